@@ -1,0 +1,1025 @@
+/*
+ * larql_oracle.c — CPU restatement of the LARQL reference algorithms on the
+ * quantised decode path (see larql_oracle.h).
+ *
+ * TEST INFRASTRUCTURE ONLY: the checker for the HIP path and the CPU baseline
+ * of the benchmark.  Never linked into, or called from, the product library.
+ *
+ * Paths in the citations are relative to the reference checkout, under
+ * crates/.  The reference is Rust: f32 arithmetic is never contracted to FMA,
+ * `f32::round` rounds half away from zero (roundf), `as u8`/`as i8`/`as i32`
+ * casts saturate and map NaN to 0, and `Iterator::sum` adds left to right.
+ * Compile with -ffp-contract=off.
+ *
+ * How each function is pinned is stated at the function.  "restatement +
+ * KATs" means no reference-held vector exists for it; the test-suite then
+ * holds it to closed-form cases and to an independent numpy restatement.
+ */
+#include "larql_oracle.h"
+
+#include <math.h>
+#include <pthread.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ------------------------------------------------------------------ bits */
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+/* Rust `x as u8` / `as i8` / `as i32` for an f32 that was already clamped:
+ * saturating, NaN -> 0. */
+static inline int32_t sat_i32(float v) {
+    if (v != v) return 0;
+    if (v >= 2147483648.0f) return INT32_MAX;
+    if (v <= -2147483648.0f) return INT32_MIN;
+    return (int32_t)v;
+}
+static inline uint8_t sat_u8(float v) {
+    if (v != v) return 0;
+    if (v <= 0.0f) return 0;
+    if (v >= 255.0f) return 255;
+    return (uint8_t)v;
+}
+static inline int8_t sat_i8(float v) {
+    if (v != v) return 0;
+    if (v <= -128.0f) return -128;
+    if (v >= 127.0f) return 127;
+    return (int8_t)v;
+}
+/* f32::clamp(lo, hi): NaN stays NaN. */
+static inline float clampf(float v, float lo, float hi) {
+    if (v < lo) return lo;
+    if (v > hi) return hi;
+    return v;
+}
+
+/* ------------------------------------------------------------ half/bf16 */
+
+/* larql-models/src/quant/half.rs:14-35 and, bit-identically,
+ * larql-compute/src/cpu/ops/q4_common/f16.rs:60-102.
+ * Pinned: all 65 536 inputs against numpy float16 (IEEE) in the tests, plus
+ * the reference's pinned subnormals (q4_common/tests/f16_subnormal_*.rs). */
+float lq_f16_to_f32(uint16_t bits) {
+    uint32_t sign = ((uint32_t)(bits >> 15)) << 31;
+    uint32_t exp = (bits >> 10) & 0x1F;
+    uint32_t mant = bits & 0x3FF;
+    if (exp == 0) {
+        if (mant == 0) return u2f(sign);
+        uint32_t e = 1, m = mant;
+        while ((m & 0x400) == 0) { m <<= 1; e += 1; }
+        return u2f(sign | ((114 - e) << 23) | ((m & 0x3FF) << 13));
+    }
+    if (exp == 31) return u2f(sign | (0xFFu << 23) | (mant << 13));
+    return u2f(sign | ((exp + 127 - 15) << 23) | (mant << 13));
+}
+
+/* larql-compute/src/cpu/ops/q4_common/f16.rs:10-41 — truncating, keeps
+ * subnormals; the Q4_K encoder's header conversion.
+ * Pinned: restatement + KATs (normals truncate, subnormals shift with the
+ * implicit one, below 2^-24 gives signed zero). */
+uint16_t lq_f32_to_f16_trunc(float val) {
+    uint32_t bits = f2u(val);
+    uint32_t sign = (bits >> 16) & 0x8000;
+    int32_t exp = (int32_t)((bits >> 23) & 0xFF);
+    uint32_t mant = bits & 0x7FFFFF;
+    if (exp == 0) return (uint16_t)sign;
+    if (exp == 255) return (uint16_t)(sign | 0x7C00 | (mant >> 13));
+    int32_t new_exp = exp - 127 + 15;
+    if (new_exp >= 31) return (uint16_t)(sign | 0x7C00);
+    if (new_exp <= 0) {
+        int32_t shift = 1 - new_exp;
+        if (13 + (uint32_t)shift >= 24) return (uint16_t)sign;
+        uint32_t sub_mant = (mant | 0x800000) >> (13 + (uint32_t)shift);
+        return (uint16_t)(sign | sub_mant);
+    }
+    return (uint16_t)(sign | ((uint32_t)new_exp << 10) | (mant >> 13));
+}
+
+/* larql-models/src/quant/half.rs:70-104 — IEEE round-to-nearest-even with
+ * subnormals; the Q8_0 encoder's scale conversion.
+ * Pinned: the reference's table (half.rs:160-200) and numpy float16 on a
+ * sweep of bit patterns. */
+uint16_t lq_f32_to_f16_nearest(float value) {
+    uint32_t bits = f2u(value);
+    uint16_t sign = (uint16_t)((bits >> 16) & 0x8000);
+    int32_t exp = (int32_t)((bits >> 23) & 0xFF);
+    uint32_t mant = bits & 0x007FFFFF;
+    if (exp == 255) return (uint16_t)(sign | (mant == 0 ? 0x7C00 : 0x7E00));
+    int32_t exp16 = exp - 127 + 15;
+    if (exp16 >= 31) return (uint16_t)(sign | 0x7C00);
+    uint32_t significand, shift;
+    if (exp16 >= 1) { significand = mant; shift = 13; }
+    else if (exp == 0 || exp16 < -10) return sign;
+    else { significand = mant | 0x00800000; shift = (uint32_t)(14 - exp16); }
+    uint32_t magnitude = significand >> shift;
+    uint32_t remainder = significand & ((1u << shift) - 1);
+    uint32_t half = 1u << (shift - 1);
+    if (remainder > half || (remainder == half && (magnitude & 1) == 1)) magnitude += 1;
+    if (exp16 >= 1) magnitude += ((uint32_t)exp16) << 10;
+    return (uint16_t)(sign | (uint16_t)magnitude);
+}
+
+/* The inline conversion inside quantize_q4_0,
+ * larql-compute/src/cpu/ops/q4_common/quantize.rs:41-58 — truncating, and
+ * everything below the f16 normal range becomes signed zero. */
+uint16_t lq_f32_to_f16_flush(float v) {
+    uint32_t bits = f2u(v);
+    uint32_t sign = (bits >> 16) & 0x8000;
+    int32_t exp = (int32_t)((bits >> 23) & 0xFF);
+    uint32_t mant = bits & 0x7FFFFF;
+    if (exp == 0) return (uint16_t)sign;
+    if (exp == 255) return (uint16_t)(sign | 0x7C00 | (mant >> 13));
+    int32_t new_exp = exp - 127 + 15;
+    if (new_exp >= 31) return (uint16_t)(sign | 0x7C00);
+    if (new_exp <= 0) return (uint16_t)sign;
+    return (uint16_t)(sign | ((uint32_t)new_exp << 10) | (mant >> 13));
+}
+
+/* larql-models/src/quant/half.rs:107-109 (truncate) and :38-40. */
+uint16_t lq_f32_to_bf16(float v) { return (uint16_t)(f2u(v) >> 16); }
+float lq_bf16_to_f32(uint16_t bits) { return u2f(((uint32_t)bits) << 16); }
+void lq_f32_to_bf16_slice(const float *src, size_t n, uint16_t *dst) {
+    for (size_t i = 0; i < n; i++) dst[i] = lq_f32_to_bf16(src[i]);
+}
+
+/* ------------------------------------------------------------------ Q4_K */
+
+/* get_scale_min_k4 unpack as every Q4_K reader in the reference writes it,
+ * e.g. q4_common/matvec_f32.rs:124-131. */
+static inline void q4k_unpack_scales(const uint8_t *p, uint8_t scales[8], uint8_t mins[8]) {
+    for (int j = 0; j < 4; j++) {
+        scales[j] = p[j] & 0x3F;
+        mins[j] = p[j + 4] & 0x3F;
+        scales[j + 4] = (uint8_t)((p[j + 8] & 0x0F) | ((p[j] >> 6) << 4));
+        mins[j + 4] = (uint8_t)((p[j + 8] >> 4) | ((p[j + 4] >> 6) << 4));
+    }
+}
+
+/* larql-compute/src/cpu/ops/q4_common/quantize.rs:89-189.
+ * Note the nibble encode uses the un-rounded f32 d/dmin, not the f16 values
+ * written to the header (:170-186).
+ * Pinned: restatement + KATs (zero block, constant blocks, two-level block)
+ * + byte-for-byte agreement with an independent numpy restatement + the
+ * round-trip bound of larql-compute/tests/test_q4k_parity.rs:48-65.
+ * No reference-held Q4_K encoder bytes exist. */
+int lq_quantize_q4_k(const float *data, size_t n, uint8_t *out) {
+    if (n % 256 != 0) return 1; /* the reference asserts */
+    size_t n_sb = n / 256;
+    for (size_t sb = 0; sb < n_sb; sb++) {
+        const float *block = data + sb * 256;
+        uint8_t *o = out + sb * 144;
+        float sub_mins[8], sub_maxs[8];
+        for (int j = 0; j < 8; j++) {
+            const float *sub = block + j * 32;
+            float mn = INFINITY, mx = -INFINITY;
+            for (int l = 0; l < 32; l++) { mn = fminf(mn, sub[l]); mx = fmaxf(mx, sub[l]); }
+            sub_mins[j] = fminf(mn, 0.0f);
+            sub_maxs[j] = fmaxf(mx, 0.0f);
+        }
+        float global_max_range = 0.0f;
+        for (int j = 0; j < 8; j++) global_max_range = fmaxf(global_max_range, sub_maxs[j] - sub_mins[j]);
+        float global_min = INFINITY;
+        for (int j = 0; j < 8; j++) global_min = fminf(global_min, sub_mins[j]);
+
+        float d = global_max_range > 0.0f ? global_max_range / (15.0f * 63.0f) : 0.0f;
+        float dmin = global_min < 0.0f ? -global_min / 63.0f : 0.0f;
+
+        uint16_t dh = lq_f32_to_f16_trunc(d), mh = lq_f32_to_f16_trunc(dmin);
+        o[0] = (uint8_t)(dh & 0xFF); o[1] = (uint8_t)(dh >> 8);
+        o[2] = (uint8_t)(mh & 0xFF); o[3] = (uint8_t)(mh >> 8);
+
+        uint8_t q_scales[8], q_mins[8];
+        for (int j = 0; j < 8; j++) {
+            float range = sub_maxs[j] - sub_mins[j];
+            q_scales[j] = d > 0.0f ? sat_u8(clampf(roundf(range / (15.0f * d)), 0.0f, 63.0f)) : 0;
+            q_mins[j] = dmin > 0.0f ? sat_u8(clampf(roundf(-sub_mins[j] / dmin), 0.0f, 63.0f)) : 0;
+        }
+        uint8_t *packed = o + 4;
+        for (int j = 0; j < 4; j++) {
+            packed[j] = (uint8_t)((q_scales[j] & 0x3F) | (((q_scales[j + 4] >> 4) & 0x03) << 6));
+            packed[j + 4] = (uint8_t)((q_mins[j] & 0x3F) | (((q_mins[j + 4] >> 4) & 0x03) << 6));
+            packed[j + 8] = (uint8_t)((q_scales[j + 4] & 0x0F) | ((q_mins[j + 4] & 0x0F) << 4));
+        }
+        uint8_t *qs = o + 16;
+        for (int g = 0; g < 4; g++) {
+            int sb_lo = 2 * g, sb_hi = 2 * g + 1;
+            float sc_lo = d * (float)q_scales[sb_lo];
+            float sc_hi = d * (float)q_scales[sb_hi];
+            float mn_lo = dmin * (float)q_mins[sb_lo];
+            float mn_hi = dmin * (float)q_mins[sb_hi];
+            float inv_lo = sc_lo > 0.0f ? 1.0f / sc_lo : 0.0f;
+            float inv_hi = sc_hi > 0.0f ? 1.0f / sc_hi : 0.0f;
+            const float *lo_sub = block + sb_lo * 32;
+            const float *hi_sub = block + sb_hi * 32;
+            for (int l = 0; l < 32; l++) {
+                uint8_t lo = sat_u8(clampf(roundf((lo_sub[l] + mn_lo) * inv_lo), 0.0f, 15.0f));
+                uint8_t hi = sat_u8(clampf(roundf((hi_sub[l] + mn_hi) * inv_hi), 0.0f, 15.0f));
+                qs[g * 32 + l] = (uint8_t)(lo | (hi << 4));
+            }
+        }
+    }
+    return 0;
+}
+
+/* larql-compute/src/cpu/ops/q4_common/dequant.rs:9-53, the same values as
+ * larql-models/src/quant/ggml/q4_k.rs:286-338.  Refusal = empty Vec.
+ * Pinned: bit-exact against the reference-held llama.cpp golden
+ * (larql-vindex/src/format/vindex3/represent/fixtures/ggml_kquant_golden.json,
+ * case q4_K). */
+int lq_dequantize_q4_k(const uint8_t *data, size_t data_len, size_t n, float *out) {
+    if (n % 256 != 0) return 1;
+    size_t n_blocks = n / 256;
+    if (data_len < n_blocks * 144) return 1;
+    for (size_t sb = 0; sb < n_blocks; sb++) {
+        const uint8_t *block = data + sb * 144;
+        float d = lq_f16_to_f32((uint16_t)(block[0] | (block[1] << 8)));
+        float dmin = lq_f16_to_f32((uint16_t)(block[2] | (block[3] << 8)));
+        uint8_t scales[8], mins[8];
+        q4k_unpack_scales(block + 4, scales, mins);
+        const uint8_t *quants = block + 16;
+        size_t sb_base = sb * 256;
+        for (int g = 0; g < 4; g++) {
+            int sb_lo = 2 * g, sb_hi = 2 * g + 1;
+            float sc_lo = d * (float)scales[sb_lo], sc_hi = d * (float)scales[sb_hi];
+            float mn_lo = dmin * (float)mins[sb_lo], mn_hi = dmin * (float)mins[sb_hi];
+            const uint8_t *chunk = quants + g * 32;
+            for (int l = 0; l < 32; l++) {
+                uint8_t byte = chunk[l];
+                out[sb_base + sb_lo * 32 + l] = sc_lo * (float)(byte & 0x0F) - mn_lo;
+                out[sb_base + sb_hi * 32 + l] = sc_hi * (float)((byte >> 4) & 0x0F) - mn_hi;
+            }
+        }
+    }
+    return 0;
+}
+
+/* KernelShapeError::check, larql-compute/src/cpu/ops/kernel_shape.rs:46-75. */
+static int kernel_shape_ok(size_t out_len, size_t rows, size_t x_len, size_t cols,
+                           size_t weight_bytes, size_t block_elems, size_t block_bytes) {
+    size_t needed = (cols / block_elems) * block_bytes * rows;
+    return out_len == rows && x_len == cols && cols % block_elems == 0 && weight_bytes >= needed;
+}
+
+/* q4_dual_dot_32, scalar arm: q4_common/dual.rs:178-199. */
+static inline void q4_dual_dot_32(const uint8_t *chunk, const float *x_lo, const float *x_hi,
+                                  float *dot_lo_out, float *dot_hi_out) {
+    float dot_lo = 0.0f, dot_hi = 0.0f;
+    for (int l = 0; l < 32; l++) {
+        uint8_t byte = chunk[l];
+        float q_lo = (float)(byte & 0x0F);
+        float q_hi = (float)((byte >> 4) & 0x0F);
+        dot_lo += q_lo * x_lo[l];
+        dot_hi += q_hi * x_hi[l];
+    }
+    *dot_lo_out = dot_lo; *dot_hi_out = dot_hi;
+}
+
+/* process_q4k_superblock: q4_common/matvec_f32.rs:116-155. */
+static inline float process_q4k_superblock(const uint8_t *w, const float *x, const float *sum_x,
+                                           size_t row_base, size_t sb) {
+    const uint8_t *block = w + row_base + sb * 144;
+    float d = lq_f16_to_f32((uint16_t)(block[0] | (block[1] << 8)));
+    float dmin = lq_f16_to_f32((uint16_t)(block[2] | (block[3] << 8)));
+    uint8_t scales[8], mins[8];
+    q4k_unpack_scales(block + 4, scales, mins);
+    const uint8_t *quants = block + 16;
+    size_t x_sb_base = sb * 256;
+    float acc = 0.0f;
+    for (int g = 0; g < 4; g++) {
+        int sb_lo = 2 * g, sb_hi = 2 * g + 1;
+        float sc_lo = d * (float)scales[sb_lo], sc_hi = d * (float)scales[sb_hi];
+        float mn_lo = dmin * (float)mins[sb_lo], mn_hi = dmin * (float)mins[sb_hi];
+        float sumy_lo = sum_x[sb * 8 + sb_lo], sumy_hi = sum_x[sb * 8 + sb_hi];
+        float dot_lo, dot_hi;
+        q4_dual_dot_32(quants + g * 32, x + x_sb_base + sb_lo * 32, x + x_sb_base + sb_hi * 32,
+                       &dot_lo, &dot_hi);
+        acc += sc_lo * dot_lo - mn_lo * sumy_lo;
+        acc += sc_hi * dot_hi - mn_hi * sumy_hi;
+    }
+    return acc;
+}
+
+static float *q4k_sum_x(const float *x, size_t n_blocks) {
+    /* q4_common/matvec_f32.rs:63-74 */
+    size_t n_sub = n_blocks * 8;
+    float *sum_x = (float *)malloc((n_sub ? n_sub : 1) * sizeof(float));
+    for (size_t sub = 0; sub < n_sub; sub++) {
+        float s = 0.0f;
+        for (int l = 0; l < 32; l++) s += x[sub * 32 + l];
+        sum_x[sub] = s;
+    }
+    return sum_x;
+}
+
+static void q4k_rows(float *out, const float *x, const uint8_t *w, const float *sum_x,
+                     size_t r0, size_t r1, size_t n_blocks) {
+    size_t row_bytes = n_blocks * 144;
+    for (size_t r = r0; r < r1; r++) {
+        float acc = 0.0f;
+        for (size_t sb = 0; sb < n_blocks; sb++)
+            acc += process_q4k_superblock(w, x, sum_x, r * row_bytes, sb);
+        out[r] = acc;
+    }
+}
+
+/* CpuBackend::q4k_matvec -> q4k_matvec_into:
+ * larql-compute/src/cpu/mod.rs:95-114, q4_common/matvec_f32.rs:37-106.
+ * Row chunking only decides which thread runs a row, so the serial loop is
+ * the same arithmetic.
+ * Pinned: equals sum(dequantize(bytes) * x) to rounding on the golden q4_K
+ * bytes and on seeded bytes (the reference's own oracle,
+ * q4_common/tests/quantize_q4_0_tests.rs:69-149), f64 brute force on small
+ * shapes, and the refusal table of quantize_q4_0_tests.rs:351-389.  The
+ * last-ulp accumulation order is restatement only. */
+int lq_q4k_matvec_into(float *out, size_t out_len, const float *x, size_t x_len,
+                       const uint8_t *w, size_t w_len, size_t rows, size_t cols) {
+    if (!kernel_shape_ok(out_len, rows, x_len, cols, w_len, 256, 144)) return 1;
+    if (rows == 0 || cols == 0) { for (size_t i = 0; i < out_len; i++) out[i] = 0.0f; return 0; }
+    size_t n_blocks = cols / 256;
+    float *sum_x = q4k_sum_x(x, n_blocks);
+    q4k_rows(out, x, w, sum_x, 0, rows, n_blocks);
+    free(sum_x);
+    return 0;
+}
+
+/* q4k_matvec::dispatch (scalar cross-backend reference):
+ * larql-compute/src/cpu/ops/q4k_matvec.rs:72-117 — association
+ * (sc*q - mn)*x per element.  Uses the powi-based f16 decode of that file
+ * (:22-50), which agrees with lq_f16_to_f32 on every finite input. */
+int lq_q4k_matvec_scalar(float *out, const float *x, const uint8_t *w, size_t rows, size_t hidden) {
+    size_t superblocks = hidden / 256, bytes_per_row = superblocks * 144;
+    for (size_t row = 0; row < rows; row++) {
+        float acc = 0.0f;
+        for (size_t sb = 0; sb < superblocks; sb++) {
+            const uint8_t *block = w + row * bytes_per_row + sb * 144;
+            float d = lq_f16_to_f32((uint16_t)(block[0] | (block[1] << 8)));
+            float dmin = lq_f16_to_f32((uint16_t)(block[2] | (block[3] << 8)));
+            uint8_t scales[8], mins[8];
+            q4k_unpack_scales(block + 4, scales, mins);
+            const uint8_t *qs = block + 16;
+            size_t x_base = sb * 256;
+            for (int g = 0; g < 4; g++) {
+                int sb_lo = 2 * g, sb_hi = 2 * g + 1;
+                float sc_lo = d * (float)scales[sb_lo], sc_hi = d * (float)scales[sb_hi];
+                float mn_lo = dmin * (float)mins[sb_lo], mn_hi = dmin * (float)mins[sb_hi];
+                for (int l = 0; l < 32; l++) {
+                    uint8_t byte = qs[g * 32 + l];
+                    float lo = (float)(byte & 0x0F), hi = (float)((byte >> 4) & 0x0F);
+                    acc += (sc_lo * lo - mn_lo) * x[x_base + sb_lo * 32 + l];
+                    acc += (sc_hi * hi - mn_hi) * x[x_base + sb_hi * 32 + l];
+                }
+            }
+        }
+        out[row] = acc;
+    }
+    return 0;
+}
+
+/* q4k_dual_matvec_into: q4_common/dual.rs:22-167 — per-row operation order
+ * is that of two q4k_matvec_into calls (the reference's own test,
+ * q4_common/neon_tests.rs:75-117). */
+int lq_q4k_dual_matvec_into(float *out_a, float *out_b, size_t out_len,
+                            const float *x, size_t x_len,
+                            const uint8_t *w_a, size_t wa_len,
+                            const uint8_t *w_b, size_t wb_len,
+                            size_t rows, size_t cols) {
+    if (!kernel_shape_ok(out_len, rows, x_len, cols, wa_len, 256, 144)) return 1;
+    if (!kernel_shape_ok(out_len, rows, x_len, cols, wb_len, 256, 144)) return 1;
+    if (rows == 0 || cols == 0) {
+        for (size_t i = 0; i < out_len; i++) { out_a[i] = 0.0f; out_b[i] = 0.0f; }
+        return 0;
+    }
+    size_t n_blocks = cols / 256;
+    float *sum_x = q4k_sum_x(x, n_blocks);
+    q4k_rows(out_a, x, w_a, sum_x, 0, rows, n_blocks);
+    q4k_rows(out_b, x, w_b, sum_x, 0, rows, n_blocks);
+    free(sum_x);
+    return 0;
+}
+
+/* decode_q4k_superblock_into: q4_common/matvec_f32.rs:166-199. */
+static void decode_q4k_superblock_into(const uint8_t *w, size_t row_base, size_t sb, float *wf) {
+    const uint8_t *block = w + row_base + sb * 144;
+    float d = lq_f16_to_f32((uint16_t)(block[0] | (block[1] << 8)));
+    float dmin = lq_f16_to_f32((uint16_t)(block[2] | (block[3] << 8)));
+    uint8_t scales[8], mins[8];
+    q4k_unpack_scales(block + 4, scales, mins);
+    const uint8_t *quants = block + 16;
+    for (int g = 0; g < 4; g++) {
+        int sb_lo = 2 * g, sb_hi = 2 * g + 1;
+        float sc_lo = d * (float)scales[sb_lo], sc_hi = d * (float)scales[sb_hi];
+        float mn_lo = dmin * (float)mins[sb_lo], mn_hi = dmin * (float)mins[sb_hi];
+        const uint8_t *chunk = quants + g * 32;
+        for (int i = 0; i < 32; i++) {
+            wf[sb_lo * 32 + i] = sc_lo * (float)(chunk[i] & 0x0F) - mn_lo;
+            wf[sb_hi * 32 + i] = sc_hi * (float)(chunk[i] >> 4) - mn_hi;
+        }
+    }
+}
+
+/* dot_256_f32_scalar: q4_common/matvec_f32.rs:250-258. */
+static float dot_256_f32_scalar(const float *wf, const float *xs) {
+    float acc[8] = {0};
+    for (int c = 0; c < 32; c++)
+        for (int l = 0; l < 8; l++) acc[l] += wf[c * 8 + l] * xs[c * 8 + l];
+    float s = 0.0f;
+    for (int l = 0; l < 8; l++) s += acc[l];
+    return s;
+}
+
+/* q4k_matmul_into / kquant_matmul_into: q4_common/matmul.rs:20-139.
+ * out is [seq, rows]; shape errors zero the output (:89-98).
+ * Pinned: rows equal stacked matvec to 1e-4 and dequant-then-matmul to 5e-3
+ * (the reference's tests, quantize_q4_0_tests.rs:155-238). */
+void lq_q4k_matmul_into(float *out, const float *x, const uint8_t *w, size_t w_len,
+                        size_t rows, size_t hidden, size_t seq) {
+    size_t out_len = seq * rows;
+    if (rows == 0 || seq == 0 || hidden == 0 || hidden % 256 != 0) {
+        for (size_t i = 0; i < out_len; i++) out[i] = 0.0f;
+        return;
+    }
+    size_t n_blocks = hidden / 256, row_bytes = n_blocks * 144;
+    if (w_len < rows * row_bytes) {
+        for (size_t i = 0; i < out_len; i++) out[i] = 0.0f;
+        return;
+    }
+    float *tmp = (float *)calloc(rows * seq, sizeof(float));
+    float wf[256];
+    for (size_t r = 0; r < rows; r++) {
+        float *out_row = tmp + r * seq;
+        for (size_t sb = 0; sb < n_blocks; sb++) {
+            decode_q4k_superblock_into(w, r * row_bytes, sb, wf);
+            size_t x_off = sb * 256;
+            for (size_t s = 0; s < seq; s++) out_row[s] += dot_256_f32_scalar(wf, x + s * hidden + x_off);
+        }
+    }
+    for (size_t r = 0; r < rows; r++)
+        for (size_t s = 0; s < seq; s++) out[s * rows + r] = tmp[r * seq + s];
+    free(tmp);
+}
+
+/* ------------------------------------------------------------------ Q8_0 */
+
+/* larql-models/src/quant/ggml/quantize.rs:50-77.  Codes use the reciprocal
+ * of the un-rounded f32 scale.
+ * Pinned: byte-for-byte against the reference-held ggml golden blocks
+ * (larql-models/src/quant/ggml/tests/q8_0_ggml_golden.rs). */
+int lq_quantize_q8_0(const float *data, size_t n, uint8_t *out) {
+    if (n % 32 != 0) return 1;
+    size_t n_blocks = n / 32;
+    for (size_t i = 0; i < n_blocks; i++) {
+        const float *block = data + i * 32;
+        float amax = 0.0f;
+        for (int j = 0; j < 32; j++) amax = fmaxf(amax, fabsf(block[j]));
+        float scale = amax / 127.0f;
+        float inv_scale = scale > 0.0f ? 1.0f / scale : 0.0f;
+        uint16_t sh = lq_f32_to_f16_nearest(scale);
+        uint8_t *o = out + i * 34;
+        o[0] = (uint8_t)(sh & 0xFF); o[1] = (uint8_t)(sh >> 8);
+        for (int j = 0; j < 32; j++)
+            o[2 + j] = (uint8_t)sat_i8(clampf(roundf(block[j] * inv_scale), -128.0f, 127.0f));
+    }
+    return 0;
+}
+
+/* larql-models/src/quant/ggml/legacy.rs:68-83.
+ * Pinned: bit-exact against ggml_kquant_golden.json case q8_0. */
+int lq_dequantize_q8_0(const uint8_t *data, size_t data_len, size_t n, float *out) {
+    if (n % 32 != 0) return 1;
+    size_t n_blocks = n / 32;
+    if (data_len < n_blocks * 34) return 1;
+    for (size_t i = 0; i < n_blocks; i++) {
+        const uint8_t *block = data + i * 34;
+        float scale = lq_f16_to_f32((uint16_t)(block[0] | (block[1] << 8)));
+        for (int j = 0; j < 32; j++) out[i * 32 + j] = (float)(int8_t)block[2 + j] * scale;
+    }
+    return 0;
+}
+
+static float q8_0_row_dot(const uint8_t *blocks, const float *x, size_t row, size_t per_row) {
+    /* larql-compute/src/cpu/kquant_gemv.rs:92-109 */
+    float acc = 0.0f;
+    for (size_t b = 0; b < per_row; b++) {
+        const uint8_t *base = blocks + (row * per_row + b) * 34;
+        float d = lq_f16_to_f32((uint16_t)(base[0] | (base[1] << 8)));
+        const float *xs = x + b * 32;
+        for (int j = 0; j < 32; j++) acc += ((float)(int8_t)base[2 + j] * d) * xs[j];
+    }
+    return acc;
+}
+
+/* q8_0_gemv: larql-compute/src/cpu/kquant_gemv.rs:67-90.  Exact length.
+ * Pinned: bit-for-bit equal to dequantize-then-multiply in element order
+ * (the reference's own assert_eq!, kquant_gemv_tests.rs:92-105), on the
+ * golden q8_0 bytes and on seeded bytes; refusals of :133-151. */
+int lq_q8_0_gemv(const uint8_t *blocks, size_t blocks_len, const float *x, size_t x_len,
+                 size_t n, size_t k, float *out) {
+    if (k == 0 || k % 32 != 0 || x_len != k) return 1;
+    size_t per_row = k / 32;
+    if (blocks_len != n * per_row * 34) return 1;
+    for (size_t r = 0; r < n; r++) out[r] = q8_0_row_dot(blocks, x, r, per_row);
+    return 0;
+}
+
+/* ------------------------------------------------------------ Q4_0 x Q8 */
+
+/* quantize_to_q8: q4_common/quantize.rs:6-22. */
+void lq_quantize_to_q8(const float *x, size_t n, int8_t *q8, float *scales) {
+    size_t n_blocks = n / 32;
+    for (size_t i = 0; i < n; i++) q8[i] = 0;
+    for (size_t b = 0; b < n_blocks; b++) {
+        const float *block = x + b * 32;
+        float amax = 0.0f;
+        for (int j = 0; j < 32; j++) amax = fmaxf(amax, fabsf(block[j]));
+        float scale = amax / 127.0f;
+        scales[b] = scale;
+        float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
+        for (int j = 0; j < 32; j++)
+            q8[b * 32 + j] = sat_i8(clampf(roundf(block[j] * inv), -128.0f, 127.0f));
+    }
+}
+
+/* quantize_q4_0: q4_common/quantize.rs:28-69 (planar nibbles). */
+int lq_quantize_q4_0(const float *data, size_t n, uint8_t *out) {
+    if (n % 32 != 0) return 1;
+    size_t n_blocks = n / 32;
+    for (size_t i = 0; i < n_blocks; i++) {
+        const float *block = data + i * 32;
+        float amax = 0.0f;
+        for (int j = 0; j < 32; j++) amax = fmaxf(amax, fabsf(block[j]));
+        float scale = amax / 7.0f;
+        float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
+        uint16_t h = lq_f32_to_f16_flush(scale);
+        uint8_t *o = out + i * 18;
+        o[0] = (uint8_t)(h & 0xFF); o[1] = (uint8_t)(h >> 8);
+        for (int j = 0; j < 16; j++) {
+            int32_t lo = sat_i32(roundf(block[j] * inv)) + 8;
+            int32_t hi = sat_i32(roundf(block[j + 16] * inv)) + 8;
+            lo = lo < 0 ? 0 : (lo > 15 ? 15 : lo);
+            hi = hi < 0 ? 0 : (hi > 15 ? 15 : hi);
+            o[2 + j] = (uint8_t)(lo | (hi << 4));
+        }
+    }
+    return 0;
+}
+
+/* q4_0_matvec_c, scalar arm: larql-compute/csrc/q4_dot.c:176-207.
+ * Pinned: bit-for-bit against that C file compiled from the reference tree
+ * (oracle/_ref/libq4dot_ref.so) wherever it builds. */
+void lq_q4_0_matvec(const uint8_t *q4, const int8_t *q8_x, const float *q8_scales,
+                    float *scores, size_t num_rows, size_t hidden) {
+    size_t blocks_per_row = hidden / 32, bytes_per_row = blocks_per_row * 18;
+    for (size_t row = 0; row < num_rows; row++) {
+        float acc = 0.0f;
+        const uint8_t *row_data = q4 + row * bytes_per_row;
+        for (size_t b = 0; b < blocks_per_row; b++) {
+            const uint8_t *block = row_data + b * 18;
+            float combined = lq_f16_to_f32((uint16_t)(block[0] | (block[1] << 8))) * q8_scales[b];
+            const int8_t *q8p = q8_x + b * 32;
+            for (int j = 0; j < 16; j++) {
+                uint8_t byte = block[2 + j];
+                int lo_v = (byte & 0x0F) - 8, hi_v = ((byte >> 4) & 0x0F) - 8;
+                acc += (float)lo_v * (float)q8p[j] * combined;
+                acc += (float)hi_v * (float)q8p[j + 16] * combined;
+            }
+        }
+        scores[row] = acc;
+    }
+}
+
+/* dequantise_q8: larql-compute/src/backend/quant_matvec.rs:24-40. */
+void lq_dequantise_q8(const int8_t *q8_x, size_t n, const float *scales, float *out) {
+    size_t n_blocks = n / 32;
+    for (size_t b = 0; b < n_blocks; b++)
+        for (int j = 0; j < 32; j++) out[b * 32 + j] = (float)q8_x[b * 32 + j] * scales[b];
+    for (size_t i = n_blocks * 32; i < n; i++) out[i] = (float)q8_x[i];
+}
+
+/* ----------------------------------------------------------------- MXFP4 */
+
+static const float MXFP4_TABLE[16] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f,
+                                      -0.0f, -0.5f, -1.0f, -1.5f, -2.0f, -3.0f, -4.0f, -6.0f};
+float lq_mxfp4_table(unsigned code) { return MXFP4_TABLE[code & 15]; }
+
+/* larql-models/src/quant/mxfp4.rs:26-35.  Pinned: KATs of mxfp4.rs:276-297. */
+float lq_e8m0_to_f32(uint8_t byte) {
+    if (byte == 0) return 0.0f;
+    if (byte == 255) return NAN;
+    return u2f(((uint32_t)byte) << 23);
+}
+
+/* larql-vindex/src/format/vindex3/opplan/exec/weights/quantize.rs:71-88. */
+uint8_t lq_nearest_mxfp4_code(float v) {
+    uint8_t sign = (f2u(v) >> 31) ? 8 : 0;
+    float mag = fminf(fabsf(v), 6.0f);
+    uint8_t best = 0;
+    float best_err = INFINITY;
+    for (unsigned code = 0; code < 8; code++) {
+        float err = fabsf(mag - MXFP4_TABLE[code]);
+        if (err < best_err || (err == best_err && code % 2 == 0)) { best = (uint8_t)code; best_err = err; }
+    }
+    return best == 0 ? 0 : (uint8_t)(sign | best);
+}
+
+/* quantize_mxfp4: .../opplan/exec/weights/load.rs:410-476.  The shared
+ * exponent is floor(log2f(max|x|)) - 2 computed in f32 with libm, as Rust's
+ * f32::log2 does.
+ * Pinned: restatement + KATs (powers of two, ties, saturation, all-zero
+ * group) + round trip through the decoder; no reference-held bytes. */
+int lq_quantize_mxfp4(const float *values, size_t rows, size_t k, uint8_t *packed, uint8_t *scales) {
+    if (k % 32 != 0) return 1;
+    size_t groups = k / 32;
+    for (size_t r = 0; r < rows; r++) {
+        for (size_t g = 0; g < groups; g++) {
+            const float *group = values + r * k + g * 32;
+            float max_abs = 0.0f;
+            for (int i = 0; i < 32; i++) max_abs = fmaxf(max_abs, fabsf(group[i]));
+            uint8_t scale_byte;
+            if (max_abs == 0.0f) scale_byte = 0;
+            else {
+                int32_t exponent = sat_i32(floorf(log2f(max_abs))) - 2;
+                int32_t e = exponent + 127;
+                e = e < 1 ? 1 : (e > 254 ? 254 : e);
+                scale_byte = (uint8_t)e;
+            }
+            scales[r * groups + g] = scale_byte;
+            float scale = lq_e8m0_to_f32(scale_byte);
+            float inv = scale == 0.0f ? 0.0f : 1.0f / scale;
+            uint8_t *bytes = packed + (r * groups + g) * 16;
+            for (int b = 0; b < 16; b++) {
+                uint8_t lo = lq_nearest_mxfp4_code(group[2 * b] * inv);
+                uint8_t hi = lq_nearest_mxfp4_code(group[2 * b + 1] * inv);
+                bytes[b] = (uint8_t)(lo | (hi << 4));
+            }
+        }
+    }
+    return 0;
+}
+
+/* dequantize_expert: larql-models/src/quant/mxfp4.rs:42-95.
+ * Pinned: KATs of mxfp4.rs:312-380. */
+int lq_dequantize_mxfp4_expert(const uint8_t *blocks, size_t blocks_len,
+                               const uint8_t *scales, size_t scales_len,
+                               size_t out_features, size_t groups, float *out) {
+    if (blocks_len < out_features * groups * 16) return 1;
+    if (scales_len < out_features * groups) return 1;
+    size_t in_features = groups * 32;
+    for (size_t row = 0; row < out_features; row++)
+        for (size_t g = 0; g < groups; g++) {
+            float scale = lq_e8m0_to_f32(scales[row * groups + g]);
+            const uint8_t *blk = blocks + (row * groups + g) * 16;
+            for (int b = 0; b < 16; b++) {
+                size_t o = row * in_features + g * 32 + (size_t)b * 2;
+                out[o] = MXFP4_TABLE[blk[b] & 0x0F] * scale;
+                out[o + 1] = MXFP4_TABLE[(blk[b] >> 4) & 0x0F] * scale;
+            }
+        }
+    return 0;
+}
+
+/* The CPU stand-in of MatMul::mxfp4_gemv: LoopDevice::mxfp4_gemv / mxfp4_loop,
+ * larql-vindex/src/format/vindex3/opplan/exec/tests/device.rs:87-127, with
+ * the validation of larql-compute/src/backend/matmul.rs:226-235 as the Metal
+ * peer applies it. */
+int lq_mxfp4_gemv(const uint8_t *packed, size_t packed_len, const uint8_t *scales, size_t scales_len,
+                  const float *x, size_t x_len, size_t n, size_t k, float *out) {
+    if (k % 32 != 0 || x_len < k) return 1;
+    if (packed_len < n * (k / 32) * 16 || scales_len < n * (k / 32)) return 1;
+    size_t groups = k / 32;
+    for (size_t row = 0; row < n; row++) {
+        float acc = 0.0f;
+        for (size_t g = 0; g < groups; g++) {
+            float scale = lq_e8m0_to_f32(scales[row * groups + g]);
+            const uint8_t *bytes = packed + (row * groups + g) * 16;
+            for (int b = 0; b < 16; b++) {
+                size_t e0 = g * 32 + 2 * (size_t)b;
+                acc += MXFP4_TABLE[bytes[b] & 0x0F] * scale * x[e0];
+                acc += MXFP4_TABLE[bytes[b] >> 4] * scale * x[e0 + 1];
+            }
+        }
+        out[row] = acc;
+    }
+    return 0;
+}
+
+/* dequantize_expert + row dot: the reference the Metal peer's tests use,
+ * larql-compute-metal/src/trait_impl/mxfp4.rs:201-206. */
+int lq_mxfp4_gemv_dequant(const uint8_t *packed, const uint8_t *scales, const float *x,
+                          size_t n, size_t k, float *out) {
+    size_t groups = k / 32;
+    float *w = (float *)malloc(n * k * sizeof(float));
+    lq_dequantize_mxfp4_expert(packed, n * groups * 16, scales, n * groups, n, groups, w);
+    for (size_t r = 0; r < n; r++) {
+        float acc = 0.0f;
+        for (size_t c = 0; c < k; c++) acc += w[r * k + c] * x[c];
+        out[r] = acc;
+    }
+    free(w);
+    return 0;
+}
+
+/* ----------------------------------------------------------- dense gemv */
+
+/* bf16_dot_portable per row:
+ * larql-vindex/src/format/vindex3/opplan/exec/cpu/kernels.rs:718-723. */
+void lq_bf16_gemv(const uint16_t *w, const float *x, size_t n, size_t k, float *out) {
+    for (size_t r = 0; r < n; r++) {
+        float acc = 0.0f;
+        for (size_t c = 0; c < k; c++) acc += lq_bf16_to_f32(w[r * k + c]) * x[c];
+        out[r] = acc;
+    }
+}
+/* f16 gates are widened then multiplied (gate_store.rs:353-444 decode cache). */
+void lq_f16_gemv(const uint16_t *w, const float *x, size_t n, size_t k, float *out) {
+    for (size_t r = 0; r < n; r++) {
+        float acc = 0.0f;
+        for (size_t c = 0; c < k; c++) acc += lq_f16_to_f32(w[r * k + c]) * x[c];
+        out[r] = acc;
+    }
+}
+/* gemv: larql-vindex/src/index/storage/gate_store.rs:119-143.  The reference
+ * calls cblas_sgemv of whatever OpenBLAS the host has (ndarray 0.16.1 /
+ * openblas-src 0.10.15, system library, unpinned): its summation order is not
+ * fixed, so this sequential row dot is parity "within fp32 reordering". */
+void lq_f32_gemv(const float *w, const float *x, size_t n, size_t k, float *out) {
+    for (size_t r = 0; r < n; r++) {
+        float acc = 0.0f;
+        for (size_t c = 0; c < k; c++) acc += w[r * k + c] * x[c];
+        out[r] = acc;
+    }
+}
+
+/* ---------------------------------------------------------------- top-K */
+
+/* top_k_by_abs: larql-vindex/src/index/compute/gate_knn/mod.rs:50-108.
+ * The min-heap is Rust's std BinaryHeap (push = sift_up, pop = swap the last
+ * element to the root, sift_down_to_bottom, sift_up), restated so that the
+ * eviction among equal |values| follows the same heap order.  The final
+ * sort_unstable leaves the order of equal |values| unspecified; a stable
+ * sort over the heap's vector order is used here.
+ * Pinned: the closed-form cases of gate_knn/mod.rs:231-287 and brute-force
+ * full sort on tie-free data; tie eviction is restatement only. */
+typedef struct { uint64_t idx; float val; } abs_score;
+
+/* heap order: a <= b  <=>  not (|a| < |b|)   (Ord reversed on |val|) */
+static inline int heap_le(const abs_score *a, const abs_score *b) {
+    return !(fabsf(a->val) < fabsf(b->val));
+}
+static size_t heap_sift_up(abs_score *d, size_t start, size_t pos) {
+    abs_score elt = d[pos];
+    while (pos > start) {
+        size_t parent = (pos - 1) / 2;
+        if (heap_le(&elt, &d[parent])) break;
+        d[pos] = d[parent];
+        pos = parent;
+    }
+    d[pos] = elt;
+    return pos;
+}
+static void heap_sift_down_to_bottom(abs_score *d, size_t len, size_t pos) {
+    size_t end = len, start = pos;
+    abs_score elt = d[pos];
+    size_t child = 2 * pos + 1;
+    size_t lim = end >= 2 ? end - 2 : 0;
+    while (child <= lim && end >= 2) {
+        child += heap_le(&d[child], &d[child + 1]) ? 1 : 0;
+        d[pos] = d[child];
+        pos = child;
+        child = 2 * pos + 1;
+    }
+    if (child == end - 1) { d[pos] = d[child]; pos = child; }
+    d[pos] = elt;
+    heap_sift_up(d, start, pos);
+}
+
+long lq_top_k_by_abs(const float *scores, size_t n, size_t top_k, uint64_t *idx_out, float *val_out) {
+    if (top_k == 0) return 0;
+    for (size_t i = 0; i < n; i++) if (scores[i] != scores[i]) return -1; /* partial_cmp().unwrap() panics */
+    size_t cap = top_k < n ? top_k : n;
+    abs_score *heap = (abs_score *)malloc((cap ? cap : 1) * sizeof(abs_score));
+    size_t len = 0;
+    for (size_t i = 0; i < n; i++) {
+        float v = scores[i];
+        if (len < top_k) {
+            heap[len].idx = i; heap[len].val = v; len++;
+            heap_sift_up(heap, 0, len - 1);
+        } else if (fabsf(v) > fabsf(heap[0].val)) {
+            /* pop */
+            abs_score item = heap[len - 1];
+            len--;
+            if (len > 0) {
+                abs_score t = heap[0]; heap[0] = item; item = t;
+                heap_sift_down_to_bottom(heap, len, 0);
+            }
+            /* push */
+            heap[len].idx = i; heap[len].val = v; len++;
+            heap_sift_up(heap, 0, len - 1);
+        }
+    }
+    /* stable insertion sort, |val| descending */
+    for (size_t i = 1; i < len; i++) {
+        abs_score e = heap[i];
+        size_t j = i;
+        while (j > 0 && fabsf(heap[j - 1].val) < fabsf(e.val)) { heap[j] = heap[j - 1]; j--; }
+        heap[j] = e;
+    }
+    for (size_t i = 0; i < len; i++) { idx_out[i] = heap[i].idx; val_out[i] = heap[i].val; }
+    free(heap);
+    return (long)len;
+}
+
+/* top_k_sorted: larql-vindex/src/index/storage/lm_head/knn.rs:315-386 —
+ * by value descending, non-finite scores skipped. */
+typedef struct { float s; uint32_t i; } val_score;
+static void vs_sift_down(val_score *h, size_t n, size_t i) {
+    for (;;) {
+        size_t smallest = i, l = 2 * i + 1, r = 2 * i + 2;
+        if (l < n && h[l].s < h[smallest].s) smallest = l;
+        if (r < n && h[r].s < h[smallest].s) smallest = r;
+        if (smallest == i) break;
+        val_score t = h[i]; h[i] = h[smallest]; h[smallest] = t;
+        i = smallest;
+    }
+}
+long lq_top_k_sorted(const float *scores, size_t n, size_t top_k, uint32_t *idx_out, float *val_out) {
+    if (n == 0 || top_k == 0) return 0;
+    size_t k = top_k < n ? top_k : n;
+    if (k == 1) {
+        uint32_t best_i = 0; float best_v = -INFINITY;
+        for (size_t i = 0; i < n; i++) if (isfinite(scores[i]) && scores[i] > best_v) { best_v = scores[i]; best_i = (uint32_t)i; }
+        if (best_v == -INFINITY) return 0;
+        idx_out[0] = best_i; val_out[0] = best_v;
+        return 1;
+    }
+    val_score *heap = (val_score *)malloc((k + 1) * sizeof(val_score));
+    size_t len = 0;
+    for (size_t i = 0; i < n; i++) {
+        float s = scores[i];
+        if (!isfinite(s)) continue;
+        if (len < k) {
+            heap[len].s = s; heap[len].i = (uint32_t)i; len++;
+            if (len == k) for (size_t j = k / 2; j-- > 0;) vs_sift_down(heap, len, j);
+        } else if (s > heap[0].s) {
+            heap[0].s = s; heap[0].i = (uint32_t)i;
+            vs_sift_down(heap, len, 0);
+        }
+    }
+    /* (the reference re-heapifies a short heap here; the sort below makes it moot) */
+    for (size_t i = 1; i < len; i++) {
+        val_score e = heap[i];
+        size_t j = i;
+        while (j > 0 && heap[j - 1].s < e.s) { heap[j] = heap[j - 1]; j--; }
+        heap[j] = e;
+    }
+    for (size_t i = 0; i < len; i++) { idx_out[i] = heap[i].i; val_out[i] = heap[i].s; }
+    free(heap);
+    return (long)len;
+}
+
+static int cmp_u64(const void *a, const void *b) {
+    uint64_t x = *(const uint64_t *)a, y = *(const uint64_t *)b;
+    return x < y ? -1 : (x > y ? 1 : 0);
+}
+
+/* gate_knn_batch: larql-vindex/src/index/compute/gate_knn/dispatch.rs:256-304
+ * — per-position top_k_by_abs over column s of scores_2d [n_features, seq],
+ * then the sorted, de-duplicated union of the indices. */
+long lq_gate_knn_batch_union(const float *scores_2d, size_t n_features, size_t seq, size_t top_k,
+                             uint64_t *idx_out, size_t idx_cap) {
+    if (seq == 0) return 0;
+    size_t k = top_k < n_features ? top_k : n_features;
+    if (k == 0) return 0;
+    float *col = (float *)malloc(n_features * sizeof(float));
+    uint64_t *all = (uint64_t *)malloc(seq * k * sizeof(uint64_t));
+    float *vals = (float *)malloc(k * sizeof(float));
+    size_t total = 0;
+    for (size_t s = 0; s < seq; s++) {
+        for (size_t f = 0; f < n_features; f++) col[f] = scores_2d[f * seq + s];
+        long got = lq_top_k_by_abs(col, n_features, k, all + total, vals);
+        if (got < 0) { free(col); free(all); free(vals); return -1; }
+        total += (size_t)got;
+    }
+    qsort(all, total, sizeof(uint64_t), cmp_u64);
+    size_t m = 0;
+    for (size_t i = 0; i < total; i++) if (i == 0 || all[i] != all[i - 1]) { if (m < idx_cap) idx_out[m] = all[i]; m++; }
+    free(col); free(all); free(vals);
+    return (long)m;
+}
+
+/* ---------------------------------------------------------- MoE routing */
+
+/* router::select: larql-compute/src/ffn/expert_weight/router.rs:33-70.
+ * Stable sort by logit descending (first index wins ties), softmax with the
+ * global max shift over all experts or over the selected ones.
+ * Pinned: KATs of router.rs:79-200 (sums to 1, matches a full softmax, ties
+ * go to the first index). */
+size_t lq_router_select(const float *logits, size_t n, size_t k, int policy,
+                        uint64_t *experts, float *weights) {
+    if (k > n) k = n;
+    if (k == 0) return 0;
+    uint64_t *ri = (uint64_t *)malloc(n * sizeof(uint64_t));
+    float *rv = (float *)malloc(n * sizeof(float));
+    for (size_t i = 0; i < n; i++) { ri[i] = i; rv[i] = logits[i]; }
+    for (size_t i = 1; i < n; i++) { /* stable, descending */
+        uint64_t ei = ri[i]; float ev = rv[i];
+        size_t j = i;
+        while (j > 0 && ev > rv[j - 1]) { ri[j] = ri[j - 1]; rv[j] = rv[j - 1]; j--; }
+        ri[j] = ei; rv[j] = ev;
+    }
+    float dmax = -INFINITY;
+    for (size_t i = 0; i < n; i++) dmax = fmaxf(dmax, logits[i]);
+    float denom = 0.0f;
+    if (policy == LQ_ROUTE_SOFTMAX_THEN_SELECT) for (size_t i = 0; i < n; i++) denom += expf(logits[i] - dmax);
+    else for (size_t i = 0; i < k; i++) denom += expf(rv[i] - dmax);
+    for (size_t i = 0; i < k; i++) {
+        experts[i] = ri[i];
+        weights[i] = denom > 0.0f ? expf(rv[i] - dmax) / denom : 0.0f;
+    }
+    free(ri); free(rv);
+    return k;
+}
+
+/* math::top_k: larql-compute/src/cpu/ops/moe/math.rs:152-164 — value
+ * descending, index ascending. */
+size_t lq_moe_top_k(const float *v, size_t n, size_t k, uint64_t *idx, float *val) {
+    if (k > n) k = n;
+    uint64_t *ri = (uint64_t *)malloc((n ? n : 1) * sizeof(uint64_t));
+    for (size_t i = 0; i < n; i++) ri[i] = i;
+    for (size_t i = 1; i < n; i++) {
+        uint64_t e = ri[i];
+        size_t j = i;
+        while (j > 0 && (v[e] > v[ri[j - 1]])) { ri[j] = ri[j - 1]; j--; }
+        ri[j] = e;
+    }
+    for (size_t i = 0; i < k; i++) { idx[i] = ri[i]; val[i] = v[ri[i]]; }
+    free(ri);
+    return k;
+}
+
+/* math::softmax: moe/math.rs:130-142. */
+void lq_softmax(float *v, size_t n) {
+    float max = -INFINITY;
+    for (size_t i = 0; i < n; i++) max = fmaxf(max, v[i]);
+    float sum = 0.0f;
+    for (size_t i = 0; i < n; i++) { v[i] = expf(v[i] - max); sum += v[i]; }
+    if (sum > 0.0f) for (size_t i = 0; i < n; i++) v[i] /= sum;
+}
+
+/* MoeGateRule::ClampedGlu: larql-compute/src/pipeline/moe.rs:88-92. */
+float lq_clamped_glu(float g, float u, float limit, float alpha) {
+    g = fminf(g, limit);
+    u = clampf(u, -limit, limit);
+    float sig = 1.0f / (1.0f + expf(-(g * alpha)));
+    return (u + 1.0f) * (g * sig);
+}
+
+/* ------------------------------------------- multi-threaded CPU baseline */
+
+typedef struct {
+    int kind; /* 0 q4k, 1 q8_0 */
+    float *out; const float *x; const uint8_t *w; const float *sum_x;
+    size_t rows, blocks_per_row; int tid, nthreads;
+} mt_job;
+
+static void *mt_worker(void *p) {
+    mt_job *j = (mt_job *)p;
+    size_t n_chunks = (j->rows + 31) / 32; /* CHUNK_ROWS = 32 in both kernels */
+    for (size_t c = (size_t)j->tid; c < n_chunks; c += (size_t)j->nthreads) {
+        size_t r0 = c * 32, r1 = r0 + 32 < j->rows ? r0 + 32 : j->rows;
+        if (j->kind == 0) q4k_rows(j->out, j->x, j->w, j->sum_x, r0, r1, j->blocks_per_row);
+        else for (size_t r = r0; r < r1; r++) j->out[r] = q8_0_row_dot(j->w, j->x, r, j->blocks_per_row);
+    }
+    return NULL;
+}
+
+static void mt_run(mt_job proto, int threads) {
+    if (threads < 1) threads = 1;
+    if (threads > 256) threads = 256;
+    pthread_t th[256]; mt_job jobs[256];
+    for (int t = 0; t < threads; t++) { jobs[t] = proto; jobs[t].tid = t; jobs[t].nthreads = threads; }
+    for (int t = 1; t < threads; t++) pthread_create(&th[t], NULL, mt_worker, &jobs[t]);
+    mt_worker(&jobs[0]);
+    for (int t = 1; t < threads; t++) pthread_join(th[t], NULL);
+}
+
+int lq_q4k_matvec_into_mt(float *out, const float *x, const uint8_t *w, size_t w_len,
+                          size_t rows, size_t cols, int threads) {
+    if (!kernel_shape_ok(rows, rows, cols, cols, w_len, 256, 144)) return 1;
+    if (rows == 0 || cols == 0) { for (size_t i = 0; i < rows; i++) out[i] = 0.0f; return 0; }
+    size_t n_blocks = cols / 256;
+    float *sum_x = q4k_sum_x(x, n_blocks);
+    mt_job j = {0, out, x, w, sum_x, rows, n_blocks, 0, 1};
+    mt_run(j, threads);
+    free(sum_x);
+    return 0;
+}
+
+int lq_q8_0_gemv_mt(const uint8_t *blocks, size_t blocks_len, const float *x,
+                    size_t n, size_t k, float *out, int threads) {
+    if (k == 0 || k % 32 != 0) return 1;
+    size_t per_row = k / 32;
+    if (blocks_len != n * per_row * 34) return 1;
+    mt_job j = {1, out, x, blocks, NULL, n, per_row, 0, 1};
+    mt_run(j, threads);
+    return 0;
+}

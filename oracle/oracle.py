@@ -1,0 +1,379 @@
+"""ctypes loader for the CPU checker (oracle/liblarql_oracle.so).
+
+TEST INFRASTRUCTURE ONLY.  Import this from tests/, from the smoke check and
+from the benchmark's cpu_baseline leg; the product package never does.
+
+The wrappers take and return numpy arrays and follow the reference's refusal
+convention: a refused call returns None.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liblarql_oracle.so")
+_REF_PATH = os.path.join(_HERE, "_ref", "libq4dot_ref.so")
+
+
+def build(force: bool = False) -> None:
+    """Compile the checker (and the reference's C kernel when its tree is present)."""
+    if force or not os.path.exists(_LIB_PATH) or os.path.exists("/root/reference"):
+        subprocess.run(["make", "-C", _HERE, "-s", "all"], check=True)
+
+
+def _load():
+    if not os.path.exists(_LIB_PATH):
+        build(force=True)
+    return C.CDLL(_LIB_PATH)
+
+
+_lib = _load()
+_u8p = C.POINTER(C.c_uint8)
+_i8p = C.POINTER(C.c_int8)
+_u16p = C.POINTER(C.c_uint16)
+_u32p = C.POINTER(C.c_uint32)
+_u64p = C.POINTER(C.c_uint64)
+_f32p = C.POINTER(C.c_float)
+_sz = C.c_size_t
+
+
+def _p(a: np.ndarray, t):
+    return a.ctypes.data_as(t)
+
+
+def _f32(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _u8(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.uint8)
+
+
+_lib.lq_f16_to_f32.restype = C.c_float
+_lib.lq_f16_to_f32.argtypes = [C.c_uint16]
+_lib.lq_bf16_to_f32.restype = C.c_float
+_lib.lq_bf16_to_f32.argtypes = [C.c_uint16]
+for _n in ("lq_f32_to_f16_trunc", "lq_f32_to_f16_nearest", "lq_f32_to_f16_flush", "lq_f32_to_bf16"):
+    getattr(_lib, _n).restype = C.c_uint16
+    getattr(_lib, _n).argtypes = [C.c_float]
+_lib.lq_e8m0_to_f32.restype = C.c_float
+_lib.lq_e8m0_to_f32.argtypes = [C.c_uint8]
+_lib.lq_mxfp4_table.restype = C.c_float
+_lib.lq_mxfp4_table.argtypes = [C.c_uint]
+_lib.lq_nearest_mxfp4_code.restype = C.c_uint8
+_lib.lq_nearest_mxfp4_code.argtypes = [C.c_float]
+_lib.lq_clamped_glu.restype = C.c_float
+_lib.lq_clamped_glu.argtypes = [C.c_float] * 4
+_lib.lq_top_k_by_abs.restype = C.c_long
+_lib.lq_top_k_sorted.restype = C.c_long
+_lib.lq_gate_knn_batch_union.restype = C.c_long
+_lib.lq_router_select.restype = _sz
+_lib.lq_moe_top_k.restype = _sz
+
+
+# ---- scalar conversions -------------------------------------------------
+def f16_to_f32(bits: int) -> float:
+    return _lib.lq_f16_to_f32(bits)
+
+
+def f32_to_f16_trunc(v: float) -> int:
+    return _lib.lq_f32_to_f16_trunc(v)
+
+
+def f32_to_f16_nearest(v: float) -> int:
+    return _lib.lq_f32_to_f16_nearest(v)
+
+
+def f32_to_f16_flush(v: float) -> int:
+    return _lib.lq_f32_to_f16_flush(v)
+
+
+def f32_to_bf16(a) -> np.ndarray:
+    a = _f32(a).ravel()
+    out = np.empty(a.size, dtype=np.uint16)
+    _lib.lq_f32_to_bf16_slice(_p(a, _f32p), _sz(a.size), _p(out, _u16p))
+    return out
+
+
+def e8m0_to_f32(b: int) -> float:
+    return _lib.lq_e8m0_to_f32(b)
+
+
+def mxfp4_table(code: int) -> float:
+    return _lib.lq_mxfp4_table(code)
+
+
+def nearest_mxfp4_code(v: float) -> int:
+    return _lib.lq_nearest_mxfp4_code(v)
+
+
+def clamped_glu(g: float, u: float, limit: float = 7.0, alpha: float = 1.702) -> float:
+    return _lib.lq_clamped_glu(g, u, limit, alpha)
+
+
+# ---- Q4_K -----------------------------------------------------------------
+def quantize_q4_k(data) -> np.ndarray:
+    data = _f32(data).ravel()
+    out = np.empty(data.size // 256 * 144, dtype=np.uint8)
+    if _lib.lq_quantize_q4_k(_p(data, _f32p), _sz(data.size), _p(out, _u8p)):
+        raise ValueError("data length must be a multiple of 256")
+    return out
+
+
+def dequantize_q4_k(data, n: int):
+    data = _u8(data).ravel()
+    out = np.empty(n, dtype=np.float32)
+    if _lib.lq_dequantize_q4_k(_p(data, _u8p), _sz(data.size), _sz(n), _p(out, _f32p)):
+        return None
+    return out
+
+
+def q4k_matvec(w, x, rows: int, cols: int, out_len: int | None = None):
+    w, x = _u8(w).ravel(), _f32(x).ravel()
+    out_len = rows if out_len is None else out_len
+    out = np.full(out_len, np.nan, dtype=np.float32)
+    rc = _lib.lq_q4k_matvec_into(_p(out, _f32p), _sz(out_len), _p(x, _f32p), _sz(x.size),
+                                 _p(w, _u8p), _sz(w.size), _sz(rows), _sz(cols))
+    return None if rc else out
+
+
+def q4k_matvec_mt(w, x, rows: int, cols: int, threads: int):
+    w, x = _u8(w).ravel(), _f32(x).ravel()
+    out = np.empty(rows, dtype=np.float32)
+    rc = _lib.lq_q4k_matvec_into_mt(_p(out, _f32p), _p(x, _f32p), _p(w, _u8p), _sz(w.size),
+                                    _sz(rows), _sz(cols), C.c_int(threads))
+    return None if rc else out
+
+
+def q4k_matvec_scalar(w, x, rows: int, hidden: int) -> np.ndarray:
+    w, x = _u8(w).ravel(), _f32(x).ravel()
+    out = np.empty(rows, dtype=np.float32)
+    _lib.lq_q4k_matvec_scalar(_p(out, _f32p), _p(x, _f32p), _p(w, _u8p), _sz(rows), _sz(hidden))
+    return out
+
+
+def q4k_dual_matvec(wa, wb, x, rows: int, cols: int):
+    wa, wb, x = _u8(wa).ravel(), _u8(wb).ravel(), _f32(x).ravel()
+    oa = np.empty(rows, dtype=np.float32)
+    ob = np.empty(rows, dtype=np.float32)
+    rc = _lib.lq_q4k_dual_matvec_into(_p(oa, _f32p), _p(ob, _f32p), _sz(rows), _p(x, _f32p), _sz(x.size),
+                                      _p(wa, _u8p), _sz(wa.size), _p(wb, _u8p), _sz(wb.size),
+                                      _sz(rows), _sz(cols))
+    return None if rc else (oa, ob)
+
+
+def q4k_matmul(w, x, rows: int, hidden: int, seq: int) -> np.ndarray:
+    w, x = _u8(w).ravel(), _f32(x).ravel()
+    out = np.full(seq * rows, np.nan, dtype=np.float32)
+    _lib.lq_q4k_matmul_into(_p(out, _f32p), _p(x, _f32p), _p(w, _u8p), _sz(w.size),
+                            _sz(rows), _sz(hidden), _sz(seq))
+    return out.reshape(seq, rows) if seq and rows else out
+
+
+# ---- Q8_0 -----------------------------------------------------------------
+def quantize_q8_0(data) -> np.ndarray:
+    data = _f32(data).ravel()
+    out = np.empty(data.size // 32 * 34, dtype=np.uint8)
+    if _lib.lq_quantize_q8_0(_p(data, _f32p), _sz(data.size), _p(out, _u8p)):
+        raise ValueError("Q8_0: element count must be multiple of 32")
+    return out
+
+
+def dequantize_q8_0(data, n: int):
+    data = _u8(data).ravel()
+    out = np.empty(n, dtype=np.float32)
+    if _lib.lq_dequantize_q8_0(_p(data, _u8p), _sz(data.size), _sz(n), _p(out, _f32p)):
+        return None
+    return out
+
+
+def q8_0_gemv(blocks, x, n: int, k: int):
+    blocks, x = _u8(blocks).ravel(), _f32(x).ravel()
+    out = np.empty(n, dtype=np.float32)
+    rc = _lib.lq_q8_0_gemv(_p(blocks, _u8p), _sz(blocks.size), _p(x, _f32p), _sz(x.size),
+                           _sz(n), _sz(k), _p(out, _f32p))
+    return None if rc else out
+
+
+def q8_0_gemv_mt(blocks, x, n: int, k: int, threads: int):
+    blocks, x = _u8(blocks).ravel(), _f32(x).ravel()
+    out = np.empty(n, dtype=np.float32)
+    rc = _lib.lq_q8_0_gemv_mt(_p(blocks, _u8p), _sz(blocks.size), _p(x, _f32p),
+                              _sz(n), _sz(k), _p(out, _f32p), C.c_int(threads))
+    return None if rc else out
+
+
+# ---- Q4_0 x Q8 --------------------------------------------------------------
+def quantize_to_q8(x):
+    x = _f32(x).ravel()
+    q8 = np.empty(x.size, dtype=np.int8)
+    scales = np.empty(x.size // 32, dtype=np.float32)
+    _lib.lq_quantize_to_q8(_p(x, _f32p), _sz(x.size), _p(q8, _i8p), _p(scales, _f32p))
+    return q8, scales
+
+
+def quantize_q4_0(data) -> np.ndarray:
+    data = _f32(data).ravel()
+    out = np.empty(data.size // 32 * 18, dtype=np.uint8)
+    if _lib.lq_quantize_q4_0(_p(data, _f32p), _sz(data.size), _p(out, _u8p)):
+        raise ValueError("data length must be a multiple of 32")
+    return out
+
+
+def q4_0_matvec(q4, q8_x, q8_scales, rows: int, hidden: int) -> np.ndarray:
+    q4 = _u8(q4).ravel()
+    q8_x = np.ascontiguousarray(q8_x, dtype=np.int8)
+    q8_scales = _f32(q8_scales)
+    assert hidden % 32 == 0 and q4.size == rows * (hidden // 32) * 18
+    assert q8_x.size == hidden and q8_scales.size == hidden // 32
+    out = np.empty(rows, dtype=np.float32)
+    _lib.lq_q4_0_matvec(_p(q4, _u8p), _p(q8_x, _i8p), _p(q8_scales, _f32p), _p(out, _f32p),
+                        _sz(rows), _sz(hidden))
+    return out
+
+
+def ref_q4_0_matvec(q4, q8_x, q8_scales, rows: int, hidden: int):
+    """The reference's own q4_0_matvec_c, compiled from its tree (None if not built)."""
+    if not os.path.exists(_REF_PATH):
+        return None
+    ref = C.CDLL(_REF_PATH)
+    q4 = _u8(q4).ravel()
+    q8_x = np.ascontiguousarray(q8_x, dtype=np.int8)
+    q8_scales = _f32(q8_scales)
+    out = np.empty(rows, dtype=np.float32)
+    ref.q4_0_matvec_c(_p(q4, _u8p), _p(q8_x, _i8p), _p(q8_scales, _f32p), _p(out, _f32p),
+                      _sz(rows), _sz(hidden))
+    return out
+
+
+def dequantise_q8(q8_x, scales) -> np.ndarray:
+    q8_x = np.ascontiguousarray(q8_x, dtype=np.int8)
+    scales = _f32(scales)
+    out = np.empty(q8_x.size, dtype=np.float32)
+    _lib.lq_dequantise_q8(_p(q8_x, _i8p), _sz(q8_x.size), _p(scales, _f32p), _p(out, _f32p))
+    return out
+
+
+# ---- MXFP4 ------------------------------------------------------------------
+def quantize_mxfp4(values, rows: int, k: int):
+    values = _f32(values).ravel()
+    assert values.size == rows * k
+    packed = np.empty(rows * (k // 32) * 16, dtype=np.uint8)
+    scales = np.empty(rows * (k // 32), dtype=np.uint8)
+    if _lib.lq_quantize_mxfp4(_p(values, _f32p), _sz(rows), _sz(k), _p(packed, _u8p), _p(scales, _u8p)):
+        return None
+    return packed, scales
+
+
+def dequantize_mxfp4_expert(blocks, scales, out_features: int, groups: int):
+    blocks, scales = _u8(blocks).ravel(), _u8(scales).ravel()
+    out = np.empty(out_features * groups * 32, dtype=np.float32)
+    rc = _lib.lq_dequantize_mxfp4_expert(_p(blocks, _u8p), _sz(blocks.size), _p(scales, _u8p),
+                                         _sz(scales.size), _sz(out_features), _sz(groups), _p(out, _f32p))
+    return None if rc else out
+
+
+def mxfp4_gemv(packed, scales, x, n: int, k: int):
+    packed, scales, x = _u8(packed).ravel(), _u8(scales).ravel(), _f32(x).ravel()
+    out = np.empty(n, dtype=np.float32)
+    rc = _lib.lq_mxfp4_gemv(_p(packed, _u8p), _sz(packed.size), _p(scales, _u8p), _sz(scales.size),
+                            _p(x, _f32p), _sz(x.size), _sz(n), _sz(k), _p(out, _f32p))
+    return None if rc else out
+
+
+def mxfp4_gemv_dequant(packed, scales, x, n: int, k: int) -> np.ndarray:
+    packed, scales, x = _u8(packed).ravel(), _u8(scales).ravel(), _f32(x).ravel()
+    out = np.empty(n, dtype=np.float32)
+    _lib.lq_mxfp4_gemv_dequant(_p(packed, _u8p), _p(scales, _u8p), _p(x, _f32p), _sz(n), _sz(k), _p(out, _f32p))
+    return out
+
+
+# ---- dense gemv -------------------------------------------------------------
+def bf16_gemv(w_bits, x, n: int, k: int) -> np.ndarray:
+    w = np.ascontiguousarray(w_bits, dtype=np.uint16).ravel()
+    x = _f32(x).ravel()
+    out = np.empty(n, dtype=np.float32)
+    _lib.lq_bf16_gemv(_p(w, _u16p), _p(x, _f32p), _sz(n), _sz(k), _p(out, _f32p))
+    return out
+
+
+def f16_gemv(w_bits, x, n: int, k: int) -> np.ndarray:
+    w = np.ascontiguousarray(w_bits, dtype=np.uint16).ravel()
+    x = _f32(x).ravel()
+    out = np.empty(n, dtype=np.float32)
+    _lib.lq_f16_gemv(_p(w, _u16p), _p(x, _f32p), _sz(n), _sz(k), _p(out, _f32p))
+    return out
+
+
+def f32_gemv(w, x, n: int, k: int) -> np.ndarray:
+    w, x = _f32(w).ravel(), _f32(x).ravel()
+    out = np.empty(n, dtype=np.float32)
+    _lib.lq_f32_gemv(_p(w, _f32p), _p(x, _f32p), _sz(n), _sz(k), _p(out, _f32p))
+    return out
+
+
+# ---- top-K ------------------------------------------------------------------
+def top_k_by_abs(scores, top_k: int):
+    """[(idx, score)] sorted by |score| descending; raises on NaN like the reference panics."""
+    scores = _f32(scores).ravel()
+    cap = max(1, min(top_k, scores.size))
+    idx = np.empty(cap, dtype=np.uint64)
+    val = np.empty(cap, dtype=np.float32)
+    got = _lib.lq_top_k_by_abs(_p(scores, _f32p), _sz(scores.size), _sz(top_k), _p(idx, _u64p), _p(val, _f32p))
+    if got < 0:
+        raise ValueError("NaN score")
+    return [(int(idx[i]), float(val[i])) for i in range(got)]
+
+
+def top_k_sorted(scores, top_k: int):
+    scores = _f32(scores).ravel()
+    cap = max(1, min(top_k, scores.size))
+    idx = np.empty(cap, dtype=np.uint32)
+    val = np.empty(cap, dtype=np.float32)
+    got = _lib.lq_top_k_sorted(_p(scores, _f32p), _sz(scores.size), _sz(top_k), _p(idx, _u32p), _p(val, _f32p))
+    return [(int(idx[i]), float(val[i])) for i in range(got)]
+
+
+def gate_knn_batch_union(scores_2d, top_k: int):
+    """scores_2d: [n_features, seq]; returns the sorted de-duplicated union of per-position hits."""
+    s = _f32(scores_2d)
+    n, seq = s.shape
+    cap = max(1, seq * min(top_k, n))
+    idx = np.empty(cap, dtype=np.uint64)
+    got = _lib.lq_gate_knn_batch_union(_p(s, _f32p), _sz(n), _sz(seq), _sz(top_k), _p(idx, _u64p), _sz(cap))
+    if got < 0:
+        raise ValueError("NaN score")
+    return [int(v) for v in idx[:got]]
+
+
+# ---- MoE routing ------------------------------------------------------------
+SOFTMAX_THEN_SELECT = 0
+NORMALISED_OVER_SELECTED = 1
+
+
+def router_select(logits, k: int, policy: int = NORMALISED_OVER_SELECTED):
+    logits = _f32(logits).ravel()
+    cap = max(1, min(k, logits.size))
+    e = np.empty(cap, dtype=np.uint64)
+    w = np.empty(cap, dtype=np.float32)
+    got = _lib.lq_router_select(_p(logits, _f32p), _sz(logits.size), _sz(k), C.c_int(policy), _p(e, _u64p), _p(w, _f32p))
+    return [(int(e[i]), float(w[i])) for i in range(got)]
+
+
+def moe_top_k(v, k: int):
+    v = _f32(v).ravel()
+    cap = max(1, min(k, v.size))
+    idx = np.empty(cap, dtype=np.uint64)
+    val = np.empty(cap, dtype=np.float32)
+    got = _lib.lq_moe_top_k(_p(v, _f32p), _sz(v.size), _sz(k), _p(idx, _u64p), _p(val, _f32p))
+    return [int(i) for i in idx[:got]], [float(x) for x in val[:got]]
+
+
+def softmax(v) -> np.ndarray:
+    v = _f32(v).ravel().copy()
+    _lib.lq_softmax(_p(v, _f32p), _sz(v.size))
+    return v
