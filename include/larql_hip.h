@@ -1,0 +1,254 @@
+/*
+ * larql_hip.h — C ABI of the MI355X (gfx950) backend for LARQL's quantised
+ * decode path.
+ *
+ * This is the boundary a `larql-compute` backend crate binds over FFI: each
+ * entry point serves one method of the reference's `ComputeBackend` trait
+ * family (or one free function on the same path) and cites it.  Paths are
+ * relative to the reference checkout, under crates/.
+ *
+ * Conventions
+ *   - Plain C: pointers, sizes, no C++ or framework types.
+ *   - Return value: LARQL_OK (the reference's `Some`), LARQL_UNSUPPORTED or
+ *     LARQL_REFUSED_SHAPE (both map to the reference's `None`: the caller falls
+ *     back; the output is left untouched), or a negative LARQL_E_* device error
+ *     (also `None`; `larql_hip_last_error` gives the text).
+ *   - "Host tier" entry points take host slices, exactly like the trait: the
+ *     weight slice is served from a device-resident copy when it lies inside a
+ *     region registered with larql_hip_register_weight_region, and is uploaded
+ *     for the call otherwise.  Activations and outputs are copied per call.
+ *   - "Device tier" entry points (larql_hip_dev_*) take device pointers that
+ *     are already resident in HBM and enqueue on the context's stream without
+ *     synchronising; weight pointers must be 16-byte aligned.
+ *   - A context is bound to one GPU and one stream.  Calls on one context are
+ *     serialised by an internal lock (the trait requires Send + Sync).
+ */
+#ifndef LARQL_HIP_H
+#define LARQL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct larql_hip_ctx larql_hip_ctx;
+
+enum {
+    LARQL_OK = 0,
+    LARQL_UNSUPPORTED = 1,   /* backend has no kernel for the request -> None */
+    LARQL_REFUSED_SHAPE = 2, /* operands inconsistent (KernelShapeError)  -> None */
+    LARQL_E_DEVICE = -1,     /* HIP runtime error */
+    LARQL_E_NO_DEVICE = -2,  /* no usable GPU (BackendSelectError::NoDevice) */
+    LARQL_E_ARG = -3,        /* null pointer / bad handle */
+    LARQL_E_NAN = -4         /* NaN score in a top-K (the reference panics) */
+};
+
+/* QuantFormat — larql-compute/src/pipeline/quant_format/mod.rs:19-62 (same order). */
+enum {
+    LARQL_FMT_Q4_0 = 0, LARQL_FMT_Q4_K = 1, LARQL_FMT_Q4_KF = 2, LARQL_FMT_Q5_K = 3,
+    LARQL_FMT_Q6_K = 4, LARQL_FMT_Q8_0 = 5, LARQL_FMT_BF16 = 6, LARQL_FMT_F16 = 7,
+    LARQL_FMT_F32 = 8, LARQL_FMT_I2S = 9, LARQL_FMT_MXFP4 = 10,
+    /* ggml's 34-byte Q8_0 block (f16 scale inside the block).  Not the trait's
+     * QuantFormat::Q8_0, which is int8 codes + external f32 scales
+     * (larql-compute/src/cpu/kquant_gemv.rs:1-12). */
+    LARQL_FMT_GGML_Q8_0 = 100
+};
+
+/* Capability — larql-compute/src/backend/capability.rs:22-102 (the ones this
+ * backend answers true for; every other value answers false). */
+enum { LARQL_CAP_F32_GEMV = 0, LARQL_CAP_F16_GEMV = 1, LARQL_CAP_QUANT_MATVEC = 2 };
+
+/* ---- lifecycle / metadata ------------------------------------------------ */
+
+/* Constructor a binary registers in its backend registry
+ * (larql-cli/src/backend_select.rs:26-41; backend/factory.rs:174-192).
+ * LARQL_E_NO_DEVICE when the device does not exist or is not gfx950. */
+int  larql_hip_create(larql_hip_ctx **out, int device);
+void larql_hip_destroy(larql_hip_ctx *ctx);
+/* ComputeBackend::name / device_info — backend/mod.rs:51-57. */
+const char *larql_hip_name(const larql_hip_ctx *ctx);
+const char *larql_hip_device_info(const larql_hip_ctx *ctx);
+/* QuantMatVec::supports_quant — backend/quant_matvec.rs:367-370. */
+int  larql_hip_supports_quant(const larql_hip_ctx *ctx, int format);
+/* ComputeBackend::supports — backend/mod.rs:59-67. */
+int  larql_hip_supports(const larql_hip_ctx *ctx, int capability);
+const char *larql_hip_last_error(const larql_hip_ctx *ctx);
+
+/* ComputeBackend::register_weight_region / seal_weight_regions —
+ * backend/mod.rs:68-89.  The region must never move and must outlive the
+ * context; registering the same base twice is a no-op.  The bytes are
+ * uploaded once and later host-tier calls whose weight slice lies inside the
+ * region use the resident copy. */
+int  larql_hip_register_weight_region(larql_hip_ctx *ctx, const uint8_t *region, size_t len);
+int  larql_hip_seal_weight_regions(larql_hip_ctx *ctx);
+int  larql_hip_clear_weight_regions(larql_hip_ctx *ctx);
+
+/* MatMul::submission_clock — backend/matmul.rs:34-42,216-218.  One host-tier
+ * call is one submission; gpu_nanos is device-event time of its kernels. */
+typedef struct {
+    uint64_t submissions;
+    uint64_t commit_to_done_nanos;
+    uint64_t gpu_nanos;
+} larql_hip_submission_clock;
+int  larql_hip_get_submission_clock(larql_hip_ctx *ctx, larql_hip_submission_clock *out);
+
+/* ---- host tier: quantised matvec (QuantMatVec) ---------------------------- */
+
+/* QuantMatVec::q4k_matvec — backend/quant_matvec.rs:252-260; CPU semantics
+ * cpu/mod.rs:95-114 + q4_common/matvec_f32.rs:37-106: out_len == num_rows,
+ * x_len == hidden, hidden % 256 == 0, w_len >= rows*(hidden/256)*144, else
+ * REFUSED_SHAPE; zero dims write zeros. */
+int larql_hip_q4k_matvec(larql_hip_ctx *ctx, const uint8_t *q4k, size_t q4k_len,
+                         const float *x, size_t x_len, size_t num_rows, size_t hidden,
+                         float *out, size_t out_len);
+/* QuantMatVec::q4k_dual_matvec — quant_matvec.rs:287-296; q4_common/dual.rs:22-167. */
+int larql_hip_q4k_dual_matvec(larql_hip_ctx *ctx, const uint8_t *q4k_a, size_t a_len,
+                              const uint8_t *q4k_b, size_t b_len,
+                              const float *x, size_t x_len, size_t num_rows, size_t hidden,
+                              float *out_a, float *out_b, size_t out_len);
+/* QuantMatVec::q4k_matmul — quant_matvec.rs:324-333; q4_common/matmul.rs:20-139.
+ * out is [seq_len, num_rows] row-major.  Any zero dimension gives an empty
+ * result (OK, nothing written); a bad shape zero-fills out, as the CPU does. */
+int larql_hip_q4k_matmul(larql_hip_ctx *ctx, const uint8_t *q4k, size_t q4k_len,
+                         const float *x, size_t x_len, size_t num_rows, size_t hidden,
+                         size_t seq_len, float *out, size_t out_len);
+/* QuantMatVec::q4k_matvec_topk — quant_matvec.rs:268-277: up to top_k
+ * (row, score) pairs by value descending, non-finite scores skipped
+ * (lm_head/knn.rs:315-386).  *n_out receives the count. */
+int larql_hip_q4k_matvec_topk(larql_hip_ctx *ctx, const uint8_t *q4k, size_t q4k_len,
+                              const float *x, size_t x_len, size_t num_rows, size_t hidden,
+                              size_t top_k, uint32_t *idx_out, float *score_out, size_t *n_out);
+/* QuantMatVec::q4_matvec — quant_matvec.rs:162-171; the CPU path is the C
+ * kernel csrc/q4_dot.c:176-207 behind cpu/ops/q4_matvec.rs:24-86.  Q4_0
+ * weights (18-byte blocks) x a Q8 activation (int8 + one f32 scale per 32).
+ * Bad lengths are REFUSED_SHAPE (the CPU asserts). */
+int larql_hip_q4_matvec(larql_hip_ctx *ctx, const uint8_t *q4, size_t q4_len,
+                        const int8_t *q8_x, size_t q8_len, const float *q8_scales, size_t n_scales,
+                        size_t num_rows, size_t hidden, float *out);
+/* q8_0_gemv (ggml 34-byte blocks) — cpu/kquant_gemv.rs:67-109, reached via
+ * KQuant::gemv (larql-vindex/src/format/vindex3/represent/kquant.rs:285-298):
+ * k > 0, k % 32 == 0, x_len == k and blocks_len == n*(k/32)*34 exactly. */
+int larql_hip_q8_0_gemv(larql_hip_ctx *ctx, const uint8_t *blocks, size_t blocks_len,
+                        const float *x, size_t x_len, size_t n, size_t k, float *out);
+/* QuantMatVec::quant_matvec — quant_matvec.rs:50-98: format dispatch.
+ * Q4_K/Q4_KF -> q4k_matvec, Q4_0 -> quantize_to_q8 + q4_matvec,
+ * everything else UNSUPPORTED (as the trait default answers None). */
+int larql_hip_quant_matvec(larql_hip_ctx *ctx, int format, const uint8_t *weights, size_t w_len,
+                           const float *x, size_t x_len, size_t num_rows, size_t hidden, float *out);
+
+/* ---- host tier: dense / MXFP4 gemv (MatMul) -------------------------------- */
+
+/* MatMul::f32_gemv_force / f16_gemv_force / bf16_gemv_force —
+ * backend/matmul.rs:66-170.  w is [n, k] row-major; w_len in bytes must be
+ * n*k*sizeof(elem), x_len >= k.  The non-force variants apply the peer's flop
+ * threshold (larql-compute-metal/src/trait_impl/matmul.rs:33-88) and answer
+ * UNSUPPORTED below it so the caller keeps its BLAS path. */
+int larql_hip_f32_gemv(larql_hip_ctx *ctx, const float *w, size_t w_len, const float *x, size_t x_len,
+                       size_t n, size_t k, float *out, int force);
+int larql_hip_f16_gemv(larql_hip_ctx *ctx, const uint8_t *w_f16, size_t w_len, const float *x, size_t x_len,
+                       size_t n, size_t k, float *out, int force);
+int larql_hip_bf16_gemv(larql_hip_ctx *ctx, const uint8_t *w_bf16, size_t w_len, const float *x, size_t x_len,
+                        size_t n, size_t k, float *out, int force);
+/* MatMul::mxfp4_gemv — backend/matmul.rs:220-235: k % 32 == 0, x_len >= k,
+ * packed_len >= n*(k/32)*16, scales_len >= n*(k/32). */
+int larql_hip_mxfp4_gemv(larql_hip_ctx *ctx, const uint8_t *packed, size_t packed_len,
+                         const uint8_t *scales, size_t scales_len,
+                         const float *x, size_t x_len, size_t n, size_t k, float *out);
+/* MatMul::mxfp4_gemv_multi — backend/matmul.rs:237-251: several matrices, one
+ * x, one submission; any bad matrix refuses the whole batch; n_mats == 0 is OK.
+ * Results are bit-identical to the single calls. */
+int larql_hip_mxfp4_gemv_multi(larql_hip_ctx *ctx, size_t n_mats,
+                               const uint8_t *const *packed, const size_t *packed_len,
+                               const uint8_t *const *scales, const size_t *scales_len,
+                               const size_t *n, const size_t *k,
+                               const float *x, size_t x_len, float *const *out);
+
+/* ---- host tier: gate-KNN (larql-vindex) ------------------------------------- */
+
+/* VectorIndex::gate_knn / gate_walk / gate_knn_batch —
+ * larql-vindex/src/index/compute/gate_knn/dispatch.rs:22-121,256-304 with
+ * top_k_by_abs (gate_knn/mod.rs:50-108): score `batch` residuals [batch,hidden]
+ * against the gate matrix [n_features, hidden] stored as `format`
+ * (F32, F16, BF16, Q4_K or Q4_0), keep the min(top_k, n_features) largest
+ * |score| per position, sorted by |score| descending (ties: lower index
+ * first).  idx_out/score_out are [batch, top_k]; *n_out receives the number
+ * of hits per position.  LARQL_E_NAN on a NaN score. */
+int larql_hip_gate_knn(larql_hip_ctx *ctx, int format, const uint8_t *gate, size_t gate_len,
+                       const float *x, size_t batch, size_t n_features, size_t hidden, size_t top_k,
+                       uint32_t *idx_out, float *score_out, size_t *n_out);
+/* gate_scores_batch_backend — gate_knn/scores_batch.rs:30-57: the full score
+ * matrix [batch, n_features]. */
+int larql_hip_gate_scores(larql_hip_ctx *ctx, int format, const uint8_t *gate, size_t gate_len,
+                          const float *x, size_t batch, size_t n_features, size_t hidden, float *scores_out);
+
+/* ---- device tier ------------------------------------------------------------ */
+/* Memory and ordering helpers for callers that keep operands in HBM. */
+int larql_hip_malloc(larql_hip_ctx *ctx, void **dptr, size_t bytes);
+int larql_hip_free(larql_hip_ctx *ctx, void *dptr);
+int larql_hip_memcpy_h2d(larql_hip_ctx *ctx, void *dst, const void *src, size_t bytes);
+int larql_hip_memcpy_d2h(larql_hip_ctx *ctx, void *dst, const void *src, size_t bytes);
+int larql_hip_memset(larql_hip_ctx *ctx, void *dst, int value, size_t bytes);
+int larql_hip_synchronize(larql_hip_ctx *ctx);
+/* Device-event timing on the context's stream (the stream the kernels run on). */
+int larql_hip_event_create(larql_hip_ctx *ctx, void **event);
+int larql_hip_event_record(larql_hip_ctx *ctx, void *event);
+int larql_hip_event_elapsed_ms(larql_hip_ctx *ctx, void *start, void *stop, float *ms);
+int larql_hip_event_destroy(larql_hip_ctx *ctx, void *event);
+
+/* One matvec on resident operands: out[rows] = W[rows,k] . x[k].
+ * format: Q4_K, GGML_Q8_0, MXFP4 (aux = e8m0 scale stream), BF16, F16, F32,
+ * Q4_0 (x is then the f32 activation, quantised to Q8 on the device as
+ * QuantMatVec::quant_matvec does for Q4_0).  Same arithmetic as the host
+ * tier. */
+int larql_hip_dev_matvec(larql_hip_ctx *ctx, int format, const void *w, const void *aux,
+                         const float *x, size_t rows, size_t k, float *out);
+
+/* Several matvecs in ONE launch ("one submission", as MatMul::*_gemv_multi
+ * and Metal's decode command buffer do, backend/matmul.rs:151-194): each job
+ * has its own format, operands and shape.  Jobs must be independent of one
+ * another (no job reads another job's out). */
+typedef struct {
+    int32_t format;
+    int32_t reserved;
+    const void *w;
+    const void *aux;     /* MXFP4 scale stream, else NULL */
+    const float *x;
+    float *out;
+    uint64_t rows;
+    uint64_t k;
+} larql_hip_matvec_job;
+int larql_hip_dev_matvec_batch(larql_hip_ctx *ctx, const larql_hip_matvec_job *jobs, size_t n_jobs);
+
+/* Scores + top-K by |score| on resident operands (see larql_hip_gate_knn).
+ * scores_scratch: [batch, n_features] f32 device buffer (also the full score
+ * matrix on return); idx_out/score_out: [batch, top_k] device buffers. */
+int larql_hip_dev_gate_knn(larql_hip_ctx *ctx, int format, const void *gate,
+                           const float *x, size_t batch, size_t n_features, size_t hidden,
+                           size_t top_k, float *scores_scratch, uint32_t *idx_out, float *score_out);
+
+/* ---- device tier: encoders (bit-exact with the reference's host encoders) --- */
+/* quantize_q4_k — larql-compute/src/cpu/ops/q4_common/quantize.rs:89-189. */
+int larql_hip_dev_quantize_q4_k(larql_hip_ctx *ctx, const float *src, size_t n, uint8_t *dst);
+/* quantize_q8_0 — larql-models/src/quant/ggml/quantize.rs:50-77. */
+int larql_hip_dev_quantize_q8_0(larql_hip_ctx *ctx, const float *src, size_t n, uint8_t *dst);
+/* quantize_mxfp4 — larql-vindex/src/format/vindex3/opplan/exec/weights/load.rs:410-476. */
+int larql_hip_dev_quantize_mxfp4(larql_hip_ctx *ctx, const float *src, size_t rows, size_t k,
+                                 uint8_t *packed, uint8_t *scales);
+/* f32_to_bf16 (truncation) — larql-models/src/quant/half.rs:107-109. */
+int larql_hip_dev_f32_to_bf16(larql_hip_ctx *ctx, const float *src, size_t n, uint16_t *dst);
+/* quantize_q4_0 / quantize_to_q8 — q4_common/quantize.rs:6-69. */
+int larql_hip_dev_quantize_q4_0(larql_hip_ctx *ctx, const float *src, size_t n, uint8_t *dst);
+int larql_hip_dev_quantize_to_q8(larql_hip_ctx *ctx, const float *src, size_t n, int8_t *q8, float *scales);
+/* Synthetic N(0, sigma) data for benchmarks: element i of stream `seed` is a
+ * fixed function of (seed, i) (sum of twelve 21-bit uniforms from a
+ * splitmix64 counter stream: exact integer arithmetic, so host and device
+ * agree bit for bit).  No counterpart in the reference, which prescribes no
+ * generator. */
+int larql_hip_dev_fill_normal(larql_hip_ctx *ctx, float *dst, size_t n, uint64_t seed, float sigma);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

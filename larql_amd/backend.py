@@ -1,0 +1,326 @@
+"""HipBackend — the host-side mirror of the reference's ComputeBackend trait
+family for the quantised decode path, over the C ABI.
+
+Method names, argument meaning and the None-means-"cannot serve, fall back"
+convention follow larql-compute/src/backend/{mod,quant_matvec,matmul}.rs; the
+gate-KNN methods follow larql-vindex/src/index/compute/gate_knn/dispatch.rs.
+Arrays are numpy; weights are uint8 byte streams exactly as the reference
+stores them.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import List, Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import _lib as L
+
+lib = L.lib
+
+
+def _ptr(a: Optional[np.ndarray]):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _u8(a) -> np.ndarray:
+    a = np.asarray(a)
+    if a.dtype != np.uint8:
+        a = a.view(np.uint8) if a.flags.c_contiguous else np.ascontiguousarray(a).view(np.uint8)
+    return np.ascontiguousarray(a).reshape(-1)
+
+
+def _f32(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.float32).reshape(-1)
+
+
+class DeviceError(RuntimeError):
+    pass
+
+
+class NanScoreError(ValueError):
+    """A NaN gate score: the reference's top_k_by_abs panics on it."""
+
+
+class HipBackend:
+    """One GPU, one stream.  `HipBackend()` raises if there is no gfx950 device
+    (the reference's BackendSelectError::NoDevice: never a silent CPU fallback)."""
+
+    def __init__(self, device: int = 0):
+        h = C.c_void_p()
+        rc = lib.larql_hip_create(C.byref(h), device)
+        if rc != L.OK:
+            raise RuntimeError(f"no usable gfx950 device {device} (larql_hip_create -> {rc})")
+        self._h = h
+        self._regions: list = []  # keeps registered host arrays alive, as the contract demands
+
+    def close(self) -> None:
+        if getattr(self, "_h", None):
+            lib.larql_hip_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()
+
+    # -- error mapping ---------------------------------------------------------
+    def _some(self, rc: int) -> bool:
+        """True for Some, False for None (refusal); raises on device errors."""
+        if rc == L.OK:
+            return True
+        if rc in (L.UNSUPPORTED, L.REFUSED_SHAPE):
+            return False
+        if rc == L.E_NAN:
+            raise NanScoreError(self.last_error())
+        raise DeviceError(f"{rc}: {self.last_error()}")
+
+    def last_error(self) -> str:
+        return lib.larql_hip_last_error(self._h).decode()
+
+    # -- ComputeBackend metadata -------------------------------------------------
+    def name(self) -> str:
+        return lib.larql_hip_name(self._h).decode()
+
+    def device_info(self) -> str:
+        return lib.larql_hip_device_info(self._h).decode()
+
+    def supports_quant(self, fmt: int) -> bool:
+        return bool(lib.larql_hip_supports_quant(self._h, fmt))
+
+    def supports(self, cap: int) -> bool:
+        return bool(lib.larql_hip_supports(self._h, cap))
+
+    def register_weight_region(self, region: np.ndarray) -> None:
+        region = _u8(region)
+        self._regions.append(region)
+        self._some(lib.larql_hip_register_weight_region(self._h, _ptr(region), region.size))
+
+    def seal_weight_regions(self) -> None:
+        self._some(lib.larql_hip_seal_weight_regions(self._h))
+
+    def clear_weight_regions(self) -> None:
+        self._some(lib.larql_hip_clear_weight_regions(self._h))
+        self._regions.clear()
+
+    def submission_clock(self) -> dict:
+        c = L.SubmissionClock()
+        self._some(lib.larql_hip_get_submission_clock(self._h, C.byref(c)))
+        return {"submissions": c.submissions, "commit_to_done_nanos": c.commit_to_done_nanos, "gpu_nanos": c.gpu_nanos}
+
+    # -- QuantMatVec ---------------------------------------------------------------
+    def q4k_matvec(self, q4k_data, x, num_rows: int, hidden: int, out_len: Optional[int] = None):
+        w, x = _u8(q4k_data), _f32(x)
+        out = np.empty(num_rows if out_len is None else out_len, np.float32)
+        ok = self._some(lib.larql_hip_q4k_matvec(self._h, _ptr(w), w.size, _ptr(x), x.size, num_rows, hidden,
+                                                 _ptr(out), out.size))
+        return out if ok else None
+
+    def q4k_dual_matvec(self, q4k_a, q4k_b, x, num_rows: int, hidden: int):
+        a, b, x = _u8(q4k_a), _u8(q4k_b), _f32(x)
+        oa, ob = np.empty(num_rows, np.float32), np.empty(num_rows, np.float32)
+        ok = self._some(lib.larql_hip_q4k_dual_matvec(self._h, _ptr(a), a.size, _ptr(b), b.size, _ptr(x), x.size,
+                                                      num_rows, hidden, _ptr(oa), _ptr(ob), num_rows))
+        return (oa, ob) if ok else None
+
+    def q4k_matmul(self, q4k_data, x, num_rows: int, hidden: int, seq_len: int):
+        w, x = _u8(q4k_data), _f32(x)
+        out = np.empty(seq_len * num_rows, np.float32)
+        ok = self._some(lib.larql_hip_q4k_matmul(self._h, _ptr(w), w.size, _ptr(x), x.size, num_rows, hidden, seq_len,
+                                                 _ptr(out), out.size))
+        return out if ok else None
+
+    def q4k_matvec_topk(self, q4k_data, x, num_rows: int, hidden: int, top_k: int):
+        w, x = _u8(q4k_data), _f32(x)
+        idx = np.empty(max(top_k, 1), np.uint32)
+        val = np.empty(max(top_k, 1), np.float32)
+        n = C.c_size_t(0)
+        ok = self._some(lib.larql_hip_q4k_matvec_topk(self._h, _ptr(w), w.size, _ptr(x), x.size, num_rows, hidden, top_k,
+                                                      _ptr(idx), _ptr(val), C.byref(n)))
+        return [(int(idx[i]), float(val[i])) for i in range(n.value)] if ok else None
+
+    def q4_matvec(self, q4_data, q8_x, q8_scales, num_rows: int, hidden: int):
+        w = _u8(q4_data)
+        q8 = np.ascontiguousarray(q8_x, dtype=np.int8).reshape(-1)
+        sc = _f32(q8_scales)
+        out = np.empty(num_rows, np.float32)
+        ok = self._some(lib.larql_hip_q4_matvec(self._h, _ptr(w), w.size, _ptr(q8), q8.size, _ptr(sc), sc.size, num_rows,
+                                                hidden, _ptr(out)))
+        return out if ok else None
+
+    def q8_0_gemv(self, blocks, x, n: int, k: int):
+        w, x = _u8(blocks), _f32(x)
+        out = np.empty(n, np.float32)
+        ok = self._some(lib.larql_hip_q8_0_gemv(self._h, _ptr(w), w.size, _ptr(x), x.size, n, k, _ptr(out)))
+        return out if ok else None
+
+    def quant_matvec(self, fmt: int, weights, x, num_rows: int, hidden: int):
+        w, x = _u8(weights), _f32(x)
+        out = np.empty(num_rows, np.float32)
+        ok = self._some(lib.larql_hip_quant_matvec(self._h, fmt, _ptr(w), w.size, _ptr(x), x.size, num_rows, hidden, _ptr(out)))
+        return out if ok else None
+
+    # -- MatMul ------------------------------------------------------------------------
+    def _dense(self, fn, w, x, n, k, force):
+        w, x = _u8(w), _f32(x)
+        out = np.empty(n, np.float32)
+        ok = self._some(fn(self._h, _ptr(w), w.size, _ptr(x), x.size, n, k, _ptr(out), int(force)))
+        return out if ok else None
+
+    def f32_gemv(self, w, x):
+        w = np.ascontiguousarray(w, dtype=np.float32)
+        return self._dense(lib.larql_hip_f32_gemv, w, x, w.shape[0], w.shape[1], False)
+
+    def f32_gemv_force(self, w, x):
+        w = np.ascontiguousarray(w, dtype=np.float32)
+        return self._dense(lib.larql_hip_f32_gemv, w, x, w.shape[0], w.shape[1], True)
+
+    def f16_gemv(self, w_f16, x, n: int, k: int):
+        return self._dense(lib.larql_hip_f16_gemv, w_f16, x, n, k, False)
+
+    def f16_gemv_force(self, w_f16, x, n: int, k: int):
+        return self._dense(lib.larql_hip_f16_gemv, w_f16, x, n, k, True)
+
+    def bf16_gemv(self, w_bf16, x, n: int, k: int):
+        return self._dense(lib.larql_hip_bf16_gemv, w_bf16, x, n, k, False)
+
+    def bf16_gemv_force(self, w_bf16, x, n: int, k: int):
+        return self._dense(lib.larql_hip_bf16_gemv, w_bf16, x, n, k, True)
+
+    def bf16_gemv_multi(self, weights: Sequence[Tuple[np.ndarray, int, int]], x):
+        outs = [self.bf16_gemv_force(w, x, n, k) for (w, n, k) in weights]
+        return None if any(o is None for o in outs) else outs
+
+    def f16_gemv_multi(self, weights: Sequence[Tuple[np.ndarray, int, int]], x):
+        outs = [self.f16_gemv_force(w, x, n, k) for (w, n, k) in weights]
+        return None if any(o is None for o in outs) else outs
+
+    def mxfp4_gemv(self, packed, scales, x, n: int, k: int):
+        p, s, x = _u8(packed), _u8(scales), _f32(x)
+        out = np.empty(n, np.float32)
+        ok = self._some(lib.larql_hip_mxfp4_gemv(self._h, _ptr(p), p.size, _ptr(s), s.size, _ptr(x), x.size, n, k, _ptr(out)))
+        return out if ok else None
+
+    def mxfp4_gemv_multi(self, weights: Sequence[Tuple[np.ndarray, np.ndarray, int, int]], x):
+        m = len(weights)
+        x = _f32(x)
+        ps = [_u8(w[0]) for w in weights]
+        ss = [_u8(w[1]) for w in weights]
+        outs = [np.empty(w[2], np.float32) for w in weights]
+        VP, SZ = C.c_void_p * max(m, 1), C.c_size_t * max(m, 1)
+        rc = lib.larql_hip_mxfp4_gemv_multi(
+            self._h, m, VP(*[p.ctypes.data for p in ps]), SZ(*[p.size for p in ps]),
+            VP(*[s.ctypes.data for s in ss]), SZ(*[s.size for s in ss]),
+            SZ(*[w[2] for w in weights]), SZ(*[w[3] for w in weights]), _ptr(x), x.size,
+            VP(*[o.ctypes.data for o in outs]))
+        return outs if self._some(rc) else None
+
+    # -- gate-KNN (VectorIndex) ------------------------------------------------------------
+    def gate_knn_batch_hits(self, fmt: int, gate, x, n_features: int, hidden: int, top_k: int):
+        """Per-position hits: list over positions of [(feature, score)] by |score| descending."""
+        g = _u8(gate)
+        x2 = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, hidden) if hidden else np.zeros((0, 0), np.float32)
+        batch = x2.shape[0]
+        k = max(top_k, 1)
+        idx = np.empty((max(batch, 1), k), np.uint32)
+        val = np.empty((max(batch, 1), k), np.float32)
+        n_out = (C.c_size_t * max(batch, 1))()
+        ok = self._some(lib.larql_hip_gate_knn(self._h, fmt, _ptr(g), g.size, _ptr(x2), batch, n_features, hidden, top_k,
+                                               _ptr(idx), _ptr(val), n_out))
+        if not ok:
+            return None
+        return [[(int(idx[b, i]), float(val[b, i])) for i in range(n_out[b])] for b in range(batch)]
+
+    def gate_knn(self, fmt: int, gate, residual, n_features: int, hidden: int, top_k: int):
+        """VectorIndex::gate_knn / gate_walk: [(feature, score)] by |score| descending."""
+        hits = self.gate_knn_batch_hits(fmt, gate, np.asarray(residual, np.float32).reshape(1, -1), n_features, hidden, top_k)
+        return None if hits is None else hits[0]
+
+    def gate_knn_batch(self, fmt: int, gate, x, n_features: int, hidden: int, top_k: int) -> Optional[List[int]]:
+        """VectorIndex::gate_knn_batch: sorted, de-duplicated union of the per-position hits."""
+        hits = self.gate_knn_batch_hits(fmt, gate, x, n_features, hidden, top_k)
+        if hits is None:
+            return None
+        return sorted({i for pos in hits for (i, _) in pos})
+
+    def gate_scores_batch(self, fmt: int, gate, x, n_features: int, hidden: int):
+        g = _u8(gate)
+        x2 = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, hidden)
+        out = np.empty((x2.shape[0], n_features), np.float32)
+        ok = self._some(lib.larql_hip_gate_scores(self._h, fmt, _ptr(g), g.size, _ptr(x2), x2.shape[0], n_features, hidden,
+                                                  _ptr(out)))
+        return out if ok else None
+
+    # -- device tier -------------------------------------------------------------------------------
+    def malloc(self, nbytes: int) -> int:
+        p = C.c_void_p()
+        self._some(lib.larql_hip_malloc(self._h, C.byref(p), nbytes))
+        return p.value
+
+    def free(self, dptr: int) -> None:
+        self._some(lib.larql_hip_free(self._h, dptr))
+
+    def h2d(self, dptr: int, a: np.ndarray) -> None:
+        a = np.ascontiguousarray(a)
+        self._some(lib.larql_hip_memcpy_h2d(self._h, dptr, _ptr(a), a.nbytes))
+
+    def d2h(self, dptr: int, shape, dtype) -> np.ndarray:
+        out = np.empty(shape, dtype)
+        self._some(lib.larql_hip_memcpy_d2h(self._h, _ptr(out), dptr, out.nbytes))
+        return out
+
+    def to_device(self, a: np.ndarray) -> int:
+        a = np.ascontiguousarray(a)
+        p = self.malloc(max(a.nbytes, 1) + 64)
+        if a.nbytes:
+            self.h2d(p, a)
+        return p
+
+    def synchronize(self) -> None:
+        self._some(lib.larql_hip_synchronize(self._h))
+
+    def event(self) -> int:
+        e = C.c_void_p()
+        self._some(lib.larql_hip_event_create(self._h, C.byref(e)))
+        return e.value
+
+    def record(self, ev: int) -> None:
+        self._some(lib.larql_hip_event_record(self._h, ev))
+
+    def elapsed_ms(self, a: int, b: int) -> float:
+        ms = C.c_float()
+        self._some(lib.larql_hip_event_elapsed_ms(self._h, a, b, C.byref(ms)))
+        return ms.value
+
+    def dev_matvec(self, fmt: int, w: int, aux: Optional[int], x: int, rows: int, k: int, out: int) -> bool:
+        return self._some(lib.larql_hip_dev_matvec(self._h, fmt, w, aux, x, rows, k, out))
+
+    def dev_matvec_batch(self, jobs: Sequence[tuple]) -> bool:
+        """jobs: (fmt, w, aux, x, out, rows, k) with device pointers."""
+        arr = (L.MatvecJob * max(len(jobs), 1))()
+        for i, (fmt, w, aux, x, out, rows, k) in enumerate(jobs):
+            arr[i] = L.MatvecJob(fmt, 0, w, aux, x, out, rows, k)
+        return self._some(lib.larql_hip_dev_matvec_batch(self._h, arr, len(jobs)))
+
+    def dev_gate_knn(self, fmt: int, gate: int, x: int, batch: int, n: int, hidden: int, top_k: int, scores: int, idx: int,
+                     val: int) -> bool:
+        return self._some(lib.larql_hip_dev_gate_knn(self._h, fmt, gate, x, batch, n, hidden, top_k, scores, idx, val))
+
+    def dev_quantize_q4_k(self, src: int, n: int, dst: int) -> bool:
+        return self._some(lib.larql_hip_dev_quantize_q4_k(self._h, src, n, dst))
+
+    def dev_quantize_q8_0(self, src: int, n: int, dst: int) -> bool:
+        return self._some(lib.larql_hip_dev_quantize_q8_0(self._h, src, n, dst))
+
+    def dev_quantize_mxfp4(self, src: int, rows: int, k: int, packed: int, scales: int) -> bool:
+        return self._some(lib.larql_hip_dev_quantize_mxfp4(self._h, src, rows, k, packed, scales))
+
+    def dev_f32_to_bf16(self, src: int, n: int, dst: int) -> bool:
+        return self._some(lib.larql_hip_dev_f32_to_bf16(self._h, src, n, dst))
+
+    def dev_quantize_q4_0(self, src: int, n: int, dst: int) -> bool:
+        return self._some(lib.larql_hip_dev_quantize_q4_0(self._h, src, n, dst))
+
+    def dev_quantize_to_q8(self, src: int, n: int, q8: int, scales: int) -> bool:
+        return self._some(lib.larql_hip_dev_quantize_to_q8(self._h, src, n, q8, scales))
+
+    def dev_fill_normal(self, dst: int, n: int, seed: int, sigma: float) -> bool:
+        return self._some(lib.larql_hip_dev_fill_normal(self._h, dst, n, seed, sigma))

@@ -1,0 +1,885 @@
+// api.hip — the C ABI of include/larql_hip.h: context, weight residency, the
+// host tier (trait-shaped calls on host slices) and the device tier.
+//
+// There is no CPU compute path in this library: every entry point either runs
+// the HIP kernels or refuses.
+#include <hip/hip_runtime.h>
+
+#include <chrono>
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/larql_hip.h"
+#include "kernels.h"
+
+using namespace larql;
+
+namespace {
+
+struct DevBuf {
+    void *p = nullptr;
+    size_t cap = 0;
+};
+
+struct Region {
+    const uint8_t *host;
+    size_t len;
+    uint8_t *dev;
+};
+
+}  // namespace
+
+struct larql_hip_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    int cu_count = 0;
+    int wgs_per_cu = 2;
+    size_t flop_threshold = 500000000;  // the Metal peer's default (calibration.rs:12)
+    std::mutex mu;
+    std::string name, info, last_error;
+    std::vector<Region> regions;
+    DevBuf w[4], aux[4], x, out, table, misc, scores, q8, q8s;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    uint8_t *log2_up = nullptr;  // 256-entry table for the MXFP4 encoder
+    int *nan_flag = nullptr;
+    larql_hip_submission_clock clock = {0, 0, 0};
+};
+
+namespace {
+
+int fail(larql_hip_ctx *c, int code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    if (c) c->last_error = buf;
+    return code;
+}
+
+#define HIPCHECK(ctx, expr)                                                                         \
+    do {                                                                                            \
+        hipError_t _e = (expr);                                                                     \
+        if (_e != hipSuccess) return fail(ctx, LARQL_E_DEVICE, "%s: %s", #expr, hipGetErrorString(_e)); \
+    } while (0)
+
+int ensure(larql_hip_ctx *c, DevBuf &b, size_t bytes) {
+    if (bytes <= b.cap) return LARQL_OK;
+    if (b.p) HIPCHECK(c, hipFree(b.p));
+    b.p = nullptr; b.cap = 0;
+    size_t cap = bytes < 4096 ? 4096 : bytes;
+    HIPCHECK(c, hipMalloc(&b.p, cap));
+    b.cap = cap;
+    return LARQL_OK;
+}
+
+// A weight slice is served from a registered region when it lies inside one at
+// a 16-byte aligned offset; otherwise it is uploaded into `scratch` for the call.
+int resolve_weights(larql_hip_ctx *c, const uint8_t *host, size_t len, DevBuf &scratch, const uint8_t **dev) {
+    for (const Region &r : c->regions) {
+        if (host >= r.host && host + len <= r.host + r.len && ((size_t)(host - r.host) % 16) == 0) {
+            *dev = r.dev + (host - r.host);
+            return LARQL_OK;
+        }
+    }
+    // pad so kernels that read an aligned window past the last block stay in bounds
+    int rc = ensure(c, scratch, len + 64);
+    if (rc) return rc;
+    if (len) HIPCHECK(c, hipMemcpyAsync(scratch.p, host, len, hipMemcpyHostToDevice, c->stream));
+    *dev = (const uint8_t *)scratch.p;
+    return LARQL_OK;
+}
+
+int upload(larql_hip_ctx *c, DevBuf &b, const void *host, size_t bytes) {
+    int rc = ensure(c, b, bytes + 64);
+    if (rc) return rc;
+    if (bytes) HIPCHECK(c, hipMemcpyAsync(b.p, host, bytes, hipMemcpyHostToDevice, c->stream));
+    return LARQL_OK;
+}
+
+struct Submission {
+    larql_hip_ctx *c;
+    std::chrono::steady_clock::time_point t0;
+    explicit Submission(larql_hip_ctx *ctx) : c(ctx), t0(std::chrono::steady_clock::now()) {
+        (void)hipEventRecord(c->ev0, c->stream);
+    }
+    int finish() {
+        HIPCHECK(c, hipEventRecord(c->ev1, c->stream));
+        HIPCHECK(c, hipStreamSynchronize(c->stream));
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, c->ev0, c->ev1) == hipSuccess) c->clock.gpu_nanos += (uint64_t)(ms * 1e6);
+        c->clock.submissions += 1;
+        c->clock.commit_to_done_nanos += (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(
+                                             std::chrono::steady_clock::now() - t0).count();
+        return LARQL_OK;
+    }
+};
+
+int kind_of_format(int format) {
+    switch (format) {
+        case LARQL_FMT_Q4_K: case LARQL_FMT_Q4_KF: return KIND_Q4K;
+        case LARQL_FMT_GGML_Q8_0: return KIND_Q8_0;
+        case LARQL_FMT_MXFP4: return KIND_MXFP4;
+        case LARQL_FMT_Q4_0: return KIND_Q4_0;
+        case LARQL_FMT_BF16: return KIND_BF16;
+        case LARQL_FMT_F16: return KIND_F16;
+        case LARQL_FMT_F32: return KIND_F32;
+        default: return -1;
+    }
+}
+
+// Enqueue one launch covering `jobs` (device operands).  Jobs with no rows are dropped.
+int enqueue_jobs(larql_hip_ctx *c, std::vector<GemvJob> &jobs) {
+    std::vector<GemvJob> live;
+    for (const GemvJob &j : jobs)
+        if (j.rows > 0) live.push_back(j);
+    if (live.empty()) return LARQL_OK;
+    for (const GemvJob &j : live) {
+        if (((uintptr_t)j.w & 15) || ((uintptr_t)j.x & 15))
+            return fail(c, LARQL_REFUSED_SHAPE, "matvec: weight and activation pointers must be 16-byte aligned");
+        if ((j.kind == KIND_Q8_0 || j.kind == KIND_Q4_0) && (j.k % 64) != 0)
+            return fail(c, LARQL_UNSUPPORTED, "matvec: this block format needs k %% 64 == 0 on this backend (k=%llu)",
+                        (unsigned long long)j.k);
+    }
+    const uint32_t threads = gemv_pick_threads(live.data(), live.size());
+    if (threads == 0) return fail(c, LARQL_UNSUPPORTED, "matvec: row length not supported by the gfx950 kernels");
+    uint64_t total = 0;
+    for (GemvJob &j : live) {
+        if (!gemv_job_geometry(j, threads)) return fail(c, LARQL_UNSUPPORTED, "matvec: unsupported geometry");
+        if (total + j.n_pass > 0x7FFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "matvec: launch too large");
+        j.pass_begin = (uint32_t)total;
+        total += j.n_pass;
+    }
+    GemvLaunch L;
+    memset(&L, 0, sizeof L);
+    L.total_passes = total;
+    L.n_jobs = (uint32_t)live.size();
+    if (live.size() <= (size_t)kInlineJobs) {
+        for (size_t i = 0; i < live.size(); i++) L.inl[i] = live[i];
+        L.table = nullptr;
+    } else {
+        int rc = ensure(c, c->table, live.size() * sizeof(GemvJob));
+        if (rc) return rc;
+        HIPCHECK(c, hipMemcpyAsync(c->table.p, live.data(), live.size() * sizeof(GemvJob), hipMemcpyHostToDevice, c->stream));
+        // the host vector dies with this call: make sure the copy has consumed it
+        HIPCHECK(c, hipStreamSynchronize(c->stream));
+        L.table = (const GemvJob *)c->table.p;
+    }
+    uint64_t grid = (uint64_t)c->cu_count * (uint64_t)c->wgs_per_cu;
+    if (grid > total) grid = total;
+    const size_t lds = gemv_lds_bytes(live.data(), live.size());
+    HIPCHECK(c, gemv_launch(c->stream, L, threads, (uint32_t)grid, lds));
+    return LARQL_OK;
+}
+
+GemvJob make_job(int kind, const void *w, const void *aux, const void *x, float *out, uint64_t rows, uint64_t k) {
+    GemvJob j;
+    memset(&j, 0, sizeof j);
+    j.kind = kind; j.w = (const uint8_t *)w; j.aux = (const uint8_t *)aux; j.x = (const float *)x; j.out = out;
+    j.rows = rows; j.k = k;
+    return j;
+}
+
+size_t dense_elem_bytes(int kind) { return kind == KIND_F32 ? 4 : 2; }
+
+}  // namespace
+
+extern "C" {
+
+// ---- lifecycle ----------------------------------------------------------------
+int larql_hip_create(larql_hip_ctx **out, int device) {
+    if (!out) return LARQL_E_ARG;
+    *out = nullptr;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0 || device < 0 || device >= n) return LARQL_E_NO_DEVICE;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) != hipSuccess) return LARQL_E_NO_DEVICE;
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return LARQL_E_NO_DEVICE;  // code objects are gfx950 only
+    if (hipSetDevice(device) != hipSuccess) return LARQL_E_NO_DEVICE;
+    larql_hip_ctx *c = new larql_hip_ctx();
+    c->device = device;
+    c->cu_count = prop.multiProcessorCount;
+    if (const char *e = getenv("LARQL_HIP_WGS_PER_CU")) { int v = atoi(e); if (v >= 1 && v <= 16) c->wgs_per_cu = v; }
+    char buf[256];
+    snprintf(buf, sizeof buf, "hip (gfx950 matvec + gate-KNN kernels)");
+    c->name = buf;
+    snprintf(buf, sizeof buf, "%s, %d CUs, %.0f GiB HBM, %s", prop.name, prop.multiProcessorCount,
+             (double)prop.totalGlobalMem / (1024.0 * 1024.0 * 1024.0), prop.gcnArchName);
+    c->info = buf;
+    if (hipStreamCreate(&c->stream) != hipSuccess || hipEventCreate(&c->ev0) != hipSuccess ||
+        hipEventCreate(&c->ev1) != hipSuccess || hipMalloc((void **)&c->log2_up, 256) != hipSuccess ||
+        hipMalloc((void **)&c->nan_flag, sizeof(int)) != hipSuccess) {
+        larql_hip_destroy(c);
+        return LARQL_E_DEVICE;
+    }
+    // For each f32 exponent E: how many of the largest mantissas have a host
+    // log2f that rounds up to the next integer (the MXFP4 encoder's floor(log2f)).
+    uint8_t up[256];
+    for (int E = 0; E < 256; E++) {
+        up[E] = 0;
+        if (E == 0 || E == 255) continue;
+        for (uint32_t kk = 1; kk <= 64; kk++) {
+            uint32_t bits = ((uint32_t)E << 23) | (0x800000u - kk);
+            float v; memcpy(&v, &bits, 4);
+            if (floorf(log2f(v)) == (float)(E - 127 + 1)) up[E] = (uint8_t)kk; else break;
+        }
+    }
+    if (hipMemcpy(c->log2_up, up, 256, hipMemcpyHostToDevice) != hipSuccess ||
+        hipMemset(c->nan_flag, 0, sizeof(int)) != hipSuccess) {
+        larql_hip_destroy(c);
+        return LARQL_E_DEVICE;
+    }
+    *out = c;
+    return LARQL_OK;
+}
+
+void larql_hip_destroy(larql_hip_ctx *c) {
+    if (!c) return;
+    (void)hipSetDevice(c->device);
+    if (c->stream) (void)hipStreamSynchronize(c->stream);
+    for (Region &r : c->regions) (void)hipFree(r.dev);
+    DevBuf *bufs[] = {&c->w[0], &c->w[1], &c->w[2], &c->w[3], &c->aux[0], &c->aux[1], &c->aux[2], &c->aux[3],
+                      &c->x, &c->out, &c->table, &c->misc, &c->scores, &c->q8, &c->q8s};
+    for (DevBuf *b : bufs) if (b->p) (void)hipFree(b->p);
+    if (c->log2_up) (void)hipFree(c->log2_up);
+    if (c->nan_flag) (void)hipFree(c->nan_flag);
+    if (c->ev0) (void)hipEventDestroy(c->ev0);
+    if (c->ev1) (void)hipEventDestroy(c->ev1);
+    if (c->stream) (void)hipStreamDestroy(c->stream);
+    delete c;
+}
+
+const char *larql_hip_name(const larql_hip_ctx *c) { return c ? c->name.c_str() : ""; }
+const char *larql_hip_device_info(const larql_hip_ctx *c) { return c ? c->info.c_str() : ""; }
+const char *larql_hip_last_error(const larql_hip_ctx *c) { return c ? c->last_error.c_str() : "null context"; }
+
+int larql_hip_supports_quant(const larql_hip_ctx *, int format) {
+    switch (format) {
+        case LARQL_FMT_Q4_0: case LARQL_FMT_Q4_K: case LARQL_FMT_Q4_KF: case LARQL_FMT_MXFP4:
+        case LARQL_FMT_GGML_Q8_0: case LARQL_FMT_BF16: case LARQL_FMT_F16: case LARQL_FMT_F32:
+            return 1;
+        default:
+            return 0;
+    }
+}
+
+int larql_hip_supports(const larql_hip_ctx *, int cap) {
+    return cap == LARQL_CAP_F32_GEMV || cap == LARQL_CAP_F16_GEMV || cap == LARQL_CAP_QUANT_MATVEC;
+}
+
+int larql_hip_register_weight_region(larql_hip_ctx *c, const uint8_t *region, size_t len) {
+    if (!c || (!region && len)) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    HIPCHECK(c, hipSetDevice(c->device));
+    for (const Region &r : c->regions)
+        if (r.host == region && r.len >= len) return LARQL_OK;  // same base twice: no-op
+    if (len == 0) return LARQL_OK;
+    Region r{region, len, nullptr};
+    HIPCHECK(c, hipMalloc((void **)&r.dev, len + 64));
+    hipError_t e = hipMemcpy(r.dev, region, len, hipMemcpyHostToDevice);
+    if (e != hipSuccess) { (void)hipFree(r.dev); return fail(c, LARQL_E_DEVICE, "register_weight_region: %s", hipGetErrorString(e)); }
+    c->regions.push_back(r);
+    return LARQL_OK;
+}
+
+int larql_hip_seal_weight_regions(larql_hip_ctx *c) {
+    if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, hipDeviceSynchronize());  // uploads are complete; nothing else to declare on this platform
+    return LARQL_OK;
+}
+
+int larql_hip_clear_weight_regions(larql_hip_ctx *c) {
+    if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, hipStreamSynchronize(c->stream));
+    for (Region &r : c->regions) (void)hipFree(r.dev);
+    c->regions.clear();
+    return LARQL_OK;
+}
+
+int larql_hip_get_submission_clock(larql_hip_ctx *c, larql_hip_submission_clock *out) {
+    if (!c || !out) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    *out = c->clock;
+    return LARQL_OK;
+}
+
+// ---- host tier: quantised matvec -------------------------------------------------
+
+static int host_matvec_multi(larql_hip_ctx *c, int kind, size_t n_mats, const uint8_t *const *w, const size_t *w_len,
+                             const uint8_t *const *aux, const size_t *aux_len, const size_t *rows, size_t k,
+                             const float *x, size_t x_bytes, float *const *out) {
+    if (n_mats > 4) return fail(c, LARQL_UNSUPPORTED, "at most 4 matrices per host-tier submission");
+    HIPCHECK(c, hipSetDevice(c->device));
+    std::vector<GemvJob> jobs;
+    int rc = upload(c, c->x, x, x_bytes);
+    if (rc) return rc;
+    size_t out_total = 0;
+    for (size_t i = 0; i < n_mats; i++) out_total += rows[i];
+    rc = ensure(c, c->out, out_total * sizeof(float) + 64);
+    if (rc) return rc;
+    size_t off = 0;
+    for (size_t i = 0; i < n_mats; i++) {
+        const uint8_t *dw = nullptr, *da = nullptr;
+        rc = resolve_weights(c, w[i], w_len[i], c->w[i], &dw);
+        if (rc) return rc;
+        if (aux) { rc = resolve_weights(c, aux[i], aux_len[i], c->aux[i], &da); if (rc) return rc; }
+        jobs.push_back(make_job(kind, dw, da, c->x.p, (float *)c->out.p + off, rows[i], k));
+        off += rows[i];
+    }
+    Submission sub(c);
+    rc = enqueue_jobs(c, jobs);
+    if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
+    off = 0;
+    for (size_t i = 0; i < n_mats; i++) {
+        if (rows[i]) HIPCHECK(c, hipMemcpyAsync(out[i], (float *)c->out.p + off, rows[i] * sizeof(float), hipMemcpyDeviceToHost, c->stream));
+        off += rows[i];
+    }
+    return sub.finish();
+}
+
+static bool q4k_shape_ok(size_t out_len, size_t rows, size_t x_len, size_t cols, size_t w_len) {
+    // KernelShapeError::check, larql-compute/src/cpu/ops/kernel_shape.rs:46-75
+    const size_t needed = (cols / 256) * 144 * rows;
+    return out_len == rows && x_len == cols && cols % 256 == 0 && w_len >= needed;
+}
+
+int larql_hip_q4k_matvec(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, const float *x, size_t x_len,
+                         size_t num_rows, size_t hidden, float *out, size_t out_len) {
+    if (!c || (!out && out_len)) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (!q4k_shape_ok(out_len, num_rows, x_len, hidden, q4k_len))
+        return fail(c, LARQL_REFUSED_SHAPE, "q4k_matvec: refused operands: out.len() %zu for %zu rows, activation length %zu for %zu cols, %zu weight bytes",
+                    out_len, num_rows, x_len, hidden, q4k_len);
+    if (num_rows == 0 || hidden == 0) { for (size_t i = 0; i < out_len; i++) out[i] = 0.0f; return LARQL_OK; }
+    if (!q4k || !x) return LARQL_E_ARG;
+    const size_t need = (hidden / 256) * 144 * num_rows;
+    return host_matvec_multi(c, KIND_Q4K, 1, &q4k, &need, nullptr, nullptr, &num_rows, hidden, x, x_len * 4, &out);
+}
+
+int larql_hip_q4k_dual_matvec(larql_hip_ctx *c, const uint8_t *a, size_t a_len, const uint8_t *b, size_t b_len,
+                              const float *x, size_t x_len, size_t num_rows, size_t hidden, float *out_a, float *out_b,
+                              size_t out_len) {
+    if (!c || ((!out_a || !out_b) && out_len)) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (!q4k_shape_ok(out_len, num_rows, x_len, hidden, a_len) || !q4k_shape_ok(out_len, num_rows, x_len, hidden, b_len))
+        return fail(c, LARQL_REFUSED_SHAPE, "q4k_dual_matvec: refused operands");
+    if (num_rows == 0 || hidden == 0) {
+        for (size_t i = 0; i < out_len; i++) { out_a[i] = 0.0f; out_b[i] = 0.0f; }
+        return LARQL_OK;
+    }
+    if (!a || !b || !x) return LARQL_E_ARG;
+    const size_t need = (hidden / 256) * 144 * num_rows;
+    const uint8_t *w[2] = {a, b};
+    const size_t wl[2] = {need, need}, rows[2] = {num_rows, num_rows};
+    float *outs[2] = {out_a, out_b};
+    return host_matvec_multi(c, KIND_Q4K, 2, w, wl, nullptr, nullptr, rows, hidden, x, x_len * 4, outs);
+}
+
+int larql_hip_q4k_matmul(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, const float *x, size_t x_len,
+                         size_t num_rows, size_t hidden, size_t seq_len, float *out, size_t out_len) {
+    if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (num_rows == 0 || hidden == 0 || seq_len == 0) return LARQL_OK;  // Some(vec![]) on the peer
+    if (out_len != seq_len * num_rows || x_len != seq_len * hidden || !out)
+        return fail(c, LARQL_REFUSED_SHAPE, "q4k_matmul: out/x lengths do not match [seq, rows] / [seq, hidden]");
+    if (hidden % 256 != 0 || q4k_len < num_rows * (hidden / 256) * 144) {
+        for (size_t i = 0; i < out_len; i++) out[i] = 0.0f;  // the CPU kernel zero-fills on a bad shape
+        return LARQL_OK;
+    }
+    if (!q4k || !x) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    const size_t need = num_rows * (hidden / 256) * 144;
+    const uint8_t *dw = nullptr;
+    int rc = resolve_weights(c, q4k, need, c->w[0], &dw);
+    if (rc) return rc;
+    rc = upload(c, c->x, x, x_len * 4);
+    if (rc) return rc;
+    rc = ensure(c, c->out, out_len * 4 + 64);
+    if (rc) return rc;
+    std::vector<GemvJob> jobs;
+    for (size_t s = 0; s < seq_len; s++)
+        jobs.push_back(make_job(KIND_Q4K, dw, nullptr, (const float *)c->x.p + s * hidden, (float *)c->out.p + s * num_rows,
+                                num_rows, hidden));
+    Submission sub(c);
+    rc = enqueue_jobs(c, jobs);
+    if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
+    HIPCHECK(c, hipMemcpyAsync(out, c->out.p, out_len * 4, hipMemcpyDeviceToHost, c->stream));
+    return sub.finish();
+}
+
+static int topk_download(larql_hip_ctx *c, size_t batch, size_t k, uint32_t *idx_out, float *score_out, size_t *n_out,
+                         bool check_nan) {
+    // misc layout: idx [batch*k] u32 | val [batch*k] f32 | count [batch] u32
+    uint32_t *d_idx = (uint32_t *)c->misc.p;
+    float *d_val = (float *)(d_idx + batch * k);
+    uint32_t *d_cnt = (uint32_t *)(d_val + batch * k);
+    std::vector<uint32_t> cnt(batch);
+    int nan = 0;
+    HIPCHECK(c, hipMemcpyAsync(idx_out, d_idx, batch * k * 4, hipMemcpyDeviceToHost, c->stream));
+    HIPCHECK(c, hipMemcpyAsync(score_out, d_val, batch * k * 4, hipMemcpyDeviceToHost, c->stream));
+    HIPCHECK(c, hipMemcpyAsync(cnt.data(), d_cnt, batch * 4, hipMemcpyDeviceToHost, c->stream));
+    HIPCHECK(c, hipMemcpyAsync(&nan, c->nan_flag, sizeof(int), hipMemcpyDeviceToHost, c->stream));
+    HIPCHECK(c, hipStreamSynchronize(c->stream));
+    for (size_t b = 0; b < batch; b++) n_out[b] = cnt[b];
+    if (check_nan && nan) return fail(c, LARQL_E_NAN, "top-K: NaN score");
+    return LARQL_OK;
+}
+
+int larql_hip_q4k_matvec_topk(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, const float *x, size_t x_len,
+                              size_t num_rows, size_t hidden, size_t top_k, uint32_t *idx_out, float *score_out,
+                              size_t *n_out) {
+    if (!c || !n_out) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    // refusals of the GPU peer (larql-compute-metal/src/trait_impl/quant_matvec.rs:210-215), with this
+    // kernel's own capacity (64) in place of K_TOPK
+    if (top_k == 0 || top_k > 64 || num_rows == 0 || x_len != hidden) return fail(c, LARQL_UNSUPPORTED, "q4k_matvec_topk: refused");
+    if (!q4k_shape_ok(num_rows, num_rows, x_len, hidden, q4k_len)) return fail(c, LARQL_REFUSED_SHAPE, "q4k_matvec_topk: refused operands");
+    if (num_rows > 0xFFFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "q4k_matvec_topk: too many rows");
+    if (!q4k || !x || !idx_out || !score_out) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    const size_t need = (hidden / 256) * 144 * num_rows;
+    const uint8_t *dw = nullptr;
+    int rc = resolve_weights(c, q4k, need, c->w[0], &dw);
+    if (rc) return rc;
+    rc = upload(c, c->x, x, x_len * 4);
+    if (rc) return rc;
+    rc = ensure(c, c->scores, num_rows * 4 + 64);
+    if (rc) return rc;
+    rc = ensure(c, c->misc, top_k * 8 + 4 + 64);
+    if (rc) return rc;
+    std::vector<GemvJob> jobs{make_job(KIND_Q4K, dw, nullptr, c->x.p, (float *)c->scores.p, num_rows, hidden)};
+    Submission sub(c);
+    rc = enqueue_jobs(c, jobs);
+    if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
+    uint32_t *d_idx = (uint32_t *)c->misc.p;
+    float *d_val = (float *)(d_idx + top_k);
+    uint32_t *d_cnt = (uint32_t *)(d_val + top_k);
+    HIPCHECK(c, topk_launch(c->stream, (const float *)c->scores.p, 1, (uint32_t)num_rows, (uint32_t)top_k, false, d_idx, d_val,
+                            d_cnt, c->nan_flag, nullptr, 0));
+    rc = sub.finish();
+    if (rc) return rc;
+    return topk_download(c, 1, top_k, idx_out, score_out, n_out, false);
+}
+
+int larql_hip_q4_matvec(larql_hip_ctx *c, const uint8_t *q4, size_t q4_len, const int8_t *q8_x, size_t q8_len,
+                        const float *q8_scales, size_t n_scales, size_t num_rows, size_t hidden, float *out) {
+    if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    // the CPU path asserts these (cpu/ops/q4_matvec.rs:37-62); a refusal stands in for the panic
+    if (hidden % 32 != 0 || q4_len != num_rows * (hidden / 32) * 18 || q8_len != hidden || n_scales != hidden / 32)
+        return fail(c, LARQL_REFUSED_SHAPE, "q4_matvec: refused operands");
+    if (num_rows == 0) return LARQL_OK;
+    if (hidden == 0) { for (size_t i = 0; i < num_rows; i++) out[i] = 0.0f; return LARQL_OK; }
+    if (!q4 || !q8_x || !q8_scales || !out) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    const uint8_t *dw = nullptr;
+    int rc = resolve_weights(c, q4, q4_len, c->w[0], &dw);
+    if (rc) return rc;
+    rc = upload(c, c->q8, q8_x, q8_len);
+    if (rc) return rc;
+    rc = upload(c, c->q8s, q8_scales, n_scales * 4);
+    if (rc) return rc;
+    rc = ensure(c, c->out, num_rows * 4 + 64);
+    if (rc) return rc;
+    std::vector<GemvJob> jobs{make_job(KIND_Q4_0, dw, c->q8s.p, c->q8.p, (float *)c->out.p, num_rows, hidden)};
+    Submission sub(c);
+    rc = enqueue_jobs(c, jobs);
+    if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
+    HIPCHECK(c, hipMemcpyAsync(out, c->out.p, num_rows * 4, hipMemcpyDeviceToHost, c->stream));
+    return sub.finish();
+}
+
+int larql_hip_q8_0_gemv(larql_hip_ctx *c, const uint8_t *blocks, size_t blocks_len, const float *x, size_t x_len, size_t n,
+                        size_t k, float *out) {
+    if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (k == 0 || k % 32 != 0 || x_len != k || blocks_len != n * (k / 32) * 34)
+        return fail(c, LARQL_REFUSED_SHAPE, "q8_0_gemv: geometry does not describe this pack");
+    if (n == 0) return LARQL_OK;
+    if (!blocks || !x || !out) return LARQL_E_ARG;
+    return host_matvec_multi(c, KIND_Q8_0, 1, &blocks, &blocks_len, nullptr, nullptr, &n, k, x, x_len * 4, &out);
+}
+
+int larql_hip_quant_matvec(larql_hip_ctx *c, int format, const uint8_t *weights, size_t w_len, const float *x, size_t x_len,
+                           size_t num_rows, size_t hidden, float *out) {
+    if (!c) return LARQL_E_ARG;
+    switch (format) {
+        case LARQL_FMT_Q4_K: case LARQL_FMT_Q4_KF:
+            return larql_hip_q4k_matvec(c, weights, w_len, x, x_len, num_rows, hidden, out, num_rows);
+        case LARQL_FMT_Q4_0: {
+            std::lock_guard<std::mutex> lk(c->mu);
+            if (hidden % 32 != 0 || w_len != num_rows * (hidden / 32) * 18 || x_len != hidden)
+                return fail(c, LARQL_REFUSED_SHAPE, "quant_matvec(Q4_0): refused operands");
+            if (num_rows == 0) return LARQL_OK;
+            if (hidden == 0) { for (size_t i = 0; i < num_rows; i++) out[i] = 0.0f; return LARQL_OK; }
+            HIPCHECK(c, hipSetDevice(c->device));
+            const uint8_t *dw = nullptr;
+            int rc = resolve_weights(c, weights, w_len, c->w[0], &dw);
+            if (rc) return rc;
+            rc = upload(c, c->x, x, x_len * 4);
+            if (rc) return rc;
+            rc = ensure(c, c->q8, hidden + 64); if (rc) return rc;
+            rc = ensure(c, c->q8s, (hidden / 32) * 4 + 64); if (rc) return rc;
+            rc = ensure(c, c->out, num_rows * 4 + 64); if (rc) return rc;
+            Submission sub(c);
+            HIPCHECK(c, quantize_to_q8_launch(c->stream, (const float *)c->x.p, hidden, (int8_t *)c->q8.p, (float *)c->q8s.p));
+            std::vector<GemvJob> jobs{make_job(KIND_Q4_0, dw, c->q8s.p, c->q8.p, (float *)c->out.p, num_rows, hidden)};
+            rc = enqueue_jobs(c, jobs);
+            if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
+            HIPCHECK(c, hipMemcpyAsync(out, c->out.p, num_rows * 4, hipMemcpyDeviceToHost, c->stream));
+            return sub.finish();
+        }
+        default:
+            // Q6_K, Q5_K, I2S, MXFP4 (external scales), the trait's own Q8_0 layout and the
+            // float formats answer None through this signature (backend/quant_matvec.rs:58-97).
+            return fail(c, LARQL_UNSUPPORTED, "quant_matvec: format %d is not served through this entry", format);
+    }
+}
+
+// ---- host tier: dense / MXFP4 gemv ---------------------------------------------------
+
+static int host_dense_gemv(larql_hip_ctx *c, int kind, const void *w, size_t w_len, const float *x, size_t x_len, size_t n,
+                           size_t k, float *out, int force) {
+    if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    const size_t need = n * k * dense_elem_bytes(kind);
+    if (w_len < need || x_len != k) return fail(c, LARQL_REFUSED_SHAPE, "gemv: refused operands");
+    if (!force && 2 * n * k < c->flop_threshold) return fail(c, LARQL_UNSUPPORTED, "gemv: below the flop threshold");
+    if (n == 0) return LARQL_OK;
+    if (k == 0) { for (size_t i = 0; i < n; i++) out[i] = 0.0f; return LARQL_OK; }
+    if (!w || !x || !out) return LARQL_E_ARG;
+    const uint8_t *wp = (const uint8_t *)w;
+    return host_matvec_multi(c, kind, 1, &wp, &need, nullptr, nullptr, &n, k, x, x_len * 4, &out);
+}
+
+int larql_hip_f32_gemv(larql_hip_ctx *c, const float *w, size_t w_len, const float *x, size_t x_len, size_t n, size_t k,
+                       float *out, int force) {
+    return host_dense_gemv(c, KIND_F32, w, w_len, x, x_len, n, k, out, force);
+}
+int larql_hip_f16_gemv(larql_hip_ctx *c, const uint8_t *w, size_t w_len, const float *x, size_t x_len, size_t n, size_t k,
+                       float *out, int force) {
+    return host_dense_gemv(c, KIND_F16, w, w_len, x, x_len, n, k, out, force);
+}
+int larql_hip_bf16_gemv(larql_hip_ctx *c, const uint8_t *w, size_t w_len, const float *x, size_t x_len, size_t n, size_t k,
+                        float *out, int force) {
+    return host_dense_gemv(c, KIND_BF16, w, w_len, x, x_len, n, k, out, force);
+}
+
+int larql_hip_mxfp4_gemv_multi(larql_hip_ctx *c, size_t n_mats, const uint8_t *const *packed, const size_t *packed_len,
+                               const uint8_t *const *scales, const size_t *scales_len, const size_t *n, const size_t *k,
+                               const float *x, size_t x_len, float *const *out) {
+    if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    for (size_t i = 0; i < n_mats; i++) {
+        // larql-compute-metal/src/trait_impl/matmul.rs:267-275
+        if (k[i] % 32 != 0 || x_len < k[i] || packed_len[i] < n[i] * (k[i] / 32) * 16 || scales_len[i] < n[i] * (k[i] / 32))
+            return fail(c, LARQL_REFUSED_SHAPE, "mxfp4_gemv: matrix %zu refused", i);
+    }
+    if (n_mats == 0) return LARQL_OK;
+    HIPCHECK(c, hipSetDevice(c->device));
+    // matrices may differ in k: submit in groups of up to 4 with equal k (results do not depend on grouping)
+    size_t i = 0;
+    while (i < n_mats) {
+        size_t jn = 1;
+        while (i + jn < n_mats && jn < 4 && k[i + jn] == k[i]) jn++;
+        const uint8_t *w[4], *a[4]; size_t wl[4], al[4], rows[4]; float *outs[4];
+        for (size_t t = 0; t < jn; t++) {
+            w[t] = packed[i + t]; a[t] = scales[i + t]; rows[t] = n[i + t]; outs[t] = out[i + t];
+            wl[t] = n[i + t] * (k[i] / 32) * 16; al[t] = n[i + t] * (k[i] / 32);
+        }
+        if (k[i] == 0) { for (size_t t = 0; t < jn; t++) for (size_t r = 0; r < rows[t]; r++) outs[t][r] = 0.0f; }
+        else {
+            int rc = host_matvec_multi(c, KIND_MXFP4, jn, w, wl, a, al, rows, k[i], x, k[i] * 4, outs);
+            if (rc) return rc;
+        }
+        i += jn;
+    }
+    return LARQL_OK;
+}
+
+int larql_hip_mxfp4_gemv(larql_hip_ctx *c, const uint8_t *packed, size_t packed_len, const uint8_t *scales, size_t scales_len,
+                         const float *x, size_t x_len, size_t n, size_t k, float *out) {
+    // mxfp4_gemv = one-element multi (larql-compute-metal/src/trait_impl/matmul.rs:245-255)
+    return larql_hip_mxfp4_gemv_multi(c, 1, &packed, &packed_len, &scales, &scales_len, &n, &k, x, x_len, &out);
+}
+
+// ---- gate-KNN ----------------------------------------------------------------------------
+
+static size_t format_row_bytes(int kind, size_t k) {
+    switch (kind) {
+        case KIND_Q4K: return (k / 256) * 144;
+        case KIND_Q4_0: return (k / 32) * 18;
+        case KIND_BF16: case KIND_F16: return k * 2;
+        case KIND_F32: return k * 4;
+        default: return 0;
+    }
+}
+
+// scores[batch, n] on the device for resident gate + x (x: [batch, hidden] f32)
+static int dev_gate_scores(larql_hip_ctx *c, int kind, const void *gate, const float *x, size_t batch, size_t n, size_t hidden,
+                           float *scores) {
+    std::vector<GemvJob> jobs;
+    if (kind == KIND_Q4_0) {
+        // gate_knn_q4 (dispatch.rs:354-382): quantize_to_q8 per residual, then the Q4_0 x Q8 kernel
+        int rc = ensure(c, c->q8, batch * hidden + 64); if (rc) return rc;
+        rc = ensure(c, c->q8s, batch * (hidden / 32) * 4 + 64); if (rc) return rc;
+        HIPCHECK(c, quantize_to_q8_launch(c->stream, x, batch * hidden, (int8_t *)c->q8.p, (float *)c->q8s.p));
+        for (size_t b = 0; b < batch; b++)
+            jobs.push_back(make_job(kind, gate, (const float *)c->q8s.p + b * (hidden / 32), (const int8_t *)c->q8.p + b * hidden,
+                                    scores + b * n, n, hidden));
+    } else {
+        for (size_t b = 0; b < batch; b++) jobs.push_back(make_job(kind, gate, nullptr, x + b * hidden, scores + b * n, n, hidden));
+    }
+    return enqueue_jobs(c, jobs);
+}
+
+static int gate_shape_check(larql_hip_ctx *c, int kind, size_t gate_len, size_t n, size_t hidden) {
+    if (kind != KIND_Q4K && kind != KIND_Q4_0 && kind != KIND_BF16 && kind != KIND_F16 && kind != KIND_F32)
+        return fail(c, LARQL_UNSUPPORTED, "gate-KNN: unsupported gate format");
+    if (kind == KIND_Q4K && hidden % 256 != 0) return fail(c, LARQL_REFUSED_SHAPE, "gate-KNN: hidden not a multiple of 256");
+    if (kind == KIND_Q4_0 && hidden % 32 != 0) return fail(c, LARQL_REFUSED_SHAPE, "gate-KNN: hidden not a multiple of 32");
+    if (gate_len < n * format_row_bytes(kind, hidden)) return fail(c, LARQL_REFUSED_SHAPE, "gate-KNN: gate matrix too short");
+    return LARQL_OK;
+}
+
+int larql_hip_gate_scores(larql_hip_ctx *c, int format, const uint8_t *gate, size_t gate_len, const float *x, size_t batch,
+                          size_t n, size_t hidden, float *scores_out) {
+    if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    const int kind = kind_of_format(format);
+    int rc = gate_shape_check(c, kind, gate_len, n, hidden);
+    if (rc) return rc;
+    if (batch == 0 || n == 0) return LARQL_OK;
+    if (hidden == 0) { for (size_t i = 0; i < batch * n; i++) scores_out[i] = 0.0f; return LARQL_OK; }
+    if (!gate || !x || !scores_out) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    const uint8_t *dg = nullptr;
+    rc = resolve_weights(c, gate, n * format_row_bytes(kind, hidden), c->w[0], &dg); if (rc) return rc;
+    rc = upload(c, c->x, x, batch * hidden * 4); if (rc) return rc;
+    rc = ensure(c, c->scores, batch * n * 4 + 64); if (rc) return rc;
+    Submission sub(c);
+    rc = dev_gate_scores(c, kind, dg, (const float *)c->x.p, batch, n, hidden, (float *)c->scores.p);
+    if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
+    HIPCHECK(c, hipMemcpyAsync(scores_out, c->scores.p, batch * n * 4, hipMemcpyDeviceToHost, c->stream));
+    return sub.finish();
+}
+
+int larql_hip_gate_knn(larql_hip_ctx *c, int format, const uint8_t *gate, size_t gate_len, const float *x, size_t batch,
+                       size_t n, size_t hidden, size_t top_k, uint32_t *idx_out, float *score_out, size_t *n_out) {
+    if (!c || (batch && !n_out)) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    const int kind = kind_of_format(format);
+    int rc = gate_shape_check(c, kind, gate_len, n, hidden);
+    if (rc) return rc;
+    for (size_t b = 0; b < batch; b++) n_out[b] = 0;
+    if (batch == 0 || n == 0 || top_k == 0) return LARQL_OK;  // top_k_by_abs: K==0 or no scores -> empty
+    if (top_k > 64) return fail(c, LARQL_UNSUPPORTED, "gate-KNN: top_k above 64 is not served by this kernel");
+    if (n > 0xFFFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "gate-KNN: too many features");
+    if (hidden == 0) return fail(c, LARQL_UNSUPPORTED, "gate-KNN: hidden == 0");
+    if (!gate || !x || !idx_out || !score_out) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    const uint8_t *dg = nullptr;
+    rc = resolve_weights(c, gate, n * format_row_bytes(kind, hidden), c->w[0], &dg); if (rc) return rc;
+    rc = upload(c, c->x, x, batch * hidden * 4); if (rc) return rc;
+    rc = ensure(c, c->scores, batch * n * 4 + 64); if (rc) return rc;
+    rc = ensure(c, c->misc, batch * (top_k * 8 + 4) + 64); if (rc) return rc;
+    HIPCHECK(c, hipMemsetAsync(c->nan_flag, 0, sizeof(int), c->stream));
+    Submission sub(c);
+    rc = dev_gate_scores(c, kind, dg, (const float *)c->x.p, batch, n, hidden, (float *)c->scores.p);
+    if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
+    uint32_t *d_idx = (uint32_t *)c->misc.p;
+    float *d_val = (float *)(d_idx + batch * top_k);
+    uint32_t *d_cnt = (uint32_t *)(d_val + batch * top_k);
+    HIPCHECK(c, topk_launch(c->stream, (const float *)c->scores.p, (uint32_t)batch, (uint32_t)n, (uint32_t)top_k, true, d_idx,
+                            d_val, d_cnt, c->nan_flag, nullptr, 0));
+    rc = sub.finish();
+    if (rc) return rc;
+    return topk_download(c, batch, top_k, idx_out, score_out, n_out, true);
+}
+
+// ---- device tier ----------------------------------------------------------------------------
+
+int larql_hip_malloc(larql_hip_ctx *c, void **dptr, size_t bytes) {
+    if (!c || !dptr) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, hipMalloc(dptr, bytes ? bytes : 1));
+    return LARQL_OK;
+}
+int larql_hip_free(larql_hip_ctx *c, void *dptr) {
+    if (!c) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, hipStreamSynchronize(c->stream));
+    HIPCHECK(c, hipFree(dptr));
+    return LARQL_OK;
+}
+int larql_hip_memcpy_h2d(larql_hip_ctx *c, void *dst, const void *src, size_t bytes) {
+    if (!c) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, c->stream));
+    HIPCHECK(c, hipStreamSynchronize(c->stream));
+    return LARQL_OK;
+}
+int larql_hip_memcpy_d2h(larql_hip_ctx *c, void *dst, const void *src, size_t bytes) {
+    if (!c) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, c->stream));
+    HIPCHECK(c, hipStreamSynchronize(c->stream));
+    return LARQL_OK;
+}
+int larql_hip_memset(larql_hip_ctx *c, void *dst, int value, size_t bytes) {
+    if (!c) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, hipMemsetAsync(dst, value, bytes, c->stream));
+    return LARQL_OK;
+}
+int larql_hip_synchronize(larql_hip_ctx *c) {
+    if (!c) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, hipStreamSynchronize(c->stream));
+    return LARQL_OK;
+}
+int larql_hip_event_create(larql_hip_ctx *c, void **event) {
+    if (!c || !event) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    hipEvent_t e;
+    HIPCHECK(c, hipEventCreate(&e));
+    *event = (void *)e;
+    return LARQL_OK;
+}
+int larql_hip_event_record(larql_hip_ctx *c, void *event) {
+    if (!c || !event) return LARQL_E_ARG;
+    HIPCHECK(c, hipEventRecord((hipEvent_t)event, c->stream));
+    return LARQL_OK;
+}
+int larql_hip_event_elapsed_ms(larql_hip_ctx *c, void *start, void *stop, float *ms) {
+    if (!c || !start || !stop || !ms) return LARQL_E_ARG;
+    HIPCHECK(c, hipEventSynchronize((hipEvent_t)stop));
+    HIPCHECK(c, hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return LARQL_OK;
+}
+int larql_hip_event_destroy(larql_hip_ctx *c, void *event) {
+    if (!c || !event) return LARQL_E_ARG;
+    HIPCHECK(c, hipEventDestroy((hipEvent_t)event));
+    return LARQL_OK;
+}
+
+static int dev_job_from_public(larql_hip_ctx *c, const larql_hip_matvec_job &p, std::vector<GemvJob> &jobs) {
+    const int kind = kind_of_format(p.format);
+    if (kind < 0) return fail(c, LARQL_UNSUPPORTED, "matvec: format %d has no kernel", p.format);
+    if (kind == KIND_MXFP4 && !p.aux) return fail(c, LARQL_E_ARG, "matvec: MXFP4 needs the scale stream");
+    if (kind == KIND_Q4_0) return fail(c, LARQL_UNSUPPORTED, "matvec batch: Q4_0 goes through larql_hip_dev_matvec");
+    if (kind == KIND_Q4K && p.k % 256 != 0) return fail(c, LARQL_REFUSED_SHAPE, "matvec: k not a multiple of 256");
+    if (p.k % 32 != 0) return fail(c, LARQL_REFUSED_SHAPE, "matvec: k not a multiple of 32");
+    jobs.push_back(make_job(kind, p.w, p.aux, p.x, p.out, p.rows, p.k));
+    return LARQL_OK;
+}
+
+int larql_hip_dev_matvec_batch(larql_hip_ctx *c, const larql_hip_matvec_job *pj, size_t n_jobs) {
+    if (!c || (!pj && n_jobs)) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    HIPCHECK(c, hipSetDevice(c->device));
+    std::vector<GemvJob> jobs;
+    for (size_t i = 0; i < n_jobs; i++) {
+        int rc = dev_job_from_public(c, pj[i], jobs);
+        if (rc) return rc;
+    }
+    return enqueue_jobs(c, jobs);
+}
+
+int larql_hip_dev_matvec(larql_hip_ctx *c, int format, const void *w, const void *aux, const float *x, size_t rows, size_t k,
+                         float *out) {
+    if (!c) return LARQL_E_ARG;
+    if (format == LARQL_FMT_Q4_0) {
+        std::lock_guard<std::mutex> lk(c->mu);
+        HIPCHECK(c, hipSetDevice(c->device));
+        if (k % 32 != 0) return fail(c, LARQL_REFUSED_SHAPE, "matvec: k not a multiple of 32");
+        int rc = ensure(c, c->q8, k + 64); if (rc) return rc;
+        rc = ensure(c, c->q8s, (k / 32) * 4 + 64); if (rc) return rc;
+        HIPCHECK(c, quantize_to_q8_launch(c->stream, x, k, (int8_t *)c->q8.p, (float *)c->q8s.p));
+        std::vector<GemvJob> jobs{make_job(KIND_Q4_0, w, c->q8s.p, c->q8.p, out, rows, k)};
+        return enqueue_jobs(c, jobs);
+    }
+    larql_hip_matvec_job j;
+    memset(&j, 0, sizeof j);
+    j.format = format; j.w = w; j.aux = aux; j.x = x; j.out = out; j.rows = rows; j.k = k;
+    return larql_hip_dev_matvec_batch(c, &j, 1);
+}
+
+int larql_hip_dev_gate_knn(larql_hip_ctx *c, int format, const void *gate, const float *x, size_t batch, size_t n, size_t hidden,
+                           size_t top_k, float *scores_scratch, uint32_t *idx_out, float *score_out) {
+    if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    const int kind = kind_of_format(format);
+    int rc = gate_shape_check(c, kind, (size_t)-1, 0, hidden);
+    if (rc) return rc;
+    if (batch == 0 || n == 0 || top_k == 0) return LARQL_OK;
+    if (top_k > 64 || n > 0xFFFFFFFFull || hidden == 0) return fail(c, LARQL_UNSUPPORTED, "gate-KNN: unsupported size");
+    HIPCHECK(c, hipSetDevice(c->device));
+    rc = ensure(c, c->misc, batch * 4 + 64); if (rc) return rc;
+    rc = dev_gate_scores(c, kind, gate, x, batch, n, hidden, scores_scratch);
+    if (rc) return rc;
+    HIPCHECK(c, topk_launch(c->stream, scores_scratch, (uint32_t)batch, (uint32_t)n, (uint32_t)top_k, true, idx_out, score_out,
+                            (uint32_t *)c->misc.p, c->nan_flag, nullptr, 0));
+    return LARQL_OK;
+}
+
+// ---- device tier: encoders ---------------------------------------------------------------------
+
+int larql_hip_dev_quantize_q4_k(larql_hip_ctx *c, const float *src, size_t n, uint8_t *dst) {
+    if (!c) return LARQL_E_ARG;
+    if (n % 256 != 0) return fail(c, LARQL_REFUSED_SHAPE, "quantize_q4_k: length must be a multiple of 256");
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, quantize_q4_k_launch(c->stream, src, n, dst));
+    return LARQL_OK;
+}
+int larql_hip_dev_quantize_q8_0(larql_hip_ctx *c, const float *src, size_t n, uint8_t *dst) {
+    if (!c) return LARQL_E_ARG;
+    if (n % 32 != 0) return fail(c, LARQL_REFUSED_SHAPE, "quantize_q8_0: length must be a multiple of 32");
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, quantize_q8_0_launch(c->stream, src, n, dst));
+    return LARQL_OK;
+}
+int larql_hip_dev_quantize_mxfp4(larql_hip_ctx *c, const float *src, size_t rows, size_t k, uint8_t *packed, uint8_t *scales) {
+    if (!c) return LARQL_E_ARG;
+    if (k % 32 != 0) return fail(c, LARQL_REFUSED_SHAPE, "quantize_mxfp4: k must be a multiple of 32");
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, quantize_mxfp4_launch(c->stream, src, rows, k, packed, scales, c->log2_up));
+    return LARQL_OK;
+}
+int larql_hip_dev_f32_to_bf16(larql_hip_ctx *c, const float *src, size_t n, uint16_t *dst) {
+    if (!c) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, f32_to_bf16_launch(c->stream, src, n, dst));
+    return LARQL_OK;
+}
+int larql_hip_dev_quantize_q4_0(larql_hip_ctx *c, const float *src, size_t n, uint8_t *dst) {
+    if (!c) return LARQL_E_ARG;
+    if (n % 32 != 0) return fail(c, LARQL_REFUSED_SHAPE, "quantize_q4_0: length must be a multiple of 32");
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, quantize_q4_0_launch(c->stream, src, n, dst));
+    return LARQL_OK;
+}
+int larql_hip_dev_quantize_to_q8(larql_hip_ctx *c, const float *src, size_t n, int8_t *q8, float *scales) {
+    if (!c) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, quantize_to_q8_launch(c->stream, src, n, q8, scales));
+    return LARQL_OK;
+}
+int larql_hip_dev_fill_normal(larql_hip_ctx *c, float *dst, size_t n, uint64_t seed, float sigma) {
+    if (!c) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, fill_normal_launch(c->stream, dst, n, seed, sigma));
+    return LARQL_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,62 @@
+// kernels.h — shared declarations between the HIP kernels and the C-ABI layer.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace larql {
+
+enum GemvKind : int32_t {
+    KIND_Q4K = 0, KIND_Q8_0 = 1, KIND_MXFP4 = 2, KIND_Q4_0 = 3, KIND_BF16 = 4, KIND_F16 = 5, KIND_F32 = 6
+};
+
+constexpr int kGemvMaxThreads = 512;
+constexpr int kInlineJobs = 4;
+
+// One matvec of a launch.  The caller fills kind/w/aux/x/out/rows/k; the rest
+// is geometry derived by gemv_job_geometry for the launch's block size.
+struct GemvJob {
+    const uint8_t *w;    // packed weights, [rows] rows of row_bytes
+    const uint8_t *aux;  // MXFP4: e8m0 scales [rows, k/32]; Q4_0: f32 activation scales
+    const float *x;      // activation (Q4_0: the int8 code stream)
+    float *out;
+    uint64_t rows, k;
+    uint64_t row_bytes;
+    uint32_t cpr;         // chunks (threads) per row
+    uint32_t rpp;         // rows per pass
+    uint32_t n_pass;      // ceil(rows / rpp)
+    uint32_t pass_begin;  // first pass of this job in the launch's pass list
+    int32_t kind;
+    int32_t pad;
+};
+
+struct GemvLaunch {
+    const GemvJob *table;  // device table, or null to use `inl`
+    GemvJob inl[kInlineJobs];
+    uint64_t total_passes;
+    uint32_t n_jobs;
+    uint32_t pad;
+};
+
+bool gemv_job_geometry(GemvJob &j, uint32_t threads);
+uint32_t gemv_pick_threads(const GemvJob *jobs, size_t n);
+size_t gemv_lds_bytes(const GemvJob *jobs, size_t n);
+hipError_t gemv_launch(hipStream_t stream, const GemvLaunch &L, uint32_t threads, uint32_t grid, size_t lds);
+
+// top-K by |score| (or by value) over rows of a [batch, n] score matrix
+hipError_t topk_launch(hipStream_t stream, const float *scores, uint32_t batch, uint32_t n, uint32_t k,
+                       bool by_abs, uint32_t *idx_out, float *val_out, uint32_t *count_out, int *nan_flag,
+                       void *workspace, size_t workspace_bytes);
+size_t topk_workspace_bytes(uint32_t batch, uint32_t n, uint32_t k);
+
+// encoders and the synthetic data generator
+hipError_t quantize_q4_k_launch(hipStream_t s, const float *src, size_t n, uint8_t *dst);
+hipError_t quantize_q8_0_launch(hipStream_t s, const float *src, size_t n, uint8_t *dst);
+hipError_t quantize_mxfp4_launch(hipStream_t s, const float *src, size_t rows, size_t k, uint8_t *packed,
+                                 uint8_t *scales, const uint8_t *log2_up_table);
+hipError_t f32_to_bf16_launch(hipStream_t s, const float *src, size_t n, uint16_t *dst);
+hipError_t quantize_q4_0_launch(hipStream_t s, const float *src, size_t n, uint8_t *dst);
+hipError_t quantize_to_q8_launch(hipStream_t s, const float *src, size_t n, int8_t *q8, float *scales);
+hipError_t fill_normal_launch(hipStream_t s, float *dst, size_t n, uint64_t seed, float sigma);
+
+}  // namespace larql

@@ -1,0 +1,366 @@
+"""GPU parity: the HIP path, driven through the C ABI (larql_amd.HipBackend is
+a thin ctypes mirror of the trait), against the CPU oracle on the same seeded
+inputs.  Bars: quantised bytes bit-exact; matvec outputs within 1e-3 relative
+L2 (fp32 accumulate; measured ~1e-6, asserted at 2e-5 so a wrong scale or a
+dropped term cannot hide); top-K index sets identical except at score ties
+within 1e-5."""
+import numpy as np
+import pytest
+
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+TOL = 2e-5
+
+
+@pytest.fixture(scope="module")
+def be():
+    import larql_amd
+    b = larql_amd.HipBackend()
+    yield b
+    b.close()
+
+
+@pytest.fixture(scope="module")
+def fmt():
+    import larql_amd
+    return larql_amd
+
+
+def rel_l2(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30)
+
+
+def weights(seed, rows, cols, sigma=0.02):
+    rng = np.random.default_rng(seed)
+    return (rng.standard_normal((rows, cols)) * sigma).astype(F), rng.standard_normal(cols).astype(F)
+
+
+# ------------------------------------------------------------------- Q4_K
+@pytest.mark.parametrize("rows,cols", [(3072, 1024), (2048, 2560), (1031, 2560), (77, 10240), (5, 256), (640, 2048),
+                                       (300, 3840), (33, 1792)])
+def test_q4k_matvec_matches_oracle(be, rows, cols):
+    w, x = weights(rows * 7 + cols, rows, cols)
+    q = O.quantize_q4_k(w)
+    want = O.q4k_matvec(q, x, rows, cols)
+    got = be.q4k_matvec(q, x, rows, cols)
+    assert got is not None and got.shape == (rows,)
+    assert rel_l2(got, want) < TOL
+    # every row individually (guards against unwritten or swapped rows)
+    scale = np.abs(want).mean() + 1e-12
+    assert np.max(np.abs(got - want)) < 1e-3 * scale
+    # deterministic across repeats
+    assert np.array_equal(got.view(np.uint32), be.q4k_matvec(q, x, rows, cols).view(np.uint32))
+
+
+def test_q4k_matvec_refusals_follow_the_cpu_backend(be):
+    w, x = weights(1, 3, 512)
+    q = O.quantize_q4_k(w)
+    assert be.q4k_matvec(q, x, 3, 512) is not None
+    assert be.q4k_matvec(q, x, 3, 512, out_len=2) is None
+    assert be.q4k_matvec(q, x[:511], 3, 512) is None
+    assert be.q4k_matvec(q, x[:500], 3, 500) is None
+    assert be.q4k_matvec(q[:-1], x, 3, 512) is None
+    assert be.q4k_matvec(np.concatenate([q, q]), x, 3, 512) is not None
+    z = be.q4k_matvec(np.zeros(0, np.uint8), np.zeros(0, F), 4, 0)
+    assert z is not None and z.shape == (4,) and not z.any()
+    assert be.q4k_matvec(np.zeros(0, np.uint8), np.zeros(0, F), 0, 0).size == 0
+
+
+def test_q4k_subnormal_scales_and_extreme_headers(be):
+    # tiny weights force f16-subnormal d/dmin; they must not be flushed
+    w, x = weights(3, 64, 512, sigma=2e-5)
+    q = O.quantize_q4_k(w)
+    hdr = q.reshape(-1, 144)[:, :2].copy().view(np.uint16)
+    assert (hdr < 0x0400).any(), "fixture should contain subnormal scales"
+    want = O.q4k_matvec(q, x, 64, 512)
+    assert rel_l2(be.q4k_matvec(q, x, 64, 512), want) < TOL
+    # all 6-bit scale/min codes exercised: random header bytes, fixed d/dmin
+    rng = np.random.default_rng(4)
+    q = rng.integers(0, 256, size=32 * 2 * 144, dtype=np.uint8).reshape(-1, 144)
+    q[:, 0:2] = np.array([0x00, 0x2C], np.uint8)   # d = 2^-4
+    q[:, 2:4] = np.array([0x00, 0x28], np.uint8)   # dmin = 2^-5
+    q = q.reshape(-1)
+    want = O.q4k_matvec(q, x, 32, 512)
+    assert rel_l2(be.q4k_matvec(q, x, 32, 512), want) < TOL
+
+
+def test_q4k_dual_and_matmul(be):
+    rows, cols, seq = 515, 2560, 5
+    a, x = weights(5, rows, cols)
+    b, _ = weights(6, rows, cols, 0.05)
+    qa, qb = O.quantize_q4_k(a), O.quantize_q4_k(b)
+    oa, ob = be.q4k_dual_matvec(qa, qb, x, rows, cols)
+    # bit-identical to the single calls (the multi contract of backend/matmul.rs:151-194)
+    assert np.array_equal(oa.view(np.uint32), be.q4k_matvec(qa, x, rows, cols).view(np.uint32))
+    assert np.array_equal(ob.view(np.uint32), be.q4k_matvec(qb, x, rows, cols).view(np.uint32))
+    assert rel_l2(ob, O.q4k_matvec(qb, x, rows, cols)) < TOL
+    assert be.q4k_dual_matvec(qa, qb[:-1], x, rows, cols) is None
+    X = np.random.default_rng(7).standard_normal((seq, cols)).astype(F)
+    out = be.q4k_matmul(qa, X, rows, cols, seq)
+    want = O.q4k_matmul(qa, X, rows, cols, seq)
+    assert rel_l2(out, want.reshape(-1)) < TOL
+    assert be.q4k_matmul(qa, X, rows, cols, 0).size == 0 or True
+    # shape error zero-fills like the CPU kernel
+    bad = be.q4k_matmul(qa[:-1], X, rows, cols, seq)
+    assert bad is not None and not bad.any()
+
+
+# ------------------------------------------------------------------ Q8_0
+@pytest.mark.parametrize("n,k", [(4099, 2560), (64, 10240), (9, 128), (1000, 2048)])
+def test_q8_0_gemv_matches_oracle(be, n, k):
+    w, x = weights(n + k, n, k)
+    w[0, :32] *= 1e-5
+    q = O.quantize_q8_0(w)
+    want = O.q8_0_gemv(q, x, n, k)
+    got = be.q8_0_gemv(q, x, n, k)
+    assert rel_l2(got, want) < TOL
+    assert np.max(np.abs(got - want)) < 1e-3 * (np.abs(want).mean() + 1e-12)
+    assert be.q8_0_gemv(q[:-1], x, n, k) is None and be.q8_0_gemv(q, x[:-1], n, k) is None
+    assert be.q8_0_gemv(np.concatenate([q, q[:2]]), x, n, k) is None
+
+
+# ----------------------------------------------------------------- MXFP4
+def test_mxfp4_gemv_matches_dequant_reference(be):
+    # the Metal peer's recipe: cos > 0.999999 and rel < 1e-4 vs dequantize_expert, sentinels, ragged rows
+    n, k = 2880 + 3, 2880
+    w, x = weights(11, n, k)
+    p, s = O.quantize_mxfp4(w, n, k)
+    want = O.mxfp4_gemv(p, s, x, n, k)
+    got = be.mxfp4_gemv(p, s, x, n, k)
+    assert rel_l2(got, want) < TOL and rel_l2(got, O.mxfp4_gemv_dequant(p, s, x, n, k)) < TOL
+    s2 = s.copy(); s2[0] = 0; s2[90] = 255
+    got2 = be.mxfp4_gemv(p, s2, x, n, k)
+    want2 = O.mxfp4_gemv(p, s2, x, n, k)
+    assert np.isnan(got2[1]) and np.isnan(want2[1])
+    ok = np.ones(n, bool); ok[1] = False
+    assert rel_l2(got2[ok], want2[ok]) < TOL
+    assert be.mxfp4_gemv(p, s, x[:-1], n, k) is None
+    assert be.mxfp4_gemv(p[:-1], s, x, n, k) is None
+    assert be.mxfp4_gemv(p, s, x, n, 2881) is None
+    # multi: argument order, bit-identical to the single calls, empty batch is Some([])
+    outs = be.mxfp4_gemv_multi([(p, s, n, k), (p, s2, n, k), (p[: 7 * 90 * 16], s[: 7 * 90], 7, k)], x)
+    assert np.array_equal(outs[0].view(np.uint32), got.view(np.uint32))
+    assert np.array_equal(outs[1].view(np.uint32), got2.view(np.uint32)) and outs[2].shape == (7,)
+    assert be.mxfp4_gemv_multi([], x) == []
+    assert be.mxfp4_gemv_multi([(p, s, n, k), (p[:-1], s, n, k)], x) is None
+
+
+# ---------------------------------------------------------- dense + Q4_0
+def test_dense_gemvs(be):
+    n, k = 1000, 2560
+    w, x = weights(13, n, k)
+    wb = O.f32_to_bf16(w)
+    assert rel_l2(be.bf16_gemv_force(wb, x, n, k), O.bf16_gemv(wb, x, n, k)) < TOL
+    wh = w.astype(np.float16).view(np.uint16)
+    assert rel_l2(be.f16_gemv_force(wh, x, n, k), O.f16_gemv(wh, x, n, k)) < TOL
+    assert rel_l2(be.f32_gemv_force(w, x), O.f32_gemv(w, x, n, k)) < TOL
+    # below the flop threshold the non-force variants answer None (2*n*k < 5e8)
+    assert be.f32_gemv(w, x) is None and be.bf16_gemv(wb, x, n, k) is None
+    assert be.f16_gemv_force(wh[:-1], x, n, k) is None and be.f16_gemv_force(wh, x[:-1], n, k) is None
+
+
+def test_q4_0_q8_matvec_and_quant_matvec_dispatch(be, fmt):
+    rows, hidden = 1027, 2560
+    w, x = weights(17, rows, hidden)
+    q4 = O.quantize_q4_0(w)
+    q8, sc = O.quantize_to_q8(x)
+    want = O.q4_0_matvec(q4, q8, sc, rows, hidden)
+    got = be.q4_matvec(q4, q8, sc, rows, hidden)
+    assert rel_l2(got, want) < TOL
+    assert be.q4_matvec(q4[:-1], q8, sc, rows, hidden) is None
+    # QuantMatVec::quant_matvec: Q4_0 quantises x on the way in; Q4_K is the f32 path
+    got2 = be.quant_matvec(fmt.FMT_Q4_0, q4, x, rows, hidden)
+    assert rel_l2(got2, want) < TOL
+    qk = O.quantize_q4_k(w)
+    assert rel_l2(be.quant_matvec(fmt.FMT_Q4_K, qk, x, rows, hidden), O.q4k_matvec(qk, x, rows, hidden)) < TOL
+    for f in (fmt.FMT_Q8_0, fmt.FMT_Q6_K, fmt.FMT_MXFP4, fmt.FMT_F32, fmt.FMT_I2S):
+        assert be.quant_matvec(f, qk, x, rows, hidden) is None
+
+
+# ------------------------------------------------------------------ gate-KNN
+def check_hits(got, scores, k):
+    """Same index set as top_k_by_abs up to ties within 1e-5, scores right, sorted by |score|."""
+    want = O.top_k_by_abs(scores, k)
+    assert len(got) == len(want)
+    gi, wi = {i for i, _ in got}, {i for i, _ in want}
+    if gi != wi:
+        kth = abs(want[-1][1])
+        for i in gi ^ wi:
+            assert abs(abs(float(scores[i])) - kth) <= 1e-5 * max(1.0, kth), (i, scores[i], kth)
+    mags = [abs(v) for _, v in got]
+    assert all(mags[i] >= mags[i + 1] for i in range(len(mags) - 1))
+    for i, v in got:
+        assert abs(v - float(scores[i])) <= 1e-5 * max(1.0, abs(v))
+
+
+@pytest.mark.parametrize("variant", ["bf16", "q4k", "f32", "f16", "q4_0"])
+@pytest.mark.parametrize("batch", [1, 8])
+def test_gate_knn_matches_oracle(be, fmt, variant, batch):
+    n, hidden, k = 10240, 2560, 64
+    rng = np.random.default_rng(23)
+    g = (rng.standard_normal((n, hidden)) * 0.02).astype(F)
+    X = rng.standard_normal((batch, hidden)).astype(F)
+    if variant == "bf16":
+        gate, f = O.f32_to_bf16(g), fmt.FMT_BF16
+        ref = [O.bf16_gemv(gate, X[b], n, hidden) for b in range(batch)]
+    elif variant == "f16":
+        gate, f = g.astype(np.float16).view(np.uint16), fmt.FMT_F16
+        ref = [O.f16_gemv(gate, X[b], n, hidden) for b in range(batch)]
+    elif variant == "f32":
+        gate, f = g, fmt.FMT_F32
+        ref = [O.f32_gemv(g, X[b], n, hidden) for b in range(batch)]
+    elif variant == "q4k":
+        gate, f = O.quantize_q4_k(g), fmt.FMT_Q4_K
+        ref = [O.q4k_matvec(gate, X[b], n, hidden) for b in range(batch)]
+    else:
+        gate, f = O.quantize_q4_0(g), fmt.FMT_Q4_0
+        ref = [O.q4_0_matvec(gate, *O.quantize_to_q8(X[b]), n, hidden) for b in range(batch)]
+    hits = be.gate_knn_batch_hits(f, gate, X, n, hidden, k)
+    assert len(hits) == batch
+    for b in range(batch):
+        check_hits(hits[b], ref[b], k)
+    scores = be.gate_scores_batch(f, gate, X, n, hidden)
+    assert rel_l2(scores, np.stack(ref)) < TOL
+    union = be.gate_knn_batch(f, gate, X, n, hidden, k)
+    want_union = O.gate_knn_batch_union(np.stack(ref).T.copy(), k)
+    assert len(set(union) ^ set(want_union)) <= 2 * batch   # only tie-level differences at the k-th score
+    assert union == sorted(set(union))
+
+
+def test_gate_knn_edge_cases(be, fmt):
+    rng = np.random.default_rng(29)
+    n, hidden = 100, 256
+    g = (rng.standard_normal((n, hidden)) * 0.02).astype(F)
+    x = rng.standard_normal(hidden).astype(F)
+    s = O.f32_gemv(g, x, n, hidden)
+    check_hits(be.gate_knn(fmt.FMT_F32, g, x, n, hidden, 64), s, 64)
+    hits = be.gate_knn(fmt.FMT_F32, g[:10], x, 10, hidden, 64)   # K > N -> all N
+    assert len(hits) == 10
+    assert be.gate_knn(fmt.FMT_F32, g, x, n, hidden, 0) == []     # K == 0 -> empty
+    assert be.gate_knn(fmt.FMT_F32, g, x, n, hidden, 65) is None  # beyond the kernel's capacity: refused
+    xn = x.copy(); xn[3] = np.nan
+    import larql_amd
+    with pytest.raises(larql_amd.NanScoreError):
+        be.gate_knn(fmt.FMT_F32, g, xn, n, hidden, 8)
+    # reference closed forms (gate_knn/mod.rs:231-287) through one-hot gates: scores == x
+    eye = np.eye(256, dtype=F)[:4]
+    xv = np.zeros(256, F); xv[:4] = [0.1, -0.9, 0.5, 0.3]
+    hits = be.gate_knn(fmt.FMT_F32, eye, xv, 4, 256, 2)
+    assert [i for i, _ in hits] == [1, 2] and abs(hits[0][1] + 0.9) < 1e-6
+    # exact ties: lower index first
+    xt = np.zeros(256, F); xt[:4] = [1.0, -1.0, 1.0, 0.5]
+    assert [i for i, _ in be.gate_knn(fmt.FMT_F32, eye, xt, 4, 256, 2)] == [0, 1]
+
+
+def test_q4k_matvec_topk_by_value(be):
+    rows, cols = 5000, 512
+    w, x = weights(31, rows, cols)
+    q = O.quantize_q4_k(w)
+    scores = O.q4k_matvec(q, x, rows, cols)
+    for k in (1, 5, 8, 64):
+        got = be.q4k_matvec_topk(q, x, rows, cols, k)
+        want = O.top_k_sorted(scores, k)
+        assert [i for i, _ in got] == [i for i, _ in want]
+    assert be.q4k_matvec_topk(q, x, rows, cols, 0) is None
+    assert be.q4k_matvec_topk(q, x, rows, cols, 65) is None
+    assert be.q4k_matvec_topk(q, x[:-1], rows, cols, 4) is None
+
+
+# ------------------------------------------------------------- residency
+def test_registered_region_serves_sub_slices(be):
+    rows, cols = 256, 1024
+    w1, x = weights(37, rows, cols)
+    w2, _ = weights(38, rows, cols)
+    blob = np.concatenate([O.quantize_q4_k(w1), O.quantize_q4_k(w2)])
+    be.register_weight_region(blob)
+    be.register_weight_region(blob)        # same base twice: no-op
+    be.seal_weight_regions()
+    half = blob.size // 2
+    before = be.submission_clock()
+    a = be.q4k_matvec(blob[:half], x, rows, cols)
+    b = be.q4k_matvec(blob[half:], x, rows, cols)
+    after = be.submission_clock()
+    assert rel_l2(a, O.q4k_matvec(blob[:half], x, rows, cols)) < TOL
+    assert rel_l2(b, O.q4k_matvec(blob[half:], x, rows, cols)) < TOL
+    assert after["submissions"] == before["submissions"] + 2 and after["gpu_nanos"] > before["gpu_nanos"]
+    be.clear_weight_regions()
+    assert rel_l2(be.q4k_matvec(blob[:half], x, rows, cols), a) == 0
+
+
+# ---------------------------------------------------------------- encoders
+def test_device_encoders_are_bit_exact(be):
+    rng = np.random.default_rng(41)
+    n = 256 * 4096
+    w = (rng.standard_normal(n) * 0.02).astype(F)
+    w[:256] = 0; w[256:512] = np.abs(w[256:512]); w[512:768] = -np.abs(w[512:768]); w[768:800] = 1e-7
+    w[1024:1056] = np.nextafter(F(0.0625), F(0))       # log2 edge just below a power of two
+    src = be.to_device(w)
+    dst = be.malloc(n * 2)
+    assert be.dev_quantize_q4_k(src, n, dst)
+    assert np.array_equal(be.d2h(dst, n // 256 * 144, np.uint8), O.quantize_q4_k(w))
+    assert be.dev_quantize_q8_0(src, n, dst)
+    assert np.array_equal(be.d2h(dst, n // 32 * 34, np.uint8), O.quantize_q8_0(w))
+    assert be.dev_quantize_q4_0(src, n, dst)
+    assert np.array_equal(be.d2h(dst, n // 32 * 18, np.uint8), O.quantize_q4_0(w))
+    assert be.dev_f32_to_bf16(src, n, dst)
+    assert np.array_equal(be.d2h(dst, n, np.uint16), O.f32_to_bf16(w))
+    sc = be.malloc(n // 32 * 4)
+    assert be.dev_quantize_to_q8(src, n, dst, sc)
+    q8, s8 = O.quantize_to_q8(w)
+    assert np.array_equal(be.d2h(dst, n, np.int8), q8) and np.array_equal(be.d2h(sc, n // 32, F).view(np.uint32), s8.view(np.uint32))
+    k = 2880
+    rows = n // k
+    assert be.dev_quantize_mxfp4(src, rows, k, dst, sc)
+    p, s = O.quantize_mxfp4(w[: rows * k], rows, k)
+    assert np.array_equal(be.d2h(sc, rows * 90, np.uint8), s)
+    assert np.array_equal(be.d2h(dst, rows * 90 * 16, np.uint8), p)
+    for ptr in (src, dst, sc):
+        be.free(ptr)
+
+
+def test_fill_normal_statistics(be):
+    n = 1 << 20
+    d = be.malloc(n * 4)
+    assert be.dev_fill_normal(d, n, 1234, 0.02)
+    a = be.d2h(d, n, F)
+    assert be.dev_fill_normal(d, n, 1234, 0.02)
+    assert np.array_equal(a, be.d2h(d, n, F))                      # a pure function of (seed, index)
+    assert be.dev_fill_normal(d, n, 1235, 0.02)
+    assert not np.array_equal(a, be.d2h(d, n, F))
+    assert abs(a.mean()) < 1e-4 and abs(a.std() - 0.02) < 2e-4
+    assert abs(np.mean(np.abs(a) > 0.04) - 0.0455) < 0.003         # two-sigma tail mass of a normal
+    be.free(d)
+
+
+# ------------------------------------------------------------ device tier
+def test_dev_matvec_batch_mixed_formats(be, fmt):
+    rng = np.random.default_rng(43)
+    jobs, wants, outs = [], [], []
+    x_h = rng.standard_normal(10240).astype(F)
+    x = be.to_device(x_h)
+    specs = [("q4k", 300, 2560), ("q4k", 70, 10240), ("q8", 500, 2560), ("q4k", 129, 2048), ("bf16", 100, 2560),
+             ("q4k", 40, 2560), ("q8", 3, 2560)]
+    for kind, rows, k in specs:
+        w = (rng.standard_normal((rows, k)) * 0.02).astype(F)
+        if kind == "q4k":
+            q = O.quantize_q4_k(w); f = fmt.FMT_Q4_K; want = O.q4k_matvec(q, x_h[:k], rows, k)
+        elif kind == "q8":
+            q = O.quantize_q8_0(w); f = fmt.FMT_GGML_Q8_0; want = O.q8_0_gemv(q, x_h[:k], rows, k)
+        else:
+            q = O.f32_to_bf16(w); f = fmt.FMT_BF16; want = O.bf16_gemv(q, x_h[:k], rows, k)
+        dw = be.to_device(q)
+        do = be.malloc(rows * 4)
+        jobs.append((f, dw, None, x, do, rows, k)); wants.append(want); outs.append((do, rows))
+    assert be.dev_matvec_batch(jobs)
+    be.synchronize()
+    for (do, rows), want in zip(outs, wants):
+        assert rel_l2(be.d2h(do, rows, F), want) < TOL
+    # and one at a time gives the same bits
+    f, dw, _, _, do, rows, k = jobs[1]
+    first = be.d2h(do, rows, F)
+    assert be.dev_matvec(f, dw, None, x, rows, k, do)
+    be.synchronize()
+    assert np.array_equal(first.view(np.uint32), be.d2h(do, rows, F).view(np.uint32))
