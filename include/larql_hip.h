@@ -197,6 +197,12 @@ int larql_hip_event_record(larql_hip_ctx *ctx, void *event);
 int larql_hip_event_elapsed_ms(larql_hip_ctx *ctx, void *start, void *stop, float *ms);
 int larql_hip_event_destroy(larql_hip_ctx *ctx, void *event);
 
+/* Plain streaming kernels: copy `bytes` from src to dst with 16-byte loads
+ * and stores, or (dst == NULL) only read src.  No counterpart in the
+ * reference: they are the yardstick for achievable HBM bandwidth and for
+ * scaling profiler byte counters. */
+int larql_hip_dev_copy(larql_hip_ctx *ctx, void *dst, const void *src, size_t bytes);
+
 /* One matvec on resident operands: out[rows] = W[rows,k] . x[k].
  * format: Q4_K, GGML_Q8_0, MXFP4 (aux = e8m0 scale stream), BF16, F16, F32,
  * Q4_0 (x is then the f32 activation, quantised to Q8 on the device as

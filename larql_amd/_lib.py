@@ -70,6 +70,7 @@ SIGNATURES = {
     "larql_hip_event_record": (ci, [vp, vp]),
     "larql_hip_event_elapsed_ms": (ci, [vp, vp, vp, C.POINTER(C.c_float)]),
     "larql_hip_event_destroy": (ci, [vp, vp]),
+    "larql_hip_dev_copy": (ci, [vp, vp, vp, sz]),
     "larql_hip_dev_matvec": (ci, [vp, ci, vp, vp, vp, sz, sz, vp]),
     "larql_hip_dev_matvec_batch": (ci, [vp, C.POINTER(MatvecJob), sz]),
     "larql_hip_dev_gate_knn": (ci, [vp, ci, vp, vp, sz, sz, sz, sz, vp, vp, vp]),

@@ -290,6 +290,9 @@ class HipBackend:
         self._some(lib.larql_hip_event_elapsed_ms(self._h, a, b, C.byref(ms)))
         return ms.value
 
+    def dev_copy(self, dst: Optional[int], src: int, nbytes: int) -> bool:
+        return self._some(lib.larql_hip_dev_copy(self._h, dst, src, nbytes))
+
     def dev_matvec(self, fmt: int, w: int, aux: Optional[int], x: int, rows: int, k: int, out: int) -> bool:
         return self._some(lib.larql_hip_dev_matvec(self._h, fmt, w, aux, x, rows, k, out))
 

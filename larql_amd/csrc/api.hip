@@ -44,7 +44,7 @@ struct larql_hip_ctx {
     std::mutex mu;
     std::string name, info, last_error;
     std::vector<Region> regions;
-    DevBuf w[4], aux[4], x, out, table, misc, scores, q8, q8s;
+    DevBuf w[4], aux[4], x, out, tables[4], misc, scores, q8, q8s;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     uint8_t *log2_up = nullptr;  // 256-entry table for the MXFP4 encoder
     int *nan_flag = nullptr;
@@ -134,19 +134,9 @@ int kind_of_format(int format) {
     }
 }
 
-// Enqueue one launch covering `jobs` (device operands).  Jobs with no rows are dropped.
-int enqueue_jobs(larql_hip_ctx *c, std::vector<GemvJob> &jobs) {
-    std::vector<GemvJob> live;
-    for (const GemvJob &j : jobs)
-        if (j.rows > 0) live.push_back(j);
-    if (live.empty()) return LARQL_OK;
-    for (const GemvJob &j : live) {
-        if (((uintptr_t)j.w & 15) || ((uintptr_t)j.x & 15))
-            return fail(c, LARQL_REFUSED_SHAPE, "matvec: weight and activation pointers must be 16-byte aligned");
-        if ((j.kind == KIND_Q8_0 || j.kind == KIND_Q4_0) && (j.k % 64) != 0)
-            return fail(c, LARQL_UNSUPPORTED, "matvec: this block format needs k %% 64 == 0 on this backend (k=%llu)",
-                        (unsigned long long)j.k);
-    }
+// One launch over jobs of a single format.
+int enqueue_same_kind(larql_hip_ctx *c, std::vector<GemvJob> &live, DevBuf &table_buf) {
+    const int kind = live[0].kind;
     const uint32_t threads = gemv_pick_threads(live.data(), live.size());
     if (threads == 0) return fail(c, LARQL_UNSUPPORTED, "matvec: row length not supported by the gfx950 kernels");
     uint64_t total = 0;
@@ -164,17 +154,43 @@ int enqueue_jobs(larql_hip_ctx *c, std::vector<GemvJob> &jobs) {
         for (size_t i = 0; i < live.size(); i++) L.inl[i] = live[i];
         L.table = nullptr;
     } else {
-        int rc = ensure(c, c->table, live.size() * sizeof(GemvJob));
+        int rc = ensure(c, table_buf, live.size() * sizeof(GemvJob));
         if (rc) return rc;
-        HIPCHECK(c, hipMemcpyAsync(c->table.p, live.data(), live.size() * sizeof(GemvJob), hipMemcpyHostToDevice, c->stream));
+        HIPCHECK(c, hipMemcpyAsync(table_buf.p, live.data(), live.size() * sizeof(GemvJob), hipMemcpyHostToDevice, c->stream));
         // the host vector dies with this call: make sure the copy has consumed it
         HIPCHECK(c, hipStreamSynchronize(c->stream));
-        L.table = (const GemvJob *)c->table.p;
+        L.table = (const GemvJob *)table_buf.p;
     }
     uint64_t grid = (uint64_t)c->cu_count * (uint64_t)c->wgs_per_cu;
     if (grid > total) grid = total;
     const size_t lds = gemv_lds_bytes(live.data(), live.size());
-    HIPCHECK(c, gemv_launch(c->stream, L, threads, (uint32_t)grid, lds));
+    HIPCHECK(c, gemv_launch(c->stream, kind, L, threads, (uint32_t)grid, lds));
+    return LARQL_OK;
+}
+
+// Enqueue `jobs` (device operands): one launch per format present, in first-seen
+// order.  Jobs with no rows are dropped.
+int enqueue_jobs(larql_hip_ctx *c, std::vector<GemvJob> &jobs) {
+    for (const GemvJob &j : jobs) {
+        if (j.rows == 0) continue;
+        if (((uintptr_t)j.w & 15) || ((uintptr_t)j.x & 15))
+            return fail(c, LARQL_REFUSED_SHAPE, "matvec: weight and activation pointers must be 16-byte aligned");
+        if ((j.kind == KIND_Q8_0 || j.kind == KIND_Q4_0) && (j.k % 64) != 0)
+            return fail(c, LARQL_UNSUPPORTED, "matvec: this block format needs k %% 64 == 0 on this backend (k=%llu)",
+                        (unsigned long long)j.k);
+    }
+    bool done[8] = {false, false, false, false, false, false, false, false};
+    int slot = 0;
+    for (size_t i = 0; i < jobs.size(); i++) {
+        const int kind = jobs[i].kind;
+        if (jobs[i].rows == 0 || kind < 0 || kind > 6 || done[kind]) continue;
+        done[kind] = true;
+        std::vector<GemvJob> live;
+        for (size_t t = i; t < jobs.size(); t++)
+            if (jobs[t].kind == kind && jobs[t].rows > 0) live.push_back(jobs[t]);
+        int rc = enqueue_same_kind(c, live, c->tables[slot++ % 4]);
+        if (rc) return rc;
+    }
     return LARQL_OK;
 }
 
@@ -245,7 +261,7 @@ void larql_hip_destroy(larql_hip_ctx *c) {
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     for (Region &r : c->regions) (void)hipFree(r.dev);
     DevBuf *bufs[] = {&c->w[0], &c->w[1], &c->w[2], &c->w[3], &c->aux[0], &c->aux[1], &c->aux[2], &c->aux[3],
-                      &c->x, &c->out, &c->table, &c->misc, &c->scores, &c->q8, &c->q8s};
+                      &c->x, &c->out, &c->tables[0], &c->tables[1], &c->tables[2], &c->tables[3], &c->misc, &c->scores, &c->q8, &c->q8s};
     for (DevBuf *b : bufs) if (b->p) (void)hipFree(b->p);
     if (c->log2_up) (void)hipFree(c->log2_up);
     if (c->nan_flag) (void)hipFree(c->nan_flag);
@@ -830,6 +846,16 @@ int larql_hip_dev_gate_knn(larql_hip_ctx *c, int format, const void *gate, const
     if (rc) return rc;
     HIPCHECK(c, topk_launch(c->stream, scores_scratch, (uint32_t)batch, (uint32_t)n, (uint32_t)top_k, true, idx_out, score_out,
                             (uint32_t *)c->misc.p, c->nan_flag, nullptr, 0));
+    return LARQL_OK;
+}
+
+int larql_hip_dev_copy(larql_hip_ctx *c, void *dst, const void *src, size_t bytes) {
+    if (!c || !src) return LARQL_E_ARG;
+    if (bytes % 16 != 0 || ((uintptr_t)src & 15) || ((uintptr_t)dst & 15)) return fail(c, LARQL_REFUSED_SHAPE, "copy: 16-byte granularity");
+    HIPCHECK(c, hipSetDevice(c->device));
+    const uint32_t grid = (uint32_t)c->cu_count * 8u;
+    if (dst) HIPCHECK(c, copy_launch(c->stream, src, dst, bytes, grid));
+    else { int rc = ensure(c, c->misc, 64); if (rc) return rc; HIPCHECK(c, read_launch(c->stream, src, (uint32_t *)c->misc.p, bytes, grid)); }
     return LARQL_OK;
 }
 

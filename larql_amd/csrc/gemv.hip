@@ -20,6 +20,7 @@
 // routine; only the summation order differs (fp32 accumulate throughout).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "kernels.h"
 
@@ -109,9 +110,8 @@ __device__ __forceinline__ float q4k_group_dot(const u32x4 hdr, const u32x4 q0, 
     const float dmin = half_bits_to_float(hdr.x >> 16);
     const uint32_t sh = (g & 1u) * 16u;
     const uint32_t a = (hdr.y >> sh) & 0xFFFFu, b = (hdr.z >> sh) & 0xFFFFu, c = (hdr.w >> sh) & 0xFFFFu;
-    uint32_t sc2, mn2;
-    if (g < 2) { sc2 = a & 0x3F3Fu; mn2 = b & 0x3F3Fu; }
-    else { sc2 = (c & 0x0F0Fu) | ((a >> 2) & 0x3030u); mn2 = ((c >> 4) & 0x0F0Fu) | ((b >> 2) & 0x3030u); }
+    const uint32_t sc_hi2 = (c & 0x0F0Fu) | ((a >> 2) & 0x3030u), mn_hi2 = ((c >> 4) & 0x0F0Fu) | ((b >> 2) & 0x3030u);
+    const uint32_t sc2 = g < 2 ? (a & 0x3F3Fu) : sc_hi2, mn2 = g < 2 ? (b & 0x3F3Fu) : mn_hi2;
     const float sc_lo = d * (float)(sc2 & 0xFFu), sc_hi = d * (float)(sc2 >> 8);
     const float mn_lo = dmin * (float)(mn2 & 0xFFu), mn_hi = dmin * (float)(mn2 >> 8);
     const float dot_lo = (alo0 + alo1) * 16777216.0f;  // * 2^24 (exact)
@@ -521,11 +521,11 @@ __device__ __forceinline__ void run_dense(const GemvJob &j, uint32_t p0, uint32_
 }
 
 // ---------------------------------------------------------------------------
-// The kernel: workgroup b sweeps passes [P*b/G, P*(b+1)/G) of the launch's
-// pass list, job by job.
+// The kernels, one per format so each gets its own register budget: workgroup
+// b sweeps passes [P*b/G, P*(b+1)/G) of the launch's pass list, job by job.
 // ---------------------------------------------------------------------------
-__global__ void __launch_bounds__(kGemvMaxThreads) gemv_kernel(GemvLaunch L) {
-    extern __shared__ float part[];
+template <int KIND, int U>
+__device__ __forceinline__ void gemv_body(const GemvLaunch &L, float *part) {
     const GemvJob *jobs = L.table ? L.table : L.inl;
     const uint64_t P = L.total_passes;
     uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
@@ -542,24 +542,41 @@ __global__ void __launch_bounds__(kGemvMaxThreads) gemv_kernel(GemvLaunch L) {
         const uint32_t jp_end = j.pass_begin + j.n_pass;
         const uint32_t seg_end = min(p_end, jp_end);
         const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin;
-        switch (j.kind) {
-            case KIND_Q4K: run_q4k<4>(j, a, b, part); break;
-            case KIND_Q8_0: run_q8_0<4>(j, a, b, part); break;
-            case KIND_MXFP4: run_mxfp4<4>(j, a, b, part); break;
-            case KIND_Q4_0: run_q4_0<4>(j, a, b, part); break;
-            case KIND_BF16: run_dense<4, 0>(j, a, b, part); break;
-            case KIND_F16: run_dense<4, 1>(j, a, b, part); break;
-            case KIND_F32: run_dense<2, 2>(j, a, b, part); break;
-            default: break;
-        }
+        if (KIND == KIND_Q4K) run_q4k<U>(j, a, b, part);
+        else if (KIND == KIND_Q8_0) run_q8_0<U>(j, a, b, part);
+        else if (KIND == KIND_MXFP4) run_mxfp4<U>(j, a, b, part);
+        else if (KIND == KIND_Q4_0) run_q4_0<U>(j, a, b, part);
+        else if (KIND == KIND_BF16) run_dense<U, 0>(j, a, b, part);
+        else if (KIND == KIND_F16) run_dense<U, 1>(j, a, b, part);
+        else run_dense<U, 2>(j, a, b, part);
         p = seg_end;
         ji++;
     }
 }
 
+#define LARQL_GEMV_KERNEL(NAME, KIND, U, WAVES)                                                                 \
+    __global__ void __launch_bounds__(kGemvMaxThreads) __attribute__((amdgpu_waves_per_eu(WAVES))) NAME(GemvLaunch L) { \
+        extern __shared__ float part[];                                                                         \
+        gemv_body<KIND, U>(L, part);                                                                            \
+    }
+LARQL_GEMV_KERNEL(gemv_q4k_u2_kernel, KIND_Q4K, 2, 4)
+LARQL_GEMV_KERNEL(gemv_q4k_u4_kernel, KIND_Q4K, 4, 3)
+LARQL_GEMV_KERNEL(gemv_q8_0_u2_kernel, KIND_Q8_0, 2, 4)
+LARQL_GEMV_KERNEL(gemv_q8_0_u4_kernel, KIND_Q8_0, 4, 3)
+LARQL_GEMV_KERNEL(gemv_mxfp4_u2_kernel, KIND_MXFP4, 2, 4)
+LARQL_GEMV_KERNEL(gemv_mxfp4_u4_kernel, KIND_MXFP4, 4, 4)
+LARQL_GEMV_KERNEL(gemv_q4_0_kernel, KIND_Q4_0, 4, 4)
+LARQL_GEMV_KERNEL(gemv_bf16_kernel, KIND_BF16, 4, 4)
+LARQL_GEMV_KERNEL(gemv_f16_kernel, KIND_F16, 4, 4)
+LARQL_GEMV_KERNEL(gemv_f32_kernel, KIND_F32, 2, 4)
+
+
 // ---------------------------------------------------------------------------
 // Host side: geometry and launch.
 // ---------------------------------------------------------------------------
+// experiment knobs (environment): passes in flight per thread, forced block size
+static int g_unroll = getenv("LARQL_HIP_UNROLL") ? atoi(getenv("LARQL_HIP_UNROLL")) : 0;  // 0: per-format default
+static int g_threads = getenv("LARQL_HIP_THREADS") ? atoi(getenv("LARQL_HIP_THREADS")) : 0;
 static uint32_t chunk_elems(int kind) {
     switch (kind) {
         case KIND_Q4K: return 64;
@@ -593,10 +610,14 @@ bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
 uint32_t gemv_pick_threads(const GemvJob *jobs, size_t n) {
     // Prefer the block size that wastes the fewest lanes over the jobs'
     // chunk counts (weighted by bytes); ties go to the smaller block.
-    static const uint32_t cand[] = {256, 320, 384, 448, 512};
+    static const uint32_t cand_all[] = {256, 320, 384, 448, 512};
+    const uint32_t forced[] = {(uint32_t)g_threads};
+    const uint32_t *cand = g_threads ? forced : cand_all;
+    const size_t n_cand = g_threads ? 1 : 5;
     double best = -1.0;
     uint32_t pick = 0;
-    for (uint32_t T : cand) {
+    for (size_t ci = 0; ci < n_cand; ci++) {
+        const uint32_t T = cand[ci];
         double used = 0.0, total = 0.0;
         bool ok = true;
         for (size_t i = 0; i < n; i++) {
@@ -623,8 +644,50 @@ size_t gemv_lds_bytes(const GemvJob *jobs, size_t n) {
     return m;
 }
 
-hipError_t gemv_launch(hipStream_t stream, const GemvLaunch &L, uint32_t threads, uint32_t grid, size_t lds) {
-    hipLaunchKernelGGL(gemv_kernel, dim3(grid), dim3(threads), lds, stream, L);
+hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32_t threads, uint32_t grid, size_t lds) {
+    switch (kind) {
+        case KIND_Q4K:
+            if (g_unroll != 4) hipLaunchKernelGGL(gemv_q4k_u2_kernel, dim3(grid), dim3(threads), lds, stream, L);
+            else hipLaunchKernelGGL(gemv_q4k_u4_kernel, dim3(grid), dim3(threads), lds, stream, L);
+            break;
+        case KIND_Q8_0:
+            if (g_unroll == 2) hipLaunchKernelGGL(gemv_q8_0_u2_kernel, dim3(grid), dim3(threads), lds, stream, L);
+            else hipLaunchKernelGGL(gemv_q8_0_u4_kernel, dim3(grid), dim3(threads), lds, stream, L);
+            break;
+        case KIND_MXFP4:
+            if (g_unroll == 2) hipLaunchKernelGGL(gemv_mxfp4_u2_kernel, dim3(grid), dim3(threads), lds, stream, L);
+            else hipLaunchKernelGGL(gemv_mxfp4_u4_kernel, dim3(grid), dim3(threads), lds, stream, L);
+            break;
+        case KIND_Q4_0: hipLaunchKernelGGL(gemv_q4_0_kernel, dim3(grid), dim3(threads), lds, stream, L); break;
+        case KIND_BF16: hipLaunchKernelGGL(gemv_bf16_kernel, dim3(grid), dim3(threads), lds, stream, L); break;
+        case KIND_F16: hipLaunchKernelGGL(gemv_f16_kernel, dim3(grid), dim3(threads), lds, stream, L); break;
+        case KIND_F32: hipLaunchKernelGGL(gemv_f32_kernel, dim3(grid), dim3(threads), lds, stream, L); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+// Plain streaming copy (one 16-byte load and store per thread per step): the
+// yardstick for achievable HBM bandwidth and for scaling profiler counters.
+__global__ void __launch_bounds__(256) copy_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst, size_t n_vec) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_vec; i += stride) dst[i] = src[i];
+}
+__global__ void __launch_bounds__(256) read_kernel(const u32x4 *__restrict__ src, uint32_t *__restrict__ sink, size_t n_vec) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    uint32_t acc = 0;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_vec; i += stride) {
+        const u32x4 v = src[i];
+        acc ^= v.x ^ v.y ^ v.z ^ v.w;
+    }
+    if (acc == 0x9E3779B9u) sink[0] = acc;  // keeps the loads alive; practically never true
+}
+hipError_t copy_launch(hipStream_t stream, const void *src, void *dst, size_t bytes, uint32_t grid) {
+    if (dst) hipLaunchKernelGGL(copy_kernel, dim3(grid), dim3(256), 0, stream, (const u32x4 *)src, (u32x4 *)dst, bytes / 16);
+    return hipGetLastError();
+}
+hipError_t read_launch(hipStream_t stream, const void *src, uint32_t *sink, size_t bytes, uint32_t grid) {
+    hipLaunchKernelGGL(read_kernel, dim3(grid), dim3(256), 0, stream, (const u32x4 *)src, sink, bytes / 16);
     return hipGetLastError();
 }
 

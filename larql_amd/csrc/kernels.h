@@ -41,7 +41,9 @@ struct GemvLaunch {
 bool gemv_job_geometry(GemvJob &j, uint32_t threads);
 uint32_t gemv_pick_threads(const GemvJob *jobs, size_t n);
 size_t gemv_lds_bytes(const GemvJob *jobs, size_t n);
-hipError_t gemv_launch(hipStream_t stream, const GemvLaunch &L, uint32_t threads, uint32_t grid, size_t lds);
+hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32_t threads, uint32_t grid, size_t lds);
+hipError_t copy_launch(hipStream_t stream, const void *src, void *dst, size_t bytes, uint32_t grid);
+hipError_t read_launch(hipStream_t stream, const void *src, uint32_t *sink, size_t bytes, uint32_t grid);
 
 // top-K by |score| (or by value) over rows of a [batch, n] score matrix
 hipError_t topk_launch(hipStream_t stream, const float *scores, uint32_t batch, uint32_t n, uint32_t k,
