@@ -1,0 +1,223 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantised decode matvec stack on one MI355X.
+
+Workload (BASELINE.json configs[1]): the full decode-step matvec stack at
+Gemma-3-4B shapes, batch 1 — per layer q 2048x2560, k/v 1024x2560, o 2560x2048,
+gate/up 10240x2560, down 2560x10240 in Q4_K, 34 distinct layers, then the
+lm_head 262144x2560 in ggml Q8_0.  Weights are N(0, 0.02) drawn on the device
+from a seeded counter generator and quantised on the device with the
+reference's encoders (bit-exact kernels); every matvec has its own N(0, 1)
+activation.  One step = one token = all 239 matvecs, submitted as two recorded
+launches (238 Q4_K jobs, 1 Q8_0 job); inputs are resident in HBM before the
+timed region.
+
+Prints ONE JSON line: whole-job HBM throughput in GB/s over the algorithmic
+bytes (weight bytes + 4*K + 4*N per matvec), plus `roofline` for the dominant
+kernel (Q4_K matvec, timed with HIP events on the launch stream inside the timed
+region) and `cpu_baseline` (the CPU oracle's restatement of the reference
+kernels, multi-threaded, on a bounded sample of the same weights).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HIDDEN, LAYERS, VOCAB = 2560, 34, 262144
+# (name, rows, k) in trait orientation [num_rows, hidden]
+LAYER_MATS = [("q", 2048, 2560), ("k", 1024, 2560), ("v", 1024, 2560), ("o", 2560, 2048),
+              ("gate", 10240, 2560), ("up", 10240, 2560), ("down", 2560, 10240)]
+HBM_PEAK_GBS = 8000.0
+CONFIG_ID = 2  # seeds: 0x5EED0000 + config*256 + tensor_id (mod 2^32 per layer below)
+
+
+def q4k_bytes(rows, k):
+    return rows * (k // 256) * 144
+
+
+def q8_0_bytes(rows, k):
+    return rows * (k // 32) * 34
+
+
+class Stack:
+    """Device-resident weights, activations and outputs of the whole stack."""
+
+    def __init__(self, be, fmt, layers=LAYERS, vocab=VOCAB):
+        self.be, self.fmt = be, fmt
+        self.q4k_jobs, self.q8_jobs, self.meta = [], [], []
+        tmp_elems = max(vocab * HIDDEN, 10240 * 2560)
+        tmp = be.malloc(tmp_elems * 4)
+        tid = 0
+        for layer in range(layers):
+            for name, rows, k in LAYER_MATS:
+                seed = 0x5EED0000 + CONFIG_ID * 256 + tid
+                tid += 1
+                w = be.malloc(q4k_bytes(rows, k) + 64)
+                assert be.dev_fill_normal(tmp, rows * k, seed, 0.02)
+                assert be.dev_quantize_q4_k(tmp, rows * k, w)
+                x = be.malloc(k * 4 + 64)
+                assert be.dev_fill_normal(x, k, seed ^ 0xA5A50000, 1.0)
+                out = be.malloc(rows * 4 + 64)
+                self.q4k_jobs.append((fmt.FMT_Q4_K, w, None, x, out, rows, k))
+                self.meta.append((f"L{layer}.{name}", "q4k", rows, k))
+        seed = 0x5EED0000 + CONFIG_ID * 256 + 0xFFFF
+        w = be.malloc(q8_0_bytes(vocab, HIDDEN) + 64)
+        assert be.dev_fill_normal(tmp, vocab * HIDDEN, seed, 0.02)
+        assert be.dev_quantize_q8_0(tmp, vocab * HIDDEN, w)
+        x = be.malloc(HIDDEN * 4 + 64)
+        assert be.dev_fill_normal(x, HIDDEN, seed ^ 0xA5A50000, 1.0)
+        out = be.malloc(vocab * 4 + 64)
+        self.q8_jobs.append((fmt.FMT_GGML_Q8_0, w, None, x, out, vocab, HIDDEN))
+        be.synchronize()
+        be.free(tmp)
+        self.q4k_weight_bytes = sum(q4k_bytes(r, k) for (_, _, _, _, _, r, k) in self.q4k_jobs)
+        self.q8_weight_bytes = q8_0_bytes(vocab, HIDDEN)
+        self.q4k_algo_bytes = self.q4k_weight_bytes + sum(4 * k + 4 * r for (_, _, _, _, _, r, k) in self.q4k_jobs)
+        self.q8_algo_bytes = self.q8_weight_bytes + 4 * HIDDEN + 4 * vocab
+        self.plan_q4k = be.plan_create(self.q4k_jobs)
+        self.plan_q8 = be.plan_create(self.q8_jobs)
+        assert self.plan_q4k and self.plan_q8, be.last_error()
+
+    def step(self):
+        self.be.plan_run(self.plan_q4k)
+        self.be.plan_run(self.plan_q8)
+
+
+def verify_and_cpu_baseline(be, stack, lm_rows=16384, min_seconds=10.0):
+    """Check the GPU outputs of a sample (layer 0 + the first lm_head rows) against the CPU
+    oracle, then time the oracle (the reference's CPU algorithm restated, row-chunk
+    threaded as the reference schedules it) on the same sample."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import oracle as O  # the checker; never the thing measured as the product
+
+    threads = min(16, len(os.sched_getaffinity(0)))
+    sample, worst = [], 0.0
+    for (f, w, _, x, out, rows, k), (name, kind, _, _) in zip(stack.q4k_jobs[:7], stack.meta[:7]):
+        wb = be.d2h(w, q4k_bytes(rows, k), np.uint8)
+        xv = be.d2h(x, k, np.float32)
+        got = be.d2h(out, rows, np.float32)
+        want = O.q4k_matvec_mt(wb, xv, rows, k, threads)
+        worst = max(worst, float(np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want)))
+        sample.append(("q4k", wb, xv, rows, k))
+    (f, w, _, x, out, rows, k) = stack.q8_jobs[0]
+    lm_rows = min(lm_rows, rows)
+    wb = be.d2h(w, q8_0_bytes(lm_rows, k), np.uint8)
+    xv = be.d2h(x, k, np.float32)
+    got = be.d2h(out, lm_rows, np.float32)
+    want = O.q8_0_gemv_mt(wb, xv, lm_rows, k, threads)
+    worst = max(worst, float(np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want)))
+    sample.append(("q8", wb, xv, lm_rows, k))
+    if not worst < 1e-3:
+        raise SystemExit(f"bench: GPU outputs differ from the CPU oracle (rel-L2 {worst:.3e}); no number recorded")
+
+    sample_bytes = sum(s[1].nbytes for s in sample)
+
+    def one_pass():
+        for kind, wb, xv, rows, k in sample:
+            (O.q4k_matvec_mt if kind == "q4k" else O.q8_0_gemv_mt)(wb, xv, rows, k, threads)
+
+    one_pass()
+    times = []
+    t_end = time.perf_counter() + min_seconds
+    while time.perf_counter() < t_end or len(times) < 5:
+        t0 = time.perf_counter()
+        one_pass()
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    return worst, {
+        "value": round(sample_bytes / med / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": f"layer 0 (7 Q4_K matvecs) + first {lm_rows} lm_head rows (Q8_0), {sample_bytes / 1e6:.1f} MB, "
+                  f"median of {len(times)} passes",
+        "tokens_per_s_extrapolated": round(1.0 / (med * (stack.q4k_weight_bytes + stack.q8_weight_bytes) / sample_bytes), 3),
+    }
+
+
+def read_traffic():
+    """HBM bytes per launch of the dominant kernel from the committed rocprof PMC summary, if any."""
+    path = os.path.join(ROOT, "profiles", "gemv_q4k_c2_stack.pmc.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return float(line.split(":", 1)[1].split()[0])
+    except OSError:
+        pass
+    return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
+    ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path runs on ONE GPU; --gpus above 1 is not part of this build "
+              "(sharding is by weight rows, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    import larql_amd as fmt
+    be = fmt.HipBackend()
+    stack = Stack(be, fmt, layers=args.layers)
+
+    stack.step()
+    be.synchronize()
+    if args.no_cpu:
+        worst, cpu = None, None
+    else:
+        worst, cpu = verify_and_cpu_baseline(be, stack, min_seconds=args.cpu_seconds)
+
+    for _ in range(args.warmup):
+        stack.step()
+    be.synchronize()
+    ev = [(be.event(), be.event(), be.event()) for _ in range(args.steps)]
+    be.synchronize()
+    t0 = time.perf_counter()
+    for a, b, c in ev:
+        be.record(a)
+        be.plan_run(stack.plan_q4k)
+        be.record(b)
+        be.plan_run(stack.plan_q8)
+        be.record(c)
+    be.synchronize()
+    t1 = time.perf_counter()
+
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    q4k_ms = float(np.mean([be.elapsed_ms(a, b) for a, b, _ in ev]))
+    q8_ms = float(np.mean([be.elapsed_ms(b, c) for _, b, c in ev]))
+    algo_bytes = stack.q4k_algo_bytes + stack.q8_algo_bytes
+    value = algo_bytes / (ms_per_step * 1e-3) / 1e9
+    achieved = stack.q4k_algo_bytes / (q4k_ms * 1e-3) / 1e9
+    out = {
+        "metric": "Q4_K/Q8_0 decode matvec stack HBM GB/s", "value": round(value, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {
+            "workload": "BASELINE configs[1]: Gemma-3-4B decode matvec stack, batch 1, "
+                        f"{args.layers} layers x 7 Q4_K matvecs + Q8_0 lm_head 262144x2560",
+            "matvecs_per_step": len(stack.q4k_jobs) + 1, "launches_per_step": 2,
+            "algorithmic_bytes_per_step": algo_bytes, "tokens_per_s": round(1e3 / ms_per_step, 1),
+            "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+            "q8_0_lm_head": {"ms": round(q8_ms, 4), "GB/s": round(stack.q8_algo_bytes / (q8_ms * 1e-3) / 1e9, 1)},
+            "verified_rel_l2_vs_oracle": worst,
+        },
+        "roofline": {"kernel": "gemv_q4k (238 Q4_K matvecs, one launch)", "bound": "hbm", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "launch_ms": round(q4k_ms, 4), "algorithmic_bytes_per_launch": stack.q4k_algo_bytes,
+                     "traffic": read_traffic()},
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -227,6 +227,18 @@ typedef struct {
 } larql_hip_matvec_job;
 int larql_hip_dev_matvec_batch(larql_hip_ctx *ctx, const larql_hip_matvec_job *jobs, size_t n_jobs);
 
+/* A recorded submission: the jobs' geometry and device job tables are
+ * prepared once, and every run enqueues the same launches (one per format
+ * present) on the context's stream without synchronising — what the Metal
+ * peer's decode command buffer is to its per-call matvecs
+ * (larql-compute-metal backend/decode.rs:338).  Operand pointers are captured
+ * by value; the buffers may be rewritten between runs. */
+typedef struct larql_hip_plan larql_hip_plan;
+int  larql_hip_plan_create(larql_hip_ctx *ctx, const larql_hip_matvec_job *jobs, size_t n_jobs, larql_hip_plan **out);
+int  larql_hip_plan_run(larql_hip_ctx *ctx, larql_hip_plan *plan);
+int  larql_hip_plan_launch_count(const larql_hip_plan *plan);
+void larql_hip_plan_destroy(larql_hip_ctx *ctx, larql_hip_plan *plan);
+
 /* Scores + top-K by |score| on resident operands (see larql_hip_gate_knn).
  * scores_scratch: [batch, n_features] f32 device buffer (also the full score
  * matrix on return); idx_out/score_out: [batch, top_k] device buffers. */

@@ -73,6 +73,10 @@ SIGNATURES = {
     "larql_hip_dev_copy": (ci, [vp, vp, vp, sz]),
     "larql_hip_dev_matvec": (ci, [vp, ci, vp, vp, vp, sz, sz, vp]),
     "larql_hip_dev_matvec_batch": (ci, [vp, C.POINTER(MatvecJob), sz]),
+    "larql_hip_plan_create": (ci, [vp, C.POINTER(MatvecJob), sz, C.POINTER(vp)]),
+    "larql_hip_plan_run": (ci, [vp, vp]),
+    "larql_hip_plan_launch_count": (ci, [vp]),
+    "larql_hip_plan_destroy": (None, [vp, vp]),
     "larql_hip_dev_gate_knn": (ci, [vp, ci, vp, vp, sz, sz, sz, sz, vp, vp, vp]),
     "larql_hip_dev_quantize_q4_k": (ci, [vp, vp, sz, vp]),
     "larql_hip_dev_quantize_q8_0": (ci, [vp, vp, sz, vp]),

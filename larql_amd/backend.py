@@ -303,6 +303,24 @@ class HipBackend:
             arr[i] = L.MatvecJob(fmt, 0, w, aux, x, out, rows, k)
         return self._some(lib.larql_hip_dev_matvec_batch(self._h, arr, len(jobs)))
 
+    def plan_create(self, jobs: Sequence[tuple]) -> Optional[int]:
+        """Record a submission of (fmt, w, aux, x, out, rows, k) jobs; returns a plan handle or None."""
+        arr = (L.MatvecJob * max(len(jobs), 1))()
+        for i, (fmt, w, aux, x, out, rows, k) in enumerate(jobs):
+            arr[i] = L.MatvecJob(fmt, 0, w, aux, x, out, rows, k)
+        p = C.c_void_p()
+        ok = self._some(lib.larql_hip_plan_create(self._h, arr, len(jobs), C.byref(p)))
+        return p.value if ok else None
+
+    def plan_run(self, plan: int) -> bool:
+        return self._some(lib.larql_hip_plan_run(self._h, plan))
+
+    def plan_launch_count(self, plan: int) -> int:
+        return lib.larql_hip_plan_launch_count(plan)
+
+    def plan_destroy(self, plan: int) -> None:
+        lib.larql_hip_plan_destroy(self._h, plan)
+
     def dev_gate_knn(self, fmt: int, gate: int, x: int, batch: int, n: int, hidden: int, top_k: int, scores: int, idx: int,
                      val: int) -> bool:
         return self._some(lib.larql_hip_dev_gate_knn(self._h, fmt, gate, x, batch, n, hidden, top_k, scores, idx, val))

@@ -134,43 +134,46 @@ int kind_of_format(int format) {
     }
 }
 
-// One launch over jobs of a single format.
-int enqueue_same_kind(larql_hip_ctx *c, std::vector<GemvJob> &live, DevBuf &table_buf) {
-    const int kind = live[0].kind;
-    const uint32_t threads = gemv_pick_threads(live.data(), live.size());
-    if (threads == 0) return fail(c, LARQL_UNSUPPORTED, "matvec: row length not supported by the gfx950 kernels");
+struct PreparedLaunch {
+    int kind;
+    GemvLaunch L;
+    uint32_t threads, grid;
+    size_t lds;
+    void *table = nullptr;  // owned device table when the jobs do not fit inline (plans only)
+};
+
+// Geometry for one launch over jobs of a single format.  When the jobs do not fit
+// inline the table is uploaded into `table_dst` (synchronously: the host vector may die).
+int prepare_same_kind(larql_hip_ctx *c, std::vector<GemvJob> &live, void *table_dst, PreparedLaunch &P) {
+    P.kind = live[0].kind;
+    P.threads = gemv_pick_threads(live.data(), live.size());
+    if (P.threads == 0) return fail(c, LARQL_UNSUPPORTED, "matvec: row length not supported by the gfx950 kernels");
     uint64_t total = 0;
     for (GemvJob &j : live) {
-        if (!gemv_job_geometry(j, threads)) return fail(c, LARQL_UNSUPPORTED, "matvec: unsupported geometry");
+        if (!gemv_job_geometry(j, P.threads)) return fail(c, LARQL_UNSUPPORTED, "matvec: unsupported geometry");
         if (total + j.n_pass > 0x7FFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "matvec: launch too large");
         j.pass_begin = (uint32_t)total;
         total += j.n_pass;
     }
-    GemvLaunch L;
-    memset(&L, 0, sizeof L);
-    L.total_passes = total;
-    L.n_jobs = (uint32_t)live.size();
+    memset(&P.L, 0, sizeof P.L);
+    P.L.total_passes = total;
+    P.L.n_jobs = (uint32_t)live.size();
     if (live.size() <= (size_t)kInlineJobs) {
-        for (size_t i = 0; i < live.size(); i++) L.inl[i] = live[i];
-        L.table = nullptr;
+        for (size_t i = 0; i < live.size(); i++) P.L.inl[i] = live[i];
+        P.L.table = nullptr;
     } else {
-        int rc = ensure(c, table_buf, live.size() * sizeof(GemvJob));
-        if (rc) return rc;
-        HIPCHECK(c, hipMemcpyAsync(table_buf.p, live.data(), live.size() * sizeof(GemvJob), hipMemcpyHostToDevice, c->stream));
-        // the host vector dies with this call: make sure the copy has consumed it
+        HIPCHECK(c, hipMemcpyAsync(table_dst, live.data(), live.size() * sizeof(GemvJob), hipMemcpyHostToDevice, c->stream));
         HIPCHECK(c, hipStreamSynchronize(c->stream));
-        L.table = (const GemvJob *)table_buf.p;
+        P.L.table = (const GemvJob *)table_dst;
     }
     uint64_t grid = (uint64_t)c->cu_count * (uint64_t)c->wgs_per_cu;
     if (grid > total) grid = total;
-    const size_t lds = gemv_lds_bytes(live.data(), live.size());
-    HIPCHECK(c, gemv_launch(c->stream, kind, L, threads, (uint32_t)grid, lds));
+    P.grid = (uint32_t)grid;
+    P.lds = gemv_lds_bytes(live.data(), live.size());
     return LARQL_OK;
 }
 
-// Enqueue `jobs` (device operands): one launch per format present, in first-seen
-// order.  Jobs with no rows are dropped.
-int enqueue_jobs(larql_hip_ctx *c, std::vector<GemvJob> &jobs) {
+int check_jobs(larql_hip_ctx *c, const std::vector<GemvJob> &jobs) {
     for (const GemvJob &j : jobs) {
         if (j.rows == 0) continue;
         if (((uintptr_t)j.w & 15) || ((uintptr_t)j.x & 15))
@@ -179,8 +182,13 @@ int enqueue_jobs(larql_hip_ctx *c, std::vector<GemvJob> &jobs) {
             return fail(c, LARQL_UNSUPPORTED, "matvec: this block format needs k %% 64 == 0 on this backend (k=%llu)",
                         (unsigned long long)j.k);
     }
+    return LARQL_OK;
+}
+
+// Split jobs into one group per format present, in first-seen order.
+std::vector<std::vector<GemvJob>> group_by_kind(const std::vector<GemvJob> &jobs) {
+    std::vector<std::vector<GemvJob>> groups;
     bool done[8] = {false, false, false, false, false, false, false, false};
-    int slot = 0;
     for (size_t i = 0; i < jobs.size(); i++) {
         const int kind = jobs[i].kind;
         if (jobs[i].rows == 0 || kind < 0 || kind > 6 || done[kind]) continue;
@@ -188,8 +196,24 @@ int enqueue_jobs(larql_hip_ctx *c, std::vector<GemvJob> &jobs) {
         std::vector<GemvJob> live;
         for (size_t t = i; t < jobs.size(); t++)
             if (jobs[t].kind == kind && jobs[t].rows > 0) live.push_back(jobs[t]);
-        int rc = enqueue_same_kind(c, live, c->tables[slot++ % 4]);
+        groups.push_back(live);
+    }
+    return groups;
+}
+
+// Enqueue `jobs` (device operands): one launch per format present, in first-seen
+// order.  Jobs with no rows are dropped.
+int enqueue_jobs(larql_hip_ctx *c, std::vector<GemvJob> &jobs) {
+    int rc = check_jobs(c, jobs);
+    if (rc) return rc;
+    int slot = 0;
+    for (std::vector<GemvJob> &live : group_by_kind(jobs)) {
+        DevBuf &tb = c->tables[slot++ % 4];
+        if (live.size() > (size_t)kInlineJobs) { rc = ensure(c, tb, live.size() * sizeof(GemvJob)); if (rc) return rc; }
+        PreparedLaunch P;
+        rc = prepare_same_kind(c, live, tb.p, P);
         if (rc) return rc;
+        HIPCHECK(c, gemv_launch(c->stream, P.kind, P.L, P.threads, P.grid, P.lds));
     }
     return LARQL_OK;
 }
@@ -810,6 +834,62 @@ int larql_hip_dev_matvec_batch(larql_hip_ctx *c, const larql_hip_matvec_job *pj,
         if (rc) return rc;
     }
     return enqueue_jobs(c, jobs);
+}
+
+struct larql_hip_plan {
+    std::vector<PreparedLaunch> launches;
+};
+
+int larql_hip_plan_create(larql_hip_ctx *c, const larql_hip_matvec_job *pj, size_t n_jobs, larql_hip_plan **out) {
+    if (!c || !out || (!pj && n_jobs)) return LARQL_E_ARG;
+    *out = nullptr;
+    std::lock_guard<std::mutex> lk(c->mu);
+    HIPCHECK(c, hipSetDevice(c->device));
+    std::vector<GemvJob> jobs;
+    for (size_t i = 0; i < n_jobs; i++) {
+        int rc = dev_job_from_public(c, pj[i], jobs);
+        if (rc) return rc;
+    }
+    int rc = check_jobs(c, jobs);
+    if (rc) return rc;
+    larql_hip_plan *plan = new larql_hip_plan();
+    for (std::vector<GemvJob> &live : group_by_kind(jobs)) {
+        PreparedLaunch P;
+        if (live.size() > (size_t)kInlineJobs) {
+            if (hipMalloc(&P.table, live.size() * sizeof(GemvJob)) != hipSuccess) {
+                for (PreparedLaunch &q : plan->launches) if (q.table) (void)hipFree(q.table);
+                delete plan;
+                return fail(c, LARQL_E_DEVICE, "plan: out of device memory");
+            }
+        }
+        rc = prepare_same_kind(c, live, P.table, P);
+        if (rc) {
+            if (P.table) (void)hipFree(P.table);
+            for (PreparedLaunch &q : plan->launches) if (q.table) (void)hipFree(q.table);
+            delete plan;
+            return rc;
+        }
+        plan->launches.push_back(P);
+    }
+    *out = plan;
+    return LARQL_OK;
+}
+
+int larql_hip_plan_run(larql_hip_ctx *c, larql_hip_plan *plan) {
+    if (!c || !plan) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    HIPCHECK(c, hipSetDevice(c->device));
+    for (const PreparedLaunch &P : plan->launches) HIPCHECK(c, gemv_launch(c->stream, P.kind, P.L, P.threads, P.grid, P.lds));
+    return LARQL_OK;
+}
+
+int larql_hip_plan_launch_count(const larql_hip_plan *plan) { return plan ? (int)plan->launches.size() : 0; }
+
+void larql_hip_plan_destroy(larql_hip_ctx *c, larql_hip_plan *plan) {
+    if (!plan) return;
+    if (c) { (void)hipSetDevice(c->device); (void)hipStreamSynchronize(c->stream); }
+    for (PreparedLaunch &P : plan->launches) if (P.table) (void)hipFree(P.table);
+    delete plan;
 }
 
 int larql_hip_dev_matvec(larql_hip_ctx *c, int format, const void *w, const void *aux, const float *x, size_t rows, size_t k,

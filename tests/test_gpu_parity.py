@@ -364,3 +364,43 @@ def test_dev_matvec_batch_mixed_formats(be, fmt):
     assert be.dev_matvec(f, dw, None, x, rows, k, do)
     be.synchronize()
     assert np.array_equal(first.view(np.uint32), be.d2h(do, rows, F).view(np.uint32))
+
+
+def test_recorded_plan_replays_and_matches_direct_launches(be, fmt):
+    rng = np.random.default_rng(47)
+    x_h = rng.standard_normal(2560).astype(F)
+    x = be.to_device(x_h)
+    jobs, wants = [], []
+    for i, (rows, kind) in enumerate([(300, "q4k"), (64, "q4k"), (500, "q8"), (1000, "q4k"), (17, "q4k"), (9, "q4k")]):
+        w = (rng.standard_normal((rows, 2560)) * 0.02).astype(F)
+        if kind == "q4k":
+            q, f, want = O.quantize_q4_k(w), fmt.FMT_Q4_K, None
+            want = O.q4k_matvec(q, x_h, rows, 2560)
+        else:
+            q, f = O.quantize_q8_0(w), fmt.FMT_GGML_Q8_0
+            want = O.q8_0_gemv(q, x_h, rows, 2560)
+        jobs.append((f, be.to_device(q), None, x, be.malloc(rows * 4), rows, 2560)); wants.append(want)
+    plan = be.plan_create(jobs)
+    assert plan and be.plan_launch_count(plan) == 2
+    outs = []
+    for rep in range(3):                                       # replays give the same bits
+        for j in jobs:
+            be.h2d(j[4], np.zeros(j[5], F))
+        assert be.plan_run(plan)
+        be.synchronize()
+        outs.append([be.d2h(j[4], j[5], F) for j in jobs])
+    for got, want in zip(outs[0], wants):
+        assert rel_l2(got, want) < TOL
+    for rep in (1, 2):
+        for a, b in zip(outs[0], outs[rep]):
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    be.plan_destroy(plan)
+
+
+def test_cpp_host_mirror():
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "larql_amd", "host", "host_test")
+    assert os.path.exists(exe), "larql_amd/host/host_test is not built (run __graft_entry__.build())"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0 and "host_test ok" in r.stdout, r.stdout + r.stderr
