@@ -159,6 +159,9 @@ def main():
     ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="only run the plain 16-byte copy kernel on 1 GiB three times (known size, for scaling "
+                         "profiler byte counters) and print its bandwidth")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on ONE GPU; --gpus above 1 is not part of this build "
@@ -167,6 +170,26 @@ def main():
 
     import larql_amd as fmt
     be = fmt.HipBackend()
+    if args.copy_probe:
+        n = 1 << 30
+        a, b = be.malloc(n + 64), be.malloc(n + 64)
+        be.dev_fill_normal(a, n // 4, 1, 1.0)
+        be.dev_copy(b, a, n)
+        e0, e1 = be.event(), be.event()
+        be.record(e0)
+        for _ in range(3):
+            be.dev_copy(b, a, n)
+        be.record(e1)
+        ms = be.elapsed_ms(e0, e1) / 3
+        e2, e3 = be.event(), be.event()
+        be.record(e2)
+        for _ in range(3):
+            be.dev_copy(None, a, n)
+        be.record(e3)
+        ms_r = be.elapsed_ms(e2, e3) / 3
+        print(json.dumps({"copy_bytes": n, "copy_GBps_read_plus_write": round(2 * n / ms / 1e6, 1),
+                          "read_only_GBps": round(n / ms_r / 1e6, 1)}))
+        return
     stack = Stack(be, fmt, layers=args.layers)
 
     stack.step()

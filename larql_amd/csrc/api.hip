@@ -249,7 +249,7 @@ int larql_hip_create(larql_hip_ctx **out, int device) {
     char buf[256];
     snprintf(buf, sizeof buf, "hip (gfx950 matvec + gate-KNN kernels)");
     c->name = buf;
-    snprintf(buf, sizeof buf, "%s, %d CUs, %.0f GiB HBM, %s", prop.name, prop.multiProcessorCount,
+    snprintf(buf, sizeof buf, "%s, %d CUs, %.0f GiB HBM, %s", prop.name[0] ? prop.name : "AMD Instinct (gfx950)", prop.multiProcessorCount,
              (double)prop.totalGlobalMem / (1024.0 * 1024.0 * 1024.0), prop.gcnArchName);
     c->info = buf;
     if (hipStreamCreate(&c->stream) != hipSuccess || hipEventCreate(&c->ev0) != hipSuccess ||
