@@ -246,6 +246,32 @@ int larql_hip_dev_gate_knn(larql_hip_ctx *ctx, int format, const void *gate,
                            const float *x, size_t batch, size_t n_features, size_t hidden,
                            size_t top_k, float *scores_scratch, uint32_t *idx_out, float *score_out);
 
+/* ---- device tier: MoE expert block (MXFP4) --------------------------------------
+ * router::select — larql-compute/src/ffn/expert_weight/router.rs:33-70: top-k
+ * of `n_experts` logits per token (ties: first index), weights softmaxed over
+ * the selected logits (policy 1, NormalisedOverSelected: GPT-OSS) or over all
+ * experts (policy 0, SoftmaxThenSelect).  experts/weights are [tokens, k].
+ * n_experts <= 64, k <= 8. */
+int larql_hip_dev_router_select(larql_hip_ctx *ctx, const float *logits, size_t tokens, size_t n_experts, size_t k,
+                                int policy, uint32_t *experts, float *weights);
+/* One bank of MXFP4 experts: gate/up are [n_experts, inter, hidden] and down is
+ * [n_experts, hidden, inter], each as packed nibbles + e8m0 scales (the layout
+ * of MatMul::mxfp4_gemv, backend/matmul.rs:220-235, expert after expert). */
+typedef struct {
+    const uint8_t *gate_packed, *gate_scales, *up_packed, *up_scales, *down_packed, *down_scales;
+    size_t n_experts, hidden, inter;
+    float limit, alpha; /* MoeGateRule::ClampedGlu — pipeline/moe.rs:88-92 (GPT-OSS: 7, 1.702) */
+} larql_hip_mxfp4_experts;
+/* The expert block of cpu_moe_forward (cpu/ops/moe/forward.rs:201-270) for
+ * MXFP4 banks, which the CPU tier refuses (forward.rs:69-75): per token and
+ * selected expert, gate/up matvec -> ClampedGlu -> down matvec, then the
+ * weighted sum in selection order.  `experts` stays on the device (the kernels
+ * index the bank with it), so routing needs no host round trip.  Five launches.
+ * workspace: larql_hip_moe_mxfp4_workspace_bytes(...) of device memory. */
+size_t larql_hip_moe_mxfp4_workspace_bytes(size_t tokens, size_t k, size_t hidden, size_t inter);
+int larql_hip_dev_moe_mxfp4(larql_hip_ctx *ctx, const larql_hip_mxfp4_experts *bank, const float *x, size_t tokens, size_t k,
+                            const uint32_t *experts, const float *weights, float *out, void *workspace, size_t workspace_bytes);
+
 /* ---- device tier: encoders (bit-exact with the reference's host encoders) --- */
 /* quantize_q4_k — larql-compute/src/cpu/ops/q4_common/quantize.rs:89-189. */
 int larql_hip_dev_quantize_q4_k(larql_hip_ctx *ctx, const float *src, size_t n, uint8_t *dst);

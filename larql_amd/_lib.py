@@ -27,6 +27,12 @@ class SubmissionClock(C.Structure):
     _fields_ = [("submissions", u64), ("commit_to_done_nanos", u64), ("gpu_nanos", u64)]
 
 
+class Mxfp4Experts(C.Structure):
+    _fields_ = [("gate_packed", vp), ("gate_scales", vp), ("up_packed", vp), ("up_scales", vp), ("down_packed", vp),
+                ("down_scales", vp), ("n_experts", sz), ("hidden", sz), ("inter", sz), ("limit", C.c_float),
+                ("alpha", C.c_float)]
+
+
 class MatvecJob(C.Structure):
     _fields_ = [("format", C.c_int32), ("reserved", C.c_int32), ("w", vp), ("aux", vp), ("x", vp),
                 ("out", vp), ("rows", u64), ("k", u64)]
@@ -78,6 +84,9 @@ SIGNATURES = {
     "larql_hip_plan_launch_count": (ci, [vp]),
     "larql_hip_plan_destroy": (None, [vp, vp]),
     "larql_hip_dev_gate_knn": (ci, [vp, ci, vp, vp, sz, sz, sz, sz, vp, vp, vp]),
+    "larql_hip_dev_router_select": (ci, [vp, vp, sz, sz, sz, ci, vp, vp]),
+    "larql_hip_moe_mxfp4_workspace_bytes": (sz, [sz, sz, sz, sz]),
+    "larql_hip_dev_moe_mxfp4": (ci, [vp, C.POINTER(Mxfp4Experts), vp, sz, sz, vp, vp, vp, vp, sz]),
     "larql_hip_dev_quantize_q4_k": (ci, [vp, vp, sz, vp]),
     "larql_hip_dev_quantize_q8_0": (ci, [vp, vp, sz, vp]),
     "larql_hip_dev_quantize_mxfp4": (ci, [vp, vp, sz, sz, vp, vp]),

@@ -325,6 +325,17 @@ class HipBackend:
                      val: int) -> bool:
         return self._some(lib.larql_hip_dev_gate_knn(self._h, fmt, gate, x, batch, n, hidden, top_k, scores, idx, val))
 
+    def dev_router_select(self, logits: int, tokens: int, n_experts: int, k: int, policy: int, experts: int, weights: int) -> bool:
+        return self._some(lib.larql_hip_dev_router_select(self._h, logits, tokens, n_experts, k, policy, experts, weights))
+
+    def moe_mxfp4_workspace_bytes(self, tokens: int, k: int, hidden: int, inter: int) -> int:
+        return lib.larql_hip_moe_mxfp4_workspace_bytes(tokens, k, hidden, inter)
+
+    def dev_moe_mxfp4(self, bank: "L.Mxfp4Experts", x: int, tokens: int, k: int, experts: int, weights: int, out: int,
+                      workspace: int, workspace_bytes: int) -> bool:
+        return self._some(lib.larql_hip_dev_moe_mxfp4(self._h, C.byref(bank), x, tokens, k, experts, weights, out, workspace,
+                                                      workspace_bytes))
+
     def dev_quantize_q4_k(self, src: int, n: int, dst: int) -> bool:
         return self._some(lib.larql_hip_dev_quantize_q4_k(self._h, src, n, dst))
 

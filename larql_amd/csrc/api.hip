@@ -939,6 +939,64 @@ int larql_hip_dev_copy(larql_hip_ctx *c, void *dst, const void *src, size_t byte
     return LARQL_OK;
 }
 
+// ---- device tier: MoE -------------------------------------------------------------------------
+
+int larql_hip_dev_router_select(larql_hip_ctx *c, const float *logits, size_t tokens, size_t n_experts, size_t k, int policy,
+                                uint32_t *experts, float *weights) {
+    if (!c) return LARQL_E_ARG;
+    if (k > n_experts) k = n_experts;  // select(): k.min(logits.len())
+    if (tokens == 0 || k == 0) return LARQL_OK;
+    if (n_experts > 64 || k > 8) return fail(c, LARQL_UNSUPPORTED, "router_select: at most 64 experts and top-8 on this backend");
+    if (!logits || !experts || !weights) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, router_select_launch(c->stream, logits, (uint32_t)tokens, (uint32_t)n_experts, (uint32_t)k, policy, experts, weights));
+    return LARQL_OK;
+}
+
+size_t larql_hip_moe_mxfp4_workspace_bytes(size_t tokens, size_t k, size_t hidden, size_t inter) {
+    const size_t slots = tokens * k;
+    return (slots * inter * 3 + slots * hidden) * sizeof(float) + 256;
+}
+
+int larql_hip_dev_moe_mxfp4(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank, const float *x, size_t tokens, size_t k,
+                            const uint32_t *experts, const float *weights, float *out, void *workspace, size_t workspace_bytes) {
+    if (!c || !bank) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    const size_t hidden = bank->hidden, inter = bank->inter;
+    if (hidden % 32 != 0 || inter % 32 != 0) return fail(c, LARQL_REFUSED_SHAPE, "moe_mxfp4: hidden and inter must be multiples of 32");
+    if (tokens == 0 || k == 0) return LARQL_OK;
+    if (workspace_bytes < larql_hip_moe_mxfp4_workspace_bytes(tokens, k, hidden, inter))
+        return fail(c, LARQL_REFUSED_SHAPE, "moe_mxfp4: workspace too small");
+    if (!x || !experts || !weights || !out || !workspace) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    const size_t slots = tokens * k;
+    float *g = (float *)workspace, *u = g + slots * inter, *h = u + slots * inter, *d = h + slots * inter;
+    const uint64_t gu_w_stride = inter * (hidden / 32) * 16, gu_s_stride = inter * (hidden / 32);
+    const uint64_t dn_w_stride = hidden * (inter / 32) * 16, dn_s_stride = hidden * (inter / 32);
+    std::vector<GemvJob> jobs;
+    for (size_t s = 0; s < slots; s++) {
+        const size_t t = s / k;
+        GemvJob a = make_job(KIND_MXFP4, bank->gate_packed, bank->gate_scales, x + t * hidden, g + s * inter, inter, hidden);
+        a.sel = experts + s; a.w_sel_stride = gu_w_stride; a.aux_sel_stride = gu_s_stride;
+        GemvJob b = make_job(KIND_MXFP4, bank->up_packed, bank->up_scales, x + t * hidden, u + s * inter, inter, hidden);
+        b.sel = experts + s; b.w_sel_stride = gu_w_stride; b.aux_sel_stride = gu_s_stride;
+        jobs.push_back(a); jobs.push_back(b);
+    }
+    int rc = enqueue_jobs(c, jobs);
+    if (rc) return rc;
+    HIPCHECK(c, clamped_glu_launch(c->stream, g, u, h, slots * inter, bank->limit, bank->alpha));
+    jobs.clear();
+    for (size_t s = 0; s < slots; s++) {
+        GemvJob a = make_job(KIND_MXFP4, bank->down_packed, bank->down_scales, h + s * inter, d + s * hidden, hidden, inter);
+        a.sel = experts + s; a.w_sel_stride = dn_w_stride; a.aux_sel_stride = dn_s_stride;
+        jobs.push_back(a);
+    }
+    rc = enqueue_jobs(c, jobs);
+    if (rc) return rc;
+    HIPCHECK(c, weighted_sum_launch(c->stream, d, weights, out, (uint32_t)tokens, (uint32_t)k, (uint32_t)hidden));
+    return LARQL_OK;
+}
+
 // ---- device tier: encoders ---------------------------------------------------------------------
 
 int larql_hip_dev_quantize_q4_k(larql_hip_ctx *c, const float *src, size_t n, uint8_t *dst) {

@@ -538,7 +538,12 @@ __device__ __forceinline__ void gemv_body(const GemvLaunch &L, float *part) {
     }
     uint32_t ji = lo;
     while (p < p_end) {
-        const GemvJob j = jobs[ji];
+        GemvJob j = jobs[ji];
+        if (j.sel) {  // run-time expert selection: one bank of equally shaped matrices
+            const uint32_t e = __builtin_amdgcn_readfirstlane(*(const GLOBAL_AS uint32_t *)j.sel);
+            j.w += (size_t)e * j.w_sel_stride;
+            j.aux += (size_t)e * j.aux_sel_stride;
+        }
         const uint32_t jp_end = j.pass_begin + j.n_pass;
         const uint32_t seg_end = min(p_end, jp_end);
         const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin;

@@ -28,6 +28,10 @@ struct GemvJob {
     uint32_t pass_begin;  // first pass of this job in the launch's pass list
     int32_t kind;
     int32_t pad;
+    // Optional run-time selection (MoE): when `sel` is set, the job reads expert id e = *sel and
+    // uses w + e*w_sel_stride, aux + e*aux_sel_stride (one bank of equally shaped matrices).
+    const uint32_t *sel;
+    uint64_t w_sel_stride, aux_sel_stride;
 };
 
 struct GemvLaunch {
@@ -60,5 +64,12 @@ hipError_t f32_to_bf16_launch(hipStream_t s, const float *src, size_t n, uint16_
 hipError_t quantize_q4_0_launch(hipStream_t s, const float *src, size_t n, uint8_t *dst);
 hipError_t quantize_to_q8_launch(hipStream_t s, const float *src, size_t n, int8_t *q8, float *scales);
 hipError_t fill_normal_launch(hipStream_t s, float *dst, size_t n, uint64_t seed, float sigma);
+
+// MoE helpers
+hipError_t router_select_launch(hipStream_t s, const float *logits, uint32_t tokens, uint32_t n_experts, uint32_t k, int policy,
+                                uint32_t *experts, float *weights);
+hipError_t clamped_glu_launch(hipStream_t s, const float *g, const float *u, float *h, size_t n, float limit, float alpha);
+hipError_t weighted_sum_launch(hipStream_t s, const float *d, const float *weights, float *out, uint32_t tokens, uint32_t k,
+                               uint32_t hidden);
 
 }  // namespace larql

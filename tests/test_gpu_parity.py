@@ -404,3 +404,68 @@ def test_cpp_host_mirror():
     assert os.path.exists(exe), "larql_amd/host/host_test is not built (run __graft_entry__.build())"
     r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
     assert r.returncode == 0 and "host_test ok" in r.stdout, r.stdout + r.stderr
+
+
+# ------------------------------------------------------------------------ MoE
+def test_router_select_matches_oracle(be):
+    rng = np.random.default_rng(53)
+    T, E, k = 64, 32, 4
+    logits = rng.standard_normal((T, E)).astype(F)
+    logits[0, :] = 1.0                                   # all tied -> first indices
+    logits[1, :4] = 2.0; logits[1, 4:] = 1.0             # router.rs logits_32()
+    logits[2, 5] = logits[2, 9] = 3.5                    # a tie inside the top-k
+    dl, de, dw = be.to_device(logits), be.malloc(T * k * 4), be.malloc(T * k * 4)
+    for policy in (O.NORMALISED_OVER_SELECTED, O.SOFTMAX_THEN_SELECT):
+        assert be.dev_router_select(dl, T, E, k, policy, de, dw)
+        e, w = be.d2h(de, (T, k), np.uint32), be.d2h(dw, (T, k), F)
+        for t in range(T):
+            want = O.router_select(logits[t], k, policy)
+            assert [int(v) for v in e[t]] == [i for i, _ in want]
+            assert np.allclose(w[t], [x for _, x in want], rtol=2e-6, atol=1e-7)
+    assert [int(v) for v in e[0]] == [0, 1, 2, 3] and [int(v) for v in e[2][:2]] == [5, 9]
+    assert be.dev_router_select(dl, T, E, 0, 1, de, dw)                  # k == 0: nothing to do
+    assert not be.dev_router_select(dl, T, 65, 4, 1, de, dw)             # beyond this kernel: refused
+
+
+@pytest.mark.parametrize("T,E,hidden,inter", [(1, 4, 2880, 2880), (16, 8, 2880, 576)])
+def test_moe_mxfp4_block_matches_oracle(be, fmt, T, E, hidden, inter):
+    rng = np.random.default_rng(59 + T)
+    k = 4
+
+    def bank(n, kk):
+        p, s = [], []
+        for _ in range(E):
+            w = (rng.standard_normal(n * kk) * 0.02).astype(F)
+            pp, ss = O.quantize_mxfp4(w, n, kk)
+            p.append(pp); s.append(ss)
+        return np.concatenate(p), np.concatenate(s)
+
+    gp, gs = bank(inter, hidden)
+    up, us = bank(inter, hidden)
+    dp, ds = bank(hidden, inter)
+    x = rng.standard_normal((T, hidden)).astype(F)
+    logits = rng.standard_normal((T, E)).astype(F)
+    # oracle: select -> per expert gate/up -> ClampedGlu -> down -> weighted sum in selection order
+    want = np.zeros((T, hidden), F)
+    gw, gsz = inter * (hidden // 32) * 16, inter * (hidden // 32)
+    dwb, dsz = hidden * (inter // 32) * 16, hidden * (inter // 32)
+    for t in range(T):
+        acc = np.zeros(hidden, F)
+        for e, w in O.router_select(logits[t], k):
+            g = O.mxfp4_gemv(gp[e * gw:(e + 1) * gw], gs[e * gsz:(e + 1) * gsz], x[t], inter, hidden)
+            u = O.mxfp4_gemv(up[e * gw:(e + 1) * gw], us[e * gsz:(e + 1) * gsz], x[t], inter, hidden)
+            h = np.array([O.clamped_glu(float(a), float(b)) for a, b in zip(g, u)], F)
+            d = O.mxfp4_gemv(dp[e * dwb:(e + 1) * dwb], ds[e * dsz:(e + 1) * dsz], h, hidden, inter)
+            acc = (acc + F(w) * d).astype(F)
+        want[t] = acc
+    dev = {n: be.to_device(a) for n, a in dict(gp=gp, gs=gs, up=up, us=us, dp=dp, ds=ds, x=x, lg=logits).items()}
+    de, dw_, do = be.malloc(T * k * 4), be.malloc(T * k * 4), be.malloc(T * hidden * 4)
+    assert be.dev_router_select(dev["lg"], T, E, k, O.NORMALISED_OVER_SELECTED, de, dw_)
+    b = fmt.Mxfp4Experts(dev["gp"], dev["gs"], dev["up"], dev["us"], dev["dp"], dev["ds"], E, hidden, inter, 7.0, 1.702)
+    wsb = be.moe_mxfp4_workspace_bytes(T, k, hidden, inter)
+    ws = be.malloc(wsb)
+    assert be.dev_moe_mxfp4(b, dev["x"], T, k, de, dw_, do, ws, wsb)
+    be.synchronize()
+    got = be.d2h(do, (T, hidden), F)
+    assert rel_l2(got, want) < 1e-5
+    assert not be.dev_moe_mxfp4(b, dev["x"], T, k, de, dw_, do, ws, wsb - 1024)   # short workspace: refused
