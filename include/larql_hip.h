@@ -246,6 +246,13 @@ int larql_hip_dev_gate_knn(larql_hip_ctx *ctx, int format, const void *gate,
                            const float *x, size_t batch, size_t n_features, size_t hidden,
                            size_t top_k, float *scores_scratch, uint32_t *idx_out, float *score_out);
 
+/* Batched-prefill GEMM on resident operands: out[seq, rows] = X[seq, hidden] . W[rows, hidden]^T,
+ * W in Q4_K, X held as bf16 (the top 16 bits of each f32).  Same contraction as
+ * QuantMatVec::q4k_matmul (backend/quant_matvec.rs:324-333): bf16 MFMA with fp32
+ * accumulate; each decoded weight enters as two bf16 terms (hi + lo). */
+int larql_hip_dev_q4k_gemm(larql_hip_ctx *ctx, const uint8_t *w, const uint16_t *x_bf16, size_t rows, size_t hidden,
+                           size_t seq, float *out);
+
 /* ---- device tier: MoE expert block (MXFP4) --------------------------------------
  * router::select — larql-compute/src/ffn/expert_weight/router.rs:33-70: top-k
  * of `n_experts` logits per token (ties: first index), weights softmaxed over

@@ -325,6 +325,9 @@ class HipBackend:
                      val: int) -> bool:
         return self._some(lib.larql_hip_dev_gate_knn(self._h, fmt, gate, x, batch, n, hidden, top_k, scores, idx, val))
 
+    def dev_q4k_gemm(self, w: int, x_bf16: int, rows: int, hidden: int, seq: int, out: int) -> bool:
+        return self._some(lib.larql_hip_dev_q4k_gemm(self._h, w, x_bf16, rows, hidden, seq, out))
+
     def dev_router_select(self, logits: int, tokens: int, n_experts: int, k: int, policy: int, experts: int, weights: int) -> bool:
         return self._some(lib.larql_hip_dev_router_select(self._h, logits, tokens, n_experts, k, policy, experts, weights))
 

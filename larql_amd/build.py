@@ -11,7 +11,7 @@ import subprocess
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "liblarql_hip.so")
-SOURCES = ["gemv.hip", "topk.hip", "quantize.hip", "moe.hip", "api.hip"]
+SOURCES = ["gemv.hip", "topk.hip", "quantize.hip", "moe.hip", "gemm.hip", "api.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-Wall",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

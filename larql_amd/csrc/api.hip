@@ -446,13 +446,29 @@ int larql_hip_q4k_matmul(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, c
     if (rc) return rc;
     rc = ensure(c, c->out, out_len * 4 + 64);
     if (rc) return rc;
-    std::vector<GemvJob> jobs;
-    for (size_t s = 0; s < seq_len; s++)
-        jobs.push_back(make_job(KIND_Q4K, dw, nullptr, (const float *)c->x.p + s * hidden, (float *)c->out.p + s * num_rows,
-                                num_rows, hidden));
     Submission sub(c);
-    rc = enqueue_jobs(c, jobs);
-    if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
+    if (seq_len >= 16 && num_rows <= 0xFFFFFFFFull && seq_len <= 0xFFFFFFFFull) {
+        // prefill shape: bf16 MFMA GEMM.  The f32 activations are split into two bf16 terms so the
+        // result keeps ~16 significant bits of x; the second pass is skipped when x is exactly bf16.
+        rc = ensure(c, c->misc, x_len * 4 + 64);
+        if (rc) return rc;
+        uint16_t *xh = (uint16_t *)c->misc.p, *xl = xh + x_len;
+        HIPCHECK(c, hipMemsetAsync(c->nan_flag, 0, sizeof(int), c->stream));
+        HIPCHECK(c, split_bf16_launch(c->stream, (const float *)c->x.p, x_len, xh, xl, c->nan_flag));
+        int any_lo = 0;
+        HIPCHECK(c, hipMemcpyAsync(&any_lo, c->nan_flag, sizeof(int), hipMemcpyDeviceToHost, c->stream));
+        HIPCHECK(c, hipStreamSynchronize(c->stream));
+        HIPCHECK(c, q4k_gemm_launch(c->stream, dw, xh, (float *)c->out.p, (uint32_t)num_rows, (uint32_t)hidden, (uint32_t)seq_len, 0));
+        if (any_lo)
+            HIPCHECK(c, q4k_gemm_launch(c->stream, dw, xl, (float *)c->out.p, (uint32_t)num_rows, (uint32_t)hidden, (uint32_t)seq_len, 1));
+    } else {
+        std::vector<GemvJob> jobs;
+        for (size_t s = 0; s < seq_len; s++)
+            jobs.push_back(make_job(KIND_Q4K, dw, nullptr, (const float *)c->x.p + s * hidden, (float *)c->out.p + s * num_rows,
+                                    num_rows, hidden));
+        rc = enqueue_jobs(c, jobs);
+        if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
+    }
     HIPCHECK(c, hipMemcpyAsync(out, c->out.p, out_len * 4, hipMemcpyDeviceToHost, c->stream));
     return sub.finish();
 }
@@ -936,6 +952,18 @@ int larql_hip_dev_copy(larql_hip_ctx *c, void *dst, const void *src, size_t byte
     const uint32_t grid = (uint32_t)c->cu_count * 8u;
     if (dst) HIPCHECK(c, copy_launch(c->stream, src, dst, bytes, grid));
     else { int rc = ensure(c, c->misc, 64); if (rc) return rc; HIPCHECK(c, read_launch(c->stream, src, (uint32_t *)c->misc.p, bytes, grid)); }
+    return LARQL_OK;
+}
+
+int larql_hip_dev_q4k_gemm(larql_hip_ctx *c, const uint8_t *w, const uint16_t *x_bf16, size_t rows, size_t hidden, size_t seq,
+                           float *out) {
+    if (!c) return LARQL_E_ARG;
+    if (rows == 0 || seq == 0 || hidden == 0) return LARQL_OK;
+    if (hidden % 256 != 0) return fail(c, LARQL_REFUSED_SHAPE, "q4k_gemm: hidden not a multiple of 256");
+    if (rows > 0xFFFFFFFFull || seq > 0xFFFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "q4k_gemm: too large");
+    if (!w || !x_bf16 || !out || ((uintptr_t)w & 15) || ((uintptr_t)x_bf16 & 15)) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, q4k_gemm_launch(c->stream, w, x_bf16, out, (uint32_t)rows, (uint32_t)hidden, (uint32_t)seq, 0));
     return LARQL_OK;
 }
 

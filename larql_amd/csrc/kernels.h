@@ -65,6 +65,11 @@ hipError_t quantize_q4_0_launch(hipStream_t s, const float *src, size_t n, uint8
 hipError_t quantize_to_q8_launch(hipStream_t s, const float *src, size_t n, int8_t *q8, float *scales);
 hipError_t fill_normal_launch(hipStream_t s, float *dst, size_t n, uint64_t seed, float sigma);
 
+// batched-prefill Q4_K GEMM (bf16 MFMA, fp32 accumulate)
+hipError_t q4k_gemm_launch(hipStream_t s, const uint8_t *w, const uint16_t *x_bf16, float *out, uint32_t rows, uint32_t hidden,
+                           uint32_t seq, int accumulate);
+hipError_t split_bf16_launch(hipStream_t s, const float *x, size_t n, uint16_t *hi, uint16_t *lo, int *any_lo);
+
 // MoE helpers
 hipError_t router_select_launch(hipStream_t s, const float *logits, uint32_t tokens, uint32_t n_experts, uint32_t k, int policy,
                                 uint32_t *experts, float *weights);

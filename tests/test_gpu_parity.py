@@ -469,3 +469,34 @@ def test_moe_mxfp4_block_matches_oracle(be, fmt, T, E, hidden, inter):
     got = be.d2h(do, (T, hidden), F)
     assert rel_l2(got, want) < 1e-5
     assert not be.dev_moe_mxfp4(b, dev["x"], T, k, de, dw_, do, ws, wsb - 1024)   # short workspace: refused
+
+
+# ------------------------------------------------------------- prefill GEMM
+@pytest.mark.parametrize("rows,hidden,seq", [(300, 512, 70), (128, 3840, 128), (1, 256, 1), (257, 768, 33)])
+def test_q4k_gemm_mfma_matches_oracle(be, rows, hidden, seq):
+    rng = np.random.default_rng(61 + rows)
+    w = (rng.standard_normal((rows, hidden)) * 0.02).astype(F)
+    q = O.quantize_q4_k(w)
+    xb = O.f32_to_bf16(rng.standard_normal((seq, hidden)).astype(F))          # activations held as bf16 (truncated)
+    X = (xb.astype(np.uint32) << 16).view(F).reshape(seq, hidden)
+    want = O.q4k_matmul(q, X, rows, hidden, seq)                                # [seq, rows]
+    dw, dx, do = be.to_device(q), be.to_device(xb), be.malloc(seq * rows * 4)
+    assert be.dev_q4k_gemm(dw, dx, rows, hidden, seq, do)
+    be.synchronize()
+    got = be.d2h(do, (seq, rows), F)
+    assert rel_l2(got, want) < 1e-4          # stated bar 1e-3; two bf16 weight terms give ~1e-5
+    # every output element (guards tile-edge and layout mistakes)
+    assert np.max(np.abs(got - want)) < 2e-3 * (np.abs(want).mean() + 1e-9)
+
+
+def test_q4k_matmul_host_tier_uses_gemm_for_prefill_shapes(be):
+    rng = np.random.default_rng(67)
+    rows, hidden, seq = 200, 1024, 40
+    q = O.quantize_q4_k((rng.standard_normal((rows, hidden)) * 0.02).astype(F))
+    X = rng.standard_normal((seq, hidden)).astype(F)                            # full f32 activations: two bf16 terms
+    got = be.q4k_matmul(q, X, rows, hidden, seq)
+    want = O.q4k_matmul(q, X, rows, hidden, seq).reshape(-1)
+    assert rel_l2(got, want) < 1e-4
+    # rows of the matmul equal the stacked matvec (quantize_q4_0_tests.rs:202-238, tol 1e-4)
+    mv = be.q4k_matvec(q, X[7], rows, hidden)
+    assert np.max(np.abs(got.reshape(seq, rows)[7] - mv)) < 1e-4
