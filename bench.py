@@ -139,6 +139,231 @@ def verify_and_cpu_baseline(be, stack, lm_rows=16384, min_seconds=10.0):
     }
 
 
+def _timeit(be, fn, reps, warm=2):
+    for _ in range(warm):
+        fn()
+    be.synchronize()
+    e0, e1 = be.event(), be.event()
+    be.record(e0)
+    for _ in range(reps):
+        fn()
+    be.record(e1)
+    return be.elapsed_ms(e0, e1) / reps
+
+
+def _oracle():
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import oracle as O  # the checker / CPU baseline; never the product
+    return O
+
+
+def _cpu_time(fn, seconds):
+    fn()
+    times, t_end = [], time.perf_counter() + seconds
+    while time.perf_counter() < t_end or len(times) < 3:
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return float(np.median(times)), len(times)
+
+
+def _emit(metric, value, unit, ms, steps, warmup, config, roofline, cpu, higher=True):
+    print(json.dumps({"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
+                      "ms_per_step": round(ms, 5), "higher_is_better": higher, "scaling": "weak", "vs_baseline": None,
+                      "dtype": "f32", "data": "synthetic", "config": config, "roofline": roofline, "cpu_baseline": cpu}))
+
+
+def run_c1(be, fmt, args):
+    """BASELINE configs[0]: Q4_K 3072x1024 matvec, batch 1 (cold: 256 distinct copies in one launch; hot: one copy)."""
+    O = _oracle()
+    rows, k, copies = 3072, 1024, 256
+    tmp = be.malloc(rows * k * 4)
+    x = be.malloc(k * 4 + 64)
+    be.dev_fill_normal(x, k, 0x5EED0100 ^ 0xA5A50000, 1.0)
+    ws, outs = [], []
+    for i in range(copies):
+        w = be.malloc(q4k_bytes(rows, k) + 64)
+        be.dev_fill_normal(tmp, rows * k, 0x5EED0100 + i, 0.02)
+        be.dev_quantize_q4_k(tmp, rows * k, w)
+        ws.append(w); outs.append(be.malloc(rows * 4 + 64))
+    cold = be.plan_create([(fmt.FMT_Q4_K, w, None, x, o, rows, k) for w, o in zip(ws, outs)])
+    hot = be.plan_create([(fmt.FMT_Q4_K, ws[0], None, x, o, rows, k) for o in outs])
+    be.plan_run(cold); be.synchronize()
+    wb, xv = be.d2h(ws[3], q4k_bytes(rows, k), np.uint8), be.d2h(x, k, np.float32)
+    want = O.q4k_matvec(wb, xv, rows, k)
+    rel = float(np.linalg.norm(be.d2h(outs[3], rows, np.float32).astype(np.float64) - want) / np.linalg.norm(want))
+    assert rel < 1e-3, rel
+    algo = q4k_bytes(rows, k) + 4 * k + 4 * rows
+    ms_cold = _timeit(be, lambda: be.plan_run(cold), args.steps)
+    ms_hot = _timeit(be, lambda: be.plan_run(hot), args.steps)
+    ms_one = _timeit(be, lambda: be.dev_matvec(fmt.FMT_Q4_K, ws[5], None, x, rows, k, outs[5]), args.steps)
+    threads = min(16, len(os.sched_getaffinity(0)))
+    med, n = _cpu_time(lambda: O.q4k_matvec_mt(wb, xv, rows, k, threads), args.cpu_seconds)
+    gbs = copies * algo / ms_cold / 1e6
+    _emit("Q4_K 3072x1024 matvec HBM GB/s (cold, 256 distinct copies per launch)", round(gbs, 1), "GB/s", ms_cold, args.steps,
+          2, {"workload": "BASELINE configs[0]: Q4_K matvec 3072x1024, batch 1", "us_per_matvec_cold": round(ms_cold * 1e3 / copies, 3),
+              "us_per_matvec_hot": round(ms_hot * 1e3 / copies, 3), "GBps_hot": round(copies * algo / ms_hot / 1e6, 1),
+              "us_single_launch_device_resident": round(ms_one * 1e3, 2), "verified_rel_l2_vs_oracle": rel},
+          {"kernel": "gemv_q4k", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+           "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+          {"value": round(algo / med / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+           "sample": f"one 3072x1024 matvec, median of {n}", "us_per_matvec": round(med * 1e6, 1)})
+
+
+def run_c3(be, fmt, args):
+    """BASELINE configs[2]: gate-KNN 10240x2560, bf16 and Q4_K gates, top-64 by |score|, 34 layers, batch 1 and 8."""
+    O = _oracle()
+    n, hidden, k, layers = 10240, 2560, 64, 34
+    tmp = be.malloc(n * hidden * 4)
+    threads = min(16, len(os.sched_getaffinity(0)))
+    for variant, f, nbytes in (("bf16", fmt.FMT_BF16, 2 * n * hidden), ("q4k", fmt.FMT_Q4_K, q4k_bytes(n, hidden))):
+        gates = []
+        for layer in range(layers):
+            g = be.malloc(nbytes + 64)
+            be.dev_fill_normal(tmp, n * hidden, 0x5EED0300 + layer, 0.02)
+            (be.dev_f32_to_bf16 if variant == "bf16" else be.dev_quantize_q4_k)(tmp, n * hidden, g)
+            gates.append(g)
+        for batch in (1, 8):
+            x = be.malloc(batch * hidden * 4 + 64)
+            be.dev_fill_normal(x, batch * hidden, 0x5EED03F0 + batch, 1.0)
+            scores = be.malloc(layers * batch * n * 4)
+            idx, val = be.malloc(layers * batch * k * 4), be.malloc(layers * batch * k * 4)
+
+            def walk():  # all 34 layers in one submission (2 launches)
+                be.dev_gate_walk(f, gates, x, 0, batch, n, hidden, k, scores, idx, val)
+            walk(); be.synchronize()
+            # verify the last layer against the oracle
+            gb, xv = be.d2h(gates[-1], nbytes, np.uint8), be.d2h(x, (batch, hidden), np.float32)
+            got_i = be.d2h(idx, (layers, batch, k), np.uint32)[-1]
+            for b in range(batch):
+                sc = (O.bf16_gemv(gb.view(np.uint16), xv[b], n, hidden) if variant == "bf16" else O.q4k_matvec(gb, xv[b], n, hidden))
+                want = O.top_k_by_abs(sc, k)
+                diff = {int(i) for i in got_i[b]} ^ {i for i, _ in want}
+                kth = abs(want[-1][1])
+                assert all(abs(abs(float(sc[i])) - kth) <= 1e-5 * max(1.0, kth) for i in diff), (variant, batch, b)
+            ms = _timeit(be, walk, max(3, args.steps // 5)) / layers
+            algo = nbytes + batch * (4 * hidden + 4 * n + 8 * k)
+
+            def cpu_one():
+                for b in range(batch):
+                    sc = (O.bf16_gemv(gb.view(np.uint16), xv[b], n, hidden) if variant == "bf16" else O.q4k_matvec_mt(gb, xv[b], n, hidden, threads))
+                    O.top_k_by_abs(sc, k)
+            med, nrep = _cpu_time(cpu_one, args.cpu_seconds / 4)
+            _emit(f"gate-KNN top-64 us/layer ({variant} gate 10240x2560, batch {batch})", round(ms * 1e3, 2), "us/layer", ms * layers,
+                  max(3, args.steps // 5), 2,
+                  {"workload": f"BASELINE configs[2]: vindex gate-KNN walk, {variant} gate, K=64, 34 layers, batch {batch}",
+                   "launches_per_walk": 2, "GBps_weights_once": round(algo / ms / 1e6, 1), "topk_identical_up_to_ties": True},
+                  {"kernel": f"gemv_{variant} + topk", "bound": "hbm", "achieved": round(algo / ms / 1e6, 1), "peak": HBM_PEAK_GBS,
+                   "unit": "GB/s", "frac": round(algo / ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": None},
+                  {"value": round(med * 1e6, 1), "unit": "us/layer", "cores": threads if variant == "q4k" else 1, "kind": "port",
+                   "sample": f"one layer, batch {batch}, median of {nrep}"}, higher=False)
+            for p in (x, scores, idx, val):
+                be.free(p)
+        for g in gates:
+            be.free(g)
+
+
+def run_c4(be, fmt, args):
+    """BASELINE configs[3]: MXFP4 MoE experts, 32 experts x (gate, up, down 2880x2880), top-4, batch 1 and 16."""
+    O = _oracle()
+    E, H, I, k = 32, 2880, 2880, 4
+    per = H * I
+    tmp = be.malloc(per * 4)
+    bufs = {}
+    for name, seed in (("gate", 0x5EED0400), ("up", 0x5EED0440), ("down", 0x5EED0480)):
+        p, s = be.malloc(E * per // 2 + 64), be.malloc(E * per // 32 + 64)
+        for e in range(E):
+            be.dev_fill_normal(tmp, per, seed + e, 0.02)
+            be.dev_quantize_mxfp4(tmp, H if name != "down" else H, I if name != "down" else I, p + e * per // 2, s + e * per // 32)
+        bufs[name] = (p, s)
+    bank = fmt.Mxfp4Experts(bufs["gate"][0], bufs["gate"][1], bufs["up"][0], bufs["up"][1], bufs["down"][0], bufs["down"][1], E, H, I,
+                            7.0, 1.702)
+    expert_bytes = 3 * (per // 2 + per // 32)
+    for T in (1, 16):
+        x, lg = be.malloc(T * H * 4 + 64), be.malloc(T * E * 4 + 64)
+        be.dev_fill_normal(x, T * H, 0x5EED04F0 + T, 1.0)
+        be.dev_fill_normal(lg, T * E, 0x5EED04E0 + T, 1.0)
+        de, dw, out = be.malloc(T * k * 4), be.malloc(T * k * 4), be.malloc(T * H * 4)
+        wsb = be.moe_mxfp4_workspace_bytes(T, k, H, I)
+        ws = be.malloc(wsb)
+
+        def block():
+            be.dev_router_select(lg, T, E, k, 1, de, dw)
+            be.dev_moe_mxfp4(bank, x, T, k, de, dw, out, ws, wsb)
+        block(); be.synchronize()
+        experts = be.d2h(de, (T, k), np.uint32)
+        distinct = len(set(int(v) for v in experts.reshape(-1)))
+        # verify token 0 against the oracle
+        xv, lv, wv = be.d2h(x, (T, H), np.float32), be.d2h(lg, (T, E), np.float32), be.d2h(dw, (T, k), np.float32)
+        acc = np.zeros(H, np.float32)
+        mats = {}
+        for (e, w) in O.router_select(lv[0], k):
+            for name in ("gate", "up", "down"):
+                mats[name] = (be.d2h(bufs[name][0] + e * per // 2, per // 2, np.uint8), be.d2h(bufs[name][1] + e * per // 32, per // 32, np.uint8))
+            g = O.mxfp4_gemv(*mats["gate"], xv[0], I, H); u = O.mxfp4_gemv(*mats["up"], xv[0], I, H)
+            h = np.array([O.clamped_glu(float(a), float(b)) for a, b in zip(g, u)], np.float32)
+            acc = (acc + np.float32(w) * O.mxfp4_gemv(*mats["down"], h, H, I)).astype(np.float32)
+        got = be.d2h(out, (T, H), np.float32)[0]
+        rel = float(np.linalg.norm(got.astype(np.float64) - acc) / np.linalg.norm(acc))
+        assert rel < 1e-3, rel
+        ms = _timeit(be, block, args.steps)
+        algo = distinct * expert_bytes + T * (8 * H + 4 * E)
+        med, nrep = _cpu_time(lambda: O.mxfp4_gemv(*mats["gate"], xv[0], I, H), args.cpu_seconds / 4)
+        _emit(f"MXFP4 MoE expert block us (32 experts, top-4, batch {T})", round(ms * 1e3, 2), "us/block", ms, args.steps, 2,
+              {"workload": f"BASELINE configs[3]: MXFP4 experts 32 x (gate, up, down 2880x2880), top-4, batch {T}",
+               "distinct_experts": distinct, "launches_per_block": 5, "GBps_over_distinct_expert_bytes": round(algo / ms / 1e6, 1),
+               "us_per_expert_matvec": round(ms * 1e3 / (3 * T * k), 2), "verified_rel_l2_vs_oracle": rel},
+              {"kernel": "gemv_mxfp4 (gate/up + down launches)", "bound": "hbm", "achieved": round(algo / ms / 1e6, 1), "peak": HBM_PEAK_GBS,
+               "unit": "GB/s", "frac": round(algo / ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": None},
+              {"value": round(med * 1e6 * 3 * T * k, 1), "unit": "us/block", "cores": 1, "kind": "port",
+               "sample": f"one 2880x2880 MXFP4 matvec (dequant-order loop), median of {nrep}, scaled by {3 * T * k} matvecs"}, higher=False)
+        for p in (x, lg, de, dw, out, ws):
+            be.free(p)
+
+
+def run_c5(be, fmt, args):
+    """BASELINE configs[4]: batched-prefill Q4_K GEMM at Gemma-3-12B shapes, 512 tokens, bf16 MFMA."""
+    O = _oracle()
+    seq = 512
+    total_fl, total_ms, rels = 0.0, 0.0, []
+    per = []
+    for name, rows, hidden in (("gate", 15360, 3840), ("up", 15360, 3840), ("down", 3840, 15360)):
+        n = rows * hidden
+        tmp, w = be.malloc(n * 4), be.malloc(q4k_bytes(rows, hidden) + 64)
+        be.dev_fill_normal(tmp, n, 0x5EED0500 + len(per), 0.02)
+        be.dev_quantize_q4_k(tmp, n, w)
+        xf, xb = be.malloc(seq * hidden * 4), be.malloc(seq * hidden * 2 + 64)
+        be.dev_fill_normal(xf, seq * hidden, 0x5EED05F0 + len(per), 1.0)
+        be.dev_f32_to_bf16(xf, seq * hidden, xb)
+        out = be.malloc(seq * rows * 4)
+        be.dev_q4k_gemm(w, xb, rows, hidden, seq, out); be.synchronize()
+        # verify 64 rows x 8 tokens against the oracle
+        r0 = 4096 % rows
+        wb = be.d2h(w + r0 * (hidden // 256) * 144, 64 * (hidden // 256) * 144, np.uint8)
+        xs = (be.d2h(xb, (seq, hidden), np.uint16)[:8].astype(np.uint32) << 16).view(np.float32)
+        want = O.q4k_matmul(wb, xs, 64, hidden, 8)
+        got = be.d2h(out, (seq, rows), np.float32)[:8, r0:r0 + 64]
+        rels.append(float(np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want)))
+        assert rels[-1] < 1e-3, rels
+        ms = _timeit(be, lambda: be.dev_q4k_gemm(w, xb, rows, hidden, seq, out), max(3, args.steps // 5))
+        fl = 2.0 * seq * rows * hidden
+        per.append({"matrix": name, "us": round(ms * 1e3, 1), "TFLOPs": round(fl / ms / 1e9, 1)})
+        total_fl += fl; total_ms += ms
+        if name == "down":
+            med, nrep = _cpu_time(lambda: O.q4k_matmul(wb, xs, 64, hidden, 8), args.cpu_seconds / 2)
+            cpu = {"value": round(2.0 * 64 * hidden * 8 / med / 1e12, 5), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                   "sample": f"64 rows x 8 tokens x {hidden} (q4k_matmul_into restated), median of {nrep}"}
+        for p in (tmp, w, xf, xb, out):
+            be.free(p)
+    tf = total_fl / total_ms / 1e9
+    _emit("Q4_K prefill GEMM TFLOP/s (bf16 MFMA, 512 tokens, Gemma-3-12B FFN)", round(tf, 1), "TFLOP/s", total_ms, max(3, args.steps // 5), 2,
+          {"workload": "BASELINE configs[4]: Q4_K GEMM 512x3840 . (15360x3840, 15360x3840, 3840x15360)", "per_matrix": per,
+           "mfma_terms_per_weight": 2, "verified_rel_l2_vs_oracle": max(rels)},
+          {"kernel": "q4k_gemm", "bound": "mfma", "achieved": round(tf, 1), "peak": 2500.0, "unit": "TFLOP/s",
+           "frac": round(tf / 2500.0, 4), "traffic": None, "note": "nominal flops 2*S*N*K; the kernel issues twice that (hi+lo weight terms)"},
+          cpu)
+
+
 def read_traffic():
     """HBM bytes per launch of the dominant kernel from the committed rocprof PMC summary, if any."""
     path = os.path.join(ROOT, "profiles", "gemv_q4k_c2_stack.pmc.txt")
@@ -159,6 +384,8 @@ def main():
     ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"],
+                    help="c2 (default) is the headline decode stack; the others are BASELINE's remaining configs")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run the plain 16-byte copy kernel on 1 GiB three times (known size, for scaling "
                          "profiler byte counters) and print its bandwidth")
@@ -189,6 +416,9 @@ def main():
         ms_r = be.elapsed_ms(e2, e3) / 3
         print(json.dumps({"copy_bytes": n, "copy_GBps_read_plus_write": round(2 * n / ms / 1e6, 1),
                           "read_only_GBps": round(n / ms_r / 1e6, 1)}))
+        return
+    if args.workload != "c2":
+        {"c1": run_c1, "c3": run_c3, "c4": run_c4, "c5": run_c5}[args.workload](be, fmt, args)
         return
     stack = Stack(be, fmt, layers=args.layers)
 

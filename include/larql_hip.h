@@ -246,6 +246,18 @@ int larql_hip_dev_gate_knn(larql_hip_ctx *ctx, int format, const void *gate,
                            const float *x, size_t batch, size_t n_features, size_t hidden,
                            size_t top_k, float *scores_scratch, uint32_t *idx_out, float *score_out);
 
+/* Gate-KNN over `n_layers` layers in ONE submission — the shape of LQL WALK / DESCRIBE, where
+ * every layer of the index is scored for one query (PatchedVindex::walk,
+ * larql-vindex/src/patch/overlay.rs:557-562 over VectorIndex::gate_knn): one matvec launch for all
+ * layers' scores and one top-K launch for all (layer, position) rows.  gates[l] is layer l's
+ * [n_features, hidden] matrix; x is [batch, hidden] (x_layer_stride == 0: the same residuals
+ * for every layer) or [n_layers, batch, hidden] (x_layer_stride == batch*hidden).
+ * scores_scratch: [n_layers, batch, n_features]; idx_out/score_out: [n_layers, batch, top_k];
+ * count_out (may be NULL): hits per row. */
+int larql_hip_dev_gate_walk(larql_hip_ctx *ctx, int format, const void *const *gates, size_t n_layers, const float *x,
+                            size_t x_layer_stride, size_t batch, size_t n_features, size_t hidden, size_t top_k,
+                            float *scores_scratch, uint32_t *idx_out, float *score_out, uint32_t *count_out);
+
 /* Batched-prefill GEMM on resident operands: out[seq, rows] = X[seq, hidden] . W[rows, hidden]^T,
  * W in Q4_K, X held as bf16 (the top 16 bits of each f32).  Same contraction as
  * QuantMatVec::q4k_matmul (backend/quant_matvec.rs:324-333): bf16 MFMA with fp32

@@ -325,6 +325,12 @@ class HipBackend:
                      val: int) -> bool:
         return self._some(lib.larql_hip_dev_gate_knn(self._h, fmt, gate, x, batch, n, hidden, top_k, scores, idx, val))
 
+    def dev_gate_walk(self, fmt: int, gates: Sequence[int], x: int, x_layer_stride: int, batch: int, n: int, hidden: int,
+                      top_k: int, scores: int, idx: int, val: int, count: Optional[int] = None) -> bool:
+        arr = (C.c_void_p * max(len(gates), 1))(*gates)
+        return self._some(lib.larql_hip_dev_gate_walk(self._h, fmt, arr, len(gates), x, x_layer_stride, batch, n, hidden, top_k,
+                                                      scores, idx, val, count))
+
     def dev_q4k_gemm(self, w: int, x_bf16: int, rows: int, hidden: int, seq: int, out: int) -> bool:
         return self._some(lib.larql_hip_dev_q4k_gemm(self._h, w, x_bf16, rows, hidden, seq, out))
 

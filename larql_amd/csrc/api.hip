@@ -1025,6 +1025,36 @@ int larql_hip_dev_moe_mxfp4(larql_hip_ctx *c, const larql_hip_mxfp4_experts *ban
     return LARQL_OK;
 }
 
+// Gate-KNN over several layers in one submission (the LQL WALK / DESCRIBE shape: every layer of
+// the index scored for one query, PatchedVindex::walk): one matvec launch for all layers' scores
+// and one top-K launch for all (layer, position) rows.
+int larql_hip_dev_gate_walk(larql_hip_ctx *c, int format, const void *const *gates, size_t n_layers, const float *x,
+                            size_t x_layer_stride, size_t batch, size_t n, size_t hidden, size_t top_k, float *scores_scratch,
+                            uint32_t *idx_out, float *score_out, uint32_t *count_out) {
+    if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    const int kind = kind_of_format(format);
+    int rc = gate_shape_check(c, kind, (size_t)-1, 0, hidden);
+    if (rc) return rc;
+    if (kind == KIND_Q4_0) return fail(c, LARQL_UNSUPPORTED, "gate_walk: Q4_0 gates go through larql_hip_dev_gate_knn");
+    if (n_layers == 0 || batch == 0 || n == 0 || top_k == 0) return LARQL_OK;
+    if (top_k > 64 || n > 0xFFFFFFFFull || hidden == 0 || n_layers * batch > 0x7FFFFFFFull)
+        return fail(c, LARQL_UNSUPPORTED, "gate_walk: unsupported size");
+    if (!gates || !x || !scores_scratch || !idx_out || !score_out) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    if (!count_out) { rc = ensure(c, c->misc, n_layers * batch * 4 + 64); if (rc) return rc; count_out = (uint32_t *)c->misc.p; }
+    std::vector<GemvJob> jobs;
+    jobs.reserve(n_layers * batch);
+    for (size_t l = 0; l < n_layers; l++)
+        for (size_t b = 0; b < batch; b++)
+            jobs.push_back(make_job(kind, gates[l], nullptr, x + l * x_layer_stride + b * hidden, scores_scratch + (l * batch + b) * n, n, hidden));
+    rc = enqueue_jobs(c, jobs);
+    if (rc) return rc;
+    HIPCHECK(c, topk_launch(c->stream, scores_scratch, (uint32_t)(n_layers * batch), (uint32_t)n, (uint32_t)top_k, true, idx_out,
+                            score_out, count_out, c->nan_flag, nullptr, 0));
+    return LARQL_OK;
+}
+
 // ---- device tier: encoders ---------------------------------------------------------------------
 
 int larql_hip_dev_quantize_q4_k(larql_hip_ctx *c, const float *src, size_t n, uint8_t *dst) {

@@ -500,3 +500,29 @@ def test_q4k_matmul_host_tier_uses_gemm_for_prefill_shapes(be):
     # rows of the matmul equal the stacked matvec (quantize_q4_0_tests.rs:202-238, tol 1e-4)
     mv = be.q4k_matvec(q, X[7], rows, hidden)
     assert np.max(np.abs(got.reshape(seq, rows)[7] - mv)) < 1e-4
+
+
+def test_gate_walk_over_layers_equals_per_layer_calls(be, fmt):
+    rng = np.random.default_rng(71)
+    L, n, hidden, k, batch = 3, 1000, 512, 64, 2
+    gates_h = [O.f32_to_bf16((rng.standard_normal((n, hidden)) * 0.02).astype(F)) for _ in range(L)]
+    X = rng.standard_normal((L, batch, hidden)).astype(F)
+    gates = [be.to_device(g) for g in gates_h]
+    x = be.to_device(X)
+    scores, idx, val, cnt = be.malloc(L * batch * n * 4), be.malloc(L * batch * k * 4), be.malloc(L * batch * k * 4), be.malloc(L * batch * 4)
+    assert be.dev_gate_walk(fmt.FMT_BF16, gates, x, batch * hidden, batch, n, hidden, k, scores, idx, val, cnt)
+    be.synchronize()
+    gi, gv = be.d2h(idx, (L, batch, k), np.uint32), be.d2h(val, (L, batch, k), F)
+    assert (be.d2h(cnt, L * batch, np.uint32) == k).all()
+    for l in range(L):
+        for b in range(batch):
+            ref = O.bf16_gemv(gates_h[l], X[l, b], n, hidden)
+            check_hits([(int(i), float(v)) for i, v in zip(gi[l, b], gv[l, b])], ref, k)
+    # shared residuals (stride 0) == per-layer host-tier calls
+    assert be.dev_gate_walk(fmt.FMT_BF16, gates, x, 0, batch, n, hidden, k, scores, idx, val)
+    be.synchronize()
+    gi0 = be.d2h(idx, (L, batch, k), np.uint32)
+    for l in range(L):
+        hits = be.gate_knn_batch_hits(fmt.FMT_BF16, gates_h[l], X[0], n, hidden, k)
+        for b in range(batch):
+            assert [i for i, _ in hits[b]] == [int(v) for v in gi0[l, b]]
