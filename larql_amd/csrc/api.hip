@@ -166,10 +166,10 @@ int prepare_same_kind(larql_hip_ctx *c, std::vector<GemvJob> &live, void *table_
         HIPCHECK(c, hipStreamSynchronize(c->stream));
         P.L.table = (const GemvJob *)table_dst;
     }
-    uint64_t grid = (uint64_t)c->cu_count * (uint64_t)c->wgs_per_cu;
+    P.lds = gemv_lds_bytes(live.data(), live.size(), P.threads);
+    uint64_t grid = (uint64_t)c->cu_count * (uint64_t)gemv_wgs_per_cu(P.kind, P.threads, P.lds, (uint32_t)c->wgs_per_cu);
     if (grid > total) grid = total;
     P.grid = (uint32_t)grid;
-    P.lds = gemv_lds_bytes(live.data(), live.size());
     return LARQL_OK;
 }
 
@@ -186,12 +186,14 @@ int check_jobs(larql_hip_ctx *c, const std::vector<GemvJob> &jobs) {
 }
 
 // Split jobs into one group per format present, in first-seen order.
-std::vector<std::vector<GemvJob>> group_by_kind(const std::vector<GemvJob> &jobs) {
+std::vector<std::vector<GemvJob>> group_by_kind(const std::vector<GemvJob> &jobs_in) {
+    std::vector<GemvJob> jobs(jobs_in);
+    for (GemvJob &j : jobs) j.kind = gemv_effective_kind(j);  // Q4_K rows the matrix-core kernel takes get their own launch
     std::vector<std::vector<GemvJob>> groups;
     bool done[8] = {false, false, false, false, false, false, false, false};
     for (size_t i = 0; i < jobs.size(); i++) {
         const int kind = jobs[i].kind;
-        if (jobs[i].rows == 0 || kind < 0 || kind > 6 || done[kind]) continue;
+        if (jobs[i].rows == 0 || kind < 0 || kind > 7 || done[kind]) continue;
         done[kind] = true;
         std::vector<GemvJob> live;
         for (size_t t = i; t < jobs.size(); t++)

@@ -375,6 +375,279 @@ __device__ __forceinline__ void run_q4k(const GemvJob &j, uint32_t p0, uint32_t 
     }
 }
 
+// ---------------------------------------------------------------------------
+// Q4_K on the matrix cores (rows of up to 48 super-blocks).
+//
+// A wavefront owns one super-block column c of a job and walks down the rows
+// 16 at a time.  Its 16 x 144 bytes of a tile stream global -> LDS directly
+// (global_load_lds, 16 bytes per lane, no VGPRs) into a private ring kQ4kStages
+// deep, so the bytes in flight are bounded by LDS, not by registers or
+// occupancy, and no wavefront ever waits for another one's loads.
+//
+// The dot products run on v_mfma_i32_16x16x64_i8, exactly, with the roles
+// swapped: the 16 "B" columns are the 16 weight rows of the tile and the "A"
+// rows carry the activation.  Per 256-wide column, x is scaled by a power of
+// two to 28-bit integers n = rint(x * 2^(27-e)) (2^e > max|x|) and n is split
+// into four balanced base-128 digits (int8 "limbs"); A row 4g + 2cl + i holds
+// limb i (first operand set) or limb 2+i (second set) of sub-block 2g+cl in
+// the k-slots that the sub-block's nibbles occupy in B, zero elsewhere.  Lane
+// (row j = lane%16, kq = lane/16) supplies, per 32-byte group, the low nibbles
+// of its bytes 8kq..8kq+7 in k-slots 0-7 and the high nibbles in slots 8-15
+// (three mask/shift instructions per 8 weights) and, after two MFMAs per group,
+// holds for weight row j and group g = kq the eight exact integer sums
+// nibbles.limb — it is the very lane that decodes that group's two scales and
+// mins from the header.  The limb sums are recombined in f32 (the only
+// rounding besides the final scale), so the result differs from an f32 FMA
+// chain over exact products only by the 2^-28 relative quantum of x.
+// Value per row as q4k_matvec_into (larql-compute/src/cpu/ops/q4_common/
+// matvec_f32.rs:116-155): sum over sub-blocks of (d*sc)*dot(q,x) - (dmin*mn)*sum(x).
+//
+// Rows longer than the workgroup has wavefronts are covered in up to 4 column
+// passes per tile (wave w owns columns w, w+nw, ...), summed in registers.
+// Row partials meet in LDS every kQ4kBatchTiles tiles: part[row][wave*4 + g],
+// folded in a fixed order that depends only on the row length.
+// ---------------------------------------------------------------------------
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) void *lds_vp;
+typedef const GLOBAL_AS void *g_vp;
+union Q4kOp { i32x4 v; uint32_t u[4]; };  // one MFMA operand: 16 int8 k-slots of a lane
+
+constexpr int kQ4kStages = 4;      // wave-tiles in flight per wavefront (ring slots of 2304 B)
+constexpr int kQ4kBatchTiles = 4;  // 16-row tiles between two folds of the row partials
+constexpr int kQ4kMaxColPasses = 4;
+constexpr int kQ4kMaxWaves = 12;
+constexpr uint32_t kQ4kTileBytes = 16 * 144;
+constexpr uint32_t kQ4kColBytes = 1024 + 64;  // a column's activation limbs for 64 lanes, then {k, -, -, -, sums of 8 sub-blocks}
+
+// s_waitcnt vmcnt(n), n < 64, leaving the other counters alone (gfx9 encoding)
+#define LARQL_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
+
+struct Q4kCol {
+    uint32_t xq[4];        // this lane's 8 activations as int8 limbs: {limb i: 2 dwords, limb 2+i: 2 dwords}, i = lane & 1
+    float k;               // 2^(e-27): integer dot -> value
+    float sum_lo, sum_hi;  // sum of x over sub-blocks 2kq and 2kq+1
+};
+
+// A column's activations as loaded
+struct Q4kRaw { f32x4 v, a, b; };
+
+__device__ __forceinline__ Q4kRaw q4k_mfma_load_col(const float *x, uint32_t c, uint32_t lane) {
+    // A-operand row j = 4g + 2cl + i feeds sub-block m = j/2 = 2g+cl: elements 8kq..8kq+7 of it
+    const uint32_t j = lane & 15u, kq = lane >> 4, m = j >> 1;
+    g_f4p xc = (g_f4p)(x + (size_t)c * 256);
+    g_f4p xs = (g_f4p)(x + (size_t)c * 256 + m * 32 + 8 * kq);
+    Q4kRaw r;
+    r.v = xc[lane];  // 4 consecutive activations per lane: column max and per-sub-block sums (8 lanes each)
+    r.a = xs[0];
+    r.b = xs[1];
+    return r;
+}
+
+__device__ __forceinline__ Q4kCol q4k_mfma_finish_col(const Q4kRaw &r, uint32_t lane) {
+    const uint32_t j = lane & 15u, kq = lane >> 4;
+    float mx = fmaxf(fmaxf(fabsf(r.v.x), fabsf(r.v.y)), fmaxf(fabsf(r.v.z), fabsf(r.v.w)));
+    float sm = (r.v.x + r.v.y) + (r.v.z + r.v.w);
+#pragma unroll
+    for (int o = 1; o < 8; o <<= 1) { sm += __shfl_xor(sm, o); mx = fmaxf(mx, __shfl_xor(mx, o)); }
+#pragma unroll
+    for (int o = 8; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    Q4kCol col;
+    col.sum_lo = __shfl(sm, 16 * kq);
+    col.sum_hi = __shfl(sm, 16 * kq + 8);
+    int ex = 0;
+    if (mx > 0.f && mx < __builtin_inff()) (void)frexpf(mx, &ex);  // mx = f * 2^ex, f in [0.5, 1)
+    ex = max(-90, min(120, ex));
+    const float to_int = ldexpf(1.f, 27 - ex);  // |x| * to_int < 2^27
+    col.k = ldexpf(1.f, ex - 27);
+    const float e[8] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w};
+    const uint32_t i = j & 1u;
+    uint32_t la[8], lb[8];  // limbs i and 2+i of the 8 elements, as unsigned bytes
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+        // n = l0*128^3 + l1*128^2 + l2*128 + l3 with l1..l3 in [-64, 63], l0 in [-64, 64]
+        const int n = (int)__builtin_rintf(e[t] * to_int);
+        const int l3 = ((n + 64) & 127) - 64, n1 = (n - l3) >> 7;
+        const int l2 = ((n1 + 64) & 127) - 64, n2 = (n1 - l2) >> 7;
+        const int l1 = ((n2 + 64) & 127) - 64, l0 = (n2 - l1) >> 7;
+        la[t] = (uint32_t)(i ? l1 : l0) & 0xFFu;
+        lb[t] = (uint32_t)(i ? l3 : l2) & 0xFFu;
+    }
+    col.xq[0] = la[0] | (la[1] << 8) | (la[2] << 16) | (la[3] << 24);
+    col.xq[1] = la[4] | (la[5] << 8) | (la[6] << 16) | (la[7] << 24);
+    col.xq[2] = lb[0] | (lb[1] << 8) | (lb[2] << 16) | (lb[3] << 24);
+    col.xq[3] = lb[4] | (lb[5] << 8) | (lb[6] << 16) | (lb[7] << 24);
+    return col;
+}
+
+// xm[2g] / xm[2g+1]: A operands (limbs 0,1 / limbs 2,3) of the MFMAs of group g.  A lane is non-zero only in
+// its own group (j/4) and only in the k-slots of its sub-block's nibbles: 0-7 (low, cl = 0) or 8-15 (high).
+__device__ __forceinline__ void q4k_mfma_operands(Q4kOp (&xm)[8], const Q4kCol &col, uint32_t j) {
+    const uint32_t my_g = j >> 2, cl = (j >> 1) & 1u;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        const bool lo = my_g == (uint32_t)g && cl == 0, hi = my_g == (uint32_t)g && cl == 1;
+        xm[2 * g].u[0] = lo ? col.xq[0] : 0u; xm[2 * g].u[1] = lo ? col.xq[1] : 0u;
+        xm[2 * g].u[2] = hi ? col.xq[0] : 0u; xm[2 * g].u[3] = hi ? col.xq[1] : 0u;
+        xm[2 * g + 1].u[0] = lo ? col.xq[2] : 0u; xm[2 * g + 1].u[1] = lo ? col.xq[3] : 0u;
+        xm[2 * g + 1].u[2] = hi ? col.xq[2] : 0u; xm[2 * g + 1].u[3] = hi ? col.xq[3] : 0u;
+    }
+}
+
+// one wave-tile from its LDS slot: 16 rows x one super-block against the column's activations
+__device__ __forceinline__ float q4k_mfma_tile(const uint8_t *slot, const Q4kOp (&xm)[8], const Q4kCol &col, uint32_t j, uint32_t kq) {
+    const uint8_t *sp = slot + j * 144;
+    const u32x4 hdr = *reinterpret_cast<const u32x4 *>(sp);
+    u32x2 q[4];
+#pragma unroll
+    for (int g = 0; g < 4; g++) q[g] = *reinterpret_cast<const u32x2 *>(sp + 16 + 32 * g + 8 * kq);
+    i32x4 Da = {0, 0, 0, 0}, Db = {0, 0, 0, 0};
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        Q4kOp b;
+        b.u[0] = q[g].x & 0x0F0F0F0Fu; b.u[1] = q[g].y & 0x0F0F0F0Fu;
+        b.u[2] = (q[g].x >> 4) & 0x0F0F0F0Fu; b.u[3] = (q[g].y >> 4) & 0x0F0F0F0Fu;
+        Da = __builtin_amdgcn_mfma_i32_16x16x64_i8(xm[2 * g].v, b.v, Da, 0, 0, 0);
+        Db = __builtin_amdgcn_mfma_i32_16x16x64_i8(xm[2 * g + 1].v, b.v, Db, 0, 0, 0);
+    }
+    // this lane's group is g = kq.  Da = [lo.l0, lo.l1, hi.l0, hi.l1], Db = [lo.l2, lo.l3, hi.l2, hi.l3]
+    float dot_lo = __builtin_fmaf((float)Da[0], 128.f, (float)Da[1]);
+    float dot_hi = __builtin_fmaf((float)Da[2], 128.f, (float)Da[3]);
+    dot_lo = __builtin_fmaf(dot_lo, 128.f, (float)Db[0]);
+    dot_hi = __builtin_fmaf(dot_hi, 128.f, (float)Db[2]);
+    dot_lo = __builtin_fmaf(dot_lo, 128.f, (float)Db[1]) * col.k;
+    dot_hi = __builtin_fmaf(dot_hi, 128.f, (float)Db[3]) * col.k;
+    // header fields as get_scale_min_k4 (matvec_f32.rs:124-131), two bytes at a time
+    const float d = half_bits_to_float(hdr.x & 0xFFFFu), dmin = half_bits_to_float(hdr.x >> 16);
+    const uint32_t sh = (kq & 1u) * 16u;
+    const uint32_t a = (hdr.y >> sh) & 0xFFFFu, b = (hdr.z >> sh) & 0xFFFFu, c = (hdr.w >> sh) & 0xFFFFu;
+    const uint32_t sc_hi2 = (c & 0x0F0Fu) | ((a >> 2) & 0x3030u), mn_hi2 = ((c >> 4) & 0x0F0Fu) | ((b >> 2) & 0x3030u);
+    const uint32_t sc2 = kq < 2 ? (a & 0x3F3Fu) : sc_hi2, mn2 = kq < 2 ? (b & 0x3F3Fu) : mn_hi2;
+    const float sc_lo = d * (float)(sc2 & 0xFFu), sc_hi = d * (float)(sc2 >> 8);
+    const float mn_lo = dmin * (float)(mn2 & 0xFFu), mn_hi = dmin * (float)(mn2 >> 8);
+    float r = sc_lo * dot_lo - mn_lo * col.sum_lo;
+    r += sc_hi * dot_hi - mn_hi * col.sum_hi;
+    return r;
+}
+
+// tiles [tile_a, tile_b) of one job; `parity` flips per batch (double-buffered partials)
+__device__ __forceinline__ void run_q4k_mfma(const GemvJob &j, uint32_t tile_a, uint32_t tile_b, uint8_t *lds, uint32_t &parity) {
+    constexpr int NS = kQ4kStages, R = kQ4kBatchTiles;
+    const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t nw_launch = blockDim.x >> 6;
+    const uint32_t jr = lane & 15u, kq = lane >> 4;
+    const uint32_t nwj = j.rpp, cpr = j.cpr, PW = nwj * 4;
+    const uint32_t rows = (uint32_t)j.rows, row_bytes = (uint32_t)j.row_bytes;
+    uint8_t *ring = lds + wv * (NS * kQ4kTileBytes);
+    float *part = reinterpret_cast<float *>(lds + nw_launch * (NS * kQ4kTileBytes));
+    const uint32_t np = wv < nwj ? (cpr - wv + nwj - 1) / nwj : 0;  // columns wv, wv+nwj, ... of this wavefront
+
+    // Column state: in registers when the wavefront has one column; with several it is prepared once per
+    // job into this wavefront's own LDS area (1 KB of operands + 64 B of scales and sums per column) and
+    // fetched at every column change.
+    uint8_t *cols = lds + nw_launch * (NS * kQ4kTileBytes) + 2 * R * 16 * nw_launch * 4 * sizeof(float) +
+                    wv * (kQ4kMaxColPasses * kQ4kColBytes);
+    Q4kCol col;
+    Q4kOp xm[8];
+    auto fetch_col = [&](uint32_t p) {
+        const uint8_t *cp = cols + p * kQ4kColBytes;
+        const u32x4 xq = *reinterpret_cast<const u32x4 *>(cp + lane * 16);
+        const float2_t sm = *reinterpret_cast<const float2_t *>(cp + 1024 + 16 + kq * 8);
+        col.xq[0] = xq.x; col.xq[1] = xq.y; col.xq[2] = xq.z; col.xq[3] = xq.w;
+        col.k = *reinterpret_cast<const float *>(cp + 1024);
+        col.sum_lo = sm.x; col.sum_hi = sm.y;
+        q4k_mfma_operands(xm, col, jr);
+    };
+    if (np == 1) {
+        col = q4k_mfma_finish_col(q4k_mfma_load_col(j.x, wv, lane), lane);
+        q4k_mfma_operands(xm, col, jr);
+    } else if (np > 1) {
+        for (uint32_t p = 0; p < np; p++) {
+            const Q4kCol c = q4k_mfma_finish_col(q4k_mfma_load_col(j.x, wv + nwj * p, lane), lane);
+            uint8_t *cp = cols + p * kQ4kColBytes;
+            *reinterpret_cast<u32x4 *>(cp + lane * 16) = (u32x4){c.xq[0], c.xq[1], c.xq[2], c.xq[3]};
+            if (lane == 0) *reinterpret_cast<float *>(cp + 1024) = c.k;
+            if (jr == 0) *reinterpret_cast<float2_t *>(cp + 1024 + 16 + kq * 8) = (float2_t){c.sum_lo, c.sum_hi};
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own writes, own reads: program order is enough
+    }
+
+    // lane's three pieces of a wave-tile, in 16-byte units u = row*9 + piece (the last 256 B go dword by dword)
+    const uint32_t u0 = lane, u1 = 64 + lane, u2 = 128 + (lane >> 2);
+    const uint32_t r0 = u0 / 9, r1 = u1 / 9, r2 = u2 / 9;
+    const uint32_t w0 = (u0 - r0 * 9) * 16, w1 = (u1 - r1 * 9) * 16, w2 = (u2 - r2 * 9) * 16 + (lane & 3u) * 4;
+    const uint8_t *wcol = j.w + (size_t)wv * 144;
+    const uint32_t nt = tile_b - tile_a;
+
+    // issue cursor: wave-tiles in the order they are consumed (batch, column pass, tile of the batch)
+    uint32_t it_tb = 0, it_p = 0, it_tl = 0, n_issue = 0;
+    auto issue = [&]() {
+        // past the end the last wave-tile is read again: every wavefront keeps the same number of loads in flight
+        const uint32_t tl = min(tile_a + it_tb + it_tl, tile_b - 1);
+        const uint8_t *gp = wcol + (size_t)it_p * nwj * 144;
+        const uint32_t rb = tl * 16;
+        const uint8_t *g0 = gp + (size_t)min(rb + r0, rows - 1) * row_bytes + w0;
+        const uint8_t *g1 = gp + (size_t)min(rb + r1, rows - 1) * row_bytes + w1;
+        const uint8_t *g2 = gp + (size_t)min(rb + r2, rows - 1) * row_bytes + w2;
+        uint8_t *lp = ring + (n_issue % NS) * kQ4kTileBytes;
+        __builtin_amdgcn_global_load_lds((g_vp)g0, (lds_vp)lp, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((g_vp)g1, (lds_vp)(lp + 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((g_vp)g2, (lds_vp)(lp + 2048), 4, 0, 0);
+        n_issue++;
+        if (it_tb < nt) {
+            const uint32_t nb = min((uint32_t)R, nt - it_tb);
+            if (++it_tl == nb) {
+                it_tl = 0;
+                if (++it_p == np) { it_p = 0; it_tb += R; }
+            }
+        }
+    };
+    if (np >= 1)
+        for (int s = 0; s < NS - 1; s++) issue();
+
+    uint32_t n_use = 0;
+    for (uint32_t tb = 0; tb < nt; tb += R) {
+        float *pb = part + parity * (R * 16 * nw_launch * 4);
+        const uint32_t nb = min((uint32_t)R, nt - tb);
+        if (np >= 1) {
+            float racc[R];
+#pragma unroll
+            for (int tl = 0; tl < R; tl++) racc[tl] = 0.f;
+#pragma unroll 1
+            for (uint32_t p = 0; p < np; p++) {
+                if (np > 1) fetch_col(p);
+#pragma unroll
+                for (int tl = 0; tl < R; tl++) {
+                    if ((uint32_t)tl < nb) {
+                        issue();
+                        LARQL_WAIT_VMCNT(3 * (NS - 1));  // at most NS-1 younger wave-tiles still in flight: the oldest has landed
+                        asm volatile("" ::: "memory");
+                        racc[tl] += q4k_mfma_tile(ring + (n_use % NS) * kQ4kTileBytes, xm, col, jr, kq);
+                        n_use++;
+                    }
+                }
+            }
+#pragma unroll
+            for (int tl = 0; tl < R; tl++)
+                if ((uint32_t)tl < nb) pb[(tl * 16 + jr) * PW + wv * 4 + kq] = racc[tl];
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        // fold: 4 lanes per row, lane q sums the group-q partial of every wavefront in order
+        const uint32_t row_base = (tile_a + tb) * 16;
+        for (uint32_t rr = threadIdx.x >> 2; rr < nb * 16; rr += blockDim.x >> 2) {
+            const uint32_t qd = threadIdx.x & 3u;
+            float s = 0.f;
+            for (uint32_t k = 0; k < nwj; k++) s += pb[rr * PW + k * 4 + qd];
+            s = dpp_add<0xB1>(s);  // quad_perm [1,0,3,2]
+            s = dpp_add<0x4E>(s);  // quad_perm [2,3,0,1]
+            if (qd == 0 && row_base + rr < rows) ((g_f32wp)j.out)[row_base + rr] = s;
+        }
+        parity ^= 1u;
+    }
+}
+
 template <int U>
 __device__ __forceinline__ void run_q8_0(const GemvJob &j, uint32_t p0, uint32_t p1, float *part) {
     const uint32_t t = threadIdx.x, cpr = j.cpr, rpp = j.rpp;
@@ -576,6 +849,33 @@ LARQL_GEMV_KERNEL(gemv_f16_kernel, KIND_F16, 4, 4)
 LARQL_GEMV_KERNEL(gemv_f32_kernel, KIND_F32, 2, 4)
 
 
+// Q4_K on the matrix cores: workgroup b sweeps its share of the launch's tile list (a tile = 16 rows of
+// a job, weighted by the job's row length so that shares are equal in bytes), job by job.
+__global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_mfma_kernel(GemvLaunch L) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t q4k_lds[];
+    const GemvJob *jobs = L.table ? L.table : L.inl;
+    const uint64_t P = L.total_passes;
+    uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
+    const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
+    uint32_t lo = 0, hi = L.n_jobs;
+    while (lo + 1 < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (jobs[mid].pass_begin <= p) lo = mid; else hi = mid;
+    }
+    uint32_t ji = lo, parity = 0;
+    while (p < p_end) {
+        const GemvJob j = jobs[ji];
+        const uint32_t seg_end = min(p_end, j.pass_begin + j.n_pass);
+        // a tile belongs to the workgroup whose share contains its first cost unit
+        const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin;
+        const uint32_t tile_a = (a + j.cpr - 1) / j.cpr, tile_b = (b + j.cpr - 1) / j.cpr;
+        if (tile_a < tile_b) run_q4k_mfma(j, tile_a, tile_b, q4k_lds, parity);
+        p = seg_end;
+        ji++;
+    }
+    LARQL_WAIT_VMCNT(0);
+}
+
 // ---------------------------------------------------------------------------
 // Host side: geometry and launch.
 // ---------------------------------------------------------------------------
@@ -590,7 +890,45 @@ static uint32_t chunk_elems(int kind) {
     }
 }
 
+// Q4_K on the matrix cores: wavefronts used for a row of `cpr` super-blocks (a function of the row
+// length alone, so a matvec sums in the same order whatever else shares its launch): one wavefront per
+// column up to 12, beyond that the count in 6..10 that wastes the fewest column slots over <= 4 passes
+// (10 wavefronts x 4 columns of prepared activations is what fits in LDS beside the weight ring).
+static uint32_t q4k_mfma_waves(uint64_t cpr) {
+    if (cpr <= (uint64_t)kQ4kMaxWaves) return (uint32_t)cpr;
+    uint32_t best = 0;
+    uint64_t best_slots = ~0ull;
+    for (uint32_t nw = 10; nw >= 6; nw--) {
+        const uint64_t passes = (cpr + nw - 1) / nw;
+        if (passes > (uint64_t)kQ4kMaxColPasses) continue;
+        if (passes * nw < best_slots) { best_slots = passes * nw; best = nw; }
+    }
+    return best;  // 0: row too long for this path
+}
+
+static int g_q4k_mfma = getenv("LARQL_HIP_Q4K_MFMA") ? atoi(getenv("LARQL_HIP_Q4K_MFMA")) : 1;
+
+int gemv_effective_kind(const GemvJob &j) {
+    if (j.kind == KIND_Q4K && g_q4k_mfma && !j.sel && j.k % 256 == 0 && j.k / 256 >= 1 && q4k_mfma_waves(j.k / 256) != 0 &&
+        j.rows < 0x7FFFFFF0ull && (j.k / 256) * 144 * j.rows < (1ull << 62))
+        return KIND_Q4K_MFMA;
+    return j.kind;
+}
+
 bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
+    if (j.kind == KIND_Q4K_MFMA) {
+        if (j.k == 0 || j.k % 256 != 0) return false;
+        const uint64_t cpr = j.k / 256;
+        const uint32_t nw = q4k_mfma_waves(cpr);
+        if (nw == 0 || nw * 64 > threads) return false;
+        j.cpr = (uint32_t)cpr;
+        j.rpp = nw;  // wavefronts that work on this job
+        j.row_bytes = cpr * 144;
+        const uint64_t tiles = (j.rows + 15) / 16;
+        if (tiles * cpr > 0x7FFFFFFFull) return false;
+        j.n_pass = (uint32_t)(tiles * cpr);  // cost units: one per tile and super-block column
+        return true;
+    }
     const uint32_t ce = chunk_elems(j.kind);
     if (j.k == 0 || j.k % ce != 0) return false;
     const uint64_t cpr = j.k / ce;
@@ -613,6 +951,15 @@ bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
 }
 
 uint32_t gemv_pick_threads(const GemvJob *jobs, size_t n) {
+    if (n > 0 && jobs[0].kind == KIND_Q4K_MFMA) {
+        uint32_t nw = 0;
+        for (size_t i = 0; i < n; i++) {
+            const uint32_t w = q4k_mfma_waves(jobs[i].k / 256);
+            if (w == 0) return 0;
+            if (w > nw) nw = w;
+        }
+        return nw * 64;
+    }
     // Prefer the block size that wastes the fewest lanes over the jobs'
     // chunk counts (weighted by bytes); ties go to the smaller block.
     static const uint32_t cand_all[] = {256, 320, 384, 448, 512};
@@ -639,7 +986,14 @@ uint32_t gemv_pick_threads(const GemvJob *jobs, size_t n) {
     return pick;
 }
 
-size_t gemv_lds_bytes(const GemvJob *jobs, size_t n) {
+size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
+    if (n > 0 && jobs[0].kind == KIND_Q4K_MFMA) {
+        const size_t nw = threads / 64;
+        bool multi = false;  // some row needs several column passes: room for the prepared activations
+        for (size_t i = 0; i < n; i++) multi = multi || jobs[i].k / 256 > (uint64_t)kQ4kMaxWaves;
+        return nw * kQ4kStages * kQ4kTileBytes + 2 * (size_t)kQ4kBatchTiles * 16 * nw * 4 * sizeof(float) +
+               (multi ? nw * kQ4kMaxColPasses * kQ4kColBytes : 0);
+    }
     size_t m = 0;
     for (size_t i = 0; i < n; i++) {
         const size_t npart = jobs[i].kind == KIND_Q4K ? jobs[i].cpr / 4 : jobs[i].cpr;
@@ -649,8 +1003,26 @@ size_t gemv_lds_bytes(const GemvJob *jobs, size_t n) {
     return m;
 }
 
+uint32_t gemv_wgs_per_cu(int kind, uint32_t threads, size_t lds, uint32_t dflt) {
+    if (kind != KIND_Q4K_MFMA) return dflt;
+    // as many workgroups as LDS (160 KB per CU) allows, up to 12 wavefronts per CU (3 per SIMD at this register count)
+    const uint32_t by_lds = (uint32_t)((160 * 1024) / lds), by_waves = 12 / (threads / 64);
+    const uint32_t w = by_lds < by_waves ? by_lds : by_waves;
+    return w < 1 ? 1 : w;
+}
+
 hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32_t threads, uint32_t grid, size_t lds) {
     switch (kind) {
+        case KIND_Q4K_MFMA: {
+            static bool attr_set = false;  // dynamic LDS above 64 KB has to be allowed once per process
+            if (!attr_set) {
+                hipError_t e = hipFuncSetAttribute((const void *)gemv_q4k_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                if (e != hipSuccess) return e;
+                attr_set = true;
+            }
+            hipLaunchKernelGGL(gemv_q4k_mfma_kernel, dim3(grid), dim3(threads), lds, stream, L);
+            break;
+        }
         case KIND_Q4K:
             if (g_unroll != 4) hipLaunchKernelGGL(gemv_q4k_u2_kernel, dim3(grid), dim3(threads), lds, stream, L);
             else hipLaunchKernelGGL(gemv_q4k_u4_kernel, dim3(grid), dim3(threads), lds, stream, L);

@@ -40,7 +40,8 @@ def weights(seed, rows, cols, sigma=0.02):
 
 # ------------------------------------------------------------------- Q4_K
 @pytest.mark.parametrize("rows,cols", [(3072, 1024), (2048, 2560), (1031, 2560), (77, 10240), (5, 256), (640, 2048),
-                                       (300, 3840), (33, 1792)])
+                                       (300, 3840), (33, 1792), (257, 4096), (130, 7168), (48, 12288), (17, 3328),
+                                       (1, 2560), (16, 2816), (4100, 512)])
 def test_q4k_matvec_matches_oracle(be, rows, cols):
     w, x = weights(rows * 7 + cols, rows, cols)
     q = O.quantize_q4_k(w)
@@ -53,6 +54,33 @@ def test_q4k_matvec_matches_oracle(be, rows, cols):
     assert np.max(np.abs(got - want)) < 1e-3 * scale
     # deterministic across repeats
     assert np.array_equal(got.view(np.uint32), be.q4k_matvec(q, x, rows, cols).view(np.uint32))
+
+
+@pytest.mark.parametrize("case", ["outliers", "zero", "tiny", "huge", "one_hot"])
+def test_q4k_matvec_activation_ranges(be, case):
+    # the matrix-core kernel rescales every 256-wide slice of x by a power of two and splits it into
+    # two f16 terms: the result must not depend on the magnitude or spread of the activations
+    rows, cols = 96, 2560
+    w, x = weights(11, rows, cols)
+    if case == "outliers":
+        x[::97] *= 1000.0
+    elif case == "zero":
+        x[:] = 0.0
+    elif case == "tiny":
+        x *= 1e-30
+    elif case == "huge":
+        x *= 1e20
+    else:
+        x[:] = 0.0
+        x[1000] = -3.5
+    q = O.quantize_q4_k(w)
+    want = O.q4k_matvec(q, x, rows, cols)
+    got = be.q4k_matvec(q, x, rows, cols)
+    assert got is not None and np.isfinite(got).all()
+    if case == "zero":
+        assert not got.any()
+    else:
+        assert rel_l2(got, want) < TOL
 
 
 def test_q4k_matvec_refusals_follow_the_cpu_backend(be):
