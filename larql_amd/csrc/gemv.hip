@@ -416,7 +416,7 @@ union Q4kOp { i32x4 v; uint32_t u[4]; };  // one MFMA operand: 16 int8 k-slots o
 constexpr int kQ4kStages = 4;      // wave-tiles in flight per wavefront (ring slots of 2304 B)
 constexpr int kQ4kBatchTiles = 4;  // 16-row tiles between two folds of the row partials
 constexpr int kQ4kMaxColPasses = 4;
-constexpr int kQ4kMaxWaves = 12;
+constexpr int kQ4kMaxWaves = 10;  // with the ring, the partials and 4 prepared columns per wavefront this fills the 160 KB of LDS
 constexpr uint32_t kQ4kTileBytes = 16 * 144;
 constexpr uint32_t kQ4kColBytes = 1024 + 64;  // a column's activation limbs for 64 lanes, then {k, -, -, -, sums of 8 sub-blocks}
 
@@ -892,7 +892,7 @@ static uint32_t chunk_elems(int kind) {
 
 // Q4_K on the matrix cores: wavefronts used for a row of `cpr` super-blocks (a function of the row
 // length alone, so a matvec sums in the same order whatever else shares its launch): one wavefront per
-// column up to 12, beyond that the count in 6..10 that wastes the fewest column slots over <= 4 passes
+// column up to 10, beyond that the count in 6..10 that wastes the fewest column slots over <= 4 passes
 // (10 wavefronts x 4 columns of prepared activations is what fits in LDS beside the weight ring).
 static uint32_t q4k_mfma_waves(uint64_t cpr) {
     if (cpr <= (uint64_t)kQ4kMaxWaves) return (uint32_t)cpr;
