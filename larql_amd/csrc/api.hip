@@ -158,6 +158,7 @@ int prepare_same_kind(larql_hip_ctx *c, std::vector<GemvJob> &live, void *table_
     memset(&P.L, 0, sizeof P.L);
     P.L.total_passes = total;
     P.L.n_jobs = (uint32_t)live.size();
+    P.L.pad = gemv_launch_param(live.data(), live.size());
     if (live.size() <= (size_t)kInlineJobs) {
         for (size_t i = 0; i < live.size(); i++) P.L.inl[i] = live[i];
         P.L.table = nullptr;
@@ -190,10 +191,10 @@ std::vector<std::vector<GemvJob>> group_by_kind(const std::vector<GemvJob> &jobs
     std::vector<GemvJob> jobs(jobs_in);
     for (GemvJob &j : jobs) j.kind = gemv_effective_kind(j);  // Q4_K rows the matrix-core kernel takes get their own launch
     std::vector<std::vector<GemvJob>> groups;
-    bool done[8] = {false, false, false, false, false, false, false, false};
+    bool done[9] = {false, false, false, false, false, false, false, false, false};
     for (size_t i = 0; i < jobs.size(); i++) {
         const int kind = jobs[i].kind;
-        if (jobs[i].rows == 0 || kind < 0 || kind > 7 || done[kind]) continue;
+        if (jobs[i].rows == 0 || kind < 0 || kind > 8 || done[kind]) continue;
         done[kind] = true;
         std::vector<GemvJob> live;
         for (size_t t = i; t < jobs.size(); t++)

@@ -22,6 +22,8 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <algorithm>
+
 #include "kernels.h"
 
 namespace larql {
@@ -542,36 +544,6 @@ __device__ __forceinline__ void run_q4k_mfma(const GemvJob &j, uint32_t tile_a, 
     float *part = reinterpret_cast<float *>(lds + nw_launch * (NS * kQ4kTileBytes));
     const uint32_t np = wv < nwj ? (cpr - wv + nwj - 1) / nwj : 0;  // columns wv, wv+nwj, ... of this wavefront
 
-    // Column state: in registers when the wavefront has one column; with several it is prepared once per
-    // job into this wavefront's own LDS area (1 KB of operands + 64 B of scales and sums per column) and
-    // fetched at every column change.
-    uint8_t *cols = lds + nw_launch * (NS * kQ4kTileBytes) + 2 * R * 16 * nw_launch * 4 * sizeof(float) +
-                    wv * (kQ4kMaxColPasses * kQ4kColBytes);
-    Q4kCol col;
-    Q4kOp xm[8];
-    auto fetch_col = [&](uint32_t p) {
-        const uint8_t *cp = cols + p * kQ4kColBytes;
-        const u32x4 xq = *reinterpret_cast<const u32x4 *>(cp + lane * 16);
-        const float2_t sm = *reinterpret_cast<const float2_t *>(cp + 1024 + 16 + kq * 8);
-        col.xq[0] = xq.x; col.xq[1] = xq.y; col.xq[2] = xq.z; col.xq[3] = xq.w;
-        col.k = *reinterpret_cast<const float *>(cp + 1024);
-        col.sum_lo = sm.x; col.sum_hi = sm.y;
-        q4k_mfma_operands(xm, col, jr);
-    };
-    if (np == 1) {
-        col = q4k_mfma_finish_col(q4k_mfma_load_col(j.x, wv, lane), lane);
-        q4k_mfma_operands(xm, col, jr);
-    } else if (np > 1) {
-        for (uint32_t p = 0; p < np; p++) {
-            const Q4kCol c = q4k_mfma_finish_col(q4k_mfma_load_col(j.x, wv + nwj * p, lane), lane);
-            uint8_t *cp = cols + p * kQ4kColBytes;
-            *reinterpret_cast<u32x4 *>(cp + lane * 16) = (u32x4){c.xq[0], c.xq[1], c.xq[2], c.xq[3]};
-            if (lane == 0) *reinterpret_cast<float *>(cp + 1024) = c.k;
-            if (jr == 0) *reinterpret_cast<float2_t *>(cp + 1024 + 16 + kq * 8) = (float2_t){c.sum_lo, c.sum_hi};
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own writes, own reads: program order is enough
-    }
-
     // lane's three pieces of a wave-tile, in 16-byte units u = row*9 + piece (the last 256 B go dword by dword)
     const uint32_t u0 = lane, u1 = 64 + lane, u2 = 128 + (lane >> 2);
     const uint32_t r0 = u0 / 9, r1 = u1 / 9, r2 = u2 / 9;
@@ -604,6 +576,37 @@ __device__ __forceinline__ void run_q4k_mfma(const GemvJob &j, uint32_t tile_a, 
     };
     if (np >= 1)
         for (int s = 0; s < NS - 1; s++) issue();
+
+    // (prepared while the first weight tiles are on their way)
+    // Column state: in registers when the wavefront has one column; with several it is prepared once per
+    // job into this wavefront's own LDS area (1 KB of operands + 64 B of scales and sums per column) and
+    // fetched at every column change.
+    uint8_t *cols = lds + nw_launch * (NS * kQ4kTileBytes) + 2 * R * 16 * nw_launch * 4 * sizeof(float) +
+                    wv * (kQ4kMaxColPasses * kQ4kColBytes);
+    Q4kCol col;
+    Q4kOp xm[8];
+    auto fetch_col = [&](uint32_t p) {
+        const uint8_t *cp = cols + p * kQ4kColBytes;
+        const u32x4 xq = *reinterpret_cast<const u32x4 *>(cp + lane * 16);
+        const float2_t sm = *reinterpret_cast<const float2_t *>(cp + 1024 + 16 + kq * 8);
+        col.xq[0] = xq.x; col.xq[1] = xq.y; col.xq[2] = xq.z; col.xq[3] = xq.w;
+        col.k = *reinterpret_cast<const float *>(cp + 1024);
+        col.sum_lo = sm.x; col.sum_hi = sm.y;
+        q4k_mfma_operands(xm, col, jr);
+    };
+    if (np == 1) {
+        col = q4k_mfma_finish_col(q4k_mfma_load_col(j.x, wv, lane), lane);
+        q4k_mfma_operands(xm, col, jr);
+    } else if (np > 1) {
+        for (uint32_t p = 0; p < np; p++) {
+            const Q4kCol c = q4k_mfma_finish_col(q4k_mfma_load_col(j.x, wv + nwj * p, lane), lane);
+            uint8_t *cp = cols + p * kQ4kColBytes;
+            *reinterpret_cast<u32x4 *>(cp + lane * 16) = (u32x4){c.xq[0], c.xq[1], c.xq[2], c.xq[3]};
+            if (lane == 0) *reinterpret_cast<float *>(cp + 1024) = c.k;
+            if (jr == 0) *reinterpret_cast<float2_t *>(cp + 1024 + 16 + kq * 8) = (float2_t){c.sum_lo, c.sum_hi};
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own writes, own reads: program order is enough
+    }
 
     uint32_t n_use = 0;
     for (uint32_t tb = 0; tb < nt; tb += R) {
@@ -643,6 +646,176 @@ __device__ __forceinline__ void run_q4k_mfma(const GemvJob &j, uint32_t tile_a, 
             s = dpp_add<0xB1>(s);  // quad_perm [1,0,3,2]
             s = dpp_add<0x4E>(s);  // quad_perm [2,3,0,1]
             if (qd == 0 && row_base + rr < rows) ((g_f32wp)j.out)[row_base + rr] = s;
+        }
+        parity ^= 1u;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// MXFP4 on the matrix cores (rows of up to 40 x 128 elements).
+//
+// gfx950's block-scaled MFMA takes the format as stored: v_mfma_scale_f32_16x16x128_f8f6f4 with an
+// FP4 (e2m1) "B" operand wants, from lane (column j = lane%16, kg = lane/16), the 32 consecutive
+// K-elements 32kg..32kg+31 as 16 packed bytes (low nibble first) plus one e8m0 scale byte — one MXFP4
+// block of weight row j, exactly as mxfp4.rs lays it out (larql-models/src/quant/mxfp4.rs:42-95), so the
+// weights go global -> LDS -> operand registers without a single unpacking instruction and the block
+// scale is applied by the hardware.  The 16 "B" columns are 16 weight rows; a wavefront owns a K-range
+// of `cw` 128-element steps of those rows and streams its (16 rows x cw steps) tiles through a private
+// LDS ring (16-byte and 1-byte global_load_lds, one per lane and step; a sub-dword load still
+// fills a whole dword slot per lane).
+//
+// The "A" rows carry the activation in FP8 (e4m3): per step, n = rint(x * 2^(23-e)) (2^e > max|x| of
+// the step) is written in six balanced base-16 digits d_t in [-8, 8] — exact in e4m3 — and row t holds
+// digit t with the row's own e8m0 scale 2^(e-23+4(5-t)), so sum_t row_t reproduces x to 2^-24 of the
+// step's maximum.  A-operand bytes 0-15 of lane (t, kg) are K = 16kg..16kg+15 of the step, bytes 16-31 are
+// K = 64+16kg..; rows 6-15 are zero.  After the wavefront's steps, lane (j, rq) holds rows 4rq..4rq+3 of
+// column j: the digit sums of weight row j, already scaled, which it adds up (rq = 0, 1 matter).
+// e8m0 0 means 0.0 in the reference (the hardware reads it as 2^-127): such blocks are zeroed; 255 is NaN.
+// ---------------------------------------------------------------------------
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+constexpr int kMx4Stages = 3;
+constexpr int kMx4BatchTiles = 4;
+constexpr int kMx4MaxSteps = 4;    // 128-element steps per wavefront
+constexpr int kMx4MaxWaves = 10;
+constexpr uint32_t kMx4StepBytes = 1024 + 256;  // per step of a wave-tile: 64 lanes x 16 B of nibbles, 64 scale bytes (one dword slot each)
+
+struct Mx4Step {
+    i32x8 a;        // this lane's 32 activation digits (FP8) of the step
+    int scale_a;    // e8m0 scale of this lane's digit row
+};
+
+// Digits of one step's 128 activations, for lane (t = lane%16, kg = lane/16); x index >= k reads as 0.
+// Every lane converts two activations into their six digits and the wavefront transposes them through
+// `scratch` (768 B of its own LDS: digit row t at t*128) into the operand layout.
+__device__ __forceinline__ Mx4Step mx4_setup_step(const float *x, uint32_t step, uint32_t k, uint32_t lane, uint8_t *scratch) {
+    const uint32_t t = lane & 15u, kg = lane >> 4;
+    const uint32_t i0 = step * 128 + 2 * lane;
+    float2_t v = {0.f, 0.f};
+    if (i0 + 2 <= k) v = *(const GLOBAL_AS float2_t *)(x + i0);  // k is even: a pair is inside or outside
+    float mx = fmaxf(fabsf(v.x), fabsf(v.y));
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    int ex = 0;
+    if (mx > 0.f && mx < __builtin_inff()) (void)frexpf(mx, &ex);  // mx = f * 2^ex, f in [0.5, 1)
+    ex = max(-100, min(100, ex));
+    const float to_int = ldexpf(1.f, 23 - ex);
+    // balanced base-16 digits: n + 0x888888 has the unsigned digits d+8 (the top one may reach 16)
+    const int n0 = (int)__builtin_rintf(v.x * to_int) + 0x888888, n1 = (int)__builtin_rintf(v.y * to_int) + 0x888888;
+#pragma unroll
+    for (int d = 0; d < 6; d++) {
+        const int sh = 4 * (5 - d);
+        const int d0 = (d == 0 ? (n0 >> 20) : ((n0 >> sh) & 15)) - 8, d1 = (d == 0 ? (n1 >> 20) : ((n1 >> sh) & 15)) - 8;
+        const int pk = __builtin_amdgcn_cvt_pk_fp8_f32((float)d0, (float)d1, 0, false);  // integers up to 8 are exact in e4m3
+        *reinterpret_cast<uint16_t *>(scratch + d * 128 + 2 * lane) = (uint16_t)pk;
+    }
+    asm volatile("" ::: "memory");  // same wavefront: LDS executes its writes before the reads that follow
+    Mx4Step st;
+    st.scale_a = 124 + ex - 4 * (int)t;  // digit t weighs 2^(ex - 23 + 4*(5 - t))
+    u32x4 lo = {0u, 0u, 0u, 0u}, hi = {0u, 0u, 0u, 0u};
+    if (t < 6) {
+        lo = *reinterpret_cast<const u32x4 *>(scratch + t * 128 + 16 * kg);       // K = 16kg .. 16kg+15
+        hi = *reinterpret_cast<const u32x4 *>(scratch + t * 128 + 64 + 16 * kg);  // K = 64+16kg ..
+    }
+    st.a[0] = (int)lo.x; st.a[1] = (int)lo.y; st.a[2] = (int)lo.z; st.a[3] = (int)lo.w;
+    st.a[4] = (int)hi.x; st.a[5] = (int)hi.y; st.a[6] = (int)hi.z; st.a[7] = (int)hi.w;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the scratch is reused by the next step
+    return st;
+}
+
+#define LARQL_MX4_WAIT_CASE(CW) case CW: LARQL_WAIT_VMCNT(2 * CW * (kMx4Stages - 1)); break;
+
+// tiles [tile_a, tile_b) of one job
+__device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a, uint32_t tile_b, uint8_t *lds, uint32_t slot_bytes,
+                                               uint32_t &parity) {
+    constexpr int NS = kMx4Stages, R = kMx4BatchTiles;
+    const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t nw_launch = blockDim.x >> 6;
+    const uint32_t jr = lane & 15u, kg = lane >> 4;
+    const uint32_t nwj = j.rpp, steps = j.cpr, cw = (uint32_t)j.pad, PW = nwj * 2;
+    const uint32_t rows = (uint32_t)j.rows, k = (uint32_t)j.k, nb = k / 32;
+    const size_t row_bytes = j.row_bytes;
+    uint8_t *ring = lds + wv * (NS * slot_bytes);
+    float *part = reinterpret_cast<float *>(lds + nw_launch * (NS * slot_bytes));
+    const uint32_t step0 = wv * cw;
+    const bool working = wv < nwj && step0 < steps;
+
+    uint32_t blk[kMx4MaxSteps];   // this lane's block of each step, clamped into the row
+    bool valid[kMx4MaxSteps];
+#pragma unroll
+    for (int s = 0; s < kMx4MaxSteps; s++) {
+        const uint32_t b = (step0 + s) * 4 + kg;
+        valid[s] = working && (uint32_t)s < cw && b < nb;
+        blk[s] = min(b, nb - 1);
+    }
+
+    const uint32_t nt = tile_b - tile_a;
+    uint32_t it_tile = tile_a, n_issue = 0;
+    auto issue = [&]() {
+        const uint32_t tl = min(it_tile, tile_b - 1);  // past the end: the last tile again (uniform load counts)
+        const uint32_t row = min(tl * 16 + jr, rows - 1);
+        const uint8_t *wrow = j.w + (size_t)row * row_bytes;
+        const uint8_t *srow = j.aux + (size_t)row * nb;
+        uint8_t *lp = ring + (n_issue % NS) * slot_bytes;
+#pragma unroll
+        for (int s = 0; s < kMx4MaxSteps; s++) {
+            if ((uint32_t)s < cw) {
+                __builtin_amdgcn_global_load_lds((g_vp)(wrow + (size_t)blk[s] * 16), (lds_vp)(lp + s * 1024), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((g_vp)(srow + blk[s]), (lds_vp)(lp + cw * 1024 + s * 256), 1, 0, 0);  // lands zero-extended in dword slot `lane`
+            }
+        }
+        n_issue++;
+        if (it_tile < tile_b) it_tile++;
+    };
+    if (working)
+        for (int s = 0; s < NS - 1; s++) issue();
+    // the activation digits are prepared while the first weight tiles are on their way (the ring's last
+    // slot is still free and serves as scratch)
+    Mx4Step st[kMx4MaxSteps];
+#pragma unroll
+    for (int s = 0; s < kMx4MaxSteps; s++)
+        if (working && (uint32_t)s < cw) st[s] = mx4_setup_step(j.x, step0 + s, k, lane, ring + (NS - 1) * slot_bytes);
+
+    uint32_t n_use = 0;
+    for (uint32_t tb = 0; tb < nt; tb += R) {
+        float *pb = part + parity * (R * 16 * nw_launch * 2);
+        const uint32_t nbt = min((uint32_t)R, nt - tb);
+        if (working) {
+            for (uint32_t tl = 0; tl < nbt; tl++) {
+                issue();
+                switch (cw) {  // at most NS-1 younger wave-tiles in flight: the oldest has landed
+                    LARQL_MX4_WAIT_CASE(1) LARQL_MX4_WAIT_CASE(2) LARQL_MX4_WAIT_CASE(3) LARQL_MX4_WAIT_CASE(4)
+                }
+                asm volatile("" ::: "memory");
+                const uint8_t *slot = ring + (n_use % NS) * slot_bytes;
+                f32x4 D = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s = 0; s < kMx4MaxSteps; s++) {
+                    if ((uint32_t)s < cw) {
+                        const u32x4 q = *reinterpret_cast<const u32x4 *>(slot + s * 1024 + lane * 16);
+                        uint32_t sc = *reinterpret_cast<const uint32_t *>(slot + cw * 1024 + s * 256 + lane * 4) & 0xFFu;
+                        const bool live = valid[s] && sc != 0;  // e8m0 0 is 0.0 here; blocks past the row end do not exist
+                        sc = valid[s] ? sc : 127u;
+                        i32x8 b = {0, 0, 0, 0, 0, 0, 0, 0};
+                        b[0] = live ? (int)q.x : 0; b[1] = live ? (int)q.y : 0; b[2] = live ? (int)q.z : 0; b[3] = live ? (int)q.w : 0;
+                        D = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st[s].a, b, D, 0, 4, 0, st[s].scale_a, 0, (int)sc);
+                    }
+                }
+                n_use++;
+                const float v = (D[0] + D[1]) + (D[2] + D[3]);  // digits 4rq..4rq+3 of weight row jr
+                if (kg < 2) pb[(tl * 16 + jr) * PW + wv * 2 + kg] = v;
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        const uint32_t row_base = (tile_a + tb) * 16;
+        const uint32_t nwork = min(nwj, (steps + cw - 1) / cw);
+        for (uint32_t rr = threadIdx.x >> 1; rr < nbt * 16; rr += blockDim.x >> 1) {
+            const uint32_t h = threadIdx.x & 1u;
+            float s = 0.f;
+            for (uint32_t w = 0; w < nwork; w++) s += pb[rr * PW + w * 2 + h];
+            s = dpp_add<0xB1>(s);  // quad_perm [1,0,3,2]
+            if (h == 0 && row_base + rr < rows) ((g_f32wp)j.out)[row_base + rr] = s;
         }
         parity ^= 1u;
     }
@@ -876,6 +1049,36 @@ __global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_mfma_kernel(GemvLa
     LARQL_WAIT_VMCNT(0);
 }
 
+// MXFP4 on the matrix cores: same sweep as the Q4_K kernel (cost unit = one tile x one 128-element step).
+__global__ void __launch_bounds__(kMx4MaxWaves * 64) gemv_mxfp4_mfma_kernel(GemvLaunch L) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t mx4_lds[];
+    const GemvJob *jobs = L.table ? L.table : L.inl;
+    const uint64_t P = L.total_passes;
+    uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
+    const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
+    uint32_t lo = 0, hi = L.n_jobs;
+    while (lo + 1 < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (jobs[mid].pass_begin <= p) lo = mid; else hi = mid;
+    }
+    uint32_t ji = lo, parity = 0;
+    while (p < p_end) {
+        GemvJob j = jobs[ji];
+        if (j.sel) {  // run-time expert selection: one bank of equally shaped matrices
+            const uint32_t e = __builtin_amdgcn_readfirstlane(*(const GLOBAL_AS uint32_t *)j.sel);
+            j.w += (size_t)e * j.w_sel_stride;
+            j.aux += (size_t)e * j.aux_sel_stride;
+        }
+        const uint32_t seg_end = min(p_end, j.pass_begin + j.n_pass);
+        const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin;
+        const uint32_t tile_a = (a + j.cpr - 1) / j.cpr, tile_b = (b + j.cpr - 1) / j.cpr;
+        if (tile_a < tile_b) run_mxfp4_mfma(j, tile_a, tile_b, mx4_lds, L.pad, parity);
+        p = seg_end;
+        ji++;
+    }
+    LARQL_WAIT_VMCNT(0);
+}
+
 // ---------------------------------------------------------------------------
 // Host side: geometry and launch.
 // ---------------------------------------------------------------------------
@@ -908,7 +1111,19 @@ static uint32_t q4k_mfma_waves(uint64_t cpr) {
 
 static int g_q4k_mfma = getenv("LARQL_HIP_Q4K_MFMA") ? atoi(getenv("LARQL_HIP_Q4K_MFMA")) : 1;
 
+static int g_mxfp4_mfma = getenv("LARQL_HIP_MXFP4_MFMA") ? atoi(getenv("LARQL_HIP_MXFP4_MFMA")) : 1;
+
+// MXFP4 on the matrix cores: 128-element steps per wavefront (1..4) so that at most 10 wavefronts cover a row
+static uint32_t mx4_steps_per_wave(uint64_t steps) {
+    for (uint32_t cw = 1; cw <= (uint32_t)kMx4MaxSteps; cw++)
+        if ((steps + cw - 1) / cw <= (uint64_t)kMx4MaxWaves) return cw;
+    return 0;  // row too long for this path
+}
+
 int gemv_effective_kind(const GemvJob &j) {
+    if (j.kind == KIND_MXFP4 && g_mxfp4_mfma && j.k >= 32 && j.k % 32 == 0 && mx4_steps_per_wave((j.k + 127) / 128) != 0 &&
+        j.rows < 0x7FFFFFF0ull)
+        return KIND_MXFP4_MFMA;
     if (j.kind == KIND_Q4K && g_q4k_mfma && !j.sel && j.k % 256 == 0 && j.k / 256 >= 1 && q4k_mfma_waves(j.k / 256) != 0 &&
         j.rows < 0x7FFFFFF0ull && (j.k / 256) * 144 * j.rows < (1ull << 62))
         return KIND_Q4K_MFMA;
@@ -916,6 +1131,22 @@ int gemv_effective_kind(const GemvJob &j) {
 }
 
 bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
+    if (j.kind == KIND_MXFP4_MFMA) {
+        if (j.k == 0 || j.k % 32 != 0) return false;
+        const uint64_t steps = (j.k + 127) / 128;
+        const uint32_t cw = mx4_steps_per_wave(steps);
+        if (cw == 0) return false;
+        const uint32_t nw = (uint32_t)((steps + cw - 1) / cw);
+        if (nw * 64 > threads) return false;
+        j.cpr = (uint32_t)steps;   // cost units per tile: one per 128-element step
+        j.rpp = nw;                // wavefronts that work on this job
+        j.pad = (int32_t)cw;       // steps per wavefront
+        j.row_bytes = (j.k / 32) * 16;
+        const uint64_t tiles = (j.rows + 15) / 16;
+        if (tiles * steps > 0x7FFFFFFFull) return false;
+        j.n_pass = (uint32_t)(tiles * steps);
+        return true;
+    }
     if (j.kind == KIND_Q4K_MFMA) {
         if (j.k == 0 || j.k % 256 != 0) return false;
         const uint64_t cpr = j.k / 256;
@@ -951,6 +1182,16 @@ bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
 }
 
 uint32_t gemv_pick_threads(const GemvJob *jobs, size_t n) {
+    if (n > 0 && jobs[0].kind == KIND_MXFP4_MFMA) {
+        uint32_t nw = 0;
+        for (size_t i = 0; i < n; i++) {
+            const uint64_t steps = (jobs[i].k + 127) / 128;
+            const uint32_t cw = mx4_steps_per_wave(steps);
+            if (cw == 0) return 0;
+            nw = std::max(nw, (uint32_t)((steps + cw - 1) / cw));
+        }
+        return nw * 64;
+    }
     if (n > 0 && jobs[0].kind == KIND_Q4K_MFMA) {
         uint32_t nw = 0;
         for (size_t i = 0; i < n; i++) {
@@ -986,7 +1227,20 @@ uint32_t gemv_pick_threads(const GemvJob *jobs, size_t n) {
     return pick;
 }
 
+uint32_t gemv_launch_param(const GemvJob *jobs, size_t n) {
+    if (n > 0 && jobs[0].kind == KIND_MXFP4_MFMA) {  // ring slot: room for the longest K-range a wavefront owns
+        uint32_t cw = 1;
+        for (size_t i = 0; i < n; i++) cw = std::max(cw, mx4_steps_per_wave((jobs[i].k + 127) / 128));
+        return cw * kMx4StepBytes;
+    }
+    return 0;
+}
+
 size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
+    if (n > 0 && jobs[0].kind == KIND_MXFP4_MFMA) {
+        const size_t nw = threads / 64;
+        return nw * kMx4Stages * gemv_launch_param(jobs, n) + 2 * (size_t)kMx4BatchTiles * 16 * nw * 2 * sizeof(float);
+    }
     if (n > 0 && jobs[0].kind == KIND_Q4K_MFMA) {
         const size_t nw = threads / 64;
         bool multi = false;  // some row needs several column passes: room for the prepared activations
@@ -1004,7 +1258,7 @@ size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
 }
 
 uint32_t gemv_wgs_per_cu(int kind, uint32_t threads, size_t lds, uint32_t dflt) {
-    if (kind != KIND_Q4K_MFMA) return dflt;
+    if (kind != KIND_Q4K_MFMA && kind != KIND_MXFP4_MFMA) return dflt;
     // as many workgroups as LDS (160 KB per CU) allows, up to 12 wavefronts per CU (3 per SIMD at this register count)
     const uint32_t by_lds = (uint32_t)((160 * 1024) / lds), by_waves = 12 / (threads / 64);
     const uint32_t w = by_lds < by_waves ? by_lds : by_waves;
@@ -1013,6 +1267,16 @@ uint32_t gemv_wgs_per_cu(int kind, uint32_t threads, size_t lds, uint32_t dflt) 
 
 hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32_t threads, uint32_t grid, size_t lds) {
     switch (kind) {
+        case KIND_MXFP4_MFMA: {
+            static bool attr_set_mx4 = false;
+            if (!attr_set_mx4) {
+                hipError_t e = hipFuncSetAttribute((const void *)gemv_mxfp4_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                if (e != hipSuccess) return e;
+                attr_set_mx4 = true;
+            }
+            hipLaunchKernelGGL(gemv_mxfp4_mfma_kernel, dim3(grid), dim3(threads), lds, stream, L);
+            break;
+        }
         case KIND_Q4K_MFMA: {
             static bool attr_set = false;  // dynamic LDS above 64 KB has to be allowed once per process
             if (!attr_set) {

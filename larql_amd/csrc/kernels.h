@@ -8,7 +8,8 @@ namespace larql {
 
 enum GemvKind : int32_t {
     KIND_Q4K = 0, KIND_Q8_0 = 1, KIND_MXFP4 = 2, KIND_Q4_0 = 3, KIND_BF16 = 4, KIND_F16 = 5, KIND_F32 = 6,
-    KIND_Q4K_MFMA = 7  // internal: Q4_K rows short enough for the matrix-core kernel (see gemv_effective_kind)
+    KIND_Q4K_MFMA = 7,   // internal: Q4_K rows short enough for the matrix-core kernel (see gemv_effective_kind)
+    KIND_MXFP4_MFMA = 8  // internal: likewise for MXFP4
 };
 
 constexpr int kGemvMaxThreads = 512;
@@ -47,6 +48,7 @@ bool gemv_job_geometry(GemvJob &j, uint32_t threads);
 uint32_t gemv_pick_threads(const GemvJob *jobs, size_t n);
 size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads);
 int gemv_effective_kind(const GemvJob &j);
+uint32_t gemv_launch_param(const GemvJob *jobs, size_t n);  // goes into GemvLaunch::pad
 uint32_t gemv_wgs_per_cu(int kind, uint32_t threads, size_t lds, uint32_t dflt);
 hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32_t threads, uint32_t grid, size_t lds);
 hipError_t copy_launch(hipStream_t stream, const void *src, void *dst, size_t bytes, uint32_t grid);
