@@ -11,11 +11,14 @@
 //
 // Each score becomes a 64-bit key (ordered score bits, then ~index), so one
 // unsigned compare decides everything and index recovery needs no side array.
-// One workgroup serves one row: every wavefront keeps a sorted top-64 in
-// registers (one key per lane), folds 64-score chunks into it with a bitonic
-// sort + bitonic merge done by cross-lane shuffles, skipping chunks that cannot
-// beat the current 64th key; the wavefronts' lists are then merged by the first
-// wavefront through LDS.
+// One workgroup serves one row, each thread a contiguous run of indices.
+// The K-th largest ordered-score value T is found exactly by a 4-pass radix
+// select (8 bits per pass, a 256-bin histogram in LDS per pass, one wavefront
+// scanning the bins from the top); scores above T are taken, and of the scores
+// equal to T the lowest indices fill the remaining places (ranked by a prefix
+// count in index order).  The <= 64 winners are gathered in LDS and one
+// wavefront orders them best-first with a bitonic sort done by cross-lane
+// shuffles.  Cost is a handful of passes over the row, whatever its order.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -66,20 +69,13 @@ __device__ __forceinline__ uint64_t sort_desc(uint64_t key, uint32_t lane) {
     return key;
 }
 
-// fold a sorted-descending list `in` into the sorted-descending `top`
-__device__ __forceinline__ uint64_t fold_sorted(uint64_t top, uint64_t in_desc, uint32_t lane) {
-    const uint64_t rev = shfl_u64(in_desc, 63 - (int)lane);
-    const uint64_t m = top > rev ? top : rev;  // the 64 largest of the union, bitonic
-    return merge_desc(m, lane);
-}
-
 template <bool BY_ABS>
 __device__ __forceinline__ uint64_t make_key(float s, uint32_t idx, int *nan_flag) {
     const uint32_t bits = __builtin_bit_cast(uint32_t, s);
     uint32_t ord;
     if (BY_ABS) {
         ord = bits & 0x7FFFFFFFu;
-        if (ord > 0x7F800000u) { atomicOr(nan_flag, 1); ord = 0; }
+        if (ord > 0x7F800000u) { if (nan_flag) atomicOr(nan_flag, 1); ord = 0; }
         ord += 1;  // keep every real score above the padding key 0
     } else {
         if ((bits & 0x7F800000u) == 0x7F800000u) return 0;  // inf / NaN are skipped
@@ -92,29 +88,98 @@ template <bool BY_ABS>
 __global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restrict__ scores, uint32_t n, uint32_t k,
                                                             uint32_t *__restrict__ idx_out, float *__restrict__ val_out,
                                                             uint32_t *__restrict__ count_out, int *nan_flag) {
-    __shared__ uint64_t lists[kTopkWaves][64];
-    const uint32_t row = blockIdx.x;
+    __shared__ uint32_t hist[256];
+    __shared__ uint32_t wave_ties[kTopkWaves];
+    __shared__ uint64_t winners[64];
+    __shared__ uint32_t sh_prefix, sh_need, sh_nwin;
+    const uint32_t row = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const float *s = scores + (size_t)row * n;
-    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    uint64_t top = 0;
-    // wave w takes chunks w, w+16, ... of 64 consecutive scores
-    for (uint32_t base = wave * 64; base < n; base += kTopkThreads) {
-        const uint32_t i = base + lane;
-        uint64_t key = i < n ? make_key<BY_ABS>(s[i], i, nan_flag) : 0;
-        const uint64_t thr = shfl_u64(top, 63);
-        if (__ballot(key > thr) == 0) continue;
-        key = sort_desc(key, lane);
-        top = fold_sorted(top, key, lane);
+    // wavefront w owns the contiguous indices [w0, w1), 64 at a time (lane = index within the 64)
+    const uint32_t perw = ((n + kTopkWaves * 64 - 1) / (kTopkWaves * 64)) * 64;
+    const uint32_t w0 = min(n, wave * perw), w1 = min(n, w0 + perw);
+
+    if (tid < 64) winners[tid] = 0;
+    if (tid == 0) { sh_prefix = 0; sh_need = k; sh_nwin = 0; }
+    // ---- radix select of the k-th largest ordered score: 8 bits per pass, top byte first ----
+    for (int pass = 0; pass < 4; pass++) {
+        const int sh = 24 - 8 * pass;
+        if (tid < 256) hist[tid] = 0;
+        __syncthreads();
+        const uint32_t prefix = sh_prefix;
+        for (uint32_t i = w0 + lane; i < w1; i += 64) {
+            const uint32_t ord = (uint32_t)(make_key<BY_ABS>(s[i], i, pass == 0 ? nan_flag : nullptr) >> 32);
+            // 64-bit shift: the first pass compares nothing (shift by 32)
+            if (ord != 0 && ((uint64_t)ord >> (sh + 8)) == ((uint64_t)prefix >> (sh + 8))) atomicAdd(&hist[(ord >> sh) & 255u], 1u);
+        }
+        __syncthreads();
+        if (wave == 0) {
+            // lane l holds bins 255-4l .. 252-4l (descending); find the bin where the running count reaches `need`
+            const uint32_t need = sh_need;
+            const uint32_t b0 = 255u - 4u * lane;
+            const uint32_t c0 = hist[b0], c1 = hist[b0 - 1], c2 = hist[b0 - 2], c3 = hist[b0 - 3];
+            const uint32_t mine = c0 + c1 + c2 + c3;
+            uint32_t incl = mine;  // inclusive scan over lanes (bins in descending order)
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const uint32_t t = (uint32_t)__shfl_up((int)incl, o, 64);
+                if (lane >= (uint32_t)o) incl += t;
+            }
+            const uint32_t before = incl - mine;
+            const bool here = before < need && incl >= need;
+            if (here) {
+                uint32_t acc = before, bin = b0, above = before;
+                const uint32_t c[4] = {c0, c1, c2, c3};
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    if (acc < need && acc + c[q] >= need) { bin = b0 - q; above = acc; }
+                    acc += c[q];
+                }
+                sh_prefix = prefix | (bin << sh);
+                sh_need = need - above;  // still to find inside the chosen bin
+            }
+            // fewer than `need` valid scores in total: nobody is `here`; prefix stays and everything valid is taken
+            const uint32_t total = (uint32_t)__shfl((int)incl, 63, 64);
+            if (lane == 0 && total < need) { sh_need = 0xFFFFFFFFu; }
+        }
+        __syncthreads();
+        if (sh_need == 0xFFFFFFFFu) break;
     }
-    lists[wave][lane] = top;
+    const bool take_all = sh_need == 0xFFFFFFFFu;
+    const uint32_t T = take_all ? 0u : sh_prefix;     // scores with ord > T are in
+    const uint32_t r = take_all ? 0xFFFFFFFFu : sh_need;  // this many of the scores with ord == T, lowest indices first
+    // ---- rank the ties in index order: per-wavefront counts, then ballots inside the wavefront ----
+    uint32_t my_ties = 0;
+    if (!take_all)
+        for (uint32_t base = w0; base < w1; base += 64) {
+            const uint32_t i = base + lane;
+            const bool tie = i < w1 && (uint32_t)(make_key<BY_ABS>(s[i], i, nullptr) >> 32) == T;
+            my_ties += (uint32_t)__popcll(__ballot(tie));
+        }
+    if (lane == 0) wave_ties[wave] = my_ties;
+    __syncthreads();
+    uint32_t tie_rank = 0;  // ties at lower indices than this wavefront's current 64
+    for (uint32_t w = 0; w < wave; w++) tie_rank += wave_ties[w];
+    // ---- gather the winners ----
+    for (uint32_t base = w0; base < w1; base += 64) {
+        const uint32_t i = base + lane;
+        const uint64_t key = i < w1 ? make_key<BY_ABS>(s[i], i, nullptr) : 0;
+        const uint32_t ord = (uint32_t)(key >> 32);
+        bool in = ord != 0 && ord > T;
+        if (!take_all) {
+            const bool tie = ord != 0 && ord == T;
+            const uint64_t m = __ballot(tie);
+            const uint32_t before = (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
+            if (tie) in = tie_rank + before < r;
+            tie_rank += (uint32_t)__popcll(m);
+        }
+        if (in) {
+            const uint32_t pos = atomicAdd(&sh_nwin, 1u);
+            if (pos < 64) winners[pos] = key;
+        }
+    }
     __syncthreads();
     if (wave == 0) {
-        for (int w = 1; w < kTopkWaves; w++) {
-            const uint64_t in = lists[w][lane];
-            const uint64_t thr = shfl_u64(top, 63);
-            if (__ballot(in > thr) == 0) continue;
-            top = fold_sorted(top, in, lane);
-        }
+        const uint64_t top = sort_desc(winners[lane], lane);
         const bool valid = top != 0 && lane < k;
         if (valid) {
             const uint32_t idx = ~(uint32_t)top;
