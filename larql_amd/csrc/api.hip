@@ -191,10 +191,10 @@ std::vector<std::vector<GemvJob>> group_by_kind(const std::vector<GemvJob> &jobs
     std::vector<GemvJob> jobs(jobs_in);
     for (GemvJob &j : jobs) j.kind = gemv_effective_kind(j);  // Q4_K rows the matrix-core kernel takes get their own launch
     std::vector<std::vector<GemvJob>> groups;
-    bool done[9] = {false, false, false, false, false, false, false, false, false};
+    bool done[10] = {false, false, false, false, false, false, false, false, false, false};
     for (size_t i = 0; i < jobs.size(); i++) {
         const int kind = jobs[i].kind;
-        if (jobs[i].rows == 0 || kind < 0 || kind > 8 || done[kind]) continue;
+        if (jobs[i].rows == 0 || kind < 0 || kind > 9 || done[kind]) continue;
         done[kind] = true;
         std::vector<GemvJob> live;
         for (size_t t = i; t < jobs.size(); t++)
@@ -684,6 +684,20 @@ static size_t format_row_bytes(int kind, size_t k) {
     }
 }
 
+// One gate matrix against `batch` residual positions (x: [batch, hidden], scores: [batch, n]): jobs that
+// carry as many positions as the kernels take at once, so the matrix is read once per group.
+static void push_gate_jobs(std::vector<GemvJob> &jobs, int kind, const void *gate, const float *x, size_t batch, size_t n,
+                           size_t hidden, float *scores) {
+    const size_t cap = gemv_batch_capacity(kind, hidden);
+    for (size_t b = 0; b < batch;) {
+        const size_t take = std::min(cap, batch - b);
+        GemvJob j = make_job(kind, gate, nullptr, x + b * hidden, scores + b * n, n, hidden);
+        if (take >= 2) { j.batch = (uint32_t)take; j.x_stride = hidden; j.out_stride = n; }
+        jobs.push_back(j);
+        b += take;
+    }
+}
+
 // scores[batch, n] on the device for resident gate + x (x: [batch, hidden] f32)
 static int dev_gate_scores(larql_hip_ctx *c, int kind, const void *gate, const float *x, size_t batch, size_t n, size_t hidden,
                            float *scores) {
@@ -697,7 +711,7 @@ static int dev_gate_scores(larql_hip_ctx *c, int kind, const void *gate, const f
             jobs.push_back(make_job(kind, gate, (const float *)c->q8s.p + b * (hidden / 32), (const int8_t *)c->q8.p + b * hidden,
                                     scores + b * n, n, hidden));
     } else {
-        for (size_t b = 0; b < batch; b++) jobs.push_back(make_job(kind, gate, nullptr, x + b * hidden, scores + b * n, n, hidden));
+        push_gate_jobs(jobs, kind, gate, x, batch, n, hidden, scores);
     }
     return enqueue_jobs(c, jobs);
 }
@@ -1049,8 +1063,7 @@ int larql_hip_dev_gate_walk(larql_hip_ctx *c, int format, const void *const *gat
     std::vector<GemvJob> jobs;
     jobs.reserve(n_layers * batch);
     for (size_t l = 0; l < n_layers; l++)
-        for (size_t b = 0; b < batch; b++)
-            jobs.push_back(make_job(kind, gates[l], nullptr, x + l * x_layer_stride + b * hidden, scores_scratch + (l * batch + b) * n, n, hidden));
+        push_gate_jobs(jobs, kind, gates[l], x + l * x_layer_stride, batch, n, hidden, scores_scratch + l * batch * n);
     rc = enqueue_jobs(c, jobs);
     if (rc) return rc;
     HIPCHECK(c, topk_launch(c->stream, scores_scratch, (uint32_t)(n_layers * batch), (uint32_t)n, (uint32_t)top_k, true, idx_out,

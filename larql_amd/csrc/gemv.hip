@@ -821,6 +821,144 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
     }
 }
 
+// ---------------------------------------------------------------------------
+// bf16 rows against 2..8 activations at once (gate-KNN over several residual positions): the gate
+// matrix is read once.  v_mfma_f32_16x16x32_bf16 with the roles swapped as above: the 16 "B" columns are
+// 16 weight rows (a lane's operand is 16 contiguous bytes of its row, straight from the LDS ring), the
+// "A" rows carry the activations: row 4t + i of set s holds term i of position 4s + t, where
+// x = hi + mid + lo is split into three bf16 terms (exact: each term takes the next 8 significant
+// bits) and row 4t + 3 is zero.  A wavefront owns 128 elements (4 MFMA steps) of the row per column pass,
+// at most 2 passes (K <= 2560), and keeps all its A operands in registers.  Lane (j, rq) ends with the
+// three term sums of position 4s + rq for weight row j.  Dot as bf16_dot_portable
+// (larql-vindex/.../opplan/exec/cpu/kernels.rs:718-723); only the summation order differs.
+// ---------------------------------------------------------------------------
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+constexpr int kBfStages = 3;
+constexpr int kBfBatchTiles = 2;
+constexpr int kBfMaxPasses = 2;
+constexpr int kBfMaxSets = 2;       // 4 positions each
+constexpr int kBfMaxWaves = 10;
+constexpr uint32_t kBfTileBytes = 4 * 1024;  // 16 rows x 4 steps x 64 B
+
+union BfOp { bf16x8_t v; uint32_t u[4]; };
+
+__device__ __forceinline__ uint32_t bf16_term_bits(float &r) {  // next 8 significant bits of r; r keeps the rest
+    const uint32_t b = __builtin_bit_cast(uint32_t, r) & 0xFFFF0000u;
+    r -= __builtin_bit_cast(float, b);  // exact
+    return b >> 16;
+}
+
+// A operand of one step: lane (i = lane%16, kq) holds term i%4 of position pos0 + i/4, elements 8kq..8kq+7
+__device__ __forceinline__ BfOp bf16_mfma_operand(const float *x, uint64_t x_stride, uint32_t pos0, uint32_t batch, uint32_t k0,
+                                                  uint32_t lane) {
+    const uint32_t i = lane & 15u, kq = lane >> 4, pos = pos0 + (i >> 2), term = i & 3u;
+    BfOp op;
+    op.u[0] = op.u[1] = op.u[2] = op.u[3] = 0u;
+    if (pos < batch && term < 3) {
+        g_f4p xp = (g_f4p)(x + (size_t)pos * x_stride + k0 + 8 * kq);
+        const f32x4 a = xp[0], b = xp[1];
+        float e[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        uint32_t h[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            uint32_t t0 = bf16_term_bits(e[q]);
+            const uint32_t t1 = bf16_term_bits(e[q]), t2 = bf16_term_bits(e[q]);
+            h[q] = term == 0 ? t0 : (term == 1 ? t1 : t2);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; q++) op.u[q] = h[2 * q] | (h[2 * q + 1] << 16);
+    }
+    return op;
+}
+
+__device__ __forceinline__ void run_bf16_mfma(const GemvJob &j, uint32_t tile_a, uint32_t tile_b, uint8_t *lds, uint32_t &parity) {
+    constexpr int NS = kBfStages, R = kBfBatchTiles;
+    const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t nw_launch = blockDim.x >> 6;
+    const uint32_t jr = lane & 15u, kq = lane >> 4;
+    const uint32_t nwj = j.rpp, cols = j.cpr, batch = j.batch, nsets = (batch + 3) / 4;
+    const uint32_t rows = (uint32_t)j.rows;
+    const size_t row_bytes = j.row_bytes;
+    uint8_t *ring = lds + wv * (NS * kBfTileBytes);
+    float *part = reinterpret_cast<float *>(lds + nw_launch * (NS * kBfTileBytes));
+    const uint32_t np = wv < nwj ? (cols - wv + nwj - 1) / nwj : 0;  // columns wv, wv+nwj of this wavefront
+    const uint32_t PW = 8 * nw_launch;                              // partials per row: [position][wavefront]
+
+    const uint32_t nt = tile_b - tile_a;
+    uint32_t it_tile = tile_a, it_p = 0, n_issue = 0;
+    auto issue = [&]() {
+        const uint32_t tl = min(it_tile, tile_b - 1);  // past the end: the last wave-tile again (uniform load counts)
+        const uint32_t row = min(tl * 16 + jr, rows - 1);
+        const uint8_t *gp = j.w + (size_t)row * row_bytes + (size_t)(wv + nwj * it_p) * 256 + kq * 16;
+        uint8_t *lp = ring + (n_issue % NS) * kBfTileBytes;
+#pragma unroll
+        for (int s = 0; s < 4; s++) __builtin_amdgcn_global_load_lds((g_vp)(gp + s * 64), (lds_vp)(lp + s * 1024), 16, 0, 0);
+        n_issue++;
+        if (it_tile < tile_b && ++it_p == np) { it_p = 0; it_tile++; }
+    };
+    if (np >= 1)
+        for (int s = 0; s < NS - 1; s++) issue();
+
+    // A operands of every (pass, step, set) of this wavefront, prepared while the first tiles are on their way
+    BfOp xa[kBfMaxPasses][4][kBfMaxSets];
+#pragma unroll
+    for (int p = 0; p < kBfMaxPasses; p++)
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+#pragma unroll
+            for (int q = 0; q < kBfMaxSets; q++)
+                if ((uint32_t)p < np && (uint32_t)q < nsets)
+                    xa[p][s][q] = bf16_mfma_operand(j.x, j.x_stride, 4 * q, batch, ((wv + nwj * p) * 4 + s) * 32, lane);
+
+    uint32_t n_use = 0;
+    for (uint32_t tb = 0; tb < nt; tb += R) {
+        float *pb = part + parity * (R * 16 * PW);
+        const uint32_t nbt = min((uint32_t)R, nt - tb);
+        if (np >= 1) {
+            for (uint32_t tl = 0; tl < nbt; tl++) {
+                f32x4 D[kBfMaxSets];
+#pragma unroll
+                for (int q = 0; q < kBfMaxSets; q++) D[q] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int p = 0; p < kBfMaxPasses; p++) {
+                    if ((uint32_t)p < np) {
+                        issue();
+                        LARQL_WAIT_VMCNT(4 * (NS - 1));  // the oldest wave-tile in flight has landed
+                        asm volatile("" ::: "memory");
+                        const uint8_t *slot = ring + (n_use % NS) * kBfTileBytes;
+#pragma unroll
+                        for (int s = 0; s < 4; s++) {
+                            BfOp b;
+                            const u32x4 q4 = *reinterpret_cast<const u32x4 *>(slot + s * 1024 + lane * 16);
+                            b.u[0] = q4.x; b.u[1] = q4.y; b.u[2] = q4.z; b.u[3] = q4.w;
+#pragma unroll
+                            for (int q = 0; q < kBfMaxSets; q++)
+                                if ((uint32_t)q < nsets) D[q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[p][s][q].v, b.v, D[q], 0, 0, 0);
+                        }
+                        n_use++;
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < kBfMaxSets; q++) {
+                    const uint32_t pos = 4 * q + kq;  // lane (jr, kq) holds the terms of position 4q + kq
+                    if ((uint32_t)q < nsets && pos < batch) pb[(tl * 16 + jr) * PW + pos * nw_launch + wv] = (D[q][0] + D[q][1]) + D[q][2];
+                }
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        const uint32_t row_base = (tile_a + tb) * 16, nwork = min(nwj, cols);
+        for (uint32_t e = threadIdx.x; e < nbt * 16 * batch; e += blockDim.x) {
+            const uint32_t rr = e / batch, pos = e - rr * batch;
+            float s = 0.f;
+            for (uint32_t w = 0; w < nwork; w++) s += pb[rr * PW + pos * nw_launch + w];
+            if (row_base + rr < rows) ((g_f32wp)j.out)[(size_t)pos * j.out_stride + row_base + rr] = s;
+        }
+        parity ^= 1u;
+    }
+}
+
 template <int U>
 __device__ __forceinline__ void run_q8_0(const GemvJob &j, uint32_t p0, uint32_t p1, float *part) {
     const uint32_t t = threadIdx.x, cpr = j.cpr, rpp = j.rpp;
@@ -1079,6 +1217,31 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) gemv_mxfp4_mfma_kernel(Gemv
     LARQL_WAIT_VMCNT(0);
 }
 
+// bf16 rows x several activations: same sweep (cost unit = one tile x one 128-element column)
+__global__ void __launch_bounds__(kBfMaxWaves * 64) gemv_bf16_mfma_kernel(GemvLaunch L) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t bf_lds[];
+    const GemvJob *jobs = L.table ? L.table : L.inl;
+    const uint64_t P = L.total_passes;
+    uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
+    const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
+    uint32_t lo = 0, hi = L.n_jobs;
+    while (lo + 1 < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (jobs[mid].pass_begin <= p) lo = mid; else hi = mid;
+    }
+    uint32_t ji = lo, parity = 0;
+    while (p < p_end) {
+        const GemvJob j = jobs[ji];
+        const uint32_t seg_end = min(p_end, j.pass_begin + j.n_pass);
+        const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin;
+        const uint32_t tile_a = (a + j.cpr - 1) / j.cpr, tile_b = (b + j.cpr - 1) / j.cpr;
+        if (tile_a < tile_b) run_bf16_mfma(j, tile_a, tile_b, bf_lds, parity);
+        p = seg_end;
+        ji++;
+    }
+    LARQL_WAIT_VMCNT(0);
+}
+
 // ---------------------------------------------------------------------------
 // Host side: geometry and launch.
 // ---------------------------------------------------------------------------
@@ -1120,7 +1283,16 @@ static uint32_t mx4_steps_per_wave(uint64_t steps) {
     return 0;  // row too long for this path
 }
 
+static int g_bf16_mfma = getenv("LARQL_HIP_BF16_MFMA") ? atoi(getenv("LARQL_HIP_BF16_MFMA")) : 1;
+
+uint32_t gemv_batch_capacity(int kind, uint64_t k) {
+    // bf16: 128-element columns, at most 10 wavefronts x 2 passes, two sets of 4 positions
+    if (kind == KIND_BF16 && g_bf16_mfma && k >= 128 && k % 128 == 0 && k / 128 <= (uint64_t)(kBfMaxWaves * kBfMaxPasses)) return 4 * kBfMaxSets;
+    return 1;
+}
+
 int gemv_effective_kind(const GemvJob &j) {
+    if (j.kind == KIND_BF16 && j.batch >= 2) return KIND_BF16_MFMA;
     if (j.kind == KIND_MXFP4 && g_mxfp4_mfma && j.k >= 32 && j.k % 32 == 0 && mx4_steps_per_wave((j.k + 127) / 128) != 0 &&
         j.rows < 0x7FFFFFF0ull)
         return KIND_MXFP4_MFMA;
@@ -1131,6 +1303,19 @@ int gemv_effective_kind(const GemvJob &j) {
 }
 
 bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
+    if (j.kind == KIND_BF16_MFMA) {
+        if (j.batch < 2 || j.batch > gemv_batch_capacity(KIND_BF16, j.k)) return false;
+        const uint64_t cols = j.k / 128;
+        const uint32_t nw = (uint32_t)std::min<uint64_t>(cols, kBfMaxWaves);
+        if (nw * 64 > threads) return false;
+        j.cpr = (uint32_t)cols;  // cost units per tile: one per 128-element column
+        j.rpp = nw;
+        j.row_bytes = j.k * 2;
+        const uint64_t tiles = (j.rows + 15) / 16;
+        if (tiles * cols > 0x7FFFFFFFull) return false;
+        j.n_pass = (uint32_t)(tiles * cols);
+        return true;
+    }
     if (j.kind == KIND_MXFP4_MFMA) {
         if (j.k == 0 || j.k % 32 != 0) return false;
         const uint64_t steps = (j.k + 127) / 128;
@@ -1182,6 +1367,11 @@ bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
 }
 
 uint32_t gemv_pick_threads(const GemvJob *jobs, size_t n) {
+    if (n > 0 && jobs[0].kind == KIND_BF16_MFMA) {
+        uint64_t nw = 0;
+        for (size_t i = 0; i < n; i++) nw = std::max<uint64_t>(nw, std::min<uint64_t>(jobs[i].k / 128, kBfMaxWaves));
+        return (uint32_t)nw * 64;
+    }
     if (n > 0 && jobs[0].kind == KIND_MXFP4_MFMA) {
         uint32_t nw = 0;
         for (size_t i = 0; i < n; i++) {
@@ -1237,6 +1427,10 @@ uint32_t gemv_launch_param(const GemvJob *jobs, size_t n) {
 }
 
 size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
+    if (n > 0 && jobs[0].kind == KIND_BF16_MFMA) {
+        const size_t nw = threads / 64;
+        return nw * kBfStages * kBfTileBytes + 2 * (size_t)kBfBatchTiles * 16 * 8 * nw * sizeof(float);
+    }
     if (n > 0 && jobs[0].kind == KIND_MXFP4_MFMA) {
         const size_t nw = threads / 64;
         return nw * kMx4Stages * gemv_launch_param(jobs, n) + 2 * (size_t)kMx4BatchTiles * 16 * nw * 2 * sizeof(float);
@@ -1258,7 +1452,7 @@ size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
 }
 
 uint32_t gemv_wgs_per_cu(int kind, uint32_t threads, size_t lds, uint32_t dflt) {
-    if (kind != KIND_Q4K_MFMA && kind != KIND_MXFP4_MFMA) return dflt;
+    if (kind != KIND_Q4K_MFMA && kind != KIND_MXFP4_MFMA && kind != KIND_BF16_MFMA) return dflt;
     // as many workgroups as LDS (160 KB per CU) allows, up to 12 wavefronts per CU (3 per SIMD at this register count)
     const uint32_t by_lds = (uint32_t)((160 * 1024) / lds), by_waves = 12 / (threads / 64);
     const uint32_t w = by_lds < by_waves ? by_lds : by_waves;
@@ -1267,6 +1461,16 @@ uint32_t gemv_wgs_per_cu(int kind, uint32_t threads, size_t lds, uint32_t dflt) 
 
 hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32_t threads, uint32_t grid, size_t lds) {
     switch (kind) {
+        case KIND_BF16_MFMA: {
+            static bool attr_set_bf = false;
+            if (!attr_set_bf) {
+                hipError_t e = hipFuncSetAttribute((const void *)gemv_bf16_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                if (e != hipSuccess) return e;
+                attr_set_bf = true;
+            }
+            hipLaunchKernelGGL(gemv_bf16_mfma_kernel, dim3(grid), dim3(threads), lds, stream, L);
+            break;
+        }
         case KIND_MXFP4_MFMA: {
             static bool attr_set_mx4 = false;
             if (!attr_set_mx4) {

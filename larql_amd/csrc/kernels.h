@@ -9,7 +9,8 @@ namespace larql {
 enum GemvKind : int32_t {
     KIND_Q4K = 0, KIND_Q8_0 = 1, KIND_MXFP4 = 2, KIND_Q4_0 = 3, KIND_BF16 = 4, KIND_F16 = 5, KIND_F32 = 6,
     KIND_Q4K_MFMA = 7,   // internal: Q4_K rows short enough for the matrix-core kernel (see gemv_effective_kind)
-    KIND_MXFP4_MFMA = 8  // internal: likewise for MXFP4
+    KIND_MXFP4_MFMA = 8, // internal: likewise for MXFP4
+    KIND_BF16_MFMA = 9   // internal: bf16 rows against 2..8 activations at once (batch field of the job)
 };
 
 constexpr int kGemvMaxThreads = 512;
@@ -34,6 +35,10 @@ struct GemvJob {
     // uses w + e*w_sel_stride, aux + e*aux_sel_stride (one bank of equally shaped matrices).
     const uint32_t *sel;
     uint64_t w_sel_stride, aux_sel_stride;
+    // Optional batch (bf16 gates): `batch` activations x + t*x_stride against the same weights, results to
+    // out + t*out_stride (strides in floats).  0 or 1 = a plain matvec.  See gemv_batch_capacity.
+    uint32_t batch, pad2;
+    uint64_t x_stride, out_stride;
 };
 
 struct GemvLaunch {
@@ -48,6 +53,7 @@ bool gemv_job_geometry(GemvJob &j, uint32_t threads);
 uint32_t gemv_pick_threads(const GemvJob *jobs, size_t n);
 size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads);
 int gemv_effective_kind(const GemvJob &j);
+uint32_t gemv_batch_capacity(int kind, uint64_t k);  // activations one job may carry (1: no batched kernel for this shape)
 uint32_t gemv_launch_param(const GemvJob *jobs, size_t n);  // goes into GemvLaunch::pad
 uint32_t gemv_wgs_per_cu(int kind, uint32_t threads, size_t lds, uint32_t dflt);
 hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32_t threads, uint32_t grid, size_t lds);

@@ -258,6 +258,25 @@ def test_gate_knn_matches_oracle(be, fmt, variant, batch):
     assert union == sorted(set(union))
 
 
+@pytest.mark.parametrize("n,hidden,batch", [(1000, 128, 2), (77, 384, 3), (4099, 2560, 5), (640, 1280, 9), (33, 2560, 17),
+                                            (500, 2688, 4), (500, 208, 3)])
+def test_bf16_gate_scores_over_several_positions(be, fmt, n, hidden, batch):
+    # several positions share one pass over a bf16 gate (up to 8 at a time where the row length allows);
+    # every position's scores must equal the single-position result, whatever the grouping
+    rng = np.random.default_rng(n + hidden + batch)
+    gate = O.f32_to_bf16((rng.standard_normal((n, hidden)) * 0.05).astype(F))
+    X = rng.standard_normal((batch, hidden)).astype(F)
+    X[0, ::7] *= 300.0           # spread of magnitudes inside a position
+    X[-1] *= 1e-12               # and between positions
+    scores = be.gate_scores_batch(fmt.FMT_BF16, gate, X, n, hidden)
+    assert scores.shape == (batch, n)
+    for b in range(batch):
+        want = O.bf16_gemv(gate, X[b], n, hidden)
+        assert rel_l2(scores[b], want) < TOL, b
+        single = be.gate_scores_batch(fmt.FMT_BF16, gate, X[b:b + 1], n, hidden)[0]
+        assert rel_l2(scores[b], single) < TOL
+
+
 def test_gate_knn_edge_cases(be, fmt):
     rng = np.random.default_rng(29)
     n, hidden = 100, 256
