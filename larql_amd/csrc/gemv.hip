@@ -959,6 +959,180 @@ __device__ __forceinline__ void run_bf16_mfma(const GemvJob &j, uint32_t tile_a,
     }
 }
 
+// ---------------------------------------------------------------------------
+// Q4_K rows against 2..4 activations at once (gate-KNN over several residual positions, rows of up to 10
+// super-blocks): same streaming and the same int8 MFMA as the single-activation kernel, with the A rows
+// re-dealt: the MFMA of group g and position pair p carries row 8t + 4cl + l = limb l of sub-block 2g+cl of
+// position 2p + t, so one MFMA per group serves two positions and lane (j, rq) ends with the four limb sums
+// of position 2p + rq/2, nibble class cl = rq%2, for its weight row j and every group.  It therefore decodes
+// the scales and mins of its class for all four groups.
+// ---------------------------------------------------------------------------
+constexpr int kQ4kBatchPairs = 2;  // positions per job: 2 * kQ4kBatchPairs
+
+struct Q4kBatchCol {
+    Q4kOp xm[4][kQ4kBatchPairs];      // A operand of (group, pair)
+    float k[kQ4kBatchPairs];          // 2^(e-27) of this lane's position in the pair
+    float sum[4][kQ4kBatchPairs];     // sum of x over sub-block 2g + cl of this lane's position
+};
+
+__device__ __forceinline__ void q4k_batch_setup(Q4kBatchCol &col, const float *x, uint64_t x_stride, uint32_t batch, uint32_t c,
+                                                uint32_t lane) {
+    const uint32_t i = lane & 15u, kq = lane >> 4;
+    const uint32_t t_a = i >> 3, cl_a = (i >> 2) & 1u, limb = i & 3u;  // this lane as A supplier: row 8t + 4cl + limb
+    const uint32_t t_p = kq >> 1, cl_p = kq & 1u;                      // this lane in the post role (rq = kq)
+#pragma unroll
+    for (int p = 0; p < kQ4kBatchPairs; p++) {
+        // column maxima and sub-block sums of both positions of the pair
+        float kk[2], sm[2];
+        int ex2[2];
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            const uint32_t pos = 2 * p + t;
+            f32x4 v = {0.f, 0.f, 0.f, 0.f};
+            if (pos < batch) v = ((g_f4p)(x + (size_t)pos * x_stride + (size_t)c * 256))[lane];
+            float mx = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+            float s4 = (v.x + v.y) + (v.z + v.w);
+#pragma unroll
+            for (int o = 1; o < 8; o <<= 1) { s4 += __shfl_xor(s4, o); mx = fmaxf(mx, __shfl_xor(mx, o)); }
+#pragma unroll
+            for (int o = 8; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+            int ex = 0;
+            if (mx > 0.f && mx < __builtin_inff()) (void)frexpf(mx, &ex);
+            ex = max(-90, min(120, ex));
+            ex2[t] = ex; kk[t] = ldexpf(1.f, ex - 27); sm[t] = s4;
+        }
+        col.k[p] = t_p ? kk[1] : kk[0];
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const float s0 = __shfl(sm[0], 8 * (2 * g + cl_p)), s1 = __shfl(sm[1], 8 * (2 * g + cl_p));
+            col.sum[g][p] = t_p ? s1 : s0;
+        }
+        // limbs of this lane's A rows
+        const uint32_t pos = 2 * p + t_a;
+        const float to_int = ldexpf(1.f, 27 - (t_a ? ex2[1] : ex2[0]));
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            f32x4 a = {0.f, 0.f, 0.f, 0.f}, b = {0.f, 0.f, 0.f, 0.f};
+            if (pos < batch) {
+                g_f4p xs = (g_f4p)(x + (size_t)pos * x_stride + (size_t)c * 256 + g * 64 + cl_a * 32 + 8 * kq);
+                a = xs[0]; b = xs[1];
+            }
+            const float e[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+            uint32_t d[8];
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                // balanced base-128 digits: n + 64*(1 + 128 + 128^2 + 128^3) has the unsigned digits l+64
+                const int n = (int)__builtin_rintf(e[q] * to_int) + 0x8102040;
+                const int dg = limb == 0 ? (n >> 21) : ((n >> (7 * (3 - (int)limb))) & 127);
+                d[q] = (uint32_t)(dg - 64) & 0xFFu;
+            }
+            const uint32_t d0 = d[0] | (d[1] << 8) | (d[2] << 16) | (d[3] << 24), d1 = d[4] | (d[5] << 8) | (d[6] << 16) | (d[7] << 24);
+            col.xm[g][p].u[0] = cl_a ? 0u : d0; col.xm[g][p].u[1] = cl_a ? 0u : d1;
+            col.xm[g][p].u[2] = cl_a ? d0 : 0u; col.xm[g][p].u[3] = cl_a ? d1 : 0u;
+        }
+    }
+}
+
+__device__ __forceinline__ void run_q4k_batch(const GemvJob &j, uint32_t tile_a, uint32_t tile_b, uint8_t *lds, uint32_t &parity) {
+    constexpr int NS = kQ4kStages, R = kQ4kBatchTiles, NP = kQ4kBatchPairs;
+    const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t nw_launch = blockDim.x >> 6;
+    const uint32_t jr = lane & 15u, kq = lane >> 4, t_p = kq >> 1, cl = kq & 1u;
+    const uint32_t nwj = j.rpp, batch = j.batch;
+    const uint32_t rows = (uint32_t)j.rows, row_bytes = (uint32_t)j.row_bytes;
+    uint8_t *ring = lds + wv * (NS * kQ4kTileBytes);
+    float *part = reinterpret_cast<float *>(lds + nw_launch * (NS * kQ4kTileBytes));
+    const bool working = wv < nwj;
+    const uint32_t PW = 2 * NP * nw_launch * 2;  // partials per row: [position][wavefront][class]
+
+    const uint32_t u0 = lane, u1 = 64 + lane, u2 = 128 + (lane >> 2);
+    const uint32_t r0 = u0 / 9, r1 = u1 / 9, r2 = u2 / 9;
+    const uint32_t w0 = (u0 - r0 * 9) * 16, w1 = (u1 - r1 * 9) * 16, w2 = (u2 - r2 * 9) * 16 + (lane & 3u) * 4;
+    const uint8_t *wcol = j.w + (size_t)wv * 144;
+    const uint32_t nt = tile_b - tile_a;
+    uint32_t it_tile = tile_a, n_issue = 0;
+    auto issue = [&]() {
+        const uint32_t rb = min(it_tile, tile_b - 1) * 16;
+        const uint8_t *g0 = wcol + (size_t)min(rb + r0, rows - 1) * row_bytes + w0;
+        const uint8_t *g1 = wcol + (size_t)min(rb + r1, rows - 1) * row_bytes + w1;
+        const uint8_t *g2 = wcol + (size_t)min(rb + r2, rows - 1) * row_bytes + w2;
+        uint8_t *lp = ring + (n_issue % NS) * kQ4kTileBytes;
+        __builtin_amdgcn_global_load_lds((g_vp)g0, (lds_vp)lp, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((g_vp)g1, (lds_vp)(lp + 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((g_vp)g2, (lds_vp)(lp + 2048), 4, 0, 0);
+        n_issue++;
+        if (it_tile < tile_b) it_tile++;
+    };
+    if (working)
+        for (int s = 0; s < NS - 1; s++) issue();
+    Q4kBatchCol col;
+    if (working) q4k_batch_setup(col, j.x, j.x_stride, batch, wv, lane);
+
+    uint32_t n_use = 0;
+    for (uint32_t tb = 0; tb < nt; tb += R) {
+        float *pb = part + parity * (R * 16 * PW);
+        const uint32_t nbt = min((uint32_t)R, nt - tb);
+        if (working) {
+            for (uint32_t tl = 0; tl < nbt; tl++) {
+                issue();
+                LARQL_WAIT_VMCNT(3 * (NS - 1));
+                asm volatile("" ::: "memory");
+                const uint8_t *sp = ring + (n_use % NS) * kQ4kTileBytes + jr * 144;
+                n_use++;
+                const u32x4 hdr = *reinterpret_cast<const u32x4 *>(sp);
+                // scales and mins of class cl for the four groups: sub-blocks cl, 2+cl, 4+cl, 6+cl (get_scale_min_k4)
+                const float d = half_bits_to_float(hdr.x & 0xFFFFu), dmin = half_bits_to_float(hdr.x >> 16);
+                const uint32_t sh01 = cl * 8u;
+                const uint32_t sc_a = hdr.y >> sh01, mn_a = hdr.z >> sh01, hi_a = hdr.w >> sh01;  // bytes cl, (cl+1), (cl+2), ...
+                float sc[4], mn[4];
+                sc[0] = d * (float)(sc_a & 63u);          mn[0] = dmin * (float)(mn_a & 63u);            // sub cl
+                sc[1] = d * (float)((sc_a >> 16) & 63u);  mn[1] = dmin * (float)((mn_a >> 16) & 63u);    // sub 2+cl
+                sc[2] = d * (float)((hi_a & 0x0Fu) | ((sc_a >> 2) & 0x30u));                             // sub 4+cl
+                mn[2] = dmin * (float)(((hi_a >> 4) & 0x0Fu) | ((mn_a >> 2) & 0x30u));
+                sc[3] = d * (float)(((hi_a >> 16) & 0x0Fu) | ((sc_a >> 18) & 0x30u));                    // sub 6+cl
+                mn[3] = dmin * (float)(((hi_a >> 20) & 0x0Fu) | ((mn_a >> 18) & 0x30u));
+                float racc[NP];
+#pragma unroll
+                for (int p = 0; p < NP; p++) racc[p] = 0.f;
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const u32x2 q = *reinterpret_cast<const u32x2 *>(sp + 16 + 32 * g + 8 * kq);
+                    Q4kOp b;
+                    b.u[0] = q.x & 0x0F0F0F0Fu; b.u[1] = q.y & 0x0F0F0F0Fu;
+                    b.u[2] = (q.x >> 4) & 0x0F0F0F0Fu; b.u[3] = (q.y >> 4) & 0x0F0F0F0Fu;
+#pragma unroll
+                    for (int p = 0; p < NP; p++) {
+                        if ((uint32_t)(2 * p) < batch) {
+                            const i32x4 z = {0, 0, 0, 0};
+                            const i32x4 D = __builtin_amdgcn_mfma_i32_16x16x64_i8(col.xm[g][p].v, b.v, z, 0, 0, 0);
+                            float dot = __builtin_fmaf((float)D[0], 128.f, (float)D[1]);
+                            dot = __builtin_fmaf(dot, 128.f, (float)D[2]);
+                            dot = __builtin_fmaf(dot, 128.f, (float)D[3]) * col.k[p];
+                            racc[p] += sc[g] * dot - mn[g] * col.sum[g][p];
+                        }
+                    }
+                }
+#pragma unroll
+                for (int p = 0; p < NP; p++) {
+                    const uint32_t pos = 2 * p + t_p;
+                    if (pos < batch) pb[(tl * 16 + jr) * PW + (pos * nw_launch + wv) * 2 + cl] = racc[p];
+                }
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        const uint32_t row_base = (tile_a + tb) * 16;
+        for (uint32_t e = threadIdx.x; e < nbt * 16 * batch; e += blockDim.x) {
+            const uint32_t rr = e / batch, pos = e - rr * batch;
+            float s = 0.f;
+            for (uint32_t w = 0; w < nwj; w++) s += pb[rr * PW + (pos * nw_launch + w) * 2] + pb[rr * PW + (pos * nw_launch + w) * 2 + 1];
+            if (row_base + rr < rows) ((g_f32wp)j.out)[(size_t)pos * j.out_stride + row_base + rr] = s;
+        }
+        parity ^= 1u;
+    }
+}
+
 template <int U>
 __device__ __forceinline__ void run_q8_0(const GemvJob &j, uint32_t p0, uint32_t p1, float *part) {
     const uint32_t t = threadIdx.x, cpr = j.cpr, rpp = j.rpp;
@@ -1242,6 +1416,31 @@ __global__ void __launch_bounds__(kBfMaxWaves * 64) gemv_bf16_mfma_kernel(GemvLa
     LARQL_WAIT_VMCNT(0);
 }
 
+// Q4_K rows x several activations: same sweep as the single-activation kernel
+__global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_batch_kernel(GemvLaunch L) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t q4kb_lds[];
+    const GemvJob *jobs = L.table ? L.table : L.inl;
+    const uint64_t P = L.total_passes;
+    uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
+    const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
+    uint32_t lo = 0, hi = L.n_jobs;
+    while (lo + 1 < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (jobs[mid].pass_begin <= p) lo = mid; else hi = mid;
+    }
+    uint32_t ji = lo, parity = 0;
+    while (p < p_end) {
+        const GemvJob j = jobs[ji];
+        const uint32_t seg_end = min(p_end, j.pass_begin + j.n_pass);
+        const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin;
+        const uint32_t tile_a = (a + j.cpr - 1) / j.cpr, tile_b = (b + j.cpr - 1) / j.cpr;
+        if (tile_a < tile_b) run_q4k_batch(j, tile_a, tile_b, q4kb_lds, parity);
+        p = seg_end;
+        ji++;
+    }
+    LARQL_WAIT_VMCNT(0);
+}
+
 // ---------------------------------------------------------------------------
 // Host side: geometry and launch.
 // ---------------------------------------------------------------------------
@@ -1288,11 +1487,14 @@ static int g_bf16_mfma = getenv("LARQL_HIP_BF16_MFMA") ? atoi(getenv("LARQL_HIP_
 uint32_t gemv_batch_capacity(int kind, uint64_t k) {
     // bf16: 128-element columns, at most 10 wavefronts x 2 passes, two sets of 4 positions
     if (kind == KIND_BF16 && g_bf16_mfma && k >= 128 && k % 128 == 0 && k / 128 <= (uint64_t)(kBfMaxWaves * kBfMaxPasses)) return 4 * kBfMaxSets;
+    // Q4_K: one wavefront per super-block column, two pairs of positions
+    if (kind == KIND_Q4K && g_q4k_mfma && k >= 256 && k % 256 == 0 && k / 256 <= (uint64_t)kQ4kMaxWaves) return 2 * kQ4kBatchPairs;
     return 1;
 }
 
 int gemv_effective_kind(const GemvJob &j) {
     if (j.kind == KIND_BF16 && j.batch >= 2) return KIND_BF16_MFMA;
+    if (j.kind == KIND_Q4K && j.batch >= 2) return KIND_Q4K_BATCH;
     if (j.kind == KIND_MXFP4 && g_mxfp4_mfma && j.k >= 32 && j.k % 32 == 0 && mx4_steps_per_wave((j.k + 127) / 128) != 0 &&
         j.rows < 0x7FFFFFF0ull)
         return KIND_MXFP4_MFMA;
@@ -1303,6 +1505,18 @@ int gemv_effective_kind(const GemvJob &j) {
 }
 
 bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
+    if (j.kind == KIND_Q4K_BATCH) {
+        if (j.batch < 2 || j.batch > gemv_batch_capacity(KIND_Q4K, j.k)) return false;
+        const uint64_t cpr = j.k / 256;
+        if (cpr * 64 > threads) return false;
+        j.cpr = (uint32_t)cpr;
+        j.rpp = (uint32_t)cpr;
+        j.row_bytes = cpr * 144;
+        const uint64_t tiles = (j.rows + 15) / 16;
+        if (tiles * cpr > 0x7FFFFFFFull) return false;
+        j.n_pass = (uint32_t)(tiles * cpr);
+        return true;
+    }
     if (j.kind == KIND_BF16_MFMA) {
         if (j.batch < 2 || j.batch > gemv_batch_capacity(KIND_BF16, j.k)) return false;
         const uint64_t cols = j.k / 128;
@@ -1367,6 +1581,11 @@ bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
 }
 
 uint32_t gemv_pick_threads(const GemvJob *jobs, size_t n) {
+    if (n > 0 && jobs[0].kind == KIND_Q4K_BATCH) {
+        uint64_t nw = 0;
+        for (size_t i = 0; i < n; i++) nw = std::max<uint64_t>(nw, jobs[i].k / 256);
+        return nw <= (uint64_t)kQ4kMaxWaves ? (uint32_t)nw * 64 : 0;
+    }
     if (n > 0 && jobs[0].kind == KIND_BF16_MFMA) {
         uint64_t nw = 0;
         for (size_t i = 0; i < n; i++) nw = std::max<uint64_t>(nw, std::min<uint64_t>(jobs[i].k / 128, kBfMaxWaves));
@@ -1427,6 +1646,10 @@ uint32_t gemv_launch_param(const GemvJob *jobs, size_t n) {
 }
 
 size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
+    if (n > 0 && jobs[0].kind == KIND_Q4K_BATCH) {
+        const size_t nw = threads / 64;
+        return nw * kQ4kStages * kQ4kTileBytes + 2 * (size_t)kQ4kBatchTiles * 16 * (2 * kQ4kBatchPairs * nw * 2) * sizeof(float);
+    }
     if (n > 0 && jobs[0].kind == KIND_BF16_MFMA) {
         const size_t nw = threads / 64;
         return nw * kBfStages * kBfTileBytes + 2 * (size_t)kBfBatchTiles * 16 * 8 * nw * sizeof(float);
@@ -1452,7 +1675,7 @@ size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
 }
 
 uint32_t gemv_wgs_per_cu(int kind, uint32_t threads, size_t lds, uint32_t dflt) {
-    if (kind != KIND_Q4K_MFMA && kind != KIND_MXFP4_MFMA && kind != KIND_BF16_MFMA) return dflt;
+    if (kind != KIND_Q4K_MFMA && kind != KIND_MXFP4_MFMA && kind != KIND_BF16_MFMA && kind != KIND_Q4K_BATCH) return dflt;
     // as many workgroups as LDS (160 KB per CU) allows, up to 12 wavefronts per CU (3 per SIMD at this register count)
     const uint32_t by_lds = (uint32_t)((160 * 1024) / lds), by_waves = 12 / (threads / 64);
     const uint32_t w = by_lds < by_waves ? by_lds : by_waves;
@@ -1461,6 +1684,16 @@ uint32_t gemv_wgs_per_cu(int kind, uint32_t threads, size_t lds, uint32_t dflt) 
 
 hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32_t threads, uint32_t grid, size_t lds) {
     switch (kind) {
+        case KIND_Q4K_BATCH: {
+            static bool attr_set_qb = false;
+            if (!attr_set_qb) {
+                hipError_t e = hipFuncSetAttribute((const void *)gemv_q4k_batch_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                if (e != hipSuccess) return e;
+                attr_set_qb = true;
+            }
+            hipLaunchKernelGGL(gemv_q4k_batch_kernel, dim3(grid), dim3(threads), lds, stream, L);
+            break;
+        }
         case KIND_BF16_MFMA: {
             static bool attr_set_bf = false;
             if (!attr_set_bf) {

@@ -277,6 +277,24 @@ def test_bf16_gate_scores_over_several_positions(be, fmt, n, hidden, batch):
         assert rel_l2(scores[b], single) < TOL
 
 
+@pytest.mark.parametrize("n,hidden,batch", [(1000, 256, 2), (77, 768, 3), (4099, 2560, 4), (640, 1280, 9), (33, 2560, 6),
+                                            (500, 2816, 4)])
+def test_q4k_gate_scores_over_several_positions(be, fmt, n, hidden, batch):
+    # up to 4 positions share one pass over a Q4_K gate (rows of up to 10 super-blocks; longer rows go one by one)
+    rng = np.random.default_rng(n + hidden + batch)
+    gate = O.quantize_q4_k((rng.standard_normal((n, hidden)) * 0.05).astype(F))
+    X = rng.standard_normal((batch, hidden)).astype(F)
+    X[0, ::7] *= 300.0
+    X[-1] *= 1e-12
+    scores = be.gate_scores_batch(fmt.FMT_Q4_K, gate, X, n, hidden)
+    assert scores.shape == (batch, n)
+    for b in range(batch):
+        want = O.q4k_matvec(gate, X[b], n, hidden)
+        assert rel_l2(scores[b], want) < TOL, b
+        single = be.gate_scores_batch(fmt.FMT_Q4_K, gate, X[b:b + 1], n, hidden)[0]
+        assert rel_l2(scores[b], single) < TOL
+
+
 def test_gate_knn_edge_cases(be, fmt):
     rng = np.random.default_rng(29)
     n, hidden = 100, 256
