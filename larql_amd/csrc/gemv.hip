@@ -1133,6 +1133,168 @@ __device__ __forceinline__ void run_q4k_batch(const GemvJob &j, uint32_t tile_a,
     }
 }
 
+// ---------------------------------------------------------------------------
+// ggml Q8_0 on the matrix cores (rows of up to 10 x 256 elements): the same streaming as Q4_K — a
+// wavefront owns a 256-element column (8 blocks of 34 B = 272 B per row, 16 rows per wave-tile, global ->
+// LDS ring) — and the same exact int8 MFMA against four-limb activations.  The weights already are int8:
+// lane (row j, kq) feeds the 16 codes of half kq%2 of block 2g + kq/2 of each block pair g (the 34-byte
+// blocks leave them 2 bytes off a dword boundary for even blocks: five aligned dwords and v_alignbit).
+// A row 4g + 2cl + i carries limb i (or 2+i) of block 2g+cl and is non-zero only in the lanes kq/2 == cl.
+// Lane (j, rq) ends with the limb sums of blocks 2rq and 2rq+1 of its row and scales them by the blocks'
+// f16 d (q8_0_gemv / row_dot, larql-compute/src/cpu/kquant_gemv.rs:67-109, sums ((q*d)*x); here d*(sum q*x)).
+// ---------------------------------------------------------------------------
+constexpr int kQ8Stages = 3;
+constexpr int kQ8BatchTiles = 4;
+constexpr int kQ8MaxWaves = 10;
+constexpr uint32_t kQ8RowBytes = 8 * 34;             // one column of one row
+constexpr uint32_t kQ8TileBytes = 16 * kQ8RowBytes;  // 4352
+
+struct Q8Col {
+    uint32_t xa[4], xb[4];  // this lane's 16 activations as limbs i / 2+i (i = lane & 1)
+    float k;                // 2^(e-27)
+};
+
+__device__ __forceinline__ Q8Col q8_mfma_setup_col(const float *x, uint32_t c, uint32_t lane) {
+    const uint32_t j = lane & 15u, kq = lane >> 4;
+    g_f4p xc = (g_f4p)(x + (size_t)c * 256);
+    const f32x4 v = xc[lane];
+    float mx = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    int ex = 0;
+    if (mx > 0.f && mx < __builtin_inff()) (void)frexpf(mx, &ex);
+    ex = max(-90, min(120, ex));
+    const float to_int = ldexpf(1.f, 27 - ex);
+    Q8Col col;
+    col.k = ldexpf(1.f, ex - 27);
+    // A row j = 4g + 2cl + i: block 2g+cl = j/2, elements 16*(kq%2) .. +15 of it
+    const uint32_t i = j & 1u;
+    g_f4p xs = (g_f4p)(x + (size_t)c * 256 + (j >> 1) * 32 + 16 * (kq & 1u));
+    uint32_t la[16], lb[16];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const f32x4 f = xs[q];
+        const float e[4] = {f.x, f.y, f.z, f.w};
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            // balanced base-128 digits: n + 64*(1 + 128 + 128^2 + 128^3) has the unsigned digits l+64
+            const int n = (int)__builtin_rintf(e[t] * to_int) + 0x8102040;
+            const int l0 = (n >> 21) - 64, l1 = ((n >> 14) & 127) - 64, l2 = ((n >> 7) & 127) - 64, l3 = (n & 127) - 64;
+            la[4 * q + t] = (uint32_t)(i ? l1 : l0) & 0xFFu;
+            lb[4 * q + t] = (uint32_t)(i ? l3 : l2) & 0xFFu;
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        col.xa[q] = la[4 * q] | (la[4 * q + 1] << 8) | (la[4 * q + 2] << 16) | (la[4 * q + 3] << 24);
+        col.xb[q] = lb[4 * q] | (lb[4 * q + 1] << 8) | (lb[4 * q + 2] << 16) | (lb[4 * q + 3] << 24);
+    }
+    return col;
+}
+
+__device__ __forceinline__ void run_q8_0_mfma(const GemvJob &j, uint32_t tile_a, uint32_t tile_b, uint8_t *lds, uint32_t &parity) {
+    constexpr int NS = kQ8Stages, R = kQ8BatchTiles;
+    const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t nw_launch = blockDim.x >> 6;
+    const uint32_t jr = lane & 15u, kq = lane >> 4;
+    const uint32_t nwj = j.rpp, PW = nwj * 4;
+    const uint32_t rows = (uint32_t)j.rows;
+    const size_t row_bytes = j.row_bytes;
+    uint8_t *ring = lds + wv * (NS * kQ8TileBytes);
+    float *part = reinterpret_cast<float *>(lds + nw_launch * (NS * kQ8TileBytes));
+    const bool working = wv < nwj;
+
+    // lane's pieces of a wave-tile in 16-byte units u = row*17 + piece: four full loads, then 256 B dword by dword
+    uint32_t rw[5], ow[5];
+#pragma unroll
+    for (int q = 0; q < 5; q++) {
+        const uint32_t u = q < 4 ? 64 * q + lane : 256 + (lane >> 2);
+        rw[q] = u / 17;
+        ow[q] = (u - rw[q] * 17) * 16 + (q < 4 ? 0 : (lane & 3u) * 4);
+    }
+    const uint8_t *wcol = j.w + (size_t)wv * kQ8RowBytes;
+    const uint32_t nt = tile_b - tile_a;
+    uint32_t it_tile = tile_a, n_issue = 0;
+    auto issue = [&]() {
+        const uint32_t rb = min(it_tile, tile_b - 1) * 16;
+        uint8_t *lp = ring + (n_issue % NS) * kQ8TileBytes;
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+            __builtin_amdgcn_global_load_lds((g_vp)(wcol + (size_t)min(rb + rw[q], rows - 1) * row_bytes + ow[q]), (lds_vp)(lp + q * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((g_vp)(wcol + (size_t)min(rb + rw[4], rows - 1) * row_bytes + ow[4]), (lds_vp)(lp + 4096), 4, 0, 0);
+        n_issue++;
+        if (it_tile < tile_b) it_tile++;
+    };
+    if (working)
+        for (int s = 0; s < NS - 1; s++) issue();
+
+    Q8Col col;
+    Q4kOp xm[8];
+    if (working) {
+        col = q8_mfma_setup_col(j.x, wv, lane);
+        const uint32_t my_g = jr >> 2, cl = (jr >> 1) & 1u;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const bool mine = my_g == (uint32_t)g && (kq >> 1) == cl;
+#pragma unroll
+            for (int q = 0; q < 4; q++) { xm[2 * g].u[q] = mine ? col.xa[q] : 0u; xm[2 * g + 1].u[q] = mine ? col.xb[q] : 0u; }
+        }
+    }
+    // this lane's 16 codes of block pair g start at byte (2g + kq/2)*34 + 2 + 16*(kq%2) of its row: the aligned
+    // dword below it and the bit offset (0 or 16)
+    const uint32_t code_off = (kq >> 1) * 34 + 2 + 16 * (kq & 1u);
+    const uint32_t code_dw = code_off & ~3u, code_sh = (code_off & 3u) * 8;
+
+    uint32_t n_use = 0;
+    for (uint32_t tb = 0; tb < nt; tb += R) {
+        float *pb = part + parity * (R * 16 * nw_launch * 4);
+        const uint32_t nbt = min((uint32_t)R, nt - tb);
+        if (working) {
+            for (uint32_t tl = 0; tl < nbt; tl++) {
+                issue();
+                LARQL_WAIT_VMCNT(5 * (NS - 1));
+                asm volatile("" ::: "memory");
+                const uint8_t *sp = ring + (n_use % NS) * kQ8TileBytes + jr * kQ8RowBytes;
+                n_use++;
+                i32x4 Da = {0, 0, 0, 0}, Db = {0, 0, 0, 0};
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const uint32_t *wp = reinterpret_cast<const uint32_t *>(sp + g * 68 + code_dw);
+                    const uint32_t w0 = wp[0], w1 = wp[1], w2 = wp[2], w3 = wp[3], w4 = wp[4];
+                    Q4kOp b;
+                    b.u[0] = __builtin_amdgcn_alignbit(w1, w0, code_sh); b.u[1] = __builtin_amdgcn_alignbit(w2, w1, code_sh);
+                    b.u[2] = __builtin_amdgcn_alignbit(w3, w2, code_sh); b.u[3] = __builtin_amdgcn_alignbit(w4, w3, code_sh);
+                    Da = __builtin_amdgcn_mfma_i32_16x16x64_i8(xm[2 * g].v, b.v, Da, 0, 0, 0);
+                    Db = __builtin_amdgcn_mfma_i32_16x16x64_i8(xm[2 * g + 1].v, b.v, Db, 0, 0, 0);
+                }
+                // this lane's pair is g = kq: Da = [b0.l0, b0.l1, b1.l0, b1.l1], Db = [b0.l2, b0.l3, b1.l2, b1.l3]
+                float dot0 = __builtin_fmaf((float)Da[0], 128.f, (float)Da[1]);
+                float dot1 = __builtin_fmaf((float)Da[2], 128.f, (float)Da[3]);
+                dot0 = __builtin_fmaf(dot0, 128.f, (float)Db[0]);
+                dot1 = __builtin_fmaf(dot1, 128.f, (float)Db[2]);
+                dot0 = __builtin_fmaf(dot0, 128.f, (float)Db[1]) * col.k;
+                dot1 = __builtin_fmaf(dot1, 128.f, (float)Db[3]) * col.k;
+                const float d0 = half_bits_to_float(*reinterpret_cast<const uint16_t *>(sp + kq * 68));
+                const float d1 = half_bits_to_float(*reinterpret_cast<const uint16_t *>(sp + kq * 68 + 34));
+                pb[(tl * 16 + jr) * PW + wv * 4 + kq] = d0 * dot0 + d1 * dot1;
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        const uint32_t row_base = (tile_a + tb) * 16;
+        for (uint32_t rr = threadIdx.x >> 2; rr < nbt * 16; rr += blockDim.x >> 2) {
+            const uint32_t qd = threadIdx.x & 3u;
+            float s = 0.f;
+            for (uint32_t k = 0; k < nwj; k++) s += pb[rr * PW + k * 4 + qd];
+            s = dpp_add<0xB1>(s);
+            s = dpp_add<0x4E>(s);
+            if (qd == 0 && row_base + rr < rows) ((g_f32wp)j.out)[row_base + rr] = s;
+        }
+        parity ^= 1u;
+    }
+}
+
 template <int U>
 __device__ __forceinline__ void run_q8_0(const GemvJob &j, uint32_t p0, uint32_t p1, float *part) {
     const uint32_t t = threadIdx.x, cpr = j.cpr, rpp = j.rpp;
@@ -1441,6 +1603,31 @@ __global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_batch_kernel(GemvL
     LARQL_WAIT_VMCNT(0);
 }
 
+// ggml Q8_0 on the matrix cores: same sweep (cost unit = one tile x one 256-element column)
+__global__ void __launch_bounds__(kQ8MaxWaves * 64) gemv_q8_0_mfma_kernel(GemvLaunch L) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t q8_lds[];
+    const GemvJob *jobs = L.table ? L.table : L.inl;
+    const uint64_t P = L.total_passes;
+    uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
+    const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
+    uint32_t lo = 0, hi = L.n_jobs;
+    while (lo + 1 < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (jobs[mid].pass_begin <= p) lo = mid; else hi = mid;
+    }
+    uint32_t ji = lo, parity = 0;
+    while (p < p_end) {
+        const GemvJob j = jobs[ji];
+        const uint32_t seg_end = min(p_end, j.pass_begin + j.n_pass);
+        const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin;
+        const uint32_t tile_a = (a + j.cpr - 1) / j.cpr, tile_b = (b + j.cpr - 1) / j.cpr;
+        if (tile_a < tile_b) run_q8_0_mfma(j, tile_a, tile_b, q8_lds, parity);
+        p = seg_end;
+        ji++;
+    }
+    LARQL_WAIT_VMCNT(0);
+}
+
 // ---------------------------------------------------------------------------
 // Host side: geometry and launch.
 // ---------------------------------------------------------------------------
@@ -1492,7 +1679,11 @@ uint32_t gemv_batch_capacity(int kind, uint64_t k) {
     return 1;
 }
 
+static int g_q8_mfma = getenv("LARQL_HIP_Q8_MFMA") ? atoi(getenv("LARQL_HIP_Q8_MFMA")) : 1;
+
 int gemv_effective_kind(const GemvJob &j) {
+    if (j.kind == KIND_Q8_0 && g_q8_mfma && j.k >= 256 && j.k % 256 == 0 && j.k / 256 <= (uint64_t)kQ8MaxWaves && j.rows < 0x7FFFFFF0ull)
+        return KIND_Q8_0_MFMA;
     if (j.kind == KIND_BF16 && j.batch >= 2) return KIND_BF16_MFMA;
     if (j.kind == KIND_Q4K && j.batch >= 2) return KIND_Q4K_BATCH;
     if (j.kind == KIND_MXFP4 && g_mxfp4_mfma && j.k >= 32 && j.k % 32 == 0 && mx4_steps_per_wave((j.k + 127) / 128) != 0 &&
@@ -1505,6 +1696,17 @@ int gemv_effective_kind(const GemvJob &j) {
 }
 
 bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
+    if (j.kind == KIND_Q8_0_MFMA) {
+        const uint64_t cpr = j.k / 256;
+        if (j.k % 256 != 0 || cpr == 0 || cpr * 64 > threads) return false;
+        j.cpr = (uint32_t)cpr;
+        j.rpp = (uint32_t)cpr;
+        j.row_bytes = (j.k / 32) * 34;
+        const uint64_t tiles = (j.rows + 15) / 16;
+        if (tiles * cpr > 0x7FFFFFFFull) return false;
+        j.n_pass = (uint32_t)(tiles * cpr);
+        return true;
+    }
     if (j.kind == KIND_Q4K_BATCH) {
         if (j.batch < 2 || j.batch > gemv_batch_capacity(KIND_Q4K, j.k)) return false;
         const uint64_t cpr = j.k / 256;
@@ -1581,7 +1783,7 @@ bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
 }
 
 uint32_t gemv_pick_threads(const GemvJob *jobs, size_t n) {
-    if (n > 0 && jobs[0].kind == KIND_Q4K_BATCH) {
+    if (n > 0 && (jobs[0].kind == KIND_Q4K_BATCH || jobs[0].kind == KIND_Q8_0_MFMA)) {
         uint64_t nw = 0;
         for (size_t i = 0; i < n; i++) nw = std::max<uint64_t>(nw, jobs[i].k / 256);
         return nw <= (uint64_t)kQ4kMaxWaves ? (uint32_t)nw * 64 : 0;
@@ -1646,6 +1848,10 @@ uint32_t gemv_launch_param(const GemvJob *jobs, size_t n) {
 }
 
 size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
+    if (n > 0 && jobs[0].kind == KIND_Q8_0_MFMA) {
+        const size_t nw = threads / 64;
+        return nw * kQ8Stages * kQ8TileBytes + 2 * (size_t)kQ8BatchTiles * 16 * nw * 4 * sizeof(float);
+    }
     if (n > 0 && jobs[0].kind == KIND_Q4K_BATCH) {
         const size_t nw = threads / 64;
         return nw * kQ4kStages * kQ4kTileBytes + 2 * (size_t)kQ4kBatchTiles * 16 * (2 * kQ4kBatchPairs * nw * 2) * sizeof(float);
@@ -1675,7 +1881,7 @@ size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
 }
 
 uint32_t gemv_wgs_per_cu(int kind, uint32_t threads, size_t lds, uint32_t dflt) {
-    if (kind != KIND_Q4K_MFMA && kind != KIND_MXFP4_MFMA && kind != KIND_BF16_MFMA && kind != KIND_Q4K_BATCH) return dflt;
+    if (kind != KIND_Q4K_MFMA && kind != KIND_MXFP4_MFMA && kind != KIND_BF16_MFMA && kind != KIND_Q4K_BATCH && kind != KIND_Q8_0_MFMA) return dflt;
     // as many workgroups as LDS (160 KB per CU) allows, up to 12 wavefronts per CU (3 per SIMD at this register count)
     const uint32_t by_lds = (uint32_t)((160 * 1024) / lds), by_waves = 12 / (threads / 64);
     const uint32_t w = by_lds < by_waves ? by_lds : by_waves;
@@ -1684,6 +1890,16 @@ uint32_t gemv_wgs_per_cu(int kind, uint32_t threads, size_t lds, uint32_t dflt) 
 
 hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32_t threads, uint32_t grid, size_t lds) {
     switch (kind) {
+        case KIND_Q8_0_MFMA: {
+            static bool attr_set_q8 = false;
+            if (!attr_set_q8) {
+                hipError_t e = hipFuncSetAttribute((const void *)gemv_q8_0_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                if (e != hipSuccess) return e;
+                attr_set_q8 = true;
+            }
+            hipLaunchKernelGGL(gemv_q8_0_mfma_kernel, dim3(grid), dim3(threads), lds, stream, L);
+            break;
+        }
         case KIND_Q4K_BATCH: {
             static bool attr_set_qb = false;
             if (!attr_set_qb) {

@@ -137,7 +137,7 @@ def test_q4k_dual_and_matmul(be):
 
 
 # ------------------------------------------------------------------ Q8_0
-@pytest.mark.parametrize("n,k", [(4099, 2560), (64, 10240), (9, 128), (1000, 2048)])
+@pytest.mark.parametrize("n,k", [(4099, 2560), (64, 10240), (9, 128), (1000, 2048), (17, 256), (333, 1792), (48, 2816)])
 def test_q8_0_gemv_matches_oracle(be, n, k):
     w, x = weights(n + k, n, k)
     w[0, :32] *= 1e-5
