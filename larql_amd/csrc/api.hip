@@ -45,6 +45,10 @@ struct larql_hip_ctx {
     std::string name, info, last_error;
     std::vector<Region> regions;
     DevBuf w[4], aux[4], x, out, tables[4], misc, scores, q8, q8s;
+    // pinned staging for job tables: the upload is asynchronous, the event says when a slot may be rewritten
+    void *table_host[4] = {nullptr, nullptr, nullptr, nullptr};
+    size_t table_host_cap[4] = {0, 0, 0, 0};
+    hipEvent_t table_ev[4] = {nullptr, nullptr, nullptr, nullptr};
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     uint8_t *log2_up = nullptr;  // 256-entry table for the MXFP4 encoder
     int *nan_flag = nullptr;
@@ -144,7 +148,7 @@ struct PreparedLaunch {
 
 // Geometry for one launch over jobs of a single format.  When the jobs do not fit
 // inline the table is uploaded into `table_dst` (synchronously: the host vector may die).
-int prepare_same_kind(larql_hip_ctx *c, std::vector<GemvJob> &live, void *table_dst, PreparedLaunch &P) {
+int prepare_same_kind(larql_hip_ctx *c, std::vector<GemvJob> &live, void *table_dst, PreparedLaunch &P, int stage_slot = -1) {
     P.kind = live[0].kind;
     P.threads = gemv_pick_threads(live.data(), live.size());
     if (P.threads == 0) return fail(c, LARQL_UNSUPPORTED, "matvec: row length not supported by the gfx950 kernels");
@@ -163,8 +167,25 @@ int prepare_same_kind(larql_hip_ctx *c, std::vector<GemvJob> &live, void *table_
         for (size_t i = 0; i < live.size(); i++) P.L.inl[i] = live[i];
         P.L.table = nullptr;
     } else {
-        HIPCHECK(c, hipMemcpyAsync(table_dst, live.data(), live.size() * sizeof(GemvJob), hipMemcpyHostToDevice, c->stream));
-        HIPCHECK(c, hipStreamSynchronize(c->stream));
+        const size_t bytes = live.size() * sizeof(GemvJob);
+        if (stage_slot >= 0) {
+            // through pinned memory: no host wait, the launch that follows on the stream sees the table
+            if (c->table_host_cap[stage_slot] < bytes) {
+                if (c->table_ev[stage_slot]) HIPCHECK(c, hipEventSynchronize(c->table_ev[stage_slot]));
+                if (c->table_host[stage_slot]) HIPCHECK(c, hipHostFree(c->table_host[stage_slot]));
+                c->table_host[stage_slot] = nullptr; c->table_host_cap[stage_slot] = 0;
+                HIPCHECK(c, hipHostMalloc(&c->table_host[stage_slot], bytes * 2, hipHostMallocDefault));
+                c->table_host_cap[stage_slot] = bytes * 2;
+            }
+            if (!c->table_ev[stage_slot]) HIPCHECK(c, hipEventCreateWithFlags(&c->table_ev[stage_slot], hipEventDisableTiming));
+            else HIPCHECK(c, hipEventSynchronize(c->table_ev[stage_slot]));  // the previous upload from this slot is done
+            memcpy(c->table_host[stage_slot], live.data(), bytes);
+            HIPCHECK(c, hipMemcpyAsync(table_dst, c->table_host[stage_slot], bytes, hipMemcpyHostToDevice, c->stream));
+            HIPCHECK(c, hipEventRecord(c->table_ev[stage_slot], c->stream));
+        } else {
+            HIPCHECK(c, hipMemcpyAsync(table_dst, live.data(), bytes, hipMemcpyHostToDevice, c->stream));
+            HIPCHECK(c, hipStreamSynchronize(c->stream));  // the host vector may die
+        }
         P.L.table = (const GemvJob *)table_dst;
     }
     P.lds = gemv_lds_bytes(live.data(), live.size(), P.threads);
@@ -211,10 +232,11 @@ int enqueue_jobs(larql_hip_ctx *c, std::vector<GemvJob> &jobs) {
     if (rc) return rc;
     int slot = 0;
     for (std::vector<GemvJob> &live : group_by_kind(jobs)) {
-        DevBuf &tb = c->tables[slot++ % 4];
+        const int sl = slot++ % 4;
+        DevBuf &tb = c->tables[sl];
         if (live.size() > (size_t)kInlineJobs) { rc = ensure(c, tb, live.size() * sizeof(GemvJob)); if (rc) return rc; }
         PreparedLaunch P;
-        rc = prepare_same_kind(c, live, tb.p, P);
+        rc = prepare_same_kind(c, live, tb.p, P, sl);
         if (rc) return rc;
         HIPCHECK(c, gemv_launch(c->stream, P.kind, P.L, P.threads, P.grid, P.lds));
     }
@@ -290,6 +312,10 @@ void larql_hip_destroy(larql_hip_ctx *c) {
     DevBuf *bufs[] = {&c->w[0], &c->w[1], &c->w[2], &c->w[3], &c->aux[0], &c->aux[1], &c->aux[2], &c->aux[3],
                       &c->x, &c->out, &c->tables[0], &c->tables[1], &c->tables[2], &c->tables[3], &c->misc, &c->scores, &c->q8, &c->q8s};
     for (DevBuf *b : bufs) if (b->p) (void)hipFree(b->p);
+    for (int i = 0; i < 4; i++) {
+        if (c->table_host[i]) (void)hipHostFree(c->table_host[i]);
+        if (c->table_ev[i]) (void)hipEventDestroy(c->table_ev[i]);
+    }
     if (c->log2_up) (void)hipFree(c->log2_up);
     if (c->nan_flag) (void)hipFree(c->nan_flag);
     if (c->ev0) (void)hipEventDestroy(c->ev0);
@@ -1029,10 +1055,14 @@ int larql_hip_dev_moe_mxfp4(larql_hip_ctx *c, const larql_hip_mxfp4_experts *ban
     }
     int rc = enqueue_jobs(c, jobs);
     if (rc) return rc;
-    HIPCHECK(c, clamped_glu_launch(c->stream, g, u, h, slots * inter, bank->limit, bank->alpha));
+    // the gated activation is applied by the down projection itself where the matrix-core kernel serves it
+    const bool fuse_glu = gemv_effective_kind(make_job(KIND_MXFP4, bank->down_packed, bank->down_scales, g, d, hidden, inter)) != KIND_MXFP4;
+    if (!fuse_glu) HIPCHECK(c, clamped_glu_launch(c->stream, g, u, h, slots * inter, bank->limit, bank->alpha));
     jobs.clear();
     for (size_t s = 0; s < slots; s++) {
-        GemvJob a = make_job(KIND_MXFP4, bank->down_packed, bank->down_scales, h + s * inter, d + s * hidden, hidden, inter);
+        GemvJob a = make_job(KIND_MXFP4, bank->down_packed, bank->down_scales, fuse_glu ? g + s * inter : h + s * inter, d + s * hidden,
+                             hidden, inter);
+        if (fuse_glu) { a.x_glu = u + s * inter; a.glu_limit = bank->limit; a.glu_alpha = bank->alpha; }
         a.sel = experts + s; a.w_sel_stride = dn_w_stride; a.aux_sel_stride = dn_s_stride;
         jobs.push_back(a);
     }

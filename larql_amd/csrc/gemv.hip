@@ -687,11 +687,25 @@ struct Mx4Step {
 // Digits of one step's 128 activations, for lane (t = lane%16, kg = lane/16); x index >= k reads as 0.
 // Every lane converts two activations into their six digits and the wavefront transposes them through
 // `scratch` (768 B of its own LDS: digit row t at t*128) into the operand layout.
-__device__ __forceinline__ Mx4Step mx4_setup_step(const float *x, uint32_t step, uint32_t k, uint32_t lane, uint8_t *scratch) {
+__device__ __forceinline__ Mx4Step mx4_setup_step(const GemvJob &j, uint32_t step, uint32_t lane, uint8_t *scratch) {
+    const float *x = j.x;
+    const uint32_t k = (uint32_t)j.k;
     const uint32_t t = lane & 15u, kg = lane >> 4;
     const uint32_t i0 = step * 128 + 2 * lane;
     float2_t v = {0.f, 0.f};
-    if (i0 + 2 <= k) v = *(const GLOBAL_AS float2_t *)(x + i0);  // k is even: a pair is inside or outside
+    if (i0 + 2 <= k) {  // k is even: a pair is inside or outside
+        v = *(const GLOBAL_AS float2_t *)(x + i0);
+        if (j.x_glu) {
+            // MoeGateRule::ClampedGlu (larql-compute/src/pipeline/moe.rs:88-92): g = min(g, L); u = clamp(u, -L, L);
+            // (u + 1) * (g * sigmoid(alpha * g))
+            const float2_t u = *(const GLOBAL_AS float2_t *)(j.x_glu + i0);
+            const float L = j.glu_limit, al = j.glu_alpha;
+            const float g0 = fminf(v.x, L), g1 = fminf(v.y, L);
+            const float u0 = u.x < -L ? -L : (u.x > L ? L : u.x), u1 = u.y < -L ? -L : (u.y > L ? L : u.y);
+            v.x = (u0 + 1.0f) * (g0 * (1.0f / (1.0f + expf(-(g0 * al)))));
+            v.y = (u1 + 1.0f) * (g1 * (1.0f / (1.0f + expf(-(g1 * al)))));
+        }
+    }
     float mx = fmaxf(fabsf(v.x), fabsf(v.y));
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
@@ -773,7 +787,7 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
     Mx4Step st[kMx4MaxSteps];
 #pragma unroll
     for (int s = 0; s < kMx4MaxSteps; s++)
-        if (working && (uint32_t)s < cw) st[s] = mx4_setup_step(j.x, step0 + s, k, lane, ring + (NS - 1) * slot_bytes);
+        if (working && (uint32_t)s < cw) st[s] = mx4_setup_step(j, step0 + s, lane, ring + (NS - 1) * slot_bytes);
 
     uint32_t n_use = 0;
     for (uint32_t tb = 0; tb < nt; tb += R) {

@@ -16,7 +16,7 @@ enum GemvKind : int32_t {
 };
 
 constexpr int kGemvMaxThreads = 512;
-constexpr int kInlineJobs = 4;
+constexpr int kInlineJobs = 8;  // jobs that travel in the kernel arguments (no table upload)
 
 // One matvec of a launch.  The caller fills kind/w/aux/x/out/rows/k; the rest
 // is geometry derived by gemv_job_geometry for the launch's block size.
@@ -41,6 +41,10 @@ struct GemvJob {
     // out + t*out_stride (strides in floats).  0 or 1 = a plain matvec.  See gemv_batch_capacity.
     uint32_t batch, pad2;
     uint64_t x_stride, out_stride;
+    // Optional gated activation (MoE down projection, MXFP4 matrix-core kernel only): when `x_glu` is set the
+    // activation is ClampedGlu(g = x[i], u = x_glu[i]) computed while the activations are prepared.
+    const float *x_glu;
+    float glu_limit, glu_alpha;
 };
 
 struct GemvLaunch {
