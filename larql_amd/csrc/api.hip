@@ -477,19 +477,27 @@ int larql_hip_q4k_matmul(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, c
     if (rc) return rc;
     Submission sub(c);
     if (seq_len >= 16 && num_rows <= 0xFFFFFFFFull && seq_len <= 0xFFFFFFFFull) {
-        // prefill shape: bf16 MFMA GEMM.  The f32 activations are split into two bf16 terms so the
-        // result keeps ~16 significant bits of x; the second pass is skipped when x is exactly bf16.
-        rc = ensure(c, c->misc, x_len * 4 + 64);
+        // prefill shape: MFMA GEMM on integer weights.  The f32 activations become two f16 terms (per-token
+        // scale), so the result keeps ~22 significant bits of x; the second pass is skipped when no lo term exists.
+        const size_t sx_len = seq_len * (hidden / 32) * 2;
+        rc = ensure(c, c->misc, x_len * 4 + sx_len * 2 + seq_len * 4 + 256);
         if (rc) return rc;
-        uint16_t *xh = (uint16_t *)c->misc.p, *xl = xh + x_len;
+        uint16_t *xh = (uint16_t *)c->misc.p, *xl = xh + x_len, *sx = xl + x_len;
+        float *ts = (float *)(((uintptr_t)(sx + sx_len) + 15) & ~(uintptr_t)15);
         HIPCHECK(c, hipMemsetAsync(c->nan_flag, 0, sizeof(int), c->stream));
-        HIPCHECK(c, split_bf16_launch(c->stream, (const float *)c->x.p, x_len, xh, xl, c->nan_flag));
+        HIPCHECK(c, q4k_gemm_prep_launch(c->stream, c->x.p, 0, (uint32_t)hidden, (uint32_t)seq_len, xh, xl, sx, ts, c->nan_flag));
         int any_lo = 0;
         HIPCHECK(c, hipMemcpyAsync(&any_lo, c->nan_flag, sizeof(int), hipMemcpyDeviceToHost, c->stream));
         HIPCHECK(c, hipStreamSynchronize(c->stream));
-        HIPCHECK(c, q4k_gemm_launch(c->stream, dw, xh, (float *)c->out.p, (uint32_t)num_rows, (uint32_t)hidden, (uint32_t)seq_len, 0));
+        HIPCHECK(c, hipMemsetAsync(c->nan_flag, 0, sizeof(int), c->stream));
+        const uint32_t splits = q4k_gemm_splits((uint32_t)num_rows, (uint32_t)hidden, (uint32_t)seq_len, (uint32_t)c->cu_count);
+        float *partial = nullptr;
+        if (splits > 1) { rc = ensure(c, c->scores, (size_t)splits * seq_len * num_rows * 4 + 64); if (rc) return rc; partial = (float *)c->scores.p; }
+        HIPCHECK(c, q4k_gemm_f16_launch(c->stream, dw, xh, sx, ts, (float *)c->out.p, (uint32_t)num_rows, (uint32_t)hidden, (uint32_t)seq_len, 1, 0,
+                                        splits, partial));
         if (any_lo)
-            HIPCHECK(c, q4k_gemm_launch(c->stream, dw, xl, (float *)c->out.p, (uint32_t)num_rows, (uint32_t)hidden, (uint32_t)seq_len, 1));
+            HIPCHECK(c, q4k_gemm_f16_launch(c->stream, dw, xl, sx, ts, (float *)c->out.p, (uint32_t)num_rows, (uint32_t)hidden, (uint32_t)seq_len, 0, 1,
+                                            splits, partial));
     } else {
         std::vector<GemvJob> jobs;
         for (size_t s = 0; s < seq_len; s++)
@@ -1005,8 +1013,23 @@ int larql_hip_dev_q4k_gemm(larql_hip_ctx *c, const uint8_t *w, const uint16_t *x
     if (hidden % 256 != 0) return fail(c, LARQL_REFUSED_SHAPE, "q4k_gemm: hidden not a multiple of 256");
     if (rows > 0xFFFFFFFFull || seq > 0xFFFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "q4k_gemm: too large");
     if (!w || !x_bf16 || !out || ((uintptr_t)w & 15) || ((uintptr_t)x_bf16 & 15)) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipSetDevice(c->device));
-    HIPCHECK(c, q4k_gemm_launch(c->stream, w, x_bf16, out, (uint32_t)rows, (uint32_t)hidden, (uint32_t)seq, 0));
+    if (getenv("LARQL_HIP_GEMM_BF16")) {  // first formulation (decoded weights split into two bf16 terms), kept for comparison
+        HIPCHECK(c, q4k_gemm_launch(c->stream, w, x_bf16, out, (uint32_t)rows, (uint32_t)hidden, (uint32_t)seq, 0));
+        return LARQL_OK;
+    }
+    // bf16 activations are exact in one f16 term after the per-token scale
+    const size_t x_len = seq * hidden, sx_len = seq * (hidden / 32) * 2;
+    int rc = ensure(c, c->misc, x_len * 2 + sx_len * 2 + seq * 4 + 256);
+    if (rc) return rc;
+    uint16_t *xh = (uint16_t *)c->misc.p, *sx = xh + x_len;
+    float *ts = (float *)(((uintptr_t)(sx + sx_len) + 15) & ~(uintptr_t)15);
+    HIPCHECK(c, q4k_gemm_prep_launch(c->stream, x_bf16, 1, (uint32_t)hidden, (uint32_t)seq, xh, nullptr, sx, ts, nullptr));
+    const uint32_t splits = q4k_gemm_splits((uint32_t)rows, (uint32_t)hidden, (uint32_t)seq, (uint32_t)c->cu_count);
+    float *partial = nullptr;
+    if (splits > 1) { rc = ensure(c, c->scores, (size_t)splits * seq * rows * 4 + 64); if (rc) return rc; partial = (float *)c->scores.p; }
+    HIPCHECK(c, q4k_gemm_f16_launch(c->stream, w, xh, sx, ts, out, (uint32_t)rows, (uint32_t)hidden, (uint32_t)seq, 1, 0, splits, partial));
     return LARQL_OK;
 }
 

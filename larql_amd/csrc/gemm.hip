@@ -141,6 +141,230 @@ __global__ void __launch_bounds__(256) q4k_gemm_kernel(const uint8_t *__restrict
         }
 }
 
+// ---------------------------------------------------------------------------
+// Second formulation (the one in use): keep the weight integer.
+//
+//   out[s, r] = sum over super-blocks of  d[r] * (sum_k (sc6*q)[r,k] * x[s,k])  -  dmin[r] * (sum_sub mn6[r,sub] * Sx[s,sub])
+//
+// sc6*q <= 945 is exact in f16, so the A operand needs no hi/lo split and costs ~1.7 VALU instructions per
+// weight (byte gather, mask into an f16 1024+q, one packed FMA against sc6) instead of ~10 for decode + split.
+// The activations are prepared once per call (q4k_gemm_prep_kernel): per token a power-of-two scale brings
+// max|x| to [2^13, 2^14), x/scale is stored as f16 (exact for bf16 inputs; f32 inputs add a second f16 term
+// and a second pass), and Sx, the sum of the represented activations over each 32-element sub-block, is stored
+// (divided by 32, to stay inside f16) as an f16 pair (hi, lo).  Per super-block a wavefront accumulates its 64x64 quadrant in D (v_mfma_f32_16x16x32_f16,
+// 32 MFMAs per 64-element step), gets sum_sub mn6*Sx from one more MFMA per tile (A slots 2*sub+h = mn6,
+// B slots = Sx_h), and folds both into the f32 result with the row's d and dmin.
+// ---------------------------------------------------------------------------
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+constexpr int LDM = 40;  // padded row of the 32-slot min tiles (f16 elements)
+
+// one block per token: scale, f16 terms, sub-block sums.  `x_is_bf16`: 16-bit inputs (exact in one term).
+__global__ void __launch_bounds__(256) q4k_gemm_prep_kernel(const void *__restrict__ x, int x_is_bf16, uint32_t hidden,
+                                                            uint16_t *__restrict__ xh, uint16_t *__restrict__ xl,
+                                                            uint16_t *__restrict__ sx, float *__restrict__ tok_scale,
+                                                            int *__restrict__ any_lo) {
+    __shared__ float red[4];
+    const uint32_t tok = blockIdx.x, t = threadIdx.x;
+    const uint16_t *xb = (const uint16_t *)x + (size_t)tok * hidden;
+    const float *xf = (const float *)x + (size_t)tok * hidden;
+    float mx = 0.f;
+    for (uint32_t k = t; k < hidden; k += 256) {
+        const float v = x_is_bf16 ? __builtin_bit_cast(float, (uint32_t)xb[k] << 16) : xf[k];
+        mx = fmaxf(mx, fabsf(v));
+    }
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    if ((t & 63u) == 0) red[t >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    int ex = 0;
+    if (mx > 0.f && mx < __builtin_inff()) (void)frexpf(mx, &ex);
+    ex = max(-100, min(110, ex));
+    const float to_h = ldexpf(1.f, 14 - ex);
+    if (t == 0) tok_scale[tok] = ldexpf(1.f, ex - 14);
+    int lo_seen = 0;
+    for (uint32_t k = t; k < hidden; k += 256) {  // hidden % 256 == 0: every wavefront half covers one sub-block
+        const float v = (x_is_bf16 ? __builtin_bit_cast(float, (uint32_t)xb[k] << 16) : xf[k]) * to_h;
+        const _Float16 h = (_Float16)v;
+        const _Float16 l = (_Float16)(v - (float)h);
+        xh[(size_t)tok * hidden + k] = __builtin_bit_cast(uint16_t, h);
+        if (xl) xl[(size_t)tok * hidden + k] = __builtin_bit_cast(uint16_t, l);
+        lo_seen |= (xl && (float)l != 0.f) ? 1 : 0;
+        float sm = (float)h + (xl ? (float)l : 0.f);  // the activation as the MFMAs will see it
+        for (int o = 1; o < 32; o <<= 1) sm += __shfl_xor(sm, o);
+        sm *= 0.03125f;  // stored as Sx/32 so that 32 x 2^14 stays inside f16; the min operand carries the 32
+        if ((t & 31u) == 0) {
+            const _Float16 sh = (_Float16)sm;
+            const _Float16 sl = (_Float16)(sm - (float)sh);
+            sx[((size_t)tok * (hidden / 32) + k / 32) * 2 + 0] = __builtin_bit_cast(uint16_t, sh);
+            sx[((size_t)tok * (hidden / 32) + k / 32) * 2 + 1] = __builtin_bit_cast(uint16_t, sl);
+        }
+    }
+    if (lo_seen && any_lo) *any_lo = 1;
+}
+
+// with_mins = 0: the activation term carries no offset part (second pass over the lo terms)
+__global__ void __launch_bounds__(256, 2) q4k_gemm_f16_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ xh,
+                                                              const uint16_t *__restrict__ sx, const float *__restrict__ tok_scale,
+                                                              float *__restrict__ out, uint32_t rows, uint32_t hidden, uint32_t seq,
+                                                              int with_mins, int accumulate, uint32_t sb_per_split, float *__restrict__ partial) {
+    __shared__ __attribute__((aligned(16))) uint16_t a_t[TM * LDK];   // f16(sc6*q), 128 rows x 64 k
+    __shared__ __attribute__((aligned(16))) uint16_t b_t[TN * LDK];   // f16 activations, 128 tokens x 64 k
+    __shared__ __attribute__((aligned(16))) uint16_t am_t[TM * LDM];  // mn6 in slots 2*sub+h
+    __shared__ __attribute__((aligned(16))) uint16_t bm_t[TN * LDM];  // Sx_h in slots 2*sub+h
+    __shared__ float d_t[TM], dmin_t[TM];
+    const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
+    const uint32_t row0 = blockIdx.x * TM, tok0 = blockIdx.y * TN;
+    const uint32_t nsb = hidden >> 8;
+    const size_t row_bytes = (size_t)nsb * 144;
+    const uint32_t sr = t >> 1, half = t & 1u;
+    const uint32_t wrow = min(row0 + sr, rows - 1), xtok = min(tok0 + sr, seq - 1);
+    const uint8_t *wp = w + (size_t)wrow * row_bytes;
+    const uint16_t *xp = xh + (size_t)xtok * hidden + half * 32;
+    const uint16_t *sxp = sx + (size_t)xtok * (hidden / 32) * 2;
+    const uint32_t wm = (wave >> 1) * 64, wn = (wave & 1u) * 64;
+    const uint32_t l16 = lane & 15u, kq = (lane >> 4) * 8;
+
+    f32x4 acc[4][4], D[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) { acc[i][jj] = (f32x4){0.f, 0.f, 0.f, 0.f}; D[i][jj] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
+    // slots 16..31 of the min tiles stay zero
+    for (uint32_t e = t; e < TM * LDM; e += 256) { am_t[e] = 0; bm_t[e] = 0; }
+
+    // split-K: blockIdx.z takes super-blocks [z*sb_per_split, ...); partial results go to their own slab
+    const uint32_t sb_begin = blockIdx.z * sb_per_split, sb_end = min(nsb, sb_begin + sb_per_split);
+    for (uint32_t sb = sb_begin; sb < sb_end; sb++) {
+      const u32x4 *blk = reinterpret_cast<const u32x4 *>(wp + (size_t)sb * 144);
+      const u32x4 hdr = blk[0];
+      for (uint32_t g = 0; g < 4; g++) {
+        // raw operands of this 64-element step (a register prefetch one step ahead cost more in spills than it hid)
+        const u32x4 q0 = blk[1 + 2 * g], q1 = blk[2 + 2 * g];
+        const u32x4 *xv = reinterpret_cast<const u32x4 *>(xp + (size_t)sb * 256 + g * 64);
+        const u32x4 x0 = xv[0], x1 = xv[1], x2 = xv[2], x3 = xv[3];
+        u32x4 sxv = {0u, 0u, 0u, 0u};
+        if (g == 0 && with_mins) sxv = *reinterpret_cast<const u32x4 *>(sxp + (size_t)sb * 16 + half * 8);
+        // ---- 32 weights of (row sr, sub-block 2g+half) as f16(sc6*q) ----
+        const uint32_t s = 2 * g + half, sh = 8u * (s & 3u);
+        const uint32_t pa = (hdr.y >> sh) & 0xFFu, pc = (hdr.w >> sh) & 0xFFu;
+        const uint32_t sc6 = s < 4 ? (pa & 63u) : ((pc & 0x0Fu) | ((pa >> 6) << 4));
+        const _Float16 scf = (_Float16)(float)sc6;
+        const f16x2 sc2 = {scf, scf};
+        const f16x2 off2 = {(_Float16)(-1024.0f * (float)sc6), (_Float16)(-1024.0f * (float)sc6)};
+        const uint32_t qd[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+        uint32_t aw[16];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const uint32_t v = half ? (qd[i] >> 4) : qd[i];
+            // bytes 0,1 -> 16-bit lanes of one dword, bytes 2,3 -> the next (k order kept)
+            const uint32_t p01 = __builtin_amdgcn_perm(0u, v, 0x0C010C00u), p23 = __builtin_amdgcn_perm(0u, v, 0x0C030C02u);
+            const f16x2 m01 = __builtin_bit_cast(f16x2, (p01 & 0x000F000Fu) | 0x64006400u);  // 1024 + q
+            const f16x2 m23 = __builtin_bit_cast(f16x2, (p23 & 0x000F000Fu) | 0x64006400u);
+            aw[2 * i] = __builtin_bit_cast(uint32_t, m01 * sc2 + off2);      // (1024+q)*sc6 - 1024*sc6, one rounding: exact
+            aw[2 * i + 1] = __builtin_bit_cast(uint32_t, m23 * sc2 + off2);
+        }
+        uint32_t mnw[4] = {0u, 0u, 0u, 0u};
+        if (g == 0 && with_mins) {
+            // this thread's half of the super-block: sub-blocks 4*half .. 4*half+3 -> slots 8*half .. 8*half+7
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const uint32_t ss = 4 * half + u, shm = 8u * (ss & 3u);
+                const uint32_t qb = (hdr.z >> shm) & 0xFFu, qc = (hdr.w >> shm) & 0xFFu;
+                const uint32_t mn6 = ss < 4 ? (qb & 63u) : ((qc >> 4) | ((qb >> 6) << 4));
+                const uint32_t hb = __builtin_bit_cast(uint16_t, (_Float16)(float)(mn6 * 32u));  // <= 2016: exact; Sx is stored /32
+                mnw[u] = hb | (hb << 16);
+            }
+        }
+        __syncthreads();  // previous step's MFMA reads are done
+        {
+            u32x4 *ah = reinterpret_cast<u32x4 *>(&a_t[sr * LDK + half * 32]);
+#pragma unroll
+            for (int i = 0; i < 4; i++) ah[i] = (u32x4){aw[4 * i], aw[4 * i + 1], aw[4 * i + 2], aw[4 * i + 3]};
+            u32x4 *bt = reinterpret_cast<u32x4 *>(&b_t[sr * LDK + half * 32]);
+            bt[0] = x0; bt[1] = x1; bt[2] = x2; bt[3] = x3;
+            if (g == 0) {
+                if (with_mins) {
+                    *reinterpret_cast<u32x4 *>(&am_t[sr * LDM + half * 8]) = (u32x4){mnw[0], mnw[1], mnw[2], mnw[3]};
+                    *reinterpret_cast<u32x4 *>(&bm_t[sr * LDM + half * 8]) = sxv;
+                }
+                if (half == 0) {
+                    d_t[sr] = half_to_float(hdr.x & 0xFFFFu);
+                    dmin_t[sr] = half_to_float(hdr.x >> 16);
+                }
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+            f16x8 af[4], bf[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                af[i] = *reinterpret_cast<const f16x8 *>(&a_t[(wm + i * 16 + l16) * LDK + kk * 32 + kq]);
+                bf[i] = *reinterpret_cast<const f16x8 *>(&b_t[(wn + i * 16 + l16) * LDK + kk * 32 + kq]);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) D[i][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bf[jj], D[i][jj], 0, 0, 0);
+        }
+        if (g == 3) {
+            // ---- end of the super-block: acc += d * D - dmin * (mn6 . Sx) ----
+            f16x8 amf[4], bmf[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                amf[i] = *reinterpret_cast<const f16x8 *>(&am_t[(wm + i * 16 + l16) * LDM + kq]);
+                bmf[i] = *reinterpret_cast<const f16x8 *>(&bm_t[(wn + i * 16 + l16) * LDM + kq]);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t rb = wm + i * 16 + (lane >> 4) * 4;
+                const f32x4 dv = *reinterpret_cast<const f32x4 *>(&d_t[rb]);
+                const f32x4 mv = *reinterpret_cast<const f32x4 *>(&dmin_t[rb]);
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) {
+                    f32x4 Dm = {0.f, 0.f, 0.f, 0.f};
+                    if (with_mins) Dm = __builtin_amdgcn_mfma_f32_16x16x32_f16(amf[i], bmf[jj], Dm, 0, 0, 0);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[i][jj][e] += dv[e] * D[i][jj][e] - mv[e] * Dm[e];
+                    D[i][jj] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                }
+            }
+        }
+    }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            const uint32_t tok = tok0 + wn + jj * 16 + l16;
+            const uint32_t r = row0 + wm + i * 16 + (lane >> 4) * 4;
+            if (tok >= seq) continue;
+            if (partial) {  // unscaled partial sums of this K-range; q4k_gemm_reduce_kernel adds the slabs in order
+                float *o = partial + ((size_t)blockIdx.z * seq + tok) * rows + r;
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (r + e < rows) o[e] = acc[i][jj][e];
+                continue;
+            }
+            const float ts = tok_scale[tok];
+            float *o = out + (size_t)tok * rows + r;
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (r + e < rows) o[e] = accumulate ? o[e] + acc[i][jj][e] * ts : acc[i][jj][e] * ts;
+        }
+}
+
+__global__ void __launch_bounds__(256) q4k_gemm_reduce_kernel(const float *__restrict__ partial, uint32_t splits, const float *__restrict__ tok_scale,
+                                                              float *__restrict__ out, uint32_t rows, uint32_t seq, int accumulate) {
+    const size_t n = (size_t)rows * seq, i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float s = 0.f;
+    for (uint32_t z = 0; z < splits; z++) s += partial[(size_t)z * n + i];
+    s *= tok_scale[i / rows];
+    out[i] = accumulate ? out[i] + s : s;
+}
+
 // f32 activations -> bf16 hi (round to nearest even) and the bf16 of the remainder
 __global__ void split_bf16_kernel(const float *__restrict__ x, size_t n, uint16_t *__restrict__ hi, uint16_t *__restrict__ lo,
                                   int *__restrict__ any_lo) {
@@ -159,6 +383,39 @@ hipError_t q4k_gemm_launch(hipStream_t s, const uint8_t *w, const uint16_t *x_bf
     if (rows == 0 || seq == 0) return hipSuccess;
     hipLaunchKernelGGL(q4k_gemm_kernel, dim3((rows + TM - 1) / TM, (seq + TN - 1) / TN), dim3(256), 0, s, w, x_bf16, out, rows, hidden,
                        seq, accumulate);
+    return hipGetLastError();
+}
+
+hipError_t q4k_gemm_prep_launch(hipStream_t s, const void *x, int x_is_bf16, uint32_t hidden, uint32_t seq, uint16_t *xh, uint16_t *xl,
+                                uint16_t *sx, float *tok_scale, int *any_lo) {
+    if (seq == 0) return hipSuccess;
+    hipLaunchKernelGGL(q4k_gemm_prep_kernel, dim3(seq), dim3(256), 0, s, x, x_is_bf16, hidden, xh, xl, sx, tok_scale, any_lo);
+    return hipGetLastError();
+}
+
+// K-ranges per output tile so that a launch has roughly two workgroups per CU (1 = no split)
+uint32_t q4k_gemm_splits(uint32_t rows, uint32_t hidden, uint32_t seq, uint32_t cu_count) {
+    const uint64_t tiles = (uint64_t)((rows + TM - 1) / TM) * ((seq + TN - 1) / TN);
+    const uint32_t nsb = hidden / 256;
+    uint32_t s = 1;
+    while (s < 8 && tiles * s < (uint64_t)cu_count * 3 / 2 && nsb / (s * 2) >= 4) s *= 2;
+    return s;
+}
+
+hipError_t q4k_gemm_f16_launch(hipStream_t s, const uint8_t *w, const uint16_t *xh, const uint16_t *sx, const float *tok_scale, float *out,
+                               uint32_t rows, uint32_t hidden, uint32_t seq, int with_mins, int accumulate, uint32_t splits, float *partial) {
+    if (rows == 0 || seq == 0) return hipSuccess;
+    const uint32_t nsb = hidden / 256;
+    if (splits <= 1 || !partial) {
+        hipLaunchKernelGGL(q4k_gemm_f16_kernel, dim3((rows + TM - 1) / TM, (seq + TN - 1) / TN, 1), dim3(256), 0, s, w, xh, sx, tok_scale, out,
+                           rows, hidden, seq, with_mins, accumulate, nsb, (float *)nullptr);
+        return hipGetLastError();
+    }
+    const uint32_t per = (nsb + splits - 1) / splits, z = (nsb + per - 1) / per;
+    hipLaunchKernelGGL(q4k_gemm_f16_kernel, dim3((rows + TM - 1) / TM, (seq + TN - 1) / TN, z), dim3(256), 0, s, w, xh, sx, tok_scale, out,
+                       rows, hidden, seq, with_mins, accumulate, per, partial);
+    const size_t n = (size_t)rows * seq;
+    hipLaunchKernelGGL(q4k_gemm_reduce_kernel, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, s, partial, z, tok_scale, out, rows, seq, accumulate);
     return hipGetLastError();
 }
 
