@@ -103,6 +103,14 @@ int  larql_hip_get_submission_clock(larql_hip_ctx *ctx, larql_hip_submission_clo
 int larql_hip_q4k_matvec(larql_hip_ctx *ctx, const uint8_t *q4k, size_t q4k_len,
                          const float *x, size_t x_len, size_t num_rows, size_t hidden,
                          float *out, size_t out_len);
+
+/* QuantMatVec::q6k_matvec — backend/quant_matvec.rs:335-345; CPU semantics
+ * cpu/mod.rs:133-141 + cpu/ops/q6k_matvec.rs:45-91 (210-byte super-blocks in ggml's
+ * planar layout, larql-models/src/quant/ggml/q6_k.rs:19-40).  x_len == hidden,
+ * hidden % 256 == 0, w_len >= rows*(hidden/256)*210, else REFUSED_SHAPE (the CPU
+ * path indexes out of range there); zero dims write zeros. */
+int larql_hip_q6k_matvec(larql_hip_ctx *ctx, const uint8_t *q6k, size_t q6k_len,
+                         const float *x, size_t x_len, size_t num_rows, size_t hidden, float *out);
 /* QuantMatVec::q4k_dual_matvec — quant_matvec.rs:287-296; q4_common/dual.rs:22-167. */
 int larql_hip_q4k_dual_matvec(larql_hip_ctx *ctx, const uint8_t *q4k_a, size_t a_len,
                               const uint8_t *q4k_b, size_t b_len,

@@ -52,6 +52,7 @@ SIGNATURES = {
     "larql_hip_clear_weight_regions": (ci, [vp]),
     "larql_hip_get_submission_clock": (ci, [vp, C.POINTER(SubmissionClock)]),
     "larql_hip_q4k_matvec": (ci, [vp, vp, sz, vp, sz, sz, sz, vp, sz]),
+    "larql_hip_q6k_matvec": (ci, [vp, vp, sz, vp, sz, sz, sz, vp]),
     "larql_hip_q4k_dual_matvec": (ci, [vp, vp, sz, vp, sz, vp, sz, sz, sz, vp, vp, sz]),
     "larql_hip_q4k_matmul": (ci, [vp, vp, sz, vp, sz, sz, sz, sz, vp, sz]),
     "larql_hip_q4k_matvec_topk": (ci, [vp, vp, sz, vp, sz, sz, sz, sz, vp, vp, C.POINTER(sz)]),

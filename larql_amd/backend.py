@@ -114,6 +114,13 @@ class HipBackend:
                                                  _ptr(out), out.size))
         return out if ok else None
 
+    def q6k_matvec(self, q6k, x, num_rows: int, hidden: int) -> Optional[np.ndarray]:
+        """QuantMatVec::q6k_matvec (backend/quant_matvec.rs:335-345)."""
+        w, xv = _u8(q6k), _f32(x)
+        out = np.empty(num_rows, np.float32)
+        ok = self._some(lib.larql_hip_q6k_matvec(self._h, _ptr(w), w.size, _ptr(xv), xv.size, num_rows, hidden, _ptr(out)))
+        return out if ok else None
+
     def q4k_dual_matvec(self, q4k_a, q4k_b, x, num_rows: int, hidden: int):
         a, b, x = _u8(q4k_a), _u8(q4k_b), _f32(x)
         oa, ob = np.empty(num_rows, np.float32), np.empty(num_rows, np.float32)

@@ -129,6 +129,7 @@ int kind_of_format(int format) {
     switch (format) {
         case LARQL_FMT_Q4_K: case LARQL_FMT_Q4_KF: return KIND_Q4K;
         case LARQL_FMT_GGML_Q8_0: return KIND_Q8_0;
+        case LARQL_FMT_Q6_K: return KIND_Q6K;
         case LARQL_FMT_MXFP4: return KIND_MXFP4;
         case LARQL_FMT_Q4_0: return KIND_Q4_0;
         case LARQL_FMT_BF16: return KIND_BF16;
@@ -212,10 +213,10 @@ std::vector<std::vector<GemvJob>> group_by_kind(const std::vector<GemvJob> &jobs
     std::vector<GemvJob> jobs(jobs_in);
     for (GemvJob &j : jobs) j.kind = gemv_effective_kind(j);  // Q4_K rows the matrix-core kernel takes get their own launch
     std::vector<std::vector<GemvJob>> groups;
-    bool done[12] = {false, false, false, false, false, false, false, false, false, false, false, false};
+    bool done[13] = {false, false, false, false, false, false, false, false, false, false, false, false, false};
     for (size_t i = 0; i < jobs.size(); i++) {
         const int kind = jobs[i].kind;
-        if (jobs[i].rows == 0 || kind < 0 || kind > 11 || done[kind]) continue;
+        if (jobs[i].rows == 0 || kind < 0 || kind > 12 || done[kind]) continue;
         done[kind] = true;
         std::vector<GemvJob> live;
         for (size_t t = i; t < jobs.size(); t++)
@@ -330,7 +331,7 @@ const char *larql_hip_last_error(const larql_hip_ctx *c) { return c ? c->last_er
 
 int larql_hip_supports_quant(const larql_hip_ctx *, int format) {
     switch (format) {
-        case LARQL_FMT_Q4_0: case LARQL_FMT_Q4_K: case LARQL_FMT_Q4_KF: case LARQL_FMT_MXFP4:
+        case LARQL_FMT_Q4_0: case LARQL_FMT_Q4_K: case LARQL_FMT_Q4_KF: case LARQL_FMT_Q6_K: case LARQL_FMT_MXFP4:
         case LARQL_FMT_GGML_Q8_0: case LARQL_FMT_BF16: case LARQL_FMT_F16: case LARQL_FMT_F32:
             return 1;
         default:
@@ -433,6 +434,19 @@ int larql_hip_q4k_matvec(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, c
     if (!q4k || !x) return LARQL_E_ARG;
     const size_t need = (hidden / 256) * 144 * num_rows;
     return host_matvec_multi(c, KIND_Q4K, 1, &q4k, &need, nullptr, nullptr, &num_rows, hidden, x, x_len * 4, &out);
+}
+
+int larql_hip_q6k_matvec(larql_hip_ctx *c, const uint8_t *q6k, size_t q6k_len, const float *x, size_t x_len, size_t num_rows,
+                         size_t hidden, float *out) {
+    if (!c || (!out && num_rows)) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    const size_t need = (hidden / 256) * 210 * num_rows;
+    if (hidden % 256 != 0 || x_len != hidden || q6k_len < need)
+        return fail(c, LARQL_REFUSED_SHAPE, "q6k_matvec: refused operands: activation length %zu for %zu cols, %zu weight bytes for %zu rows",
+                    x_len, hidden, q6k_len, num_rows);
+    if (num_rows == 0 || hidden == 0) { for (size_t i = 0; i < num_rows; i++) out[i] = 0.0f; return LARQL_OK; }
+    if (!q6k || !x) return LARQL_E_ARG;
+    return host_matvec_multi(c, KIND_Q6K, 1, &q6k, &need, nullptr, nullptr, &num_rows, hidden, x, x_len * 4, &out);
 }
 
 int larql_hip_q4k_dual_matvec(larql_hip_ctx *c, const uint8_t *a, size_t a_len, const uint8_t *b, size_t b_len,
@@ -609,6 +623,8 @@ int larql_hip_quant_matvec(larql_hip_ctx *c, int format, const uint8_t *weights,
     switch (format) {
         case LARQL_FMT_Q4_K: case LARQL_FMT_Q4_KF:
             return larql_hip_q4k_matvec(c, weights, w_len, x, x_len, num_rows, hidden, out, num_rows);
+        case LARQL_FMT_Q6_K:
+            return larql_hip_q6k_matvec(c, weights, w_len, x, x_len, num_rows, hidden, out);
         case LARQL_FMT_Q4_0: {
             std::lock_guard<std::mutex> lk(c->mu);
             if (hidden % 32 != 0 || w_len != num_rows * (hidden / 32) * 18 || x_len != hidden)
@@ -633,7 +649,7 @@ int larql_hip_quant_matvec(larql_hip_ctx *c, int format, const uint8_t *weights,
             return sub.finish();
         }
         default:
-            // Q6_K, Q5_K, I2S, MXFP4 (external scales), the trait's own Q8_0 layout and the
+            // Q5_K, I2S, MXFP4 (external scales), the trait's own Q8_0 layout and the
             // float formats answer None through this signature (backend/quant_matvec.rs:58-97).
             return fail(c, LARQL_UNSUPPORTED, "quant_matvec: format %d is not served through this entry", format);
     }
@@ -885,7 +901,7 @@ static int dev_job_from_public(larql_hip_ctx *c, const larql_hip_matvec_job &p, 
     if (kind < 0) return fail(c, LARQL_UNSUPPORTED, "matvec: format %d has no kernel", p.format);
     if (kind == KIND_MXFP4 && !p.aux) return fail(c, LARQL_E_ARG, "matvec: MXFP4 needs the scale stream");
     if (kind == KIND_Q4_0) return fail(c, LARQL_UNSUPPORTED, "matvec batch: Q4_0 goes through larql_hip_dev_matvec");
-    if (kind == KIND_Q4K && p.k % 256 != 0) return fail(c, LARQL_REFUSED_SHAPE, "matvec: k not a multiple of 256");
+    if ((kind == KIND_Q4K || kind == KIND_Q6K) && p.k % 256 != 0) return fail(c, LARQL_REFUSED_SHAPE, "matvec: k not a multiple of 256");
     if (p.k % 32 != 0) return fail(c, LARQL_REFUSED_SHAPE, "matvec: k not a multiple of 32");
     jobs.push_back(make_job(kind, p.w, p.aux, p.x, p.out, p.rows, p.k));
     return LARQL_OK;

@@ -174,6 +174,93 @@ __device__ __forceinline__ float q8_0_block_dot(const Q8Raw &r, const X32Slice &
 }
 
 // ---------------------------------------------------------------------------
+// Q6_K (K-slice kernel): one thread = one 32-byte row of ql of one 128-element half of a 210-byte
+// super-block, i.e. 64 weights: the low nibbles are plane r (elements r*32 .. r*32+31 of the half), the
+// high nibbles plane r+2; qh of the half carries their two top bits at shifts 2r and 2r+4
+// (q6k_subblock_vals, larql-models/src/quant/ggml/q6_k.rs:19-40).  Value per row as q6k_matvec
+// (larql-compute/src/cpu/ops/q6k_matvec.rs:45-91): sum over 16-element sub-blocks of (d*scale) * sum (q-32)*x,
+// with the -32 taken out through the sub-block sums of x.  Blocks are only 2-byte aligned: every field is read as
+// the aligned dwords that cover it and shifted into place (v_alignbit).
+// ---------------------------------------------------------------------------
+struct Q6KSlice {
+    float x[64];     // plane r (32), then plane r+2 (32)
+    float sum[4];    // sums of x over the four 16-element sub-blocks, in that order
+};
+
+__device__ __forceinline__ void q6k_load_x(Q6KSlice &s, const float *x, uint32_t c) {
+    const uint32_t sb = c >> 2, h = (c >> 1) & 1u, r = c & 1u;
+    g_f4p lo = (g_f4p)(x + (size_t)sb * 256 + h * 128 + r * 32);
+    g_f4p hi = (g_f4p)(x + (size_t)sb * 256 + h * 128 + (r + 2) * 32);
+    float sm[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const f32x4 a = lo[i], b = hi[i];
+        s.x[4 * i + 0] = a.x; s.x[4 * i + 1] = a.y; s.x[4 * i + 2] = a.z; s.x[4 * i + 3] = a.w;
+        s.x[32 + 4 * i + 0] = b.x; s.x[32 + 4 * i + 1] = b.y; s.x[32 + 4 * i + 2] = b.z; s.x[32 + 4 * i + 3] = b.w;
+        sm[i >> 2] += (a.x + a.y) + (a.z + a.w);
+        sm[2 + (i >> 2)] += (b.x + b.y) + (b.z + b.w);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) s.sum[i] = sm[i];
+}
+
+struct Q6KRaw { uint32_t ql[9], qh[9], sc[2], d; };
+
+// 32 bytes starting at the 2-byte-aligned address p, as the 9 aligned dwords that cover them
+__device__ __forceinline__ void load9(uint32_t (&dst)[9], const uint8_t *p) {
+    g_u32p a = (g_u32p)((uintptr_t)p & ~(uintptr_t)3);
+#pragma unroll
+    for (int i = 0; i < 9; i++) dst[i] = a[i];
+}
+
+__device__ __forceinline__ Q6KRaw q6k_load(const uint8_t *row, uint32_t c) {
+    const uint32_t sb = c >> 2, h = (c >> 1) & 1u, r = c & 1u;
+    const uint8_t *blk = row + (size_t)sb * 210;
+    Q6KRaw raw;
+    load9(raw.ql, blk + h * 64 + r * 32);
+    load9(raw.qh, blk + 128 + h * 32);
+    g_u32p sp = (g_u32p)((uintptr_t)(blk + 192 + h * 8 + 2 * r) & ~(uintptr_t)3);  // scales 2r, 2r+1 and 2r+4, 2r+5 of the half
+    raw.sc[0] = sp[0]; raw.sc[1] = sp[1];  // the six bytes needed start at most 2 bytes into this window
+    raw.d = *(const GLOBAL_AS uint16_t *)(blk + 208);
+    return raw;
+}
+
+__device__ __forceinline__ float q6k_chunk_dot(const Q6KRaw &raw, const Q6KSlice &s, const uint8_t *row, uint32_t c) {
+    const uint32_t sb = c >> 2, r = c & 1u;
+    // all fields of a block share the block's misalignment (0 or 2 bytes): block offset sb*210 on a 4-byte aligned row
+    const uint32_t mis = (uint32_t)(((uintptr_t)row + (size_t)sb * 210) & 2u), sh = mis * 8;
+    const float d = half_bits_to_float(raw.d);
+    // scale bytes: 8 bytes from (block + 192 + h*8 + 2r): parity of (mis + 2r)
+    const uint32_t ssh = ((mis + 2 * r) & 2u) * 8;
+    const uint32_t s01 = __builtin_amdgcn_alignbit(raw.sc[1], raw.sc[0], ssh), s45 = raw.sc[1] >> ssh;
+    const float sc0 = (float)(int)(int8_t)(s01 & 0xFF), sc1 = (float)(int)(int8_t)((s01 >> 8) & 0xFF);
+    const float sc2 = (float)(int)(int8_t)(s45 & 0xFF), sc3 = (float)(int)(int8_t)((s45 >> 8) & 0xFF);
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    const uint32_t hs = 2 * r;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const uint32_t ql = __builtin_amdgcn_alignbit(raw.ql[i + 1], raw.ql[i], sh);
+        const uint32_t qh = __builtin_amdgcn_alignbit(raw.qh[i + 1], raw.qh[i], sh);
+        const uint32_t a = (ql & 0x0F0F0F0Fu) | (((qh >> hs) & 0x03030303u) << 4);              // plane r, elements 4i..4i+3
+        const uint32_t b = ((ql >> 4) & 0x0F0F0F0Fu) | (((qh >> (hs + 4)) & 0x03030303u) << 4);  // plane r+2
+        float &al = acc[i >> 2], &bh = acc[2 + (i >> 2)];
+        al = __builtin_fmaf((float)(a & 0xFFu), s.x[4 * i + 0], al);
+        al = __builtin_fmaf((float)((a >> 8) & 0xFFu), s.x[4 * i + 1], al);
+        al = __builtin_fmaf((float)((a >> 16) & 0xFFu), s.x[4 * i + 2], al);
+        al = __builtin_fmaf((float)(a >> 24), s.x[4 * i + 3], al);
+        bh = __builtin_fmaf((float)(b & 0xFFu), s.x[32 + 4 * i + 0], bh);
+        bh = __builtin_fmaf((float)((b >> 8) & 0xFFu), s.x[32 + 4 * i + 1], bh);
+        bh = __builtin_fmaf((float)((b >> 16) & 0xFFu), s.x[32 + 4 * i + 2], bh);
+        bh = __builtin_fmaf((float)(b >> 24), s.x[32 + 4 * i + 3], bh);
+    }
+    float v = sc0 * (acc[0] - 32.0f * s.sum[0]);
+    v += sc1 * (acc[1] - 32.0f * s.sum[1]);
+    v += sc2 * (acc[2] - 32.0f * s.sum[2]);
+    v += sc3 * (acc[3] - 32.0f * s.sum[3]);
+    return d * v;
+}
+
+// ---------------------------------------------------------------------------
 // MXFP4: one thread = one 32-element group: 16 packed bytes (element 2b in the
 // low nibble of byte b) + one e8m0 scale byte.  Value as mxfp4_loop computes it
 // (larql-vindex/src/format/vindex3/opplan/exec/tests/device.rs:109-127):
@@ -1344,6 +1431,42 @@ __device__ __forceinline__ void run_q8_0(const GemvJob &j, uint32_t p0, uint32_t
 }
 
 template <int U>
+__device__ __forceinline__ void run_q6k(const GemvJob &j, uint32_t p0, uint32_t p1, float *part) {
+    const uint32_t t = threadIdx.x, cpr = j.cpr, rpp = j.rpp;
+    const bool active = t < cpr * rpp;
+    const uint32_t c = active ? t % cpr : 0, rl = active ? t / cpr : 0;
+    Q6KSlice xs;
+    q6k_load_x(xs, j.x, c);
+    const size_t row_bytes = j.row_bytes;
+    for (uint32_t tp = p0; tp < p1; tp += kTilePasses) {
+        const uint32_t tp_end = min(p1, tp + kTilePasses);
+        const uint32_t row_base = tp * rpp;
+        const uint32_t tile_rows = min((uint32_t)j.rows, tp_end * rpp) - row_base;
+        if (active) {
+            for (uint32_t lr = rl; lr < tile_rows; lr += rpp * U) {
+                Q6KRaw raw[U];
+                const uint8_t *rowp[U];
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    const uint32_t r = min(lr + u * rpp, tile_rows - 1) + row_base;
+                    rowp[u] = j.w + (size_t)r * row_bytes;
+                    raw[u] = q6k_load(rowp[u], c);
+                }
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    const uint32_t r = lr + u * rpp;
+                    const float v = q6k_chunk_dot(raw[u], xs, rowp[u], c);
+                    if (r < tile_rows) part[r * cpr + c] = v;
+                }
+            }
+        }
+        __syncthreads();
+        tile_epilogue(part, cpr, tile_rows, j.out, row_base);
+        __syncthreads();
+    }
+}
+
+template <int U>
 __device__ __forceinline__ void run_mxfp4(const GemvJob &j, uint32_t p0, uint32_t p1, float *part) {
     const uint32_t t = threadIdx.x, cpr = j.cpr, rpp = j.rpp;
     const bool active = t < cpr * rpp;
@@ -1484,6 +1607,7 @@ __device__ __forceinline__ void gemv_body(const GemvLaunch &L, float *part) {
         if (KIND == KIND_Q4K) run_q4k<U>(j, a, b, part);
         else if (KIND == KIND_Q8_0) run_q8_0<U>(j, a, b, part);
         else if (KIND == KIND_MXFP4) run_mxfp4<U>(j, a, b, part);
+        else if (KIND == KIND_Q6K) run_q6k<U>(j, a, b, part);
         else if (KIND == KIND_Q4_0) run_q4_0<U>(j, a, b, part);
         else if (KIND == KIND_BF16) run_dense<U, 0>(j, a, b, part);
         else if (KIND == KIND_F16) run_dense<U, 1>(j, a, b, part);
@@ -1505,6 +1629,7 @@ LARQL_GEMV_KERNEL(gemv_q8_0_u4_kernel, KIND_Q8_0, 4, 3)
 LARQL_GEMV_KERNEL(gemv_mxfp4_u2_kernel, KIND_MXFP4, 2, 4)
 LARQL_GEMV_KERNEL(gemv_mxfp4_u4_kernel, KIND_MXFP4, 4, 4)
 LARQL_GEMV_KERNEL(gemv_q4_0_kernel, KIND_Q4_0, 4, 4)
+LARQL_GEMV_KERNEL(gemv_q6k_kernel, KIND_Q6K, 2, 3)
 LARQL_GEMV_KERNEL(gemv_bf16_kernel, KIND_BF16, 4, 4)
 LARQL_GEMV_KERNEL(gemv_f16_kernel, KIND_F16, 4, 4)
 LARQL_GEMV_KERNEL(gemv_f32_kernel, KIND_F32, 2, 4)
@@ -1650,7 +1775,7 @@ static int g_unroll = getenv("LARQL_HIP_UNROLL") ? atoi(getenv("LARQL_HIP_UNROLL
 static int g_threads = getenv("LARQL_HIP_THREADS") ? atoi(getenv("LARQL_HIP_THREADS")) : 0;
 static uint32_t chunk_elems(int kind) {
     switch (kind) {
-        case KIND_Q4K: return 64;
+        case KIND_Q4K: case KIND_Q6K: return 64;
         case KIND_Q8_0: case KIND_MXFP4: case KIND_Q4_0: return 32;
         default: return 16;
     }
@@ -1784,6 +1909,7 @@ bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
     switch (j.kind) {
         case KIND_Q4K: j.row_bytes = (j.k / 256) * 144; break;
         case KIND_Q8_0: j.row_bytes = (j.k / 32) * 34; break;
+        case KIND_Q6K: if (j.k % 256 != 0) return false; j.row_bytes = (j.k / 256) * 210; break;
         case KIND_MXFP4: j.row_bytes = (j.k / 32) * 16; break;
         case KIND_Q4_0: j.row_bytes = (j.k / 32) * 18; break;
         case KIND_BF16: case KIND_F16: j.row_bytes = j.k * 2; break;
@@ -1967,6 +2093,7 @@ hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32
             else hipLaunchKernelGGL(gemv_mxfp4_u4_kernel, dim3(grid), dim3(threads), lds, stream, L);
             break;
         case KIND_Q4_0: hipLaunchKernelGGL(gemv_q4_0_kernel, dim3(grid), dim3(threads), lds, stream, L); break;
+        case KIND_Q6K: hipLaunchKernelGGL(gemv_q6k_kernel, dim3(grid), dim3(threads), lds, stream, L); break;
         case KIND_BF16: hipLaunchKernelGGL(gemv_bf16_kernel, dim3(grid), dim3(threads), lds, stream, L); break;
         case KIND_F16: hipLaunchKernelGGL(gemv_f16_kernel, dim3(grid), dim3(threads), lds, stream, L); break;
         case KIND_F32: hipLaunchKernelGGL(gemv_f32_kernel, dim3(grid), dim3(threads), lds, stream, L); break;

@@ -12,7 +12,8 @@ enum GemvKind : int32_t {
     KIND_MXFP4_MFMA = 8, // internal: likewise for MXFP4
     KIND_BF16_MFMA = 9,  // internal: bf16 rows against 2..8 activations at once (batch field of the job)
     KIND_Q4K_BATCH = 10, // internal: Q4_K rows against 2..4 activations at once
-    KIND_Q8_0_MFMA = 11  // internal: ggml Q8_0 rows short enough for the matrix-core kernel
+    KIND_Q8_0_MFMA = 11, // internal: ggml Q8_0 rows short enough for the matrix-core kernel
+    KIND_Q6K = 12        // Q6_K, 210-byte super-blocks (K-slice kernel)
 };
 
 constexpr int kGemvMaxThreads = 512;

@@ -63,6 +63,10 @@ class HipBackend {
         std::vector<float> out(num_rows);
         return some(larql_hip_q4k_matvec(ctx_, q4k.ptr, q4k.len, x.ptr, x.len, num_rows, hidden, out.data(), out.size()), out);
     }
+    std::optional<std::vector<float>> q6k_matvec(Slice<uint8_t> q6k, Slice<float> x, size_t num_rows, size_t hidden) {
+        std::vector<float> out(num_rows);
+        return some(larql_hip_q6k_matvec(ctx_, q6k.ptr, q6k.len, x.ptr, x.len, num_rows, hidden, out.data()), out);
+    }
     std::optional<std::pair<std::vector<float>, std::vector<float>>> q4k_dual_matvec(Slice<uint8_t> a, Slice<uint8_t> b,
                                                                                        Slice<float> x, size_t num_rows,
                                                                                        size_t hidden) {

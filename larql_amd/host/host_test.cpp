@@ -31,7 +31,19 @@ int main() {
     larql::HipBackend be;
     std::printf("%s | %s\n", be.name().c_str(), be.device_info().c_str());
     CHECK(be.supports_quant(larql::QuantFormat::Q4_K) && be.supports_quant(larql::QuantFormat::MXFP4));
-    CHECK(!be.supports_quant(larql::QuantFormat::Q6_K));
+    CHECK(be.supports_quant(larql::QuantFormat::Q6_K) && !be.supports_quant(larql::QuantFormat::Q5_K));
+    {
+        // one Q6_K super-block: every code 32 + 5 (low nibble 5, high bits 2), scale 3, d = 0.5 -> weight 7.5; x = 1 -> 1920
+        std::vector<uint8_t> b6(210, 0);
+        for (int i = 0; i < 128; i++) b6[i] = 0x55;
+        for (int i = 128; i < 192; i++) b6[i] = 0xAA;
+        for (int i = 192; i < 208; i++) b6[i] = 3;
+        b6[208] = 0x00; b6[209] = 0x38;  // f16 0.5
+        std::vector<float> x6(256, 1.0f);
+        auto o6 = be.q6k_matvec({b6.data(), b6.size()}, {x6.data(), x6.size()}, 1, 256);
+        CHECK(o6 && std::fabs((*o6)[0] - 1920.0f) < 1e-2f);
+        CHECK(!be.q6k_matvec({b6.data(), b6.size() - 1}, {x6.data(), x6.size()}, 1, 256));
+    }
 
     const size_t rows = 70, hidden = 512;
     std::vector<uint8_t> w(rows * 2 * 144);

@@ -460,6 +460,113 @@ void lq_q4k_matmul_into(float *out, const float *x, const uint8_t *w, size_t w_l
 
 /* ------------------------------------------------------------------ Q8_0 */
 
+/* ------------------------------------------------------------------------------------------------
+ * Q6_K.  Block of 256 values = 210 bytes: ql[128] low nibbles, qh[64] high bit pairs, 16 int8
+ * sub-block scales, f16 d.  Value = d * scale[j] * q, q = (lo4 | hi2 << 4) - 32.
+ * ---------------------------------------------------------------------------------------------- */
+
+/* quantize_q6_k — larql-compute/src/cpu/ops/q4_common/quantize.rs:197-276 */
+int lq_quantize_q6_k(const float *data, size_t n, uint8_t *out) {
+    if (n % 256 != 0) return 1;
+    size_t nsb = n / 256;
+    for (size_t sb = 0; sb < nsb; sb++) {
+        const float *block = data + sb * 256;
+        uint8_t *o = out + sb * 210;
+        float amax = 0.0f;
+        for (int i = 0; i < 256; i++) { float a = fabsf(block[i]); amax = fmaxf(amax, a); }
+        float d = amax / (31.0f * 127.0f);
+        int8_t sub_scales[16];
+        for (int j = 0; j < 16; j++) {
+            float sub_max = 0.0f;
+            for (int i = 0; i < 16; i++) sub_max = fmaxf(sub_max, fabsf(block[j * 16 + i]));
+            float sc = d > 0.0f ? sub_max / (31.0f * d) : 0.0f;
+            float r = roundf(sc);
+            if (r < -128.0f) r = -128.0f;
+            if (r > 127.0f) r = 127.0f;
+            sub_scales[j] = (int8_t)r;
+        }
+        uint8_t q6[256];
+        for (int j = 0; j < 16; j++) {
+            float sc = d * (float)sub_scales[j];
+            float inv_sc = fabsf(sc) > 1e-10f ? 1.0f / sc : 0.0f;
+            for (int i = 0; i < 16; i++) {
+                float r = roundf(block[j * 16 + i] * inv_sc);
+                if (r < -32.0f) r = -32.0f;
+                if (r > 31.0f) r = 31.0f;
+                q6[j * 16 + i] = (uint8_t)((int)r + 32);
+            }
+        }
+        for (int half = 0; half < 2; half++) {
+            int e = half * 128;
+            for (int l = 0; l < 32; l++) {
+                uint8_t q1 = q6[e + l], q2 = q6[e + l + 32], q3 = q6[e + l + 64], q4 = q6[e + l + 96];
+                o[half * 64 + l] = (uint8_t)((q1 & 0x0F) | ((q3 & 0x0F) << 4));
+                o[half * 64 + l + 32] = (uint8_t)((q2 & 0x0F) | ((q4 & 0x0F) << 4));
+                o[128 + half * 32 + l] = (uint8_t)(((q1 >> 4) & 3) | (((q2 >> 4) & 3) << 2) | (((q3 >> 4) & 3) << 4) | (((q4 >> 4) & 3) << 6));
+            }
+        }
+        for (int j = 0; j < 16; j++) o[192 + j] = (uint8_t)sub_scales[j];
+        uint16_t db = lq_f32_to_f16_trunc(d);
+        o[208] = (uint8_t)(db & 0xFF);
+        o[209] = (uint8_t)(db >> 8);
+    }
+    return 0;
+}
+
+/* q6k_subblock_vals — larql-models/src/quant/ggml/q6_k.rs:19-40 */
+void lq_q6k_subblock_vals(const uint8_t *block, size_t j, int8_t *out16) {
+    const uint8_t *ql = block, *qh = block + 128;
+    size_t half = j / 8, g = j % 8, plane = g / 2, lbase = (g % 2) * 16;
+    size_t ql_off = half * 64 + (plane & 1) * 32 + lbase, qh_off = half * 32 + lbase;
+    unsigned shift = (unsigned)plane * 2;
+    for (int i = 0; i < 16; i++) {
+        int lo4 = plane < 2 ? (ql[ql_off + i] & 0x0F) : (ql[ql_off + i] >> 4);
+        int hi2 = (qh[qh_off + i] >> shift) & 0x03;
+        out16[i] = (int8_t)((lo4 | (hi2 << 4)) - 32);
+    }
+}
+
+/* dequantize_q6_k — q6_k.rs:173-195 */
+int lq_dequantize_q6_k(const uint8_t *data, size_t data_len, size_t n, float *out) {
+    if (n % 256 != 0) return 1;
+    size_t nsb = n / 256;
+    if (data_len < nsb * 210) return 1;
+    for (size_t sb = 0; sb < nsb; sb++) {
+        const uint8_t *block = data + sb * 210;
+        float d = lq_f16_to_f32((uint16_t)(block[208] | (block[209] << 8)));
+        for (size_t j = 0; j < 16; j++) {
+            float sc = d * (float)(int8_t)block[192 + j];
+            int8_t vals[16];
+            lq_q6k_subblock_vals(block, j, vals);
+            for (int i = 0; i < 16; i++) out[sb * 256 + j * 16 + i] = sc * (float)vals[i];
+        }
+    }
+    return 0;
+}
+
+/* q6k_matvec::dispatch — larql-compute/src/cpu/ops/q6k_matvec.rs:45-91 (per sub-block: sub = sum v*x; acc += sc*sub) */
+int lq_q6k_matvec(const uint8_t *w, size_t w_len, const float *x, size_t rows, size_t hidden, float *out) {
+    size_t nsb = hidden / 256, bpr = nsb * 210;
+    if (hidden % 256 != 0 || w_len < rows * bpr) return 1;
+    for (size_t row = 0; row < rows; row++) {
+        float acc = 0.0f;
+        for (size_t sb = 0; sb < nsb; sb++) {
+            const uint8_t *block = w + row * bpr + sb * 210;
+            float d = lq_f16_to_f32((uint16_t)(block[208] | (block[209] << 8)));
+            for (size_t j = 0; j < 16; j++) {
+                float sc = d * (float)(int8_t)block[192 + j];
+                int8_t vals[16];
+                lq_q6k_subblock_vals(block, j, vals);
+                float sub = 0.0f;
+                for (int i = 0; i < 16; i++) sub += (float)vals[i] * x[sb * 256 + j * 16 + i];
+                acc += sc * sub;
+            }
+        }
+        out[row] = acc;
+    }
+    return 0;
+}
+
 /* larql-models/src/quant/ggml/quantize.rs:50-77.  Codes use the reciprocal
  * of the un-rounded f32 scale.
  * Pinned: byte-for-byte against the reference-held ggml golden blocks

@@ -50,6 +50,12 @@ void lq_q4k_matmul_into(float *out, const float *x, const uint8_t *w, size_t w_l
                         size_t rows, size_t hidden, size_t seq);
 
 /* ---- Q8_0 (ggml, 34-byte blocks) ------------------------------------- */
+/* Q6_K: 210-byte super-blocks (ggml planar layout) */
+int  lq_quantize_q6_k(const float *data, size_t n, uint8_t *out);              /* q4_common/quantize.rs:197-276 */
+void lq_q6k_subblock_vals(const uint8_t *block, size_t j, int8_t *out16);     /* larql-models/src/quant/ggml/q6_k.rs:19-40 */
+int  lq_dequantize_q6_k(const uint8_t *data, size_t data_len, size_t n, float *out); /* q6_k.rs:173-195 */
+int  lq_q6k_matvec(const uint8_t *w, size_t w_len, const float *x, size_t rows, size_t hidden, float *out); /* cpu/ops/q6k_matvec.rs:45-91 */
+
 int  lq_quantize_q8_0(const float *data, size_t n, uint8_t *out);
 int  lq_dequantize_q8_0(const uint8_t *data, size_t data_len, size_t n, float *out);
 int  lq_q8_0_gemv(const uint8_t *blocks, size_t blocks_len, const float *x, size_t x_len,

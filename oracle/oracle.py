@@ -175,6 +175,30 @@ def q4k_matmul(w, x, rows: int, hidden: int, seq: int) -> np.ndarray:
 
 
 # ---- Q8_0 -----------------------------------------------------------------
+def quantize_q6_k(data) -> np.ndarray:
+    data = _f32(data).ravel()
+    out = np.empty(data.size // 256 * 210, dtype=np.uint8)
+    if _lib.lq_quantize_q6_k(_p(data, _f32p), _sz(data.size), _p(out, _u8p)):
+        raise ValueError("Q6_K: element count must be multiple of 256")
+    return out
+
+
+def dequantize_q6_k(data, n: int):
+    data = _u8(data).ravel()
+    out = np.empty(n, dtype=np.float32)
+    if _lib.lq_dequantize_q6_k(_p(data, _u8p), _sz(data.size), _sz(n), _p(out, _f32p)):
+        return None
+    return out
+
+
+def q6k_matvec(w, x, rows: int, hidden: int):
+    w, x = _u8(w).ravel(), _f32(x).ravel()
+    out = np.empty(rows, dtype=np.float32)
+    if x.size != hidden or _lib.lq_q6k_matvec(_p(w, _u8p), _sz(w.size), _p(x, _f32p), _sz(rows), _sz(hidden), _p(out, _f32p)):
+        return None
+    return out
+
+
 def quantize_q8_0(data) -> np.ndarray:
     data = _f32(data).ravel()
     out = np.empty(data.size // 32 * 34, dtype=np.uint8)

@@ -100,6 +100,50 @@ def quantize_q4_k(data):
     return out.reshape(-1)
 
 
+def dequantize_q6_k(data, n):
+    """larql-models/src/quant/ggml/q6_k.rs:19-40,173-195 (ggml planar layout), written plane by plane."""
+    nb = n // 256
+    blocks = np.asarray(data, np.uint8)[: nb * 210].reshape(nb, 210)
+    ql = blocks[:, :128].reshape(nb, 2, 2, 32)          # [block, half, row, l]
+    qh = blocks[:, 128:192].reshape(nb, 2, 32)          # [block, half, l]
+    sc = blocks[:, 192:208].view(np.int8).astype(F)     # [block, 16]
+    d = f16_bits_to_f32(blocks[:, 208].astype(np.uint16) | (blocks[:, 209].astype(np.uint16) << 8))
+    q = np.empty((nb, 2, 4, 32), np.int32)              # [block, half, plane, l]: element half*128 + plane*32 + l
+    for plane in range(4):
+        lo4 = (ql[:, :, plane & 1, :] & 0x0F) if plane < 2 else (ql[:, :, plane & 1, :] >> 4)
+        hi2 = (qh >> (2 * plane)) & 3
+        q[:, :, plane, :] = (lo4.astype(np.int32) | (hi2.astype(np.int32) << 4)) - 32
+    q = q.reshape(nb, 16, 16).astype(F)                 # 16 sub-blocks of 16 in element order
+    scale = (d[:, None] * sc).astype(F)
+    return (scale[:, :, None] * q).astype(F).reshape(-1)
+
+
+def quantize_q6_k(data):
+    """larql-compute/src/cpu/ops/q4_common/quantize.rs:197-276."""
+    x = np.asarray(data, F).reshape(-1, 16, 16)
+    nb = x.shape[0]
+    amax = np.abs(x).max((1, 2)).astype(F)
+    d = (amax / F(31.0 * 127.0)).astype(F)
+    sub_max = np.abs(x).max(-1).astype(F)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        sc = np.where(d[:, None] > 0, sub_max / (F(31.0) * d)[:, None], F(0)).astype(F)
+        ss = np.clip(rust_round(sc), -128, 127).astype(np.int8)
+        scale = (d[:, None] * ss.astype(F)).astype(F)
+        inv = np.where(np.abs(scale) > F(1e-10), F(1.0) / scale, F(0)).astype(F)
+        q = (np.clip(rust_round((x * inv[:, :, None]).astype(F)), -32, 31).astype(np.int32) + 32).astype(np.uint8)
+    q = q.reshape(nb, 2, 4, 32)                          # [block, half, plane, l]
+    out = np.zeros((nb, 210), np.uint8)
+    ql = np.empty((nb, 2, 2, 32), np.uint8)
+    ql[:, :, 0, :] = (q[:, :, 0, :] & 0x0F) | ((q[:, :, 2, :] & 0x0F) << 4)
+    ql[:, :, 1, :] = (q[:, :, 1, :] & 0x0F) | ((q[:, :, 3, :] & 0x0F) << 4)
+    qh = ((q[:, :, 0, :] >> 4) & 3) | (((q[:, :, 1, :] >> 4) & 3) << 2) | (((q[:, :, 2, :] >> 4) & 3) << 4) | (((q[:, :, 3, :] >> 4) & 3) << 6)
+    out[:, :128] = ql.reshape(nb, 128)
+    out[:, 128:192] = qh.reshape(nb, 64)
+    out[:, 192:208] = ss.view(np.uint8)
+    out[:, 208:210] = f32_to_f16_trunc(d).reshape(nb, 1).view(np.uint8)
+    return out.reshape(-1)
+
+
 def quantize_q8_0(data):
     """larql-models/src/quant/ggml/quantize.rs:50-77."""
     x = np.asarray(data, F).reshape(-1, 32)

@@ -136,6 +136,33 @@ def test_q4k_dual_and_matmul(be):
     assert bad is not None and not bad.any()
 
 
+# ------------------------------------------------------------------ Q6_K
+@pytest.mark.parametrize("rows,cols", [(2560, 10240), (1031, 2560), (77, 256), (5, 768), (640, 2304), (4100, 512), (1, 5120)])
+def test_q6k_matvec_matches_oracle(be, fmt, rows, cols):
+    # rows of an odd number of 210-byte super-blocks leave every other row 2 bytes off a dword boundary
+    w, x = weights(rows * 3 + cols, rows, cols)
+    w[0, :16] *= 1e-4
+    q = O.quantize_q6_k(w)
+    want = O.q6k_matvec(q, x, rows, cols)
+    got = be.q6k_matvec(q, x, rows, cols)
+    assert got is not None and got.shape == (rows,)
+    assert rel_l2(got, want) < TOL
+    assert np.max(np.abs(got - want)) < 1e-3 * (np.abs(want).mean() + 1e-12)
+    assert np.array_equal(got.view(np.uint32), be.q6k_matvec(q, x, rows, cols).view(np.uint32))
+    assert be.q6k_matvec(q[:-1], x, rows, cols) is None and be.q6k_matvec(q, x[:-1], rows, cols) is None
+    assert be.q6k_matvec(np.concatenate([q, q[:7]]), x, rows, cols) is not None
+    # the trait's format dispatcher reaches the same kernel
+    via = be.quant_matvec(fmt.FMT_Q6_K, q, x, rows, cols)
+    assert via is not None and np.array_equal(via.view(np.uint32), got.view(np.uint32))
+
+
+def test_q6k_matvec_shape_rules(be):
+    assert be.q6k_matvec(np.zeros(210, np.uint8), np.zeros(255, F), 1, 255) is None      # hidden % 256
+    z = be.q6k_matvec(np.zeros(0, np.uint8), np.zeros(0, F), 3, 0)
+    assert z is not None and z.shape == (3,) and not z.any()
+    assert be.q6k_matvec(np.zeros(0, np.uint8), np.zeros(256, F), 0, 256).size == 0
+
+
 # ------------------------------------------------------------------ Q8_0
 @pytest.mark.parametrize("n,k", [(4099, 2560), (64, 10240), (9, 128), (1000, 2048), (17, 256), (333, 1792), (48, 2816)])
 def test_q8_0_gemv_matches_oracle(be, n, k):

@@ -119,16 +119,64 @@ def ggml_golden():
     return d
 
 
-@pytest.mark.parametrize("enc", ["q4_K", "q8_0"])
+@pytest.mark.parametrize("enc", ["q4_K", "q8_0", "q6_K"])
 def test_decoders_bit_exact_on_llama_cpp_golden(ggml_golden, enc):
     case = next(c for c in ggml_golden["cases"] if c["encoding"] == enc)
     raw = np.frombuffer(bytes.fromhex(case["quantised_hex"]), np.uint8)
     want = np.array(case["dequantised_bits"], np.uint32)
     n = case["elements"]
-    got = O.dequantize_q4_k(raw, n) if enc == "q4_K" else O.dequantize_q8_0(raw, n)
-    assert np.array_equal(bits(got), want)
-    alt = npr.dequantize_q4_k(raw, n) if enc == "q4_K" else npr.dequantize_q8_0(raw, n)
-    assert np.array_equal(bits(alt), want)
+    dec = {"q4_K": (O.dequantize_q4_k, npr.dequantize_q4_k), "q8_0": (O.dequantize_q8_0, npr.dequantize_q8_0),
+           "q6_K": (O.dequantize_q6_k, npr.dequantize_q6_k)}[enc]
+    assert np.array_equal(bits(dec[0](raw, n)), want)
+    assert np.array_equal(bits(dec[1](raw, n)), want)
+
+
+def test_q6k_matvec_on_golden_bytes_matches_decode(ggml_golden):
+    # the kernel must equal decode-then-dot on llama.cpp's own bytes (f64 reference, 5e-6 as for Q4_K)
+    case = next(c for c in ggml_golden["cases"] if c["encoding"] == "q6_K")
+    raw = np.frombuffer(bytes.fromhex(case["quantised_hex"]), np.uint8)
+    w = np.array(case["dequantised_bits"], np.uint32).view(F).reshape(2, 256)
+    x = np.random.default_rng(5).standard_normal(256).astype(F)
+    got = O.q6k_matvec(raw, x, 2, 256)
+    exact = w.astype(np.float64) @ x.astype(np.float64)
+    assert np.max(np.abs(got - exact) / np.maximum(np.abs(exact), 1e-6)) < 5e-6
+    assert O.q6k_matvec(raw[:-1], x, 2, 256) is None and O.q6k_matvec(raw, x[:-1], 2, 256) is None
+
+
+def test_q6k_encoder_closed_forms_and_second_restatement():
+    # all-zero block -> 210 zero bytes except the biased codes (q = 0 -> 32: low nibble 0, high bits 2)
+    z = O.quantize_q6_k(np.zeros(256, F))
+    assert z.size == 210 and not z[:128].any() and (z[128:192] == 0xAA).all() and not z[192:].any()
+    assert not O.dequantize_q6_k(z, 256).any()
+    # constant block c > 0: amax = c, d = c/3937, every sub-scale 127, every q = round(c / (d*127)) = 31
+    c = F(0.75)
+    b = O.quantize_q6_k(np.full(256, c, F))
+    d = F(c / F(31.0 * 127.0))
+    assert (b[192:208].view(np.int8) == 127).all()
+    assert (int(b[208]) | (int(b[209]) << 8)) == int(npr.f32_to_f16_trunc(np.array([d], F))[0])
+    assert (b[:128] == 0xFF).all() and (b[128:192] == 0xFF).all()          # 31 + 32 = 63 = 0b111111 everywhere
+    # negative constant: q = -31 -> 1: low nibble 1, high bits 0
+    n = O.quantize_q6_k(np.full(256, -c, F))
+    assert (n[:128] == 0x11).all() and not n[128:192].any()
+    # one sub-block 4x larger than the rest: its scale saturates at 127, the others land near 32
+    rng = np.random.default_rng(9)
+    x = (rng.standard_normal(256) * 0.01).astype(F)
+    x[48:64] *= 4
+    e = O.quantize_q6_k(x)
+    sc = e[192:208].view(np.int8)
+    assert sc.max() == sc[np.abs(x.reshape(16, 16)).max(1).argmax()] and sc.max() >= 100
+    # two independent restatements agree byte for byte, and the round trip is within half a level
+    for seed, scale in ((1, 0.02), (2, 1.0), (3, 30.0)):
+        w = (np.random.default_rng(seed).standard_normal(256 * 24) * scale).astype(F)
+        q = O.quantize_q6_k(w)
+        assert np.array_equal(q, npr.quantize_q6_k(w))
+        dq = O.dequantize_q6_k(q, w.size)
+        assert np.array_equal(bits(dq), bits(npr.dequantize_q6_k(q, w.size)))
+        # half a level of the sub-block (level = d*scale ~ sub_max/31, scale rounded to an integer: +- d/2),
+        # plus what the clamp at +-31 levels can cut off when the scale rounds down (31 * d/2)
+        d = np.repeat(np.abs(w.reshape(-1, 256)).max(1) / (31.0 * 127.0), 256)
+        sub_max = np.repeat(np.abs(w.reshape(-1, 16)).max(1), 16)
+        assert np.all(np.abs(dq - w) <= 0.5 * sub_max / 31.0 + 16.0 * d + 1e-12)
 
 
 def test_direct_gemv_on_golden_bytes_matches_decode(ggml_golden):
