@@ -635,6 +635,7 @@ __device__ __forceinline__ void run_q4k_mfma(const GemvJob &j, uint32_t tile_a, 
     const uint32_t u0 = lane, u1 = 64 + lane, u2 = 128 + (lane >> 2);
     const uint32_t r0 = u0 / 9, r1 = u1 / 9, r2 = u2 / 9;
     const uint32_t w0 = (u0 - r0 * 9) * 16, w1 = (u1 - r1 * 9) * 16, w2 = (u2 - r2 * 9) * 16 + (lane & 3u) * 4;
+    const uint32_t o0 = r0 * row_bytes + w0, o1 = r1 * row_bytes + w1, o2 = r2 * row_bytes + w2;
     const uint8_t *wcol = j.w + (size_t)wv * 144;
     const uint32_t nt = tile_b - tile_a;
 
@@ -643,11 +644,17 @@ __device__ __forceinline__ void run_q4k_mfma(const GemvJob &j, uint32_t tile_a, 
     auto issue = [&]() {
         // past the end the last wave-tile is read again: every wavefront keeps the same number of loads in flight
         const uint32_t tl = min(tile_a + it_tb + it_tl, tile_b - 1);
-        const uint8_t *gp = wcol + (size_t)it_p * nwj * 144;
+        // wave-uniform 64-bit base + per-lane 32-bit offset; only a ragged last tile recomputes the offsets
         const uint32_t rb = tl * 16;
-        const uint8_t *g0 = gp + (size_t)min(rb + r0, rows - 1) * row_bytes + w0;
-        const uint8_t *g1 = gp + (size_t)min(rb + r1, rows - 1) * row_bytes + w1;
-        const uint8_t *g2 = gp + (size_t)min(rb + r2, rows - 1) * row_bytes + w2;
+        const uint8_t *gp = wcol + (size_t)it_p * nwj * 144 + (size_t)rb * row_bytes;
+        uint32_t a0 = o0, a1 = o1, a2 = o2;
+        if (rb + 16 > rows) {
+            const uint32_t lim = rows - 1 - rb;
+            a0 = min(r0, lim) * row_bytes + w0;
+            a1 = min(r1, lim) * row_bytes + w1;
+            a2 = min(r2, lim) * row_bytes + w2;
+        }
+        const uint8_t *g0 = gp + a0, *g1 = gp + a1, *g2 = gp + a2;
         uint8_t *lp = ring + (n_issue % NS) * kQ4kTileBytes;
         __builtin_amdgcn_global_load_lds((g_vp)g0, (lds_vp)lp, 16, 0, 0);
         __builtin_amdgcn_global_load_lds((g_vp)g1, (lds_vp)(lp + 1024), 16, 0, 0);
@@ -661,10 +668,15 @@ __device__ __forceinline__ void run_q4k_mfma(const GemvJob &j, uint32_t tile_a, 
             }
         }
     };
+    // the activations of all this wavefront's columns are requested first and together (one memory round
+    // trip, ahead of the weight tiles in the in-order return queue), then prepared while the tiles fly
+    Q4kRaw raw[kQ4kMaxColPasses];
+#pragma unroll
+    for (int p = 0; p < kQ4kMaxColPasses; p++)
+        if ((uint32_t)p < np) raw[p] = q4k_mfma_load_col(j.x, wv + nwj * p, lane);
     if (np >= 1)
         for (int s = 0; s < NS - 1; s++) issue();
 
-    // (prepared while the first weight tiles are on their way)
     // Column state: in registers when the wavefront has one column; with several it is prepared once per
     // job into this wavefront's own LDS area (1 KB of operands + 64 B of scales and sums per column) and
     // fetched at every column change.
@@ -682,15 +694,18 @@ __device__ __forceinline__ void run_q4k_mfma(const GemvJob &j, uint32_t tile_a, 
         q4k_mfma_operands(xm, col, jr);
     };
     if (np == 1) {
-        col = q4k_mfma_finish_col(q4k_mfma_load_col(j.x, wv, lane), lane);
+        col = q4k_mfma_finish_col(raw[0], lane);
         q4k_mfma_operands(xm, col, jr);
     } else if (np > 1) {
-        for (uint32_t p = 0; p < np; p++) {
-            const Q4kCol c = q4k_mfma_finish_col(q4k_mfma_load_col(j.x, wv + nwj * p, lane), lane);
-            uint8_t *cp = cols + p * kQ4kColBytes;
-            *reinterpret_cast<u32x4 *>(cp + lane * 16) = (u32x4){c.xq[0], c.xq[1], c.xq[2], c.xq[3]};
-            if (lane == 0) *reinterpret_cast<float *>(cp + 1024) = c.k;
-            if (jr == 0) *reinterpret_cast<float2_t *>(cp + 1024 + 16 + kq * 8) = (float2_t){c.sum_lo, c.sum_hi};
+#pragma unroll
+        for (int p = 0; p < kQ4kMaxColPasses; p++) {
+            if ((uint32_t)p < np) {
+                const Q4kCol c = q4k_mfma_finish_col(raw[p], lane);
+                uint8_t *cp = cols + p * kQ4kColBytes;
+                *reinterpret_cast<u32x4 *>(cp + lane * 16) = (u32x4){c.xq[0], c.xq[1], c.xq[2], c.xq[3]};
+                if (lane == 0) *reinterpret_cast<float *>(cp + 1024) = c.k;
+                if (jr == 0) *reinterpret_cast<float2_t *>(cp + 1024 + 16 + kq * 8) = (float2_t){c.sum_lo, c.sum_hi};
+            }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own writes, own reads: program order is enough
     }
@@ -833,8 +848,7 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
     const uint32_t nw_launch = blockDim.x >> 6;
     const uint32_t jr = lane & 15u, kg = lane >> 4;
     const uint32_t nwj = j.rpp, steps = j.cpr, cw = (uint32_t)j.pad, PW = nwj * 2;
-    const uint32_t rows = (uint32_t)j.rows, k = (uint32_t)j.k, nb = k / 32;
-    const size_t row_bytes = j.row_bytes;
+    const uint32_t rows = (uint32_t)j.rows, k = (uint32_t)j.k, nb = k / 32, row_bytes = (uint32_t)j.row_bytes;
     uint8_t *ring = lds + wv * (NS * slot_bytes);
     float *part = reinterpret_cast<float *>(lds + nw_launch * (NS * slot_bytes));
     const uint32_t step0 = wv * cw;
@@ -849,19 +863,27 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
         blk[s] = min(b, nb - 1);
     }
 
+    const uint32_t wro_full = jr * row_bytes, sro_full = jr * nb;
     const uint32_t nt = tile_b - tile_a;
     uint32_t it_tile = tile_a, n_issue = 0;
     auto issue = [&]() {
         const uint32_t tl = min(it_tile, tile_b - 1);  // past the end: the last tile again (uniform load counts)
-        const uint32_t row = min(tl * 16 + jr, rows - 1);
-        const uint8_t *wrow = j.w + (size_t)row * row_bytes;
-        const uint8_t *srow = j.aux + (size_t)row * nb;
+        // wave-uniform 64-bit bases + per-lane 32-bit offsets (the lane's row within the tile, clamped into the matrix)
+        const uint32_t rb = tl * 16;
+        const uint8_t *wbase = j.w + (size_t)rb * row_bytes;
+        const uint8_t *sbase = j.aux + (size_t)rb * nb;
+        uint32_t wro = wro_full, sro = sro_full;
+        if (rb + 16 > rows) {  // ragged last tile only
+            const uint32_t rl = min(jr, rows - 1 - rb);
+            wro = rl * row_bytes;
+            sro = rl * nb;
+        }
         uint8_t *lp = ring + (n_issue % NS) * slot_bytes;
 #pragma unroll
         for (int s = 0; s < kMx4MaxSteps; s++) {
             if ((uint32_t)s < cw) {
-                __builtin_amdgcn_global_load_lds((g_vp)(wrow + (size_t)blk[s] * 16), (lds_vp)(lp + s * 1024), 16, 0, 0);
-                __builtin_amdgcn_global_load_lds((g_vp)(srow + blk[s]), (lds_vp)(lp + cw * 1024 + s * 256), 1, 0, 0);  // lands zero-extended in dword slot `lane`
+                __builtin_amdgcn_global_load_lds((g_vp)(wbase + (wro + blk[s] * 16)), (lds_vp)(lp + s * 1024), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((g_vp)(sbase + (sro + blk[s])), (lds_vp)(lp + cw * 1024 + s * 256), 1, 0, 0);  // lands zero-extended in dword slot `lane`
             }
         }
         n_issue++;
@@ -978,19 +1000,23 @@ __device__ __forceinline__ void run_bf16_mfma(const GemvJob &j, uint32_t tile_a,
     const uint32_t nw_launch = blockDim.x >> 6;
     const uint32_t jr = lane & 15u, kq = lane >> 4;
     const uint32_t nwj = j.rpp, cols = j.cpr, batch = j.batch, nsets = (batch + 3) / 4;
-    const uint32_t rows = (uint32_t)j.rows;
-    const size_t row_bytes = j.row_bytes;
+    const uint32_t rows = (uint32_t)j.rows, row_bytes = (uint32_t)j.row_bytes;
     uint8_t *ring = lds + wv * (NS * kBfTileBytes);
     float *part = reinterpret_cast<float *>(lds + nw_launch * (NS * kBfTileBytes));
     const uint32_t np = wv < nwj ? (cols - wv + nwj - 1) / nwj : 0;  // columns wv, wv+nwj of this wavefront
     const uint32_t PW = 8 * nw_launch;                              // partials per row: [position][wavefront]
 
+    const uint32_t lane_off = jr * row_bytes + kq * 16;
     const uint32_t nt = tile_b - tile_a;
     uint32_t it_tile = tile_a, it_p = 0, n_issue = 0;
     auto issue = [&]() {
         const uint32_t tl = min(it_tile, tile_b - 1);  // past the end: the last wave-tile again (uniform load counts)
-        const uint32_t row = min(tl * 16 + jr, rows - 1);
-        const uint8_t *gp = j.w + (size_t)row * row_bytes + (size_t)(wv + nwj * it_p) * 256 + kq * 16;
+        // wave-uniform 64-bit base + per-lane 32-bit offset (the lane's row within the tile, clamped into the matrix)
+        const uint32_t rb = tl * 16;
+        const uint8_t *gb = j.w + (size_t)rb * row_bytes + (size_t)(wv + nwj * it_p) * 256;
+        uint32_t lo = lane_off;
+        if (rb + 16 > rows) lo = min(jr, rows - 1 - rb) * row_bytes + kq * 16;  // ragged last tile only
+        const uint8_t *gp = gb + lo;
         uint8_t *lp = ring + (n_issue % NS) * kBfTileBytes;
 #pragma unroll
         for (int s = 0; s < 4; s++) __builtin_amdgcn_global_load_lds((g_vp)(gp + s * 64), (lds_vp)(lp + s * 1024), 16, 0, 0);
@@ -1149,14 +1175,22 @@ __device__ __forceinline__ void run_q4k_batch(const GemvJob &j, uint32_t tile_a,
     const uint32_t u0 = lane, u1 = 64 + lane, u2 = 128 + (lane >> 2);
     const uint32_t r0 = u0 / 9, r1 = u1 / 9, r2 = u2 / 9;
     const uint32_t w0 = (u0 - r0 * 9) * 16, w1 = (u1 - r1 * 9) * 16, w2 = (u2 - r2 * 9) * 16 + (lane & 3u) * 4;
+    const uint32_t o0 = r0 * row_bytes + w0, o1 = r1 * row_bytes + w1, o2 = r2 * row_bytes + w2;
     const uint8_t *wcol = j.w + (size_t)wv * 144;
     const uint32_t nt = tile_b - tile_a;
     uint32_t it_tile = tile_a, n_issue = 0;
     auto issue = [&]() {
+        // wave-uniform 64-bit base + per-lane 32-bit offset; only a ragged last tile recomputes the offsets
         const uint32_t rb = min(it_tile, tile_b - 1) * 16;
-        const uint8_t *g0 = wcol + (size_t)min(rb + r0, rows - 1) * row_bytes + w0;
-        const uint8_t *g1 = wcol + (size_t)min(rb + r1, rows - 1) * row_bytes + w1;
-        const uint8_t *g2 = wcol + (size_t)min(rb + r2, rows - 1) * row_bytes + w2;
+        const uint8_t *gp = wcol + (size_t)rb * row_bytes;
+        uint32_t a0 = o0, a1 = o1, a2 = o2;
+        if (rb + 16 > rows) {
+            const uint32_t lim = rows - 1 - rb;
+            a0 = min(r0, lim) * row_bytes + w0;
+            a1 = min(r1, lim) * row_bytes + w1;
+            a2 = min(r2, lim) * row_bytes + w2;
+        }
+        const uint8_t *g0 = gp + a0, *g1 = gp + a1, *g2 = gp + a2;
         uint8_t *lp = ring + (n_issue % NS) * kQ4kTileBytes;
         __builtin_amdgcn_global_load_lds((g_vp)g0, (lds_vp)lp, 16, 0, 0);
         __builtin_amdgcn_global_load_lds((g_vp)g1, (lds_vp)(lp + 1024), 16, 0, 0);
@@ -1299,19 +1333,19 @@ __device__ __forceinline__ void run_q8_0_mfma(const GemvJob &j, uint32_t tile_a,
     const uint32_t nw_launch = blockDim.x >> 6;
     const uint32_t jr = lane & 15u, kq = lane >> 4;
     const uint32_t nwj = j.rpp, PW = nwj * 4;
-    const uint32_t rows = (uint32_t)j.rows;
-    const size_t row_bytes = j.row_bytes;
+    const uint32_t rows = (uint32_t)j.rows, row_bytes = (uint32_t)j.row_bytes;
     uint8_t *ring = lds + wv * (NS * kQ8TileBytes);
     float *part = reinterpret_cast<float *>(lds + nw_launch * (NS * kQ8TileBytes));
     const bool working = wv < nwj;
 
     // lane's pieces of a wave-tile in 16-byte units u = row*17 + piece: four full loads, then 256 B dword by dword
-    uint32_t rw[5], ow[5];
+    uint32_t rw[5], ow[5], off[5];
 #pragma unroll
     for (int q = 0; q < 5; q++) {
         const uint32_t u = q < 4 ? 64 * q + lane : 256 + (lane >> 2);
         rw[q] = u / 17;
         ow[q] = (u - rw[q] * 17) * 16 + (q < 4 ? 0 : (lane & 3u) * 4);
+        off[q] = rw[q] * row_bytes + ow[q];
     }
     const uint8_t *wcol = j.w + (size_t)wv * kQ8RowBytes;
     const uint32_t nt = tile_b - tile_a;
@@ -1319,10 +1353,20 @@ __device__ __forceinline__ void run_q8_0_mfma(const GemvJob &j, uint32_t tile_a,
     auto issue = [&]() {
         const uint32_t rb = min(it_tile, tile_b - 1) * 16;
         uint8_t *lp = ring + (n_issue % NS) * kQ8TileBytes;
+        // wave-uniform 64-bit base + per-lane 32-bit offset; only a ragged last tile recomputes the offsets
+        const uint8_t *gp = wcol + (size_t)rb * row_bytes;
+        uint32_t a[5];
+#pragma unroll
+        for (int q = 0; q < 5; q++) a[q] = off[q];
+        if (rb + 16 > rows) {
+            const uint32_t lim = rows - 1 - rb;
+#pragma unroll
+            for (int q = 0; q < 5; q++) a[q] = min(rw[q], lim) * row_bytes + ow[q];
+        }
 #pragma unroll
         for (int q = 0; q < 4; q++)
-            __builtin_amdgcn_global_load_lds((g_vp)(wcol + (size_t)min(rb + rw[q], rows - 1) * row_bytes + ow[q]), (lds_vp)(lp + q * 1024), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((g_vp)(wcol + (size_t)min(rb + rw[4], rows - 1) * row_bytes + ow[4]), (lds_vp)(lp + 4096), 4, 0, 0);
+            __builtin_amdgcn_global_load_lds((g_vp)(gp + a[q]), (lds_vp)(lp + q * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((g_vp)(gp + a[4]), (lds_vp)(lp + 4096), 4, 0, 0);
         n_issue++;
         if (it_tile < tile_b) it_tile++;
     };
@@ -1577,6 +1621,22 @@ __device__ __forceinline__ void run_dense(const GemvJob &j, uint32_t p0, uint32_
     }
 }
 
+// A job descriptor as wave-uniform values.  The table pointer is generic (it may name the kernel-argument
+// block or device memory), and the compiler treats whatever a generic load returns as different per lane:
+// every address and loop bound derived from it would be computed 64 times over in vector registers.
+// Broadcasting the words from the first lane puts the descriptor, and all arithmetic on it, on the scalar side.
+__device__ __forceinline__ GemvJob uniform_job(const GemvJob *src) {
+    static_assert(sizeof(GemvJob) % 4 == 0, "descriptor is a whole number of dwords");
+    constexpr int N = sizeof(GemvJob) / 4;
+    uint32_t w[N];
+    __builtin_memcpy(w, src, sizeof(GemvJob));
+#pragma unroll
+    for (int i = 0; i < N; i++) w[i] = __builtin_amdgcn_readfirstlane(w[i]);
+    GemvJob j;
+    __builtin_memcpy(&j, w, sizeof(GemvJob));
+    return j;
+}
+
 // ---------------------------------------------------------------------------
 // The kernels, one per format so each gets its own register budget: workgroup
 // b sweeps passes [P*b/G, P*(b+1)/G) of the launch's pass list, job by job.
@@ -1591,11 +1651,11 @@ __device__ __forceinline__ void gemv_body(const GemvLaunch &L, float *part) {
     uint32_t lo = 0, hi = L.n_jobs;
     while (lo + 1 < hi) {
         const uint32_t mid = (lo + hi) >> 1;
-        if (jobs[mid].pass_begin <= p) lo = mid; else hi = mid;
+        if ((uint32_t)__builtin_amdgcn_readfirstlane(jobs[mid].pass_begin) <= p) lo = mid; else hi = mid;
     }
     uint32_t ji = lo;
     while (p < p_end) {
-        GemvJob j = jobs[ji];
+        GemvJob j = uniform_job(jobs + ji);
         if (j.sel) {  // run-time expert selection: one bank of equally shaped matrices
             const uint32_t e = __builtin_amdgcn_readfirstlane(*(const GLOBAL_AS uint32_t *)j.sel);
             j.w += (size_t)e * j.w_sel_stride;
@@ -1646,15 +1706,16 @@ __global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_mfma_kernel(GemvLa
     uint32_t lo = 0, hi = L.n_jobs;
     while (lo + 1 < hi) {
         const uint32_t mid = (lo + hi) >> 1;
-        if (jobs[mid].pass_begin <= p) lo = mid; else hi = mid;
+        if ((uint32_t)__builtin_amdgcn_readfirstlane(jobs[mid].pass_begin) <= p) lo = mid; else hi = mid;
     }
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
-        const GemvJob j = jobs[ji];
+        const GemvJob j = uniform_job(jobs + ji);
         const uint32_t seg_end = min(p_end, j.pass_begin + j.n_pass);
         // a tile belongs to the workgroup whose share contains its first cost unit
-        const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin;
-        const uint32_t tile_a = (a + j.cpr - 1) / j.cpr, tile_b = (b + j.cpr - 1) / j.cpr;
+        // (the job's cost range opens with its start-up allowance; tile t covers [su + t*cpt, su + (t+1)*cpt))
+        const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin, cpt = (uint32_t)j.pad, su = j.pad2;
+        const uint32_t tile_a = a > su ? (a - su + cpt - 1) / cpt : 0, tile_b = b > su ? (b - su + cpt - 1) / cpt : 0;
         if (tile_a < tile_b) run_q4k_mfma(j, tile_a, tile_b, q4k_lds, parity);
         p = seg_end;
         ji++;
@@ -1672,11 +1733,11 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) gemv_mxfp4_mfma_kernel(Gemv
     uint32_t lo = 0, hi = L.n_jobs;
     while (lo + 1 < hi) {
         const uint32_t mid = (lo + hi) >> 1;
-        if (jobs[mid].pass_begin <= p) lo = mid; else hi = mid;
+        if ((uint32_t)__builtin_amdgcn_readfirstlane(jobs[mid].pass_begin) <= p) lo = mid; else hi = mid;
     }
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
-        GemvJob j = jobs[ji];
+        GemvJob j = uniform_job(jobs + ji);
         if (j.sel) {  // run-time expert selection: one bank of equally shaped matrices
             const uint32_t e = __builtin_amdgcn_readfirstlane(*(const GLOBAL_AS uint32_t *)j.sel);
             j.w += (size_t)e * j.w_sel_stride;
@@ -1702,11 +1763,11 @@ __global__ void __launch_bounds__(kBfMaxWaves * 64) gemv_bf16_mfma_kernel(GemvLa
     uint32_t lo = 0, hi = L.n_jobs;
     while (lo + 1 < hi) {
         const uint32_t mid = (lo + hi) >> 1;
-        if (jobs[mid].pass_begin <= p) lo = mid; else hi = mid;
+        if ((uint32_t)__builtin_amdgcn_readfirstlane(jobs[mid].pass_begin) <= p) lo = mid; else hi = mid;
     }
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
-        const GemvJob j = jobs[ji];
+        const GemvJob j = uniform_job(jobs + ji);
         const uint32_t seg_end = min(p_end, j.pass_begin + j.n_pass);
         const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin;
         const uint32_t tile_a = (a + j.cpr - 1) / j.cpr, tile_b = (b + j.cpr - 1) / j.cpr;
@@ -1727,11 +1788,11 @@ __global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_batch_kernel(GemvL
     uint32_t lo = 0, hi = L.n_jobs;
     while (lo + 1 < hi) {
         const uint32_t mid = (lo + hi) >> 1;
-        if (jobs[mid].pass_begin <= p) lo = mid; else hi = mid;
+        if ((uint32_t)__builtin_amdgcn_readfirstlane(jobs[mid].pass_begin) <= p) lo = mid; else hi = mid;
     }
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
-        const GemvJob j = jobs[ji];
+        const GemvJob j = uniform_job(jobs + ji);
         const uint32_t seg_end = min(p_end, j.pass_begin + j.n_pass);
         const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin;
         const uint32_t tile_a = (a + j.cpr - 1) / j.cpr, tile_b = (b + j.cpr - 1) / j.cpr;
@@ -1752,11 +1813,11 @@ __global__ void __launch_bounds__(kQ8MaxWaves * 64) gemv_q8_0_mfma_kernel(GemvLa
     uint32_t lo = 0, hi = L.n_jobs;
     while (lo + 1 < hi) {
         const uint32_t mid = (lo + hi) >> 1;
-        if (jobs[mid].pass_begin <= p) lo = mid; else hi = mid;
+        if ((uint32_t)__builtin_amdgcn_readfirstlane(jobs[mid].pass_begin) <= p) lo = mid; else hi = mid;
     }
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
-        const GemvJob j = jobs[ji];
+        const GemvJob j = uniform_job(jobs + ji);
         const uint32_t seg_end = min(p_end, j.pass_begin + j.n_pass);
         const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin;
         const uint32_t tile_a = (a + j.cpr - 1) / j.cpr, tile_b = (b + j.cpr - 1) / j.cpr;
@@ -1896,8 +1957,17 @@ bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
         j.rpp = nw;  // wavefronts that work on this job
         j.row_bytes = cpr * 144;
         const uint64_t tiles = (j.rows + 15) / 16;
-        if (tiles * cpr > 0x7FFFFFFFull) return false;
-        j.n_pass = (uint32_t)(tiles * cpr);  // cost units: one per tile and super-block column
+        // Cost model of the share-out, in sixteenths of the time a wavefront takes for one wave-tile (measured
+        // per workgroup and job segment on a mixed 238-job launch): a tile costs one wave-tile time per column
+        // pass whatever the number of columns (narrow rows leave wavefronts idle, they do not finish sooner),
+        // multi-pass tiles come ~19 % dearer per pass, and every job start costs a pipeline refill and the
+        // activation set-up (~4 us, ~10 us with several columns per wavefront).
+        const uint64_t np = (cpr + nw - 1) / nw;
+        const uint64_t cpt = np == 1 ? 16 : np * 19, startup = np == 1 ? 72 : 180;
+        j.pad = (int32_t)cpt;
+        j.pad2 = (uint32_t)startup;
+        if (startup + tiles * cpt > 0x7FFFFFFFull) return false;
+        j.n_pass = (uint32_t)(startup + tiles * cpt);
         return true;
     }
     const uint32_t ce = chunk_elems(j.kind);
