@@ -15,6 +15,7 @@
 // an operand read hit 16 distinct 16-byte slots.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "kernels.h"
 
@@ -160,18 +161,36 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 constexpr int LDM = 40;  // padded row of the 32-slot min tiles (f16 elements)
 
 // one block per token: scale, f16 terms, sub-block sums.  `x_is_bf16`: 16-bit inputs (exact in one term).
+// A thread takes 8 consecutive elements at a time (one or two 16-byte loads); four neighbouring threads hold a
+// 32-element sub-block.
 __global__ void __launch_bounds__(256) q4k_gemm_prep_kernel(const void *__restrict__ x, int x_is_bf16, uint32_t hidden,
                                                             uint16_t *__restrict__ xh, uint16_t *__restrict__ xl,
                                                             uint16_t *__restrict__ sx, float *__restrict__ tok_scale,
                                                             int *__restrict__ any_lo) {
     __shared__ float red[4];
-    const uint32_t tok = blockIdx.x, t = threadIdx.x;
-    const uint16_t *xb = (const uint16_t *)x + (size_t)tok * hidden;
-    const float *xf = (const float *)x + (size_t)tok * hidden;
+    const uint32_t tok = blockIdx.x, t = threadIdx.x, nvec = hidden >> 3;  // hidden % 256 == 0
+    const u32x4 *xb = reinterpret_cast<const u32x4 *>((const uint16_t *)x + (size_t)tok * hidden);
+    const f32x4 *xf = reinterpret_cast<const f32x4 *>((const float *)x + (size_t)tok * hidden);
+    auto load8 = [&](uint32_t v, float (&o)[8]) {
+        if (x_is_bf16) {
+            const u32x4 r = xb[v];
+            const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                o[2 * i] = __builtin_bit_cast(float, w[i] << 16);
+                o[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xFFFF0000u);
+            }
+        } else {
+            const f32x4 a = xf[2 * v], b = xf[2 * v + 1];
+            o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+        }
+    };
     float mx = 0.f;
-    for (uint32_t k = t; k < hidden; k += 256) {
-        const float v = x_is_bf16 ? __builtin_bit_cast(float, (uint32_t)xb[k] << 16) : xf[k];
-        mx = fmaxf(mx, fabsf(v));
+    for (uint32_t v = t; v < nvec; v += 256) {
+        float o[8];
+        load8(v, o);
+#pragma unroll
+        for (int i = 0; i < 8; i++) mx = fmaxf(mx, fabsf(o[i]));
     }
     for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
     if ((t & 63u) == 0) red[t >> 6] = mx;
@@ -183,21 +202,33 @@ __global__ void __launch_bounds__(256) q4k_gemm_prep_kernel(const void *__restri
     const float to_h = ldexpf(1.f, 14 - ex);
     if (t == 0) tok_scale[tok] = ldexpf(1.f, ex - 14);
     int lo_seen = 0;
-    for (uint32_t k = t; k < hidden; k += 256) {  // hidden % 256 == 0: every wavefront half covers one sub-block
-        const float v = (x_is_bf16 ? __builtin_bit_cast(float, (uint32_t)xb[k] << 16) : xf[k]) * to_h;
-        const _Float16 h = (_Float16)v;
-        const _Float16 l = (_Float16)(v - (float)h);
-        xh[(size_t)tok * hidden + k] = __builtin_bit_cast(uint16_t, h);
-        if (xl) xl[(size_t)tok * hidden + k] = __builtin_bit_cast(uint16_t, l);
-        lo_seen |= (xl && (float)l != 0.f) ? 1 : 0;
-        float sm = (float)h + (xl ? (float)l : 0.f);  // the activation as the MFMAs will see it
-        for (int o = 1; o < 32; o <<= 1) sm += __shfl_xor(sm, o);
+    u32x4 *oh = reinterpret_cast<u32x4 *>(xh + (size_t)tok * hidden);
+    u32x4 *ol = xl ? reinterpret_cast<u32x4 *>(xl + (size_t)tok * hidden) : nullptr;
+    for (uint32_t v = t; v < nvec; v += 256) {  // nvec % 32 == 0: the four threads of a sub-block run together
+        float o[8];
+        load8(v, o);
+        uint32_t hw[4], lw[4];
+        float sm = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const float sv = o[i] * to_h;
+            const _Float16 h = (_Float16)sv;
+            const _Float16 l = (_Float16)(sv - (float)h);
+            const uint32_t hb = __builtin_bit_cast(uint16_t, h), lb = __builtin_bit_cast(uint16_t, l);
+            if (i & 1) { hw[i >> 1] |= hb << 16; lw[i >> 1] |= lb << 16; } else { hw[i >> 1] = hb; lw[i >> 1] = lb; }
+            lo_seen |= (ol && (float)l != 0.f) ? 1 : 0;
+            sm += (float)h + (ol ? (float)l : 0.f);  // the activation as the MFMAs will see it
+        }
+        oh[v] = (u32x4){hw[0], hw[1], hw[2], hw[3]};
+        if (ol) ol[v] = (u32x4){lw[0], lw[1], lw[2], lw[3]};
+        sm += __shfl_xor(sm, 1);
+        sm += __shfl_xor(sm, 2);
         sm *= 0.03125f;  // stored as Sx/32 so that 32 x 2^14 stays inside f16; the min operand carries the 32
-        if ((t & 31u) == 0) {
+        if ((t & 3u) == 0) {
             const _Float16 sh = (_Float16)sm;
             const _Float16 sl = (_Float16)(sm - (float)sh);
-            sx[((size_t)tok * (hidden / 32) + k / 32) * 2 + 0] = __builtin_bit_cast(uint16_t, sh);
-            sx[((size_t)tok * (hidden / 32) + k / 32) * 2 + 1] = __builtin_bit_cast(uint16_t, sl);
+            const uint32_t pair = (uint32_t)__builtin_bit_cast(uint16_t, sh) | ((uint32_t)__builtin_bit_cast(uint16_t, sl) << 16);
+            reinterpret_cast<uint32_t *>(sx)[(size_t)tok * (hidden / 32) + (v >> 2)] = pair;
         }
     }
     if (lo_seen && any_lo) *any_lo = 1;
@@ -365,6 +396,289 @@ __global__ void __launch_bounds__(256) q4k_gemm_reduce_kernel(const float *__res
     out[i] = accumulate ? out[i] + s : s;
 }
 
+// ---------------------------------------------------------------------------
+// The same arithmetic, software-pipelined (the kernel in use).
+//
+// One workgroup of 8 wavefronts per CU owns a 256-row x 128-token tile; every wavefront keeps a 64x64
+// quadrant.  Everything a step needs from global memory was copied global -> LDS (global_load_lds, 16 bytes
+// per lane, no registers involved) two steps before:
+//   * the f16 activations of a step, into a ring of three stages.  Rows are 128 bytes (64 f16) without
+//     padding; the 16-byte chunk c of row r is kept at position c ^ (r & 7), chosen on the global side of the
+//     copy, so that the eight lanes of an operand read phase hit eight different bank groups;
+//   * the raw weight bytes of a step (32 per row), into a ring of three stages; each step the bytes of the
+//     next one are converted to f16(sc6*q) and written to the other of two A stages (same swizzle);
+//   * per super-block the 16-byte headers and the Sx of the tile's tokens; sum mn6*Sx is taken at the
+//     super-block's first step, d*D is folded in at its last.
+// One barrier per step.  No load returns into a register, so the compiler places no waits of its own (it
+// would wait for *all* outstanding loads as soon as register loads and LDS copies are in flight together);
+// outstanding copies are counted by hand: at the end of a step only that step's requests may still fly.
+// ---------------------------------------------------------------------------
+constexpr int PM = 256, PN = 128, PTHREADS = 512;
+constexpr int P_A_STAGE = PM * 128, P_B_STAGE = PN * 128, P_R_STAGE = PM * 32;  // bytes per stage
+constexpr int P_A_OFF = 0, P_B_OFF = 2 * P_A_STAGE, P_R_OFF = P_B_OFF + 3 * P_B_STAGE, P_H_OFF = P_R_OFF + 3 * P_R_STAGE,
+              P_AM_OFF = P_H_OFF + PM * 16, P_BM_OFF = P_AM_OFF + PM * 32, P_D_OFF = P_BM_OFF + PN * 32,
+              P_DMIN_OFF = P_D_OFF + 2 * PM * 4, P_LDS_BYTES = P_DMIN_OFF + 2 * PM * 4;
+static_assert(P_LDS_BYTES <= 160 * 1024, "one workgroup per CU");
+typedef __attribute__((address_space(3))) void *p_lds_vp;
+typedef const __attribute__((address_space(1))) void *p_g_vp;
+#define GEMM_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
+
+// 32 weights of sub-block s = 2g + half of a row as f16(sc6*q): exact (sc6*q <= 945)
+__device__ __forceinline__ void q4k_gemm_convert(const u32x4 &q0, const u32x4 &q1, uint32_t hdr_y, uint32_t hdr_w, uint32_t g, uint32_t half,
+                                                 uint32_t (&aw)[16]) {
+    const uint32_t s = 2 * g + half, sh = 8u * (s & 3u);
+    const uint32_t pa = (hdr_y >> sh) & 0xFFu, pc = (hdr_w >> sh) & 0xFFu;
+    const uint32_t sc6 = s < 4 ? (pa & 63u) : ((pc & 0x0Fu) | ((pa >> 6) << 4));
+    const _Float16 scf = (_Float16)(float)sc6;
+    const f16x2 sc2 = {scf, scf};
+    const f16x2 off2 = {(_Float16)(-1024.0f * (float)sc6), (_Float16)(-1024.0f * (float)sc6)};
+    const uint32_t qd[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const uint32_t v = half ? (qd[i] >> 4) : qd[i];
+        const uint32_t p01 = __builtin_amdgcn_perm(0u, v, 0x0C010C00u), p23 = __builtin_amdgcn_perm(0u, v, 0x0C030C02u);
+        const f16x2 m01 = __builtin_bit_cast(f16x2, (p01 & 0x000F000Fu) | 0x64006400u);  // 1024 + q
+        const f16x2 m23 = __builtin_bit_cast(f16x2, (p23 & 0x000F000Fu) | 0x64006400u);
+        aw[2 * i] = __builtin_bit_cast(uint32_t, m01 * sc2 + off2);  // (1024+q)*sc6 - 1024*sc6, one rounding: exact
+        aw[2 * i + 1] = __builtin_bit_cast(uint32_t, m23 * sc2 + off2);
+    }
+}
+
+__global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_t *w, const uint16_t *xh, const uint16_t *sx,
+                                                                    const float *__restrict__ tok_scale, float *__restrict__ out,
+                                                                    uint32_t rows, uint32_t hidden, uint32_t seq, int with_mins,
+                                                                    int accumulate, uint32_t sb_per_split, float *__restrict__ partial) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t plds[];
+    const uint32_t t = threadIdx.x, lane = t & 63u, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const uint32_t row0 = blockIdx.x * PM, tok0 = blockIdx.y * PN;
+    const uint32_t nsb = hidden >> 8, row_bytes = nsb * 144;
+    const uint32_t sb_begin = blockIdx.z * sb_per_split, sb_end = min(nsb, sb_begin + sb_per_split);
+    if (sb_begin >= sb_end) return;
+    const uint32_t nsteps = (sb_end - sb_begin) * 4;
+
+    // staging role: thread -> (tile row, half of the 64-wide k step)
+    const uint32_t sr = t >> 1, half = t & 1u;
+    // copy roles.  Raw weights: thread -> (row t/2, 16-byte half t&1) of a step, i.e. wavefront w brings rows 32w .. 32w+31.
+    const uint8_t *wt = w + (size_t)row0 * row_bytes;                                          // uniform
+    const uint32_t r_off = (min(row0 + sr, rows - 1) - row0) * row_bytes + half * 16;
+    // headers: wavefronts w and w+4 both bring rows 64*(w&3) .. +63
+    const uint32_t h_off = (min(row0 + (wave & 3u) * 64 + lane, rows - 1) - row0) * row_bytes;
+    // activations: wavefront -> tokens 16w .. 16w+15 (two copies of 8 tokens x 128 bytes), lane -> (token, chunk)
+    const uint8_t *xt = (const uint8_t *)xh + (size_t)tok0 * hidden * 2;                       // uniform
+    uint32_t b_off[2];
+#pragma unroll
+    for (int q = 0; q < 2; q++) {
+        const uint32_t r = (wave * 2 + q) * 8 + (lane >> 3);
+        b_off[q] = (min(tok0 + r, seq - 1) - tok0) * hidden * 2 + (((lane & 7u) ^ (lane >> 3)) * 16);
+    }
+    // Sx: wavefronts w and w+4 both bring tokens 32*(w&3) .. +31 (two 16-byte halves each)
+    const uint8_t *st = (const uint8_t *)sx + (size_t)tok0 * (hidden / 32) * 4;                // uniform
+    const uint32_t m_off = (min(tok0 + (wave & 3u) * 32 + (lane >> 1), seq - 1) - tok0) * (hidden / 32) * 4 + (lane & 1u) * 16;
+
+    // compute role
+    const uint32_t wm = (wave >> 1) * 64, wn = (wave & 1u) * 64;
+    const uint32_t l16 = lane & 15u, kg = lane >> 4, sw = l16 & 7u;
+
+    // (requests past the end are clamped: same number of copies in flight, results unused)
+    auto issue_raw = [&](uint32_t s) {
+        const uint32_t sc = min(s, nsteps - 1);
+        const uint8_t *src = wt + ((size_t)(sb_begin + (sc >> 2)) * 144 + 16 + 32 * (sc & 3u));
+        __builtin_amdgcn_global_load_lds((p_g_vp)(src + r_off), (p_lds_vp)(plds + P_R_OFF + (s % 3u) * P_R_STAGE + wave * 1024), 16, 0, 0);
+    };
+    auto issue_b = [&](uint32_t s) {
+        const uint32_t sc = min(s, nsteps - 1);
+        const uint8_t *src = xt + ((size_t)sb_begin * 256 + (size_t)sc * 64) * 2;
+        uint8_t *dst = plds + P_B_OFF + (s % 3u) * P_B_STAGE + wave * 2048;
+        __builtin_amdgcn_global_load_lds((p_g_vp)(src + b_off[0]), (p_lds_vp)dst, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((p_g_vp)(src + b_off[1]), (p_lds_vp)(dst + 1024), 16, 0, 0);
+    };
+    auto issue_sb = [&](uint32_t sb) {  // header and Sx of a super-block
+        const uint32_t sbc = min(sb, sb_end - 1);
+        __builtin_amdgcn_global_load_lds((p_g_vp)((wt + (size_t)sbc * 144) + h_off), (p_lds_vp)(plds + P_H_OFF + (wave & 3u) * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((p_g_vp)((st + (size_t)sbc * 32) + m_off), (p_lds_vp)(plds + P_BM_OFF + (wave & 3u) * 1024), 16, 0, 0);
+    };
+    uint32_t hdr_y = 0, hdr_w = 0;  // the scale words of the super-block being staged
+    auto stage_a = [&](uint32_t s, uint32_t g) {  // step s (k group g of its super-block): raw bytes -> f16(sc6*q)
+        const u32x4 *rp = reinterpret_cast<const u32x4 *>(plds + P_R_OFF + (s % 3u) * P_R_STAGE + sr * 32);
+        const u32x4 q0 = rp[0], q1 = rp[1];
+        uint32_t aw[16];
+        q4k_gemm_convert(q0, q1, hdr_y, hdr_w, g, half, aw);
+        uint8_t *base = plds + P_A_OFF + (s & 1u) * P_A_STAGE + sr * 128;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            *reinterpret_cast<u32x4 *>(base + (((half * 4 + i) ^ (sr & 7u)) << 4)) = (u32x4){aw[4 * i], aw[4 * i + 1], aw[4 * i + 2], aw[4 * i + 3]};
+    };
+    auto stage_sb = [&](uint32_t par) {  // a super-block's header: scale words to registers, mn6 / d / dmin to LDS
+        const u32x4 hdr = *reinterpret_cast<const u32x4 *>(plds + P_H_OFF + sr * 16);
+        hdr_y = hdr.y; hdr_w = hdr.w;
+        if (with_mins) {
+            uint32_t mnw[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {  // this thread's half of the super-block: sub-blocks 4*half .. +3 -> slots 8*half .. +7
+                const uint32_t ss = 4 * half + u, shm = 8u * (ss & 3u);
+                const uint32_t qb = (hdr.z >> shm) & 0xFFu, qc = (hdr.w >> shm) & 0xFFu;
+                const uint32_t mn6 = ss < 4 ? (qb & 63u) : ((qc >> 4) | ((qb >> 6) << 4));
+                const uint32_t hb = __builtin_bit_cast(uint16_t, (_Float16)(float)(mn6 * 32u));  // <= 2016: exact; Sx is stored /32
+                mnw[u] = hb | (hb << 16);
+            }
+            *reinterpret_cast<u32x4 *>(plds + P_AM_OFF + sr * 32 + half * 16) = (u32x4){mnw[0], mnw[1], mnw[2], mnw[3]};
+        }
+        if (half == 0) {
+            reinterpret_cast<float *>(plds + P_D_OFF)[par * PM + sr] = half_to_float(hdr.x & 0xFFFFu);
+            reinterpret_cast<float *>(plds + P_DMIN_OFF)[par * PM + sr] = half_to_float(hdr.x >> 16);
+        }
+    };
+
+    f32x4 acc[4][4], D[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) { acc[i][jj] = (f32x4){0.f, 0.f, 0.f, 0.f}; D[i][jj] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
+
+    // ---- prologue: first super-block's header and Sx, raw steps 0..2, activation steps 0..1; step 0 staged ----
+    issue_sb(sb_begin);
+    issue_raw(0); issue_raw(1); issue_raw(2);
+    issue_b(0); issue_b(1);
+    GEMM_WAIT_VMCNT(0);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    stage_sb(0);
+    stage_a(0, 0);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+
+    uint32_t s = 0;
+    for (uint32_t sb = sb_begin; sb < sb_end; sb++) {
+        const uint32_t par = (sb - sb_begin) & 1u;
+#pragma unroll
+        for (int g = 0; g < 4; g++, s++) {
+            // ---- requests: raw weights of step s+3, activations of step s+2, (next super-block's header and Sx) ----
+            issue_raw(s + 3);
+            issue_b(s + 2);
+            if (g == 1) issue_sb(sb + 1);
+            // ---- stage step s+1 and run step s on the matrix cores, interleaved ----
+            const uint8_t *A = plds + P_A_OFF + (s & 1u) * P_A_STAGE, *B = plds + P_B_OFF + (s % 3u) * P_B_STAGE;
+            if (g == 0 && with_mins) {
+                // offsets of the super-block: sum_sub mn6 * Sx (A slots 2*sub+h = 32*mn6, B slots = Sx_h/32; slots 16..31 are zero)
+                const uint32_t kgc = min(kg, 1u);
+                f16x8 amf[4], bmf[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    u32x4 av = *reinterpret_cast<const u32x4 *>(plds + P_AM_OFF + (wm + i * 16 + l16) * 32 + kgc * 16);
+                    u32x4 bv = *reinterpret_cast<const u32x4 *>(plds + P_BM_OFF + (wn + i * 16 + l16) * 32 + kgc * 16);
+                    if (kg >= 2) { av = (u32x4){0u, 0u, 0u, 0u}; bv = (u32x4){0u, 0u, 0u, 0u}; }
+                    amf[i] = __builtin_bit_cast(f16x8, av);
+                    bmf[i] = __builtin_bit_cast(f16x8, bv);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const f32x4 mv = *reinterpret_cast<const f32x4 *>(plds + P_DMIN_OFF + (par * PM + wm + i * 16 + kg * 4) * 4);
+#pragma unroll
+                    for (int jj = 0; jj < 4; jj++) {
+                        const f32x4 Dm = __builtin_amdgcn_mfma_f32_16x16x32_f16(amf[i], bmf[jj], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) acc[i][jj][e] = __builtin_fmaf(-mv[e], Dm[e], acc[i][jj][e]);
+                    }
+                }
+            }
+            if (g == 3) stage_sb(par ^ 1u);
+            __builtin_amdgcn_sched_barrier(0);
+            // Operand fragments: the A side of a 32-wide k half stays (4 registers x 4 tiles), the B side streams one
+            // 16-token tile ahead of the MFMAs that use it.  The conversion of step s+1 runs in the MFMAs' shadow.
+            auto a_frag = [&](int kk, int i) {
+                return *reinterpret_cast<const f16x8 *>(A + (wm + i * 16 + l16) * 128 + ((((uint32_t)kk * 4 + kg) ^ sw) << 4));
+            };
+            auto b_frag = [&](int kk, int jj) {
+                return *reinterpret_cast<const f16x8 *>(B + (wn + jj * 16 + l16) * 128 + ((((uint32_t)kk * 4 + kg) ^ sw) << 4));
+            };
+            // raw bytes of step s+1 and their scale
+            const u32x4 *rp = reinterpret_cast<const u32x4 *>(plds + P_R_OFF + ((s + 1) % 3u) * P_R_STAGE + sr * 32);
+            const u32x4 q0 = rp[0], q1 = rp[1];
+            const uint32_t qd[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+            const uint32_t cs = 2 * ((g + 1) & 3) + half, csh = 8u * (cs & 3u);
+            const uint32_t pa = (hdr_y >> csh) & 0xFFu, pc = (hdr_w >> csh) & 0xFFu;
+            const uint32_t sc6 = cs < 4 ? (pa & 63u) : ((pc & 0x0Fu) | ((pa >> 6) << 4));
+            const _Float16 scf = (_Float16)(float)sc6;
+            const f16x2 sc2 = {scf, scf};
+            const f16x2 off2 = {(_Float16)(-1024.0f * (float)sc6), (_Float16)(-1024.0f * (float)sc6)};
+            uint8_t *abase = plds + P_A_OFF + ((s + 1) & 1u) * P_A_STAGE + sr * 128;
+            f16x8 af[2][4], bf[2];
+#pragma unroll
+            for (int i = 0; i < 4; i++) af[0][i] = a_frag(0, i);
+            bf[0] = b_frag(0, 0);
+            uint32_t aw[16];
+            __builtin_amdgcn_sched_barrier(0);
+            // eight groups of four MFMAs; each carries one eighth of the conversion (4 weights -> two dwords of
+            // f16(sc6*q)) and the next operand reads in its shadow
+#pragma unroll
+            for (int n = 0; n < 8; n++) {
+                const int kk = n >> 2, jj = n & 3;
+                if (n + 1 < 8) bf[(n + 1) & 1] = b_frag((n + 1) >> 2, (n + 1) & 3);
+                if (kk == 0) af[1][jj] = a_frag(1, jj);
+                {
+                    const uint32_t v = qd[n] >> (half * 4u);  // low or high nibbles (the mask below drops the rest)
+                    // bytes 0,1 -> 16-bit lanes of one dword, bytes 2,3 -> the next (k order kept)
+                    const uint32_t p01 = __builtin_amdgcn_perm(0u, v, 0x0C010C00u), p23 = __builtin_amdgcn_perm(0u, v, 0x0C030C02u);
+                    const f16x2 m01 = __builtin_bit_cast(f16x2, (p01 & 0x000F000Fu) | 0x64006400u);  // 1024 + q
+                    const f16x2 m23 = __builtin_bit_cast(f16x2, (p23 & 0x000F000Fu) | 0x64006400u);
+                    aw[2 * n] = __builtin_bit_cast(uint32_t, m01 * sc2 + off2);  // (1024+q)*sc6 - 1024*sc6, one rounding: exact
+                    aw[2 * n + 1] = __builtin_bit_cast(uint32_t, m23 * sc2 + off2);
+                }
+                if (n & 1) {
+                    const int c = n >> 1;
+                    *reinterpret_cast<u32x4 *>(abase + (((half * 4 + c) ^ (sr & 7u)) << 4)) = (u32x4){aw[4 * c], aw[4 * c + 1], aw[4 * c + 2], aw[4 * c + 3]};
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++) D[i][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[kk][i], bf[n & 1], D[i][jj], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (g == 3) {
+                // ---- end of the super-block: acc += d * D ----
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const f32x4 dv = *reinterpret_cast<const f32x4 *>(plds + P_D_OFF + (par * PM + wm + i * 16 + kg * 4) * 4);
+#pragma unroll
+                    for (int jj = 0; jj < 4; jj++) {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) acc[i][jj][e] = __builtin_fmaf(dv[e], D[i][jj][e], acc[i][jj][e]);
+                        D[i][jj] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                    }
+                }
+            }
+            // ---- end of step: only this step's copies (3, or 5 with the super-block's) may still fly ----
+            asm volatile("" ::: "memory");
+            if (g == 1) GEMM_WAIT_VMCNT(5);
+            else GEMM_WAIT_VMCNT(3);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        }
+    }
+    GEMM_WAIT_VMCNT(0);  // the clamped requests past the end
+
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            const uint32_t tok = tok0 + wn + jj * 16 + l16;
+            const uint32_t r = row0 + wm + i * 16 + kg * 4;
+            if (tok >= seq) continue;
+            if (partial) {  // unscaled partial sums of this K-range; q4k_gemm_reduce_kernel adds the slabs in order
+                float *o = partial + ((size_t)blockIdx.z * seq + tok) * rows + r;
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (r + e < rows) o[e] = acc[i][jj][e];
+                continue;
+            }
+            const float ts = tok_scale[tok];
+            float *o = out + (size_t)tok * rows + r;
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (r + e < rows) o[e] = accumulate ? o[e] + acc[i][jj][e] * ts : acc[i][jj][e] * ts;
+        }
+}
+
 // f32 activations -> bf16 hi (round to nearest even) and the bf16 of the remainder
 __global__ void split_bf16_kernel(const float *__restrict__ x, size_t n, uint16_t *__restrict__ hi, uint16_t *__restrict__ lo,
                                   int *__restrict__ any_lo) {
@@ -393,11 +707,21 @@ hipError_t q4k_gemm_prep_launch(hipStream_t s, const void *x, int x_is_bf16, uin
     return hipGetLastError();
 }
 
-// K-ranges per output tile so that a launch has roughly two workgroups per CU (1 = no split)
+static bool gemm_pipe_enabled() {
+    static const bool on = !(getenv("LARQL_HIP_GEMM_PIPE") && atoi(getenv("LARQL_HIP_GEMM_PIPE")) == 0);
+    return on;
+}
+
+// K-ranges per output tile so that a launch fills the CUs (1 = no split)
 uint32_t q4k_gemm_splits(uint32_t rows, uint32_t hidden, uint32_t seq, uint32_t cu_count) {
-    const uint64_t tiles = (uint64_t)((rows + TM - 1) / TM) * ((seq + TN - 1) / TN);
     const uint32_t nsb = hidden / 256;
     uint32_t s = 1;
+    if (gemm_pipe_enabled()) {  // one 256x128 workgroup per CU
+        const uint64_t tiles = (uint64_t)((rows + PM - 1) / PM) * ((seq + PN - 1) / PN);
+        while (s < 8 && tiles * s * 2 <= (uint64_t)cu_count && nsb / (s * 2) >= 4) s *= 2;
+        return s;
+    }
+    const uint64_t tiles = (uint64_t)((rows + TM - 1) / TM) * ((seq + TN - 1) / TN);
     while (s < 8 && tiles * s < (uint64_t)cu_count * 3 / 2 && nsb / (s * 2) >= 4) s *= 2;
     return s;
 }
@@ -406,16 +730,25 @@ hipError_t q4k_gemm_f16_launch(hipStream_t s, const uint8_t *w, const uint16_t *
                                uint32_t rows, uint32_t hidden, uint32_t seq, int with_mins, int accumulate, uint32_t splits, float *partial) {
     if (rows == 0 || seq == 0) return hipSuccess;
     const uint32_t nsb = hidden / 256;
-    if (splits <= 1 || !partial) {
-        hipLaunchKernelGGL(q4k_gemm_f16_kernel, dim3((rows + TM - 1) / TM, (seq + TN - 1) / TN, 1), dim3(256), 0, s, w, xh, sx, tok_scale, out,
-                           rows, hidden, seq, with_mins, accumulate, nsb, (float *)nullptr);
-        return hipGetLastError();
+    const bool split = splits > 1 && partial;
+    const uint32_t per = split ? (nsb + splits - 1) / splits : nsb, z = split ? (nsb + per - 1) / per : 1;
+    if (gemm_pipe_enabled()) {
+        static bool attr_set = false;  // dynamic LDS above 64 KB has to be allowed once per process
+        if (!attr_set) {
+            hipError_t e = hipFuncSetAttribute((const void *)q4k_gemm_pipe_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return e;
+            attr_set = true;
+        }
+        hipLaunchKernelGGL(q4k_gemm_pipe_kernel, dim3((rows + PM - 1) / PM, (seq + PN - 1) / PN, z), dim3(PTHREADS), P_LDS_BYTES, s, w, xh, sx,
+                           tok_scale, out, rows, hidden, seq, with_mins, accumulate, per, split ? partial : (float *)nullptr);
+    } else {
+        hipLaunchKernelGGL(q4k_gemm_f16_kernel, dim3((rows + TM - 1) / TM, (seq + TN - 1) / TN, z), dim3(256), 0, s, w, xh, sx, tok_scale, out,
+                           rows, hidden, seq, with_mins, accumulate, per, split ? partial : (float *)nullptr);
     }
-    const uint32_t per = (nsb + splits - 1) / splits, z = (nsb + per - 1) / per;
-    hipLaunchKernelGGL(q4k_gemm_f16_kernel, dim3((rows + TM - 1) / TM, (seq + TN - 1) / TN, z), dim3(256), 0, s, w, xh, sx, tok_scale, out,
-                       rows, hidden, seq, with_mins, accumulate, per, partial);
-    const size_t n = (size_t)rows * seq;
-    hipLaunchKernelGGL(q4k_gemm_reduce_kernel, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, s, partial, z, tok_scale, out, rows, seq, accumulate);
+    if (split) {
+        const size_t n = (size_t)rows * seq;
+        hipLaunchKernelGGL(q4k_gemm_reduce_kernel, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, s, partial, z, tok_scale, out, rows, seq, accumulate);
+    }
     return hipGetLastError();
 }
 
