@@ -400,22 +400,26 @@ __global__ void __launch_bounds__(256) q4k_gemm_reduce_kernel(const float *__res
 // The same arithmetic, software-pipelined (the kernel in use).
 //
 // One workgroup of 8 wavefronts per CU owns a 256-row x 128-token tile; every wavefront keeps a 64x64
-// quadrant.  Everything a step needs from global memory was copied global -> LDS (global_load_lds, 16 bytes
-// per lane, no registers involved) two steps before:
-//   * the f16 activations of a step, into a ring of three stages.  Rows are 128 bytes (64 f16) without
+// quadrant.  Everything a step (64 k) needs from global memory was copied global -> LDS (global_load_lds,
+// 16 bytes per lane, no registers involved) at least two steps before:
+//   * the f16 activations of a step, into a ring of four stages.  Rows are 128 bytes (64 f16) without
 //     padding; the 16-byte chunk c of row r is kept at position c ^ (r & 7), chosen on the global side of the
 //     copy, so that the eight lanes of an operand read phase hit eight different bank groups;
-//   * the raw weight bytes of a step (32 per row), into a ring of three stages; each step the bytes of the
-//     next one are converted to f16(sc6*q) and written to the other of two A stages (same swizzle);
+//   * the raw weight bytes of a step (32 per row), into a ring of five stages;
 //   * per super-block the 16-byte headers and the Sx of the tile's tokens; sum mn6*Sx is taken at the
 //     super-block's first step, d*D is folded in at its last.
-// One barrier per step.  No load returns into a register, so the compiler places no waits of its own (it
-// would wait for *all* outstanding loads as soon as register loads and LDS copies are in flight together);
-// outstanding copies are counted by hand: at the end of a step only that step's requests may still fly.
+// The f16(sc6*q) operand exists once (256 rows x 64 k, chunk c of row r at c ^ swz(r), swz a bit permutation
+// that also spreads the converting threads over the banks).  A step has two halves with a barrier after each:
+// while the matrix cores work on k 0..31 the threads convert this step's k 32..63 (high nibbles) into the
+// other half of the operand, and while they work on k 32..63 the next step's k 0..31 (low nibbles) replace the
+// half just used.  No load returns into a register, so the compiler places no waits of its own (it would wait
+// for *all* outstanding loads as soon as register loads and LDS copies are in flight together); outstanding
+// copies are counted by hand: at the end of a step only the requests of the last two steps may still fly.
 // ---------------------------------------------------------------------------
 constexpr int PM = 256, PN = 128, PTHREADS = 512;
-constexpr int P_A_STAGE = PM * 128, P_B_STAGE = PN * 128, P_R_STAGE = PM * 32;  // bytes per stage
-constexpr int P_A_OFF = 0, P_B_OFF = 2 * P_A_STAGE, P_R_OFF = P_B_OFF + 3 * P_B_STAGE, P_H_OFF = P_R_OFF + 3 * P_R_STAGE,
+constexpr int P_NB = 4, P_NR = 5;                                               // ring depths: activations, raw weights
+constexpr int P_A_BYTES = PM * 128, P_B_STAGE = PN * 128, P_R_STAGE = PM * 32;  // bytes
+constexpr int P_A_OFF = 0, P_B_OFF = P_A_BYTES, P_R_OFF = P_B_OFF + P_NB * P_B_STAGE, P_H_OFF = P_R_OFF + P_NR * P_R_STAGE,
               P_AM_OFF = P_H_OFF + PM * 16, P_BM_OFF = P_AM_OFF + PM * 32, P_D_OFF = P_BM_OFF + PN * 32,
               P_DMIN_OFF = P_D_OFF + 2 * PM * 4, P_LDS_BYTES = P_DMIN_OFF + 2 * PM * 4;
 static_assert(P_LDS_BYTES <= 160 * 1024, "one workgroup per CU");
@@ -423,26 +427,9 @@ typedef __attribute__((address_space(3))) void *p_lds_vp;
 typedef const __attribute__((address_space(1))) void *p_g_vp;
 #define GEMM_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
 
-// 32 weights of sub-block s = 2g + half of a row as f16(sc6*q): exact (sc6*q <= 945)
-__device__ __forceinline__ void q4k_gemm_convert(const u32x4 &q0, const u32x4 &q1, uint32_t hdr_y, uint32_t hdr_w, uint32_t g, uint32_t half,
-                                                 uint32_t (&aw)[16]) {
-    const uint32_t s = 2 * g + half, sh = 8u * (s & 3u);
-    const uint32_t pa = (hdr_y >> sh) & 0xFFu, pc = (hdr_w >> sh) & 0xFFu;
-    const uint32_t sc6 = s < 4 ? (pa & 63u) : ((pc & 0x0Fu) | ((pa >> 6) << 4));
-    const _Float16 scf = (_Float16)(float)sc6;
-    const f16x2 sc2 = {scf, scf};
-    const f16x2 off2 = {(_Float16)(-1024.0f * (float)sc6), (_Float16)(-1024.0f * (float)sc6)};
-    const uint32_t qd[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const uint32_t v = half ? (qd[i] >> 4) : qd[i];
-        const uint32_t p01 = __builtin_amdgcn_perm(0u, v, 0x0C010C00u), p23 = __builtin_amdgcn_perm(0u, v, 0x0C030C02u);
-        const f16x2 m01 = __builtin_bit_cast(f16x2, (p01 & 0x000F000Fu) | 0x64006400u);  // 1024 + q
-        const f16x2 m23 = __builtin_bit_cast(f16x2, (p23 & 0x000F000Fu) | 0x64006400u);
-        aw[2 * i] = __builtin_bit_cast(uint32_t, m01 * sc2 + off2);  // (1024+q)*sc6 - 1024*sc6, one rounding: exact
-        aw[2 * i + 1] = __builtin_bit_cast(uint32_t, m23 * sc2 + off2);
-    }
-}
+// position swizzle of the weight operand: bit 0 of the row picks the half of the row's eight chunk positions,
+// bits 1..2 the position inside it (a bijection of r & 7, so 8 consecutive rows still hit 8 bank groups)
+__device__ __forceinline__ uint32_t q4k_gemm_swz(uint32_t r) { return ((r & 1u) << 2) | ((r >> 1) & 3u); }
 
 __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_t *w, const uint16_t *xh, const uint16_t *sx,
                                                                     const float *__restrict__ tok_scale, float *__restrict__ out,
@@ -456,11 +443,11 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
     if (sb_begin >= sb_end) return;
     const uint32_t nsteps = (sb_end - sb_begin) * 4;
 
-    // staging role: thread -> (tile row, half of the 64-wide k step)
-    const uint32_t sr = t >> 1, half = t & 1u;
-    // copy roles.  Raw weights: thread -> (row t/2, 16-byte half t&1) of a step, i.e. wavefront w brings rows 32w .. 32w+31.
+    // conversion role: thread -> (tile row, 16-byte part of the row's 32 raw bytes = 16 k of a 32-wide half)
+    const uint32_t sr = t >> 1, part = t & 1u;
+    // copy roles.  Raw weights: thread -> (row t/2, part t&1) of a step, i.e. wavefront w brings rows 32w .. 32w+31.
     const uint8_t *wt = w + (size_t)row0 * row_bytes;                                          // uniform
-    const uint32_t r_off = (min(row0 + sr, rows - 1) - row0) * row_bytes + half * 16;
+    const uint32_t r_off = (min(row0 + sr, rows - 1) - row0) * row_bytes + part * 16;
     // headers: wavefronts w and w+4 both bring rows 64*(w&3) .. +63
     const uint32_t h_off = (min(row0 + (wave & 3u) * 64 + lane, rows - 1) - row0) * row_bytes;
     // activations: wavefront -> tokens 16w .. 16w+15 (two copies of 8 tokens x 128 bytes), lane -> (token, chunk)
@@ -477,18 +464,18 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
 
     // compute role
     const uint32_t wm = (wave >> 1) * 64, wn = (wave & 1u) * 64;
-    const uint32_t l16 = lane & 15u, kg = lane >> 4, sw = l16 & 7u;
+    const uint32_t l16 = lane & 15u, kg = lane >> 4, sw_a = q4k_gemm_swz(l16), sw_b = l16 & 7u;
 
     // (requests past the end are clamped: same number of copies in flight, results unused)
     auto issue_raw = [&](uint32_t s) {
         const uint32_t sc = min(s, nsteps - 1);
         const uint8_t *src = wt + ((size_t)(sb_begin + (sc >> 2)) * 144 + 16 + 32 * (sc & 3u));
-        __builtin_amdgcn_global_load_lds((p_g_vp)(src + r_off), (p_lds_vp)(plds + P_R_OFF + (s % 3u) * P_R_STAGE + wave * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((p_g_vp)(src + r_off), (p_lds_vp)(plds + P_R_OFF + (s % P_NR) * P_R_STAGE + wave * 1024), 16, 0, 0);
     };
     auto issue_b = [&](uint32_t s) {
         const uint32_t sc = min(s, nsteps - 1);
         const uint8_t *src = xt + ((size_t)sb_begin * 256 + (size_t)sc * 64) * 2;
-        uint8_t *dst = plds + P_B_OFF + (s % 3u) * P_B_STAGE + wave * 2048;
+        uint8_t *dst = plds + P_B_OFF + (s % P_NB) * P_B_STAGE + wave * 2048;
         __builtin_amdgcn_global_load_lds((p_g_vp)(src + b_off[0]), (p_lds_vp)dst, 16, 0, 0);
         __builtin_amdgcn_global_load_lds((p_g_vp)(src + b_off[1]), (p_lds_vp)(dst + 1024), 16, 0, 0);
     };
@@ -497,36 +484,51 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
         __builtin_amdgcn_global_load_lds((p_g_vp)((wt + (size_t)sbc * 144) + h_off), (p_lds_vp)(plds + P_H_OFF + (wave & 3u) * 1024), 16, 0, 0);
         __builtin_amdgcn_global_load_lds((p_g_vp)((st + (size_t)sbc * 32) + m_off), (p_lds_vp)(plds + P_BM_OFF + (wave & 3u) * 1024), 16, 0, 0);
     };
-    uint32_t hdr_y = 0, hdr_w = 0;  // the scale words of the super-block being staged
-    auto stage_a = [&](uint32_t s, uint32_t g) {  // step s (k group g of its super-block): raw bytes -> f16(sc6*q)
-        const u32x4 *rp = reinterpret_cast<const u32x4 *>(plds + P_R_OFF + (s % 3u) * P_R_STAGE + sr * 32);
-        const u32x4 q0 = rp[0], q1 = rp[1];
-        uint32_t aw[16];
-        q4k_gemm_convert(q0, q1, hdr_y, hdr_w, g, half, aw);
-        uint8_t *base = plds + P_A_OFF + (s & 1u) * P_A_STAGE + sr * 128;
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            *reinterpret_cast<u32x4 *>(base + (((half * 4 + i) ^ (sr & 7u)) << 4)) = (u32x4){aw[4 * i], aw[4 * i + 1], aw[4 * i + 2], aw[4 * i + 3]};
-    };
+    uint32_t hdr_y = 0, hdr_w = 0;  // the scale words of the super-block being converted
     auto stage_sb = [&](uint32_t par) {  // a super-block's header: scale words to registers, mn6 / d / dmin to LDS
         const u32x4 hdr = *reinterpret_cast<const u32x4 *>(plds + P_H_OFF + sr * 16);
         hdr_y = hdr.y; hdr_w = hdr.w;
         if (with_mins) {
             uint32_t mnw[4];
 #pragma unroll
-            for (int u = 0; u < 4; u++) {  // this thread's half of the super-block: sub-blocks 4*half .. +3 -> slots 8*half .. +7
-                const uint32_t ss = 4 * half + u, shm = 8u * (ss & 3u);
+            for (int u = 0; u < 4; u++) {  // this thread's half of the super-block: sub-blocks 4*part .. +3 -> slots 8*part .. +7
+                const uint32_t ss = 4 * part + u, shm = 8u * (ss & 3u);
                 const uint32_t qb = (hdr.z >> shm) & 0xFFu, qc = (hdr.w >> shm) & 0xFFu;
                 const uint32_t mn6 = ss < 4 ? (qb & 63u) : ((qc >> 4) | ((qb >> 6) << 4));
                 const uint32_t hb = __builtin_bit_cast(uint16_t, (_Float16)(float)(mn6 * 32u));  // <= 2016: exact; Sx is stored /32
                 mnw[u] = hb | (hb << 16);
             }
-            *reinterpret_cast<u32x4 *>(plds + P_AM_OFF + sr * 32 + half * 16) = (u32x4){mnw[0], mnw[1], mnw[2], mnw[3]};
+            *reinterpret_cast<u32x4 *>(plds + P_AM_OFF + sr * 32 + part * 16) = (u32x4){mnw[0], mnw[1], mnw[2], mnw[3]};
         }
-        if (half == 0) {
+        if (part == 0) {
             reinterpret_cast<float *>(plds + P_D_OFF)[par * PM + sr] = half_to_float(hdr.x & 0xFFFFu);
             reinterpret_cast<float *>(plds + P_DMIN_OFF)[par * PM + sr] = half_to_float(hdr.x >> 16);
         }
+    };
+    // scale of sub-block `sub` (0..7) of the current header as the packed-FMA operands (sc6, -1024*sc6)
+    auto scale_of = [&](uint32_t sub, f16x2 &sc2, f16x2 &off2) {
+        const uint32_t sh = 8u * (sub & 3u);
+        const uint32_t pa = (hdr_y >> sh) & 0xFFu, pc = (hdr_w >> sh) & 0xFFu;
+        const uint32_t sc6 = sub < 4 ? (pa & 63u) : ((pc & 0x0Fu) | ((pa >> 6) << 4));
+        const _Float16 scf = (_Float16)(float)sc6, of = (_Float16)(-1024.0f * (float)sc6);
+        sc2 = (f16x2){scf, scf};
+        off2 = (f16x2){of, of};
+    };
+    // 4 raw bytes (nibble h) -> two dwords of f16(sc6*q): exact (sc6*q <= 945)
+    auto convert4 = [&](uint32_t raw, uint32_t h, f16x2 sc2, f16x2 off2, uint32_t &o0, uint32_t &o1) {
+        const uint32_t v = raw >> (h * 4u);  // low or high nibbles (the mask below drops the rest)
+        // bytes 0,1 -> 16-bit lanes of one dword, bytes 2,3 -> the next (k order kept)
+        const uint32_t p01 = __builtin_amdgcn_perm(0u, v, 0x0C010C00u), p23 = __builtin_amdgcn_perm(0u, v, 0x0C030C02u);
+        const f16x2 m01 = __builtin_bit_cast(f16x2, (p01 & 0x000F000Fu) | 0x64006400u);  // 1024 + q
+        const f16x2 m23 = __builtin_bit_cast(f16x2, (p23 & 0x000F000Fu) | 0x64006400u);
+        o0 = __builtin_bit_cast(uint32_t, m01 * sc2 + off2);  // (1024+q)*sc6 - 1024*sc6, one rounding: exact
+        o1 = __builtin_bit_cast(uint32_t, m23 * sc2 + off2);
+    };
+    // where this thread's two chunks of k-half h go
+    uint8_t *const a_row = plds + P_A_OFF + sr * 128;
+    const uint32_t a_swz = q4k_gemm_swz(sr);
+    auto a_frag = [&](int kk, int i) {
+        return *reinterpret_cast<const f16x8 *>(plds + P_A_OFF + (wm + i * 16 + l16) * 128 + ((((uint32_t)kk * 4 + kg) ^ sw_a) << 4));
     };
 
     f32x4 acc[4][4], D[4][4];
@@ -535,15 +537,25 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
 #pragma unroll
         for (int jj = 0; jj < 4; jj++) { acc[i][jj] = (f32x4){0.f, 0.f, 0.f, 0.f}; D[i][jj] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
 
-    // ---- prologue: first super-block's header and Sx, raw steps 0..2, activation steps 0..1; step 0 staged ----
+    // ---- prologue: first super-block's header and Sx, raw steps 0..3, activation steps 0..2; k 0..31 of step 0 converted ----
     issue_sb(sb_begin);
-    issue_raw(0); issue_raw(1); issue_raw(2);
-    issue_b(0); issue_b(1);
+    issue_raw(0); issue_raw(1); issue_raw(2); issue_raw(3);
+    issue_b(0); issue_b(1); issue_b(2);
     GEMM_WAIT_VMCNT(0);
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     stage_sb(0);
-    stage_a(0, 0);
+    {
+        const u32x4 q = *reinterpret_cast<const u32x4 *>(plds + P_R_OFF + sr * 32 + part * 16);
+        const uint32_t qd[4] = {q.x, q.y, q.z, q.w};
+        f16x2 sc2, off2;
+        scale_of(0, sc2, off2);
+        uint32_t aw[8];
+#pragma unroll
+        for (int n = 0; n < 4; n++) convert4(qd[n], 0, sc2, off2, aw[2 * n], aw[2 * n + 1]);
+        *reinterpret_cast<u32x4 *>(a_row + (((2 * part) ^ a_swz) << 4)) = (u32x4){aw[0], aw[1], aw[2], aw[3]};
+        *reinterpret_cast<u32x4 *>(a_row + (((2 * part + 1) ^ a_swz) << 4)) = (u32x4){aw[4], aw[5], aw[6], aw[7]};
+    }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
@@ -553,12 +565,13 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
         const uint32_t par = (sb - sb_begin) & 1u;
 #pragma unroll
         for (int g = 0; g < 4; g++, s++) {
-            // ---- requests: raw weights of step s+3, activations of step s+2, (next super-block's header and Sx) ----
-            issue_raw(s + 3);
-            issue_b(s + 2);
-            if (g == 1) issue_sb(sb + 1);
-            // ---- stage step s+1 and run step s on the matrix cores, interleaved ----
-            const uint8_t *A = plds + P_A_OFF + (s & 1u) * P_A_STAGE, *B = plds + P_B_OFF + (s % 3u) * P_B_STAGE;
+            // ---- requests: raw weights of step s+4, activations of step s+3 ----
+            issue_raw(s + 4);
+            issue_b(s + 3);
+            const uint8_t *B = plds + P_B_OFF + (s % P_NB) * P_B_STAGE;
+            auto b_frag = [&](int kk, int jj) {
+                return *reinterpret_cast<const f16x8 *>(B + (wn + jj * 16 + l16) * 128 + ((((uint32_t)kk * 4 + kg) ^ sw_b) << 4));
+            };
             if (g == 0 && with_mins) {
                 // offsets of the super-block: sum_sub mn6 * Sx (A slots 2*sub+h = 32*mn6, B slots = Sx_h/32; slots 16..31 are zero)
                 const uint32_t kgc = min(kg, 1u);
@@ -582,101 +595,104 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
                     }
                 }
             }
-            if (g == 3) stage_sb(par ^ 1u);
-            __builtin_amdgcn_sched_barrier(0);
-            // Operand fragments: the A side of a 32-wide k half stays (4 registers x 4 tiles), the B side streams one
-            // 16-token tile ahead of the MFMAs that use it.  The conversion of step s+1 runs in the MFMAs' shadow.
-            auto a_frag = [&](int kk, int i) {
-                return *reinterpret_cast<const f16x8 *>(A + (wm + i * 16 + l16) * 128 + ((((uint32_t)kk * 4 + kg) ^ sw) << 4));
-            };
-            auto b_frag = [&](int kk, int jj) {
-                return *reinterpret_cast<const f16x8 *>(B + (wn + jj * 16 + l16) * 128 + ((((uint32_t)kk * 4 + kg) ^ sw) << 4));
-            };
-            // raw bytes of step s+1 and their scale
-            const u32x4 *rp = reinterpret_cast<const u32x4 *>(plds + P_R_OFF + ((s + 1) % 3u) * P_R_STAGE + sr * 32);
-            const u32x4 q0 = rp[0], q1 = rp[1];
-            const uint32_t qd[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
-            const uint32_t cs = 2 * ((g + 1) & 3) + half, csh = 8u * (cs & 3u);
-            const uint32_t pa = (hdr_y >> csh) & 0xFFu, pc = (hdr_w >> csh) & 0xFFu;
-            const uint32_t sc6 = cs < 4 ? (pa & 63u) : ((pc & 0x0Fu) | ((pa >> 6) << 4));
-            const _Float16 scf = (_Float16)(float)sc6;
-            const f16x2 sc2 = {scf, scf};
-            const f16x2 off2 = {(_Float16)(-1024.0f * (float)sc6), (_Float16)(-1024.0f * (float)sc6)};
-            uint8_t *abase = plds + P_A_OFF + ((s + 1) & 1u) * P_A_STAGE + sr * 128;
-            f16x8 af[2][4], bf[2];
 #pragma unroll
-            for (int i = 0; i < 4; i++) af[0][i] = a_frag(0, i);
-            bf[0] = b_frag(0, 0);
-            uint32_t aw[16];
-            __builtin_amdgcn_sched_barrier(0);
-            // eight groups of four MFMAs; each carries one eighth of the conversion (4 weights -> two dwords of
-            // f16(sc6*q)) and the next operand reads in its shadow
-#pragma unroll
-            for (int n = 0; n < 8; n++) {
-                const int kk = n >> 2, jj = n & 3;
-                if (n + 1 < 8) bf[(n + 1) & 1] = b_frag((n + 1) >> 2, (n + 1) & 3);
-                if (kk == 0) af[1][jj] = a_frag(1, jj);
-                {
-                    const uint32_t v = qd[n] >> (half * 4u);  // low or high nibbles (the mask below drops the rest)
-                    // bytes 0,1 -> 16-bit lanes of one dword, bytes 2,3 -> the next (k order kept)
-                    const uint32_t p01 = __builtin_amdgcn_perm(0u, v, 0x0C010C00u), p23 = __builtin_amdgcn_perm(0u, v, 0x0C030C02u);
-                    const f16x2 m01 = __builtin_bit_cast(f16x2, (p01 & 0x000F000Fu) | 0x64006400u);  // 1024 + q
-                    const f16x2 m23 = __builtin_bit_cast(f16x2, (p23 & 0x000F000Fu) | 0x64006400u);
-                    aw[2 * n] = __builtin_bit_cast(uint32_t, m01 * sc2 + off2);  // (1024+q)*sc6 - 1024*sc6, one rounding: exact
-                    aw[2 * n + 1] = __builtin_bit_cast(uint32_t, m23 * sc2 + off2);
-                }
-                if (n & 1) {
-                    const int c = n >> 1;
-                    *reinterpret_cast<u32x4 *>(abase + (((half * 4 + c) ^ (sr & 7u)) << 4)) = (u32x4){aw[4 * c], aw[4 * c + 1], aw[4 * c + 2], aw[4 * c + 3]};
-                }
-#pragma unroll
-                for (int i = 0; i < 4; i++) D[i][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[kk][i], bf[n & 1], D[i][jj], 0, 0, 0);
+            for (int h = 0; h < 2; h++) {
+                // ---- half h: the matrix cores take k 32h .. 32h+31 of step s; the threads convert, for h = 0, this step's
+                //      k 32..63 (high nibbles of raw step s) and, for h = 1, the next step's k 0..31 (low nibbles of s+1) ----
+                if (h == 1 && g == 0) issue_sb(sb + 1);  // (everybody is past this super-block's Sx and header now)
+                if (h == 1 && g == 3) stage_sb(par ^ 1u);
                 __builtin_amdgcn_sched_barrier(0);
-            }
-            if (g == 3) {
-                // ---- end of the super-block: acc += d * D ----
+                const uint32_t rs = s + h;                                  // raw step being converted
+                const uint32_t nib = 1 - h;                                 // its nibble
+                const u32x4 q = *reinterpret_cast<const u32x4 *>(plds + P_R_OFF + (rs % P_NR) * P_R_STAGE + sr * 32 + part * 16);
+                const uint32_t qd[4] = {q.x, q.y, q.z, q.w};
+                f16x2 sc2, off2;
+                scale_of(h == 0 ? 2 * g + 1 : 2 * ((g + 1) & 3), sc2, off2);
+                const uint32_t c0 = 4 * nib + 2 * part;                     // destination chunks c0, c0+1
+                f16x8 af[4], bf[2];
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const f32x4 dv = *reinterpret_cast<const f32x4 *>(plds + P_D_OFF + (par * PM + wm + i * 16 + kg * 4) * 4);
+                for (int i = 0; i < 4; i++) af[i] = a_frag(h, i);
+                bf[0] = b_frag(h, 0);
+                uint32_t aw[8];
+                __builtin_amdgcn_sched_barrier(0);
+                // four groups of four MFMAs; each carries a quarter of the conversion and the next operand read
 #pragma unroll
-                    for (int jj = 0; jj < 4; jj++) {
+                for (int jj = 0; jj < 4; jj++) {
+                    if (jj + 1 < 4) bf[(jj + 1) & 1] = b_frag(h, jj + 1);
+                    convert4(qd[jj], nib, sc2, off2, aw[2 * jj], aw[2 * jj + 1]);
+                    if (jj & 1) {
+                        const int c = jj >> 1;
+                        *reinterpret_cast<u32x4 *>(a_row + (((c0 + c) ^ a_swz) << 4)) = (u32x4){aw[4 * c], aw[4 * c + 1], aw[4 * c + 2], aw[4 * c + 3]};
+                    }
 #pragma unroll
-                        for (int e = 0; e < 4; e++) acc[i][jj][e] = __builtin_fmaf(dv[e], D[i][jj][e], acc[i][jj][e]);
-                        D[i][jj] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                    for (int i = 0; i < 4; i++)  // (a super-block's first MFMAs start from zero: D is never cleared)
+                        D[i][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bf[jj & 1], (g == 0 && h == 0) ? (f32x4){0.f, 0.f, 0.f, 0.f} : D[i][jj], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if (h == 1 && g == 3) {
+                    // ---- end of the super-block: acc += d * D ----
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const f32x4 dv = *reinterpret_cast<const f32x4 *>(plds + P_D_OFF + (par * PM + wm + i * 16 + kg * 4) * 4);
+#pragma unroll
+                        for (int jj = 0; jj < 4; jj++) {
+#pragma unroll
+                            for (int e = 0; e < 4; e++) acc[i][jj][e] = __builtin_fmaf(dv[e], D[i][jj][e], acc[i][jj][e]);
+                        }
                     }
                 }
+                asm volatile("" ::: "memory");
+                if (h == 1) {
+                    // ---- end of step: only the copies requested in this step and the one before may still fly
+                    //      (3 per step, 5 in a super-block's first) ----
+                    if (g == 0 || g == 1) GEMM_WAIT_VMCNT(8);
+                    else GEMM_WAIT_VMCNT(6);
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
             }
-            // ---- end of step: only this step's copies (3, or 5 with the super-block's) may still fly ----
-            asm volatile("" ::: "memory");
-            if (g == 1) GEMM_WAIT_VMCNT(5);
-            else GEMM_WAIT_VMCNT(3);
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            __builtin_amdgcn_s_barrier();
-            asm volatile("" ::: "memory");
         }
     }
     GEMM_WAIT_VMCNT(0);  // the clamped requests past the end
 
+    // Results leave through LDS so that a store instruction writes whole lines: each wavefront parks its 64x64
+    // block as [token][row] (token rows padded to 68 floats: the 8 lanes of a write phase hit 8 bank groups) in
+    // its own 17 KB, then every lane stores 16 bytes of a 256-byte run of one token.
+    __builtin_amdgcn_s_barrier();  // nobody's copies are still landing in what becomes another wavefront's block
+    asm volatile("" ::: "memory");
+    constexpr uint32_t EP_LD = 68;
+    float *blk = reinterpret_cast<float *>(plds) + wave * (64 * EP_LD);
+    static_assert(8 * 64 * EP_LD * 4 <= P_LDS_BYTES, "the eight blocks fit");
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
-        for (int jj = 0; jj < 4; jj++) {
-            const uint32_t tok = tok0 + wn + jj * 16 + l16;
-            const uint32_t r = row0 + wm + i * 16 + kg * 4;
-            if (tok >= seq) continue;
-            if (partial) {  // unscaled partial sums of this K-range; q4k_gemm_reduce_kernel adds the slabs in order
-                float *o = partial + ((size_t)blockIdx.z * seq + tok) * rows + r;
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    if (r + e < rows) o[e] = acc[i][jj][e];
-                continue;
-            }
+        for (int jj = 0; jj < 4; jj++)
+            *reinterpret_cast<f32x4 *>(blk + (jj * 16 + l16) * EP_LD + i * 16 + kg * 4) = acc[i][jj];
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own writes, own reads
+    const bool vec_ok = (rows & 3u) == 0 && (((uintptr_t)(partial ? partial : out)) & 15u) == 0;
+    const uint32_t rc = (lane & 15u) * 4, r = row0 + wm + rc;
+#pragma unroll 4
+    for (int it = 0; it < 16; it++) {
+        const uint32_t tl = it * 4 + (lane >> 4), tok = tok0 + wn + tl;
+        if (tok >= seq) continue;
+        f32x4 v = *reinterpret_cast<const f32x4 *>(blk + tl * EP_LD + rc);
+        float *o = partial ? partial + ((size_t)blockIdx.z * seq + tok) * rows + r : out + (size_t)tok * rows + r;
+        if (!partial) {  // (partial sums stay unscaled; q4k_gemm_reduce_kernel adds the slabs in order and scales)
             const float ts = tok_scale[tok];
-            float *o = out + (size_t)tok * rows + r;
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] *= ts;
+        }
+        if (vec_ok && r + 3 < rows) {
+            f32x4 *ov = reinterpret_cast<f32x4 *>(o);
+            if (!partial && accumulate) { const f32x4 old = *ov; v += old; }
+            *ov = v;
+        } else {
 #pragma unroll
             for (int e = 0; e < 4; e++)
-                if (r + e < rows) o[e] = accumulate ? o[e] + acc[i][jj][e] * ts : acc[i][jj][e] * ts;
+                if (r + e < rows) o[e] = (!partial && accumulate) ? o[e] + v[e] : v[e];
         }
+    }
 }
 
 // f32 activations -> bf16 hi (round to nearest even) and the bf16 of the remainder

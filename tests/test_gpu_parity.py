@@ -564,7 +564,7 @@ def test_moe_mxfp4_block_matches_oracle(be, fmt, T, E, hidden, inter):
 
 
 # ------------------------------------------------------------- prefill GEMM
-@pytest.mark.parametrize("rows,hidden,seq", [(300, 512, 70), (128, 3840, 128), (1, 256, 1), (257, 768, 33)])
+@pytest.mark.parametrize("rows,hidden,seq", [(300, 512, 70), (128, 3840, 128), (1, 256, 1), (257, 768, 33), (520, 8192, 200)])
 def test_q4k_gemm_mfma_matches_oracle(be, rows, hidden, seq):
     rng = np.random.default_rng(61 + rows)
     w = (rng.standard_normal((rows, hidden)) * 0.02).astype(F)
