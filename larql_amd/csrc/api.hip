@@ -1083,6 +1083,46 @@ int larql_hip_dev_moe_mxfp4(larql_hip_ctx *c, const larql_hip_mxfp4_experts *ban
     float *g = (float *)workspace, *u = g + slots * inter, *h = u + slots * inter, *d = h + slots * inter;
     const uint64_t gu_w_stride = inter * (hidden / 32) * 16, gu_s_stride = inter * (hidden / 32);
     const uint64_t dn_w_stride = hidden * (inter / 32) * 16, dn_s_stride = hidden * (inter / 32);
+    // Several tokens: slots that chose the same expert share its weights two at a time.  The job lists are built on
+    // the device from the router's choice (moe_plan_kernel) into the workspace's spare activation area.
+    {
+        GemvJob tg = make_job(KIND_MXFP4, bank->gate_packed, bank->gate_scales, x, g, inter, hidden);
+        GemvJob tu = make_job(KIND_MXFP4, bank->up_packed, bank->up_scales, x, u, inter, hidden);
+        GemvJob td = make_job(KIND_MXFP4, bank->down_packed, bank->down_scales, g, d, hidden, inter);
+        td.x_glu = u; td.glu_limit = bank->limit; td.glu_alpha = bank->alpha;
+        const size_t table_bytes = slots * 3 * sizeof(GemvJob) + 64;
+        const bool mfma = gemv_effective_kind(tg) == KIND_MXFP4_MFMA && gemv_effective_kind(td) == KIND_MXFP4_MFMA;
+        static const bool pairing = !(getenv("LARQL_HIP_MOE_PAIRS") && atoi(getenv("LARQL_HIP_MOE_PAIRS")) == 0);
+        if (pairing && mfma && tokens > 1 && slots <= 4096 && bank->n_experts <= 1024 && slots * inter * sizeof(float) >= table_bytes) {
+            tg.kind = tu.kind = td.kind = KIND_MXFP4_MFMA;
+            uint32_t *hdr = (uint32_t *)h;  // {gate/up count, passes, down count, passes}
+            GemvJob *gu_table = (GemvJob *)((uint8_t *)h + 64), *dn_table = gu_table + 2 * slots;
+            PreparedLaunch Pg, Pd;
+            for (int which = 0; which < 2; which++) {
+                GemvJob &tj = which == 0 ? tg : td;
+                PreparedLaunch &P = which == 0 ? Pg : Pd;
+                P.kind = KIND_MXFP4_MFMA;
+                P.threads = gemv_pick_threads(&tj, 1);
+                if (P.threads == 0 || !gemv_job_geometry(tj, P.threads)) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: unsupported geometry");
+                const uint64_t max_jobs = which == 0 ? 2 * slots : slots;
+                if (max_jobs * tj.n_pass > 0x7FFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: launch too large");
+                memset(&P.L, 0, sizeof P.L);
+                P.L.table = which == 0 ? gu_table : dn_table;
+                P.L.dyn = hdr + 2 * which;
+                P.L.pad = gemv_launch_param(&tj, 1);
+                P.lds = gemv_lds_bytes(&tj, 1, P.threads);
+                P.grid = (uint32_t)((uint64_t)c->cu_count * gemv_wgs_per_cu(P.kind, P.threads, P.lds, (uint32_t)c->wgs_per_cu));
+            }
+            if (!gemv_job_geometry(tu, Pg.threads)) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: unsupported geometry");
+            HIPCHECK(c, moe_plan_launch(c->stream, experts, (uint32_t)slots, (uint32_t)k, (uint32_t)bank->n_experts, tg, tu, td, gu_w_stride,
+                                        gu_s_stride, dn_w_stride, dn_s_stride, (uint32_t)hidden, (uint32_t)inter, gu_table, hdr, dn_table,
+                                        hdr + 2));
+            HIPCHECK(c, gemv_launch(c->stream, Pg.kind, Pg.L, Pg.threads, Pg.grid, Pg.lds));
+            HIPCHECK(c, gemv_launch(c->stream, Pd.kind, Pd.L, Pd.threads, Pd.grid, Pd.lds));
+            HIPCHECK(c, weighted_sum_launch(c->stream, d, weights, out, (uint32_t)tokens, (uint32_t)k, (uint32_t)hidden));
+            return LARQL_OK;
+        }
+    }
     std::vector<GemvJob> jobs;
     for (size_t s = 0; s < slots; s++) {
         const size_t t = s / k;

@@ -790,51 +790,58 @@ struct Mx4Step {
 // Every lane converts two activations into their six digits and the wavefront transposes them through
 // `scratch` (768 B of its own LDS: digit row t at t*128) into the operand layout.
 __device__ __forceinline__ Mx4Step mx4_setup_step(const GemvJob &j, uint32_t step, uint32_t lane, uint8_t *scratch) {
-    const float *x = j.x;
     const uint32_t k = (uint32_t)j.k;
     const uint32_t t = lane & 15u, kg = lane >> 4;
     const uint32_t i0 = step * 128 + 2 * lane;
-    float2_t v = {0.f, 0.f};
-    if (i0 + 2 <= k) {  // k is even: a pair is inside or outside
-        v = *(const GLOBAL_AS float2_t *)(x + i0);
-        if (j.x_glu) {
-            // MoeGateRule::ClampedGlu (larql-compute/src/pipeline/moe.rs:88-92): g = min(g, L); u = clamp(u, -L, L);
-            // (u + 1) * (g * sigmoid(alpha * g))
-            const float2_t u = *(const GLOBAL_AS float2_t *)(j.x_glu + i0);
-            const float L = j.glu_limit, al = j.glu_alpha;
-            const float g0 = fminf(v.x, L), g1 = fminf(v.y, L);
-            const float u0 = u.x < -L ? -L : (u.x > L ? L : u.x), u1 = u.y < -L ? -L : (u.y > L ? L : u.y);
-            v.x = (u0 + 1.0f) * (g0 * (1.0f / (1.0f + expf(-(g0 * al)))));
-            v.y = (u1 + 1.0f) * (g1 * (1.0f / (1.0f + expf(-(g1 * al)))));
-        }
-    }
-    float mx = fmaxf(fabsf(v.x), fabsf(v.y));
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
-    int ex = 0;
-    if (mx > 0.f && mx < __builtin_inff()) (void)frexpf(mx, &ex);  // mx = f * 2^ex, f in [0.5, 1)
-    ex = max(-100, min(100, ex));
-    const float to_int = ldexpf(1.f, 23 - ex);
-    // balanced base-16 digits: n + 0x888888 has the unsigned digits d+8 (the top one may reach 16)
-    const int n0 = (int)__builtin_rintf(v.x * to_int) + 0x888888, n1 = (int)__builtin_rintf(v.y * to_int) + 0x888888;
-#pragma unroll
-    for (int d = 0; d < 6; d++) {
-        const int sh = 4 * (5 - d);
-        const int d0 = (d == 0 ? (n0 >> 20) : ((n0 >> sh) & 15)) - 8, d1 = (d == 0 ? (n1 >> 20) : ((n1 >> sh) & 15)) - 8;
-        const int pk = __builtin_amdgcn_cvt_pk_fp8_f32((float)d0, (float)d1, 0, false);  // integers up to 8 are exact in e4m3
-        *reinterpret_cast<uint16_t *>(scratch + d * 128 + 2 * lane) = (uint16_t)pk;
-    }
-    asm volatile("" ::: "memory");  // same wavefront: LDS executes its writes before the reads that follow
+    const uint32_t ntok = j.batch > 1 ? 2u : 1u;
     Mx4Step st;
-    st.scale_a = 124 + ex - 4 * (int)t;  // digit t weighs 2^(ex - 23 + 4*(5 - t))
-    u32x4 lo = {0u, 0u, 0u, 0u}, hi = {0u, 0u, 0u, 0u};
-    if (t < 6) {
-        lo = *reinterpret_cast<const u32x4 *>(scratch + t * 128 + 16 * kg);       // K = 16kg .. 16kg+15
-        hi = *reinterpret_cast<const u32x4 *>(scratch + t * 128 + 64 + 16 * kg);  // K = 64+16kg ..
+#pragma unroll
+    for (int q = 0; q < 8; q++) st.a[q] = 0;
+    st.scale_a = 127;
+    // token q's six digit rows are A rows 8q .. 8q+5 (rows 6, 7, 14, 15 stay zero): its sums come out in D rows of their own
+    for (uint32_t q = 0; q < ntok; q++) {
+        const float *x = j.x + (int64_t)(q * j.x_stride);
+        float2_t v = {0.f, 0.f};
+        if (i0 + 2 <= k) {  // k is even: a pair is inside or outside
+            v = *(const GLOBAL_AS float2_t *)(x + i0);
+            if (j.x_glu) {
+                // MoeGateRule::ClampedGlu (larql-compute/src/pipeline/moe.rs:88-92): g = min(g, L); u = clamp(u, -L, L);
+                // (u + 1) * (g * sigmoid(alpha * g))
+                const float2_t u = *(const GLOBAL_AS float2_t *)(j.x_glu + (int64_t)(q * j.x_stride) + i0);
+                const float L = j.glu_limit, al = j.glu_alpha;
+                const float g0 = fminf(v.x, L), g1 = fminf(v.y, L);
+                const float u0 = u.x < -L ? -L : (u.x > L ? L : u.x), u1 = u.y < -L ? -L : (u.y > L ? L : u.y);
+                v.x = (u0 + 1.0f) * (g0 * (1.0f / (1.0f + expf(-(g0 * al)))));
+                v.y = (u1 + 1.0f) * (g1 * (1.0f / (1.0f + expf(-(g1 * al)))));
+            }
+        }
+        float mx = fmaxf(fabsf(v.x), fabsf(v.y));
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+        int ex = 0;
+        if (mx > 0.f && mx < __builtin_inff()) (void)frexpf(mx, &ex);  // mx = f * 2^ex, f in [0.5, 1)
+        ex = max(-100, min(100, ex));
+        const float to_int = ldexpf(1.f, 23 - ex);
+        // balanced base-16 digits: n + 0x888888 has the unsigned digits d+8 (the top one may reach 16)
+        const int n0 = (int)__builtin_rintf(v.x * to_int) + 0x888888, n1 = (int)__builtin_rintf(v.y * to_int) + 0x888888;
+#pragma unroll
+        for (int d = 0; d < 6; d++) {
+            const int sh = 4 * (5 - d);
+            const int d0 = (d == 0 ? (n0 >> 20) : ((n0 >> sh) & 15)) - 8, d1 = (d == 0 ? (n1 >> 20) : ((n1 >> sh) & 15)) - 8;
+            const int pk = __builtin_amdgcn_cvt_pk_fp8_f32((float)d0, (float)d1, 0, false);  // integers up to 8 are exact in e4m3
+            *reinterpret_cast<uint16_t *>(scratch + d * 128 + 2 * lane) = (uint16_t)pk;
+        }
+        asm volatile("" ::: "memory");  // same wavefront: LDS executes its writes before the reads that follow
+        const uint32_t row = t - 8 * q;  // (wraps for the rows of the other token)
+        if (row < 6) {
+            const u32x4 lo = *reinterpret_cast<const u32x4 *>(scratch + row * 128 + 16 * kg);       // K = 16kg .. 16kg+15
+            const u32x4 hi = *reinterpret_cast<const u32x4 *>(scratch + row * 128 + 64 + 16 * kg);  // K = 64+16kg ..
+            st.a[0] = (int)lo.x; st.a[1] = (int)lo.y; st.a[2] = (int)lo.z; st.a[3] = (int)lo.w;
+            st.a[4] = (int)hi.x; st.a[5] = (int)hi.y; st.a[6] = (int)hi.z; st.a[7] = (int)hi.w;
+            st.scale_a = 124 + ex - 4 * (int)row;  // digit `row` weighs 2^(ex - 23 + 4*(5 - row))
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the scratch is reused by the next token / step
     }
-    st.a[0] = (int)lo.x; st.a[1] = (int)lo.y; st.a[2] = (int)lo.z; st.a[3] = (int)lo.w;
-    st.a[4] = (int)hi.x; st.a[5] = (int)hi.y; st.a[6] = (int)hi.z; st.a[7] = (int)hi.w;
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the scratch is reused by the next step
     return st;
 }
 
@@ -847,7 +854,8 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
     const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t nw_launch = blockDim.x >> 6;
     const uint32_t jr = lane & 15u, kg = lane >> 4;
-    const uint32_t nwj = j.rpp, steps = j.cpr, cw = (uint32_t)j.pad, PW = nwj * 2;
+    const bool two = j.batch > 1;  // two tokens share the weights: their sums leave in D rows 0..7 and 8..15
+    const uint32_t nwj = j.rpp, steps = j.cpr, cw = (uint32_t)j.pad, PW = nwj * (two ? 4u : 2u);
     const uint32_t rows = (uint32_t)j.rows, k = (uint32_t)j.k, nb = k / 32, row_bytes = (uint32_t)j.row_bytes;
     uint8_t *ring = lds + wv * (NS * slot_bytes);
     float *part = reinterpret_cast<float *>(lds + nw_launch * (NS * slot_bytes));
@@ -900,7 +908,7 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
 
     uint32_t n_use = 0;
     for (uint32_t tb = 0; tb < nt; tb += R) {
-        float *pb = part + parity * (R * 16 * nw_launch * 2);
+        float *pb = part + parity * (R * 16 * nw_launch * 4);
         const uint32_t nbt = min((uint32_t)R, nt - tb);
         if (working) {
             for (uint32_t tl = 0; tl < nbt; tl++) {
@@ -925,7 +933,8 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
                 }
                 n_use++;
                 const float v = (D[0] + D[1]) + (D[2] + D[3]);  // digits 4rq..4rq+3 of weight row jr
-                if (kg < 2) pb[(tl * 16 + jr) * PW + wv * 2 + kg] = v;
+                if (two) pb[(tl * 16 + jr) * PW + wv * 4 + kg] = v;
+                else if (kg < 2) pb[(tl * 16 + jr) * PW + wv * 2 + kg] = v;
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -933,12 +942,22 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
         asm volatile("" ::: "memory");
         const uint32_t row_base = (tile_a + tb) * 16;
         const uint32_t nwork = min(nwj, (steps + cw - 1) / cw);
-        for (uint32_t rr = threadIdx.x >> 1; rr < nbt * 16; rr += blockDim.x >> 1) {
-            const uint32_t h = threadIdx.x & 1u;
-            float s = 0.f;
-            for (uint32_t w = 0; w < nwork; w++) s += pb[rr * PW + w * 2 + h];
-            s = dpp_add<0xB1>(s);  // quad_perm [1,0,3,2]
-            if (h == 0 && row_base + rr < rows) ((g_f32wp)j.out)[row_base + rr] = s;
+        if (two) {  // same order of additions per token as the single-token fold: the result does not depend on the pairing
+            for (uint32_t rr = threadIdx.x >> 2; rr < nbt * 16; rr += blockDim.x >> 2) {
+                const uint32_t h = threadIdx.x & 3u;
+                float s = 0.f;
+                for (uint32_t w = 0; w < nwork; w++) s += pb[rr * PW + w * 4 + h];
+                s = dpp_add<0xB1>(s);  // quad_perm [1,0,3,2]
+                if ((h & 1u) == 0 && row_base + rr < rows) ((g_f32wp)(j.out + (int64_t)((h >> 1) * j.out_stride)))[row_base + rr] = s;
+            }
+        } else {
+            for (uint32_t rr = threadIdx.x >> 1; rr < nbt * 16; rr += blockDim.x >> 1) {
+                const uint32_t h = threadIdx.x & 1u;
+                float s = 0.f;
+                for (uint32_t w = 0; w < nwork; w++) s += pb[rr * PW + w * 2 + h];
+                s = dpp_add<0xB1>(s);  // quad_perm [1,0,3,2]
+                if (h == 0 && row_base + rr < rows) ((g_f32wp)j.out)[row_base + rr] = s;
+            }
         }
         parity ^= 1u;
     }
@@ -1727,10 +1746,13 @@ __global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_mfma_kernel(GemvLa
 __global__ void __launch_bounds__(kMx4MaxWaves * 64) gemv_mxfp4_mfma_kernel(GemvLaunch L) {
     extern __shared__ __attribute__((aligned(16))) uint8_t mx4_lds[];
     const GemvJob *jobs = L.table ? L.table : L.inl;
-    const uint64_t P = L.total_passes;
+    // (a job list built on the device brings its own count and pass total)
+    const uint32_t n_jobs = L.dyn ? (uint32_t)__builtin_amdgcn_readfirstlane(((const GLOBAL_AS uint32_t *)L.dyn)[0]) : L.n_jobs;
+    const uint64_t P = L.dyn ? (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane(((const GLOBAL_AS uint32_t *)L.dyn)[1]) : L.total_passes;
+    if (P == 0 || n_jobs == 0) return;
     uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
     const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
-    uint32_t lo = 0, hi = L.n_jobs;
+    uint32_t lo = 0, hi = n_jobs;
     while (lo + 1 < hi) {
         const uint32_t mid = (lo + hi) >> 1;
         if ((uint32_t)__builtin_amdgcn_readfirstlane(jobs[mid].pass_begin) <= p) lo = mid; else hi = mid;
@@ -2072,7 +2094,7 @@ size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
     }
     if (n > 0 && jobs[0].kind == KIND_MXFP4_MFMA) {
         const size_t nw = threads / 64;
-        return nw * kMx4Stages * gemv_launch_param(jobs, n) + 2 * (size_t)kMx4BatchTiles * 16 * nw * 2 * sizeof(float);
+        return nw * kMx4Stages * gemv_launch_param(jobs, n) + 2 * (size_t)kMx4BatchTiles * 16 * nw * 4 * sizeof(float);
     }
     if (n > 0 && jobs[0].kind == KIND_Q4K_MFMA) {
         const size_t nw = threads / 64;

@@ -38,8 +38,9 @@ struct GemvJob {
     // uses w + e*w_sel_stride, aux + e*aux_sel_stride (one bank of equally shaped matrices).
     const uint32_t *sel;
     uint64_t w_sel_stride, aux_sel_stride;
-    // Optional batch (bf16 gates): `batch` activations x + t*x_stride against the same weights, results to
-    // out + t*out_stride (strides in floats).  0 or 1 = a plain matvec.  See gemv_batch_capacity.
+    // Optional batch (bf16 / Q4_K gates, MXFP4 experts shared by two tokens): `batch` activations x + t*x_stride
+    // against the same weights, results to out + t*out_stride (strides in floats; they may wrap, i.e. be
+    // negative, for the MXFP4 pair).  0 or 1 = a plain matvec.  See gemv_batch_capacity.
     uint32_t batch, pad2;
     uint64_t x_stride, out_stride;
     // Optional gated activation (MoE down projection, MXFP4 matrix-core kernel only): when `x_glu` is set the
@@ -54,6 +55,9 @@ struct GemvLaunch {
     uint64_t total_passes;
     uint32_t n_jobs;
     uint32_t pad;
+    // Optional: the job count and pass total live in device memory ({n_jobs, total_passes}, written by a kernel
+    // earlier on the stream) and override the two fields above.  MXFP4 matrix-core kernel only.
+    const uint32_t *dyn;
 };
 
 bool gemv_job_geometry(GemvJob &j, uint32_t threads);
@@ -97,6 +101,10 @@ hipError_t split_bf16_launch(hipStream_t s, const float *x, size_t n, uint16_t *
 // MoE helpers
 hipError_t router_select_launch(hipStream_t s, const float *logits, uint32_t tokens, uint32_t n_experts, uint32_t k, int policy,
                                 uint32_t *experts, float *weights);
+hipError_t moe_plan_launch(hipStream_t s, const uint32_t *experts, uint32_t slots, uint32_t k, uint32_t n_experts, const GemvJob &tg,
+                           const GemvJob &tu, const GemvJob &td, uint64_t gu_w_stride, uint64_t gu_s_stride, uint64_t dn_w_stride,
+                           uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, GemvJob *gu_table, uint32_t *gu_hdr, GemvJob *dn_table,
+                           uint32_t *dn_hdr);
 hipError_t clamped_glu_launch(hipStream_t s, const float *g, const float *u, float *h, size_t n, float limit, float alpha);
 hipError_t weighted_sum_launch(hipStream_t s, const float *d, const float *weights, float *out, uint32_t tokens, uint32_t k,
                                uint32_t hidden);

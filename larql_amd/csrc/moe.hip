@@ -85,6 +85,87 @@ __global__ void weighted_sum_kernel(const float *__restrict__ d, const float *__
     out[(size_t)t * hidden + i] = acc;
 }
 
+// Job lists of an expert block, built on the device from the router's choice (no host round trip): the slots
+// (token, rank) that chose the same expert are paired, in slot order, and every pair (or single) becomes one
+// gate, one up and one down job whose two activations share the expert's weights (GemvJob::batch = 2; the
+// second activation / result sits x_stride / out_stride floats away from the first, in either direction).
+// tg / tu / td are the jobs of slot 0 with expert 0 (geometry filled in); tables: [gate jobs | up jobs], [down jobs];
+// headers: {job count, pass total}.  One block; a thread per slot, O(slots) work each.
+__global__ void __launch_bounds__(256) moe_plan_kernel(const uint32_t *__restrict__ experts, uint32_t slots, uint32_t k, uint32_t n_experts,
+                                                       GemvJob tg, GemvJob tu, GemvJob td, uint64_t gu_w_stride, uint64_t gu_s_stride,
+                                                       uint64_t dn_w_stride, uint64_t dn_s_stride, uint32_t hidden, uint32_t inter,
+                                                       GemvJob *__restrict__ gu_table, uint32_t *__restrict__ gu_hdr,
+                                                       GemvJob *__restrict__ dn_table, uint32_t *__restrict__ dn_hdr) {
+    __shared__ uint32_t first_job[1025];  // first job of expert e; [n_experts] = total
+    __shared__ uint32_t cnt[1024];        // slots per expert
+    __shared__ uint32_t ex[4096];         // the router's choice, read once
+    __shared__ uint32_t partner[4096];    // second slot of a job (or ~0)
+    const uint32_t t = threadIdx.x;
+    for (uint32_t e = t; e < n_experts; e += blockDim.x) cnt[e] = 0;
+    for (uint32_t s = t; s < slots; s += blockDim.x) { ex[s] = experts[s]; partner[s] = 0xFFFFFFFFu; }
+    __syncthreads();
+    for (uint32_t s = t; s < slots; s += blockDim.x)
+        if (ex[s] < n_experts) atomicAdd(&cnt[ex[s]], 1u);
+    __syncthreads();
+    for (uint32_t e = t; e <= n_experts; e += blockDim.x) {
+        uint32_t f = 0;
+        for (uint32_t q = 0; q < e; q++) f += (cnt[q] + 1) / 2;
+        first_job[e] = f;
+    }
+    __syncthreads();
+    const uint32_t n_jobs = first_job[n_experts];
+    // a slot's rank among the slots of its expert, in slot order: even ranks open a job, odd ranks join it
+    for (uint32_t s = t; s < slots; s += blockDim.x) {
+        const uint32_t e = ex[s];
+        if (e >= n_experts) continue;
+        uint32_t r = 0;
+        for (uint32_t q = 0; q < s; q++) r += ex[q] == e ? 1u : 0u;
+        if (r & 1u) partner[first_job[e] + r / 2] = s;
+    }
+    __syncthreads();
+    for (uint32_t s1 = t; s1 < slots; s1 += blockDim.x) {
+        const uint32_t e = ex[s1];
+        if (e >= n_experts) continue;
+        uint32_t r = 0;
+        for (uint32_t q = 0; q < s1; q++) r += ex[q] == e ? 1u : 0u;
+        if (r & 1u) continue;
+        const uint32_t jb = first_job[e] + r / 2;
+        const bool pair = partner[jb] != 0xFFFFFFFFu;
+        const uint32_t s2 = pair ? partner[jb] : s1, nb = pair ? 2u : 1u;
+        const uint32_t tok1 = s1 / k, tok2 = s2 / k;
+        GemvJob a = tg, b = tu, c = td;
+        a.w += (size_t)e * gu_w_stride; a.aux += (size_t)e * gu_s_stride;
+        b.w += (size_t)e * gu_w_stride; b.aux += (size_t)e * gu_s_stride;
+        c.w += (size_t)e * dn_w_stride; c.aux += (size_t)e * dn_s_stride;
+        a.x += (size_t)tok1 * hidden; b.x += (size_t)tok1 * hidden;
+        a.out += (size_t)s1 * inter; b.out += (size_t)s1 * inter;
+        c.x += (size_t)s1 * inter; c.x_glu += (size_t)s1 * inter; c.out += (size_t)s1 * hidden;
+        a.batch = b.batch = c.batch = nb;
+        a.x_stride = b.x_stride = (uint64_t)(((int64_t)tok2 - (int64_t)tok1) * (int64_t)hidden);
+        a.out_stride = b.out_stride = (uint64_t)(((int64_t)s2 - (int64_t)s1) * (int64_t)inter);
+        c.x_stride = (uint64_t)(((int64_t)s2 - (int64_t)s1) * (int64_t)inter);
+        c.out_stride = (uint64_t)(((int64_t)s2 - (int64_t)s1) * (int64_t)hidden);
+        a.pass_begin = jb * tg.n_pass;
+        b.pass_begin = (n_jobs + jb) * tg.n_pass;
+        c.pass_begin = jb * td.n_pass;
+        gu_table[jb] = a; gu_table[n_jobs + jb] = b; dn_table[jb] = c;
+    }
+    if (t == 0) {
+        gu_hdr[0] = 2 * n_jobs; gu_hdr[1] = 2 * n_jobs * tg.n_pass;
+        dn_hdr[0] = n_jobs; dn_hdr[1] = n_jobs * td.n_pass;
+    }
+}
+
+hipError_t moe_plan_launch(hipStream_t s, const uint32_t *experts, uint32_t slots, uint32_t k, uint32_t n_experts, const GemvJob &tg,
+                           const GemvJob &tu, const GemvJob &td, uint64_t gu_w_stride, uint64_t gu_s_stride, uint64_t dn_w_stride,
+                           uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, GemvJob *gu_table, uint32_t *gu_hdr, GemvJob *dn_table,
+                           uint32_t *dn_hdr) {
+    if (n_experts > 1024) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(256), 0, s, experts, slots, k, n_experts, tg, tu, td, gu_w_stride, gu_s_stride,
+                       dn_w_stride, dn_s_stride, hidden, inter, gu_table, gu_hdr, dn_table, dn_hdr);
+    return hipGetLastError();
+}
+
 hipError_t router_select_launch(hipStream_t s, const float *logits, uint32_t tokens, uint32_t n_experts, uint32_t k, int policy,
                                 uint32_t *experts, float *weights) {
     if (tokens == 0) return hipSuccess;

@@ -563,6 +563,48 @@ def test_moe_mxfp4_block_matches_oracle(be, fmt, T, E, hidden, inter):
     assert not be.dev_moe_mxfp4(b, dev["x"], T, k, de, dw_, do, ws, wsb - 1024)   # short workspace: refused
 
 
+def test_moe_mxfp4_tokens_sharing_an_expert_equal_single_token_calls(be, fmt):
+    """Slots that chose the same expert are served two at a time from one read of its weights; a token's result
+    must not depend on who it was paired with: the 13-token block equals 13 one-token blocks bit for bit."""
+    rng = np.random.default_rng(83)
+    T, E, hidden, inter, k = 13, 6, 384, 320, 4          # 52 slots over 6 experts: pairs, odd leftovers, far-apart partners
+
+    def bank(n, kk):
+        p, s = [], []
+        for _ in range(E):
+            pp, ss = O.quantize_mxfp4((rng.standard_normal(n * kk) * 0.05).astype(F), n, kk)
+            p.append(pp); s.append(ss)
+        return np.concatenate(p), np.concatenate(s)
+
+    gp, gs = bank(inter, hidden); up, us = bank(inter, hidden); dp, ds = bank(hidden, inter)
+    x = rng.standard_normal((T, hidden)).astype(F)
+    logits = rng.standard_normal((T, E)).astype(F)
+    dev = {n: be.to_device(a) for n, a in dict(gp=gp, gs=gs, up=up, us=us, dp=dp, ds=ds, x=x, lg=logits).items()}
+    b = fmt.Mxfp4Experts(dev["gp"], dev["gs"], dev["up"], dev["us"], dev["dp"], dev["ds"], E, hidden, inter, 7.0, 1.702)
+    de, dw_, do = be.malloc(T * k * 4), be.malloc(T * k * 4), be.malloc(T * hidden * 4)
+    assert be.dev_router_select(dev["lg"], T, E, k, O.NORMALISED_OVER_SELECTED, de, dw_)
+    wsb = be.moe_mxfp4_workspace_bytes(T, k, hidden, inter)
+    ws = be.malloc(wsb)
+    assert be.dev_moe_mxfp4(b, dev["x"], T, k, de, dw_, do, ws, wsb)
+    be.synchronize()
+    got = be.d2h(do, (T, hidden), F)
+    one = be.malloc(hidden * 4)
+    for t in range(T):
+        assert be.dev_moe_mxfp4(b, dev["x"] + t * hidden * 4, 1, k, de + t * k * 4, dw_ + t * k * 4, one, ws, wsb)
+        be.synchronize()
+        assert np.array_equal(be.d2h(one, hidden, F), got[t]), t
+    # and the oracle, token 5
+    acc = np.zeros(hidden, F)
+    gw, gsz = inter * (hidden // 32) * 16, inter * (hidden // 32)
+    dwb, dsz = hidden * (inter // 32) * 16, hidden * (inter // 32)
+    for e, w in O.router_select(logits[5], k):
+        g = O.mxfp4_gemv(gp[e * gw:(e + 1) * gw], gs[e * gsz:(e + 1) * gsz], x[5], inter, hidden)
+        u = O.mxfp4_gemv(up[e * gw:(e + 1) * gw], us[e * gsz:(e + 1) * gsz], x[5], inter, hidden)
+        hh = np.array([O.clamped_glu(float(a), float(b_)) for a, b_ in zip(g, u)], F)
+        acc = (acc + F(w) * O.mxfp4_gemv(dp[e * dwb:(e + 1) * dwb], ds[e * dsz:(e + 1) * dsz], hh, hidden, inter)).astype(F)
+    assert rel_l2(got[5], acc) < 1e-5
+
+
 # ------------------------------------------------------------- prefill GEMM
 @pytest.mark.parametrize("rows,hidden,seq", [(300, 512, 70), (128, 3840, 128), (1, 256, 1), (257, 768, 33), (520, 8192, 200)])
 def test_q4k_gemm_mfma_matches_oracle(be, rows, hidden, seq):
