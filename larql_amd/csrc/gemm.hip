@@ -166,7 +166,7 @@ constexpr int LDM = 40;  // padded row of the 32-slot min tiles (f16 elements)
 __global__ void __launch_bounds__(256) q4k_gemm_prep_kernel(const void *__restrict__ x, int x_is_bf16, uint32_t hidden,
                                                             uint16_t *__restrict__ xh, uint16_t *__restrict__ xl,
                                                             uint16_t *__restrict__ sx, float *__restrict__ tok_scale,
-                                                            int *__restrict__ any_lo) {
+                                                            int *__restrict__ any_lo, int swap12) {
     __shared__ float red[4];
     const uint32_t tok = blockIdx.x, t = threadIdx.x, nvec = hidden >> 3;  // hidden % 256 == 0
     const u32x4 *xb = reinterpret_cast<const u32x4 *>((const uint16_t *)x + (size_t)tok * hidden);
@@ -207,7 +207,7 @@ __global__ void __launch_bounds__(256) q4k_gemm_prep_kernel(const void *__restri
     for (uint32_t v = t; v < nvec; v += 256) {  // nvec % 32 == 0: the four threads of a sub-block run together
         float o[8];
         load8(v, o);
-        uint32_t hw[4], lw[4];
+        uint32_t hw[4] = {0u, 0u, 0u, 0u}, lw[4] = {0u, 0u, 0u, 0u};
         float sm = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
@@ -215,7 +215,10 @@ __global__ void __launch_bounds__(256) q4k_gemm_prep_kernel(const void *__restri
             const _Float16 h = (_Float16)sv;
             const _Float16 l = (_Float16)(sv - (float)h);
             const uint32_t hb = __builtin_bit_cast(uint16_t, h), lb = __builtin_bit_cast(uint16_t, l);
-            if (i & 1) { hw[i >> 1] |= hb << 16; lw[i >> 1] |= lb << 16; } else { hw[i >> 1] = hb; lw[i >> 1] = lb; }
+            // `swap12`: elements 1 and 2 of every four change places (the pipelined GEMM's weight operand comes out of
+            // its nibble masks as the pairs (k0, k2), (k1, k3); the MFMA only needs both operands to agree)
+            const int pos = swap12 ? ((i & 4) | ((i & 1) << 1) | ((i >> 1) & 1)) : i;
+            if (pos & 1) { hw[pos >> 1] |= hb << 16; lw[pos >> 1] |= lb << 16; } else { hw[pos >> 1] |= hb; lw[pos >> 1] |= lb; }
             lo_seen |= (ol && (float)l != 0.f) ? 1 : 0;
             sm += (float)h + (ol ? (float)l : 0.f);  // the activation as the MFMAs will see it
         }
@@ -506,23 +509,29 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
         }
     };
     // scale of sub-block `sub` (0..7) of the current header as the packed-FMA operands (sc6, -1024*sc6)
+    // (odd sub-blocks are the high nibbles: their masked value is 1024 + 16q, so the factor is sc6/16 and the offset -64*sc6)
     auto scale_of = [&](uint32_t sub, f16x2 &sc2, f16x2 &off2) {
         const uint32_t sh = 8u * (sub & 3u);
         const uint32_t pa = (hdr_y >> sh) & 0xFFu, pc = (hdr_w >> sh) & 0xFFu;
         const uint32_t sc6 = sub < 4 ? (pa & 63u) : ((pc & 0x0Fu) | ((pa >> 6) << 4));
-        const _Float16 scf = (_Float16)(float)sc6, of = (_Float16)(-1024.0f * (float)sc6);
+        const float f = (float)sc6;
+        const _Float16 scf = (_Float16)((sub & 1u) ? f * 0.0625f : f), of = (_Float16)((sub & 1u) ? -64.0f * f : -1024.0f * f);
         sc2 = (f16x2){scf, scf};
         off2 = (f16x2){of, of};
     };
-    // 4 raw bytes (nibble h) -> two dwords of f16(sc6*q): exact (sc6*q <= 945)
+    // 4 raw bytes (nibble h) -> two dwords of f16(sc6*q), exact (sc6*q <= 945), as the pairs (k0, k2) and (k1, k3):
+    // the nibbles of bytes 0 and 2 are masked in place into the mantissas of two f16 (1024 + q, or 1024 + 16q for
+    // the high nibbles), those of bytes 1 and 3 after one shift; one packed FMA takes the 1024 away and applies
+    // sc6 (sc6/16) with a single rounding.  `magic` is 0x64006400 held in a register so that mask-and-or is one
+    // instruction.
+    uint32_t magic;
+    asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
     auto convert4 = [&](uint32_t raw, uint32_t h, f16x2 sc2, f16x2 off2, uint32_t &o0, uint32_t &o1) {
-        const uint32_t v = raw >> (h * 4u);  // low or high nibbles (the mask below drops the rest)
-        // bytes 0,1 -> 16-bit lanes of one dword, bytes 2,3 -> the next (k order kept)
-        const uint32_t p01 = __builtin_amdgcn_perm(0u, v, 0x0C010C00u), p23 = __builtin_amdgcn_perm(0u, v, 0x0C030C02u);
-        const f16x2 m01 = __builtin_bit_cast(f16x2, (p01 & 0x000F000Fu) | 0x64006400u);  // 1024 + q
-        const f16x2 m23 = __builtin_bit_cast(f16x2, (p23 & 0x000F000Fu) | 0x64006400u);
-        o0 = __builtin_bit_cast(uint32_t, m01 * sc2 + off2);  // (1024+q)*sc6 - 1024*sc6, one rounding: exact
-        o1 = __builtin_bit_cast(uint32_t, m23 * sc2 + off2);
+        const uint32_t mask = h ? 0x00F000F0u : 0x000F000Fu;
+        const f16x2 m02 = __builtin_bit_cast(f16x2, (raw & mask) | magic);
+        const f16x2 m13 = __builtin_bit_cast(f16x2, ((raw >> 8) & mask) | magic);
+        o0 = __builtin_bit_cast(uint32_t, m02 * sc2 + off2);
+        o1 = __builtin_bit_cast(uint32_t, m13 * sc2 + off2);
     };
     // where this thread's two chunks of k-half h go
     uint8_t *const a_row = plds + P_A_OFF + sr * 128;
@@ -584,15 +593,19 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
                     amf[i] = __builtin_bit_cast(f16x8, av);
                     bmf[i] = __builtin_bit_cast(f16x8, bv);
                 }
+                // (D is free here: the sixteen products go there back to back, then they are folded in)
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int jj = 0; jj < 4; jj++)
+                        D[i][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(amf[i], bmf[jj], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const f32x4 mv = *reinterpret_cast<const f32x4 *>(plds + P_DMIN_OFF + (par * PM + wm + i * 16 + kg * 4) * 4);
 #pragma unroll
-                    for (int jj = 0; jj < 4; jj++) {
-                        const f32x4 Dm = __builtin_amdgcn_mfma_f32_16x16x32_f16(amf[i], bmf[jj], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    for (int jj = 0; jj < 4; jj++)
 #pragma unroll
-                        for (int e = 0; e < 4; e++) acc[i][jj][e] = __builtin_fmaf(-mv[e], Dm[e], acc[i][jj][e]);
-                    }
+                        for (int e = 0; e < 4; e++) acc[i][jj][e] = __builtin_fmaf(-mv[e], D[i][jj][e], acc[i][jj][e]);
                 }
             }
 #pragma unroll
@@ -609,16 +622,17 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
                 f16x2 sc2, off2;
                 scale_of(h == 0 ? 2 * g + 1 : 2 * ((g + 1) & 3), sc2, off2);
                 const uint32_t c0 = 4 * nib + 2 * part;                     // destination chunks c0, c0+1
-                f16x8 af[4], bf[2];
+                f16x8 af[4], bf[4];
 #pragma unroll
                 for (int i = 0; i < 4; i++) af[i] = a_frag(h, i);
                 bf[0] = b_frag(h, 0);
+                bf[1] = b_frag(h, 1);
                 uint32_t aw[8];
                 __builtin_amdgcn_sched_barrier(0);
-                // four groups of four MFMAs; each carries a quarter of the conversion and the next operand read
+                // four groups of four MFMAs; each carries a quarter of the conversion and an operand read two groups ahead
 #pragma unroll
                 for (int jj = 0; jj < 4; jj++) {
-                    if (jj + 1 < 4) bf[(jj + 1) & 1] = b_frag(h, jj + 1);
+                    if (jj + 2 < 4) bf[jj + 2] = b_frag(h, jj + 2);
                     convert4(qd[jj], nib, sc2, off2, aw[2 * jj], aw[2 * jj + 1]);
                     if (jj & 1) {
                         const int c = jj >> 1;
@@ -626,7 +640,7 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
                     }
 #pragma unroll
                     for (int i = 0; i < 4; i++)  // (a super-block's first MFMAs start from zero: D is never cleared)
-                        D[i][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bf[jj & 1], (g == 0 && h == 0) ? (f32x4){0.f, 0.f, 0.f, 0.f} : D[i][jj], 0, 0, 0);
+                        D[i][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bf[jj], (g == 0 && h == 0) ? (f32x4){0.f, 0.f, 0.f, 0.f} : D[i][jj], 0, 0, 0);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 if (h == 1 && g == 3) {
@@ -708,6 +722,11 @@ __global__ void split_bf16_kernel(const float *__restrict__ x, size_t n, uint16_
     if ((l & 0x7FFFu) != 0) *any_lo = 1;
 }
 
+static bool gemm_pipe_enabled() {
+    static const bool on = !(getenv("LARQL_HIP_GEMM_PIPE") && atoi(getenv("LARQL_HIP_GEMM_PIPE")) == 0);
+    return on;
+}
+
 hipError_t q4k_gemm_launch(hipStream_t s, const uint8_t *w, const uint16_t *x_bf16, float *out, uint32_t rows, uint32_t hidden,
                            uint32_t seq, int accumulate) {
     if (rows == 0 || seq == 0) return hipSuccess;
@@ -719,14 +738,11 @@ hipError_t q4k_gemm_launch(hipStream_t s, const uint8_t *w, const uint16_t *x_bf
 hipError_t q4k_gemm_prep_launch(hipStream_t s, const void *x, int x_is_bf16, uint32_t hidden, uint32_t seq, uint16_t *xh, uint16_t *xl,
                                 uint16_t *sx, float *tok_scale, int *any_lo) {
     if (seq == 0) return hipSuccess;
-    hipLaunchKernelGGL(q4k_gemm_prep_kernel, dim3(seq), dim3(256), 0, s, x, x_is_bf16, hidden, xh, xl, sx, tok_scale, any_lo);
+    hipLaunchKernelGGL(q4k_gemm_prep_kernel, dim3(seq), dim3(256), 0, s, x, x_is_bf16, hidden, xh, xl, sx, tok_scale, any_lo,
+                       gemm_pipe_enabled() ? 1 : 0);
     return hipGetLastError();
 }
 
-static bool gemm_pipe_enabled() {
-    static const bool on = !(getenv("LARQL_HIP_GEMM_PIPE") && atoi(getenv("LARQL_HIP_GEMM_PIPE")) == 0);
-    return on;
-}
 
 // K-ranges per output tile so that a launch fills the CUs (1 = no split)
 uint32_t q4k_gemm_splits(uint32_t rows, uint32_t hidden, uint32_t seq, uint32_t cu_count) {
