@@ -423,7 +423,7 @@ constexpr int PM = 256, PN = 128, PTHREADS = 512;
 constexpr int P_NB = 4, P_NR = 5;                                               // ring depths: activations, raw weights
 constexpr int P_A_BYTES = PM * 128, P_B_STAGE = PN * 128, P_R_STAGE = PM * 32;  // bytes
 constexpr int P_A_OFF = 0, P_B_OFF = P_A_BYTES, P_R_OFF = P_B_OFF + P_NB * P_B_STAGE, P_H_OFF = P_R_OFF + P_NR * P_R_STAGE,
-              P_AM_OFF = P_H_OFF + PM * 16, P_BM_OFF = P_AM_OFF + PM * 32, P_D_OFF = P_BM_OFF + PN * 32,
+              P_AM_OFF = P_H_OFF + PM * 32, P_BM_OFF = P_AM_OFF + PM * 32, P_D_OFF = P_BM_OFF + PN * 32,
               P_DMIN_OFF = P_D_OFF + 2 * PM * 4, P_LDS_BYTES = P_DMIN_OFF + 2 * PM * 4;
 static_assert(P_LDS_BYTES <= 160 * 1024, "one workgroup per CU");
 typedef __attribute__((address_space(3))) void *p_lds_vp;
@@ -451,8 +451,8 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
     // copy roles.  Raw weights: thread -> (row t/2, part t&1) of a step, i.e. wavefront w brings rows 32w .. 32w+31.
     const uint8_t *wt = w + (size_t)row0 * row_bytes;                                          // uniform
     const uint32_t r_off = (min(row0 + sr, rows - 1) - row0) * row_bytes + part * 16;
-    // headers: wavefronts w and w+4 both bring rows 64*(w&3) .. +63
-    const uint32_t h_off = (min(row0 + (wave & 3u) * 64 + lane, rows - 1) - row0) * row_bytes;
+    // headers: a wavefront brings those of its own 32 rows (lanes 32..63 a second copy: the copy is 64 lanes wide)
+    const uint32_t h_off = (min(row0 + wave * 32 + (lane & 31u), rows - 1) - row0) * row_bytes;
     // activations: wavefront -> tokens 16w .. 16w+15 (two copies of 8 tokens x 128 bytes), lane -> (token, chunk)
     const uint8_t *xt = (const uint8_t *)xh + (size_t)tok0 * hidden * 2;                       // uniform
     uint32_t b_off[2];
@@ -465,8 +465,9 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
     const uint8_t *st = (const uint8_t *)sx + (size_t)tok0 * (hidden / 32) * 4;                // uniform
     const uint32_t m_off = (min(tok0 + (wave & 3u) * 32 + (lane >> 1), seq - 1) - tok0) * (hidden / 32) * 4 + (lane & 1u) * 16;
 
-    // compute role
-    const uint32_t wm = (wave >> 1) * 64, wn = (wave & 1u) * 64;
+    // compute role: a wavefront owns the 32 rows it converts, against all 128 tokens: the weight operand, the raw
+    // bytes, the headers and the per-row constants never cross wavefronts, only the activations (and Sx) do
+    const uint32_t wm = wave * 32;
     const uint32_t l16 = lane & 15u, kg = lane >> 4, sw_a = q4k_gemm_swz(l16), sw_b = l16 & 7u;
 
     // (requests past the end are clamped: same number of copies in flight, results unused)
@@ -484,12 +485,12 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
     };
     auto issue_sb = [&](uint32_t sb) {  // header and Sx of a super-block
         const uint32_t sbc = min(sb, sb_end - 1);
-        __builtin_amdgcn_global_load_lds((p_g_vp)((wt + (size_t)sbc * 144) + h_off), (p_lds_vp)(plds + P_H_OFF + (wave & 3u) * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((p_g_vp)((wt + (size_t)sbc * 144) + h_off), (p_lds_vp)(plds + P_H_OFF + wave * 1024), 16, 0, 0);
         __builtin_amdgcn_global_load_lds((p_g_vp)((st + (size_t)sbc * 32) + m_off), (p_lds_vp)(plds + P_BM_OFF + (wave & 3u) * 1024), 16, 0, 0);
     };
     uint32_t hdr_y = 0, hdr_w = 0;  // the scale words of the super-block being converted
     auto stage_sb = [&](uint32_t par) {  // a super-block's header: scale words to registers, mn6 / d / dmin to LDS
-        const u32x4 hdr = *reinterpret_cast<const u32x4 *>(plds + P_H_OFF + sr * 16);
+        const u32x4 hdr = *reinterpret_cast<const u32x4 *>(plds + P_H_OFF + wave * 1024 + (lane >> 1) * 16);
         hdr_y = hdr.y; hdr_w = hdr.w;
         if (with_mins) {
             uint32_t mnw[4];
@@ -540,11 +541,11 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
         return *reinterpret_cast<const f16x8 *>(plds + P_A_OFF + (wm + i * 16 + l16) * 128 + ((((uint32_t)kk * 4 + kg) ^ sw_a) << 4));
     };
 
-    f32x4 acc[4][4], D[4][4];
+    f32x4 acc[2][8], D[2][8];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int jj = 0; jj < 4; jj++) { acc[i][jj] = (f32x4){0.f, 0.f, 0.f, 0.f}; D[i][jj] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
+        for (int jj = 0; jj < 8; jj++) { acc[i][jj] = (f32x4){0.f, 0.f, 0.f, 0.f}; D[i][jj] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
 
     // ---- prologue: first super-block's header and Sx, raw steps 0..3, activation steps 0..2; k 0..31 of step 0 converted ----
     issue_sb(sb_begin);
@@ -574,36 +575,41 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
         const uint32_t par = (sb - sb_begin) & 1u;
 #pragma unroll
         for (int g = 0; g < 4; g++, s++) {
-            // ---- requests: raw weights of step s+4, activations of step s+3 ----
+            // ---- requests: raw weights of step s+4, activations of step s+3, (at g = 1) the next super-block's header and Sx ----
             issue_raw(s + 4);
             issue_b(s + 3);
+            if (g == 1) issue_sb(sb + 1);  // (after the barrier that ended g = 0: everybody is past this super-block's Sx)
             const uint8_t *B = plds + P_B_OFF + (s % P_NB) * P_B_STAGE;
             auto b_frag = [&](int kk, int jj) {
-                return *reinterpret_cast<const f16x8 *>(B + (wn + jj * 16 + l16) * 128 + ((((uint32_t)kk * 4 + kg) ^ sw_b) << 4));
+                return *reinterpret_cast<const f16x8 *>(B + (jj * 16 + l16) * 128 + ((((uint32_t)kk * 4 + kg) ^ sw_b) << 4));
             };
             if (g == 0 && with_mins) {
                 // offsets of the super-block: sum_sub mn6 * Sx (A slots 2*sub+h = 32*mn6, B slots = Sx_h/32; slots 16..31 are zero)
                 const uint32_t kgc = min(kg, 1u);
-                f16x8 amf[4], bmf[4];
+                f16x8 amf[2], bmf[8];
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
+                for (int i = 0; i < 2; i++) {
                     u32x4 av = *reinterpret_cast<const u32x4 *>(plds + P_AM_OFF + (wm + i * 16 + l16) * 32 + kgc * 16);
-                    u32x4 bv = *reinterpret_cast<const u32x4 *>(plds + P_BM_OFF + (wn + i * 16 + l16) * 32 + kgc * 16);
-                    if (kg >= 2) { av = (u32x4){0u, 0u, 0u, 0u}; bv = (u32x4){0u, 0u, 0u, 0u}; }
+                    if (kg >= 2) av = (u32x4){0u, 0u, 0u, 0u};
                     amf[i] = __builtin_bit_cast(f16x8, av);
-                    bmf[i] = __builtin_bit_cast(f16x8, bv);
+                }
+#pragma unroll
+                for (int jj = 0; jj < 8; jj++) {
+                    u32x4 bv = *reinterpret_cast<const u32x4 *>(plds + P_BM_OFF + (jj * 16 + l16) * 32 + kgc * 16);
+                    if (kg >= 2) bv = (u32x4){0u, 0u, 0u, 0u};
+                    bmf[jj] = __builtin_bit_cast(f16x8, bv);
                 }
                 // (D is free here: the sixteen products go there back to back, then they are folded in)
 #pragma unroll
-                for (int i = 0; i < 4; i++)
+                for (int i = 0; i < 2; i++)
 #pragma unroll
-                    for (int jj = 0; jj < 4; jj++)
+                    for (int jj = 0; jj < 8; jj++)
                         D[i][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(amf[i], bmf[jj], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
+                for (int i = 0; i < 2; i++) {
                     const f32x4 mv = *reinterpret_cast<const f32x4 *>(plds + P_DMIN_OFF + (par * PM + wm + i * 16 + kg * 4) * 4);
 #pragma unroll
-                    for (int jj = 0; jj < 4; jj++)
+                    for (int jj = 0; jj < 8; jj++)
 #pragma unroll
                         for (int e = 0; e < 4; e++) acc[i][jj][e] = __builtin_fmaf(-mv[e], D[i][jj][e], acc[i][jj][e]);
                 }
@@ -611,8 +617,8 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
 #pragma unroll
             for (int h = 0; h < 2; h++) {
                 // ---- half h: the matrix cores take k 32h .. 32h+31 of step s; the threads convert, for h = 0, this step's
-                //      k 32..63 (high nibbles of raw step s) and, for h = 1, the next step's k 0..31 (low nibbles of s+1) ----
-                if (h == 1 && g == 0) issue_sb(sb + 1);  // (everybody is past this super-block's Sx and header now)
+                //      k 32..63 (high nibbles of raw step s) and, for h = 1, the next step's k 0..31 (low nibbles of s+1).
+                //      Both halves of the operand belong to this wavefront alone: no barrier between them ----
                 if (h == 1 && g == 3) stage_sb(par ^ 1u);
                 __builtin_amdgcn_sched_barrier(0);
                 const uint32_t rs = s + h;                                  // raw step being converted
@@ -622,73 +628,78 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
                 f16x2 sc2, off2;
                 scale_of(h == 0 ? 2 * g + 1 : 2 * ((g + 1) & 3), sc2, off2);
                 const uint32_t c0 = 4 * nib + 2 * part;                     // destination chunks c0, c0+1
-                f16x8 af[4], bf[4];
+                f16x8 af[2], bf[8];
 #pragma unroll
-                for (int i = 0; i < 4; i++) af[i] = a_frag(h, i);
+                for (int i = 0; i < 2; i++) af[i] = a_frag(h, i);
                 bf[0] = b_frag(h, 0);
                 bf[1] = b_frag(h, 1);
                 uint32_t aw[8];
                 __builtin_amdgcn_sched_barrier(0);
-                // four groups of four MFMAs; each carries a quarter of the conversion and an operand read two groups ahead
+                // eight groups of two MFMAs; every other one carries a quarter of the conversion, each an operand read two groups ahead
 #pragma unroll
-                for (int jj = 0; jj < 4; jj++) {
-                    if (jj + 2 < 4) bf[jj + 2] = b_frag(h, jj + 2);
-                    convert4(qd[jj], nib, sc2, off2, aw[2 * jj], aw[2 * jj + 1]);
-                    if (jj & 1) {
-                        const int c = jj >> 1;
+                for (int jj = 0; jj < 8; jj++) {
+                    if (jj + 2 < 8) bf[jj + 2] = b_frag(h, jj + 2);
+                    if ((jj & 1) == 0) convert4(qd[jj >> 1], nib, sc2, off2, aw[jj], aw[jj + 1]);
+                    if ((jj & 3) == 3) {
+                        const int c = jj >> 2;
                         *reinterpret_cast<u32x4 *>(a_row + (((c0 + c) ^ a_swz) << 4)) = (u32x4){aw[4 * c], aw[4 * c + 1], aw[4 * c + 2], aw[4 * c + 3]};
                     }
 #pragma unroll
-                    for (int i = 0; i < 4; i++)  // (a super-block's first MFMAs start from zero: D is never cleared)
+                    for (int i = 0; i < 2; i++)  // (a super-block's first MFMAs start from zero: D is never cleared)
                         D[i][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bf[jj], (g == 0 && h == 0) ? (f32x4){0.f, 0.f, 0.f, 0.f} : D[i][jj], 0, 0, 0);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 if (h == 1 && g == 3) {
                     // ---- end of the super-block: acc += d * D ----
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
+                    for (int i = 0; i < 2; i++) {
                         const f32x4 dv = *reinterpret_cast<const f32x4 *>(plds + P_D_OFF + (par * PM + wm + i * 16 + kg * 4) * 4);
 #pragma unroll
-                        for (int jj = 0; jj < 4; jj++) {
+                        for (int jj = 0; jj < 8; jj++) {
 #pragma unroll
                             for (int e = 0; e < 4; e++) acc[i][jj][e] = __builtin_fmaf(dv[e], D[i][jj][e], acc[i][jj][e]);
                         }
                     }
                 }
                 asm volatile("" ::: "memory");
-                if (h == 1) {
-                    // ---- end of step: only the copies requested in this step and the one before may still fly
-                    //      (3 per step, 5 in a super-block's first) ----
-                    if (g == 0 || g == 1) GEMM_WAIT_VMCNT(8);
+                if (h == 0) {
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own conversion stores before own operand reads
+                } else {
+                    // ---- end of step: only the copies requested in this step and the one before may still fly (3 per
+                    //      step, 5 at g = 1); at g = 2 only this step's, so that the header requested at g = 1 is there
+                    //      for the conversion that opens the next super-block ----
+                    if (g == 0) GEMM_WAIT_VMCNT(6);
+                    else if (g == 1) GEMM_WAIT_VMCNT(8);
+                    else if (g == 2) GEMM_WAIT_VMCNT(3);
                     else GEMM_WAIT_VMCNT(6);
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    __builtin_amdgcn_s_barrier();  // everybody's activation copies are visible; everybody is done with stage s
                 }
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
             }
         }
     }
     GEMM_WAIT_VMCNT(0);  // the clamped requests past the end
 
-    // Results leave through LDS so that a store instruction writes whole lines: each wavefront parks its 64x64
-    // block as [token][row] (token rows padded to 68 floats: the 8 lanes of a write phase hit 8 bank groups) in
-    // its own 17 KB, then every lane stores 16 bytes of a 256-byte run of one token.
+    // Results leave through LDS so that a store instruction writes whole lines: each wavefront parks its 32-row x
+    // 128-token block as [token][row] (token rows padded to 36 floats: the 8 lanes of a write phase hit 8 bank
+    // groups) in its own 18 KB, then every lane stores 16 bytes of a 128-byte run of one token.
     __builtin_amdgcn_s_barrier();  // nobody's copies are still landing in what becomes another wavefront's block
     asm volatile("" ::: "memory");
-    constexpr uint32_t EP_LD = 68;
-    float *blk = reinterpret_cast<float *>(plds) + wave * (64 * EP_LD);
-    static_assert(8 * 64 * EP_LD * 4 <= P_LDS_BYTES, "the eight blocks fit");
+    constexpr uint32_t EP_LD = 36;
+    float *blk = reinterpret_cast<float *>(plds) + wave * (PN * EP_LD);
+    static_assert(8 * PN * EP_LD * 4 <= P_LDS_BYTES, "the eight blocks fit");
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int jj = 0; jj < 4; jj++)
+        for (int jj = 0; jj < 8; jj++)
             *reinterpret_cast<f32x4 *>(blk + (jj * 16 + l16) * EP_LD + i * 16 + kg * 4) = acc[i][jj];
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own writes, own reads
     const bool vec_ok = (rows & 3u) == 0 && (((uintptr_t)(partial ? partial : out)) & 15u) == 0;
-    const uint32_t rc = (lane & 15u) * 4, r = row0 + wm + rc;
+    const uint32_t rc = (lane & 7u) * 4, r = row0 + wm + rc;
 #pragma unroll 4
     for (int it = 0; it < 16; it++) {
-        const uint32_t tl = it * 4 + (lane >> 4), tok = tok0 + wn + tl;
+        const uint32_t tl = it * 8 + (lane >> 3), tok = tok0 + tl;
         if (tok >= seq) continue;
         f32x4 v = *reinterpret_cast<const f32x4 *>(blk + tl * EP_LD + rc);
         float *o = partial ? partial + ((size_t)blockIdx.z * seq + tok) * rows + r : out + (size_t)tok * rows + r;
