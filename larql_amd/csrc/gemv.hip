@@ -1300,6 +1300,12 @@ __device__ __forceinline__ void run_q4k_batch(const GemvJob &j, uint32_t tile_a,
 constexpr int kQ8Stages = 3;
 constexpr int kQ8BatchTiles = 4;
 constexpr int kQ8MaxWaves = 10;
+constexpr int kQ8MaxPasses = 2;  // columns per wavefront (both columns' activations stay in registers): K <= 5120
+// wavefronts that work on a row of `cpr` 256-element columns (0: the row is too long for this kernel)
+__host__ __device__ inline uint32_t q8_mfma_waves(uint64_t cpr) {
+    if (cpr == 0 || cpr > (uint64_t)kQ8MaxWaves * kQ8MaxPasses) return 0;
+    return cpr <= (uint64_t)kQ8MaxWaves ? (uint32_t)cpr : (uint32_t)((cpr + 1) / 2);
+}
 constexpr uint32_t kQ8RowBytes = 8 * 34;             // one column of one row
 constexpr uint32_t kQ8TileBytes = 16 * kQ8RowBytes;  // 4352
 
@@ -1347,15 +1353,16 @@ __device__ __forceinline__ Q8Col q8_mfma_setup_col(const float *x, uint32_t c, u
 }
 
 __device__ __forceinline__ void run_q8_0_mfma(const GemvJob &j, uint32_t tile_a, uint32_t tile_b, uint8_t *lds, uint32_t &parity) {
-    constexpr int NS = kQ8Stages, R = kQ8BatchTiles;
+    constexpr int NS = kQ8Stages, R = kQ8BatchTiles, NP = kQ8MaxPasses;
     const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t nw_launch = blockDim.x >> 6;
     const uint32_t jr = lane & 15u, kq = lane >> 4;
-    const uint32_t nwj = j.rpp, PW = nwj * 4;
+    const uint32_t nwj = j.rpp, cpr = j.cpr, PW = nwj * 4;
     const uint32_t rows = (uint32_t)j.rows, row_bytes = (uint32_t)j.row_bytes;
     uint8_t *ring = lds + wv * (NS * kQ8TileBytes);
     float *part = reinterpret_cast<float *>(lds + nw_launch * (NS * kQ8TileBytes));
-    const bool working = wv < nwj;
+    const uint32_t np = wv < nwj ? (cpr - wv + nwj - 1) / nwj : 0;  // columns wv, wv + nwj of this wavefront
+    const bool working = np >= 1;
 
     // lane's pieces of a wave-tile in 16-byte units u = row*17 + piece: four full loads, then 256 B dword by dword
     uint32_t rw[5], ow[5], off[5];
@@ -1368,12 +1375,13 @@ __device__ __forceinline__ void run_q8_0_mfma(const GemvJob &j, uint32_t tile_a,
     }
     const uint8_t *wcol = j.w + (size_t)wv * kQ8RowBytes;
     const uint32_t nt = tile_b - tile_a;
-    uint32_t it_tile = tile_a, n_issue = 0;
+    // issue cursor: wave-tiles in the order they are consumed (tile, then column pass: the workgroup reads whole rows)
+    uint32_t it_tile = tile_a, it_p = 0, n_issue = 0;
     auto issue = [&]() {
-        const uint32_t rb = min(it_tile, tile_b - 1) * 16;
+        const uint32_t rb = min(it_tile, tile_b - 1) * 16;  // past the end: the last tile again (uniform load counts)
         uint8_t *lp = ring + (n_issue % NS) * kQ8TileBytes;
         // wave-uniform 64-bit base + per-lane 32-bit offset; only a ragged last tile recomputes the offsets
-        const uint8_t *gp = wcol + (size_t)rb * row_bytes;
+        const uint8_t *gp = wcol + (size_t)it_p * nwj * kQ8RowBytes + (size_t)rb * row_bytes;
         uint32_t a[5];
 #pragma unroll
         for (int q = 0; q < 5; q++) a[q] = off[q];
@@ -1387,21 +1395,31 @@ __device__ __forceinline__ void run_q8_0_mfma(const GemvJob &j, uint32_t tile_a,
             __builtin_amdgcn_global_load_lds((g_vp)(gp + a[q]), (lds_vp)(lp + q * 1024), 16, 0, 0);
         __builtin_amdgcn_global_load_lds((g_vp)(gp + a[4]), (lds_vp)(lp + 4096), 4, 0, 0);
         n_issue++;
-        if (it_tile < tile_b) it_tile++;
+        if (it_tile < tile_b && ++it_p == np) { it_p = 0; it_tile++; }
     };
     if (working)
         for (int s = 0; s < NS - 1; s++) issue();
 
-    Q8Col col;
-    Q4kOp xm[8];
-    if (working) {
-        col = q8_mfma_setup_col(j.x, wv, lane);
-        const uint32_t my_g = jr >> 2, cl = (jr >> 1) & 1u;
+    float colk[NP];
+    Q4kOp xm[NP][8];
 #pragma unroll
-        for (int g = 0; g < 4; g++) {
-            const bool mine = my_g == (uint32_t)g && (kq >> 1) == cl;
+    for (int p = 0; p < NP; p++) {
+        colk[p] = 0.f;
+        if ((uint32_t)p < np) {
+            const Q8Col col = q8_mfma_setup_col(j.x, wv + nwj * p, lane);
+            colk[p] = col.k;
+            const uint32_t my_g = jr >> 2, cl = (jr >> 1) & 1u;
 #pragma unroll
-            for (int q = 0; q < 4; q++) { xm[2 * g].u[q] = mine ? col.xa[q] : 0u; xm[2 * g + 1].u[q] = mine ? col.xb[q] : 0u; }
+            for (int g = 0; g < 4; g++) {
+                const bool mine = my_g == (uint32_t)g && (kq >> 1) == cl;
+#pragma unroll
+                for (int q = 0; q < 4; q++) { xm[p][2 * g].u[q] = mine ? col.xa[q] : 0u; xm[p][2 * g + 1].u[q] = mine ? col.xb[q] : 0u; }
+            }
+        } else {
+#pragma unroll
+            for (int g = 0; g < 8; g++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) xm[p][g].u[q] = 0u;
         }
     }
     // this lane's 16 codes of block pair g start at byte (2g + kq/2)*34 + 2 + 16*(kq%2) of its row: the aligned
@@ -1415,32 +1433,39 @@ __device__ __forceinline__ void run_q8_0_mfma(const GemvJob &j, uint32_t tile_a,
         const uint32_t nbt = min((uint32_t)R, nt - tb);
         if (working) {
             for (uint32_t tl = 0; tl < nbt; tl++) {
-                issue();
-                LARQL_WAIT_VMCNT(5 * (NS - 1));
-                asm volatile("" ::: "memory");
-                const uint8_t *sp = ring + (n_use % NS) * kQ8TileBytes + jr * kQ8RowBytes;
-                n_use++;
-                i32x4 Da = {0, 0, 0, 0}, Db = {0, 0, 0, 0};
+                float racc = 0.f;
 #pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const uint32_t *wp = reinterpret_cast<const uint32_t *>(sp + g * 68 + code_dw);
-                    const uint32_t w0 = wp[0], w1 = wp[1], w2 = wp[2], w3 = wp[3], w4 = wp[4];
-                    Q4kOp b;
-                    b.u[0] = __builtin_amdgcn_alignbit(w1, w0, code_sh); b.u[1] = __builtin_amdgcn_alignbit(w2, w1, code_sh);
-                    b.u[2] = __builtin_amdgcn_alignbit(w3, w2, code_sh); b.u[3] = __builtin_amdgcn_alignbit(w4, w3, code_sh);
-                    Da = __builtin_amdgcn_mfma_i32_16x16x64_i8(xm[2 * g].v, b.v, Da, 0, 0, 0);
-                    Db = __builtin_amdgcn_mfma_i32_16x16x64_i8(xm[2 * g + 1].v, b.v, Db, 0, 0, 0);
+                for (int p = 0; p < NP; p++) {
+                    if ((uint32_t)p < np) {
+                        issue();
+                        LARQL_WAIT_VMCNT(5 * (NS - 1));
+                        asm volatile("" ::: "memory");
+                        const uint8_t *sp = ring + (n_use % NS) * kQ8TileBytes + jr * kQ8RowBytes;
+                        n_use++;
+                        i32x4 Da = {0, 0, 0, 0}, Db = {0, 0, 0, 0};
+#pragma unroll
+                        for (int g = 0; g < 4; g++) {
+                            const uint32_t *wp = reinterpret_cast<const uint32_t *>(sp + g * 68 + code_dw);
+                            const uint32_t w0 = wp[0], w1 = wp[1], w2 = wp[2], w3 = wp[3], w4 = wp[4];
+                            Q4kOp b;
+                            b.u[0] = __builtin_amdgcn_alignbit(w1, w0, code_sh); b.u[1] = __builtin_amdgcn_alignbit(w2, w1, code_sh);
+                            b.u[2] = __builtin_amdgcn_alignbit(w3, w2, code_sh); b.u[3] = __builtin_amdgcn_alignbit(w4, w3, code_sh);
+                            Da = __builtin_amdgcn_mfma_i32_16x16x64_i8(xm[p][2 * g].v, b.v, Da, 0, 0, 0);
+                            Db = __builtin_amdgcn_mfma_i32_16x16x64_i8(xm[p][2 * g + 1].v, b.v, Db, 0, 0, 0);
+                        }
+                        // this lane's pair is g = kq: Da = [b0.l0, b0.l1, b1.l0, b1.l1], Db = [b0.l2, b0.l3, b1.l2, b1.l3]
+                        float dot0 = __builtin_fmaf((float)Da[0], 128.f, (float)Da[1]);
+                        float dot1 = __builtin_fmaf((float)Da[2], 128.f, (float)Da[3]);
+                        dot0 = __builtin_fmaf(dot0, 128.f, (float)Db[0]);
+                        dot1 = __builtin_fmaf(dot1, 128.f, (float)Db[2]);
+                        dot0 = __builtin_fmaf(dot0, 128.f, (float)Db[1]) * colk[p];
+                        dot1 = __builtin_fmaf(dot1, 128.f, (float)Db[3]) * colk[p];
+                        const float d0 = half_bits_to_float(*reinterpret_cast<const uint16_t *>(sp + kq * 68));
+                        const float d1 = half_bits_to_float(*reinterpret_cast<const uint16_t *>(sp + kq * 68 + 34));
+                        racc += d0 * dot0 + d1 * dot1;
+                    }
                 }
-                // this lane's pair is g = kq: Da = [b0.l0, b0.l1, b1.l0, b1.l1], Db = [b0.l2, b0.l3, b1.l2, b1.l3]
-                float dot0 = __builtin_fmaf((float)Da[0], 128.f, (float)Da[1]);
-                float dot1 = __builtin_fmaf((float)Da[2], 128.f, (float)Da[3]);
-                dot0 = __builtin_fmaf(dot0, 128.f, (float)Db[0]);
-                dot1 = __builtin_fmaf(dot1, 128.f, (float)Db[2]);
-                dot0 = __builtin_fmaf(dot0, 128.f, (float)Db[1]) * col.k;
-                dot1 = __builtin_fmaf(dot1, 128.f, (float)Db[3]) * col.k;
-                const float d0 = half_bits_to_float(*reinterpret_cast<const uint16_t *>(sp + kq * 68));
-                const float d1 = half_bits_to_float(*reinterpret_cast<const uint16_t *>(sp + kq * 68 + 34));
-                pb[(tl * 16 + jr) * PW + wv * 4 + kq] = d0 * dot0 + d1 * dot1;
+                pb[(tl * 16 + jr) * PW + wv * 4 + kq] = racc;
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -1904,7 +1929,7 @@ uint32_t gemv_batch_capacity(int kind, uint64_t k) {
 static int g_q8_mfma = getenv("LARQL_HIP_Q8_MFMA") ? atoi(getenv("LARQL_HIP_Q8_MFMA")) : 1;
 
 int gemv_effective_kind(const GemvJob &j) {
-    if (j.kind == KIND_Q8_0 && g_q8_mfma && j.k >= 256 && j.k % 256 == 0 && j.k / 256 <= (uint64_t)kQ8MaxWaves && j.rows < 0x7FFFFFF0ull)
+    if (j.kind == KIND_Q8_0 && g_q8_mfma && j.k >= 256 && j.k % 256 == 0 && q8_mfma_waves(j.k / 256) != 0 && j.rows < 0x7FFFFFF0ull)
         return KIND_Q8_0_MFMA;
     if (j.kind == KIND_BF16 && j.batch >= 2) return KIND_BF16_MFMA;
     if (j.kind == KIND_Q4K && j.batch >= 2) return KIND_Q4K_BATCH;
@@ -1920,9 +1945,10 @@ int gemv_effective_kind(const GemvJob &j) {
 bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
     if (j.kind == KIND_Q8_0_MFMA) {
         const uint64_t cpr = j.k / 256;
-        if (j.k % 256 != 0 || cpr == 0 || cpr * 64 > threads) return false;
+        const uint32_t nw = q8_mfma_waves(cpr);
+        if (j.k % 256 != 0 || nw == 0 || nw * 64 > threads) return false;
         j.cpr = (uint32_t)cpr;
-        j.rpp = (uint32_t)cpr;
+        j.rpp = nw;  // wavefronts that work on this job
         j.row_bytes = (j.k / 32) * 34;
         const uint64_t tiles = (j.rows + 15) / 16;
         if (tiles * cpr > 0x7FFFFFFFull) return false;
@@ -2015,7 +2041,16 @@ bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
 }
 
 uint32_t gemv_pick_threads(const GemvJob *jobs, size_t n) {
-    if (n > 0 && (jobs[0].kind == KIND_Q4K_BATCH || jobs[0].kind == KIND_Q8_0_MFMA)) {
+    if (n > 0 && jobs[0].kind == KIND_Q8_0_MFMA) {
+        uint32_t nw = 0;
+        for (size_t i = 0; i < n; i++) {
+            const uint32_t w = q8_mfma_waves(jobs[i].k / 256);
+            if (w == 0) return 0;
+            nw = std::max(nw, w);
+        }
+        return nw * 64;
+    }
+    if (n > 0 && jobs[0].kind == KIND_Q4K_BATCH) {
         uint64_t nw = 0;
         for (size_t i = 0; i < n; i++) nw = std::max<uint64_t>(nw, jobs[i].k / 256);
         return nw <= (uint64_t)kQ4kMaxWaves ? (uint32_t)nw * 64 : 0;

@@ -164,7 +164,8 @@ def test_q6k_matvec_shape_rules(be):
 
 
 # ------------------------------------------------------------------ Q8_0
-@pytest.mark.parametrize("n,k", [(4099, 2560), (64, 10240), (9, 128), (1000, 2048), (17, 256), (333, 1792), (48, 2816)])
+@pytest.mark.parametrize("n,k", [(4099, 2560), (64, 10240), (9, 128), (1000, 2048), (17, 256), (333, 1792), (48, 2816),
+                                 (531, 3840), (2050, 4096), (77, 5120), (40, 5376)])   # two column passes per wavefront; odd column count; just above
 def test_q8_0_gemv_matches_oracle(be, n, k):
     w, x = weights(n + k, n, k)
     w[0, :32] *= 1e-5
