@@ -175,10 +175,10 @@ def _cpu_time(fn, seconds):
     return float(np.median(times)), len(times)
 
 
-def _emit(metric, value, unit, ms, steps, warmup, config, roofline, cpu, higher=True):
+def _emit(metric, value, unit, ms, steps, warmup, config, roofline, cpu, higher=True, dtype="f32"):
     print(json.dumps({"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
                       "ms_per_step": round(ms, 5), "higher_is_better": higher, "scaling": "weak", "vs_baseline": None,
-                      "dtype": "f32", "data": "synthetic", "config": config, "roofline": roofline, "cpu_baseline": cpu}))
+                      "dtype": dtype, "data": "synthetic", "config": config, "roofline": roofline, "cpu_baseline": cpu}))
 
 
 def run_c1(be, fmt, args):
@@ -372,6 +372,64 @@ def run_c5(be, fmt, args):
           cpu)
 
 
+def run_q8k(be, fmt, args):
+    """The Gemma-3-4B decode stack through the Q8_K-activation integer path (quantize_x_to_q8k + q4k_q8k_matvec), the
+    path the reference's CPU decode runs: 34 layers x 7 Q4_K matvecs, one launch, activations quantised on the device."""
+    O = _oracle()
+    layers = args.layers
+    shapes = [("q", 2048, 2560), ("k", 1024, 2560), ("v", 1024, 2560), ("o", 2560, 2048), ("gate", 10240, 2560), ("up", 10240, 2560),
+              ("down", 2560, 10240)]
+    acts = {}
+    for k in (2560, 2048, 10240):
+        x = be.malloc(k * 4 + 64)
+        be.dev_fill_normal(x, k, 0x5EED0600 + k, 1.0)
+        q = be.malloc(be.q8k_bytes(k) + 64)
+        assert be.dev_quantize_x_to_q8k(x, k, q)
+        acts[k] = (x, q)
+    tmp = be.malloc(10240 * 2560 * 4)
+    jobs, keep = [], []
+    algo = 0
+    for layer in range(layers):
+        for i, (name, rows, k) in enumerate(shapes):
+            w = be.malloc(q4k_bytes(rows, k) + 64)
+            be.dev_fill_normal(tmp, rows * k, 0x5EED0610 + layer * 8 + i, 0.02)
+            be.dev_quantize_q4_k(tmp, rows * k, w)
+            o = be.malloc(rows * 4 + 64)
+            jobs.append((fmt.FMT_Q4_K_Q8K, w, None, acts[k][1], o, rows, k))
+            keep.append((w, o, rows, k))
+            algo += q4k_bytes(rows, k) + be.q8k_bytes(k) + 4 * rows
+    plan = be.plan_create(jobs)
+    assert plan is not None and be.plan_launch_count(plan) == 1
+    be.plan_run(plan); be.synchronize()
+    # bit-exact against the oracle on two matvecs of layer 0 (the reference's SIMD kernels equal its scalar one bit for bit)
+    exact = True
+    cpu_ops = []
+    for idx in (1, 6):
+        w, o, rows, k = keep[idx]
+        wb, xv = be.d2h(w, q4k_bytes(rows, k), np.uint8), be.d2h(acts[k][0], k, np.float32)
+        a = O.quantize_x_to_q8k(xv)
+        dev_a = be.d2h(acts[k][1], be.q8k_bytes(k), np.uint8)
+        exact &= bool(np.array_equal(dev_a[:k].view(np.int8), a[0]) and np.array_equal(dev_a[k:k + k // 64].view(np.float32), a[1]))
+        want = O.q4k_q8k_matvec(wb, *a, rows, k)
+        exact &= bool(np.array_equal(be.d2h(o, rows, np.float32).view(np.uint32), want.view(np.uint32)))
+        cpu_ops.append((wb, a, rows, k))
+    assert exact
+    ms = _timeit(be, lambda: be.plan_run(plan), args.steps)
+    ms_q = _timeit(be, lambda: be.dev_quantize_x_to_q8k(acts[10240][0], 10240, acts[10240][1]), args.steps)
+    gbs = algo / ms / 1e6
+    med, n = _cpu_time(lambda: [O.q4k_q8k_matvec(wb, *a, rows, k) for wb, a, rows, k in cpu_ops], args.cpu_seconds)
+    cpu_bytes = sum(q4k_bytes(rows, k) for _, _, rows, k in cpu_ops)
+    _emit("Q4_K x Q8_K decode matvec stack HBM GB/s (integer-dot path)", round(gbs, 1), "GB/s", ms, args.steps, 2,
+          {"workload": f"Gemma-3-4B decode stack, batch 1, {layers} layers x 7 Q4_K matvecs against Q8_K activations, one launch",
+           "matvecs_per_step": len(jobs), "algorithmic_bytes_per_step": algo, "bit_exact_vs_oracle": exact,
+           "quantize_x_to_q8k_us_10240": round(ms_q * 1e3, 2)},
+          {"kernel": "gemv_q4k_q8k", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+           "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+          {"value": round(cpu_bytes / med / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+           "sample": f"k 1024x2560 and down 2560x10240 of layer 0 (q4k_q8k_matvec_scalar restated), median of {n}"},
+          dtype="i32")
+
+
 def read_traffic():
     """HBM bytes per launch of the dominant kernel from the committed rocprof PMC summary, if any."""
     path = os.path.join(ROOT, "profiles", "gemv_q4k_c2_stack.pmc.txt")
@@ -393,7 +451,7 @@ def main():
     ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"],
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "q8k"],
                     help="c2 (default) is the headline decode stack; the others are BASELINE's remaining configs")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run the plain 16-byte copy kernel on 1 GiB three times (known size, for scaling "
@@ -427,7 +485,7 @@ def main():
                           "read_only_GBps": round(n / ms_r / 1e6, 1)}))
         return
     if args.workload != "c2":
-        {"c1": run_c1, "c3": run_c3, "c4": run_c4, "c5": run_c5}[args.workload](be, fmt, args)
+        {"c1": run_c1, "c3": run_c3, "c4": run_c4, "c5": run_c5, "q8k": run_q8k}[args.workload](be, fmt, args)
         return
     stack = Stack(be, fmt, layers=args.layers)
 

@@ -53,7 +53,11 @@ enum {
     /* ggml's 34-byte Q8_0 block (f16 scale inside the block).  Not the trait's
      * QuantFormat::Q8_0, which is int8 codes + external f32 scales
      * (larql-compute/src/cpu/kquant_gemv.rs:1-12). */
-    LARQL_FMT_GGML_Q8_0 = 100
+    LARQL_FMT_GGML_Q8_0 = 100,
+    /* Q4_K weights against a Q8_K activation (the integer-dot decode path,
+     * larql-compute/src/cpu/ops/q4k_q8k_dot): in a device-tier job `x` is the
+     * activation in the layout larql_hip_dev_quantize_x_to_q8k writes. */
+    LARQL_FMT_Q4_K_Q8K = 101
 };
 
 /* Capability — larql-compute/src/backend/capability.rs:22-102 (the ones this
@@ -111,6 +115,19 @@ int larql_hip_q4k_matvec(larql_hip_ctx *ctx, const uint8_t *q4k, size_t q4k_len,
  * path indexes out of range there); zero dims write zeros. */
 int larql_hip_q6k_matvec(larql_hip_ctx *ctx, const uint8_t *q6k, size_t q6k_len,
                          const float *x, size_t x_len, size_t num_rows, size_t hidden, float *out);
+/* quantize_x_to_q8k — larql-compute/src/cpu/ops/q4k_q8k_dot/q8k_activation.rs:84-109
+ * (Q8KActivation { qs, d, sums }): n % 256 == 0, qs[n], d[n/256], sums[n/32].
+ * Bit-exact with the reference. */
+int larql_hip_quantize_x_to_q8k(larql_hip_ctx *ctx, const float *x, size_t n, int8_t *qs, float *d, int16_t *sums);
+/* q4k_q8k_matvec_into / q4k_q8k_matvec_parallel with format "Q4_K" —
+ * cpu/ops/q4k_q8k_dot/dispatch.rs:15-148; value and bits of q4k_q8k_matvec_scalar
+ * (q4k_scalar.rs:15-84), which every SIMD kernel of the reference equals bit for
+ * bit and so does this one.  Shape rule KernelShapeError::check
+ * (cpu/ops/kernel_shape.rs:47-75): out_len == rows, qs_len == cols, cols % 256 == 0,
+ * q4k_len >= rows*(cols/256)*144, else REFUSED_SHAPE with `out` untouched; zero
+ * dims write zeros.  cols <= 10240 on this backend (longer: UNSUPPORTED). */
+int larql_hip_q4k_q8k_matvec(larql_hip_ctx *ctx, const uint8_t *q4k, size_t q4k_len, const int8_t *qs, size_t qs_len,
+                             const float *d, const int16_t *sums, size_t num_rows, size_t cols, float *out, size_t out_len);
 /* QuantMatVec::q4k_dual_matvec — quant_matvec.rs:287-296; q4_common/dual.rs:22-167. */
 int larql_hip_q4k_dual_matvec(larql_hip_ctx *ctx, const uint8_t *q4k_a, size_t a_len,
                               const uint8_t *q4k_b, size_t b_len,
@@ -312,6 +329,12 @@ int larql_hip_dev_f32_to_bf16(larql_hip_ctx *ctx, const float *src, size_t n, ui
 /* quantize_q4_0 / quantize_to_q8 — q4_common/quantize.rs:6-69. */
 int larql_hip_dev_quantize_q4_0(larql_hip_ctx *ctx, const float *src, size_t n, uint8_t *dst);
 int larql_hip_dev_quantize_to_q8(larql_hip_ctx *ctx, const float *src, size_t n, int8_t *q8, float *scales);
+/* quantize_x_to_q8k on the device (q8k_activation.rs:84-109).  `q8k` receives the
+ * activation in one buffer of larql_hip_q8k_bytes(n) bytes: n int8 codes, then
+ * n/256 f32 scales, then n/32 i16 sub-block sums; that buffer is the `x` of a
+ * LARQL_FMT_Q4_K_Q8K job.  Both pointers 16-byte aligned. */
+size_t larql_hip_q8k_bytes(size_t n);
+int larql_hip_dev_quantize_x_to_q8k(larql_hip_ctx *ctx, const float *x, size_t n, void *q8k);
 /* Synthetic N(0, sigma) data for benchmarks: element i of stream `seed` is a
  * fixed function of (seed, i) (sum of twelve 21-bit uniforms from a
  * splitmix64 counter stream: exact integer arithmetic, so host and device

@@ -121,6 +121,27 @@ class HipBackend:
         ok = self._some(lib.larql_hip_q6k_matvec(self._h, _ptr(w), w.size, _ptr(xv), xv.size, num_rows, hidden, _ptr(out)))
         return out if ok else None
 
+    def quantize_x_to_q8k(self, x):
+        """quantize_x_to_q8k (cpu/ops/q4k_q8k_dot/q8k_activation.rs:84-109) -> (qs int8, d f32, sums int16) or None."""
+        xv = _f32(x)
+        n = xv.size
+        qs, d, sums = np.empty(n, np.int8), np.empty(n // 256, np.float32), np.empty(n // 32, np.int16)
+        ok = self._some(lib.larql_hip_quantize_x_to_q8k(self._h, _ptr(xv), n, _ptr(qs), _ptr(d), _ptr(sums)))
+        return (qs, d, sums) if ok else None
+
+    def q4k_q8k_matvec(self, q4k, qs, d, sums, num_rows: int, cols: int, out_len: Optional[int] = None) -> Optional[np.ndarray]:
+        """q4k_q8k_matvec_into (cpu/ops/q4k_q8k_dot/dispatch.rs:15-51): Q4_K rows against a Q8_K activation."""
+        w = _u8(q4k)
+        qs = np.ascontiguousarray(qs, dtype=np.int8).reshape(-1)
+        d = _f32(d)
+        sums = np.ascontiguousarray(sums, dtype=np.int16).reshape(-1)
+        if d.size * 256 != qs.size or sums.size * 32 != qs.size:
+            return None
+        out = np.empty(num_rows if out_len is None else out_len, np.float32)
+        ok = self._some(lib.larql_hip_q4k_q8k_matvec(self._h, _ptr(w), w.size, _ptr(qs), qs.size, _ptr(d), _ptr(sums), num_rows, cols,
+                                                     _ptr(out), out.size))
+        return out if ok else None
+
     def q4k_dual_matvec(self, q4k_a, q4k_b, x, num_rows: int, hidden: int):
         a, b, x = _u8(q4k_a), _u8(q4k_b), _f32(x)
         oa, ob = np.empty(num_rows, np.float32), np.empty(num_rows, np.float32)
@@ -369,6 +390,12 @@ class HipBackend:
 
     def dev_quantize_to_q8(self, src: int, n: int, q8: int, scales: int) -> bool:
         return self._some(lib.larql_hip_dev_quantize_to_q8(self._h, src, n, q8, scales))
+
+    def q8k_bytes(self, n: int) -> int:
+        return int(lib.larql_hip_q8k_bytes(n))
+
+    def dev_quantize_x_to_q8k(self, x: int, n: int, q8k: int) -> bool:
+        return self._some(lib.larql_hip_dev_quantize_x_to_q8k(self._h, x, n, q8k))
 
     def dev_fill_normal(self, dst: int, n: int, seed: int, sigma: float) -> bool:
         return self._some(lib.larql_hip_dev_fill_normal(self._h, dst, n, seed, sigma))

@@ -130,6 +130,7 @@ int kind_of_format(int format) {
         case LARQL_FMT_Q4_K: case LARQL_FMT_Q4_KF: return KIND_Q4K;
         case LARQL_FMT_GGML_Q8_0: return KIND_Q8_0;
         case LARQL_FMT_Q6_K: return KIND_Q6K;
+        case LARQL_FMT_Q4_K_Q8K: return KIND_Q4K_Q8K;
         case LARQL_FMT_MXFP4: return KIND_MXFP4;
         case LARQL_FMT_Q4_0: return KIND_Q4_0;
         case LARQL_FMT_BF16: return KIND_BF16;
@@ -213,10 +214,10 @@ std::vector<std::vector<GemvJob>> group_by_kind(const std::vector<GemvJob> &jobs
     std::vector<GemvJob> jobs(jobs_in);
     for (GemvJob &j : jobs) j.kind = gemv_effective_kind(j);  // Q4_K rows the matrix-core kernel takes get their own launch
     std::vector<std::vector<GemvJob>> groups;
-    bool done[13] = {false, false, false, false, false, false, false, false, false, false, false, false, false};
+    bool done[14] = {false, false, false, false, false, false, false, false, false, false, false, false, false, false};
     for (size_t i = 0; i < jobs.size(); i++) {
         const int kind = jobs[i].kind;
-        if (jobs[i].rows == 0 || kind < 0 || kind > 12 || done[kind]) continue;
+        if (jobs[i].rows == 0 || kind < 0 || kind > 13 || done[kind]) continue;
         done[kind] = true;
         std::vector<GemvJob> live;
         for (size_t t = i; t < jobs.size(); t++)
@@ -447,6 +448,59 @@ int larql_hip_q6k_matvec(larql_hip_ctx *c, const uint8_t *q6k, size_t q6k_len, c
     if (num_rows == 0 || hidden == 0) { for (size_t i = 0; i < num_rows; i++) out[i] = 0.0f; return LARQL_OK; }
     if (!q6k || !x) return LARQL_E_ARG;
     return host_matvec_multi(c, KIND_Q6K, 1, &q6k, &need, nullptr, nullptr, &num_rows, hidden, x, x_len * 4, &out);
+}
+
+// ---- Q8_K-activation integer path (larql-compute/src/cpu/ops/q4k_q8k_dot) --------------------------------
+
+size_t larql_hip_q8k_bytes(size_t n) { return q8k_bytes(n); }
+
+int larql_hip_dev_quantize_x_to_q8k(larql_hip_ctx *c, const float *x, size_t n, void *q8k) {
+    if (!c) return LARQL_E_ARG;
+    if (n % 256 != 0) return fail(c, LARQL_REFUSED_SHAPE, "quantize_x_to_q8k: length must be a multiple of 256");
+    if (n == 0) return LARQL_OK;
+    if (!x || !q8k || ((uintptr_t)x & 15) || ((uintptr_t)q8k & 15)) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, quantize_x_to_q8k_launch(c->stream, x, n, (uint8_t *)q8k));
+    return LARQL_OK;
+}
+
+int larql_hip_quantize_x_to_q8k(larql_hip_ctx *c, const float *x, size_t n, int8_t *qs, float *d, int16_t *sums) {
+    if (!c) return LARQL_E_ARG;
+    if (n % 256 != 0) return fail(c, LARQL_REFUSED_SHAPE, "quantize_x_to_q8k: length must be a multiple of 256");
+    if (n == 0) return LARQL_OK;
+    if (!x || !qs || !d || !sums) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    HIPCHECK(c, hipSetDevice(c->device));
+    int rc = upload(c, c->x, x, n * 4);
+    if (rc) return rc;
+    rc = ensure(c, c->misc, q8k_bytes(n) + 64);
+    if (rc) return rc;
+    Submission sub(c);
+    HIPCHECK(c, quantize_x_to_q8k_launch(c->stream, (const float *)c->x.p, n, (uint8_t *)c->misc.p));
+    const uint8_t *p = (const uint8_t *)c->misc.p;
+    HIPCHECK(c, hipMemcpyAsync(qs, p, n, hipMemcpyDeviceToHost, c->stream));
+    HIPCHECK(c, hipMemcpyAsync(d, p + n, (n / 256) * 4, hipMemcpyDeviceToHost, c->stream));
+    HIPCHECK(c, hipMemcpyAsync(sums, p + n + (n / 256) * 4, (n / 32) * 2, hipMemcpyDeviceToHost, c->stream));
+    return sub.finish();
+}
+
+int larql_hip_q4k_q8k_matvec(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, const int8_t *qs, size_t qs_len, const float *d,
+                             const int16_t *sums, size_t num_rows, size_t cols, float *out, size_t out_len) {
+    if (!c || (!out && out_len)) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (!q4k_shape_ok(out_len, num_rows, qs_len, cols, q4k_len))
+        return fail(c, LARQL_REFUSED_SHAPE, "q4k_q8k_matvec: refused operands: out.len() %zu for %zu rows, activation length %zu for %zu cols, %zu weight bytes",
+                    out_len, num_rows, qs_len, cols, q4k_len);
+    if (num_rows == 0 || cols == 0) { for (size_t i = 0; i < out_len; i++) out[i] = 0.0f; return LARQL_OK; }
+    if (!q4k || !qs || !d || !sums) return LARQL_E_ARG;
+    if (cols / 256 > 40) return fail(c, LARQL_UNSUPPORTED, "q4k_q8k_matvec: rows longer than 10240 have no kernel");
+    // the activation travels in its device layout: [codes | scales | sums]
+    std::vector<uint8_t> packed(q8k_bytes(cols));
+    memcpy(packed.data(), qs, cols);
+    memcpy(packed.data() + cols, d, (cols / 256) * 4);
+    memcpy(packed.data() + cols + (cols / 256) * 4, sums, (cols / 32) * 2);
+    const size_t need = (cols / 256) * 144 * num_rows;
+    return host_matvec_multi(c, KIND_Q4K_Q8K, 1, &q4k, &need, nullptr, nullptr, &num_rows, cols, (const float *)packed.data(), packed.size(), &out);
 }
 
 int larql_hip_q4k_dual_matvec(larql_hip_ctx *c, const uint8_t *a, size_t a_len, const uint8_t *b, size_t b_len,
@@ -901,7 +955,9 @@ static int dev_job_from_public(larql_hip_ctx *c, const larql_hip_matvec_job &p, 
     if (kind < 0) return fail(c, LARQL_UNSUPPORTED, "matvec: format %d has no kernel", p.format);
     if (kind == KIND_MXFP4 && !p.aux) return fail(c, LARQL_E_ARG, "matvec: MXFP4 needs the scale stream");
     if (kind == KIND_Q4_0) return fail(c, LARQL_UNSUPPORTED, "matvec batch: Q4_0 goes through larql_hip_dev_matvec");
-    if ((kind == KIND_Q4K || kind == KIND_Q6K) && p.k % 256 != 0) return fail(c, LARQL_REFUSED_SHAPE, "matvec: k not a multiple of 256");
+    if ((kind == KIND_Q4K || kind == KIND_Q6K || kind == KIND_Q4K_Q8K) && p.k % 256 != 0)
+        return fail(c, LARQL_REFUSED_SHAPE, "matvec: k not a multiple of 256");
+    if (kind == KIND_Q4K_Q8K && p.k / 256 > 40) return fail(c, LARQL_UNSUPPORTED, "matvec: Q4_K x Q8_K rows longer than 10240 have no kernel");
     if (p.k % 32 != 0) return fail(c, LARQL_REFUSED_SHAPE, "matvec: k not a multiple of 32");
     jobs.push_back(make_job(kind, p.w, p.aux, p.x, p.out, p.rows, p.k));
     return LARQL_OK;

@@ -754,6 +754,158 @@ __device__ __forceinline__ void run_q4k_mfma(const GemvJob &j, uint32_t tile_a, 
 }
 
 // ---------------------------------------------------------------------------
+// Q4_K weights against a Q8_K activation (q4k_q8k_matvec_scalar, larql-compute/src/cpu/ops/q4k_q8k_dot/
+// q4k_scalar.rs:15-84): the activation is already int8, so one operand set replaces the four digit sets of the
+// f32 kernel.  A row m of the "A" operand is sub-block m (rows 8..15 are zero): its 32 codes sit in the k-slots
+// where "B" carries that sub-block's nibbles (slots 16kq+0..7 = low nibbles = sub-block 2g, 16kq+8..15 = high =
+// sub-block 2g+1), so after four MFMAs lane (row j, kq < 2) holds the eight exact integer dots of weight row j,
+// four per lane.  sum1 = sum sc*dot and sum2 = sum mn*bsum are formed in integers, the two halves meet by one
+// cross-lane add, and the reference's float expression d_w*d_y*sum1 - dmin_w*d_y*sum2 is evaluated once per
+// (row, super-block) without contraction.  Every column keeps its own partial and a row is summed by one lane
+// in super-block order: the result equals the reference's bit for bit.
+// All columns of a wavefront (up to 4) keep their operands in registers; tiles are walked column-innermost, so
+// the workgroup reads whole rows.
+// ---------------------------------------------------------------------------
+struct Q8kCol {
+    Q4kOp xm[4];      // operand of group g: this lane's 8 codes in the low or high k-slots if its row is sub-block 2g or 2g+1
+    uint32_t bs[2];   // the four i16 sub-block sums of this lane's half (4kq..4kq+3), packed
+    float dy;
+};
+
+__device__ __forceinline__ Q8kCol q8k_load_col(const uint8_t *q8k, uint32_t k, uint32_t c, uint32_t lane) {
+    const uint32_t r = lane & 15u, kq = lane >> 4;
+    const GLOBAL_AS uint8_t *base = (const GLOBAL_AS uint8_t *)q8k;
+    const u32x2 codes = *(const GLOBAL_AS u32x2 *)(base + (size_t)c * 256 + (r & 7u) * 32 + kq * 8);
+    const u32x2 sums = *(const GLOBAL_AS u32x2 *)(base + k + (k / 256) * 4 + (size_t)c * 16 + (kq & 1u) * 8);
+    Q8kCol col;
+    col.dy = *(const GLOBAL_AS float *)(base + k + (size_t)c * 4);
+    col.bs[0] = sums.x; col.bs[1] = sums.y;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        const bool lo = r == (uint32_t)(2 * g), hi = r == (uint32_t)(2 * g + 1);
+        col.xm[g].u[0] = lo ? codes.x : 0u; col.xm[g].u[1] = lo ? codes.y : 0u;
+        col.xm[g].u[2] = hi ? codes.x : 0u; col.xm[g].u[3] = hi ? codes.y : 0u;
+    }
+    return col;
+}
+
+// one wave-tile: 16 rows x one super-block; returns this (row, super-block)'s term in lanes kq == 0
+__device__ __forceinline__ float q4k_q8k_tile(const uint8_t *slot, const Q8kCol &col, uint32_t j, uint32_t kq) {
+#pragma clang fp contract(off)
+    const uint8_t *sp = slot + j * 144;
+    const u32x4 hdr = *reinterpret_cast<const u32x4 *>(sp);
+    u32x2 q[4];
+#pragma unroll
+    for (int g = 0; g < 4; g++) q[g] = *reinterpret_cast<const u32x2 *>(sp + 16 + 32 * g + 8 * kq);
+    i32x4 D = {0, 0, 0, 0};
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        Q4kOp b;
+        b.u[0] = q[g].x & 0x0F0F0F0Fu; b.u[1] = q[g].y & 0x0F0F0F0Fu;
+        b.u[2] = (q[g].x >> 4) & 0x0F0F0F0Fu; b.u[3] = (q[g].y >> 4) & 0x0F0F0F0Fu;
+        D = __builtin_amdgcn_mfma_i32_16x16x64_i8(col.xm[g].v, b.v, D, 0, 0, 0);
+    }
+    // D[i] = dot of sub-block 4kq + i (lanes kq >= 2 hold the zero rows: they compute with kq & 1 and are ignored)
+    const bool upper = (kq & 1u) != 0;
+    const uint32_t sc4 = upper ? ((hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u)) : (hdr.y & 0x3F3F3F3Fu);
+    const uint32_t mn4 = upper ? (((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u)) : (hdr.z & 0x3F3F3F3Fu);
+    // |dot| <= 32*15*127 and |bsum| <= 32*127: the products fit 24-bit multiplies
+    int s1 = __mul24((int)(sc4 & 0xFFu), D[0]) + __mul24((int)((sc4 >> 8) & 0xFFu), D[1]) +
+             __mul24((int)((sc4 >> 16) & 0xFFu), D[2]) + __mul24((int)(sc4 >> 24), D[3]);
+    const int b0 = (int)(int16_t)(col.bs[0] & 0xFFFFu), b1 = (int)col.bs[0] >> 16;
+    const int b2 = (int)(int16_t)(col.bs[1] & 0xFFFFu), b3 = (int)col.bs[1] >> 16;
+    int s2 = __mul24((int)(mn4 & 0xFFu), b0) + __mul24((int)((mn4 >> 8) & 0xFFu), b1) +
+             __mul24((int)((mn4 >> 16) & 0xFFu), b2) + __mul24((int)(mn4 >> 24), b3);
+    s1 += __shfl_xor(s1, 16);  // sub-blocks 0..3 + 4..7
+    s2 += __shfl_xor(s2, 16);
+    const float d_w = half_bits_to_float(hdr.x & 0xFFFFu), dmin_w = half_bits_to_float(hdr.x >> 16);
+    float t1 = d_w * col.dy;
+    t1 = t1 * (float)s1;
+    float t2 = dmin_w * col.dy;
+    t2 = t2 * (float)s2;
+    return t1 - t2;
+}
+
+// tiles [tile_a, tile_b) of one job; `parity` flips per batch (double-buffered partials)
+__device__ __forceinline__ void run_q4k_q8k(const GemvJob &j, uint32_t tile_a, uint32_t tile_b, uint8_t *lds, uint32_t &parity) {
+    constexpr int NS = kQ4kStages, R = kQ4kBatchTiles, NP = kQ4kMaxColPasses;
+    const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t nw_launch = blockDim.x >> 6;
+    const uint32_t jr = lane & 15u, kq = lane >> 4;
+    const uint32_t nwj = j.rpp, cpr = j.cpr, PW = cpr;  // one partial per (row, super-block)
+    const uint32_t rows = (uint32_t)j.rows, row_bytes = (uint32_t)j.row_bytes;
+    uint8_t *ring = lds + wv * (NS * kQ4kTileBytes);
+    float *part = reinterpret_cast<float *>(lds + nw_launch * (NS * kQ4kTileBytes));
+    const uint32_t np = wv < nwj ? (cpr - wv + nwj - 1) / nwj : 0;  // columns wv, wv+nwj, ... of this wavefront
+
+    const uint32_t u0 = lane, u1 = 64 + lane, u2 = 128 + (lane >> 2);
+    const uint32_t r0 = u0 / 9, r1 = u1 / 9, r2 = u2 / 9;
+    const uint32_t w0 = (u0 - r0 * 9) * 16, w1 = (u1 - r1 * 9) * 16, w2 = (u2 - r2 * 9) * 16 + (lane & 3u) * 4;
+    const uint32_t o0 = r0 * row_bytes + w0, o1 = r1 * row_bytes + w1, o2 = r2 * row_bytes + w2;
+    const uint8_t *wcol = j.w + (size_t)wv * 144;
+    const uint32_t nt = tile_b - tile_a;
+
+    // issue cursor: wave-tiles in the order they are consumed (tile, then column pass)
+    uint32_t it_tile = tile_a, it_p = 0, n_issue = 0;
+    auto issue = [&]() {
+        const uint32_t rb = min(it_tile, tile_b - 1) * 16;  // past the end: the last tile again (uniform load counts)
+        const uint8_t *gp = wcol + (size_t)it_p * nwj * 144 + (size_t)rb * row_bytes;
+        uint32_t a0 = o0, a1 = o1, a2 = o2;
+        if (rb + 16 > rows) {
+            const uint32_t lim = rows - 1 - rb;
+            a0 = min(r0, lim) * row_bytes + w0;
+            a1 = min(r1, lim) * row_bytes + w1;
+            a2 = min(r2, lim) * row_bytes + w2;
+        }
+        uint8_t *lp = ring + (n_issue % NS) * kQ4kTileBytes;
+        __builtin_amdgcn_global_load_lds((g_vp)(gp + a0), (lds_vp)lp, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((g_vp)(gp + a1), (lds_vp)(lp + 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((g_vp)(gp + a2), (lds_vp)(lp + 2048), 4, 0, 0);
+        n_issue++;
+        if (it_tile < tile_b && ++it_p == np) { it_p = 0; it_tile++; }
+    };
+    // the activation columns are requested first (ahead of the weight tiles in the in-order return queue)
+    Q8kCol col[NP];
+#pragma unroll
+    for (int p = 0; p < NP; p++)
+        col[p] = q8k_load_col((const uint8_t *)j.x, (uint32_t)j.k, min(wv + nwj * (uint32_t)p, cpr - 1), lane);
+    if (np >= 1)
+        for (int s = 0; s < NS - 1; s++) issue();
+
+    uint32_t n_use = 0;
+    for (uint32_t tb = 0; tb < nt; tb += R) {
+        float *pb = part + parity * (R * 16 * PW);
+        const uint32_t nb = min((uint32_t)R, nt - tb);
+        if (np >= 1) {
+            for (uint32_t tl = 0; tl < nb; tl++) {
+#pragma unroll
+                for (int p = 0; p < NP; p++) {
+                    if ((uint32_t)p < np) {
+                        issue();
+                        LARQL_WAIT_VMCNT(3 * (NS - 1));  // at most NS-1 younger wave-tiles still in flight: the oldest has landed
+                        asm volatile("" ::: "memory");
+                        const float term = q4k_q8k_tile(ring + (n_use % NS) * kQ4kTileBytes, col[p], jr, kq);
+                        n_use++;
+                        if (kq == 0) pb[(tl * 16 + jr) * PW + wv + nwj * p] = term;
+                    }
+                }
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        // a lane per row: acc += term, super-blocks in order (q4k_scalar.rs:39,79)
+        const uint32_t row_base = (tile_a + tb) * 16;
+        for (uint32_t rr = threadIdx.x; rr < nb * 16; rr += blockDim.x) {
+            float acc = 0.f;
+            for (uint32_t c = 0; c < cpr; c++) acc += pb[rr * PW + c];
+            if (row_base + rr < rows) ((g_f32wp)j.out)[row_base + rr] = acc;
+        }
+        parity ^= 1u;
+    }
+}
+
+// ---------------------------------------------------------------------------
 // MXFP4 on the matrix cores (rows of up to 40 x 128 elements).
 //
 // gfx950's block-scaled MFMA takes the format as stored: v_mfma_scale_f32_16x16x128_f8f6f4 with an
@@ -1767,6 +1919,31 @@ __global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_mfma_kernel(GemvLa
     LARQL_WAIT_VMCNT(0);
 }
 
+// Q4_K x Q8_K: the same sweep and cost model as the Q4_K kernel.
+__global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_q8k_kernel(GemvLaunch L) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t q8k_lds[];
+    const GemvJob *jobs = L.table ? L.table : L.inl;
+    const uint64_t P = L.total_passes;
+    uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
+    const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
+    uint32_t lo = 0, hi = L.n_jobs;
+    while (lo + 1 < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if ((uint32_t)__builtin_amdgcn_readfirstlane(jobs[mid].pass_begin) <= p) lo = mid; else hi = mid;
+    }
+    uint32_t ji = lo, parity = 0;
+    while (p < p_end) {
+        const GemvJob j = uniform_job(jobs + ji);
+        const uint32_t seg_end = min(p_end, j.pass_begin + j.n_pass);
+        const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin, cpt = (uint32_t)j.pad, su = j.pad2;
+        const uint32_t tile_a = a > su ? (a - su + cpt - 1) / cpt : 0, tile_b = b > su ? (b - su + cpt - 1) / cpt : 0;
+        if (tile_a < tile_b) run_q4k_q8k(j, tile_a, tile_b, q8k_lds, parity);
+        p = seg_end;
+        ji++;
+    }
+    LARQL_WAIT_VMCNT(0);
+}
+
 // MXFP4 on the matrix cores: same sweep as the Q4_K kernel (cost unit = one tile x one 128-element step).
 __global__ void __launch_bounds__(kMx4MaxWaves * 64) gemv_mxfp4_mfma_kernel(GemvLaunch L) {
     extern __shared__ __attribute__((aligned(16))) uint8_t mx4_lds[];
@@ -1996,7 +2173,7 @@ bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
         j.n_pass = (uint32_t)(tiles * steps);
         return true;
     }
-    if (j.kind == KIND_Q4K_MFMA) {
+    if (j.kind == KIND_Q4K_MFMA || j.kind == KIND_Q4K_Q8K) {
         if (j.k == 0 || j.k % 256 != 0) return false;
         const uint64_t cpr = j.k / 256;
         const uint32_t nw = q4k_mfma_waves(cpr);
@@ -2070,7 +2247,7 @@ uint32_t gemv_pick_threads(const GemvJob *jobs, size_t n) {
         }
         return nw * 64;
     }
-    if (n > 0 && jobs[0].kind == KIND_Q4K_MFMA) {
+    if (n > 0 && (jobs[0].kind == KIND_Q4K_MFMA || jobs[0].kind == KIND_Q4K_Q8K)) {
         uint32_t nw = 0;
         for (size_t i = 0; i < n; i++) {
             const uint32_t w = q4k_mfma_waves(jobs[i].k / 256);
@@ -2131,6 +2308,12 @@ size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
         const size_t nw = threads / 64;
         return nw * kMx4Stages * gemv_launch_param(jobs, n) + 2 * (size_t)kMx4BatchTiles * 16 * nw * 4 * sizeof(float);
     }
+    if (n > 0 && jobs[0].kind == KIND_Q4K_Q8K) {  // rings + one partial per (row, super-block), double-buffered
+        const size_t nw = threads / 64;
+        uint64_t cpr = 1;
+        for (size_t i = 0; i < n; i++) cpr = std::max<uint64_t>(cpr, jobs[i].k / 256);
+        return nw * kQ4kStages * kQ4kTileBytes + 2 * (size_t)kQ4kBatchTiles * 16 * cpr * sizeof(float);
+    }
     if (n > 0 && jobs[0].kind == KIND_Q4K_MFMA) {
         const size_t nw = threads / 64;
         bool multi = false;  // some row needs several column passes: room for the prepared activations
@@ -2148,7 +2331,9 @@ size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
 }
 
 uint32_t gemv_wgs_per_cu(int kind, uint32_t threads, size_t lds, uint32_t dflt) {
-    if (kind != KIND_Q4K_MFMA && kind != KIND_MXFP4_MFMA && kind != KIND_BF16_MFMA && kind != KIND_Q4K_BATCH && kind != KIND_Q8_0_MFMA) return dflt;
+    if (kind != KIND_Q4K_MFMA && kind != KIND_MXFP4_MFMA && kind != KIND_BF16_MFMA && kind != KIND_Q4K_BATCH && kind != KIND_Q8_0_MFMA &&
+        kind != KIND_Q4K_Q8K)
+        return dflt;
     // as many workgroups as LDS (160 KB per CU) allows, up to 12 wavefronts per CU (3 per SIMD at this register count)
     const uint32_t by_lds = (uint32_t)((160 * 1024) / lds), by_waves = 12 / (threads / 64);
     const uint32_t w = by_lds < by_waves ? by_lds : by_waves;
@@ -2205,6 +2390,16 @@ hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32
                 attr_set = true;
             }
             hipLaunchKernelGGL(gemv_q4k_mfma_kernel, dim3(grid), dim3(threads), lds, stream, L);
+            break;
+        }
+        case KIND_Q4K_Q8K: {
+            static bool attr_set = false;  // dynamic LDS above 64 KB has to be allowed once per process
+            if (!attr_set) {
+                hipError_t e = hipFuncSetAttribute((const void *)gemv_q4k_q8k_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                if (e != hipSuccess) return e;
+                attr_set = true;
+            }
+            hipLaunchKernelGGL(gemv_q4k_q8k_kernel, dim3(grid), dim3(threads), lds, stream, L);
             break;
         }
         case KIND_Q4K:

@@ -13,7 +13,8 @@ enum GemvKind : int32_t {
     KIND_BF16_MFMA = 9,  // internal: bf16 rows against 2..8 activations at once (batch field of the job)
     KIND_Q4K_BATCH = 10, // internal: Q4_K rows against 2..4 activations at once
     KIND_Q8_0_MFMA = 11, // internal: ggml Q8_0 rows short enough for the matrix-core kernel
-    KIND_Q6K = 12        // Q6_K, 210-byte super-blocks (K-slice kernel)
+    KIND_Q6K = 12,       // Q6_K, 210-byte super-blocks (K-slice kernel)
+    KIND_Q4K_Q8K = 13    // Q4_K weights against a Q8_K activation (integer dots on the matrix cores); x = the Q8_K device layout
 };
 
 constexpr int kGemvMaxThreads = 512;
@@ -84,6 +85,9 @@ hipError_t quantize_mxfp4_launch(hipStream_t s, const float *src, size_t rows, s
                                  uint8_t *scales, const uint8_t *log2_up_table);
 hipError_t f32_to_bf16_launch(hipStream_t s, const float *src, size_t n, uint16_t *dst);
 hipError_t quantize_q4_0_launch(hipStream_t s, const float *src, size_t n, uint8_t *dst);
+// Q8_K activation of n elements in its device layout: [n int8 codes | n/256 f32 scales | n/32 i16 sub-block sums]
+inline size_t q8k_bytes(size_t n) { return n + (n / 256) * 4 + (n / 32) * 2; }
+hipError_t quantize_x_to_q8k_launch(hipStream_t s, const float *src, size_t n, uint8_t *dst);
 hipError_t quantize_to_q8_launch(hipStream_t s, const float *src, size_t n, int8_t *q8, float *scales);
 hipError_t fill_normal_launch(hipStream_t s, float *dst, size_t n, uint64_t seed, float sigma);
 

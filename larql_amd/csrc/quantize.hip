@@ -187,6 +187,33 @@ __global__ void quantize_to_q8_kernel(const float *__restrict__ src, size_t n_bl
     for (int i = 0; i < 32; i++) q8[b * 32 + i] = (int8_t)sat_i8(clampf(roundf(src[b * 32 + i] * inv), -128.0f, 127.0f));
 }
 
+// quantize_x_to_q8k — larql-compute/src/cpu/ops/q4k_q8k_dot/q8k_activation.rs:84-109: per 256-element super-block
+// d = amax/127, codes round(x * (1/d)) clamped to +-127, and the sum of every 32 codes.  One wavefront per
+// super-block, four elements per lane; the eight lanes of a sub-block add their codes by shuffles (integers: any
+// order).  Output is the device layout of a Q8_K activation of n elements: [n codes | n/256 f32 scales | n/32 i16 sums].
+__global__ void __launch_bounds__(256) quantize_x_to_q8k_kernel(const float *__restrict__ src, size_t n_blocks, uint8_t *__restrict__ dst) {
+    const size_t sb = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (sb >= n_blocks) return;
+    const uint32_t lane = threadIdx.x & 63u;
+    const float4 v = reinterpret_cast<const float4 *>(src + sb * 256)[lane];
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));  // fmaxf ignores a NaN operand, as f32::max does
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+    const float scale = amax > 0.0f ? amax / 127.0f : 0.0f;
+    const float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
+    const int q0 = sat_i8(clampf(roundf(v.x * inv), -127.0f, 127.0f)), q1 = sat_i8(clampf(roundf(v.y * inv), -127.0f, 127.0f));
+    const int q2 = sat_i8(clampf(roundf(v.z * inv), -127.0f, 127.0f)), q3 = sat_i8(clampf(roundf(v.w * inv), -127.0f, 127.0f));
+    int sum = q0 + q1 + q2 + q3;
+    sum += __shfl_xor(sum, 1);
+    sum += __shfl_xor(sum, 2);
+    sum += __shfl_xor(sum, 4);
+    const size_t n = n_blocks * 256;
+    reinterpret_cast<uint32_t *>(dst)[sb * 64 + lane] =
+        ((uint32_t)q0 & 0xFFu) | (((uint32_t)q1 & 0xFFu) << 8) | (((uint32_t)q2 & 0xFFu) << 16) | (((uint32_t)q3 & 0xFFu) << 24);
+    if (lane == 0) reinterpret_cast<float *>(dst + n)[sb] = scale;
+    if ((lane & 7u) == 0) reinterpret_cast<int16_t *>(dst + n + n_blocks * 4)[sb * 8 + (lane >> 3)] = (int16_t)sum;
+}
+
 __device__ __forceinline__ int sat_i32(float v) {
     if (v != v) return 0;
     if (v >= 2147483648.0f) return 2147483647;
@@ -317,6 +344,12 @@ hipError_t quantize_q8_0_launch(hipStream_t s, const float *src, size_t n, uint8
     const size_t nb = n / 32;
     if (nb == 0) return hipSuccess;
     hipLaunchKernelGGL(quantize_q8_0_kernel, blocks_for(nb, 256), dim3(256), 0, s, src, nb, dst);
+    return hipGetLastError();
+}
+hipError_t quantize_x_to_q8k_launch(hipStream_t s, const float *src, size_t n, uint8_t *dst) {
+    const size_t nb = n / 256;
+    if (nb == 0) return hipSuccess;
+    hipLaunchKernelGGL(quantize_x_to_q8k_kernel, blocks_for(nb, 4), dim3(256), 0, s, src, nb, dst);
     return hipGetLastError();
 }
 hipError_t quantize_mxfp4_launch(hipStream_t s, const float *src, size_t rows, size_t k, uint8_t *packed, uint8_t *scales,

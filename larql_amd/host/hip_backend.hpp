@@ -67,6 +67,18 @@ class HipBackend {
         std::vector<float> out(num_rows);
         return some(larql_hip_q6k_matvec(ctx_, q6k.ptr, q6k.len, x.ptr, x.len, num_rows, hidden, out.data()), out);
     }
+    // Q8_K-activation integer path (cpu/ops/q4k_q8k_dot): Q8KActivation { qs, d, sums }
+    struct Q8KActivation { std::vector<int8_t> qs; std::vector<float> d; std::vector<int16_t> sums; };
+    std::optional<Q8KActivation> quantize_x_to_q8k(Slice<float> x) {
+        Q8KActivation a{std::vector<int8_t>(x.len), std::vector<float>(x.len / 256), std::vector<int16_t>(x.len / 32)};
+        if (larql_hip_quantize_x_to_q8k(ctx_, x.ptr, x.len, a.qs.data(), a.d.data(), a.sums.data()) != LARQL_OK) return std::nullopt;
+        return a;
+    }
+    std::optional<std::vector<float>> q4k_q8k_matvec(Slice<uint8_t> q4k, const Q8KActivation &a, size_t num_rows, size_t cols) {
+        std::vector<float> out(num_rows);
+        return some(larql_hip_q4k_q8k_matvec(ctx_, q4k.ptr, q4k.len, a.qs.data(), a.qs.size(), a.d.data(), a.sums.data(), num_rows, cols,
+                                             out.data(), out.size()), out);
+    }
     std::optional<std::pair<std::vector<float>, std::vector<float>>> q4k_dual_matvec(Slice<uint8_t> a, Slice<uint8_t> b,
                                                                                        Slice<float> x, size_t num_rows,
                                                                                        size_t hidden) {

@@ -56,6 +56,20 @@ int main() {
     CHECK(out.has_value() && out->size() == rows);
     for (float v : *out) CHECK(std::fabs(v - 2 * per_sb) < 1e-3);
 
+    {
+        // Q8_K-activation path on the same matrix: x = 1 quantises to d = 1/127, every code 127, every sub-block sum 32*127;
+        // the integer sums are exact, so the output is 2 * ((d_w*d_y)*sum1 - (dmin_w*d_y)*sum2) up to the two f32 roundings
+        auto a = be.quantize_x_to_q8k({x.data(), x.size()});
+        CHECK(a && a->qs.size() == hidden && a->d.size() == 2 && a->sums.size() == 16);
+        for (int8_t q : a->qs) CHECK(q == 127);
+        CHECK(a->d[0] == 1.0f / 127.0f && a->sums[5] == 32 * 127);
+        auto o8 = be.q4k_q8k_matvec(w, *a, rows, hidden);
+        CHECK(o8.has_value() && o8->size() == rows);
+        for (float v : *o8) CHECK(std::fabs(v - 2 * per_sb) < 2e-3 * per_sb);
+        a->qs.pop_back();
+        CHECK(!be.q4k_q8k_matvec(w, *a, rows, hidden));  // activation of the wrong length: refused
+    }
+
     // refusals: None, never a wrong vector (backend/quant_matvec.rs:378-427, kernel_shape.rs)
     std::vector<float> x_short(hidden - 1, 1.0f);
     CHECK(!be.q4k_matvec(w, x_short, rows, hidden).has_value());

@@ -567,6 +567,80 @@ int lq_q6k_matvec(const uint8_t *w, size_t w_len, const float *x, size_t rows, s
     return 0;
 }
 
+/* quantize_x_to_q8k — larql-compute/src/cpu/ops/q4k_q8k_dot/q8k_activation.rs:84-109 (and its in-place twin :44-77):
+ * per 256-element super-block d = amax/127 (0 for an all-zero block), codes round(x * (1/d)) clamped to +-127
+ * (f32::round: half away from zero), sums[8] = the i32 sum of each 32-code sub-block stored as i16.
+ * Pinned by the reference's own properties (tests/q8k_quantize_and_matvec.rs:18-50: reconstruction within one
+ * step on its ramp input, sums equal the literal sums, zero input clean), closed forms and the numpy restatement;
+ * no reference-held vector exists: parity unpinned. */
+int lq_quantize_x_to_q8k(const float *x, size_t n, int8_t *qs, float *d, int16_t *sums) {
+    if (n % 256 != 0) return 1;
+    for (size_t sb = 0; sb < n / 256; sb++) {
+        const float *block = x + sb * 256;
+        float amax = 0.0f;
+        for (int i = 0; i < 256; i++) { float a = fabsf(block[i]); amax = a > amax ? a : amax; }  /* f32::max: a NaN operand is ignored */
+        float scale = amax > 0.0f ? amax / 127.0f : 0.0f;
+        float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
+        d[sb] = scale;
+        for (int s = 0; s < 8; s++) {
+            int32_t acc = 0;
+            for (int j = 0; j < 32; j++) {
+                float v = roundf(block[s * 32 + j] * inv);
+                v = v < -127.0f ? -127.0f : (v > 127.0f ? 127.0f : v);
+                int8_t q = (int8_t)v;  /* `as i8` saturates and maps NaN to 0; after the clamp only NaN differs: (int8_t)NaN is undefined in C */
+                if (v != v) q = 0;
+                qs[sb * 256 + s * 32 + j] = q;
+                acc += q;
+            }
+            sums[sb * 8 + s] = (int16_t)acc;
+        }
+    }
+    return 0;
+}
+
+/* q4k_q8k_matvec_scalar — larql-compute/src/cpu/ops/q4k_q8k_dot/q4k_scalar.rs:15-84, the reference every SIMD
+ * kernel of the module is held to bit for bit (NEON, AVX2, the hand assembly; dispatch.rs:15-51):
+ * per super-block sum1 = sum_sub sc*dot(q4, q8), sum2 = sum_sub mn*bsum in i32, then
+ * acc += d_w*d_y*(f32)sum1 - dmin_w*d_y*(f32)sum2 (left to right, no fused multiply-add), super-blocks in order.
+ * Shape rule: KernelShapeError::check (cpu/ops/kernel_shape.rs:47-75): out_len == rows, qs_len == cols,
+ * cols % 256 == 0, w_len >= rows*(cols/256)*144; rows == 0 or cols == 0 fill `out` with zeros. */
+int lq_q4k_q8k_matvec(float *out, size_t out_len, const int8_t *qs, size_t qs_len, const float *d, const int16_t *sums,
+                      const uint8_t *w, size_t w_len, size_t rows, size_t cols) {
+    size_t nb = cols / 256, row_bytes = nb * 144;
+    if (out_len != rows || qs_len != cols || cols % 256 != 0 || w_len < rows * row_bytes) return 1;
+    if (rows == 0 || cols == 0) { for (size_t r = 0; r < out_len; r++) out[r] = 0.0f; return 0; }
+    for (size_t r = 0; r < rows; r++) {
+        float acc = 0.0f;
+        for (size_t sb = 0; sb < nb; sb++) {
+            const uint8_t *block = w + r * row_bytes + sb * 144;
+            float d_w = lq_f16_to_f32((uint16_t)(block[0] | (block[1] << 8)));
+            float dmin_w = lq_f16_to_f32((uint16_t)(block[2] | (block[3] << 8)));
+            uint8_t scales[8], mins[8];
+            q4k_unpack_scales(block + 4, scales, mins);
+            const uint8_t *quants = block + 16;
+            const int8_t *y = qs + sb * 256;
+            const int16_t *bs = sums + sb * 8;
+            float d_y = d[sb];
+            int32_t sum1 = 0, sum2 = 0;
+            for (int g = 0; g < 4; g++) {
+                int32_t dot_lo = 0, dot_hi = 0;
+                for (int l = 0; l < 32; l++) {
+                    uint8_t byte = quants[g * 32 + l];
+                    dot_lo += (int32_t)(byte & 0x0F) * y[(2 * g) * 32 + l];
+                    dot_hi += (int32_t)(byte >> 4) * y[(2 * g + 1) * 32 + l];
+                }
+                sum1 += (int32_t)scales[2 * g] * dot_lo + (int32_t)scales[2 * g + 1] * dot_hi;
+                sum2 += (int32_t)mins[2 * g] * bs[2 * g] + (int32_t)mins[2 * g + 1] * bs[2 * g + 1];
+            }
+            float t1 = d_w * d_y; t1 = t1 * (float)sum1;
+            float t2 = dmin_w * d_y; t2 = t2 * (float)sum2;
+            acc += t1 - t2;
+        }
+        out[r] = acc;
+    }
+    return 0;
+}
+
 /* larql-models/src/quant/ggml/quantize.rs:50-77.  Codes use the reciprocal
  * of the un-rounded f32 scale.
  * Pinned: byte-for-byte against the reference-held ggml golden blocks

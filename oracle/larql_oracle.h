@@ -54,6 +54,9 @@ void lq_q4k_matmul_into(float *out, const float *x, const uint8_t *w, size_t w_l
 int  lq_quantize_q6_k(const float *data, size_t n, uint8_t *out);              /* q4_common/quantize.rs:197-276 */
 void lq_q6k_subblock_vals(const uint8_t *block, size_t j, int8_t *out16);     /* larql-models/src/quant/ggml/q6_k.rs:19-40 */
 int  lq_dequantize_q6_k(const uint8_t *data, size_t data_len, size_t n, float *out); /* q6_k.rs:173-195 */
+int  lq_quantize_x_to_q8k(const float *x, size_t n, int8_t *qs, float *d, int16_t *sums); /* cpu/ops/q4k_q8k_dot/q8k_activation.rs:84-109 */
+int  lq_q4k_q8k_matvec(float *out, size_t out_len, const int8_t *qs, size_t qs_len, const float *d, const int16_t *sums,
+                       const uint8_t *w, size_t w_len, size_t rows, size_t cols); /* cpu/ops/q4k_q8k_dot/q4k_scalar.rs:15-84 */
 int  lq_q6k_matvec(const uint8_t *w, size_t w_len, const float *x, size_t rows, size_t hidden, float *out); /* cpu/ops/q6k_matvec.rs:45-91 */
 
 int  lq_quantize_q8_0(const float *data, size_t n, uint8_t *out);

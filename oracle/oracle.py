@@ -199,6 +199,33 @@ def q6k_matvec(w, x, rows: int, hidden: int):
     return out
 
 
+def quantize_x_to_q8k(x):
+    """Q8_K activation: (qs int8 [n], d f32 [n/256], sums int16 [n/32]); n % 256 == 0."""
+    x = _f32(x).ravel()
+    if x.size % 256 != 0:
+        raise ValueError("Q8_K: element count must be a multiple of 256")
+    qs = np.empty(x.size, dtype=np.int8)
+    d = np.empty(x.size // 256, dtype=np.float32)
+    sums = np.empty(x.size // 32, dtype=np.int16)
+    _lib.lq_quantize_x_to_q8k(_p(x, _f32p), _sz(x.size), _p(qs, _i8p), _p(d, _f32p), _p(sums, C.POINTER(C.c_int16)))
+    return qs, d, sums
+
+
+def q4k_q8k_matvec(w, qs, d, sums, rows: int, cols: int):
+    """q4k_q8k_matvec_scalar: None where the reference refuses the operands."""
+    w = _u8(w).ravel()
+    qs = np.ascontiguousarray(qs, dtype=np.int8).ravel()
+    d = _f32(d).ravel()
+    sums = np.ascontiguousarray(sums, dtype=np.int16).ravel()
+    out = np.empty(rows, dtype=np.float32)
+    if d.size * 256 != qs.size or sums.size * 32 != qs.size:
+        return None
+    if _lib.lq_q4k_q8k_matvec(_p(out, _f32p), _sz(rows), _p(qs, _i8p), _sz(qs.size), _p(d, _f32p), _p(sums, C.POINTER(C.c_int16)),
+                              _p(w, _u8p), _sz(w.size), _sz(rows), _sz(cols)):
+        return None
+    return out
+
+
 def quantize_q8_0(data) -> np.ndarray:
     data = _f32(data).ravel()
     out = np.empty(data.size // 32 * 34, dtype=np.uint8)

@@ -217,3 +217,40 @@ def quantize_mxfp4(values, rows, k):
     code = np.where(best == 0, 0, sign | best).astype(np.uint8)
     packed = (code[..., 0::2] | (code[..., 1::2] << 4)).astype(np.uint8)
     return packed.reshape(-1), byte.reshape(-1)
+
+
+def quantize_x_to_q8k(x):
+    """Q8_K activation, written from the description in q4k_q8k_dot/mod.rs:12-27 and llama.cpp's convention:
+    symmetric int8 over [-127, 127] per 256 values, d = absmax/127, per-32 sums of the codes."""
+    x = np.asarray(x, np.float32).reshape(-1, 256)
+    amax = np.abs(x).max(axis=1)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        d = np.where(amax > 0, amax / np.float32(127.0), np.float32(0.0)).astype(np.float32)
+        inv = np.where(d > 0, np.float32(1.0) / d, np.float32(0.0)).astype(np.float32)
+    q = np.clip(rust_round((x * inv[:, None]).astype(np.float32)), -127.0, 127.0).astype(np.int8)
+    sums = q.reshape(-1, 32).astype(np.int32).sum(axis=1).astype(np.int16)
+    return q.reshape(-1), d, sums
+
+
+def q4k_q8k_matvec(w, qs, d, sums, rows, cols):
+    """Q4_K x Q8_K integer-dot matvec, vectorised differently from the oracle's loops: all integer sums first
+    (exact), then the reference's float expression per super-block in f32, accumulated in order."""
+    nb = cols // 256
+    blocks = np.asarray(w, np.uint8)[: rows * nb * 144].reshape(rows, nb, 144)
+    d_w, dmin_w, sc, mn = q4k_unpack_header(blocks.reshape(-1, 144))
+    d_w, dmin_w = d_w.reshape(rows, nb), dmin_w.reshape(rows, nb)
+    sc, mn = sc.reshape(rows, nb, 8).astype(np.int64), mn.reshape(rows, nb, 8).astype(np.int64)
+    q = blocks[:, :, 16:].reshape(rows, nb, 4, 32)
+    nib = np.stack([q & 0x0F, q >> 4], axis=3).reshape(rows, nb, 8, 32).astype(np.int64)  # sub-block 2g = low, 2g+1 = high
+    y = np.asarray(qs, np.int8).reshape(nb, 8, 32).astype(np.int64)
+    dots = (nib * y[None]).sum(axis=3)                                        # [rows, nb, 8]
+    sum1 = (sc * dots).sum(axis=2)
+    sum2 = (mn * np.asarray(sums, np.int16).reshape(nb, 8).astype(np.int64)[None]).sum(axis=2)
+    dy = np.asarray(d, np.float32)[None, :]
+    t1 = ((d_w * dy).astype(np.float32) * sum1.astype(np.float32)).astype(np.float32)
+    t2 = ((dmin_w * dy).astype(np.float32) * sum2.astype(np.float32)).astype(np.float32)
+    term = (t1 - t2).astype(np.float32)
+    acc = np.zeros(rows, np.float32)
+    for b in range(nb):
+        acc = (acc + term[:, b]).astype(np.float32)
+    return acc

@@ -163,6 +163,100 @@ def test_q6k_matvec_shape_rules(be):
     assert be.q6k_matvec(np.zeros(0, np.uint8), np.zeros(256, F), 0, 256).size == 0
 
 
+# ------------------------------------------------- Q8_K-activation integer path
+@pytest.mark.parametrize("n,scale", [(256, 1.0), (2560, 3.0), (10240, 1e-3), (256 * 7, 2e4)])
+def test_quantize_x_to_q8k_bit_exact(be, n, scale):
+    rng = np.random.default_rng(n)
+    x = (rng.standard_normal(n) * scale).astype(F)
+    x[3] = 0.0
+    if n > 512:
+        x[256:512] = 0.0                       # an all-zero super-block
+    x[n - 1] = F(scale) * 9                    # an outlier
+    x[10:16] = np.array([0.5, -0.5, 1.5, -1.5, 2.5, -2.5], F) * (np.abs(x[:256]).max() / F(127.0))   # near half-way cases
+    want = O.quantize_x_to_q8k(x)
+    got = be.quantize_x_to_q8k(x)
+    assert got is not None
+    for g, w in zip(got, want):
+        assert np.array_equal(g, w)
+    assert be.quantize_x_to_q8k(np.zeros(255, F)) is None
+
+
+@pytest.mark.parametrize("rows,cols", [(3072, 1024), (2048, 2560), (1031, 2560), (77, 10240), (5, 256), (300, 3840), (33, 1792),
+                                       (257, 4096), (130, 7168), (1, 2560), (4100, 512), (19, 2816)])
+def test_q4k_q8k_matvec_bit_exact(be, rows, cols):
+    """Every SIMD kernel of the reference equals q4k_q8k_matvec_scalar bit for bit (dispatch.rs:15-51); so does this one."""
+    w, x = weights(rows * 3 + cols, rows, cols)
+    q = O.quantize_q4_k(w)
+    a = O.quantize_x_to_q8k(x * F(2.5))
+    want = O.q4k_q8k_matvec(q, *a, rows, cols)
+    got = be.q4k_q8k_matvec(q, *a, rows, cols)
+    assert got is not None
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_q4k_q8k_matvec_extreme_codes_and_scales(be):
+    # all codes at +-127, all nibbles 15, scales and mins 63: the largest integer sums the kernel can meet
+    rows, cols = 48, 2560
+    nb = cols // 256
+    blk = np.zeros(144, np.uint8)
+    blk[0:2] = np.array([1.0], np.float16).view(np.uint8)
+    blk[2:4] = np.array([0.5], np.float16).view(np.uint8)
+    blk[4:16] = 0xFF                           # every 6-bit scale and min = 63
+    blk[16:] = 0xFF                            # every nibble = 15
+    q = np.tile(blk, rows * nb)
+    qs = np.where(np.arange(cols) % 3 == 0, -127, 127).astype(np.int8)
+    d = np.full(nb, 0.75, F)
+    sums = qs.reshape(-1, 32).astype(np.int32).sum(axis=1).astype(np.int16)
+    want = O.q4k_q8k_matvec(q, qs, d, sums, rows, cols)
+    got = be.q4k_q8k_matvec(q, qs, d, sums, rows, cols)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # sums are an operand (not recomputed from the codes): the min term follows them
+    sums2 = (sums // 2).astype(np.int16)
+    assert np.array_equal(be.q4k_q8k_matvec(q, qs, d, sums2, rows, cols).view(np.uint32),
+                          O.q4k_q8k_matvec(q, qs, d, sums2, rows, cols).view(np.uint32))
+
+
+def test_q4k_q8k_matvec_shape_rules(be):
+    # KernelShapeError::check (cpu/ops/kernel_shape.rs:47-75) as the reference's tests exercise it
+    # (fused_and_q6k_paths.rs:53-84, public_execution_path_q4k_q8k_matvec_par.rs:33-78)
+    w = O.quantize_q4_k(np.ones(2 * 512, F))
+    a = O.quantize_x_to_q8k(np.ones(512, F))
+    assert be.q4k_q8k_matvec(w, *a, 2, 512) is not None
+    assert be.q4k_q8k_matvec(w[:-1], *a, 2, 512) is None                                   # short weight slab
+    assert be.q4k_q8k_matvec(w, *O.quantize_x_to_q8k(np.ones(768, F)), 2, 512) is None      # activation of the wrong length
+    assert be.q4k_q8k_matvec(w, *a, 2, 512, out_len=1) is None                             # output shorter than rows
+    z = be.q4k_q8k_matvec(np.zeros(0, np.uint8), np.zeros(0, np.int8), np.zeros(0, F), np.zeros(0, np.int16), 3, 0)
+    assert z is not None and z.shape == (3,) and not z.any()                               # zero dims give zeros
+    big = O.quantize_x_to_q8k(np.ones(10496, F))                                           # 41 super-blocks: no kernel
+    assert be.q4k_q8k_matvec(np.zeros(41 * 144, np.uint8), *big, 1, 10496) is None
+
+
+def test_q4k_q8k_device_tier_plan_matches_host_tier(be, fmt):
+    # activation quantised on the device into its device layout, several matvecs in one plan
+    rng = np.random.default_rng(97)
+    shapes = [(640, 2560), (96, 2560), (200, 10240), (31, 1024)]
+    x = {k: rng.standard_normal(k).astype(F) for k in (2560, 10240, 1024)}
+    dq = {}
+    for k, xv in x.items():
+        dx, buf = be.to_device(xv), be.malloc(be.q8k_bytes(k) + 64)
+        assert be.dev_quantize_x_to_q8k(dx, k, buf)
+        dq[k] = buf
+    jobs, outs, wants = [], [], []
+    for rows, k in shapes:
+        q = O.quantize_q4_k((rng.standard_normal(rows * k) * 0.03).astype(F))
+        o = be.malloc(rows * 4)
+        jobs.append((fmt.FMT_Q4_K_Q8K, be.to_device(q), None, dq[k], o, rows, k))
+        outs.append((o, rows))
+        wants.append(O.q4k_q8k_matvec(q, *O.quantize_x_to_q8k(x[k]), rows, k))
+    plan = be.plan_create(jobs)
+    assert plan is not None and be.plan_launch_count(plan) == 1
+    assert be.plan_run(plan) and be.plan_run(plan)
+    be.synchronize()
+    for (o, rows), want in zip(outs, wants):
+        assert np.array_equal(be.d2h(o, rows, F).view(np.uint32), want.view(np.uint32))
+    be.plan_destroy(plan)
+
+
 # ------------------------------------------------------------------ Q8_0
 @pytest.mark.parametrize("n,k", [(4099, 2560), (64, 10240), (9, 128), (1000, 2048), (17, 256), (333, 1792), (48, 2816),
                                  (531, 3840), (2050, 4096), (77, 5120), (40, 5376)])   # two column passes per wavefront; odd column count; just above
