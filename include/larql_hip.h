@@ -57,7 +57,9 @@ enum {
     /* Q4_K weights against a Q8_K activation (the integer-dot decode path,
      * larql-compute/src/cpu/ops/q4k_q8k_dot): in a device-tier job `x` is the
      * activation in the layout larql_hip_dev_quantize_x_to_q8k writes. */
-    LARQL_FMT_Q4_K_Q8K = 101
+    LARQL_FMT_Q4_K_Q8K = 101,
+    /* Q6_K weights against the same activation layout (cpu/ops/q4k_q8k_dot/q6k.rs). */
+    LARQL_FMT_Q6_K_Q8K = 102
 };
 
 /* Capability — larql-compute/src/backend/capability.rs:22-102 (the ones this
@@ -128,6 +130,14 @@ int larql_hip_quantize_x_to_q8k(larql_hip_ctx *ctx, const float *x, size_t n, in
  * dims write zeros.  cols <= 10240 on this backend (longer: UNSUPPORTED). */
 int larql_hip_q4k_q8k_matvec(larql_hip_ctx *ctx, const uint8_t *q4k, size_t q4k_len, const int8_t *qs, size_t qs_len,
                              const float *d, const int16_t *sums, size_t num_rows, size_t cols, float *out, size_t out_len);
+/* q6k_q8k_matvec_into / q4k_q8k_matvec_parallel with format "Q6_K" —
+ * cpu/ops/q4k_q8k_dot/q6k.rs:15-92, dispatch.rs:100-148: per super-block
+ * acc += d_w*d_y*(f32)(sum over the 16 groups of scale_g * dot(q6 - 32, q8)), in
+ * super-block order; bit-exact with q6k_q8k_matvec_scalar (the reference's NEON
+ * kernel is checked against it to 1e-3).  The activation's `sums` are not used by
+ * this format.  Shape rule as above with 210-byte blocks. */
+int larql_hip_q6k_q8k_matvec(larql_hip_ctx *ctx, const uint8_t *q6k, size_t q6k_len, const int8_t *qs, size_t qs_len,
+                             const float *d, size_t num_rows, size_t cols, float *out, size_t out_len);
 /* QuantMatVec::q4k_dual_matvec — quant_matvec.rs:287-296; q4_common/dual.rs:22-167. */
 int larql_hip_q4k_dual_matvec(larql_hip_ctx *ctx, const uint8_t *q4k_a, size_t a_len,
                               const uint8_t *q4k_b, size_t b_len,

@@ -16,7 +16,7 @@ OK, UNSUPPORTED, REFUSED_SHAPE = 0, 1, 2
 E_DEVICE, E_NO_DEVICE, E_ARG, E_NAN = -1, -2, -3, -4
 
 FMT_Q4_0, FMT_Q4_K, FMT_Q4_KF, FMT_Q5_K, FMT_Q6_K, FMT_Q8_0 = 0, 1, 2, 3, 4, 5
-FMT_BF16, FMT_F16, FMT_F32, FMT_I2S, FMT_MXFP4, FMT_GGML_Q8_0, FMT_Q4_K_Q8K = 6, 7, 8, 9, 10, 100, 101
+FMT_BF16, FMT_F16, FMT_F32, FMT_I2S, FMT_MXFP4, FMT_GGML_Q8_0, FMT_Q4_K_Q8K, FMT_Q6_K_Q8K = 6, 7, 8, 9, 10, 100, 101, 102
 CAP_F32_GEMV, CAP_F16_GEMV, CAP_QUANT_MATVEC = 0, 1, 2
 
 vp, sz, ci = C.c_void_p, C.c_size_t, C.c_int
@@ -55,6 +55,7 @@ SIGNATURES = {
     "larql_hip_q6k_matvec": (ci, [vp, vp, sz, vp, sz, sz, sz, vp]),
     "larql_hip_quantize_x_to_q8k": (ci, [vp, vp, sz, vp, vp, vp]),
     "larql_hip_q4k_q8k_matvec": (ci, [vp, vp, sz, vp, sz, vp, vp, sz, sz, vp, sz]),
+    "larql_hip_q6k_q8k_matvec": (ci, [vp, vp, sz, vp, sz, vp, sz, sz, vp, sz]),
     "larql_hip_q8k_bytes": (sz, [sz]),
     "larql_hip_dev_quantize_x_to_q8k": (ci, [vp, vp, sz, vp]),
     "larql_hip_q4k_dual_matvec": (ci, [vp, vp, sz, vp, sz, vp, sz, sz, sz, vp, vp, sz]),

@@ -142,6 +142,18 @@ class HipBackend:
                                                      _ptr(out), out.size))
         return out if ok else None
 
+    def q6k_q8k_matvec(self, q6k, qs, d, num_rows: int, cols: int, out_len: Optional[int] = None) -> Optional[np.ndarray]:
+        """q6k_q8k_matvec_into (cpu/ops/q4k_q8k_dot/q6k.rs:15-92): Q6_K rows against a Q8_K activation (qs and d; no sums)."""
+        w = _u8(q6k)
+        qs = np.ascontiguousarray(qs, dtype=np.int8).reshape(-1)
+        d = _f32(d)
+        if d.size * 256 != qs.size:
+            return None
+        out = np.empty(num_rows if out_len is None else out_len, np.float32)
+        ok = self._some(lib.larql_hip_q6k_q8k_matvec(self._h, _ptr(w), w.size, _ptr(qs), qs.size, _ptr(d), num_rows, cols,
+                                                     _ptr(out), out.size))
+        return out if ok else None
+
     def q4k_dual_matvec(self, q4k_a, q4k_b, x, num_rows: int, hidden: int):
         a, b, x = _u8(q4k_a), _u8(q4k_b), _f32(x)
         oa, ob = np.empty(num_rows, np.float32), np.empty(num_rows, np.float32)

@@ -131,6 +131,7 @@ int kind_of_format(int format) {
         case LARQL_FMT_GGML_Q8_0: return KIND_Q8_0;
         case LARQL_FMT_Q6_K: return KIND_Q6K;
         case LARQL_FMT_Q4_K_Q8K: return KIND_Q4K_Q8K;
+        case LARQL_FMT_Q6_K_Q8K: return KIND_Q6K_Q8K;
         case LARQL_FMT_MXFP4: return KIND_MXFP4;
         case LARQL_FMT_Q4_0: return KIND_Q4_0;
         case LARQL_FMT_BF16: return KIND_BF16;
@@ -214,10 +215,10 @@ std::vector<std::vector<GemvJob>> group_by_kind(const std::vector<GemvJob> &jobs
     std::vector<GemvJob> jobs(jobs_in);
     for (GemvJob &j : jobs) j.kind = gemv_effective_kind(j);  // Q4_K rows the matrix-core kernel takes get their own launch
     std::vector<std::vector<GemvJob>> groups;
-    bool done[14] = {false, false, false, false, false, false, false, false, false, false, false, false, false, false};
+    bool done[15] = {};
     for (size_t i = 0; i < jobs.size(); i++) {
         const int kind = jobs[i].kind;
-        if (jobs[i].rows == 0 || kind < 0 || kind > 13 || done[kind]) continue;
+        if (jobs[i].rows == 0 || kind < 0 || kind > 14 || done[kind]) continue;
         done[kind] = true;
         std::vector<GemvJob> live;
         for (size_t t = i; t < jobs.size(); t++)
@@ -501,6 +502,23 @@ int larql_hip_q4k_q8k_matvec(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_le
     memcpy(packed.data() + cols + (cols / 256) * 4, sums, (cols / 32) * 2);
     const size_t need = (cols / 256) * 144 * num_rows;
     return host_matvec_multi(c, KIND_Q4K_Q8K, 1, &q4k, &need, nullptr, nullptr, &num_rows, cols, (const float *)packed.data(), packed.size(), &out);
+}
+
+int larql_hip_q6k_q8k_matvec(larql_hip_ctx *c, const uint8_t *q6k, size_t q6k_len, const int8_t *qs, size_t qs_len, const float *d,
+                             size_t num_rows, size_t cols, float *out, size_t out_len) {
+    if (!c || (!out && out_len)) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    // KernelShapeError::check with 210-byte blocks (cpu/ops/q4k_q8k_dot/q6k.rs:15-36)
+    const size_t need = (cols / 256) * 210 * num_rows;
+    if (out_len != num_rows || qs_len != cols || cols % 256 != 0 || q6k_len < need)
+        return fail(c, LARQL_REFUSED_SHAPE, "q6k_q8k_matvec: refused operands: out.len() %zu for %zu rows, activation length %zu for %zu cols, %zu weight bytes",
+                    out_len, num_rows, qs_len, cols, q6k_len);
+    if (num_rows == 0 || cols == 0) { for (size_t i = 0; i < out_len; i++) out[i] = 0.0f; return LARQL_OK; }
+    if (!q6k || !qs || !d) return LARQL_E_ARG;
+    std::vector<uint8_t> packed(q8k_bytes(cols), 0);  // [codes | scales | sums]: this kernel forms its own sums of codes
+    memcpy(packed.data(), qs, cols);
+    memcpy(packed.data() + cols, d, (cols / 256) * 4);
+    return host_matvec_multi(c, KIND_Q6K_Q8K, 1, &q6k, &need, nullptr, nullptr, &num_rows, cols, (const float *)packed.data(), packed.size(), &out);
 }
 
 int larql_hip_q4k_dual_matvec(larql_hip_ctx *c, const uint8_t *a, size_t a_len, const uint8_t *b, size_t b_len,
@@ -955,7 +973,7 @@ static int dev_job_from_public(larql_hip_ctx *c, const larql_hip_matvec_job &p, 
     if (kind < 0) return fail(c, LARQL_UNSUPPORTED, "matvec: format %d has no kernel", p.format);
     if (kind == KIND_MXFP4 && !p.aux) return fail(c, LARQL_E_ARG, "matvec: MXFP4 needs the scale stream");
     if (kind == KIND_Q4_0) return fail(c, LARQL_UNSUPPORTED, "matvec batch: Q4_0 goes through larql_hip_dev_matvec");
-    if ((kind == KIND_Q4K || kind == KIND_Q6K || kind == KIND_Q4K_Q8K) && p.k % 256 != 0)
+    if ((kind == KIND_Q4K || kind == KIND_Q6K || kind == KIND_Q4K_Q8K || kind == KIND_Q6K_Q8K) && p.k % 256 != 0)
         return fail(c, LARQL_REFUSED_SHAPE, "matvec: k not a multiple of 256");
     if (kind == KIND_Q4K_Q8K && p.k / 256 > 40) return fail(c, LARQL_UNSUPPORTED, "matvec: Q4_K x Q8_K rows longer than 10240 have no kernel");
     if (p.k % 32 != 0) return fail(c, LARQL_REFUSED_SHAPE, "matvec: k not a multiple of 32");

@@ -260,6 +260,60 @@ __device__ __forceinline__ float q6k_chunk_dot(const Q6KRaw &raw, const Q6KSlice
     return d * v;
 }
 
+// Q6_K against a Q8_K activation (q6k_q8k_matvec_scalar, larql-compute/src/cpu/ops/q4k_q8k_dot/q6k.rs:38-92): the same
+// 64-weight chunk per thread, but the activation is int8: the 6-bit codes (0..63) meet the codes of x in v_dot4_i32_i8,
+// the -32 goes through the sums of x's codes per 16-element group, and the four chunks of a super-block (four
+// neighbouring lanes) add their integer sums so that one of them can evaluate d_w*d_y*(f32)sum1 as the reference does.
+struct Q6KQ8Slice {
+    uint32_t y[16];  // codes of plane r (8 dwords), then plane r+2
+    int ysum[4];     // sums of the codes over the four 16-element groups, in that order
+    float dy;
+};
+
+__device__ __forceinline__ void q6k_q8k_load_x(Q6KQ8Slice &s, const uint8_t *q8k, uint32_t k, uint32_t c) {
+    const uint32_t sb = c >> 2, h = (c >> 1) & 1u, r = c & 1u;
+    g_u4p lo = (g_u4p)(q8k + (size_t)sb * 256 + h * 128 + r * 32);
+    g_u4p hi = (g_u4p)(q8k + (size_t)sb * 256 + h * 128 + (r + 2) * 32);
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const u32x4 a = lo[i], b = hi[i];
+        s.y[4 * i + 0] = a.x; s.y[4 * i + 1] = a.y; s.y[4 * i + 2] = a.z; s.y[4 * i + 3] = a.w;
+        s.y[8 + 4 * i + 0] = b.x; s.y[8 + 4 * i + 1] = b.y; s.y[8 + 4 * i + 2] = b.z; s.y[8 + 4 * i + 3] = b.w;
+    }
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        int sm = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) sm = __builtin_amdgcn_sdot4(0x01010101, (int)s.y[4 * g + i], sm, false);
+        s.ysum[g] = sm;
+    }
+    s.dy = *(const GLOBAL_AS float *)(q8k + k + (size_t)sb * 4);
+}
+
+// this chunk's integer share of its super-block's sum1
+__device__ __forceinline__ int q6k_q8k_chunk(const Q6KRaw &raw, const Q6KQ8Slice &s, const uint8_t *row, uint32_t c) {
+    const uint32_t sb = c >> 2, r = c & 1u;
+    const uint32_t mis = (uint32_t)(((uintptr_t)row + (size_t)sb * 210) & 2u), sh = mis * 8;
+    const uint32_t ssh = ((mis + 2 * r) & 2u) * 8;
+    const uint32_t s01 = __builtin_amdgcn_alignbit(raw.sc[1], raw.sc[0], ssh), s45 = raw.sc[1] >> ssh;
+    const int sc0 = (int)(int8_t)(s01 & 0xFF), sc1 = (int)(int8_t)((s01 >> 8) & 0xFF);
+    const int sc2 = (int)(int8_t)(s45 & 0xFF), sc3 = (int)(int8_t)((s45 >> 8) & 0xFF);
+    int acc[4] = {0, 0, 0, 0};
+    const uint32_t hs = 2 * r;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const uint32_t ql = __builtin_amdgcn_alignbit(raw.ql[i + 1], raw.ql[i], sh);
+        const uint32_t qh = __builtin_amdgcn_alignbit(raw.qh[i + 1], raw.qh[i], sh);
+        const uint32_t a = (ql & 0x0F0F0F0Fu) | (((qh >> hs) & 0x03030303u) << 4);              // plane r, elements 4i..4i+3
+        const uint32_t b = ((ql >> 4) & 0x0F0F0F0Fu) | (((qh >> (hs + 4)) & 0x03030303u) << 4);  // plane r+2
+        acc[i >> 2] = __builtin_amdgcn_sdot4((int)a, (int)s.y[i], acc[i >> 2], false);          // codes <= 63: positive as int8
+        acc[2 + (i >> 2)] = __builtin_amdgcn_sdot4((int)b, (int)s.y[8 + i], acc[2 + (i >> 2)], false);
+    }
+    // |sum (q-32)*y| <= 16*32*127 over a group: the products with the int8 scales fit 24-bit multiplies
+    return __mul24(sc0, acc[0] - 32 * s.ysum[0]) + __mul24(sc1, acc[1] - 32 * s.ysum[1]) +
+           __mul24(sc2, acc[2] - 32 * s.ysum[2]) + __mul24(sc3, acc[3] - 32 * s.ysum[3]);
+}
+
 // ---------------------------------------------------------------------------
 // MXFP4: one thread = one 32-element group: 16 packed bytes (element 2b in the
 // low nibble of byte b) + one e8m0 scale byte.  Value as mxfp4_loop computes it
@@ -1707,6 +1761,53 @@ __device__ __forceinline__ void run_q6k(const GemvJob &j, uint32_t p0, uint32_t 
 }
 
 template <int U>
+__device__ __forceinline__ void run_q6k_q8k(const GemvJob &j, uint32_t p0, uint32_t p1, float *part) {
+#pragma clang fp contract(off)
+    const uint32_t t = threadIdx.x, cpr = j.cpr, rpp = j.rpp, nsb = cpr >> 2;
+    const bool active = t < cpr * rpp;
+    const uint32_t c = active ? t % cpr : 0, rl = active ? t / cpr : 0;
+    Q6KQ8Slice xs;
+    q6k_q8k_load_x(xs, (const uint8_t *)j.x, (uint32_t)j.k, c);
+    const size_t row_bytes = j.row_bytes;
+    for (uint32_t tp = p0; tp < p1; tp += kTilePasses) {
+        const uint32_t tp_end = min(p1, tp + kTilePasses);
+        const uint32_t row_base = tp * rpp;
+        const uint32_t tile_rows = min((uint32_t)j.rows, tp_end * rpp) - row_base;
+        if (active) {
+            for (uint32_t lr = rl; lr < tile_rows; lr += rpp * U) {
+                Q6KRaw raw[U];
+                const uint8_t *rowp[U];
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    const uint32_t r = min(lr + u * rpp, tile_rows - 1) + row_base;
+                    rowp[u] = j.w + (size_t)r * row_bytes;
+                    raw[u] = q6k_load(rowp[u], c);
+                }
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    const uint32_t r = lr + u * rpp;
+                    int s1 = q6k_q8k_chunk(raw[u], xs, rowp[u], c);
+                    // the four chunks of a super-block are four neighbouring lanes (cpr % 4 == 0)
+                    s1 += __builtin_amdgcn_mov_dpp(s1, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+                    s1 += __builtin_amdgcn_mov_dpp(s1, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+                    float term = half_bits_to_float(raw[u].d) * xs.dy;       // d_w * d_y
+                    term = term * (float)s1;
+                    if ((c & 3u) == 0 && r < tile_rows) part[r * nsb + (c >> 2)] = term;
+                }
+            }
+        }
+        __syncthreads();
+        // a lane per row: acc += term, super-blocks in order (q6k.rs:63-89)
+        for (uint32_t r = t; r < tile_rows; r += blockDim.x) {
+            float acc = 0.f;
+            for (uint32_t sb = 0; sb < nsb; sb++) acc += part[r * nsb + sb];
+            ((g_f32wp)j.out)[row_base + r] = acc;
+        }
+        __syncthreads();
+    }
+}
+
+template <int U>
 __device__ __forceinline__ void run_mxfp4(const GemvJob &j, uint32_t p0, uint32_t p1, float *part) {
     const uint32_t t = threadIdx.x, cpr = j.cpr, rpp = j.rpp;
     const bool active = t < cpr * rpp;
@@ -1864,6 +1965,7 @@ __device__ __forceinline__ void gemv_body(const GemvLaunch &L, float *part) {
         else if (KIND == KIND_Q8_0) run_q8_0<U>(j, a, b, part);
         else if (KIND == KIND_MXFP4) run_mxfp4<U>(j, a, b, part);
         else if (KIND == KIND_Q6K) run_q6k<U>(j, a, b, part);
+        else if (KIND == KIND_Q6K_Q8K) run_q6k_q8k<U>(j, a, b, part);
         else if (KIND == KIND_Q4_0) run_q4_0<U>(j, a, b, part);
         else if (KIND == KIND_BF16) run_dense<U, 0>(j, a, b, part);
         else if (KIND == KIND_F16) run_dense<U, 1>(j, a, b, part);
@@ -1886,6 +1988,7 @@ LARQL_GEMV_KERNEL(gemv_mxfp4_u2_kernel, KIND_MXFP4, 2, 4)
 LARQL_GEMV_KERNEL(gemv_mxfp4_u4_kernel, KIND_MXFP4, 4, 4)
 LARQL_GEMV_KERNEL(gemv_q4_0_kernel, KIND_Q4_0, 4, 4)
 LARQL_GEMV_KERNEL(gemv_q6k_kernel, KIND_Q6K, 2, 3)
+LARQL_GEMV_KERNEL(gemv_q6k_q8k_kernel, KIND_Q6K_Q8K, 2, 4)
 LARQL_GEMV_KERNEL(gemv_bf16_kernel, KIND_BF16, 4, 4)
 LARQL_GEMV_KERNEL(gemv_f16_kernel, KIND_F16, 4, 4)
 LARQL_GEMV_KERNEL(gemv_f32_kernel, KIND_F32, 2, 4)
@@ -2060,7 +2163,7 @@ static int g_unroll = getenv("LARQL_HIP_UNROLL") ? atoi(getenv("LARQL_HIP_UNROLL
 static int g_threads = getenv("LARQL_HIP_THREADS") ? atoi(getenv("LARQL_HIP_THREADS")) : 0;
 static uint32_t chunk_elems(int kind) {
     switch (kind) {
-        case KIND_Q4K: case KIND_Q6K: return 64;
+        case KIND_Q4K: case KIND_Q6K: case KIND_Q6K_Q8K: return 64;
         case KIND_Q8_0: case KIND_MXFP4: case KIND_Q4_0: return 32;
         default: return 16;
     }
@@ -2204,7 +2307,7 @@ bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
     switch (j.kind) {
         case KIND_Q4K: j.row_bytes = (j.k / 256) * 144; break;
         case KIND_Q8_0: j.row_bytes = (j.k / 32) * 34; break;
-        case KIND_Q6K: if (j.k % 256 != 0) return false; j.row_bytes = (j.k / 256) * 210; break;
+        case KIND_Q6K: case KIND_Q6K_Q8K: if (j.k % 256 != 0) return false; j.row_bytes = (j.k / 256) * 210; break;
         case KIND_MXFP4: j.row_bytes = (j.k / 32) * 16; break;
         case KIND_Q4_0: j.row_bytes = (j.k / 32) * 18; break;
         case KIND_BF16: case KIND_F16: j.row_bytes = j.k * 2; break;
@@ -2416,6 +2519,7 @@ hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32
             break;
         case KIND_Q4_0: hipLaunchKernelGGL(gemv_q4_0_kernel, dim3(grid), dim3(threads), lds, stream, L); break;
         case KIND_Q6K: hipLaunchKernelGGL(gemv_q6k_kernel, dim3(grid), dim3(threads), lds, stream, L); break;
+        case KIND_Q6K_Q8K: hipLaunchKernelGGL(gemv_q6k_q8k_kernel, dim3(grid), dim3(threads), lds, stream, L); break;
         case KIND_BF16: hipLaunchKernelGGL(gemv_bf16_kernel, dim3(grid), dim3(threads), lds, stream, L); break;
         case KIND_F16: hipLaunchKernelGGL(gemv_f16_kernel, dim3(grid), dim3(threads), lds, stream, L); break;
         case KIND_F32: hipLaunchKernelGGL(gemv_f32_kernel, dim3(grid), dim3(threads), lds, stream, L); break;

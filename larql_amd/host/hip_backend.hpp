@@ -79,6 +79,11 @@ class HipBackend {
         return some(larql_hip_q4k_q8k_matvec(ctx_, q4k.ptr, q4k.len, a.qs.data(), a.qs.size(), a.d.data(), a.sums.data(), num_rows, cols,
                                              out.data(), out.size()), out);
     }
+    std::optional<std::vector<float>> q6k_q8k_matvec(Slice<uint8_t> q6k, const Q8KActivation &a, size_t num_rows, size_t cols) {
+        std::vector<float> out(num_rows);
+        return some(larql_hip_q6k_q8k_matvec(ctx_, q6k.ptr, q6k.len, a.qs.data(), a.qs.size(), a.d.data(), num_rows, cols, out.data(),
+                                             out.size()), out);
+    }
     std::optional<std::pair<std::vector<float>, std::vector<float>>> q4k_dual_matvec(Slice<uint8_t> a, Slice<uint8_t> b,
                                                                                        Slice<float> x, size_t num_rows,
                                                                                        size_t hidden) {

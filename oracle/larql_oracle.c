@@ -641,6 +641,40 @@ int lq_q4k_q8k_matvec(float *out, size_t out_len, const int8_t *qs, size_t qs_le
     return 0;
 }
 
+/* q6k_q8k_matvec_scalar — larql-compute/src/cpu/ops/q4k_q8k_dot/q6k.rs:38-92 (the reference its NEON kernel equals bit
+ * for bit): per super-block sum1 = sum over the 16 groups of scale_g * dot(q6 - 32, q8) in i32, acc += d_w*d_y*(f32)sum1,
+ * super-blocks in order.  Shape rule: KernelShapeError::check with 210-byte blocks; `out` is zero-filled first.
+ * Pinned by the reference's own test inputs and bound (tests/fused_and_q6k_paths.rs:87-110: within 1.2e-1 of the f32
+ * Q6_K path, which is itself pinned on the golden Q6_K bytes), a block worked by hand with distinct scales per group,
+ * linearity in d_y, and an independently written numpy restatement, bit for bit. */
+int lq_q6k_q8k_matvec(float *out, size_t out_len, const int8_t *qs, size_t qs_len, const float *d,
+                      const uint8_t *w, size_t w_len, size_t rows, size_t cols) {
+    size_t nb = cols / 256, row_bytes = nb * 210;
+    if (out_len != rows || qs_len != cols || cols % 256 != 0 || w_len < rows * row_bytes) return 1;
+    for (size_t r = 0; r < out_len; r++) out[r] = 0.0f;
+    if (rows == 0 || cols == 0) return 0;
+    for (size_t r = 0; r < rows; r++) {
+        float acc = 0.0f;
+        for (size_t sb = 0; sb < nb; sb++) {
+            const uint8_t *block = w + r * row_bytes + sb * 210;
+            float d_w = lq_f16_to_f32((uint16_t)(block[208] | (block[209] << 8)));
+            float d_y = d[sb];
+            int32_t sum1 = 0;
+            for (size_t g = 0; g < 16; g++) {
+                int8_t vals[16];
+                lq_q6k_subblock_vals(block, g, vals);
+                int32_t dot = 0;
+                for (int k = 0; k < 16; k++) dot += (int32_t)vals[k] * qs[sb * 256 + g * 16 + k];
+                sum1 += (int32_t)(int8_t)block[192 + g] * dot;
+            }
+            float t = d_w * d_y;
+            acc += t * (float)sum1;
+        }
+        out[r] = acc;
+    }
+    return 0;
+}
+
 /* larql-models/src/quant/ggml/quantize.rs:50-77.  Codes use the reciprocal
  * of the un-rounded f32 scale.
  * Pinned: byte-for-byte against the reference-held ggml golden blocks

@@ -57,6 +57,8 @@ int  lq_dequantize_q6_k(const uint8_t *data, size_t data_len, size_t n, float *o
 int  lq_quantize_x_to_q8k(const float *x, size_t n, int8_t *qs, float *d, int16_t *sums); /* cpu/ops/q4k_q8k_dot/q8k_activation.rs:84-109 */
 int  lq_q4k_q8k_matvec(float *out, size_t out_len, const int8_t *qs, size_t qs_len, const float *d, const int16_t *sums,
                        const uint8_t *w, size_t w_len, size_t rows, size_t cols); /* cpu/ops/q4k_q8k_dot/q4k_scalar.rs:15-84 */
+int  lq_q6k_q8k_matvec(float *out, size_t out_len, const int8_t *qs, size_t qs_len, const float *d,
+                       const uint8_t *w, size_t w_len, size_t rows, size_t cols); /* cpu/ops/q4k_q8k_dot/q6k.rs:38-92 */
 int  lq_q6k_matvec(const uint8_t *w, size_t w_len, const float *x, size_t rows, size_t hidden, float *out); /* cpu/ops/q6k_matvec.rs:45-91 */
 
 int  lq_quantize_q8_0(const float *data, size_t n, uint8_t *out);

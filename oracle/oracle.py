@@ -226,6 +226,20 @@ def q4k_q8k_matvec(w, qs, d, sums, rows: int, cols: int):
     return out
 
 
+def q6k_q8k_matvec(w, qs, d, rows: int, cols: int):
+    """q6k_q8k_matvec_scalar: None where the reference refuses the operands."""
+    w = _u8(w).ravel()
+    qs = np.ascontiguousarray(qs, dtype=np.int8).ravel()
+    d = _f32(d).ravel()
+    out = np.empty(rows, dtype=np.float32)
+    if d.size * 256 != qs.size:
+        return None
+    if _lib.lq_q6k_q8k_matvec(_p(out, _f32p), _sz(rows), _p(qs, _i8p), _sz(qs.size), _p(d, _f32p), _p(w, _u8p), _sz(w.size), _sz(rows),
+                              _sz(cols)):
+        return None
+    return out
+
+
 def quantize_q8_0(data) -> np.ndarray:
     data = _f32(data).ravel()
     out = np.empty(data.size // 32 * 34, dtype=np.uint8)

@@ -254,3 +254,28 @@ def q4k_q8k_matvec(w, qs, d, sums, rows, cols):
     for b in range(nb):
         acc = (acc + term[:, b]).astype(np.float32)
     return acc
+
+
+def q6k_q8k_matvec(w, qs, d, rows, cols):
+    """Q6_K x Q8_K integer-dot matvec from the layout description alone (ql[128] | qh[64] | 16 int8 scales | f16 d):
+    element half*128 + plane*32 + l has the low nibble of ql[half*64 + (plane&1)*32 + l] for plane < 2 and the high
+    nibble otherwise, and bits 2*plane, 2*plane+1 of qh[half*32 + l]; value = code - 32; scale per 16 elements."""
+    nb = cols // 256
+    blocks = np.asarray(w, np.uint8)[: rows * nb * 210].reshape(rows, nb, 210)
+    ql = blocks[:, :, :128].reshape(rows, nb, 2, 2, 32)          # [half][ql row][l]
+    qh = blocks[:, :, 128:192].reshape(rows, nb, 2, 32)
+    sc = blocks[:, :, 192:208].view(np.int8).astype(np.int64)    # [rows, nb, 16]
+    dw = f16_bits_to_f32(blocks[:, :, 208:210].copy().view(np.uint16)[:, :, 0])
+    vals = np.empty((rows, nb, 2, 4, 32), np.int64)
+    for plane in range(4):
+        nib = (ql[:, :, :, plane & 1, :] & 0x0F) if plane < 2 else (ql[:, :, :, plane & 1, :] >> 4)
+        hi = (qh >> (2 * plane)) & 3
+        vals[:, :, :, plane, :] = (nib | (hi << 4)).astype(np.int64) - 32
+    vals = vals.reshape(rows, nb, 16, 16)
+    y = np.asarray(qs, np.int8).reshape(nb, 16, 16).astype(np.int64)
+    sum1 = (sc * (vals * y[None]).sum(axis=3)).sum(axis=2)
+    term = ((dw * np.asarray(d, np.float32)[None, :]).astype(np.float32) * sum1.astype(np.float32)).astype(np.float32)
+    acc = np.zeros(rows, np.float32)
+    for b in range(nb):
+        acc = (acc + term[:, b]).astype(np.float32)
+    return acc

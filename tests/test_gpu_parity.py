@@ -257,6 +257,77 @@ def test_q4k_q8k_device_tier_plan_matches_host_tier(be, fmt):
     be.plan_destroy(plan)
 
 
+@pytest.mark.parametrize("rows,cols", [(2560, 10240), (1031, 2560), (262, 4096), (5, 512), (1, 256), (77, 7168), (4100, 768),
+                                       (33, 1792), (300, 3840), (19, 16384)])
+def test_q6k_q8k_matvec_bit_exact(be, rows, cols):
+    """q6k_q8k_matvec_scalar (q6k.rs:38-92): integer group dots, d_w*d_y*(f32)sum1 added in super-block order."""
+    w, x = weights(rows * 5 + cols, rows, cols)
+    q = O.quantize_q6_k(w)
+    qs, d, _ = O.quantize_x_to_q8k(x * F(1.75))
+    want = O.q6k_q8k_matvec(q, qs, d, rows, cols)
+    got = be.q6k_q8k_matvec(q, qs, d, rows, cols)
+    assert got is not None
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_q6k_q8k_matvec_extreme_codes_and_scales(be):
+    # codes 63 and 0 (q - 32 = +31 / -32), scales +127 / -128, activation codes +-127: the widest integer sums
+    rows, cols = 24, 1536
+    nb = cols // 256
+    rng = np.random.default_rng(5)
+    blocks = np.zeros((rows * nb, 210), np.uint8)
+    blocks[:, 0:192] = np.where(rng.random((rows * nb, 1)) < 0.5, 0xFF, 0x00).astype(np.uint8)
+    blocks[:, 192:208] = np.where(rng.random((rows * nb, 16)) < 0.5, 127, 128).astype(np.uint8)   # int8 +127 / -128
+    blocks[:, 208:210] = np.array([0.25], np.float16).view(np.uint8)
+    q = blocks.reshape(-1)
+    qs = np.where(rng.random(cols) < 0.5, -127, 127).astype(np.int8)
+    d = np.full(nb, 1.5, F)
+    want = O.q6k_q8k_matvec(q, qs, d, rows, cols)
+    got = be.q6k_q8k_matvec(q, qs, d, rows, cols)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    qs[:] = 127                                           # every product of one sign within a group
+    assert np.array_equal(be.q6k_q8k_matvec(q, qs, d, rows, cols).view(np.uint32),
+                          O.q6k_q8k_matvec(q, qs, d, rows, cols).view(np.uint32))
+
+
+def test_q6k_q8k_matvec_shape_rules(be):
+    # q6k_q8k_zero_dims_are_empty_and_short_weights_are_refused (fused_and_q6k_paths.rs:137-166)
+    w = O.quantize_q6_k(np.ones(2 * 512, F))
+    qs, d, _ = O.quantize_x_to_q8k(np.ones(512, F))
+    assert be.q6k_q8k_matvec(w, qs, d, 2, 512) is not None
+    assert be.q6k_q8k_matvec(w[:-1], qs, d, 2, 512) is None                   # short weight slab
+    q3, d3, _ = O.quantize_x_to_q8k(np.ones(768, F))
+    assert be.q6k_q8k_matvec(w, q3, d3, 2, 512) is None                       # activation of the wrong length
+    assert be.q6k_q8k_matvec(w, qs, d, 2, 512, out_len=3) is None             # output length != rows
+    z = be.q6k_q8k_matvec(np.zeros(0, np.uint8), np.zeros(0, np.int8), np.zeros(0, F), 3, 0)
+    assert z is not None and z.shape == (3,) and not z.any()
+
+
+def test_q6k_q8k_and_q4k_q8k_jobs_share_one_activation_in_a_plan(be, fmt):
+    # the reference's decode mixes Q4_K and Q6_K tensors against one quantised activation (q4k_q8k_matvec_parallel's format switch)
+    rng = np.random.default_rng(98)
+    k = 2560
+    xv = rng.standard_normal(k).astype(F)
+    buf = be.malloc(be.q8k_bytes(k) + 64)
+    assert be.dev_quantize_x_to_q8k(be.to_device(xv), k, buf)
+    a = O.quantize_x_to_q8k(xv)
+    jobs, outs, wants = [], [], []
+    for f, rows in ((fmt.FMT_Q6_K_Q8K, 513), (fmt.FMT_Q4_K_Q8K, 640), (fmt.FMT_Q6_K_Q8K, 40)):
+        wf = (rng.standard_normal(rows * k) * 0.05).astype(F)
+        q = O.quantize_q6_k(wf) if f == fmt.FMT_Q6_K_Q8K else O.quantize_q4_k(wf)
+        o = be.malloc(rows * 4)
+        jobs.append((f, be.to_device(q), None, buf, o, rows, k))
+        outs.append((o, rows))
+        wants.append(O.q6k_q8k_matvec(q, a[0], a[1], rows, k) if f == fmt.FMT_Q6_K_Q8K else O.q4k_q8k_matvec(q, *a, rows, k))
+    plan = be.plan_create(jobs)
+    assert plan is not None and be.plan_launch_count(plan) == 2
+    assert be.plan_run(plan) and be.plan_run(plan)
+    be.synchronize()
+    for (o, rows), want in zip(outs, wants):
+        assert np.array_equal(be.d2h(o, rows, F).view(np.uint32), want.view(np.uint32))
+    be.plan_destroy(plan)
+
+
 # ------------------------------------------------------------------ Q8_0
 @pytest.mark.parametrize("n,k", [(4099, 2560), (64, 10240), (9, 128), (1000, 2048), (17, 256), (333, 1792), (48, 2816),
                                  (531, 3840), (2050, 4096), (77, 5120), (40, 5376)])   # two column passes per wavefront; odd column count; just above

@@ -134,3 +134,54 @@ def test_q4k_q8k_matvec_shape_rules():
     assert O.q4k_q8k_matvec(np.concatenate([w, w]), *q, 2, 512) is not None   # longer slab is fine
     z = O.q4k_q8k_matvec(np.zeros(0, np.uint8), np.zeros(0, np.int8), np.zeros(0, F), np.zeros(0, np.int16), 3, 0)
     assert z is not None and z.shape == (3,) and not z.any()                  # zero dims give zeros
+
+
+# ------------------------------------------------------------------ the Q6_K twin
+def test_q6k_q8k_matvec_within_noise_of_the_f32_path_on_the_reference_inputs():
+    # q6k_q8k_matvec_matches_q6k_f32_dispatch_within_noise (fused_and_q6k_paths.rs:87-110): diff < 1.2e-1 on these inputs
+    rows, cols = 5, 512
+    x = np.array([np.sin(F(i) * F(0.017)) * F(1.5) for i in range(cols)], F)
+    w = O.quantize_q6_k(np.array([np.cos(F(i) * F(0.006)) * F(0.7) for i in range(rows * cols)], F))
+    qs, d, _ = O.quantize_x_to_q8k(x)
+    f32 = O.q6k_matvec(w, x, rows, cols)
+    q8 = O.q6k_q8k_matvec(w, qs, d, rows, cols)
+    assert np.all(np.abs(f32 - q8) < 1.2e-1)
+
+
+def test_q6k_q8k_matvec_hand_computed_block():
+    # every code 32 + 5 (low nibble 5, high bits 2), scale 3 for even groups and -2 for odd ones, d = 0.5; y = +2 / -1 per group
+    b = np.zeros(210, np.uint8)
+    b[:128] = 0x55
+    b[128:192] = 0xAA
+    b[192:208] = np.array([3, -2] * 8, np.int8).view(np.uint8)
+    b[208:210] = np.array([0.5], np.float16).view(np.uint8)
+    qs = np.concatenate([np.full(16, 2 if g % 3 == 0 else -1, np.int8) for g in range(16)])
+    d = np.array([0.25], F)
+    sum1 = sum((3 if g % 2 == 0 else -2) * 5 * 16 * (2 if g % 3 == 0 else -1) for g in range(16))
+    want = F(F(0.5) * F(0.25)) * F(sum1)
+    assert O.q6k_q8k_matvec(b, qs, d, 1, 256)[0] == want
+    assert O.q6k_q8k_matvec(b, qs, d * F(4), 1, 256)[0] == want * F(4)
+
+
+@pytest.mark.parametrize("rows,cols,seed", [(7, 1024, 0), (33, 2560, 1), (3, 10240, 2), (1, 256, 3)])
+def test_q6k_q8k_matvec_agrees_with_numpy_restatement_bit_for_bit(rows, cols, seed):
+    rng = np.random.default_rng(200 + seed)
+    w = O.quantize_q6_k((rng.standard_normal(rows * cols) * 0.05).astype(F))
+    qs, d, _ = O.quantize_x_to_q8k((rng.standard_normal(cols) * 2).astype(F))
+    a, b = O.q6k_q8k_matvec(w, qs, d, rows, cols), npr.q6k_q8k_matvec(w, qs, d, rows, cols)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    deq = O.dequantize_q6_k(w, rows * cols).reshape(rows, cols).astype(np.float64)
+    y = np.repeat(d.astype(np.float64), 256) * qs.astype(np.float64)
+    assert np.allclose(a, deq @ y, rtol=0, atol=1e-4 * np.abs(deq @ y).max() + 1e-6)
+
+
+def test_q6k_q8k_matvec_shape_rules():
+    # fused_and_q6k_paths.rs:137-166: zero dims zero the output, a short weight slab is refused
+    w = O.quantize_q6_k(np.ones(2 * 512, F))
+    qs, d, _ = O.quantize_x_to_q8k(np.ones(512, F))
+    assert O.q6k_q8k_matvec(w, qs, d, 2, 512) is not None
+    assert O.q6k_q8k_matvec(w[:-1], qs, d, 2, 512) is None
+    qs2, d2, _ = O.quantize_x_to_q8k(np.ones(768, F))
+    assert O.q6k_q8k_matvec(w, qs2, d2, 2, 512) is None
+    z = O.q6k_q8k_matvec(np.zeros(0, np.uint8), np.zeros(0, np.int8), np.zeros(0, F), 3, 0)
+    assert z is not None and z.shape == (3,) and not z.any()
