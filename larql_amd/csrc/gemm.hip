@@ -24,6 +24,7 @@ namespace larql {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int TM = 128, TN = 128, KS = 64, LDK = 72;  // tile rows, tile tokens, k per step, padded LDS row (bf16 elements)
 
@@ -158,6 +159,7 @@ __global__ void __launch_bounds__(256) q4k_gemm_kernel(const uint8_t *__restrict
 // ---------------------------------------------------------------------------
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 constexpr int LDM = 40;  // padded row of the 32-slot min tiles (f16 elements)
 
 // one block per token: scale, f16 terms, sub-block sums.  `x_is_bf16`: 16-bit inputs (exact in one term).
@@ -402,37 +404,38 @@ __global__ void __launch_bounds__(256) q4k_gemm_reduce_kernel(const float *__res
 // ---------------------------------------------------------------------------
 // The same arithmetic, software-pipelined (the kernel in use).
 //
-// One workgroup of 8 wavefronts per CU owns a 256-row x 128-token tile; every wavefront keeps a 64x64
-// quadrant.  Everything a step (64 k) needs from global memory was copied global -> LDS (global_load_lds,
+// One workgroup of 8 wavefronts per CU owns a 256-row x 128-token tile; a wavefront owns 32 of the rows against
+// all 128 tokens.  Everything a step (64 k) needs from global memory was copied global -> LDS (global_load_lds,
 // 16 bytes per lane, no registers involved) at least two steps before:
 //   * the f16 activations of a step, into a ring of four stages.  Rows are 128 bytes (64 f16) without
 //     padding; the 16-byte chunk c of row r is kept at position c ^ (r & 7), chosen on the global side of the
 //     copy, so that the eight lanes of an operand read phase hit eight different bank groups;
-//   * the raw weight bytes of a step (32 per row), into a ring of five stages;
+//   * the raw weight bytes of a step (32 per row), into a ring of five stages (a wavefront copies its own rows);
 //   * per super-block the 16-byte headers and the Sx of the tile's tokens; sum mn6*Sx is taken at the
 //     super-block's first step, d*D is folded in at its last.
-// The f16(sc6*q) operand exists once (256 rows x 64 k, chunk c of row r at c ^ swz(r), swz a bit permutation
-// that also spreads the converting threads over the banks).  A step has two halves with a barrier after each:
-// while the matrix cores work on k 0..31 the threads convert this step's k 32..63 (high nibbles) into the
-// other half of the operand, and while they work on k 32..63 the next step's k 0..31 (low nibbles) replace the
-// half just used.  No load returns into a register, so the compiler places no waits of its own (it would wait
-// for *all* outstanding loads as soon as register loads and LDS copies are in flight together); outstanding
-// copies are counted by hand: at the end of a step only the requests of the last two steps may still fly.
+// The f16(sc6*q) operand never exists in memory: lane (l16, kg) of an MFMA holds row l16, k 8kg .. 8kg+7 of a
+// 32-wide half, i.e. the low or the high nibbles of 8 raw bytes of that row, so every lane reads the 8 bytes of
+// its two rows once per step and converts them, in the MFMAs' shadow, into the operand of the next half.  Only
+// the activations cross wavefronts: one barrier per step.  No global load returns into a register, so the
+// compiler places no vmcnt waits of its own (it would wait for *all* outstanding loads as soon as register loads
+// and LDS copies are in flight together); outstanding copies are counted by hand: at the end of a step only the
+// requests of the last two steps may still fly.  For the same reason (an LDS copy in flight makes the compiler
+// wait for lgkmcnt(0) at every LDS read) the operand reads of the loop are written as instructions with counted
+// waits, P_LA reads ahead of the MFMA group that consumes them.
 // ---------------------------------------------------------------------------
 constexpr int PM = 256, PN = 128, PTHREADS = 512;
+constexpr int P_LA = 4;                                                         // operand reads in flight ahead of the MFMAs
 constexpr int P_NB = 4, P_NR = 5;                                               // ring depths: activations, raw weights
-constexpr int P_A_BYTES = PM * 128, P_B_STAGE = PN * 128, P_R_STAGE = PM * 32;  // bytes
-constexpr int P_A_OFF = 0, P_B_OFF = P_A_BYTES, P_R_OFF = P_B_OFF + P_NB * P_B_STAGE, P_H_OFF = P_R_OFF + P_NR * P_R_STAGE,
+constexpr int P_B_STAGE = PN * 128, P_R_STAGE = PM * 32;                        // bytes
+constexpr int P_B_OFF = 0, P_R_OFF = P_B_OFF + P_NB * P_B_STAGE, P_H_OFF = P_R_OFF + P_NR * P_R_STAGE,
               P_AM_OFF = P_H_OFF + PM * 32, P_BM_OFF = P_AM_OFF + PM * 32, P_D_OFF = P_BM_OFF + PN * 32,
-              P_DMIN_OFF = P_D_OFF + 2 * PM * 4, P_LDS_BYTES = P_DMIN_OFF + 2 * PM * 4;
+              P_DMIN_OFF = P_D_OFF + 2 * PM * 4, P_LOOP_BYTES = P_DMIN_OFF + 2 * PM * 4;
+constexpr int P_EP_LD = 36, P_EP_BYTES = 8 * PN * P_EP_LD * 4;                  // the results leave through LDS (see the epilogue)
+constexpr int P_LDS_BYTES = P_LOOP_BYTES > P_EP_BYTES ? P_LOOP_BYTES : P_EP_BYTES;
 static_assert(P_LDS_BYTES <= 160 * 1024, "one workgroup per CU");
 typedef __attribute__((address_space(3))) void *p_lds_vp;
 typedef const __attribute__((address_space(1))) void *p_g_vp;
 #define GEMM_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
-
-// position swizzle of the weight operand: bit 0 of the row picks the half of the row's eight chunk positions,
-// bits 1..2 the position inside it (a bijection of r & 7, so 8 consecutive rows still hit 8 bank groups)
-__device__ __forceinline__ uint32_t q4k_gemm_swz(uint32_t r) { return ((r & 1u) << 2) | ((r >> 1) & 3u); }
 
 __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_t *w, const uint16_t *xh, const uint16_t *sx,
                                                                     const float *__restrict__ tok_scale, float *__restrict__ out,
@@ -468,7 +471,7 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
     // compute role: a wavefront owns the 32 rows it converts, against all 128 tokens: the weight operand, the raw
     // bytes, the headers and the per-row constants never cross wavefronts, only the activations (and Sx) do
     const uint32_t wm = wave * 32;
-    const uint32_t l16 = lane & 15u, kg = lane >> 4, sw_a = q4k_gemm_swz(l16), sw_b = l16 & 7u;
+    const uint32_t l16 = lane & 15u, kg = lane >> 4, sw_b = l16 & 7u;
 
     // (requests past the end are clamped: same number of copies in flight, results unused)
     auto issue_raw = [&](uint32_t s) {
@@ -488,10 +491,14 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
         __builtin_amdgcn_global_load_lds((p_g_vp)((wt + (size_t)sbc * 144) + h_off), (p_lds_vp)(plds + P_H_OFF + wave * 1024), 16, 0, 0);
         __builtin_amdgcn_global_load_lds((p_g_vp)((st + (size_t)sbc * 32) + m_off), (p_lds_vp)(plds + P_BM_OFF + (wave & 3u) * 1024), 16, 0, 0);
     };
-    uint32_t hdr_y = 0, hdr_w = 0;  // the scale words of the super-block being converted
+    uint32_t hdr_y[2] = {0, 0}, hdr_w[2] = {0, 0};  // the scale words of this lane's two operand rows, super-block being converted
     auto stage_sb = [&](uint32_t par) {  // a super-block's header: scale words to registers, mn6 / d / dmin to LDS
         const u32x4 hdr = *reinterpret_cast<const u32x4 *>(plds + P_H_OFF + wave * 1024 + (lane >> 1) * 16);
-        hdr_y = hdr.y; hdr_w = hdr.w;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const u32x4 hi = *reinterpret_cast<const u32x4 *>(plds + P_H_OFF + wave * 1024 + (i * 16 + l16) * 16);
+            hdr_y[i] = hi.y; hdr_w[i] = hi.w;
+        }
         if (with_mins) {
             uint32_t mnw[4];
 #pragma unroll
@@ -511,14 +518,14 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
     };
     // scale of sub-block `sub` (0..7) of the current header as the packed-FMA operands (sc6, -1024*sc6)
     // (odd sub-blocks are the high nibbles: their masked value is 1024 + 16q, so the factor is sc6/16 and the offset -64*sc6)
-    auto scale_of = [&](uint32_t sub, f16x2 &sc2, f16x2 &off2) {
+    auto scale_of = [&](int i, uint32_t sub, _Float16 &sc1, _Float16 &off1) {
         const uint32_t sh = 8u * (sub & 3u);
-        const uint32_t pa = (hdr_y >> sh) & 0xFFu, pc = (hdr_w >> sh) & 0xFFu;
+        const uint32_t pa = (hdr_y[i] >> sh) & 0xFFu, pc = (hdr_w[i] >> sh) & 0xFFu;
         const uint32_t sc6 = sub < 4 ? (pa & 63u) : ((pc & 0x0Fu) | ((pa >> 6) << 4));
         const float f = (float)sc6;
         const _Float16 scf = (_Float16)((sub & 1u) ? f * 0.0625f : f), of = (_Float16)((sub & 1u) ? -64.0f * f : -1024.0f * f);
-        sc2 = (f16x2){scf, scf};
-        off2 = (f16x2){of, of};
+        sc1 = scf;
+        off1 = of;
     };
     // 4 raw bytes (nibble h) -> two dwords of f16(sc6*q), exact (sc6*q <= 945), as the pairs (k0, k2) and (k1, k3):
     // the nibbles of bytes 0 and 2 are masked in place into the mantissas of two f16 (1024 + q, or 1024 + 16q for
@@ -527,19 +534,33 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
     // instruction.
     uint32_t magic;
     asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
-    auto convert4 = [&](uint32_t raw, uint32_t h, f16x2 sc2, f16x2 off2, uint32_t &o0, uint32_t &o1) {
+    auto convert4 = [&](uint32_t raw, uint32_t h, _Float16 sc1, _Float16 off1, uint32_t &o0, uint32_t &o1) {
+        const f16x2 sc2 = {sc1, sc1}, off2 = {off1, off1};  // (broadcast by the instruction's operand selects, not by a pack)
         const uint32_t mask = h ? 0x00F000F0u : 0x000F000Fu;
         const f16x2 m02 = __builtin_bit_cast(f16x2, (raw & mask) | magic);
         const f16x2 m13 = __builtin_bit_cast(f16x2, ((raw >> 8) & mask) | magic);
         o0 = __builtin_bit_cast(uint32_t, m02 * sc2 + off2);
         o1 = __builtin_bit_cast(uint32_t, m13 * sc2 + off2);
     };
-    // where this thread's two chunks of k-half h go
-    uint8_t *const a_row = plds + P_A_OFF + sr * 128;
-    const uint32_t a_swz = q4k_gemm_swz(sr);
-    auto a_frag = [&](int kk, int i) {
-        return *reinterpret_cast<const f16x8 *>(plds + P_A_OFF + (wm + i * 16 + l16) * 128 + ((((uint32_t)kk * 4 + kg) ^ sw_a) << 4));
+    // The weight operand never exists in memory: lane (l16, kg) of an MFMA holds row l16, k 8kg .. 8kg+7 of a
+    // 32-wide half, which are the low (first half) or high (second half) nibbles of the row's raw bytes
+    // 8kg .. 8kg+7 of the step; the lane reads those 8 bytes of its two rows once per step and converts them
+    // into the operand of the next half while the matrix cores work on the current one.
+    //
+    // The operand reads of the main loop are written as instructions with hand-counted waits: while LDS copies
+    // are in flight the compiler's own wait for an LDS read is lgkmcnt(0), i.e. it would drain the reads issued
+    // ahead with the one that is needed.  LDS reads return in order, so "all but the last n" is exact.
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(p_lds_vp)plds;
+    const uint32_t raw_lane = lds0 + P_R_OFF + wave * 1024 + l16 * 32 + kg * 8;
+    auto raw_of = [&](uint32_t rs, u32x2 (&rq)[2]) {
+        const uint32_t a = raw_lane + (rs % P_NR) * P_R_STAGE;
+        asm volatile("ds_read_b64 %0, %1" : "=v"(rq[0]) : "v"(a));
+        asm volatile("ds_read_b64 %0, %1 offset:512" : "=v"(rq[1]) : "v"(a));
     };
+    const uint32_t b_lane = lds0 + P_B_OFF + l16 * 128;
+    uint32_t b_col[2];  // byte position of this lane's chunk in a token's row, for the two halves of a step
+#pragma unroll
+    for (int kk = 0; kk < 2; kk++) b_col[kk] = (((uint32_t)kk * 4 + kg) ^ sw_b) << 4;
 
     f32x4 acc[2][8], D[2][8];
 #pragma unroll
@@ -555,19 +576,19 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     stage_sb(0);
-    {
-        const u32x4 q = *reinterpret_cast<const u32x4 *>(plds + P_R_OFF + sr * 32 + part * 16);
-        const uint32_t qd[4] = {q.x, q.y, q.z, q.w};
-        f16x2 sc2, off2;
-        scale_of(0, sc2, off2);
-        uint32_t aw[8];
+    u32x2 rq[2];       // this lane's raw bytes of the step whose halves are being converted
+    uint32_t an[2][4]; // the operand of the coming half, rows l16 and 16 + l16
+    raw_of(0, rq);
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(rq[0]), "+v"(rq[1]));
 #pragma unroll
-        for (int n = 0; n < 4; n++) convert4(qd[n], 0, sc2, off2, aw[2 * n], aw[2 * n + 1]);
-        *reinterpret_cast<u32x4 *>(a_row + (((2 * part) ^ a_swz) << 4)) = (u32x4){aw[0], aw[1], aw[2], aw[3]};
-        *reinterpret_cast<u32x4 *>(a_row + (((2 * part + 1) ^ a_swz) << 4)) = (u32x4){aw[4], aw[5], aw[6], aw[7]};
+    for (int i = 0; i < 2; i++) {
+        _Float16 sc2, off2;
+        scale_of(i, 0, sc2, off2);
+        convert4(rq[i].x, 0, sc2, off2, an[i][0], an[i][1]);
+        convert4(rq[i].y, 0, sc2, off2, an[i][2], an[i][3]);
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_s_barrier();  // the mn6 / d / dmin that stage_sb wrote are visible
     asm volatile("" ::: "memory");
 
     uint32_t s = 0;
@@ -579,32 +600,21 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
             issue_raw(s + 4);
             issue_b(s + 3);
             if (g == 1) issue_sb(sb + 1);  // (after the barrier that ended g = 0: everybody is past this super-block's Sx)
-            const uint8_t *B = plds + P_B_OFF + (s % P_NB) * P_B_STAGE;
-            auto b_frag = [&](int kk, int jj) {
-                return *reinterpret_cast<const f16x8 *>(B + (jj * 16 + l16) * 128 + ((((uint32_t)kk * 4 + kg) ^ sw_b) << 4));
-            };
+            const uint32_t b_stage = b_lane + (s % P_NB) * P_B_STAGE;
             if (g == 0 && with_mins) {
-                // offsets of the super-block: sum_sub mn6 * Sx (A slots 2*sub+h = 32*mn6, B slots = Sx_h/32; slots 16..31 are zero)
-                const uint32_t kgc = min(kg, 1u);
-                f16x8 amf[2], bmf[8];
+                // offsets of the super-block: sum_sub mn6 * Sx as one 16-deep MFMA per block (A slots 2*sub+h = 32*mn6,
+                // B slots = Sx_h/32: lane (l16, kg) holds slots 4kg .. 4kg+3)
+                f16x4 amf[2], bmf[8];
 #pragma unroll
-                for (int i = 0; i < 2; i++) {
-                    u32x4 av = *reinterpret_cast<const u32x4 *>(plds + P_AM_OFF + (wm + i * 16 + l16) * 32 + kgc * 16);
-                    if (kg >= 2) av = (u32x4){0u, 0u, 0u, 0u};
-                    amf[i] = __builtin_bit_cast(f16x8, av);
-                }
+                for (int i = 0; i < 2; i++) amf[i] = *reinterpret_cast<const f16x4 *>(plds + P_AM_OFF + (wm + i * 16 + l16) * 32 + kg * 8);
 #pragma unroll
-                for (int jj = 0; jj < 8; jj++) {
-                    u32x4 bv = *reinterpret_cast<const u32x4 *>(plds + P_BM_OFF + (jj * 16 + l16) * 32 + kgc * 16);
-                    if (kg >= 2) bv = (u32x4){0u, 0u, 0u, 0u};
-                    bmf[jj] = __builtin_bit_cast(f16x8, bv);
-                }
+                for (int jj = 0; jj < 8; jj++) bmf[jj] = *reinterpret_cast<const f16x4 *>(plds + P_BM_OFF + (jj * 16 + l16) * 32 + kg * 8);
                 // (D is free here: the sixteen products go there back to back, then they are folded in)
 #pragma unroll
                 for (int i = 0; i < 2; i++)
 #pragma unroll
                     for (int jj = 0; jj < 8; jj++)
-                        D[i][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(amf[i], bmf[jj], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                        D[i][jj] = __builtin_amdgcn_mfma_f32_16x16x16f16(amf[i], bmf[jj], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
 #pragma unroll
                 for (int i = 0; i < 2; i++) {
                     const f32x4 mv = *reinterpret_cast<const f32x4 *>(plds + P_DMIN_OFF + (par * PM + wm + i * 16 + kg * 4) * 4);
@@ -614,39 +624,75 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
                         for (int e = 0; e < 4; e++) acc[i][jj][e] = __builtin_fmaf(-mv[e], D[i][jj][e], acc[i][jj][e]);
                 }
             }
+            // ---- the step's sixteen operand reads (two halves x eight token blocks) run P_LA groups ahead of the MFMAs that
+            //      use them, across the two halves; the raw bytes of the next step are requested before the first of them ----
+            u32x4 bf[16];
+            u32x2 rqn[2];
+            uint32_t b_addr[2];
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++) b_addr[kk] = b_stage + b_col[kk];
+#define LARQL_RD(G) case G: asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(bf[G]) : "v"(b_addr[(G) >> 3]), "n"(((G) & 7) * 2048)); break;
+            auto b_read = [&](int G) {
+                switch (G) { LARQL_RD(0) LARQL_RD(1) LARQL_RD(2) LARQL_RD(3) LARQL_RD(4) LARQL_RD(5) LARQL_RD(6) LARQL_RD(7)
+                             LARQL_RD(8) LARQL_RD(9) LARQL_RD(10) LARQL_RD(11) LARQL_RD(12) LARQL_RD(13) LARQL_RD(14) LARQL_RD(15) default: break; }
+            };
+#undef LARQL_RD
+            // operand G has arrived when at most the reads issued after it are outstanding (reads return in order; anything
+            // else issued in between only makes the wait stricter)
+#define LARQL_WT(N) case N: asm volatile("s_waitcnt lgkmcnt(" #N ")" : "+v"(bf[G])); break;
+            auto b_wait = [&](int G) {
+                switch (min(P_LA, 15 - G)) { LARQL_WT(0) LARQL_WT(1) LARQL_WT(2) LARQL_WT(3) LARQL_WT(4) LARQL_WT(5) LARQL_WT(6) LARQL_WT(7) LARQL_WT(8) default: break; }
+            };
+#undef LARQL_WT
+            asm volatile("" ::: "memory");  // (nothing of the above sinks below the counted reads)
+            __builtin_amdgcn_sched_barrier(0);
+            raw_of(s + 1, rqn);             // (its copy landed two steps ago: own rows, own copy)
+#pragma unroll
+            for (int G = 0; G < P_LA; G++) b_read(G);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int h = 0; h < 2; h++) {
                 // ---- half h: the matrix cores take k 32h .. 32h+31 of step s; the threads convert, for h = 0, this step's
                 //      k 32..63 (high nibbles of raw step s) and, for h = 1, the next step's k 0..31 (low nibbles of s+1).
                 //      Both halves of the operand belong to this wavefront alone: no barrier between them ----
-                if (h == 1 && g == 3) stage_sb(par ^ 1u);
-                __builtin_amdgcn_sched_barrier(0);
-                const uint32_t rs = s + h;                                  // raw step being converted
-                const uint32_t nib = 1 - h;                                 // its nibble
-                const u32x4 q = *reinterpret_cast<const u32x4 *>(plds + P_R_OFF + (rs % P_NR) * P_R_STAGE + sr * 32 + part * 16);
-                const uint32_t qd[4] = {q.x, q.y, q.z, q.w};
-                f16x2 sc2, off2;
-                scale_of(h == 0 ? 2 * g + 1 : 2 * ((g + 1) & 3), sc2, off2);
-                const uint32_t c0 = 4 * nib + 2 * part;                     // destination chunks c0, c0+1
-                f16x8 af[2], bf[8];
+                if (h == 1 && g == 3) {
+                    stage_sb(par ^ 1u);
+                    asm volatile("" ::: "memory");
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if (h == 1) { rq[0] = rqn[0]; rq[1] = rqn[1]; }
+                const uint32_t nib = 1 - h;                                 // nibble of the half being converted
+                const uint32_t nsub = h == 0 ? 2 * g + 1 : 2 * ((g + 1) & 3);
+                f16x8 af[2];
 #pragma unroll
-                for (int i = 0; i < 2; i++) af[i] = a_frag(h, i);
-                bf[0] = b_frag(h, 0);
-                bf[1] = b_frag(h, 1);
-                uint32_t aw[8];
+                for (int i = 0; i < 2; i++) af[i] = __builtin_bit_cast(f16x8, (u32x4){an[i][0], an[i][1], an[i][2], an[i][3]});
+                _Float16 sc2[2], off2[2];
                 __builtin_amdgcn_sched_barrier(0);
-                // eight groups of two MFMAs; every other one carries a quarter of the conversion, each an operand read two groups ahead
+                // eight groups of two MFMAs; six of them carry a piece of the conversion
 #pragma unroll
                 for (int jj = 0; jj < 8; jj++) {
-                    if (jj + 2 < 8) bf[jj + 2] = b_frag(h, jj + 2);
-                    if ((jj & 1) == 0) convert4(qd[jj >> 1], nib, sc2, off2, aw[jj], aw[jj + 1]);
-                    if ((jj & 3) == 3) {
-                        const int c = jj >> 2;
-                        *reinterpret_cast<u32x4 *>(a_row + (((c0 + c) ^ a_swz) << 4)) = (u32x4){aw[4 * c], aw[4 * c + 1], aw[4 * c + 2], aw[4 * c + 3]};
-                    }
+                    const int G = h * 8 + jj;
+                    if (G + P_LA < 16) b_read(G + P_LA);
+                    b_wait(G);
+                    // (these name what the group before produced: they keep each piece of the conversion between two
+                    // groups instead of wherever its first use is; the raw bytes came back before operand 0)
+                    if (G == 0) asm volatile("" : "+v"(rqn[0]), "+v"(rqn[1]));
+                    if (jj == 1) asm volatile("" : "+v"(sc2[0]), "+v"(off2[0]));
+                    if (jj == 2) asm volatile("" : "+v"(sc2[1]), "+v"(off2[1]));
+                    if (jj == 3) asm volatile("" : "+v"(an[0][0]), "+v"(an[0][1]));
+                    if (jj == 4) asm volatile("" : "+v"(an[0][2]), "+v"(an[0][3]));
+                    if (jj == 5) asm volatile("" : "+v"(an[1][0]), "+v"(an[1][1]));
+                    if (jj == 6) asm volatile("" : "+v"(an[1][2]), "+v"(an[1][3]));
+                    if (jj == 0) scale_of(0, nsub, sc2[0], off2[0]);
+                    if (jj == 1) scale_of(1, nsub, sc2[1], off2[1]);
+                    if (jj == 2) convert4(rq[0].x, nib, sc2[0], off2[0], an[0][0], an[0][1]);
+                    if (jj == 3) convert4(rq[0].y, nib, sc2[0], off2[0], an[0][2], an[0][3]);
+                    if (jj == 4) convert4(rq[1].x, nib, sc2[1], off2[1], an[1][0], an[1][1]);
+                    if (jj == 5) convert4(rq[1].y, nib, sc2[1], off2[1], an[1][2], an[1][3]);
+                    const f16x8 bv = __builtin_bit_cast(f16x8, bf[G]);
 #pragma unroll
                     for (int i = 0; i < 2; i++)  // (a super-block's first MFMAs start from zero: D is never cleared)
-                        D[i][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bf[jj], (g == 0 && h == 0) ? (f32x4){0.f, 0.f, 0.f, 0.f} : D[i][jj], 0, 0, 0);
+                        D[i][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bv, (g == 0 && h == 0) ? (f32x4){0.f, 0.f, 0.f, 0.f} : D[i][jj], 0, 0, 0);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 if (h == 1 && g == 3) {
@@ -662,9 +708,7 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
                     }
                 }
                 asm volatile("" ::: "memory");
-                if (h == 0) {
-                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own conversion stores before own operand reads
-                } else {
+                if (h == 1) {
                     // ---- end of step: only the copies requested in this step and the one before may still fly (3 per
                     //      step, 5 at g = 1); at g = 2 only this step's, so that the header requested at g = 1 is there
                     //      for the conversion that opens the next super-block ----
@@ -686,9 +730,8 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
     // groups) in its own 18 KB, then every lane stores 16 bytes of a 128-byte run of one token.
     __builtin_amdgcn_s_barrier();  // nobody's copies are still landing in what becomes another wavefront's block
     asm volatile("" ::: "memory");
-    constexpr uint32_t EP_LD = 36;
+    constexpr uint32_t EP_LD = P_EP_LD;
     float *blk = reinterpret_cast<float *>(plds) + wave * (PN * EP_LD);
-    static_assert(8 * PN * EP_LD * 4 <= P_LDS_BYTES, "the eight blocks fit");
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
