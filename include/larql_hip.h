@@ -130,6 +130,22 @@ int larql_hip_quantize_x_to_q8k(larql_hip_ctx *ctx, const float *x, size_t n, in
  * dims write zeros.  cols <= 10240 on this backend (longer: UNSUPPORTED). */
 int larql_hip_q4k_q8k_matvec(larql_hip_ctx *ctx, const uint8_t *q4k, size_t q4k_len, const int8_t *qs, size_t qs_len,
                              const float *d, const int16_t *sums, size_t num_rows, size_t cols, float *out, size_t out_len);
+/* q4k_q8k_gate_up_into — cpu/ops/q4k_q8k_dot/gate_up.rs:30-57 (shape checks :68-87):
+ * gate and up rows against one Q8_K activation in one launch; each output is
+ * bit-identical to larql_hip_q4k_q8k_matvec on its matrix (the reference holds its
+ * fused kernels to the scalar one bit for bit).  Both shape rules are checked
+ * before anything is written. */
+int larql_hip_q4k_q8k_gate_up(larql_hip_ctx *ctx, const uint8_t *gate_w, size_t gate_len, const uint8_t *up_w, size_t up_len,
+                              const int8_t *qs, size_t qs_len, const float *d, const int16_t *sums, size_t num_rows,
+                              size_t cols, float *gate_out, float *up_out, size_t out_len);
+/* q4k_q8k_gemm_into — cpu/ops/q4k_q8k_dot/gemm.rs:42-112: out[s*rows + r] = W[r,:] . X[s,:]
+ * for `seq` activation rows quantised to Q8_K (`qs` seq*cols codes, `d` seq*cols/256,
+ * `sums` seq*cols/32, row after row); every activation row bit-identical to the
+ * row-at-a-time matvec (gemm.rs:141-170).  One launch, one job per activation row.
+ * The reference asserts out_len == seq*rows, cols % 256 == 0 and the slab length;
+ * here those are REFUSED_SHAPE. */
+int larql_hip_q4k_q8k_gemm(larql_hip_ctx *ctx, const uint8_t *q4k, size_t q4k_len, const int8_t *qs, const float *d,
+                           const int16_t *sums, size_t seq, size_t num_rows, size_t cols, float *out, size_t out_len);
 /* q6k_q8k_matvec_into / q4k_q8k_matvec_parallel with format "Q6_K" —
  * cpu/ops/q4k_q8k_dot/q6k.rs:15-92, dispatch.rs:100-148: per super-block
  * acc += d_w*d_y*(f32)(sum over the 16 groups of scale_g * dot(q6 - 32, q8)), in

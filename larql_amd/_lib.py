@@ -56,6 +56,8 @@ SIGNATURES = {
     "larql_hip_quantize_x_to_q8k": (ci, [vp, vp, sz, vp, vp, vp]),
     "larql_hip_q4k_q8k_matvec": (ci, [vp, vp, sz, vp, sz, vp, vp, sz, sz, vp, sz]),
     "larql_hip_q6k_q8k_matvec": (ci, [vp, vp, sz, vp, sz, vp, sz, sz, vp, sz]),
+    "larql_hip_q4k_q8k_gate_up": (ci, [vp, vp, sz, vp, sz, vp, sz, vp, vp, sz, sz, vp, vp, sz]),
+    "larql_hip_q4k_q8k_gemm": (ci, [vp, vp, sz, vp, vp, vp, sz, sz, sz, vp, sz]),
     "larql_hip_q8k_bytes": (sz, [sz]),
     "larql_hip_dev_quantize_x_to_q8k": (ci, [vp, vp, sz, vp]),
     "larql_hip_q4k_dual_matvec": (ci, [vp, vp, sz, vp, sz, vp, sz, sz, sz, vp, vp, sz]),

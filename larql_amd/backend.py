@@ -142,6 +142,32 @@ class HipBackend:
                                                      _ptr(out), out.size))
         return out if ok else None
 
+    def q4k_q8k_gate_up(self, gate_w, up_w, qs, d, sums, num_rows: int, cols: int):
+        """q4k_q8k_gate_up_into (cpu/ops/q4k_q8k_dot/gate_up.rs:30-57) -> (gate_out, up_out) or None."""
+        gw, uw = _u8(gate_w), _u8(up_w)
+        qs = np.ascontiguousarray(qs, dtype=np.int8).reshape(-1)
+        d = _f32(d)
+        sums = np.ascontiguousarray(sums, dtype=np.int16).reshape(-1)
+        if d.size * 256 != qs.size or sums.size * 32 != qs.size:
+            return None
+        go, uo = np.empty(num_rows, np.float32), np.empty(num_rows, np.float32)
+        ok = self._some(lib.larql_hip_q4k_q8k_gate_up(self._h, _ptr(gw), gw.size, _ptr(uw), uw.size, _ptr(qs), qs.size, _ptr(d), _ptr(sums),
+                                                      num_rows, cols, _ptr(go), _ptr(uo), num_rows))
+        return (go, uo) if ok else None
+
+    def q4k_q8k_gemm(self, q4k, acts, num_rows: int, cols: int) -> Optional[np.ndarray]:
+        """q4k_q8k_gemm_into (cpu/ops/q4k_q8k_dot/gemm.rs:42-112): `acts` is a sequence of (qs, d, sums); -> [seq, rows]."""
+        w = _u8(q4k)
+        seq = len(acts)
+        if any(np.asarray(a[0]).size != cols for a in acts):
+            return None
+        qs = np.ascontiguousarray(np.concatenate([np.asarray(a[0], np.int8).reshape(-1) for a in acts])) if seq else np.zeros(0, np.int8)
+        d = np.ascontiguousarray(np.concatenate([_f32(a[1]) for a in acts])) if seq else np.zeros(0, np.float32)
+        sums = np.ascontiguousarray(np.concatenate([np.asarray(a[2], np.int16).reshape(-1) for a in acts])) if seq else np.zeros(0, np.int16)
+        out = np.empty(seq * num_rows, np.float32)
+        ok = self._some(lib.larql_hip_q4k_q8k_gemm(self._h, _ptr(w), w.size, _ptr(qs), _ptr(d), _ptr(sums), seq, num_rows, cols, _ptr(out), out.size))
+        return out.reshape(seq, num_rows) if ok else None
+
     def q6k_q8k_matvec(self, q6k, qs, d, num_rows: int, cols: int, out_len: Optional[int] = None) -> Optional[np.ndarray]:
         """q6k_q8k_matvec_into (cpu/ops/q4k_q8k_dot/q6k.rs:15-92): Q6_K rows against a Q8_K activation (qs and d; no sums)."""
         w = _u8(q6k)

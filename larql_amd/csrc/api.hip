@@ -485,6 +485,12 @@ int larql_hip_quantize_x_to_q8k(larql_hip_ctx *c, const float *x, size_t n, int8
     return sub.finish();
 }
 
+static void pack_q8k(uint8_t *dst, const int8_t *qs, const float *d, const int16_t *sums, size_t cols) {
+    memcpy(dst, qs, cols);  // the activation travels in its device layout: [codes | scales | sums]
+    memcpy(dst + cols, d, (cols / 256) * 4);
+    memcpy(dst + cols + (cols / 256) * 4, sums, (cols / 32) * 2);
+}
+
 int larql_hip_q4k_q8k_matvec(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, const int8_t *qs, size_t qs_len, const float *d,
                              const int16_t *sums, size_t num_rows, size_t cols, float *out, size_t out_len) {
     if (!c || (!out && out_len)) return LARQL_E_ARG;
@@ -495,13 +501,69 @@ int larql_hip_q4k_q8k_matvec(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_le
     if (num_rows == 0 || cols == 0) { for (size_t i = 0; i < out_len; i++) out[i] = 0.0f; return LARQL_OK; }
     if (!q4k || !qs || !d || !sums) return LARQL_E_ARG;
     if (cols / 256 > 40) return fail(c, LARQL_UNSUPPORTED, "q4k_q8k_matvec: rows longer than 10240 have no kernel");
-    // the activation travels in its device layout: [codes | scales | sums]
     std::vector<uint8_t> packed(q8k_bytes(cols));
-    memcpy(packed.data(), qs, cols);
-    memcpy(packed.data() + cols, d, (cols / 256) * 4);
-    memcpy(packed.data() + cols + (cols / 256) * 4, sums, (cols / 32) * 2);
+    pack_q8k(packed.data(), qs, d, sums, cols);
     const size_t need = (cols / 256) * 144 * num_rows;
     return host_matvec_multi(c, KIND_Q4K_Q8K, 1, &q4k, &need, nullptr, nullptr, &num_rows, cols, (const float *)packed.data(), packed.size(), &out);
+}
+
+int larql_hip_q4k_q8k_gate_up(larql_hip_ctx *c, const uint8_t *gate_w, size_t gate_len, const uint8_t *up_w, size_t up_len,
+                              const int8_t *qs, size_t qs_len, const float *d, const int16_t *sums, size_t num_rows, size_t cols,
+                              float *gate_out, float *up_out, size_t out_len) {
+    if (!c || ((!gate_out || !up_out) && out_len)) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    // both halves are checked before anything is written (gate_up.rs:68-87): a refusal touches neither output
+    if (!q4k_shape_ok(out_len, num_rows, qs_len, cols, gate_len) || !q4k_shape_ok(out_len, num_rows, qs_len, cols, up_len))
+        return fail(c, LARQL_REFUSED_SHAPE, "q4k_q8k_gate_up: refused operands: out.len() %zu for %zu rows, activation length %zu for %zu cols, %zu / %zu weight bytes",
+                    out_len, num_rows, qs_len, cols, gate_len, up_len);
+    if (num_rows == 0 || cols == 0) { for (size_t i = 0; i < out_len; i++) { gate_out[i] = 0.0f; up_out[i] = 0.0f; } return LARQL_OK; }
+    if (!gate_w || !up_w || !qs || !d || !sums) return LARQL_E_ARG;
+    if (cols / 256 > 40) return fail(c, LARQL_UNSUPPORTED, "q4k_q8k_gate_up: rows longer than 10240 have no kernel");
+    std::vector<uint8_t> packed(q8k_bytes(cols));
+    pack_q8k(packed.data(), qs, d, sums, cols);
+    const size_t need = (cols / 256) * 144 * num_rows;
+    const uint8_t *w[2] = {gate_w, up_w};
+    const size_t needs[2] = {need, need}, rows[2] = {num_rows, num_rows};
+    float *outs[2] = {gate_out, up_out};
+    return host_matvec_multi(c, KIND_Q4K_Q8K, 2, w, needs, nullptr, nullptr, rows, cols, (const float *)packed.data(), packed.size(), outs);
+}
+
+int larql_hip_q4k_q8k_gemm(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, const int8_t *qs, const float *d, const int16_t *sums,
+                           size_t seq, size_t num_rows, size_t cols, float *out, size_t out_len) {
+    if (!c || (!out && out_len)) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    const size_t need = (cols / 256) * 144 * num_rows;
+    if (out_len != seq * num_rows || cols % 256 != 0 || q4k_len < need)  // (the reference asserts these)
+        return fail(c, LARQL_REFUSED_SHAPE, "q4k_q8k_gemm: refused operands: out.len() %zu for %zu x %zu, %zu cols, %zu weight bytes", out_len, seq,
+                    num_rows, cols, q4k_len);
+    if (seq == 0 || num_rows == 0) return LARQL_OK;
+    if (cols == 0) { for (size_t i = 0; i < out_len; i++) out[i] = 0.0f; return LARQL_OK; }
+    if (!q4k || !qs || !d || !sums) return LARQL_E_ARG;
+    if (cols / 256 > 40) return fail(c, LARQL_UNSUPPORTED, "q4k_q8k_gemm: rows longer than 10240 have no kernel");
+    if (seq > 65536) return fail(c, LARQL_UNSUPPORTED, "q4k_q8k_gemm: more than 65536 activation rows");
+    HIPCHECK(c, hipSetDevice(c->device));
+    // one launch: a job per activation row against the one resident copy of the weights (the reference runs the
+    // row-at-a-time kernel per activation row and holds the result to it bit for bit)
+    const size_t stride = (q8k_bytes(cols) + 63) & ~(size_t)63;
+    std::vector<uint8_t> packed(stride * seq);
+    for (size_t s = 0; s < seq; s++)
+        pack_q8k(packed.data() + s * stride, qs + s * cols, d + s * (cols / 256), sums + s * (cols / 32), cols);
+    int rc = upload(c, c->x, (const float *)packed.data(), packed.size());
+    if (rc) return rc;
+    rc = ensure(c, c->out, out_len * sizeof(float) + 64);
+    if (rc) return rc;
+    const uint8_t *dw = nullptr;
+    rc = resolve_weights(c, q4k, need, c->w[0], &dw);
+    if (rc) return rc;
+    std::vector<GemvJob> jobs;
+    jobs.reserve(seq);
+    for (size_t s = 0; s < seq; s++)
+        jobs.push_back(make_job(KIND_Q4K_Q8K, dw, nullptr, (const uint8_t *)c->x.p + s * stride, (float *)c->out.p + s * num_rows, num_rows, cols));
+    Submission sub(c);
+    rc = enqueue_jobs(c, jobs);
+    if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
+    HIPCHECK(c, hipMemcpyAsync(out, c->out.p, out_len * sizeof(float), hipMemcpyDeviceToHost, c->stream));
+    return sub.finish();
 }
 
 int larql_hip_q6k_q8k_matvec(larql_hip_ctx *c, const uint8_t *q6k, size_t q6k_len, const int8_t *qs, size_t qs_len, const float *d,

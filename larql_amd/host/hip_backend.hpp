@@ -79,6 +79,25 @@ class HipBackend {
         return some(larql_hip_q4k_q8k_matvec(ctx_, q4k.ptr, q4k.len, a.qs.data(), a.qs.size(), a.d.data(), a.sums.data(), num_rows, cols,
                                              out.data(), out.size()), out);
     }
+    std::optional<std::pair<std::vector<float>, std::vector<float>>> q4k_q8k_gate_up(Slice<uint8_t> gate_w, Slice<uint8_t> up_w,
+                                                                                       const Q8KActivation &a, size_t num_rows,
+                                                                                       size_t cols) {
+        std::vector<float> g(num_rows), u(num_rows);
+        if (larql_hip_q4k_q8k_gate_up(ctx_, gate_w.ptr, gate_w.len, up_w.ptr, up_w.len, a.qs.data(), a.qs.size(), a.d.data(), a.sums.data(),
+                                      num_rows, cols, g.data(), u.data(), num_rows) != LARQL_OK)
+            return std::nullopt;
+        return std::make_pair(std::move(g), std::move(u));
+    }
+    // q4k_q8k_gemm_into: [seq, rows] from `seq` quantised activation rows
+    std::optional<std::vector<float>> q4k_q8k_gemm(Slice<uint8_t> q4k, const std::vector<Q8KActivation> &acts, size_t num_rows, size_t cols) {
+        std::vector<int8_t> qs; std::vector<float> d; std::vector<int16_t> sums;
+        for (const Q8KActivation &a : acts) {
+            if (a.qs.size() != cols || a.d.size() != cols / 256 || a.sums.size() != cols / 32) return std::nullopt;
+            qs.insert(qs.end(), a.qs.begin(), a.qs.end()); d.insert(d.end(), a.d.begin(), a.d.end()); sums.insert(sums.end(), a.sums.begin(), a.sums.end());
+        }
+        std::vector<float> out(acts.size() * num_rows);
+        return some(larql_hip_q4k_q8k_gemm(ctx_, q4k.ptr, q4k.len, qs.data(), d.data(), sums.data(), acts.size(), num_rows, cols, out.data(), out.size()), out);
+    }
     std::optional<std::vector<float>> q6k_q8k_matvec(Slice<uint8_t> q6k, const Q8KActivation &a, size_t num_rows, size_t cols) {
         std::vector<float> out(num_rows);
         return some(larql_hip_q6k_q8k_matvec(ctx_, q6k.ptr, q6k.len, a.qs.data(), a.qs.size(), a.d.data(), num_rows, cols, out.data(),

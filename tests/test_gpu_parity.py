@@ -303,6 +303,48 @@ def test_q6k_q8k_matvec_shape_rules(be):
     assert z is not None and z.shape == (3,) and not z.any()
 
 
+def test_q4k_q8k_gate_up_equals_two_matvecs_bit_for_bit(be):
+    # q8k_gate_up_fused_matches_separate_matvecs (fused_and_q6k_paths.rs:7-50) at a decode shape and a ragged one
+    for rows, cols, seed in ((10240, 2560, 3), (37, 768, 4)):
+        rng = np.random.default_rng(seed)
+        gw = O.quantize_q4_k((rng.standard_normal(rows * cols) * 0.03).astype(F))
+        uw = O.quantize_q4_k((rng.standard_normal(rows * cols) * 0.03).astype(F))
+        a = O.quantize_x_to_q8k(rng.standard_normal(cols).astype(F))
+        got = be.q4k_q8k_gate_up(gw, uw, *a, rows, cols)
+        assert got is not None
+        assert np.array_equal(got[0].view(np.uint32), O.q4k_q8k_matvec(gw, *a, rows, cols).view(np.uint32))
+        assert np.array_equal(got[1].view(np.uint32), O.q4k_q8k_matvec(uw, *a, rows, cols).view(np.uint32))
+    # a short gate or up slab refuses the pair (fused_and_q6k_paths.rs:296-337); zero dims give zeros
+    a = O.quantize_x_to_q8k(np.full(256, 0.5, F))
+    full, short = np.zeros(2 * 144, np.uint8), np.zeros(144, np.uint8)
+    assert be.q4k_q8k_gate_up(short, full, *a, 2, 256) is None
+    assert be.q4k_q8k_gate_up(full, short, *a, 2, 256) is None
+    assert be.q4k_q8k_gate_up(full, full, *a, 2, 256) is not None
+    z = be.q4k_q8k_gate_up(np.zeros(0, np.uint8), np.zeros(0, np.uint8), np.zeros(0, np.int8), np.zeros(0, F), np.zeros(0, np.int16), 4, 0)
+    assert z is not None and not z[0].any() and not z[1].any() and z[0].shape == (4,)
+
+
+def test_q4k_q8k_gemm_rows_equal_the_row_at_a_time_matvec(be):
+    # gemm_is_bit_identical_to_row_at_a_time_matvec (gemm.rs:141-170), on the reference's own inputs and a larger case
+    rows, cols, seq = 96, 512, 7
+    w = O.quantize_q4_k(np.array([((i * 31 + 7) % 23) * 0.01 - 0.11 for i in range(rows * cols)], F))
+    xs = [np.array([((s * 13 + c * 3) % 19) * 0.01 - 0.09 for c in range(cols)], F) for s in range(seq)]
+    acts = [O.quantize_x_to_q8k(x) for x in xs]
+    got = be.q4k_q8k_gemm(w, acts, rows, cols)
+    assert got is not None and got.shape == (seq, rows)
+    for s in range(seq):
+        assert np.array_equal(got[s].view(np.uint32), O.q4k_q8k_matvec(w, *acts[s], rows, cols).view(np.uint32))
+    rng = np.random.default_rng(11)
+    rows, cols, seq = 1031, 2560, 33
+    w = O.quantize_q4_k((rng.standard_normal(rows * cols) * 0.03).astype(F))
+    acts = [O.quantize_x_to_q8k(rng.standard_normal(cols).astype(F)) for _ in range(seq)]
+    got = be.q4k_q8k_gemm(w, acts, rows, cols)
+    for s in (0, 16, 32):
+        assert np.array_equal(got[s].view(np.uint32), O.q4k_q8k_matvec(w, *acts[s], rows, cols).view(np.uint32))
+    assert be.q4k_q8k_gemm(w[:-1], acts, rows, cols) is None            # short slab
+    assert be.q4k_q8k_gemm(w, [], rows, cols).shape == (0, rows)        # no activation rows: nothing to do
+
+
 def test_q6k_q8k_and_q4k_q8k_jobs_share_one_activation_in_a_plan(be, fmt):
     # the reference's decode mixes Q4_K and Q6_K tensors against one quantised activation (q4k_q8k_matvec_parallel's format switch)
     rng = np.random.default_rng(98)
