@@ -19,6 +19,10 @@
 // count in index order).  The <= 64 winners are gathered in LDS and one
 // wavefront orders them best-first with a bitonic sort done by cross-lane
 // shuffles.  Cost is a handful of passes over the row, whatever its order.
+// Rows of up to 16384 scores (every gate matrix) are read once: a thread keeps
+// its up to 16 ordered scores in registers and all passes run from there (the
+// passes are short, so from memory each would cost a dependent load latency
+// per 64 scores of a wavefront); longer rows (a vocabulary) are streamed.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -84,7 +88,9 @@ __device__ __forceinline__ uint64_t make_key(float s, uint32_t idx, int *nan_fla
     return ((uint64_t)ord << 32) | (uint32_t)(~idx);
 }
 
-template <bool BY_ABS>
+constexpr int kTopkCached = 16;  // rounds of 64 scores per wavefront held in registers
+
+template <bool BY_ABS, bool CACHED>
 __global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restrict__ scores, uint32_t n, uint32_t k,
                                                             uint32_t *__restrict__ idx_out, float *__restrict__ val_out,
                                                             uint32_t *__restrict__ count_out, int *nan_flag) {
@@ -98,6 +104,28 @@ __global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restr
     const uint32_t perw = ((n + kTopkWaves * 64 - 1) / (kTopkWaves * 64)) * 64;
     const uint32_t w0 = min(n, wave * perw), w1 = min(n, w0 + perw);
 
+    // the ordered score of index i (0: nothing there), from the register copy or from memory
+    uint32_t cache[CACHED ? kTopkCached : 1];
+    if (CACHED) {
+#pragma unroll
+        for (int it = 0; it < kTopkCached; it++) {
+            const uint32_t i = w0 + it * 64 + lane;
+            cache[it] = i < w1 ? (uint32_t)(make_key<BY_ABS>(s[i], i, nan_flag) >> 32) : 0u;
+        }
+    }
+    // f(ord, i) for every index of this wavefront, 64 at a time, all lanes taking part in every round
+    auto for_each = [&](auto &&f, int *flag) {
+        if (CACHED) {
+#pragma unroll
+            for (int it = 0; it < kTopkCached; it++) f(cache[it], w0 + it * 64 + lane);
+        } else {
+            for (uint32_t base = w0; base < w1; base += 64) {
+                const uint32_t i = base + lane;
+                f(i < w1 ? (uint32_t)(make_key<BY_ABS>(s[i], i, flag) >> 32) : 0u, i);
+            }
+        }
+    };
+
     if (tid < 64) winners[tid] = 0;
     if (tid == 0) { sh_prefix = 0; sh_need = k; sh_nwin = 0; }
     // ---- radix select of the k-th largest ordered score: 8 bits per pass, top byte first ----
@@ -106,11 +134,10 @@ __global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restr
         if (tid < 256) hist[tid] = 0;
         __syncthreads();
         const uint32_t prefix = sh_prefix;
-        for (uint32_t i = w0 + lane; i < w1; i += 64) {
-            const uint32_t ord = (uint32_t)(make_key<BY_ABS>(s[i], i, pass == 0 ? nan_flag : nullptr) >> 32);
+        for_each([&](uint32_t ord, uint32_t) {
             // 64-bit shift: the first pass compares nothing (shift by 32)
             if (ord != 0 && ((uint64_t)ord >> (sh + 8)) == ((uint64_t)prefix >> (sh + 8))) atomicAdd(&hist[(ord >> sh) & 255u], 1u);
-        }
+        }, pass == 0 ? nan_flag : nullptr);
         __syncthreads();
         if (wave == 0) {
             // lane l holds bins 255-4l .. 252-4l (descending); find the bin where the running count reaches `need`
@@ -150,20 +177,14 @@ __global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restr
     // ---- rank the ties in index order: per-wavefront counts, then ballots inside the wavefront ----
     uint32_t my_ties = 0;
     if (!take_all)
-        for (uint32_t base = w0; base < w1; base += 64) {
-            const uint32_t i = base + lane;
-            const bool tie = i < w1 && (uint32_t)(make_key<BY_ABS>(s[i], i, nullptr) >> 32) == T;
-            my_ties += (uint32_t)__popcll(__ballot(tie));
-        }
+        for_each([&](uint32_t ord, uint32_t) { my_ties += (uint32_t)__popcll(__ballot(ord != 0 && ord == T)); }, nullptr);
     if (lane == 0) wave_ties[wave] = my_ties;
     __syncthreads();
     uint32_t tie_rank = 0;  // ties at lower indices than this wavefront's current 64
     for (uint32_t w = 0; w < wave; w++) tie_rank += wave_ties[w];
     // ---- gather the winners ----
-    for (uint32_t base = w0; base < w1; base += 64) {
-        const uint32_t i = base + lane;
-        const uint64_t key = i < w1 ? make_key<BY_ABS>(s[i], i, nullptr) : 0;
-        const uint32_t ord = (uint32_t)(key >> 32);
+    for_each([&](uint32_t ord, uint32_t i) {
+        const uint64_t key = ((uint64_t)ord << 32) | (uint32_t)(~i);
         bool in = ord != 0 && ord > T;
         if (!take_all) {
             const bool tie = ord != 0 && ord == T;
@@ -176,7 +197,7 @@ __global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restr
             const uint32_t pos = atomicAdd(&sh_nwin, 1u);
             if (pos < 64) winners[pos] = key;
         }
-    }
+    }, nullptr);
     __syncthreads();
     if (wave == 0) {
         const uint64_t top = sort_desc(winners[lane], lane);
@@ -196,12 +217,11 @@ size_t topk_workspace_bytes(uint32_t, uint32_t, uint32_t) { return 0; }
 hipError_t topk_launch(hipStream_t stream, const float *scores, uint32_t batch, uint32_t n, uint32_t k, bool by_abs,
                        uint32_t *idx_out, float *val_out, uint32_t *count_out, int *nan_flag, void *, size_t) {
     if (batch == 0) return hipSuccess;
-    if (by_abs)
-        hipLaunchKernelGGL(topk_kernel<true>, dim3(batch), dim3(kTopkThreads), 0, stream, scores, n, k, idx_out, val_out,
-                           count_out, nan_flag);
-    else
-        hipLaunchKernelGGL(topk_kernel<false>, dim3(batch), dim3(kTopkThreads), 0, stream, scores, n, k, idx_out, val_out,
-                           count_out, nan_flag);
+    const bool cached = n <= (uint32_t)(kTopkWaves * 64 * kTopkCached);
+#define LARQL_TOPK(ABS, C) hipLaunchKernelGGL((topk_kernel<ABS, C>), dim3(batch), dim3(kTopkThreads), 0, stream, scores, n, k, idx_out, val_out, count_out, nan_flag)
+    if (by_abs) { if (cached) LARQL_TOPK(true, true); else LARQL_TOPK(true, false); }
+    else { if (cached) LARQL_TOPK(false, true); else LARQL_TOPK(false, false); }
+#undef LARQL_TOPK
     return hipGetLastError();
 }
 
