@@ -20,9 +20,11 @@
 // wavefront orders them best-first with a bitonic sort done by cross-lane
 // shuffles.  Cost is a handful of passes over the row, whatever its order.
 // Rows of up to 16384 scores (every gate matrix) are read once: a thread keeps
-// its up to 16 ordered scores in registers and all passes run from there (the
-// passes are short, so from memory each would cost a dependent load latency
-// per 64 scores of a wavefront); longer rows (a vocabulary) are streamed.
+// its up to 16 ordered scores in registers, and a bound with at least 64 scores
+// at or above it (the smallest maximum of 64 slices of the row) usually leaves
+// a few hundred candidates, which are ranked directly; the radix passes remain
+// for rows with more than 1024 candidates and for longer rows (a vocabulary),
+// which are streamed.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -89,6 +91,7 @@ __device__ __forceinline__ uint64_t make_key(float s, uint32_t idx, int *nan_fla
 }
 
 constexpr int kTopkCached = 16;  // rounds of 64 scores per wavefront held in registers
+constexpr int kTopkCandidates = kTopkThreads;  // candidates of the short way: one per thread
 
 template <bool BY_ABS, bool CACHED>
 __global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restrict__ scores, uint32_t n, uint32_t k,
@@ -97,7 +100,9 @@ __global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restr
     __shared__ uint32_t hist[256];
     __shared__ uint32_t wave_ties[kTopkWaves];
     __shared__ uint64_t winners[64];
-    __shared__ uint32_t sh_prefix, sh_need, sh_nwin;
+    __shared__ uint32_t sh_prefix, sh_need, sh_nwin, sh_ncand;
+    __shared__ uint32_t group_max[64];
+    __shared__ uint64_t cand[CACHED ? kTopkCandidates : 1];
     const uint32_t row = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const float *s = scores + (size_t)row * n;
     // wavefront w owns the contiguous indices [w0, w1), 64 at a time (lane = index within the 64)
@@ -127,7 +132,58 @@ __global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restr
     };
 
     if (tid < 64) winners[tid] = 0;
-    if (tid == 0) { sh_prefix = 0; sh_need = k; sh_nwin = 0; }
+    if (tid == 0) { sh_prefix = 0; sh_need = k; sh_nwin = 0; sh_ncand = 0; }
+    if (CACHED) {
+        // ---- short way for a row held in registers.  The 64 groups of 16 lanes each own a slice of the row; the
+        //      smallest of the 64 group maxima, L, has at least 64 scores at or above it (one per group), so the
+        //      winners are among the scores >= L: a few hundred of a typical row.  Those are collected and each one
+        //      counts the candidates with a larger key: that count is its place in the output.  A row whose
+        //      candidates do not fit (sorted input, a group without valid scores) takes the radix passes below. ----
+        uint32_t gmax = 0;
+#pragma unroll
+        for (int it = 0; it < kTopkCached; it++) gmax = max(gmax, cache[it]);
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) gmax = max(gmax, (uint32_t)__shfl_xor((int)gmax, o, 64));
+        if ((lane & 15u) == 0) group_max[wave * 4 + (lane >> 4)] = gmax;
+        __syncthreads();
+        uint32_t L = group_max[lane];
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) L = min(L, (uint32_t)__shfl_xor((int)L, o, 64));
+        if (L != 0) {
+            // a wavefront reserves room for all its candidates at once, then places them round by round
+            uint32_t mine = 0;
+#pragma unroll
+            for (int it = 0; it < kTopkCached; it++) mine += (uint32_t)__popcll(__ballot(cache[it] >= L));
+            uint32_t base = 0;
+            if (lane == 0 && mine) base = atomicAdd(&sh_ncand, mine);
+            base = (uint32_t)__builtin_amdgcn_readfirstlane((int)base);
+#pragma unroll
+            for (int it = 0; it < kTopkCached; it++) {
+                const bool c = cache[it] >= L;
+                const uint64_t m = __ballot(c);
+                const uint32_t pos = base + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
+                if (c && pos < (uint32_t)kTopkCandidates) cand[pos] = ((uint64_t)cache[it] << 32) | (uint32_t)(~(w0 + it * 64 + lane));
+                base += (uint32_t)__popcll(m);
+            }
+            __syncthreads();
+            const uint32_t nc = sh_ncand;
+            if (nc <= (uint32_t)kTopkCandidates) {  // (uniform over the workgroup)
+                if (tid < nc) {
+                    const uint64_t key = cand[tid];
+                    uint32_t rank = 0;
+                    for (uint32_t j = 0; j < nc; j++) rank += cand[j] > key ? 1u : 0u;
+                    if (rank < k) {
+                        const uint32_t idx = ~(uint32_t)key;
+                        idx_out[(size_t)row * k + rank] = idx;
+                        val_out[(size_t)row * k + rank] = s[idx];
+                    }
+                }
+                if (tid == 0) count_out[row] = min(k, nc);
+                return;
+            }
+        }
+        __syncthreads();
+    }
     // ---- radix select of the k-th largest ordered score: 8 bits per pass, top byte first ----
     for (int pass = 0; pass < 4; pass++) {
         const int sh = 24 - 8 * pass;

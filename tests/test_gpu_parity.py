@@ -555,6 +555,41 @@ def test_gate_knn_edge_cases(be, fmt):
     assert [i for i, _ in be.gate_knn(fmt.FMT_F32, eye, xt, 4, 256, 2)] == [0, 1]
 
 
+@pytest.mark.parametrize("case", ["normal", "sorted", "constant", "coarse", "tie_block", "max_cached", "streamed", "ragged"])
+def test_top_k_selection_paths(be, fmt, case):
+    # top_k_by_abs on prescribed score rows (scores = gate[:, 0] through a unit residual), over the selection paths
+    # of the kernel: candidates ranked directly, the radix passes (sorted / constant rows have too many candidates),
+    # rows streamed from memory.  Ties go to the lower index, so the expected list is unique.
+    rng = np.random.default_rng(len(case))
+    n, k = 10240, 64
+    if case == "normal":
+        sc = rng.standard_normal(n)
+    elif case == "sorted":
+        sc = np.linspace(3.0, -3.0, n)
+    elif case == "constant":
+        sc = np.full(n, -0.75)
+    elif case == "coarse":
+        sc = np.round(rng.standard_normal(n) * 2) / 2            # many exact ties everywhere
+    elif case == "tie_block":
+        sc = rng.standard_normal(n) * 0.1
+        sc[rng.choice(n, 100, replace=False)] = 5.0              # 100 equal scores straddle the K boundary
+        sc[rng.choice(n, 20, replace=False)] = -7.0
+    elif case == "max_cached":
+        n = 16384; sc = rng.standard_normal(n)
+    elif case == "streamed":
+        n = 16385; sc = rng.standard_normal(n)
+    else:
+        n = 1000; k = 7; sc = rng.standard_normal(n)
+    sc = sc.astype(F)
+    hidden = 32
+    gate = np.zeros((n, hidden), F); gate[:, 0] = sc
+    x = np.zeros(hidden, F); x[0] = 1.0
+    hits = be.gate_knn(fmt.FMT_F32, gate, x, n, hidden, k)
+    order = np.lexsort((np.arange(n), -np.abs(sc)))[:k]
+    assert [i for i, _ in hits] == order.tolist()
+    assert [v for _, v in hits] == sc[order].tolist()
+
+
 def test_q4k_matvec_topk_by_value(be):
     rows, cols = 5000, 512
     w, x = weights(31, rows, cols)
