@@ -284,10 +284,19 @@ def run_c4(be, fmt, args):
             be.dev_fill_normal(tmp, per, seed + e, 0.02)
             be.dev_quantize_mxfp4(tmp, H if name != "down" else H, I if name != "down" else I, p + e * per // 2, s + e * per // 32)
         bufs[name] = (p, s)
-    bank = fmt.Mxfp4Experts(bufs["gate"][0], bufs["gate"][1], bufs["up"][0], bufs["up"][1], bufs["down"][0], bufs["down"][1], E, H, I,
-                            7.0, 1.702)
+    # the same experts as one fused gate_up region each, gate on the even and up on the odd rows (what a GPT-OSS checkpoint ships)
+    fp, fs = be.malloc(E * per + 64), be.malloc(E * per // 16 + 64)
+    tmp2 = be.malloc(2 * per * 4)
+    for e in range(E):
+        be.dev_fill_normal(tmp2, 2 * per, 0x5EED04C0 + e, 0.02)
+        be.dev_quantize_mxfp4(tmp2, 2 * I, H, fp + e * per, fs + e * per // 16)
+    be.free(tmp2)
+    banks = {"separate": fmt.Mxfp4Experts(bufs["gate"][0], bufs["gate"][1], bufs["up"][0], bufs["up"][1], bufs["down"][0], bufs["down"][1],
+                                          E, H, I, 7.0, 1.702, 0),
+             "interleaved": fmt.Mxfp4Experts(fp, fs, None, None, bufs["down"][0], bufs["down"][1], E, H, I, 7.0, 1.702, 1)}
     expert_bytes = 3 * (per // 2 + per // 32)
-    for T in (1, 16):
+    for T, layout in ((1, "separate"), (1, "interleaved"), (16, "separate"), (16, "interleaved")):
+        bank = banks[layout]
         x, lg = be.malloc(T * H * 4 + 64), be.malloc(T * E * 4 + 64)
         be.dev_fill_normal(x, T * H, 0x5EED04F0 + T, 1.0)
         be.dev_fill_normal(lg, T * E, 0x5EED04E0 + T, 1.0)
@@ -308,6 +317,11 @@ def run_c4(be, fmt, args):
         for (e, w) in O.router_select(lv[0], k):
             for name in ("gate", "up", "down"):
                 mats[name] = (be.d2h(bufs[name][0] + e * per // 2, per // 2, np.uint8), be.d2h(bufs[name][1] + e * per // 32, per // 32, np.uint8))
+            if layout == "interleaved":
+                G = H // 32
+                fpe, fse = be.d2h(fp + e * per, per, np.uint8).reshape(2 * I, G * 16), be.d2h(fs + e * per // 16, per // 16, np.uint8).reshape(2 * I, G)
+                mats["gate"] = (fpe[0::2].reshape(-1).copy(), fse[0::2].reshape(-1).copy())
+                mats["up"] = (fpe[1::2].reshape(-1).copy(), fse[1::2].reshape(-1).copy())
             g = O.mxfp4_gemv(*mats["gate"], xv[0], I, H); u = O.mxfp4_gemv(*mats["up"], xv[0], I, H)
             h = np.array([O.clamped_glu(float(a), float(b)) for a, b in zip(g, u)], np.float32)
             acc = (acc + np.float32(w) * O.mxfp4_gemv(*mats["down"], h, H, I)).astype(np.float32)
@@ -317,9 +331,9 @@ def run_c4(be, fmt, args):
         ms = _timeit(be, block, args.steps)
         algo = distinct * expert_bytes + T * (8 * H + 4 * E)
         med, nrep = _cpu_time(lambda: O.mxfp4_gemv(*mats["gate"], xv[0], I, H), args.cpu_seconds / 4)
-        _emit(f"MXFP4 MoE expert block us (32 experts, top-4, batch {T})", round(ms * 1e3, 2), "us/block", ms, args.steps, 2,
+        _emit(f"MXFP4 MoE expert block us (32 experts, top-4, batch {T}, gate/up {layout})", round(ms * 1e3, 2), "us/block", ms, args.steps, 2,
               {"workload": f"BASELINE configs[3]: MXFP4 experts 32 x (gate, up, down 2880x2880), top-4, batch {T}",
-               "distinct_experts": distinct, "launches_per_block": 5, "GBps_over_distinct_expert_bytes": round(algo / ms / 1e6, 1),
+               "gate_up_layout": layout, "distinct_experts": distinct, "launches_per_block": 5 if T > 1 else 4, "GBps_over_distinct_expert_bytes": round(algo / ms / 1e6, 1),
                "us_per_expert_matvec": round(ms * 1e3 / (3 * T * k), 2), "verified_rel_l2_vs_oracle": rel},
               {"kernel": "gemv_mxfp4 (gate/up + down launches)", "bound": "hbm", "achieved": round(algo / ms / 1e6, 1), "peak": HBM_PEAK_GBS,
                "unit": "GB/s", "frac": round(algo / ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": None},

@@ -331,6 +331,13 @@ typedef struct {
     const uint8_t *gate_packed, *gate_scales, *up_packed, *up_scales, *down_packed, *down_scales;
     size_t n_experts, hidden, inter;
     float limit, alpha; /* MoeGateRule::ClampedGlu — pipeline/moe.rs:88-92 (GPT-OSS: 7, 1.702) */
+    /* MoeFusedRowLayout — pipeline/moe.rs:294-332.  0 = the gate and up projections are given
+     * apart (ContiguousHalves: up_* = gate_* + inter rows of the same region).  1 = Interleaved,
+     * what a GPT-OSS checkpoint ships: gate_packed / gate_scales hold each expert's fused
+     * [2*inter, hidden/32] rows with gate = rows 0, 2, 4, ... and up = rows 1, 3, 5, ...
+     * (FusedHalf::fused_row, larql-models/src/quant/mxfp4.rs:179-191); up_* are not read.
+     * The fused rows are walked in place, one pass over 2*inter rows per (token, expert). */
+    int gate_up_interleaved;
 } larql_hip_mxfp4_experts;
 /* The expert block of cpu_moe_forward (cpu/ops/moe/forward.rs:201-270) for
  * MXFP4 banks, which the CPU tier refuses (forward.rs:69-75): per token and

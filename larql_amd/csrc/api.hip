@@ -1214,18 +1214,25 @@ int larql_hip_dev_moe_mxfp4(larql_hip_ctx *c, const larql_hip_mxfp4_experts *ban
     if (workspace_bytes < larql_hip_moe_mxfp4_workspace_bytes(tokens, k, hidden, inter))
         return fail(c, LARQL_REFUSED_SHAPE, "moe_mxfp4: workspace too small");
     if (!x || !experts || !weights || !out || !workspace) return LARQL_E_ARG;
+    if (!bank->gate_packed || !bank->gate_scales || !bank->down_packed || !bank->down_scales ||
+        (!bank->gate_up_interleaved && (!bank->up_packed || !bank->up_scales)))
+        return LARQL_E_ARG;
     HIPCHECK(c, hipSetDevice(c->device));
     const size_t slots = tokens * k;
     float *g = (float *)workspace, *u = g + slots * inter, *h = u + slots * inter, *d = h + slots * inter;
-    const uint64_t gu_w_stride = inter * (hidden / 32) * 16, gu_s_stride = inter * (hidden / 32);
+    // fused: every expert's gate_up region is one matrix of 2*inter interleaved rows (gate even, up odd), walked in
+    // place by one job per slot; its 2*inter results (g0 u0 g1 u1 ...) fill the slot's share of the g and u areas
+    const bool fused = bank->gate_up_interleaved != 0;
+    const size_t gu_rows = fused ? 2 * inter : inter;
+    const uint64_t gu_w_stride = gu_rows * (hidden / 32) * 16, gu_s_stride = gu_rows * (hidden / 32);
     const uint64_t dn_w_stride = hidden * (inter / 32) * 16, dn_s_stride = hidden * (inter / 32);
     // Several tokens: slots that chose the same expert share its weights two at a time.  The job lists are built on
     // the device from the router's choice (moe_plan_kernel) into the workspace's spare activation area.
     {
-        GemvJob tg = make_job(KIND_MXFP4, bank->gate_packed, bank->gate_scales, x, g, inter, hidden);
-        GemvJob tu = make_job(KIND_MXFP4, bank->up_packed, bank->up_scales, x, u, inter, hidden);
+        GemvJob tg = make_job(KIND_MXFP4, bank->gate_packed, bank->gate_scales, x, g, gu_rows, hidden);
+        GemvJob tu = fused ? tg : make_job(KIND_MXFP4, bank->up_packed, bank->up_scales, x, u, inter, hidden);
         GemvJob td = make_job(KIND_MXFP4, bank->down_packed, bank->down_scales, g, d, hidden, inter);
-        td.x_glu = u; td.glu_limit = bank->limit; td.glu_alpha = bank->alpha;
+        td.x_glu = fused ? g : u; td.glu_limit = bank->limit; td.glu_alpha = bank->alpha;
         const size_t table_bytes = slots * 3 * sizeof(GemvJob) + 64;
         const bool mfma = gemv_effective_kind(tg) == KIND_MXFP4_MFMA && gemv_effective_kind(td) == KIND_MXFP4_MFMA;
         static const bool pairing = !(getenv("LARQL_HIP_MOE_PAIRS") && atoi(getenv("LARQL_HIP_MOE_PAIRS")) == 0);
@@ -1240,7 +1247,7 @@ int larql_hip_dev_moe_mxfp4(larql_hip_ctx *c, const larql_hip_mxfp4_experts *ban
                 P.kind = KIND_MXFP4_MFMA;
                 P.threads = gemv_pick_threads(&tj, 1);
                 if (P.threads == 0 || !gemv_job_geometry(tj, P.threads)) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: unsupported geometry");
-                const uint64_t max_jobs = which == 0 ? 2 * slots : slots;
+                const uint64_t max_jobs = which == 0 && !fused ? 2 * slots : slots;
                 if (max_jobs * tj.n_pass > 0x7FFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: launch too large");
                 memset(&P.L, 0, sizeof P.L);
                 P.L.table = which == 0 ? gu_table : dn_table;
@@ -1251,8 +1258,8 @@ int larql_hip_dev_moe_mxfp4(larql_hip_ctx *c, const larql_hip_mxfp4_experts *ban
             }
             if (!gemv_job_geometry(tu, Pg.threads)) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: unsupported geometry");
             HIPCHECK(c, moe_plan_launch(c->stream, experts, (uint32_t)slots, (uint32_t)k, (uint32_t)bank->n_experts, tg, tu, td, gu_w_stride,
-                                        gu_s_stride, dn_w_stride, dn_s_stride, (uint32_t)hidden, (uint32_t)inter, gu_table, hdr, dn_table,
-                                        hdr + 2));
+                                        gu_s_stride, dn_w_stride, dn_s_stride, (uint32_t)hidden, (uint32_t)inter, fused, gu_table, hdr,
+                                        dn_table, hdr + 2));
             HIPCHECK(c, gemv_launch(c->stream, Pg.kind, Pg.L, Pg.threads, Pg.grid, Pg.lds));
             HIPCHECK(c, gemv_launch(c->stream, Pd.kind, Pd.L, Pd.threads, Pd.grid, Pd.lds));
             HIPCHECK(c, weighted_sum_launch(c->stream, d, weights, out, (uint32_t)tokens, (uint32_t)k, (uint32_t)hidden));
@@ -1262,22 +1269,28 @@ int larql_hip_dev_moe_mxfp4(larql_hip_ctx *c, const larql_hip_mxfp4_experts *ban
     std::vector<GemvJob> jobs;
     for (size_t s = 0; s < slots; s++) {
         const size_t t = s / k;
-        GemvJob a = make_job(KIND_MXFP4, bank->gate_packed, bank->gate_scales, x + t * hidden, g + s * inter, inter, hidden);
+        GemvJob a = make_job(KIND_MXFP4, bank->gate_packed, bank->gate_scales, x + t * hidden, g + s * gu_rows, gu_rows, hidden);
         a.sel = experts + s; a.w_sel_stride = gu_w_stride; a.aux_sel_stride = gu_s_stride;
+        jobs.push_back(a);
+        if (fused) continue;
         GemvJob b = make_job(KIND_MXFP4, bank->up_packed, bank->up_scales, x + t * hidden, u + s * inter, inter, hidden);
         b.sel = experts + s; b.w_sel_stride = gu_w_stride; b.aux_sel_stride = gu_s_stride;
-        jobs.push_back(a); jobs.push_back(b);
+        jobs.push_back(b);
     }
     int rc = enqueue_jobs(c, jobs);
     if (rc) return rc;
     // the gated activation is applied by the down projection itself where the matrix-core kernel serves it
     const bool fuse_glu = gemv_effective_kind(make_job(KIND_MXFP4, bank->down_packed, bank->down_scales, g, d, hidden, inter)) != KIND_MXFP4;
-    if (!fuse_glu) HIPCHECK(c, clamped_glu_launch(c->stream, g, u, h, slots * inter, bank->limit, bank->alpha));
+    if (!fuse_glu) {
+        if (fused) HIPCHECK(c, clamped_glu_interleaved_launch(c->stream, g, h, slots * inter, bank->limit, bank->alpha));
+        else HIPCHECK(c, clamped_glu_launch(c->stream, g, u, h, slots * inter, bank->limit, bank->alpha));
+    }
     jobs.clear();
     for (size_t s = 0; s < slots; s++) {
-        GemvJob a = make_job(KIND_MXFP4, bank->down_packed, bank->down_scales, fuse_glu ? g + s * inter : h + s * inter, d + s * hidden,
+        const float *gx = fused ? g + s * 2 * inter : g + s * inter;
+        GemvJob a = make_job(KIND_MXFP4, bank->down_packed, bank->down_scales, fuse_glu ? gx : h + s * inter, d + s * hidden,
                              hidden, inter);
-        if (fuse_glu) { a.x_glu = u + s * inter; a.glu_limit = bank->limit; a.glu_alpha = bank->alpha; }
+        if (fuse_glu) { a.x_glu = fused ? gx : u + s * inter; a.glu_limit = bank->limit; a.glu_alpha = bank->alpha; }
         a.sel = experts + s; a.w_sel_stride = dn_w_stride; a.aux_sel_stride = dn_s_stride;
         jobs.push_back(a);
     }

@@ -1009,11 +1009,18 @@ __device__ __forceinline__ Mx4Step mx4_setup_step(const GemvJob &j, uint32_t ste
         const float *x = j.x + (int64_t)(q * j.x_stride);
         float2_t v = {0.f, 0.f};
         if (i0 + 2 <= k) {  // k is even: a pair is inside or outside
-            v = *(const GLOBAL_AS float2_t *)(x + i0);
+            float2_t u = {0.f, 0.f};
+            if (j.x_glu == j.x) {
+                // gate and up values interleaved (the result rows of a fused gate_up matrix walked in place): g0 u0 g1 u1
+                const f32x4 w = *(const GLOBAL_AS f32x4 *)(x + 2 * (size_t)i0);
+                v.x = w.x; v.y = w.z; u.x = w.y; u.y = w.w;
+            } else {
+                v = *(const GLOBAL_AS float2_t *)(x + i0);
+                if (j.x_glu) u = *(const GLOBAL_AS float2_t *)(j.x_glu + (int64_t)(q * j.x_stride) + i0);
+            }
             if (j.x_glu) {
                 // MoeGateRule::ClampedGlu (larql-compute/src/pipeline/moe.rs:88-92): g = min(g, L); u = clamp(u, -L, L);
                 // (u + 1) * (g * sigmoid(alpha * g))
-                const float2_t u = *(const GLOBAL_AS float2_t *)(j.x_glu + (int64_t)(q * j.x_stride) + i0);
                 const float L = j.glu_limit, al = j.glu_alpha;
                 const float g0 = fminf(v.x, L), g1 = fminf(v.y, L);
                 const float u0 = u.x < -L ? -L : (u.x > L ? L : u.x), u1 = u.y < -L ? -L : (u.y > L ? L : u.y);

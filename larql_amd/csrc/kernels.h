@@ -46,7 +46,8 @@ struct GemvJob {
     uint32_t batch, pad2;
     uint64_t x_stride, out_stride;
     // Optional gated activation (MoE down projection, MXFP4 matrix-core kernel only): when `x_glu` is set the
-    // activation is ClampedGlu(g = x[i], u = x_glu[i]) computed while the activations are prepared.
+    // activation is ClampedGlu(g = x[i], u = x_glu[i]) computed while the activations are prepared; x_glu == x means
+    // that g and u are interleaved in x (g = x[2i], u = x[2i+1]: the result of a fused gate_up matrix walked in place).
     const float *x_glu;
     float glu_limit, glu_alpha;
 };
@@ -108,8 +109,9 @@ hipError_t router_select_launch(hipStream_t s, const float *logits, uint32_t tok
                                 uint32_t *experts, float *weights);
 hipError_t moe_plan_launch(hipStream_t s, const uint32_t *experts, uint32_t slots, uint32_t k, uint32_t n_experts, const GemvJob &tg,
                            const GemvJob &tu, const GemvJob &td, uint64_t gu_w_stride, uint64_t gu_s_stride, uint64_t dn_w_stride,
-                           uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, GemvJob *gu_table, uint32_t *gu_hdr, GemvJob *dn_table,
-                           uint32_t *dn_hdr);
+                           uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, bool fused, GemvJob *gu_table, uint32_t *gu_hdr,
+                           GemvJob *dn_table, uint32_t *dn_hdr);
+hipError_t clamped_glu_interleaved_launch(hipStream_t s, const float *gu, float *h, size_t n, float limit, float alpha);
 hipError_t clamped_glu_launch(hipStream_t s, const float *g, const float *u, float *h, size_t n, float limit, float alpha);
 hipError_t weighted_sum_launch(hipStream_t s, const float *d, const float *weights, float *out, uint32_t tokens, uint32_t k,
                                uint32_t hidden);

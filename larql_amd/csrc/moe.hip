@@ -73,6 +73,17 @@ __global__ void clamped_glu_kernel(const float *__restrict__ g, const float *__r
     h[i] = (uv + 1.0f) * (gv * sig);
 }
 
+// the same on the interleaved result of a fused gate_up matrix: g = gu[2i], u = gu[2i+1]
+__global__ void clamped_glu_interleaved_kernel(const float *__restrict__ gu, float *__restrict__ h, size_t n, float limit, float alpha) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float gv = fminf(gu[2 * i], limit);
+    float uv = gu[2 * i + 1];
+    uv = uv < -limit ? -limit : (uv > limit ? limit : uv);
+    const float sig = 1.0f / (1.0f + expf(-(gv * alpha)));
+    h[i] = (uv + 1.0f) * (gv * sig);
+}
+
 // out[t] = sum over the token's k selected experts, in selection order, of w * down-output
 // (larql-compute/src/cpu/ops/moe/forward.rs:266-270).
 __global__ void weighted_sum_kernel(const float *__restrict__ d, const float *__restrict__ weights, float *__restrict__ out,
@@ -91,9 +102,11 @@ __global__ void weighted_sum_kernel(const float *__restrict__ d, const float *__
 // second activation / result sits x_stride / out_stride floats away from the first, in either direction).
 // tg / tu / td are the jobs of slot 0 with expert 0 (geometry filled in); tables: [gate jobs | up jobs], [down jobs];
 // headers: {job count, pass total}.  One block; a thread per slot, O(slots) work each.
+// `fused`: tg walks a fused gate_up matrix of 2*inter interleaved rows (no up jobs; a slot's results and the down
+// job's activation are 2*inter floats, gate and up values alternating).
 __global__ void __launch_bounds__(256) moe_plan_kernel(const uint32_t *__restrict__ experts, uint32_t slots, uint32_t k, uint32_t n_experts,
                                                        GemvJob tg, GemvJob tu, GemvJob td, uint64_t gu_w_stride, uint64_t gu_s_stride,
-                                                       uint64_t dn_w_stride, uint64_t dn_s_stride, uint32_t hidden, uint32_t inter,
+                                                       uint64_t dn_w_stride, uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, uint32_t fused,
                                                        GemvJob *__restrict__ gu_table, uint32_t *__restrict__ gu_hdr,
                                                        GemvJob *__restrict__ dn_table, uint32_t *__restrict__ dn_hdr) {
     __shared__ uint32_t first_job[1025];  // first job of expert e; [n_experts] = total
@@ -138,31 +151,34 @@ __global__ void __launch_bounds__(256) moe_plan_kernel(const uint32_t *__restric
         b.w += (size_t)e * gu_w_stride; b.aux += (size_t)e * gu_s_stride;
         c.w += (size_t)e * dn_w_stride; c.aux += (size_t)e * dn_s_stride;
         a.x += (size_t)tok1 * hidden; b.x += (size_t)tok1 * hidden;
-        a.out += (size_t)s1 * inter; b.out += (size_t)s1 * inter;
-        c.x += (size_t)s1 * inter; c.x_glu += (size_t)s1 * inter; c.out += (size_t)s1 * hidden;
+        const size_t gs = fused ? 2 * (size_t)inter : (size_t)inter;  // floats of gate/up results per slot and half
+        a.out += (size_t)s1 * gs; b.out += (size_t)s1 * gs;
+        c.x += (size_t)s1 * gs; c.x_glu += (size_t)s1 * gs; c.out += (size_t)s1 * hidden;
         a.batch = b.batch = c.batch = nb;
         a.x_stride = b.x_stride = (uint64_t)(((int64_t)tok2 - (int64_t)tok1) * (int64_t)hidden);
-        a.out_stride = b.out_stride = (uint64_t)(((int64_t)s2 - (int64_t)s1) * (int64_t)inter);
-        c.x_stride = (uint64_t)(((int64_t)s2 - (int64_t)s1) * (int64_t)inter);
+        a.out_stride = b.out_stride = (uint64_t)(((int64_t)s2 - (int64_t)s1) * (int64_t)gs);
+        c.x_stride = (uint64_t)(((int64_t)s2 - (int64_t)s1) * (int64_t)gs);
         c.out_stride = (uint64_t)(((int64_t)s2 - (int64_t)s1) * (int64_t)hidden);
         a.pass_begin = jb * tg.n_pass;
         b.pass_begin = (n_jobs + jb) * tg.n_pass;
         c.pass_begin = jb * td.n_pass;
-        gu_table[jb] = a; gu_table[n_jobs + jb] = b; dn_table[jb] = c;
+        gu_table[jb] = a; dn_table[jb] = c;
+        if (!fused) gu_table[n_jobs + jb] = b;
     }
     if (t == 0) {
-        gu_hdr[0] = 2 * n_jobs; gu_hdr[1] = 2 * n_jobs * tg.n_pass;
+        const uint32_t gu_jobs = fused ? n_jobs : 2 * n_jobs;
+        gu_hdr[0] = gu_jobs; gu_hdr[1] = gu_jobs * tg.n_pass;
         dn_hdr[0] = n_jobs; dn_hdr[1] = n_jobs * td.n_pass;
     }
 }
 
 hipError_t moe_plan_launch(hipStream_t s, const uint32_t *experts, uint32_t slots, uint32_t k, uint32_t n_experts, const GemvJob &tg,
                            const GemvJob &tu, const GemvJob &td, uint64_t gu_w_stride, uint64_t gu_s_stride, uint64_t dn_w_stride,
-                           uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, GemvJob *gu_table, uint32_t *gu_hdr, GemvJob *dn_table,
-                           uint32_t *dn_hdr) {
+                           uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, bool fused, GemvJob *gu_table, uint32_t *gu_hdr,
+                           GemvJob *dn_table, uint32_t *dn_hdr) {
     if (n_experts > 1024) return hipErrorInvalidValue;
     hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(256), 0, s, experts, slots, k, n_experts, tg, tu, td, gu_w_stride, gu_s_stride,
-                       dn_w_stride, dn_s_stride, hidden, inter, gu_table, gu_hdr, dn_table, dn_hdr);
+                       dn_w_stride, dn_s_stride, hidden, inter, fused ? 1u : 0u, gu_table, gu_hdr, dn_table, dn_hdr);
     return hipGetLastError();
 }
 
@@ -170,6 +186,11 @@ hipError_t router_select_launch(hipStream_t s, const float *logits, uint32_t tok
                                 uint32_t *experts, float *weights) {
     if (tokens == 0) return hipSuccess;
     hipLaunchKernelGGL(router_select_kernel, dim3(tokens), dim3(64), 0, s, logits, n_experts, k, policy, experts, weights);
+    return hipGetLastError();
+}
+hipError_t clamped_glu_interleaved_launch(hipStream_t s, const float *gu, float *h, size_t n, float limit, float alpha) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(clamped_glu_interleaved_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, gu, h, n, limit, alpha);
     return hipGetLastError();
 }
 hipError_t clamped_glu_launch(hipStream_t s, const float *g, const float *u, float *h, size_t n, float limit, float alpha) {

@@ -420,6 +420,25 @@ SOFTMAX_THEN_SELECT = 0
 NORMALISED_OVER_SELECTED = 1
 
 
+# MoeFusedRowLayout / FusedHalf — larql-compute/src/pipeline/moe.rs:294-332, larql-models/src/quant/mxfp4.rs:168-191
+CONTIGUOUS_HALVES, INTERLEAVED = 0, 1
+HALF_GATE, HALF_UP = 0, 1
+
+
+def fused_row_walk(layout: int, half: int, inter: int):
+    """MoeFusedRowLayout::row_walk: (first row, row stride) of one half's rows in a fused gate_up region of 2*inter rows."""
+    if layout == CONTIGUOUS_HALVES:
+        return (0, 1) if half == HALF_GATE else (inter, 1)
+    return (2 * 0 + (0 if half == HALF_GATE else 1), 2)  # FusedHalf::fused_row(0), FUSED_HALVES
+
+
+def deinterleave_fused_half(data, out_features: int, in_features: int, half: int) -> np.ndarray:
+    """deinterleave_fused_half (mxfp4.rs:218-231): the rows of one projection out of a fused [out_features, in_features] matrix."""
+    m = np.asarray(data).reshape(out_features, in_features)
+    first, step = fused_row_walk(INTERLEAVED, half, out_features // 2)
+    return m[first::step].reshape(-1).copy()
+
+
 def router_select(logits, k: int, policy: int = NORMALISED_OVER_SELECTED):
     logits = _f32(logits).ravel()
     cap = max(1, min(k, logits.size))

@@ -848,6 +848,52 @@ def test_moe_mxfp4_tokens_sharing_an_expert_equal_single_token_calls(be, fmt):
     assert rel_l2(got[5], acc) < 1e-5
 
 
+@pytest.mark.parametrize("T,E,hidden,inter", [(1, 4, 2880, 2880), (13, 6, 384, 320), (16, 8, 2880, 576)])
+def test_moe_mxfp4_interleaved_gate_up_bank_equals_separate_banks(be, fmt, T, E, hidden, inter):
+    """MoeFusedRowLayout::Interleaved (pipeline/moe.rs:294-332; FusedHalf::fused_row, mxfp4.rs:179-191): a GPT-OSS
+    gate_up region holds gate on the even and up on the odd fused rows.  Walking it in place gives the block the
+    de-interleaved banks give, bit for bit (a row's sum does not depend on its neighbours)."""
+    rng = np.random.default_rng(7 * T + E)
+    k = 4
+
+    def bank(n, kk):
+        p, s = [], []
+        for _ in range(E):
+            pp, ss = O.quantize_mxfp4((rng.standard_normal(n * kk) * 0.04).astype(F), n, kk)
+            p.append(pp); s.append(ss)
+        return np.concatenate(p), np.concatenate(s)
+
+    gp, gs = bank(inter, hidden); up, us = bank(inter, hidden); dp, ds = bank(hidden, inter)
+    G = hidden // 32
+    # the fused region of expert e: row 2r = gate row r, row 2r+1 = up row r (16 G packed bytes and G scale bytes per row)
+    fp = np.empty((E, 2 * inter, G * 16), np.uint8); fs = np.empty((E, 2 * inter, G), np.uint8)
+    fp[:, 0::2] = gp.reshape(E, inter, G * 16); fp[:, 1::2] = up.reshape(E, inter, G * 16)
+    fs[:, 0::2] = gs.reshape(E, inter, G); fs[:, 1::2] = us.reshape(E, inter, G)
+    assert O.fused_row_walk(O.INTERLEAVED, O.HALF_UP, inter) == (1, 2) and O.fused_row_walk(O.CONTIGUOUS_HALVES, O.HALF_UP, inter) == (inter, 1)
+    x = rng.standard_normal((T, hidden)).astype(F)
+    logits = rng.standard_normal((T, E)).astype(F)
+    dev = {n: be.to_device(a) for n, a in dict(gp=gp, gs=gs, up=up, us=us, dp=dp, ds=ds, fp=fp.reshape(-1), fs=fs.reshape(-1), x=x,
+                                                lg=logits).items()}
+    de, dw_ = be.malloc(T * k * 4), be.malloc(T * k * 4)
+    assert be.dev_router_select(dev["lg"], T, E, k, O.NORMALISED_OVER_SELECTED, de, dw_)
+    wsb = be.moe_mxfp4_workspace_bytes(T, k, hidden, inter)
+    ws = be.malloc(wsb)
+    outs = []
+    for b in (fmt.Mxfp4Experts(dev["gp"], dev["gs"], dev["up"], dev["us"], dev["dp"], dev["ds"], E, hidden, inter, 7.0, 1.702, 0),
+              fmt.Mxfp4Experts(dev["fp"], dev["fs"], None, None, dev["dp"], dev["ds"], E, hidden, inter, 7.0, 1.702, 1)):
+        do = be.malloc(T * hidden * 4)
+        assert be.dev_moe_mxfp4(b, dev["x"], T, k, de, dw_, do, ws, wsb)
+        be.synchronize()
+        outs.append(be.d2h(do, (T, hidden), F))
+    assert np.isfinite(outs[0]).all() and np.abs(outs[0]).max() > 0
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+    # a bank that says "separate" but brings no up half is an argument error
+    import larql_amd
+    with pytest.raises(larql_amd.DeviceError):
+        be.dev_moe_mxfp4(fmt.Mxfp4Experts(dev["fp"], dev["fs"], None, None, dev["dp"], dev["ds"], E, hidden, inter, 7.0, 1.702, 0),
+                         dev["x"], T, k, de, dw_, do, ws, wsb)
+
+
 # ------------------------------------------------------------- prefill GEMM
 @pytest.mark.parametrize("rows,hidden,seq", [(300, 512, 70), (128, 3840, 128), (1, 256, 1), (257, 768, 33), (520, 8192, 200)])
 def test_q4k_gemm_mfma_matches_oracle(be, rows, hidden, seq):

@@ -299,3 +299,25 @@ def test_moe_top_k_softmax_and_clamped_glu():
         gc, uc = min(g, 7.0), max(-7.0, min(7.0, u))
         want = (uc + 1.0) * gc / (1.0 + np.exp(-1.702 * gc))
         assert abs(O.clamped_glu(g, u) - want) < 1e-5 * max(1.0, abs(want))
+
+
+def test_fused_gate_up_row_walk_is_interleaved_not_contiguous_halves():
+    # FusedHalf::fused_row / deinterleave_fused_half / split_gate_up_experts (larql-models/src/quant/mxfp4.rs:179-268) and
+    # MoeFusedRowLayout::row_walk (larql-compute/src/pipeline/moe.rs:313-332), on the reference's own fixtures
+    # (mxfp4.rs:485-535: fused_row_indices_interleave, deinterleave_takes_even_rows_for_gate_and_odd_for_up,
+    # split_gate_up_is_interleaved_not_contiguous_halves)
+    first, step = O.fused_row_walk(O.INTERLEAVED, O.HALF_GATE, 8)
+    assert [first + step * r for r in (0, 1, 7)] == [0, 2, 14]
+    first, step = O.fused_row_walk(O.INTERLEAVED, O.HALF_UP, 8)
+    assert [first + step * r for r in (0, 1, 7)] == [1, 3, 15]
+    assert O.fused_row_walk(O.CONTIGUOUS_HALVES, O.HALF_GATE, 8) == (0, 1)
+    assert O.fused_row_walk(O.CONTIGUOUS_HALVES, O.HALF_UP, 8) == (8, 1)
+    data = np.array([0, 0, 1, 1, 2, 2, 3, 3], F)
+    assert O.deinterleave_fused_half(data, 4, 2, O.HALF_GATE).tolist() == [0, 0, 2, 2]
+    assert O.deinterleave_fused_half(data, 4, 2, O.HALF_UP).tolist() == [1, 1, 3, 3]
+    # four fused rows whose value is their own scale (nibble 2 = 1.0): rows = [1, 2, 4, 8]
+    blocks, scales = np.full(4 * 16, 0x22, np.uint8), np.array([127, 128, 129, 130], np.uint8)
+    dense = O.dequantize_mxfp4_expert(blocks, scales, 4, 1)
+    gate = O.deinterleave_fused_half(dense, 4, 32, O.HALF_GATE).reshape(2, 32)[:, 0].tolist()
+    up = O.deinterleave_fused_half(dense, 4, 32, O.HALF_UP).reshape(2, 32)[:, 0].tolist()
+    assert gate == [1.0, 4.0] and up == [2.0, 8.0]
