@@ -473,7 +473,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on ONE GPU; --gpus above 1 is not part of this build "
-              "(sharding is by weight rows, see DESIGN.md)", file=sys.stderr)
+              "(it would shard by weight rows: x broadcast, outputs concatenated, no reduction across GPUs)", file=sys.stderr)
         sys.exit(2)
 
     import larql_amd as fmt
