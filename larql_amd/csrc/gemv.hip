@@ -56,6 +56,20 @@ __device__ __forceinline__ float dpp_add(float v) {
     return v + __builtin_bit_cast(float, moved);
 }
 
+// max of a non-negative value over the wavefront, the same in every lane: four steps inside the rows of 16 lanes
+// and two row broadcasts (data-parallel primitives, a few cycles each; cross-lane shuffles go through LDS hardware
+// and cost a round trip each), then lane 63 holds the result
+__device__ __forceinline__ float wave_max_nonneg(float v) {
+    int m = __builtin_bit_cast(int, v);  // (non-negative floats order like their bit patterns)
+    m = max(m, __builtin_amdgcn_update_dpp(0, m, 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+    m = max(m, __builtin_amdgcn_update_dpp(0, m, 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+    m = max(m, __builtin_amdgcn_update_dpp(0, m, 0x141, 0xF, 0xF, true));  // row_half_mirror
+    m = max(m, __builtin_amdgcn_update_dpp(0, m, 0x140, 0xF, 0xF, true));  // row_mirror
+    m = max(m, __builtin_amdgcn_update_dpp(0, m, 0x142, 0xA, 0xF, false)); // row_bcast:15 into rows 1 and 3
+    m = max(m, __builtin_amdgcn_update_dpp(0, m, 0x143, 0xC, 0xF, false)); // row_bcast:31 into rows 2 and 3
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(m, 63));
+}
+
 // ---------------------------------------------------------------------------
 // Q4_K: one thread = one 32-byte nibble group (sub-blocks 2g and 2g+1 of
 // super-block sb, 64 consecutive activations).  Value per row, as
@@ -995,67 +1009,95 @@ struct Mx4Step {
 // Digits of one step's 128 activations, for lane (t = lane%16, kg = lane/16); x index >= k reads as 0.
 // Every lane converts two activations into their six digits and the wavefront transposes them through
 // `scratch` (768 B of its own LDS: digit row t at t*128) into the operand layout.
-__device__ __forceinline__ Mx4Step mx4_setup_step(const GemvJob &j, uint32_t step, uint32_t lane, uint8_t *scratch) {
-    const uint32_t k = (uint32_t)j.k;
-    const uint32_t t = lane & 15u, kg = lane >> 4;
-    const uint32_t i0 = step * 128 + 2 * lane;
+// The two activations of lane `lane` in step `step`, for up to two tokens (the gate and up values of a gated job):
+// loaded apart from their conversion so that all steps' loads fly together (a load's first use waits for
+// everything in flight, the weight tiles included, so loads issued one step at a time cost a round trip each).
+struct Mx4In { float2_t v[2], u[2]; };
+
+__device__ __forceinline__ Mx4In mx4_load_step(const GemvJob &j, uint32_t step, uint32_t lane) {
+    const uint32_t k = (uint32_t)j.k, i0 = step * 128 + 2 * lane;
     const uint32_t ntok = j.batch > 1 ? 2u : 1u;
-    Mx4Step st;
+    Mx4In in;
 #pragma unroll
-    for (int q = 0; q < 8; q++) st.a[q] = 0;
-    st.scale_a = 127;
-    // token q's six digit rows are A rows 8q .. 8q+5 (rows 6, 7, 14, 15 stay zero): its sums come out in D rows of their own
-    for (uint32_t q = 0; q < ntok; q++) {
-        const float *x = j.x + (int64_t)(q * j.x_stride);
-        float2_t v = {0.f, 0.f};
-        if (i0 + 2 <= k) {  // k is even: a pair is inside or outside
-            float2_t u = {0.f, 0.f};
+    for (int q = 0; q < 2; q++) {
+        in.v[q] = (float2_t){0.f, 0.f}; in.u[q] = (float2_t){0.f, 0.f};
+        if ((uint32_t)q < ntok && i0 + 2 <= k) {  // k is even: a pair is inside or outside
+            const float *x = j.x + (int64_t)(q * j.x_stride);
             if (j.x_glu == j.x) {
                 // gate and up values interleaved (the result rows of a fused gate_up matrix walked in place): g0 u0 g1 u1
                 const f32x4 w = *(const GLOBAL_AS f32x4 *)(x + 2 * (size_t)i0);
-                v.x = w.x; v.y = w.z; u.x = w.y; u.y = w.w;
+                in.v[q].x = w.x; in.v[q].y = w.z; in.u[q].x = w.y; in.u[q].y = w.w;
             } else {
-                v = *(const GLOBAL_AS float2_t *)(x + i0);
-                if (j.x_glu) u = *(const GLOBAL_AS float2_t *)(j.x_glu + (int64_t)(q * j.x_stride) + i0);
+                in.v[q] = *(const GLOBAL_AS float2_t *)(x + i0);
+                if (j.x_glu) in.u[q] = *(const GLOBAL_AS float2_t *)(j.x_glu + (int64_t)(q * j.x_stride) + i0);
             }
+        }
+    }
+    return in;
+}
+
+// The operands of all `cw` steps of a wavefront.  Per token, the digits of every step go to `scratch` (768 bytes per
+// step: digit row d at d*128) first and are read back in the operand layout afterwards, so the LDS round trip is paid
+// once per token, not once per step.
+__device__ __forceinline__ void mx4_setup_steps(const GemvJob &j, const Mx4In (&in)[kMx4MaxSteps], Mx4Step (&st)[kMx4MaxSteps], uint32_t cw,
+                                                uint32_t lane, uint8_t *scratch) {
+    const uint32_t t = lane & 15u, kg = lane >> 4;
+    const uint32_t ntok = j.batch > 1 ? 2u : 1u;
+#pragma unroll
+    for (int s = 0; s < kMx4MaxSteps; s++) {
+#pragma unroll
+        for (int q = 0; q < 8; q++) st[s].a[q] = 0;
+        st[s].scale_a = 127;
+    }
+    // token q's six digit rows are A rows 8q .. 8q+5 (rows 6, 7, 14, 15 stay zero): its sums come out in D rows of their own
+#pragma unroll
+    for (int q = 0; q < 2; q++) {
+        if ((uint32_t)q >= ntok) break;
+        int ex[kMx4MaxSteps];
+#pragma unroll
+        for (int s = 0; s < kMx4MaxSteps; s++) {
+            if ((uint32_t)s >= cw) continue;
+            float2_t v = in[s].v[q];
             if (j.x_glu) {
                 // MoeGateRule::ClampedGlu (larql-compute/src/pipeline/moe.rs:88-92): g = min(g, L); u = clamp(u, -L, L);
-                // (u + 1) * (g * sigmoid(alpha * g))
+                // (u + 1) * (g * sigmoid(alpha * g))   (activations past the row end are zeros: they stay zero)
+                const float2_t u = in[s].u[q];
                 const float L = j.glu_limit, al = j.glu_alpha;
                 const float g0 = fminf(v.x, L), g1 = fminf(v.y, L);
                 const float u0 = u.x < -L ? -L : (u.x > L ? L : u.x), u1 = u.y < -L ? -L : (u.y > L ? L : u.y);
                 v.x = (u0 + 1.0f) * (g0 * (1.0f / (1.0f + expf(-(g0 * al)))));
                 v.y = (u1 + 1.0f) * (g1 * (1.0f / (1.0f + expf(-(g1 * al)))));
             }
-        }
-        float mx = fmaxf(fabsf(v.x), fabsf(v.y));
+            const float mx = wave_max_nonneg(fmaxf(fabsf(v.x), fabsf(v.y)));
+            // mx = f * 2^ex, f in [0.5, 1): the exponent field less 126 (zero, subnormal, infinite and NaN maxima end at the clamps)
+            const int ef = (int)((__builtin_bit_cast(uint32_t, mx) >> 23) & 0xFFu);
+            ex[s] = (ef == 0 || ef == 255) ? (ef == 0 && mx > 0.f ? -100 : 0) : max(-100, min(100, ef - 126));
+            const float to_int = __builtin_bit_cast(float, (uint32_t)(127 + 23 - ex[s]) << 23);  // 2^(23 - ex)
+            // balanced base-16 digits: n + 0x888888 has the unsigned digits d+8 (the top one may reach 16)
+            const int n0 = (int)__builtin_rintf(v.x * to_int) + 0x888888, n1 = (int)__builtin_rintf(v.y * to_int) + 0x888888;
 #pragma unroll
-        for (int o = 1; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
-        int ex = 0;
-        if (mx > 0.f && mx < __builtin_inff()) (void)frexpf(mx, &ex);  // mx = f * 2^ex, f in [0.5, 1)
-        ex = max(-100, min(100, ex));
-        const float to_int = ldexpf(1.f, 23 - ex);
-        // balanced base-16 digits: n + 0x888888 has the unsigned digits d+8 (the top one may reach 16)
-        const int n0 = (int)__builtin_rintf(v.x * to_int) + 0x888888, n1 = (int)__builtin_rintf(v.y * to_int) + 0x888888;
-#pragma unroll
-        for (int d = 0; d < 6; d++) {
-            const int sh = 4 * (5 - d);
-            const int d0 = (d == 0 ? (n0 >> 20) : ((n0 >> sh) & 15)) - 8, d1 = (d == 0 ? (n1 >> 20) : ((n1 >> sh) & 15)) - 8;
-            const int pk = __builtin_amdgcn_cvt_pk_fp8_f32((float)d0, (float)d1, 0, false);  // integers up to 8 are exact in e4m3
-            *reinterpret_cast<uint16_t *>(scratch + d * 128 + 2 * lane) = (uint16_t)pk;
+            for (int d = 0; d < 6; d++) {
+                const int sh = 4 * (5 - d);
+                const int d0 = (d == 0 ? (n0 >> 20) : ((n0 >> sh) & 15)) - 8, d1 = (d == 0 ? (n1 >> 20) : ((n1 >> sh) & 15)) - 8;
+                const int pk = __builtin_amdgcn_cvt_pk_fp8_f32((float)d0, (float)d1, 0, false);  // integers up to 8 are exact in e4m3
+                *reinterpret_cast<uint16_t *>(scratch + s * 768 + d * 128 + 2 * lane) = (uint16_t)pk;
+            }
         }
         asm volatile("" ::: "memory");  // same wavefront: LDS executes its writes before the reads that follow
-        const uint32_t row = t - 8 * q;  // (wraps for the rows of the other token)
-        if (row < 6) {
-            const u32x4 lo = *reinterpret_cast<const u32x4 *>(scratch + row * 128 + 16 * kg);       // K = 16kg .. 16kg+15
-            const u32x4 hi = *reinterpret_cast<const u32x4 *>(scratch + row * 128 + 64 + 16 * kg);  // K = 64+16kg ..
-            st.a[0] = (int)lo.x; st.a[1] = (int)lo.y; st.a[2] = (int)lo.z; st.a[3] = (int)lo.w;
-            st.a[4] = (int)hi.x; st.a[5] = (int)hi.y; st.a[6] = (int)hi.z; st.a[7] = (int)hi.w;
-            st.scale_a = 124 + ex - 4 * (int)row;  // digit `row` weighs 2^(ex - 23 + 4*(5 - row))
+        const uint32_t row = t - 8 * (uint32_t)q;  // (wraps for the rows of the other token)
+#pragma unroll
+        for (int s = 0; s < kMx4MaxSteps; s++) {
+            if ((uint32_t)s >= cw) continue;
+            if (row < 6) {
+                const u32x4 lo = *reinterpret_cast<const u32x4 *>(scratch + s * 768 + row * 128 + 16 * kg);       // K = 16kg .. 16kg+15
+                const u32x4 hi = *reinterpret_cast<const u32x4 *>(scratch + s * 768 + row * 128 + 64 + 16 * kg);  // K = 64+16kg ..
+                st[s].a[0] = (int)lo.x; st[s].a[1] = (int)lo.y; st[s].a[2] = (int)lo.z; st[s].a[3] = (int)lo.w;
+                st[s].a[4] = (int)hi.x; st[s].a[5] = (int)hi.y; st[s].a[6] = (int)hi.z; st[s].a[7] = (int)hi.w;
+                st[s].scale_a = 124 + ex[s] - 4 * (int)row;  // digit `row` weighs 2^(ex - 23 + 4*(5 - row))
+            }
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the scratch is reused by the next token / step
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the scratch is reused by the next token
     }
-    return st;
 }
 
 #define LARQL_MX4_WAIT_CASE(CW) case CW: LARQL_WAIT_VMCNT(2 * CW * (kMx4Stages - 1)); break;
@@ -1110,14 +1152,17 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
         n_issue++;
         if (it_tile < tile_b) it_tile++;
     };
-    if (working)
-        for (int s = 0; s < NS - 1; s++) issue();
-    // the activation digits are prepared while the first weight tiles are on their way (the ring's last
+    // the activations of all this wavefront's steps are requested first and together, ahead of the weight tiles in
+    // the in-order return queue; their digits are prepared while the first tiles are on their way (the ring's last
     // slot is still free and serves as scratch)
-    Mx4Step st[kMx4MaxSteps];
+    Mx4In xin[kMx4MaxSteps];
 #pragma unroll
     for (int s = 0; s < kMx4MaxSteps; s++)
-        if (working && (uint32_t)s < cw) st[s] = mx4_setup_step(j, step0 + s, lane, ring + (NS - 1) * slot_bytes);
+        if (working && (uint32_t)s < cw) xin[s] = mx4_load_step(j, step0 + s, lane);
+    if (working)
+        for (int s = 0; s < NS - 1; s++) issue();
+    Mx4Step st[kMx4MaxSteps];
+    if (working) mx4_setup_steps(j, xin, st, cw, lane, ring + (NS - 1) * slot_bytes);  // (768 bytes per step fit the 1280 of a slot's step)
 
     uint32_t n_use = 0;
     for (uint32_t tb = 0; tb < nt; tb += R) {
