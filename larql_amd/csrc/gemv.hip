@@ -603,15 +603,20 @@ __device__ __forceinline__ Q4kRaw q4k_mfma_load_col(const float *x, uint32_t c, 
 
 __device__ __forceinline__ Q4kCol q4k_mfma_finish_col(const Q4kRaw &r, uint32_t lane) {
     const uint32_t j = lane & 15u, kq = lane >> 4;
-    float mx = fmaxf(fmaxf(fabsf(r.v.x), fabsf(r.v.y)), fmaxf(fabsf(r.v.z), fabsf(r.v.w)));
+    float mx = wave_max_nonneg(fmaxf(fmaxf(fabsf(r.v.x), fabsf(r.v.y)), fmaxf(fabsf(r.v.z), fabsf(r.v.w))));
     float sm = (r.v.x + r.v.y) + (r.v.z + r.v.w);
-#pragma unroll
-    for (int o = 1; o < 8; o <<= 1) { sm += __shfl_xor(sm, o); mx = fmaxf(mx, __shfl_xor(mx, o)); }
-#pragma unroll
-    for (int o = 8; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    // sum over the 8 lanes of a sub-block: the exchange pattern of a butterfly (partners 1, 2, 4 lanes away), by DPP
+    sm = dpp_add<0xB1>(sm);   // quad_perm [1,0,3,2]
+    sm = dpp_add<0x4E>(sm);   // quad_perm [2,3,0,1]
+    sm = dpp_add<0x141>(sm);  // row_half_mirror: the other quad of the eight
     Q4kCol col;
-    col.sum_lo = __shfl(sm, 16 * kq);
-    col.sum_hi = __shfl(sm, 16 * kq + 8);
+    {   // sub-block m's sum sits in lanes 8m .. 8m+7; this lane wants sub-blocks 2kq and 2kq+1
+        float sb[8];
+#pragma unroll
+        for (int m = 0; m < 8; m++) sb[m] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sm), 8 * m));
+        col.sum_lo = kq == 0 ? sb[0] : (kq == 1 ? sb[2] : (kq == 2 ? sb[4] : sb[6]));
+        col.sum_hi = kq == 0 ? sb[1] : (kq == 1 ? sb[3] : (kq == 2 ? sb[5] : sb[7]));
+    }
     int ex = 0;
     if (mx > 0.f && mx < __builtin_inff()) (void)frexpf(mx, &ex);  // mx = f * 2^ex, f in [0.5, 1)
     ex = max(-90, min(120, ex));
