@@ -142,13 +142,21 @@ __global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restr
         uint32_t gmax = 0;
 #pragma unroll
         for (int it = 0; it < kTopkCached; it++) gmax = max(gmax, cache[it]);
-#pragma unroll
-        for (int o = 1; o < 16; o <<= 1) gmax = max(gmax, (uint32_t)__shfl_xor((int)gmax, o, 64));
+        // (reductions by DPP row operations: a few cycles each, where a cross-lane shuffle costs an LDS round trip)
+        gmax = max(gmax, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)gmax, 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+        gmax = max(gmax, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)gmax, 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+        gmax = max(gmax, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)gmax, 0x141, 0xF, 0xF, true));  // row_half_mirror
+        gmax = max(gmax, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)gmax, 0x140, 0xF, 0xF, true));  // row_mirror
         if ((lane & 15u) == 0) group_max[wave * 4 + (lane >> 4)] = gmax;
         __syncthreads();
         uint32_t L = group_max[lane];
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) L = min(L, (uint32_t)__shfl_xor((int)L, o, 64));
+        L = min(L, (uint32_t)__builtin_amdgcn_update_dpp(-1, (int)L, 0xB1, 0xF, 0xF, false));
+        L = min(L, (uint32_t)__builtin_amdgcn_update_dpp(-1, (int)L, 0x4E, 0xF, 0xF, false));
+        L = min(L, (uint32_t)__builtin_amdgcn_update_dpp(-1, (int)L, 0x141, 0xF, 0xF, false));
+        L = min(L, (uint32_t)__builtin_amdgcn_update_dpp(-1, (int)L, 0x140, 0xF, 0xF, false));
+        L = min(L, (uint32_t)__builtin_amdgcn_update_dpp((int)L, (int)L, 0x142, 0xA, 0xF, false));     // row_bcast:15 into rows 1 and 3
+        L = min(L, (uint32_t)__builtin_amdgcn_update_dpp((int)L, (int)L, 0x143, 0xC, 0xF, false));     // row_bcast:31 into rows 2 and 3
+        L = (uint32_t)__builtin_amdgcn_readlane((int)L, 63);
         if (L != 0) {
             // a wavefront reserves room for all its candidates at once, then places them round by round
             uint32_t mine = 0;
