@@ -1248,7 +1248,8 @@ int larql_hip_dev_moe_mxfp4(larql_hip_ctx *c, const larql_hip_mxfp4_experts *ban
                 P.threads = gemv_pick_threads(&tj, 1);
                 if (P.threads == 0 || !gemv_job_geometry(tj, P.threads)) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: unsupported geometry");
                 const uint64_t max_jobs = which == 0 && !fused ? 2 * slots : slots;
-                if (max_jobs * tj.n_pass > 0x7FFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: launch too large");
+                // (the planner's cost per job: at most 6 start-up tiles' worth and 7/6 per tile)
+                if (max_jobs * (2 * (uint64_t)tj.n_pass + 8 * (uint64_t)tj.cpr) > 0x7FFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: launch too large");
                 memset(&P.L, 0, sizeof P.L);
                 P.L.table = which == 0 ? gu_table : dn_table;
                 P.L.dyn = hdr + 2 * which;

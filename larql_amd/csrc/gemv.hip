@@ -2128,8 +2128,10 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) gemv_mxfp4_mfma_kernel(Gemv
             j.aux += (size_t)e * j.aux_sel_stride;
         }
         const uint32_t seg_end = min(p_end, j.pass_begin + j.n_pass);
-        const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin;
-        const uint32_t tile_a = (a + j.cpr - 1) / j.cpr, tile_b = (b + j.cpr - 1) / j.cpr;
+        // a tile belongs to the workgroup whose share contains its first cost unit (the job's range opens with its
+        // start-up allowance, if it has one)
+        const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin, cpt = j.cpt ? j.cpt : j.cpr, su = j.su;
+        const uint32_t tile_a = a > su ? (a - su + cpt - 1) / cpt : 0, tile_b = b > su ? (b - su + cpt - 1) / cpt : 0;
         if (tile_a < tile_b) run_mxfp4_mfma(j, tile_a, tile_b, mx4_lds, L.pad, parity);
         p = seg_end;
         ji++;

@@ -50,6 +50,9 @@ struct GemvJob {
     // that g and u are interleaved in x (g = x[2i], u = x[2i+1]: the result of a fused gate_up matrix walked in place).
     const float *x_glu;
     float glu_limit, glu_alpha;
+    // Optional cost model of the job in the launch's pass list (MXFP4 matrix-core kernel): the job's n_pass is
+    // su + tiles * cpt (a start-up allowance, then cpt units per 16-row tile); cpt == 0 means cpr units per tile, no allowance.
+    uint32_t cpt, su;
 };
 
 struct GemvLaunch {

@@ -110,6 +110,7 @@ __global__ void __launch_bounds__(256) moe_plan_kernel(const uint32_t *__restric
                                                        GemvJob *__restrict__ gu_table, uint32_t *__restrict__ gu_hdr,
                                                        GemvJob *__restrict__ dn_table, uint32_t *__restrict__ dn_hdr) {
     __shared__ uint32_t first_job[1025];  // first job of expert e; [n_experts] = total
+    __shared__ uint32_t first_gcost[1025], first_dcost[1025];  // the same for the jobs' places in the two pass lists
     __shared__ uint32_t cnt[1024];        // slots per expert
     __shared__ uint32_t ex[4096];         // the router's choice, read once
     __shared__ uint32_t partner[4096];    // second slot of a job (or ~0)
@@ -120,13 +121,24 @@ __global__ void __launch_bounds__(256) moe_plan_kernel(const uint32_t *__restric
     for (uint32_t s = t; s < slots; s += blockDim.x)
         if (ex[s] < n_experts) atomicAdd(&cnt[ex[s]], 1u);
     __syncthreads();
+    // Cost of a job in the launches' pass lists, from cycle counts of the kernel: a tile costs the same whether one
+    // or two tokens share it (its bytes set the pace), and a job segment starts with the preparation of its
+    // activations, worth 4 (one token) or 6 (two) tiles.  Units: steps (a tile = cpr of them).
+    const uint32_t g_tiles = ((uint32_t)tg.rows + 15) / 16, d_tiles = ((uint32_t)td.rows + 15) / 16;
+    const uint32_t g_c1 = tg.cpr, g_c2 = tg.cpr, d_c1 = td.cpr, d_c2 = td.cpr;
+    const uint32_t g_p1 = 4 * g_c1 + g_tiles * g_c1, g_p2 = 6 * g_c1 + g_tiles * g_c2;
+    const uint32_t d_p1 = 4 * d_c1 + d_tiles * d_c1, d_p2 = 6 * d_c1 + d_tiles * d_c2;
     for (uint32_t e = t; e <= n_experts; e += blockDim.x) {
-        uint32_t f = 0;
-        for (uint32_t q = 0; q < e; q++) f += (cnt[q] + 1) / 2;
-        first_job[e] = f;
+        uint32_t f = 0, gc = 0, dc = 0;
+        for (uint32_t q = 0; q < e; q++) {
+            f += (cnt[q] + 1) / 2;
+            gc += (cnt[q] / 2) * g_p2 + (cnt[q] & 1u) * g_p1;
+            dc += (cnt[q] / 2) * d_p2 + (cnt[q] & 1u) * d_p1;
+        }
+        first_job[e] = f; first_gcost[e] = gc; first_dcost[e] = dc;
     }
     __syncthreads();
-    const uint32_t n_jobs = first_job[n_experts];
+    const uint32_t n_jobs = first_job[n_experts], g_total = first_gcost[n_experts], d_total = first_dcost[n_experts];
     // a slot's rank among the slots of its expert, in slot order: even ranks open a job, odd ranks join it
     for (uint32_t s = t; s < slots; s += blockDim.x) {
         const uint32_t e = ex[s];
@@ -159,16 +171,19 @@ __global__ void __launch_bounds__(256) moe_plan_kernel(const uint32_t *__restric
         a.out_stride = b.out_stride = (uint64_t)(((int64_t)s2 - (int64_t)s1) * (int64_t)gs);
         c.x_stride = (uint64_t)(((int64_t)s2 - (int64_t)s1) * (int64_t)gs);
         c.out_stride = (uint64_t)(((int64_t)s2 - (int64_t)s1) * (int64_t)hidden);
-        a.pass_begin = jb * tg.n_pass;
-        b.pass_begin = (n_jobs + jb) * tg.n_pass;
-        c.pass_begin = jb * td.n_pass;
+        // (the earlier jobs of this expert are all shared by two tokens)
+        a.pass_begin = first_gcost[e] + (r / 2) * g_p2;
+        b.pass_begin = g_total + a.pass_begin;
+        c.pass_begin = first_dcost[e] + (r / 2) * d_p2;
+        a.n_pass = b.n_pass = pair ? g_p2 : g_p1; c.n_pass = pair ? d_p2 : d_p1;
+        a.cpt = b.cpt = pair ? g_c2 : g_c1; c.cpt = pair ? d_c2 : d_c1;
+        a.su = b.su = (pair ? 6u : 4u) * g_c1; c.su = (pair ? 6u : 4u) * d_c1;
         gu_table[jb] = a; dn_table[jb] = c;
         if (!fused) gu_table[n_jobs + jb] = b;
     }
     if (t == 0) {
-        const uint32_t gu_jobs = fused ? n_jobs : 2 * n_jobs;
-        gu_hdr[0] = gu_jobs; gu_hdr[1] = gu_jobs * tg.n_pass;
-        dn_hdr[0] = n_jobs; dn_hdr[1] = n_jobs * td.n_pass;
+        gu_hdr[0] = fused ? n_jobs : 2 * n_jobs; gu_hdr[1] = fused ? g_total : 2 * g_total;
+        dn_hdr[0] = n_jobs; dn_hdr[1] = d_total;
     }
 }
 
