@@ -1226,7 +1226,7 @@ int larql_hip_dev_moe_mxfp4(larql_hip_ctx *c, const larql_hip_mxfp4_experts *ban
     const size_t gu_rows = fused ? 2 * inter : inter;
     const uint64_t gu_w_stride = gu_rows * (hidden / 32) * 16, gu_s_stride = gu_rows * (hidden / 32);
     const uint64_t dn_w_stride = hidden * (inter / 32) * 16, dn_s_stride = hidden * (inter / 32);
-    // Several tokens: slots that chose the same expert share its weights two at a time.  The job lists are built on
+    // Several tokens: slots that chose the same expert share its weights up to four at a time.  The job lists are built on
     // the device from the router's choice (moe_plan_kernel) into the workspace's spare activation area.
     {
         GemvJob tg = make_job(KIND_MXFP4, bank->gate_packed, bank->gate_scales, x, g, gu_rows, hidden);
@@ -1241,6 +1241,15 @@ int larql_hip_dev_moe_mxfp4(larql_hip_ctx *c, const larql_hip_mxfp4_experts *ban
             uint32_t *hdr = (uint32_t *)h;  // {gate/up count, passes, down count, passes}
             GemvJob *gu_table = (GemvJob *)((uint8_t *)h + 64), *dn_table = gu_table + 2 * slots;
             PreparedLaunch Pg, Pd;
+            // four tokens per job where the launches' LDS has room for their partial sums, else two
+            static const uint32_t group_cap = getenv("LARQL_HIP_MOE_GROUP") && atoi(getenv("LARQL_HIP_MOE_GROUP")) == 2 ? 2u : 4u;
+            uint32_t group = group_cap;
+            for (int which = 0; which < 2 && group > 2; which++) {
+                GemvJob tj = which == 0 ? tg : td;
+                const uint32_t th = gemv_pick_threads(&tj, 1);
+                tj.batch = group;
+                if (th == 0 || !gemv_job_geometry(tj, th) || gemv_lds_bytes(&tj, 1, th) > 160 * 1024) group = 2;
+            }
             for (int which = 0; which < 2; which++) {
                 GemvJob &tj = which == 0 ? tg : td;
                 PreparedLaunch &P = which == 0 ? Pg : Pd;
@@ -1248,18 +1257,19 @@ int larql_hip_dev_moe_mxfp4(larql_hip_ctx *c, const larql_hip_mxfp4_experts *ban
                 P.threads = gemv_pick_threads(&tj, 1);
                 if (P.threads == 0 || !gemv_job_geometry(tj, P.threads)) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: unsupported geometry");
                 const uint64_t max_jobs = which == 0 && !fused ? 2 * slots : slots;
-                // (the planner's cost per job: at most 6 start-up tiles' worth and 7/6 per tile)
-                if (max_jobs * (2 * (uint64_t)tj.n_pass + 8 * (uint64_t)tj.cpr) > 0x7FFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: launch too large");
+                // (the planner's cost per job: the tiles and at most 10 more tiles' worth of start-up)
+                if (max_jobs * ((uint64_t)tj.n_pass + 10 * (uint64_t)tj.cpr) > 0x7FFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: launch too large");
                 memset(&P.L, 0, sizeof P.L);
                 P.L.table = which == 0 ? gu_table : dn_table;
                 P.L.dyn = hdr + 2 * which;
                 P.L.pad = gemv_launch_param(&tj, 1);
+                tj.batch = group;  // (sizes the partial sums; the planner sets every job's own count)
                 P.lds = gemv_lds_bytes(&tj, 1, P.threads);
                 P.grid = (uint32_t)((uint64_t)c->cu_count * gemv_wgs_per_cu(P.kind, P.threads, P.lds, (uint32_t)c->wgs_per_cu));
             }
             if (!gemv_job_geometry(tu, Pg.threads)) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: unsupported geometry");
             HIPCHECK(c, moe_plan_launch(c->stream, experts, (uint32_t)slots, (uint32_t)k, (uint32_t)bank->n_experts, tg, tu, td, gu_w_stride,
-                                        gu_s_stride, dn_w_stride, dn_s_stride, (uint32_t)hidden, (uint32_t)inter, fused, gu_table, hdr,
+                                        gu_s_stride, dn_w_stride, dn_s_stride, (uint32_t)hidden, (uint32_t)inter, fused, group, gu_table, hdr,
                                         dn_table, hdr + 2));
             HIPCHECK(c, gemv_launch(c->stream, Pg.kind, Pg.L, Pg.threads, Pg.grid, Pg.lds));
             HIPCHECK(c, gemv_launch(c->stream, Pd.kind, Pd.L, Pd.threads, Pd.grid, Pd.lds));

@@ -991,12 +991,13 @@ __device__ __forceinline__ void run_q4k_q8k(const GemvJob &j, uint32_t tile_a, u
 // LDS ring (16-byte and 1-byte global_load_lds, one per lane and step; a sub-dword load still
 // fills a whole dword slot per lane).
 //
-// The "A" rows carry the activation in FP8 (e4m3): per step, n = rint(x * 2^(23-e)) (2^e > max|x| of
-// the step) is written in six balanced base-16 digits d_t in [-8, 8] — exact in e4m3 — and row t holds
-// digit t with the row's own e8m0 scale 2^(e-23+4(5-t)), so sum_t row_t reproduces x to 2^-24 of the
-// step's maximum.  A-operand bytes 0-15 of lane (t, kg) are K = 16kg..16kg+15 of the step, bytes 16-31 are
-// K = 64+16kg..; rows 6-15 are zero.  After the wavefront's steps, lane (j, rq) holds rows 4rq..4rq+3 of
-// column j: the digit sums of weight row j, already scaled, which it adds up (rq = 0, 1 matter).
+// The "A" rows carry the activation in FP4 as well: per step, n = rint(x * 2^(23-e)) (2^e > max|x| of
+// the step) is written in eight balanced base-8 digits d_t in [-4, 4] — all of them e2m1 values — and row t
+// holds digit t with the row's own e8m0 scale 2^(e-23+3(7-t)), so sum_t row_t reproduces x to 2^-24 of the
+// step's maximum; with both operands FP4 the instruction takes half the matrix-pipe time of an FP8 x FP4 one.
+// The A operand of lane (t, kg) is K = 32kg..32kg+31 of the step, laid out like the weights'.  A token takes
+// rows 0-7, a second token rows 8-15.  After the wavefront's steps, lane (j, rq) holds rows 4rq..4rq+3 of
+// column j: the digit sums of weight row j, already scaled, which it adds up (rq = 0, 1 are the first token).
 // e8m0 0 means 0.0 in the reference (the hardware reads it as 2^-127): such blocks are zeroed; 255 is NaN.
 // ---------------------------------------------------------------------------
 typedef int i32x8 __attribute__((ext_vector_type(8)));
@@ -1007,56 +1008,64 @@ constexpr int kMx4MaxWaves = 10;
 constexpr uint32_t kMx4StepBytes = 1024 + 256;  // per step of a wave-tile: 64 lanes x 16 B of nibbles, 64 scale bytes (one dword slot each)
 
 struct Mx4Step {
-    i32x8 a;        // this lane's 32 activation digits (FP8) of the step
+    i32x8 a;        // this lane's 32 activation digits (FP4, in a[0..3]) of the step
     int scale_a;    // e8m0 scale of this lane's digit row
 };
 
 // Digits of one step's 128 activations, for lane (t = lane%16, kg = lane/16); x index >= k reads as 0.
-// Every lane converts two activations into their six digits and the wavefront transposes them through
-// `scratch` (768 B of its own LDS: digit row t at t*128) into the operand layout.
-// The two activations of lane `lane` in step `step`, for up to two tokens (the gate and up values of a gated job):
+// Every lane converts two activations into their eight digits and the wavefront transposes them through
+// `scratch` (512 B of its own LDS per step: digit row t at t*64) into the operand layout.
+// The two activations of lane `lane` in step `step`, for every token of the job (the gate and up values of a gated job):
 // loaded apart from their conversion so that all steps' loads fly together (a load's first use waits for
 // everything in flight, the weight tiles included, so loads issued one step at a time cost a round trip each).
-struct Mx4In { float2_t v[2], u[2]; };
+constexpr int kMx4MaxTokens = 4;    // tokens that share one job's weights: two per 16-row A operand
+struct Mx4In { float2_t v[kMx4MaxTokens], u[kMx4MaxTokens]; };
+
+__device__ __forceinline__ uint32_t mx4_tokens(const GemvJob &j) { return j.batch > 1 ? min(j.batch, (uint32_t)kMx4MaxTokens) : 1u; }
+__device__ __forceinline__ int64_t mx4_x_off(const GemvJob &j, int q) { return q == 0 ? 0 : q == 1 ? (int64_t)j.x_stride : q == 2 ? j.x_off[0] : j.x_off[1]; }
+__device__ __forceinline__ int64_t mx4_out_off(const GemvJob &j, uint32_t q) { return q == 0 ? 0 : q == 1 ? (int64_t)j.out_stride : q == 2 ? j.out_off[0] : j.out_off[1]; }
 
 __device__ __forceinline__ Mx4In mx4_load_step(const GemvJob &j, uint32_t step, uint32_t lane) {
     const uint32_t k = (uint32_t)j.k, i0 = step * 128 + 2 * lane;
-    const uint32_t ntok = j.batch > 1 ? 2u : 1u;
+    const uint32_t ntok = mx4_tokens(j);
     Mx4In in;
 #pragma unroll
-    for (int q = 0; q < 2; q++) {
+    for (int q = 0; q < kMx4MaxTokens; q++) {
         in.v[q] = (float2_t){0.f, 0.f}; in.u[q] = (float2_t){0.f, 0.f};
         if ((uint32_t)q < ntok && i0 + 2 <= k) {  // k is even: a pair is inside or outside
-            const float *x = j.x + (int64_t)(q * j.x_stride);
+            const float *x = j.x + mx4_x_off(j, q);
             if (j.x_glu == j.x) {
                 // gate and up values interleaved (the result rows of a fused gate_up matrix walked in place): g0 u0 g1 u1
                 const f32x4 w = *(const GLOBAL_AS f32x4 *)(x + 2 * (size_t)i0);
                 in.v[q].x = w.x; in.v[q].y = w.z; in.u[q].x = w.y; in.u[q].y = w.w;
             } else {
                 in.v[q] = *(const GLOBAL_AS float2_t *)(x + i0);
-                if (j.x_glu) in.u[q] = *(const GLOBAL_AS float2_t *)(j.x_glu + (int64_t)(q * j.x_stride) + i0);
+                if (j.x_glu) in.u[q] = *(const GLOBAL_AS float2_t *)(j.x_glu + mx4_x_off(j, q) + i0);
             }
         }
     }
     return in;
 }
 
-// The operands of all `cw` steps of a wavefront.  Per token, the digits of every step go to `scratch` (768 bytes per
-// step: digit row d at d*128) first and are read back in the operand layout afterwards, so the LDS round trip is paid
+// The operands of all `cw` steps of a wavefront.  Per token, the digits of every step go to `scratch` (512 bytes per
+// step: digit row d at d*64) first and are read back in the operand layout afterwards, so the LDS round trip is paid
 // once per token, not once per step.
-__device__ __forceinline__ void mx4_setup_steps(const GemvJob &j, const Mx4In (&in)[kMx4MaxSteps], Mx4Step (&st)[kMx4MaxSteps], uint32_t cw,
+__device__ __forceinline__ void mx4_setup_steps(const GemvJob &j, const Mx4In (&in)[kMx4MaxSteps], Mx4Step (&st)[2][kMx4MaxSteps], uint32_t cw,
                                                 uint32_t lane, uint8_t *scratch) {
     const uint32_t t = lane & 15u, kg = lane >> 4;
-    const uint32_t ntok = j.batch > 1 ? 2u : 1u;
+    const uint32_t ntok = mx4_tokens(j);
 #pragma unroll
-    for (int s = 0; s < kMx4MaxSteps; s++) {
+    for (int g = 0; g < 2; g++) {
 #pragma unroll
-        for (int q = 0; q < 8; q++) st[s].a[q] = 0;
-        st[s].scale_a = 127;
+        for (int s = 0; s < kMx4MaxSteps; s++) {
+#pragma unroll
+            for (int q = 0; q < 8; q++) st[g][s].a[q] = 0;
+            st[g][s].scale_a = 127;
+        }
     }
-    // token q's six digit rows are A rows 8q .. 8q+5 (rows 6, 7, 14, 15 stay zero): its sums come out in D rows of their own
+    // token q's eight digit rows are A rows 8(q%2) .. 8(q%2)+7 of operand q/2: its sums come out in D rows of their own
 #pragma unroll
-    for (int q = 0; q < 2; q++) {
+    for (int q = 0; q < kMx4MaxTokens; q++) {
         if ((uint32_t)q >= ntok) break;
         int ex[kMx4MaxSteps];
 #pragma unroll
@@ -1078,27 +1087,35 @@ __device__ __forceinline__ void mx4_setup_steps(const GemvJob &j, const Mx4In (&
             const int ef = (int)((__builtin_bit_cast(uint32_t, mx) >> 23) & 0xFFu);
             ex[s] = (ef == 0 || ef == 255) ? (ef == 0 && mx > 0.f ? -100 : 0) : max(-100, min(100, ef - 126));
             const float to_int = __builtin_bit_cast(float, (uint32_t)(127 + 23 - ex[s]) << 23);  // 2^(23 - ex)
-            // balanced base-16 digits: n + 0x888888 has the unsigned digits d+8 (the top one may reach 16)
-            const int n0 = (int)__builtin_rintf(v.x * to_int) + 0x888888, n1 = (int)__builtin_rintf(v.y * to_int) + 0x888888;
+            // balanced base-8 digits: n + 0o44444444 has the unsigned digits d+4 (the top one may reach 8)
+            const uint32_t n0 = (uint32_t)((int)__builtin_rintf(v.x * to_int) + 0x924924), n1 = (uint32_t)((int)__builtin_rintf(v.y * to_int) + 0x924924);
+            // e2m1 codes of -4 .. 3 by unsigned digit, a nibble each: -4 = 0xE, -3 = 0xD, -2 = 0xC, -1 = 0xA, 0, 1 = 2, 2 = 4, 3 = 5 (and 4 = 6)
+            constexpr uint32_t kCodes = 0x5420ACDEu;
 #pragma unroll
-            for (int d = 0; d < 6; d++) {
-                const int sh = 4 * (5 - d);
-                const int d0 = (d == 0 ? (n0 >> 20) : ((n0 >> sh) & 15)) - 8, d1 = (d == 0 ? (n1 >> 20) : ((n1 >> sh) & 15)) - 8;
-                const int pk = __builtin_amdgcn_cvt_pk_fp8_f32((float)d0, (float)d1, 0, false);  // integers up to 8 are exact in e4m3
-                *reinterpret_cast<uint16_t *>(scratch + s * 768 + d * 128 + 2 * lane) = (uint16_t)pk;
+            for (int d = 0; d < 8; d++) {
+                const int sh = 3 * (7 - d);
+                uint32_t c0, c1;
+                if (d == 0) {
+                    const uint32_t u0 = n0 >> 21, u1 = n1 >> 21;
+                    c0 = u0 == 8u ? 6u : (kCodes >> (4 * u0)) & 15u;
+                    c1 = u1 == 8u ? 6u : (kCodes >> (4 * u1)) & 15u;
+                } else {
+                    c0 = (kCodes >> (4 * ((n0 >> sh) & 7u))) & 15u;
+                    c1 = (kCodes >> (4 * ((n1 >> sh) & 7u))) & 15u;
+                }
+                scratch[s * 512 + d * 64 + lane] = (uint8_t)(c0 | (c1 << 4));  // low nibble first
             }
         }
         asm volatile("" ::: "memory");  // same wavefront: LDS executes its writes before the reads that follow
-        const uint32_t row = t - 8 * (uint32_t)q;  // (wraps for the rows of the other token)
+        const uint32_t row = t - 8 * (uint32_t)(q & 1);  // (wraps for the rows of the other token)
+        Mx4Step (&sq)[kMx4MaxSteps] = st[q >> 1];
 #pragma unroll
         for (int s = 0; s < kMx4MaxSteps; s++) {
             if ((uint32_t)s >= cw) continue;
-            if (row < 6) {
-                const u32x4 lo = *reinterpret_cast<const u32x4 *>(scratch + s * 768 + row * 128 + 16 * kg);       // K = 16kg .. 16kg+15
-                const u32x4 hi = *reinterpret_cast<const u32x4 *>(scratch + s * 768 + row * 128 + 64 + 16 * kg);  // K = 64+16kg ..
-                st[s].a[0] = (int)lo.x; st[s].a[1] = (int)lo.y; st[s].a[2] = (int)lo.z; st[s].a[3] = (int)lo.w;
-                st[s].a[4] = (int)hi.x; st[s].a[5] = (int)hi.y; st[s].a[6] = (int)hi.z; st[s].a[7] = (int)hi.w;
-                st[s].scale_a = 124 + ex[s] - 4 * (int)row;  // digit `row` weighs 2^(ex - 23 + 4*(5 - row))
+            if (row < 8) {
+                const u32x4 op = *reinterpret_cast<const u32x4 *>(scratch + s * 512 + row * 64 + 16 * kg);  // K = 32kg .. 32kg+31
+                sq[s].a[0] = (int)op.x; sq[s].a[1] = (int)op.y; sq[s].a[2] = (int)op.z; sq[s].a[3] = (int)op.w;
+                sq[s].scale_a = 125 + ex[s] - 3 * (int)row;  // digit `row` weighs 2^(ex - 23 + 3*(7 - row))
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the scratch is reused by the next token
@@ -1114,8 +1131,11 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
     const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t nw_launch = blockDim.x >> 6;
     const uint32_t jr = lane & 15u, kg = lane >> 4;
-    const bool two = j.batch > 1;  // two tokens share the weights: their sums leave in D rows 0..7 and 8..15
-    const uint32_t nwj = j.rpp, steps = j.cpr, cw = (uint32_t)j.pad, PW = nwj * (two ? 4u : 2u);
+    // up to four tokens share the weights: tokens 2q and 2q+1 ride in A operand q, their sums leave in D rows 0..7 and 8..15
+    const uint32_t ntok = mx4_tokens(j);
+    const bool second = ntok > 2;
+    const uint32_t hw_sh = ntok == 1 ? 1u : (ntok == 2 ? 2u : 3u), hw = 1u << hw_sh;  // partial sums per weight row and wavefront
+    const uint32_t nwj = j.rpp, steps = j.cpr, cw = (uint32_t)j.pad, PW = nwj * hw;
     const uint32_t rows = (uint32_t)j.rows, k = (uint32_t)j.k, nb = k / 32, row_bytes = (uint32_t)j.row_bytes;
     uint8_t *ring = lds + wv * (NS * slot_bytes);
     float *part = reinterpret_cast<float *>(lds + nw_launch * (NS * slot_bytes));
@@ -1166,8 +1186,8 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
         if (working && (uint32_t)s < cw) xin[s] = mx4_load_step(j, step0 + s, lane);
     if (working)
         for (int s = 0; s < NS - 1; s++) issue();
-    Mx4Step st[kMx4MaxSteps];
-    if (working) mx4_setup_steps(j, xin, st, cw, lane, ring + (NS - 1) * slot_bytes);  // (768 bytes per step fit the 1280 of a slot's step)
+    Mx4Step st[2][kMx4MaxSteps];
+    if (working) mx4_setup_steps(j, xin, st, cw, lane, ring + (NS - 1) * slot_bytes);  // (512 bytes per step fit the 1280 of a slot's step)
 
     uint32_t n_use = 0;
     for (uint32_t tb = 0; tb < nt; tb += R) {
@@ -1181,7 +1201,7 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
                 }
                 asm volatile("" ::: "memory");
                 const uint8_t *slot = ring + (n_use % NS) * slot_bytes;
-                f32x4 D = {0.f, 0.f, 0.f, 0.f};
+                f32x4 D = {0.f, 0.f, 0.f, 0.f}, D2 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int s = 0; s < kMx4MaxSteps; s++) {
                     if ((uint32_t)s < cw) {
@@ -1191,13 +1211,16 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
                         sc = valid[s] ? sc : 127u;
                         i32x8 b = {0, 0, 0, 0, 0, 0, 0, 0};
                         b[0] = live ? (int)q.x : 0; b[1] = live ? (int)q.y : 0; b[2] = live ? (int)q.z : 0; b[3] = live ? (int)q.w : 0;
-                        D = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st[s].a, b, D, 0, 4, 0, st[s].scale_a, 0, (int)sc);
+                        D = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st[0][s].a, b, D, 4, 4, 0, st[0][s].scale_a, 0, (int)sc);
+                        if (second) D2 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st[1][s].a, b, D2, 4, 4, 0, st[1][s].scale_a, 0, (int)sc);
                     }
                 }
                 n_use++;
                 const float v = (D[0] + D[1]) + (D[2] + D[3]);  // digits 4rq..4rq+3 of weight row jr
-                if (two) pb[(tl * 16 + jr) * PW + wv * 4 + kg] = v;
-                else if (kg < 2) pb[(tl * 16 + jr) * PW + wv * 2 + kg] = v;
+                float *pr = pb + (tl * 16 + jr) * PW + wv * hw;
+                if (ntok == 1) { if (kg < 2) pr[kg] = v; }
+                else pr[kg] = v;
+                if (second) pr[4 + kg] = (D2[0] + D2[1]) + (D2[2] + D2[3]);
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -1205,22 +1228,14 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
         asm volatile("" ::: "memory");
         const uint32_t row_base = (tile_a + tb) * 16;
         const uint32_t nwork = min(nwj, (steps + cw - 1) / cw);
-        if (two) {  // same order of additions per token as the single-token fold: the result does not depend on the pairing
-            for (uint32_t rr = threadIdx.x >> 2; rr < nbt * 16; rr += blockDim.x >> 2) {
-                const uint32_t h = threadIdx.x & 3u;
-                float s = 0.f;
-                for (uint32_t w = 0; w < nwork; w++) s += pb[rr * PW + w * 4 + h];
-                s = dpp_add<0xB1>(s);  // quad_perm [1,0,3,2]
-                if ((h & 1u) == 0 && row_base + rr < rows) ((g_f32wp)(j.out + (int64_t)((h >> 1) * j.out_stride)))[row_base + rr] = s;
-            }
-        } else {
-            for (uint32_t rr = threadIdx.x >> 1; rr < nbt * 16; rr += blockDim.x >> 1) {
-                const uint32_t h = threadIdx.x & 1u;
-                float s = 0.f;
-                for (uint32_t w = 0; w < nwork; w++) s += pb[rr * PW + w * 2 + h];
-                s = dpp_add<0xB1>(s);  // quad_perm [1,0,3,2]
-                if (h == 0 && row_base + rr < rows) ((g_f32wp)j.out)[row_base + rr] = s;
-            }
+        // hw threads per weight row: thread h adds up slot h of every wavefront, the two halves of a token meet in one
+        // DPP step (the same order of additions per token whatever the number of tokens that share the job)
+        for (uint32_t rr = threadIdx.x >> hw_sh; rr < nbt * 16; rr += blockDim.x >> hw_sh) {
+            const uint32_t h = threadIdx.x & (hw - 1u);
+            float s = 0.f;
+            for (uint32_t w = 0; w < nwork; w++) s += pb[rr * PW + w * hw + h];
+            s = dpp_add<0xB1>(s);  // quad_perm [1,0,3,2]
+            if ((h & 1u) == 0 && row_base + rr < rows) ((g_f32wp)(j.out + mx4_out_off(j, h >> 1)))[row_base + rr] = s;
         }
         parity ^= 1u;
     }
@@ -2468,7 +2483,7 @@ size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
     }
     if (n > 0 && jobs[0].kind == KIND_MXFP4_MFMA) {
         const size_t nw = threads / 64;
-        return nw * kMx4Stages * gemv_launch_param(jobs, n) + 2 * (size_t)kMx4BatchTiles * 16 * nw * 4 * sizeof(float);
+        return nw * kMx4Stages * gemv_launch_param(jobs, n) + 2 * (size_t)kMx4BatchTiles * 16 * nw * (jobs[0].batch > 2 ? 8 : 4) * sizeof(float);
     }
     if (n > 0 && jobs[0].kind == KIND_Q4K_Q8K) {  // rings + one partial per (row, super-block), double-buffered
         const size_t nw = threads / 64;

@@ -40,11 +40,13 @@ struct GemvJob {
     // uses w + e*w_sel_stride, aux + e*aux_sel_stride (one bank of equally shaped matrices).
     const uint32_t *sel;
     uint64_t w_sel_stride, aux_sel_stride;
-    // Optional batch (bf16 / Q4_K gates, MXFP4 experts shared by two tokens): `batch` activations x + t*x_stride
-    // against the same weights, results to out + t*out_stride (strides in floats; they may wrap, i.e. be
-    // negative, for the MXFP4 pair).  0 or 1 = a plain matvec.  See gemv_batch_capacity.
+    // Optional batch (bf16 / Q4_K gates, MXFP4 experts shared by up to four tokens): `batch` activations x + t*x_stride
+    // against the same weights, results to out + t*out_stride (strides in floats).  0 or 1 = a plain matvec.
+    // See gemv_batch_capacity.  The MXFP4 matrix-core kernel's tokens sit anywhere: token 1 at x + x_stride (which may
+    // wrap, i.e. be negative), tokens 2 and 3 at x + x_off[0], x + x_off[1]; results likewise with out_stride, out_off.
     uint32_t batch, pad2;
     uint64_t x_stride, out_stride;
+    int64_t x_off[2], out_off[2];
     // Optional gated activation (MoE down projection, MXFP4 matrix-core kernel only): when `x_glu` is set the
     // activation is ClampedGlu(g = x[i], u = x_glu[i]) computed while the activations are prepared; x_glu == x means
     // that g and u are interleaved in x (g = x[2i], u = x[2i+1]: the result of a fused gate_up matrix walked in place).
@@ -53,6 +55,7 @@ struct GemvJob {
     // Optional cost model of the job in the launch's pass list (MXFP4 matrix-core kernel): the job's n_pass is
     // su + tiles * cpt (a start-up allowance, then cpt units per 16-row tile); cpt == 0 means cpr units per tile, no allowance.
     uint32_t cpt, su;
+    uint64_t pad3;        // (the descriptor is a whole number of 16-byte words)
 };
 
 struct GemvLaunch {
@@ -112,7 +115,7 @@ hipError_t router_select_launch(hipStream_t s, const float *logits, uint32_t tok
                                 uint32_t *experts, float *weights);
 hipError_t moe_plan_launch(hipStream_t s, const uint32_t *experts, uint32_t slots, uint32_t k, uint32_t n_experts, const GemvJob &tg,
                            const GemvJob &tu, const GemvJob &td, uint64_t gu_w_stride, uint64_t gu_s_stride, uint64_t dn_w_stride,
-                           uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, bool fused, GemvJob *gu_table, uint32_t *gu_hdr,
+                           uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, bool fused, uint32_t group, GemvJob *gu_table, uint32_t *gu_hdr,
                            GemvJob *dn_table, uint32_t *dn_hdr);
 hipError_t clamped_glu_interleaved_launch(hipStream_t s, const float *gu, float *h, size_t n, float limit, float alpha);
 hipError_t clamped_glu_launch(hipStream_t s, const float *g, const float *u, float *h, size_t n, float limit, float alpha);

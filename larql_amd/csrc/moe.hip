@@ -15,15 +15,40 @@ namespace larql {
 // over the selected logits in rank order (policy 1, NormalisedOverSelected) or
 // over all experts in index order (policy 0, SoftmaxThenSelect).
 // ---------------------------------------------------------------------------
+// Reductions over the wavefront by data-parallel primitives (four steps inside the rows of 16 lanes, two row
+// broadcasts, then lane 63 holds the result): a few cycles per step, where a cross-lane shuffle costs an LDS round trip.
+template <int CTRL, int ROW_MASK, bool BOUND>
+__device__ __forceinline__ uint64_t dpp_max_u64(uint64_t v) {  // lanes without a source read 0: the identity here
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)v, CTRL, ROW_MASK, 0xF, BOUND);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(v >> 32), CTRL, ROW_MASK, 0xF, BOUND);
+    const uint64_t other = ((uint64_t)hi << 32) | lo;
+    return other > v ? other : v;
+}
 __device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
-    for (int o = 32; o > 0; o >>= 1) {
-        uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
-        lo = (uint32_t)__shfl_xor((int)lo, o, 64);
-        hi = (uint32_t)__shfl_xor((int)hi, o, 64);
-        const uint64_t other = ((uint64_t)hi << 32) | lo;
-        v = other > v ? other : v;
-    }
-    return v;
+    v = dpp_max_u64<0xB1, 0xF, true>(v);    // quad_perm [1,0,3,2]
+    v = dpp_max_u64<0x4E, 0xF, true>(v);    // quad_perm [2,3,0,1]
+    v = dpp_max_u64<0x141, 0xF, true>(v);   // row_half_mirror
+    v = dpp_max_u64<0x140, 0xF, true>(v);   // row_mirror
+    v = dpp_max_u64<0x142, 0xA, false>(v);  // row_bcast:15 into rows 1 and 3
+    v = dpp_max_u64<0x143, 0xC, false>(v);  // row_bcast:31 into rows 2 and 3
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, 63), hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), 63);
+    return ((uint64_t)hi << 32) | lo;
+}
+template <int CTRL, int ROW_MASK, bool BOUND>
+__device__ __forceinline__ float dpp_fmax(float v) {  // lanes without a source read -inf
+    return fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp((int)0xFF800000u, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, BOUND)));
+}
+__device__ __forceinline__ float wave_fmax(float v) {
+    v = dpp_fmax<0xB1, 0xF, false>(v);
+    v = dpp_fmax<0x4E, 0xF, false>(v);
+    v = dpp_fmax<0x141, 0xF, false>(v);
+    v = dpp_fmax<0x140, 0xF, false>(v);
+    v = dpp_fmax<0x142, 0xA, false>(v);
+    v = dpp_fmax<0x143, 0xC, false>(v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+__device__ __forceinline__ float lane_value(float v, uint32_t lane_uniform) {  // the lane index must be the same in every lane
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), (int)lane_uniform));
 }
 
 __global__ void __launch_bounds__(64) router_select_kernel(const float *__restrict__ logits, uint32_t n_experts, uint32_t k,
@@ -36,19 +61,18 @@ __global__ void __launch_bounds__(64) router_select_kernel(const float *__restri
     const uint32_t bits = __builtin_bit_cast(uint32_t, l);
     const uint32_t ord = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
     uint64_t key = has ? (((uint64_t)ord << 32) | (uint32_t)(~lane)) : 0;
-    float dmax = has ? l : -__builtin_inff();
-    for (int o = 32; o > 0; o >>= 1) dmax = fmaxf(dmax, __shfl_xor(dmax, o, 64));
+    const float dmax = wave_fmax(has ? l : -__builtin_inff());
     const float ex = has ? expf(l - dmax) : 0.0f;
     float denom = 0.0f;
     if (policy == 0)
-        for (uint32_t i = 0; i < n_experts; i++) denom += __shfl(ex, (int)i, 64);  // index order, as the iterator sums
+        for (uint32_t i = 0; i < n_experts; i++) denom += lane_value(ex, i);  // index order, as the iterator sums
     uint32_t sel_idx[8];
     float sel_ex[8];
     for (uint32_t r = 0; r < k; r++) {
         const uint64_t best = wave_max_u64(key);
-        const uint32_t idx = ~(uint32_t)best;
+        const uint32_t idx = ~(uint32_t)best & 63u;  // (k <= n_experts: a key is always left; the mask keeps the lane index in range regardless)
         sel_idx[r] = idx;
-        sel_ex[r] = __shfl(ex, (int)idx, 64);
+        sel_ex[r] = lane_value(ex, idx);
         if (lane == idx) key = 0;
     }
     if (policy != 0)
@@ -92,14 +116,25 @@ __global__ void weighted_sum_kernel(const float *__restrict__ d, const float *__
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= hidden) return;
     float acc = 0.0f;
-    for (uint32_t r = 0; r < k; r++) acc += weights[(size_t)t * k + r] * d[((size_t)t * k + r) * hidden + i];
+    for (uint32_t r0 = 0; r0 < k; r0 += 4) {  // four loads in flight, added in selection order
+        float w[4], v[4];
+#pragma unroll
+        for (uint32_t q = 0; q < 4; q++) {
+            const bool in = r0 + q < k;
+            w[q] = in ? weights[(size_t)t * k + r0 + q] : 0.0f;
+            v[q] = in ? d[((size_t)t * k + r0 + q) * hidden + i] : 0.0f;
+        }
+#pragma unroll
+        for (uint32_t q = 0; q < 4; q++)
+            if (r0 + q < k) acc += w[q] * v[q];
+    }
     out[(size_t)t * hidden + i] = acc;
 }
 
 // Job lists of an expert block, built on the device from the router's choice (no host round trip): the slots
-// (token, rank) that chose the same expert are paired, in slot order, and every pair (or single) becomes one
-// gate, one up and one down job whose two activations share the expert's weights (GemvJob::batch = 2; the
-// second activation / result sits x_stride / out_stride floats away from the first, in either direction).
+// (token, rank) that chose the same expert are grouped by `group` (2 or 4), in slot order, and every group becomes one
+// gate, one up and one down job whose activations share the expert's weights (GemvJob::batch = tokens in the group;
+// the other activations / results sit x_stride, x_off[] / out_stride, out_off[] floats away from the first).
 // tg / tu / td are the jobs of slot 0 with expert 0 (geometry filled in); tables: [gate jobs | up jobs], [down jobs];
 // headers: {job count, pass total}.  One block; a thread per slot, O(slots) work each.
 // `fused`: tg walks a fused gate_up matrix of 2*inter interleaved rows (no up jobs; a slot's results and the down
@@ -107,79 +142,120 @@ __global__ void weighted_sum_kernel(const float *__restrict__ d, const float *__
 __global__ void __launch_bounds__(256) moe_plan_kernel(const uint32_t *__restrict__ experts, uint32_t slots, uint32_t k, uint32_t n_experts,
                                                        GemvJob tg, GemvJob tu, GemvJob td, uint64_t gu_w_stride, uint64_t gu_s_stride,
                                                        uint64_t dn_w_stride, uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, uint32_t fused,
-                                                       GemvJob *__restrict__ gu_table, uint32_t *__restrict__ gu_hdr,
+                                                       uint32_t group, GemvJob *__restrict__ gu_table, uint32_t *__restrict__ gu_hdr,
                                                        GemvJob *__restrict__ dn_table, uint32_t *__restrict__ dn_hdr) {
     __shared__ uint32_t first_job[1025];  // first job of expert e; [n_experts] = total
     __shared__ uint32_t first_gcost[1025], first_dcost[1025];  // the same for the jobs' places in the two pass lists
-    __shared__ uint32_t cnt[1024];        // slots per expert
-    __shared__ uint32_t ex[4096];         // the router's choice, read once
-    __shared__ uint32_t partner[4096];    // second slot of a job (or ~0)
+    __shared__ __attribute__((aligned(16))) uint32_t cnt[1024];  // slots per expert
+    __shared__ __attribute__((aligned(16))) uint32_t ex[4096];   // the router's choice, read once
+    __shared__ uint32_t first_slot[1025]; // slots of the experts before e
+    __shared__ uint16_t rank[4096];       // a slot's rank among the slots of its expert, in slot order
+    __shared__ uint16_t by_expert[4096];  // the slots ordered by (expert, rank)
     const uint32_t t = threadIdx.x;
-    for (uint32_t e = t; e < n_experts; e += blockDim.x) cnt[e] = 0;
-    for (uint32_t s = t; s < slots; s += blockDim.x) { ex[s] = experts[s]; partner[s] = 0xFFFFFFFFu; }
+    const uint32_t gsh = group == 4 ? 2u : 1u, gmask = group - 1;  // (group is 2 or 4: no divisions below)
+    for (uint32_t e = t; e < ((n_experts + 3u) & ~3u); e += blockDim.x) cnt[e] = 0;
+    for (uint32_t s = t; s < ((slots + 3u) & ~3u); s += blockDim.x) ex[s] = s < slots ? experts[s] : 0xFFFFFFFFu;
     __syncthreads();
-    for (uint32_t s = t; s < slots; s += blockDim.x)
-        if (ex[s] < n_experts) atomicAdd(&cnt[ex[s]], 1u);
-    __syncthreads();
-    // Cost of a job in the launches' pass lists, from cycle counts of the kernel: a tile costs the same whether one
-    // or two tokens share it (its bytes set the pace), and a job segment starts with the preparation of its
-    // activations, worth 4 (one token) or 6 (two) tiles.  Units: steps (a tile = cpr of them).
-    const uint32_t g_tiles = ((uint32_t)tg.rows + 15) / 16, d_tiles = ((uint32_t)td.rows + 15) / 16;
-    const uint32_t g_c1 = tg.cpr, g_c2 = tg.cpr, d_c1 = td.cpr, d_c2 = td.cpr;
-    const uint32_t g_p1 = 4 * g_c1 + g_tiles * g_c1, g_p2 = 6 * g_c1 + g_tiles * g_c2;
-    const uint32_t d_p1 = 4 * d_c1 + d_tiles * d_c1, d_p2 = 6 * d_c1 + d_tiles * d_c2;
-    for (uint32_t e = t; e <= n_experts; e += blockDim.x) {
-        uint32_t f = 0, gc = 0, dc = 0;
-        for (uint32_t q = 0; q < e; q++) {
-            f += (cnt[q] + 1) / 2;
-            gc += (cnt[q] / 2) * g_p2 + (cnt[q] & 1u) * g_p1;
-            dc += (cnt[q] / 2) * d_p2 + (cnt[q] & 1u) * d_p1;
+    // ranks: four earlier slots per LDS read, the reads of a round independent of each other
+    for (uint32_t s = t; s < slots; s += blockDim.x) {
+        const uint32_t e = ex[s];
+        uint32_t r = 0;
+#pragma unroll 4
+        for (uint32_t q = 0; q < s; q += 4) {
+            const uint4 v = *reinterpret_cast<const uint4 *>(&ex[q]);
+            r += (v.x == e ? 1u : 0u) + (q + 1 < s && v.y == e ? 1u : 0u) + (q + 2 < s && v.z == e ? 1u : 0u) + (q + 3 < s && v.w == e ? 1u : 0u);
         }
-        first_job[e] = f; first_gcost[e] = gc; first_dcost[e] = dc;
+        rank[s] = (uint16_t)r;
+        if (e < n_experts) atomicAdd(&cnt[e], 1u);
+    }
+    __syncthreads();
+    // Cost of a job in the launches' pass lists, from cycle counts of the kernel: a tile costs the same however many
+    // tokens share it (its bytes set the pace), and a job segment starts with the preparation of its
+    // activations, worth 4 tiles for one token and 2 more for every further one.  Units: steps (a tile = cpr of them).
+    const uint32_t g_tiles = ((uint32_t)tg.rows + 15) / 16, d_tiles = ((uint32_t)td.rows + 15) / 16;
+    const uint32_t g_c = tg.cpr, d_c = td.cpr;
+    auto g_cost = [&](uint32_t n) { return n ? (2 + 2 * n + g_tiles) * g_c : 0u; };
+    auto d_cost = [&](uint32_t n) { return n ? (2 + 2 * n + d_tiles) * d_c : 0u; };
+    const uint32_t g_full = g_cost(group), d_full = d_cost(group);
+    for (uint32_t e = t; e <= n_experts; e += blockDim.x) {
+        uint32_t f = 0, gc = 0, dc = 0, fs = 0;
+        auto add = [&](uint32_t c) {
+            fs += c;
+            f += (c + gmask) >> gsh;
+            gc += (c >> gsh) * g_full + g_cost(c & gmask);
+            dc += (c >> gsh) * d_full + d_cost(c & gmask);
+        };
+#pragma unroll 2
+        for (uint32_t q = 0; q < e; q += 4) {
+            const uint4 v = *reinterpret_cast<const uint4 *>(&cnt[q]);
+            add(v.x);
+            if (q + 1 < e) add(v.y);
+            if (q + 2 < e) add(v.z);
+            if (q + 3 < e) add(v.w);
+        }
+        first_job[e] = f; first_gcost[e] = gc; first_dcost[e] = dc; first_slot[e] = fs;
     }
     __syncthreads();
     const uint32_t n_jobs = first_job[n_experts], g_total = first_gcost[n_experts], d_total = first_dcost[n_experts];
-    // a slot's rank among the slots of its expert, in slot order: even ranks open a job, odd ranks join it
     for (uint32_t s = t; s < slots; s += blockDim.x) {
         const uint32_t e = ex[s];
-        if (e >= n_experts) continue;
-        uint32_t r = 0;
-        for (uint32_t q = 0; q < s; q++) r += ex[q] == e ? 1u : 0u;
-        if (r & 1u) partner[first_job[e] + r / 2] = s;
+        if (e < n_experts) by_expert[first_slot[e] + rank[s]] = (uint16_t)s;
     }
     __syncthreads();
+    // ranks that are multiples of `group` open a job, the `group - 1` that follow join it
     for (uint32_t s1 = t; s1 < slots; s1 += blockDim.x) {
-        const uint32_t e = ex[s1];
-        if (e >= n_experts) continue;
-        uint32_t r = 0;
-        for (uint32_t q = 0; q < s1; q++) r += ex[q] == e ? 1u : 0u;
-        if (r & 1u) continue;
-        const uint32_t jb = first_job[e] + r / 2;
-        const bool pair = partner[jb] != 0xFFFFFFFFu;
-        const uint32_t s2 = pair ? partner[jb] : s1, nb = pair ? 2u : 1u;
-        const uint32_t tok1 = s1 / k, tok2 = s2 / k;
-        GemvJob a = tg, b = tu, c = td;
-        a.w += (size_t)e * gu_w_stride; a.aux += (size_t)e * gu_s_stride;
-        b.w += (size_t)e * gu_w_stride; b.aux += (size_t)e * gu_s_stride;
-        c.w += (size_t)e * dn_w_stride; c.aux += (size_t)e * dn_s_stride;
-        a.x += (size_t)tok1 * hidden; b.x += (size_t)tok1 * hidden;
+        const uint32_t e = ex[s1], r = rank[s1];
+        if (e >= n_experts || (r & gmask)) continue;
+        const uint32_t jb = first_job[e] + (r >> gsh);
+        const uint32_t nb = min(group, cnt[e] - r);
+        uint32_t sm[4];
+#pragma unroll
+        for (uint32_t q = 0; q < 4; q++) sm[q] = q < nb ? by_expert[first_slot[e] + r + q] : s1;
+        const uint32_t tok1 = s1 / k;
         const size_t gs = fused ? 2 * (size_t)inter : (size_t)inter;  // floats of gate/up results per slot and half
-        a.out += (size_t)s1 * gs; b.out += (size_t)s1 * gs;
-        c.x += (size_t)s1 * gs; c.x_glu += (size_t)s1 * gs; c.out += (size_t)s1 * hidden;
-        a.batch = b.batch = c.batch = nb;
-        a.x_stride = b.x_stride = (uint64_t)(((int64_t)tok2 - (int64_t)tok1) * (int64_t)hidden);
-        a.out_stride = b.out_stride = (uint64_t)(((int64_t)s2 - (int64_t)s1) * (int64_t)gs);
-        c.x_stride = (uint64_t)(((int64_t)s2 - (int64_t)s1) * (int64_t)gs);
-        c.out_stride = (uint64_t)(((int64_t)s2 - (int64_t)s1) * (int64_t)hidden);
-        // (the earlier jobs of this expert are all shared by two tokens)
-        a.pass_begin = first_gcost[e] + (r / 2) * g_p2;
-        b.pass_begin = g_total + a.pass_begin;
-        c.pass_begin = first_dcost[e] + (r / 2) * d_p2;
-        a.n_pass = b.n_pass = pair ? g_p2 : g_p1; c.n_pass = pair ? d_p2 : d_p1;
-        a.cpt = b.cpt = pair ? g_c2 : g_c1; c.cpt = pair ? d_c2 : d_c1;
-        a.su = b.su = (pair ? 6u : 4u) * g_c1; c.su = (pair ? 6u : 4u) * d_c1;
-        gu_table[jb] = a; dn_table[jb] = c;
-        if (!fused) gu_table[n_jobs + jb] = b;
+        const auto tok_off = [&](uint32_t q) { return ((int64_t)(sm[q] / k) - (int64_t)tok1) * (int64_t)hidden; };
+        const auto slot_off = [&](uint32_t q, size_t unit) { return ((int64_t)sm[q] - (int64_t)s1) * (int64_t)unit; };
+        // a job = the template's words with the fields that differ replaced, kept in registers as plain dwords
+        // and stored 16 bytes at a time
+        const auto emit = [&](GemvJob *dst, const GemvJob &tm, size_t w_off, size_t aux_off, size_t x_off, size_t out_off, bool x_by_token,
+                              size_t out_unit, uint32_t pass_begin, uint32_t tiles_cost, uint32_t c1) {
+            static_assert(sizeof(GemvJob) % 16 == 0 && alignof(GemvJob) == 8, "descriptor is a whole number of 16-byte stores");
+            constexpr int N = sizeof(GemvJob) / 4;
+            const uint32_t *src = reinterpret_cast<const uint32_t *>(&tm);
+            uint32_t d[N];
+#pragma unroll
+            for (int i = 0; i < N; i++) d[i] = src[i];
+            const auto put32 = [&](size_t byte_off, uint32_t v) { d[byte_off / 4] = v; };
+            const auto put64 = [&](size_t byte_off, uint64_t v) { d[byte_off / 4] = (uint32_t)v; d[byte_off / 4 + 1] = (uint32_t)(v >> 32); };
+            put64(offsetof(GemvJob, w), (uint64_t)(tm.w + w_off));
+            put64(offsetof(GemvJob, aux), (uint64_t)(tm.aux + aux_off));
+            put64(offsetof(GemvJob, x), (uint64_t)(tm.x + x_off));
+            put64(offsetof(GemvJob, out), (uint64_t)(tm.out + out_off));
+            if (tm.x_glu) put64(offsetof(GemvJob, x_glu), (uint64_t)(tm.x_glu + x_off));
+            put32(offsetof(GemvJob, batch), nb);
+            put64(offsetof(GemvJob, x_stride), (uint64_t)(x_by_token ? tok_off(1) : slot_off(1, gs)));
+            put64(offsetof(GemvJob, out_stride), (uint64_t)slot_off(1, out_unit));
+            put64(offsetof(GemvJob, x_off), (uint64_t)(x_by_token ? tok_off(2) : slot_off(2, gs)));
+            put64(offsetof(GemvJob, x_off) + 8, (uint64_t)(x_by_token ? tok_off(3) : slot_off(3, gs)));
+            put64(offsetof(GemvJob, out_off), (uint64_t)slot_off(2, out_unit));
+            put64(offsetof(GemvJob, out_off) + 8, (uint64_t)slot_off(3, out_unit));
+            put32(offsetof(GemvJob, pass_begin), pass_begin);
+            put32(offsetof(GemvJob, n_pass), (2 + 2 * nb) * c1 + tiles_cost);
+            put32(offsetof(GemvJob, cpt), c1);
+            put32(offsetof(GemvJob, su), (2 + 2 * nb) * c1);
+            uint4 *o = reinterpret_cast<uint4 *>(dst);  // (the tables are 16-byte aligned)
+#pragma unroll
+            for (int i = 0; i < N / 4; i++) o[i] = make_uint4(d[4 * i], d[4 * i + 1], d[4 * i + 2], d[4 * i + 3]);
+        };
+        // (the earlier jobs of this expert are all full groups)
+        const uint32_t g_begin = first_gcost[e] + (r >> gsh) * g_full, d_begin = first_dcost[e] + (r >> gsh) * d_full;
+        emit(gu_table + jb, tg, (size_t)e * gu_w_stride, (size_t)e * gu_s_stride, (size_t)tok1 * hidden, (size_t)s1 * gs, true, gs, g_begin,
+             g_tiles * g_c, g_c);
+        if (!fused)
+            emit(gu_table + n_jobs + jb, tu, (size_t)e * gu_w_stride, (size_t)e * gu_s_stride, (size_t)tok1 * hidden, (size_t)s1 * gs, true, gs,
+                 g_total + g_begin, g_tiles * g_c, g_c);
+        emit(dn_table + jb, td, (size_t)e * dn_w_stride, (size_t)e * dn_s_stride, (size_t)s1 * gs, (size_t)s1 * hidden, false, hidden, d_begin,
+             d_tiles * d_c, d_c);
     }
     if (t == 0) {
         gu_hdr[0] = fused ? n_jobs : 2 * n_jobs; gu_hdr[1] = fused ? g_total : 2 * g_total;
@@ -189,11 +265,11 @@ __global__ void __launch_bounds__(256) moe_plan_kernel(const uint32_t *__restric
 
 hipError_t moe_plan_launch(hipStream_t s, const uint32_t *experts, uint32_t slots, uint32_t k, uint32_t n_experts, const GemvJob &tg,
                            const GemvJob &tu, const GemvJob &td, uint64_t gu_w_stride, uint64_t gu_s_stride, uint64_t dn_w_stride,
-                           uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, bool fused, GemvJob *gu_table, uint32_t *gu_hdr,
+                           uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, bool fused, uint32_t group, GemvJob *gu_table, uint32_t *gu_hdr,
                            GemvJob *dn_table, uint32_t *dn_hdr) {
-    if (n_experts > 1024) return hipErrorInvalidValue;
+    if (n_experts > 1024 || slots > 4096 || (group != 2 && group != 4)) return hipErrorInvalidValue;
     hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(256), 0, s, experts, slots, k, n_experts, tg, tu, td, gu_w_stride, gu_s_stride,
-                       dn_w_stride, dn_s_stride, hidden, inter, fused ? 1u : 0u, gu_table, gu_hdr, dn_table, dn_hdr);
+                       dn_w_stride, dn_s_stride, hidden, inter, fused ? 1u : 0u, group, gu_table, gu_hdr, dn_table, dn_hdr);
     return hipGetLastError();
 }
 

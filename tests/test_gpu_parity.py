@@ -807,10 +807,10 @@ def test_moe_mxfp4_block_matches_oracle(be, fmt, T, E, hidden, inter):
 
 
 def test_moe_mxfp4_tokens_sharing_an_expert_equal_single_token_calls(be, fmt):
-    """Slots that chose the same expert are served two at a time from one read of its weights; a token's result
-    must not depend on who it was paired with: the 13-token block equals 13 one-token blocks bit for bit."""
+    """Slots that chose the same expert are served up to four at a time from one read of its weights; a token's result
+    must not depend on who it shared a job with: the 13-token block equals 13 one-token blocks bit for bit."""
     rng = np.random.default_rng(83)
-    T, E, hidden, inter, k = 13, 6, 384, 320, 4          # 52 slots over 6 experts: pairs, odd leftovers, far-apart partners
+    T, E, hidden, inter, k = 13, 6, 384, 320, 4          # 52 slots over 6 experts: full groups, leftovers of one to three, far-apart companions
 
     def bank(n, kk):
         p, s = [], []
@@ -846,6 +846,47 @@ def test_moe_mxfp4_tokens_sharing_an_expert_equal_single_token_calls(be, fmt):
         hh = np.array([O.clamped_glu(float(a), float(b_)) for a, b_ in zip(g, u)], F)
         acc = (acc + F(w) * O.mxfp4_gemv(dp[e * dwb:(e + 1) * dwb], ds[e * dsz:(e + 1) * dsz], hh, hidden, inter)).astype(F)
     assert rel_l2(got[5], acc) < 1e-5
+
+
+def test_moe_mxfp4_job_groups_of_every_size(be, fmt):
+    """Experts chosen by 1, 2, 3, 4 and 5 slots: jobs of one, two, three and four tokens and a second job for the
+    fifth.  Every token's result equals its one-token call bit for bit."""
+    rng = np.random.default_rng(97)
+    E, hidden, inter, k = 6, 384, 320, 2
+    picks = [(4, 5)] * 5 + [(0, 3), (1, 3), (1, 2), (2, 3), (2, 3)]
+    order = rng.permutation(len(picks))
+    picks = [picks[i] for i in order]
+    T = len(picks)
+    logits = (rng.standard_normal((T, E)) * 0.1).astype(F)
+    for t, (a, b_) in enumerate(picks):
+        logits[t, a] = 5.0 + 0.01 * t
+        logits[t, b_] = 4.0
+
+    def bank(n, kk):
+        p, s = [], []
+        for _ in range(E):
+            pp, ss = O.quantize_mxfp4((rng.standard_normal(n * kk) * 0.05).astype(F), n, kk)
+            p.append(pp); s.append(ss)
+        return np.concatenate(p), np.concatenate(s)
+
+    gp, gs = bank(inter, hidden); up, us = bank(inter, hidden); dp, ds = bank(hidden, inter)
+    x = rng.standard_normal((T, hidden)).astype(F)
+    dev = {n: be.to_device(a) for n, a in dict(gp=gp, gs=gs, up=up, us=us, dp=dp, ds=ds, x=x, lg=logits).items()}
+    b = fmt.Mxfp4Experts(dev["gp"], dev["gs"], dev["up"], dev["us"], dev["dp"], dev["ds"], E, hidden, inter, 7.0, 1.702)
+    de, dw_, do = be.malloc(T * k * 4), be.malloc(T * k * 4), be.malloc(T * hidden * 4)
+    assert be.dev_router_select(dev["lg"], T, E, k, O.NORMALISED_OVER_SELECTED, de, dw_)
+    chosen = be.d2h(de, (T, k), np.uint32)
+    assert sorted(np.bincount(chosen.reshape(-1), minlength=E).tolist()) == [1, 2, 3, 4, 5, 5]
+    wsb = be.moe_mxfp4_workspace_bytes(T, k, hidden, inter)
+    ws = be.malloc(wsb)
+    assert be.dev_moe_mxfp4(b, dev["x"], T, k, de, dw_, do, ws, wsb)
+    be.synchronize()
+    got = be.d2h(do, (T, hidden), F)
+    one = be.malloc(hidden * 4)
+    for t in range(T):
+        assert be.dev_moe_mxfp4(b, dev["x"] + t * hidden * 4, 1, k, de + t * k * 4, dw_ + t * k * 4, one, ws, wsb)
+        be.synchronize()
+        assert np.array_equal(be.d2h(one, hidden, F), got[t]), t
 
 
 @pytest.mark.parametrize("T,E,hidden,inter", [(1, 4, 2880, 2880), (13, 6, 384, 320), (16, 8, 2880, 576)])
