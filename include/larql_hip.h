@@ -344,7 +344,8 @@ typedef struct {
  * selected expert, gate/up matvec -> ClampedGlu -> down matvec, then the
  * weighted sum in selection order.  `experts` stays on the device (the kernels
  * index the bank with it), so routing needs no host round trip.  Five launches.
- * workspace: larql_hip_moe_mxfp4_workspace_bytes(...) of device memory. */
+ * workspace: larql_hip_moe_mxfp4_workspace_bytes(...) of device memory; workspace, x and the packed streams
+ * 16-byte aligned (else LARQL_REFUSED_SHAPE). */
 size_t larql_hip_moe_mxfp4_workspace_bytes(size_t tokens, size_t k, size_t hidden, size_t inter);
 int larql_hip_dev_moe_mxfp4(larql_hip_ctx *ctx, const larql_hip_mxfp4_experts *bank, const float *x, size_t tokens, size_t k,
                             const uint32_t *experts, const float *weights, float *out, void *workspace, size_t workspace_bytes);

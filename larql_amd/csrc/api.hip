@@ -1214,6 +1214,9 @@ int larql_hip_dev_moe_mxfp4(larql_hip_ctx *c, const larql_hip_mxfp4_experts *ban
     if (workspace_bytes < larql_hip_moe_mxfp4_workspace_bytes(tokens, k, hidden, inter))
         return fail(c, LARQL_REFUSED_SHAPE, "moe_mxfp4: workspace too small");
     if (!x || !experts || !weights || !out || !workspace) return LARQL_E_ARG;
+    if (((uintptr_t)workspace & 15) || ((uintptr_t)x & 15) || ((uintptr_t)bank->gate_packed & 15) || ((uintptr_t)bank->up_packed & 15) ||
+        ((uintptr_t)bank->down_packed & 15))
+        return fail(c, LARQL_REFUSED_SHAPE, "moe_mxfp4: workspace, activation and packed-weight pointers must be 16-byte aligned");
     if (!bank->gate_packed || !bank->gate_scales || !bank->down_packed || !bank->down_scales ||
         (!bank->gate_up_interleaved && (!bank->up_packed || !bank->up_scales)))
         return LARQL_E_ARG;

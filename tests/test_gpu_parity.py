@@ -804,6 +804,8 @@ def test_moe_mxfp4_block_matches_oracle(be, fmt, T, E, hidden, inter):
     got = be.d2h(do, (T, hidden), F)
     assert rel_l2(got, want) < 1e-5
     assert not be.dev_moe_mxfp4(b, dev["x"], T, k, de, dw_, do, ws, wsb - 1024)   # short workspace: refused
+    ws2 = be.malloc(wsb + 16)
+    assert not be.dev_moe_mxfp4(b, dev["x"], T, k, de, dw_, do, ws2 + 4, wsb)     # workspace off a 16-byte boundary: refused
 
 
 def test_moe_mxfp4_tokens_sharing_an_expert_equal_single_token_calls(be, fmt):
