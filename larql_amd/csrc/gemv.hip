@@ -988,8 +988,8 @@ __device__ __forceinline__ void run_q4k_q8k(const GemvJob &j, uint32_t tile_a, u
 // weights go global -> LDS -> operand registers without a single unpacking instruction and the block
 // scale is applied by the hardware.  The 16 "B" columns are 16 weight rows; a wavefront owns a K-range
 // of `cw` 128-element steps of those rows and streams its (16 rows x cw steps) tiles through a private
-// LDS ring (16-byte and 1-byte global_load_lds, one per lane and step; a sub-dword load still
-// fills a whole dword slot per lane).
+// LDS ring: a 16-byte global_load_lds per lane and step for the nibbles and one 4-byte copy per tile for the scale
+// bytes of all its steps (a dword per row and step, at whatever alignment the row has; rows need at least 4 blocks).
 //
 // The "A" rows carry the activation in FP4 as well: per step, n = rint(x * 2^(23-e)) (2^e > max|x| of
 // the step) is written in eight balanced base-8 digits d_t in [-4, 4] — all of them e2m1 values — and row t
@@ -1005,7 +1005,8 @@ constexpr int kMx4Stages = 3;
 constexpr int kMx4BatchTiles = 4;
 constexpr int kMx4MaxSteps = 4;    // 128-element steps per wavefront
 constexpr int kMx4MaxWaves = 10;
-constexpr uint32_t kMx4StepBytes = 1024 + 256;  // per step of a wave-tile: 64 lanes x 16 B of nibbles, 64 scale bytes (one dword slot each)
+constexpr uint32_t kMx4StepBytes = 1024;      // per step of a wave-tile: 64 lanes x 16 B of nibbles
+constexpr uint32_t kMx4ScaleBytes = 256;      // per wave-tile: the scale bytes of all its steps, a dword slot per (row, step)
 
 struct Mx4Step {
     i32x8 a;        // this lane's 32 activation digits (FP4, in a[0..3]) of the step
@@ -1122,7 +1123,7 @@ __device__ __forceinline__ void mx4_setup_steps(const GemvJob &j, const Mx4In (&
     }
 }
 
-#define LARQL_MX4_WAIT_CASE(CW) case CW: LARQL_WAIT_VMCNT(2 * CW * (kMx4Stages - 1)); break;
+#define LARQL_MX4_WAIT_CASE(CW) case CW: LARQL_WAIT_VMCNT((CW + 1) * (kMx4Stages - 1)); break;
 
 // tiles [tile_a, tile_b) of one job
 __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a, uint32_t tile_b, uint8_t *lds, uint32_t slot_bytes,
@@ -1151,6 +1152,12 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
         blk[s] = min(b, nb - 1);
     }
 
+    // scale bytes: lane (jr, c) copies the dword that holds blocks 4(step0+c) .. +3 of row jr, moved back to end with the
+    // row where the row has fewer; lane (jr, kg) then finds the byte of its block of step s in slot 16s + jr
+    const uint32_t sc_dw = min((step0 + kg) * 4, nb - 4);
+    uint32_t sc_at[kMx4MaxSteps];
+#pragma unroll
+    for (int s = 0; s < kMx4MaxSteps; s++) sc_at[s] = (16u * s + jr) * 4 + (blk[s] - min((step0 + s) * 4, nb - 4));
     const uint32_t wro_full = jr * row_bytes, sro_full = jr * nb;
     const uint32_t nt = tile_b - tile_a;
     uint32_t it_tile = tile_a, n_issue = 0;
@@ -1168,12 +1175,11 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
         }
         uint8_t *lp = ring + (n_issue % NS) * slot_bytes;
 #pragma unroll
-        for (int s = 0; s < kMx4MaxSteps; s++) {
-            if ((uint32_t)s < cw) {
-                __builtin_amdgcn_global_load_lds((g_vp)(wbase + (wro + blk[s] * 16)), (lds_vp)(lp + s * 1024), 16, 0, 0);
-                __builtin_amdgcn_global_load_lds((g_vp)(sbase + (sro + blk[s])), (lds_vp)(lp + cw * 1024 + s * 256), 1, 0, 0);  // lands zero-extended in dword slot `lane`
-            }
-        }
+        for (int s = 0; s < kMx4MaxSteps; s++)
+            if ((uint32_t)s < cw) __builtin_amdgcn_global_load_lds((g_vp)(wbase + (wro + blk[s] * 16)), (lds_vp)(lp + s * 1024), 16, 0, 0);
+        // the e8m0 bytes of all the wavefront's steps in one copy: lane (row jr, step c = lane/16 < cw) brings the four
+        // scale bytes of its row and step as one dword into slot `lane` (the dword is not aligned in general)
+        if (lane < 16 * cw) __builtin_amdgcn_global_load_lds((g_vp)(sbase + (sro + sc_dw)), (lds_vp)(lp + cw * 1024), 4, 0, 0);
         n_issue++;
         if (it_tile < tile_b) it_tile++;
     };
@@ -1187,7 +1193,7 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
     if (working)
         for (int s = 0; s < NS - 1; s++) issue();
     Mx4Step st[2][kMx4MaxSteps];
-    if (working) mx4_setup_steps(j, xin, st, cw, lane, ring + (NS - 1) * slot_bytes);  // (512 bytes per step fit the 1280 of a slot's step)
+    if (working) mx4_setup_steps(j, xin, st, cw, lane, ring + (NS - 1) * slot_bytes);  // (512 bytes per step fit the 1024 of a slot's step)
 
     uint32_t n_use = 0;
     for (uint32_t tb = 0; tb < nt; tb += R) {
@@ -1206,7 +1212,7 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
                 for (int s = 0; s < kMx4MaxSteps; s++) {
                     if ((uint32_t)s < cw) {
                         const u32x4 q = *reinterpret_cast<const u32x4 *>(slot + s * 1024 + lane * 16);
-                        uint32_t sc = *reinterpret_cast<const uint32_t *>(slot + cw * 1024 + s * 256 + lane * 4) & 0xFFu;
+                        uint32_t sc = slot[cw * 1024 + sc_at[s]];
                         const bool live = valid[s] && sc != 0;  // e8m0 0 is 0.0 here; blocks past the row end do not exist
                         sc = valid[s] ? sc : 127u;
                         i32x8 b = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -2287,7 +2293,7 @@ int gemv_effective_kind(const GemvJob &j) {
         return KIND_Q8_0_MFMA;
     if (j.kind == KIND_BF16 && j.batch >= 2) return KIND_BF16_MFMA;
     if (j.kind == KIND_Q4K && j.batch >= 2) return KIND_Q4K_BATCH;
-    if (j.kind == KIND_MXFP4 && g_mxfp4_mfma && j.k >= 32 && j.k % 32 == 0 && mx4_steps_per_wave((j.k + 127) / 128) != 0 &&
+    if (j.kind == KIND_MXFP4 && g_mxfp4_mfma && j.k >= 128 && j.k % 32 == 0 && mx4_steps_per_wave((j.k + 127) / 128) != 0 &&
         j.rows < 0x7FFFFFF0ull)
         return KIND_MXFP4_MFMA;
     if (j.kind == KIND_Q4K && g_q4k_mfma && !j.sel && j.k % 256 == 0 && j.k / 256 >= 1 && q4k_mfma_waves(j.k / 256) != 0 &&
@@ -2463,7 +2469,7 @@ uint32_t gemv_launch_param(const GemvJob *jobs, size_t n) {
     if (n > 0 && jobs[0].kind == KIND_MXFP4_MFMA) {  // ring slot: room for the longest K-range a wavefront owns
         uint32_t cw = 1;
         for (size_t i = 0; i < n; i++) cw = std::max(cw, mx4_steps_per_wave((jobs[i].k + 127) / 128));
-        return cw * kMx4StepBytes;
+        return cw * kMx4StepBytes + kMx4ScaleBytes;
     }
     return 0;
 }

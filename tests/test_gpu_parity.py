@@ -411,6 +411,21 @@ def test_mxfp4_gemv_matches_dequant_reference(be):
     assert be.mxfp4_gemv_multi([(p, s, n, k), (p[:-1], s, n, k)], x) is None
 
 
+@pytest.mark.parametrize("n,k", [(33, 128), (50, 160), (19, 224), (70, 384), (40, 992), (37, 4096), (21, 5120), (16, 96)])
+def test_mxfp4_gemv_row_lengths_and_block_scales(be, n, k):
+    """Rows of 3 to 160 blocks (odd block counts put a row's scale bytes at odd addresses; partial last steps; k = 96 is
+    below what the matrix-core kernel takes), every block with its own power-of-two magnitude so that a scale byte
+    taken from the wrong block or row shows."""
+    rng = np.random.default_rng(1000 + k)
+    w = (rng.standard_normal((n, k // 32, 32)) * 0.02).astype(F)
+    w *= np.exp2(rng.integers(-6, 7, size=(n, k // 32, 1))).astype(F)
+    w = w.reshape(-1)
+    x = rng.standard_normal(k).astype(F)
+    p, s = O.quantize_mxfp4(w, n, k)
+    assert len(set(s.tolist())) >= 8
+    assert rel_l2(be.mxfp4_gemv(p, s, x, n, k), O.mxfp4_gemv(p, s, x, n, k)) < TOL
+
+
 # ---------------------------------------------------------- dense + Q4_0
 def test_dense_gemvs(be):
     n, k = 1000, 2560
