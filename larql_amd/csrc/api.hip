@@ -215,10 +215,10 @@ std::vector<std::vector<GemvJob>> group_by_kind(const std::vector<GemvJob> &jobs
     std::vector<GemvJob> jobs(jobs_in);
     for (GemvJob &j : jobs) j.kind = gemv_effective_kind(j);  // Q4_K rows the matrix-core kernel takes get their own launch
     std::vector<std::vector<GemvJob>> groups;
-    bool done[15] = {};
+    bool done[16] = {};
     for (size_t i = 0; i < jobs.size(); i++) {
         const int kind = jobs[i].kind;
-        if (jobs[i].rows == 0 || kind < 0 || kind > 14 || done[kind]) continue;
+        if (jobs[i].rows == 0 || kind < 0 || kind > 15 || done[kind]) continue;
         done[kind] = true;
         std::vector<GemvJob> live;
         for (size_t t = i; t < jobs.size(); t++)

@@ -827,6 +827,233 @@ __device__ __forceinline__ void run_q4k_mfma(const GemvJob &j, uint32_t tile_a, 
 }
 
 // ---------------------------------------------------------------------------
+// Q6_K on the matrix cores: the scheme of the Q4_K kernel above for 210-byte super-blocks (q6k_matvec::dispatch,
+// larql-compute/src/cpu/ops/q6k_matvec.rs:45-91: per 16-element group sub = sum (q - 32) * x; acc += (d * sc) * sub).
+//
+// A wave-tile is 16 rows x one super-block, copied global -> LDS as 13 sixteen-byte pieces per row (ql, qh, scales)
+// plus a two-byte piece for d.  The blocks are only 2-byte aligned in memory: the copies take any alignment (at
+// ~12 % of the bandwidth that aligned ones reach) and land on a 208-byte pitch, so that every LDS read is an aligned
+// ds_read_b128.  (Copying the 14 aligned pieces that contain a block instead moves the misalignment to the LDS side,
+// where it costs more: a misaligned ds_read_b128 is correct but slow, five aligned dwords and a byte rotation per
+// field add instructions to a kernel that is within reach of the vector issue limit; both were measured slower.)
+// One v_mfma_i32_16x16x64_i8 covers 64 weights = four scale
+// groups: lane (row j, kq) supplies in its 16 k-slots the 16 six-bit codes of group 4m + kq of weight row j (its 16
+// ql bytes serve MFMAs 2h (low nibbles) and 2h+1 (high nibbles) of half h, its 16 qh bytes give both their top bits:
+// four instructions per four codes), and A row 4g + i carries limb i of the activations of group 4m + g in that
+// group's k-slots, zero elsewhere.  After the MFMA lane (j, rq) holds the four exact limb sums of group 4m + rq of
+// row j — the group whose int8 scale it applies.  The -32 goes through the group's sum of x.  Four MFMAs per tile,
+// none accumulates into another.  The activations of a column (256 elements) are turned into limbs by all 64 lanes,
+// four elements each, and go through LDS (limb planes) into the operand layout; they stay there for the job.
+// ---------------------------------------------------------------------------
+constexpr int kQ6kStages = 3;
+constexpr int kQ6kBatchTiles = 2;
+constexpr int kQ6kMaxColPasses = 4;
+constexpr int kQ6kMaxWaves = 10;
+constexpr uint32_t kQ6kPitch = 208;                          // ql 128, qh 64, scales 16
+constexpr uint32_t kQ6kTileBytes = 16 * kQ6kPitch + 64;      // + a dword slot per row for d
+constexpr uint32_t kQ6kColBytes = 1024 + 64 + 16;            // four limb planes of 256 bytes, 16 group sums, k
+
+struct Q6kCol {
+    Q4kOp xm[4];     // A operand of MFMA m: limb (row % 4) of group 4m + kq in this lane's k-slots if row / 4 == kq, else zero
+    float sumx[4];   // -32 * the sum of x over group 4m + kq
+    float k;         // 2^(e-27)
+};
+
+// turns the lane's four activations (elements 4*lane .. 4*lane+3 of the column) into limbs and group sums at `cp`
+__device__ __forceinline__ void q6k_mfma_prepare_col(const f32x4 v, uint32_t lane, uint8_t *cp) {
+    const float mx = wave_max_nonneg(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+    int ex = 0;
+    if (mx > 0.f && mx < __builtin_inff()) (void)frexpf(mx, &ex);  // mx = f * 2^ex, f in [0.5, 1)
+    ex = max(-90, min(120, ex));
+    const float to_int = ldexpf(1.f, 27 - ex);  // |x| * to_int < 2^27
+    const float e[4] = {v.x, v.y, v.z, v.w};
+    uint32_t pl[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        // n = l0*128^3 + l1*128^2 + l2*128 + l3 with l1..l3 in [-64, 63], l0 in [-64, 64]
+        const int n = (int)__builtin_rintf(e[t] * to_int);
+        const int l3 = ((n + 64) & 127) - 64, n1 = (n - l3) >> 7;
+        const int l2 = ((n1 + 64) & 127) - 64, n2 = (n1 - l2) >> 7;
+        const int l1 = ((n2 + 64) & 127) - 64, l0 = (n2 - l1) >> 7;
+        pl[0] |= ((uint32_t)l0 & 0xFFu) << (8 * t); pl[1] |= ((uint32_t)l1 & 0xFFu) << (8 * t);
+        pl[2] |= ((uint32_t)l2 & 0xFFu) << (8 * t); pl[3] |= ((uint32_t)l3 & 0xFFu) << (8 * t);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) *reinterpret_cast<uint32_t *>(cp + i * 256 + 4 * lane) = pl[i];
+    float sm = (v.x + v.y) + (v.z + v.w);
+    sm = dpp_add<0xB1>(sm);  // quad_perm [1,0,3,2]
+    sm = dpp_add<0x4E>(sm);  // quad_perm [2,3,0,1]: the 16 elements of group lane / 4
+    const uint32_t g = lane >> 2;
+    if ((lane & 3u) == 0) *reinterpret_cast<float *>(cp + 1024 + 4 * ((g & 3u) * 4 + (g >> 2))) = sm;  // [g % 4][g / 4]
+    if (lane == 0) *reinterpret_cast<float *>(cp + 1024 + 64) = ldexpf(1.f, ex - 27);
+}
+
+__device__ __forceinline__ void q6k_mfma_fetch_col(Q6kCol &col, const uint8_t *cp, uint32_t jr, uint32_t kq) {
+    const bool mine = (jr >> 2) == kq;
+    const uint8_t *lp = cp + (jr & 3u) * 256 + 16 * kq;
+#pragma unroll
+    for (int m = 0; m < 4; m++) {
+        const u32x4 t = *reinterpret_cast<const u32x4 *>(lp + 64 * m);  // group 4m + kq
+        col.xm[m].u[0] = mine ? t.x : 0u; col.xm[m].u[1] = mine ? t.y : 0u;
+        col.xm[m].u[2] = mine ? t.z : 0u; col.xm[m].u[3] = mine ? t.w : 0u;
+    }
+    const f32x4 sm = *reinterpret_cast<const f32x4 *>(cp + 1024 + 16 * kq);
+    col.sumx[0] = -32.f * sm.x; col.sumx[1] = -32.f * sm.y; col.sumx[2] = -32.f * sm.z; col.sumx[3] = -32.f * sm.w;
+    col.k = *reinterpret_cast<const float *>(cp + 1024 + 64);
+}
+
+// one wave-tile from its LDS slot: 16 rows x one super-block against the column's activations
+__device__ __forceinline__ float q6k_mfma_tile(const uint8_t *slot, const Q6kCol &col, uint32_t j, uint32_t kq) {
+    const uint8_t *sp = slot + j * kQ6kPitch;
+    u32x4 ql[2], qh[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        ql[h] = *reinterpret_cast<const u32x4 *>(sp + 64 * h + 16 * kq);
+        qh[h] = *reinterpret_cast<const u32x4 *>(sp + 128 + 32 * h + 16 * (kq & 1u));
+    }
+    const u32x4 scs = *reinterpret_cast<const u32x4 *>(sp + 192);
+    const float d = half_bits_to_float(*reinterpret_cast<const uint32_t *>(slot + 16 * kQ6kPitch + 4 * j) & 0xFFFFu);
+    // top bits: MFMA 2h wants bits s0, s0+1 of the qh bytes in bits 4-5 (a left shift by 4 - s0), MFMA 2h+1 bits
+    // s0+4, s0+5 (a right shift by s0); what crosses a byte boundary falls outside the mask
+    const uint32_t s0 = 2u * (kq >> 1), sl = 4u - s0;
+    const i32x4 zero = {0, 0, 0, 0};
+    float acc = 0.f;
+#pragma unroll
+    for (int m = 0; m < 4; m++) {
+        const int h = m >> 1;
+        Q4kOp b;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            if (m & 1) b.u[i] = ((qh[h][i] >> s0) & 0x30303030u) | ((ql[h][i] >> 4) & 0x0F0F0F0Fu);
+            else b.u[i] = ((qh[h][i] << sl) & 0x30303030u) | (ql[h][i] & 0x0F0F0F0Fu);
+        }
+        const i32x4 D = __builtin_amdgcn_mfma_i32_16x16x64_i8(col.xm[m].v, b.v, zero, 0, 0, 0);
+        // this lane's group is 4m + kq: D = its four limb sums; pairs of limbs meet as integers (exact, below 2^24)
+        const float hi = (float)(D[0] * 128 + D[1]), lo = (float)(D[2] * 128 + D[3]);
+        const float dot = __builtin_fmaf(hi, 16384.f, lo);
+        const float sc = (float)(int)(int8_t)(scs[m] >> (8u * kq));
+        acc = __builtin_fmaf(sc, __builtin_fmaf(dot, col.k, col.sumx[m]), acc);  // (sumx holds -32 * the group's sum of x)
+    }
+    return d * acc;
+}
+
+// tiles [tile_a, tile_b) of one job; `parity` flips per batch (double-buffered partials); `cols_pitch` = columns per
+// wavefront the launch keeps room for
+__device__ __forceinline__ void run_q6k_mfma(const GemvJob &j, uint32_t tile_a, uint32_t tile_b, uint8_t *lds, uint32_t cols_pitch,
+                                             uint32_t &parity) {
+    constexpr int NS = kQ6kStages, R = kQ6kBatchTiles;
+    const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t nw_launch = blockDim.x >> 6;
+    const uint32_t jr = lane & 15u, kq = lane >> 4;
+    const uint32_t nwj = j.rpp, cpr = j.cpr, PW = nwj * 4;
+    const uint32_t rows = (uint32_t)j.rows, row_bytes = (uint32_t)j.row_bytes;
+    uint8_t *ring = lds + wv * (NS * kQ6kTileBytes);
+    float *part = reinterpret_cast<float *>(lds + nw_launch * (NS * kQ6kTileBytes));
+    uint8_t *cols = lds + nw_launch * (NS * kQ6kTileBytes) + 2 * R * 16 * nw_launch * 4 * sizeof(float) + wv * (cols_pitch * kQ6kColBytes);
+    const uint32_t np = wv < nwj ? (cpr - wv + nwj - 1) / nwj : 0;  // columns wv, wv+nwj, ... of this wavefront
+
+    // lane's pieces of a wave-tile: 16-byte piece u = 13 * row + piece (u < 208), and d of row `lane` (lane < 16)
+    uint32_t pr[4], po[4], o[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t u = min(64u * i + lane, 207u);
+        pr[i] = u / 13;
+        po[i] = (u - pr[i] * 13) * 16;
+        o[i] = pr[i] * row_bytes + po[i];
+    }
+    const uint32_t od = (lane & 15u) * row_bytes + 208;
+    const uint8_t *wcol = j.w + (size_t)wv * 210;
+    const uint32_t nt = tile_b - tile_a;
+
+    // issue cursor: wave-tiles in the order they are consumed (batch, column pass, tile of the batch)
+    uint32_t it_tb = 0, it_p = 0, it_tl = 0, n_issue = 0;
+    auto issue = [&]() {
+        // past the end the last wave-tile is read again: every wavefront keeps the same number of loads in flight
+        const uint32_t tl = min(tile_a + it_tb + it_tl, tile_b - 1);
+        const uint32_t rb = tl * 16, lim = min(15u, rows - 1 - rb);  // (rows of a ragged last tile are clamped)
+        const uint8_t *gp = wcol + (size_t)it_p * nwj * 210 + (size_t)rb * row_bytes;
+        uint8_t *lp = ring + (n_issue % NS) * kQ6kTileBytes;
+        // wave-uniform 64-bit base + per-lane 32-bit offset; only a ragged last tile recomputes the offsets
+        uint32_t a0 = o[0], a1 = o[1], a2 = o[2], a3 = o[3], ad = od;
+        if (rb + 16 > rows) {
+            a0 = min(pr[0], lim) * row_bytes + po[0]; a1 = min(pr[1], lim) * row_bytes + po[1];
+            a2 = min(pr[2], lim) * row_bytes + po[2]; a3 = min(pr[3], lim) * row_bytes + po[3];
+            ad = min(lane & 15u, lim) * row_bytes + 208;
+        }
+        __builtin_amdgcn_global_load_lds((g_vp)(gp + a0), (lds_vp)lp, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((g_vp)(gp + a1), (lds_vp)(lp + 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((g_vp)(gp + a2), (lds_vp)(lp + 2048), 16, 0, 0);
+        if (lane < 16) {
+            __builtin_amdgcn_global_load_lds((g_vp)(gp + a3), (lds_vp)(lp + 3072), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((g_vp)(gp + ad), (lds_vp)(lp + 16 * kQ6kPitch), 2, 0, 0);
+        }
+        n_issue++;
+        if (it_tb < nt) {
+            const uint32_t nb = min((uint32_t)R, nt - it_tb);
+            if (++it_tl == nb) {
+                it_tl = 0;
+                if (++it_p == np) { it_p = 0; it_tb += R; }
+            }
+        }
+    };
+    // the activations of all this wavefront's columns are requested first and together, then prepared while the tiles fly
+    f32x4 raw[kQ6kMaxColPasses];
+#pragma unroll
+    for (int p = 0; p < kQ6kMaxColPasses; p++)
+        if ((uint32_t)p < np) raw[p] = ((g_f4p)(j.x + (size_t)(wv + nwj * p) * 256))[lane];
+    if (np >= 1)
+        for (int s = 0; s < NS - 1; s++) issue();
+#pragma unroll
+    for (int p = 0; p < kQ6kMaxColPasses; p++)
+        if ((uint32_t)p < np) q6k_mfma_prepare_col(raw[p], lane, cols + p * kQ6kColBytes);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own writes, own reads: program order is enough
+    Q6kCol col;
+    if (np == 1) q6k_mfma_fetch_col(col, cols, jr, kq);
+
+    uint32_t n_use = 0;
+    for (uint32_t tb = 0; tb < nt; tb += R) {
+        float *pb = part + parity * (R * 16 * nw_launch * 4);
+        const uint32_t nb = min((uint32_t)R, nt - tb);
+        if (np >= 1) {
+            float racc[R];
+#pragma unroll
+            for (int tl = 0; tl < R; tl++) racc[tl] = 0.f;
+#pragma unroll 1
+            for (uint32_t p = 0; p < np; p++) {
+                if (np > 1) q6k_mfma_fetch_col(col, cols + p * kQ6kColBytes, jr, kq);
+#pragma unroll
+                for (int tl = 0; tl < R; tl++) {
+                    if ((uint32_t)tl < nb) {
+                        issue();
+                        LARQL_WAIT_VMCNT(5 * (NS - 1));  // at most NS-1 younger wave-tiles still in flight: the oldest has landed
+                        asm volatile("" ::: "memory");
+                        racc[tl] += q6k_mfma_tile(ring + (n_use % NS) * kQ6kTileBytes, col, jr, kq);
+                        n_use++;
+                    }
+                }
+            }
+#pragma unroll
+            for (int tl = 0; tl < R; tl++)
+                if ((uint32_t)tl < nb) pb[(tl * 16 + jr) * PW + wv * 4 + kq] = racc[tl];
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        // fold: 4 lanes per row, lane q sums the group-q partial of every wavefront in order
+        const uint32_t row_base = (tile_a + tb) * 16;
+        for (uint32_t rr = threadIdx.x >> 2; rr < nb * 16; rr += blockDim.x >> 2) {
+            const uint32_t qd = threadIdx.x & 3u;
+            float s = 0.f;
+            for (uint32_t k = 0; k < nwj; k++) s += pb[rr * PW + k * 4 + qd];
+            s = dpp_add<0xB1>(s);  // quad_perm [1,0,3,2]
+            s = dpp_add<0x4E>(s);  // quad_perm [2,3,0,1]
+            if (qd == 0 && row_base + rr < rows) ((g_f32wp)j.out)[row_base + rr] = s;
+        }
+        parity ^= 1u;
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Q4_K weights against a Q8_K activation (q4k_q8k_matvec_scalar, larql-compute/src/cpu/ops/q4k_q8k_dot/
 // q4k_scalar.rs:15-84): the activation is already int8, so one operand set replaces the four digit sets of the
 // f32 kernel.  A row m of the "A" operand is sub-block m (rows 8..15 are zero): its 32 codes sit in the k-slots
@@ -2100,6 +2327,31 @@ __global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_mfma_kernel(GemvLa
     LARQL_WAIT_VMCNT(0);
 }
 
+// Q6_K on the matrix cores: the same sweep and cost model as the Q4_K kernel.
+__global__ void __launch_bounds__(kQ6kMaxWaves * 64) gemv_q6k_mfma_kernel(GemvLaunch L) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t q6k_lds[];
+    const GemvJob *jobs = L.table ? L.table : L.inl;
+    const uint64_t P = L.total_passes;
+    uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
+    const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
+    uint32_t lo = 0, hi = L.n_jobs;
+    while (lo + 1 < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if ((uint32_t)__builtin_amdgcn_readfirstlane(jobs[mid].pass_begin) <= p) lo = mid; else hi = mid;
+    }
+    uint32_t ji = lo, parity = 0;
+    while (p < p_end) {
+        const GemvJob j = uniform_job(jobs + ji);
+        const uint32_t seg_end = min(p_end, j.pass_begin + j.n_pass);
+        const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin, cpt = (uint32_t)j.pad, su = j.pad2;
+        const uint32_t tile_a = a > su ? (a - su + cpt - 1) / cpt : 0, tile_b = b > su ? (b - su + cpt - 1) / cpt : 0;
+        if (tile_a < tile_b) run_q6k_mfma(j, tile_a, tile_b, q6k_lds, L.pad, parity);
+        p = seg_end;
+        ji++;
+    }
+    LARQL_WAIT_VMCNT(0);
+}
+
 // Q4_K x Q8_K: the same sweep and cost model as the Q4_K kernel.
 __global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_q8k_kernel(GemvLaunch L) {
     extern __shared__ __attribute__((aligned(16))) uint8_t q8k_lds[];
@@ -2265,6 +2517,20 @@ static uint32_t q4k_mfma_waves(uint64_t cpr) {
     return best;  // 0: row too long for this path
 }
 
+static uint32_t q6k_mfma_waves(uint64_t cpr) {  // as q4k_mfma_waves: up to 10 wavefronts, up to 4 columns each
+    if (cpr <= (uint64_t)kQ6kMaxWaves) return (uint32_t)cpr;
+    uint32_t best = 0;
+    uint64_t best_slots = ~0ull;
+    for (uint32_t nw = 10; nw >= 6; nw--) {
+        const uint64_t passes = (cpr + nw - 1) / nw;
+        if (passes > (uint64_t)kQ6kMaxColPasses) continue;
+        if (passes * nw < best_slots) { best_slots = passes * nw; best = nw; }
+    }
+    return best;  // 0: row too long for this path
+}
+
+static int g_q6k_mfma = getenv("LARQL_HIP_Q6K_MFMA") ? atoi(getenv("LARQL_HIP_Q6K_MFMA")) : 1;
+
 static int g_q4k_mfma = getenv("LARQL_HIP_Q4K_MFMA") ? atoi(getenv("LARQL_HIP_Q4K_MFMA")) : 1;
 
 static int g_mxfp4_mfma = getenv("LARQL_HIP_MXFP4_MFMA") ? atoi(getenv("LARQL_HIP_MXFP4_MFMA")) : 1;
@@ -2299,6 +2565,9 @@ int gemv_effective_kind(const GemvJob &j) {
     if (j.kind == KIND_Q4K && g_q4k_mfma && !j.sel && j.k % 256 == 0 && j.k / 256 >= 1 && q4k_mfma_waves(j.k / 256) != 0 &&
         j.rows < 0x7FFFFFF0ull && (j.k / 256) * 144 * j.rows < (1ull << 62))
         return KIND_Q4K_MFMA;
+    if (j.kind == KIND_Q6K && g_q6k_mfma && !j.sel && j.k % 256 == 0 && j.k / 256 >= 1 && q6k_mfma_waves(j.k / 256) != 0 &&
+        j.rows < 0x7FFFFFF0ull && (j.k / 256) * 210 * j.rows < (1ull << 62))
+        return KIND_Q6K_MFMA;
     return j.kind;
 }
 
@@ -2354,6 +2623,23 @@ bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
         const uint64_t tiles = (j.rows + 15) / 16;
         if (tiles * steps > 0x7FFFFFFFull) return false;
         j.n_pass = (uint32_t)(tiles * steps);
+        return true;
+    }
+    if (j.kind == KIND_Q6K_MFMA) {  // geometry and cost model as for the Q4_K matrix-core kernel
+        if (j.k == 0 || j.k % 256 != 0) return false;
+        const uint64_t cpr = j.k / 256;
+        const uint32_t nw = q6k_mfma_waves(cpr);
+        if (nw == 0 || nw * 64 > threads) return false;
+        j.cpr = (uint32_t)cpr;
+        j.rpp = nw;
+        j.row_bytes = cpr * 210;
+        const uint64_t tiles = (j.rows + 15) / 16;
+        const uint64_t np = (cpr + nw - 1) / nw;
+        const uint64_t cpt = np == 1 ? 16 : np * 19, startup = np == 1 ? 72 : 180;
+        j.pad = (int32_t)cpt;
+        j.pad2 = (uint32_t)startup;
+        if (startup + tiles * cpt > 0x7FFFFFFFull) return false;
+        j.n_pass = (uint32_t)(startup + tiles * cpt);
         return true;
     }
     if (j.kind == KIND_Q4K_MFMA || j.kind == KIND_Q4K_Q8K) {
@@ -2430,6 +2716,15 @@ uint32_t gemv_pick_threads(const GemvJob *jobs, size_t n) {
         }
         return nw * 64;
     }
+    if (n > 0 && jobs[0].kind == KIND_Q6K_MFMA) {
+        uint32_t nw = 0;
+        for (size_t i = 0; i < n; i++) {
+            const uint32_t w = q6k_mfma_waves(jobs[i].k / 256);
+            if (w == 0) return 0;
+            if (w > nw) nw = w;
+        }
+        return nw * 64;
+    }
     if (n > 0 && (jobs[0].kind == KIND_Q4K_MFMA || jobs[0].kind == KIND_Q4K_Q8K)) {
         uint32_t nw = 0;
         for (size_t i = 0; i < n; i++) {
@@ -2471,6 +2766,15 @@ uint32_t gemv_launch_param(const GemvJob *jobs, size_t n) {
         for (size_t i = 0; i < n; i++) cw = std::max(cw, mx4_steps_per_wave((jobs[i].k + 127) / 128));
         return cw * kMx4StepBytes + kMx4ScaleBytes;
     }
+    if (n > 0 && jobs[0].kind == KIND_Q6K_MFMA) {  // columns per wavefront to keep room for
+        uint32_t np = 1;
+        for (size_t i = 0; i < n; i++) {
+            const uint64_t cpr = jobs[i].k / 256;
+            const uint32_t nw = q6k_mfma_waves(cpr);
+            if (nw) np = std::max(np, (uint32_t)((cpr + nw - 1) / nw));
+        }
+        return np;
+    }
     return 0;
 }
 
@@ -2497,6 +2801,11 @@ size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
         for (size_t i = 0; i < n; i++) cpr = std::max<uint64_t>(cpr, jobs[i].k / 256);
         return nw * kQ4kStages * kQ4kTileBytes + 2 * (size_t)kQ4kBatchTiles * 16 * cpr * sizeof(float);
     }
+    if (n > 0 && jobs[0].kind == KIND_Q6K_MFMA) {
+        const size_t nw = threads / 64;
+        return nw * kQ6kStages * kQ6kTileBytes + 2 * (size_t)kQ6kBatchTiles * 16 * nw * 4 * sizeof(float) +
+               nw * gemv_launch_param(jobs, n) * kQ6kColBytes;
+    }
     if (n > 0 && jobs[0].kind == KIND_Q4K_MFMA) {
         const size_t nw = threads / 64;
         bool multi = false;  // some row needs several column passes: room for the prepared activations
@@ -2515,7 +2824,7 @@ size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
 
 uint32_t gemv_wgs_per_cu(int kind, uint32_t threads, size_t lds, uint32_t dflt) {
     if (kind != KIND_Q4K_MFMA && kind != KIND_MXFP4_MFMA && kind != KIND_BF16_MFMA && kind != KIND_Q4K_BATCH && kind != KIND_Q8_0_MFMA &&
-        kind != KIND_Q4K_Q8K)
+        kind != KIND_Q4K_Q8K && kind != KIND_Q6K_MFMA)
         return dflt;
     // as many workgroups as LDS (160 KB per CU) allows, up to 12 wavefronts per CU (3 per SIMD at this register count)
     const uint32_t by_lds = (uint32_t)((160 * 1024) / lds), by_waves = 12 / (threads / 64);
@@ -2573,6 +2882,16 @@ hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32
                 attr_set = true;
             }
             hipLaunchKernelGGL(gemv_q4k_mfma_kernel, dim3(grid), dim3(threads), lds, stream, L);
+            break;
+        }
+        case KIND_Q6K_MFMA: {
+            static bool attr_set = false;  // dynamic LDS above 64 KB has to be allowed once per process
+            if (!attr_set) {
+                hipError_t e = hipFuncSetAttribute((const void *)gemv_q6k_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                if (e != hipSuccess) return e;
+                attr_set = true;
+            }
+            hipLaunchKernelGGL(gemv_q6k_mfma_kernel, dim3(grid), dim3(threads), lds, stream, L);
             break;
         }
         case KIND_Q4K_Q8K: {

@@ -15,7 +15,8 @@ enum GemvKind : int32_t {
     KIND_Q8_0_MFMA = 11, // internal: ggml Q8_0 rows short enough for the matrix-core kernel
     KIND_Q6K = 12,       // Q6_K, 210-byte super-blocks (K-slice kernel)
     KIND_Q4K_Q8K = 13,   // Q4_K weights against a Q8_K activation (integer dots on the matrix cores); x = the Q8_K device layout
-    KIND_Q6K_Q8K = 14    // Q6_K weights against a Q8_K activation (K-slice kernel, v_dot4)
+    KIND_Q6K_Q8K = 14,   // Q6_K weights against a Q8_K activation (K-slice kernel, v_dot4)
+    KIND_Q6K_MFMA = 15   // internal: Q6_K rows short enough for the matrix-core kernel
 };
 
 constexpr int kGemvMaxThreads = 512;

@@ -137,9 +137,11 @@ def test_q4k_dual_and_matmul(be):
 
 
 # ------------------------------------------------------------------ Q6_K
-@pytest.mark.parametrize("rows,cols", [(2560, 10240), (1031, 2560), (77, 256), (5, 768), (640, 2304), (4100, 512), (1, 5120)])
+@pytest.mark.parametrize("rows,cols", [(2560, 10240), (1031, 2560), (77, 256), (5, 768), (640, 2304), (4100, 512), (1, 5120), (33, 7936),
+                                       (19, 12800)])
 def test_q6k_matvec_matches_oracle(be, fmt, rows, cols):
-    # rows of an odd number of 210-byte super-blocks leave every other row 2 bytes off a dword boundary
+    # rows of an odd number of 210-byte super-blocks leave every other row 2 bytes off a dword boundary; 31 super-blocks
+    # take 4 columns per wavefront of the matrix-core kernel, 50 are beyond it (K-slice kernel)
     w, x = weights(rows * 3 + cols, rows, cols)
     w[0, :16] *= 1e-4
     q = O.quantize_q6_k(w)
