@@ -49,6 +49,8 @@ struct larql_hip_ctx {
     void *table_host[4] = {nullptr, nullptr, nullptr, nullptr};
     size_t table_host_cap[4] = {0, 0, 0, 0};
     hipEvent_t table_ev[4] = {nullptr, nullptr, nullptr, nullptr};
+    void *table_sent_dst[4] = {nullptr, nullptr, nullptr, nullptr};  // where the table staged in table_host[i] went, and its size:
+    size_t table_sent_bytes[4] = {0, 0, 0, 0};                      // an identical table for the same place is not sent again
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     uint8_t *log2_up = nullptr;  // 256-entry table for the MXFP4 encoder
     int *nan_flag = nullptr;
@@ -171,8 +173,13 @@ int prepare_same_kind(larql_hip_ctx *c, std::vector<GemvJob> &live, void *table_
         P.L.table = nullptr;
     } else {
         const size_t bytes = live.size() * sizeof(GemvJob);
-        if (stage_slot >= 0) {
+        if (stage_slot >= 0 && c->table_sent_dst[stage_slot] == table_dst && c->table_sent_bytes[stage_slot] == bytes &&
+            memcmp(c->table_host[stage_slot], live.data(), bytes) == 0) {
+            // the same jobs as the last call through this slot (a decode loop): the device table is already (or, in
+            // stream order, about to be) what this launch needs
+        } else if (stage_slot >= 0) {
             // through pinned memory: no host wait, the launch that follows on the stream sees the table
+            c->table_sent_dst[stage_slot] = nullptr;
             if (c->table_host_cap[stage_slot] < bytes) {
                 if (c->table_ev[stage_slot]) HIPCHECK(c, hipEventSynchronize(c->table_ev[stage_slot]));
                 if (c->table_host[stage_slot]) HIPCHECK(c, hipHostFree(c->table_host[stage_slot]));
@@ -185,6 +192,8 @@ int prepare_same_kind(larql_hip_ctx *c, std::vector<GemvJob> &live, void *table_
             memcpy(c->table_host[stage_slot], live.data(), bytes);
             HIPCHECK(c, hipMemcpyAsync(table_dst, c->table_host[stage_slot], bytes, hipMemcpyHostToDevice, c->stream));
             HIPCHECK(c, hipEventRecord(c->table_ev[stage_slot], c->stream));
+            c->table_sent_dst[stage_slot] = table_dst;
+            c->table_sent_bytes[stage_slot] = bytes;
         } else {
             HIPCHECK(c, hipMemcpyAsync(table_dst, live.data(), bytes, hipMemcpyHostToDevice, c->stream));
             HIPCHECK(c, hipStreamSynchronize(c->stream));  // the host vector may die
@@ -237,7 +246,12 @@ int enqueue_jobs(larql_hip_ctx *c, std::vector<GemvJob> &jobs) {
     for (std::vector<GemvJob> &live : group_by_kind(jobs)) {
         const int sl = slot++ % 4;
         DevBuf &tb = c->tables[sl];
-        if (live.size() > (size_t)kInlineJobs) { rc = ensure(c, tb, live.size() * sizeof(GemvJob)); if (rc) return rc; }
+        if (live.size() > (size_t)kInlineJobs) {
+            const void *before = tb.p;
+            rc = ensure(c, tb, live.size() * sizeof(GemvJob));
+            if (rc) return rc;
+            if (tb.p != before) c->table_sent_dst[sl] = nullptr;  // a new allocation holds nothing yet
+        }
         PreparedLaunch P;
         rc = prepare_same_kind(c, live, tb.p, P, sl);
         if (rc) return rc;
