@@ -1617,14 +1617,15 @@ __device__ __forceinline__ void run_bf16_mfma(const GemvJob &j, uint32_t tile_a,
 }
 
 // ---------------------------------------------------------------------------
-// Q4_K rows against 2..4 activations at once (gate-KNN over several residual positions, rows of up to 10
+// Q4_K rows against 2..8 activations at once (gate-KNN over several residual positions, rows of up to 10
 // super-blocks): same streaming and the same int8 MFMA as the single-activation kernel, with the A rows
 // re-dealt: the MFMA of group g and position pair p carries row 8t + 4cl + l = limb l of sub-block 2g+cl of
 // position 2p + t, so one MFMA per group serves two positions and lane (j, rq) ends with the four limb sums
 // of position 2p + rq/2, nibble class cl = rq%2, for its weight row j and every group.  It therefore decodes
 // the scales and mins of its class for all four groups.
 // ---------------------------------------------------------------------------
-constexpr int kQ4kBatchPairs = 2;  // positions per job: 2 * kQ4kBatchPairs
+constexpr int kQ4kBatchPairs = 4;  // positions per job: 2 * kQ4kBatchPairs
+constexpr int kQ4kBatchR = 2;      // 16-row tiles between two folds of the row partials (16 * wavefronts partials per row)
 
 struct Q4kBatchCol {
     Q4kOp xm[4][kQ4kBatchPairs];      // A operand of (group, pair)
@@ -1690,8 +1691,39 @@ __device__ __forceinline__ void q4k_batch_setup(Q4kBatchCol &col, const float *x
     }
 }
 
+// the products of one wave-tile for the first NPA position pairs: value of (row, position) = k * sum_g sc_g * dot_g -
+// sum_g mn_g * sum_g(x); the limb sums meet pairwise as integers (exact, below 2^24) before they become floats
+template <int NPA>
+__device__ __forceinline__ void q4k_batch_tile(const uint8_t *sp, uint32_t kq, const Q4kBatchCol &col, const float (&sc)[4], const float (&mn)[4],
+                                               float (&racc)[kQ4kBatchPairs]) {
+    float rdot[NPA], rmin[NPA];
+#pragma unroll
+    for (int p = 0; p < NPA; p++) {
+        rdot[p] = 0.f;
+        rmin[p] = mn[0] * col.sum[0][p];
+#pragma unroll
+        for (int g = 1; g < 4; g++) rmin[p] = __builtin_fmaf(mn[g], col.sum[g][p], rmin[p]);
+    }
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        const u32x2 q = *reinterpret_cast<const u32x2 *>(sp + 16 + 32 * g + 8 * kq);
+        Q4kOp b;
+        b.u[0] = q.x & 0x0F0F0F0Fu; b.u[1] = q.y & 0x0F0F0F0Fu;
+        b.u[2] = (q.x >> 4) & 0x0F0F0F0Fu; b.u[3] = (q.y >> 4) & 0x0F0F0F0Fu;
+#pragma unroll
+        for (int p = 0; p < NPA; p++) {
+            const i32x4 z = {0, 0, 0, 0};
+            const i32x4 D = __builtin_amdgcn_mfma_i32_16x16x64_i8(col.xm[g][p].v, b.v, z, 0, 0, 0);
+            const float hi = (float)(D[0] * 128 + D[1]), lo = (float)(D[2] * 128 + D[3]);
+            rdot[p] = __builtin_fmaf(sc[g], __builtin_fmaf(hi, 16384.f, lo), rdot[p]);
+        }
+    }
+#pragma unroll
+    for (int p = 0; p < kQ4kBatchPairs; p++) racc[p] = p < NPA ? __builtin_fmaf(rdot[p < NPA ? p : 0], col.k[p], -rmin[p < NPA ? p : 0]) : 0.f;
+}
+
 __device__ __forceinline__ void run_q4k_batch(const GemvJob &j, uint32_t tile_a, uint32_t tile_b, uint8_t *lds, uint32_t &parity) {
-    constexpr int NS = kQ4kStages, R = kQ4kBatchTiles, NP = kQ4kBatchPairs;
+    constexpr int NS = kQ4kStages, R = kQ4kBatchR, NP = kQ4kBatchPairs;
     const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t nw_launch = blockDim.x >> 6;
     const uint32_t jr = lane & 15u, kq = lane >> 4, t_p = kq >> 1, cl = kq & 1u;
@@ -1757,25 +1789,11 @@ __device__ __forceinline__ void run_q4k_batch(const GemvJob &j, uint32_t tile_a,
                 sc[3] = d * (float)(((hi_a >> 16) & 0x0Fu) | ((sc_a >> 18) & 0x30u));                    // sub 6+cl
                 mn[3] = dmin * (float)(((hi_a >> 20) & 0x0Fu) | ((mn_a >> 18) & 0x30u));
                 float racc[NP];
-#pragma unroll
-                for (int p = 0; p < NP; p++) racc[p] = 0.f;
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const u32x2 q = *reinterpret_cast<const u32x2 *>(sp + 16 + 32 * g + 8 * kq);
-                    Q4kOp b;
-                    b.u[0] = q.x & 0x0F0F0F0Fu; b.u[1] = q.y & 0x0F0F0F0Fu;
-                    b.u[2] = (q.x >> 4) & 0x0F0F0F0Fu; b.u[3] = (q.y >> 4) & 0x0F0F0F0Fu;
-#pragma unroll
-                    for (int p = 0; p < NP; p++) {
-                        if ((uint32_t)(2 * p) < batch) {
-                            const i32x4 z = {0, 0, 0, 0};
-                            const i32x4 D = __builtin_amdgcn_mfma_i32_16x16x64_i8(col.xm[g][p].v, b.v, z, 0, 0, 0);
-                            float dot = __builtin_fmaf((float)D[0], 128.f, (float)D[1]);
-                            dot = __builtin_fmaf(dot, 128.f, (float)D[2]);
-                            dot = __builtin_fmaf(dot, 128.f, (float)D[3]) * col.k[p];
-                            racc[p] += sc[g] * dot - mn[g] * col.sum[g][p];
-                        }
-                    }
+                switch ((batch + 1) / 2) {  // (no branch inside the MFMA sequence: the products of a tile are independent)
+                    case 1: q4k_batch_tile<1>(sp, kq, col, sc, mn, racc); break;
+                    case 2: q4k_batch_tile<2>(sp, kq, col, sc, mn, racc); break;
+                    case 3: q4k_batch_tile<3>(sp, kq, col, sc, mn, racc); break;
+                    default: q4k_batch_tile<4>(sp, kq, col, sc, mn, racc); break;
                 }
 #pragma unroll
                 for (int p = 0; p < NP; p++) {
@@ -2547,7 +2565,7 @@ static int g_bf16_mfma = getenv("LARQL_HIP_BF16_MFMA") ? atoi(getenv("LARQL_HIP_
 uint32_t gemv_batch_capacity(int kind, uint64_t k) {
     // bf16: 128-element columns, at most 10 wavefronts x 2 passes, two sets of 4 positions
     if (kind == KIND_BF16 && g_bf16_mfma && k >= 128 && k % 128 == 0 && k / 128 <= (uint64_t)(kBfMaxWaves * kBfMaxPasses)) return 4 * kBfMaxSets;
-    // Q4_K: one wavefront per super-block column, two pairs of positions
+    // Q4_K: one wavefront per super-block column, four pairs of positions
     if (kind == KIND_Q4K && g_q4k_mfma && k >= 256 && k % 256 == 0 && k / 256 <= (uint64_t)kQ4kMaxWaves) return 2 * kQ4kBatchPairs;
     return 1;
 }
@@ -2785,7 +2803,7 @@ size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
     }
     if (n > 0 && jobs[0].kind == KIND_Q4K_BATCH) {
         const size_t nw = threads / 64;
-        return nw * kQ4kStages * kQ4kTileBytes + 2 * (size_t)kQ4kBatchTiles * 16 * (2 * kQ4kBatchPairs * nw * 2) * sizeof(float);
+        return nw * kQ4kStages * kQ4kTileBytes + 2 * (size_t)kQ4kBatchR * 16 * (2 * kQ4kBatchPairs * nw * 2) * sizeof(float);
     }
     if (n > 0 && jobs[0].kind == KIND_BF16_MFMA) {
         const size_t nw = threads / 64;

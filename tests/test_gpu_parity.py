@@ -530,9 +530,9 @@ def test_bf16_gate_scores_over_several_positions(be, fmt, n, hidden, batch):
 
 
 @pytest.mark.parametrize("n,hidden,batch", [(1000, 256, 2), (77, 768, 3), (4099, 2560, 4), (640, 1280, 9), (33, 2560, 6),
-                                            (500, 2816, 4)])
+                                            (500, 2816, 4), (2051, 2560, 8), (130, 512, 7), (300, 2304, 17), (64, 256, 5)])
 def test_q4k_gate_scores_over_several_positions(be, fmt, n, hidden, batch):
-    # up to 4 positions share one pass over a Q4_K gate (rows of up to 10 super-blocks; longer rows go one by one)
+    # up to 8 positions share one pass over a Q4_K gate (rows of up to 10 super-blocks; longer rows go one by one)
     rng = np.random.default_rng(n + hidden + batch)
     gate = O.quantize_q4_k((rng.standard_normal((n, hidden)) * 0.05).astype(F))
     X = rng.standard_normal((batch, hidden)).astype(F)
