@@ -304,9 +304,8 @@ def run_c4(be, fmt, args):
         wsb = be.moe_mxfp4_workspace_bytes(T, k, H, I)
         ws = be.malloc(wsb)
 
-        def block():
-            be.dev_router_select(lg, T, E, k, 1, de, dw)
-            be.dev_moe_mxfp4(bank, x, T, k, de, dw, out, ws, wsb)
+        def block():  # Router::select + the expert block (one token: the selection runs inside the first matvec launch)
+            be.dev_moe_mxfp4_routed(bank, x, T, k, lg, 1, de, dw, out, ws, wsb)
         block(); be.synchronize()
         experts = be.d2h(de, (T, k), np.uint32)
         distinct = len(set(int(v) for v in experts.reshape(-1)))
@@ -333,7 +332,7 @@ def run_c4(be, fmt, args):
         med, nrep = _cpu_time(lambda: O.mxfp4_gemv(*mats["gate"], xv[0], I, H), args.cpu_seconds / 4)
         _emit(f"MXFP4 MoE expert block us (32 experts, top-4, batch {T}, gate/up {layout})", round(ms * 1e3, 2), "us/block", ms, args.steps, 2,
               {"workload": f"BASELINE configs[3]: MXFP4 experts 32 x (gate, up, down 2880x2880), top-4, batch {T}",
-               "gate_up_layout": layout, "distinct_experts": distinct, "launches_per_block": 5 if T > 1 else 4, "GBps_over_distinct_expert_bytes": round(algo / ms / 1e6, 1),
+               "gate_up_layout": layout, "distinct_experts": distinct, "launches_per_block": 5 if T > 1 else 3, "GBps_over_distinct_expert_bytes": round(algo / ms / 1e6, 1),
                "us_per_expert_matvec": round(ms * 1e3 / (3 * T * k), 2), "verified_rel_l2_vs_oracle": rel},
               {"kernel": "gemv_mxfp4 (gate/up + down launches)", "bound": "hbm", "achieved": round(algo / ms / 1e6, 1), "peak": HBM_PEAK_GBS,
                "unit": "GB/s", "frac": round(algo / ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": None},

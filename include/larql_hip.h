@@ -349,6 +349,13 @@ typedef struct {
 size_t larql_hip_moe_mxfp4_workspace_bytes(size_t tokens, size_t k, size_t hidden, size_t inter);
 int larql_hip_dev_moe_mxfp4(larql_hip_ctx *ctx, const larql_hip_mxfp4_experts *bank, const float *x, size_t tokens, size_t k,
                             const uint32_t *experts, const float *weights, float *out, void *workspace, size_t workspace_bytes);
+/* Router::select (ffn/expert_weight/router.rs:33-70) and the expert block above as one call: the same results as
+ * larql_hip_dev_router_select followed by larql_hip_dev_moe_mxfp4, experts / weights [tokens, min(k, n_experts)]
+ * written as the former writes them.  For one token the selection runs inside the first matvec launch (one launch
+ * fewer: a decode step's expert block is bound by its launches, not by its bytes).  Limits as the two calls. */
+int larql_hip_dev_moe_mxfp4_routed(larql_hip_ctx *ctx, const larql_hip_mxfp4_experts *bank, const float *x, size_t tokens, size_t k,
+                                   const float *router_logits, int policy, uint32_t *experts, float *weights, float *out,
+                                   void *workspace, size_t workspace_bytes);
 
 /* ---- device tier: encoders (bit-exact with the reference's host encoders) --- */
 /* quantize_q4_k — larql-compute/src/cpu/ops/q4_common/quantize.rs:89-189. */

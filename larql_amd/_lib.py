@@ -97,6 +97,7 @@ SIGNATURES = {
     "larql_hip_dev_router_select": (ci, [vp, vp, sz, sz, sz, ci, vp, vp]),
     "larql_hip_moe_mxfp4_workspace_bytes": (sz, [sz, sz, sz, sz]),
     "larql_hip_dev_moe_mxfp4": (ci, [vp, C.POINTER(Mxfp4Experts), vp, sz, sz, vp, vp, vp, vp, sz]),
+    "larql_hip_dev_moe_mxfp4_routed": (ci, [vp, C.POINTER(Mxfp4Experts), vp, sz, sz, vp, ci, vp, vp, vp, vp, sz]),
     "larql_hip_dev_quantize_q4_k": (ci, [vp, vp, sz, vp]),
     "larql_hip_dev_quantize_q8_0": (ci, [vp, vp, sz, vp]),
     "larql_hip_dev_quantize_mxfp4": (ci, [vp, vp, sz, sz, vp, vp]),

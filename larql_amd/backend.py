@@ -411,6 +411,13 @@ class HipBackend:
         return self._some(lib.larql_hip_dev_moe_mxfp4(self._h, C.byref(bank), x, tokens, k, experts, weights, out, workspace,
                                                       workspace_bytes))
 
+    def dev_moe_mxfp4_routed(self, bank: "L.Mxfp4Experts", x: int, tokens: int, k: int, logits: int, policy: int, experts: int,
+                             weights: int, out: int, workspace: int, workspace_bytes: int) -> bool:
+        """Router::select and the expert block in one call (one launch fewer for a single token); experts / weights are
+        written as dev_router_select writes them."""
+        return self._some(lib.larql_hip_dev_moe_mxfp4_routed(self._h, C.byref(bank), x, tokens, k, logits, policy, experts, weights,
+                                                             out, workspace, workspace_bytes))
+
     def dev_quantize_q4_k(self, src: int, n: int, dst: int) -> bool:
         return self._some(lib.larql_hip_dev_quantize_q4_k(self._h, src, n, dst))
 

@@ -1218,10 +1218,11 @@ size_t larql_hip_moe_mxfp4_workspace_bytes(size_t tokens, size_t k, size_t hidde
     return (slots * inter * 3 + slots * hidden) * sizeof(float) + 256;
 }
 
-int larql_hip_dev_moe_mxfp4(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank, const float *x, size_t tokens, size_t k,
-                            const uint32_t *experts, const float *weights, float *out, void *workspace, size_t workspace_bytes) {
-    if (!c || !bank) return LARQL_E_ARG;
-    std::lock_guard<std::mutex> lk(c->mu);
+// The expert block; with `route_logits` the selection is part of it (written to experts / weights as
+// larql_hip_dev_router_select would): inside the first matvec launch for one token, by the selection kernel otherwise.
+static int moe_mxfp4_block(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank, const float *x, size_t tokens, size_t k,
+                           uint32_t *experts, float *weights, float *out, void *workspace, size_t workspace_bytes,
+                           const float *route_logits, int route_policy) {
     const size_t hidden = bank->hidden, inter = bank->inter;
     if (hidden % 32 != 0 || inter % 32 != 0) return fail(c, LARQL_REFUSED_SHAPE, "moe_mxfp4: hidden and inter must be multiples of 32");
     if (tokens == 0 || k == 0) return LARQL_OK;
@@ -1243,6 +1244,13 @@ int larql_hip_dev_moe_mxfp4(larql_hip_ctx *c, const larql_hip_mxfp4_experts *ban
     const size_t gu_rows = fused ? 2 * inter : inter;
     const uint64_t gu_w_stride = gu_rows * (hidden / 32) * 16, gu_s_stride = gu_rows * (hidden / 32);
     const uint64_t dn_w_stride = hidden * (inter / 32) * 16, dn_s_stride = hidden * (inter / 32);
+    // one token: the gate/up launch can select for itself (every wavefront repeats the token's selection, the
+    // workgroup that opens the first job writes it out for the launches that follow)
+    const bool route_in_launch = route_logits && tokens == 1 &&
+        gemv_effective_kind(make_job(KIND_MXFP4, bank->gate_packed, bank->gate_scales, x, g, gu_rows, hidden)) == KIND_MXFP4_MFMA;
+    if (route_logits && !route_in_launch)
+        HIPCHECK(c, router_select_launch(c->stream, route_logits, (uint32_t)tokens, (uint32_t)bank->n_experts, (uint32_t)k, route_policy,
+                                         experts, weights));
     // Several tokens: slots that chose the same expert share its weights up to four at a time.  The job lists are built on
     // the device from the router's choice (moe_plan_kernel) into the workspace's spare activation area.
     {
@@ -1299,10 +1307,16 @@ int larql_hip_dev_moe_mxfp4(larql_hip_ctx *c, const larql_hip_mxfp4_experts *ban
         const size_t t = s / k;
         GemvJob a = make_job(KIND_MXFP4, bank->gate_packed, bank->gate_scales, x + t * hidden, g + s * gu_rows, gu_rows, hidden);
         a.sel = experts + s; a.w_sel_stride = gu_w_stride; a.aux_sel_stride = gu_s_stride;
+        if (route_in_launch) {
+            a.sel = nullptr;
+            a.route_logits = route_logits; a.route_n = (uint32_t)bank->n_experts; a.route_k = (uint32_t)k; a.route_rank = (uint32_t)s;
+            a.route_policy = route_policy;
+        }
+        GemvJob b = a;
+        if (route_in_launch && s == 0) { a.route_experts = experts; a.route_weights = weights; }
         jobs.push_back(a);
         if (fused) continue;
-        GemvJob b = make_job(KIND_MXFP4, bank->up_packed, bank->up_scales, x + t * hidden, u + s * inter, inter, hidden);
-        b.sel = experts + s; b.w_sel_stride = gu_w_stride; b.aux_sel_stride = gu_s_stride;
+        b.w = (const uint8_t *)bank->up_packed; b.aux = (const uint8_t *)bank->up_scales; b.out = u + s * inter; b.rows = inter;
         jobs.push_back(b);
     }
     int rc = enqueue_jobs(c, jobs);
@@ -1326,6 +1340,26 @@ int larql_hip_dev_moe_mxfp4(larql_hip_ctx *c, const larql_hip_mxfp4_experts *ban
     if (rc) return rc;
     HIPCHECK(c, weighted_sum_launch(c->stream, d, weights, out, (uint32_t)tokens, (uint32_t)k, (uint32_t)hidden));
     return LARQL_OK;
+}
+
+int larql_hip_dev_moe_mxfp4(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank, const float *x, size_t tokens, size_t k,
+                            const uint32_t *experts, const float *weights, float *out, void *workspace, size_t workspace_bytes) {
+    if (!c || !bank) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    return moe_mxfp4_block(c, bank, x, tokens, k, const_cast<uint32_t *>(experts), const_cast<float *>(weights), out, workspace,
+                           workspace_bytes, nullptr, 0);  // (without logits nothing is written to experts / weights)
+}
+
+int larql_hip_dev_moe_mxfp4_routed(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank, const float *x, size_t tokens, size_t k,
+                                   const float *router_logits, int policy, uint32_t *experts, float *weights, float *out,
+                                   void *workspace, size_t workspace_bytes) {
+    if (!c || !bank) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (k > bank->n_experts) k = bank->n_experts;  // select(): k.min(logits.len())
+    if (tokens == 0 || k == 0) return LARQL_OK;
+    if (bank->n_experts > 64 || k > 8) return fail(c, LARQL_UNSUPPORTED, "router_select: at most 64 experts and top-8 on this backend");
+    if (!router_logits) return LARQL_E_ARG;
+    return moe_mxfp4_block(c, bank, x, tokens, k, experts, weights, out, workspace, workspace_bytes, router_logits, policy);
 }
 
 // Gate-KNN over several layers in one submission (the LQL WALK / DESCRIBE shape: every layer of

@@ -25,6 +25,7 @@
 #include <algorithm>
 
 #include "kernels.h"
+#include "router.h"
 
 namespace larql {
 
@@ -2413,7 +2414,24 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) gemv_mxfp4_mfma_kernel(Gemv
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
         GemvJob j = uniform_job(jobs + ji);
-        if (j.sel) {  // run-time expert selection: one bank of equally shaped matrices
+        if (j.route_logits) {  // the selection itself, by every wavefront for itself (a load and ~200 instructions)
+            uint32_t idx[kRouterMaxK];
+            float wt[kRouterMaxK];
+            const bool writer = j.route_experts && p == j.pass_begin && threadIdx.x < 64;  // (one workgroup opens the job)
+            if (writer) router_select_wave<true>(j.route_logits, j.route_n, j.route_k, j.route_policy, threadIdx.x & 63u, idx, wt);
+            else router_select_wave<false>(j.route_logits, j.route_n, j.route_k, j.route_policy, threadIdx.x & 63u, idx, wt);
+            uint32_t e = idx[0];
+#pragma unroll
+            for (int r = 1; r < kRouterMaxK; r++) e = j.route_rank == (uint32_t)r ? idx[r] : e;
+            e = __builtin_amdgcn_readfirstlane(e);
+            j.w += (size_t)e * j.w_sel_stride;
+            j.aux += (size_t)e * j.aux_sel_stride;
+            if (writer && threadIdx.x == 0) {
+#pragma unroll
+                for (int r = 0; r < kRouterMaxK; r++)
+                    if ((uint32_t)r < j.route_k) { j.route_experts[r] = idx[r]; j.route_weights[r] = wt[r]; }
+            }
+        } else if (j.sel) {  // run-time expert selection: one bank of equally shaped matrices
             const uint32_t e = __builtin_amdgcn_readfirstlane(*(const GLOBAL_AS uint32_t *)j.sel);
             j.w += (size_t)e * j.w_sel_stride;
             j.aux += (size_t)e * j.aux_sel_stride;

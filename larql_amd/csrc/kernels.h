@@ -56,8 +56,17 @@ struct GemvJob {
     // Optional cost model of the job in the launch's pass list (MXFP4 matrix-core kernel): the job's n_pass is
     // su + tiles * cpt (a start-up allowance, then cpt units per 16-row tile); cpt == 0 means cpr units per tile, no allowance.
     uint32_t cpt, su;
-    uint64_t pad3;        // (the descriptor is a whole number of 16-byte words)
+    // Optional selection inside the kernel (MXFP4 matrix-core kernel, one token): when `route_logits` is set the job
+    // takes the expert of rank `route_rank` of Router::select over those logits (route_n experts <= 64, route_k <= 8,
+    // policy as router_select_launch) where it would read *sel, and the workgroup that opens the job also writes the
+    // token's selection to route_experts / route_weights if they are set.
+    const float *route_logits;
+    uint32_t *route_experts;
+    float *route_weights;
+    uint32_t route_n, route_k, route_rank;
+    int32_t route_policy;
 };
+static_assert(sizeof(GemvJob) % 16 == 0, "the descriptor is a whole number of 16-byte words (moe_plan_kernel stores it that way)");
 
 struct GemvLaunch {
     const GemvJob *table;  // device table, or null to use `inl`

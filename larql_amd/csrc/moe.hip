@@ -4,84 +4,26 @@
 #include <stdint.h>
 
 #include "kernels.h"
+#include "router.h"
 
 namespace larql {
 
-// ---------------------------------------------------------------------------
-// router::select — larql-compute/src/ffn/expert_weight/router.rs:33-70.
-// One wavefront per token, lane i holds logit i (n_experts <= 64).  Rank by
-// logit descending, first index wins ties (the reference's stable sort);
-// weights are exp(l - max_all) / denominator, the denominator summed in f32
-// over the selected logits in rank order (policy 1, NormalisedOverSelected) or
-// over all experts in index order (policy 0, SoftmaxThenSelect).
-// ---------------------------------------------------------------------------
-// Reductions over the wavefront by data-parallel primitives (four steps inside the rows of 16 lanes, two row
-// broadcasts, then lane 63 holds the result): a few cycles per step, where a cross-lane shuffle costs an LDS round trip.
-template <int CTRL, int ROW_MASK, bool BOUND>
-__device__ __forceinline__ uint64_t dpp_max_u64(uint64_t v) {  // lanes without a source read 0: the identity here
-    const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)v, CTRL, ROW_MASK, 0xF, BOUND);
-    const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(v >> 32), CTRL, ROW_MASK, 0xF, BOUND);
-    const uint64_t other = ((uint64_t)hi << 32) | lo;
-    return other > v ? other : v;
-}
-__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
-    v = dpp_max_u64<0xB1, 0xF, true>(v);    // quad_perm [1,0,3,2]
-    v = dpp_max_u64<0x4E, 0xF, true>(v);    // quad_perm [2,3,0,1]
-    v = dpp_max_u64<0x141, 0xF, true>(v);   // row_half_mirror
-    v = dpp_max_u64<0x140, 0xF, true>(v);   // row_mirror
-    v = dpp_max_u64<0x142, 0xA, false>(v);  // row_bcast:15 into rows 1 and 3
-    v = dpp_max_u64<0x143, 0xC, false>(v);  // row_bcast:31 into rows 2 and 3
-    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, 63), hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), 63);
-    return ((uint64_t)hi << 32) | lo;
-}
-template <int CTRL, int ROW_MASK, bool BOUND>
-__device__ __forceinline__ float dpp_fmax(float v) {  // lanes without a source read -inf
-    return fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp((int)0xFF800000u, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, BOUND)));
-}
-__device__ __forceinline__ float wave_fmax(float v) {
-    v = dpp_fmax<0xB1, 0xF, false>(v);
-    v = dpp_fmax<0x4E, 0xF, false>(v);
-    v = dpp_fmax<0x141, 0xF, false>(v);
-    v = dpp_fmax<0x140, 0xF, false>(v);
-    v = dpp_fmax<0x142, 0xA, false>(v);
-    v = dpp_fmax<0x143, 0xC, false>(v);
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
-}
-__device__ __forceinline__ float lane_value(float v, uint32_t lane_uniform) {  // the lane index must be the same in every lane
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), (int)lane_uniform));
-}
-
+// router::select for every token: one wavefront per token (router.h).
 __global__ void __launch_bounds__(64) router_select_kernel(const float *__restrict__ logits, uint32_t n_experts, uint32_t k,
                                                            int policy, uint32_t *__restrict__ experts,
                                                            float *__restrict__ weights) {
     const uint32_t t = blockIdx.x, lane = threadIdx.x;
-    const bool has = lane < n_experts;
-    const float l = has ? logits[(size_t)t * n_experts + lane] : 0.0f;
-    // orderable key: logit bits made monotone, then ~index so the lower index wins a tie; 0 = absent
-    const uint32_t bits = __builtin_bit_cast(uint32_t, l);
-    const uint32_t ord = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
-    uint64_t key = has ? (((uint64_t)ord << 32) | (uint32_t)(~lane)) : 0;
-    const float dmax = wave_fmax(has ? l : -__builtin_inff());
-    const float ex = has ? expf(l - dmax) : 0.0f;
-    float denom = 0.0f;
-    if (policy == 0)
-        for (uint32_t i = 0; i < n_experts; i++) denom += lane_value(ex, i);  // index order, as the iterator sums
-    uint32_t sel_idx[8];
-    float sel_ex[8];
-    for (uint32_t r = 0; r < k; r++) {
-        const uint64_t best = wave_max_u64(key);
-        const uint32_t idx = ~(uint32_t)best & 63u;  // (k <= n_experts: a key is always left; the mask keeps the lane index in range regardless)
-        sel_idx[r] = idx;
-        sel_ex[r] = lane_value(ex, idx);
-        if (lane == idx) key = 0;
+    uint32_t sel_idx[kRouterMaxK];
+    float sel_w[kRouterMaxK];
+    router_select_wave(logits + (size_t)t * n_experts, n_experts, k, policy, lane, sel_idx, sel_w);
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < kRouterMaxK; r++)
+            if ((uint32_t)r < k) {
+                experts[(size_t)t * k + r] = sel_idx[r];
+                weights[(size_t)t * k + r] = sel_w[r];
+            }
     }
-    if (policy != 0)
-        for (uint32_t r = 0; r < k; r++) denom += sel_ex[r];  // rank order
-    if (lane == 0)
-        for (uint32_t r = 0; r < k; r++) {
-            experts[(size_t)t * k + r] = sel_idx[r];
-            weights[(size_t)t * k + r] = denom > 0.0f ? sel_ex[r] / denom : 0.0f;
-        }
 }
 
 // MoeGateRule::ClampedGlu — larql-compute/src/pipeline/moe.rs:88-92:

@@ -867,6 +867,49 @@ def test_moe_mxfp4_tokens_sharing_an_expert_equal_single_token_calls(be, fmt):
     assert rel_l2(got[5], acc) < 1e-5
 
 
+@pytest.mark.parametrize("T,E,hidden,inter,interleaved,policy", [(1, 8, 2880, 2880, 0, 1), (1, 8, 2880, 2880, 1, 1), (1, 6, 384, 320, 0, 0),
+                                                                 (1, 64, 384, 320, 1, 1), (5, 6, 384, 320, 0, 1), (1, 3, 96, 64, 0, 1)])
+def test_moe_mxfp4_routed_equals_select_then_block(be, fmt, T, E, hidden, inter, interleaved, policy):
+    """Selection and expert block as one call: experts, weights and output bit for bit those of the two calls (one
+    token: the selection runs inside the first matvec launch; k = 96 rows are below what that kernel takes and
+    several tokens go through the selection kernel)."""
+    rng = np.random.default_rng(500 + E + T)
+    k = min(4, E)
+    g_rows = 2 * inter if interleaved else inter
+    gp, gs = O.quantize_mxfp4((rng.standard_normal(E * g_rows * hidden) * 0.03).astype(F), E * g_rows, hidden)
+    dp, ds = O.quantize_mxfp4((rng.standard_normal(E * hidden * inter) * 0.03).astype(F), E * hidden, inter)
+    dev = {n: be.to_device(a) for n, a in dict(gp=gp, gs=gs, dp=dp, ds=ds).items()}
+    if interleaved:
+        b = fmt.Mxfp4Experts(dev["gp"], dev["gs"], None, None, dev["dp"], dev["ds"], E, hidden, inter, 7.0, 1.702, 1)
+    else:
+        up, us = O.quantize_mxfp4((rng.standard_normal(E * inter * hidden) * 0.03).astype(F), E * inter, hidden)
+        dev["up"], dev["us"] = be.to_device(up), be.to_device(us)
+        b = fmt.Mxfp4Experts(dev["gp"], dev["gs"], dev["up"], dev["us"], dev["dp"], dev["ds"], E, hidden, inter, 7.0, 1.702, 0)
+    x = be.to_device(rng.standard_normal((T, hidden)).astype(F))
+    lg = rng.standard_normal((T, E)).astype(F)
+    lg[0, 1] = lg[0, 2]                                   # a tie: the lower index first
+    dl = be.to_device(lg)
+    wsb = be.moe_mxfp4_workspace_bytes(T, k, hidden, inter)
+    ws = be.malloc(wsb)
+    e1, w1, o1 = be.malloc(T * k * 4), be.malloc(T * k * 4), be.malloc(T * hidden * 4)
+    e2, w2, o2 = be.malloc(T * k * 4), be.malloc(T * k * 4), be.malloc(T * hidden * 4)
+    assert be.dev_router_select(dl, T, E, k, policy, e1, w1)
+    assert be.dev_moe_mxfp4(b, x, T, k, e1, w1, o1, ws, wsb)
+    be.synchronize()
+    want = (be.d2h(e1, (T, k), np.uint32), be.d2h(w1, (T, k), F), be.d2h(o1, (T, hidden), F))
+    for rep in range(2):                                   # (the second call finds its job tables already on the device)
+        assert be.dev_moe_mxfp4_routed(b, x, T, k, dl, policy, e2, w2, o2, ws, wsb)
+        be.synchronize()
+        got = (be.d2h(e2, (T, k), np.uint32), be.d2h(w2, (T, k), F), be.d2h(o2, (T, hidden), F))
+        assert np.array_equal(got[0], want[0])
+        assert np.array_equal(got[1].view(np.uint32), want[1].view(np.uint32))
+        assert np.array_equal(got[2].view(np.uint32), want[2].view(np.uint32))
+    assert [int(v) for v in want[0][0]] == [i for i, _ in O.router_select(lg[0], k, policy)]
+    import larql_amd
+    with pytest.raises(larql_amd.DeviceError):                                        # no logits: an argument error
+        be.dev_moe_mxfp4_routed(b, x, T, k, 0, policy, e2, w2, o2, ws, wsb)
+
+
 def test_moe_mxfp4_job_groups_of_every_size(be, fmt):
     """Experts chosen by 1, 2, 3, 4 and 5 slots: jobs of one, two, three and four tokens and a second job for the
     fifth.  Every token's result equals its one-token call bit for bit."""
