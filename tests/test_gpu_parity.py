@@ -868,7 +868,8 @@ def test_moe_mxfp4_tokens_sharing_an_expert_equal_single_token_calls(be, fmt):
 
 
 @pytest.mark.parametrize("T,E,hidden,inter,interleaved,policy", [(1, 8, 2880, 2880, 0, 1), (1, 8, 2880, 2880, 1, 1), (1, 6, 384, 320, 0, 0),
-                                                                 (1, 64, 384, 320, 1, 1), (5, 6, 384, 320, 0, 1), (1, 3, 96, 64, 0, 1)])
+                                                                 (1, 64, 384, 320, 1, 1), (5, 6, 384, 320, 0, 1), (1, 3, 96, 64, 0, 1), (16, 32, 384, 320, 1, 1),
+                                                                 (32, 9, 384, 320, 0, 0), (40, 12, 384, 320, 0, 1)])
 def test_moe_mxfp4_routed_equals_select_then_block(be, fmt, T, E, hidden, inter, interleaved, policy):
     """Selection and expert block as one call: experts, weights and output bit for bit those of the two calls (one
     token: the selection runs inside the first matvec launch; k = 96 rows are below what that kernel takes and
