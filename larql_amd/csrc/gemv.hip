@@ -832,7 +832,7 @@ __device__ __forceinline__ void run_q4k_mfma(const GemvJob &j, uint32_t tile_a, 
 // larql-compute/src/cpu/ops/q6k_matvec.rs:45-91: per 16-element group sub = sum (q - 32) * x; acc += (d * sc) * sub).
 //
 // A wave-tile is 16 rows x one super-block, copied global -> LDS as 13 sixteen-byte pieces per row (ql, qh, scales)
-// plus a two-byte piece for d.  The blocks are only 2-byte aligned in memory: the copies take any alignment (at
+// plus the block's last 16 bytes again for d.  The blocks are only 2-byte aligned in memory: the copies take any alignment (at
 // ~12 % of the bandwidth that aligned ones reach) and land on a 208-byte pitch, so that every LDS read is an aligned
 // ds_read_b128.  (Copying the 14 aligned pieces that contain a block instead moves the misalignment to the LDS side,
 // where it costs more: a misaligned ds_read_b128 is correct but slow, five aligned dwords and a byte rotation per
@@ -851,7 +851,7 @@ constexpr int kQ6kBatchTiles = 2;
 constexpr int kQ6kMaxColPasses = 4;
 constexpr int kQ6kMaxWaves = 10;
 constexpr uint32_t kQ6kPitch = 208;                          // ql 128, qh 64, scales 16
-constexpr uint32_t kQ6kTileBytes = 16 * kQ6kPitch + 64;      // + a dword slot per row for d
+constexpr uint32_t kQ6kTileBytes = 16 * kQ6kPitch + 256;     // + a 16-byte slot per row whose last two bytes are d
 constexpr uint32_t kQ6kColBytes = 1024 + 64 + 16;            // four limb planes of 256 bytes, 16 group sums, k
 
 struct Q6kCol {
@@ -913,7 +913,7 @@ __device__ __forceinline__ float q6k_mfma_tile(const uint8_t *slot, const Q6kCol
         qh[h] = *reinterpret_cast<const u32x4 *>(sp + 128 + 32 * h + 16 * (kq & 1u));
     }
     const u32x4 scs = *reinterpret_cast<const u32x4 *>(sp + 192);
-    const float d = half_bits_to_float(*reinterpret_cast<const uint32_t *>(slot + 16 * kQ6kPitch + 4 * j) & 0xFFFFu);
+    const float d = half_bits_to_float(*reinterpret_cast<const uint32_t *>(slot + 16 * kQ6kPitch + 16 * j + 12) >> 16);
     // top bits: MFMA 2h wants bits s0, s0+1 of the qh bytes in bits 4-5 (a left shift by 4 - s0), MFMA 2h+1 bits
     // s0+4, s0+5 (a right shift by s0); what crosses a byte boundary falls outside the mask
     const uint32_t s0 = 2u * (kq >> 1), sl = 4u - s0;
@@ -953,16 +953,17 @@ __device__ __forceinline__ void run_q6k_mfma(const GemvJob &j, uint32_t tile_a, 
     uint8_t *cols = lds + nw_launch * (NS * kQ6kTileBytes) + 2 * R * 16 * nw_launch * 4 * sizeof(float) + wv * (cols_pitch * kQ6kColBytes);
     const uint32_t np = wv < nwj ? (cpr - wv + nwj - 1) / nwj : 0;  // columns wv, wv+nwj, ... of this wavefront
 
-    // lane's pieces of a wave-tile: 16-byte piece u = 13 * row + piece (u < 208), and d of row `lane` (lane < 16)
+    // lane's pieces of a wave-tile: 16-byte piece u = 13 * row + piece (u < 208); lanes 16..31 of the fourth copy bring
+    // the last 16 bytes of the block of row lane - 16 (bytes 194..209: d is the end of it)
     uint32_t pr[4], po[4], o[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const uint32_t u = min(64u * i + lane, 207u);
         pr[i] = u / 13;
         po[i] = (u - pr[i] * 13) * 16;
+        if (i == 3 && lane >= 16) { pr[i] = lane & 15u; po[i] = 194; }
         o[i] = pr[i] * row_bytes + po[i];
     }
-    const uint32_t od = (lane & 15u) * row_bytes + 208;
     const uint8_t *wcol = j.w + (size_t)wv * 210;
     const uint32_t nt = tile_b - tile_a;
 
@@ -975,19 +976,15 @@ __device__ __forceinline__ void run_q6k_mfma(const GemvJob &j, uint32_t tile_a, 
         const uint8_t *gp = wcol + (size_t)it_p * nwj * 210 + (size_t)rb * row_bytes;
         uint8_t *lp = ring + (n_issue % NS) * kQ6kTileBytes;
         // wave-uniform 64-bit base + per-lane 32-bit offset; only a ragged last tile recomputes the offsets
-        uint32_t a0 = o[0], a1 = o[1], a2 = o[2], a3 = o[3], ad = od;
+        uint32_t a0 = o[0], a1 = o[1], a2 = o[2], a3 = o[3];
         if (rb + 16 > rows) {
             a0 = min(pr[0], lim) * row_bytes + po[0]; a1 = min(pr[1], lim) * row_bytes + po[1];
             a2 = min(pr[2], lim) * row_bytes + po[2]; a3 = min(pr[3], lim) * row_bytes + po[3];
-            ad = min(lane & 15u, lim) * row_bytes + 208;
         }
         __builtin_amdgcn_global_load_lds((g_vp)(gp + a0), (lds_vp)lp, 16, 0, 0);
         __builtin_amdgcn_global_load_lds((g_vp)(gp + a1), (lds_vp)(lp + 1024), 16, 0, 0);
         __builtin_amdgcn_global_load_lds((g_vp)(gp + a2), (lds_vp)(lp + 2048), 16, 0, 0);
-        if (lane < 16) {
-            __builtin_amdgcn_global_load_lds((g_vp)(gp + a3), (lds_vp)(lp + 3072), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((g_vp)(gp + ad), (lds_vp)(lp + 16 * kQ6kPitch), 2, 0, 0);
-        }
+        if (lane < 32) __builtin_amdgcn_global_load_lds((g_vp)(gp + a3), (lds_vp)(lp + 3072), 16, 0, 0);
         n_issue++;
         if (it_tb < nt) {
             const uint32_t nb = min((uint32_t)R, nt - it_tb);
@@ -1026,7 +1023,7 @@ __device__ __forceinline__ void run_q6k_mfma(const GemvJob &j, uint32_t tile_a, 
                 for (int tl = 0; tl < R; tl++) {
                     if ((uint32_t)tl < nb) {
                         issue();
-                        LARQL_WAIT_VMCNT(5 * (NS - 1));  // at most NS-1 younger wave-tiles still in flight: the oldest has landed
+                        LARQL_WAIT_VMCNT(4 * (NS - 1));  // at most NS-1 younger wave-tiles still in flight: the oldest has landed
                         asm volatile("" ::: "memory");
                         racc[tl] += q6k_mfma_tile(ring + (n_use % NS) * kQ6kTileBytes, col, jr, kq);
                         n_use++;
