@@ -844,10 +844,11 @@ __device__ __forceinline__ void run_q4k_mfma(const GemvJob &j, uint32_t tile_a, 
 // group's k-slots, zero elsewhere.  After the MFMA lane (j, rq) holds the four exact limb sums of group 4m + rq of
 // row j — the group whose int8 scale it applies.  The -32 goes through the group's sum of x.  Four MFMAs per tile,
 // none accumulates into another.  The activations of a column (256 elements) are turned into limbs by all 64 lanes,
-// four elements each, and go through LDS (limb planes) into the operand layout; they stay there for the job.
+// four elements each, and go through LDS (limb planes) into the operand layout; the operands of all the wavefront's
+// columns (up to 4) stay in registers and tiles are walked column-innermost.
 // ---------------------------------------------------------------------------
 constexpr int kQ6kStages = 3;
-constexpr int kQ6kBatchTiles = 2;
+constexpr int kQ6kBatchTiles = 4;
 constexpr int kQ6kMaxColPasses = 4;
 constexpr int kQ6kMaxWaves = 10;
 constexpr uint32_t kQ6kPitch = 208;                          // ql 128, qh 64, scales 16
@@ -938,10 +939,9 @@ __device__ __forceinline__ float q6k_mfma_tile(const uint8_t *slot, const Q6kCol
     return d * acc;
 }
 
-// tiles [tile_a, tile_b) of one job; `parity` flips per batch (double-buffered partials); `cols_pitch` = columns per
-// wavefront the launch keeps room for
-__device__ __forceinline__ void run_q6k_mfma(const GemvJob &j, uint32_t tile_a, uint32_t tile_b, uint8_t *lds, uint32_t cols_pitch,
-                                             uint32_t &parity) {
+// tiles [tile_a, tile_b) of one job, columns innermost (the workgroup reads whole rows); `parity` flips per batch
+// (double-buffered partials)
+__device__ __forceinline__ void run_q6k_mfma(const GemvJob &j, uint32_t tile_a, uint32_t tile_b, uint8_t *lds, uint32_t &parity) {
     constexpr int NS = kQ6kStages, R = kQ6kBatchTiles;
     const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t nw_launch = blockDim.x >> 6;
@@ -950,7 +950,6 @@ __device__ __forceinline__ void run_q6k_mfma(const GemvJob &j, uint32_t tile_a, 
     const uint32_t rows = (uint32_t)j.rows, row_bytes = (uint32_t)j.row_bytes;
     uint8_t *ring = lds + wv * (NS * kQ6kTileBytes);
     float *part = reinterpret_cast<float *>(lds + nw_launch * (NS * kQ6kTileBytes));
-    uint8_t *cols = lds + nw_launch * (NS * kQ6kTileBytes) + 2 * R * 16 * nw_launch * 4 * sizeof(float) + wv * (cols_pitch * kQ6kColBytes);
     const uint32_t np = wv < nwj ? (cpr - wv + nwj - 1) / nwj : 0;  // columns wv, wv+nwj, ... of this wavefront
 
     // lane's pieces of a wave-tile: 16-byte piece u = 13 * row + piece (u < 208); lanes 16..31 of the fourth copy bring
@@ -986,13 +985,7 @@ __device__ __forceinline__ void run_q6k_mfma(const GemvJob &j, uint32_t tile_a, 
         __builtin_amdgcn_global_load_lds((g_vp)(gp + a2), (lds_vp)(lp + 2048), 16, 0, 0);
         if (lane < 32) __builtin_amdgcn_global_load_lds((g_vp)(gp + a3), (lds_vp)(lp + 3072), 16, 0, 0);
         n_issue++;
-        if (it_tb < nt) {
-            const uint32_t nb = min((uint32_t)R, nt - it_tb);
-            if (++it_tl == nb) {
-                it_tl = 0;
-                if (++it_p == np) { it_p = 0; it_tb += R; }
-            }
-        }
+        if (it_tb + it_tl < nt && ++it_p == np) { it_p = 0; it_tl++; }  // (it_tb stays 0: tiles in order, columns innermost)
     };
     // the activations of all this wavefront's columns are requested first and together, then prepared while the tiles fly
     f32x4 raw[kQ6kMaxColPasses];
@@ -1001,12 +994,19 @@ __device__ __forceinline__ void run_q6k_mfma(const GemvJob &j, uint32_t tile_a, 
         if ((uint32_t)p < np) raw[p] = ((g_f4p)(j.x + (size_t)(wv + nwj * p) * 256))[lane];
     if (np >= 1)
         for (int s = 0; s < NS - 1; s++) issue();
+    // every column's operands stay in registers for the job; a column passes through the ring's last slot, still
+    // free at this point, on its way into the operand layout
+    Q6kCol col[kQ6kMaxColPasses];
+    uint8_t *scratch = ring + (NS - 1) * kQ6kTileBytes;
 #pragma unroll
-    for (int p = 0; p < kQ6kMaxColPasses; p++)
-        if ((uint32_t)p < np) q6k_mfma_prepare_col(raw[p], lane, cols + p * kQ6kColBytes);
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own writes, own reads: program order is enough
-    Q6kCol col;
-    if (np == 1) q6k_mfma_fetch_col(col, cols, jr, kq);
+    for (int p = 0; p < kQ6kMaxColPasses; p++) {
+        if ((uint32_t)p < np) {
+            q6k_mfma_prepare_col(raw[p], lane, scratch);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own writes, own reads: program order is enough
+            q6k_mfma_fetch_col(col[p], scratch, jr, kq);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // (read before the next column overwrites it)
+        }
+    }
 
     uint32_t n_use = 0;
     for (uint32_t tb = 0; tb < nt; tb += R) {
@@ -1015,18 +1015,18 @@ __device__ __forceinline__ void run_q6k_mfma(const GemvJob &j, uint32_t tile_a, 
         if (np >= 1) {
             float racc[R];
 #pragma unroll
-            for (int tl = 0; tl < R; tl++) racc[tl] = 0.f;
-#pragma unroll 1
-            for (uint32_t p = 0; p < np; p++) {
-                if (np > 1) q6k_mfma_fetch_col(col, cols + p * kQ6kColBytes, jr, kq);
+            for (int tl = 0; tl < R; tl++) {
+                racc[tl] = 0.f;
+                if ((uint32_t)tl < nb) {
 #pragma unroll
-                for (int tl = 0; tl < R; tl++) {
-                    if ((uint32_t)tl < nb) {
-                        issue();
-                        LARQL_WAIT_VMCNT(4 * (NS - 1));  // at most NS-1 younger wave-tiles still in flight: the oldest has landed
-                        asm volatile("" ::: "memory");
-                        racc[tl] += q6k_mfma_tile(ring + (n_use % NS) * kQ6kTileBytes, col, jr, kq);
-                        n_use++;
+                    for (int p = 0; p < kQ6kMaxColPasses; p++) {
+                        if ((uint32_t)p < np) {
+                            issue();
+                            LARQL_WAIT_VMCNT(4 * (NS - 1));  // at most NS-1 younger wave-tiles still in flight: the oldest has landed
+                            asm volatile("" ::: "memory");
+                            racc[tl] += q6k_mfma_tile(ring + (n_use % NS) * kQ6kTileBytes, col[p], jr, kq);
+                            n_use++;
+                        }
                     }
                 }
             }
@@ -2361,7 +2361,7 @@ __global__ void __launch_bounds__(kQ6kMaxWaves * 64) gemv_q6k_mfma_kernel(GemvLa
         const uint32_t seg_end = min(p_end, j.pass_begin + j.n_pass);
         const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin, cpt = (uint32_t)j.pad, su = j.pad2;
         const uint32_t tile_a = a > su ? (a - su + cpt - 1) / cpt : 0, tile_b = b > su ? (b - su + cpt - 1) / cpt : 0;
-        if (tile_a < tile_b) run_q6k_mfma(j, tile_a, tile_b, q6k_lds, L.pad, parity);
+        if (tile_a < tile_b) run_q6k_mfma(j, tile_a, tile_b, q6k_lds, parity);
         p = seg_end;
         ji++;
     }
@@ -2836,8 +2836,7 @@ size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
     }
     if (n > 0 && jobs[0].kind == KIND_Q6K_MFMA) {
         const size_t nw = threads / 64;
-        return nw * kQ6kStages * kQ6kTileBytes + 2 * (size_t)kQ6kBatchTiles * 16 * nw * 4 * sizeof(float) +
-               nw * gemv_launch_param(jobs, n) * kQ6kColBytes;
+        return nw * kQ6kStages * kQ6kTileBytes + 2 * (size_t)kQ6kBatchTiles * 16 * nw * 4 * sizeof(float);
     }
     if (n > 0 && jobs[0].kind == KIND_Q4K_MFMA) {
         const size_t nw = threads / 64;
