@@ -443,6 +443,74 @@ def run_q8k(be, fmt, args):
           dtype="i32")
 
 
+def run_formats(be, fmt, args):
+    """The other block formats of the matvec family at decode shapes, cache-cold (distinct copies of each matrix in one
+    launch, 0.5-1 GB per launch): Q6_K at the Gemma-3-4B FFN shapes, MXFP4 at the gpt-oss expert shape and at 4096 x 4096."""
+    O = _oracle()
+    rng = np.random.default_rng(0x5EED0700)
+    x_all = be.malloc(16384 * 4)
+    be.dev_fill_normal(x_all, 16384, 0x5EED0701, 1.0)
+    cases = [("Q6_K", 10240, 2560, 24), ("Q6_K", 2560, 10240, 24), ("MXFP4", 2880, 2880, 128), ("MXFP4", 4096, 4096, 64)]
+    for name, rows, k, copies in cases:
+        if name == "Q6_K":
+            # any bytes are valid 6-bit codes and int8 scales; d a small f16
+            blocks = rng.integers(0, 256, size=(rows * (k // 256), 210), dtype=np.uint8)
+            blocks[:, 208:210] = np.frombuffer(np.float16(rng.uniform(1e-4, 3e-4, size=rows * (k // 256))).tobytes(), np.uint8).reshape(-1, 2)
+            host = [blocks.reshape(-1)]
+            job = lambda bufs, o: (fmt.FMT_Q6_K, bufs[0], None, x_all, o, rows, k)
+            want = lambda r: O.q6k_matvec(host[0][:r * (k // 256) * 210], be.d2h(x_all, k, np.float32), r, k)
+        else:
+            tmp = be.malloc(rows * k * 4)
+            be.dev_fill_normal(tmp, rows * k, 0x5EED0710 + rows, 0.02)
+            p0, s0 = be.malloc(rows * k // 2 + 64), be.malloc(rows * k // 32 + 64)
+            assert be.dev_quantize_mxfp4(tmp, rows, k, p0, s0)
+            be.synchronize()
+            host = [be.d2h(p0, rows * k // 2, np.uint8), be.d2h(s0, rows * k // 32, np.uint8)]
+            for q in (tmp, p0, s0):
+                be.free(q)
+            job = lambda bufs, o: (fmt.FMT_MXFP4, bufs[0], bufs[1], x_all, o, rows, k)
+            want = lambda r: O.mxfp4_gemv(host[0][:r * k // 2], host[1][:r * k // 32], be.d2h(x_all, k, np.float32), r, k)
+        first = [be.to_device(h) for h in host]
+        bufs_all, outs = [first], []
+        for _ in range(copies - 1):  # exact copies at distinct addresses: nothing of a launch is served from a cache
+            cp = []
+            for h, src in zip(host, first):
+                assert h.size % 16 == 0
+                d = be.malloc(h.size + 64)
+                assert be.dev_copy(d, src, h.size)
+                cp.append(d)
+            bufs_all.append(cp)
+        jobs = []
+        for bufs in bufs_all:
+            o = be.malloc(rows * 4 + 64)
+            outs.append(o)
+            jobs.append(job(bufs, o))
+        plan = be.plan_create(jobs)
+        assert plan is not None
+        be.plan_run(plan); be.synchronize()
+        sample = 64
+        ref = want(sample)
+        rel = max(float(np.linalg.norm(be.d2h(o, sample, np.float32).astype(np.float64) - ref) / np.linalg.norm(ref)) for o in (outs[0], outs[-1]))
+        assert rel < 1e-3, (name, rows, k, rel)
+        ms = _timeit(be, lambda: be.plan_run(plan), args.steps)
+        algo = copies * (sum(h.size for h in host) + 4 * rows) + 4 * k
+        gbs = algo / ms / 1e6
+        med, n = _cpu_time(lambda: want(sample), args.cpu_seconds / 4)
+        _emit(f"{name} {rows}x{k} matvec HBM GB/s (cold, {copies} distinct copies per launch)", round(gbs, 1), "GB/s", ms, args.steps, 2,
+              {"workload": f"{name} matvec {rows}x{k}, batch 1, {copies} copies in one launch", "us_per_matvec": round(ms * 1e3 / copies, 3),
+               "verified_rel_l2_vs_oracle": rel},
+              {"kernel": "gemv_q6k_mfma" if name == "Q6_K" else "gemv_mxfp4_mfma", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+               "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+              {"value": round(sample * sum(h.size for h in host) / rows / med / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+               "sample": f"first {sample} rows, median of {n}"})
+        be.plan_destroy(plan)
+        for bufs in bufs_all:
+            for d in bufs:
+                be.free(d)
+        for o in outs:
+            be.free(o)
+
+
 def read_traffic():
     """HBM bytes per launch of the dominant kernel from the committed rocprof PMC summary, if any."""
     path = os.path.join(ROOT, "profiles", "gemv_q4k_c2_stack.pmc.txt")
@@ -464,7 +532,7 @@ def main():
     ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "q8k"],
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "q8k", "formats"],
                     help="c2 (default) is the headline decode stack; the others are BASELINE's remaining configs")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run the plain 16-byte copy kernel on 1 GiB three times (known size, for scaling "
@@ -498,7 +566,7 @@ def main():
                           "read_only_GBps": round(n / ms_r / 1e6, 1)}))
         return
     if args.workload != "c2":
-        {"c1": run_c1, "c3": run_c3, "c4": run_c4, "c5": run_c5, "q8k": run_q8k}[args.workload](be, fmt, args)
+        {"c1": run_c1, "c3": run_c3, "c4": run_c4, "c5": run_c5, "q8k": run_q8k, "formats": run_formats}[args.workload](be, fmt, args)
         return
     stack = Stack(be, fmt, layers=args.layers)
 
