@@ -1188,6 +1188,136 @@ float lq_clamped_glu(float g, float u, float limit, float alpha) {
     return (u + 1.0f) * (g * sig);
 }
 
+/* ------------------------------------------------------ MoE expert block */
+
+/* One weight row against x.  f32 banks: `w` is [rows, k] f32 (dot_proj =
+ * x . w^T, larql-compute/src/forward/ops.rs:43-48; the reference's BLAS sums
+ * in an order it does not fix, a sequential f32 dot stands in for it).
+ * MXFP4 banks: the row loop of lq_mxfp4_gemv above. */
+typedef struct {
+    int mxfp4;
+    const float *w_f32;
+    const uint8_t *packed, *scales;
+} moe_matrix;
+
+static float moe_row_dot(const moe_matrix *m, size_t row, size_t k, const float *x) {
+    float acc = 0.0f;
+    if (!m->mxfp4) {
+        const float *w = m->w_f32 + row * k;
+        for (size_t c = 0; c < k; c++) acc += w[c] * x[c];
+        return acc;
+    }
+    size_t groups = k / 32;
+    for (size_t g = 0; g < groups; g++) {
+        float scale = lq_e8m0_to_f32(m->scales[row * groups + g]);
+        const uint8_t *bytes = m->packed + (row * groups + g) * 16;
+        for (int b = 0; b < 16; b++) {
+            size_t e0 = g * 32 + 2 * (size_t)b;
+            acc += MXFP4_TABLE[bytes[b] & 0x0F] * scale * x[e0];
+            acc += MXFP4_TABLE[bytes[b] >> 4] * scale * x[e0 + 1];
+        }
+    }
+    return acc;
+}
+
+/* The expert block for one token, given its routing — the composition both
+ * tiers of the reference share:
+ *   ExpertWeightFfn::run_expert_observed + moe_block's weighted accumulation,
+ *     larql-compute/src/ffn/expert_weight/mod.rs:150-262 (f32 experts);
+ *   cpu_moe_forward's add_expert, cpu/ops/moe/forward.rs:201-270, and the Metal
+ *     combine h + sum_s w_s*(dot_s + bias_s),
+ *     larql-compute-metal/src/shaders/mxfp4_grouped_experts/kernels.rs:482-541.
+ * act[j] = rule.combine(gate.x + gate_bias[j], up.x + up_bias[j]); the fused bias
+ * row is interleaved (gate bias j at 2j, up bias j at 2j+1: ExpertMlp::gate_bias /
+ * up_bias, pipeline/moe.rs:150-166, FusedHalf::fused_row) whatever the weight
+ * layout; contribution = down.act + down_bias; out += w * contribution in
+ * selection order.  An expert id outside the bank is skipped (forward.rs:203-208).
+ * gate/up/down describe expert 0; expert e lies e*stride further on.
+ * `interleaved`: gate row j is fused row 2j and up row j is fused row 2j+1 of
+ * the gate matrix ([2*inter, hidden] per expert); `up` is not read. */
+static void moe_token(const float *x, size_t hidden, size_t inter, size_t n_experts, size_t top_k, const uint64_t *experts,
+                      const float *weights, const moe_matrix *gate, const moe_matrix *up, const moe_matrix *down,
+                      int interleaved, const float *gate_up_bias, const float *down_bias, float limit, float alpha,
+                      float *act, float *out) {
+    for (size_t c = 0; c < hidden; c++) out[c] = 0.0f;
+    for (size_t s = 0; s < top_k; s++) {
+        size_t e = (size_t)experts[s];
+        float w = weights[s];
+        if (e >= n_experts) continue;
+        size_t gu_rows = interleaved ? 2 * inter : inter;
+        moe_matrix g = *gate, u = interleaved ? *gate : *up, d = *down;
+        if (g.mxfp4) {
+            g.packed += e * gu_rows * (hidden / 32) * 16; g.scales += e * gu_rows * (hidden / 32);
+            u.packed += e * gu_rows * (hidden / 32) * 16; u.scales += e * gu_rows * (hidden / 32);
+            d.packed += e * hidden * (inter / 32) * 16; d.scales += e * hidden * (inter / 32);
+        } else {
+            g.w_f32 += e * gu_rows * hidden; u.w_f32 += e * gu_rows * hidden; d.w_f32 += e * hidden * inter;
+        }
+        for (size_t j = 0; j < inter; j++) {
+            size_t gr = interleaved ? 2 * j : j, ur = interleaved ? 2 * j + 1 : j;
+            float gv = moe_row_dot(&g, gr, hidden, x), uv = moe_row_dot(&u, ur, hidden, x);
+            if (gate_up_bias) { gv += gate_up_bias[e * 2 * inter + 2 * j]; uv += gate_up_bias[e * 2 * inter + 2 * j + 1]; }
+            act[j] = lq_clamped_glu(gv, uv, limit, alpha);
+        }
+        for (size_t c = 0; c < hidden; c++) {
+            float v = moe_row_dot(&d, c, inter, act);
+            if (down_bias) v += down_bias[e * hidden + c];
+            out[c] += w * v;
+        }
+    }
+}
+
+/* ExpertWeightFfn::moe_block for a GPT-OSS-shaped f32 layer —
+ * larql-compute/src/ffn/expert_weight/mod.rs:100-262: router logits = x . W_r^T
+ * + b_r, router::select per token, then the block above.  `fused` is
+ * [n_experts, 2*inter, hidden] as a checkpoint ships it (gate = even rows,
+ * up = odd rows: deinterleave_fused_half, larql-models/src/quant/mxfp4.rs:218-231).
+ * The reference groups tokens per expert and so adds a token's contributions in
+ * expert-index order; here they are added in selection order, as the served tier
+ * does (forward.rs) — the two differ by fp32 reordering only.
+ * Pinned: EXPECTED[48] of larql-compute/tests/test_moe_reference_parity.rs:72-85
+ * (values of an independent transcription of the GPT-OSS reference model). */
+int lq_moe_block_f32(const float *x, size_t tokens, size_t hidden, size_t inter, size_t n_experts, size_t top_k, int policy,
+                     const float *router_w, const float *router_b, const float *fused, const float *down,
+                     const float *gate_up_bias, const float *down_bias, float limit, float alpha, float *out) {
+    if (n_experts == 0 || top_k == 0) { for (size_t i = 0; i < tokens * hidden; i++) out[i] = 0.0f; return 0; }
+    float *logits = (float *)malloc(n_experts * sizeof(float));
+    float *act = (float *)malloc((inter ? inter : 1) * sizeof(float));
+    uint64_t *ex = (uint64_t *)malloc(top_k * sizeof(uint64_t));
+    float *wt = (float *)malloc(top_k * sizeof(float));
+    moe_matrix g = {0, fused, NULL, NULL}, d = {0, down, NULL, NULL};
+    for (size_t t = 0; t < tokens; t++) {
+        const float *xt = x + t * hidden;
+        for (size_t e = 0; e < n_experts; e++) {
+            float acc = 0.0f;
+            for (size_t c = 0; c < hidden; c++) acc += xt[c] * router_w[e * hidden + c];
+            logits[e] = router_b ? acc + router_b[e] : acc;
+        }
+        size_t k = lq_router_select(logits, n_experts, top_k, policy, ex, wt);
+        moe_token(xt, hidden, inter, n_experts, k, ex, wt, &g, &g, &d, 1, gate_up_bias, down_bias, limit, alpha, act,
+                  out + t * hidden);
+    }
+    free(logits); free(act); free(ex); free(wt);
+    return 0;
+}
+
+/* The same block over an MXFP4 bank with the routing given (experts / weights
+ * [tokens, top_k], as router::select returns them): the CPU tier refuses MXFP4
+ * banks (forward.rs:69-75), the Metal peer serves them with this composition. */
+int lq_moe_block_mxfp4(const float *x, size_t tokens, size_t hidden, size_t inter, size_t n_experts, size_t top_k,
+                       const uint64_t *experts, const float *weights, const uint8_t *gate_packed, const uint8_t *gate_scales,
+                       const uint8_t *up_packed, const uint8_t *up_scales, const uint8_t *down_packed, const uint8_t *down_scales,
+                       int interleaved, const float *gate_up_bias, const float *down_bias, float limit, float alpha, float *out) {
+    if (hidden % 32 != 0 || inter % 32 != 0) return 1;
+    float *act = (float *)malloc((inter ? inter : 1) * sizeof(float));
+    moe_matrix g = {1, NULL, gate_packed, gate_scales}, u = {1, NULL, up_packed, up_scales}, d = {1, NULL, down_packed, down_scales};
+    for (size_t t = 0; t < tokens; t++)
+        moe_token(x + t * hidden, hidden, inter, n_experts, top_k, experts + t * top_k, weights + t * top_k, &g, &u, &d, interleaved,
+                  gate_up_bias, down_bias, limit, alpha, act, out + t * hidden);
+    free(act);
+    return 0;
+}
+
 /* ------------------------------------------- multi-threaded CPU baseline */
 
 typedef struct {

@@ -112,6 +112,16 @@ size_t lq_router_select(const float *logits, size_t n, size_t k, int policy,
 size_t lq_moe_top_k(const float *v, size_t n, size_t k, uint64_t *idx, float *val);
 void   lq_softmax(float *v, size_t n);
 float  lq_clamped_glu(float g, float u, float limit, float alpha);
+/* ExpertWeightFfn::moe_block (ffn/expert_weight/mod.rs:100-262) on a GPT-OSS-shaped f32 layer; pinned on EXPECTED[48]
+ * of larql-compute/tests/test_moe_reference_parity.rs.  router_b / gate_up_bias / down_bias may be NULL. */
+int lq_moe_block_f32(const float *x, size_t tokens, size_t hidden, size_t inter, size_t n_experts, size_t top_k, int policy,
+                     const float *router_w, const float *router_b, const float *fused, const float *down,
+                     const float *gate_up_bias, const float *down_bias, float limit, float alpha, float *out);
+/* the same composition over an MXFP4 bank, routing given */
+int lq_moe_block_mxfp4(const float *x, size_t tokens, size_t hidden, size_t inter, size_t n_experts, size_t top_k,
+                       const uint64_t *experts, const float *weights, const uint8_t *gate_packed, const uint8_t *gate_scales,
+                       const uint8_t *up_packed, const uint8_t *up_scales, const uint8_t *down_packed, const uint8_t *down_scales,
+                       int interleaved, const float *gate_up_bias, const float *down_bias, float limit, float alpha, float *out);
 
 /* ---- multi-threaded drivers for the CPU baseline ----------------------- */
 /* Row-chunk parallel versions (32-row chunks, as the reference schedules

@@ -461,3 +461,55 @@ def softmax(v) -> np.ndarray:
     v = _f32(v).ravel().copy()
     _lib.lq_softmax(_p(v, _f32p), _sz(v.size))
     return v
+
+
+# ---- MoE expert block -------------------------------------------------------
+def _opt_f32(a):
+    if a is None:
+        return None, None
+    a = _f32(a).ravel()
+    return a, _p(a, _f32p)
+
+
+def moe_block_f32(x, router_w, router_b, fused, down, gate_up_bias, down_bias, top_k: int, policy: int = NORMALISED_OVER_SELECTED,
+                  limit: float = 7.0, alpha: float = 1.702) -> np.ndarray:
+    """ExpertWeightFfn::moe_block (ffn/expert_weight/mod.rs:100-262) on a GPT-OSS-shaped f32 layer.
+    x [T, hidden]; router_w [E, hidden]; fused [E, 2*inter, hidden] (gate = even rows, up = odd rows);
+    down [E, hidden, inter]; gate_up_bias [E, 2*inter] (interleaved) / down_bias [E, hidden] / router_b [E] or None."""
+    x, router_w, fused, down = _f32(x), _f32(router_w), _f32(fused), _f32(down)
+    tokens, hidden = x.shape
+    n_experts = router_w.shape[0]
+    inter = fused.shape[1] // 2
+    assert fused.shape == (n_experts, 2 * inter, hidden) and down.shape == (n_experts, hidden, inter)
+    rb, rbp = _opt_f32(router_b)
+    gb, gbp = _opt_f32(gate_up_bias)
+    db, dbp = _opt_f32(down_bias)
+    out = np.empty((tokens, hidden), np.float32)
+    _lib.lq_moe_block_f32(_p(x, _f32p), _sz(tokens), _sz(hidden), _sz(inter), _sz(n_experts), _sz(top_k), C.c_int(policy),
+                          _p(router_w, _f32p), rbp, _p(fused, _f32p), _p(down, _f32p), gbp, dbp, C.c_float(limit), C.c_float(alpha),
+                          _p(out, _f32p))
+    return out
+
+
+def moe_block_mxfp4(x, experts, weights, gate, up, down, n_experts: int, hidden: int, inter: int, interleaved: bool = False,
+                    gate_up_bias=None, down_bias=None, limit: float = 7.0, alpha: float = 1.702) -> np.ndarray:
+    """The expert block over an MXFP4 bank with the routing given.  gate / up / down are (packed, scales) pairs, expert
+    after expert; with `interleaved` gate holds each expert's fused [2*inter, hidden/32] rows and `up` is ignored.
+    experts / weights: [T, k]."""
+    x = _f32(x)
+    tokens = x.shape[0]
+    ex = np.ascontiguousarray(experts, dtype=np.uint64).reshape(tokens, -1)
+    wt = _f32(weights).reshape(tokens, -1)
+    k = ex.shape[1]
+    gp, gs = _u8(gate[0]), _u8(gate[1])
+    up_, us = (gp, gs) if interleaved else (_u8(up[0]), _u8(up[1]))
+    dp, ds = _u8(down[0]), _u8(down[1])
+    gb, gbp = _opt_f32(gate_up_bias)
+    db, dbp = _opt_f32(down_bias)
+    out = np.empty((tokens, hidden), np.float32)
+    rc = _lib.lq_moe_block_mxfp4(_p(x, _f32p), _sz(tokens), _sz(hidden), _sz(inter), _sz(n_experts), _sz(k), _p(ex, _u64p),
+                                 _p(wt, _f32p), _p(gp, _u8p), _p(gs, _u8p), _p(up_, _u8p), _p(us, _u8p), _p(dp, _u8p), _p(ds, _u8p),
+                                 C.c_int(1 if interleaved else 0), gbp, dbp, C.c_float(limit), C.c_float(alpha), _p(out, _f32p))
+    if rc:
+        raise ValueError("hidden and inter must be multiples of 32")
+    return out
