@@ -297,6 +297,24 @@ int larql_hip_dev_gate_knn(larql_hip_ctx *ctx, int format, const void *gate,
                            const float *x, size_t batch, size_t n_features, size_t hidden,
                            size_t top_k, float *scores_scratch, uint32_t *idx_out, float *score_out);
 
+/* larql_hip_dev_gate_knn for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same results as
+ * larql_hip_dev_gate_knn, bit for bit, but the score matrix, the hit counts and the quantised activation of
+ * Q4_0 gates live in a fixed array in device memory that the library holds on every GPU it runs on until the
+ * process ends (larql_hip_static_scratch_bytes(), about 0.7 MiB); the call itself performs no hipMalloc /
+ * hipFree, no host allocation and no table upload.  Limits (beyond them: LARQL_REFUSED_SHAPE with a message):
+ * batch <= LARQL_HIP_STATIC_MAX_BATCH, batch * n_features <= LARQL_HIP_STATIC_MAX_SCORES, and for Q4_0 gates
+ * hidden <= LARQL_HIP_STATIC_MAX_HIDDEN.  count_out (may be NULL): hits per position.  All calls on one GPU
+ * share that GPU's array, which keeps the previous call's contents: calls that overlap on one GPU (two
+ * contexts, or two streams) race; calls through one context are serialised. */
+#define LARQL_HIP_STATIC_MAX_BATCH 8
+#define LARQL_HIP_STATIC_MAX_SCORES 131072
+#define LARQL_HIP_STATIC_MAX_HIDDEN 16384
+size_t larql_hip_static_scratch_bytes(void);
+int larql_hip_dev_gate_knn_static(larql_hip_ctx *ctx, int format, const void *gate, const float *x, size_t batch,
+                                  size_t n_features, size_t hidden, size_t top_k, uint32_t *idx_out, float *score_out,
+                                  uint32_t *count_out);
+
 /* Gate-KNN over `n_layers` layers in ONE submission — the shape of LQL WALK / DESCRIBE, where
  * every layer of the index is scored for one query (PatchedVindex::walk,
  * larql-vindex/src/patch/overlay.rs:557-562 over VectorIndex::gate_knn): one matvec launch for all

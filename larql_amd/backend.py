@@ -391,6 +391,14 @@ class HipBackend:
                      val: int) -> bool:
         return self._some(lib.larql_hip_dev_gate_knn(self._h, fmt, gate, x, batch, n, hidden, top_k, scores, idx, val))
 
+    def static_scratch_bytes(self) -> int:
+        return int(lib.larql_hip_static_scratch_bytes())
+
+    def dev_gate_knn_static(self, fmt: int, gate: int, x: int, batch: int, n: int, hidden: int, top_k: int, idx: int,
+                            val: int, counts: Optional[int] = None) -> bool:
+        """larql_hip_dev_gate_knn without any allocation (scores live in the library's static device array)."""
+        return self._some(lib.larql_hip_dev_gate_knn_static(self._h, fmt, gate, x, batch, n, hidden, top_k, idx, val, counts))
+
     def dev_gate_walk(self, fmt: int, gates: Sequence[int], x: int, x_layer_stride: int, batch: int, n: int, hidden: int,
                       top_k: int, scores: int, idx: int, val: int, count: Optional[int] = None) -> bool:
         arr = (C.c_void_p * max(len(gates), 1))(*gates)

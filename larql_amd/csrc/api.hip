@@ -20,6 +20,26 @@
 
 using namespace larql;
 
+// Scratch memory of larql_hip_dev_gate_knn_static, the entry point that allocates nothing: the score matrix, the hit
+// counts and (Q4_0 gates) the quantised activation live here instead of in caller-provided or per-context buffers.
+// Every GPU holds its own copy of the array; host code reaches it only through the address hipGetSymbolAddress
+// returns for the current device (larql_hip_create keeps it in the context), never through the array's name.
+// Layout: [scores: MAX_SCORES f32][counts: MAX_BATCH u32, padded to 256 B][Q8 codes: MAX_BATCH*MAX_HIDDEN i8]
+//         [Q8 block scales: MAX_BATCH*MAX_HIDDEN/32 f32]
+constexpr size_t kStaticScoresBytes = (size_t)LARQL_HIP_STATIC_MAX_SCORES * 4;
+constexpr size_t kStaticCountsBytes = 256;
+constexpr size_t kStaticQ8Bytes = (size_t)LARQL_HIP_STATIC_MAX_BATCH * LARQL_HIP_STATIC_MAX_HIDDEN;
+constexpr size_t kStaticQ8ScaleBytes = kStaticQ8Bytes / 32 * 4;
+constexpr size_t kStaticScratchBytes = kStaticScoresBytes + kStaticCountsBytes + kStaticQ8Bytes + kStaticQ8ScaleBytes;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Clears a few words on the stream (a kernel, not hipMemsetAsync: memset nodes recorded into a captured graph have
+// given wrong results on replays).
+__global__ void zero_words_kernel(uint32_t *p, uint32_t n) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
 namespace {
 
 struct DevBuf {
@@ -54,6 +74,7 @@ struct larql_hip_ctx {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     uint8_t *log2_up = nullptr;  // 256-entry table for the MXFP4 encoder
     int *nan_flag = nullptr;
+    uint8_t *static_scratch = nullptr;  // this device's copy of `scratch` (hipGetSymbolAddress at create)
     larql_hip_submission_clock clock = {0, 0, 0};
 };
 
@@ -86,8 +107,8 @@ int ensure(larql_hip_ctx *c, DevBuf &b, size_t bytes) {
 }
 
 // A weight slice is served from a registered region when it lies inside one at
-// a 16-byte aligned offset; otherwise it is uploaded into `scratch` for the call.
-int resolve_weights(larql_hip_ctx *c, const uint8_t *host, size_t len, DevBuf &scratch, const uint8_t **dev) {
+// a 16-byte aligned offset; otherwise it is uploaded into `staging` for the call.
+int resolve_weights(larql_hip_ctx *c, const uint8_t *host, size_t len, DevBuf &staging, const uint8_t **dev) {
     for (const Region &r : c->regions) {
         if (host >= r.host && host + len <= r.host + r.len && ((size_t)(host - r.host) % 16) == 0) {
             *dev = r.dev + (host - r.host);
@@ -95,10 +116,10 @@ int resolve_weights(larql_hip_ctx *c, const uint8_t *host, size_t len, DevBuf &s
         }
     }
     // pad so kernels that read an aligned window past the last block stay in bounds
-    int rc = ensure(c, scratch, len + 64);
+    int rc = ensure(c, staging, len + 64);
     if (rc) return rc;
-    if (len) HIPCHECK(c, hipMemcpyAsync(scratch.p, host, len, hipMemcpyHostToDevice, c->stream));
-    *dev = (const uint8_t *)scratch.p;
+    if (len) HIPCHECK(c, hipMemcpyAsync(staging.p, host, len, hipMemcpyHostToDevice, c->stream));
+    *dev = (const uint8_t *)staging.p;
     return LARQL_OK;
 }
 
@@ -153,12 +174,13 @@ struct PreparedLaunch {
 
 // Geometry for one launch over jobs of a single format.  When the jobs do not fit
 // inline the table is uploaded into `table_dst` (synchronously: the host vector may die).
-int prepare_same_kind(larql_hip_ctx *c, std::vector<GemvJob> &live, void *table_dst, PreparedLaunch &P, int stage_slot = -1) {
+int prepare_same_kind(larql_hip_ctx *c, GemvJob *live, size_t n_live, void *table_dst, PreparedLaunch &P, int stage_slot = -1) {
     P.kind = live[0].kind;
-    P.threads = gemv_pick_threads(live.data(), live.size());
+    P.threads = gemv_pick_threads(live, n_live);
     if (P.threads == 0) return fail(c, LARQL_UNSUPPORTED, "matvec: row length not supported by the gfx950 kernels");
     uint64_t total = 0;
-    for (GemvJob &j : live) {
+    for (size_t ji = 0; ji < n_live; ji++) {
+        GemvJob &j = live[ji];
         if (!gemv_job_geometry(j, P.threads)) return fail(c, LARQL_UNSUPPORTED, "matvec: unsupported geometry");
         if (total + j.n_pass > 0x7FFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "matvec: launch too large");
         j.pass_begin = (uint32_t)total;
@@ -166,15 +188,15 @@ int prepare_same_kind(larql_hip_ctx *c, std::vector<GemvJob> &live, void *table_
     }
     memset(&P.L, 0, sizeof P.L);
     P.L.total_passes = total;
-    P.L.n_jobs = (uint32_t)live.size();
-    P.L.pad = gemv_launch_param(live.data(), live.size());
-    if (live.size() <= (size_t)kInlineJobs) {
-        for (size_t i = 0; i < live.size(); i++) P.L.inl[i] = live[i];
+    P.L.n_jobs = (uint32_t)n_live;
+    P.L.pad = gemv_launch_param(live, n_live);
+    if (n_live <= (size_t)kInlineJobs) {
+        for (size_t i = 0; i < n_live; i++) P.L.inl[i] = live[i];
         P.L.table = nullptr;
     } else {
-        const size_t bytes = live.size() * sizeof(GemvJob);
+        const size_t bytes = n_live * sizeof(GemvJob);
         if (stage_slot >= 0 && c->table_sent_dst[stage_slot] == table_dst && c->table_sent_bytes[stage_slot] == bytes &&
-            memcmp(c->table_host[stage_slot], live.data(), bytes) == 0) {
+            memcmp(c->table_host[stage_slot], live, bytes) == 0) {
             // the same jobs as the last call through this slot (a decode loop): the device table is already (or, in
             // stream order, about to be) what this launch needs
         } else if (stage_slot >= 0) {
@@ -189,18 +211,18 @@ int prepare_same_kind(larql_hip_ctx *c, std::vector<GemvJob> &live, void *table_
             }
             if (!c->table_ev[stage_slot]) HIPCHECK(c, hipEventCreateWithFlags(&c->table_ev[stage_slot], hipEventDisableTiming));
             else HIPCHECK(c, hipEventSynchronize(c->table_ev[stage_slot]));  // the previous upload from this slot is done
-            memcpy(c->table_host[stage_slot], live.data(), bytes);
+            memcpy(c->table_host[stage_slot], live, bytes);
             HIPCHECK(c, hipMemcpyAsync(table_dst, c->table_host[stage_slot], bytes, hipMemcpyHostToDevice, c->stream));
             HIPCHECK(c, hipEventRecord(c->table_ev[stage_slot], c->stream));
             c->table_sent_dst[stage_slot] = table_dst;
             c->table_sent_bytes[stage_slot] = bytes;
         } else {
-            HIPCHECK(c, hipMemcpyAsync(table_dst, live.data(), bytes, hipMemcpyHostToDevice, c->stream));
+            HIPCHECK(c, hipMemcpyAsync(table_dst, live, bytes, hipMemcpyHostToDevice, c->stream));
             HIPCHECK(c, hipStreamSynchronize(c->stream));  // the host vector may die
         }
         P.L.table = (const GemvJob *)table_dst;
     }
-    P.lds = gemv_lds_bytes(live.data(), live.size(), P.threads);
+    P.lds = gemv_lds_bytes(live, n_live, P.threads);
     uint64_t grid = (uint64_t)c->cu_count * (uint64_t)gemv_wgs_per_cu(P.kind, P.threads, P.lds, (uint32_t)c->wgs_per_cu);
     if (grid > total) grid = total;
     P.grid = (uint32_t)grid;
@@ -253,7 +275,7 @@ int enqueue_jobs(larql_hip_ctx *c, std::vector<GemvJob> &jobs) {
             if (tb.p != before) c->table_sent_dst[sl] = nullptr;  // a new allocation holds nothing yet
         }
         PreparedLaunch P;
-        rc = prepare_same_kind(c, live, tb.p, P, sl);
+        rc = prepare_same_kind(c, live.data(), live.size(), tb.p, P, sl);
         if (rc) return rc;
         HIPCHECK(c, gemv_launch(c->stream, P.kind, P.L, P.threads, P.grid, P.lds));
     }
@@ -317,6 +339,13 @@ int larql_hip_create(larql_hip_ctx **out, int device) {
         larql_hip_destroy(c);
         return LARQL_E_DEVICE;
     }
+    // the address of this device's copy of the static scratch array (the device is current: hipSetDevice above)
+    void *sp = nullptr;
+    if (hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch)) != hipSuccess || !sp) {
+        larql_hip_destroy(c);
+        return LARQL_E_DEVICE;
+    }
+    c->static_scratch = (uint8_t *)sp;
     *out = c;
     return LARQL_OK;
 }
@@ -1095,7 +1124,7 @@ int larql_hip_plan_create(larql_hip_ctx *c, const larql_hip_matvec_job *pj, size
                 return fail(c, LARQL_E_DEVICE, "plan: out of device memory");
             }
         }
-        rc = prepare_same_kind(c, live, P.table, P);
+        rc = prepare_same_kind(c, live.data(), live.size(), P.table, P);
         if (rc) {
             if (P.table) (void)hipFree(P.table);
             for (PreparedLaunch &q : plan->launches) if (q.table) (void)hipFree(q.table);
@@ -1159,6 +1188,74 @@ int larql_hip_dev_gate_knn(larql_hip_ctx *c, int format, const void *gate, const
     if (rc) return rc;
     HIPCHECK(c, topk_launch(c->stream, scores_scratch, (uint32_t)batch, (uint32_t)n, (uint32_t)top_k, true, idx_out, score_out,
                             (uint32_t *)c->misc.p, c->nan_flag, nullptr, 0));
+    return LARQL_OK;
+}
+
+size_t larql_hip_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+// larql_hip_dev_gate_knn without any allocation: scores, hit counts and the Q8 activation of Q4_0 gates use this
+// device's static scratch array; job descriptors travel in the kernel arguments (at most kInlineJobs per launch,
+// which batch <= LARQL_HIP_STATIC_MAX_BATCH guarantees); no vector, no staging buffer, no table upload.
+int larql_hip_dev_gate_knn_static(larql_hip_ctx *c, int format, const void *gate, const float *x, size_t batch, size_t n,
+                                  size_t hidden, size_t top_k, uint32_t *idx_out, float *score_out, uint32_t *count_out) {
+    if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    const int kind = kind_of_format(format);
+    int rc = gate_shape_check(c, kind, (size_t)-1, 0, hidden);
+    if (rc) return rc;
+    if (batch == 0 || n == 0 || top_k == 0) return LARQL_OK;
+    if (top_k > kTopkMaxK || hidden == 0) return fail(c, LARQL_UNSUPPORTED, "gate-KNN: unsupported size");
+    if (batch > LARQL_HIP_STATIC_MAX_BATCH || n > LARQL_HIP_STATIC_MAX_SCORES || batch * n > LARQL_HIP_STATIC_MAX_SCORES)
+        return fail(c, LARQL_REFUSED_SHAPE, "gate_knn_static: batch %zu x %zu features exceeds the static scratch (at most %d positions, %d scores)",
+                    batch, n, LARQL_HIP_STATIC_MAX_BATCH, LARQL_HIP_STATIC_MAX_SCORES);
+    if (kind == KIND_Q4_0 && hidden > LARQL_HIP_STATIC_MAX_HIDDEN)
+        return fail(c, LARQL_REFUSED_SHAPE, "gate_knn_static: Q4_0 gates take rows of at most %d elements here", LARQL_HIP_STATIC_MAX_HIDDEN);
+    if (!gate || !x || !idx_out || !score_out || !c->static_scratch) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    float *scores = (float *)c->static_scratch;
+    uint32_t *counts = (uint32_t *)(c->static_scratch + kStaticScoresBytes);
+    int8_t *q8 = (int8_t *)(c->static_scratch + kStaticScoresBytes + kStaticCountsBytes);
+    float *q8s = (float *)(c->static_scratch + kStaticScoresBytes + kStaticCountsBytes + kStaticQ8Bytes);
+    GemvJob jobs[LARQL_HIP_STATIC_MAX_BATCH];
+    size_t n_jobs = 0;
+    if (kind == KIND_Q4_0) {
+        HIPCHECK(c, quantize_to_q8_launch(c->stream, x, batch * hidden, q8, q8s));
+        for (size_t b = 0; b < batch; b++)
+            jobs[n_jobs++] = make_job(kind, gate, q8s + b * (hidden / 32), q8 + b * hidden, scores + b * n, n, hidden);
+    } else {
+        const size_t cap = gemv_batch_capacity(kind, hidden);
+        for (size_t b = 0; b < batch;) {
+            const size_t take = std::min(cap, batch - b);
+            GemvJob j = make_job(kind, gate, nullptr, x + b * hidden, scores + b * n, n, hidden);
+            if (take >= 2) { j.batch = (uint32_t)take; j.x_stride = hidden; j.out_stride = n; }
+            jobs[n_jobs++] = j;
+            b += take;
+        }
+    }
+    for (size_t i = 0; i < n_jobs; i++) {
+        if (((uintptr_t)jobs[i].w & 15) || ((uintptr_t)jobs[i].x & 15))
+            return fail(c, LARQL_REFUSED_SHAPE, "matvec: weight and activation pointers must be 16-byte aligned");
+        if (kind == KIND_Q4_0 && (hidden % 64) != 0) return fail(c, LARQL_UNSUPPORTED, "matvec: this block format needs k %% 64 == 0 on this backend");
+        jobs[i].kind = gemv_effective_kind(jobs[i]);
+    }
+    // one launch per kernel the jobs map to (a full group of positions and a single left-over position may differ)
+    bool done[LARQL_HIP_STATIC_MAX_BATCH] = {};
+    for (size_t i = 0; i < n_jobs; i++) {
+        if (done[i]) continue;
+        GemvJob live[LARQL_HIP_STATIC_MAX_BATCH];
+        size_t n_live = 0;
+        for (size_t t = i; t < n_jobs; t++)
+            if (!done[t] && jobs[t].kind == jobs[i].kind) { live[n_live++] = jobs[t]; done[t] = true; }
+        static_assert(LARQL_HIP_STATIC_MAX_BATCH <= kInlineJobs, "the jobs of a launch must fit the kernel arguments");
+        PreparedLaunch P;
+        rc = prepare_same_kind(c, live, n_live, nullptr, P);
+        if (rc) return rc;
+        HIPCHECK(c, gemv_launch(c->stream, P.kind, P.L, P.threads, P.grid, P.lds));
+    }
+    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, c->stream, (uint32_t *)c->nan_flag, 1u);
+    HIPCHECK(c, hipGetLastError());
+    HIPCHECK(c, topk_launch(c->stream, scores, (uint32_t)batch, (uint32_t)n, (uint32_t)top_k, true, idx_out, score_out,
+                            count_out ? count_out : counts, c->nan_flag, nullptr, 0));
     return LARQL_OK;
 }
 
