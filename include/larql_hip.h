@@ -356,12 +356,21 @@ typedef struct {
      * (FusedHalf::fused_row, larql-models/src/quant/mxfp4.rs:179-191); up_* are not read.
      * The fused rows are walked in place, one pass over 2*inter rows per (token, expert). */
     int gate_up_interleaved;
+    /* Biases of MoeLayerWeights — pipeline/moe.rs:505-516, read by ExpertMlp::{gate_bias, up_bias, add_down_bias}
+     * (pipeline/moe.rs:150-176); each may be NULL (none).  router_bias [n_experts] is added to the router logits
+     * before the selection (larql_hip_dev_moe_mxfp4_routed only).  gate_up_bias [n_experts, 2*inter] is the fused
+     * row as the checkpoint ships it — gate bias j at 2j, up bias j at 2j+1 — whatever the weight layout.
+     * down_bias [n_experts, hidden].  The block computes sum_s w_s * (down_e(ClampedGlu(gate_e.x + bg, up_e.x + bu)) + bd). */
+    const float *router_bias, *gate_up_bias, *down_bias;
 } larql_hip_mxfp4_experts;
 /* The expert block of cpu_moe_forward (cpu/ops/moe/forward.rs:201-270) for
  * MXFP4 banks, which the CPU tier refuses (forward.rs:69-75): per token and
- * selected expert, gate/up matvec -> ClampedGlu -> down matvec, then the
+ * selected expert, gate/up matvec (+ bias) -> ClampedGlu -> down matvec (+ bias), then the
  * weighted sum in selection order.  `experts` stays on the device (the kernels
- * index the bank with it), so routing needs no host round trip.  Five launches.
+ * index the bank with it), so routing needs no host round trip; an expert id >= n_experts is skipped,
+ * as the reference skips it (forward.rs:203-208).  One token with k <= 4: two launches — the down
+ * projection folds the k experts and the weighted sum into one pass over the output rows (the shape of
+ * the Metal peer's mxfp4g_down_combine4, larql-compute-metal/src/shaders/mxfp4_grouped_experts/kernels.rs:482-541).
  * workspace: larql_hip_moe_mxfp4_workspace_bytes(...) of device memory; workspace, x and the packed streams
  * 16-byte aligned (else LARQL_REFUSED_SHAPE). */
 size_t larql_hip_moe_mxfp4_workspace_bytes(size_t tokens, size_t k, size_t hidden, size_t inter);

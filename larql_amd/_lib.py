@@ -30,7 +30,7 @@ class SubmissionClock(C.Structure):
 class Mxfp4Experts(C.Structure):
     _fields_ = [("gate_packed", vp), ("gate_scales", vp), ("up_packed", vp), ("up_scales", vp), ("down_packed", vp),
                 ("down_scales", vp), ("n_experts", sz), ("hidden", sz), ("inter", sz), ("limit", C.c_float),
-                ("alpha", C.c_float), ("gate_up_interleaved", C.c_int)]
+                ("alpha", C.c_float), ("gate_up_interleaved", C.c_int), ("router_bias", vp), ("gate_up_bias", vp), ("down_bias", vp)]
 
 
 class MatvecJob(C.Structure):

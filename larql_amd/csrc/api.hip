@@ -1306,7 +1306,7 @@ int larql_hip_dev_router_select(larql_hip_ctx *c, const float *logits, size_t to
     if (n_experts > 64 || k > 8) return fail(c, LARQL_UNSUPPORTED, "router_select: at most 64 experts and top-8 on this backend");
     if (!logits || !experts || !weights) return LARQL_E_ARG;
     HIPCHECK(c, hipSetDevice(c->device));
-    HIPCHECK(c, router_select_launch(c->stream, logits, (uint32_t)tokens, (uint32_t)n_experts, (uint32_t)k, policy, experts, weights));
+    HIPCHECK(c, router_select_launch(c->stream, logits, nullptr, (uint32_t)tokens, (uint32_t)n_experts, (uint32_t)k, policy, experts, weights));
     return LARQL_OK;
 }
 
@@ -1343,18 +1343,33 @@ static int moe_mxfp4_block(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank
     const uint64_t dn_w_stride = hidden * (inter / 32) * 16, dn_s_stride = hidden * (inter / 32);
     // one token: the gate/up launch can select for itself (every wavefront repeats the token's selection, the
     // workgroup that opens the first job writes it out for the launches that follow)
+    // Expert biases ride in the jobs: the fused bias row is interleaved (gate bias j at 2j, up bias j at 2j+1) whatever the
+    // weight layout, so a fused job adds it element for element and separate gate / up jobs take every second element.
+    const auto set_gate_up_bias = [&](GemvJob &jb, int half) {
+        if (!bank->gate_up_bias) return;
+        jb.bias = bank->gate_up_bias + (fused ? 0 : half);
+        jb.bias_step = fused ? 1u : 2u;
+        jb.bias_sel_stride = 2 * inter;
+    };
+    const auto set_down_bias = [&](GemvJob &jb) {
+        if (!bank->down_bias) return;
+        jb.bias = bank->down_bias; jb.bias_step = 1; jb.bias_sel_stride = hidden;
+    };
     const bool route_in_launch = route_logits && tokens == 1 &&
         gemv_effective_kind(make_job(KIND_MXFP4, bank->gate_packed, bank->gate_scales, x, g, gu_rows, hidden)) == KIND_MXFP4_MFMA;
     if (route_logits && !route_in_launch)
-        HIPCHECK(c, router_select_launch(c->stream, route_logits, (uint32_t)tokens, (uint32_t)bank->n_experts, (uint32_t)k, route_policy,
-                                         experts, weights));
+        HIPCHECK(c, router_select_launch(c->stream, route_logits, bank->router_bias, (uint32_t)tokens, (uint32_t)bank->n_experts, (uint32_t)k,
+                                         route_policy, experts, weights));
     // Several tokens: slots that chose the same expert share its weights up to four at a time.  The job lists are built on
     // the device from the router's choice (moe_plan_kernel) into the workspace's spare activation area.
     {
         GemvJob tg = make_job(KIND_MXFP4, bank->gate_packed, bank->gate_scales, x, g, gu_rows, hidden);
+        set_gate_up_bias(tg, 0);
         GemvJob tu = fused ? tg : make_job(KIND_MXFP4, bank->up_packed, bank->up_scales, x, u, inter, hidden);
+        if (!fused) set_gate_up_bias(tu, 1);
         GemvJob td = make_job(KIND_MXFP4, bank->down_packed, bank->down_scales, g, d, hidden, inter);
         td.x_glu = fused ? g : u; td.glu_limit = bank->limit; td.glu_alpha = bank->alpha;
+        set_down_bias(td);
         const size_t table_bytes = slots * 3 * sizeof(GemvJob) + 64;
         const bool mfma = gemv_effective_kind(tg) == KIND_MXFP4_MFMA && gemv_effective_kind(td) == KIND_MXFP4_MFMA;
         static const bool pairing = !(getenv("LARQL_HIP_MOE_PAIRS") && atoi(getenv("LARQL_HIP_MOE_PAIRS")) == 0);
@@ -1395,7 +1410,8 @@ static int moe_mxfp4_block(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank
                                         dn_table, hdr + 2));
             HIPCHECK(c, gemv_launch(c->stream, Pg.kind, Pg.L, Pg.threads, Pg.grid, Pg.lds));
             HIPCHECK(c, gemv_launch(c->stream, Pd.kind, Pd.L, Pd.threads, Pd.grid, Pd.lds));
-            HIPCHECK(c, weighted_sum_launch(c->stream, d, weights, out, (uint32_t)tokens, (uint32_t)k, (uint32_t)hidden));
+            HIPCHECK(c, weighted_sum_launch(c->stream, d, weights, experts, (uint32_t)bank->n_experts, out, (uint32_t)tokens, (uint32_t)k,
+                                            (uint32_t)hidden));
             return LARQL_OK;
         }
     }
@@ -1403,17 +1419,19 @@ static int moe_mxfp4_block(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank
     for (size_t s = 0; s < slots; s++) {
         const size_t t = s / k;
         GemvJob a = make_job(KIND_MXFP4, bank->gate_packed, bank->gate_scales, x + t * hidden, g + s * gu_rows, gu_rows, hidden);
-        a.sel = experts + s; a.w_sel_stride = gu_w_stride; a.aux_sel_stride = gu_s_stride;
+        a.sel = experts + s; a.w_sel_stride = gu_w_stride; a.aux_sel_stride = gu_s_stride; a.sel_count = (uint32_t)bank->n_experts;
+        set_gate_up_bias(a, 0);
         if (route_in_launch) {
             a.sel = nullptr;
-            a.route_logits = route_logits; a.route_n = (uint32_t)bank->n_experts; a.route_k = (uint32_t)k; a.route_rank = (uint32_t)s;
-            a.route_policy = route_policy;
+            a.route_logits = route_logits; a.route_bias = bank->router_bias; a.route_n = (uint32_t)bank->n_experts; a.route_k = (uint32_t)k;
+            a.route_rank = (uint32_t)s; a.route_policy = route_policy;
         }
         GemvJob b = a;
         if (route_in_launch && s == 0) { a.route_experts = experts; a.route_weights = weights; }
         jobs.push_back(a);
         if (fused) continue;
         b.w = (const uint8_t *)bank->up_packed; b.aux = (const uint8_t *)bank->up_scales; b.out = u + s * inter; b.rows = inter;
+        set_gate_up_bias(b, 1);
         jobs.push_back(b);
     }
     int rc = enqueue_jobs(c, jobs);
@@ -1425,17 +1443,32 @@ static int moe_mxfp4_block(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank
         else HIPCHECK(c, clamped_glu_launch(c->stream, g, u, h, slots * inter, bank->limit, bank->alpha));
     }
     jobs.clear();
+    if (fuse_glu && tokens == 1 && k <= 4) {
+        // One token: the down projection folds its k experts and the weighted sum — every workgroup walks its output rows
+        // through the k experts' matrices, each activation scaled by its routing weight, and writes
+        // sum_s w_s * (down_s . act_s + bias_s) itself.  No third launch.
+        const size_t gs = fused ? 2 * inter : inter;  // floats of gate/up results per slot
+        GemvJob a = make_job(KIND_MXFP4, bank->down_packed, bank->down_scales, g, out, hidden, inter);
+        a.x_glu = fused ? g : u; a.glu_limit = bank->limit; a.glu_alpha = bank->alpha;
+        a.batch = (uint32_t)k; a.x_stride = gs; a.x_off[0] = (int64_t)(2 * gs); a.x_off[1] = (int64_t)(3 * gs);
+        a.sel = experts; a.w_sel_stride = dn_w_stride; a.aux_sel_stride = dn_s_stride; a.sel_count = (uint32_t)bank->n_experts;
+        a.combine_w = weights;
+        set_down_bias(a);
+        jobs.push_back(a);
+        return enqueue_jobs(c, jobs);
+    }
     for (size_t s = 0; s < slots; s++) {
         const float *gx = fused ? g + s * 2 * inter : g + s * inter;
         GemvJob a = make_job(KIND_MXFP4, bank->down_packed, bank->down_scales, fuse_glu ? gx : h + s * inter, d + s * hidden,
                              hidden, inter);
         if (fuse_glu) { a.x_glu = fused ? gx : u + s * inter; a.glu_limit = bank->limit; a.glu_alpha = bank->alpha; }
-        a.sel = experts + s; a.w_sel_stride = dn_w_stride; a.aux_sel_stride = dn_s_stride;
+        a.sel = experts + s; a.w_sel_stride = dn_w_stride; a.aux_sel_stride = dn_s_stride; a.sel_count = (uint32_t)bank->n_experts;
+        set_down_bias(a);
         jobs.push_back(a);
     }
     rc = enqueue_jobs(c, jobs);
     if (rc) return rc;
-    HIPCHECK(c, weighted_sum_launch(c->stream, d, weights, out, (uint32_t)tokens, (uint32_t)k, (uint32_t)hidden));
+    HIPCHECK(c, weighted_sum_launch(c->stream, d, weights, experts, (uint32_t)bank->n_experts, out, (uint32_t)tokens, (uint32_t)k, (uint32_t)hidden));
     return LARQL_OK;
 }
 

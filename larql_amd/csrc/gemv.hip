@@ -473,7 +473,7 @@ __device__ __forceinline__ float f32x16_dot(const f32x4 *__restrict__ w, const X
 // DPP reduction inside the 16-lane row.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ void tile_epilogue(const float *part, uint32_t npart, uint32_t tile_rows,
-                                              float *out, uint32_t row_base) {
+                                              float *out, uint32_t row_base, const float *bias = nullptr, uint32_t bias_step = 1) {
     const uint32_t lane16 = threadIdx.x & 15u;
     for (uint32_t r = threadIdx.x >> 4; r < tile_rows; r += blockDim.x >> 4) {
         float v = 0.f;
@@ -482,7 +482,10 @@ __device__ __forceinline__ void tile_epilogue(const float *part, uint32_t npart,
         v = dpp_add<0x114>(v);  // row_shr:4
         v = dpp_add<0x112>(v);  // row_shr:2
         v = dpp_add<0x111>(v);  // row_shr:1
-        if (lane16 == 15u) ((g_f32wp)out)[row_base + r] = v;
+        if (lane16 == 15u) {
+            if (bias) v += ((const GLOBAL_AS float *)bias)[(size_t)(row_base + r) * bias_step];
+            ((g_f32wp)out)[row_base + r] = v;
+        }
     }
 }
 
@@ -1247,6 +1250,15 @@ struct Mx4Step {
 constexpr int kMx4MaxTokens = 4;    // tokens that share one job's weights: two per 16-row A operand
 struct Mx4In { float2_t v[kMx4MaxTokens], u[kMx4MaxTokens]; };
 
+// The weight matrices a job reads (wave-uniform): one, or — a job folded over experts (GemvJob::combine_w) — one per
+// activation, each with its expert's bias row and combine weight; `ok` is false for an expert id outside the bank.
+struct Mx4Sel {
+    const uint8_t *w[kMx4MaxTokens], *aux[kMx4MaxTokens];
+    const float *bias[kMx4MaxTokens];
+    float cw[kMx4MaxTokens];
+    bool ok[kMx4MaxTokens];
+};
+
 __device__ __forceinline__ uint32_t mx4_tokens(const GemvJob &j) { return j.batch > 1 ? min(j.batch, (uint32_t)kMx4MaxTokens) : 1u; }
 __device__ __forceinline__ int64_t mx4_x_off(const GemvJob &j, int q) { return q == 0 ? 0 : q == 1 ? (int64_t)j.x_stride : q == 2 ? j.x_off[0] : j.x_off[1]; }
 __device__ __forceinline__ int64_t mx4_out_off(const GemvJob &j, uint32_t q) { return q == 0 ? 0 : q == 1 ? (int64_t)j.out_stride : q == 2 ? j.out_off[0] : j.out_off[1]; }
@@ -1273,86 +1285,95 @@ __device__ __forceinline__ Mx4In mx4_load_step(const GemvJob &j, uint32_t step, 
     return in;
 }
 
-// The operands of all `cw` steps of a wavefront.  Per token, the digits of every step go to `scratch` (512 bytes per
-// step: digit row d at d*64) first and are read back in the operand layout afterwards, so the LDS round trip is paid
-// once per token, not once per step.
-__device__ __forceinline__ void mx4_setup_steps(const GemvJob &j, const Mx4In (&in)[kMx4MaxSteps], Mx4Step (&st)[2][kMx4MaxSteps], uint32_t cw,
-                                                uint32_t lane, uint8_t *scratch) {
+// One token's operands of all `cw` steps of a wavefront: the digits of every step go to `scratch` (512 bytes per step:
+// digit row d at d*64) first and are read back in the operand layout afterwards, so the LDS round trip is paid once
+// per token, not once per step.  The token's eight digit rows become A rows 8*half .. 8*half+7 of `sq` (the other
+// rows are left as they are); `wq` scales the activation (a folded job's routing weight) when `scaled` is set.
+template <int Q>
+__device__ __forceinline__ void mx4_setup_token(const GemvJob &j, bool scaled, float wq, const Mx4In (&in)[kMx4MaxSteps],
+                                                Mx4Step (&sq)[kMx4MaxSteps], uint32_t half, uint32_t cw, uint32_t lane, uint8_t *scratch) {
     const uint32_t t = lane & 15u, kg = lane >> 4;
+    int ex[kMx4MaxSteps];
+#pragma unroll
+    for (int s = 0; s < kMx4MaxSteps; s++) {
+        if ((uint32_t)s >= cw) continue;
+        float2_t v = in[s].v[Q];
+        if (j.x_glu) {
+            // MoeGateRule::ClampedGlu (larql-compute/src/pipeline/moe.rs:88-92): g = min(g, L); u = clamp(u, -L, L);
+            // (u + 1) * (g * sigmoid(alpha * g))   (activations past the row end are zeros: they stay zero)
+            const float2_t u = in[s].u[Q];
+            const float L = j.glu_limit, al = j.glu_alpha;
+            const float g0 = fminf(v.x, L), g1 = fminf(v.y, L);
+            const float u0 = u.x < -L ? -L : (u.x > L ? L : u.x), u1 = u.y < -L ? -L : (u.y > L ? L : u.y);
+            v.x = (u0 + 1.0f) * (g0 * (1.0f / (1.0f + expf(-(g0 * al)))));
+            v.y = (u1 + 1.0f) * (g1 * (1.0f / (1.0f + expf(-(g1 * al)))));
+        }
+        if (scaled) { v.x *= wq; v.y *= wq; }  // the expert's routing weight rides in its activation
+        const float mx = wave_max_nonneg(fmaxf(fabsf(v.x), fabsf(v.y)));
+        // mx = f * 2^ex, f in [0.5, 1): the exponent field less 126 (zero, subnormal, infinite and NaN maxima end at the clamps)
+        const int ef = (int)((__builtin_bit_cast(uint32_t, mx) >> 23) & 0xFFu);
+        ex[s] = (ef == 0 || ef == 255) ? (ef == 0 && mx > 0.f ? -100 : 0) : max(-100, min(100, ef - 126));
+        const float to_int = __builtin_bit_cast(float, (uint32_t)(127 + 23 - ex[s]) << 23);  // 2^(23 - ex)
+        // balanced base-8 digits: n + 0o44444444 has the unsigned digits d+4 (the top one may reach 8)
+        const uint32_t n0 = (uint32_t)((int)__builtin_rintf(v.x * to_int) + 0x924924), n1 = (uint32_t)((int)__builtin_rintf(v.y * to_int) + 0x924924);
+        // e2m1 codes of -4 .. 3 by unsigned digit, a nibble each: -4 = 0xE, -3 = 0xD, -2 = 0xC, -1 = 0xA, 0, 1 = 2, 2 = 4, 3 = 5 (and 4 = 6)
+        constexpr uint32_t kCodes = 0x5420ACDEu;
+#pragma unroll
+        for (int d = 0; d < 8; d++) {
+            const int sh = 3 * (7 - d);
+            uint32_t c0, c1;
+            if (d == 0) {
+                const uint32_t u0 = n0 >> 21, u1 = n1 >> 21;
+                c0 = u0 == 8u ? 6u : (kCodes >> (4 * u0)) & 15u;
+                c1 = u1 == 8u ? 6u : (kCodes >> (4 * u1)) & 15u;
+            } else {
+                c0 = (kCodes >> (4 * ((n0 >> sh) & 7u))) & 15u;
+                c1 = (kCodes >> (4 * ((n1 >> sh) & 7u))) & 15u;
+            }
+            scratch[s * 512 + d * 64 + lane] = (uint8_t)(c0 | (c1 << 4));  // low nibble first
+        }
+    }
+    asm volatile("" ::: "memory");  // same wavefront: LDS executes its writes before the reads that follow
+    const uint32_t row = t - 8 * half;  // (wraps for the rows of the other token)
+#pragma unroll
+    for (int s = 0; s < kMx4MaxSteps; s++) {
+        if ((uint32_t)s >= cw) continue;
+        if (row < 8) {
+            const u32x4 op = *reinterpret_cast<const u32x4 *>(scratch + s * 512 + row * 64 + 16 * kg);  // K = 32kg .. 32kg+31
+            sq[s].a[0] = (int)op.x; sq[s].a[1] = (int)op.y; sq[s].a[2] = (int)op.z; sq[s].a[3] = (int)op.w;
+            sq[s].scale_a = 125 + ex[s] - 3 * (int)row;  // digit `row` weighs 2^(ex - 23 + 3*(7 - row))
+        }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the scratch is reused by the next token
+}
+
+__device__ __forceinline__ void mx4_clear_steps(Mx4Step (&sq)[kMx4MaxSteps]) {
+#pragma unroll
+    for (int s = 0; s < kMx4MaxSteps; s++) {
+#pragma unroll
+        for (int q = 0; q < 8; q++) sq[s].a[q] = 0;
+        sq[s].scale_a = 127;
+    }
+}
+
+// The operands of every token of a job: token q's eight digit rows are A rows 8(q%2) .. 8(q%2)+7 of operand q/2, so
+// its sums come out in D rows of their own.
+__device__ __forceinline__ void mx4_setup_steps(const GemvJob &j, const Mx4In (&in)[kMx4MaxSteps], Mx4Step (&st)[2][kMx4MaxSteps],
+                                                uint32_t cw, uint32_t lane, uint8_t *scratch) {
     const uint32_t ntok = mx4_tokens(j);
-#pragma unroll
-    for (int g = 0; g < 2; g++) {
-#pragma unroll
-        for (int s = 0; s < kMx4MaxSteps; s++) {
-#pragma unroll
-            for (int q = 0; q < 8; q++) st[g][s].a[q] = 0;
-            st[g][s].scale_a = 127;
-        }
-    }
-    // token q's eight digit rows are A rows 8(q%2) .. 8(q%2)+7 of operand q/2: its sums come out in D rows of their own
-#pragma unroll
-    for (int q = 0; q < kMx4MaxTokens; q++) {
-        if ((uint32_t)q >= ntok) break;
-        int ex[kMx4MaxSteps];
-#pragma unroll
-        for (int s = 0; s < kMx4MaxSteps; s++) {
-            if ((uint32_t)s >= cw) continue;
-            float2_t v = in[s].v[q];
-            if (j.x_glu) {
-                // MoeGateRule::ClampedGlu (larql-compute/src/pipeline/moe.rs:88-92): g = min(g, L); u = clamp(u, -L, L);
-                // (u + 1) * (g * sigmoid(alpha * g))   (activations past the row end are zeros: they stay zero)
-                const float2_t u = in[s].u[q];
-                const float L = j.glu_limit, al = j.glu_alpha;
-                const float g0 = fminf(v.x, L), g1 = fminf(v.y, L);
-                const float u0 = u.x < -L ? -L : (u.x > L ? L : u.x), u1 = u.y < -L ? -L : (u.y > L ? L : u.y);
-                v.x = (u0 + 1.0f) * (g0 * (1.0f / (1.0f + expf(-(g0 * al)))));
-                v.y = (u1 + 1.0f) * (g1 * (1.0f / (1.0f + expf(-(g1 * al)))));
-            }
-            const float mx = wave_max_nonneg(fmaxf(fabsf(v.x), fabsf(v.y)));
-            // mx = f * 2^ex, f in [0.5, 1): the exponent field less 126 (zero, subnormal, infinite and NaN maxima end at the clamps)
-            const int ef = (int)((__builtin_bit_cast(uint32_t, mx) >> 23) & 0xFFu);
-            ex[s] = (ef == 0 || ef == 255) ? (ef == 0 && mx > 0.f ? -100 : 0) : max(-100, min(100, ef - 126));
-            const float to_int = __builtin_bit_cast(float, (uint32_t)(127 + 23 - ex[s]) << 23);  // 2^(23 - ex)
-            // balanced base-8 digits: n + 0o44444444 has the unsigned digits d+4 (the top one may reach 8)
-            const uint32_t n0 = (uint32_t)((int)__builtin_rintf(v.x * to_int) + 0x924924), n1 = (uint32_t)((int)__builtin_rintf(v.y * to_int) + 0x924924);
-            // e2m1 codes of -4 .. 3 by unsigned digit, a nibble each: -4 = 0xE, -3 = 0xD, -2 = 0xC, -1 = 0xA, 0, 1 = 2, 2 = 4, 3 = 5 (and 4 = 6)
-            constexpr uint32_t kCodes = 0x5420ACDEu;
-#pragma unroll
-            for (int d = 0; d < 8; d++) {
-                const int sh = 3 * (7 - d);
-                uint32_t c0, c1;
-                if (d == 0) {
-                    const uint32_t u0 = n0 >> 21, u1 = n1 >> 21;
-                    c0 = u0 == 8u ? 6u : (kCodes >> (4 * u0)) & 15u;
-                    c1 = u1 == 8u ? 6u : (kCodes >> (4 * u1)) & 15u;
-                } else {
-                    c0 = (kCodes >> (4 * ((n0 >> sh) & 7u))) & 15u;
-                    c1 = (kCodes >> (4 * ((n1 >> sh) & 7u))) & 15u;
-                }
-                scratch[s * 512 + d * 64 + lane] = (uint8_t)(c0 | (c1 << 4));  // low nibble first
-            }
-        }
-        asm volatile("" ::: "memory");  // same wavefront: LDS executes its writes before the reads that follow
-        const uint32_t row = t - 8 * (uint32_t)(q & 1);  // (wraps for the rows of the other token)
-        Mx4Step (&sq)[kMx4MaxSteps] = st[q >> 1];
-#pragma unroll
-        for (int s = 0; s < kMx4MaxSteps; s++) {
-            if ((uint32_t)s >= cw) continue;
-            if (row < 8) {
-                const u32x4 op = *reinterpret_cast<const u32x4 *>(scratch + s * 512 + row * 64 + 16 * kg);  // K = 32kg .. 32kg+31
-                sq[s].a[0] = (int)op.x; sq[s].a[1] = (int)op.y; sq[s].a[2] = (int)op.z; sq[s].a[3] = (int)op.w;
-                sq[s].scale_a = 125 + ex[s] - 3 * (int)row;  // digit `row` weighs 2^(ex - 23 + 3*(7 - row))
-            }
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the scratch is reused by the next token
-    }
+    mx4_clear_steps(st[0]);
+    mx4_clear_steps(st[1]);
+    mx4_setup_token<0>(j, false, 1.0f, in, st[0], 0, cw, lane, scratch);
+    if (ntok > 1) mx4_setup_token<1>(j, false, 1.0f, in, st[0], 1, cw, lane, scratch);
+    if (ntok > 2) mx4_setup_token<2>(j, false, 1.0f, in, st[1], 0, cw, lane, scratch);
+    if (ntok > 3) mx4_setup_token<3>(j, false, 1.0f, in, st[1], 1, cw, lane, scratch);
 }
 
 #define LARQL_MX4_WAIT_CASE(CW) case CW: LARQL_WAIT_VMCNT((CW + 1) * (kMx4Stages - 1)); break;
 
 // tiles [tile_a, tile_b) of one job
-__device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a, uint32_t tile_b, uint8_t *lds, uint32_t slot_bytes,
-                                               uint32_t &parity) {
+__device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, const Mx4Sel &sel, uint32_t tile_a, uint32_t tile_b, uint8_t *lds,
+                                               uint32_t slot_bytes, uint32_t &parity) {
     constexpr int NS = kMx4Stages, R = kMx4BatchTiles;
     const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t nw_launch = blockDim.x >> 6;
@@ -1390,8 +1411,8 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
         const uint32_t tl = min(it_tile, tile_b - 1);  // past the end: the last tile again (uniform load counts)
         // wave-uniform 64-bit bases + per-lane 32-bit offsets (the lane's row within the tile, clamped into the matrix)
         const uint32_t rb = tl * 16;
-        const uint8_t *wbase = j.w + (size_t)rb * row_bytes;
-        const uint8_t *sbase = j.aux + (size_t)rb * nb;
+        const uint8_t *wbase = sel.w[0] + (size_t)rb * row_bytes;
+        const uint8_t *sbase = sel.aux[0] + (size_t)rb * nb;
         uint32_t wro = wro_full, sro = sro_full;
         if (rb + 16 > rows) {  // ragged last tile only
             const uint32_t rl = min(jr, rows - 1 - rb);
@@ -1420,9 +1441,12 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
     Mx4Step st[2][kMx4MaxSteps];
     if (working) mx4_setup_steps(j, xin, st, cw, lane, ring + (NS - 1) * slot_bytes);  // (512 bytes per step fit the 1024 of a slot's step)
 
+    // The two partial-sum areas are laid out for this job's own `hw`; the job this workgroup served before may have used
+    // another layout, and its last row sums may still be read by a slower wavefront: wait for everybody before writing.
+    __builtin_amdgcn_s_barrier();
     uint32_t n_use = 0;
     for (uint32_t tb = 0; tb < nt; tb += R) {
-        float *pb = part + parity * (R * 16 * nw_launch * 4);
+        float *pb = part + parity * (R * 16 * nw_launch * hw);
         const uint32_t nbt = min((uint32_t)R, nt - tb);
         if (working) {
             for (uint32_t tl = 0; tl < nbt; tl++) {
@@ -1466,7 +1490,159 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, uint32_t tile_a
             float s = 0.f;
             for (uint32_t w = 0; w < nwork; w++) s += pb[rr * PW + w * hw + h];
             s = dpp_add<0xB1>(s);  // quad_perm [1,0,3,2]
-            if ((h & 1u) == 0 && row_base + rr < rows) ((g_f32wp)(j.out + mx4_out_off(j, h >> 1)))[row_base + rr] = s;
+            const uint32_t row = row_base + rr;
+            if ((h & 1u) == 0 && row < rows) {
+                if (!sel.ok[0]) s = 0.0f;  // an expert outside the bank: no contribution (its stand-in's bytes were read, not used)
+                else if (j.bias) s += ((const GLOBAL_AS float *)sel.bias[0])[(size_t)row * j.bias_step];
+                ((g_f32wp)(j.out + mx4_out_off(j, h >> 1)))[row] = s;
+            }
+        }
+        parity ^= 1u;
+    }
+}
+
+// A job folded over experts (GemvJob::combine_w): row tiles [tile_a, tile_b) of the result, each the sum over the job's
+// `nq` experts of (that expert's 16 weight rows) . (that expert's activation, scaled by its routing weight).  The walk is
+// expert-outermost within a batch of R row tiles: one expert's operands are prepared while its tiles are already on their
+// way, its tiles accumulate into the row tiles' own D registers, then the next expert follows; the D registers hold
+// sum_q w_q * (W_q . act_q) when the batch is written out.  One operand set lives at a time.
+__device__ __forceinline__ void run_mxfp4_fold(const GemvJob &j, const Mx4Sel &sel, uint32_t tile_a, uint32_t tile_b, uint8_t *lds,
+                                               uint32_t slot_bytes, uint32_t &parity) {
+    constexpr int NS = kMx4Stages, R = kMx4BatchTiles;
+    const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t nw_launch = blockDim.x >> 6;
+    const uint32_t jr = lane & 15u, kg = lane >> 4;
+    const uint32_t nq = mx4_tokens(j);
+    constexpr uint32_t hw = 2, hw_sh = 1;  // the digit rows 0-7 of the one live operand: two partial sums per weight row and wavefront
+    const uint32_t nwj = j.rpp, steps = j.cpr, cw = (uint32_t)j.pad, PW = nwj * hw;
+    const uint32_t rows = (uint32_t)j.rows, k = (uint32_t)j.k, nb = k / 32, row_bytes = (uint32_t)j.row_bytes;
+    uint8_t *ring = lds + wv * (NS * slot_bytes);
+    float *part = reinterpret_cast<float *>(lds + nw_launch * (NS * slot_bytes));
+    const uint32_t step0 = wv * cw;
+    const bool working = wv < nwj && step0 < steps;
+
+    uint32_t blk[kMx4MaxSteps];
+    bool valid[kMx4MaxSteps];
+#pragma unroll
+    for (int s = 0; s < kMx4MaxSteps; s++) {
+        const uint32_t b = (step0 + s) * 4 + kg;
+        valid[s] = working && (uint32_t)s < cw && b < nb;
+        blk[s] = min(b, nb - 1);
+    }
+    const uint32_t sc_dw = min((step0 + kg) * 4, nb - 4);
+    uint32_t sc_at[kMx4MaxSteps];
+#pragma unroll
+    for (int s = 0; s < kMx4MaxSteps; s++) sc_at[s] = (16u * s + jr) * 4 + (blk[s] - min((step0 + s) * 4, nb - 4));
+    const uint32_t wro_full = jr * row_bytes, sro_full = jr * nb;
+    const uint32_t nt = tile_b - tile_a;
+    // the order of the virtual tiles: batch of R row tiles, then expert, then row tile of the batch
+    uint32_t it_tb = 0, it_q = 0, it_tl = 0, n_issue = 0;
+    auto issue = [&]() {
+        const uint32_t tl = min(tile_a + it_tb + it_tl, tile_b - 1);  // past the end: the last tile again (uniform load counts)
+        const uint32_t rb = tl * 16;
+        const uint8_t *wq = it_q == 1 ? sel.w[1] : (it_q == 2 ? sel.w[2] : (it_q == 3 ? sel.w[3] : sel.w[0]));
+        const uint8_t *aq = it_q == 1 ? sel.aux[1] : (it_q == 2 ? sel.aux[2] : (it_q == 3 ? sel.aux[3] : sel.aux[0]));
+        const uint8_t *wbase = wq + (size_t)rb * row_bytes;
+        const uint8_t *sbase = aq + (size_t)rb * nb;
+        uint32_t wro = wro_full, sro = sro_full;
+        if (rb + 16 > rows) {
+            const uint32_t rl = min(jr, rows - 1 - rb);
+            wro = rl * row_bytes;
+            sro = rl * nb;
+        }
+        uint8_t *lp = ring + (n_issue % NS) * slot_bytes;
+#pragma unroll
+        for (int s = 0; s < kMx4MaxSteps; s++)
+            if ((uint32_t)s < cw) __builtin_amdgcn_global_load_lds((g_vp)(wbase + (wro + blk[s] * 16)), (lds_vp)(lp + s * 1024), 16, 0, 0);
+        if (lane < 16 * cw) __builtin_amdgcn_global_load_lds((g_vp)(sbase + (sro + sc_dw)), (lds_vp)(lp + cw * 1024), 4, 0, 0);
+        n_issue++;
+        if (it_tb < nt) {  // next virtual tile (stays on the last one once the list is exhausted)
+            const uint32_t nbt = min((uint32_t)R, nt - it_tb);
+            if (++it_tl >= nbt) {
+                it_tl = 0;
+                if (++it_q >= nq) { it_q = 0; it_tb += R; }
+            }
+            if (it_tb >= nt) { it_tb = nt - 1 - ((nt - 1) % R); it_q = nq - 1; it_tl = (nt - 1) % R; }
+        }
+    };
+    Mx4In xin[kMx4MaxSteps];
+#pragma unroll
+    for (int s = 0; s < kMx4MaxSteps; s++)
+        if (working && (uint32_t)s < cw) xin[s] = mx4_load_step(j, step0 + s, lane);
+    if (working)
+        for (int s = 0; s < NS - 1; s++) issue();
+
+    __builtin_amdgcn_s_barrier();  // (the partial-sum areas follow this job's layout: see run_mxfp4_mfma)
+    uint32_t n_use = 0;
+    Mx4Step st[kMx4MaxSteps];
+    for (uint32_t tb = 0; tb < nt; tb += R) {
+        float *pb = part + parity * (R * 16 * nw_launch * hw);
+        const uint32_t nbt = min((uint32_t)R, nt - tb);
+        if (working) {
+            f32x4 D[R];
+#pragma unroll
+            for (int t = 0; t < R; t++) D[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int q = 0; q < kMx4MaxTokens; q++) {
+                if ((uint32_t)q >= nq) break;
+                // this expert's operands; the scratch is the ring slot the next copy will fill (nothing is in flight into it)
+                mx4_clear_steps(st);
+                uint8_t *scratch = ring + ((n_use + NS - 1) % NS) * slot_bytes;
+                if (q == 0) mx4_setup_token<0>(j, true, sel.cw[0], xin, st, 0, cw, lane, scratch);
+                else if (q == 1) mx4_setup_token<1>(j, true, sel.cw[1], xin, st, 0, cw, lane, scratch);
+                else if (q == 2) mx4_setup_token<2>(j, true, sel.cw[2], xin, st, 0, cw, lane, scratch);
+                else mx4_setup_token<3>(j, true, sel.cw[3], xin, st, 0, cw, lane, scratch);
+#pragma unroll
+                for (int tl = 0; tl < R; tl++) {
+                    if ((uint32_t)tl >= nbt) break;
+                    issue();
+                    switch (cw) {
+                        LARQL_MX4_WAIT_CASE(1) LARQL_MX4_WAIT_CASE(2) LARQL_MX4_WAIT_CASE(3) LARQL_MX4_WAIT_CASE(4)
+                    }
+                    asm volatile("" ::: "memory");
+                    const uint8_t *slot = ring + (n_use % NS) * slot_bytes;
+#pragma unroll
+                    for (int s = 0; s < kMx4MaxSteps; s++) {
+                        if ((uint32_t)s < cw) {
+                            const u32x4 qw = *reinterpret_cast<const u32x4 *>(slot + s * 1024 + lane * 16);
+                            uint32_t sc = slot[cw * 1024 + sc_at[s]];
+                            // e8m0 0 is 0.0 here; blocks past the row end do not exist; an expert outside the bank has no weights
+                            const bool live = valid[s] && sc != 0 && sel.ok[q];
+                            sc = valid[s] ? sc : 127u;
+                            i32x8 b = {0, 0, 0, 0, 0, 0, 0, 0};
+                            b[0] = live ? (int)qw.x : 0; b[1] = live ? (int)qw.y : 0; b[2] = live ? (int)qw.z : 0; b[3] = live ? (int)qw.w : 0;
+                            D[tl] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st[s].a, b, D[tl], 4, 4, 0, st[s].scale_a, 0, (int)sc);
+                        }
+                    }
+                    n_use++;
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the slot's reads are done before anything reuses it
+                }
+            }
+#pragma unroll
+            for (int tl = 0; tl < R; tl++) {
+                if ((uint32_t)tl >= nbt) break;
+                if (kg < 2) pb[(tl * 16 + jr) * PW + wv * hw + kg] = (D[tl][0] + D[tl][1]) + (D[tl][2] + D[tl][3]);
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        const uint32_t row_base = (tile_a + tb) * 16;
+        const uint32_t nwork = min(nwj, (steps + cw - 1) / cw);
+        for (uint32_t rr = threadIdx.x >> hw_sh; rr < nbt * 16; rr += blockDim.x >> hw_sh) {
+            const uint32_t h = threadIdx.x & (hw - 1u);
+            float s = 0.f;
+            for (uint32_t w = 0; w < nwork; w++) s += pb[rr * PW + w * hw + h];
+            s = dpp_add<0xB1>(s);  // quad_perm [1,0,3,2]
+            const uint32_t row = row_base + rr;
+            if (h == 0 && row < rows) {
+                if (j.bias) {  // + sum_q w_q * bias_q[row], in selection order
+#pragma unroll
+                    for (int q = 0; q < kMx4MaxTokens; q++)
+                        if ((uint32_t)q < nq && sel.ok[q]) s += sel.cw[q] * ((const GLOBAL_AS float *)sel.bias[q])[(size_t)row * j.bias_step];
+                }
+                ((g_f32wp)j.out)[row] = s;
+            }
         }
         parity ^= 1u;
     }
@@ -2159,7 +2335,7 @@ __device__ __forceinline__ void run_mxfp4(const GemvJob &j, uint32_t p0, uint32_
             }
         }
         __syncthreads();
-        tile_epilogue(part, cpr, tile_rows, j.out, row_base);
+        tile_epilogue(part, cpr, tile_rows, j.out, row_base, j.bias, j.bias_step);
         __syncthreads();
     }
 }
@@ -2274,15 +2450,21 @@ __device__ __forceinline__ void gemv_body(const GemvLaunch &L, float *part) {
     uint32_t ji = lo;
     while (p < p_end) {
         GemvJob j = uniform_job(jobs + ji);
+        bool dead = false;
         if (j.sel) {  // run-time expert selection: one bank of equally shaped matrices
             const uint32_t e = __builtin_amdgcn_readfirstlane(*(const GLOBAL_AS uint32_t *)j.sel);
-            j.w += (size_t)e * j.w_sel_stride;
-            j.aux += (size_t)e * j.aux_sel_stride;
+            dead = j.sel_count != 0 && e >= j.sel_count;  // an id outside the bank: zeros, and no byte of the bank is read
+            j.w += (size_t)(dead ? 0u : e) * j.w_sel_stride;
+            j.aux += (size_t)(dead ? 0u : e) * j.aux_sel_stride;
+            if (j.bias) j.bias += (size_t)(dead ? 0u : e) * j.bias_sel_stride;
         }
         const uint32_t jp_end = j.pass_begin + j.n_pass;
         const uint32_t seg_end = min(p_end, jp_end);
         const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin;
-        if (KIND == KIND_Q4K) run_q4k<U>(j, a, b, part);
+        if (dead) {
+            const uint64_t r0 = (uint64_t)a * j.rpp, r1 = min(j.rows, (uint64_t)b * j.rpp);
+            for (uint64_t r = r0 + threadIdx.x; r < r1; r += blockDim.x) ((g_f32wp)j.out)[r] = 0.0f;
+        } else if (KIND == KIND_Q4K) run_q4k<U>(j, a, b, part);
         else if (KIND == KIND_Q8_0) run_q8_0<U>(j, a, b, part);
         else if (KIND == KIND_MXFP4) run_mxfp4<U>(j, a, b, part);
         else if (KIND == KIND_Q6K) run_q6k<U>(j, a, b, part);
@@ -2411,34 +2593,53 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) gemv_mxfp4_mfma_kernel(Gemv
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
         GemvJob j = uniform_job(jobs + ji);
+        Mx4Sel S;
+#pragma unroll
+        for (int q = 0; q < kMx4MaxTokens; q++) { S.w[q] = j.w; S.aux[q] = j.aux; S.bias[q] = j.bias; S.cw[q] = 1.0f; S.ok[q] = true; }
         if (j.route_logits) {  // the selection itself, by every wavefront for itself (a load and ~200 instructions)
             uint32_t idx[kRouterMaxK];
             float wt[kRouterMaxK];
             const bool writer = j.route_experts && p == j.pass_begin && threadIdx.x < 64;  // (one workgroup opens the job)
-            if (writer) router_select_wave<true>(j.route_logits, j.route_n, j.route_k, j.route_policy, threadIdx.x & 63u, idx, wt);
-            else router_select_wave<false>(j.route_logits, j.route_n, j.route_k, j.route_policy, threadIdx.x & 63u, idx, wt);
+            if (writer) router_select_wave<true>(j.route_logits, j.route_bias, j.route_n, j.route_k, j.route_policy, threadIdx.x & 63u, idx, wt);
+            else router_select_wave<false>(j.route_logits, j.route_bias, j.route_n, j.route_k, j.route_policy, threadIdx.x & 63u, idx, wt);
             uint32_t e = idx[0];
 #pragma unroll
             for (int r = 1; r < kRouterMaxK; r++) e = j.route_rank == (uint32_t)r ? idx[r] : e;
             e = __builtin_amdgcn_readfirstlane(e);
-            j.w += (size_t)e * j.w_sel_stride;
-            j.aux += (size_t)e * j.aux_sel_stride;
+            S.w[0] = j.w + (size_t)e * j.w_sel_stride;
+            S.aux[0] = j.aux + (size_t)e * j.aux_sel_stride;
+            if (j.bias) S.bias[0] = j.bias + (size_t)e * j.bias_sel_stride;
             if (writer && threadIdx.x == 0) {
 #pragma unroll
                 for (int r = 0; r < kRouterMaxK; r++)
                     if ((uint32_t)r < j.route_k) { j.route_experts[r] = idx[r]; j.route_weights[r] = wt[r]; }
             }
-        } else if (j.sel) {  // run-time expert selection: one bank of equally shaped matrices
-            const uint32_t e = __builtin_amdgcn_readfirstlane(*(const GLOBAL_AS uint32_t *)j.sel);
-            j.w += (size_t)e * j.w_sel_stride;
-            j.aux += (size_t)e * j.aux_sel_stride;
+        } else if (j.sel) {  // run-time expert selection: one bank of equally shaped matrices (one expert per activation in a folded job)
+            const uint32_t n_sel = j.combine_w ? mx4_tokens(j) : 1u;
+#pragma unroll
+            for (int q = 0; q < kMx4MaxTokens; q++) {
+                if ((uint32_t)q >= n_sel) break;
+                uint32_t e = __builtin_amdgcn_readfirstlane(((const GLOBAL_AS uint32_t *)j.sel)[q]);
+                S.ok[q] = j.sel_count == 0 || e < j.sel_count;  // an id outside the bank contributes nothing and reads nothing of it
+                e = S.ok[q] ? e : 0u;
+                S.w[q] = j.w + (size_t)e * j.w_sel_stride;
+                S.aux[q] = j.aux + (size_t)e * j.aux_sel_stride;
+                if (j.bias) S.bias[q] = j.bias + (size_t)e * j.bias_sel_stride;
+                if (j.combine_w) {
+                    const float wq = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, ((const GLOBAL_AS float *)j.combine_w)[q])));
+                    S.cw[q] = S.ok[q] ? wq : 0.0f;
+                }
+            }
         }
         const uint32_t seg_end = min(p_end, j.pass_begin + j.n_pass);
         // a tile belongs to the workgroup whose share contains its first cost unit (the job's range opens with its
         // start-up allowance, if it has one)
         const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin, cpt = j.cpt ? j.cpt : j.cpr, su = j.su;
         const uint32_t tile_a = a > su ? (a - su + cpt - 1) / cpt : 0, tile_b = b > su ? (b - su + cpt - 1) / cpt : 0;
-        if (tile_a < tile_b) run_mxfp4_mfma(j, tile_a, tile_b, mx4_lds, L.pad, parity);
+        if (tile_a < tile_b) {
+            if (j.combine_w) run_mxfp4_fold(j, S, tile_a, tile_b, mx4_lds, L.pad, parity);
+            else run_mxfp4_mfma(j, S, tile_a, tile_b, mx4_lds, L.pad, parity);
+        }
         p = seg_end;
         ji++;
     }
@@ -2654,8 +2855,11 @@ bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
         j.pad = (int32_t)cw;       // steps per wavefront
         j.row_bytes = (j.k / 32) * 16;
         const uint64_t tiles = (j.rows + 15) / 16;
-        if (tiles * steps > 0x7FFFFFFFull) return false;
-        j.n_pass = (uint32_t)(tiles * steps);
+        const uint64_t fold = j.combine_w ? std::min<uint64_t>(std::max<uint64_t>(j.batch, 1), kMx4MaxTokens) : 1;  // matrices read per row tile
+        if (tiles * steps * fold > 0x7FFFFFFFull) return false;
+        j.n_pass = (uint32_t)(tiles * steps * fold);
+        j.cpt = fold > 1 ? (uint32_t)(steps * fold) : 0;
+        j.su = 0;
         return true;
     }
     if (j.kind == KIND_Q6K_MFMA) {  // geometry and cost model as for the Q4_K matrix-core kernel
@@ -2826,7 +3030,9 @@ size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
     }
     if (n > 0 && jobs[0].kind == KIND_MXFP4_MFMA) {
         const size_t nw = threads / 64;
-        return nw * kMx4Stages * gemv_launch_param(jobs, n) + 2 * (size_t)kMx4BatchTiles * 16 * nw * (jobs[0].batch > 2 ? 8 : 4) * sizeof(float);
+        uint32_t batch = 1;  // the partial sums per weight row and wavefront follow the largest job (a folded job never needs more than 4)
+        for (size_t i = 0; i < n; i++) batch = std::max(batch, jobs[i].combine_w ? 1u : jobs[i].batch);
+        return nw * kMx4Stages * gemv_launch_param(jobs, n) + 2 * (size_t)kMx4BatchTiles * 16 * nw * (batch > 2 ? 8 : 4) * sizeof(float);
     }
     if (n > 0 && jobs[0].kind == KIND_Q4K_Q8K) {  // rings + one partial per (row, super-block), double-buffered
         const size_t nw = threads / 64;

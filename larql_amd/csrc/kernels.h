@@ -65,6 +65,22 @@ struct GemvJob {
     float *route_weights;
     uint32_t route_n, route_k, route_rank;
     int32_t route_policy;
+    // Optional bias (MoE expert biases; MXFP4 kernels only): out[r] = dot + bias[r * bias_step].  With a run-time
+    // selection the bias row of expert e starts e * bias_sel_stride floats further on.
+    const float *bias;
+    uint64_t bias_sel_stride;
+    uint32_t bias_step;
+    // Experts in the bank: a selected id >= sel_count contributes nothing (the job writes zeros, no bias; in a folded
+    // job that expert's share is dropped) and no byte of the bank is read through it.  0 = unchecked.
+    uint32_t sel_count;
+    // Optional fold over experts (MXFP4 matrix-core kernel, MoE down projection of one token): when `combine_w` is set
+    // the job's `batch` activations (x, x + x_stride, x + x_off[..]) belong to `batch` <= 4 DIFFERENT experts
+    // sel[0..batch) of the bank, and the single result row is sum_q combine_w[q] * (W_{sel[q]} . act_q + bias_{sel[q]}):
+    // activation q is scaled by its weight before it meets the matrix, so the sum forms in the accumulators.
+    const float *combine_w;
+    // Optional router bias [route_n], added to route_logits before the selection (it changes which experts win).
+    const float *route_bias;
+    uint64_t pad3;
 };
 static_assert(sizeof(GemvJob) % 16 == 0, "the descriptor is a whole number of 16-byte words (moe_plan_kernel stores it that way)");
 
@@ -122,15 +138,15 @@ uint32_t q4k_gemm_splits(uint32_t rows, uint32_t hidden, uint32_t seq, uint32_t 
 hipError_t split_bf16_launch(hipStream_t s, const float *x, size_t n, uint16_t *hi, uint16_t *lo, int *any_lo);
 
 // MoE helpers
-hipError_t router_select_launch(hipStream_t s, const float *logits, uint32_t tokens, uint32_t n_experts, uint32_t k, int policy,
-                                uint32_t *experts, float *weights);
+hipError_t router_select_launch(hipStream_t s, const float *logits, const float *bias, uint32_t tokens, uint32_t n_experts, uint32_t k,
+                                int policy, uint32_t *experts, float *weights);
 hipError_t moe_plan_launch(hipStream_t s, const uint32_t *experts, uint32_t slots, uint32_t k, uint32_t n_experts, const GemvJob &tg,
                            const GemvJob &tu, const GemvJob &td, uint64_t gu_w_stride, uint64_t gu_s_stride, uint64_t dn_w_stride,
                            uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, bool fused, uint32_t group, GemvJob *gu_table, uint32_t *gu_hdr,
                            GemvJob *dn_table, uint32_t *dn_hdr);
 hipError_t clamped_glu_interleaved_launch(hipStream_t s, const float *gu, float *h, size_t n, float limit, float alpha);
 hipError_t clamped_glu_launch(hipStream_t s, const float *g, const float *u, float *h, size_t n, float limit, float alpha);
-hipError_t weighted_sum_launch(hipStream_t s, const float *d, const float *weights, float *out, uint32_t tokens, uint32_t k,
-                               uint32_t hidden);
+hipError_t weighted_sum_launch(hipStream_t s, const float *d, const float *weights, const uint32_t *experts, uint32_t n_experts, float *out,
+                               uint32_t tokens, uint32_t k, uint32_t hidden);
 
 }  // namespace larql

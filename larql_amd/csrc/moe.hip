@@ -9,13 +9,13 @@
 namespace larql {
 
 // router::select for every token: one wavefront per token (router.h).
-__global__ void __launch_bounds__(64) router_select_kernel(const float *__restrict__ logits, uint32_t n_experts, uint32_t k,
-                                                           int policy, uint32_t *__restrict__ experts,
+__global__ void __launch_bounds__(64) router_select_kernel(const float *__restrict__ logits, const float *__restrict__ bias, uint32_t n_experts,
+                                                           uint32_t k, int policy, uint32_t *__restrict__ experts,
                                                            float *__restrict__ weights) {
     const uint32_t t = blockIdx.x, lane = threadIdx.x;
     uint32_t sel_idx[kRouterMaxK];
     float sel_w[kRouterMaxK];
-    router_select_wave(logits + (size_t)t * n_experts, n_experts, k, policy, lane, sel_idx, sel_w);
+    router_select_wave(logits + (size_t)t * n_experts, bias, n_experts, k, policy, lane, sel_idx, sel_w);
     if (lane == 0) {
 #pragma unroll
         for (int r = 0; r < kRouterMaxK; r++)
@@ -51,9 +51,10 @@ __global__ void clamped_glu_interleaved_kernel(const float *__restrict__ gu, flo
 }
 
 // out[t] = sum over the token's k selected experts, in selection order, of w * down-output
-// (larql-compute/src/cpu/ops/moe/forward.rs:266-270).
-__global__ void weighted_sum_kernel(const float *__restrict__ d, const float *__restrict__ weights, float *__restrict__ out,
-                                    uint32_t k, uint32_t hidden) {
+// (larql-compute/src/cpu/ops/moe/forward.rs:266-270).  A slot whose expert id lies outside the bank is skipped
+// (forward.rs:203-208): its rows of `d` were never written and are not read.
+__global__ void weighted_sum_kernel(const float *__restrict__ d, const float *__restrict__ weights, const uint32_t *__restrict__ experts,
+                                    uint32_t n_experts, float *__restrict__ out, uint32_t k, uint32_t hidden) {
     const uint32_t t = blockIdx.y;
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= hidden) return;
@@ -62,13 +63,13 @@ __global__ void weighted_sum_kernel(const float *__restrict__ d, const float *__
         float w[4], v[4];
 #pragma unroll
         for (uint32_t q = 0; q < 4; q++) {
-            const bool in = r0 + q < k;
+            const bool in = r0 + q < k && experts[(size_t)t * k + r0 + q] < n_experts;
             w[q] = in ? weights[(size_t)t * k + r0 + q] : 0.0f;
             v[q] = in ? d[((size_t)t * k + r0 + q) * hidden + i] : 0.0f;
         }
 #pragma unroll
         for (uint32_t q = 0; q < 4; q++)
-            if (r0 + q < k) acc += w[q] * v[q];
+            if (r0 + q < k && experts[(size_t)t * k + r0 + q] < n_experts) acc += w[q] * v[q];
     }
     out[(size_t)t * hidden + i] = acc;
 }
@@ -174,6 +175,7 @@ __global__ void __launch_bounds__(256) moe_plan_kernel(const uint32_t *__restric
             put64(offsetof(GemvJob, x), (uint64_t)(tm.x + x_off));
             put64(offsetof(GemvJob, out), (uint64_t)(tm.out + out_off));
             if (tm.x_glu) put64(offsetof(GemvJob, x_glu), (uint64_t)(tm.x_glu + x_off));
+            if (tm.bias) put64(offsetof(GemvJob, bias), (uint64_t)(tm.bias + (size_t)e * tm.bias_sel_stride));  // this expert's bias row
             put32(offsetof(GemvJob, batch), nb);
             put64(offsetof(GemvJob, x_stride), (uint64_t)(x_by_token ? tok_off(1) : slot_off(1, gs)));
             put64(offsetof(GemvJob, out_stride), (uint64_t)slot_off(1, out_unit));
@@ -215,10 +217,10 @@ hipError_t moe_plan_launch(hipStream_t s, const uint32_t *experts, uint32_t slot
     return hipGetLastError();
 }
 
-hipError_t router_select_launch(hipStream_t s, const float *logits, uint32_t tokens, uint32_t n_experts, uint32_t k, int policy,
-                                uint32_t *experts, float *weights) {
+hipError_t router_select_launch(hipStream_t s, const float *logits, const float *bias, uint32_t tokens, uint32_t n_experts, uint32_t k,
+                                int policy, uint32_t *experts, float *weights) {
     if (tokens == 0) return hipSuccess;
-    hipLaunchKernelGGL(router_select_kernel, dim3(tokens), dim3(64), 0, s, logits, n_experts, k, policy, experts, weights);
+    hipLaunchKernelGGL(router_select_kernel, dim3(tokens), dim3(64), 0, s, logits, bias, n_experts, k, policy, experts, weights);
     return hipGetLastError();
 }
 hipError_t clamped_glu_interleaved_launch(hipStream_t s, const float *gu, float *h, size_t n, float limit, float alpha) {
@@ -231,10 +233,10 @@ hipError_t clamped_glu_launch(hipStream_t s, const float *g, const float *u, flo
     hipLaunchKernelGGL(clamped_glu_kernel, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, s, g, u, h, n, limit, alpha);
     return hipGetLastError();
 }
-hipError_t weighted_sum_launch(hipStream_t s, const float *d, const float *weights, float *out, uint32_t tokens, uint32_t k,
-                               uint32_t hidden) {
+hipError_t weighted_sum_launch(hipStream_t s, const float *d, const float *weights, const uint32_t *experts, uint32_t n_experts, float *out,
+                               uint32_t tokens, uint32_t k, uint32_t hidden) {
     if (tokens == 0 || hidden == 0) return hipSuccess;
-    hipLaunchKernelGGL(weighted_sum_kernel, dim3((hidden + 255) / 256, tokens), dim3(256), 0, s, d, weights, out, k, hidden);
+    hipLaunchKernelGGL(weighted_sum_kernel, dim3((hidden + 255) / 256, tokens), dim3(256), 0, s, d, weights, experts, n_experts, out, k, hidden);
     return hipGetLastError();
 }
 

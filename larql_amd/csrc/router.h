@@ -51,10 +51,11 @@ constexpr int kRouterMaxK = 8;
 // Every lane ends with the same sel_idx / sel_w (entries from k on are 0).  WEIGHTS = false leaves sel_w at 0 (a
 // caller that only needs to know which experts).
 template <bool WEIGHTS = true>
-__device__ __forceinline__ void router_select_wave(const float *logits, uint32_t n_experts, uint32_t k, int policy, uint32_t lane,
+__device__ __forceinline__ void router_select_wave(const float *logits, const float *bias, uint32_t n_experts, uint32_t k, int policy, uint32_t lane,
                                                    uint32_t (&sel_idx)[kRouterMaxK], float (&sel_w)[kRouterMaxK]) {
     const bool has = lane < n_experts;
-    const float l = has ? logits[lane] : 0.0f;
+    // the router bias joins the logit before anything else (MoeLayerWeights::router_bias, larql-compute/src/pipeline/moe.rs:505-508)
+    const float l = has ? (bias ? logits[lane] + bias[lane] : logits[lane]) : 0.0f;
     // orderable key: logit bits made monotone, then ~index so the lower index wins a tie; 0 = absent
     const uint32_t bits = __builtin_bit_cast(uint32_t, l);
     const uint32_t ord = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);

@@ -278,16 +278,39 @@ def test_moe_block_full_size_weight_scaling_and_token_permutation(be, fmt):
     # tokens in another order: the same results, row for row (who shares an expert's read with whom does not matter)
     perm = rng.permutation(T)
     assert np.array_equal(block(X[perm], logits[perm])[0].view(np.uint32), base[perm].view(np.uint32))
-    # one token against the oracle
+    # one token of the 16 against the oracle's block (the four experts it chose, downloaded and renumbered 0..3)
+    def chosen_bank(ids):
+        m = {nm: (np.concatenate([be.d2h(bufs[nm][0] + int(e) * per // 2, per // 2, np.uint8) for e in ids]),
+                  np.concatenate([be.d2h(bufs[nm][1] + int(e) * per // 32, per // 32, np.uint8) for e in ids])) for nm in bufs}
+        return m
     t = 11
-    acc = np.zeros(H, F)
-    for e, wgt in O.router_select(logits[t], k):
-        m = {nm: (be.d2h(bufs[nm][0] + e * per // 2, per // 2, np.uint8), be.d2h(bufs[nm][1] + e * per // 32, per // 32, np.uint8))
-             for nm in bufs}
-        g, u = O.mxfp4_gemv(*m["gate"], X[t], I, H), O.mxfp4_gemv(*m["up"], X[t], I, H)
-        h = np.array([O.clamped_glu(float(a), float(b)) for a, b in zip(g, u)], F)
-        acc = (acc + F(wgt) * O.mxfp4_gemv(*m["down"], h, H, I)).astype(F)
-    assert rel_l2(base[t], acc) < 1e-5
+    sel = O.router_select(logits[t], k)
+    m = chosen_bank([e for e, _ in sel])
+    want = O.moe_block_mxfp4(X[t:t + 1], np.arange(k, dtype=np.uint64)[None], np.array([[w for _, w in sel]], F), m["gate"], m["up"],
+                             m["down"], k, H, I)
+    assert rel_l2(base[t], want[0]) < 1e-5
+    # configs[3] at batch 1 on the same 32-expert bank, with router / gate_up / down biases: selection inside the first
+    # launch, experts and weighted sum folded into the down projection (two launches)
+    rb = rng.standard_normal(E).astype(F)
+    gub = (rng.standard_normal((E, 2 * I)) * 0.5).astype(F)
+    db = (rng.standard_normal((E, H)) * 0.5).astype(F)
+    drb, dgub, ddb = be.to_device(rb), be.to_device(gub), be.to_device(db)
+    bank_b = fmt.Mxfp4Experts(bufs["gate"][0], bufs["gate"][1], bufs["up"][0], bufs["up"][1], bufs["down"][0], bufs["down"][1], E, H, I,
+                              7.0, 1.702, 0, drb, dgub, ddb)
+    for t in (0, 5, 11):
+        dx, dl = be.to_device(X[t]), be.to_device(logits[t])
+        de, dw, do = be.malloc(k * 4), be.malloc(k * 4), be.malloc(H * 4)
+        assert be.dev_moe_mxfp4_routed(bank_b, dx, 1, k, dl, O.NORMALISED_OVER_SELECTED, de, dw, do, ws, wsb)
+        be.synchronize()
+        ex, wt, got = be.d2h(de, k, np.uint32), be.d2h(dw, k, F), be.d2h(do, H, F)
+        sel = O.router_select(logits[t] + rb, k)
+        assert [int(e) for e in ex] == [e for e, _ in sel]
+        m = chosen_bank(ex)
+        want = O.moe_block_mxfp4(X[t:t + 1], np.arange(k, dtype=np.uint64)[None], wt[None], m["gate"], m["up"], m["down"], k, H, I,
+                                 gate_up_bias=gub[ex], down_bias=db[ex])
+        assert rel_l2(got, want[0]) < 1e-5, t
+        for p in (dx, dl, de, dw, do):
+            be.free(p)
     for p, s in bufs.values():
         be.free(p); be.free(s)
     be.free(ws)

@@ -779,55 +779,111 @@ def test_router_select_matches_oracle(be):
     assert not be.dev_router_select(dl, T, 65, 4, 1, de, dw)             # beyond this kernel: refused
 
 
-@pytest.mark.parametrize("T,E,hidden,inter", [(1, 4, 2880, 2880), (16, 8, 2880, 576)])
-def test_moe_mxfp4_block_matches_oracle(be, fmt, T, E, hidden, inter):
-    rng = np.random.default_rng(59 + T)
+def _mx_bank(rng, E, n, kk, sigma=0.02):
+    p, s = O.quantize_mxfp4((rng.standard_normal(E * n * kk) * sigma).astype(F), E * n, kk)
+    return p, s
+
+
+def _moe_case(rng, T, E, hidden, inter, biases, interleaved):
+    """A bank (separate or fused-interleaved), activations, logits and optional biases, on the host."""
+    c = {"T": T, "E": E, "hidden": hidden, "inter": inter, "interleaved": interleaved}
+    gp, gs = _mx_bank(rng, E, inter, hidden)
+    up, us = _mx_bank(rng, E, inter, hidden)
+    c["dp"], c["ds"] = _mx_bank(rng, E, hidden, inter)
+    if interleaved:       # fused region of expert e: row 2r = gate row r, row 2r+1 = up row r
+        G = hidden // 32
+        fp = np.empty((E, 2 * inter, G * 16), np.uint8); fs = np.empty((E, 2 * inter, G), np.uint8)
+        fp[:, 0::2] = gp.reshape(E, inter, G * 16); fp[:, 1::2] = up.reshape(E, inter, G * 16)
+        fs[:, 0::2] = gs.reshape(E, inter, G); fs[:, 1::2] = us.reshape(E, inter, G)
+        c["gp"], c["gs"], c["up"], c["us"] = fp.reshape(-1), fs.reshape(-1), None, None
+    else:
+        c["gp"], c["gs"], c["up"], c["us"] = gp, gs, up, us
+    c["x"] = rng.standard_normal((T, hidden)).astype(F)
+    c["logits"] = rng.standard_normal((T, E)).astype(F)
+    c["rb"] = rng.standard_normal(E).astype(F) if biases else None
+    c["gub"] = (rng.standard_normal((E, 2 * inter)) * 0.5).astype(F) if biases else None
+    c["db"] = (rng.standard_normal((E, hidden)) * 0.5).astype(F) if biases else None
+    return c
+
+
+def _moe_device_bank(be, fmt, c):
+    dev = {n: (be.to_device(c[n]) if c[n] is not None else None) for n in ("gp", "gs", "up", "us", "dp", "ds", "rb", "gub", "db")}
+    bank = fmt.Mxfp4Experts(dev["gp"], dev["gs"], dev["up"], dev["us"], dev["dp"], dev["ds"], c["E"], c["hidden"], c["inter"], 7.0, 1.702,
+                            1 if c["interleaved"] else 0, dev["rb"], dev["gub"], dev["db"])
+    return bank, dev
+
+
+def _moe_oracle(c, experts, weights):
+    return O.moe_block_mxfp4(c["x"], experts, weights, (c["gp"], c["gs"]), None if c["interleaved"] else (c["up"], c["us"]),
+                             (c["dp"], c["ds"]), c["E"], c["hidden"], c["inter"], interleaved=bool(c["interleaved"]),
+                             gate_up_bias=c["gub"], down_bias=c["db"])
+
+
+@pytest.mark.parametrize("T,E,hidden,inter,biases,interleaved", [(1, 4, 2880, 2880, False, 0), (1, 6, 2880, 2880, True, 1), (1, 5, 384, 320, True, 0),
+                                                                 (16, 8, 2880, 576, False, 0), (16, 8, 2880, 576, True, 1), (7, 6, 384, 320, True, 0),
+                                                                 (1, 4, 96, 64, True, 0), (3, 4, 96, 64, True, 1)])
+def test_moe_mxfp4_block_matches_oracle(be, fmt, T, E, hidden, inter, biases, interleaved):
+    """The expert block (gate/up + bias -> ClampedGlu -> down + bias -> weighted sum) against the checker's block, whose
+    composition is pinned on the reference's GPT-OSS fixture; with and without biases, both bank layouts, one token
+    (the down projection folds experts and weighted sum) and several (device-built job lists); 96-wide rows take the
+    kernels without matrix-core support."""
+    rng = np.random.default_rng(59 + T + E)
     k = 4
-
-    def bank(n, kk):
-        p, s = [], []
-        for _ in range(E):
-            w = (rng.standard_normal(n * kk) * 0.02).astype(F)
-            pp, ss = O.quantize_mxfp4(w, n, kk)
-            p.append(pp); s.append(ss)
-        return np.concatenate(p), np.concatenate(s)
-
-    gp, gs = bank(inter, hidden)
-    up, us = bank(inter, hidden)
-    dp, ds = bank(hidden, inter)
-    x = rng.standard_normal((T, hidden)).astype(F)
-    logits = rng.standard_normal((T, E)).astype(F)
-    # oracle: select -> per expert gate/up -> ClampedGlu -> down -> weighted sum in selection order
-    want = np.zeros((T, hidden), F)
-    gw, gsz = inter * (hidden // 32) * 16, inter * (hidden // 32)
-    dwb, dsz = hidden * (inter // 32) * 16, hidden * (inter // 32)
-    for t in range(T):
-        acc = np.zeros(hidden, F)
-        for e, w in O.router_select(logits[t], k):
-            g = O.mxfp4_gemv(gp[e * gw:(e + 1) * gw], gs[e * gsz:(e + 1) * gsz], x[t], inter, hidden)
-            u = O.mxfp4_gemv(up[e * gw:(e + 1) * gw], us[e * gsz:(e + 1) * gsz], x[t], inter, hidden)
-            h = np.array([O.clamped_glu(float(a), float(b)) for a, b in zip(g, u)], F)
-            d = O.mxfp4_gemv(dp[e * dwb:(e + 1) * dwb], ds[e * dsz:(e + 1) * dsz], h, hidden, inter)
-            acc = (acc + F(w) * d).astype(F)
-        want[t] = acc
-    dev = {n: be.to_device(a) for n, a in dict(gp=gp, gs=gs, up=up, us=us, dp=dp, ds=ds, x=x, lg=logits).items()}
+    c = _moe_case(rng, T, E, hidden, inter, biases, interleaved)
+    bank, dev = _moe_device_bank(be, fmt, c)
+    dx, dl = be.to_device(c["x"]), be.to_device(c["logits"])
     de, dw_, do = be.malloc(T * k * 4), be.malloc(T * k * 4), be.malloc(T * hidden * 4)
-    assert be.dev_router_select(dev["lg"], T, E, k, O.NORMALISED_OVER_SELECTED, de, dw_)
-    b = fmt.Mxfp4Experts(dev["gp"], dev["gs"], dev["up"], dev["us"], dev["dp"], dev["ds"], E, hidden, inter, 7.0, 1.702)
     wsb = be.moe_mxfp4_workspace_bytes(T, k, hidden, inter)
     ws = be.malloc(wsb)
-    assert be.dev_moe_mxfp4(b, dev["x"], T, k, de, dw_, do, ws, wsb)
+    # the selection with the router bias, as one call with the block
+    assert be.dev_moe_mxfp4_routed(bank, dx, T, k, dl, O.NORMALISED_OVER_SELECTED, de, dw_, do, ws, wsb)
     be.synchronize()
+    experts, weights = be.d2h(de, (T, k), np.uint32), be.d2h(dw_, (T, k), F)
+    for t in range(T):
+        want_sel = O.router_select(c["logits"][t] + (c["rb"] if biases else 0), k)
+        assert [int(e) for e in experts[t]] == [e for e, _ in want_sel]
+        assert np.allclose(weights[t], [w for _, w in want_sel], rtol=2e-6, atol=0)
+    want = _moe_oracle(c, experts, weights)
     got = be.d2h(do, (T, hidden), F)
     assert rel_l2(got, want) < 1e-5
-    assert not be.dev_moe_mxfp4(b, dev["x"], T, k, de, dw_, do, ws, wsb - 1024)   # short workspace: refused
+    # the block with the routing given: the same bits
+    do2 = be.malloc(T * hidden * 4)
+    assert be.dev_moe_mxfp4(bank, dx, T, k, de, dw_, do2, ws, wsb)
+    be.synchronize()
+    assert np.array_equal(be.d2h(do2, (T, hidden), F).view(np.uint32), got.view(np.uint32))
+    assert not be.dev_moe_mxfp4(bank, dx, T, k, de, dw_, do, ws, wsb - 1024)   # short workspace: refused
     ws2 = be.malloc(wsb + 16)
-    assert not be.dev_moe_mxfp4(b, dev["x"], T, k, de, dw_, do, ws2 + 4, wsb)     # workspace off a 16-byte boundary: refused
+    assert not be.dev_moe_mxfp4(bank, dx, T, k, de, dw_, do, ws2 + 4, wsb)     # workspace off a 16-byte boundary: refused
+
+
+@pytest.mark.parametrize("T,hidden,inter", [(1, 384, 320), (6, 384, 320), (1, 96, 64)])
+def test_moe_mxfp4_expert_id_outside_the_bank_is_skipped(be, fmt, T, hidden, inter):
+    """cpu_moe_forward skips an expert the bank does not have (`moe.experts_gate_up.get(ei)` else return,
+    cpu/ops/moe/forward.rs:203-208): the slot contributes nothing, and no byte beyond the bank is read."""
+    rng = np.random.default_rng(5 + T)
+    E, k = 4, 3
+    c = _moe_case(rng, T, E, hidden, inter, True, 0)
+    bank, dev = _moe_device_bank(be, fmt, c)
+    experts = np.array([rng.permutation(E)[:k] for _ in range(T)], np.uint32)
+    experts[0, 1] = E + 7                        # outside the bank
+    if T > 2:
+        experts[2, 0] = 0xFFFFFFFF
+    weights = rng.random((T, k)).astype(F)
+    dx, de, dw_, do = be.to_device(c["x"]), be.to_device(experts), be.to_device(weights), be.malloc(T * hidden * 4)
+    wsb = be.moe_mxfp4_workspace_bytes(T, k, hidden, inter)
+    ws = be.malloc(wsb)
+    be.h2d(ws, np.full(wsb // 4, np.nan, F))     # whatever a skipped slot leaves unwritten must not reach the output
+    assert be.dev_moe_mxfp4(bank, dx, T, k, de, dw_, do, ws, wsb)
+    be.synchronize()
+    got = be.d2h(do, (T, hidden), F)
+    want = _moe_oracle(c, experts, weights)
+    assert np.isfinite(got).all() and rel_l2(got, want) < 1e-5
 
 
 def test_moe_mxfp4_tokens_sharing_an_expert_equal_single_token_calls(be, fmt):
     """Slots that chose the same expert are served up to four at a time from one read of its weights; a token's result
-    must not depend on who it shared a job with: the 13-token block equals 13 one-token blocks bit for bit."""
+    must not depend on who it shared a job with: the 13-token block equals, bit for bit, the two-token blocks of its
+    neighbouring tokens."""
     rng = np.random.default_rng(83)
     T, E, hidden, inter, k = 13, 6, 384, 320, 4          # 52 slots over 6 experts: full groups, leftovers of one to three, far-apart companions
 
@@ -850,21 +906,20 @@ def test_moe_mxfp4_tokens_sharing_an_expert_equal_single_token_calls(be, fmt):
     assert be.dev_moe_mxfp4(b, dev["x"], T, k, de, dw_, do, ws, wsb)
     be.synchronize()
     got = be.d2h(do, (T, hidden), F)
-    one = be.malloc(hidden * 4)
-    for t in range(T):
+    # every pair of neighbouring tokens as a block of its own: other companions, the same bits; the one-token call folds
+    # the experts inside its down projection (another order of additions) and agrees to rounding
+    two, one = be.malloc(2 * hidden * 4), be.malloc(hidden * 4)
+    for t in range(T - 1):
+        assert be.dev_moe_mxfp4(b, dev["x"] + t * hidden * 4, 2, k, de + t * k * 4, dw_ + t * k * 4, two, ws, wsb)
+        be.synchronize()
+        assert np.array_equal(be.d2h(two, (2, hidden), F), got[t:t + 2]), t
         assert be.dev_moe_mxfp4(b, dev["x"] + t * hidden * 4, 1, k, de + t * k * 4, dw_ + t * k * 4, one, ws, wsb)
         be.synchronize()
-        assert np.array_equal(be.d2h(one, hidden, F), got[t]), t
-    # and the oracle, token 5
-    acc = np.zeros(hidden, F)
-    gw, gsz = inter * (hidden // 32) * 16, inter * (hidden // 32)
-    dwb, dsz = hidden * (inter // 32) * 16, hidden * (inter // 32)
-    for e, w in O.router_select(logits[5], k):
-        g = O.mxfp4_gemv(gp[e * gw:(e + 1) * gw], gs[e * gsz:(e + 1) * gsz], x[5], inter, hidden)
-        u = O.mxfp4_gemv(up[e * gw:(e + 1) * gw], us[e * gsz:(e + 1) * gsz], x[5], inter, hidden)
-        hh = np.array([O.clamped_glu(float(a), float(b_)) for a, b_ in zip(g, u)], F)
-        acc = (acc + F(w) * O.mxfp4_gemv(dp[e * dwb:(e + 1) * dwb], ds[e * dsz:(e + 1) * dsz], hh, hidden, inter)).astype(F)
-    assert rel_l2(got[5], acc) < 1e-5
+        assert rel_l2(be.d2h(one, hidden, F), got[t]) < 2e-6, t
+    # and the oracle
+    experts, weights = be.d2h(de, (T, k), np.uint32), be.d2h(dw_, (T, k), F)
+    want = O.moe_block_mxfp4(x, experts, weights, (gp, gs), (up, us), (dp, ds), E, hidden, inter)
+    assert rel_l2(got, want) < 1e-5
 
 
 @pytest.mark.parametrize("T,E,hidden,inter,interleaved,policy", [(1, 8, 2880, 2880, 0, 1), (1, 8, 2880, 2880, 1, 1), (1, 6, 384, 320, 0, 0),
@@ -913,7 +968,7 @@ def test_moe_mxfp4_routed_equals_select_then_block(be, fmt, T, E, hidden, inter,
 
 def test_moe_mxfp4_job_groups_of_every_size(be, fmt):
     """Experts chosen by 1, 2, 3, 4 and 5 slots: jobs of one, two, three and four tokens and a second job for the
-    fifth.  Every token's result equals its one-token call bit for bit."""
+    fifth.  Every token's result equals, bit for bit, what it is in a two-token block."""
     rng = np.random.default_rng(97)
     E, hidden, inter, k = 6, 384, 320, 2
     picks = [(4, 5)] * 5 + [(0, 3), (1, 3), (1, 2), (2, 3), (2, 3)]
@@ -945,11 +1000,13 @@ def test_moe_mxfp4_job_groups_of_every_size(be, fmt):
     assert be.dev_moe_mxfp4(b, dev["x"], T, k, de, dw_, do, ws, wsb)
     be.synchronize()
     got = be.d2h(do, (T, hidden), F)
-    one = be.malloc(hidden * 4)
-    for t in range(T):
-        assert be.dev_moe_mxfp4(b, dev["x"] + t * hidden * 4, 1, k, de + t * k * 4, dw_ + t * k * 4, one, ws, wsb)
+    two = be.malloc(2 * hidden * 4)
+    for t in range(T - 1):
+        assert be.dev_moe_mxfp4(b, dev["x"] + t * hidden * 4, 2, k, de + t * k * 4, dw_ + t * k * 4, two, ws, wsb)
         be.synchronize()
-        assert np.array_equal(be.d2h(one, hidden, F), got[t]), t
+        assert np.array_equal(be.d2h(two, (2, hidden), F), got[t:t + 2]), t
+    experts, weights = be.d2h(de, (T, k), np.uint32), be.d2h(dw_, (T, k), F)
+    assert rel_l2(got, O.moe_block_mxfp4(x, experts, weights, (gp, gs), (up, us), (dp, ds), E, hidden, inter)) < 1e-5
 
 
 @pytest.mark.parametrize("T,E,hidden,inter", [(1, 4, 2880, 2880), (13, 6, 384, 320), (16, 8, 2880, 576)])
