@@ -160,14 +160,15 @@ int larql_hip_q4k_dual_matvec(larql_hip_ctx *ctx, const uint8_t *q4k_a, size_t a
                               const float *x, size_t x_len, size_t num_rows, size_t hidden,
                               float *out_a, float *out_b, size_t out_len);
 /* QuantMatVec::q4k_matmul — quant_matvec.rs:324-333; q4_common/matmul.rs:20-139.
- * out is [seq_len, num_rows] row-major.  Any zero dimension gives an empty
- * result (OK, nothing written); a bad shape zero-fills out, as the CPU does. */
+ * out is [seq_len, num_rows] row-major; out_len / x_len must be seq*rows / seq*hidden
+ * (else REFUSED_SHAPE).  A zero dimension or a bad shape zero-fills out, as the CPU
+ * does (matmul.rs:89-98): hidden == 0 leaves seq*rows zeros. */
 int larql_hip_q4k_matmul(larql_hip_ctx *ctx, const uint8_t *q4k, size_t q4k_len,
                          const float *x, size_t x_len, size_t num_rows, size_t hidden,
                          size_t seq_len, float *out, size_t out_len);
 /* QuantMatVec::q4k_matvec_topk — quant_matvec.rs:268-277: up to top_k
  * (row, score) pairs by value descending, non-finite scores skipped
- * (lm_head/knn.rs:315-386).  *n_out receives the count. */
+ * (lm_head/knn.rs:315-386).  *n_out receives the count.  top_k up to 16384. */
 int larql_hip_q4k_matvec_topk(larql_hip_ctx *ctx, const uint8_t *q4k, size_t q4k_len,
                               const float *x, size_t x_len, size_t num_rows, size_t hidden,
                               size_t top_k, uint32_t *idx_out, float *score_out, size_t *n_out);
@@ -184,7 +185,7 @@ int larql_hip_q4_matvec(larql_hip_ctx *ctx, const uint8_t *q4, size_t q4_len,
 int larql_hip_q8_0_gemv(larql_hip_ctx *ctx, const uint8_t *blocks, size_t blocks_len,
                         const float *x, size_t x_len, size_t n, size_t k, float *out);
 /* QuantMatVec::quant_matvec — quant_matvec.rs:50-98: format dispatch.
- * Q4_K/Q4_KF -> q4k_matvec, Q4_0 -> quantize_to_q8 + q4_matvec,
+ * Q4_K/Q4_KF -> q4k_matvec, Q6_K -> q6k_matvec, Q4_0 -> quantize_to_q8 + q4_matvec,
  * everything else UNSUPPORTED (as the trait default answers None). */
 int larql_hip_quant_matvec(larql_hip_ctx *ctx, int format, const uint8_t *weights, size_t w_len,
                            const float *x, size_t x_len, size_t num_rows, size_t hidden, float *out);
@@ -225,7 +226,9 @@ int larql_hip_mxfp4_gemv_multi(larql_hip_ctx *ctx, size_t n_mats,
  * (F32, F16, BF16, Q4_K or Q4_0), keep the min(top_k, n_features) largest
  * |score| per position, sorted by |score| descending (ties: lower index
  * first).  idx_out/score_out are [batch, top_k]; *n_out receives the number
- * of hits per position.  LARQL_E_NAN on a NaN score. */
+ * of hits per position.  top_k up to 16384 (top_k_by_abs takes any K; WalkFfn's
+ * default is every feature, larql-inference/src/vindex/walk_ffn/mod.rs:186-190);
+ * above that LARQL_UNSUPPORTED.  LARQL_E_NAN on a NaN score. */
 int larql_hip_gate_knn(larql_hip_ctx *ctx, int format, const uint8_t *gate, size_t gate_len,
                        const float *x, size_t batch, size_t n_features, size_t hidden, size_t top_k,
                        uint32_t *idx_out, float *score_out, size_t *n_out);
@@ -292,10 +295,17 @@ void larql_hip_plan_destroy(larql_hip_ctx *ctx, larql_hip_plan *plan);
 
 /* Scores + top-K by |score| on resident operands (see larql_hip_gate_knn).
  * scores_scratch: [batch, n_features] f32 device buffer (also the full score
- * matrix on return); idx_out/score_out: [batch, top_k] device buffers. */
+ * matrix on return); idx_out/score_out: [batch, top_k] device buffers, of which
+ * the first count_out[b] entries of row b are written (min(top_k, n_features), fewer
+ * when scores are NaN); count_out (device, [batch]) may be NULL.  A NaN score does not
+ * stop the call — it only enqueues — but raises a flag: see larql_hip_dev_take_nan_flag. */
 int larql_hip_dev_gate_knn(larql_hip_ctx *ctx, int format, const void *gate,
                            const float *x, size_t batch, size_t n_features, size_t hidden,
-                           size_t top_k, float *scores_scratch, uint32_t *idx_out, float *score_out);
+                           size_t top_k, float *scores_scratch, uint32_t *idx_out, float *score_out, uint32_t *count_out);
+/* Waits for the context's stream, reports whether the last device-tier gate-KNN / gate walk met a NaN score
+ * (the host tier answers LARQL_E_NAN there, the reference panics: gate_knn/mod.rs:84) and clears the flag.
+ * Every device-tier gate-KNN call clears the flag before its own selection, so the answer belongs to the last one. */
+int larql_hip_dev_take_nan_flag(larql_hip_ctx *ctx, int *flag_out);
 
 /* larql_hip_dev_gate_knn for callers that cannot allocate (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same results as

@@ -91,7 +91,8 @@ SIGNATURES = {
     "larql_hip_plan_run": (ci, [vp, vp]),
     "larql_hip_plan_launch_count": (ci, [vp]),
     "larql_hip_plan_destroy": (None, [vp, vp]),
-    "larql_hip_dev_gate_knn": (ci, [vp, ci, vp, vp, sz, sz, sz, sz, vp, vp, vp]),
+    "larql_hip_dev_gate_knn": (ci, [vp, ci, vp, vp, sz, sz, sz, sz, vp, vp, vp, vp]),
+    "larql_hip_dev_take_nan_flag": (ci, [vp, C.POINTER(ci)]),
     "larql_hip_static_scratch_bytes": (sz, []),
     "larql_hip_dev_gate_knn_static": (ci, [vp, ci, vp, vp, sz, sz, sz, sz, vp, vp, vp]),
     "larql_hip_dev_gate_walk": (ci, [vp, ci, C.POINTER(vp), sz, vp, sz, sz, sz, sz, sz, vp, vp, vp, vp]),

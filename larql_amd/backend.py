@@ -388,8 +388,14 @@ class HipBackend:
         lib.larql_hip_plan_destroy(self._h, plan)
 
     def dev_gate_knn(self, fmt: int, gate: int, x: int, batch: int, n: int, hidden: int, top_k: int, scores: int, idx: int,
-                     val: int) -> bool:
-        return self._some(lib.larql_hip_dev_gate_knn(self._h, fmt, gate, x, batch, n, hidden, top_k, scores, idx, val))
+                     val: int, counts: Optional[int] = None) -> bool:
+        return self._some(lib.larql_hip_dev_gate_knn(self._h, fmt, gate, x, batch, n, hidden, top_k, scores, idx, val, counts))
+
+    def dev_take_nan_flag(self) -> bool:
+        """True if the last device-tier gate-KNN / gate walk met a NaN score (waits for the stream, clears the flag)."""
+        f = C.c_int(0)
+        self._some(lib.larql_hip_dev_take_nan_flag(self._h, C.byref(f)))
+        return bool(f.value)
 
     def static_scratch_bytes(self) -> int:
         return int(lib.larql_hip_static_scratch_bytes())

@@ -500,6 +500,7 @@ size_t larql_hip_q8k_bytes(size_t n) { return q8k_bytes(n); }
 
 int larql_hip_dev_quantize_x_to_q8k(larql_hip_ctx *c, const float *x, size_t n, void *q8k) {
     if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     if (n % 256 != 0) return fail(c, LARQL_REFUSED_SHAPE, "quantize_x_to_q8k: length must be a multiple of 256");
     if (n == 0) return LARQL_OK;
     if (!x || !q8k || ((uintptr_t)x & 15) || ((uintptr_t)q8k & 15)) return LARQL_E_ARG;
@@ -510,10 +511,10 @@ int larql_hip_dev_quantize_x_to_q8k(larql_hip_ctx *c, const float *x, size_t n, 
 
 int larql_hip_quantize_x_to_q8k(larql_hip_ctx *c, const float *x, size_t n, int8_t *qs, float *d, int16_t *sums) {
     if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     if (n % 256 != 0) return fail(c, LARQL_REFUSED_SHAPE, "quantize_x_to_q8k: length must be a multiple of 256");
     if (n == 0) return LARQL_OK;
     if (!x || !qs || !d || !sums) return LARQL_E_ARG;
-    std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipSetDevice(c->device));
     int rc = upload(c, c->x, x, n * 4);
     if (rc) return rc;
@@ -649,9 +650,11 @@ int larql_hip_q4k_matmul(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, c
                          size_t num_rows, size_t hidden, size_t seq_len, float *out, size_t out_len) {
     if (!c) return LARQL_E_ARG;
     std::lock_guard<std::mutex> lk(c->mu);
-    if (num_rows == 0 || hidden == 0 || seq_len == 0) return LARQL_OK;  // Some(vec![]) on the peer
-    if (out_len != seq_len * num_rows || x_len != seq_len * hidden || !out)
+    if (out_len != seq_len * num_rows || x_len != seq_len * hidden || (!out && out_len))
         return fail(c, LARQL_REFUSED_SHAPE, "q4k_matmul: out/x lengths do not match [seq, rows] / [seq, hidden]");
+    // a zero dimension zero-fills whatever `out` there is (kquant_matmul_into, q4_common/matmul.rs:89-92): hidden == 0
+    // with rows and positions leaves seq * rows zeros, the other two leave an empty result
+    if (num_rows == 0 || hidden == 0 || seq_len == 0) { for (size_t i = 0; i < out_len; i++) out[i] = 0.0f; return LARQL_OK; }
     if (hidden % 256 != 0 || q4k_len < num_rows * (hidden / 256) * 144) {
         for (size_t i = 0; i < out_len; i++) out[i] = 0.0f;  // the CPU kernel zero-fills on a bad shape
         return LARQL_OK;
@@ -725,8 +728,8 @@ int larql_hip_q4k_matvec_topk(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_l
     if (!c || !n_out) return LARQL_E_ARG;
     std::lock_guard<std::mutex> lk(c->mu);
     // refusals of the GPU peer (larql-compute-metal/src/trait_impl/quant_matvec.rs:210-215), with this
-    // kernel's own capacity (64) in place of K_TOPK
-    if (top_k == 0 || top_k > 64 || num_rows == 0 || x_len != hidden) return fail(c, LARQL_UNSUPPORTED, "q4k_matvec_topk: refused");
+    // kernel's own capacity (kTopkMaxK) in place of K_TOPK
+    if (top_k == 0 || top_k > kTopkMaxK || num_rows == 0 || x_len != hidden) return fail(c, LARQL_UNSUPPORTED, "q4k_matvec_topk: refused");
     if (!q4k_shape_ok(num_rows, num_rows, x_len, hidden, q4k_len)) return fail(c, LARQL_REFUSED_SHAPE, "q4k_matvec_topk: refused operands");
     if (num_rows > 0xFFFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "q4k_matvec_topk: too many rows");
     if (!q4k || !x || !idx_out || !score_out) return LARQL_E_ARG;
@@ -828,7 +831,10 @@ int larql_hip_quant_matvec(larql_hip_ctx *c, int format, const uint8_t *weights,
         default:
             // Q5_K, I2S, MXFP4 (external scales), the trait's own Q8_0 layout and the
             // float formats answer None through this signature (backend/quant_matvec.rs:58-97).
+        {
+            std::lock_guard<std::mutex> lk(c->mu);
             return fail(c, LARQL_UNSUPPORTED, "quant_matvec: format %d is not served through this entry", format);
+        }
     }
 }
 
@@ -983,7 +989,7 @@ int larql_hip_gate_knn(larql_hip_ctx *c, int format, const uint8_t *gate, size_t
     if (rc) return rc;
     for (size_t b = 0; b < batch; b++) n_out[b] = 0;
     if (batch == 0 || n == 0 || top_k == 0) return LARQL_OK;  // top_k_by_abs: K==0 or no scores -> empty
-    if (top_k > 64) return fail(c, LARQL_UNSUPPORTED, "gate-KNN: top_k above 64 is not served by this kernel");
+    if (top_k > kTopkMaxK) return fail(c, LARQL_UNSUPPORTED, "gate-KNN: top_k above %u is not served by this kernel", kTopkMaxK);
     if (n > 0xFFFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "gate-KNN: too many features");
     if (hidden == 0) return fail(c, LARQL_UNSUPPORTED, "gate-KNN: hidden == 0");
     if (!gate || !x || !idx_out || !score_out) return LARQL_E_ARG;
@@ -1011,12 +1017,14 @@ int larql_hip_gate_knn(larql_hip_ctx *c, int format, const uint8_t *gate, size_t
 
 int larql_hip_malloc(larql_hip_ctx *c, void **dptr, size_t bytes) {
     if (!c || !dptr) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipSetDevice(c->device));
     HIPCHECK(c, hipMalloc(dptr, bytes ? bytes : 1));
     return LARQL_OK;
 }
 int larql_hip_free(larql_hip_ctx *c, void *dptr) {
     if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipSetDevice(c->device));
     HIPCHECK(c, hipStreamSynchronize(c->stream));
     HIPCHECK(c, hipFree(dptr));
@@ -1024,6 +1032,7 @@ int larql_hip_free(larql_hip_ctx *c, void *dptr) {
 }
 int larql_hip_memcpy_h2d(larql_hip_ctx *c, void *dst, const void *src, size_t bytes) {
     if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipSetDevice(c->device));
     HIPCHECK(c, hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, c->stream));
     HIPCHECK(c, hipStreamSynchronize(c->stream));
@@ -1031,6 +1040,7 @@ int larql_hip_memcpy_h2d(larql_hip_ctx *c, void *dst, const void *src, size_t by
 }
 int larql_hip_memcpy_d2h(larql_hip_ctx *c, void *dst, const void *src, size_t bytes) {
     if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipSetDevice(c->device));
     HIPCHECK(c, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, c->stream));
     HIPCHECK(c, hipStreamSynchronize(c->stream));
@@ -1038,18 +1048,21 @@ int larql_hip_memcpy_d2h(larql_hip_ctx *c, void *dst, const void *src, size_t by
 }
 int larql_hip_memset(larql_hip_ctx *c, void *dst, int value, size_t bytes) {
     if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipSetDevice(c->device));
     HIPCHECK(c, hipMemsetAsync(dst, value, bytes, c->stream));
     return LARQL_OK;
 }
 int larql_hip_synchronize(larql_hip_ctx *c) {
     if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipSetDevice(c->device));
     HIPCHECK(c, hipStreamSynchronize(c->stream));
     return LARQL_OK;
 }
 int larql_hip_event_create(larql_hip_ctx *c, void **event) {
     if (!c || !event) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipSetDevice(c->device));
     hipEvent_t e;
     HIPCHECK(c, hipEventCreate(&e));
@@ -1058,17 +1071,20 @@ int larql_hip_event_create(larql_hip_ctx *c, void **event) {
 }
 int larql_hip_event_record(larql_hip_ctx *c, void *event) {
     if (!c || !event) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipEventRecord((hipEvent_t)event, c->stream));
     return LARQL_OK;
 }
 int larql_hip_event_elapsed_ms(larql_hip_ctx *c, void *start, void *stop, float *ms) {
     if (!c || !start || !stop || !ms) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipEventSynchronize((hipEvent_t)stop));
     HIPCHECK(c, hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
     return LARQL_OK;
 }
 int larql_hip_event_destroy(larql_hip_ctx *c, void *event) {
     if (!c || !event) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipEventDestroy((hipEvent_t)event));
     return LARQL_OK;
 }
@@ -1173,21 +1189,42 @@ int larql_hip_dev_matvec(larql_hip_ctx *c, int format, const void *w, const void
     return larql_hip_dev_matvec_batch(c, &j, 1);
 }
 
+// Clears the NaN flag on the stream (a kernel, not a memset node: see zero_words_kernel).
+static int clear_nan_flag(larql_hip_ctx *c) {
+    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, c->stream, (uint32_t *)c->nan_flag, 1u);
+    HIPCHECK(c, hipGetLastError());
+    return LARQL_OK;
+}
+
 int larql_hip_dev_gate_knn(larql_hip_ctx *c, int format, const void *gate, const float *x, size_t batch, size_t n, size_t hidden,
-                           size_t top_k, float *scores_scratch, uint32_t *idx_out, float *score_out) {
+                           size_t top_k, float *scores_scratch, uint32_t *idx_out, float *score_out, uint32_t *count_out) {
     if (!c) return LARQL_E_ARG;
     std::lock_guard<std::mutex> lk(c->mu);
     const int kind = kind_of_format(format);
     int rc = gate_shape_check(c, kind, (size_t)-1, 0, hidden);
     if (rc) return rc;
     if (batch == 0 || n == 0 || top_k == 0) return LARQL_OK;
-    if (top_k > 64 || n > 0xFFFFFFFFull || hidden == 0) return fail(c, LARQL_UNSUPPORTED, "gate-KNN: unsupported size");
+    if (top_k > kTopkMaxK || n > 0xFFFFFFFFull || hidden == 0) return fail(c, LARQL_UNSUPPORTED, "gate-KNN: unsupported size");
     HIPCHECK(c, hipSetDevice(c->device));
-    rc = ensure(c, c->misc, batch * 4 + 64); if (rc) return rc;
+    if (!count_out) { rc = ensure(c, c->misc, batch * 4 + 64); if (rc) return rc; count_out = (uint32_t *)c->misc.p; }
     rc = dev_gate_scores(c, kind, gate, x, batch, n, hidden, scores_scratch);
     if (rc) return rc;
+    rc = clear_nan_flag(c);
+    if (rc) return rc;
     HIPCHECK(c, topk_launch(c->stream, scores_scratch, (uint32_t)batch, (uint32_t)n, (uint32_t)top_k, true, idx_out, score_out,
-                            (uint32_t *)c->misc.p, c->nan_flag, nullptr, 0));
+                            count_out, c->nan_flag, nullptr, 0));
+    return LARQL_OK;
+}
+
+int larql_hip_dev_take_nan_flag(larql_hip_ctx *c, int *flag_out) {
+    if (!c || !flag_out) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    HIPCHECK(c, hipSetDevice(c->device));
+    int v = 0;
+    HIPCHECK(c, hipMemcpyAsync(&v, c->nan_flag, sizeof(int), hipMemcpyDeviceToHost, c->stream));
+    HIPCHECK(c, hipStreamSynchronize(c->stream));
+    *flag_out = v != 0;
+    if (v) { int rc = clear_nan_flag(c); if (rc) return rc; }
     return LARQL_OK;
 }
 
@@ -1252,8 +1289,8 @@ int larql_hip_dev_gate_knn_static(larql_hip_ctx *c, int format, const void *gate
         if (rc) return rc;
         HIPCHECK(c, gemv_launch(c->stream, P.kind, P.L, P.threads, P.grid, P.lds));
     }
-    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, c->stream, (uint32_t *)c->nan_flag, 1u);
-    HIPCHECK(c, hipGetLastError());
+    rc = clear_nan_flag(c);
+    if (rc) return rc;
     HIPCHECK(c, topk_launch(c->stream, scores, (uint32_t)batch, (uint32_t)n, (uint32_t)top_k, true, idx_out, score_out,
                             count_out ? count_out : counts, c->nan_flag, nullptr, 0));
     return LARQL_OK;
@@ -1261,6 +1298,7 @@ int larql_hip_dev_gate_knn_static(larql_hip_ctx *c, int format, const void *gate
 
 int larql_hip_dev_copy(larql_hip_ctx *c, void *dst, const void *src, size_t bytes) {
     if (!c || !src) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     if (bytes % 16 != 0 || ((uintptr_t)src & 15) || ((uintptr_t)dst & 15)) return fail(c, LARQL_REFUSED_SHAPE, "copy: 16-byte granularity");
     HIPCHECK(c, hipSetDevice(c->device));
     const uint32_t grid = (uint32_t)c->cu_count * 8u;
@@ -1272,11 +1310,11 @@ int larql_hip_dev_copy(larql_hip_ctx *c, void *dst, const void *src, size_t byte
 int larql_hip_dev_q4k_gemm(larql_hip_ctx *c, const uint8_t *w, const uint16_t *x_bf16, size_t rows, size_t hidden, size_t seq,
                            float *out) {
     if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     if (rows == 0 || seq == 0 || hidden == 0) return LARQL_OK;
     if (hidden % 256 != 0) return fail(c, LARQL_REFUSED_SHAPE, "q4k_gemm: hidden not a multiple of 256");
     if (rows > 0xFFFFFFFFull || seq > 0xFFFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "q4k_gemm: too large");
     if (!w || !x_bf16 || !out || ((uintptr_t)w & 15) || ((uintptr_t)x_bf16 & 15)) return LARQL_E_ARG;
-    std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipSetDevice(c->device));
     if (getenv("LARQL_HIP_GEMM_BF16")) {  // first formulation (decoded weights split into two bf16 terms), kept for comparison
         HIPCHECK(c, q4k_gemm_launch(c->stream, w, x_bf16, out, (uint32_t)rows, (uint32_t)hidden, (uint32_t)seq, 0));
@@ -1301,6 +1339,7 @@ int larql_hip_dev_q4k_gemm(larql_hip_ctx *c, const uint8_t *w, const uint16_t *x
 int larql_hip_dev_router_select(larql_hip_ctx *c, const float *logits, size_t tokens, size_t n_experts, size_t k, int policy,
                                 uint32_t *experts, float *weights) {
     if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     if (k > n_experts) k = n_experts;  // select(): k.min(logits.len())
     if (tokens == 0 || k == 0) return LARQL_OK;
     if (n_experts > 64 || k > 8) return fail(c, LARQL_UNSUPPORTED, "router_select: at most 64 experts and top-8 on this backend");
@@ -1505,7 +1544,7 @@ int larql_hip_dev_gate_walk(larql_hip_ctx *c, int format, const void *const *gat
     if (rc) return rc;
     if (kind == KIND_Q4_0) return fail(c, LARQL_UNSUPPORTED, "gate_walk: Q4_0 gates go through larql_hip_dev_gate_knn");
     if (n_layers == 0 || batch == 0 || n == 0 || top_k == 0) return LARQL_OK;
-    if (top_k > 64 || n > 0xFFFFFFFFull || hidden == 0 || n_layers * batch > 0x7FFFFFFFull)
+    if (top_k > kTopkMaxK || n > 0xFFFFFFFFull || hidden == 0 || n_layers * batch > 0x7FFFFFFFull)
         return fail(c, LARQL_UNSUPPORTED, "gate_walk: unsupported size");
     if (!gates || !x || !scores_scratch || !idx_out || !score_out) return LARQL_E_ARG;
     HIPCHECK(c, hipSetDevice(c->device));
@@ -1516,6 +1555,8 @@ int larql_hip_dev_gate_walk(larql_hip_ctx *c, int format, const void *const *gat
         push_gate_jobs(jobs, kind, gates[l], x + l * x_layer_stride, batch, n, hidden, scores_scratch + l * batch * n);
     rc = enqueue_jobs(c, jobs);
     if (rc) return rc;
+    rc = clear_nan_flag(c);
+    if (rc) return rc;
     HIPCHECK(c, topk_launch(c->stream, scores_scratch, (uint32_t)(n_layers * batch), (uint32_t)n, (uint32_t)top_k, true, idx_out,
                             score_out, count_out, c->nan_flag, nullptr, 0));
     return LARQL_OK;
@@ -1525,6 +1566,7 @@ int larql_hip_dev_gate_walk(larql_hip_ctx *c, int format, const void *const *gat
 
 int larql_hip_dev_quantize_q4_k(larql_hip_ctx *c, const float *src, size_t n, uint8_t *dst) {
     if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     if (n % 256 != 0) return fail(c, LARQL_REFUSED_SHAPE, "quantize_q4_k: length must be a multiple of 256");
     HIPCHECK(c, hipSetDevice(c->device));
     HIPCHECK(c, quantize_q4_k_launch(c->stream, src, n, dst));
@@ -1532,6 +1574,7 @@ int larql_hip_dev_quantize_q4_k(larql_hip_ctx *c, const float *src, size_t n, ui
 }
 int larql_hip_dev_quantize_q8_0(larql_hip_ctx *c, const float *src, size_t n, uint8_t *dst) {
     if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     if (n % 32 != 0) return fail(c, LARQL_REFUSED_SHAPE, "quantize_q8_0: length must be a multiple of 32");
     HIPCHECK(c, hipSetDevice(c->device));
     HIPCHECK(c, quantize_q8_0_launch(c->stream, src, n, dst));
@@ -1539,6 +1582,7 @@ int larql_hip_dev_quantize_q8_0(larql_hip_ctx *c, const float *src, size_t n, ui
 }
 int larql_hip_dev_quantize_mxfp4(larql_hip_ctx *c, const float *src, size_t rows, size_t k, uint8_t *packed, uint8_t *scales) {
     if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     if (k % 32 != 0) return fail(c, LARQL_REFUSED_SHAPE, "quantize_mxfp4: k must be a multiple of 32");
     HIPCHECK(c, hipSetDevice(c->device));
     HIPCHECK(c, quantize_mxfp4_launch(c->stream, src, rows, k, packed, scales, c->log2_up));
@@ -1546,12 +1590,14 @@ int larql_hip_dev_quantize_mxfp4(larql_hip_ctx *c, const float *src, size_t rows
 }
 int larql_hip_dev_f32_to_bf16(larql_hip_ctx *c, const float *src, size_t n, uint16_t *dst) {
     if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipSetDevice(c->device));
     HIPCHECK(c, f32_to_bf16_launch(c->stream, src, n, dst));
     return LARQL_OK;
 }
 int larql_hip_dev_quantize_q4_0(larql_hip_ctx *c, const float *src, size_t n, uint8_t *dst) {
     if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     if (n % 32 != 0) return fail(c, LARQL_REFUSED_SHAPE, "quantize_q4_0: length must be a multiple of 32");
     HIPCHECK(c, hipSetDevice(c->device));
     HIPCHECK(c, quantize_q4_0_launch(c->stream, src, n, dst));
@@ -1559,12 +1605,14 @@ int larql_hip_dev_quantize_q4_0(larql_hip_ctx *c, const float *src, size_t n, ui
 }
 int larql_hip_dev_quantize_to_q8(larql_hip_ctx *c, const float *src, size_t n, int8_t *q8, float *scales) {
     if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipSetDevice(c->device));
     HIPCHECK(c, quantize_to_q8_launch(c->stream, src, n, q8, scales));
     return LARQL_OK;
 }
 int larql_hip_dev_fill_normal(larql_hip_ctx *c, float *dst, size_t n, uint64_t seed, float sigma) {
     if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipSetDevice(c->device));
     HIPCHECK(c, fill_normal_launch(c->stream, dst, n, seed, sigma));
     return LARQL_OK;

@@ -14,6 +14,8 @@
 // per tile: hi and lo).  LDS rows are padded to 72 elements so the 16 lanes of
 // an operand read hit 16 distinct 16-byte slots.
 #include <hip/hip_runtime.h>
+
+#include <atomic>
 #include <stdint.h>
 #include <stdlib.h>
 
@@ -819,7 +821,7 @@ hipError_t q4k_gemm_f16_launch(hipStream_t s, const uint8_t *w, const uint16_t *
     const bool split = splits > 1 && partial;
     const uint32_t per = split ? (nsb + splits - 1) / splits : nsb, z = split ? (nsb + per - 1) / per : 1;
     if (gemm_pipe_enabled()) {
-        static bool attr_set = false;  // dynamic LDS above 64 KB has to be allowed once per process
+        static std::atomic<bool> attr_set{false};  // dynamic LDS above 64 KB has to be allowed once per process
         if (!attr_set) {
             hipError_t e = hipFuncSetAttribute((const void *)q4k_gemm_pipe_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             if (e != hipSuccess) return e;

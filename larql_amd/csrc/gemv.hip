@@ -19,6 +19,8 @@
 // The arithmetic restates, per format, the reference CPU kernels cited at each
 // routine; only the summation order differs (fp32 accumulate throughout).
 #include <hip/hip_runtime.h>
+
+#include <atomic>
 #include <stdint.h>
 #include <stdlib.h>
 
@@ -3073,7 +3075,7 @@ uint32_t gemv_wgs_per_cu(int kind, uint32_t threads, size_t lds, uint32_t dflt) 
 hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32_t threads, uint32_t grid, size_t lds) {
     switch (kind) {
         case KIND_Q8_0_MFMA: {
-            static bool attr_set_q8 = false;
+            static std::atomic<bool> attr_set_q8{false};
             if (!attr_set_q8) {
                 hipError_t e = hipFuncSetAttribute((const void *)gemv_q8_0_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
                 if (e != hipSuccess) return e;
@@ -3083,7 +3085,7 @@ hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32
             break;
         }
         case KIND_Q4K_BATCH: {
-            static bool attr_set_qb = false;
+            static std::atomic<bool> attr_set_qb{false};
             if (!attr_set_qb) {
                 hipError_t e = hipFuncSetAttribute((const void *)gemv_q4k_batch_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
                 if (e != hipSuccess) return e;
@@ -3093,7 +3095,7 @@ hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32
             break;
         }
         case KIND_BF16_MFMA: {
-            static bool attr_set_bf = false;
+            static std::atomic<bool> attr_set_bf{false};
             if (!attr_set_bf) {
                 hipError_t e = hipFuncSetAttribute((const void *)gemv_bf16_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
                 if (e != hipSuccess) return e;
@@ -3103,7 +3105,7 @@ hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32
             break;
         }
         case KIND_MXFP4_MFMA: {
-            static bool attr_set_mx4 = false;
+            static std::atomic<bool> attr_set_mx4{false};
             if (!attr_set_mx4) {
                 hipError_t e = hipFuncSetAttribute((const void *)gemv_mxfp4_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
                 if (e != hipSuccess) return e;
@@ -3113,7 +3115,7 @@ hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32
             break;
         }
         case KIND_Q4K_MFMA: {
-            static bool attr_set = false;  // dynamic LDS above 64 KB has to be allowed once per process
+            static std::atomic<bool> attr_set{false};  // dynamic LDS above 64 KB has to be allowed once per process
             if (!attr_set) {
                 hipError_t e = hipFuncSetAttribute((const void *)gemv_q4k_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
                 if (e != hipSuccess) return e;
@@ -3123,7 +3125,7 @@ hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32
             break;
         }
         case KIND_Q6K_MFMA: {
-            static bool attr_set = false;  // dynamic LDS above 64 KB has to be allowed once per process
+            static std::atomic<bool> attr_set{false};  // dynamic LDS above 64 KB has to be allowed once per process
             if (!attr_set) {
                 hipError_t e = hipFuncSetAttribute((const void *)gemv_q6k_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
                 if (e != hipSuccess) return e;
@@ -3133,7 +3135,7 @@ hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32
             break;
         }
         case KIND_Q4K_Q8K: {
-            static bool attr_set = false;  // dynamic LDS above 64 KB has to be allowed once per process
+            static std::atomic<bool> attr_set{false};  // dynamic LDS above 64 KB has to be allowed once per process
             if (!attr_set) {
                 hipError_t e = hipFuncSetAttribute((const void *)gemv_q4k_q8k_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
                 if (e != hipSuccess) return e;

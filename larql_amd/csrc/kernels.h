@@ -107,7 +107,7 @@ hipError_t copy_launch(hipStream_t stream, const void *src, void *dst, size_t by
 hipError_t read_launch(hipStream_t stream, const void *src, uint32_t *sink, size_t bytes, uint32_t grid);
 
 // top-K by |score| (or by value) over rows of a [batch, n] score matrix
-constexpr uint32_t kTopkMaxK = 64;  // winners the selection kernel orders per row
+constexpr uint32_t kTopkMaxK = 16384;  // winners the selection kernel orders per row (above 64: a bitonic sort in LDS, 8 bytes per winner)
 hipError_t topk_launch(hipStream_t stream, const float *scores, uint32_t batch, uint32_t n, uint32_t k,
                        bool by_abs, uint32_t *idx_out, float *val_out, uint32_t *count_out, int *nan_flag,
                        void *workspace, size_t workspace_bytes);

@@ -28,6 +28,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "kernels.h"
 
 namespace larql {
@@ -93,10 +95,14 @@ __device__ __forceinline__ uint64_t make_key(float s, uint32_t idx, int *nan_fla
 constexpr int kTopkCached = 16;  // rounds of 64 scores per wavefront held in registers
 constexpr int kTopkCandidates = kTopkThreads;  // candidates of the short way: one per thread
 
-template <bool BY_ABS, bool CACHED>
+// LARGE (K above 64, up to kTopkMaxK): the selection is the same radix select; the winners are gathered into a
+// power-of-two array in dynamic LDS (`cap` keys, zero-padded) and ordered by a bitonic sort of the whole workgroup.
+template <bool BY_ABS, bool CACHED, bool LARGE>
 __global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restrict__ scores, uint32_t n, uint32_t k,
                                                             uint32_t *__restrict__ idx_out, float *__restrict__ val_out,
-                                                            uint32_t *__restrict__ count_out, int *nan_flag) {
+                                                            uint32_t *__restrict__ count_out, int *nan_flag, uint32_t cap) {
+    static_assert(!(LARGE && CACHED), "the candidate short cut bounds 64 winners only");
+    extern __shared__ __attribute__((aligned(16))) uint64_t big[];  // LARGE: cap keys
     __shared__ uint32_t hist[256];
     __shared__ uint32_t wave_ties[kTopkWaves];
     __shared__ uint64_t winners[64];
@@ -132,6 +138,8 @@ __global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restr
     };
 
     if (tid < 64) winners[tid] = 0;
+    if (LARGE)
+        for (uint32_t i = tid; i < cap; i += kTopkThreads) big[i] = 0;
     if (tid == 0) { sh_prefix = 0; sh_need = k; sh_nwin = 0; sh_ncand = 0; }
     if (CACHED) {
         // ---- short way for a row held in registers.  The 64 groups of 16 lanes each own a slice of the row; the
@@ -259,10 +267,34 @@ __global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restr
         }
         if (in) {
             const uint32_t pos = atomicAdd(&sh_nwin, 1u);
-            if (pos < 64) winners[pos] = key;
+            if (LARGE) { if (pos < cap) big[pos] = key; }
+            else if (pos < 64) winners[pos] = key;
         }
     }, nullptr);
     __syncthreads();
+    if (LARGE) {
+        // bitonic sort of the cap keys, descending (the padding keys 0 sink to the end): log2(cap)*(log2(cap)+1)/2 rounds of
+        // cap/2 compare-exchanges; thread t's pair in a round with distance j is (i, i+j), i = t with a 0 inserted at bit log2(j)
+        for (uint32_t size = 2; size <= cap; size <<= 1) {
+            for (uint32_t jd = size >> 1; jd > 0; jd >>= 1) {
+                for (uint32_t t = tid; t < (cap >> 1); t += kTopkThreads) {
+                    const uint32_t lo = 2 * t - (t & (jd - 1)), hi = lo + jd;
+                    const bool desc = (lo & size) == 0;
+                    const uint64_t a = big[lo], b = big[hi];
+                    if ((a < b) == desc) { big[lo] = b; big[hi] = a; }
+                }
+                __syncthreads();
+            }
+        }
+        const uint32_t nw = min(min(sh_nwin, cap), k);
+        for (uint32_t i = tid; i < nw; i += kTopkThreads) {
+            const uint32_t idx = ~(uint32_t)big[i];
+            idx_out[(size_t)row * k + i] = idx;
+            val_out[(size_t)row * k + i] = s[idx];
+        }
+        if (tid == 0) count_out[row] = nw;
+        return;
+    }
     if (wave == 0) {
         const uint64_t top = sort_desc(winners[lane], lane);
         const bool valid = top != 0 && lane < k;
@@ -281,8 +313,26 @@ size_t topk_workspace_bytes(uint32_t, uint32_t, uint32_t) { return 0; }
 hipError_t topk_launch(hipStream_t stream, const float *scores, uint32_t batch, uint32_t n, uint32_t k, bool by_abs,
                        uint32_t *idx_out, float *val_out, uint32_t *count_out, int *nan_flag, void *, size_t) {
     if (batch == 0) return hipSuccess;
+    if (k > kTopkMaxK) return hipErrorInvalidValue;
+    if (k > 64 && n > 64) {
+        // more than 64 winners: ordered in LDS (room for the next power of two above min(k, n) keys)
+        uint32_t cap = 128;
+        while (cap < k && cap < n) cap <<= 1;
+        const size_t lds = (size_t)cap * sizeof(uint64_t);
+        static std::atomic<bool> attr_abs{false}, attr_val{false};
+        std::atomic<bool> &flag = by_abs ? attr_abs : attr_val;
+        if (!flag) {  // dynamic LDS above 64 KB has to be allowed once per process
+            const void *fn = by_abs ? (const void *)topk_kernel<true, false, true> : (const void *)topk_kernel<false, false, true>;
+            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kTopkMaxK * sizeof(uint64_t)));
+            if (e != hipSuccess) return e;
+            flag = true;
+        }
+        if (by_abs) hipLaunchKernelGGL((topk_kernel<true, false, true>), dim3(batch), dim3(kTopkThreads), lds, stream, scores, n, k, idx_out, val_out, count_out, nan_flag, cap);
+        else hipLaunchKernelGGL((topk_kernel<false, false, true>), dim3(batch), dim3(kTopkThreads), lds, stream, scores, n, k, idx_out, val_out, count_out, nan_flag, cap);
+        return hipGetLastError();
+    }
     const bool cached = n <= (uint32_t)(kTopkWaves * 64 * kTopkCached);
-#define LARQL_TOPK(ABS, C) hipLaunchKernelGGL((topk_kernel<ABS, C>), dim3(batch), dim3(kTopkThreads), 0, stream, scores, n, k, idx_out, val_out, count_out, nan_flag)
+#define LARQL_TOPK(ABS, C) hipLaunchKernelGGL((topk_kernel<ABS, C, false>), dim3(batch), dim3(kTopkThreads), 0, stream, scores, n, k, idx_out, val_out, count_out, nan_flag, 0u)
     if (by_abs) { if (cached) LARQL_TOPK(true, true); else LARQL_TOPK(true, false); }
     else { if (cached) LARQL_TOPK(false, true); else LARQL_TOPK(false, false); }
 #undef LARQL_TOPK

@@ -130,7 +130,13 @@ def test_q4k_dual_and_matmul(be):
     out = be.q4k_matmul(qa, X, rows, cols, seq)
     want = O.q4k_matmul(qa, X, rows, cols, seq)
     assert rel_l2(out, want.reshape(-1)) < TOL
-    assert be.q4k_matmul(qa, X, rows, cols, 0).size == 0 or True
+    # zero dimensions (kquant_matmul_into, matmul.rs:89-92): no positions / no rows -> an empty result; hidden == 0 with
+    # rows and positions -> seq * rows zeros; lengths that do not describe [seq, rows] / [seq, hidden] are refused
+    assert be.q4k_matmul(qa, X[:0], rows, cols, 0).size == 0
+    assert be.q4k_matmul(qa[:0], X, 0, cols, seq).size == 0
+    z = be.q4k_matmul(qa[:0], X[:, :0], rows, 0, seq)
+    assert z is not None and z.size == seq * rows and not z.any()
+    assert be.q4k_matmul(qa, X, rows, cols, 0) is None          # x brings 5 positions, seq says 0
     # shape error zero-fills like the CPU kernel
     bad = be.q4k_matmul(qa[:-1], X, rows, cols, seq)
     assert bad is not None and not bad.any()
@@ -456,8 +462,14 @@ def test_q4_0_q8_matvec_and_quant_matvec_dispatch(be, fmt):
     assert rel_l2(got2, want) < TOL
     qk = O.quantize_q4_k(w)
     assert rel_l2(be.quant_matvec(fmt.FMT_Q4_K, qk, x, rows, hidden), O.q4k_matvec(qk, x, rows, hidden)) < TOL
-    for f in (fmt.FMT_Q8_0, fmt.FMT_Q6_K, fmt.FMT_MXFP4, fmt.FMT_F32, fmt.FMT_I2S):
-        assert be.quant_matvec(f, qk, x, rows, hidden) is None
+    # Q6_K is routed to q6k_matvec (quant_matvec.rs:66-68)
+    q6 = O.quantize_q6_k(w)
+    assert rel_l2(be.quant_matvec(fmt.FMT_Q6_K, q6, x, rows, hidden), O.q6k_matvec(q6, x, rows, hidden)) < TOL
+    assert be.quant_matvec(fmt.FMT_Q6_K, qk, x, rows, hidden) is None      # Q4_K bytes are too short for Q6_K rows: refused
+    # the trait's own Q8_0 layout, Q5_K, MXFP4 (external scales), the float formats and I2S answer None through this signature
+    for f in (fmt.FMT_Q8_0, fmt.FMT_Q5_K, fmt.FMT_MXFP4, fmt.FMT_BF16, fmt.FMT_F16, fmt.FMT_F32, fmt.FMT_I2S):
+        for bytes_ in (qk, q6, w):
+            assert be.quant_matvec(f, bytes_, x, rows, hidden) is None
 
 
 # ------------------------------------------------------------------ gate-KNN
@@ -557,7 +569,8 @@ def test_gate_knn_edge_cases(be, fmt):
     hits = be.gate_knn(fmt.FMT_F32, g[:10], x, 10, hidden, 64)   # K > N -> all N
     assert len(hits) == 10
     assert be.gate_knn(fmt.FMT_F32, g, x, n, hidden, 0) == []     # K == 0 -> empty
-    assert be.gate_knn(fmt.FMT_F32, g, x, n, hidden, 65) is None  # beyond the kernel's capacity: refused
+    assert len(be.gate_knn(fmt.FMT_F32, g, x, n, hidden, 65)) == 65  # above 64: served (ordered in LDS)
+    assert be.gate_knn(fmt.FMT_F32, g, x, n, hidden, 16385) is None  # beyond the kernel's capacity: refused
     xn = x.copy(); xn[3] = np.nan
     import larql_amd
     with pytest.raises(larql_amd.NanScoreError):
@@ -1110,3 +1123,115 @@ def test_gate_walk_over_layers_equals_per_layer_calls(be, fmt):
         hits = be.gate_knn_batch_hits(fmt.FMT_BF16, gates_h[l], X[0], n, hidden, k)
         for b in range(batch):
             assert [i for i, _ in hits[b]] == [int(v) for v in gi0[l, b]]
+
+
+def test_dev_gate_knn_reports_counts_and_nan(be, fmt):
+    """Device tier: hits per position come back through count_out (top_k above the feature count leaves the tail of a row
+    unwritten, exactly count entries are valid), and a NaN score — a panic in the reference (gate_knn/mod.rs:84),
+    LARQL_E_NAN on the host tier — raises a flag that larql_hip_dev_take_nan_flag reads and clears."""
+    rng = np.random.default_rng(73)
+    n, hidden, k, batch = 40, 256, 64, 3
+    w = (rng.standard_normal((n, hidden)) * 0.02).astype(F)
+    X = rng.standard_normal((batch, hidden)).astype(F)
+    g, x = be.to_device(w), be.to_device(X)
+    sc, idx, val, cnt = be.malloc(batch * n * 4), be.malloc(batch * k * 4), be.malloc(batch * k * 4), be.malloc(batch * 4)
+    assert be.dev_gate_knn(fmt.FMT_F32, g, x, batch, n, hidden, k, sc, idx, val, cnt)
+    assert be.dev_take_nan_flag() is False
+    counts = be.d2h(cnt, batch, np.uint32)
+    assert list(counts) == [n] * batch                                      # K > N: all features, as top_k_by_abs
+    gi, gv = be.d2h(idx, (batch, k), np.uint32), be.d2h(val, (batch, k), F)
+    for b in range(batch):
+        check_hits([(int(i), float(v)) for i, v in zip(gi[b, :n], gv[b, :n])], O.f32_gemv(w, X[b], n, hidden), k)
+    # one NaN activation poisons every score of position 1
+    X[1, 5] = np.nan
+    be.h2d(x, X)
+    assert be.dev_gate_knn(fmt.FMT_F32, g, x, batch, n, hidden, k, sc, idx, val, cnt)
+    assert be.dev_take_nan_flag() is True and be.dev_take_nan_flag() is False   # read once, then clear
+    X[1, 5] = 0.0
+    be.h2d(x, X)
+    assert be.dev_gate_knn(fmt.FMT_F32, g, x, batch, n, hidden, k, sc, idx, val)  # (count_out is optional)
+    assert be.dev_take_nan_flag() is False
+    with pytest.raises(Exception):                                               # host tier: the error code
+        Xn = X.copy(); Xn[0, 0] = np.nan
+        be.gate_knn_batch_hits(fmt.FMT_F32, w, Xn, n, hidden, k)
+
+
+def test_one_context_from_eight_threads(be, fmt):
+    """The trait is Send + Sync and its callers are rayon workers (gate_store.rs:40-45): one context driven from eight
+    threads at once (ctypes releases the GIL during a call), every result checked.  Calls are serialised inside the
+    library; what must hold is that no call sees another call's staging buffers or error text."""
+    import threading
+    rng = np.random.default_rng(79)
+    cases = []
+    for i in range(8):
+        rows, cols = 64 + 37 * i, 256 * (1 + i % 4)
+        w = (rng.standard_normal((rows, cols)) * 0.02).astype(F)
+        x = rng.standard_normal(cols).astype(F)
+        q = O.quantize_q4_k(w)
+        q8 = O.quantize_q8_0(w)
+        cases.append((rows, cols, q, q8, x, O.q4k_matvec(q, x, rows, cols), O.q8_0_gemv(q8, x, rows, cols), O.top_k_by_abs(O.q4k_matvec(q, x, rows, cols), 8)))
+    errors = []
+    start = threading.Barrier(8)
+
+    def work(i):
+        rows, cols, q, q8, x, want4, want8, hits = cases[i]
+        try:
+            start.wait()
+            for rep in range(25):
+                got = be.q4k_matvec(q, x, rows, cols)
+                assert got is not None and rel_l2(got, want4) < TOL
+                got8 = be.q8_0_gemv(q8, x, rows, cols) if cols % 64 == 0 else want8
+                assert rel_l2(got8, want8) < TOL
+                assert be.q4k_matvec(q[:-1], x, rows, cols) is None            # a refusal in the middle of the others' calls
+                h = be.gate_knn(fmt.FMT_Q4_K, q, x, rows, cols, 8)
+                assert sorted(j for j, _ in h) == sorted(j for j, _ in hits)
+        except Exception as e:  # noqa: BLE001 - collected and re-raised in the main thread
+            errors.append((i, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    assert not any(t.is_alive() for t in threads)
+
+
+@pytest.mark.parametrize("n,k", [(10240, 256), (10240, 2048), (10240, 10240), (3000, 65), (3000, 16384), (100, 1000), (70, 65), (16384, 16384)])
+def test_top_k_above_64(be, fmt, n, k):
+    """top_k_by_abs takes any K (gate_knn/mod.rs:50-108) and WalkFfn's default is every feature
+    (larql-inference/src/vindex/walk_ffn/mod.rs:186-190): K = 256, 2048, N and K > N against the oracle's heap —
+    same index set, |score| descending, ties to the lower index."""
+    rng = np.random.default_rng(n + k)
+    hidden = 256
+    w = (rng.standard_normal((n, hidden)) * 0.02).astype(F)
+    w[5] = w[9]; w[17] = -w[9]                       # three equal |scores|
+    x = rng.standard_normal(hidden).astype(F)
+    hits = be.gate_knn(fmt.FMT_F32, w, x, n, hidden, k)
+    scores = be.gate_scores_batch(fmt.FMT_F32, w, x.reshape(1, -1), n, hidden).reshape(-1)
+    m = min(k, n)
+    assert hits is not None and len(hits) == m
+    idx = np.array([i for i, _ in hits]); val = np.array([v for _, v in hits], F)
+    assert np.array_equal(val.view(np.uint32), scores[idx].view(np.uint32))
+    a = np.abs(val)
+    assert np.all(a[:-1] >= a[1:])
+    tie = (a[:-1] == a[1:])
+    assert np.all(idx[:-1][tie] < idx[1:][tie])                                # equal |score|: the lower index first
+    want = O.top_k_by_abs(scores, k)
+    assert sorted(idx.tolist()) == sorted(i for i, _ in want) or abs(abs(want[-1][1]) - a[-1]) <= 1e-5
+    if m == n:
+        assert sorted(idx.tolist()) == list(range(n))
+
+
+def test_top_k_above_64_limits_and_by_value(be, fmt):
+    rng = np.random.default_rng(3)
+    rows, hidden = 5000, 512
+    w = (rng.standard_normal((rows, hidden)) * 0.02).astype(F)
+    x = rng.standard_normal(hidden).astype(F)
+    q = O.quantize_q4_k(w)
+    hits = be.q4k_matvec_topk(q, x, rows, hidden, 300)                          # by value, descending
+    scores = be.q4k_matvec(q, x, rows, hidden)
+    want = O.top_k_sorted(scores, 300)
+    assert [i for i, _ in hits] == [i for i, _ in want]
+    assert be.gate_knn(fmt.FMT_F32, w, x, rows, hidden, 16385) is None           # above the kernel's capacity: the caller's fallback
+    assert be.q4k_matvec_topk(q, x, rows, hidden, 16385) is None
