@@ -184,11 +184,25 @@ int larql_hip_q4_matvec(larql_hip_ctx *ctx, const uint8_t *q4, size_t q4_len,
  * k > 0, k % 32 == 0, x_len == k and blocks_len == n*(k/32)*34 exactly. */
 int larql_hip_q8_0_gemv(larql_hip_ctx *ctx, const uint8_t *blocks, size_t blocks_len,
                         const float *x, size_t x_len, size_t n, size_t k, float *out);
+/* lm_head KNN over a ggml Q8_0 head — larql-vindex/src/index/storage/lm_head/knn.rs:126-185 with top_k_sorted
+ * (:315-386): larql_hip_q8_0_gemv followed by the top_k (<= 16384) largest scores by value, descending, non-finite
+ * scores skipped; the vocabulary's scores stay on the device (1 MB per token for a 262144-row head).  Shape rule of
+ * larql_hip_q8_0_gemv.  *n_out receives the count. */
+int larql_hip_q8_0_gemv_topk(larql_hip_ctx *ctx, const uint8_t *blocks, size_t blocks_len, const float *x, size_t x_len,
+                             size_t n, size_t k, size_t top_k, uint32_t *idx_out, float *score_out, size_t *n_out);
 /* QuantMatVec::quant_matvec — quant_matvec.rs:50-98: format dispatch.
  * Q4_K/Q4_KF -> q4k_matvec, Q6_K -> q6k_matvec, Q4_0 -> quantize_to_q8 + q4_matvec,
  * everything else UNSUPPORTED (as the trait default answers None). */
 int larql_hip_quant_matvec(larql_hip_ctx *ctx, int format, const uint8_t *weights, size_t w_len,
                            const float *x, size_t x_len, size_t num_rows, size_t hidden, float *out);
+
+/* QuantMatVec::quant_matvec_q8_input — quant_matvec.rs:100-151: the activation arrives as Q8 (int8 codes + one f32
+ * scale per 32).  Q4_0 -> q4_matvec; Q4_K / Q4_KF / Q6_K -> dequantise_q8 (quant_matvec.rs:24-39) + the f32 path;
+ * the trait's own Q8_0 layout (q8_matvec: None on the CPU backend too), Q5_K, I2S, MXFP4 and the float formats
+ * UNSUPPORTED. */
+int larql_hip_quant_matvec_q8_input(larql_hip_ctx *ctx, int format, const uint8_t *weights, size_t w_len, const int8_t *q8_x,
+                                    size_t q8_len, const float *q8_scales, size_t n_scales, size_t num_rows, size_t hidden,
+                                    float *out);
 
 /* ---- host tier: dense / MXFP4 gemv (MatMul) -------------------------------- */
 
@@ -203,6 +217,14 @@ int larql_hip_f16_gemv(larql_hip_ctx *ctx, const uint8_t *w_f16, size_t w_len, c
                        size_t n, size_t k, float *out, int force);
 int larql_hip_bf16_gemv(larql_hip_ctx *ctx, const uint8_t *w_bf16, size_t w_len, const float *x, size_t x_len,
                         size_t n, size_t k, float *out, int force);
+/* MatMul::bf16_gemv_multi / f16_gemv_multi — backend/matmul.rs:151-194: several [n_i, k_i] matrices against one
+ * x as ONE submission (groups of up to 8 matrices per launch); every k_i must equal x_len and w_len[i] >= n_i*k_i*2,
+ * any bad matrix refuses the whole batch before anything is written, n_mats == 0 is OK (Some(vec![])); results are
+ * in argument order and bit-identical to the sequential *_gemv_force calls. */
+int larql_hip_bf16_gemv_multi(larql_hip_ctx *ctx, size_t n_mats, const uint8_t *const *w_bf16, const size_t *w_len,
+                              const size_t *n, const size_t *k, const float *x, size_t x_len, float *const *out);
+int larql_hip_f16_gemv_multi(larql_hip_ctx *ctx, size_t n_mats, const uint8_t *const *w_f16, const size_t *w_len,
+                             const size_t *n, const size_t *k, const float *x, size_t x_len, float *const *out);
 /* MatMul::mxfp4_gemv — backend/matmul.rs:220-235: k % 32 == 0, x_len >= k,
  * packed_len >= n*(k/32)*16, scales_len >= n*(k/32). */
 int larql_hip_mxfp4_gemv(larql_hip_ctx *ctx, const uint8_t *packed, size_t packed_len,
@@ -397,6 +419,8 @@ int larql_hip_dev_moe_mxfp4_routed(larql_hip_ctx *ctx, const larql_hip_mxfp4_exp
 /* ---- device tier: encoders (bit-exact with the reference's host encoders) --- */
 /* quantize_q4_k — larql-compute/src/cpu/ops/q4_common/quantize.rs:89-189. */
 int larql_hip_dev_quantize_q4_k(larql_hip_ctx *ctx, const float *src, size_t n, uint8_t *dst);
+/* quantize_q6_k — larql-compute/src/cpu/ops/q4_common/quantize.rs:198-276 (210-byte super-blocks, ggml's planar layout). */
+int larql_hip_dev_quantize_q6_k(larql_hip_ctx *ctx, const float *src, size_t n, uint8_t *dst);
 /* quantize_q8_0 — larql-models/src/quant/ggml/quantize.rs:50-77. */
 int larql_hip_dev_quantize_q8_0(larql_hip_ctx *ctx, const float *src, size_t n, uint8_t *dst);
 /* quantize_mxfp4 — larql-vindex/src/format/vindex3/opplan/exec/weights/load.rs:410-476. */

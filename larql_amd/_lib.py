@@ -66,6 +66,10 @@ SIGNATURES = {
     "larql_hip_q4_matvec": (ci, [vp, vp, sz, vp, sz, vp, sz, sz, sz, vp]),
     "larql_hip_q8_0_gemv": (ci, [vp, vp, sz, vp, sz, sz, sz, vp]),
     "larql_hip_quant_matvec": (ci, [vp, ci, vp, sz, vp, sz, sz, sz, vp]),
+    "larql_hip_quant_matvec_q8_input": (ci, [vp, ci, vp, sz, vp, sz, vp, sz, sz, sz, vp]),
+    "larql_hip_q8_0_gemv_topk": (ci, [vp, vp, sz, vp, sz, sz, sz, sz, vp, vp, C.POINTER(sz)]),
+    "larql_hip_bf16_gemv_multi": (ci, [vp, sz, C.POINTER(vp), C.POINTER(sz), C.POINTER(sz), C.POINTER(sz), vp, sz, C.POINTER(vp)]),
+    "larql_hip_f16_gemv_multi": (ci, [vp, sz, C.POINTER(vp), C.POINTER(sz), C.POINTER(sz), C.POINTER(sz), vp, sz, C.POINTER(vp)]),
     "larql_hip_f32_gemv": (ci, [vp, vp, sz, vp, sz, sz, sz, vp, ci]),
     "larql_hip_f16_gemv": (ci, [vp, vp, sz, vp, sz, sz, sz, vp, ci]),
     "larql_hip_bf16_gemv": (ci, [vp, vp, sz, vp, sz, sz, sz, vp, ci]),
@@ -102,6 +106,7 @@ SIGNATURES = {
     "larql_hip_dev_moe_mxfp4": (ci, [vp, C.POINTER(Mxfp4Experts), vp, sz, sz, vp, vp, vp, vp, sz]),
     "larql_hip_dev_moe_mxfp4_routed": (ci, [vp, C.POINTER(Mxfp4Experts), vp, sz, sz, vp, ci, vp, vp, vp, vp, sz]),
     "larql_hip_dev_quantize_q4_k": (ci, [vp, vp, sz, vp]),
+    "larql_hip_dev_quantize_q6_k": (ci, [vp, vp, sz, vp]),
     "larql_hip_dev_quantize_q8_0": (ci, [vp, vp, sz, vp]),
     "larql_hip_dev_quantize_mxfp4": (ci, [vp, vp, sz, sz, vp, vp]),
     "larql_hip_dev_f32_to_bf16": (ci, [vp, vp, sz, vp]),

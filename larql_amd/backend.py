@@ -224,6 +224,26 @@ class HipBackend:
         ok = self._some(lib.larql_hip_quant_matvec(self._h, fmt, _ptr(w), w.size, _ptr(x), x.size, num_rows, hidden, _ptr(out)))
         return out if ok else None
 
+    def quant_matvec_q8_input(self, fmt: int, weights, q8_x, q8_scales, num_rows: int, hidden: int):
+        """QuantMatVec::quant_matvec_q8_input (backend/quant_matvec.rs:100-151)."""
+        w = _u8(weights)
+        q8 = np.ascontiguousarray(q8_x, dtype=np.int8).reshape(-1)
+        sc = _f32(q8_scales)
+        out = np.empty(num_rows, np.float32)
+        ok = self._some(lib.larql_hip_quant_matvec_q8_input(self._h, fmt, _ptr(w), w.size, _ptr(q8), q8.size, _ptr(sc), sc.size,
+                                                            num_rows, hidden, _ptr(out)))
+        return out if ok else None
+
+    def q8_0_gemv_topk(self, blocks, x, n: int, k: int, top_k: int):
+        """lm_head KNN over a ggml Q8_0 head (lm_head/knn.rs:126-185): [(row, score)] by value descending."""
+        w, x = _u8(blocks), _f32(x)
+        idx = np.empty(max(top_k, 1), np.uint32)
+        val = np.empty(max(top_k, 1), np.float32)
+        cnt = C.c_size_t(0)
+        ok = self._some(lib.larql_hip_q8_0_gemv_topk(self._h, _ptr(w), w.size, _ptr(x), x.size, n, k, top_k, _ptr(idx), _ptr(val),
+                                                     C.byref(cnt)))
+        return [(int(idx[i]), float(val[i])) for i in range(cnt.value)] if ok else None
+
     # -- MatMul ------------------------------------------------------------------------
     def _dense(self, fn, w, x, n, k, force):
         w, x = _u8(w), _f32(x)
@@ -251,13 +271,23 @@ class HipBackend:
     def bf16_gemv_force(self, w_bf16, x, n: int, k: int):
         return self._dense(lib.larql_hip_bf16_gemv, w_bf16, x, n, k, True)
 
+    def _dense_multi(self, fn, weights: Sequence[Tuple[np.ndarray, int, int]], x):
+        m = len(weights)
+        x = _f32(x)
+        ws = [_u8(w[0]) for w in weights]
+        outs = [np.empty(w[1], np.float32) for w in weights]
+        VP, SZ = C.c_void_p * max(m, 1), C.c_size_t * max(m, 1)
+        rc = fn(self._h, m, VP(*[w.ctypes.data for w in ws]), SZ(*[w.size for w in ws]), SZ(*[w[1] for w in weights]),
+                SZ(*[w[2] for w in weights]), _ptr(x), x.size, VP(*[o.ctypes.data for o in outs]))
+        return outs if self._some(rc) else None
+
     def bf16_gemv_multi(self, weights: Sequence[Tuple[np.ndarray, int, int]], x):
-        outs = [self.bf16_gemv_force(w, x, n, k) for (w, n, k) in weights]
-        return None if any(o is None for o in outs) else outs
+        """MatMul::bf16_gemv_multi (backend/matmul.rs:151-170): [(w_bf16, n, k)] against one x, one submission."""
+        return self._dense_multi(lib.larql_hip_bf16_gemv_multi, weights, x)
 
     def f16_gemv_multi(self, weights: Sequence[Tuple[np.ndarray, int, int]], x):
-        outs = [self.f16_gemv_force(w, x, n, k) for (w, n, k) in weights]
-        return None if any(o is None for o in outs) else outs
+        """MatMul::f16_gemv_multi (backend/matmul.rs:172-194)."""
+        return self._dense_multi(lib.larql_hip_f16_gemv_multi, weights, x)
 
     def mxfp4_gemv(self, packed, scales, x, n: int, k: int):
         p, s, x = _u8(packed), _u8(scales), _f32(x)
@@ -434,6 +464,9 @@ class HipBackend:
 
     def dev_quantize_q4_k(self, src: int, n: int, dst: int) -> bool:
         return self._some(lib.larql_hip_dev_quantize_q4_k(self._h, src, n, dst))
+
+    def dev_quantize_q6_k(self, src: int, n: int, dst: int) -> bool:
+        return self._some(lib.larql_hip_dev_quantize_q6_k(self._h, src, n, dst))
 
     def dev_quantize_q8_0(self, src: int, n: int, dst: int) -> bool:
         return self._some(lib.larql_hip_dev_quantize_q8_0(self._h, src, n, dst))

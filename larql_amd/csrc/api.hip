@@ -55,6 +55,8 @@ struct Region {
 
 }  // namespace
 
+constexpr size_t kHostMats = 8;  // matrices one host-tier submission stages (their jobs travel in the kernel arguments)
+
 struct larql_hip_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
@@ -64,7 +66,7 @@ struct larql_hip_ctx {
     std::mutex mu;
     std::string name, info, last_error;
     std::vector<Region> regions;
-    DevBuf w[4], aux[4], x, out, tables[4], misc, scores, q8, q8s;
+    DevBuf w[kHostMats], aux[kHostMats], x, out, tables[4], misc, scores, q8, q8s;
     // pinned staging for job tables: the upload is asynchronous, the event says when a slot may be rewritten
     void *table_host[4] = {nullptr, nullptr, nullptr, nullptr};
     size_t table_host_cap[4] = {0, 0, 0, 0};
@@ -355,9 +357,12 @@ void larql_hip_destroy(larql_hip_ctx *c) {
     (void)hipSetDevice(c->device);
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     for (Region &r : c->regions) (void)hipFree(r.dev);
-    DevBuf *bufs[] = {&c->w[0], &c->w[1], &c->w[2], &c->w[3], &c->aux[0], &c->aux[1], &c->aux[2], &c->aux[3],
-                      &c->x, &c->out, &c->tables[0], &c->tables[1], &c->tables[2], &c->tables[3], &c->misc, &c->scores, &c->q8, &c->q8s};
+    DevBuf *bufs[] = {&c->x, &c->out, &c->tables[0], &c->tables[1], &c->tables[2], &c->tables[3], &c->misc, &c->scores, &c->q8, &c->q8s};
     for (DevBuf *b : bufs) if (b->p) (void)hipFree(b->p);
+    for (size_t i = 0; i < kHostMats; i++) {
+        if (c->w[i].p) (void)hipFree(c->w[i].p);
+        if (c->aux[i].p) (void)hipFree(c->aux[i].p);
+    }
     for (int i = 0; i < 4; i++) {
         if (c->table_host[i]) (void)hipHostFree(c->table_host[i]);
         if (c->table_ev[i]) (void)hipEventDestroy(c->table_ev[i]);
@@ -433,7 +438,7 @@ int larql_hip_get_submission_clock(larql_hip_ctx *c, larql_hip_submission_clock 
 static int host_matvec_multi(larql_hip_ctx *c, int kind, size_t n_mats, const uint8_t *const *w, const size_t *w_len,
                              const uint8_t *const *aux, const size_t *aux_len, const size_t *rows, size_t k,
                              const float *x, size_t x_bytes, float *const *out) {
-    if (n_mats > 4) return fail(c, LARQL_UNSUPPORTED, "at most 4 matrices per host-tier submission");
+    if (n_mats > kHostMats) return fail(c, LARQL_UNSUPPORTED, "at most %zu matrices per host-tier submission", kHostMats);
     HIPCHECK(c, hipSetDevice(c->device));
     std::vector<GemvJob> jobs;
     int rc = upload(c, c->x, x, x_bytes);
@@ -722,21 +727,12 @@ static int topk_download(larql_hip_ctx *c, size_t batch, size_t k, uint32_t *idx
     return LARQL_OK;
 }
 
-int larql_hip_q4k_matvec_topk(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, const float *x, size_t x_len,
-                              size_t num_rows, size_t hidden, size_t top_k, uint32_t *idx_out, float *score_out,
-                              size_t *n_out) {
-    if (!c || !n_out) return LARQL_E_ARG;
-    std::lock_guard<std::mutex> lk(c->mu);
-    // refusals of the GPU peer (larql-compute-metal/src/trait_impl/quant_matvec.rs:210-215), with this
-    // kernel's own capacity (kTopkMaxK) in place of K_TOPK
-    if (top_k == 0 || top_k > kTopkMaxK || num_rows == 0 || x_len != hidden) return fail(c, LARQL_UNSUPPORTED, "q4k_matvec_topk: refused");
-    if (!q4k_shape_ok(num_rows, num_rows, x_len, hidden, q4k_len)) return fail(c, LARQL_REFUSED_SHAPE, "q4k_matvec_topk: refused operands");
-    if (num_rows > 0xFFFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "q4k_matvec_topk: too many rows");
-    if (!q4k || !x || !idx_out || !score_out) return LARQL_E_ARG;
+// matvec + top-K by value with the scores kept on the device (lm_head KNN: lm_head/knn.rs:126-185)
+static int host_matvec_topk(larql_hip_ctx *c, int kind, const uint8_t *w, size_t need, const float *x, size_t x_len, size_t num_rows,
+                            size_t hidden, size_t top_k, uint32_t *idx_out, float *score_out, size_t *n_out) {
     HIPCHECK(c, hipSetDevice(c->device));
-    const size_t need = (hidden / 256) * 144 * num_rows;
     const uint8_t *dw = nullptr;
-    int rc = resolve_weights(c, q4k, need, c->w[0], &dw);
+    int rc = resolve_weights(c, w, need, c->w[0], &dw);
     if (rc) return rc;
     rc = upload(c, c->x, x, x_len * 4);
     if (rc) return rc;
@@ -744,7 +740,7 @@ int larql_hip_q4k_matvec_topk(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_l
     if (rc) return rc;
     rc = ensure(c, c->misc, top_k * 8 + 4 + 64);
     if (rc) return rc;
-    std::vector<GemvJob> jobs{make_job(KIND_Q4K, dw, nullptr, c->x.p, (float *)c->scores.p, num_rows, hidden)};
+    std::vector<GemvJob> jobs{make_job(kind, dw, nullptr, c->x.p, (float *)c->scores.p, num_rows, hidden)};
     Submission sub(c);
     rc = enqueue_jobs(c, jobs);
     if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
@@ -756,6 +752,31 @@ int larql_hip_q4k_matvec_topk(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_l
     rc = sub.finish();
     if (rc) return rc;
     return topk_download(c, 1, top_k, idx_out, score_out, n_out, false);
+}
+
+int larql_hip_q4k_matvec_topk(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, const float *x, size_t x_len,
+                              size_t num_rows, size_t hidden, size_t top_k, uint32_t *idx_out, float *score_out,
+                              size_t *n_out) {
+    if (!c || !n_out) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    // refusals of the GPU peer (larql-compute-metal/src/trait_impl/quant_matvec.rs:210-215), with this
+    // kernel's own capacity (kTopkMaxK) in place of K_TOPK
+    if (top_k == 0 || top_k > kTopkMaxK || num_rows == 0 || x_len != hidden) return fail(c, LARQL_UNSUPPORTED, "q4k_matvec_topk: refused");
+    if (!q4k_shape_ok(num_rows, num_rows, x_len, hidden, q4k_len)) return fail(c, LARQL_REFUSED_SHAPE, "q4k_matvec_topk: refused operands");
+    if (num_rows > 0xFFFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "q4k_matvec_topk: too many rows");
+    if (!q4k || !x || !idx_out || !score_out) return LARQL_E_ARG;
+    return host_matvec_topk(c, KIND_Q4K, q4k, (hidden / 256) * 144 * num_rows, x, x_len, num_rows, hidden, top_k, idx_out, score_out, n_out);
+}
+
+int larql_hip_q8_0_gemv_topk(larql_hip_ctx *c, const uint8_t *blocks, size_t blocks_len, const float *x, size_t x_len, size_t n, size_t k,
+                             size_t top_k, uint32_t *idx_out, float *score_out, size_t *n_out) {
+    if (!c || !n_out) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (k == 0 || k % 32 != 0 || x_len != k || blocks_len != n * (k / 32) * 34)
+        return fail(c, LARQL_REFUSED_SHAPE, "q8_0_gemv_topk: geometry does not describe this pack");
+    if (top_k == 0 || top_k > kTopkMaxK || n == 0 || n > 0xFFFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "q8_0_gemv_topk: refused");
+    if (!blocks || !x || !idx_out || !score_out) return LARQL_E_ARG;
+    return host_matvec_topk(c, KIND_Q8_0, blocks, blocks_len, x, x_len, n, k, top_k, idx_out, score_out, n_out);
 }
 
 int larql_hip_q4_matvec(larql_hip_ctx *c, const uint8_t *q4, size_t q4_len, const int8_t *q8_x, size_t q8_len,
@@ -838,6 +859,35 @@ int larql_hip_quant_matvec(larql_hip_ctx *c, int format, const uint8_t *weights,
     }
 }
 
+int larql_hip_quant_matvec_q8_input(larql_hip_ctx *c, int format, const uint8_t *weights, size_t w_len, const int8_t *q8_x, size_t q8_len,
+                                    const float *q8_scales, size_t n_scales, size_t num_rows, size_t hidden, float *out) {
+    if (!c) return LARQL_E_ARG;
+    switch (format) {
+        case LARQL_FMT_Q4_0:
+            return larql_hip_q4_matvec(c, weights, w_len, q8_x, q8_len, q8_scales, n_scales, num_rows, hidden, out);
+        case LARQL_FMT_Q4_K: case LARQL_FMT_Q4_KF: case LARQL_FMT_Q6_K: {
+            // f32-input kernels: dequantise_q8 first (quant_matvec.rs:24-39), then the f32 path
+            if ((!q8_x && q8_len) || (!q8_scales && n_scales)) return LARQL_E_ARG;
+            const size_t n_blocks = q8_len / 32;
+            if (n_scales < n_blocks) {
+                std::lock_guard<std::mutex> lk(c->mu);
+                return fail(c, LARQL_REFUSED_SHAPE, "quant_matvec_q8_input: %zu scales for %zu blocks", n_scales, n_blocks);
+            }
+            std::vector<float> xf(q8_len);
+            for (size_t b = 0; b < n_blocks; b++)
+                for (size_t j = 0; j < 32; j++) xf[b * 32 + j] = (float)q8_x[b * 32 + j] * q8_scales[b];
+            for (size_t i = n_blocks * 32; i < q8_len; i++) xf[i] = (float)q8_x[i];
+            return larql_hip_quant_matvec(c, format, weights, w_len, xf.data(), xf.size(), num_rows, hidden, out);
+        }
+        default: {
+            // the trait's own Q8_0 layout has no kernel here (as on the CPU backend: q8_matvec -> None); Q5_K, I2S, MXFP4
+            // and the float formats answer None through this signature (quant_matvec.rs:126-150)
+            std::lock_guard<std::mutex> lk(c->mu);
+            return fail(c, LARQL_UNSUPPORTED, "quant_matvec_q8_input: format %d is not served through this entry", format);
+        }
+    }
+}
+
 // ---- host tier: dense / MXFP4 gemv ---------------------------------------------------
 
 static int host_dense_gemv(larql_hip_ctx *c, int kind, const void *w, size_t w_len, const float *x, size_t x_len, size_t n,
@@ -865,6 +915,38 @@ int larql_hip_f16_gemv(larql_hip_ctx *c, const uint8_t *w, size_t w_len, const f
 int larql_hip_bf16_gemv(larql_hip_ctx *c, const uint8_t *w, size_t w_len, const float *x, size_t x_len, size_t n, size_t k,
                         float *out, int force) {
     return host_dense_gemv(c, KIND_BF16, w, w_len, x, x_len, n, k, out, force);
+}
+
+// MatMul::{bf16,f16}_gemv_multi — backend/matmul.rs:151-194: several matrices against one x as one submission (up to
+// kHostMats per launch; more are submitted in groups), results bit-identical to the sequential force gemvs.
+static int host_dense_gemv_multi(larql_hip_ctx *c, int kind, size_t n_mats, const uint8_t *const *w, const size_t *w_len, const size_t *n,
+                                 const size_t *k, const float *x, size_t x_len, float *const *out) {
+    if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (n_mats && (!w || !w_len || !n || !k || !out)) return LARQL_E_ARG;
+    // any one bad matrix refuses the whole batch, before anything is written (larql-compute-metal/src/trait_impl/matmul.rs:97-126)
+    for (size_t i = 0; i < n_mats; i++)
+        if (k[i] != x_len || w_len[i] < n[i] * k[i] * dense_elem_bytes(kind))
+            return fail(c, LARQL_REFUSED_SHAPE, "gemv_multi: matrix %zu refused (k %zu against x.len() %zu, %zu bytes)", i, k[i], x_len, w_len[i]);
+    if (n_mats == 0) return LARQL_OK;  // Some(vec![])
+    if (x_len == 0) { for (size_t i = 0; i < n_mats; i++) for (size_t r = 0; r < n[i]; r++) out[i][r] = 0.0f; return LARQL_OK; }
+    if (!x) return LARQL_E_ARG;
+    for (size_t i = 0; i < n_mats; i += kHostMats) {
+        const size_t jn = std::min(kHostMats, n_mats - i);
+        size_t need[kHostMats];
+        for (size_t t = 0; t < jn; t++) need[t] = n[i + t] * x_len * dense_elem_bytes(kind);
+        int rc = host_matvec_multi(c, kind, jn, w + i, need, nullptr, nullptr, n + i, x_len, x, x_len * 4, out + i);
+        if (rc) return rc;
+    }
+    return LARQL_OK;
+}
+int larql_hip_bf16_gemv_multi(larql_hip_ctx *c, size_t n_mats, const uint8_t *const *w, const size_t *w_len, const size_t *n, const size_t *k,
+                              const float *x, size_t x_len, float *const *out) {
+    return host_dense_gemv_multi(c, KIND_BF16, n_mats, w, w_len, n, k, x, x_len, out);
+}
+int larql_hip_f16_gemv_multi(larql_hip_ctx *c, size_t n_mats, const uint8_t *const *w, const size_t *w_len, const size_t *n, const size_t *k,
+                             const float *x, size_t x_len, float *const *out) {
+    return host_dense_gemv_multi(c, KIND_F16, n_mats, w, w_len, n, k, x, x_len, out);
 }
 
 int larql_hip_mxfp4_gemv_multi(larql_hip_ctx *c, size_t n_mats, const uint8_t *const *packed, const size_t *packed_len,
@@ -1570,6 +1652,15 @@ int larql_hip_dev_quantize_q4_k(larql_hip_ctx *c, const float *src, size_t n, ui
     if (n % 256 != 0) return fail(c, LARQL_REFUSED_SHAPE, "quantize_q4_k: length must be a multiple of 256");
     HIPCHECK(c, hipSetDevice(c->device));
     HIPCHECK(c, quantize_q4_k_launch(c->stream, src, n, dst));
+    return LARQL_OK;
+}
+int larql_hip_dev_quantize_q6_k(larql_hip_ctx *c, const float *src, size_t n, uint8_t *dst) {
+    if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (n % 256 != 0) return fail(c, LARQL_REFUSED_SHAPE, "quantize_q6_k: length must be a multiple of 256");
+    if (n && ((uintptr_t)src & 15)) return fail(c, LARQL_REFUSED_SHAPE, "quantize_q6_k: the source must be 16-byte aligned");
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, quantize_q6_k_launch(c->stream, src, n, dst));
     return LARQL_OK;
 }
 int larql_hip_dev_quantize_q8_0(larql_hip_ctx *c, const float *src, size_t n, uint8_t *dst) {

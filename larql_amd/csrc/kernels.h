@@ -115,6 +115,7 @@ size_t topk_workspace_bytes(uint32_t batch, uint32_t n, uint32_t k);
 
 // encoders and the synthetic data generator
 hipError_t quantize_q4_k_launch(hipStream_t s, const float *src, size_t n, uint8_t *dst);
+hipError_t quantize_q6_k_launch(hipStream_t s, const float *src, size_t n, uint8_t *dst);
 hipError_t quantize_q8_0_launch(hipStream_t s, const float *src, size_t n, uint8_t *dst);
 hipError_t quantize_mxfp4_launch(hipStream_t s, const float *src, size_t rows, size_t k, uint8_t *packed,
                                  uint8_t *scales, const uint8_t *log2_up_table);

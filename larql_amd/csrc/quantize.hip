@@ -18,6 +18,7 @@ __device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(flo
 __device__ __forceinline__ float clampf(float v, float lo, float hi) { return v < lo ? lo : (v > hi ? hi : v); }
 // Rust `as u8` after a clamp: NaN -> 0
 __device__ __forceinline__ uint32_t sat_u8(float v) { return v != v ? 0u : (uint32_t)v; }
+__device__ __forceinline__ int sat_i8(float v) { return v != v ? 0 : (int)v; }
 
 // larql-compute/src/cpu/ops/q4_common/f16.rs:10-41 (truncate, keep subnormals)
 __device__ __forceinline__ uint32_t f32_to_f16_trunc(float val) {
@@ -147,11 +148,58 @@ __global__ void __launch_bounds__(256) quantize_q4_k_kernel(const float *__restr
 }
 
 // ---------------------------------------------------------------------------
+// quantize_q6_k — larql-compute/src/cpu/ops/q4_common/quantize.rs:198-276.
+// One wavefront per 256-element super-block; lane l owns elements 4l..4l+3, all
+// inside the 16-element sub-block l/4.  d = amax / (31*127); sub-block scale =
+// round(sub_max / (31 d)) as i8; code = round(v * (1 / (d * scale))) clamped to
+// -32..31, biased by 32.  The 256 six-bit codes pass through LDS into ggml's
+// planar layout: ql[64h + p] = code[128h + p] & 15 | (code[128h + p + 64] & 15) << 4,
+// qh[32h + l] = the top two bits of codes 128h + l + {0, 32, 64, 96}; then the 16
+// scales and the truncated f16 d (210 bytes, 2-byte aligned).
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) quantize_q6_k_kernel(const float *__restrict__ src, size_t n_sb, uint8_t *__restrict__ dst) {
+    __shared__ uint8_t codes[4][256];
+    const uint32_t lane = threadIdx.x & 63u, wv = threadIdx.x >> 6;
+    const size_t sb = (size_t)blockIdx.x * 4 + wv;
+    if (sb >= n_sb) return;  // (whole wavefronts leave together: no workgroup barrier below)
+    const float4 v = reinterpret_cast<const float4 *>(src + sb * 256)[lane];
+    const float e[4] = {v.x, v.y, v.z, v.w};
+    float sub_max = fmaxf(fmaxf(fabsf(e[0]), fabsf(e[1])), fmaxf(fabsf(e[2]), fabsf(e[3])));
+    sub_max = wave_max_span(sub_max, 4);
+    float amax = sub_max;
+    for (int o = 4; o < 64; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+    const float d = amax / (31.0f * 127.0f);
+    const float scf = d > 0.0f ? sub_max / (31.0f * d) : 0.0f;
+    const int sub_scale = sat_i8(clampf(roundf(scf), -128.0f, 127.0f));
+    const float sc = d * (float)sub_scale;
+    const float inv = fabsf(sc) > 1e-10f ? 1.0f / sc : 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) codes[wv][4 * lane + i] = (uint8_t)(sat_i8(clampf(roundf(e[i] * inv), -32.0f, 31.0f)) + 32);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const uint8_t *c = codes[wv];
+    uint8_t *o = dst + sb * 210;
+    {   // ql bytes 2*lane, 2*lane + 1
+        const uint32_t i0 = 2 * lane, h = i0 >> 6, p = i0 & 63u;
+        const uint32_t b0 = (c[128 * h + p] & 15u) | ((c[128 * h + p + 64] & 15u) << 4);
+        const uint32_t b1 = (c[128 * h + p + 1] & 15u) | ((c[128 * h + p + 65] & 15u) << 4);
+        *reinterpret_cast<uint16_t *>(o + i0) = (uint16_t)(b0 | (b1 << 8));
+    }
+    {   // qh byte `lane`
+        const uint32_t h = lane >> 5, l = lane & 31u, b = 128 * h + l;
+        o[128 + lane] = (uint8_t)(((c[b] >> 4) & 3u) | (((c[b + 32] >> 4) & 3u) << 2) | (((c[b + 64] >> 4) & 3u) << 4) | (((c[b + 96] >> 4) & 3u) << 6));
+    }
+    const int scale_of = __shfl(sub_scale, (int)((lane & 15u) * 4), 64);  // sub-block j lives in lanes 4j..4j+3
+    if (lane < 16) o[192 + lane] = (uint8_t)scale_of;
+    if (lane == 0) *reinterpret_cast<uint16_t *>(o + 208) = (uint16_t)f32_to_f16_trunc(d);
+}
+
+// ---------------------------------------------------------------------------
 // quantize_q8_0 — larql-models/src/quant/ggml/quantize.rs:50-77; and the two
 // Q4_0-path encoders, q4_common/quantize.rs:6-69.  One thread per 32-element
 // block (the fold over |v| is order-independent).
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ int sat_i8(float v) { return v != v ? 0 : (int)v; }
 
 __global__ void quantize_q8_0_kernel(const float *__restrict__ src, size_t n_blocks, uint8_t *__restrict__ dst) {
     const size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -338,6 +386,12 @@ hipError_t quantize_q4_k_launch(hipStream_t s, const float *src, size_t n, uint8
     const size_t n_sb = n / 256;
     if (n_sb == 0) return hipSuccess;
     hipLaunchKernelGGL(quantize_q4_k_kernel, blocks_for(n_sb, 4), dim3(256), 0, s, src, n_sb, dst);
+    return hipGetLastError();
+}
+hipError_t quantize_q6_k_launch(hipStream_t s, const float *src, size_t n, uint8_t *dst) {
+    const size_t n_sb = n / 256;
+    if (n_sb == 0) return hipSuccess;
+    hipLaunchKernelGGL(quantize_q6_k_kernel, blocks_for(n_sb, 4), dim3(256), 0, s, src, n_sb, dst);
     return hipGetLastError();
 }
 hipError_t quantize_q8_0_launch(hipStream_t s, const float *src, size_t n, uint8_t *dst) {

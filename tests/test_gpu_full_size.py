@@ -35,6 +35,21 @@ def q4k_bytes(rows, k):
     return rows * (k // 256) * 144
 
 
+def assert_same_hits_up_to_ties(hits, want, scores):
+    """Both lists by value descending with the same values; indices may differ only inside a run of equal scores (the
+    reference sorts with sort_unstable_by and its heap evicts equal minima in heap order: lm_head/knn.rs:340-383), and
+    this backend puts the lower index first."""
+    hv, wv = np.array([v for _, v in hits], F), np.array([v for _, v in want], F)
+    assert np.array_equal(hv.view(np.uint32), wv.view(np.uint32))
+    hi, wi = [i for i, _ in hits], [i for i, _ in want]
+    assert np.array_equal(scores[hi].view(np.uint32), hv.view(np.uint32)) and len(set(hi)) == len(hi)
+    for v in np.unique(hv[np.array(hi) != np.array(wi)]) if hi != wi else []:
+        run = hv == v
+        assert run.sum() > 1 or v == hv[-1]                  # a tie inside the list, or at its boundary
+        ours = sorted(np.array(hi)[run])
+        assert ours == sorted(np.flatnonzero(scores == v)[:len(ours)])   # the lowest indices of that score
+
+
 def dev_q4k_matrix(be, rows, k, seed):
     n = rows * k
     tmp, w = be.malloc(n * 4), be.malloc(q4k_bytes(rows, k) + 64)
@@ -132,7 +147,38 @@ def test_lm_head_q8_0_full_vocabulary_linearity_and_sampled_rows(be, fmt):
     for r0 in (0, 131072 + 48, n - 64):
         wb = be.d2h(w + r0 * (k // 32) * 34, 64 * (k // 32) * 34, np.uint8)
         assert rel_l2(fx[r0:r0 + 64], O.q8_0_gemv(wb, x, 64, k)) < 2e-5
+    # lm_head KNN at vocabulary size (lm_head/knn.rs:126-185): the fused call on the 713 MB head as a registered region
+    # (no upload per call), against top_k_sorted over the device's own scores
+    wh = be.d2h(w, nb, np.uint8)
     be.free(w)
+    be.register_weight_region(wh)
+    be.seal_weight_regions()
+    for top in (8, 64, 1000):
+        assert_same_hits_up_to_ties(be.q8_0_gemv_topk(wh, x, n, k, top), O.top_k_sorted(fx, top), fx)
+    be.clear_weight_regions()
+
+
+def test_q4k_matvec_topk_at_vocabulary_size(be, fmt):
+    """q4k_matvec_topk (quant_matvec.rs:268-277) over a 262144 x 2560 Q4_K head: by value, descending, against the oracle's
+    top_k_sorted over the full score vector of the same device matvec."""
+    rng = np.random.default_rng(6)
+    n, k = 262144, 2560
+    chunk = 32768
+    wb = np.empty(q4k_bytes(n, k), np.uint8)
+    tmp, wq = be.malloc(chunk * k * 4), be.malloc(q4k_bytes(chunk, k) + 64)
+    for c in range(n // chunk):
+        assert be.dev_fill_normal(tmp, chunk * k, 0x5EED0280 + c, 0.02) and be.dev_quantize_q4_k(tmp, chunk * k, wq)
+        wb[c * q4k_bytes(chunk, k):(c + 1) * q4k_bytes(chunk, k)] = be.d2h(wq, q4k_bytes(chunk, k), np.uint8)
+    be.free(tmp); be.free(wq)
+    x = rng.standard_normal(k).astype(F)
+    be.register_weight_region(wb)
+    be.seal_weight_regions()
+    scores = be.q4k_matvec(wb, x, n, k)
+    r0 = 200000
+    assert rel_l2(scores[r0:r0 + 32], O.q4k_matvec(wb[q4k_bytes(r0, k):q4k_bytes(r0 + 32, k)], x, 32, k)) < 2e-5
+    for top in (1, 8, 64, 4096):
+        assert_same_hits_up_to_ties(be.q4k_matvec_topk(wb, x, n, k, top), O.top_k_sorted(scores, top), scores)
+    be.clear_weight_regions()
 
 
 @pytest.mark.parametrize("gate_fmt", ["bf16", "q4k"])
@@ -196,10 +242,12 @@ def test_gate_walk_full_size_selection_and_order_invariants(be, fmt, gate_fmt):
         be.free(g)
 
 
-def test_prefill_gemm_full_size_exact_scaling_and_token_permutation(be, fmt):
-    """configs[4]: 15360 x 3840 against 512 tokens of bf16 activations."""
-    rows, hidden, seq = 15360, 3840, 512
-    tmp, w = dev_q4k_matrix(be, rows, hidden, 0x5EED0500)
+@pytest.mark.parametrize("rows,hidden", [(15360, 3840), (3840, 15360)])
+def test_prefill_gemm_full_size_exact_scaling_and_token_permutation(be, fmt, rows, hidden):
+    """configs[4]: gate/up 15360 x 3840 and down 3840 x 15360 (the leg that splits K over workgroups and adds the
+    partial slabs in a fixed order) against 512 tokens of bf16 activations."""
+    seq = 512
+    tmp, w = dev_q4k_matrix(be, rows, hidden, 0x5EED0500 + (hidden > rows))
     be.free(tmp)
     rng = np.random.default_rng(5)
     X = rng.standard_normal((seq, hidden)).astype(F)
@@ -224,7 +272,7 @@ def test_prefill_gemm_full_size_exact_scaling_and_token_permutation(be, fmt):
     x4 = O.f32_to_bf16((Xr * F(4.0)).astype(F)).reshape(seq, hidden)
     assert np.array_equal(gemm(x4).view(np.uint32), (base * F(4.0)).view(np.uint32))
     # rows of the product equal the matvec of that token (the reference's contract for q4k_matmul), on a sample
-    r0 = 7168
+    r0 = (rows // 2 - 512) & ~15
     wb = be.d2h(w + r0 * (hidden // 256) * 144, 64 * (hidden // 256) * 144, np.uint8)
     for t in (0, 255, 511):
         want = O.q4k_matvec(wb, Xr[t], 64, hidden)

@@ -163,3 +163,10 @@ def test_device_mxfp4_encoder_on_exact_arithmetic_groups(be):
     finally:
         for p in (src, pk, sc):
             be.free(p)
+
+
+@pytest.mark.parametrize("name", ["q6k_exact_halves", "q6k_f32_header"])
+def test_device_q6k_encoder_on_exact_arithmetic_blocks(be, name):
+    x = kat_inputs(name)
+    got = _device_encode(be, "dev_quantize_q6_k", x, x.size // 256 * 210, x.size)
+    assert got.tobytes().hex() == KATS[name]["hex"]

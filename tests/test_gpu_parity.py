@@ -1235,3 +1235,79 @@ def test_top_k_above_64_limits_and_by_value(be, fmt):
     assert [i for i, _ in hits] == [i for i, _ in want]
     assert be.gate_knn(fmt.FMT_F32, w, x, rows, hidden, 16385) is None           # above the kernel's capacity: the caller's fallback
     assert be.q4k_matvec_topk(q, x, rows, hidden, 16385) is None
+
+
+@pytest.mark.parametrize("seed,scale", [(0, 0.02), (1, 1.0), (2, 1e-4), (3, 30.0)])
+def test_device_q6k_encoder_is_bit_exact(be, seed, scale):
+    """quantize_q6_k (q4_common/quantize.rs:198-276) on the device, byte for byte, incl. all-zero and constant blocks."""
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal(256 * 333) * scale).astype(F)
+    x[:256] = 0
+    x[256:512] = F(0.37 * scale)
+    x[512:528] = 0                      # a zero sub-block: scale 0, reciprocal 0
+    src, dst = be.to_device(x), be.malloc(x.size // 256 * 210)
+    assert be.dev_quantize_q6_k(src, x.size, dst)
+    assert np.array_equal(be.d2h(dst, x.size // 256 * 210, np.uint8), O.quantize_q6_k(x))
+    assert not be.dev_quantize_q6_k(src, 255, dst)
+
+
+def test_q8_0_gemv_topk_keeps_the_scores_on_the_device(be):
+    """lm_head KNN over a ggml Q8_0 head (lm_head/knn.rs:126-185, top_k_sorted :315-386): by value, descending."""
+    rng = np.random.default_rng(41)
+    n, k = 5003, 512
+    w = (rng.standard_normal((n, k)) * 0.02).astype(F)
+    x = rng.standard_normal(k).astype(F)
+    q = O.quantize_q8_0(w)
+    scores = be.q8_0_gemv(q, x, n, k)
+    for top in (1, 8, 64, 500):
+        hits = be.q8_0_gemv_topk(q, x, n, k, top)
+        want = O.top_k_sorted(scores, top)
+        assert [i for i, _ in hits] == [i for i, _ in want]
+        assert np.array_equal(np.array([v for _, v in hits], F).view(np.uint32), scores[[i for i, _ in hits]].view(np.uint32))
+    assert be.q8_0_gemv_topk(q[:-1], x, n, k, 8) is None and be.q8_0_gemv_topk(q, x, n, k, 0) is None
+    assert be.q8_0_gemv_topk(q, x[:-1], n, k, 8) is None
+
+
+def test_quant_matvec_q8_input_dispatch(be, fmt):
+    """QuantMatVec::quant_matvec_q8_input (quant_matvec.rs:100-151)."""
+    rows, hidden = 257, 1024
+    w, x = weights(23, rows, hidden)
+    q8, sc = O.quantize_to_q8(x)
+    q4 = O.quantize_q4_0(w)
+    a = be.quant_matvec_q8_input(fmt.FMT_Q4_0, q4, q8, sc, rows, hidden)
+    assert np.array_equal(a.view(np.uint32), be.q4_matvec(q4, q8, sc, rows, hidden).view(np.uint32))
+    xd = O.dequantise_q8(q8, sc)
+    for f, q in ((fmt.FMT_Q4_K, O.quantize_q4_k(w)), (fmt.FMT_Q6_K, O.quantize_q6_k(w))):
+        got = be.quant_matvec_q8_input(f, q, q8, sc, rows, hidden)
+        assert np.array_equal(got.view(np.uint32), be.quant_matvec(f, q, xd, rows, hidden).view(np.uint32))
+        want = O.q4k_matvec(q, xd, rows, hidden) if f == fmt.FMT_Q4_K else O.q6k_matvec(q, xd, rows, hidden)
+        assert rel_l2(got, want) < TOL
+    for f in (fmt.FMT_Q8_0, fmt.FMT_Q5_K, fmt.FMT_I2S, fmt.FMT_MXFP4, fmt.FMT_BF16, fmt.FMT_F32):
+        assert be.quant_matvec_q8_input(f, q4, q8, sc, rows, hidden) is None
+    assert be.quant_matvec_q8_input(fmt.FMT_Q4_K, O.quantize_q4_k(w), q8, sc[:-1], rows, hidden) is None   # a scale short
+
+
+@pytest.mark.parametrize("half", ["bf16", "f16"])
+def test_dense_gemv_multi_is_one_submission_of_the_single_calls(be, half):
+    """MatMul::{bf16,f16}_gemv_multi (backend/matmul.rs:151-194): results in argument order, bit-identical to the
+    sequential force gemvs; an empty list is Some(vec![]); one bad matrix refuses the whole batch."""
+    rng = np.random.default_rng(43)
+    k = 640
+    x = rng.standard_normal(k).astype(F)
+    shapes = [300, 17, 1024, 5, 64, 999, 128, 256, 33, 700, 2]          # eleven matrices: two launches' worth
+    mats = []
+    for n in shapes:
+        w = (rng.standard_normal((n, k)) * 0.05).astype(F)
+        mats.append((O.f32_to_bf16(w) if half == "bf16" else w.astype(np.float16), n, k))
+    multi = getattr(be, f"{half}_gemv_multi")
+    single = getattr(be, f"{half}_gemv_force")
+    before = be.submission_clock()["submissions"]
+    outs = multi(mats, x)
+    assert be.submission_clock()["submissions"] - before == 2
+    assert outs is not None and len(outs) == len(shapes)
+    for (w, n, _), o in zip(mats, outs):
+        assert np.array_equal(o.view(np.uint32), single(w, x, n, k).view(np.uint32))
+    assert multi([], x) == []
+    bad = list(mats[:3]) + [(mats[3][0][:-1], mats[3][1], k)]
+    assert multi(bad, x) is None
+    assert multi([(mats[0][0], shapes[0], k - 64)], x) is None            # k must equal x.len()
