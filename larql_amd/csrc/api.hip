@@ -311,7 +311,6 @@ int larql_hip_create(larql_hip_ctx **out, int device) {
     larql_hip_ctx *c = new larql_hip_ctx();
     c->device = device;
     c->cu_count = prop.multiProcessorCount;
-    if (const char *e = getenv("LARQL_HIP_WGS_PER_CU")) { int v = atoi(e); if (v >= 1 && v <= 16) c->wgs_per_cu = v; }
     char buf[256];
     snprintf(buf, sizeof buf, "hip (gfx950 matvec + gate-KNN kernels)");
     c->name = buf;
@@ -1398,10 +1397,6 @@ int larql_hip_dev_q4k_gemm(larql_hip_ctx *c, const uint8_t *w, const uint16_t *x
     if (rows > 0xFFFFFFFFull || seq > 0xFFFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "q4k_gemm: too large");
     if (!w || !x_bf16 || !out || ((uintptr_t)w & 15) || ((uintptr_t)x_bf16 & 15)) return LARQL_E_ARG;
     HIPCHECK(c, hipSetDevice(c->device));
-    if (getenv("LARQL_HIP_GEMM_BF16")) {  // first formulation (decoded weights split into two bf16 terms), kept for comparison
-        HIPCHECK(c, q4k_gemm_launch(c->stream, w, x_bf16, out, (uint32_t)rows, (uint32_t)hidden, (uint32_t)seq, 0));
-        return LARQL_OK;
-    }
     // bf16 activations are exact in one f16 term after the per-token scale
     const size_t x_len = seq * hidden, sx_len = seq * (hidden / 32) * 2;
     int rc = ensure(c, c->misc, x_len * 2 + sx_len * 2 + seq * 4 + 256);
@@ -1493,15 +1488,13 @@ static int moe_mxfp4_block(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank
         set_down_bias(td);
         const size_t table_bytes = slots * 3 * sizeof(GemvJob) + 64;
         const bool mfma = gemv_effective_kind(tg) == KIND_MXFP4_MFMA && gemv_effective_kind(td) == KIND_MXFP4_MFMA;
-        static const bool pairing = !(getenv("LARQL_HIP_MOE_PAIRS") && atoi(getenv("LARQL_HIP_MOE_PAIRS")) == 0);
-        if (pairing && mfma && tokens > 1 && slots <= 4096 && bank->n_experts <= 1024 && slots * inter * sizeof(float) >= table_bytes) {
+        if (mfma && tokens > 1 && slots <= 4096 && bank->n_experts <= 1024 && slots * inter * sizeof(float) >= table_bytes) {
             tg.kind = tu.kind = td.kind = KIND_MXFP4_MFMA;
             uint32_t *hdr = (uint32_t *)h;  // {gate/up count, passes, down count, passes}
             GemvJob *gu_table = (GemvJob *)((uint8_t *)h + 64), *dn_table = gu_table + 2 * slots;
             PreparedLaunch Pg, Pd;
             // four tokens per job where the launches' LDS has room for their partial sums, else two
-            static const uint32_t group_cap = getenv("LARQL_HIP_MOE_GROUP") && atoi(getenv("LARQL_HIP_MOE_GROUP")) == 2 ? 2u : 4u;
-            uint32_t group = group_cap;
+            uint32_t group = 4;
             for (int which = 0; which < 2 && group > 2; which++) {
                 GemvJob tj = which == 0 ? tg : td;
                 const uint32_t th = gemv_pick_threads(&tj, 1);

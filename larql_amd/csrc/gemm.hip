@@ -1,18 +1,10 @@
 // gemm.hip — batched-prefill Q4_K GEMM on the gfx950 matrix cores.
 //
-//   out[s, r] = sum_k W[r, k] * X[s, k]      W: [rows, hidden] Q4_K,  X: [seq, hidden] bf16
+//   out[s, r] = sum_k W[r, k] * X[s, k]      W: [rows, hidden] Q4_K,  X: [seq, hidden] bf16 or f32
 //
 // the contraction q4k_matmul_into computes (larql-compute/src/cpu/ops/q4_common/
-// matmul.rs:20-139; `out` is [seq, rows] row-major).  A workgroup owns a
-// 128-row x 128-token tile of `out` and walks K in steps of 64 (one nibble
-// group = two 32-element sub-blocks).  Per step it decodes its 128x64 weights
-// exactly as decode_q4k_superblock_into does (w = sc*q - mn in f32,
-// matvec_f32.rs:166-199), splits each into two bf16 terms hi + lo (so the
-// bf16 operand carries 16 significant bits and the product is good to ~2^-17,
-// not the 2^-9 of a single bf16 rounding), stages them and the activation tile
-// in LDS, and feeds v_mfma_f32_16x16x32_bf16 with fp32 accumulators (two MFMAs
-// per tile: hi and lo).  LDS rows are padded to 72 elements so the 16 lanes of
-// an operand read hit 16 distinct 16-byte slots.
+// matmul.rs:20-139; `out` is [seq, rows] row-major), on f16 MFMA over the integer
+// weights (see the formulation below).
 #include <hip/hip_runtime.h>
 
 #include <atomic>
@@ -28,125 +20,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int TM = 128, TN = 128, KS = 64, LDK = 72;  // tile rows, tile tokens, k per step, padded LDS row (bf16 elements)
-
-__device__ __forceinline__ uint32_t bf16_rne_bits(float f) {
-    const uint32_t b = __builtin_bit_cast(uint32_t, f);
-    return (b + 0x7FFFu + ((b >> 16) & 1u)) >> 16;  // finite inputs only (weights and activations)
-}
-
-__device__ __forceinline__ float half_to_float(uint32_t lo16) { return (float)__builtin_bit_cast(_Float16, (uint16_t)lo16); }
-
-__global__ void __launch_bounds__(256) q4k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
-                                                       float *__restrict__ out, uint32_t rows, uint32_t hidden, uint32_t seq,
-                                                       int accumulate) {
-    __shared__ __attribute__((aligned(16))) uint16_t a_hi[TM * LDK];
-    __shared__ __attribute__((aligned(16))) uint16_t a_lo[TM * LDK];
-    __shared__ __attribute__((aligned(16))) uint16_t b_t[TN * LDK];
-    const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
-    const uint32_t row0 = blockIdx.x * TM, tok0 = blockIdx.y * TN;
-    const uint32_t nsb = hidden >> 8;
-    const size_t row_bytes = (size_t)nsb * 144;
-
-    // staging role: thread -> (tile row / token, half of the 64-wide k step)
-    const uint32_t sr = t >> 1, half = t & 1u;
-    const uint32_t wrow = min(row0 + sr, rows - 1), xtok = min(tok0 + sr, seq - 1);
-    const uint8_t *wp = w + (size_t)wrow * row_bytes;
-    const uint16_t *xp = x + (size_t)xtok * hidden + half * 32;
-
-    // compute role: wave -> 64x64 quadrant, lane -> (row / token within a 16-wide tile, k octet)
-    const uint32_t wm = (wave >> 1) * 64, wn = (wave & 1u) * 64;
-    const uint32_t l16 = lane & 15u, kq = (lane >> 4) * 8;
-
-    f32x4 acc[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
-
-    for (uint32_t ks = 0; ks < hidden; ks += KS) {
-        const uint32_t sb = ks >> 8, g = (ks >> 6) & 3u;
-        // ---- decode 32 weights of (row sr, sub-block 2g+half) ----
-        const u32x4 *blk = reinterpret_cast<const u32x4 *>(wp + (size_t)sb * 144);
-        const u32x4 hdr = blk[0], q0 = blk[1 + 2 * g], q1 = blk[2 + 2 * g];
-        const float d = half_to_float(hdr.x & 0xFFFFu), dmin = half_to_float(hdr.x >> 16);
-        const uint32_t s = 2 * g + half;  // sub-block index 0..7 (get_scale_min_k4)
-        const uint32_t sh = 8u * (s & 3u);
-        const uint32_t pa = (hdr.y >> sh) & 0xFFu, pb = (hdr.z >> sh) & 0xFFu, pc = (hdr.w >> sh) & 0xFFu;
-        const uint32_t sc6 = s < 4 ? (pa & 63u) : ((pc & 0x0Fu) | ((pa >> 6) << 4));
-        const uint32_t mn6 = s < 4 ? (pb & 63u) : ((pc >> 4) | ((pb >> 6) << 4));
-        const float sc = d * (float)sc6, mn = dmin * (float)mn6;
-        const uint32_t qd[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
-        uint32_t hi_w[16], lo_w[16];
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const uint32_t v = half ? (qd[i] >> 4) : qd[i];
-            uint32_t hb[4], lb[4];
-#pragma unroll
-            for (int b = 0; b < 4; b++) {
-                const float wf = sc * (float)((v >> (8 * b)) & 0x0Fu) - mn;
-                hb[b] = bf16_rne_bits(wf);
-                lb[b] = bf16_rne_bits(wf - __builtin_bit_cast(float, hb[b] << 16));
-            }
-            hi_w[2 * i] = hb[0] | (hb[1] << 16); hi_w[2 * i + 1] = hb[2] | (hb[3] << 16);
-            lo_w[2 * i] = lb[0] | (lb[1] << 16); lo_w[2 * i + 1] = lb[2] | (lb[3] << 16);
-        }
-        // ---- activation tile: 32 bf16 of token sr ----
-        const u32x4 *xv = reinterpret_cast<const u32x4 *>(xp + ks);
-        const u32x4 x0 = xv[0], x1 = xv[1], x2 = xv[2], x3 = xv[3];
-
-        __syncthreads();  // previous step's MFMA reads are done
-        {
-            u32x4 *ah = reinterpret_cast<u32x4 *>(&a_hi[sr * LDK + half * 32]);
-            u32x4 *al = reinterpret_cast<u32x4 *>(&a_lo[sr * LDK + half * 32]);
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                ah[i] = (u32x4){hi_w[4 * i], hi_w[4 * i + 1], hi_w[4 * i + 2], hi_w[4 * i + 3]};
-                al[i] = (u32x4){lo_w[4 * i], lo_w[4 * i + 1], lo_w[4 * i + 2], lo_w[4 * i + 3]};
-            }
-            u32x4 *bt = reinterpret_cast<u32x4 *>(&b_t[sr * LDK + half * 32]);
-            bt[0] = x0; bt[1] = x1; bt[2] = x2; bt[3] = x3;
-        }
-        __syncthreads();
-
-        // ---- 64x64 quadrant: 2 k-slices x 16 tiles x (hi, lo) ----
-#pragma unroll
-        for (int kk = 0; kk < 2; kk++) {
-            bf16x8 ah[4], al[4], bb[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const uint32_t off = (wm + i * 16 + l16) * LDK + kk * 32 + kq;
-                ah[i] = *reinterpret_cast<const bf16x8 *>(&a_hi[off]);
-                al[i] = *reinterpret_cast<const bf16x8 *>(&a_lo[off]);
-                bb[i] = *reinterpret_cast<const bf16x8 *>(&b_t[(wn + i * 16 + l16) * LDK + kk * 32 + kq]);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah[i], bb[j], acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al[i], bb[j], acc[i][j], 0, 0, 0);
-                }
-        }
-    }
-
-    // ---- store: lane holds rows 4*(lane/16)..+3 of column (token) lane%16 of each 16x16 tile ----
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const uint32_t tok = tok0 + wn + j * 16 + l16;
-            const uint32_t r = row0 + wm + i * 16 + (lane >> 4) * 4;
-            if (tok >= seq) continue;
-            float *o = out + (size_t)tok * rows + r;
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-                if (r + e < rows) o[e] = accumulate ? o[e] + acc[i][j][e] : acc[i][j][e];
-        }
-}
-
 // ---------------------------------------------------------------------------
-// Second formulation (the one in use): keep the weight integer.
+// The formulation: keep the weight integer.
 //
 //   out[s, r] = sum over super-blocks of  d[r] * (sum_k (sc6*q)[r,k] * x[s,k])  -  dmin[r] * (sum_sub mn6[r,sub] * Sx[s,sub])
 //
@@ -159,10 +34,11 @@ __global__ void __launch_bounds__(256) q4k_gemm_kernel(const uint8_t *__restrict
 // 32 MFMAs per 64-element step), gets sum_sub mn6*Sx from one more MFMA per tile (A slots 2*sub+h = mn6,
 // B slots = Sx_h), and folds both into the f32 result with the row's d and dmin.
 // ---------------------------------------------------------------------------
+__device__ __forceinline__ float half_to_float(uint32_t lo16) { return (float)__builtin_bit_cast(_Float16, (uint16_t)lo16); }
+
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
-constexpr int LDM = 40;  // padded row of the 32-slot min tiles (f16 elements)
 
 // one block per token: scale, f16 terms, sub-block sums.  `x_is_bf16`: 16-bit inputs (exact in one term).
 // A thread takes 8 consecutive elements at a time (one or two 16-byte loads); four neighbouring threads hold a
@@ -241,158 +117,7 @@ __global__ void __launch_bounds__(256) q4k_gemm_prep_kernel(const void *__restri
     if (lo_seen && any_lo) *any_lo = 1;
 }
 
-// with_mins = 0: the activation term carries no offset part (second pass over the lo terms)
-__global__ void __launch_bounds__(256, 2) q4k_gemm_f16_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ xh,
-                                                              const uint16_t *__restrict__ sx, const float *__restrict__ tok_scale,
-                                                              float *__restrict__ out, uint32_t rows, uint32_t hidden, uint32_t seq,
-                                                              int with_mins, int accumulate, uint32_t sb_per_split, float *__restrict__ partial) {
-    __shared__ __attribute__((aligned(16))) uint16_t a_t[TM * LDK];   // f16(sc6*q), 128 rows x 64 k
-    __shared__ __attribute__((aligned(16))) uint16_t b_t[TN * LDK];   // f16 activations, 128 tokens x 64 k
-    __shared__ __attribute__((aligned(16))) uint16_t am_t[TM * LDM];  // mn6 in slots 2*sub+h
-    __shared__ __attribute__((aligned(16))) uint16_t bm_t[TN * LDM];  // Sx_h in slots 2*sub+h
-    __shared__ float d_t[TM], dmin_t[TM];
-    const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
-    const uint32_t row0 = blockIdx.x * TM, tok0 = blockIdx.y * TN;
-    const uint32_t nsb = hidden >> 8;
-    const size_t row_bytes = (size_t)nsb * 144;
-    const uint32_t sr = t >> 1, half = t & 1u;
-    const uint32_t wrow = min(row0 + sr, rows - 1), xtok = min(tok0 + sr, seq - 1);
-    const uint8_t *wp = w + (size_t)wrow * row_bytes;
-    const uint16_t *xp = xh + (size_t)xtok * hidden + half * 32;
-    const uint16_t *sxp = sx + (size_t)xtok * (hidden / 32) * 2;
-    const uint32_t wm = (wave >> 1) * 64, wn = (wave & 1u) * 64;
-    const uint32_t l16 = lane & 15u, kq = (lane >> 4) * 8;
-
-    f32x4 acc[4][4], D[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int jj = 0; jj < 4; jj++) { acc[i][jj] = (f32x4){0.f, 0.f, 0.f, 0.f}; D[i][jj] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
-    // slots 16..31 of the min tiles stay zero
-    for (uint32_t e = t; e < TM * LDM; e += 256) { am_t[e] = 0; bm_t[e] = 0; }
-
-    // split-K: blockIdx.z takes super-blocks [z*sb_per_split, ...); partial results go to their own slab
-    const uint32_t sb_begin = blockIdx.z * sb_per_split, sb_end = min(nsb, sb_begin + sb_per_split);
-    for (uint32_t sb = sb_begin; sb < sb_end; sb++) {
-      const u32x4 *blk = reinterpret_cast<const u32x4 *>(wp + (size_t)sb * 144);
-      const u32x4 hdr = blk[0];
-      for (uint32_t g = 0; g < 4; g++) {
-        // raw operands of this 64-element step (a register prefetch one step ahead cost more in spills than it hid)
-        const u32x4 q0 = blk[1 + 2 * g], q1 = blk[2 + 2 * g];
-        const u32x4 *xv = reinterpret_cast<const u32x4 *>(xp + (size_t)sb * 256 + g * 64);
-        const u32x4 x0 = xv[0], x1 = xv[1], x2 = xv[2], x3 = xv[3];
-        u32x4 sxv = {0u, 0u, 0u, 0u};
-        if (g == 0 && with_mins) sxv = *reinterpret_cast<const u32x4 *>(sxp + (size_t)sb * 16 + half * 8);
-        // ---- 32 weights of (row sr, sub-block 2g+half) as f16(sc6*q) ----
-        const uint32_t s = 2 * g + half, sh = 8u * (s & 3u);
-        const uint32_t pa = (hdr.y >> sh) & 0xFFu, pc = (hdr.w >> sh) & 0xFFu;
-        const uint32_t sc6 = s < 4 ? (pa & 63u) : ((pc & 0x0Fu) | ((pa >> 6) << 4));
-        const _Float16 scf = (_Float16)(float)sc6;
-        const f16x2 sc2 = {scf, scf};
-        const f16x2 off2 = {(_Float16)(-1024.0f * (float)sc6), (_Float16)(-1024.0f * (float)sc6)};
-        const uint32_t qd[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
-        uint32_t aw[16];
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const uint32_t v = half ? (qd[i] >> 4) : qd[i];
-            // bytes 0,1 -> 16-bit lanes of one dword, bytes 2,3 -> the next (k order kept)
-            const uint32_t p01 = __builtin_amdgcn_perm(0u, v, 0x0C010C00u), p23 = __builtin_amdgcn_perm(0u, v, 0x0C030C02u);
-            const f16x2 m01 = __builtin_bit_cast(f16x2, (p01 & 0x000F000Fu) | 0x64006400u);  // 1024 + q
-            const f16x2 m23 = __builtin_bit_cast(f16x2, (p23 & 0x000F000Fu) | 0x64006400u);
-            aw[2 * i] = __builtin_bit_cast(uint32_t, m01 * sc2 + off2);      // (1024+q)*sc6 - 1024*sc6, one rounding: exact
-            aw[2 * i + 1] = __builtin_bit_cast(uint32_t, m23 * sc2 + off2);
-        }
-        uint32_t mnw[4] = {0u, 0u, 0u, 0u};
-        if (g == 0 && with_mins) {
-            // this thread's half of the super-block: sub-blocks 4*half .. 4*half+3 -> slots 8*half .. 8*half+7
-#pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const uint32_t ss = 4 * half + u, shm = 8u * (ss & 3u);
-                const uint32_t qb = (hdr.z >> shm) & 0xFFu, qc = (hdr.w >> shm) & 0xFFu;
-                const uint32_t mn6 = ss < 4 ? (qb & 63u) : ((qc >> 4) | ((qb >> 6) << 4));
-                const uint32_t hb = __builtin_bit_cast(uint16_t, (_Float16)(float)(mn6 * 32u));  // <= 2016: exact; Sx is stored /32
-                mnw[u] = hb | (hb << 16);
-            }
-        }
-        __syncthreads();  // previous step's MFMA reads are done
-        {
-            u32x4 *ah = reinterpret_cast<u32x4 *>(&a_t[sr * LDK + half * 32]);
-#pragma unroll
-            for (int i = 0; i < 4; i++) ah[i] = (u32x4){aw[4 * i], aw[4 * i + 1], aw[4 * i + 2], aw[4 * i + 3]};
-            u32x4 *bt = reinterpret_cast<u32x4 *>(&b_t[sr * LDK + half * 32]);
-            bt[0] = x0; bt[1] = x1; bt[2] = x2; bt[3] = x3;
-            if (g == 0) {
-                if (with_mins) {
-                    *reinterpret_cast<u32x4 *>(&am_t[sr * LDM + half * 8]) = (u32x4){mnw[0], mnw[1], mnw[2], mnw[3]};
-                    *reinterpret_cast<u32x4 *>(&bm_t[sr * LDM + half * 8]) = sxv;
-                }
-                if (half == 0) {
-                    d_t[sr] = half_to_float(hdr.x & 0xFFFFu);
-                    dmin_t[sr] = half_to_float(hdr.x >> 16);
-                }
-            }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int kk = 0; kk < 2; kk++) {
-            f16x8 af[4], bf[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                af[i] = *reinterpret_cast<const f16x8 *>(&a_t[(wm + i * 16 + l16) * LDK + kk * 32 + kq]);
-                bf[i] = *reinterpret_cast<const f16x8 *>(&b_t[(wn + i * 16 + l16) * LDK + kk * 32 + kq]);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int jj = 0; jj < 4; jj++) D[i][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bf[jj], D[i][jj], 0, 0, 0);
-        }
-        if (g == 3) {
-            // ---- end of the super-block: acc += d * D - dmin * (mn6 . Sx) ----
-            f16x8 amf[4], bmf[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                amf[i] = *reinterpret_cast<const f16x8 *>(&am_t[(wm + i * 16 + l16) * LDM + kq]);
-                bmf[i] = *reinterpret_cast<const f16x8 *>(&bm_t[(wn + i * 16 + l16) * LDM + kq]);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const uint32_t rb = wm + i * 16 + (lane >> 4) * 4;
-                const f32x4 dv = *reinterpret_cast<const f32x4 *>(&d_t[rb]);
-                const f32x4 mv = *reinterpret_cast<const f32x4 *>(&dmin_t[rb]);
-#pragma unroll
-                for (int jj = 0; jj < 4; jj++) {
-                    f32x4 Dm = {0.f, 0.f, 0.f, 0.f};
-                    if (with_mins) Dm = __builtin_amdgcn_mfma_f32_16x16x32_f16(amf[i], bmf[jj], Dm, 0, 0, 0);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) acc[i][jj][e] += dv[e] * D[i][jj][e] - mv[e] * Dm[e];
-                    D[i][jj] = (f32x4){0.f, 0.f, 0.f, 0.f};
-                }
-            }
-        }
-    }
-    }
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int jj = 0; jj < 4; jj++) {
-            const uint32_t tok = tok0 + wn + jj * 16 + l16;
-            const uint32_t r = row0 + wm + i * 16 + (lane >> 4) * 4;
-            if (tok >= seq) continue;
-            if (partial) {  // unscaled partial sums of this K-range; q4k_gemm_reduce_kernel adds the slabs in order
-                float *o = partial + ((size_t)blockIdx.z * seq + tok) * rows + r;
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    if (r + e < rows) o[e] = acc[i][jj][e];
-                continue;
-            }
-            const float ts = tok_scale[tok];
-            float *o = out + (size_t)tok * rows + r;
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-                if (r + e < rows) o[e] = accumulate ? o[e] + acc[i][jj][e] * ts : acc[i][jj][e] * ts;
-        }
-}
-
+// adds the partial slabs of a K-split in slab order and applies the token scale
 __global__ void __launch_bounds__(256) q4k_gemm_reduce_kernel(const float *__restrict__ partial, uint32_t splits, const float *__restrict__ tok_scale,
                                                               float *__restrict__ out, uint32_t rows, uint32_t seq, int accumulate) {
     const size_t n = (size_t)rows * seq, i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -404,7 +129,7 @@ __global__ void __launch_bounds__(256) q4k_gemm_reduce_kernel(const float *__res
 }
 
 // ---------------------------------------------------------------------------
-// The same arithmetic, software-pipelined (the kernel in use).
+// The kernel: software-pipelined; with_mins = 0: the activation term carries no offset part (second pass over the lo terms).
 //
 // One workgroup of 8 wavefronts per CU owns a 256-row x 128-token tile; a wavefront owns 32 of the rows against
 // all 128 tokens.  Everything a step (64 k) needs from global memory was copied global -> LDS (global_load_lds,
@@ -766,36 +491,11 @@ __global__ void __launch_bounds__(PTHREADS, 1) q4k_gemm_pipe_kernel(const uint8_
 }
 
 // f32 activations -> bf16 hi (round to nearest even) and the bf16 of the remainder
-__global__ void split_bf16_kernel(const float *__restrict__ x, size_t n, uint16_t *__restrict__ hi, uint16_t *__restrict__ lo,
-                                  int *__restrict__ any_lo) {
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    const float v = x[i];
-    const uint32_t h = bf16_rne_bits(v);
-    const uint32_t l = bf16_rne_bits(v - __builtin_bit_cast(float, h << 16));
-    hi[i] = (uint16_t)h;
-    lo[i] = (uint16_t)l;
-    if ((l & 0x7FFFu) != 0) *any_lo = 1;
-}
-
-static bool gemm_pipe_enabled() {
-    static const bool on = !(getenv("LARQL_HIP_GEMM_PIPE") && atoi(getenv("LARQL_HIP_GEMM_PIPE")) == 0);
-    return on;
-}
-
-hipError_t q4k_gemm_launch(hipStream_t s, const uint8_t *w, const uint16_t *x_bf16, float *out, uint32_t rows, uint32_t hidden,
-                           uint32_t seq, int accumulate) {
-    if (rows == 0 || seq == 0) return hipSuccess;
-    hipLaunchKernelGGL(q4k_gemm_kernel, dim3((rows + TM - 1) / TM, (seq + TN - 1) / TN), dim3(256), 0, s, w, x_bf16, out, rows, hidden,
-                       seq, accumulate);
-    return hipGetLastError();
-}
-
 hipError_t q4k_gemm_prep_launch(hipStream_t s, const void *x, int x_is_bf16, uint32_t hidden, uint32_t seq, uint16_t *xh, uint16_t *xl,
                                 uint16_t *sx, float *tok_scale, int *any_lo) {
     if (seq == 0) return hipSuccess;
     hipLaunchKernelGGL(q4k_gemm_prep_kernel, dim3(seq), dim3(256), 0, s, x, x_is_bf16, hidden, xh, xl, sx, tok_scale, any_lo,
-                       gemm_pipe_enabled() ? 1 : 0);
+                       1);
     return hipGetLastError();
 }
 
@@ -804,13 +504,9 @@ hipError_t q4k_gemm_prep_launch(hipStream_t s, const void *x, int x_is_bf16, uin
 uint32_t q4k_gemm_splits(uint32_t rows, uint32_t hidden, uint32_t seq, uint32_t cu_count) {
     const uint32_t nsb = hidden / 256;
     uint32_t s = 1;
-    if (gemm_pipe_enabled()) {  // one 256x128 workgroup per CU
-        const uint64_t tiles = (uint64_t)((rows + PM - 1) / PM) * ((seq + PN - 1) / PN);
-        while (s < 8 && tiles * s * 2 <= (uint64_t)cu_count && nsb / (s * 2) >= 4) s *= 2;
-        return s;
-    }
-    const uint64_t tiles = (uint64_t)((rows + TM - 1) / TM) * ((seq + TN - 1) / TN);
-    while (s < 8 && tiles * s < (uint64_t)cu_count * 3 / 2 && nsb / (s * 2) >= 4) s *= 2;
+    // one 256x128 workgroup per CU
+    const uint64_t tiles = (uint64_t)((rows + PM - 1) / PM) * ((seq + PN - 1) / PN);
+    while (s < 8 && tiles * s * 2 <= (uint64_t)cu_count && nsb / (s * 2) >= 4) s *= 2;
     return s;
 }
 
@@ -820,29 +516,18 @@ hipError_t q4k_gemm_f16_launch(hipStream_t s, const uint8_t *w, const uint16_t *
     const uint32_t nsb = hidden / 256;
     const bool split = splits > 1 && partial;
     const uint32_t per = split ? (nsb + splits - 1) / splits : nsb, z = split ? (nsb + per - 1) / per : 1;
-    if (gemm_pipe_enabled()) {
-        static std::atomic<bool> attr_set{false};  // dynamic LDS above 64 KB has to be allowed once per process
-        if (!attr_set) {
-            hipError_t e = hipFuncSetAttribute((const void *)q4k_gemm_pipe_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-            if (e != hipSuccess) return e;
-            attr_set = true;
-        }
-        hipLaunchKernelGGL(q4k_gemm_pipe_kernel, dim3((rows + PM - 1) / PM, (seq + PN - 1) / PN, z), dim3(PTHREADS), P_LDS_BYTES, s, w, xh, sx,
-                           tok_scale, out, rows, hidden, seq, with_mins, accumulate, per, split ? partial : (float *)nullptr);
-    } else {
-        hipLaunchKernelGGL(q4k_gemm_f16_kernel, dim3((rows + TM - 1) / TM, (seq + TN - 1) / TN, z), dim3(256), 0, s, w, xh, sx, tok_scale, out,
-                           rows, hidden, seq, with_mins, accumulate, per, split ? partial : (float *)nullptr);
+    static std::atomic<bool> attr_set{false};  // dynamic LDS above 64 KB has to be allowed once per process
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void *)q4k_gemm_pipe_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        attr_set = true;
     }
+    hipLaunchKernelGGL(q4k_gemm_pipe_kernel, dim3((rows + PM - 1) / PM, (seq + PN - 1) / PN, z), dim3(PTHREADS), P_LDS_BYTES, s, w, xh, sx,
+                       tok_scale, out, rows, hidden, seq, with_mins, accumulate, per, split ? partial : (float *)nullptr);
     if (split) {
         const size_t n = (size_t)rows * seq;
         hipLaunchKernelGGL(q4k_gemm_reduce_kernel, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, s, partial, z, tok_scale, out, rows, seq, accumulate);
     }
-    return hipGetLastError();
-}
-
-hipError_t split_bf16_launch(hipStream_t s, const float *x, size_t n, uint16_t *hi, uint16_t *lo, int *any_lo) {
-    if (n == 0) return hipSuccess;
-    hipLaunchKernelGGL(split_bf16_kernel, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, s, x, n, hi, lo, any_lo);
     return hipGetLastError();
 }
 

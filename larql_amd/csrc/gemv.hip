@@ -858,7 +858,6 @@ constexpr int kQ6kMaxColPasses = 4;
 constexpr int kQ6kMaxWaves = 10;
 constexpr uint32_t kQ6kPitch = 208;                          // ql 128, qh 64, scales 16
 constexpr uint32_t kQ6kTileBytes = 16 * kQ6kPitch + 256;     // + a 16-byte slot per row whose last two bytes are d
-constexpr uint32_t kQ6kColBytes = 1024 + 64 + 16;            // four limb planes of 256 bytes, 16 group sums, k
 
 struct Q6kCol {
     Q4kOp xm[4];     // A operand of MFMA m: limb (row % 4) of group 4m + kq in this lane's k-slots if row / 4 == kq, else zero
@@ -2486,10 +2485,7 @@ __device__ __forceinline__ void gemv_body(const GemvLaunch &L, float *part) {
         gemv_body<KIND, U>(L, part);                                                                            \
     }
 LARQL_GEMV_KERNEL(gemv_q4k_u2_kernel, KIND_Q4K, 2, 4)
-LARQL_GEMV_KERNEL(gemv_q4k_u4_kernel, KIND_Q4K, 4, 3)
-LARQL_GEMV_KERNEL(gemv_q8_0_u2_kernel, KIND_Q8_0, 2, 4)
 LARQL_GEMV_KERNEL(gemv_q8_0_u4_kernel, KIND_Q8_0, 4, 3)
-LARQL_GEMV_KERNEL(gemv_mxfp4_u2_kernel, KIND_MXFP4, 2, 4)
 LARQL_GEMV_KERNEL(gemv_mxfp4_u4_kernel, KIND_MXFP4, 4, 4)
 LARQL_GEMV_KERNEL(gemv_q4_0_kernel, KIND_Q4_0, 4, 4)
 LARQL_GEMV_KERNEL(gemv_q6k_kernel, KIND_Q6K, 2, 3)
@@ -2727,8 +2723,6 @@ __global__ void __launch_bounds__(kQ8MaxWaves * 64) gemv_q8_0_mfma_kernel(GemvLa
 // Host side: geometry and launch.
 // ---------------------------------------------------------------------------
 // experiment knobs (environment): passes in flight per thread, forced block size
-static int g_unroll = getenv("LARQL_HIP_UNROLL") ? atoi(getenv("LARQL_HIP_UNROLL")) : 0;  // 0: per-format default
-static int g_threads = getenv("LARQL_HIP_THREADS") ? atoi(getenv("LARQL_HIP_THREADS")) : 0;
 static uint32_t chunk_elems(int kind) {
     switch (kind) {
         case KIND_Q4K: case KIND_Q6K: case KIND_Q6K_Q8K: return 64;
@@ -2765,11 +2759,8 @@ static uint32_t q6k_mfma_waves(uint64_t cpr) {  // as q4k_mfma_waves: up to 10 w
     return best;  // 0: row too long for this path
 }
 
-static int g_q6k_mfma = getenv("LARQL_HIP_Q6K_MFMA") ? atoi(getenv("LARQL_HIP_Q6K_MFMA")) : 1;
 
-static int g_q4k_mfma = getenv("LARQL_HIP_Q4K_MFMA") ? atoi(getenv("LARQL_HIP_Q4K_MFMA")) : 1;
 
-static int g_mxfp4_mfma = getenv("LARQL_HIP_MXFP4_MFMA") ? atoi(getenv("LARQL_HIP_MXFP4_MFMA")) : 1;
 
 // MXFP4 on the matrix cores: 128-element steps per wavefront (1..4) so that at most 10 wavefronts cover a row
 static uint32_t mx4_steps_per_wave(uint64_t steps) {
@@ -2778,30 +2769,28 @@ static uint32_t mx4_steps_per_wave(uint64_t steps) {
     return 0;  // row too long for this path
 }
 
-static int g_bf16_mfma = getenv("LARQL_HIP_BF16_MFMA") ? atoi(getenv("LARQL_HIP_BF16_MFMA")) : 1;
 
 uint32_t gemv_batch_capacity(int kind, uint64_t k) {
     // bf16: 128-element columns, at most 10 wavefronts x 2 passes, two sets of 4 positions
-    if (kind == KIND_BF16 && g_bf16_mfma && k >= 128 && k % 128 == 0 && k / 128 <= (uint64_t)(kBfMaxWaves * kBfMaxPasses)) return 4 * kBfMaxSets;
+    if (kind == KIND_BF16 && k >= 128 && k % 128 == 0 && k / 128 <= (uint64_t)(kBfMaxWaves * kBfMaxPasses)) return 4 * kBfMaxSets;
     // Q4_K: one wavefront per super-block column, four pairs of positions
-    if (kind == KIND_Q4K && g_q4k_mfma && k >= 256 && k % 256 == 0 && k / 256 <= (uint64_t)kQ4kMaxWaves) return 2 * kQ4kBatchPairs;
+    if (kind == KIND_Q4K && k >= 256 && k % 256 == 0 && k / 256 <= (uint64_t)kQ4kMaxWaves) return 2 * kQ4kBatchPairs;
     return 1;
 }
 
-static int g_q8_mfma = getenv("LARQL_HIP_Q8_MFMA") ? atoi(getenv("LARQL_HIP_Q8_MFMA")) : 1;
 
 int gemv_effective_kind(const GemvJob &j) {
-    if (j.kind == KIND_Q8_0 && g_q8_mfma && j.k >= 256 && j.k % 256 == 0 && q8_mfma_waves(j.k / 256) != 0 && j.rows < 0x7FFFFFF0ull)
+    if (j.kind == KIND_Q8_0 && j.k >= 256 && j.k % 256 == 0 && q8_mfma_waves(j.k / 256) != 0 && j.rows < 0x7FFFFFF0ull)
         return KIND_Q8_0_MFMA;
     if (j.kind == KIND_BF16 && j.batch >= 2) return KIND_BF16_MFMA;
     if (j.kind == KIND_Q4K && j.batch >= 2) return KIND_Q4K_BATCH;
-    if (j.kind == KIND_MXFP4 && g_mxfp4_mfma && j.k >= 128 && j.k % 32 == 0 && mx4_steps_per_wave((j.k + 127) / 128) != 0 &&
+    if (j.kind == KIND_MXFP4 && j.k >= 128 && j.k % 32 == 0 && mx4_steps_per_wave((j.k + 127) / 128) != 0 &&
         j.rows < 0x7FFFFFF0ull)
         return KIND_MXFP4_MFMA;
-    if (j.kind == KIND_Q4K && g_q4k_mfma && !j.sel && j.k % 256 == 0 && j.k / 256 >= 1 && q4k_mfma_waves(j.k / 256) != 0 &&
+    if (j.kind == KIND_Q4K && !j.sel && j.k % 256 == 0 && j.k / 256 >= 1 && q4k_mfma_waves(j.k / 256) != 0 &&
         j.rows < 0x7FFFFFF0ull && (j.k / 256) * 144 * j.rows < (1ull << 62))
         return KIND_Q4K_MFMA;
-    if (j.kind == KIND_Q6K && g_q6k_mfma && !j.sel && j.k % 256 == 0 && j.k / 256 >= 1 && q6k_mfma_waves(j.k / 256) != 0 &&
+    if (j.kind == KIND_Q6K && !j.sel && j.k % 256 == 0 && j.k / 256 >= 1 && q6k_mfma_waves(j.k / 256) != 0 &&
         j.rows < 0x7FFFFFF0ull && (j.k / 256) * 210 * j.rows < (1ull << 62))
         return KIND_Q6K_MFMA;
     return j.kind;
@@ -2976,9 +2965,8 @@ uint32_t gemv_pick_threads(const GemvJob *jobs, size_t n) {
     // Prefer the block size that wastes the fewest lanes over the jobs'
     // chunk counts (weighted by bytes); ties go to the smaller block.
     static const uint32_t cand_all[] = {256, 320, 384, 448, 512};
-    const uint32_t forced[] = {(uint32_t)g_threads};
-    const uint32_t *cand = g_threads ? forced : cand_all;
-    const size_t n_cand = g_threads ? 1 : 5;
+    const uint32_t *cand = cand_all;
+    const size_t n_cand = 5;
     double best = -1.0;
     uint32_t pick = 0;
     for (size_t ci = 0; ci < n_cand; ci++) {
@@ -3145,16 +3133,13 @@ hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32
             break;
         }
         case KIND_Q4K:
-            if (g_unroll != 4) hipLaunchKernelGGL(gemv_q4k_u2_kernel, dim3(grid), dim3(threads), lds, stream, L);
-            else hipLaunchKernelGGL(gemv_q4k_u4_kernel, dim3(grid), dim3(threads), lds, stream, L);
+            hipLaunchKernelGGL(gemv_q4k_u2_kernel, dim3(grid), dim3(threads), lds, stream, L);
             break;
         case KIND_Q8_0:
-            if (g_unroll == 2) hipLaunchKernelGGL(gemv_q8_0_u2_kernel, dim3(grid), dim3(threads), lds, stream, L);
-            else hipLaunchKernelGGL(gemv_q8_0_u4_kernel, dim3(grid), dim3(threads), lds, stream, L);
+            hipLaunchKernelGGL(gemv_q8_0_u4_kernel, dim3(grid), dim3(threads), lds, stream, L);
             break;
         case KIND_MXFP4:
-            if (g_unroll == 2) hipLaunchKernelGGL(gemv_mxfp4_u2_kernel, dim3(grid), dim3(threads), lds, stream, L);
-            else hipLaunchKernelGGL(gemv_mxfp4_u4_kernel, dim3(grid), dim3(threads), lds, stream, L);
+            hipLaunchKernelGGL(gemv_mxfp4_u4_kernel, dim3(grid), dim3(threads), lds, stream, L);
             break;
         case KIND_Q4_0: hipLaunchKernelGGL(gemv_q4_0_kernel, dim3(grid), dim3(threads), lds, stream, L); break;
         case KIND_Q6K: hipLaunchKernelGGL(gemv_q6k_kernel, dim3(grid), dim3(threads), lds, stream, L); break;

@@ -127,16 +127,13 @@ hipError_t quantize_x_to_q8k_launch(hipStream_t s, const float *src, size_t n, u
 hipError_t quantize_to_q8_launch(hipStream_t s, const float *src, size_t n, int8_t *q8, float *scales);
 hipError_t fill_normal_launch(hipStream_t s, float *dst, size_t n, uint64_t seed, float sigma);
 
-// batched-prefill Q4_K GEMM (bf16 MFMA, fp32 accumulate)
-hipError_t q4k_gemm_launch(hipStream_t s, const uint8_t *w, const uint16_t *x_bf16, float *out, uint32_t rows, uint32_t hidden,
-                           uint32_t seq, int accumulate);
+// batched-prefill Q4_K GEMM (f16 MFMA over the integer weights, fp32 accumulate)
 // integer-weight formulation: activations prepared once (per-token scale, f16 terms, sub-block sums)
 hipError_t q4k_gemm_prep_launch(hipStream_t s, const void *x, int x_is_bf16, uint32_t hidden, uint32_t seq, uint16_t *xh, uint16_t *xl,
                                 uint16_t *sx, float *tok_scale, int *any_lo);
 hipError_t q4k_gemm_f16_launch(hipStream_t s, const uint8_t *w, const uint16_t *xh, const uint16_t *sx, const float *tok_scale, float *out,
                                uint32_t rows, uint32_t hidden, uint32_t seq, int with_mins, int accumulate, uint32_t splits, float *partial);
 uint32_t q4k_gemm_splits(uint32_t rows, uint32_t hidden, uint32_t seq, uint32_t cu_count);  // partial: [splits][seq][rows] floats
-hipError_t split_bf16_launch(hipStream_t s, const float *x, size_t n, uint16_t *hi, uint16_t *lo, int *any_lo);
 
 // MoE helpers
 hipError_t router_select_launch(hipStream_t s, const float *logits, const float *bias, uint32_t tokens, uint32_t n_experts, uint32_t k,
