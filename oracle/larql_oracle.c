@@ -1321,18 +1321,33 @@ int lq_moe_block_mxfp4(const float *x, size_t tokens, size_t hidden, size_t inte
 /* ------------------------------------------- multi-threaded CPU baseline */
 
 typedef struct {
-    int kind; /* 0 q4k, 1 q8_0 */
+    int kind; /* 0 q4k matvec, 1 q8_0 gemv, 2 mxfp4 gemv, 3 q4k matmul */
     float *out; const float *x; const uint8_t *w; const float *sum_x;
     size_t rows, blocks_per_row; int tid, nthreads;
+    const uint8_t *aux; size_t seq; float *tmp; /* mxfp4 scales; matmul positions and its [rows, seq] scratch */
 } mt_job;
 
 static void *mt_worker(void *p) {
     mt_job *j = (mt_job *)p;
-    size_t n_chunks = (j->rows + 31) / 32; /* CHUNK_ROWS = 32 in both kernels */
+    size_t n_chunks = (j->rows + 31) / 32; /* CHUNK_ROWS = 32 in the reference's row-parallel kernels */
     for (size_t c = (size_t)j->tid; c < n_chunks; c += (size_t)j->nthreads) {
         size_t r0 = c * 32, r1 = r0 + 32 < j->rows ? r0 + 32 : j->rows;
         if (j->kind == 0) q4k_rows(j->out, j->x, j->w, j->sum_x, r0, r1, j->blocks_per_row);
-        else for (size_t r = r0; r < r1; r++) j->out[r] = q8_0_row_dot(j->w, j->x, r, j->blocks_per_row);
+        else if (j->kind == 1) for (size_t r = r0; r < r1; r++) j->out[r] = q8_0_row_dot(j->w, j->x, r, j->blocks_per_row);
+        else if (j->kind == 2) {
+            moe_matrix m = {1, NULL, j->w, j->aux};
+            for (size_t r = r0; r < r1; r++) j->out[r] = moe_row_dot(&m, r, j->blocks_per_row * 32, j->x);
+        } else { /* the row loop of lq_q4k_matmul_into for rows r0..r1 */
+            float wf[256];
+            size_t n_blocks = j->blocks_per_row, row_bytes = n_blocks * 144, hidden = n_blocks * 256;
+            for (size_t r = r0; r < r1; r++) {
+                float *out_row = j->tmp + r * j->seq;
+                for (size_t sb = 0; sb < n_blocks; sb++) {
+                    decode_q4k_superblock_into(j->w, r * row_bytes, sb, wf);
+                    for (size_t s = 0; s < j->seq; s++) out_row[s] += dot_256_f32_scalar(wf, j->x + s * hidden + sb * 256);
+                }
+            }
+        }
     }
     return NULL;
 }
@@ -1347,13 +1362,34 @@ static void mt_run(mt_job proto, int threads) {
     for (int t = 1; t < threads; t++) pthread_join(th[t], NULL);
 }
 
+/* lq_mxfp4_gemv with its rows shared out in chunks of 32 (timing baseline; same bits per row) */
+int lq_mxfp4_gemv_mt(const uint8_t *packed, const uint8_t *scales, const float *x, size_t n, size_t k, float *out, int threads) {
+    if (k % 32 != 0) return 1;
+    mt_job j = {2, out, x, packed, NULL, n, k / 32, 0, 1, scales, 0, NULL};
+    mt_run(j, threads);
+    return 0;
+}
+
+/* lq_q4k_matmul_into with its rows shared out in chunks of 32, as kquant_matmul_into schedules them
+ * (q4_common/matmul.rs:100-139); same bits. */
+int lq_q4k_matmul_into_mt(float *out, const float *x, const uint8_t *w, size_t w_len, size_t rows, size_t hidden, size_t seq, int threads) {
+    if (rows == 0 || seq == 0 || hidden == 0 || hidden % 256 != 0 || w_len < rows * (hidden / 256) * 144) return 1;
+    float *tmp = (float *)calloc(rows * seq, sizeof(float));
+    mt_job j = {3, NULL, x, w, NULL, rows, hidden / 256, 0, 1, NULL, seq, tmp};
+    mt_run(j, threads);
+    for (size_t r = 0; r < rows; r++)
+        for (size_t s = 0; s < seq; s++) out[s * rows + r] = tmp[r * seq + s];
+    free(tmp);
+    return 0;
+}
+
 int lq_q4k_matvec_into_mt(float *out, const float *x, const uint8_t *w, size_t w_len,
                           size_t rows, size_t cols, int threads) {
     if (!kernel_shape_ok(rows, rows, cols, cols, w_len, 256, 144)) return 1;
     if (rows == 0 || cols == 0) { for (size_t i = 0; i < rows; i++) out[i] = 0.0f; return 0; }
     size_t n_blocks = cols / 256;
     float *sum_x = q4k_sum_x(x, n_blocks);
-    mt_job j = {0, out, x, w, sum_x, rows, n_blocks, 0, 1};
+    mt_job j = {0, out, x, w, sum_x, rows, n_blocks, 0, 1, NULL, 0, NULL};
     mt_run(j, threads);
     free(sum_x);
     return 0;
@@ -1364,7 +1400,7 @@ int lq_q8_0_gemv_mt(const uint8_t *blocks, size_t blocks_len, const float *x,
     if (k == 0 || k % 32 != 0) return 1;
     size_t per_row = k / 32;
     if (blocks_len != n * per_row * 34) return 1;
-    mt_job j = {1, out, x, blocks, NULL, n, per_row, 0, 1};
+    mt_job j = {1, out, x, blocks, NULL, n, per_row, 0, 1, NULL, 0, NULL};
     mt_run(j, threads);
     return 0;
 }

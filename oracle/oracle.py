@@ -32,6 +32,29 @@ def _load():
 
 
 _lib = _load()
+_tlib = _lib  # the library the *_mt timing baselines run in (see enable_native_timing)
+
+
+def enable_native_timing() -> str:
+    """Build the same C file for the host this runs on (-O3 -march=native, contraction still off: the reference is
+    Rust and never fuses a*b+c) and route the multi-threaded timing baselines (*_mt) through it.  The checker
+    functions keep the portable -O2 build.  Returns the flags in use; falls back to the portable build if the host
+    has no compiler."""
+    global _tlib
+    import tempfile
+    flags = ["-O3", "-march=native", "-fPIC", "-shared", "-std=c11", "-ffp-contract=off", "-fno-fast-math", "-pthread"]
+    for d in (os.path.join(_HERE, "_native"), tempfile.mkdtemp(prefix="larql_oracle_")):
+        try:
+            os.makedirs(d, exist_ok=True)
+            out = os.path.join(d, "liblarql_oracle_native.so")
+            subprocess.run(["gcc", *flags, "-o", out, os.path.join(_HERE, "larql_oracle.c"), "-lm"], check=True,
+                           capture_output=True)
+            _tlib = C.CDLL(out)
+            return " ".join(["gcc", *flags])
+        except (OSError, subprocess.CalledProcessError):
+            continue
+    _tlib = _lib
+    return "portable build (gcc -O2): no compiler on this host"
 _u8p = C.POINTER(C.c_uint8)
 _i8p = C.POINTER(C.c_int8)
 _u16p = C.POINTER(C.c_uint16)
@@ -144,7 +167,7 @@ def q4k_matvec(w, x, rows: int, cols: int, out_len: int | None = None):
 def q4k_matvec_mt(w, x, rows: int, cols: int, threads: int):
     w, x = _u8(w).ravel(), _f32(x).ravel()
     out = np.empty(rows, dtype=np.float32)
-    rc = _lib.lq_q4k_matvec_into_mt(_p(out, _f32p), _p(x, _f32p), _p(w, _u8p), _sz(w.size),
+    rc = _tlib.lq_q4k_matvec_into_mt(_p(out, _f32p), _p(x, _f32p), _p(w, _u8p), _sz(w.size),
                                     _sz(rows), _sz(cols), C.c_int(threads))
     return None if rc else out
 
@@ -267,7 +290,7 @@ def q8_0_gemv(blocks, x, n: int, k: int):
 def q8_0_gemv_mt(blocks, x, n: int, k: int, threads: int):
     blocks, x = _u8(blocks).ravel(), _f32(x).ravel()
     out = np.empty(n, dtype=np.float32)
-    rc = _lib.lq_q8_0_gemv_mt(_p(blocks, _u8p), _sz(blocks.size), _p(x, _f32p),
+    rc = _tlib.lq_q8_0_gemv_mt(_p(blocks, _u8p), _sz(blocks.size), _p(x, _f32p),
                               _sz(n), _sz(k), _p(out, _f32p), C.c_int(threads))
     return None if rc else out
 
@@ -513,3 +536,19 @@ def moe_block_mxfp4(x, experts, weights, gate, up, down, n_experts: int, hidden:
     if rc:
         raise ValueError("hidden and inter must be multiples of 32")
     return out
+
+
+# ---- multi-threaded timing baselines for the other configurations ------------------------------------------
+def mxfp4_gemv_mt(packed, scales, x, n: int, k: int, threads: int):
+    p, sc, x = _u8(packed).ravel(), _u8(scales).ravel(), _f32(x).ravel()
+    out = np.empty(n, dtype=np.float32)
+    rc = _tlib.lq_mxfp4_gemv_mt(_p(p, _u8p), _p(sc, _u8p), _p(x, _f32p), _sz(n), _sz(k), _p(out, _f32p), C.c_int(threads))
+    return None if rc else out
+
+
+def q4k_matmul_mt(w, x, rows: int, hidden: int, seq: int, threads: int):
+    w, x = _u8(w).ravel(), _f32(x).ravel()
+    out = np.empty((seq, rows), dtype=np.float32)
+    rc = _tlib.lq_q4k_matmul_into_mt(_p(out, _f32p), _p(x, _f32p), _p(w, _u8p), _sz(w.size), _sz(rows), _sz(hidden), _sz(seq),
+                                     C.c_int(threads))
+    return None if rc else out
