@@ -168,7 +168,8 @@ int larql_hip_q4k_matmul(larql_hip_ctx *ctx, const uint8_t *q4k, size_t q4k_len,
                          size_t seq_len, float *out, size_t out_len);
 /* QuantMatVec::q4k_matvec_topk — quant_matvec.rs:268-277: up to top_k
  * (row, score) pairs by value descending, non-finite scores skipped
- * (lm_head/knn.rs:315-386).  *n_out receives the count.  top_k up to 16384. */
+ * (lm_head/knn.rs:315-386).  idx_out/score_out hold top_k entries (all copied back);
+ * *n_out receives how many of them are hits.  top_k up to 16384. */
 int larql_hip_q4k_matvec_topk(larql_hip_ctx *ctx, const uint8_t *q4k, size_t q4k_len,
                               const float *x, size_t x_len, size_t num_rows, size_t hidden,
                               size_t top_k, uint32_t *idx_out, float *score_out, size_t *n_out);
@@ -187,7 +188,7 @@ int larql_hip_q8_0_gemv(larql_hip_ctx *ctx, const uint8_t *blocks, size_t blocks
 /* lm_head KNN over a ggml Q8_0 head — larql-vindex/src/index/storage/lm_head/knn.rs:126-185 with top_k_sorted
  * (:315-386): larql_hip_q8_0_gemv followed by the top_k (<= 16384) largest scores by value, descending, non-finite
  * scores skipped; the vocabulary's scores stay on the device (1 MB per token for a 262144-row head).  Shape rule of
- * larql_hip_q8_0_gemv.  *n_out receives the count. */
+ * larql_hip_q8_0_gemv.  idx_out/score_out hold top_k entries; *n_out receives how many of them are hits. */
 int larql_hip_q8_0_gemv_topk(larql_hip_ctx *ctx, const uint8_t *blocks, size_t blocks_len, const float *x, size_t x_len,
                              size_t n, size_t k, size_t top_k, uint32_t *idx_out, float *score_out, size_t *n_out);
 /* QuantMatVec::quant_matvec — quant_matvec.rs:50-98: format dispatch.
@@ -247,8 +248,9 @@ int larql_hip_mxfp4_gemv_multi(larql_hip_ctx *ctx, size_t n_mats,
  * against the gate matrix [n_features, hidden] stored as `format`
  * (F32, F16, BF16, Q4_K or Q4_0), keep the min(top_k, n_features) largest
  * |score| per position, sorted by |score| descending (ties: lower index
- * first).  idx_out/score_out are [batch, top_k]; *n_out receives the number
- * of hits per position.  top_k up to 16384 (top_k_by_abs takes any K; WalkFfn's
+ * first).  idx_out/score_out are [batch, top_k] (all of it is written; entries
+ * past a position's count are unspecified); n_out is [batch] and receives the
+ * number of hits of each position.  top_k up to 16384 (top_k_by_abs takes any K; WalkFfn's
  * default is every feature, larql-inference/src/vindex/walk_ffn/mod.rs:186-190);
  * above that LARQL_UNSUPPORTED.  LARQL_E_NAN on a NaN score. */
 int larql_hip_gate_knn(larql_hip_ctx *ctx, int format, const uint8_t *gate, size_t gate_len,
