@@ -40,3 +40,31 @@ def test_product_never_imports_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".hpp", ".cpp")):
                 src = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in src.lower(), f"{f} mentions the oracle"
+
+
+def _c_params(decl):
+    inner = decl[decl.index("(") + 1:decl.rindex(")")].strip()
+    return [] if inner in ("", "void") else [p.strip() for p in inner.split(",")]
+
+
+def test_rust_crate_declares_what_the_header_declares():
+    """larql-compute-hip/src/ffi.rs cannot be compiled here, so its declarations are held to the header textually:
+    every extern fn exists in include/larql_hip.h with the same number of parameters, pointer parameters line up, and
+    lib.rs calls only functions ffi.rs declares."""
+    header = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "larql_hip.h")).read(), flags=re.S)
+    c_decls = {m.group(1): m.group(0) for m in re.finditer(r"\b(larql_hip_[a-z0-9_]+)\s*\([^;{]*\)\s*;", header)}
+    ffi = open(os.path.join(ROOT, "larql-compute-hip", "src", "ffi.rs")).read()
+    rust = {m.group(1): m.group(2) for m in re.finditer(r"pub fn (larql_hip_[a-z0-9_]+)\s*\(([^)]*)\)", ffi)}
+    assert len(rust) >= 30
+    for name, params in rust.items():
+        assert name in c_decls, f"{name} is in ffi.rs but not in the header"
+        r = [p.strip() for p in params.split(",") if p.strip()]
+        c = _c_params(c_decls[name])
+        assert len(r) == len(c), (name, r, c)
+        for rp, cp in zip(r, c):
+            assert ("*" in rp.split(":", 1)[1]) == ("*" in cp), (name, rp, cp)
+            # pointer depth: `*const *const u8` <-> `const uint8_t *const *`
+            assert rp.split(":", 1)[1].count("*") == cp.count("*"), (name, rp, cp)
+    lib_rs = open(os.path.join(ROOT, "larql-compute-hip", "src", "lib.rs")).read()
+    called = set(re.findall(r"ffi::(larql_hip_[a-z0-9_]+)", lib_rs))
+    assert called and called <= set(rust), called - set(rust)
