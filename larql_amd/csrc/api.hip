@@ -236,9 +236,6 @@ int check_jobs(larql_hip_ctx *c, const std::vector<GemvJob> &jobs) {
         if (j.rows == 0) continue;
         if (((uintptr_t)j.w & 15) || ((uintptr_t)j.x & 15))
             return fail(c, LARQL_REFUSED_SHAPE, "matvec: weight and activation pointers must be 16-byte aligned");
-        if ((j.kind == KIND_Q8_0 || j.kind == KIND_Q4_0) && (j.k % 64) != 0)
-            return fail(c, LARQL_UNSUPPORTED, "matvec: this block format needs k %% 64 == 0 on this backend (k=%llu)",
-                        (unsigned long long)j.k);
     }
     return LARQL_OK;
 }
@@ -1353,7 +1350,6 @@ int larql_hip_dev_gate_knn_static(larql_hip_ctx *c, int format, const void *gate
     for (size_t i = 0; i < n_jobs; i++) {
         if (((uintptr_t)jobs[i].w & 15) || ((uintptr_t)jobs[i].x & 15))
             return fail(c, LARQL_REFUSED_SHAPE, "matvec: weight and activation pointers must be 16-byte aligned");
-        if (kind == KIND_Q4_0 && (hidden % 64) != 0) return fail(c, LARQL_UNSUPPORTED, "matvec: this block format needs k %% 64 == 0 on this backend");
         jobs[i].kind = gemv_effective_kind(jobs[i]);
     }
     // one launch per kernel the jobs map to (a full group of positions and a single left-over position may differ)

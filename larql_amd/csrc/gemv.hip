@@ -159,19 +159,25 @@ __device__ __forceinline__ void load_x32(X32Slice &s, const float *x, uint32_t c
     }
 }
 
-struct Q8Raw { uint32_t d[9]; };
+struct Q8Raw { uint32_t d[9]; bool odd; };
 
-__device__ __forceinline__ Q8Raw q8_0_load(const uint8_t *row, uint32_t c) {
-    // block c starts at 34c; the aligned window starts at 34c (c even) or 34c-2 (c odd)
-    g_u32p p = (g_u32p)(row + (size_t)c * 34 - ((c & 1u) * 2u));
+// `blk` is the block's index in the whole matrix (row * blocks_per_row + c): with an odd number of blocks per row the
+// rows themselves alternate between 4-byte and 2-byte alignment, so the parity is the matrix-wide one.
+__device__ __forceinline__ Q8Raw q8_0_load(const uint8_t *base, uint64_t blk) {
+    // block `blk` starts at 34*blk; the aligned window starts there (even) or 2 bytes earlier (odd)
     Q8Raw r;
+    r.odd = (blk & 1u) != 0;
+    const uint8_t *b = base + blk * 34 - (r.odd ? 2u : 0u);
+    g_u32p p = (g_u32p)b;
 #pragma unroll
-    for (int i = 0; i < 9; i++) r.d[i] = p[i];
+    for (int i = 0; i < 8; i++) r.d[i] = p[i];
+    // an even block's last two codes are half a dword: a 16-bit read, so the last block of a buffer is not overrun
+    r.d[8] = r.odd ? p[8] : (uint32_t)*(const GLOBAL_AS uint16_t *)(b + 32);
     return r;
 }
 
-__device__ __forceinline__ float q8_0_block_dot(const Q8Raw &r, const X32Slice &s, uint32_t c) {
-    const bool odd = (c & 1u) != 0;
+__device__ __forceinline__ float q8_0_block_dot(const Q8Raw &r, const X32Slice &s) {
+    const bool odd = r.odd;
     // even: [d | q0 q1][q2..q5]...[q30 q31 | next]   odd: [prev | d][q0..q3]...[q28..q31]
     const float d = half_bits_to_float(odd ? (r.d[0] >> 16) : (r.d[0] & 0xFFFFu));
     float acc0 = 0.f, acc1 = 0.f;
@@ -387,19 +393,23 @@ __device__ __forceinline__ void load_q8act(Q8ActSlice &s, const int8_t *q8, cons
     s.code_sum = cs;
 }
 
-struct Q40Raw { uint32_t d[5]; };
+struct Q40Raw { uint32_t d[5]; bool odd; };
 
-__device__ __forceinline__ Q40Raw q4_0_load(const uint8_t *row, uint32_t c) {
-    // block c at 18c: 4-byte aligned when c is even, else window starts at 18c-2
-    g_u32p p = (g_u32p)(row + (size_t)c * 18 - ((c & 1u) * 2u));
+// `blk` is the block's index in the whole matrix, as for q8_0_load.
+__device__ __forceinline__ Q40Raw q4_0_load(const uint8_t *base, uint64_t blk) {
+    // block `blk` at 18*blk: 4-byte aligned when even, else the window starts 2 bytes earlier
     Q40Raw r;
+    r.odd = (blk & 1u) != 0;
+    const uint8_t *b = base + blk * 18 - (r.odd ? 2u : 0u);
+    g_u32p p = (g_u32p)b;
 #pragma unroll
-    for (int i = 0; i < 5; i++) r.d[i] = p[i];
+    for (int i = 0; i < 4; i++) r.d[i] = p[i];
+    r.d[4] = r.odd ? p[4] : (uint32_t)*(const GLOBAL_AS uint16_t *)(b + 16);
     return r;
 }
 
-__device__ __forceinline__ float q4_0_block_dot(const Q40Raw &r, const Q8ActSlice &s, uint32_t c) {
-    const bool odd = (c & 1u) != 0;
+__device__ __forceinline__ float q4_0_block_dot(const Q40Raw &r, const Q8ActSlice &s) {
+    const bool odd = r.odd;
     const float d = half_bits_to_float(odd ? (r.d[0] >> 16) : (r.d[0] & 0xFFFFu));
     int isum = 0;
 #pragma unroll
@@ -2206,12 +2216,12 @@ __device__ __forceinline__ void run_q8_0(const GemvJob &j, uint32_t p0, uint32_t
 #pragma unroll
                 for (int u = 0; u < U; u++) {
                     const uint32_t r = min(lr + u * rpp, tile_rows - 1) + row_base;
-                    raw[u] = q8_0_load(j.w + (size_t)r * row_bytes, c);
+                    raw[u] = q8_0_load(j.w, (uint64_t)r * cpr + c);
                 }
 #pragma unroll
                 for (int u = 0; u < U; u++) {
                     const uint32_t r = lr + u * rpp;
-                    const float v = q8_0_block_dot(raw[u], xs, c);
+                    const float v = q8_0_block_dot(raw[u], xs);
                     if (r < tile_rows) part[r * cpr + c] = v;
                 }
             }
@@ -2360,12 +2370,12 @@ __device__ __forceinline__ void run_q4_0(const GemvJob &j, uint32_t p0, uint32_t
 #pragma unroll
                 for (int u = 0; u < U; u++) {
                     const uint32_t r = min(lr + u * rpp, tile_rows - 1) + row_base;
-                    raw[u] = q4_0_load(j.w + (size_t)r * row_bytes, c);
+                    raw[u] = q4_0_load(j.w, (uint64_t)r * cpr + c);
                 }
 #pragma unroll
                 for (int u = 0; u < U; u++) {
                     const uint32_t r = lr + u * rpp;
-                    const float v = q4_0_block_dot(raw[u], xs, c);
+                    const float v = q4_0_block_dot(raw[u], xs);
                     if (r < tile_rows) part[r * cpr + c] = v;
                 }
             }

@@ -393,6 +393,30 @@ def test_q8_0_gemv_matches_oracle(be, n, k):
     assert be.q8_0_gemv(np.concatenate([q, q[:2]]), x, n, k) is None
 
 
+@pytest.mark.parametrize("n,k", [(1, 32), (3, 32), (7, 96), (1001, 160), (64, 2592), (33, 4128), (5, 16352)])
+def test_q8_0_and_q4_0_rows_with_an_odd_number_of_blocks(be, fmt, n, k):
+    """K % 32 == 0 is all the reference asks (kquant_gemv.rs:67-90, q4_matvec.rs:24-86).  With an odd block count every
+    other row starts 2 bytes off a dword boundary, and an odd total leaves the last block half a dword short of one:
+    each block carries its own magnitude so that a scale or code taken from a neighbour shows."""
+    rng = np.random.default_rng(k * 7 + n)
+    w = (rng.standard_normal((n, k // 32, 32)) * 0.02).astype(F)
+    w *= np.exp2(rng.integers(-5, 6, size=(n, k // 32, 1))).astype(F)
+    w = w.reshape(-1)
+    x = rng.standard_normal(k).astype(F)
+    q8w = O.quantize_q8_0(w)
+    assert rel_l2(be.q8_0_gemv(q8w, x, n, k), O.q8_0_gemv(q8w, x, n, k)) < TOL
+    q4 = O.quantize_q4_0(w)
+    q8, sc = O.quantize_to_q8(x)
+    want = O.q4_0_matvec(q4, q8, sc, n, k)
+    assert rel_l2(be.q4_matvec(q4, q8, sc, n, k), want) < TOL
+    assert rel_l2(be.quant_matvec(fmt.FMT_Q4_0, q4, x, n, k), want) < TOL
+    hits = be.gate_knn(fmt.FMT_Q4_0, q4, x, n, k, 5)
+    assert [i for i, _ in hits] == [i for i, _ in O.top_k_by_abs(want, 5)]
+    if n >= 64:
+        top = be.q8_0_gemv_topk(q8w, x, n, k, 9)
+        assert [i for i, _ in top] == [i for i, _ in O.top_k_sorted(O.q8_0_gemv(q8w, x, n, k), 9)]
+
+
 # ----------------------------------------------------------------- MXFP4
 def test_mxfp4_gemv_matches_dequant_reference(be):
     # the Metal peer's recipe: cos > 0.999999 and rel < 1e-4 vs dequantize_expert, sentinels, ragged rows
@@ -1180,7 +1204,7 @@ def test_one_context_from_eight_threads(be, fmt):
             for rep in range(25):
                 got = be.q4k_matvec(q, x, rows, cols)
                 assert got is not None and rel_l2(got, want4) < TOL
-                got8 = be.q8_0_gemv(q8, x, rows, cols) if cols % 64 == 0 else want8
+                got8 = be.q8_0_gemv(q8, x, rows, cols)
                 assert rel_l2(got8, want8) < TOL
                 assert be.q4k_matvec(q[:-1], x, rows, cols) is None            # a refusal in the middle of the others' calls
                 h = be.gate_knn(fmt.FMT_Q4_K, q, x, rows, cols, 8)
