@@ -1467,6 +1467,53 @@ static int moe_mxfp4_block(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank
         if (!bank->down_bias) return;
         jb.bias = bank->down_bias; jb.bias_step = 1; jb.bias_sel_stride = hidden;
     };
+    if (tokens == 1 && k <= kMoe1MaxK) {
+        // One token: a launch for the selected experts' gate / up projections (which selects for itself when it is
+        // given the logits) and a launch for their down projections, gated on the way in, folded over the experts,
+        // weighted and biased on the way out.
+        Moe1Args ga = {}, da = {};
+        ga.logits = route_logits; ga.router_bias = bank->router_bias; ga.experts = experts; ga.weights = weights;
+        ga.n_experts = (uint32_t)bank->n_experts; ga.k = (uint32_t)k; ga.policy = route_policy;
+        ga.n_mats = fused ? 1u : 2u;
+        ga.w[0] = (const uint8_t *)bank->gate_packed; ga.aux[0] = (const uint8_t *)bank->gate_scales;
+        ga.w[1] = (const uint8_t *)bank->up_packed; ga.aux[1] = (const uint8_t *)bank->up_scales;
+        ga.w_stride = gu_w_stride; ga.aux_stride = gu_s_stride;
+        if (bank->gate_up_bias) {  // the fused bias row is interleaved (gate bias j at 2j, up bias j at 2j+1) whatever the weight layout
+            ga.bias[0] = bank->gate_up_bias; ga.bias[1] = bank->gate_up_bias + 1;
+            ga.bias_stride = 2 * inter; ga.bias_step = fused ? 1u : 2u;
+        }
+        ga.rows = (uint32_t)gu_rows; ga.kdim = (uint32_t)hidden;
+        ga.x = x;
+        ga.out[0] = g; ga.out[1] = u; ga.out_slot_stride = gu_rows;
+        da.experts = experts; da.weights = weights; da.n_experts = (uint32_t)bank->n_experts; da.k = (uint32_t)k; da.n_mats = 1;
+        da.w[0] = (const uint8_t *)bank->down_packed; da.aux[0] = (const uint8_t *)bank->down_scales;
+        da.w_stride = dn_w_stride; da.aux_stride = dn_s_stride;
+        if (bank->down_bias) { da.bias[0] = bank->down_bias; da.bias_stride = hidden; da.bias_step = 1; }
+        da.rows = (uint32_t)hidden; da.kdim = (uint32_t)inter;
+        da.x = g; da.x_glu = fused ? g : u; da.x_slot_stride = gu_rows;
+        da.glu_limit = bank->limit; da.glu_alpha = bank->alpha;
+        da.out[0] = out;
+        if (fused) {
+            // the stages hand the gated activation over as operand terms: 3 x k x kpad bf16 in the workspace's gate / up areas
+            // (6 bytes per element where the raw results would take 8)
+            const size_t kpad = (inter + 127) / 128 * 128;
+            if (3 * k * kpad * sizeof(uint16_t) <= 2 * slots * inter * sizeof(float)) {
+                ga.terms = da.terms = (uint16_t *)g;
+                ga.terms_kpad = da.terms_kpad = (uint32_t)kpad;
+                ga.glu_limit = bank->limit; ga.glu_alpha = bank->alpha;
+            }
+        }
+        uint32_t gt = 0, dt = 0;
+        size_t gl = 0, dl = 0;
+        if (gu_rows < (1u << 22) && hidden < (1u << 22) && c->cu_count <= 512 && (!route_logits || bank->n_experts <= 64) && moe1_geometry(ga, &gt, &gl) &&
+            moe1_geometry(da, &dt, &dl)) {
+            const uint32_t cus = (uint32_t)c->cu_count;
+            const uint32_t g_units = (uint32_t)(k * ga.n_mats * ((gu_rows + 15) / 16)), d_units = (uint32_t)((hidden + 15) / 16);
+            HIPCHECK(c, moe1_launch(c->stream, ga, false, std::min(cus, g_units), gt, gl));
+            HIPCHECK(c, moe1_launch(c->stream, da, true, std::min(cus, d_units), dt, dl));
+            return LARQL_OK;
+        }
+    }
     const bool route_in_launch = route_logits && tokens == 1 &&
         gemv_effective_kind(make_job(KIND_MXFP4, bank->gate_packed, bank->gate_scales, x, g, gu_rows, hidden)) == KIND_MXFP4_MFMA;
     if (route_logits && !route_in_launch)

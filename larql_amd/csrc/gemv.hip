@@ -1220,46 +1220,49 @@ __device__ __forceinline__ void run_q4k_q8k(const GemvJob &j, uint32_t tile_a, u
 // ---------------------------------------------------------------------------
 // MXFP4 on the matrix cores (rows of up to 40 x 128 elements).
 //
-// gfx950's block-scaled MFMA takes the format as stored: v_mfma_scale_f32_16x16x128_f8f6f4 with an
-// FP4 (e2m1) "B" operand wants, from lane (column j = lane%16, kg = lane/16), the 32 consecutive
-// K-elements 32kg..32kg+31 as 16 packed bytes (low nibble first) plus one e8m0 scale byte — one MXFP4
-// block of weight row j, exactly as mxfp4.rs lays it out (larql-models/src/quant/mxfp4.rs:42-95), so the
-// weights go global -> LDS -> operand registers without a single unpacking instruction and the block
-// scale is applied by the hardware.  The 16 "B" columns are 16 weight rows; a wavefront owns a K-range
-// of `cw` 128-element steps of those rows and streams its (16 rows x cw steps) tiles through a private
-// LDS ring: a 16-byte global_load_lds per lane and step for the nibbles and one 4-byte copy per tile for the scale
-// bytes of all its steps (a dword per row and step, at whatever alignment the row has; rows need at least 4 blocks).
+// v_mfma_f32_16x16x32_bf16 with the roles swapped as in the Q4_K kernel: the 16 "B" columns are 16 weight rows, the
+// "A" rows carry the activations.  Lane (column j = lane%16, kg = lane/16) owns one MXFP4 block of weight row j per
+// 128-element step — 16 packed bytes (low nibble first) and one e8m0 scale byte, exactly as mxfp4.rs lays it out
+// (larql-models/src/quant/mxfp4.rs:42-95) — and turns it into four B operands of eight bf16 each with
+// v_cvt_scalef32_pk_bf16_fp4 (two e2m1 codes times the block's power of two per instruction; every product of an e2m1
+// value and a power of two is a bf16 number, so the conversion is exact).  The weights go global -> LDS -> registers
+// as stored: a wavefront owns a K-range of `cw` 128-element steps of the tile's rows and streams its (16 rows x cw
+// steps) tiles through a private LDS ring: a 16-byte global_load_lds per lane and step for the nibbles and one 4-byte
+// copy per tile for the scale bytes of all its steps (a dword per row and step, at whatever alignment the row has;
+// rows need at least 4 blocks).
 //
-// The "A" rows carry the activation in FP4 as well: per step, n = rint(x * 2^(23-e)) (2^e > max|x| of
-// the step) is written in eight balanced base-8 digits d_t in [-4, 4] — all of them e2m1 values — and row t
-// holds digit t with the row's own e8m0 scale 2^(e-23+3(7-t)), so sum_t row_t reproduces x to 2^-24 of the
-// step's maximum; with both operands FP4 the instruction takes half the matrix-pipe time of an FP8 x FP4 one.
-// The A operand of lane (t, kg) is K = 32kg..32kg+31 of the step, laid out like the weights'.  A token takes
-// rows 0-7, a second token rows 8-15.  After the wavefront's steps, lane (j, rq) holds rows 4rq..4rq+3 of
-// column j: the digit sums of weight row j, already scaled, which it adds up (rq = 0, 1 are the first token).
-// e8m0 0 means 0.0 in the reference (the hardware reads it as 2^-127): such blocks are zeroed; 255 is NaN.
+// The activations ride in bf16 as well: x = hi + mid + lo, each term the next 8 significant bits of x (exact, so the
+// three terms reproduce the f32 value), and A row 4t + i holds term i of token t (row 4t + 3 is zero): up to four
+// tokens share one read of the weights.  MFMA m of a step takes from lane (row, kg) the elements 32kg + 8m .. + 7 of
+// the step on both sides (dword m of the lane's block), so neither operand is shuffled.  After the wavefront's steps
+// lane (j, rq) holds the three term sums of token rq for weight row j and adds them up.  Products are exact in f32
+// (8 x 8 significant bits) and accumulate in f32.
+// e8m0 0 means 0.0 in the reference and 255 NaN: the scale handed to the conversion is (byte << 23) as an f32, i.e.
+// 2^(byte-127) for 1..254 and 0.0 for 0, and a NaN for 255.
 // ---------------------------------------------------------------------------
-typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+union BfOp { bf16x8_t v; uint32_t u[4]; };
 constexpr int kMx4Stages = 3;
 constexpr int kMx4BatchTiles = 4;
-constexpr int kMx4MaxSteps = 4;    // 128-element steps per wavefront
-constexpr int kMx4MaxWaves = 10;
+constexpr int kMx4FoldTiles = 4;   // row tiles per batch of a job folded over experts
+constexpr int kMx4MaxSteps = 5;    // 128-element steps per wavefront
+constexpr int kMx4MaxWaves = 8;    // (512 threads: a 256-register budget per lane)
 constexpr uint32_t kMx4StepBytes = 1024;      // per step of a wave-tile: 64 lanes x 16 B of nibbles
-constexpr uint32_t kMx4ScaleBytes = 256;      // per wave-tile: the scale bytes of all its steps, a dword slot per (row, step)
+constexpr uint32_t kMx4ScaleBytes = 320;      // per wave-tile: the scale bytes of all its steps, a dword slot per (row, step)
+constexpr uint32_t kMx4TermBytes = 768;       // per step: three planes of 128 bf16 terms (the operand scratch)
 
-struct Mx4Step {
-    i32x8 a;        // this lane's 32 activation digits (FP4, in a[0..3]) of the step
-    int scale_a;    // e8m0 scale of this lane's digit row
-};
+// A operands of a wavefront's K-range: [step][MFMA of the step]
+struct Mx4Ops { BfOp a[kMx4MaxSteps][4]; };
 
-// Digits of one step's 128 activations, for lane (t = lane%16, kg = lane/16); x index >= k reads as 0.
-// Every lane converts two activations into their eight digits and the wavefront transposes them through
-// `scratch` (512 B of its own LDS per step: digit row t at t*64) into the operand layout.
-// The two activations of lane `lane` in step `step`, for every token of the job (the gate and up values of a gated job):
-// loaded apart from their conversion so that all steps' loads fly together (a load's first use waits for
+// The two activations of lane `lane` in step `step`, for every token of the job (the gate and up values of a gated
+// job): loaded apart from their conversion so that all steps' loads fly together (a load's first use waits for
 // everything in flight, the weight tiles included, so loads issued one step at a time cost a round trip each).
-constexpr int kMx4MaxTokens = 4;    // tokens that share one job's weights: two per 16-row A operand
-struct Mx4In { float2_t v[kMx4MaxTokens], u[kMx4MaxTokens]; };
+constexpr int kMx4MaxTokens = 4;    // tokens that share one job's weights: four A rows each
+// (As loaded: `a` and `b` are the two 8-byte reads of a lane — plain: a = x0 x1 (b repeats it); gate and up apart: a = g0 g1,
+// b = u0 u1; interleaved g0 u0 g1 u1: a = g0 u0, b = g1 u1 — taken apart when the operands are made, so that no move of
+// loaded data sits between the loads: the compiler waits for a load where its result is first touched.)
+struct Mx4In { float2_t a[kMx4MaxTokens], b[kMx4MaxTokens]; bool inside; };
 
 // The weight matrices a job reads (wave-uniform): one, or — a job folded over experts (GemvJob::combine_w) — one per
 // activation, each with its expert's bias row and combine weight; `ok` is false for an expert id outside the bank.
@@ -1278,109 +1281,136 @@ __device__ __forceinline__ Mx4In mx4_load_step(const GemvJob &j, uint32_t step, 
     const uint32_t k = (uint32_t)j.k, i0 = step * 128 + 2 * lane;
     const uint32_t ntok = mx4_tokens(j);
     Mx4In in;
+    in.inside = i0 + 2 <= k;  // k is even: a pair is inside or outside
+    const uint32_t ic = in.inside ? i0 : 0u;  // (a pair past the row end reads the row's first pair and is zeroed later)
+    const bool il = j.x_glu == j.x;
+    const float *xg = j.x_glu ? j.x_glu : j.x;
 #pragma unroll
     for (int q = 0; q < kMx4MaxTokens; q++) {
-        in.v[q] = (float2_t){0.f, 0.f}; in.u[q] = (float2_t){0.f, 0.f};
-        if ((uint32_t)q < ntok && i0 + 2 <= k) {  // k is even: a pair is inside or outside
-            const float *x = j.x + mx4_x_off(j, q);
-            if (j.x_glu == j.x) {
-                // gate and up values interleaved (the result rows of a fused gate_up matrix walked in place): g0 u0 g1 u1
-                const f32x4 w = *(const GLOBAL_AS f32x4 *)(x + 2 * (size_t)i0);
-                in.v[q].x = w.x; in.v[q].y = w.z; in.u[q].x = w.y; in.u[q].y = w.w;
-            } else {
-                in.v[q] = *(const GLOBAL_AS float2_t *)(x + i0);
-                if (j.x_glu) in.u[q] = *(const GLOBAL_AS float2_t *)(j.x_glu + mx4_x_off(j, q) + i0);
-            }
+        if ((uint32_t)q < ntok) {
+            const int64_t off = mx4_x_off(j, q);
+            const float *pa = il ? j.x + off + 2 * (size_t)ic : j.x + off + ic;
+            const float *pb = il ? j.x + off + 2 * (size_t)ic + 2 : xg + off + ic;
+            in.a[q] = *(const GLOBAL_AS float2_t *)pa;
+            in.b[q] = *(const GLOBAL_AS float2_t *)pb;
         }
     }
     return in;
 }
 
-// One token's operands of all `cw` steps of a wavefront: the digits of every step go to `scratch` (512 bytes per step:
-// digit row d at d*64) first and are read back in the operand layout afterwards, so the LDS round trip is paid once
-// per token, not once per step.  The token's eight digit rows become A rows 8*half .. 8*half+7 of `sq` (the other
-// rows are left as they are); `wq` scales the activation (a folded job's routing weight) when `scaled` is set.
+// The activation pair of token Q as the job means it: v = the values (gate values of a gated job), u = the up values
+__device__ __forceinline__ void mx4_pair(const GemvJob &j, const Mx4In &in, int q, float2_t &v, float2_t &u) {
+    const bool il = j.x_glu == j.x;
+    v.x = in.a[q].x; v.y = il ? in.b[q].x : in.a[q].y;
+    u.x = il ? in.a[q].y : in.b[q].x; u.y = in.b[q].y;
+    if (!in.inside) { v = (float2_t){0.f, 0.f}; u = (float2_t){0.f, 0.f}; }
+}
+
+// MoeGateRule::ClampedGlu (larql-compute/src/pipeline/moe.rs:88-92): g = min(g, L); u = clamp(u, -L, L);
+// (u + 1) * (g * sigmoid(alpha * g))
+__device__ __forceinline__ float clamped_glu(float g, float u, float L, float al) {
+    const float gc = fminf(g, L);
+    const float uc = u < -L ? -L : (u > L ? L : u);
+    return (uc + 1.0f) * (gc * (1.0f / (1.0f + expf(-(gc * al)))));
+}
+
+// The three bf16 terms of two activations, packed pairwise (a in the low half): x = t0 + t1 + t2 exactly.  An infinite
+// or NaN activation stays in the first term alone (its residual would be a NaN of its own making).
+__device__ __forceinline__ void mx4_terms(float a, float b, uint32_t (&t)[3]) {
+    const uint32_t ab = __builtin_bit_cast(uint32_t, a), bb = __builtin_bit_cast(uint32_t, b);
+    uint32_t a0 = ab & 0xFFFF0000u, b0 = bb & 0xFFFF0000u;
+    float ra = a - __builtin_bit_cast(float, a0), rb = b - __builtin_bit_cast(float, b0);  // exact
+    if ((ab & 0x7F800000u) == 0x7F800000u) { ra = 0.f; a0 = (ab & 0x007FFFFFu) ? (a0 | 0x00400000u) : a0; }
+    if ((bb & 0x7F800000u) == 0x7F800000u) { rb = 0.f; b0 = (bb & 0x007FFFFFu) ? (b0 | 0x00400000u) : b0; }
+    const uint32_t a1 = __builtin_bit_cast(uint32_t, ra) & 0xFFFF0000u, b1 = __builtin_bit_cast(uint32_t, rb) & 0xFFFF0000u;
+    ra -= __builtin_bit_cast(float, a1);
+    rb -= __builtin_bit_cast(float, b1);
+    const uint32_t a2 = __builtin_bit_cast(uint32_t, ra) & 0xFFFF0000u, b2 = __builtin_bit_cast(uint32_t, rb) & 0xFFFF0000u;
+    t[0] = (a0 >> 16) | b0;
+    t[1] = (a1 >> 16) | b1;
+    t[2] = (a2 >> 16) | b2;
+}
+
+// One token's operands of all `cw` steps of a wavefront: every lane splits its two activations of a step into terms
+// and the wavefront transposes them through `scratch` (768 bytes per step: term plane i at i*256, element e at 2e)
+// into the operand layout, so the LDS round trip is paid once per token.  The token's terms become A rows
+// 4*trow .. 4*trow+2 of `ops` (the other rows are left as they are); `wq` scales the activation (a folded job's
+// routing weight) when `scaled` is set.
 template <int Q>
 __device__ __forceinline__ void mx4_setup_token(const GemvJob &j, bool scaled, float wq, const Mx4In (&in)[kMx4MaxSteps],
-                                                Mx4Step (&sq)[kMx4MaxSteps], uint32_t half, uint32_t cw, uint32_t lane, uint8_t *scratch) {
-    const uint32_t t = lane & 15u, kg = lane >> 4;
-    int ex[kMx4MaxSteps];
+                                                Mx4Ops &ops, uint32_t trow, uint32_t cw, uint32_t lane, uint8_t *scratch) {
+    const uint32_t i = lane & 15u, kg = lane >> 4;
 #pragma unroll
     for (int s = 0; s < kMx4MaxSteps; s++) {
         if ((uint32_t)s >= cw) continue;
-        float2_t v = in[s].v[Q];
-        if (j.x_glu) {
-            // MoeGateRule::ClampedGlu (larql-compute/src/pipeline/moe.rs:88-92): g = min(g, L); u = clamp(u, -L, L);
-            // (u + 1) * (g * sigmoid(alpha * g))   (activations past the row end are zeros: they stay zero)
-            const float2_t u = in[s].u[Q];
-            const float L = j.glu_limit, al = j.glu_alpha;
-            const float g0 = fminf(v.x, L), g1 = fminf(v.y, L);
-            const float u0 = u.x < -L ? -L : (u.x > L ? L : u.x), u1 = u.y < -L ? -L : (u.y > L ? L : u.y);
-            v.x = (u0 + 1.0f) * (g0 * (1.0f / (1.0f + expf(-(g0 * al)))));
-            v.y = (u1 + 1.0f) * (g1 * (1.0f / (1.0f + expf(-(g1 * al)))));
+        float2_t v, u;
+        mx4_pair(j, in[s], Q, v, u);
+        if (j.x_glu) {  // (activations past the row end are zeros: they stay zero)
+            v.x = clamped_glu(v.x, u.x, j.glu_limit, j.glu_alpha);
+            v.y = clamped_glu(v.y, u.y, j.glu_limit, j.glu_alpha);
         }
         if (scaled) { v.x *= wq; v.y *= wq; }  // the expert's routing weight rides in its activation
-        const float mx = wave_max_nonneg(fmaxf(fabsf(v.x), fabsf(v.y)));
-        // mx = f * 2^ex, f in [0.5, 1): the exponent field less 126 (zero, subnormal, infinite and NaN maxima end at the clamps)
-        const int ef = (int)((__builtin_bit_cast(uint32_t, mx) >> 23) & 0xFFu);
-        ex[s] = (ef == 0 || ef == 255) ? (ef == 0 && mx > 0.f ? -100 : 0) : max(-100, min(100, ef - 126));
-        const float to_int = __builtin_bit_cast(float, (uint32_t)(127 + 23 - ex[s]) << 23);  // 2^(23 - ex)
-        // balanced base-8 digits: n + 0o44444444 has the unsigned digits d+4 (the top one may reach 8)
-        const uint32_t n0 = (uint32_t)((int)__builtin_rintf(v.x * to_int) + 0x924924), n1 = (uint32_t)((int)__builtin_rintf(v.y * to_int) + 0x924924);
-        // e2m1 codes of -4 .. 3 by unsigned digit, a nibble each: -4 = 0xE, -3 = 0xD, -2 = 0xC, -1 = 0xA, 0, 1 = 2, 2 = 4, 3 = 5 (and 4 = 6)
-        constexpr uint32_t kCodes = 0x5420ACDEu;
-#pragma unroll
-        for (int d = 0; d < 8; d++) {
-            const int sh = 3 * (7 - d);
-            uint32_t c0, c1;
-            if (d == 0) {
-                const uint32_t u0 = n0 >> 21, u1 = n1 >> 21;
-                c0 = u0 == 8u ? 6u : (kCodes >> (4 * u0)) & 15u;
-                c1 = u1 == 8u ? 6u : (kCodes >> (4 * u1)) & 15u;
-            } else {
-                c0 = (kCodes >> (4 * ((n0 >> sh) & 7u))) & 15u;
-                c1 = (kCodes >> (4 * ((n1 >> sh) & 7u))) & 15u;
-            }
-            scratch[s * 512 + d * 64 + lane] = (uint8_t)(c0 | (c1 << 4));  // low nibble first
-        }
+        uint32_t t[3];
+        mx4_terms(v.x, v.y, t);
+        uint32_t *sp = reinterpret_cast<uint32_t *>(scratch + s * kMx4TermBytes) + lane;
+        sp[0] = t[0]; sp[64] = t[1]; sp[128] = t[2];
     }
     asm volatile("" ::: "memory");  // same wavefront: LDS executes its writes before the reads that follow
-    const uint32_t row = t - 8 * half;  // (wraps for the rows of the other token)
+    if ((i >> 2) == trow && (i & 3u) < 3u) {
 #pragma unroll
-    for (int s = 0; s < kMx4MaxSteps; s++) {
-        if ((uint32_t)s >= cw) continue;
-        if (row < 8) {
-            const u32x4 op = *reinterpret_cast<const u32x4 *>(scratch + s * 512 + row * 64 + 16 * kg);  // K = 32kg .. 32kg+31
-            sq[s].a[0] = (int)op.x; sq[s].a[1] = (int)op.y; sq[s].a[2] = (int)op.z; sq[s].a[3] = (int)op.w;
-            sq[s].scale_a = 125 + ex[s] - 3 * (int)row;  // digit `row` weighs 2^(ex - 23 + 3*(7 - row))
+        for (int s = 0; s < kMx4MaxSteps; s++) {
+            if ((uint32_t)s >= cw) continue;
+            const uint8_t *rp = scratch + s * kMx4TermBytes + (i & 3u) * 256 + kg * 64;  // elements 32kg .. 32kg+31 of term i%4
+#pragma unroll
+            for (int m = 0; m < 4; m++) {
+                const u32x4 op = *reinterpret_cast<const u32x4 *>(rp + 16 * m);
+                ops.a[s][m].u[0] = op.x; ops.a[s][m].u[1] = op.y; ops.a[s][m].u[2] = op.z; ops.a[s][m].u[3] = op.w;
+            }
         }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the scratch is reused by the next token
 }
 
-__device__ __forceinline__ void mx4_clear_steps(Mx4Step (&sq)[kMx4MaxSteps]) {
+__device__ __forceinline__ void mx4_clear_ops(Mx4Ops &ops) {
 #pragma unroll
-    for (int s = 0; s < kMx4MaxSteps; s++) {
+    for (int s = 0; s < kMx4MaxSteps; s++)
 #pragma unroll
-        for (int q = 0; q < 8; q++) sq[s].a[q] = 0;
-        sq[s].scale_a = 127;
-    }
+        for (int m = 0; m < 4; m++) ops.a[s][m].u[0] = ops.a[s][m].u[1] = ops.a[s][m].u[2] = ops.a[s][m].u[3] = 0u;
 }
 
-// The operands of every token of a job: token q's eight digit rows are A rows 8(q%2) .. 8(q%2)+7 of operand q/2, so
-// its sums come out in D rows of their own.
-__device__ __forceinline__ void mx4_setup_steps(const GemvJob &j, const Mx4In (&in)[kMx4MaxSteps], Mx4Step (&st)[2][kMx4MaxSteps],
-                                                uint32_t cw, uint32_t lane, uint8_t *scratch) {
+// The operands of every token of a job: token q's terms are A rows 4q .. 4q+2, so its sums come out in D rows of
+// their own (lanes with rq = q).
+__device__ __forceinline__ void mx4_setup_ops(const GemvJob &j, const Mx4In (&in)[kMx4MaxSteps], Mx4Ops &ops, uint32_t cw,
+                                              uint32_t lane, uint8_t *scratch) {
     const uint32_t ntok = mx4_tokens(j);
-    mx4_clear_steps(st[0]);
-    mx4_clear_steps(st[1]);
-    mx4_setup_token<0>(j, false, 1.0f, in, st[0], 0, cw, lane, scratch);
-    if (ntok > 1) mx4_setup_token<1>(j, false, 1.0f, in, st[0], 1, cw, lane, scratch);
-    if (ntok > 2) mx4_setup_token<2>(j, false, 1.0f, in, st[1], 0, cw, lane, scratch);
-    if (ntok > 3) mx4_setup_token<3>(j, false, 1.0f, in, st[1], 1, cw, lane, scratch);
+    mx4_clear_ops(ops);
+    mx4_setup_token<0>(j, false, 1.0f, in, ops, 0, cw, lane, scratch);
+    if (ntok > 1) mx4_setup_token<1>(j, false, 1.0f, in, ops, 1, cw, lane, scratch);
+    if (ntok > 2) mx4_setup_token<2>(j, false, 1.0f, in, ops, 2, cw, lane, scratch);
+    if (ntok > 3) mx4_setup_token<3>(j, false, 1.0f, in, ops, 3, cw, lane, scratch);
 }
 
-#define LARQL_MX4_WAIT_CASE(CW) case CW: LARQL_WAIT_VMCNT((CW + 1) * (kMx4Stages - 1)); break;
+// One step of a wave-tile from its LDS slot: the lane's block (16 bytes of nibbles, scale byte `sc`) against the four
+// operands of the step.  `live` is false for a block past the row end or of an expert outside the bank.
+__device__ __forceinline__ f32x4 mx4_step_mfma(const BfOp (&a)[4], const u32x4 q, uint32_t sc, bool live, f32x4 D) {
+    float scale = __builtin_bit_cast(float, sc << 23);                       // 2^(sc-127); 0 -> 0.0 as the reference reads it
+    scale = sc == 255u ? __builtin_bit_cast(float, 0x7FC00000u) : scale;     // 255 -> NaN
+    scale = live ? scale : 0.0f;
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int m = 0; m < 4; m++) {
+        BfOp b;
+        b.u[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[m], scale, 0));
+        b.u[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[m], scale, 1));
+        b.u[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[m], scale, 2));
+        b.u[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[m], scale, 3));
+        D = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[m].v, b.v, D, 0, 0, 0);
+    }
+    return D;
+}
+
+// loads of the younger wave-tiles that may still be in flight: CW nibble copies and one scale copy each (two with five steps)
+#define LARQL_MX4_WAIT_CASE(CW) case CW: LARQL_WAIT_VMCNT((CW + 1 + (CW > 4)) * (kMx4Stages - 1)); break;
 
 // tiles [tile_a, tile_b) of one job
 __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, const Mx4Sel &sel, uint32_t tile_a, uint32_t tile_b, uint8_t *lds,
@@ -1389,10 +1419,9 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, const Mx4Sel &s
     const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t nw_launch = blockDim.x >> 6;
     const uint32_t jr = lane & 15u, kg = lane >> 4;
-    // up to four tokens share the weights: tokens 2q and 2q+1 ride in A operand q, their sums leave in D rows 0..7 and 8..15
+    // up to four tokens share the weights: token q rides in A rows 4q .. 4q+2, its sums leave in D rows 4q .. 4q+2 (lanes rq = q)
     const uint32_t ntok = mx4_tokens(j);
-    const bool second = ntok > 2;
-    const uint32_t hw_sh = ntok == 1 ? 1u : (ntok == 2 ? 2u : 3u), hw = 1u << hw_sh;  // partial sums per weight row and wavefront
+    const uint32_t hw_sh = ntok == 1 ? 0u : (ntok == 2 ? 1u : 2u), hw = 1u << hw_sh;  // partial sums per weight row and wavefront
     const uint32_t nwj = j.rpp, steps = j.cpr, cw = (uint32_t)j.pad, PW = nwj * hw;
     const uint32_t rows = (uint32_t)j.rows, k = (uint32_t)j.k, nb = k / 32, row_bytes = (uint32_t)j.row_bytes;
     uint8_t *ring = lds + wv * (NS * slot_bytes);
@@ -1412,6 +1441,7 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, const Mx4Sel &s
     // scale bytes: lane (jr, c) copies the dword that holds blocks 4(step0+c) .. +3 of row jr, moved back to end with the
     // row where the row has fewer; lane (jr, kg) then finds the byte of its block of step s in slot 16s + jr
     const uint32_t sc_dw = min((step0 + kg) * 4, nb - 4);
+    const uint32_t sc_dw4 = min((step0 + 4) * 4, nb - 4);
     uint32_t sc_at[kMx4MaxSteps];
 #pragma unroll
     for (int s = 0; s < kMx4MaxSteps; s++) sc_at[s] = (16u * s + jr) * 4 + (blk[s] - min((step0 + s) * 4, nb - 4));
@@ -1437,11 +1467,12 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, const Mx4Sel &s
         // the e8m0 bytes of all the wavefront's steps in one copy: lane (row jr, step c = lane/16 < cw) brings the four
         // scale bytes of its row and step as one dword into slot `lane` (the dword is not aligned in general)
         if (lane < 16 * cw) __builtin_amdgcn_global_load_lds((g_vp)(sbase + (sro + sc_dw)), (lds_vp)(lp + cw * 1024), 4, 0, 0);
+        if (cw > 4 && lane < 16) __builtin_amdgcn_global_load_lds((g_vp)(sbase + (sro + sc_dw4)), (lds_vp)(lp + cw * 1024 + 256), 4, 0, 0);  // a fifth step's
         n_issue++;
         if (it_tile < tile_b) it_tile++;
     };
     // the activations of all this wavefront's steps are requested first and together, ahead of the weight tiles in
-    // the in-order return queue; their digits are prepared while the first tiles are on their way (the ring's last
+    // the in-order return queue; their terms are prepared while the first tiles are on their way (the ring's last
     // slot is still free and serves as scratch)
     Mx4In xin[kMx4MaxSteps];
 #pragma unroll
@@ -1449,8 +1480,8 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, const Mx4Sel &s
         if (working && (uint32_t)s < cw) xin[s] = mx4_load_step(j, step0 + s, lane);
     if (working)
         for (int s = 0; s < NS - 1; s++) issue();
-    Mx4Step st[2][kMx4MaxSteps];
-    if (working) mx4_setup_steps(j, xin, st, cw, lane, ring + (NS - 1) * slot_bytes);  // (512 bytes per step fit the 1024 of a slot's step)
+    Mx4Ops ops;
+    if (working) mx4_setup_ops(j, xin, ops, cw, lane, ring + (NS - 1) * slot_bytes);  // (768 bytes per step fit the 1024 of a slot's step)
 
     // The two partial-sum areas are laid out for this job's own `hw`; the job this workgroup served before may have used
     // another layout, and its last row sums may still be read by a slower wavefront: wait for everybody before writing.
@@ -1463,30 +1494,22 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, const Mx4Sel &s
             for (uint32_t tl = 0; tl < nbt; tl++) {
                 issue();
                 switch (cw) {  // at most NS-1 younger wave-tiles in flight: the oldest has landed
-                    LARQL_MX4_WAIT_CASE(1) LARQL_MX4_WAIT_CASE(2) LARQL_MX4_WAIT_CASE(3) LARQL_MX4_WAIT_CASE(4)
+                    LARQL_MX4_WAIT_CASE(1) LARQL_MX4_WAIT_CASE(2) LARQL_MX4_WAIT_CASE(3) LARQL_MX4_WAIT_CASE(4) LARQL_MX4_WAIT_CASE(5)
                 }
                 asm volatile("" ::: "memory");
                 const uint8_t *slot = ring + (n_use % NS) * slot_bytes;
-                f32x4 D = {0.f, 0.f, 0.f, 0.f}, D2 = {0.f, 0.f, 0.f, 0.f};
+                f32x4 D = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int s = 0; s < kMx4MaxSteps; s++) {
                     if ((uint32_t)s < cw) {
                         const u32x4 q = *reinterpret_cast<const u32x4 *>(slot + s * 1024 + lane * 16);
-                        uint32_t sc = slot[cw * 1024 + sc_at[s]];
-                        const bool live = valid[s] && sc != 0;  // e8m0 0 is 0.0 here; blocks past the row end do not exist
-                        sc = valid[s] ? sc : 127u;
-                        i32x8 b = {0, 0, 0, 0, 0, 0, 0, 0};
-                        b[0] = live ? (int)q.x : 0; b[1] = live ? (int)q.y : 0; b[2] = live ? (int)q.z : 0; b[3] = live ? (int)q.w : 0;
-                        D = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st[0][s].a, b, D, 4, 4, 0, st[0][s].scale_a, 0, (int)sc);
-                        if (second) D2 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st[1][s].a, b, D2, 4, 4, 0, st[1][s].scale_a, 0, (int)sc);
+                        const uint32_t sc = slot[cw * 1024 + sc_at[s]];
+                        D = mx4_step_mfma(ops.a[s], q, sc, valid[s], D);  // (blocks past the row end do not exist)
                     }
                 }
                 n_use++;
-                const float v = (D[0] + D[1]) + (D[2] + D[3]);  // digits 4rq..4rq+3 of weight row jr
-                float *pr = pb + (tl * 16 + jr) * PW + wv * hw;
-                if (ntok == 1) { if (kg < 2) pr[kg] = v; }
-                else pr[kg] = v;
-                if (second) pr[4 + kg] = (D2[0] + D2[1]) + (D2[2] + D2[3]);
+                // the three term sums of token kg for weight row jr
+                if (kg < hw) pb[(tl * 16 + jr) * PW + wv * hw + kg] = (D[0] + D[1]) + D[2];
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -1494,18 +1517,17 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, const Mx4Sel &s
         asm volatile("" ::: "memory");
         const uint32_t row_base = (tile_a + tb) * 16;
         const uint32_t nwork = min(nwj, (steps + cw - 1) / cw);
-        // hw threads per weight row: thread h adds up slot h of every wavefront, the two halves of a token meet in one
-        // DPP step (the same order of additions per token whatever the number of tokens that share the job)
+        // hw threads per weight row: thread h adds up token h's slot of every wavefront (the same order of additions
+        // per token whatever the number of tokens that share the job)
         for (uint32_t rr = threadIdx.x >> hw_sh; rr < nbt * 16; rr += blockDim.x >> hw_sh) {
             const uint32_t h = threadIdx.x & (hw - 1u);
             float s = 0.f;
             for (uint32_t w = 0; w < nwork; w++) s += pb[rr * PW + w * hw + h];
-            s = dpp_add<0xB1>(s);  // quad_perm [1,0,3,2]
             const uint32_t row = row_base + rr;
-            if ((h & 1u) == 0 && row < rows) {
+            if (h < ntok && row < rows) {
                 if (!sel.ok[0]) s = 0.0f;  // an expert outside the bank: no contribution (its stand-in's bytes were read, not used)
                 else if (j.bias) s += ((const GLOBAL_AS float *)sel.bias[0])[(size_t)row * j.bias_step];
-                ((g_f32wp)(j.out + mx4_out_off(j, h >> 1)))[row] = s;
+                ((g_f32wp)(j.out + mx4_out_off(j, h)))[row] = s;
             }
         }
         parity ^= 1u;
@@ -1513,18 +1535,19 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, const Mx4Sel &s
 }
 
 // A job folded over experts (GemvJob::combine_w): row tiles [tile_a, tile_b) of the result, each the sum over the job's
-// `nq` experts of (that expert's 16 weight rows) . (that expert's activation, scaled by its routing weight).  The walk is
-// expert-outermost within a batch of R row tiles: one expert's operands are prepared while its tiles are already on their
-// way, its tiles accumulate into the row tiles' own D registers, then the next expert follows; the D registers hold
-// sum_q w_q * (W_q . act_q) when the batch is written out.  One operand set lives at a time.
+// `nq` experts of (that expert's 16 weight rows) . (that expert's activation, scaled by its routing weight).  Expert q's
+// activation terms are A rows 4q .. 4q+2 of ONE operand set, prepared once per job; expert q's weights meet the whole
+// set and accumulate into that expert's own D registers, of which only rows 4q .. 4q+2 (lanes rq = q) mean anything:
+// lane (j, rq) ends with expert rq's three term sums for weight row j, and the experts meet in the fold of the row
+// partials.  The walk is expert-outermost within a batch of R row tiles.
 __device__ __forceinline__ void run_mxfp4_fold(const GemvJob &j, const Mx4Sel &sel, uint32_t tile_a, uint32_t tile_b, uint8_t *lds,
                                                uint32_t slot_bytes, uint32_t &parity) {
-    constexpr int NS = kMx4Stages, R = kMx4BatchTiles;
+    constexpr int NS = kMx4Stages, R = kMx4FoldTiles;
     const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t nw_launch = blockDim.x >> 6;
     const uint32_t jr = lane & 15u, kg = lane >> 4;
     const uint32_t nq = mx4_tokens(j);
-    constexpr uint32_t hw = 2, hw_sh = 1;  // the digit rows 0-7 of the one live operand: two partial sums per weight row and wavefront
+    constexpr uint32_t hw = 4, hw_sh = 2;  // one partial sum per expert, weight row and wavefront
     const uint32_t nwj = j.rpp, steps = j.cpr, cw = (uint32_t)j.pad, PW = nwj * hw;
     const uint32_t rows = (uint32_t)j.rows, k = (uint32_t)j.k, nb = k / 32, row_bytes = (uint32_t)j.row_bytes;
     uint8_t *ring = lds + wv * (NS * slot_bytes);
@@ -1541,6 +1564,7 @@ __device__ __forceinline__ void run_mxfp4_fold(const GemvJob &j, const Mx4Sel &s
         blk[s] = min(b, nb - 1);
     }
     const uint32_t sc_dw = min((step0 + kg) * 4, nb - 4);
+    const uint32_t sc_dw4 = min((step0 + 4) * 4, nb - 4);
     uint32_t sc_at[kMx4MaxSteps];
 #pragma unroll
     for (int s = 0; s < kMx4MaxSteps; s++) sc_at[s] = (16u * s + jr) * 4 + (blk[s] - min((step0 + s) * 4, nb - 4));
@@ -1566,6 +1590,7 @@ __device__ __forceinline__ void run_mxfp4_fold(const GemvJob &j, const Mx4Sel &s
         for (int s = 0; s < kMx4MaxSteps; s++)
             if ((uint32_t)s < cw) __builtin_amdgcn_global_load_lds((g_vp)(wbase + (wro + blk[s] * 16)), (lds_vp)(lp + s * 1024), 16, 0, 0);
         if (lane < 16 * cw) __builtin_amdgcn_global_load_lds((g_vp)(sbase + (sro + sc_dw)), (lds_vp)(lp + cw * 1024), 4, 0, 0);
+        if (cw > 4 && lane < 16) __builtin_amdgcn_global_load_lds((g_vp)(sbase + (sro + sc_dw4)), (lds_vp)(lp + cw * 1024 + 256), 4, 0, 0);  // a fifth step's
         n_issue++;
         if (it_tb < nt) {  // next virtual tile (stays on the last one once the list is exhausted)
             const uint32_t nbt = min((uint32_t)R, nt - it_tb);
@@ -1583,56 +1608,57 @@ __device__ __forceinline__ void run_mxfp4_fold(const GemvJob &j, const Mx4Sel &s
     if (working)
         for (int s = 0; s < NS - 1; s++) issue();
 
+    // every expert's operands, once per job (the ring's last slot is still free and serves as scratch)
+    Mx4Ops ops;
+    if (working) {
+        uint8_t *scratch = ring + (NS - 1) * slot_bytes;
+        mx4_clear_ops(ops);
+        mx4_setup_token<0>(j, true, sel.cw[0], xin, ops, 0, cw, lane, scratch);
+        if (nq > 1) mx4_setup_token<1>(j, true, sel.cw[1], xin, ops, 1, cw, lane, scratch);
+        if (nq > 2) mx4_setup_token<2>(j, true, sel.cw[2], xin, ops, 2, cw, lane, scratch);
+        if (nq > 3) mx4_setup_token<3>(j, true, sel.cw[3], xin, ops, 3, cw, lane, scratch);
+    }
     __builtin_amdgcn_s_barrier();  // (the partial-sum areas follow this job's layout: see run_mxfp4_mfma)
     uint32_t n_use = 0;
-    Mx4Step st[kMx4MaxSteps];
     for (uint32_t tb = 0; tb < nt; tb += R) {
         float *pb = part + parity * (R * 16 * nw_launch * hw);
         const uint32_t nbt = min((uint32_t)R, nt - tb);
         if (working) {
-            f32x4 D[R];
+            float acc[R];  // this lane's expert (rq = kg) only
 #pragma unroll
-            for (int t = 0; t < R; t++) D[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            for (int t = 0; t < R; t++) acc[t] = 0.f;
 #pragma unroll
             for (int q = 0; q < kMx4MaxTokens; q++) {
                 if ((uint32_t)q >= nq) break;
-                // this expert's operands; the scratch is the ring slot the next copy will fill (nothing is in flight into it)
-                mx4_clear_steps(st);
-                uint8_t *scratch = ring + ((n_use + NS - 1) % NS) * slot_bytes;
-                if (q == 0) mx4_setup_token<0>(j, true, sel.cw[0], xin, st, 0, cw, lane, scratch);
-                else if (q == 1) mx4_setup_token<1>(j, true, sel.cw[1], xin, st, 0, cw, lane, scratch);
-                else if (q == 2) mx4_setup_token<2>(j, true, sel.cw[2], xin, st, 0, cw, lane, scratch);
-                else mx4_setup_token<3>(j, true, sel.cw[3], xin, st, 0, cw, lane, scratch);
 #pragma unroll
                 for (int tl = 0; tl < R; tl++) {
                     if ((uint32_t)tl >= nbt) break;
                     issue();
                     switch (cw) {
-                        LARQL_MX4_WAIT_CASE(1) LARQL_MX4_WAIT_CASE(2) LARQL_MX4_WAIT_CASE(3) LARQL_MX4_WAIT_CASE(4)
+                        LARQL_MX4_WAIT_CASE(1) LARQL_MX4_WAIT_CASE(2) LARQL_MX4_WAIT_CASE(3) LARQL_MX4_WAIT_CASE(4) LARQL_MX4_WAIT_CASE(5)
                     }
                     asm volatile("" ::: "memory");
                     const uint8_t *slot = ring + (n_use % NS) * slot_bytes;
+                    f32x4 D = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                     for (int s = 0; s < kMx4MaxSteps; s++) {
                         if ((uint32_t)s < cw) {
                             const u32x4 qw = *reinterpret_cast<const u32x4 *>(slot + s * 1024 + lane * 16);
-                            uint32_t sc = slot[cw * 1024 + sc_at[s]];
-                            // e8m0 0 is 0.0 here; blocks past the row end do not exist; an expert outside the bank has no weights
-                            const bool live = valid[s] && sc != 0 && sel.ok[q];
-                            sc = valid[s] ? sc : 127u;
-                            i32x8 b = {0, 0, 0, 0, 0, 0, 0, 0};
-                            b[0] = live ? (int)qw.x : 0; b[1] = live ? (int)qw.y : 0; b[2] = live ? (int)qw.z : 0; b[3] = live ? (int)qw.w : 0;
-                            D[tl] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(st[s].a, b, D[tl], 4, 4, 0, st[s].scale_a, 0, (int)sc);
+                            const uint32_t sc = slot[cw * 1024 + sc_at[s]];
+                            // blocks past the row end do not exist; an expert outside the bank has no weights
+                            D = mx4_step_mfma(ops.a[s], qw, sc, valid[s] && sel.ok[q], D);
                         }
                     }
                     n_use++;
+                    // rows 4q .. 4q+2 of D are expert q's term sums; the other rows met another expert's activation
+                    if (kg == (uint32_t)q) acc[tl] = (D[0] + D[1]) + D[2];
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the slot's reads are done before anything reuses it
                 }
             }
 #pragma unroll
             for (int tl = 0; tl < R; tl++) {
                 if ((uint32_t)tl >= nbt) break;
-                if (kg < 2) pb[(tl * 16 + jr) * PW + wv * hw + kg] = (D[tl][0] + D[tl][1]) + (D[tl][2] + D[tl][3]);
+                pb[(tl * 16 + jr) * PW + wv * hw + kg] = kg < nq ? acc[tl] : 0.f;
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -1644,7 +1670,8 @@ __device__ __forceinline__ void run_mxfp4_fold(const GemvJob &j, const Mx4Sel &s
             const uint32_t h = threadIdx.x & (hw - 1u);
             float s = 0.f;
             for (uint32_t w = 0; w < nwork; w++) s += pb[rr * PW + w * hw + h];
-            s = dpp_add<0xB1>(s);  // quad_perm [1,0,3,2]
+            s = dpp_add<0xB1>(s);  // quad_perm [1,0,3,2]: experts 0+1, 2+3
+            s = dpp_add<0x4E>(s);  // quad_perm [2,3,0,1]: all four
             const uint32_t row = row_base + rr;
             if (h == 0 && row < rows) {
                 if (j.bias) {  // + sum_q w_q * bias_q[row], in selection order
@@ -1660,6 +1687,290 @@ __device__ __forceinline__ void run_mxfp4_fold(const GemvJob &j, const Mx4Sel &s
 }
 
 // ---------------------------------------------------------------------------
+// One token through k <= 4 experts of an MXFP4 bank (the decode shape of ExpertWeightFfn::moe_block,
+// larql-compute/src/ffn/expert_weight/mod.rs, with the pipeline of larql-compute/src/pipeline/moe.rs:469-541): one launch for the gate / up
+// projections of the selected experts, one for the down projections folded over the experts.  The arithmetic is the
+// matrix-core scheme above (same operands, same order of additions per row as a one-token job of the general kernel);
+// what differs is the way in: the arguments are a small block in the kernel's own argument space, the token's
+// activations are requested before anything else, the selection (or the read of it) overlaps them, and a deeper ring
+// (up to four wave-tiles in flight per wavefront) covers the memory latency of a launch that lasts only a few
+// round trips.
+//   gate/up stage: the 16-row tiles of the k x n_mats matrices form one list, shared out evenly over the workgroups.
+//                  With a fused interleaved matrix (gate row 2i, up row 2i+1) the fold of the row partials has both
+//                  halves of an output side by side: it applies ClampedGlu and writes the activation of the down stage
+//                  already split into its three bf16 terms (`terms`: [term][slot < k][kpad] bf16), so the down stage
+//                  loads its A operands as stored.
+//   down stage:    a workgroup owns row tiles of the result; expert q's activation is A rows 4q .. 4q+2 of one operand
+//                  set, each expert's tile meets the whole set and lane (j, rq) keeps expert rq's sums, scaled by the
+//                  expert's routing weight; the experts meet in the fold of the row partials, the biases (weighted)
+//                  join there.  Without `terms` (gate and up apart) the activations are gated and split here.
+// ---------------------------------------------------------------------------
+constexpr int kMoe1BatchTiles = 4;
+constexpr int moe1_stages(int cw) { return cw <= 3 ? 5 : 3; }  // ring slots per wavefront that fit the LDS beside the partials
+
+// CW: 128-element steps per wavefront (the row length decides); NS: ring slots per wavefront
+template <bool DOWN, int CW, int NS>
+__global__ void __launch_bounds__(kMx4MaxWaves * 64) moe1_kernel(const Moe1Args A) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t m1_lds[];
+    constexpr int R = kMoe1BatchTiles;
+    constexpr uint32_t cw = CW, slot_bytes = CW * kMx4StepBytes + kMx4ScaleBytes;
+    const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t nw_launch = blockDim.x >> 6;
+    const uint32_t jr = lane & 15u, kg = lane >> 4;
+    const uint32_t kdim = A.kdim, nb = kdim / 32, row_bytes = nb * 16, steps = (kdim + 127) / 128, nwj = A.nw;
+    const uint32_t rows = A.rows, nq = min(A.k, kMoe1MaxK);
+    uint8_t *ring = m1_lds + wv * (NS * slot_bytes);
+    float *part = reinterpret_cast<float *>(m1_lds + nw_launch * (NS * slot_bytes));
+    const uint32_t step0 = wv * cw;
+    const bool working = wv < nwj && step0 < steps;
+
+    // 1. the activations of this wavefront's K-range: nothing they need has to be waited for
+    GemvJob jx = {};  // (the fields the activation helpers read)
+    jx.k = kdim; jx.x = A.x; jx.x_glu = A.x_glu; jx.glu_limit = A.glu_limit; jx.glu_alpha = A.glu_alpha;
+    if (DOWN) { jx.batch = nq; jx.x_stride = A.x_slot_stride; jx.x_off[0] = (int64_t)(2 * A.x_slot_stride); jx.x_off[1] = (int64_t)(3 * A.x_slot_stride); }
+    Mx4In xin[kMx4MaxSteps];
+    Mx4Ops ops;
+    const bool pre = DOWN && A.terms != nullptr;  // the activations arrive as operand terms
+    if (pre) {
+        // lane (row i = 4q + term, kg): eight consecutive bf16 of term plane `term`, slot q, per MFMA
+        const uint32_t tq = jr >> 2, term = jr & 3u;
+        const bool mine = working && tq < nq && term < 3u;
+        const uint16_t *tp = A.terms + ((size_t)(mine ? term : 0u) * nq + (mine ? tq : 0u)) * A.terms_kpad;
+#pragma unroll
+        for (int s = 0; s < CW; s++) {
+#pragma unroll
+            for (int m = 0; m < 4; m++) {
+                const uint32_t el = (step0 + s) * 128 + 32 * kg + 8 * m;
+                const bool in_row = mine && el < kdim;  // (kdim % 32 == 0: a group of eight is inside or outside)
+                const u32x4 t = *(const GLOBAL_AS u32x4 *)(tp + (in_row ? el : 0u));
+                ops.a[s][m].u[0] = in_row ? t.x : 0u; ops.a[s][m].u[1] = in_row ? t.y : 0u;
+                ops.a[s][m].u[2] = in_row ? t.z : 0u; ops.a[s][m].u[3] = in_row ? t.w : 0u;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int s = 0; s < CW; s++)
+            if (working) xin[s] = mx4_load_step(jx, step0 + s, lane);
+    }
+
+    // 2. the selection
+    uint32_t e[kMoe1MaxK];
+    float cwt[kMoe1MaxK];
+    bool ok[kMoe1MaxK];
+    if (A.logits) {
+        uint32_t idx[kRouterMaxK];
+        float wt[kRouterMaxK];
+        const bool writer = A.experts && blockIdx.x == 0 && wv == 0;  // (wave-uniform)
+        if (writer || DOWN) router_select_wave<true>(A.logits, A.router_bias, A.n_experts, nq, A.policy, lane, idx, wt);
+        else router_select_wave<false>(A.logits, A.router_bias, A.n_experts, nq, A.policy, lane, idx, wt);
+#pragma unroll
+        for (int q = 0; q < (int)kMoe1MaxK; q++) {
+            e[q] = __builtin_amdgcn_readfirstlane(idx[q]);
+            cwt[q] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, wt[q])));
+        }
+        if (writer && lane == 0) {
+#pragma unroll
+            for (int r = 0; r < (int)kMoe1MaxK; r++)
+                if ((uint32_t)r < nq) { A.experts[r] = idx[r]; A.weights[r] = wt[r]; }
+        }
+    } else {
+        const uint32_t ev = lane < nq ? ((const GLOBAL_AS uint32_t *)A.experts)[lane] : 0u;
+        const float wl = (DOWN && lane < nq) ? ((const GLOBAL_AS float *)A.weights)[lane] : 0.0f;
+#pragma unroll
+        for (int q = 0; q < (int)kMoe1MaxK; q++) {
+            e[q] = (uint32_t)__builtin_amdgcn_readlane((int)ev, q);
+            cwt[q] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wl), q));
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < (int)kMoe1MaxK; q++) {
+        ok[q] = (uint32_t)q < nq && e[q] < A.n_experts;  // an id outside the bank contributes nothing and reads nothing of it
+        e[q] = ok[q] ? e[q] : 0u;
+        cwt[q] = ok[q] ? cwt[q] : 0.0f;
+    }
+    auto expert_of = [&](uint32_t q) { return q == 1 ? e[1] : (q == 2 ? e[2] : (q == 3 ? e[3] : e[0])); };
+    auto ok_of = [&](uint32_t q) { return q == 1 ? ok[1] : (q == 2 ? ok[2] : (q == 3 ? ok[3] : ok[0])); };
+    auto weight_of = [&](uint32_t q) { return q == 1 ? cwt[1] : (q == 2 ? cwt[2] : (q == 3 ? cwt[3] : cwt[0])); };
+
+    // 3. this workgroup's share.  Gate/up: virtual tiles [va, vb) of the list (slot, matrix, row tile); down: row tiles.
+    const uint32_t tpm = (rows + 15) / 16;
+    const uint32_t n_units = DOWN ? tpm : nq * A.n_mats * tpm;
+    const uint32_t va = n_units * blockIdx.x / gridDim.x, vb = n_units * (blockIdx.x + 1) / gridDim.x;  // (the host keeps the products below 2^32)
+    if (va >= vb) return;
+    const uint32_t nt = vb - va;
+
+    // per-lane parts of a wave-tile's addresses: the lane's row within the tile and its block of each step
+    uint32_t woff[CW], sc_at[CW];
+    bool valid[CW];
+    bool all_valid = true;
+#pragma unroll
+    for (int s = 0; s < CW; s++) {
+        const uint32_t b = (step0 + s) * 4 + kg, bc = min(b, nb - 1);
+        valid[s] = working && b < nb;
+        all_valid = all_valid && valid[s];
+        woff[s] = jr * row_bytes + bc * 16;
+        sc_at[s] = (16u * s + jr) * 4 + (bc - min((step0 + s) * 4, nb - 4));
+    }
+    const uint32_t sc_dw = min((step0 + kg) * 4, nb - 4), sc_dw4 = min((step0 + 4) * 4, nb - 4);
+    const uint32_t soff = jr * nb + sc_dw, soff4 = jr * nb + sc_dw4;
+    const uint32_t tile_w = 16 * row_bytes, tile_s = 16 * nb;
+
+    // issue cursor.  Gate/up: (segment = slot * n_mats + matrix, row tile) walking the list; down: (batch, expert, tile of the batch)
+    uint32_t it_seg = DOWN ? 0u : va / tpm, it_t = DOWN ? 0u : va - (va / tpm) * tpm, it_left = nt;
+    uint32_t it_tb = 0, it_q = 0, it_tl = 0, slot_i = 0;
+    auto issue = [&]() {
+        uint32_t q, m, t;
+        if (DOWN) { q = it_q; m = 0; t = min(va + it_tb + it_tl, vb - 1); }
+        else { q = A.n_mats == 2 ? it_seg >> 1 : it_seg; m = A.n_mats == 2 ? (it_seg & 1u) : 0u; t = it_t; }
+        const uint32_t ex = expert_of(q);
+        const uint8_t *wbase = (m ? A.w[1] : A.w[0]) + ((size_t)ex * A.w_stride + (size_t)t * tile_w);
+        const uint8_t *sbase = (m ? A.aux[1] : A.aux[0]) + ((size_t)ex * A.aux_stride + (size_t)t * tile_s);
+        uint8_t *lp = ring + slot_i * slot_bytes;
+        if (t * 16 + 16 > rows) {  // ragged last tile of a matrix: the lane's row is clamped into it
+            const uint32_t rl = min(jr, rows - 1 - t * 16), back = (jr - rl);
+#pragma unroll
+            for (int s = 0; s < CW; s++)
+                __builtin_amdgcn_global_load_lds((g_vp)(wbase + (woff[s] - back * row_bytes)), (lds_vp)(lp + s * 1024), 16, 0, 0);
+            if (CW >= 4 || lane < 16 * cw) __builtin_amdgcn_global_load_lds((g_vp)(sbase + (soff - back * nb)), (lds_vp)(lp + cw * 1024), 4, 0, 0);
+            if (CW > 4 && lane < 16) __builtin_amdgcn_global_load_lds((g_vp)(sbase + (soff4 - back * nb)), (lds_vp)(lp + cw * 1024 + 256), 4, 0, 0);
+        } else {
+#pragma unroll
+            for (int s = 0; s < CW; s++)
+                __builtin_amdgcn_global_load_lds((g_vp)(wbase + woff[s]), (lds_vp)(lp + s * 1024), 16, 0, 0);
+            if (CW >= 4 || lane < 16 * cw) __builtin_amdgcn_global_load_lds((g_vp)(sbase + soff), (lds_vp)(lp + cw * 1024), 4, 0, 0);
+            if (CW > 4 && lane < 16) __builtin_amdgcn_global_load_lds((g_vp)(sbase + soff4), (lds_vp)(lp + cw * 1024 + 256), 4, 0, 0);
+        }
+        slot_i = slot_i + 1 == NS ? 0u : slot_i + 1;
+        // next wave-tile; past the end the last one again (uniform load counts)
+        if (DOWN) {
+            if (it_tb < nt) {
+                const uint32_t nbt = min((uint32_t)R, nt - it_tb);
+                if (++it_tl >= nbt) {
+                    it_tl = 0;
+                    if (++it_q >= nq) { it_q = 0; it_tb += R; }
+                }
+                if (it_tb >= nt) { it_tb = nt - 1 - ((nt - 1) % R); it_q = nq - 1; it_tl = (nt - 1) % R; }
+            }
+        } else if (it_left > 1) {
+            it_left--;
+            if (++it_t >= tpm) { it_t = 0; it_seg++; }
+        }
+    };
+    if (working)
+        for (int s = 0; s + 1 < NS; s++) issue();
+
+    // 4. operands, while the first tiles fly (the ring's last slot is still free and serves as scratch)
+    if (working && !pre) {
+        uint8_t *scratch = ring + (NS - 1) * slot_bytes;
+        mx4_clear_ops(ops);
+        mx4_setup_token<0>(jx, false, 1.0f, xin, ops, 0, cw, lane, scratch);
+        if (DOWN) {
+            if (nq > 1) mx4_setup_token<1>(jx, false, 1.0f, xin, ops, 1, cw, lane, scratch);
+            if (nq > 2) mx4_setup_token<2>(jx, false, 1.0f, xin, ops, 2, cw, lane, scratch);
+            if (nq > 3) mx4_setup_token<3>(jx, false, 1.0f, xin, ops, 3, cw, lane, scratch);
+        }
+    }
+
+    constexpr uint32_t hw = DOWN ? 4u : 1u;  // partial sums per weight row and wavefront (down: one per expert)
+    const uint32_t PW = nwj * hw, nwork = min(nwj, (steps + cw - 1) / cw);
+    uint32_t use_i = 0, parity = 0;
+    uint32_t f_seg = DOWN ? 0u : va / tpm, f_t = DOWN ? va : va - (va / tpm) * tpm;  // the fold's cursor (first tile of the batch)
+    for (uint32_t tb = 0; tb < nt; tb += R) {
+        float *pb = part + parity * (R * 16 * nw_launch * hw);
+        const uint32_t nbt = min((uint32_t)R, nt - tb);
+        if (working) {
+            float acc[R];
+#pragma unroll
+            for (int t = 0; t < R; t++) acc[t] = 0.f;
+#pragma unroll
+            for (int q = 0; q < (int)kMoe1MaxK; q++) {
+                if (DOWN ? (uint32_t)q >= nq : q >= 1) break;
+#pragma unroll
+                for (int tl = 0; tl < R; tl++) {
+                    if ((uint32_t)tl >= nbt) break;
+                    issue();
+                    LARQL_WAIT_VMCNT((CW + 1 + (CW > 4)) * (NS - 1));  // at most NS-1 younger wave-tiles in flight: the oldest has landed
+                    asm volatile("" ::: "memory");
+                    const uint8_t *slot = ring + use_i * slot_bytes;
+                    f32x4 D = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int s = 0; s < CW; s++) {
+                        const u32x4 qw = *reinterpret_cast<const u32x4 *>(slot + s * 1024 + lane * 16);
+                        const uint32_t sc = slot[cw * 1024 + sc_at[s]];
+                        D = mx4_step_mfma(ops.a[s], qw, sc, all_valid || valid[s], D);  // (an expert outside the bank: its result is dropped in the fold)
+                    }
+                    use_i = use_i + 1 == NS ? 0u : use_i + 1;
+                    if (kg == (uint32_t)q) acc[tl] = (D[0] + D[1]) + D[2];  // (rows 4q .. 4q+2: this expert's / the token's term sums)
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the slot's reads are done before anything reuses it
+                }
+            }
+#pragma unroll
+            for (int tl = 0; tl < R; tl++) {
+                if ((uint32_t)tl >= nbt) break;
+                if (DOWN) pb[(tl * 16 + jr) * PW + wv * hw + kg] = ok_of(kg) ? acc[tl] * weight_of(kg) : 0.f;
+                else if (kg == 0) pb[(tl * 16 + jr) * PW + wv] = acc[tl];
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (DOWN) {
+            // four threads per result row: thread h adds up expert h's slot of every wavefront, then the experts meet
+            const uint32_t row_base = (va + tb) * 16;
+            for (uint32_t rr = threadIdx.x >> 2; rr < nbt * 16; rr += blockDim.x >> 2) {
+                const uint32_t h = threadIdx.x & 3u;
+                float s = 0.f;
+                for (uint32_t w = 0; w < nwork; w++) s += pb[rr * PW + w * hw + h];
+                s = dpp_add<0xB1>(s);  // quad_perm [1,0,3,2]: experts 0+1, 2+3
+                s = dpp_add<0x4E>(s);  // quad_perm [2,3,0,1]: all four
+                const uint32_t row = row_base + rr;
+                if (h == 0 && row < rows) {
+                    if (A.bias[0]) {  // + sum_q w_q * bias_q[row], in selection order
+#pragma unroll
+                        for (int q = 0; q < (int)kMoe1MaxK; q++)
+                            if (ok[q]) s += cwt[q] * ((const GLOBAL_AS float *)A.bias[0])[(size_t)e[q] * A.bias_stride + (size_t)row * A.bias_step];
+                    }
+                    ((g_f32wp)A.out[0])[row] = s;
+                }
+            }
+        } else {
+            for (uint32_t rr = threadIdx.x; rr < nbt * 16; rr += blockDim.x) {
+                float s = 0.f;
+                for (uint32_t w = 0; w < nwork; w++) s += pb[rr * PW + w];
+                // the tile of this row: `rr / 16` tiles past the batch's first
+                uint32_t seg = f_seg, t = f_t + (rr >> 4);
+                while (t >= tpm) { t -= tpm; seg++; }
+                const uint32_t q = A.n_mats == 2 ? seg >> 1 : seg, m = A.n_mats == 2 ? (seg & 1u) : 0u;
+                const uint32_t row = t * 16 + (rr & 15u);
+                if (row < rows) {
+                    const float *bias = m ? A.bias[1] : A.bias[0];
+                    if (!ok_of(q)) s = 0.0f;  // an expert outside the bank: no contribution (its stand-in's bytes were read, not used)
+                    else if (bias) s += ((const GLOBAL_AS float *)bias)[(size_t)expert_of(q) * A.bias_stride + (size_t)row * A.bias_step];
+                }
+                if (A.terms) {
+                    // rows 2i (gate) and 2i+1 (up) sit in neighbouring lanes (rows and the block size are even)
+                    const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, s), 0xB1, 0xF, 0xF, false));  // quad_perm [1,0,3,2]
+                    if ((row & 1u) == 0 && row + 1 < rows) {
+                        const float hv = ok_of(q) ? clamped_glu(s, other, A.glu_limit, A.glu_alpha) : 0.0f;
+                        uint32_t t[3];
+                        mx4_terms(hv, 0.0f, t);
+                        uint16_t *tp = A.terms + (size_t)q * A.terms_kpad + (row >> 1);
+                        const size_t plane = (size_t)nq * A.terms_kpad;
+                        tp[0] = (uint16_t)t[0]; tp[plane] = (uint16_t)t[1]; tp[2 * plane] = (uint16_t)t[2];
+                    }
+                } else if (row < rows) {
+                    ((g_f32wp)((m ? A.out[1] : A.out[0]) + (size_t)q * A.out_slot_stride))[row] = s;
+                }
+            }
+            f_t += nbt;
+            while (f_t >= tpm) { f_t -= tpm; f_seg++; }
+        }
+        parity ^= 1u;
+    }
+    LARQL_WAIT_VMCNT(0);
+}
+
+// ---------------------------------------------------------------------------
 // bf16 rows against 2..8 activations at once (gate-KNN over several residual positions): the gate
 // matrix is read once.  v_mfma_f32_16x16x32_bf16 with the roles swapped as above: the 16 "B" columns are
 // 16 weight rows (a lane's operand is 16 contiguous bytes of its row, straight from the LDS ring), the
@@ -1670,15 +1981,12 @@ __device__ __forceinline__ void run_mxfp4_fold(const GemvJob &j, const Mx4Sel &s
 // three term sums of position 4s + rq for weight row j.  Dot as bf16_dot_portable
 // (larql-vindex/.../opplan/exec/cpu/kernels.rs:718-723); only the summation order differs.
 // ---------------------------------------------------------------------------
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 constexpr int kBfStages = 3;
 constexpr int kBfBatchTiles = 2;
 constexpr int kBfMaxPasses = 2;
 constexpr int kBfMaxSets = 2;       // 4 positions each
 constexpr int kBfMaxWaves = 10;
 constexpr uint32_t kBfTileBytes = 4 * 1024;  // 16 rows x 4 steps x 64 B
-
-union BfOp { bf16x8_t v; uint32_t u[4]; };
 
 __device__ __forceinline__ uint32_t bf16_term_bits(float &r) {  // next 8 significant bits of r; r keeps the rest
     const uint32_t b = __builtin_bit_cast(uint32_t, r) & 0xFFFF0000u;
@@ -2205,7 +2513,6 @@ __device__ __forceinline__ void run_q8_0(const GemvJob &j, uint32_t p0, uint32_t
     const uint32_t c = active ? t % cpr : 0, rl = active ? t / cpr : 0;
     X32Slice xs;
     load_x32(xs, j.x, c);
-    const size_t row_bytes = j.row_bytes;
     for (uint32_t tp = p0; tp < p1; tp += kTilePasses) {
         const uint32_t tp_end = min(p1, tp + kTilePasses);
         const uint32_t row_base = tp * rpp;
@@ -2359,7 +2666,6 @@ __device__ __forceinline__ void run_q4_0(const GemvJob &j, uint32_t p0, uint32_t
     Q8ActSlice xs;
     // for Q4_0 the job's x is the int8 code stream and aux the f32 block scales
     load_q8act(xs, reinterpret_cast<const int8_t *>(j.x), reinterpret_cast<const float *>(j.aux), c);
-    const size_t row_bytes = j.row_bytes;
     for (uint32_t tp = p0; tp < p1; tp += kTilePasses) {
         const uint32_t tp_end = min(p1, tp + kTilePasses);
         const uint32_t row_base = tp * rpp;
@@ -3030,9 +3336,8 @@ size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
     }
     if (n > 0 && jobs[0].kind == KIND_MXFP4_MFMA) {
         const size_t nw = threads / 64;
-        uint32_t batch = 1;  // the partial sums per weight row and wavefront follow the largest job (a folded job never needs more than 4)
-        for (size_t i = 0; i < n; i++) batch = std::max(batch, jobs[i].combine_w ? 1u : jobs[i].batch);
-        return nw * kMx4Stages * gemv_launch_param(jobs, n) + 2 * (size_t)kMx4BatchTiles * 16 * nw * (batch > 2 ? 8 : 4) * sizeof(float);
+        // ring + two partial-sum areas of up to four sums (tokens, or folded experts) per weight row and wavefront
+        return nw * kMx4Stages * gemv_launch_param(jobs, n) + 2 * (size_t)kMx4BatchTiles * 16 * nw * 4 * sizeof(float);
     }
     if (n > 0 && jobs[0].kind == KIND_Q4K_Q8K) {  // rings + one partial per (row, super-block), double-buffered
         const size_t nw = threads / 64;
@@ -3068,6 +3373,50 @@ uint32_t gemv_wgs_per_cu(int kind, uint32_t threads, size_t lds, uint32_t dflt) 
     const uint32_t by_lds = (uint32_t)((160 * 1024) / lds), by_waves = 12 / (threads / 64);
     const uint32_t w = by_lds < by_waves ? by_lds : by_waves;
     return w < 1 ? 1 : w;
+}
+
+bool moe1_geometry(Moe1Args &A, uint32_t *threads, size_t *lds) {
+    if (A.kdim < 128 || A.kdim % 32 != 0 || A.rows == 0 || A.rows >= (1u << 22) || A.k == 0 || A.k > kMoe1MaxK) return false;
+    const uint64_t steps = ((uint64_t)A.kdim + 127) / 128;
+    const uint32_t cw = mx4_steps_per_wave(steps);
+    if (cw == 0) return false;
+    const uint32_t nw = (uint32_t)((steps + cw - 1) / cw);
+    const size_t slot = (size_t)cw * kMx4StepBytes + kMx4ScaleBytes;
+    const size_t partials = 2 * (size_t)kMoe1BatchTiles * 16 * nw * 4 * sizeof(float);
+    A.cw = cw;
+    A.nw = nw;
+    A.stages = (uint32_t)moe1_stages((int)cw);
+    *threads = nw * 64;
+    *lds = nw * A.stages * slot + partials;
+    return *lds <= 160 * 1024;
+}
+
+template <bool DOWN, int CW>
+static hipError_t moe1_launch_cw(hipStream_t s, const Moe1Args &A, uint32_t grid, uint32_t threads, size_t lds) {
+    static std::atomic<bool> attr_set{false};  // dynamic LDS above 64 KB has to be allowed once per kernel
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void *)moe1_kernel<DOWN, CW, moe1_stages(CW)>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((moe1_kernel<DOWN, CW, moe1_stages(CW)>), dim3(grid), dim3(threads), lds, s, A);
+    return hipGetLastError();
+}
+
+template <bool DOWN>
+static hipError_t moe1_launch_stage(hipStream_t s, const Moe1Args &A, uint32_t grid, uint32_t threads, size_t lds) {
+    switch (A.cw) {
+        case 1: return moe1_launch_cw<DOWN, 1>(s, A, grid, threads, lds);
+        case 2: return moe1_launch_cw<DOWN, 2>(s, A, grid, threads, lds);
+        case 3: return moe1_launch_cw<DOWN, 3>(s, A, grid, threads, lds);
+        case 4: return moe1_launch_cw<DOWN, 4>(s, A, grid, threads, lds);
+        case 5: return moe1_launch_cw<DOWN, 5>(s, A, grid, threads, lds);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t moe1_launch(hipStream_t s, const Moe1Args &A, bool down, uint32_t grid, uint32_t threads, size_t lds) {
+    return down ? moe1_launch_stage<true>(s, A, grid, threads, lds) : moe1_launch_stage<false>(s, A, grid, threads, lds);
 }
 
 hipError_t gemv_launch(hipStream_t stream, int kind, const GemvLaunch &L, uint32_t threads, uint32_t grid, size_t lds) {

@@ -135,6 +135,44 @@ hipError_t q4k_gemm_f16_launch(hipStream_t s, const uint8_t *w, const uint16_t *
                                uint32_t rows, uint32_t hidden, uint32_t seq, int with_mins, int accumulate, uint32_t splits, float *partial);
 uint32_t q4k_gemm_splits(uint32_t rows, uint32_t hidden, uint32_t seq, uint32_t cu_count);  // partial: [splits][seq][rows] floats
 
+// One token through a bank of MXFP4 experts, a launch per projection stage (moe1_launch): a small argument block
+// instead of a job table, so a workgroup's first loads leave as soon as the kernel starts.
+constexpr uint32_t kMoe1MaxK = 4;  // selected experts per token
+struct Moe1Args {
+    // The token's selection.  With `logits` set every wavefront selects for itself (Router::select over n_experts <= 64
+    // logits, policy as router_select_launch) and workgroup 0 writes experts / weights; without, both are read.
+    const float *logits, *router_bias;
+    uint32_t *experts;
+    float *weights;
+    uint32_t n_experts, k;
+    int32_t policy;
+    uint32_t n_mats;        // matrices per expert in this stage: 2 = gate and up apart, 1 = fused gate_up / down
+    // Expert 0's matrices; expert e's start e * stride bytes further on.  An expert id >= n_experts contributes nothing.
+    const uint8_t *w[2], *aux[2];
+    uint64_t w_stride, aux_stride;
+    const float *bias[2];   // optional; expert e's row e * bias_stride floats further on, element r at r * bias_step
+    uint64_t bias_stride;
+    uint32_t bias_step;
+    uint32_t rows, kdim;    // of every matrix
+    // Activations: gate/up stage: the token (`x`, the same for every expert).  Down stage: slot q's gate/up results at
+    // x + q * x_slot_stride and x_glu + q * x_slot_stride (x_glu == x: interleaved g0 u0 g1 u1 ...), gated on the way in.
+    const float *x, *x_glu;
+    uint64_t x_slot_stride;
+    float glu_limit, glu_alpha;
+    // Results: gate/up stage: matrix m of slot q to out[m] + q * out_slot_stride; down stage: out[0], the weighted sum.
+    float *out[2];
+    uint64_t out_slot_stride;
+    uint32_t cw, nw, stages;  // 128-element steps per wavefront, working wavefronts, ring slots per wavefront (3 or 5)
+    uint32_t terms_kpad;      // elements per (term, slot) row of `terms`
+    // Optional hand-over between the stages (fused interleaved gate_up only): the gate/up stage writes the gated
+    // activation of slot q, element i, as its three bf16 terms terms[(t * k + q) * terms_kpad + i] instead of
+    // the raw results; the down stage reads its operands from there (and glu_limit / glu_alpha belong to the gate/up
+    // stage then).
+    uint16_t *terms;
+};
+bool moe1_geometry(Moe1Args &A, uint32_t *threads, size_t *lds);  // fills cw / nw / stages; false: not served
+hipError_t moe1_launch(hipStream_t s, const Moe1Args &A, bool down, uint32_t grid, uint32_t threads, size_t lds);
+
 // MoE helpers
 hipError_t router_select_launch(hipStream_t s, const float *logits, const float *bias, uint32_t tokens, uint32_t n_experts, uint32_t k,
                                 int policy, uint32_t *experts, float *weights);
