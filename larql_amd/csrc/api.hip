@@ -1508,7 +1508,10 @@ static int moe_mxfp4_block(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank
         if (gu_rows < (1u << 22) && hidden < (1u << 22) && c->cu_count <= 512 && (!route_logits || bank->n_experts <= 64) && moe1_geometry(ga, &gt, &gl) &&
             moe1_geometry(da, &dt, &dl)) {
             const uint32_t cus = (uint32_t)c->cu_count;
-            const uint32_t g_units = (uint32_t)(k * ga.n_mats * ((gu_rows + 15) / 16)), d_units = (uint32_t)((hidden + 15) / 16);
+            // a short result is cut into tiles of fewer than 16 rows so that every compute unit gets the same share
+            const uint32_t per_wg = (uint32_t)(((hidden + 15) / 16 + cus - 1) / cus);
+            da.tile_rows = (uint32_t)std::min<size_t>(16, (hidden + (size_t)cus * per_wg - 1) / ((size_t)cus * per_wg));
+            const uint32_t g_units = (uint32_t)(k * ga.n_mats * ((gu_rows + 15) / 16)), d_units = (uint32_t)((hidden + da.tile_rows - 1) / da.tile_rows);
             HIPCHECK(c, moe1_launch(c->stream, ga, false, std::min(cus, g_units), gt, gl));
             HIPCHECK(c, moe1_launch(c->stream, da, true, std::min(cus, d_units), dt, dl));
             return LARQL_OK;

@@ -1706,23 +1706,29 @@ __device__ __forceinline__ void run_mxfp4_fold(const GemvJob &j, const Mx4Sel &s
 //                  join there.  Without `terms` (gate and up apart) the activations are gated and split here.
 // ---------------------------------------------------------------------------
 constexpr int kMoe1BatchTiles = 4;
-constexpr int moe1_stages(int cw) { return cw <= 3 ? 5 : 3; }  // ring slots per wavefront that fit the LDS beside the partials
+constexpr int moe1_stages(int cw) { return cw <= 3 ? 3 : 3; }  // ring slots per wavefront that fit the LDS beside the partials
+constexpr uint32_t moe1_slot_bytes(int cw) { return (uint32_t)cw * kMx4StepBytes + (cw > 4 ? 512u : 256u); }  // steps, then a scale dword per lane (two with five steps)
+__device__ const uint32_t kMoe1Zeros[4] = {0u, 0u, 0u, 0u};      // what an operand lane without an activation loads
 
 // CW: 128-element steps per wavefront (the row length decides); NS: ring slots per wavefront
 template <bool DOWN, int CW, int NS>
 __global__ void __launch_bounds__(kMx4MaxWaves * 64) moe1_kernel(const Moe1Args A) {
     extern __shared__ __attribute__((aligned(16))) uint8_t m1_lds[];
     constexpr int R = kMoe1BatchTiles;
-    constexpr uint32_t cw = CW, slot_bytes = CW * kMx4StepBytes + kMx4ScaleBytes;
+    constexpr uint32_t cw = CW, slot_bytes = moe1_slot_bytes(CW);
     const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t nw_launch = blockDim.x >> 6;
     const uint32_t jr = lane & 15u, kg = lane >> 4;
     const uint32_t kdim = A.kdim, nb = kdim / 32, row_bytes = nb * 16, steps = (kdim + 127) / 128, nwj = A.nw;
-    const uint32_t rows = A.rows, nq = min(A.k, kMoe1MaxK);
+    const uint32_t rows = A.rows, nq = min(A.k, kMoe1MaxK), TR = A.tile_rows;  // (rows per tile: 16, or fewer to share a short result out evenly)
     uint8_t *ring = m1_lds + wv * (NS * slot_bytes);
     float *part = reinterpret_cast<float *>(m1_lds + nw_launch * (NS * slot_bytes));
     const uint32_t step0 = wv * cw;
     const bool working = wv < nwj && step0 < steps;
+
+    // 0. the selection as stored, where an earlier launch made it
+    const uint32_t ev = (!A.logits && lane < nq) ? ((const GLOBAL_AS uint32_t *)A.experts)[lane] : 0u;
+    const float wl = (!A.logits && DOWN && lane < nq) ? ((const GLOBAL_AS float *)A.weights)[lane] : 0.0f;
 
     // 1. the activations of this wavefront's K-range: nothing they need has to be waited for
     GemvJob jx = {};  // (the fields the activation helpers read)
@@ -1732,19 +1738,19 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) moe1_kernel(const Moe1Args 
     Mx4Ops ops;
     const bool pre = DOWN && A.terms != nullptr;  // the activations arrive as operand terms
     if (pre) {
-        // lane (row i = 4q + term, kg): eight consecutive bf16 of term plane `term`, slot q, per MFMA
+        // lane (row i = 4q + term, kg): eight consecutive bf16 of term plane `term`, slot q, per MFMA; a lane without an
+        // activation (fourth row of a slot, slot >= k, elements past the row end) reads zeros
         const uint32_t tq = jr >> 2, term = jr & 3u;
         const bool mine = working && tq < nq && term < 3u;
-        const uint16_t *tp = A.terms + ((size_t)(mine ? term : 0u) * nq + (mine ? tq : 0u)) * A.terms_kpad;
+        const uint16_t *tp = A.terms + ((size_t)term * nq + tq) * A.terms_kpad;
 #pragma unroll
         for (int s = 0; s < CW; s++) {
 #pragma unroll
             for (int m = 0; m < 4; m++) {
-                const uint32_t el = (step0 + s) * 128 + 32 * kg + 8 * m;
-                const bool in_row = mine && el < kdim;  // (kdim % 32 == 0: a group of eight is inside or outside)
-                const u32x4 t = *(const GLOBAL_AS u32x4 *)(tp + (in_row ? el : 0u));
-                ops.a[s][m].u[0] = in_row ? t.x : 0u; ops.a[s][m].u[1] = in_row ? t.y : 0u;
-                ops.a[s][m].u[2] = in_row ? t.z : 0u; ops.a[s][m].u[3] = in_row ? t.w : 0u;
+                const uint32_t el = (step0 + s) * 128 + 32 * kg + 8 * m;  // (kdim % 32 == 0: a group of eight is inside or outside)
+                const uint16_t *src = (mine && el < kdim) ? tp + el : reinterpret_cast<const uint16_t *>(kMoe1Zeros);
+                const u32x4 t = *(const GLOBAL_AS u32x4 *)src;
+                ops.a[s][m].u[0] = t.x; ops.a[s][m].u[1] = t.y; ops.a[s][m].u[2] = t.z; ops.a[s][m].u[3] = t.w;
             }
         }
     } else {
@@ -1774,90 +1780,89 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) moe1_kernel(const Moe1Args 
                 if ((uint32_t)r < nq) { A.experts[r] = idx[r]; A.weights[r] = wt[r]; }
         }
     } else {
-        const uint32_t ev = lane < nq ? ((const GLOBAL_AS uint32_t *)A.experts)[lane] : 0u;
-        const float wl = (DOWN && lane < nq) ? ((const GLOBAL_AS float *)A.weights)[lane] : 0.0f;
 #pragma unroll
         for (int q = 0; q < (int)kMoe1MaxK; q++) {
             e[q] = (uint32_t)__builtin_amdgcn_readlane((int)ev, q);
             cwt[q] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wl), q));
         }
     }
+    // expert q's matrices (wave-uniform 64-bit bases); an id outside the bank contributes nothing and reads nothing of it
+    const uint8_t *wq[kMoe1MaxK], *sq[kMoe1MaxK];
 #pragma unroll
     for (int q = 0; q < (int)kMoe1MaxK; q++) {
-        ok[q] = (uint32_t)q < nq && e[q] < A.n_experts;  // an id outside the bank contributes nothing and reads nothing of it
+        ok[q] = (uint32_t)q < nq && e[q] < A.n_experts;
         e[q] = ok[q] ? e[q] : 0u;
         cwt[q] = ok[q] ? cwt[q] : 0.0f;
+        wq[q] = A.w[0] + (size_t)e[q] * A.w_stride;
+        sq[q] = A.aux[0] + (size_t)e[q] * A.aux_stride;
     }
+    // (second matrix of a slot: the same expert in the up bank)
+    const size_t m1_w = A.n_mats == 2 ? (size_t)(A.w[1] - A.w[0]) : 0, m1_s = A.n_mats == 2 ? (size_t)(A.aux[1] - A.aux[0]) : 0;
     auto expert_of = [&](uint32_t q) { return q == 1 ? e[1] : (q == 2 ? e[2] : (q == 3 ? e[3] : e[0])); };
     auto ok_of = [&](uint32_t q) { return q == 1 ? ok[1] : (q == 2 ? ok[2] : (q == 3 ? ok[3] : ok[0])); };
     auto weight_of = [&](uint32_t q) { return q == 1 ? cwt[1] : (q == 2 ? cwt[2] : (q == 3 ? cwt[3] : cwt[0])); };
 
-    // 3. this workgroup's share.  Gate/up: virtual tiles [va, vb) of the list (slot, matrix, row tile); down: row tiles.
-    const uint32_t tpm = (rows + 15) / 16;
+    // 3. this workgroup's share.  Gate/up: row tiles [va, vb) of the list (slot, matrix, row tile); down: row tiles of
+    // the result, each met by the k experts in turn (expert innermost).
+    const uint32_t tpm = (rows + TR - 1) / TR;
     const uint32_t n_units = DOWN ? tpm : nq * A.n_mats * tpm;
     const uint32_t va = n_units * blockIdx.x / gridDim.x, vb = n_units * (blockIdx.x + 1) / gridDim.x;  // (the host keeps the products below 2^32)
     if (va >= vb) return;
-    const uint32_t nt = vb - va;
+    const uint32_t nt = vb - va, n_virtual = DOWN ? nt * nq : nt;
 
     // per-lane parts of a wave-tile's addresses: the lane's row within the tile and its block of each step
+    // (a block past the row end is the row's last block again: its activations are zeros, so it adds nothing)
     uint32_t woff[CW], sc_at[CW];
-    bool valid[CW];
-    bool all_valid = true;
 #pragma unroll
     for (int s = 0; s < CW; s++) {
         const uint32_t b = (step0 + s) * 4 + kg, bc = min(b, nb - 1);
-        valid[s] = working && b < nb;
-        all_valid = all_valid && valid[s];
         woff[s] = jr * row_bytes + bc * 16;
         sc_at[s] = (16u * s + jr) * 4 + (bc - min((step0 + s) * 4, nb - 4));
     }
-    const uint32_t sc_dw = min((step0 + kg) * 4, nb - 4), sc_dw4 = min((step0 + 4) * 4, nb - 4);
-    const uint32_t soff = jr * nb + sc_dw, soff4 = jr * nb + sc_dw4;
-    const uint32_t tile_w = 16 * row_bytes, tile_s = 16 * nb;
+    const uint32_t soff = jr * nb + min((step0 + kg) * 4, nb - 4), soff4 = jr * nb + min((step0 + 4) * 4, nb - 4);
+    const uint32_t tile_w = TR * row_bytes, tile_s = TR * nb;
 
-    // issue cursor.  Gate/up: (segment = slot * n_mats + matrix, row tile) walking the list; down: (batch, expert, tile of the batch)
-    uint32_t it_seg = DOWN ? 0u : va / tpm, it_t = DOWN ? 0u : va - (va / tpm) * tpm, it_left = nt;
-    uint32_t it_tb = 0, it_q = 0, it_tl = 0, slot_i = 0;
-    auto issue = [&]() {
-        uint32_t q, m, t;
-        if (DOWN) { q = it_q; m = 0; t = min(va + it_tb + it_tl, vb - 1); }
-        else { q = A.n_mats == 2 ? it_seg >> 1 : it_seg; m = A.n_mats == 2 ? (it_seg & 1u) : 0u; t = it_t; }
-        const uint32_t ex = expert_of(q);
-        const uint8_t *wbase = (m ? A.w[1] : A.w[0]) + ((size_t)ex * A.w_stride + (size_t)t * tile_w);
-        const uint8_t *sbase = (m ? A.aux[1] : A.aux[0]) + ((size_t)ex * A.aux_stride + (size_t)t * tile_s);
+    // issue cursor: (segment = slot * n_mats + matrix, row tile) / (row tile, expert)
+    uint32_t it_seg = DOWN ? 0u : va / tpm, it_t = DOWN ? va : va - (va / tpm) * tpm, it_q = 0, it_left = n_virtual, slot_i = 0;
+    // the loads of the cursor's wave-tile (every lane takes part: no branch sits between the loads, so what is in flight
+    // can be counted; lanes whose step does not exist copy a neighbouring block that nothing reads)
+    auto issue_loads = [&]() {
+        const uint32_t q = DOWN ? it_q : (A.n_mats == 2 ? it_seg >> 1 : it_seg);
+        const uint8_t *wbase = q == 1 ? wq[1] : (q == 2 ? wq[2] : (q == 3 ? wq[3] : wq[0]));
+        const uint8_t *sbase = q == 1 ? sq[1] : (q == 2 ? sq[2] : (q == 3 ? sq[3] : sq[0]));
+        if (!DOWN && A.n_mats == 2 && (it_seg & 1u)) { wbase += m1_w; sbase += m1_s; }
+        wbase += (size_t)it_t * tile_w;
+        sbase += (size_t)it_t * tile_s;
+        // lanes past the tile's last row (a tile of fewer than 16 rows, a ragged last tile) read that row again
+        const uint32_t last = min(TR - 1, rows - 1 - it_t * TR), back = jr > last ? jr - last : 0u;
+        const uint32_t bw = back * row_bytes, bs = back * nb;
         uint8_t *lp = ring + slot_i * slot_bytes;
-        if (t * 16 + 16 > rows) {  // ragged last tile of a matrix: the lane's row is clamped into it
-            const uint32_t rl = min(jr, rows - 1 - t * 16), back = (jr - rl);
 #pragma unroll
-            for (int s = 0; s < CW; s++)
-                __builtin_amdgcn_global_load_lds((g_vp)(wbase + (woff[s] - back * row_bytes)), (lds_vp)(lp + s * 1024), 16, 0, 0);
-            if (CW >= 4 || lane < 16 * cw) __builtin_amdgcn_global_load_lds((g_vp)(sbase + (soff - back * nb)), (lds_vp)(lp + cw * 1024), 4, 0, 0);
-            if (CW > 4 && lane < 16) __builtin_amdgcn_global_load_lds((g_vp)(sbase + (soff4 - back * nb)), (lds_vp)(lp + cw * 1024 + 256), 4, 0, 0);
-        } else {
-#pragma unroll
-            for (int s = 0; s < CW; s++)
-                __builtin_amdgcn_global_load_lds((g_vp)(wbase + woff[s]), (lds_vp)(lp + s * 1024), 16, 0, 0);
-            if (CW >= 4 || lane < 16 * cw) __builtin_amdgcn_global_load_lds((g_vp)(sbase + soff), (lds_vp)(lp + cw * 1024), 4, 0, 0);
-            if (CW > 4 && lane < 16) __builtin_amdgcn_global_load_lds((g_vp)(sbase + soff4), (lds_vp)(lp + cw * 1024 + 256), 4, 0, 0);
-        }
+        for (int s = 0; s < CW; s++)
+            __builtin_amdgcn_global_load_lds((g_vp)(wbase + (woff[s] - bw)), (lds_vp)(lp + s * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((g_vp)(sbase + (soff - bs)), (lds_vp)(lp + cw * 1024), 4, 0, 0);
+        if (CW > 4) __builtin_amdgcn_global_load_lds((g_vp)(sbase + (soff4 - bs)), (lds_vp)(lp + cw * 1024 + 256), 4, 0, 0);
         slot_i = slot_i + 1 == NS ? 0u : slot_i + 1;
-        // next wave-tile; past the end the last one again (uniform load counts)
-        if (DOWN) {
-            if (it_tb < nt) {
-                const uint32_t nbt = min((uint32_t)R, nt - it_tb);
-                if (++it_tl >= nbt) {
-                    it_tl = 0;
-                    if (++it_q >= nq) { it_q = 0; it_tb += R; }
-                }
-                if (it_tb >= nt) { it_tb = nt - 1 - ((nt - 1) % R); it_q = nq - 1; it_tl = (nt - 1) % R; }
-            }
-        } else if (it_left > 1) {
-            it_left--;
-            if (++it_t >= tpm) { it_t = 0; it_seg++; }
-        }
     };
-    if (working)
-        for (int s = 0; s + 1 < NS; s++) issue();
+    auto advance = [&]() {
+        if (DOWN) {
+            if (++it_q >= nq) { it_q = 0; it_t++; }
+        } else if (++it_t >= tpm) { it_t = 0; it_seg++; }
+    };
+    auto issue = [&]() {  // the next wave-tile, if there is one (nothing is read twice: the waits below count what is really in flight)
+        if (it_left == 0) return;
+        issue_loads();
+        it_left--;
+        advance();
+    };
+    // the first NS-1 wave-tiles without a branch around their loads (a share of fewer tiles reads its last one again)
+    if (working) {
+#pragma unroll
+        for (int s = 0; s + 1 < NS; s++) {
+            issue_loads();
+            if (it_left > 1) { it_left--; advance(); } else it_left = 0;
+        }
+    }
 
     // 4. operands, while the first tiles fly (the ring's last slot is still free and serves as scratch)
     if (working && !pre) {
@@ -1874,57 +1879,57 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) moe1_kernel(const Moe1Args 
     constexpr uint32_t hw = DOWN ? 4u : 1u;  // partial sums per weight row and wavefront (down: one per expert)
     const uint32_t PW = nwj * hw, nwork = min(nwj, (steps + cw - 1) / cw);
     uint32_t use_i = 0, parity = 0;
-    uint32_t f_seg = DOWN ? 0u : va / tpm, f_t = DOWN ? va : va - (va / tpm) * tpm;  // the fold's cursor (first tile of the batch)
-    for (uint32_t tb = 0; tb < nt; tb += R) {
+    uint32_t f_seg = DOWN ? 0u : va / tpm, f_t = DOWN ? va : va - (va / tpm) * tpm;  // the fold's cursor: first tile of the batch
+    uint32_t tl = 0, cq = 0;   // row tile within the batch, expert within the tile
+    float acc = 0.f;
+    for (uint32_t v = 0; v < n_virtual; v++) {
         float *pb = part + parity * (R * 16 * nw_launch * hw);
-        const uint32_t nbt = min((uint32_t)R, nt - tb);
         if (working) {
-            float acc[R];
-#pragma unroll
-            for (int t = 0; t < R; t++) acc[t] = 0.f;
-#pragma unroll
-            for (int q = 0; q < (int)kMoe1MaxK; q++) {
-                if (DOWN ? (uint32_t)q >= nq : q >= 1) break;
-#pragma unroll
-                for (int tl = 0; tl < R; tl++) {
-                    if ((uint32_t)tl >= nbt) break;
-                    issue();
-                    LARQL_WAIT_VMCNT((CW + 1 + (CW > 4)) * (NS - 1));  // at most NS-1 younger wave-tiles in flight: the oldest has landed
-                    asm volatile("" ::: "memory");
-                    const uint8_t *slot = ring + use_i * slot_bytes;
-                    f32x4 D = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int s = 0; s < CW; s++) {
-                        const u32x4 qw = *reinterpret_cast<const u32x4 *>(slot + s * 1024 + lane * 16);
-                        const uint32_t sc = slot[cw * 1024 + sc_at[s]];
-                        D = mx4_step_mfma(ops.a[s], qw, sc, all_valid || valid[s], D);  // (an expert outside the bank: its result is dropped in the fold)
-                    }
-                    use_i = use_i + 1 == NS ? 0u : use_i + 1;
-                    if (kg == (uint32_t)q) acc[tl] = (D[0] + D[1]) + D[2];  // (rows 4q .. 4q+2: this expert's / the token's term sums)
-                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the slot's reads are done before anything reuses it
-                }
+            issue();
+            {   // wave-tiles younger than the one about to be used: it has landed when only their loads are outstanding
+                constexpr int L = CW + 1 + (CW > 4);  // loads per wave-tile
+                const uint32_t younger = min(n_virtual - 1 - v, (uint32_t)(NS - 1));
+                if (younger >= 4) LARQL_WAIT_VMCNT(L * (NS - 1 < 4 ? NS - 1 : 4));
+                else if (younger == 3) LARQL_WAIT_VMCNT(L * (NS - 1 < 3 ? NS - 1 : 3));
+                else if (younger == 2) LARQL_WAIT_VMCNT(L * 2);
+                else if (younger == 1) LARQL_WAIT_VMCNT(L * 1);
+                else LARQL_WAIT_VMCNT(0);
             }
+            asm volatile("" ::: "memory");
+            const uint8_t *slot = ring + use_i * slot_bytes;
+            f32x4 D = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int tl = 0; tl < R; tl++) {
-                if ((uint32_t)tl >= nbt) break;
-                if (DOWN) pb[(tl * 16 + jr) * PW + wv * hw + kg] = ok_of(kg) ? acc[tl] * weight_of(kg) : 0.f;
-                else if (kg == 0) pb[(tl * 16 + jr) * PW + wv] = acc[tl];
+            for (int s = 0; s < CW; s++) {
+                const u32x4 qw = *reinterpret_cast<const u32x4 *>(slot + s * 1024 + lane * 16);
+                const uint32_t sc = slot[cw * 1024 + sc_at[s]];
+                D = mx4_step_mfma(ops.a[s], qw, sc, true, D);  // (an expert outside the bank: its result is dropped in the fold)
             }
+            use_i = use_i + 1 == NS ? 0u : use_i + 1;
+            const float sum = (D[0] + D[1]) + D[2];  // rows 4rq .. 4rq+2: the term sums of slot rq's activation
+            if (DOWN) {
+                if (kg == cq) acc = sum * weight_of(cq);
+                if (cq + 1 == nq) pb[(tl * 16 + jr) * PW + wv * hw + kg] = ok_of(kg) ? acc : 0.f;
+            } else if (kg == 0) {
+                pb[(tl * 16 + jr) * PW + wv] = sum;
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the slot's reads are done before anything reuses it
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (DOWN && ++cq < nq) continue;
+        cq = 0;
+        if (++tl < (uint32_t)R && v + 1 < n_virtual) continue;
+        // a batch of `tl` row tiles is complete: the row partials meet
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         if (DOWN) {
             // four threads per result row: thread h adds up expert h's slot of every wavefront, then the experts meet
-            const uint32_t row_base = (va + tb) * 16;
-            for (uint32_t rr = threadIdx.x >> 2; rr < nbt * 16; rr += blockDim.x >> 2) {
+            for (uint32_t rr = threadIdx.x >> 2; rr < tl * 16; rr += blockDim.x >> 2) {
                 const uint32_t h = threadIdx.x & 3u;
                 float s = 0.f;
                 for (uint32_t w = 0; w < nwork; w++) s += pb[rr * PW + w * hw + h];
                 s = dpp_add<0xB1>(s);  // quad_perm [1,0,3,2]: experts 0+1, 2+3
                 s = dpp_add<0x4E>(s);  // quad_perm [2,3,0,1]: all four
-                const uint32_t row = row_base + rr;
-                if (h == 0 && row < rows) {
+                const uint32_t jt = rr & 15u, row = (f_t + (rr >> 4)) * TR + jt;
+                if (h == 0 && jt < TR && row < rows) {
                     if (A.bias[0]) {  // + sum_q w_q * bias_q[row], in selection order
 #pragma unroll
                         for (int q = 0; q < (int)kMoe1MaxK; q++)
@@ -1933,16 +1938,18 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) moe1_kernel(const Moe1Args 
                     ((g_f32wp)A.out[0])[row] = s;
                 }
             }
+            f_t += tl;
         } else {
-            for (uint32_t rr = threadIdx.x; rr < nbt * 16; rr += blockDim.x) {
+            for (uint32_t rr = threadIdx.x; rr < tl * 16; rr += blockDim.x) {
                 float s = 0.f;
                 for (uint32_t w = 0; w < nwork; w++) s += pb[rr * PW + w];
                 // the tile of this row: `rr / 16` tiles past the batch's first
                 uint32_t seg = f_seg, t = f_t + (rr >> 4);
                 while (t >= tpm) { t -= tpm; seg++; }
                 const uint32_t q = A.n_mats == 2 ? seg >> 1 : seg, m = A.n_mats == 2 ? (seg & 1u) : 0u;
-                const uint32_t row = t * 16 + (rr & 15u);
-                if (row < rows) {
+                const uint32_t jt = rr & 15u, row = t * TR + jt;
+                const bool live = jt < TR && row < rows;
+                if (live) {
                     const float *bias = m ? A.bias[1] : A.bias[0];
                     if (!ok_of(q)) s = 0.0f;  // an expert outside the bank: no contribution (its stand-in's bytes were read, not used)
                     else if (bias) s += ((const GLOBAL_AS float *)bias)[(size_t)expert_of(q) * A.bias_stride + (size_t)row * A.bias_step];
@@ -1950,21 +1957,22 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) moe1_kernel(const Moe1Args 
                 if (A.terms) {
                     // rows 2i (gate) and 2i+1 (up) sit in neighbouring lanes (rows and the block size are even)
                     const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, s), 0xB1, 0xF, 0xF, false));  // quad_perm [1,0,3,2]
-                    if ((row & 1u) == 0 && row + 1 < rows) {
+                    if (live && (row & 1u) == 0 && row + 1 < rows) {  // (an even tile height keeps the pair in one tile)
                         const float hv = ok_of(q) ? clamped_glu(s, other, A.glu_limit, A.glu_alpha) : 0.0f;
-                        uint32_t t[3];
-                        mx4_terms(hv, 0.0f, t);
+                        uint32_t t3[3];
+                        mx4_terms(hv, 0.0f, t3);
                         uint16_t *tp = A.terms + (size_t)q * A.terms_kpad + (row >> 1);
                         const size_t plane = (size_t)nq * A.terms_kpad;
-                        tp[0] = (uint16_t)t[0]; tp[plane] = (uint16_t)t[1]; tp[2 * plane] = (uint16_t)t[2];
+                        tp[0] = (uint16_t)t3[0]; tp[plane] = (uint16_t)t3[1]; tp[2 * plane] = (uint16_t)t3[2];
                     }
-                } else if (row < rows) {
+                } else if (live) {
                     ((g_f32wp)((m ? A.out[1] : A.out[0]) + (size_t)q * A.out_slot_stride))[row] = s;
                 }
             }
-            f_t += nbt;
+            f_t += tl;
             while (f_t >= tpm) { f_t -= tpm; f_seg++; }
         }
+        tl = 0;
         parity ^= 1u;
     }
     LARQL_WAIT_VMCNT(0);
@@ -3381,11 +3389,12 @@ bool moe1_geometry(Moe1Args &A, uint32_t *threads, size_t *lds) {
     const uint32_t cw = mx4_steps_per_wave(steps);
     if (cw == 0) return false;
     const uint32_t nw = (uint32_t)((steps + cw - 1) / cw);
-    const size_t slot = (size_t)cw * kMx4StepBytes + kMx4ScaleBytes;
+    const size_t slot = moe1_slot_bytes((int)cw);
     const size_t partials = 2 * (size_t)kMoe1BatchTiles * 16 * nw * 4 * sizeof(float);
     A.cw = cw;
     A.nw = nw;
     A.stages = (uint32_t)moe1_stages((int)cw);
+    if (A.tile_rows == 0 || A.tile_rows > 16) A.tile_rows = 16;
     *threads = nw * 64;
     *lds = nw * A.stages * slot + partials;
     return *lds <= 160 * 1024;

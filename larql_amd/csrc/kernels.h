@@ -164,6 +164,8 @@ struct Moe1Args {
     uint64_t out_slot_stride;
     uint32_t cw, nw, stages;  // 128-element steps per wavefront, working wavefronts, ring slots per wavefront (3 or 5)
     uint32_t terms_kpad;      // elements per (term, slot) row of `terms`
+    uint32_t tile_rows;       // result rows per tile, 1..16 (0: 16); even where `terms` is written
+    uint32_t pad;
     // Optional hand-over between the stages (fused interleaved gate_up only): the gate/up stage writes the gated
     // activation of slot q, element i, as its three bf16 terms terms[(t * k + q) * terms_kpad + i] instead of
     // the raw results; the down stage reads its operands from there (and glu_limit / glu_alpha belong to the gate/up
