@@ -1714,7 +1714,7 @@ __device__ const uint32_t kMoe1Zeros[4] = {0u, 0u, 0u, 0u};      // what an oper
 template <bool DOWN, int CW, int NS>
 __global__ void __launch_bounds__(kMx4MaxWaves * 64) moe1_kernel(const Moe1Args A) {
     extern __shared__ __attribute__((aligned(16))) uint8_t m1_lds[];
-    constexpr int R = kMoe1BatchTiles;
+    constexpr int R = DOWN ? kMoe1BatchTiles : 2 * kMoe1BatchTiles;  // row tiles between two folds of the row partials
     constexpr uint32_t cw = CW, slot_bytes = moe1_slot_bytes(CW);
     const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t nw_launch = blockDim.x >> 6;
@@ -1726,7 +1726,10 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) moe1_kernel(const Moe1Args 
     const uint32_t step0 = wv * cw;
     const bool working = wv < nwj && step0 < steps;
 
-    // 0. the selection as stored, where an earlier launch made it
+    // 0. what the selection needs: the logits, or the selection as stored where an earlier launch made it
+    const bool has_logit = A.logits && lane < A.n_experts;
+    float logit = has_logit ? ((const GLOBAL_AS float *)A.logits)[lane] : 0.0f;
+    if (has_logit && A.router_bias) logit += ((const GLOBAL_AS float *)A.router_bias)[lane];
     const uint32_t ev = (!A.logits && lane < nq) ? ((const GLOBAL_AS uint32_t *)A.experts)[lane] : 0u;
     const float wl = (!A.logits && DOWN && lane < nq) ? ((const GLOBAL_AS float *)A.weights)[lane] : 0.0f;
 
@@ -1737,7 +1740,7 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) moe1_kernel(const Moe1Args 
     Mx4In xin[kMx4MaxSteps];
     Mx4Ops ops;
     const bool pre = DOWN && A.terms != nullptr;  // the activations arrive as operand terms
-    if (pre) {
+    auto load_operands = [&]() {
         // lane (row i = 4q + term, kg): eight consecutive bf16 of term plane `term`, slot q, per MFMA; a lane without an
         // activation (fourth row of a slot, slot >= k, elements past the row end) reads zeros
         const uint32_t tq = jr >> 2, term = jr & 3u;
@@ -1753,6 +1756,9 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) moe1_kernel(const Moe1Args 
                 ops.a[s][m].u[0] = t.x; ops.a[s][m].u[1] = t.y; ops.a[s][m].u[2] = t.z; ops.a[s][m].u[3] = t.w;
             }
         }
+    };
+    if (pre) {
+        // (fetched below, behind the first weight tile)
     } else {
 #pragma unroll
         for (int s = 0; s < CW; s++)
@@ -1767,8 +1773,8 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) moe1_kernel(const Moe1Args 
         uint32_t idx[kRouterMaxK];
         float wt[kRouterMaxK];
         const bool writer = A.experts && blockIdx.x == 0 && wv == 0;  // (wave-uniform)
-        if (writer || DOWN) router_select_wave<true>(A.logits, A.router_bias, A.n_experts, nq, A.policy, lane, idx, wt);
-        else router_select_wave<false>(A.logits, A.router_bias, A.n_experts, nq, A.policy, lane, idx, wt);
+        if (writer || DOWN) router_select_lane<true>(logit, A.n_experts, nq, A.policy, lane, idx, wt);
+        else router_select_lane<false>(logit, A.n_experts, nq, A.policy, lane, idx, wt);
 #pragma unroll
         for (int q = 0; q < (int)kMoe1MaxK; q++) {
             e[q] = __builtin_amdgcn_readfirstlane(idx[q]);
@@ -1861,7 +1867,12 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) moe1_kernel(const Moe1Args 
         for (int s = 0; s + 1 < NS; s++) {
             issue_loads();
             if (it_left > 1) { it_left--; advance(); } else it_left = 0;
+            if (s == 0 && pre) load_operands();  // behind the first tile: they return in order, the tile first
         }
+    }
+    if (pre) {
+        // the operands are in (and the first tile before them) once only the younger tiles' loads are outstanding
+        LARQL_WAIT_VMCNT((CW + 1 + (CW > 4)) * (NS - 2));
     }
 
     // 4. operands, while the first tiles fly (the ring's last slot is still free and serves as scratch)

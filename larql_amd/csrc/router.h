@@ -50,12 +50,12 @@ constexpr int kRouterMaxK = 8;
 // order (policy 1, NormalisedOverSelected) or over all experts in index order (policy 0, SoftmaxThenSelect).
 // Every lane ends with the same sel_idx / sel_w (entries from k on are 0).  WEIGHTS = false leaves sel_w at 0 (a
 // caller that only needs to know which experts).
+// (router_select_lane: lane i brings its logit, bias already added; lanes from n_experts on bring anything)
 template <bool WEIGHTS = true>
-__device__ __forceinline__ void router_select_wave(const float *logits, const float *bias, uint32_t n_experts, uint32_t k, int policy, uint32_t lane,
+__device__ __forceinline__ void router_select_lane(float l, uint32_t n_experts, uint32_t k, int policy, uint32_t lane,
                                                    uint32_t (&sel_idx)[kRouterMaxK], float (&sel_w)[kRouterMaxK]) {
     const bool has = lane < n_experts;
-    // the router bias joins the logit before anything else (MoeLayerWeights::router_bias, larql-compute/src/pipeline/moe.rs:505-508)
-    const float l = has ? (bias ? logits[lane] + bias[lane] : logits[lane]) : 0.0f;
+    l = has ? l : 0.0f;
     // orderable key: logit bits made monotone, then ~index so the lower index wins a tie; 0 = absent
     const uint32_t bits = __builtin_bit_cast(uint32_t, l);
     const uint32_t ord = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
@@ -86,6 +86,14 @@ __device__ __forceinline__ void router_select_wave(const float *logits, const fl
     }
 #pragma unroll
     for (int r = 0; r < kRouterMaxK; r++) sel_w[r] = (WEIGHTS && (uint32_t)r < k && denom > 0.0f) ? sel_ex[r] / denom : 0.0f;
+}
+
+template <bool WEIGHTS = true>
+__device__ __forceinline__ void router_select_wave(const float *logits, const float *bias, uint32_t n_experts, uint32_t k, int policy, uint32_t lane,
+                                                   uint32_t (&sel_idx)[kRouterMaxK], float (&sel_w)[kRouterMaxK]) {
+    // the router bias joins the logit before anything else (MoeLayerWeights::router_bias, larql-compute/src/pipeline/moe.rs:505-508)
+    const float l = lane < n_experts ? (bias ? logits[lane] + bias[lane] : logits[lane]) : 0.0f;
+    router_select_lane<WEIGHTS>(l, n_experts, k, policy, lane, sel_idx, sel_w);
 }
 
 }  // namespace larql
