@@ -326,9 +326,9 @@ void larql_hip_plan_destroy(larql_hip_ctx *ctx, larql_hip_plan *plan);
 int larql_hip_dev_gate_knn(larql_hip_ctx *ctx, int format, const void *gate,
                            const float *x, size_t batch, size_t n_features, size_t hidden,
                            size_t top_k, float *scores_scratch, uint32_t *idx_out, float *score_out, uint32_t *count_out);
-/* Waits for the context's stream, reports whether the last device-tier gate-KNN / gate walk met a NaN score
- * (the host tier answers LARQL_E_NAN there, the reference panics: gate_knn/mod.rs:84) and clears the flag.
- * Every device-tier gate-KNN call clears the flag before its own selection, so the answer belongs to the last one. */
+/* Waits for the context's stream, reports whether any device-tier gate-KNN / gate walk since the flag was last taken
+ * met a NaN score (the host tier answers LARQL_E_NAN there, the reference panics: gate_knn/mod.rs:84) and clears the
+ * flag.  The calls themselves only raise it: take it after the calls whose scores matter. */
 int larql_hip_dev_take_nan_flag(larql_hip_ctx *ctx, int *flag_out);
 
 /* larql_hip_dev_gate_knn for callers that cannot allocate (code under HIP graph capture, tight serving loops,

@@ -75,7 +75,7 @@ struct larql_hip_ctx {
     size_t table_sent_bytes[4] = {0, 0, 0, 0};                      // an identical table for the same place is not sent again
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     uint8_t *log2_up = nullptr;  // 256-entry table for the MXFP4 encoder
-    int *nan_flag = nullptr;
+    int *nan_flag = nullptr;       // [0]: device tier, raised by any call, cleared when taken; [1]: host tier, cleared by every call
     uint8_t *static_scratch = nullptr;  // this device's copy of `scratch` (hipGetSymbolAddress at create)
     larql_hip_submission_clock clock = {0, 0, 0};
 };
@@ -316,7 +316,7 @@ int larql_hip_create(larql_hip_ctx **out, int device) {
     c->info = buf;
     if (hipStreamCreate(&c->stream) != hipSuccess || hipEventCreate(&c->ev0) != hipSuccess ||
         hipEventCreate(&c->ev1) != hipSuccess || hipMalloc((void **)&c->log2_up, 256) != hipSuccess ||
-        hipMalloc((void **)&c->nan_flag, sizeof(int)) != hipSuccess) {
+        hipMalloc((void **)&c->nan_flag, 2 * sizeof(int)) != hipSuccess) {
         larql_hip_destroy(c);
         return LARQL_E_DEVICE;
     }
@@ -333,7 +333,7 @@ int larql_hip_create(larql_hip_ctx **out, int device) {
         }
     }
     if (hipMemcpy(c->log2_up, up, 256, hipMemcpyHostToDevice) != hipSuccess ||
-        hipMemset(c->nan_flag, 0, sizeof(int)) != hipSuccess) {
+        hipMemset(c->nan_flag, 0, 2 * sizeof(int)) != hipSuccess) {
         larql_hip_destroy(c);
         return LARQL_E_DEVICE;
     }
@@ -679,12 +679,12 @@ int larql_hip_q4k_matmul(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, c
         if (rc) return rc;
         uint16_t *xh = (uint16_t *)c->misc.p, *xl = xh + x_len, *sx = xl + x_len;
         float *ts = (float *)(((uintptr_t)(sx + sx_len) + 15) & ~(uintptr_t)15);
-        HIPCHECK(c, hipMemsetAsync(c->nan_flag, 0, sizeof(int), c->stream));
-        HIPCHECK(c, q4k_gemm_prep_launch(c->stream, c->x.p, 0, (uint32_t)hidden, (uint32_t)seq_len, xh, xl, sx, ts, c->nan_flag));
+        HIPCHECK(c, hipMemsetAsync(c->nan_flag + 1, 0, sizeof(int), c->stream));
+        HIPCHECK(c, q4k_gemm_prep_launch(c->stream, c->x.p, 0, (uint32_t)hidden, (uint32_t)seq_len, xh, xl, sx, ts, c->nan_flag + 1));
         int any_lo = 0;
-        HIPCHECK(c, hipMemcpyAsync(&any_lo, c->nan_flag, sizeof(int), hipMemcpyDeviceToHost, c->stream));
+        HIPCHECK(c, hipMemcpyAsync(&any_lo, c->nan_flag + 1, sizeof(int), hipMemcpyDeviceToHost, c->stream));
         HIPCHECK(c, hipStreamSynchronize(c->stream));
-        HIPCHECK(c, hipMemsetAsync(c->nan_flag, 0, sizeof(int), c->stream));
+        HIPCHECK(c, hipMemsetAsync(c->nan_flag + 1, 0, sizeof(int), c->stream));
         const uint32_t splits = q4k_gemm_splits((uint32_t)num_rows, (uint32_t)hidden, (uint32_t)seq_len, (uint32_t)c->cu_count);
         float *partial = nullptr;
         if (splits > 1) { rc = ensure(c, c->scores, (size_t)splits * seq_len * num_rows * 4 + 64); if (rc) return rc; partial = (float *)c->scores.p; }
@@ -716,7 +716,7 @@ static int topk_download(larql_hip_ctx *c, size_t batch, size_t k, uint32_t *idx
     HIPCHECK(c, hipMemcpyAsync(idx_out, d_idx, batch * k * 4, hipMemcpyDeviceToHost, c->stream));
     HIPCHECK(c, hipMemcpyAsync(score_out, d_val, batch * k * 4, hipMemcpyDeviceToHost, c->stream));
     HIPCHECK(c, hipMemcpyAsync(cnt.data(), d_cnt, batch * 4, hipMemcpyDeviceToHost, c->stream));
-    HIPCHECK(c, hipMemcpyAsync(&nan, c->nan_flag, sizeof(int), hipMemcpyDeviceToHost, c->stream));
+    HIPCHECK(c, hipMemcpyAsync(&nan, c->nan_flag + 1, sizeof(int), hipMemcpyDeviceToHost, c->stream));
     HIPCHECK(c, hipStreamSynchronize(c->stream));
     for (size_t b = 0; b < batch; b++) n_out[b] = cnt[b];
     if (check_nan && nan) return fail(c, LARQL_E_NAN, "top-K: NaN score");
@@ -744,7 +744,7 @@ static int host_matvec_topk(larql_hip_ctx *c, int kind, const uint8_t *w, size_t
     float *d_val = (float *)(d_idx + top_k);
     uint32_t *d_cnt = (uint32_t *)(d_val + top_k);
     HIPCHECK(c, topk_launch(c->stream, (const float *)c->scores.p, 1, (uint32_t)num_rows, (uint32_t)top_k, false, d_idx, d_val,
-                            d_cnt, c->nan_flag, nullptr, 0));
+                            d_cnt, c->nan_flag + 1, nullptr, 0));
     rc = sub.finish();
     if (rc) return rc;
     return topk_download(c, 1, top_k, idx_out, score_out, n_out, false);
@@ -1077,7 +1077,7 @@ int larql_hip_gate_knn(larql_hip_ctx *c, int format, const uint8_t *gate, size_t
     rc = upload(c, c->x, x, batch * hidden * 4); if (rc) return rc;
     rc = ensure(c, c->scores, batch * n * 4 + 64); if (rc) return rc;
     rc = ensure(c, c->misc, batch * (top_k * 8 + 4) + 64); if (rc) return rc;
-    HIPCHECK(c, hipMemsetAsync(c->nan_flag, 0, sizeof(int), c->stream));
+    HIPCHECK(c, hipMemsetAsync(c->nan_flag + 1, 0, sizeof(int), c->stream));
     Submission sub(c);
     rc = dev_gate_scores(c, kind, dg, (const float *)c->x.p, batch, n, hidden, (float *)c->scores.p);
     if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
@@ -1085,7 +1085,7 @@ int larql_hip_gate_knn(larql_hip_ctx *c, int format, const uint8_t *gate, size_t
     float *d_val = (float *)(d_idx + batch * top_k);
     uint32_t *d_cnt = (uint32_t *)(d_val + batch * top_k);
     HIPCHECK(c, topk_launch(c->stream, (const float *)c->scores.p, (uint32_t)batch, (uint32_t)n, (uint32_t)top_k, true, d_idx,
-                            d_val, d_cnt, c->nan_flag, nullptr, 0));
+                            d_val, d_cnt, c->nan_flag + 1, nullptr, 0));
     rc = sub.finish();
     if (rc) return rc;
     return topk_download(c, batch, top_k, idx_out, score_out, n_out, true);
@@ -1287,8 +1287,6 @@ int larql_hip_dev_gate_knn(larql_hip_ctx *c, int format, const void *gate, const
     if (!count_out) { rc = ensure(c, c->misc, batch * 4 + 64); if (rc) return rc; count_out = (uint32_t *)c->misc.p; }
     rc = dev_gate_scores(c, kind, gate, x, batch, n, hidden, scores_scratch);
     if (rc) return rc;
-    rc = clear_nan_flag(c);
-    if (rc) return rc;
     HIPCHECK(c, topk_launch(c->stream, scores_scratch, (uint32_t)batch, (uint32_t)n, (uint32_t)top_k, true, idx_out, score_out,
                             count_out, c->nan_flag, nullptr, 0));
     return LARQL_OK;
@@ -1366,8 +1364,6 @@ int larql_hip_dev_gate_knn_static(larql_hip_ctx *c, int format, const void *gate
         if (rc) return rc;
         HIPCHECK(c, gemv_launch(c->stream, P.kind, P.L, P.threads, P.grid, P.lds));
     }
-    rc = clear_nan_flag(c);
-    if (rc) return rc;
     HIPCHECK(c, topk_launch(c->stream, scores, (uint32_t)batch, (uint32_t)n, (uint32_t)top_k, true, idx_out, score_out,
                             count_out ? count_out : counts, c->nan_flag, nullptr, 0));
     return LARQL_OK;
@@ -1675,8 +1671,6 @@ int larql_hip_dev_gate_walk(larql_hip_ctx *c, int format, const void *const *gat
     for (size_t l = 0; l < n_layers; l++)
         push_gate_jobs(jobs, kind, gates[l], x + l * x_layer_stride, batch, n, hidden, scores_scratch + l * batch * n);
     rc = enqueue_jobs(c, jobs);
-    if (rc) return rc;
-    rc = clear_nan_flag(c);
     if (rc) return rc;
     HIPCHECK(c, topk_launch(c->stream, scores_scratch, (uint32_t)(n_layers * batch), (uint32_t)n, (uint32_t)top_k, true, idx_out,
                             score_out, count_out, c->nan_flag, nullptr, 0));

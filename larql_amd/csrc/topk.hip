@@ -108,7 +108,7 @@ __global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restr
     __shared__ uint64_t winners[64];
     __shared__ uint32_t sh_prefix, sh_need, sh_nwin, sh_ncand;
     __shared__ uint32_t group_max[64];
-    __shared__ uint64_t cand[CACHED ? kTopkCandidates : 1];
+    __shared__ __attribute__((aligned(16))) uint64_t cand[CACHED ? kTopkCandidates + 4 : 1];
     const uint32_t row = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const float *s = scores + (size_t)row * n;
     // wavefront w owns the contiguous indices [w0, w1), 64 at a time (lane = index within the 64)
@@ -118,10 +118,15 @@ __global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restr
     // the ordered score of index i (0: nothing there), from the register copy or from memory
     uint32_t cache[CACHED ? kTopkCached : 1];
     if (CACHED) {
+        // every load leaves before the first score is looked at (a load inside a condition is waited for where it
+        // stands: sixteen round trips instead of one); an index past the wavefront's range reads the row's last score
+        float raw[kTopkCached];
+#pragma unroll
+        for (int it = 0; it < kTopkCached; it++) raw[it] = s[min(w0 + it * 64 + lane, n - 1)];
 #pragma unroll
         for (int it = 0; it < kTopkCached; it++) {
             const uint32_t i = w0 + it * 64 + lane;
-            cache[it] = i < w1 ? (uint32_t)(make_key<BY_ABS>(s[i], i, nan_flag) >> 32) : 0u;
+            cache[it] = i < w1 ? (uint32_t)(make_key<BY_ABS>(raw[it], i, nan_flag) >> 32) : 0u;
         }
     }
     // f(ord, i) for every index of this wavefront, 64 at a time, all lanes taking part in every round
@@ -184,10 +189,19 @@ __global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restr
             __syncthreads();
             const uint32_t nc = sh_ncand;
             if (nc <= (uint32_t)kTopkCandidates) {  // (uniform over the workgroup)
+                // (the list is read four keys at a time: zero keys, below every real one, fill it up to a multiple of four)
+                if (tid < 4) cand[nc + tid] = 0;
+                __syncthreads();
                 if (tid < nc) {
                     const uint64_t key = cand[tid];
                     uint32_t rank = 0;
-                    for (uint32_t j = 0; j < nc; j++) rank += cand[j] > key ? 1u : 0u;
+                    typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
+                    const u64x2 *c2 = reinterpret_cast<const u64x2 *>(cand);
+#pragma unroll 2
+                    for (uint32_t j = 0; j < (nc + 3) / 4; j++) {
+                        const u64x2 a = c2[2 * j], b = c2[2 * j + 1];
+                        rank += (a.x > key ? 1u : 0u) + (a.y > key ? 1u : 0u) + (b.x > key ? 1u : 0u) + (b.y > key ? 1u : 0u);
+                    }
                     if (rank < k) {
                         const uint32_t idx = ~(uint32_t)key;
                         idx_out[(size_t)row * k + rank] = idx;

@@ -1171,9 +1171,13 @@ def test_dev_gate_knn_reports_counts_and_nan(be, fmt):
     be.h2d(x, X)
     assert be.dev_gate_knn(fmt.FMT_F32, g, x, batch, n, hidden, k, sc, idx, val, cnt)
     assert be.dev_take_nan_flag() is True and be.dev_take_nan_flag() is False   # read once, then clear
+    # the flag stays up until it is taken: a clean call after the poisoned one does not lower it
+    assert be.dev_gate_knn(fmt.FMT_F32, g, x, batch, n, hidden, k, sc, idx, val, cnt)
     X[1, 5] = 0.0
     be.h2d(x, X)
     assert be.dev_gate_knn(fmt.FMT_F32, g, x, batch, n, hidden, k, sc, idx, val)  # (count_out is optional)
+    assert be.dev_take_nan_flag() is True and be.dev_take_nan_flag() is False
+    assert be.dev_gate_knn(fmt.FMT_F32, g, x, batch, n, hidden, k, sc, idx, val)
     assert be.dev_take_nan_flag() is False
     with pytest.raises(Exception):                                               # host tier: the error code
         Xn = X.copy(); Xn[0, 0] = np.nan
