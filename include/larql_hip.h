@@ -317,6 +317,18 @@ int  larql_hip_plan_run(larql_hip_ctx *ctx, larql_hip_plan *plan);
 int  larql_hip_plan_launch_count(const larql_hip_plan *plan);
 void larql_hip_plan_destroy(larql_hip_ctx *ctx, larql_hip_plan *plan);
 
+/* Plans that depend on one another, in order, as one replayable submission: what a token's stages are to the decode
+ * loop (q,k,v | o | gate,up | down per layer, each reading what the stage before wrote).  The peers submit a token's
+ * matvecs as one command buffer (DecodeBackend::decode_token, larql-compute/src/backend/decode.rs:219-); here the
+ * plans' launches are recorded once into a HIP graph — a plan's launches run in order, a plan after the one before
+ * it — and a run replays it on the context's stream without synchronising: the per-launch submission cost is paid
+ * by the graph, not by the caller.  Creating the sequence runs the plans once.  The plans must outlive it. */
+typedef struct larql_hip_sequence larql_hip_sequence;
+int  larql_hip_sequence_create(larql_hip_ctx *ctx, larql_hip_plan *const *plans, size_t n_plans, larql_hip_sequence **out);
+int  larql_hip_sequence_run(larql_hip_ctx *ctx, larql_hip_sequence *seq);
+int  larql_hip_sequence_launch_count(const larql_hip_sequence *seq);
+void larql_hip_sequence_destroy(larql_hip_ctx *ctx, larql_hip_sequence *seq);
+
 /* Scores + top-K by |score| on resident operands (see larql_hip_gate_knn).
  * scores_scratch: [batch, n_features] f32 device buffer (also the full score
  * matrix on return); idx_out/score_out: [batch, top_k] device buffers, of which

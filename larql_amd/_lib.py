@@ -95,6 +95,10 @@ SIGNATURES = {
     "larql_hip_plan_run": (ci, [vp, vp]),
     "larql_hip_plan_launch_count": (ci, [vp]),
     "larql_hip_plan_destroy": (None, [vp, vp]),
+    "larql_hip_sequence_create": (ci, [vp, C.POINTER(vp), sz, C.POINTER(vp)]),
+    "larql_hip_sequence_run": (ci, [vp, vp]),
+    "larql_hip_sequence_launch_count": (ci, [vp]),
+    "larql_hip_sequence_destroy": (None, [vp, vp]),
     "larql_hip_dev_gate_knn": (ci, [vp, ci, vp, vp, sz, sz, sz, sz, vp, vp, vp, vp]),
     "larql_hip_dev_take_nan_flag": (ci, [vp, C.POINTER(ci)]),
     "larql_hip_static_scratch_bytes": (sz, []),

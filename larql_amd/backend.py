@@ -417,6 +417,22 @@ class HipBackend:
     def plan_destroy(self, plan: int) -> None:
         lib.larql_hip_plan_destroy(self._h, plan)
 
+    def sequence_create(self, plans: Sequence[int]) -> Optional[int]:
+        """Plans that depend on one another, in order, as one replayable submission (a HIP graph); None on failure."""
+        arr = (C.c_void_p * max(len(plans), 1))(*plans)
+        p = C.c_void_p()
+        ok = self._some(lib.larql_hip_sequence_create(self._h, arr, len(plans), C.byref(p)))
+        return p.value if ok else None
+
+    def sequence_run(self, seq: int) -> bool:
+        return self._some(lib.larql_hip_sequence_run(self._h, seq))
+
+    def sequence_launch_count(self, seq: int) -> int:
+        return lib.larql_hip_sequence_launch_count(seq)
+
+    def sequence_destroy(self, seq: int) -> None:
+        lib.larql_hip_sequence_destroy(self._h, seq)
+
     def dev_gate_knn(self, fmt: int, gate: int, x: int, batch: int, n: int, hidden: int, top_k: int, scores: int, idx: int,
                      val: int, counts: Optional[int] = None) -> bool:
         return self._some(lib.larql_hip_dev_gate_knn(self._h, fmt, gate, x, batch, n, hidden, top_k, scores, idx, val, counts))

@@ -1241,6 +1241,66 @@ int larql_hip_plan_run(larql_hip_ctx *c, larql_hip_plan *plan) {
 
 int larql_hip_plan_launch_count(const larql_hip_plan *plan) { return plan ? (int)plan->launches.size() : 0; }
 
+struct larql_hip_sequence {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    int launches = 0;
+};
+
+int larql_hip_sequence_create(larql_hip_ctx *c, larql_hip_plan *const *plans, size_t n_plans, larql_hip_sequence **out) {
+    if (!c || !out || (!plans && n_plans)) return LARQL_E_ARG;
+    *out = nullptr;
+    for (size_t i = 0; i < n_plans; i++)
+        if (!plans[i]) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    HIPCHECK(c, hipSetDevice(c->device));
+    // once eagerly: whatever a kernel's first launch sets up (its LDS limit) happens outside the recording
+    for (size_t i = 0; i < n_plans; i++)
+        for (const PreparedLaunch &P : plans[i]->launches) HIPCHECK(c, gemv_launch(c->stream, P.kind, P.L, P.threads, P.grid, P.lds));
+    HIPCHECK(c, hipStreamSynchronize(c->stream));
+    larql_hip_sequence *seq = new larql_hip_sequence();
+    hipError_t e = hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal);
+    if (e == hipSuccess) {
+        for (size_t i = 0; i < n_plans && e == hipSuccess; i++)
+            for (const PreparedLaunch &P : plans[i]->launches) {
+                e = gemv_launch(c->stream, P.kind, P.L, P.threads, P.grid, P.lds);
+                if (e != hipSuccess) break;
+                seq->launches++;
+            }
+        hipGraph_t g = nullptr;
+        const hipError_t e2 = hipStreamEndCapture(c->stream, &g);  // (always ends the recording, also after a failed launch)
+        seq->graph = g;
+        if (e == hipSuccess) e = e2;
+    }
+    if (e == hipSuccess) e = hipGraphInstantiate(&seq->exec, seq->graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        if (seq->exec) (void)hipGraphExecDestroy(seq->exec);
+        if (seq->graph) (void)hipGraphDestroy(seq->graph);
+        delete seq;
+        return fail(c, LARQL_E_DEVICE, "sequence: %s", hipGetErrorString(e));
+    }
+    *out = seq;
+    return LARQL_OK;
+}
+
+int larql_hip_sequence_run(larql_hip_ctx *c, larql_hip_sequence *seq) {
+    if (!c || !seq) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, hipGraphLaunch(seq->exec, c->stream));
+    return LARQL_OK;
+}
+
+int larql_hip_sequence_launch_count(const larql_hip_sequence *seq) { return seq ? seq->launches : 0; }
+
+void larql_hip_sequence_destroy(larql_hip_ctx *c, larql_hip_sequence *seq) {
+    if (!seq) return;
+    if (c) { (void)hipSetDevice(c->device); (void)hipStreamSynchronize(c->stream); }
+    if (seq->exec) (void)hipGraphExecDestroy(seq->exec);
+    if (seq->graph) (void)hipGraphDestroy(seq->graph);
+    delete seq;
+}
+
 void larql_hip_plan_destroy(larql_hip_ctx *c, larql_hip_plan *plan) {
     if (!plan) return;
     if (c) { (void)hipSetDevice(c->device); (void)hipStreamSynchronize(c->stream); }

@@ -19,6 +19,7 @@
 // The arithmetic restates, per format, the reference CPU kernels cited at each
 // routine; only the summation order differs (fp32 accumulate throughout).
 #include <hip/hip_runtime.h>
+#include <cstddef>
 
 #include <atomic>
 #include <stdint.h>
@@ -2751,17 +2752,24 @@ __device__ __forceinline__ void run_dense(const GemvJob &j, uint32_t p0, uint32_
     }
 }
 
-// A job descriptor as wave-uniform values.  The table pointer is generic (it may name the kernel-argument
-// block or device memory), and the compiler treats whatever a generic load returns as different per lane:
-// every address and loop bound derived from it would be computed 64 times over in vector registers.
-// Broadcasting the words from the first lane puts the descriptor, and all arithmetic on it, on the scalar side.
-__device__ __forceinline__ GemvJob uniform_job(const GemvJob *src) {
+// A job descriptor as wave-uniform values.  The table sits in the kernel-argument block or in device memory that
+// nothing writes while the kernel runs (a table built on the device was built by an earlier kernel), so it is read
+// through the constant address space: with a wave-uniform address those are scalar loads — a handful of instructions
+// and the short scalar path, where a vector load of the same words is repeated by every lane and has to be
+// broadcast back word by word — and everything computed from the descriptor stays on the scalar side.
+#define CONST_AS __attribute__((address_space(4)))
+typedef const CONST_AS GemvJob *job_cp;
+__device__ __forceinline__ job_cp job_table(const GemvLaunch &L) { return L.table ? (job_cp)L.table : (job_cp)L.inl; }
+__device__ __forceinline__ uint32_t job_pass_begin(job_cp jobs, uint32_t i) {
+    return *(const CONST_AS uint32_t *)((const CONST_AS uint8_t *)(jobs + i) + offsetof(GemvJob, pass_begin));
+}
+__device__ __forceinline__ GemvJob uniform_job(job_cp src) {
     static_assert(sizeof(GemvJob) % 4 == 0, "descriptor is a whole number of dwords");
     constexpr int N = sizeof(GemvJob) / 4;
+    const CONST_AS uint32_t *p = (const CONST_AS uint32_t *)src;
     uint32_t w[N];
-    __builtin_memcpy(w, src, sizeof(GemvJob));
 #pragma unroll
-    for (int i = 0; i < N; i++) w[i] = __builtin_amdgcn_readfirstlane(w[i]);
+    for (int i = 0; i < N; i++) w[i] = p[i];
     GemvJob j;
     __builtin_memcpy(&j, w, sizeof(GemvJob));
     return j;
@@ -2773,7 +2781,7 @@ __device__ __forceinline__ GemvJob uniform_job(const GemvJob *src) {
 // ---------------------------------------------------------------------------
 template <int KIND, int U>
 __device__ __forceinline__ void gemv_body(const GemvLaunch &L, float *part) {
-    const GemvJob *jobs = L.table ? L.table : L.inl;
+    const job_cp jobs = job_table(L);
     const uint64_t P = L.total_passes;
     uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
     const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
@@ -2781,7 +2789,7 @@ __device__ __forceinline__ void gemv_body(const GemvLaunch &L, float *part) {
     uint32_t lo = 0, hi = L.n_jobs;
     while (lo + 1 < hi) {
         const uint32_t mid = (lo + hi) >> 1;
-        if ((uint32_t)__builtin_amdgcn_readfirstlane(jobs[mid].pass_begin) <= p) lo = mid; else hi = mid;
+        if (job_pass_begin(jobs, mid) <= p) lo = mid; else hi = mid;
     }
     uint32_t ji = lo;
     while (p < p_end) {
@@ -2834,14 +2842,14 @@ LARQL_GEMV_KERNEL(gemv_f32_kernel, KIND_F32, 2, 4)
 // a job, weighted by the job's row length so that shares are equal in bytes), job by job.
 __global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_mfma_kernel(GemvLaunch L) {
     extern __shared__ __attribute__((aligned(16))) uint8_t q4k_lds[];
-    const GemvJob *jobs = L.table ? L.table : L.inl;
+    const job_cp jobs = job_table(L);
     const uint64_t P = L.total_passes;
     uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
     const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
     uint32_t lo = 0, hi = L.n_jobs;
     while (lo + 1 < hi) {
         const uint32_t mid = (lo + hi) >> 1;
-        if ((uint32_t)__builtin_amdgcn_readfirstlane(jobs[mid].pass_begin) <= p) lo = mid; else hi = mid;
+        if (job_pass_begin(jobs, mid) <= p) lo = mid; else hi = mid;
     }
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
@@ -2861,14 +2869,14 @@ __global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_mfma_kernel(GemvLa
 // Q6_K on the matrix cores: the same sweep and cost model as the Q4_K kernel.
 __global__ void __launch_bounds__(kQ6kMaxWaves * 64) gemv_q6k_mfma_kernel(GemvLaunch L) {
     extern __shared__ __attribute__((aligned(16))) uint8_t q6k_lds[];
-    const GemvJob *jobs = L.table ? L.table : L.inl;
+    const job_cp jobs = job_table(L);
     const uint64_t P = L.total_passes;
     uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
     const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
     uint32_t lo = 0, hi = L.n_jobs;
     while (lo + 1 < hi) {
         const uint32_t mid = (lo + hi) >> 1;
-        if ((uint32_t)__builtin_amdgcn_readfirstlane(jobs[mid].pass_begin) <= p) lo = mid; else hi = mid;
+        if (job_pass_begin(jobs, mid) <= p) lo = mid; else hi = mid;
     }
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
@@ -2886,14 +2894,14 @@ __global__ void __launch_bounds__(kQ6kMaxWaves * 64) gemv_q6k_mfma_kernel(GemvLa
 // Q4_K x Q8_K: the same sweep and cost model as the Q4_K kernel.
 __global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_q8k_kernel(GemvLaunch L) {
     extern __shared__ __attribute__((aligned(16))) uint8_t q8k_lds[];
-    const GemvJob *jobs = L.table ? L.table : L.inl;
+    const job_cp jobs = job_table(L);
     const uint64_t P = L.total_passes;
     uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
     const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
     uint32_t lo = 0, hi = L.n_jobs;
     while (lo + 1 < hi) {
         const uint32_t mid = (lo + hi) >> 1;
-        if ((uint32_t)__builtin_amdgcn_readfirstlane(jobs[mid].pass_begin) <= p) lo = mid; else hi = mid;
+        if (job_pass_begin(jobs, mid) <= p) lo = mid; else hi = mid;
     }
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
@@ -2911,7 +2919,7 @@ __global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_q8k_kernel(GemvLau
 // MXFP4 on the matrix cores: same sweep as the Q4_K kernel (cost unit = one tile x one 128-element step).
 __global__ void __launch_bounds__(kMx4MaxWaves * 64) gemv_mxfp4_mfma_kernel(GemvLaunch L) {
     extern __shared__ __attribute__((aligned(16))) uint8_t mx4_lds[];
-    const GemvJob *jobs = L.table ? L.table : L.inl;
+    const job_cp jobs = job_table(L);
     // (a job list built on the device brings its own count and pass total)
     const uint32_t n_jobs = L.dyn ? (uint32_t)__builtin_amdgcn_readfirstlane(((const GLOBAL_AS uint32_t *)L.dyn)[0]) : L.n_jobs;
     const uint64_t P = L.dyn ? (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane(((const GLOBAL_AS uint32_t *)L.dyn)[1]) : L.total_passes;
@@ -2921,7 +2929,7 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) gemv_mxfp4_mfma_kernel(Gemv
     uint32_t lo = 0, hi = n_jobs;
     while (lo + 1 < hi) {
         const uint32_t mid = (lo + hi) >> 1;
-        if ((uint32_t)__builtin_amdgcn_readfirstlane(jobs[mid].pass_begin) <= p) lo = mid; else hi = mid;
+        if (job_pass_begin(jobs, mid) <= p) lo = mid; else hi = mid;
     }
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
@@ -2982,14 +2990,14 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) gemv_mxfp4_mfma_kernel(Gemv
 // bf16 rows x several activations: same sweep (cost unit = one tile x one 128-element column)
 __global__ void __launch_bounds__(kBfMaxWaves * 64) gemv_bf16_mfma_kernel(GemvLaunch L) {
     extern __shared__ __attribute__((aligned(16))) uint8_t bf_lds[];
-    const GemvJob *jobs = L.table ? L.table : L.inl;
+    const job_cp jobs = job_table(L);
     const uint64_t P = L.total_passes;
     uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
     const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
     uint32_t lo = 0, hi = L.n_jobs;
     while (lo + 1 < hi) {
         const uint32_t mid = (lo + hi) >> 1;
-        if ((uint32_t)__builtin_amdgcn_readfirstlane(jobs[mid].pass_begin) <= p) lo = mid; else hi = mid;
+        if (job_pass_begin(jobs, mid) <= p) lo = mid; else hi = mid;
     }
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
@@ -3007,14 +3015,14 @@ __global__ void __launch_bounds__(kBfMaxWaves * 64) gemv_bf16_mfma_kernel(GemvLa
 // Q4_K rows x several activations: same sweep as the single-activation kernel
 __global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_batch_kernel(GemvLaunch L) {
     extern __shared__ __attribute__((aligned(16))) uint8_t q4kb_lds[];
-    const GemvJob *jobs = L.table ? L.table : L.inl;
+    const job_cp jobs = job_table(L);
     const uint64_t P = L.total_passes;
     uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
     const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
     uint32_t lo = 0, hi = L.n_jobs;
     while (lo + 1 < hi) {
         const uint32_t mid = (lo + hi) >> 1;
-        if ((uint32_t)__builtin_amdgcn_readfirstlane(jobs[mid].pass_begin) <= p) lo = mid; else hi = mid;
+        if (job_pass_begin(jobs, mid) <= p) lo = mid; else hi = mid;
     }
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
@@ -3032,14 +3040,14 @@ __global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_batch_kernel(GemvL
 // ggml Q8_0 on the matrix cores: same sweep (cost unit = one tile x one 256-element column)
 __global__ void __launch_bounds__(kQ8MaxWaves * 64) gemv_q8_0_mfma_kernel(GemvLaunch L) {
     extern __shared__ __attribute__((aligned(16))) uint8_t q8_lds[];
-    const GemvJob *jobs = L.table ? L.table : L.inl;
+    const job_cp jobs = job_table(L);
     const uint64_t P = L.total_passes;
     uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
     const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
     uint32_t lo = 0, hi = L.n_jobs;
     while (lo + 1 < hi) {
         const uint32_t mid = (lo + hi) >> 1;
-        if ((uint32_t)__builtin_amdgcn_readfirstlane(jobs[mid].pass_begin) <= p) lo = mid; else hi = mid;
+        if (job_pass_begin(jobs, mid) <= p) lo = mid; else hi = mid;
     }
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {

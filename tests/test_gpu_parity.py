@@ -786,6 +786,46 @@ def test_recorded_plan_replays_and_matches_direct_launches(be, fmt):
     be.plan_destroy(plan)
 
 
+def test_sequence_of_dependent_plans_replays_like_the_eager_launches(be, fmt):
+    """Three stages, each reading what the one before wrote (x -> a,b | a -> c | c,b -> d,e), recorded as one graph.
+    Every replay — with the input rewritten and eager launches of other work on the same stream between them — has to
+    give the bits of the same plans run one by one."""
+    rng = np.random.default_rng(59)
+    k0, ra, rb, rc, rd = 2560, 2048, 1024, 2560, 300
+    q = {}
+    for name, (rows, k, kind) in {"a": (ra, k0, "q4k"), "b": (rb, k0, "q8"), "c": (rc, ra, "q4k"), "d": (rd, rc, "q4k"), "e": (77, rb, "q8")}.items():
+        w = (rng.standard_normal((rows, k)) * 0.02).astype(F)
+        q[name] = (be.to_device(O.quantize_q4_k(w) if kind == "q4k" else O.quantize_q8_0(w)), fmt.FMT_Q4_K if kind == "q4k" else fmt.FMT_GGML_Q8_0, rows, k)
+    x = be.malloc(k0 * 4)
+    buf = {n: be.malloc(v[2] * 4) for n, v in q.items()}
+    job = lambda n, src: (q[n][1], q[n][0], None, src, buf[n], q[n][2], q[n][3])
+    stages = [[job("a", x), job("b", x)], [job("c", buf["a"])], [job("d", buf["c"]), job("e", buf["b"])]]
+    plans = [be.plan_create(st) for st in stages]
+    assert all(plans)
+    seq = be.sequence_create(plans)
+    assert seq and be.sequence_launch_count(seq) == sum(be.plan_launch_count(p) for p in plans) == 5
+    other_x, other_out = be.to_device(rng.standard_normal(k0).astype(F)), be.malloc(ra * 4)
+    for rep in range(4):
+        be.h2d(x, (rng.standard_normal(k0) * (1.0 + rep)).astype(F))
+        for p in plans:                                         # eager, one by one
+            assert be.plan_run(p)
+        be.synchronize()
+        want = {n: be.d2h(buf[n], q[n][2], F) for n in buf}
+        for n in buf:
+            be.h2d(buf[n], np.full(q[n][2], np.nan, F))         # nothing of the eager run may survive into the replay's answer
+        assert be.dev_matvec(q["a"][1], q["a"][0], None, other_x, ra, k0, other_out)   # other work on the stream
+        assert be.sequence_run(seq)
+        assert be.dev_matvec(q["a"][1], q["a"][0], None, other_x, ra, k0, other_out)
+        be.synchronize()
+        for n in buf:
+            got = be.d2h(buf[n], q[n][2], F)
+            assert np.array_equal(got.view(np.uint32), want[n].view(np.uint32)), (rep, n)
+    assert rel_l2(want["a"], O.q4k_matvec(be.d2h(q["a"][0], ra * (k0 // 256) * 144, np.uint8), be.d2h(x, k0, F), ra, k0)) < TOL
+    be.sequence_destroy(seq)
+    for p in plans:
+        be.plan_destroy(p)
+
+
 def test_cpp_host_mirror():
     import os
     import subprocess
