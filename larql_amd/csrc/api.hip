@@ -680,7 +680,7 @@ int larql_hip_q4k_matmul(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, c
         uint16_t *xh = (uint16_t *)c->misc.p, *xl = xh + x_len, *sx = xl + x_len;
         float *ts = (float *)(((uintptr_t)(sx + sx_len) + 15) & ~(uintptr_t)15);
         HIPCHECK(c, hipMemsetAsync(c->nan_flag + 1, 0, sizeof(int), c->stream));
-        HIPCHECK(c, q4k_gemm_prep_launch(c->stream, c->x.p, 0, (uint32_t)hidden, (uint32_t)seq_len, xh, xl, sx, ts, c->nan_flag + 1));
+        HIPCHECK(c, q4k_gemm_prep_launch(c->stream, c->x.p, 0, (uint32_t)hidden, (uint32_t)seq_len, xh, xl, sx, ts, c->nan_flag + 1, nullptr, 0, nullptr));
         int any_lo = 0;
         HIPCHECK(c, hipMemcpyAsync(&any_lo, c->nan_flag + 1, sizeof(int), hipMemcpyDeviceToHost, c->stream));
         HIPCHECK(c, hipStreamSynchronize(c->stream));
@@ -688,10 +688,10 @@ int larql_hip_q4k_matmul(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, c
         const uint32_t splits = q4k_gemm_splits((uint32_t)num_rows, (uint32_t)hidden, (uint32_t)seq_len, (uint32_t)c->cu_count);
         float *partial = nullptr;
         if (splits > 1) { rc = ensure(c, c->scores, (size_t)splits * seq_len * num_rows * 4 + 64); if (rc) return rc; partial = (float *)c->scores.p; }
-        HIPCHECK(c, q4k_gemm_f16_launch(c->stream, dw, xh, sx, ts, (float *)c->out.p, (uint32_t)num_rows, (uint32_t)hidden, (uint32_t)seq_len, 1, 0,
+        HIPCHECK(c, q4k_gemm_f16_launch(c->stream, dw, xh, sx, nullptr, ts, (float *)c->out.p, (uint32_t)num_rows, (uint32_t)hidden, (uint32_t)seq_len, 1, 0,
                                         splits, partial));
         if (any_lo)
-            HIPCHECK(c, q4k_gemm_f16_launch(c->stream, dw, xl, sx, ts, (float *)c->out.p, (uint32_t)num_rows, (uint32_t)hidden, (uint32_t)seq_len, 0, 1,
+            HIPCHECK(c, q4k_gemm_f16_launch(c->stream, dw, xl, sx, nullptr, ts, (float *)c->out.p, (uint32_t)num_rows, (uint32_t)hidden, (uint32_t)seq_len, 0, 1,
                                             splits, partial));
     } else {
         std::vector<GemvJob> jobs;
@@ -1451,15 +1451,16 @@ int larql_hip_dev_q4k_gemm(larql_hip_ctx *c, const uint8_t *w, const uint16_t *x
     HIPCHECK(c, hipSetDevice(c->device));
     // bf16 activations are exact in one f16 term after the per-token scale
     const size_t x_len = seq * hidden, sx_len = seq * (hidden / 32) * 2;
-    int rc = ensure(c, c->misc, x_len * 2 + sx_len * 2 + seq * 4 + 256);
+    int rc = ensure(c, c->misc, x_len * 2 + sx_len * 2 + seq * 4 + rows * 4 + 256);
     if (rc) return rc;
     uint16_t *xh = (uint16_t *)c->misc.p, *sx = xh + x_len;
     float *ts = (float *)(((uintptr_t)(sx + sx_len) + 15) & ~(uintptr_t)15);
-    HIPCHECK(c, q4k_gemm_prep_launch(c->stream, x_bf16, 1, (uint32_t)hidden, (uint32_t)seq, xh, nullptr, sx, ts, nullptr));
+    int *rexp = (int *)(ts + seq);  // the rows' exponents: the rows' scales ride in the f16 weight operand (1.4e-4 of the CPU value)
+    HIPCHECK(c, q4k_gemm_prep_launch(c->stream, x_bf16, 1, (uint32_t)hidden, (uint32_t)seq, xh, nullptr, sx, ts, nullptr, w, (uint32_t)rows, rexp));
     const uint32_t splits = q4k_gemm_splits((uint32_t)rows, (uint32_t)hidden, (uint32_t)seq, (uint32_t)c->cu_count);
     float *partial = nullptr;
     if (splits > 1) { rc = ensure(c, c->scores, (size_t)splits * seq * rows * 4 + 64); if (rc) return rc; partial = (float *)c->scores.p; }
-    HIPCHECK(c, q4k_gemm_f16_launch(c->stream, w, xh, sx, ts, out, (uint32_t)rows, (uint32_t)hidden, (uint32_t)seq, 1, 0, splits, partial));
+    HIPCHECK(c, q4k_gemm_f16_launch(c->stream, w, xh, sx, rexp, ts, out, (uint32_t)rows, (uint32_t)hidden, (uint32_t)seq, 1, 0, splits, partial));
     return LARQL_OK;
 }
 

@@ -130,9 +130,10 @@ hipError_t fill_normal_launch(hipStream_t s, float *dst, size_t n, uint64_t seed
 // batched-prefill Q4_K GEMM (f16 MFMA over the integer weights, fp32 accumulate)
 // integer-weight formulation: activations prepared once (per-token scale, f16 terms, sub-block sums)
 hipError_t q4k_gemm_prep_launch(hipStream_t s, const void *x, int x_is_bf16, uint32_t hidden, uint32_t seq, uint16_t *xh, uint16_t *xl,
-                                uint16_t *sx, float *tok_scale, int *any_lo);
-hipError_t q4k_gemm_f16_launch(hipStream_t s, const uint8_t *w, const uint16_t *xh, const uint16_t *sx, const float *tok_scale, float *out,
-                               uint32_t rows, uint32_t hidden, uint32_t seq, int with_mins, int accumulate, uint32_t splits, float *partial);
+                                uint16_t *sx, float *tok_scale, int *any_lo, const uint8_t *w, uint32_t rows, int *rexp);
+hipError_t q4k_gemm_f16_launch(hipStream_t s, const uint8_t *w, const uint16_t *xh, const uint16_t *sx, const int *rexp, const float *tok_scale,
+                               float *out, uint32_t rows, uint32_t hidden, uint32_t seq, int with_mins, int accumulate, uint32_t splits,
+                               float *partial);
 uint32_t q4k_gemm_splits(uint32_t rows, uint32_t hidden, uint32_t seq, uint32_t cu_count);  // partial: [splits][seq][rows] floats
 
 // One token through a bank of MXFP4 experts, a launch per projection stage (moe1_launch): a small argument block

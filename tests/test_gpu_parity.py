@@ -1145,7 +1145,7 @@ def test_q4k_gemm_mfma_matches_oracle(be, rows, hidden, seq):
     assert be.dev_q4k_gemm(dw, dx, rows, hidden, seq, do)
     be.synchronize()
     got = be.d2h(do, (seq, rows), F)
-    assert rel_l2(got, want) < 1e-4          # stated bar 1e-3; two bf16 weight terms give ~1e-5
+    assert rel_l2(got, want) < 5e-4          # stated bar 1e-3; f16 roundings of the sub-block scales and weights give ~3e-4
     # every output element (guards tile-edge and layout mistakes)
     assert np.max(np.abs(got - want)) < 2e-3 * (np.abs(want).mean() + 1e-9)
 
