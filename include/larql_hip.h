@@ -375,8 +375,12 @@ int larql_hip_dev_gate_walk(larql_hip_ctx *ctx, int format, const void *const *g
 
 /* Batched-prefill GEMM on resident operands: out[seq, rows] = X[seq, hidden] . W[rows, hidden]^T,
  * W in Q4_K, X held as bf16 (the top 16 bits of each f32).  Same contraction as
- * QuantMatVec::q4k_matmul (backend/quant_matvec.rs:324-333): bf16 MFMA with fp32
- * accumulate; each decoded weight enters as two bf16 terms (hi + lo). */
+ * QuantMatVec::q4k_matmul (backend/quant_matvec.rs:324-333), on f16 MFMA with fp32 accumulate: the
+ * activations are exact in f16 after a per-token power-of-two scale, a weight enters as
+ * f16(d 2^E sc6) * (q - 8) (E per row), the sub-blocks' offsets through the sums of the activations.
+ * ~3e-4 relative L2 from the CPU value (the f16 roundings of the sub-block scales and weights);
+ * larql_hip_q4k_matmul keeps exact integer sums instead (~3e-7).  hidden % 256 == 0; w and x_bf16
+ * 16-byte aligned. */
 int larql_hip_dev_q4k_gemm(larql_hip_ctx *ctx, const uint8_t *w, const uint16_t *x_bf16, size_t rows, size_t hidden,
                            size_t seq, float *out);
 

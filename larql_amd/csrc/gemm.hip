@@ -738,23 +738,20 @@ __global__ void __launch_bounds__(QTHREADS) q4k_gemm_pair_kernel(const uint8_t *
         else GEMM_WAIT_VMCNT(9);
         __builtin_amdgcn_s_setprio(3);  // (the multiply phase comes next)
     };
-    // ---- M: the sixteen MFMAs of a prepared step, back to back; at a super-block's second step its offsets first:
-    //      sum_sub (8 d sc6 - dmin mn6) * Sx as one 16-deep MFMA per block, this wavefront taking the token blocks 2kh, 2kh+1 ----
+    // ---- M: the sixteen MFMAs of a prepared step, back to back.  At a super-block's second step the wavefront kh = 0
+    //      first adds the super-block's offsets, sum_sub (8 d sc6 - dmin mn6) * Sx, one 16-deep MFMA per block (all of
+    //      them in one wavefront: a token's sum is then formed in the same order whichever token block it sits in) ----
     auto multiply = [&](const int khc, const int g) {
-        // (the multiplying wavefront runs at high priority, raised at the end of its prepare phase so that it already holds
-        // for the instruction fetches behind the barrier: at equal priority the older wavefront of a SIMD goes first, and
-        // the preparing wavefront's long instruction stream kept the younger one's sixteen MFMAs waiting for their code)
-        if (g == 1 && with_mins) {
-            f16x8 amf[2], bmf[2];
+        if (g == 1 && khc == 0 && with_mins) {
+            f16x8 amf[2], bmf[4];
 #pragma unroll
             for (int i = 0; i < 2; i++) amf[i] = *reinterpret_cast<const f16x8 *>(glds + G_AM_OFF + (wm + i * 32 + row32) * 32 + kgrp * 16);
 #pragma unroll
-            for (int jj = 0; jj < 2; jj++) bmf[jj] = *reinterpret_cast<const f16x8 *>(glds + G_BM_OFF + ((2 * khc + jj) * 32 + row32) * 32 + kgrp * 16);
+            for (int jj = 0; jj < 4; jj++) bmf[jj] = *reinterpret_cast<const f16x8 *>(glds + G_BM_OFF + (jj * 32 + row32) * 32 + kgrp * 16);
 #pragma unroll
             for (int i = 0; i < 2; i++)
 #pragma unroll
-                for (int jj = 0; jj < 2; jj++)
-                    acc[i][2 * khc + jj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(amf[i], bmf[jj], acc[i][2 * khc + jj], 0, 0, 0);
+                for (int jj = 0; jj < 4; jj++) acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(amf[i], bmf[jj], acc[i][jj], 0, 0, 0);
         }
         f16x8 af[2][2];
 #pragma unroll

@@ -276,7 +276,7 @@ def test_prefill_gemm_full_size_exact_scaling_and_token_permutation(be, fmt, row
     wb = be.d2h(w + r0 * (hidden // 256) * 144, 64 * (hidden // 256) * 144, np.uint8)
     for t in (0, 255, 511):
         want = O.q4k_matvec(wb, Xr[t], 64, hidden)
-        assert rel_l2(base[t, r0:r0 + 64], want) < 1e-4
+        assert rel_l2(base[t, r0:r0 + 64], want) < 5e-4     # stated bar 1e-3; the f16 weight operand carries the rows' scales: ~3e-4
     be.free(w); be.free(out)
 
 
