@@ -482,7 +482,7 @@ def run_c5(be, fmt, args):
           {"workload": "BASELINE configs[4]: Q4_K GEMM 512x3840 . (15360x3840, 15360x3840, 3840x15360)", "per_matrix": per,
            "mfma_terms_per_weight": 1, "verified_rel_l2_vs_oracle": max(rels)},
           {"kernel": "q4k_gemm", "bound": "mfma", "achieved": round(tf, 1), "peak": 2500.0, "unit": "TFLOP/s",
-           "frac": round(tf / 2500.0, 4), "traffic": None, "note": "nominal flops 2*S*N*K; one f16 MFMA term per weight (exact integer weight sc6*q), plus one small MFMA per tile and super-block for the mins"},
+           "frac": round(tf / 2500.0, 4), "traffic": None, "note": "nominal flops 2*S*N*K; one f16 MFMA term per weight (the row scales ride in the f16 operand: ~3e-4 from the CPU value), plus one small MFMA per tile and super-block for the offsets"},
           cpu)
 
 

@@ -56,19 +56,23 @@ __global__ void __launch_bounds__(256) q4k_gemm_prep_kernel(const void *__restri
     __shared__ float red[4];
     const uint32_t t = threadIdx.x, nvec = hidden >> 3;  // hidden % 256 == 0
     if (blockIdx.x >= seq) {
-        // the blocks behind the tokens: one thread per weight row, E with max(|d|, |dmin|/16) * 2^E in [0.5, 1) over the row,
-        // so that d 2^E sc6 <= 63 (its -1032-fold stays inside f16) and 32 (8 d sc6 + dmin mn6) 2^E <= 48384
-        const uint32_t row = (blockIdx.x - seq) * 256 + t, nsb = hidden >> 8;
-        if (row >= rows) return;
-        const uint8_t *p = w + (size_t)row * nsb * 144;
+        // the blocks behind the tokens: 16 lanes per weight row, E with max(|d|, |dmin|/16) * 2^E in [0.5, 1) over the row,
+        // so that d 2^E sc6 <= 63 and 32 (8 d sc6 + dmin mn6) 2^E <= 48384 stay well inside f16
+        const uint32_t row = (blockIdx.x - seq) * 16 + (t >> 4), nsb = hidden >> 8;
         float m = 0.f;
-        for (uint32_t sb = 0; sb < nsb; sb++) {
-            const uint32_t h = *reinterpret_cast<const uint32_t *>(p + (size_t)sb * 144);
-            m = fmaxf(m, fmaxf(fabsf(half_to_float(h & 0xFFFFu)), 0.0625f * fabsf(half_to_float(h >> 16))));
+        if (row < rows) {
+            const uint8_t *p = w + (size_t)row * nsb * 144;
+            for (uint32_t sb = t & 15u; sb < nsb; sb += 16) {
+                const uint32_t h = *reinterpret_cast<const uint32_t *>(p + (size_t)sb * 144);
+                m = fmaxf(m, fmaxf(fabsf(half_to_float(h & 0xFFFFu)), 0.0625f * fabsf(half_to_float(h >> 16))));
+            }
         }
-        int e = 0;
-        if (m > 0.f && m < __builtin_inff()) (void)frexpf(m, &e);
-        rexp[row] = -e;
+        for (int o = 8; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+        if (row < rows && (t & 15u) == 0) {
+            int e = 0;
+            if (m > 0.f && m < __builtin_inff()) (void)frexpf(m, &e);
+            rexp[row] = -e;
+        }
         return;
     }
     const uint32_t tok = blockIdx.x;
@@ -105,8 +109,9 @@ __global__ void __launch_bounds__(256) q4k_gemm_prep_kernel(const void *__restri
     const float to_h = ldexpf(1.f, 14 - ex);
     if (t == 0) tok_scale[tok] = ldexpf(1.f, ex - 14);
     int lo_seen = 0;
-    // the f16 terms are kept as [step of 64 k][token][64] and the sums as [super-block][token][8]: what a GEMM workgroup
-    // copies for a step or a super-block is one contiguous run
+    // the f16 terms are kept as [token][hidden] (a step's 128 bytes of a token are one cache line; a [step][token] order
+    // was measured: no faster for the GEMM, slower here) and the sums as [super-block][token][8], so that what a GEMM
+    // workgroup copies of them for a super-block is one contiguous run
     u32x4 *oh = reinterpret_cast<u32x4 *>(xh);
     u32x4 *ol = xl ? reinterpret_cast<u32x4 *>(xl) : nullptr;
     for (uint32_t v = t; v < nvec; v += 256) {  // nvec % 32 == 0: the four threads of a sub-block run together
@@ -127,7 +132,7 @@ __global__ void __launch_bounds__(256) q4k_gemm_prep_kernel(const void *__restri
             lo_seen |= (ol && (float)l != 0.f) ? 1 : 0;
             sm += (float)h + (ol ? (float)l : 0.f);  // the activation as the MFMAs will see it
         }
-        const size_t at = ((size_t)(v >> 3) * seq + tok) * 8 + (v & 7u);
+        const size_t at = (size_t)tok * nvec + v;
         oh[at] = (u32x4){hw[0], hw[1], hw[2], hw[3]};
         if (ol) ol[at] = (u32x4){lw[0], lw[1], lw[2], lw[3]};
         sm += __shfl_xor(sm, 1);
@@ -222,13 +227,13 @@ __global__ void __launch_bounds__(GTHREADS, 1) q4k_gemm_exact_kernel(const uint8
         const uint32_t idx = p9 * 64 + lane;
         r_off[p9] = (min(row0 + wave * 64 + idx / 9, rows - 1) - row0) * row_bytes + (idx % 9) * 16;
     }
-    // activations ([step][token][64 f16]): wavefront -> tokens 32w .. 32w+31 (four copies of 8 tokens x 128 bytes), lane -> (token, chunk)
+    // activations ([token][hidden] f16): wavefront -> tokens 32w .. 32w+31 (four copies of 8 tokens x 128 bytes), lane -> (token, chunk)
     const uint8_t *xt = (const uint8_t *)xh;                                                   // uniform
     uint32_t b_off[4];
 #pragma unroll
     for (int q = 0; q < 4; q++) {
         const uint32_t r = (wave * 4 + q) * 8 + (lane >> 3);
-        b_off[q] = min(tok0 + r, seq - 1) * 128 + (((lane & 7u) ^ ((r >> 1) & 7u)) * 16);
+        b_off[q] = min(tok0 + r, seq - 1) * hidden * 2 + (((lane & 7u) ^ ((r >> 1) & 7u)) * 16);
     }
     // Sx ([super-block][token][8 pairs]): wavefront -> tokens 32w .. 32w+31 (two 16-byte halves each)
     const uint8_t *st = (const uint8_t *)sx;                                                   // uniform
@@ -247,7 +252,7 @@ __global__ void __launch_bounds__(GTHREADS, 1) q4k_gemm_exact_kernel(const uint8
     };
     auto issue_b = [&](uint32_t s, uint32_t slot, int q) {  // one of the four pieces of a step
         const uint32_t sc = min(s, nsteps - 1);
-        const uint8_t *src = xt + ((size_t)sb_begin * 4 + sc) * seq * 128;
+        const uint8_t *src = xt + ((size_t)sb_begin * 4 + sc) * 128;
         uint8_t *dst = glds + G_B_OFF + slot * G_B_STAGE + wave * 4096;
         __builtin_amdgcn_global_load_lds((p_g_vp)(src + b_off[q]), (p_lds_vp)(dst + q * 1024), 16, 0, 0);
     };
@@ -597,13 +602,13 @@ __global__ void __launch_bounds__(QTHREADS) q4k_gemm_pair_kernel(const uint8_t *
         r_off[p] = (min(row0 + wm + idx / 9, rows - 1) - row0) * row_bytes + (idx % 9) * 16;
     }
     const uint32_t own_row = min(row0 + wm + lane, rows - 1);   // the row whose table entries this thread writes
-    // activations ([step][token][64 f16]): wavefront -> tokens 16w .. 16w+15 (two copies of 8 tokens x 128 bytes)
+    // activations ([token][hidden] f16): wavefront -> tokens 16w .. 16w+15 (two copies of 8 tokens x 128 bytes)
     const uint8_t *xt = (const uint8_t *)xh;                                                   // uniform
     uint32_t b_off[2];
 #pragma unroll
     for (int q = 0; q < 2; q++) {
         const uint32_t r = (wave * 2 + q) * 8 + (lane >> 3);
-        b_off[q] = min(tok0 + r, seq - 1) * 128 + (((lane & 7u) ^ ((r >> 1) & 7u)) * 16);
+        b_off[q] = min(tok0 + r, seq - 1) * hidden * 2 + (((lane & 7u) ^ ((r >> 1) & 7u)) * 16);
     }
     // Sx ([super-block][token][8 pairs]): the wavefronts kh = 1 -> tokens 32wq .. 32wq+31 (two 16-byte halves each)
     const uint8_t *st = (const uint8_t *)sx;                                                   // uniform
@@ -620,7 +625,7 @@ __global__ void __launch_bounds__(QTHREADS) q4k_gemm_pair_kernel(const uint8_t *
     };
     auto issue_b = [&](uint32_t s, uint32_t slot, int q) {  // one of the two pieces of a step
         const uint32_t sc = min(s, nsteps - 1);
-        const uint8_t *src = xt + ((size_t)sb_begin * 4 + sc) * seq * 128;
+        const uint8_t *src = xt + ((size_t)sb_begin * 4 + sc) * 128;
         copy16_to_lds(src, b_off[q], lds0 + G_B_OFF + slot * G_B_STAGE + wave * 2048 + q * 1024);
     };
     auto issue_sx = [&](uint32_t sb) {  // a quarter of a super-block's Sx
@@ -876,7 +881,7 @@ __global__ void __launch_bounds__(QTHREADS) q4k_gemm_pair_kernel(const uint8_t *
 hipError_t q4k_gemm_prep_launch(hipStream_t s, const void *x, int x_is_bf16, uint32_t hidden, uint32_t seq, uint16_t *xh, uint16_t *xl,
                                 uint16_t *sx, float *tok_scale, int *any_lo, const uint8_t *w, uint32_t rows, int *rexp) {
     if (seq == 0) return hipSuccess;
-    const uint32_t row_blocks = rexp ? (rows + 255) / 256 : 0;
+    const uint32_t row_blocks = rexp ? (rows + 15) / 16 : 0;
     hipLaunchKernelGGL(q4k_gemm_prep_kernel, dim3(seq + row_blocks), dim3(256), 0, s, x, x_is_bf16, hidden, xh, xl, sx, tok_scale, any_lo,
                        1, seq, w, rows, rexp);
     return hipGetLastError();
