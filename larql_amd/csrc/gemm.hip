@@ -48,23 +48,27 @@ typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 // one block per token: scale, f16 terms, sub-block sums.  `x_is_bf16`: 16-bit inputs (exact in one term).
 // A thread takes 8 consecutive elements at a time (one or two 16-byte loads); four neighbouring threads hold a
 // 32-element sub-block.
-__global__ void __launch_bounds__(256) q4k_gemm_prep_kernel(const void *__restrict__ x, int x_is_bf16, uint32_t hidden,
+__global__ void __launch_bounds__(1024) q4k_gemm_prep_kernel(const void *__restrict__ x, int x_is_bf16, uint32_t hidden,
                                                             uint16_t *__restrict__ xh, uint16_t *__restrict__ xl,
                                                             uint16_t *__restrict__ sx, float *__restrict__ tok_scale,
                                                             int *__restrict__ any_lo, int swap12, uint32_t seq,
                                                             const uint8_t *__restrict__ w, uint32_t rows, int *__restrict__ rexp) {
-    __shared__ float red[4];
+    __shared__ float red[16];
     const uint32_t t = threadIdx.x, nvec = hidden >> 3;  // hidden % 256 == 0
     if (blockIdx.x >= seq) {
         // the blocks behind the tokens: 16 lanes per weight row, E with max(|d|, |dmin|/16) * 2^E in [0.5, 1) over the row,
         // so that d 2^E sc6 <= 63 and 32 (8 d sc6 + dmin mn6) 2^E <= 48384 stay well inside f16
-        const uint32_t row = (blockIdx.x - seq) * 16 + (t >> 4), nsb = hidden >> 8;
+        const uint32_t row = (blockIdx.x - seq) * (blockDim.x >> 4) + (t >> 4), nsb = hidden >> 8;
         float m = 0.f;
         if (row < rows) {
             const uint8_t *p = w + (size_t)row * nsb * 144;
-            for (uint32_t sb = t & 15u; sb < nsb; sb += 16) {
-                const uint32_t h = *reinterpret_cast<const uint32_t *>(p + (size_t)sb * 144);
-                m = fmaxf(m, fmaxf(fabsf(half_to_float(h & 0xFFFFu)), 0.0625f * fabsf(half_to_float(h >> 16))));
+            for (uint32_t sb0 = t & 15u; sb0 < nsb; sb0 += 64) {  // four independent loads in flight per lane
+                uint32_t h[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) h[u] = sb0 + 16 * u < nsb ? *reinterpret_cast<const uint32_t *>(p + (size_t)(sb0 + 16 * u) * 144) : 0u;
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+                    m = fmaxf(m, fmaxf(fabsf(half_to_float(h[u] & 0xFFFFu)), 0.0625f * fabsf(half_to_float(h[u] >> 16))));
             }
         }
         for (int o = 8; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
@@ -93,7 +97,7 @@ __global__ void __launch_bounds__(256) q4k_gemm_prep_kernel(const void *__restri
         }
     };
     float mx = 0.f;
-    for (uint32_t v = t; v < nvec; v += 256) {
+    for (uint32_t v = t; v < nvec; v += blockDim.x) {
         float o[8];
         load8(v, o);
 #pragma unroll
@@ -102,7 +106,8 @@ __global__ void __launch_bounds__(256) q4k_gemm_prep_kernel(const void *__restri
     for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
     if ((t & 63u) == 0) red[t >> 6] = mx;
     __syncthreads();
-    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    mx = 0.f;
+    for (uint32_t wv = 0; wv < (blockDim.x >> 6); wv++) mx = fmaxf(mx, red[wv]);
     int ex = 0;
     if (mx > 0.f && mx < __builtin_inff()) (void)frexpf(mx, &ex);
     ex = max(-100, min(110, ex));
@@ -114,7 +119,7 @@ __global__ void __launch_bounds__(256) q4k_gemm_prep_kernel(const void *__restri
     // workgroup copies of them for a super-block is one contiguous run
     u32x4 *oh = reinterpret_cast<u32x4 *>(xh);
     u32x4 *ol = xl ? reinterpret_cast<u32x4 *>(xl) : nullptr;
-    for (uint32_t v = t; v < nvec; v += 256) {  // nvec % 32 == 0: the four threads of a sub-block run together
+    for (uint32_t v = t; v < nvec; v += blockDim.x) {  // nvec % 32 == 0: the four threads of a sub-block run together
         float o[8];
         load8(v, o);
         uint32_t hw[4] = {0u, 0u, 0u, 0u}, lw[4] = {0u, 0u, 0u, 0u};
@@ -148,15 +153,34 @@ __global__ void __launch_bounds__(256) q4k_gemm_prep_kernel(const void *__restri
     if (lo_seen && any_lo) *any_lo = 1;
 }
 
-// adds the partial slabs of a K-split in slab order and applies the token scale
+// adds the partial slabs of a K-split in slab order and applies the token scale; VEC elements per thread (4 when
+// rows % 4 == 0 and everything is 16-byte aligned: the four are then of one token)
+template <int VEC>
 __global__ void __launch_bounds__(256) q4k_gemm_reduce_kernel(const float *__restrict__ partial, uint32_t splits, const float *__restrict__ tok_scale,
                                                               float *__restrict__ out, uint32_t rows, uint32_t seq, int accumulate) {
-    const size_t n = (size_t)rows * seq, i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t n = (size_t)rows * seq, i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
     if (i >= n) return;
-    float s = 0.f;
-    for (uint32_t z = 0; z < splits; z++) s += partial[(size_t)z * n + i];
-    s *= tok_scale[i / rows];
-    out[i] = accumulate ? out[i] + s : s;
+    float s[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) s[e] = 0.f;
+    for (uint32_t z = 0; z < splits; z++) {
+        if (VEC == 4) {
+            const f32x4 v = *reinterpret_cast<const f32x4 *>(partial + (size_t)z * n + i);
+#pragma unroll
+            for (int e = 0; e < VEC; e++) s[e] += v[e];
+        } else {
+            s[0] += partial[(size_t)z * n + i];
+        }
+    }
+    const float ts = tok_scale[i / rows];
+    if (VEC == 4) {
+        f32x4 r = {s[0] * ts, s[VEC > 1 ? 1 : 0] * ts, s[VEC > 2 ? 2 : 0] * ts, s[VEC > 3 ? 3 : 0] * ts};
+        f32x4 *o = reinterpret_cast<f32x4 *>(out + i);
+        if (accumulate) r += *o;
+        *o = r;
+    } else {
+        out[i] = accumulate ? out[i] + s[0] * ts : s[0] * ts;
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -881,8 +905,11 @@ __global__ void __launch_bounds__(QTHREADS) q4k_gemm_pair_kernel(const uint8_t *
 hipError_t q4k_gemm_prep_launch(hipStream_t s, const void *x, int x_is_bf16, uint32_t hidden, uint32_t seq, uint16_t *xh, uint16_t *xl,
                                 uint16_t *sx, float *tok_scale, int *any_lo, const uint8_t *w, uint32_t rows, int *rexp) {
     if (seq == 0) return hipSuccess;
-    const uint32_t row_blocks = rexp ? (rows + 15) / 16 : 0;
-    hipLaunchKernelGGL(q4k_gemm_prep_kernel, dim3(seq + row_blocks), dim3(256), 0, s, x, x_is_bf16, hidden, xh, xl, sx, tok_scale, any_lo,
+    // a token per block; wide activations take more threads per token (two passes over the token: 256 threads on 15360
+    // elements are 15 dependent rounds of loads)
+    const uint32_t threads = hidden >= 8192 ? 1024u : 256u;
+    const uint32_t row_blocks = rexp ? (rows + threads / 16 - 1) / (threads / 16) : 0;
+    hipLaunchKernelGGL(q4k_gemm_prep_kernel, dim3(seq + row_blocks), dim3(threads), 0, s, x, x_is_bf16, hidden, xh, xl, sx, tok_scale, any_lo,
                        1, seq, w, rows, rexp);
     return hipGetLastError();
 }
@@ -924,7 +951,10 @@ hipError_t q4k_gemm_f16_launch(hipStream_t s, const uint8_t *w, const uint16_t *
                            accumulate, per, slab);
     if (split) {
         const size_t n = (size_t)rows * seq;
-        hipLaunchKernelGGL(q4k_gemm_reduce_kernel, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, s, partial, z, tok_scale, out, rows, seq, accumulate);
+        if (rows % 4 == 0 && (((uintptr_t)partial | (uintptr_t)out) & 15u) == 0)
+            hipLaunchKernelGGL(q4k_gemm_reduce_kernel<4>, dim3((uint32_t)((n / 4 + 255) / 256)), dim3(256), 0, s, partial, z, tok_scale, out, rows, seq, accumulate);
+        else
+            hipLaunchKernelGGL(q4k_gemm_reduce_kernel<1>, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, s, partial, z, tok_scale, out, rows, seq, accumulate);
     }
     return hipGetLastError();
 }
