@@ -1150,6 +1150,43 @@ def test_q4k_gemm_mfma_matches_oracle(be, rows, hidden, seq):
     assert np.max(np.abs(got - want)) < 2e-3 * (np.abs(want).mean() + 1e-9)
 
 
+def test_q4k_gemm_row_scales_of_any_size_and_uneven_blocks(be):
+    """The device tier's GEMM carries each row's scale in an f16 operand behind a per-row exponent: rows whose weights
+    differ by twelve orders of magnitude, rows of zeros, and a row with one super-block far larger than the others
+    all have to come out to the same relative accuracy (per row, against the oracle)."""
+    rng = np.random.default_rng(97)
+    rows, hidden, seq = 320, 1024, 48
+    w = (rng.standard_normal((rows, hidden)) * 0.02).astype(F)
+    w *= (10.0 ** rng.uniform(-8, 4, size=(rows, 1))).astype(F)        # row scales from 1e-8 to 1e4
+    w[5] = 0.0                                                          # a row of zeros
+    w[17] = 0.0; w[17, 256:512] = (rng.standard_normal(256) * 3.0).astype(F)   # only one super-block holds anything
+    w[33, :256] *= F(4096.0)                                            # one super-block 4096 times the others
+    w[40, 512:768] *= F(1.0 / 4096.0)
+    q = O.quantize_q4_k(w)
+    xb = O.f32_to_bf16(rng.standard_normal((seq, hidden)).astype(F))
+    X = (xb.astype(np.uint32) << 16).view(F).reshape(seq, hidden)
+    want = O.q4k_matmul(q, X, rows, hidden, seq)                        # [seq, rows]
+    dw, dx, do = be.to_device(q), be.to_device(xb), be.malloc(seq * rows * 4)
+    assert be.dev_q4k_gemm(dw, dx, rows, hidden, seq, do)
+    be.synchronize()
+    got = be.d2h(do, (seq, rows), F)
+    assert np.isfinite(got).all()
+    assert np.array_equal(got[:, 5], np.zeros(seq, F))
+    for r in range(rows):
+        n = np.linalg.norm(want[:, r].astype(np.float64))
+        if n > 0:
+            assert np.linalg.norm(got[:, r].astype(np.float64) - want[:, r]) / n < 1e-3, r   # the stated bar, row by row
+    assert rel_l2(got / np.maximum(np.abs(want).max(axis=0), 1e-30), want / np.maximum(np.abs(want).max(axis=0), 1e-30)) < 5e-4
+    # the host tier keeps exact integer sums: the same matrix to ~1e-6 of the oracle per row
+    Xf = rng.standard_normal((seq, hidden)).astype(F)
+    got_h = be.q4k_matmul(q, Xf, rows, hidden, seq).reshape(seq, rows)
+    want_h = O.q4k_matmul(q, Xf, rows, hidden, seq)
+    for r in range(rows):
+        n = np.linalg.norm(want_h[:, r].astype(np.float64))
+        if n > 0:
+            assert np.linalg.norm(got_h[:, r].astype(np.float64) - want_h[:, r]) / n < 2e-5, r
+
+
 def test_q4k_matmul_host_tier_uses_gemm_for_prefill_shapes(be):
     rng = np.random.default_rng(67)
     rows, hidden, seq = 200, 1024, 40
