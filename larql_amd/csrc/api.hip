@@ -1576,9 +1576,8 @@ static int moe_mxfp4_block(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank
     }
     const bool route_in_launch = route_logits && tokens == 1 &&
         gemv_effective_kind(make_job(KIND_MXFP4, bank->gate_packed, bank->gate_scales, x, g, gu_rows, hidden)) == KIND_MXFP4_MFMA;
-    if (route_logits && !route_in_launch)
-        HIPCHECK(c, router_select_launch(c->stream, route_logits, bank->router_bias, (uint32_t)tokens, (uint32_t)bank->n_experts, (uint32_t)k,
-                                         route_policy, experts, weights));
+    // (the selection kernel, unless the planner below does the selecting itself)
+    bool router_pending = route_logits && !route_in_launch;
     // Several tokens: slots that chose the same expert share its weights up to four at a time.  The job lists are built on
     // the device from the router's choice (moe_plan_kernel) into the workspace's spare activation area.
     {
@@ -1622,7 +1621,8 @@ static int moe_mxfp4_block(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank
                 P.grid = (uint32_t)((uint64_t)c->cu_count * gemv_wgs_per_cu(P.kind, P.threads, P.lds, (uint32_t)c->wgs_per_cu));
             }
             if (!gemv_job_geometry(tu, Pg.threads)) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: unsupported geometry");
-            HIPCHECK(c, moe_plan_launch(c->stream, experts, (uint32_t)slots, (uint32_t)k, (uint32_t)bank->n_experts, tg, tu, td, gu_w_stride,
+            HIPCHECK(c, moe_plan_launch(c->stream, router_pending ? route_logits : nullptr, bank->router_bias, route_policy, weights, experts,
+                                        (uint32_t)slots, (uint32_t)k, (uint32_t)bank->n_experts, tg, tu, td, gu_w_stride,
                                         gu_s_stride, dn_w_stride, dn_s_stride, (uint32_t)hidden, (uint32_t)inter, fused, group, gu_table, hdr,
                                         dn_table, hdr + 2));
             HIPCHECK(c, gemv_launch(c->stream, Pg.kind, Pg.L, Pg.threads, Pg.grid, Pg.lds));
@@ -1632,6 +1632,9 @@ static int moe_mxfp4_block(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank
             return LARQL_OK;
         }
     }
+    if (router_pending)
+        HIPCHECK(c, router_select_launch(c->stream, route_logits, bank->router_bias, (uint32_t)tokens, (uint32_t)bank->n_experts, (uint32_t)k,
+                                         route_policy, experts, weights));
     std::vector<GemvJob> jobs;
     for (size_t s = 0; s < slots; s++) {
         const size_t t = s / k;

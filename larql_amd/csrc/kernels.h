@@ -179,7 +179,9 @@ hipError_t moe1_launch(hipStream_t s, const Moe1Args &A, bool down, uint32_t gri
 // MoE helpers
 hipError_t router_select_launch(hipStream_t s, const float *logits, const float *bias, uint32_t tokens, uint32_t n_experts, uint32_t k,
                                 int policy, uint32_t *experts, float *weights);
-hipError_t moe_plan_launch(hipStream_t s, const uint32_t *experts, uint32_t slots, uint32_t k, uint32_t n_experts, const GemvJob &tg,
+// (logits != nullptr: the kernel selects the experts itself first — at most 64 experts, top-kRouterMaxK — and writes experts / weights)
+hipError_t moe_plan_launch(hipStream_t s, const float *logits, const float *router_bias, int policy, float *weights, uint32_t *experts,
+                           uint32_t slots, uint32_t k, uint32_t n_experts, const GemvJob &tg,
                            const GemvJob &tu, const GemvJob &td, uint64_t gu_w_stride, uint64_t gu_s_stride, uint64_t dn_w_stride,
                            uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, bool fused, uint32_t group, GemvJob *gu_table, uint32_t *gu_hdr,
                            GemvJob *dn_table, uint32_t *dn_hdr);

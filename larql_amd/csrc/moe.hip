@@ -82,7 +82,10 @@ __global__ void weighted_sum_kernel(const float *__restrict__ d, const float *__
 // headers: {job count, pass total}.  One block; a thread per slot, O(slots) work each.
 // `fused`: tg walks a fused gate_up matrix of 2*inter interleaved rows (no up jobs; a slot's results and the down
 // job's activation are 2*inter floats, gate and up values alternating).
-__global__ void __launch_bounds__(256) moe_plan_kernel(const uint32_t *__restrict__ experts, uint32_t slots, uint32_t k, uint32_t n_experts,
+// With `logits` the kernel is the router as well (one launch fewer in front of the matvecs): a wavefront per token
+// selects as router_select_kernel does and writes `experts` / `weights` before the planning reads the choice.
+__global__ void __launch_bounds__(1024) moe_plan_kernel(const float *__restrict__ logits, const float *__restrict__ router_bias, int policy,
+                                                       float *__restrict__ weights, uint32_t *__restrict__ experts, uint32_t slots, uint32_t k, uint32_t n_experts,
                                                        GemvJob tg, GemvJob tu, GemvJob td, uint64_t gu_w_stride, uint64_t gu_s_stride,
                                                        uint64_t dn_w_stride, uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, uint32_t fused,
                                                        uint32_t group, GemvJob *__restrict__ gu_table, uint32_t *__restrict__ gu_hdr,
@@ -97,7 +100,26 @@ __global__ void __launch_bounds__(256) moe_plan_kernel(const uint32_t *__restric
     const uint32_t t = threadIdx.x;
     const uint32_t gsh = group == 4 ? 2u : 1u, gmask = group - 1;  // (group is 2 or 4: no divisions below)
     for (uint32_t e = t; e < ((n_experts + 3u) & ~3u); e += blockDim.x) cnt[e] = 0;
-    for (uint32_t s = t; s < ((slots + 3u) & ~3u); s += blockDim.x) ex[s] = s < slots ? experts[s] : 0xFFFFFFFFu;
+    if (logits) {
+        const uint32_t lane = t & 63u, tokens = slots / k;
+        for (uint32_t tok = t >> 6; tok < tokens; tok += blockDim.x >> 6) {
+            uint32_t sel_idx[kRouterMaxK];
+            float sel_w[kRouterMaxK];
+            router_select_wave(logits + (size_t)tok * n_experts, router_bias, n_experts, k, policy, lane, sel_idx, sel_w);
+            if (lane == 0) {
+#pragma unroll
+                for (int r = 0; r < kRouterMaxK; r++)
+                    if ((uint32_t)r < k) {
+                        experts[(size_t)tok * k + r] = sel_idx[r];
+                        weights[(size_t)tok * k + r] = sel_w[r];
+                        ex[tok * k + r] = sel_idx[r];
+                    }
+            }
+        }
+        for (uint32_t s2 = slots + t; s2 < ((slots + 3u) & ~3u); s2 += blockDim.x) ex[s2] = 0xFFFFFFFFu;
+    } else {
+        for (uint32_t s = t; s < ((slots + 3u) & ~3u); s += blockDim.x) ex[s] = s < slots ? experts[s] : 0xFFFFFFFFu;
+    }
     __syncthreads();
     // ranks: four earlier slots per LDS read, the reads of a round independent of each other
     for (uint32_t s = t; s < slots; s += blockDim.x) {
@@ -207,12 +229,15 @@ __global__ void __launch_bounds__(256) moe_plan_kernel(const uint32_t *__restric
     }
 }
 
-hipError_t moe_plan_launch(hipStream_t s, const uint32_t *experts, uint32_t slots, uint32_t k, uint32_t n_experts, const GemvJob &tg,
+hipError_t moe_plan_launch(hipStream_t s, const float *logits, const float *router_bias, int policy, float *weights, uint32_t *experts,
+                           uint32_t slots, uint32_t k, uint32_t n_experts, const GemvJob &tg,
                            const GemvJob &tu, const GemvJob &td, uint64_t gu_w_stride, uint64_t gu_s_stride, uint64_t dn_w_stride,
                            uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, bool fused, uint32_t group, GemvJob *gu_table, uint32_t *gu_hdr,
                            GemvJob *dn_table, uint32_t *dn_hdr) {
     if (n_experts > 1024 || slots > 4096 || (group != 2 && group != 4)) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(256), 0, s, experts, slots, k, n_experts, tg, tu, td, gu_w_stride, gu_s_stride,
+    // (a wavefront per token while selecting: 16 wavefronts when the kernel routes)
+    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(logits ? 1024 : 256), 0, s, logits, router_bias, policy, weights, experts, slots, k, n_experts, tg, tu, td,
+                       gu_w_stride, gu_s_stride,
                        dn_w_stride, dn_s_stride, hidden, inter, fused ? 1u : 0u, group, gu_table, gu_hdr, dn_table, dn_hdr);
     return hipGetLastError();
 }
