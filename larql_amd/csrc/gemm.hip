@@ -591,7 +591,11 @@ __global__ void __launch_bounds__(GTHREADS, 1) q4k_gemm_exact_kernel(const uint8
 // step's k: wavefront kh takes the nibbles kh (k 32kh .. 32kh+31 of the step: sub-block 2g + kh) of the same raw bytes
 // against the same tokens.  No weight is converted twice and no activation read twice; each wavefront keeps a full
 // set of partial sums (128 registers), which the pair adds up through LDS at the end.  The rows' scales ride in the
-// operand (see above); the exact variant does not fit in 256 registers and stays with the 4-wavefront kernel.
+// operand (the formulation at the top of this file); with a second set of accumulators the exact variant does not
+// fit in the 256 registers a wavefront has here and stays with q4k_gemm_exact_kernel.
+// The two wavefronts of a SIMD take turns (see the loop): while one issues a step's 16 MFMAs back to back, the other
+// prepares its next step; with both doing a bit of everything all the time, a workgroup barrier per step made them
+// run one after the other, each at about half the matrix pipe's rate.
 // ---------------------------------------------------------------------------
 constexpr int QTHREADS = 512;
 // one global -> LDS copy of 16 bytes per lane: uniform base + per-lane 32-bit offset on the global side (no 64-bit
@@ -616,8 +620,10 @@ __global__ void __launch_bounds__(QTHREADS) q4k_gemm_pair_kernel(const uint8_t *
     const uint32_t nsteps = (sb_end - sb_begin) * 4;
     const uint32_t wm = wq * 64;
 
-    // copy roles.  Weights: the nine pieces of a row group's super-block (see the 4-wavefront kernel) are shared out 5 : 4
-    // over the pair; the wavefront with 4 brings a quarter of Sx as its fifth copy.
+    // copy roles.  Weights: a super-block of a row group's 64 rows (144 bytes each, header included) is nine copies; piece p,
+    // lane l brings 16-byte chunk (64p + l) % 9 of row (64p + l) / 9, so that the rows lie in LDS one after the other and
+    // a row's two or three cache lines are asked for by neighbouring lanes of one instruction.  The nine are shared out
+    // 5 : 4 over the pair; the wavefront with 4 brings a quarter of Sx as its fifth copy.
     const uint8_t *wt = w + (size_t)row0 * row_bytes;                                          // uniform
     uint32_t r_off[5];
 #pragma unroll
@@ -656,8 +662,12 @@ __global__ void __launch_bounds__(QTHREADS) q4k_gemm_pair_kernel(const uint8_t *
         const uint32_t sbc = min(sb, sb_end - 1);
         copy16_to_lds(st + (size_t)sbc * seq * 32, m_off, lds0 + G_BM_OFF + wq * 1024);
     };
-    // a super-block's header -> this row's table entries: the scales of the sub-blocks 2u + kh (the ones this wavefront
-    // converts) and the offsets' operand of the sub-blocks 4kh .. 4kh+3 (see the 4-wavefront kernel for both)
+    // a super-block's header -> this row's table entries (one thread per row).  Scales: s = f16(d 2^E sc6) of the
+    // sub-blocks 2u + kh, the ones this wavefront converts; the operand is s (q - 8): centred weights, so that the
+    // weight term and the offset term are both of the result's size and their f16 roundings are not magnified by a
+    // cancellation (with s q and -dmin mn6 Sx the error was 8e-4, so 2.9e-4).  The high nibbles' masked value is
+    // 1024 + 16q, so kh = 1 carries s/16.  Offsets' operand of the sub-blocks 4kh .. 4kh+3: 32 (8 d sc6 - dmin mn6) 2^E,
+    // twice, for the two f16 halves of Sx/32.
     auto stage_sb = [&](uint32_t par) {
         const u32x4 hdr = *reinterpret_cast<const u32x4 *>(glds + G_R_OFF + par * G_R_STAGE + wq * 9216 + lane * 144);
         const float d = half_to_float(hdr.x & 0xFFFFu), dmin = half_to_float(hdr.x >> 16);
@@ -682,7 +692,11 @@ __global__ void __launch_bounds__(QTHREADS) q4k_gemm_pair_kernel(const uint8_t *
         }
         *reinterpret_cast<u32x4 *>(glds + G_AM_OFF + (wm + lane) * 32 + kh * 16) = (u32x4){mnw[0], mnw[1], mnw[2], mnw[3]};
     };
-    // 4 raw bytes (nibble kh) -> two dwords of f16(s (q - 8)) as the pairs (k0, k2) and (k1, k3) (see the 4-wavefront kernel)
+    // 4 raw bytes (nibble kh) -> two dwords of f16(s (q - 8)) as the pairs (k0, k2) and (k1, k3): the nibbles of bytes 0
+    // and 2 are masked in place into the mantissas of two f16 (1024 + q, or 1024 + 16q for the high nibbles), those of
+    // bytes 1 and 3 after one shift; a packed add takes 1032 (1152) away, which is exact, and a packed multiply applies s:
+    // one rounding (-1032 s itself has no f16, so a single FMA cannot do it).  `magic` is 0x64006400 held in a register
+    // so that mask-and-or is one instruction.
     uint32_t magic;
     asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
     const uint32_t take = kh ? 0xE480E480u : 0xE408E408u;  // -1152 | -1032, twice
