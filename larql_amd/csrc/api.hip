@@ -1610,8 +1610,8 @@ static int moe_mxfp4_block(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank
                 P.threads = gemv_pick_threads(&tj, 1);
                 if (P.threads == 0 || !gemv_job_geometry(tj, P.threads)) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: unsupported geometry");
                 const uint64_t max_jobs = which == 0 && !fused ? 2 * slots : slots;
-                // (the planner's cost per job: the tiles and at most 10 more tiles' worth of start-up)
-                if (max_jobs * ((uint64_t)tj.n_pass + 10 * (uint64_t)tj.cpr) > 0x7FFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: launch too large");
+                // (the planner's cost per job: at most 1060 units a tile and under 11 more tiles' worth of start-up)
+                if (max_jobs * (((uint64_t)tj.rows + 15) / 16 + 11) * 1060 > 0x7FFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: launch too large");
                 memset(&P.L, 0, sizeof P.L);
                 P.L.table = which == 0 ? gu_table : dn_table;
                 P.L.dyn = hdr + 2 * which;
@@ -1623,8 +1623,8 @@ static int moe_mxfp4_block(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank
             if (!gemv_job_geometry(tu, Pg.threads)) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: unsupported geometry");
             HIPCHECK(c, moe_plan_launch(c->stream, router_pending ? route_logits : nullptr, bank->router_bias, route_policy, weights, experts,
                                         (uint32_t)slots, (uint32_t)k, (uint32_t)bank->n_experts, tg, tu, td, gu_w_stride,
-                                        gu_s_stride, dn_w_stride, dn_s_stride, (uint32_t)hidden, (uint32_t)inter, fused, group, gu_table, hdr,
-                                        dn_table, hdr + 2));
+                                        gu_s_stride, dn_w_stride, dn_s_stride, (uint32_t)hidden, (uint32_t)inter, fused, group, Pg.grid, Pd.grid, gu_table,
+                                        hdr, dn_table, hdr + 2));
             HIPCHECK(c, gemv_launch(c->stream, Pg.kind, Pg.L, Pg.threads, Pg.grid, Pg.lds));
             HIPCHECK(c, gemv_launch(c->stream, Pd.kind, Pd.L, Pd.threads, Pd.grid, Pd.lds));
             HIPCHECK(c, weighted_sum_launch(c->stream, d, weights, experts, (uint32_t)bank->n_experts, out, (uint32_t)tokens, (uint32_t)k,

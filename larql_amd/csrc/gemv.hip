@@ -2131,121 +2131,144 @@ __device__ __forceinline__ void run_bf16_mfma(const GemvJob &j, uint32_t tile_a,
 
 // ---------------------------------------------------------------------------
 // Q4_K rows against 2..8 activations at once (gate-KNN over several residual positions, rows of up to 10
-// super-blocks): same streaming and the same int8 MFMA as the single-activation kernel, with the A rows
-// re-dealt: the MFMA of group g and position pair p carries row 8t + 4cl + l = limb l of sub-block 2g+cl of
-// position 2p + t, so one MFMA per group serves two positions and lane (j, rq) ends with the four limb sums
-// of position 2p + rq/2, nibble class cl = rq%2, for its weight row j and every group.  It therefore decodes
-// the scales and mins of its class for all four groups.
+// super-blocks): the streaming of the single-activation kernel (a wavefront owns a 256-element column, 16 rows per
+// wave-tile, global -> LDS ring), the products on the f16 matrix cores.  A weight is converted once for all
+// positions: its nibble is masked in place into the mantissa of an f16 (1024 + q, or 1024 + 16 q for the high
+// nibbles) and one packed FMA takes the 1024 away and applies the sub-block's 6-bit scale, so the operand is the
+// integer sc6 * q <= 945, exact in f16.  One v_mfma_f32_16x16x32_f16 per sub-block (32 weights of 16 rows): its other
+// operand has the activations as rows (position, part), part = the f16 nearest the scaled activation or the f16
+// of what that leaves (together 22 bits of the activation; the scale is a power of two per position and column that
+// puts the column's largest value below 2^15).  A ninth MFMA multiplies the 6-bit mins by the sub-blocks' activation
+// sums, prepared the same way.  The eight products of a (row, position) share one accumulator; the row's f32 d and
+// dmin and the column's power of two are applied to the two sums once per tile: d * sum sc6 q x - dmin * sum mn6 Sx,
+// the value of q4k_matvec (larql-compute/src/cpu/ops/q4_common/matvec.rs) with the terms in another order.
+// Lane (j, kq) supplies row j of the 16 weight rows (k-slots 8 kq .. 8 kq + 7 of every sub-block) and ends with the
+// sums of positions 2 kq and 2 kq + 1 of that row.
 // ---------------------------------------------------------------------------
 constexpr int kQ4kBatchPairs = 4;  // positions per job: 2 * kQ4kBatchPairs
 constexpr int kQ4kBatchR = 2;      // 16-row tiles between two folds of the row partials (16 * wavefronts partials per row)
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 
 struct Q4kBatchCol {
-    Q4kOp xm[4][kQ4kBatchPairs];      // A operand of (group, pair)
-    float k[kQ4kBatchPairs];          // 2^(e-27) of this lane's position in the pair
-    float sum[4][kQ4kBatchPairs];     // sum of x over sub-block 2g + cl of this lane's position
+    u32x4 xa[8];   // activations' operand of sub-block m: row a = (position 2 (a / 4) + (a / 2) % 2, part a % 2)
+    uint32_t xs;   // the sums' operand: sub-blocks 2 kq and 2 kq + 1 of this lane's row, scaled by 2^-6 more
+    float k[2];    // 2^(e - 15) of positions 2 kq and 2 kq + 1 (the lane's results)
 };
+
+// the slots of a lane's eight k in the operand registers: (0, 2), (1, 3), (4, 6), (5, 7) — the order in which the
+// weights' nibbles leave their dwords (bytes 0 and 2 by a mask, bytes 1 and 3 after one shift)
+__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
+    const half2_t h = {(_Float16)lo, (_Float16)hi};
+    return __builtin_bit_cast(uint32_t, h);
+}
 
 __device__ __forceinline__ void q4k_batch_setup(Q4kBatchCol &col, const float *x, uint64_t x_stride, uint32_t batch, uint32_t c,
                                                 uint32_t lane) {
-    const uint32_t i = lane & 15u, kq = lane >> 4;
-    const uint32_t t_a = i >> 3, cl_a = (i >> 2) & 1u, limb = i & 3u;  // this lane as A supplier: row 8t + 4cl + limb
-    const uint32_t t_p = kq >> 1, cl_p = kq & 1u;                      // this lane in the post role (rq = kq)
+    const uint32_t a = lane & 15u, kq = lane >> 4;
+    const uint32_t pos_a = 2 * (a >> 2) + ((a >> 1) & 1u), part = a & 1u;
+    float to_s = 0.f, sx0 = 0.f, sx1 = 0.f;
+    col.k[0] = col.k[1] = 0.f;
 #pragma unroll
-    for (int p = 0; p < kQ4kBatchPairs; p++) {
-        // column maxima and sub-block sums of both positions of the pair
-        float kk[2], sm[2];
-        int ex2[2];
+    for (uint32_t pos = 0; pos < 2 * kQ4kBatchPairs; pos++) {
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        if (pos < batch) v = ((g_f4p)(x + (size_t)pos * x_stride + (size_t)c * 256))[lane];
+        float mx = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        float s4 = (v.x + v.y) + (v.z + v.w);  // lanes 8s .. 8s+7 hold sub-block s
 #pragma unroll
-        for (int t = 0; t < 2; t++) {
-            const uint32_t pos = 2 * p + t;
-            f32x4 v = {0.f, 0.f, 0.f, 0.f};
-            if (pos < batch) v = ((g_f4p)(x + (size_t)pos * x_stride + (size_t)c * 256))[lane];
-            float mx = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-            float s4 = (v.x + v.y) + (v.z + v.w);
+        for (int o = 1; o < 8; o <<= 1) { s4 += __shfl_xor(s4, o); mx = fmaxf(mx, __shfl_xor(mx, o)); }
 #pragma unroll
-            for (int o = 1; o < 8; o <<= 1) { s4 += __shfl_xor(s4, o); mx = fmaxf(mx, __shfl_xor(mx, o)); }
+        for (int o = 8; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+        int ex = 0;
+        if (mx > 0.f && mx < __builtin_inff()) (void)frexpf(mx, &ex);
+        ex = max(-90, min(100, ex));
+        const float s_a = __shfl(s4, 16 * kq), s_b = __shfl(s4, 16 * kq + 8);
+        if (pos == pos_a) { to_s = ldexpf(1.f, 15 - ex); sx0 = s_a; sx1 = s_b; }
+        if (pos == 2 * kq) col.k[0] = ldexpf(1.f, ex - 15);
+        if (pos == 2 * kq + 1) col.k[1] = ldexpf(1.f, ex - 15);
+    }
+    const bool live = pos_a < batch;
+    {
+        const float t0 = sx0 * to_s * 0.015625f, t1 = sx1 * to_s * 0.015625f;
+        const float h0 = (float)(_Float16)t0, h1 = (float)(_Float16)t1;
+        col.xs = !live ? 0u : part ? pack_f16(t0 - h0, t1 - h1) : pack_f16(h0, h1);
+    }
 #pragma unroll
-            for (int o = 8; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
-            int ex = 0;
-            if (mx > 0.f && mx < __builtin_inff()) (void)frexpf(mx, &ex);
-            ex = max(-90, min(120, ex));
-            ex2[t] = ex; kk[t] = ldexpf(1.f, ex - 27); sm[t] = s4;
+    for (int m = 0; m < 8; m++) {
+        f32x4 u = {0.f, 0.f, 0.f, 0.f}, w = {0.f, 0.f, 0.f, 0.f};
+        if (live) {
+            g_f4p xs = (g_f4p)(x + (size_t)pos_a * x_stride + (size_t)c * 256 + m * 32 + 8 * kq);
+            u = xs[0]; w = xs[1];
         }
-        col.k[p] = t_p ? kk[1] : kk[0];
+        float e[8] = {u.x, u.y, u.z, u.w, w.x, w.y, w.z, w.w};
 #pragma unroll
-        for (int g = 0; g < 4; g++) {
-            const float s0 = __shfl(sm[0], 8 * (2 * g + cl_p)), s1 = __shfl(sm[1], 8 * (2 * g + cl_p));
-            col.sum[g][p] = t_p ? s1 : s0;
+        for (int q = 0; q < 8; q++) {
+            const float t = e[q] * to_s;
+            const float h = (float)(_Float16)t;
+            e[q] = part ? t - h : h;
         }
-        // limbs of this lane's A rows
-        const uint32_t pos = 2 * p + t_a;
-        const float to_int = ldexpf(1.f, 27 - (t_a ? ex2[1] : ex2[0]));
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-            f32x4 a = {0.f, 0.f, 0.f, 0.f}, b = {0.f, 0.f, 0.f, 0.f};
-            if (pos < batch) {
-                g_f4p xs = (g_f4p)(x + (size_t)pos * x_stride + (size_t)c * 256 + g * 64 + cl_a * 32 + 8 * kq);
-                a = xs[0]; b = xs[1];
-            }
-            const float e[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-            uint32_t d[8];
-#pragma unroll
-            for (int q = 0; q < 8; q++) {
-                // balanced base-128 digits: n + 64*(1 + 128 + 128^2 + 128^3) has the unsigned digits l+64
-                const int n = (int)__builtin_rintf(e[q] * to_int) + 0x8102040;
-                const int dg = limb == 0 ? (n >> 21) : ((n >> (7 * (3 - (int)limb))) & 127);
-                d[q] = (uint32_t)(dg - 64) & 0xFFu;
-            }
-            const uint32_t d0 = d[0] | (d[1] << 8) | (d[2] << 16) | (d[3] << 24), d1 = d[4] | (d[5] << 8) | (d[6] << 16) | (d[7] << 24);
-            col.xm[g][p].u[0] = cl_a ? 0u : d0; col.xm[g][p].u[1] = cl_a ? 0u : d1;
-            col.xm[g][p].u[2] = cl_a ? d0 : 0u; col.xm[g][p].u[3] = cl_a ? d1 : 0u;
-        }
+        col.xa[m] = (u32x4){pack_f16(e[0], e[2]), pack_f16(e[1], e[3]), pack_f16(e[4], e[6]), pack_f16(e[5], e[7])};
     }
 }
 
-// the products of one wave-tile for the first NPA position pairs: value of (row, position) = k * sum_g sc_g * dot_g -
-// sum_g mn_g * sum_g(x); the limb sums meet pairwise as integers (exact, below 2^24) before they become floats
-template <int NPA>
-__device__ __forceinline__ void q4k_batch_tile(const uint8_t *sp, uint32_t kq, const Q4kBatchCol &col, const float (&sc)[4], const float (&mn)[4],
-                                               float (&racc)[kQ4kBatchPairs]) {
-    float rdot[NPA], rmin[NPA];
+// the products of one wave-tile: D rows = (position, part) as dealt in q4k_batch_setup, columns = the 16 weight rows
+__device__ __forceinline__ void q4k_batch_tile(const uint8_t *sp, uint32_t kq, const Q4kBatchCol &col, uint32_t magic, float (&racc)[2]) {
+    const u32x4 hdr = *reinterpret_cast<const u32x4 *>(sp);
+    u32x2 q[4];
 #pragma unroll
-    for (int p = 0; p < NPA; p++) {
-        rdot[p] = 0.f;
-        rmin[p] = mn[0] * col.sum[0][p];
+    for (int g = 0; g < 4; g++) q[g] = *reinterpret_cast<const u32x2 *>(sp + 16 + 32 * g + 8 * kq);
+    const float d = half_bits_to_float(hdr.x & 0xFFFFu), dmin64 = half_bits_to_float(hdr.x >> 16) * 64.f;
+    // the 6-bit scales and mins of the eight sub-blocks, a byte each (get_scale_min_k4)
+    const uint32_t sc_lo = hdr.y & 0x3F3F3F3Fu, mn_lo = hdr.z & 0x3F3F3F3Fu;
+    const uint32_t sc_hi = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
+    const uint32_t mn_hi = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
+    const half2_t m1024 = {(_Float16)-1024.f, (_Float16)-1024.f};
+    const half2_t k_lo = {(_Float16)1.f, (_Float16)-1024.f}, k_hi = {(_Float16)0.0625f, (_Float16)-64.f};
+    f32x4 D = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int g = 1; g < 4; g++) rmin[p] = __builtin_fmaf(mn[g], col.sum[g][p], rmin[p]);
-    }
+    for (int m = 0; m < 8; m++) {
+        const int g = m >> 1, h = m & 1;
+        // (1024 + sc6) twice as f16 by a byte shuffle (0x64 is the high byte of f16 1024 + n), then (s, -1024 s) / (s / 16, -64 s)
+        const uint32_t sel = 0x04000400u | (uint32_t)(m & 3) | ((uint32_t)(m & 3) << 16);
+        const uint32_t both = __builtin_amdgcn_perm(0x64646464u, m < 4 ? sc_lo : sc_hi, sel);
+        const half2_t s2 = __builtin_bit_cast(half2_t, both) + m1024;
+        const half2_t p = s2 * (h ? k_hi : k_lo);
+        const half2_t sc2 = {p[0], p[0]}, off2 = {p[1], p[1]};  // (broadcast by the instruction's operand selects)
+        const uint32_t mask = h ? 0x00F000F0u : 0x000F000Fu;
+        u32x4 bw;
 #pragma unroll
-    for (int g = 0; g < 4; g++) {
-        const u32x2 q = *reinterpret_cast<const u32x2 *>(sp + 16 + 32 * g + 8 * kq);
-        Q4kOp b;
-        b.u[0] = q.x & 0x0F0F0F0Fu; b.u[1] = q.y & 0x0F0F0F0Fu;
-        b.u[2] = (q.x >> 4) & 0x0F0F0F0Fu; b.u[3] = (q.y >> 4) & 0x0F0F0F0Fu;
-#pragma unroll
-        for (int p = 0; p < NPA; p++) {
-            const i32x4 z = {0, 0, 0, 0};
-            const i32x4 D = __builtin_amdgcn_mfma_i32_16x16x64_i8(col.xm[g][p].v, b.v, z, 0, 0, 0);
-            const float hi = (float)(D[0] * 128 + D[1]), lo = (float)(D[2] * 128 + D[3]);
-            rdot[p] = __builtin_fmaf(sc[g], __builtin_fmaf(hi, 16384.f, lo), rdot[p]);
+        for (int w = 0; w < 2; w++) {
+            const uint32_t raw = w ? q[g].y : q[g].x;
+            const half2_t m02 = __builtin_bit_cast(half2_t, (raw & mask) | magic);
+            const half2_t m13 = __builtin_bit_cast(half2_t, ((raw >> 8) & mask) | magic);
+            bw[2 * w] = __builtin_bit_cast(uint32_t, m02 * sc2 + off2);
+            bw[2 * w + 1] = __builtin_bit_cast(uint32_t, m13 * sc2 + off2);
         }
+        D = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, col.xa[m]), __builtin_bit_cast(f16x8_t, bw), D, 0, 0, 0);
     }
-#pragma unroll
-    for (int p = 0; p < kQ4kBatchPairs; p++) racc[p] = p < NPA ? __builtin_fmaf(rdot[p < NPA ? p : 0], col.k[p], -rmin[p < NPA ? p : 0]) : 0.f;
+    // the mins of sub-blocks 2 kq and 2 kq + 1 against their activation sums
+    const uint32_t msel = (kq & 1u) ? 0x04030402u : 0x04010400u;
+    const uint32_t mboth = __builtin_amdgcn_perm(0x64646464u, kq < 2 ? mn_lo : mn_hi, msel);
+    const half2_t mn2 = __builtin_bit_cast(half2_t, mboth) + m1024;
+    const u32x4 bm = {__builtin_bit_cast(uint32_t, mn2), 0u, 0u, 0u}, am = {col.xs, 0u, 0u, 0u};
+    const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+    const f32x4 Dm = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, am), __builtin_bit_cast(f16x8_t, bm), z, 0, 0, 0);
+    racc[0] = col.k[0] * __builtin_fmaf(d, D[0] + D[1], -dmin64 * (Dm[0] + Dm[1]));
+    racc[1] = col.k[1] * __builtin_fmaf(d, D[2] + D[3], -dmin64 * (Dm[2] + Dm[3]));
 }
 
 __device__ __forceinline__ void run_q4k_batch(const GemvJob &j, uint32_t tile_a, uint32_t tile_b, uint8_t *lds, uint32_t &parity) {
     constexpr int NS = kQ4kStages, R = kQ4kBatchR, NP = kQ4kBatchPairs;
     const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t nw_launch = blockDim.x >> 6;
-    const uint32_t jr = lane & 15u, kq = lane >> 4, t_p = kq >> 1, cl = kq & 1u;
+    const uint32_t jr = lane & 15u, kq = lane >> 4;
     const uint32_t nwj = j.rpp, batch = j.batch;
     const uint32_t rows = (uint32_t)j.rows, row_bytes = (uint32_t)j.row_bytes;
     uint8_t *ring = lds + wv * (NS * kQ4kTileBytes);
     float *part = reinterpret_cast<float *>(lds + nw_launch * (NS * kQ4kTileBytes));
     const bool working = wv < nwj;
-    const uint32_t PW = 2 * NP * nw_launch * 2;  // partials per row: [position][wavefront][class]
+    const uint32_t PW = 2 * NP * nw_launch;  // partials per row: [position][wavefront]
+    uint32_t magic;
+    asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));  // (in a register, so that mask-and-or is one instruction)
 
     const uint32_t u0 = lane, u1 = 64 + lane, u2 = 128 + (lane >> 2);
     const uint32_t r0 = u0 / 9, r1 = u1 / 9, r2 = u2 / 9;
@@ -2289,29 +2312,12 @@ __device__ __forceinline__ void run_q4k_batch(const GemvJob &j, uint32_t tile_a,
                 asm volatile("" ::: "memory");
                 const uint8_t *sp = ring + (n_use % NS) * kQ4kTileBytes + jr * 144;
                 n_use++;
-                const u32x4 hdr = *reinterpret_cast<const u32x4 *>(sp);
-                // scales and mins of class cl for the four groups: sub-blocks cl, 2+cl, 4+cl, 6+cl (get_scale_min_k4)
-                const float d = half_bits_to_float(hdr.x & 0xFFFFu), dmin = half_bits_to_float(hdr.x >> 16);
-                const uint32_t sh01 = cl * 8u;
-                const uint32_t sc_a = hdr.y >> sh01, mn_a = hdr.z >> sh01, hi_a = hdr.w >> sh01;  // bytes cl, (cl+1), (cl+2), ...
-                float sc[4], mn[4];
-                sc[0] = d * (float)(sc_a & 63u);          mn[0] = dmin * (float)(mn_a & 63u);            // sub cl
-                sc[1] = d * (float)((sc_a >> 16) & 63u);  mn[1] = dmin * (float)((mn_a >> 16) & 63u);    // sub 2+cl
-                sc[2] = d * (float)((hi_a & 0x0Fu) | ((sc_a >> 2) & 0x30u));                             // sub 4+cl
-                mn[2] = dmin * (float)(((hi_a >> 4) & 0x0Fu) | ((mn_a >> 2) & 0x30u));
-                sc[3] = d * (float)(((hi_a >> 16) & 0x0Fu) | ((sc_a >> 18) & 0x30u));                    // sub 6+cl
-                mn[3] = dmin * (float)(((hi_a >> 20) & 0x0Fu) | ((mn_a >> 18) & 0x30u));
-                float racc[NP];
-                switch ((batch + 1) / 2) {  // (no branch inside the MFMA sequence: the products of a tile are independent)
-                    case 1: q4k_batch_tile<1>(sp, kq, col, sc, mn, racc); break;
-                    case 2: q4k_batch_tile<2>(sp, kq, col, sc, mn, racc); break;
-                    case 3: q4k_batch_tile<3>(sp, kq, col, sc, mn, racc); break;
-                    default: q4k_batch_tile<4>(sp, kq, col, sc, mn, racc); break;
-                }
+                float racc[2];
+                q4k_batch_tile(sp, kq, col, magic, racc);
 #pragma unroll
-                for (int p = 0; p < NP; p++) {
-                    const uint32_t pos = 2 * p + t_p;
-                    if (pos < batch) pb[(tl * 16 + jr) * PW + (pos * nw_launch + wv) * 2 + cl] = racc[p];
+                for (int t = 0; t < 2; t++) {
+                    const uint32_t pos = 2 * kq + t;
+                    if (pos < batch) pb[(tl * 16 + jr) * PW + pos * nw_launch + wv] = racc[t];
                 }
             }
         }
@@ -2322,7 +2328,7 @@ __device__ __forceinline__ void run_q4k_batch(const GemvJob &j, uint32_t tile_a,
         for (uint32_t e = threadIdx.x; e < nbt * 16 * batch; e += blockDim.x) {
             const uint32_t rr = e / batch, pos = e - rr * batch;
             float s = 0.f;
-            for (uint32_t w = 0; w < nwj; w++) s += pb[rr * PW + (pos * nw_launch + w) * 2] + pb[rr * PW + (pos * nw_launch + w) * 2 + 1];
+            for (uint32_t w = 0; w < nwj; w++) s += pb[rr * PW + pos * nw_launch + w];
             if (row_base + rr < rows) ((g_f32wp)j.out)[(size_t)pos * j.out_stride + row_base + rr] = s;
         }
         parity ^= 1u;
@@ -3355,7 +3361,7 @@ size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
     }
     if (n > 0 && jobs[0].kind == KIND_Q4K_BATCH) {
         const size_t nw = threads / 64;
-        return nw * kQ4kStages * kQ4kTileBytes + 2 * (size_t)kQ4kBatchR * 16 * (2 * kQ4kBatchPairs * nw * 2) * sizeof(float);
+        return nw * kQ4kStages * kQ4kTileBytes + 2 * (size_t)kQ4kBatchR * 16 * (2 * kQ4kBatchPairs * nw) * sizeof(float);
     }
     if (n > 0 && jobs[0].kind == KIND_BF16_MFMA) {
         const size_t nw = threads / 64;

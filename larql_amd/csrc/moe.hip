@@ -88,10 +88,10 @@ __global__ void __launch_bounds__(1024) moe_plan_kernel(const float *__restrict_
                                                        float *__restrict__ weights, uint32_t *__restrict__ experts, uint32_t slots, uint32_t k, uint32_t n_experts,
                                                        GemvJob tg, GemvJob tu, GemvJob td, uint64_t gu_w_stride, uint64_t gu_s_stride,
                                                        uint64_t dn_w_stride, uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, uint32_t fused,
-                                                       uint32_t group, GemvJob *__restrict__ gu_table, uint32_t *__restrict__ gu_hdr,
-                                                       GemvJob *__restrict__ dn_table, uint32_t *__restrict__ dn_hdr) {
+                                                       uint32_t group, uint32_t g_grid, uint32_t d_grid, GemvJob *__restrict__ gu_table,
+                                                       uint32_t *__restrict__ gu_hdr, GemvJob *__restrict__ dn_table, uint32_t *__restrict__ dn_hdr) {
     __shared__ uint32_t first_job[1025];  // first job of expert e; [n_experts] = total
-    __shared__ uint32_t first_gcost[1025], first_dcost[1025];  // the same for the jobs' places in the two pass lists
+    __shared__ uint32_t first_kind_a[1025], first_kind_b[1025];  // the jobs before expert e by kind: {full groups, of 1 slot}, {of 2, of 3}
     __shared__ __attribute__((aligned(16))) uint32_t cnt[1024];  // slots per expert
     __shared__ __attribute__((aligned(16))) uint32_t ex[4096];   // the router's choice, read once
     __shared__ uint32_t first_slot[1025]; // slots of the experts before e
@@ -134,21 +134,15 @@ __global__ void __launch_bounds__(1024) moe_plan_kernel(const float *__restrict_
         if (e < n_experts) atomicAdd(&cnt[e], 1u);
     }
     __syncthreads();
-    // Cost of a job in the launches' pass lists, from cycle counts of the kernel: a tile costs the same however many
-    // tokens share it (its bytes set the pace), and a job segment starts with the preparation of its
-    // activations, worth 4 tiles for one token and 2 more for every further one.  Units: steps (a tile = cpr of them).
-    const uint32_t g_tiles = ((uint32_t)tg.rows + 15) / 16, d_tiles = ((uint32_t)td.rows + 15) / 16;
-    const uint32_t g_c = tg.cpr, d_c = td.cpr;
-    auto g_cost = [&](uint32_t n) { return n ? (2 + 2 * n + g_tiles) * g_c : 0u; };
-    auto d_cost = [&](uint32_t n) { return n ? (2 + 2 * n + d_tiles) * d_c : 0u; };
-    const uint32_t g_full = g_cost(group), d_full = d_cost(group);
+    // Per expert: the jobs before it, counted by kind (full groups, and groups of 1, 2 or 3 slots), 16 bits a count.
     for (uint32_t e = t; e <= n_experts; e += blockDim.x) {
-        uint32_t f = 0, gc = 0, dc = 0, fs = 0;
+        uint32_t f = 0, ka = 0, kb = 0, fs = 0;
         auto add = [&](uint32_t c) {
             fs += c;
             f += (c + gmask) >> gsh;
-            gc += (c >> gsh) * g_full + g_cost(c & gmask);
-            dc += (c >> gsh) * d_full + d_cost(c & gmask);
+            const uint32_t m = c & gmask;
+            ka += (c >> gsh) + (m == 1 ? 0x10000u : 0u);
+            kb += (m == 2 ? 1u : 0u) + (m == 3 ? 0x10000u : 0u);
         };
 #pragma unroll 2
         for (uint32_t q = 0; q < e; q += 4) {
@@ -158,10 +152,36 @@ __global__ void __launch_bounds__(1024) moe_plan_kernel(const float *__restrict_
             if (q + 2 < e) add(v.z);
             if (q + 3 < e) add(v.w);
         }
-        first_job[e] = f; first_gcost[e] = gc; first_dcost[e] = dc; first_slot[e] = fs;
+        first_job[e] = f; first_kind_a[e] = ka; first_kind_b[e] = kb; first_slot[e] = fs;
     }
     __syncthreads();
-    const uint32_t n_jobs = first_job[n_experts], g_total = first_gcost[n_experts], d_total = first_dcost[n_experts];
+    const uint32_t n_jobs = first_job[n_experts];
+    // Cost of a job in a launch's pass list.  A workgroup prepares the activations of every job it takes a share of
+    // before the share's first tile: about 3 tiles' time for one token and 2 more for every further one (time
+    // stamps of the kernel), whether the share opens the job or not.  A job cut into n shares pays that n times, and
+    // n = 1 + tiles / (tiles per workgroup) on average: so a job costs one preparation up front (GemvJob::su) and each
+    // of its tiles carries the preparation's part, cpt = 4 * tpw + prep in quarter tiles where a tile's own time is
+    // 4 * tpw units (tpw = the launch's tiles per workgroup).  The workgroup that opens a job mid-share also lets its
+    // stream of weights run dry in between: 2 tiles more up front.  Launches whose workgroups walk more than 256
+    // tiles each leave the parts out (under 4 % of a share).
+    struct JobCost {  // of a job with m tokens, in one launch
+        uint32_t tiles, unit;  // unit = tpw, or 0 where the parts are left out
+        __device__ uint32_t prep(uint32_t m) const { return 12 + 8 * (m - 1); }
+        __device__ uint32_t cpt(uint32_t m) const { return unit ? 4 * unit + prep(m) : 4u; }
+        __device__ uint32_t su(uint32_t m) const { return (prep(m) + 8) * (unit ? unit : 1u); }
+        __device__ uint32_t job(uint32_t m) const { return su(m) + tiles * cpt(m); }
+    };
+    const auto cost_model = [&](uint32_t tiles, uint32_t grid, uint32_t lists) {
+        const uint64_t tpw = max((uint64_t)1, (uint64_t)lists * n_jobs * tiles / max(grid, 1u));
+        return JobCost{tiles, tpw <= 256 ? (uint32_t)tpw : 0u};
+    };
+    const uint32_t g_tiles = ((uint32_t)tg.rows + 15) / 16, d_tiles = ((uint32_t)td.rows + 15) / 16;
+    const JobCost gc = cost_model(g_tiles, g_grid, fused ? 1u : 2u), dc = cost_model(d_tiles, d_grid, 1u);
+    const auto jobs_cost = [&](const JobCost &c, uint32_t e) {  // the jobs of the experts before e
+        const uint32_t ka = first_kind_a[e], kb = first_kind_b[e];
+        return (ka & 0xFFFFu) * c.job(group) + (ka >> 16) * c.job(1) + (kb & 0xFFFFu) * c.job(2) + (kb >> 16) * c.job(3);
+    };
+    const uint32_t g_total = jobs_cost(gc, n_experts), d_total = jobs_cost(dc, n_experts);
     for (uint32_t s = t; s < slots; s += blockDim.x) {
         const uint32_t e = ex[s];
         if (e < n_experts) by_expert[first_slot[e] + rank[s]] = (uint16_t)s;
@@ -183,7 +203,7 @@ __global__ void __launch_bounds__(1024) moe_plan_kernel(const float *__restrict_
         // a job = the template's words with the fields that differ replaced, kept in registers as plain dwords
         // and stored 16 bytes at a time
         const auto emit = [&](GemvJob *dst, const GemvJob &tm, size_t w_off, size_t aux_off, size_t x_off, size_t out_off, bool x_by_token,
-                              size_t out_unit, uint32_t pass_begin, uint32_t tiles_cost, uint32_t c1) {
+                              size_t out_unit, uint32_t pass_begin, const JobCost &c) {
             static_assert(sizeof(GemvJob) % 16 == 0 && alignof(GemvJob) == 8, "descriptor is a whole number of 16-byte stores");
             constexpr int N = sizeof(GemvJob) / 4;
             const uint32_t *src = reinterpret_cast<const uint32_t *>(&tm);
@@ -206,22 +226,20 @@ __global__ void __launch_bounds__(1024) moe_plan_kernel(const float *__restrict_
             put64(offsetof(GemvJob, out_off), (uint64_t)slot_off(2, out_unit));
             put64(offsetof(GemvJob, out_off) + 8, (uint64_t)slot_off(3, out_unit));
             put32(offsetof(GemvJob, pass_begin), pass_begin);
-            put32(offsetof(GemvJob, n_pass), (2 + 2 * nb) * c1 + tiles_cost);
-            put32(offsetof(GemvJob, cpt), c1);
-            put32(offsetof(GemvJob, su), (2 + 2 * nb) * c1);
+            put32(offsetof(GemvJob, n_pass), c.job(nb));
+            put32(offsetof(GemvJob, cpt), c.cpt(nb));
+            put32(offsetof(GemvJob, su), c.su(nb));
             uint4 *o = reinterpret_cast<uint4 *>(dst);  // (the tables are 16-byte aligned)
 #pragma unroll
             for (int i = 0; i < N / 4; i++) o[i] = make_uint4(d[4 * i], d[4 * i + 1], d[4 * i + 2], d[4 * i + 3]);
         };
         // (the earlier jobs of this expert are all full groups)
-        const uint32_t g_begin = first_gcost[e] + (r >> gsh) * g_full, d_begin = first_dcost[e] + (r >> gsh) * d_full;
-        emit(gu_table + jb, tg, (size_t)e * gu_w_stride, (size_t)e * gu_s_stride, (size_t)tok1 * hidden, (size_t)s1 * gs, true, gs, g_begin,
-             g_tiles * g_c, g_c);
+        const uint32_t g_begin = jobs_cost(gc, e) + (r >> gsh) * gc.job(group), d_begin = jobs_cost(dc, e) + (r >> gsh) * dc.job(group);
+        emit(gu_table + jb, tg, (size_t)e * gu_w_stride, (size_t)e * gu_s_stride, (size_t)tok1 * hidden, (size_t)s1 * gs, true, gs, g_begin, gc);
         if (!fused)
             emit(gu_table + n_jobs + jb, tu, (size_t)e * gu_w_stride, (size_t)e * gu_s_stride, (size_t)tok1 * hidden, (size_t)s1 * gs, true, gs,
-                 g_total + g_begin, g_tiles * g_c, g_c);
-        emit(dn_table + jb, td, (size_t)e * dn_w_stride, (size_t)e * dn_s_stride, (size_t)s1 * gs, (size_t)s1 * hidden, false, hidden, d_begin,
-             d_tiles * d_c, d_c);
+                 g_total + g_begin, gc);
+        emit(dn_table + jb, td, (size_t)e * dn_w_stride, (size_t)e * dn_s_stride, (size_t)s1 * gs, (size_t)s1 * hidden, false, hidden, d_begin, dc);
     }
     if (t == 0) {
         gu_hdr[0] = fused ? n_jobs : 2 * n_jobs; gu_hdr[1] = fused ? g_total : 2 * g_total;
@@ -232,13 +250,13 @@ __global__ void __launch_bounds__(1024) moe_plan_kernel(const float *__restrict_
 hipError_t moe_plan_launch(hipStream_t s, const float *logits, const float *router_bias, int policy, float *weights, uint32_t *experts,
                            uint32_t slots, uint32_t k, uint32_t n_experts, const GemvJob &tg,
                            const GemvJob &tu, const GemvJob &td, uint64_t gu_w_stride, uint64_t gu_s_stride, uint64_t dn_w_stride,
-                           uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, bool fused, uint32_t group, GemvJob *gu_table, uint32_t *gu_hdr,
-                           GemvJob *dn_table, uint32_t *dn_hdr) {
+                           uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, bool fused, uint32_t group, uint32_t g_grid, uint32_t d_grid, GemvJob *gu_table,
+                           uint32_t *gu_hdr, GemvJob *dn_table, uint32_t *dn_hdr) {
     if (n_experts > 1024 || slots > 4096 || (group != 2 && group != 4)) return hipErrorInvalidValue;
     // (a wavefront per token while selecting: 16 wavefronts when the kernel routes)
     hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(logits ? 1024 : 256), 0, s, logits, router_bias, policy, weights, experts, slots, k, n_experts, tg, tu, td,
                        gu_w_stride, gu_s_stride,
-                       dn_w_stride, dn_s_stride, hidden, inter, fused ? 1u : 0u, group, gu_table, gu_hdr, dn_table, dn_hdr);
+                       dn_w_stride, dn_s_stride, hidden, inter, fused ? 1u : 0u, group, g_grid, d_grid, gu_table, gu_hdr, dn_table, dn_hdr);
     return hipGetLastError();
 }
 
