@@ -2147,6 +2147,7 @@ __device__ __forceinline__ void run_bf16_mfma(const GemvJob &j, uint32_t tile_a,
 // ---------------------------------------------------------------------------
 constexpr int kQ4kBatchPairs = 4;  // positions per job: 2 * kQ4kBatchPairs
 constexpr int kQ4kBatchR = 2;      // 16-row tiles between two folds of the row partials (16 * wavefronts partials per row)
+constexpr int kQ4kBatchStages = 4;  // wave-tiles in flight per wavefront
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 
 struct Q4kBatchCol {
@@ -2211,11 +2212,18 @@ __device__ __forceinline__ void q4k_batch_setup(Q4kBatchCol &col, const float *x
 }
 
 // the products of one wave-tile: D rows = (position, part) as dealt in q4k_batch_setup, columns = the 16 weight rows
-__device__ __forceinline__ void q4k_batch_tile(const uint8_t *sp, uint32_t kq, const Q4kBatchCol &col, uint32_t magic, float (&racc)[2]) {
-    const u32x4 hdr = *reinterpret_cast<const u32x4 *>(sp);
+struct Q4kBatchRaw {  // a lane's bytes of one wave-tile: its row's header and the 8 bytes kq of the four 32-byte chunks
+    u32x4 hdr;
     u32x2 q[4];
+};
+__device__ __forceinline__ void q4k_batch_read(Q4kBatchRaw &r, const uint8_t *sp, uint32_t kq) {
+    r.hdr = *reinterpret_cast<const u32x4 *>(sp);
 #pragma unroll
-    for (int g = 0; g < 4; g++) q[g] = *reinterpret_cast<const u32x2 *>(sp + 16 + 32 * g + 8 * kq);
+    for (int g = 0; g < 4; g++) r.q[g] = *reinterpret_cast<const u32x2 *>(sp + 16 + 32 * g + 8 * kq);
+}
+__device__ __forceinline__ void q4k_batch_tile(const Q4kBatchRaw &raw_in, uint32_t kq, const Q4kBatchCol &col, uint32_t magic, float (&racc)[2]) {
+    const u32x4 hdr = raw_in.hdr;
+    const u32x2 (&q)[4] = raw_in.q;
     const float d = half_bits_to_float(hdr.x & 0xFFFFu), dmin64 = half_bits_to_float(hdr.x >> 16) * 64.f;
     // the 6-bit scales and mins of the eight sub-blocks, a byte each (get_scale_min_k4)
     const uint32_t sc_lo = hdr.y & 0x3F3F3F3Fu, mn_lo = hdr.z & 0x3F3F3F3Fu;
@@ -2227,10 +2235,15 @@ __device__ __forceinline__ void q4k_batch_tile(const uint8_t *sp, uint32_t kq, c
 #pragma unroll
     for (int m = 0; m < 8; m++) {
         const int g = m >> 1, h = m & 1;
-        // (1024 + sc6) twice as f16 by a byte shuffle (0x64 is the high byte of f16 1024 + n), then (s, -1024 s) / (s / 16, -64 s)
-        const uint32_t sel = 0x04000400u | (uint32_t)(m & 3) | ((uint32_t)(m & 3) << 16);
-        const uint32_t both = __builtin_amdgcn_perm(0x64646464u, m < 4 ? sc_lo : sc_hi, sel);
-        const half2_t s2 = __builtin_bit_cast(half2_t, both) + m1024;
+        // f16(sc6) straight from its byte, then (s, -1024 s) / (s / 16, -64 s) by one packed multiply
+        uint32_t sfb;
+        const uint32_t scw = m < 4 ? sc_lo : sc_hi;
+        if ((m & 3) == 0) asm("v_cvt_f16_u16_sdwa %0, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0" : "=v"(sfb) : "v"(scw));
+        else if ((m & 3) == 1) asm("v_cvt_f16_u16_sdwa %0, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1" : "=v"(sfb) : "v"(scw));
+        else if ((m & 3) == 2) asm("v_cvt_f16_u16_sdwa %0, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2" : "=v"(sfb) : "v"(scw));
+        else asm("v_cvt_f16_u16_sdwa %0, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3" : "=v"(sfb) : "v"(scw));
+        const _Float16 sf = __builtin_bit_cast(half2_t, sfb)[0];
+        const half2_t s2 = {sf, sf};
         const half2_t p = s2 * (h ? k_hi : k_lo);
         const half2_t sc2 = {p[0], p[0]}, off2 = {p[1], p[1]};  // (broadcast by the instruction's operand selects)
         const uint32_t mask = h ? 0x00F000F0u : 0x000F000Fu;
@@ -2257,7 +2270,7 @@ __device__ __forceinline__ void q4k_batch_tile(const uint8_t *sp, uint32_t kq, c
 }
 
 __device__ __forceinline__ void run_q4k_batch(const GemvJob &j, uint32_t tile_a, uint32_t tile_b, uint8_t *lds, uint32_t &parity) {
-    constexpr int NS = kQ4kStages, R = kQ4kBatchR, NP = kQ4kBatchPairs;
+    constexpr int NS = kQ4kBatchStages, R = kQ4kBatchR, NP = kQ4kBatchPairs;
     const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t nw_launch = blockDim.x >> 6;
     const uint32_t jr = lane & 15u, kq = lane >> 4;
@@ -2266,7 +2279,7 @@ __device__ __forceinline__ void run_q4k_batch(const GemvJob &j, uint32_t tile_a,
     uint8_t *ring = lds + wv * (NS * kQ4kTileBytes);
     float *part = reinterpret_cast<float *>(lds + nw_launch * (NS * kQ4kTileBytes));
     const bool working = wv < nwj;
-    const uint32_t PW = 2 * NP * nw_launch;  // partials per row: [position][wavefront]
+    const uint32_t PW = 2 * NP * nw_launch + 1;  // partials per row: [position][wavefront], an odd stride (the fold reads down the rows)
     uint32_t magic;
     asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));  // (in a register, so that mask-and-or is one instruction)
 
@@ -2276,7 +2289,7 @@ __device__ __forceinline__ void run_q4k_batch(const GemvJob &j, uint32_t tile_a,
     const uint32_t o0 = r0 * row_bytes + w0, o1 = r1 * row_bytes + w1, o2 = r2 * row_bytes + w2;
     const uint8_t *wcol = j.w + (size_t)wv * 144;
     const uint32_t nt = tile_b - tile_a;
-    uint32_t it_tile = tile_a, n_issue = 0;
+    uint32_t it_tile = tile_a, slot_issue = 0;  // (ring slots by wrapping counters)
     auto issue = [&]() {
         // wave-uniform 64-bit base + per-lane 32-bit offset; only a ragged last tile recomputes the offsets
         const uint32_t rb = min(it_tile, tile_b - 1) * 16;
@@ -2289,11 +2302,11 @@ __device__ __forceinline__ void run_q4k_batch(const GemvJob &j, uint32_t tile_a,
             a2 = min(r2, lim) * row_bytes + w2;
         }
         const uint8_t *g0 = gp + a0, *g1 = gp + a1, *g2 = gp + a2;
-        uint8_t *lp = ring + (n_issue % NS) * kQ4kTileBytes;
+        uint8_t *lp = ring + slot_issue * kQ4kTileBytes;
         __builtin_amdgcn_global_load_lds((g_vp)g0, (lds_vp)lp, 16, 0, 0);
         __builtin_amdgcn_global_load_lds((g_vp)g1, (lds_vp)(lp + 1024), 16, 0, 0);
         __builtin_amdgcn_global_load_lds((g_vp)g2, (lds_vp)(lp + 2048), 4, 0, 0);
-        n_issue++;
+        slot_issue = slot_issue + 1 == (uint32_t)NS ? 0u : slot_issue + 1;
         if (it_tile < tile_b) it_tile++;
     };
     if (working)
@@ -2301,19 +2314,20 @@ __device__ __forceinline__ void run_q4k_batch(const GemvJob &j, uint32_t tile_a,
     Q4kBatchCol col;
     if (working) q4k_batch_setup(col, j.x, j.x_stride, batch, wv, lane);
 
-    uint32_t n_use = 0;
+    uint32_t slot_use = 0;
     for (uint32_t tb = 0; tb < nt; tb += R) {
         float *pb = part + parity * (R * 16 * PW);
         const uint32_t nbt = min((uint32_t)R, nt - tb);
         if (working) {
             for (uint32_t tl = 0; tl < nbt; tl++) {
                 issue();
-                LARQL_WAIT_VMCNT(3 * (NS - 1));
+                LARQL_WAIT_VMCNT(3 * (NS - 1));  // at most NS-1 younger wave-tiles still in flight: the oldest has landed
                 asm volatile("" ::: "memory");
-                const uint8_t *sp = ring + (n_use % NS) * kQ4kTileBytes + jr * 144;
-                n_use++;
+                Q4kBatchRaw raw;
+                q4k_batch_read(raw, ring + slot_use * kQ4kTileBytes + jr * 144, kq);
+                slot_use = slot_use + 1 == (uint32_t)NS ? 0u : slot_use + 1;
                 float racc[2];
-                q4k_batch_tile(sp, kq, col, magic, racc);
+                q4k_batch_tile(raw, kq, col, magic, racc);
 #pragma unroll
                 for (int t = 0; t < 2; t++) {
                     const uint32_t pos = 2 * kq + t;
@@ -2325,8 +2339,11 @@ __device__ __forceinline__ void run_q4k_batch(const GemvJob &j, uint32_t tile_a,
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         const uint32_t row_base = (tile_a + tb) * 16;
-        for (uint32_t e = threadIdx.x; e < nbt * 16 * batch; e += blockDim.x) {
-            const uint32_t rr = e / batch, pos = e - rr * batch;
+        // a thread per (position, row): consecutive threads write consecutive rows of a position
+        static_assert(R == 1 || R == 2, "rows of a fold: 16 or 32");
+        const uint32_t rsh = nbt == 2 ? 5u : 4u;
+        for (uint32_t e = threadIdx.x; e < (batch << rsh); e += blockDim.x) {
+            const uint32_t pos = e >> rsh, rr = e & ((1u << rsh) - 1u);
             float s = 0.f;
             for (uint32_t w = 0; w < nwj; w++) s += pb[rr * PW + pos * nw_launch + w];
             if (row_base + rr < rows) ((g_f32wp)j.out)[(size_t)pos * j.out_stride + row_base + rr] = s;
@@ -3361,7 +3378,7 @@ size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads) {
     }
     if (n > 0 && jobs[0].kind == KIND_Q4K_BATCH) {
         const size_t nw = threads / 64;
-        return nw * kQ4kStages * kQ4kTileBytes + 2 * (size_t)kQ4kBatchR * 16 * (2 * kQ4kBatchPairs * nw) * sizeof(float);
+        return nw * kQ4kBatchStages * kQ4kTileBytes + 2 * (size_t)kQ4kBatchR * 16 * (2 * kQ4kBatchPairs * nw + 1) * sizeof(float);
     }
     if (n > 0 && jobs[0].kind == KIND_BF16_MFMA) {
         const size_t nw = threads / 64;
