@@ -2340,9 +2340,17 @@ __device__ __forceinline__ void run_q4k_batch(const GemvJob &j, uint32_t tile_a,
         asm volatile("" ::: "memory");
         const uint32_t row_base = (tile_a + tb) * 16;
         // a thread per (position, row): consecutive threads write consecutive rows of a position
+        // The fold belongs to the wavefronts without a column when the launch has at least two of them (it is
+        // launched with two more than its widest job has columns: ten column wavefronts lie 3, 3, 2, 2 on the four
+        // SIMDs, the kernel is bound by the instructions of the SIMDs with three, and wavefronts 10 and 11 go to the
+        // other two): they add up batch b while the column wavefronts are at batch b + 1 — the partials are double-
+        // buffered, and the next barrier comes after both.
         static_assert(R == 1 || R == 2, "rows of a fold: 16 or 32");
         const uint32_t rsh = nbt == 2 ? 5u : 4u;
-        for (uint32_t e = threadIdx.x; e < (batch << rsh); e += blockDim.x) {
+        const bool spare = nw_launch >= nwj + 2;
+        if (spare && working) { parity ^= 1u; continue; }
+        const uint32_t f0 = spare ? threadIdx.x - nwj * 64 : threadIdx.x, fstep = spare ? blockDim.x - nwj * 64 : blockDim.x;
+        for (uint32_t e = f0; e < (batch << rsh); e += fstep) {
             const uint32_t pos = e >> rsh, rr = e & ((1u << rsh) - 1u);
             float s = 0.f;
             for (uint32_t w = 0; w < nwj; w++) s += pb[rr * PW + pos * nw_launch + w];
@@ -3036,7 +3044,7 @@ __global__ void __launch_bounds__(kBfMaxWaves * 64) gemv_bf16_mfma_kernel(GemvLa
 }
 
 // Q4_K rows x several activations: same sweep as the single-activation kernel
-__global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_batch_kernel(GemvLaunch L) {
+__global__ void __launch_bounds__((kQ4kMaxWaves + 2) * 64) gemv_q4k_batch_kernel(GemvLaunch L) {
     extern __shared__ __attribute__((aligned(16))) uint8_t q4kb_lds[];
     const job_cp jobs = job_table(L);
     const uint64_t P = L.total_passes;
@@ -3293,7 +3301,7 @@ uint32_t gemv_pick_threads(const GemvJob *jobs, size_t n) {
     if (n > 0 && jobs[0].kind == KIND_Q4K_BATCH) {
         uint64_t nw = 0;
         for (size_t i = 0; i < n; i++) nw = std::max<uint64_t>(nw, jobs[i].k / 256);
-        return nw <= (uint64_t)kQ4kMaxWaves ? (uint32_t)nw * 64 : 0;
+        return nw <= (uint64_t)kQ4kMaxWaves ? (uint32_t)(nw + 2) * 64 : 0;  // (two wavefronts more: they fold the partial sums)
     }
     if (n > 0 && jobs[0].kind == KIND_BF16_MFMA) {
         uint64_t nw = 0;
