@@ -97,8 +97,10 @@ constexpr int kTopkCandidates = kTopkThreads;  // candidates of the short way: o
 
 // LARGE (K above 64, up to kTopkMaxK): the selection is the same radix select; the winners are gathered into a
 // power-of-two array in dynamic LDS (`cap` keys, zero-padded) and ordered by a bitonic sort of the whole workgroup.
+// (80 scalar registers: with the 96 the compiler would take, a second 16-wavefront workgroup was not placed on a CU
+// until half of the first one's wavefronts had left — more rows than CUs then ran in two rounds)
 template <bool BY_ABS, bool CACHED, bool LARGE>
-__global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restrict__ scores, uint32_t n, uint32_t k,
+__global__ void __launch_bounds__(kTopkThreads) __attribute__((amdgpu_num_sgpr(80))) topk_kernel(const float *__restrict__ scores, uint32_t n, uint32_t k,
                                                             uint32_t *__restrict__ idx_out, float *__restrict__ val_out,
                                                             uint32_t *__restrict__ count_out, int *nan_flag, uint32_t cap) {
     static_assert(!(LARGE && CACHED), "the candidate short cut bounds 64 winners only");
@@ -109,6 +111,7 @@ __global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restr
     __shared__ uint32_t sh_prefix, sh_need, sh_nwin, sh_ncand;
     __shared__ uint32_t group_max[64];
     __shared__ __attribute__((aligned(16))) uint64_t cand[CACHED ? kTopkCandidates + 4 : 1];
+    __shared__ uint32_t rank_sh[CACHED ? kTopkCandidates : 1];  // ranks counted in shares (short way)
     const uint32_t row = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const float *s = scores + (size_t)row * n;
     // wavefront w owns the contiguous indices [w0, w1), 64 at a time (lane = index within the 64)
@@ -191,22 +194,37 @@ __global__ void __launch_bounds__(kTopkThreads) topk_kernel(const float *__restr
             if (nc <= (uint32_t)kTopkCandidates) {  // (uniform over the workgroup)
                 // (the list is read four keys at a time: zero keys, below every real one, fill it up to a multiple of four)
                 if (tid < 4) cand[nc + tid] = 0;
+                // A candidate's rank = the candidates above it.  The threads beyond the list take part: with the list
+                // rounded up to a power of two, thread t counts for candidate t % that over the t / that -th share of
+                // the list, and the shares meet in an LDS counter (half as long for the usual 300-500 candidates).
+                uint32_t ncr = 64;
+                while (ncr < nc) ncr <<= 1;
+                const uint32_t parts = (uint32_t)kTopkThreads / ncr, ci = tid & (ncr - 1u), part = tid / ncr;
+                if (parts > 1 && tid < nc) rank_sh[tid] = 0;
                 __syncthreads();
-                if (tid < nc) {
-                    const uint64_t key = cand[tid];
-                    uint32_t rank = 0;
+                uint64_t key = 0;
+                uint32_t rank = 0;
+                if (ci < nc) {
+                    key = cand[ci];
                     typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
                     const u64x2 *c2 = reinterpret_cast<const u64x2 *>(cand);
+                    const uint32_t quads = (nc + 3) / 4, per = (quads + parts - 1) / parts;
+                    const uint32_t j0 = part * per, j1 = min(quads, j0 + per);
 #pragma unroll 2
-                    for (uint32_t j = 0; j < (nc + 3) / 4; j++) {
+                    for (uint32_t j = j0; j < j1; j++) {
                         const u64x2 a = c2[2 * j], b = c2[2 * j + 1];
                         rank += (a.x > key ? 1u : 0u) + (a.y > key ? 1u : 0u) + (b.x > key ? 1u : 0u) + (b.y > key ? 1u : 0u);
                     }
-                    if (rank < k) {
-                        const uint32_t idx = ~(uint32_t)key;
-                        idx_out[(size_t)row * k + rank] = idx;
-                        val_out[(size_t)row * k + rank] = s[idx];
-                    }
+                    if (parts > 1 && rank != 0) atomicAdd(&rank_sh[ci], rank);
+                }
+                if (parts > 1) {
+                    __syncthreads();
+                    if (tid < nc) rank = rank_sh[tid];
+                }
+                if (tid < nc && rank < k) {  // (tid < nc: ci == tid, the key is this thread's candidate)
+                    const uint32_t idx = ~(uint32_t)key;
+                    idx_out[(size_t)row * k + rank] = idx;
+                    val_out[(size_t)row * k + rank] = s[idx];
                 }
                 if (tid == 0) count_out[row] = min(k, nc);
                 return;
