@@ -2006,7 +2006,7 @@ constexpr int kBfBatchTiles = 2;
 constexpr int kBfMaxPasses = 2;
 constexpr int kBfMaxSets = 2;       // 4 positions each
 constexpr int kBfMaxWaves = 10;
-constexpr uint32_t kBfTileBytes = 4 * 1024;  // 16 rows x 4 steps x 64 B
+constexpr uint32_t kBfTileBytes = 4 * 1024;  // 16 rows x 256 B (four steps of 32 elements)
 
 __device__ __forceinline__ uint32_t bf16_term_bits(float &r) {  // next 8 significant bits of r; r keeps the rest
     const uint32_t b = __builtin_bit_cast(uint32_t, r) & 0xFFFF0000u;
@@ -2049,7 +2049,14 @@ __device__ __forceinline__ void run_bf16_mfma(const GemvJob &j, uint32_t tile_a,
     const uint32_t np = wv < nwj ? (cols - wv + nwj - 1) / nwj : 0;  // columns wv, wv+nwj of this wavefront
     const uint32_t PW = 8 * nw_launch;                              // partials per row: [position][wavefront]
 
-    const uint32_t lane_off = jr * row_bytes + kq * 16;
+    // A copy instruction brings whole 128-byte lines: 8 rows x one half of the column's 256 bytes, eight consecutive
+    // lanes to a line (instruction i: rows 8 (i % 2) .., half i / 2).  LDS receives a lane's 16 bytes at 16 * lane, so
+    // within its line a lane fetches chunk (lane % 8) ^ ((row / 2) % 8): the operand reads below (16 rows, one chunk
+    // each) then fall on 16 different bank groups.
+    const uint32_t cr8 = lane >> 3, cc8 = lane & 7u;
+    uint32_t copy_off[2];
+#pragma unroll
+    for (int g = 0; g < 2; g++) copy_off[g] = (g * 8 + cr8) * row_bytes + ((cc8 ^ ((g * 4 + (cr8 >> 1)) & 7u)) * 16);
     const uint32_t nt = tile_b - tile_a;
     uint32_t it_tile = tile_a, it_p = 0, n_issue = 0;
     auto issue = [&]() {
@@ -2057,12 +2064,14 @@ __device__ __forceinline__ void run_bf16_mfma(const GemvJob &j, uint32_t tile_a,
         // wave-uniform 64-bit base + per-lane 32-bit offset (the lane's row within the tile, clamped into the matrix)
         const uint32_t rb = tl * 16;
         const uint8_t *gb = j.w + (size_t)rb * row_bytes + (size_t)(wv + nwj * it_p) * 256;
-        uint32_t lo = lane_off;
-        if (rb + 16 > rows) lo = min(jr, rows - 1 - rb) * row_bytes + kq * 16;  // ragged last tile only
-        const uint8_t *gp = gb + lo;
+        uint32_t lo[2] = {copy_off[0], copy_off[1]};
+        if (rb + 16 > rows) {  // ragged last tile only: rows past the end read the last one
+#pragma unroll
+            for (int g = 0; g < 2; g++) lo[g] = min(g * 8 + cr8, rows - 1 - rb) * row_bytes + ((cc8 ^ ((g * 4 + (cr8 >> 1)) & 7u)) * 16);
+        }
         uint8_t *lp = ring + (n_issue % NS) * kBfTileBytes;
 #pragma unroll
-        for (int s = 0; s < 4; s++) __builtin_amdgcn_global_load_lds((g_vp)(gp + s * 64), (lds_vp)(lp + s * 1024), 16, 0, 0);
+        for (int i = 0; i < 4; i++) __builtin_amdgcn_global_load_lds((g_vp)(gb + lo[i & 1] + (i >> 1) * 128), (lds_vp)(lp + i * 1024), 16, 0, 0);
         n_issue++;
         if (it_tile < tile_b && ++it_p == np) { it_p = 0; it_tile++; }
     };
@@ -2099,7 +2108,9 @@ __device__ __forceinline__ void run_bf16_mfma(const GemvJob &j, uint32_t tile_a,
 #pragma unroll
                         for (int s = 0; s < 4; s++) {
                             BfOp b;
-                            const u32x4 q4 = *reinterpret_cast<const u32x4 *>(slot + s * 1024 + lane * 16);
+                            // row jr, chunk 4 (s % 2) + kq of half s / 2: instruction jr / 8 + 2 (s / 2), swizzled as it was copied
+                            const u32x4 q4 = *reinterpret_cast<const u32x4 *>(slot + ((jr >> 3) + 2 * (s >> 1)) * 1024 +
+                                                                              (8 * (jr & 7u) + (((s & 1) * 4 + kq) ^ ((jr >> 1) & 7u))) * 16);
                             b.u[0] = q4.x; b.u[1] = q4.y; b.u[2] = q4.z; b.u[3] = q4.w;
 #pragma unroll
                             for (int q = 0; q < kBfMaxSets; q++)
