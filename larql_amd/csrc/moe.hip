@@ -172,8 +172,10 @@ __global__ void __launch_bounds__(1024) moe_plan_kernel(const float *__restrict_
         __device__ uint32_t job(uint32_t m) const { return su(m) + tiles * cpt(m); }
     };
     const auto cost_model = [&](uint32_t tiles, uint32_t grid, uint32_t lists) {
-        const uint64_t tpw = max((uint64_t)1, (uint64_t)lists * n_jobs * tiles / max(grid, 1u));
-        return JobCost{tiles, tpw <= 256 ? (uint32_t)tpw : 0u};
+        // (float arithmetic: a rough figure is all the model needs, and a 64-bit division is a hundred instructions)
+        const float tpw_f = (float)(lists * n_jobs) * (float)tiles / (float)max(grid, 1u);
+        const uint32_t tpw = tpw_f < 1.0f ? 1u : tpw_f > 256.0f ? 0u : (uint32_t)tpw_f;
+        return JobCost{tiles, tpw};
     };
     const uint32_t g_tiles = ((uint32_t)tg.rows + 15) / 16, d_tiles = ((uint32_t)td.rows + 15) / 16;
     const JobCost gc = cost_model(g_tiles, g_grid, fused ? 1u : 2u), dc = cost_model(d_tiles, d_grid, 1u);
