@@ -647,9 +647,6 @@ int larql_hip_q4k_dual_matvec(larql_hip_ctx *c, const uint8_t *a, size_t a_len, 
     return host_matvec_multi(c, KIND_Q4K, 2, w, wl, nullptr, nullptr, rows, hidden, x, x_len * 4, outs);
 }
 
-static void push_gate_jobs(std::vector<GemvJob> &jobs, int kind, const void *gate, const float *x, size_t batch, size_t n,
-                           size_t hidden, float *scores);
-
 int larql_hip_q4k_matmul(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, const float *x, size_t x_len,
                          size_t num_rows, size_t hidden, size_t seq_len, float *out, size_t out_len) {
     if (!c) return LARQL_E_ARG;
@@ -697,9 +694,10 @@ int larql_hip_q4k_matmul(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, c
             HIPCHECK(c, q4k_gemm_f16_launch(c->stream, dw, xl, sx, nullptr, ts, (float *)c->out.p, (uint32_t)num_rows, (uint32_t)hidden, (uint32_t)seq_len, 0, 1,
                                             splits, partial));
     } else {
-        // a few positions: matvec jobs, up to eight positions per pass over the matrix where the rows are short enough
         std::vector<GemvJob> jobs;
-        push_gate_jobs(jobs, KIND_Q4K, dw, (const float *)c->x.p, seq_len, num_rows, hidden, (float *)c->out.p);
+        for (size_t s = 0; s < seq_len; s++)
+            jobs.push_back(make_job(KIND_Q4K, dw, nullptr, (const float *)c->x.p + s * hidden, (float *)c->out.p + s * num_rows,
+                                    num_rows, hidden));
         rc = enqueue_jobs(c, jobs);
         if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
     }

@@ -130,6 +130,9 @@ def test_q4k_dual_and_matmul(be):
     out = be.q4k_matmul(qa, X, rows, cols, seq)
     want = O.q4k_matmul(qa, X, rows, cols, seq)
     assert rel_l2(out, want.reshape(-1)) < TOL
+    # below 16 positions a row of the product is the matvec of that position, bit for bit
+    for s in range(seq):
+        assert np.array_equal(out.reshape(seq, rows)[s].view(np.uint32), be.q4k_matvec(qa, X[s], rows, cols).view(np.uint32)), s
     # zero dimensions (kquant_matmul_into, matmul.rs:89-92): no positions / no rows -> an empty result; hidden == 0 with
     # rows and positions -> seq * rows zeros; lengths that do not describe [seq, rows] / [seq, hidden] are refused
     assert be.q4k_matmul(qa, X[:0], rows, cols, 0).size == 0
