@@ -612,7 +612,8 @@ def test_gate_knn_edge_cases(be, fmt):
     assert [i for i, _ in be.gate_knn(fmt.FMT_F32, eye, xt, 4, 256, 2)] == [0, 1]
 
 
-@pytest.mark.parametrize("case", ["normal", "sorted", "constant", "coarse", "tie_block", "max_cached", "streamed", "ragged"])
+@pytest.mark.parametrize("case", ["normal", "sorted", "constant", "coarse", "tie_block", "max_cached", "streamed", "ragged",
+                                  "few_candidates", "many_candidates"])
 def test_top_k_selection_paths(be, fmt, case):
     # top_k_by_abs on prescribed score rows (scores = gate[:, 0] through a unit residual), over the selection paths
     # of the kernel: candidates ranked directly, the radix passes (sorted / constant rows have too many candidates),
@@ -631,6 +632,18 @@ def test_top_k_selection_paths(be, fmt, case):
         sc = rng.standard_normal(n) * 0.1
         sc[rng.choice(n, 100, replace=False)] = 5.0              # 100 equal scores straddle the K boundary
         sc[rng.choice(n, 20, replace=False)] = -7.0
+    elif case == "few_candidates":
+        # exactly 64 scores stand out, one in each of the 64 slices of the row (a slice = wavefront w, 16 lanes g of it:
+        # indices 640 w + 64 it + 16 g + j): the candidate list is as short as it gets, every thread counts a 16th of it
+        sc = rng.uniform(-1.0, 1.0, n)
+        for w in range(16):
+            for g in range(4):
+                sc[640 * w + 64 * int(rng.integers(10)) + 16 * g + int(rng.integers(16))] = 10.0 + rng.uniform(0.0, 1.0) * (1 if (w + g) % 2 else -1)
+    elif case == "many_candidates":
+        # one slice stays below 0.93, the rest is uniform on (0, 1): ~700 candidates, a list that is not split into shares
+        sc = rng.uniform(0.0, 1.0, n) * rng.choice([-1.0, 1.0], n)
+        sl = np.array([640 * 5 + 64 * it + 16 * 2 + j for it in range(10) for j in range(16)])
+        sc[sl] *= 0.93
     elif case == "max_cached":
         n = 16384; sc = rng.standard_normal(n)
     elif case == "streamed":
