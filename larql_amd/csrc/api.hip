@@ -188,6 +188,17 @@ int prepare_same_kind(larql_hip_ctx *c, GemvJob *live, size_t n_live, void *tabl
         j.pass_begin = (uint32_t)total;
         total += j.n_pass;
     }
+    P.lds = gemv_lds_bytes(live, n_live, P.threads);
+    uint64_t grid = (uint64_t)c->cu_count * (uint64_t)gemv_wgs_per_cu(P.kind, P.threads, P.lds, (uint32_t)c->wgs_per_cu);
+    // the share-out's cost model wants to know how long a workgroup's share is: a second pass over the costs
+    if (gemv_refine_costs(live, n_live, (uint32_t)std::min<uint64_t>(grid, 0xFFFFFFFFull))) {
+        total = 0;
+        for (size_t ji = 0; ji < n_live; ji++) {
+            if (total + live[ji].n_pass > 0x7FFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "matvec: launch too large");
+            live[ji].pass_begin = (uint32_t)total;
+            total += live[ji].n_pass;
+        }
+    }
     memset(&P.L, 0, sizeof P.L);
     P.L.total_passes = total;
     P.L.n_jobs = (uint32_t)n_live;
@@ -224,8 +235,6 @@ int prepare_same_kind(larql_hip_ctx *c, GemvJob *live, size_t n_live, void *tabl
         }
         P.L.table = (const GemvJob *)table_dst;
     }
-    P.lds = gemv_lds_bytes(live, n_live, P.threads);
-    uint64_t grid = (uint64_t)c->cu_count * (uint64_t)gemv_wgs_per_cu(P.kind, P.threads, P.lds, (uint32_t)c->wgs_per_cu);
     if (grid > total) grid = total;
     P.grid = (uint32_t)grid;
     return LARQL_OK;

@@ -3181,6 +3181,41 @@ int gemv_effective_kind(const GemvJob &j) {
     return j.kind;
 }
 
+// Cost model of the share-out for the matrix-core Q4_K kernels, in 128ths of the time a ten-column tile takes
+// (fitted on time stamps per workgroup and job segment of a mixed 238-job launch: set-up + tiles x cost per job kind):
+// a tile of nw columns costs 58 + 7 nw (eight columns: 0.89 of ten), a tile walked in several column passes 19/16 of
+// that per pass, and every share of a job — the one that opens it or not — starts with a pipeline refill and the
+// activation set-up, worth 4.5 tiles (8.2 with several columns per wavefront).
+static void q4k_tile_cost(uint64_t cpr, uint32_t nw, uint64_t *cpt, uint64_t *startup) {
+    const uint64_t np = (cpr + nw - 1) / nw;
+    const uint64_t one = 58 + 7 * (uint64_t)nw;
+    *cpt = np == 1 ? one : (np * one * 19) / 16;
+    *startup = np == 1 ? 576 : 1050;
+}
+
+// The opening share's set-up is in the job's cost (GemvJob::pad2); the later shares' set-ups ride on the tiles: a
+// share of U units holds U / cpt tiles and pays one set-up, so a tile costs cpt (1 + set-up / U), U = the launch's
+// units per workgroup.
+bool gemv_refine_costs(GemvJob *jobs, size_t n, uint32_t grid) {
+    if (n == 0 || grid == 0 || (jobs[0].kind != KIND_Q4K_MFMA && jobs[0].kind != KIND_Q4K_Q8K)) return false;
+    uint64_t total = 0;
+    for (size_t i = 0; i < n; i++) total += (uint64_t)jobs[i].n_pass;
+    const uint64_t U = std::max<uint64_t>(total / grid, 1);
+    const auto refined = [&](const GemvJob &j) {  // (a share shorter than its set-up: the tile cost at most doubles)
+        const uint64_t cpt = (uint64_t)j.pad, su = j.pad2;
+        return cpt + std::min<uint64_t>(cpt, (cpt * su + U / 2) / U);
+    };
+    for (size_t i = 0; i < n; i++)
+        if (jobs[i].pad2 + ((jobs[i].rows + 15) / 16) * refined(jobs[i]) > 0x7FFFFFFFull) return false;  // (nothing changed yet)
+    for (size_t i = 0; i < n; i++) {
+        GemvJob &j = jobs[i];
+        const uint64_t cpt = refined(j);
+        j.pad = (int32_t)cpt;
+        j.n_pass = (uint32_t)(j.pad2 + ((j.rows + 15) / 16) * cpt);
+    }
+    return true;
+}
+
 bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
     if (j.kind == KIND_Q8_0_MFMA) {
         const uint64_t cpr = j.k / 256;
@@ -3264,13 +3299,8 @@ bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
         j.rpp = nw;  // wavefronts that work on this job
         j.row_bytes = cpr * 144;
         const uint64_t tiles = (j.rows + 15) / 16;
-        // Cost model of the share-out, in sixteenths of the time a wavefront takes for one wave-tile (measured
-        // per workgroup and job segment on a mixed 238-job launch): a tile costs one wave-tile time per column
-        // pass whatever the number of columns (narrow rows leave wavefronts idle, they do not finish sooner),
-        // multi-pass tiles come ~19 % dearer per pass, and every job start costs a pipeline refill and the
-        // activation set-up (~4 us, ~10 us with several columns per wavefront).
-        const uint64_t np = (cpr + nw - 1) / nw;
-        const uint64_t cpt = np == 1 ? 16 : np * 19, startup = np == 1 ? 72 : 180;
+        uint64_t cpt, startup;
+        q4k_tile_cost(cpr, nw, &cpt, &startup);
         j.pad = (int32_t)cpt;
         j.pad2 = (uint32_t)startup;
         if (startup + tiles * cpt > 0x7FFFFFFFull) return false;

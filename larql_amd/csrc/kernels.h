@@ -96,6 +96,9 @@ struct GemvLaunch {
 };
 
 bool gemv_job_geometry(GemvJob &j, uint32_t threads);
+// Second pass of the share-out's cost model over the jobs of one launch, once the grid is known (the matrix-core Q4_K
+// kernels: a share's set-up is spread over its tiles).  True when costs (n_pass) changed: pass_begin is the caller's to redo.
+bool gemv_refine_costs(GemvJob *jobs, size_t n, uint32_t grid);
 uint32_t gemv_pick_threads(const GemvJob *jobs, size_t n);
 size_t gemv_lds_bytes(const GemvJob *jobs, size_t n, uint32_t threads);
 int gemv_effective_kind(const GemvJob &j);
