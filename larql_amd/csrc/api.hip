@@ -176,6 +176,10 @@ struct PreparedLaunch {
 
 // Geometry for one launch over jobs of a single format.  When the jobs do not fit
 // inline the table is uploaded into `table_dst` (synchronously: the host vector may die).
+// A device table's size: the jobs and the first job of up to kTableFirstMax workgroups' shares.
+constexpr size_t kTableFirstMax = 4096;
+static size_t table_bytes_for(size_t n_jobs) { return n_jobs * sizeof(GemvJob) + kTableFirstMax * sizeof(uint32_t); }
+
 int prepare_same_kind(larql_hip_ctx *c, GemvJob *live, size_t n_live, void *table_dst, PreparedLaunch &P, int stage_slot = -1) {
     P.kind = live[0].kind;
     P.threads = gemv_pick_threads(live, n_live);
@@ -199,6 +203,8 @@ int prepare_same_kind(larql_hip_ctx *c, GemvJob *live, size_t n_live, void *tabl
             total += live[ji].n_pass;
         }
     }
+    if (grid > total) grid = total;
+    P.grid = (uint32_t)grid;
     memset(&P.L, 0, sizeof P.L);
     P.L.total_passes = total;
     P.L.n_jobs = (uint32_t)n_live;
@@ -207,9 +213,24 @@ int prepare_same_kind(larql_hip_ctx *c, GemvJob *live, size_t n_live, void *tabl
         for (size_t i = 0; i < n_live; i++) P.L.inl[i] = live[i];
         P.L.table = nullptr;
     } else {
-        const size_t bytes = n_live * sizeof(GemvJob);
+        // the table: the jobs, then the first job of every workgroup's share (what a workgroup would otherwise find by
+        // bisection over the jobs' pass ranges, a dependent load per step)
+        const size_t job_bytes = n_live * sizeof(GemvJob);
+        const bool with_first = grid >= 1 && grid <= (uint64_t)kTableFirstMax;
+        const size_t bytes = job_bytes + (with_first ? (size_t)grid * sizeof(uint32_t) : 0);
+        std::vector<uint8_t> blob(bytes);
+        memcpy(blob.data(), live, job_bytes);
+        if (with_first) {
+            uint32_t *first = (uint32_t *)(blob.data() + job_bytes);
+            size_t ji = 0;
+            for (uint64_t b = 0; b < grid; b++) {
+                const uint64_t pb = total * b / grid;
+                while (ji + 1 < n_live && (uint64_t)live[ji + 1].pass_begin <= pb) ji++;
+                first[b] = (uint32_t)ji;
+            }
+        }
         if (stage_slot >= 0 && c->table_sent_dst[stage_slot] == table_dst && c->table_sent_bytes[stage_slot] == bytes &&
-            memcmp(c->table_host[stage_slot], live, bytes) == 0) {
+            memcmp(c->table_host[stage_slot], blob.data(), bytes) == 0) {
             // the same jobs as the last call through this slot (a decode loop): the device table is already (or, in
             // stream order, about to be) what this launch needs
         } else if (stage_slot >= 0) {
@@ -224,19 +245,18 @@ int prepare_same_kind(larql_hip_ctx *c, GemvJob *live, size_t n_live, void *tabl
             }
             if (!c->table_ev[stage_slot]) HIPCHECK(c, hipEventCreateWithFlags(&c->table_ev[stage_slot], hipEventDisableTiming));
             else HIPCHECK(c, hipEventSynchronize(c->table_ev[stage_slot]));  // the previous upload from this slot is done
-            memcpy(c->table_host[stage_slot], live, bytes);
+            memcpy(c->table_host[stage_slot], blob.data(), bytes);
             HIPCHECK(c, hipMemcpyAsync(table_dst, c->table_host[stage_slot], bytes, hipMemcpyHostToDevice, c->stream));
             HIPCHECK(c, hipEventRecord(c->table_ev[stage_slot], c->stream));
             c->table_sent_dst[stage_slot] = table_dst;
             c->table_sent_bytes[stage_slot] = bytes;
         } else {
-            HIPCHECK(c, hipMemcpyAsync(table_dst, live, bytes, hipMemcpyHostToDevice, c->stream));
+            HIPCHECK(c, hipMemcpyAsync(table_dst, blob.data(), bytes, hipMemcpyHostToDevice, c->stream));
             HIPCHECK(c, hipStreamSynchronize(c->stream));  // the host vector may die
         }
         P.L.table = (const GemvJob *)table_dst;
+        if (with_first) P.L.wg_first = (const uint32_t *)((const uint8_t *)table_dst + job_bytes);
     }
-    if (grid > total) grid = total;
-    P.grid = (uint32_t)grid;
     return LARQL_OK;
 }
 
@@ -278,7 +298,7 @@ int enqueue_jobs(larql_hip_ctx *c, std::vector<GemvJob> &jobs) {
         DevBuf &tb = c->tables[sl];
         if (live.size() > (size_t)kInlineJobs) {
             const void *before = tb.p;
-            rc = ensure(c, tb, live.size() * sizeof(GemvJob));
+            rc = ensure(c, tb, table_bytes_for(live.size()));
             if (rc) return rc;
             if (tb.p != before) c->table_sent_dst[sl] = nullptr;  // a new allocation holds nothing yet
         }
@@ -1221,7 +1241,7 @@ int larql_hip_plan_create(larql_hip_ctx *c, const larql_hip_matvec_job *pj, size
     for (std::vector<GemvJob> &live : group_by_kind(jobs)) {
         PreparedLaunch P;
         if (live.size() > (size_t)kInlineJobs) {
-            if (hipMalloc(&P.table, live.size() * sizeof(GemvJob)) != hipSuccess) {
+            if (hipMalloc(&P.table, table_bytes_for(live.size())) != hipSuccess) {
                 for (PreparedLaunch &q : plan->launches) if (q.table) (void)hipFree(q.table);
                 delete plan;
                 return fail(c, LARQL_E_DEVICE, "plan: out of device memory");

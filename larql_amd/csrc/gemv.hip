@@ -2805,6 +2805,17 @@ __device__ __forceinline__ job_cp job_table(const GemvLaunch &L) { return L.tabl
 __device__ __forceinline__ uint32_t job_pass_begin(job_cp jobs, uint32_t i) {
     return *(const CONST_AS uint32_t *)((const CONST_AS uint8_t *)(jobs + i) + offsetof(GemvJob, pass_begin));
 }
+// The job that holds pass p, the first of workgroup blockIdx.x: read from the launch's table of first jobs where it has
+// one (a single scalar load), else found by bisection over the jobs' pass ranges (a dependent load per step).
+__device__ __forceinline__ uint32_t first_job_of_share(const GemvLaunch &L, job_cp jobs, uint32_t n_jobs, uint32_t p) {
+    if (L.wg_first) return *((const CONST_AS uint32_t *)L.wg_first + blockIdx.x);
+    uint32_t lo = 0, hi = n_jobs;
+    while (lo + 1 < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (job_pass_begin(jobs, mid) <= p) lo = mid; else hi = mid;
+    }
+    return lo;
+}
 __device__ __forceinline__ GemvJob uniform_job(job_cp src) {
     static_assert(sizeof(GemvJob) % 4 == 0, "descriptor is a whole number of dwords");
     constexpr int N = sizeof(GemvJob) / 4;
@@ -2827,12 +2838,7 @@ __device__ __forceinline__ void gemv_body(const GemvLaunch &L, float *part) {
     const uint64_t P = L.total_passes;
     uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
     const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
-    // first job whose pass range ends after p
-    uint32_t lo = 0, hi = L.n_jobs;
-    while (lo + 1 < hi) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (job_pass_begin(jobs, mid) <= p) lo = mid; else hi = mid;
-    }
+    const uint32_t lo = first_job_of_share(L, jobs, L.n_jobs, p);
     uint32_t ji = lo;
     while (p < p_end) {
         GemvJob j = uniform_job(jobs + ji);
@@ -2888,11 +2894,7 @@ __global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_mfma_kernel(GemvLa
     const uint64_t P = L.total_passes;
     uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
     const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
-    uint32_t lo = 0, hi = L.n_jobs;
-    while (lo + 1 < hi) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (job_pass_begin(jobs, mid) <= p) lo = mid; else hi = mid;
-    }
+    const uint32_t lo = first_job_of_share(L, jobs, L.n_jobs, p);
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
         const GemvJob j = uniform_job(jobs + ji);
@@ -2915,11 +2917,7 @@ __global__ void __launch_bounds__(kQ6kMaxWaves * 64) gemv_q6k_mfma_kernel(GemvLa
     const uint64_t P = L.total_passes;
     uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
     const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
-    uint32_t lo = 0, hi = L.n_jobs;
-    while (lo + 1 < hi) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (job_pass_begin(jobs, mid) <= p) lo = mid; else hi = mid;
-    }
+    const uint32_t lo = first_job_of_share(L, jobs, L.n_jobs, p);
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
         const GemvJob j = uniform_job(jobs + ji);
@@ -2940,11 +2938,7 @@ __global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_q8k_kernel(GemvLau
     const uint64_t P = L.total_passes;
     uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
     const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
-    uint32_t lo = 0, hi = L.n_jobs;
-    while (lo + 1 < hi) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (job_pass_begin(jobs, mid) <= p) lo = mid; else hi = mid;
-    }
+    const uint32_t lo = first_job_of_share(L, jobs, L.n_jobs, p);
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
         const GemvJob j = uniform_job(jobs + ji);
@@ -2968,11 +2962,7 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) gemv_mxfp4_mfma_kernel(Gemv
     if (P == 0 || n_jobs == 0) return;
     uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
     const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
-    uint32_t lo = 0, hi = n_jobs;
-    while (lo + 1 < hi) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (job_pass_begin(jobs, mid) <= p) lo = mid; else hi = mid;
-    }
+    const uint32_t lo = first_job_of_share(L, jobs, n_jobs, p);
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
         GemvJob j = uniform_job(jobs + ji);
@@ -3036,11 +3026,7 @@ __global__ void __launch_bounds__(kBfMaxWaves * 64) gemv_bf16_mfma_kernel(GemvLa
     const uint64_t P = L.total_passes;
     uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
     const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
-    uint32_t lo = 0, hi = L.n_jobs;
-    while (lo + 1 < hi) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (job_pass_begin(jobs, mid) <= p) lo = mid; else hi = mid;
-    }
+    const uint32_t lo = first_job_of_share(L, jobs, L.n_jobs, p);
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
         const GemvJob j = uniform_job(jobs + ji);
@@ -3061,11 +3047,7 @@ __global__ void __launch_bounds__((kQ4kMaxWaves + 2) * 64) gemv_q4k_batch_kernel
     const uint64_t P = L.total_passes;
     uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
     const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
-    uint32_t lo = 0, hi = L.n_jobs;
-    while (lo + 1 < hi) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (job_pass_begin(jobs, mid) <= p) lo = mid; else hi = mid;
-    }
+    const uint32_t lo = first_job_of_share(L, jobs, L.n_jobs, p);
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
         const GemvJob j = uniform_job(jobs + ji);
@@ -3086,11 +3068,7 @@ __global__ void __launch_bounds__(kQ8MaxWaves * 64) gemv_q8_0_mfma_kernel(GemvLa
     const uint64_t P = L.total_passes;
     uint32_t p = (uint32_t)(P * blockIdx.x / gridDim.x);
     const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
-    uint32_t lo = 0, hi = L.n_jobs;
-    while (lo + 1 < hi) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (job_pass_begin(jobs, mid) <= p) lo = mid; else hi = mid;
-    }
+    const uint32_t lo = first_job_of_share(L, jobs, L.n_jobs, p);
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
         const GemvJob j = uniform_job(jobs + ji);

@@ -93,6 +93,9 @@ struct GemvLaunch {
     // Optional: the job count and pass total live in device memory ({n_jobs, total_passes}, written by a kernel
     // earlier on the stream) and override the two fields above.  MXFP4 matrix-core kernel only.
     const uint32_t *dyn;
+    // Optional: the first job of every workgroup's share ([grid] indices in device memory), so that a workgroup need not
+    // search the jobs' pass ranges for it.
+    const uint32_t *wg_first;
 };
 
 bool gemv_job_geometry(GemvJob &j, uint32_t threads);
