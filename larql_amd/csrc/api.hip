@@ -1617,7 +1617,8 @@ static int moe_mxfp4_block(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank
         GemvJob td = make_job(KIND_MXFP4, bank->down_packed, bank->down_scales, g, d, hidden, inter);
         td.x_glu = fused ? g : u; td.glu_limit = bank->limit; td.glu_alpha = bank->alpha;
         set_down_bias(td);
-        const size_t table_bytes = slots * 3 * sizeof(GemvJob) + 64;
+        constexpr uint32_t kFirstMax = 1024;  // workgroups per launch whose first jobs the planner looks up
+        const size_t table_bytes = slots * 3 * sizeof(GemvJob) + 64 + 2 * kFirstMax * sizeof(uint32_t);
         const bool mfma = gemv_effective_kind(tg) == KIND_MXFP4_MFMA && gemv_effective_kind(td) == KIND_MXFP4_MFMA;
         if (mfma && tokens > 1 && slots <= 4096 && bank->n_experts <= 1024 && slots * inter * sizeof(float) >= table_bytes) {
             tg.kind = tu.kind = td.kind = KIND_MXFP4_MFMA;
@@ -1650,10 +1651,17 @@ static int moe_mxfp4_block(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank
                 P.grid = (uint32_t)((uint64_t)c->cu_count * gemv_wgs_per_cu(P.kind, P.threads, P.lds, (uint32_t)c->wgs_per_cu));
             }
             if (!gemv_job_geometry(tu, Pg.threads)) return fail(c, LARQL_UNSUPPORTED, "moe_mxfp4: unsupported geometry");
+            uint32_t *gu_first = nullptr, *dn_first = nullptr;
+            if (Pg.grid <= kFirstMax && Pd.grid <= kFirstMax) {
+                gu_first = (uint32_t *)(dn_table + slots);
+                dn_first = gu_first + kFirstMax;
+                Pg.L.wg_first = gu_first;
+                Pd.L.wg_first = dn_first;
+            }
             HIPCHECK(c, moe_plan_launch(c->stream, router_pending ? route_logits : nullptr, bank->router_bias, route_policy, weights, experts,
                                         (uint32_t)slots, (uint32_t)k, (uint32_t)bank->n_experts, tg, tu, td, gu_w_stride,
                                         gu_s_stride, dn_w_stride, dn_s_stride, (uint32_t)hidden, (uint32_t)inter, fused, group, Pg.grid, Pd.grid, gu_table,
-                                        hdr, dn_table, hdr + 2));
+                                        hdr, dn_table, hdr + 2, gu_first, dn_first));
             HIPCHECK(c, gemv_launch(c->stream, Pg.kind, Pg.L, Pg.threads, Pg.grid, Pg.lds));
             HIPCHECK(c, gemv_launch(c->stream, Pd.kind, Pd.L, Pd.threads, Pd.grid, Pd.lds));
             HIPCHECK(c, weighted_sum_launch(c->stream, d, weights, experts, (uint32_t)bank->n_experts, out, (uint32_t)tokens, (uint32_t)k,

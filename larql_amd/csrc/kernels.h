@@ -190,7 +190,7 @@ hipError_t moe_plan_launch(hipStream_t s, const float *logits, const float *rout
                            uint32_t slots, uint32_t k, uint32_t n_experts, const GemvJob &tg,
                            const GemvJob &tu, const GemvJob &td, uint64_t gu_w_stride, uint64_t gu_s_stride, uint64_t dn_w_stride,
                            uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, bool fused, uint32_t group, uint32_t g_grid, uint32_t d_grid,
-                           GemvJob *gu_table, uint32_t *gu_hdr, GemvJob *dn_table, uint32_t *dn_hdr);
+                           GemvJob *gu_table, uint32_t *gu_hdr, GemvJob *dn_table, uint32_t *dn_hdr, uint32_t *gu_first, uint32_t *dn_first);
 hipError_t clamped_glu_interleaved_launch(hipStream_t s, const float *gu, float *h, size_t n, float limit, float alpha);
 hipError_t clamped_glu_launch(hipStream_t s, const float *g, const float *u, float *h, size_t n, float limit, float alpha);
 hipError_t weighted_sum_launch(hipStream_t s, const float *d, const float *weights, const uint32_t *experts, uint32_t n_experts, float *out,

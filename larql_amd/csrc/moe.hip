@@ -89,7 +89,8 @@ __global__ void __launch_bounds__(1024) moe_plan_kernel(const float *__restrict_
                                                        GemvJob tg, GemvJob tu, GemvJob td, uint64_t gu_w_stride, uint64_t gu_s_stride,
                                                        uint64_t dn_w_stride, uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, uint32_t fused,
                                                        uint32_t group, uint32_t g_grid, uint32_t d_grid, GemvJob *__restrict__ gu_table,
-                                                       uint32_t *__restrict__ gu_hdr, GemvJob *__restrict__ dn_table, uint32_t *__restrict__ dn_hdr) {
+                                                       uint32_t *__restrict__ gu_hdr, GemvJob *__restrict__ dn_table, uint32_t *__restrict__ dn_hdr,
+                                                       uint32_t *__restrict__ gu_first, uint32_t *__restrict__ dn_first) {
     __shared__ uint32_t first_job[1025];  // first job of expert e; [n_experts] = total
     __shared__ uint32_t first_kind_a[1025], first_kind_b[1025];  // the jobs before expert e by kind: {full groups, of 1 slot}, {of 2, of 3}
     __shared__ __attribute__((aligned(16))) uint32_t cnt[1024];  // slots per expert
@@ -121,40 +122,78 @@ __global__ void __launch_bounds__(1024) moe_plan_kernel(const float *__restrict_
         for (uint32_t s = t; s < ((slots + 3u) & ~3u); s += blockDim.x) ex[s] = s < slots ? experts[s] : 0xFFFFFFFFu;
     }
     __syncthreads();
-    // ranks: four earlier slots per LDS read, the reads of a round independent of each other
-    for (uint32_t s = t; s < slots; s += blockDim.x) {
-        const uint32_t e = ex[s];
-        uint32_t r = 0;
-#pragma unroll 4
-        for (uint32_t q = 0; q < s; q += 4) {
-            const uint4 v = *reinterpret_cast<const uint4 *>(&ex[q]);
-            r += (v.x == e ? 1u : 0u) + (q + 1 < s && v.y == e ? 1u : 0u) + (q + 2 < s && v.z == e ? 1u : 0u) + (q + 3 < s && v.w == e ? 1u : 0u);
+    if (slots <= 64 && n_experts <= 64) {
+        // A block of up to 64 slots and 64 experts is planned by one wavefront without a barrier in between: lane s is
+        // slot s (its rank = the earlier lanes with the same expert, one ballot per expert), lane e is expert e (its
+        // count from the same ballots, the sums over the experts before it by a scan across the lanes).
+        if (t < 64) {
+            const uint32_t e = t < slots ? ex[t] : 0xFFFFFFFFu;
+            uint32_t r = 0, c = 0;
+            for (uint32_t q = 0; q < n_experts; q++) {
+                const uint64_t m = __ballot(e == q);
+                if (e == q) r = (uint32_t)__popcll(m & ((1ull << t) - 1ull));
+                if (t == q) c = (uint32_t)__popcll(m);
+            }
+            if (t < slots) rank[t] = (uint16_t)r;
+            if (t < n_experts) cnt[t] = c;
+            // what expert t adds to the sums (lanes from n_experts on add nothing): jobs | slots << 16, and the jobs by kind
+            // in one word (full groups, groups of 1, 2, 3 slots: a byte each, at most 64)
+            const uint32_t mm = c & gmask;
+            uint32_t js = ((c + gmask) >> gsh) | (c << 16);
+            uint32_t kk = (c >> gsh) | (mm == 1 ? 0x100u : 0u) | (mm == 2 ? 0x10000u : 0u) | (mm == 3 ? 0x1000000u : 0u);
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {  // inclusive sums over the lanes
+                const uint32_t a = (uint32_t)__shfl_up((int)js, o, 64), bq = (uint32_t)__shfl_up((int)kk, o, 64);
+                if (t >= (uint32_t)o) { js += a; kk += bq; }
+            }
+            // entry e = the experts before e: lane e - 1's inclusive sums (entry 0 = nothing, entry n_experts = everything)
+            const uint32_t at = t + 1;
+            if (at <= n_experts) {
+                first_job[at] = js & 0xFFFFu; first_slot[at] = js >> 16;
+                first_kind_a[at] = (kk & 0xFFu) | (((kk >> 8) & 0xFFu) << 16);
+                first_kind_b[at] = ((kk >> 16) & 0xFFu) | ((kk >> 24) << 16);
+            }
+            if (t == 0) { first_job[0] = 0; first_slot[0] = 0; first_kind_a[0] = 0; first_kind_b[0] = 0; }
+            // (the same wavefront reads what it has just written: LDS executes a wavefront's operations in order)
+            if (e < n_experts) by_expert[first_slot[e] + r] = (uint16_t)t;
         }
-        rank[s] = (uint16_t)r;
-        if (e < n_experts) atomicAdd(&cnt[e], 1u);
-    }
-    __syncthreads();
-    // Per expert: the jobs before it, counted by kind (full groups, and groups of 1, 2 or 3 slots), 16 bits a count.
-    for (uint32_t e = t; e <= n_experts; e += blockDim.x) {
-        uint32_t f = 0, ka = 0, kb = 0, fs = 0;
-        auto add = [&](uint32_t c) {
-            fs += c;
-            f += (c + gmask) >> gsh;
-            const uint32_t m = c & gmask;
-            ka += (c >> gsh) + (m == 1 ? 0x10000u : 0u);
-            kb += (m == 2 ? 1u : 0u) + (m == 3 ? 0x10000u : 0u);
-        };
-#pragma unroll 2
-        for (uint32_t q = 0; q < e; q += 4) {
-            const uint4 v = *reinterpret_cast<const uint4 *>(&cnt[q]);
-            add(v.x);
-            if (q + 1 < e) add(v.y);
-            if (q + 2 < e) add(v.z);
-            if (q + 3 < e) add(v.w);
+        __syncthreads();
+    } else {
+        // ranks: four earlier slots per LDS read, the reads of a round independent of each other
+        for (uint32_t s = t; s < slots; s += blockDim.x) {
+            const uint32_t e = ex[s];
+            uint32_t r = 0;
+    #pragma unroll 4
+            for (uint32_t q = 0; q < s; q += 4) {
+                const uint4 v = *reinterpret_cast<const uint4 *>(&ex[q]);
+                r += (v.x == e ? 1u : 0u) + (q + 1 < s && v.y == e ? 1u : 0u) + (q + 2 < s && v.z == e ? 1u : 0u) + (q + 3 < s && v.w == e ? 1u : 0u);
+            }
+            rank[s] = (uint16_t)r;
+            if (e < n_experts) atomicAdd(&cnt[e], 1u);
         }
-        first_job[e] = f; first_kind_a[e] = ka; first_kind_b[e] = kb; first_slot[e] = fs;
+        __syncthreads();
+        // Per expert: the jobs before it, counted by kind (full groups, and groups of 1, 2 or 3 slots), 16 bits a count.
+        for (uint32_t e = t; e <= n_experts; e += blockDim.x) {
+            uint32_t f = 0, ka = 0, kb = 0, fs = 0;
+            auto add = [&](uint32_t c) {
+                fs += c;
+                f += (c + gmask) >> gsh;
+                const uint32_t m = c & gmask;
+                ka += (c >> gsh) + (m == 1 ? 0x10000u : 0u);
+                kb += (m == 2 ? 1u : 0u) + (m == 3 ? 0x10000u : 0u);
+            };
+    #pragma unroll 2
+            for (uint32_t q = 0; q < e; q += 4) {
+                const uint4 v = *reinterpret_cast<const uint4 *>(&cnt[q]);
+                add(v.x);
+                if (q + 1 < e) add(v.y);
+                if (q + 2 < e) add(v.z);
+                if (q + 3 < e) add(v.w);
+            }
+            first_job[e] = f; first_kind_a[e] = ka; first_kind_b[e] = kb; first_slot[e] = fs;
+        }
+        __syncthreads();
     }
-    __syncthreads();
     const uint32_t n_jobs = first_job[n_experts];
     // Cost of a job in a launch's pass list.  A workgroup prepares the activations of every job it takes a share of
     // before the share's first tile: about 3 tiles' time for one token and 2 more for every further one (time
@@ -184,13 +223,19 @@ __global__ void __launch_bounds__(1024) moe_plan_kernel(const float *__restrict_
         return (ka & 0xFFFFu) * c.job(group) + (ka >> 16) * c.job(1) + (kb & 0xFFFFu) * c.job(2) + (kb >> 16) * c.job(3);
     };
     const uint32_t g_total = jobs_cost(gc, n_experts), d_total = jobs_cost(dc, n_experts);
-    for (uint32_t s = t; s < slots; s += blockDim.x) {
-        const uint32_t e = ex[s];
-        if (e < n_experts) by_expert[first_slot[e] + rank[s]] = (uint16_t)s;
+    if (!(slots <= 64 && n_experts <= 64)) {  // (the one-wavefront path has done this)
+        for (uint32_t s = t; s < slots; s += blockDim.x) {
+            const uint32_t e = ex[s];
+            if (e < n_experts) by_expert[first_slot[e] + rank[s]] = (uint16_t)s;
+        }
     }
     __syncthreads();
-    // ranks that are multiples of `group` open a job, the `group - 1` that follow join it
-    for (uint32_t s1 = t; s1 < slots; s1 += blockDim.x) {
+    // Ranks that are multiples of `group` open a job, the `group - 1` that follow join it.  The three descriptors of a
+    // job (gate, up, down) are written by three different wavefronts: thread idx serves slot idx % span as kind idx / span.
+    const uint32_t span = (slots + 63u) & ~63u;
+    for (uint32_t idx = t; idx < 3 * span; idx += blockDim.x) {
+        const uint32_t which = idx / span, s1 = idx - which * span;  // (span is a multiple of 64: `which` is the same in a wavefront)
+        if (s1 >= slots || (which == 1 && fused)) continue;
         const uint32_t e = ex[s1], r = rank[s1];
         if (e >= n_experts || (r & gmask)) continue;
         const uint32_t jb = first_job[e] + (r >> gsh);
@@ -237,11 +282,24 @@ __global__ void __launch_bounds__(1024) moe_plan_kernel(const float *__restrict_
         };
         // (the earlier jobs of this expert are all full groups)
         const uint32_t g_begin = jobs_cost(gc, e) + (r >> gsh) * gc.job(group), d_begin = jobs_cost(dc, e) + (r >> gsh) * dc.job(group);
-        emit(gu_table + jb, tg, (size_t)e * gu_w_stride, (size_t)e * gu_s_stride, (size_t)tok1 * hidden, (size_t)s1 * gs, true, gs, g_begin, gc);
-        if (!fused)
+        if (gu_first) {
+            // The first job of every workgroup's share (what a workgroup would otherwise find by bisection over the jobs'
+            // pass ranges, a dependent load per step): workgroup b starts at pass floor(P b / grid), so this job, whose
+            // passes are [begin, begin + cost), is the first of the workgroups from ceil(begin grid / P) up to that of its end.
+            const bool dn = which == 2;
+            const uint32_t grid = dn ? d_grid : g_grid;
+            const uint64_t P = dn ? (uint64_t)d_total : (uint64_t)g_total * (fused ? 1u : 2u);
+            const uint64_t begin = dn ? d_begin : (which == 1 ? g_total + g_begin : g_begin), end = begin + (dn ? dc.job(nb) : gc.job(nb));
+            const uint32_t b0 = (uint32_t)((begin * grid + P - 1) / P), b1 = min(grid, (uint32_t)((end * grid + P - 1) / P));
+            for (uint32_t bb = b0; bb < b1; bb++) (dn ? dn_first : gu_first)[bb] = (which == 1 ? n_jobs : 0u) + jb;
+        }
+        if (which == 0)
+            emit(gu_table + jb, tg, (size_t)e * gu_w_stride, (size_t)e * gu_s_stride, (size_t)tok1 * hidden, (size_t)s1 * gs, true, gs, g_begin, gc);
+        else if (which == 1)
             emit(gu_table + n_jobs + jb, tu, (size_t)e * gu_w_stride, (size_t)e * gu_s_stride, (size_t)tok1 * hidden, (size_t)s1 * gs, true, gs,
                  g_total + g_begin, gc);
-        emit(dn_table + jb, td, (size_t)e * dn_w_stride, (size_t)e * dn_s_stride, (size_t)s1 * gs, (size_t)s1 * hidden, false, hidden, d_begin, dc);
+        else
+            emit(dn_table + jb, td, (size_t)e * dn_w_stride, (size_t)e * dn_s_stride, (size_t)s1 * gs, (size_t)s1 * hidden, false, hidden, d_begin, dc);
     }
     if (t == 0) {
         gu_hdr[0] = fused ? n_jobs : 2 * n_jobs; gu_hdr[1] = fused ? g_total : 2 * g_total;
@@ -253,12 +311,12 @@ hipError_t moe_plan_launch(hipStream_t s, const float *logits, const float *rout
                            uint32_t slots, uint32_t k, uint32_t n_experts, const GemvJob &tg,
                            const GemvJob &tu, const GemvJob &td, uint64_t gu_w_stride, uint64_t gu_s_stride, uint64_t dn_w_stride,
                            uint64_t dn_s_stride, uint32_t hidden, uint32_t inter, bool fused, uint32_t group, uint32_t g_grid, uint32_t d_grid, GemvJob *gu_table,
-                           uint32_t *gu_hdr, GemvJob *dn_table, uint32_t *dn_hdr) {
+                           uint32_t *gu_hdr, GemvJob *dn_table, uint32_t *dn_hdr, uint32_t *gu_first, uint32_t *dn_first) {
     if (n_experts > 1024 || slots > 4096 || (group != 2 && group != 4)) return hipErrorInvalidValue;
     // (a wavefront per token while selecting: 16 wavefronts when the kernel routes)
     hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(logits ? 1024 : 256), 0, s, logits, router_bias, policy, weights, experts, slots, k, n_experts, tg, tu, td,
                        gu_w_stride, gu_s_stride,
-                       dn_w_stride, dn_s_stride, hidden, inter, fused ? 1u : 0u, group, g_grid, d_grid, gu_table, gu_hdr, dn_table, dn_hdr);
+                       dn_w_stride, dn_s_stride, hidden, inter, fused ? 1u : 0u, group, g_grid, d_grid, gu_table, gu_hdr, dn_table, dn_hdr, gu_first, dn_first);
     return hipGetLastError();
 }
 
