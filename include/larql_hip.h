@@ -383,6 +383,15 @@ int larql_hip_dev_gate_walk(larql_hip_ctx *ctx, int format, const void *const *g
  * 16-byte aligned. */
 int larql_hip_dev_q4k_gemm(larql_hip_ctx *ctx, const uint8_t *w, const uint16_t *x_bf16, size_t rows, size_t hidden,
                            size_t seq, float *out);
+/* The same GEMM for a matrix whose rows' exponents E were computed once (they depend on the weights alone:
+ * max(|d|, |dmin|/16) 2^E in [0.5, 1) over the row's super-blocks): larql_hip_dev_q4k_row_exponents fills
+ * row_exp[rows] (int32, device memory), larql_hip_dev_q4k_gemm_prepared takes them and skips the pass over the
+ * matrix's block headers that larql_hip_dev_q4k_gemm makes on every call.  Results are bit-identical to
+ * larql_hip_dev_q4k_gemm.  (No counterpart in the reference: its q4k_matmul dequantises on the fly, matmul.rs:20-139;
+ * this is the load-time half of the device-tier call.) */
+int larql_hip_dev_q4k_row_exponents(larql_hip_ctx *ctx, const uint8_t *w, size_t rows, size_t hidden, int32_t *row_exp);
+int larql_hip_dev_q4k_gemm_prepared(larql_hip_ctx *ctx, const uint8_t *w, const int32_t *row_exp, const uint16_t *x_bf16,
+                                    size_t rows, size_t hidden, size_t seq, float *out);
 
 /* ---- device tier: MoE expert block (MXFP4) --------------------------------------
  * router::select — larql-compute/src/ffn/expert_weight/router.rs:33-70: top-k

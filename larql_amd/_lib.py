@@ -105,6 +105,8 @@ SIGNATURES = {
     "larql_hip_dev_gate_knn_static": (ci, [vp, ci, vp, vp, sz, sz, sz, sz, vp, vp, vp]),
     "larql_hip_dev_gate_walk": (ci, [vp, ci, C.POINTER(vp), sz, vp, sz, sz, sz, sz, sz, vp, vp, vp, vp]),
     "larql_hip_dev_q4k_gemm": (ci, [vp, vp, vp, sz, sz, sz, vp]),
+    "larql_hip_dev_q4k_row_exponents": (ci, [vp, vp, sz, sz, vp]),
+    "larql_hip_dev_q4k_gemm_prepared": (ci, [vp, vp, vp, vp, sz, sz, sz, vp]),
     "larql_hip_dev_router_select": (ci, [vp, vp, sz, sz, sz, ci, vp, vp]),
     "larql_hip_moe_mxfp4_workspace_bytes": (sz, [sz, sz, sz, sz]),
     "larql_hip_dev_moe_mxfp4": (ci, [vp, C.POINTER(Mxfp4Experts), vp, sz, sz, vp, vp, vp, vp, sz]),

@@ -460,6 +460,14 @@ class HipBackend:
     def dev_q4k_gemm(self, w: int, x_bf16: int, rows: int, hidden: int, seq: int, out: int) -> bool:
         return self._some(lib.larql_hip_dev_q4k_gemm(self._h, w, x_bf16, rows, hidden, seq, out))
 
+    def dev_q4k_row_exponents(self, w: int, rows: int, hidden: int, row_exp: int) -> bool:
+        """The rows' exponents of a resident Q4_K matrix (int32[rows], device memory): once per matrix."""
+        return self._some(lib.larql_hip_dev_q4k_row_exponents(self._h, w, rows, hidden, row_exp))
+
+    def dev_q4k_gemm_prepared(self, w: int, row_exp: int, x_bf16: int, rows: int, hidden: int, seq: int, out: int) -> bool:
+        """dev_q4k_gemm with the rows' exponents from dev_q4k_row_exponents (bit-identical results)."""
+        return self._some(lib.larql_hip_dev_q4k_gemm_prepared(self._h, w, row_exp, x_bf16, rows, hidden, seq, out))
+
     def dev_router_select(self, logits: int, tokens: int, n_experts: int, k: int, policy: int, experts: int, weights: int) -> bool:
         return self._some(lib.larql_hip_dev_router_select(self._h, logits, tokens, n_experts, k, policy, experts, weights))
 

@@ -1477,10 +1477,9 @@ int larql_hip_dev_copy(larql_hip_ctx *c, void *dst, const void *src, size_t byte
     return LARQL_OK;
 }
 
-int larql_hip_dev_q4k_gemm(larql_hip_ctx *c, const uint8_t *w, const uint16_t *x_bf16, size_t rows, size_t hidden, size_t seq,
-                           float *out) {
-    if (!c) return LARQL_E_ARG;
-    std::lock_guard<std::mutex> lk(c->mu);
+// The GEMM with the rows' exponents either given (row_exp: computed once per matrix) or computed on the way.
+static int dev_q4k_gemm(larql_hip_ctx *c, const uint8_t *w, const int32_t *row_exp, const uint16_t *x_bf16, size_t rows, size_t hidden,
+                        size_t seq, float *out) {
     if (rows == 0 || seq == 0 || hidden == 0) return LARQL_OK;
     if (hidden % 256 != 0) return fail(c, LARQL_REFUSED_SHAPE, "q4k_gemm: hidden not a multiple of 256");
     if (rows > 0xFFFFFFFFull || seq > 0xFFFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "q4k_gemm: too large");
@@ -1492,12 +1491,42 @@ int larql_hip_dev_q4k_gemm(larql_hip_ctx *c, const uint8_t *w, const uint16_t *x
     if (rc) return rc;
     uint16_t *xh = (uint16_t *)c->misc.p, *sx = xh + x_len;
     float *ts = (float *)(((uintptr_t)(sx + sx_len) + 15) & ~(uintptr_t)15);
-    int *rexp = (int *)(ts + seq);  // the rows' exponents: the rows' scales ride in the f16 weight operand (1.4e-4 of the CPU value)
-    HIPCHECK(c, q4k_gemm_prep_launch(c->stream, x_bf16, 1, (uint32_t)hidden, (uint32_t)seq, xh, nullptr, sx, ts, nullptr, w, (uint32_t)rows, rexp));
+    // the rows' exponents: the rows' scales ride in the f16 weight operand (1.4e-4 of the CPU value)
+    int *rexp = row_exp ? const_cast<int *>((const int *)row_exp) : (int *)(ts + seq);
+    HIPCHECK(c, q4k_gemm_prep_launch(c->stream, x_bf16, 1, (uint32_t)hidden, (uint32_t)seq, xh, nullptr, sx, ts, nullptr, row_exp ? nullptr : w,
+                                     (uint32_t)rows, row_exp ? nullptr : rexp));
     const uint32_t splits = q4k_gemm_splits((uint32_t)rows, (uint32_t)hidden, (uint32_t)seq, (uint32_t)c->cu_count);
     float *partial = nullptr;
     if (splits > 1) { rc = ensure(c, c->scores, (size_t)splits * seq * rows * 4 + 64); if (rc) return rc; partial = (float *)c->scores.p; }
     HIPCHECK(c, q4k_gemm_f16_launch(c->stream, w, xh, sx, rexp, ts, out, (uint32_t)rows, (uint32_t)hidden, (uint32_t)seq, 1, 0, splits, partial));
+    return LARQL_OK;
+}
+
+int larql_hip_dev_q4k_gemm(larql_hip_ctx *c, const uint8_t *w, const uint16_t *x_bf16, size_t rows, size_t hidden, size_t seq,
+                           float *out) {
+    if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    return dev_q4k_gemm(c, w, nullptr, x_bf16, rows, hidden, seq, out);
+}
+
+int larql_hip_dev_q4k_gemm_prepared(larql_hip_ctx *c, const uint8_t *w, const int32_t *row_exp, const uint16_t *x_bf16, size_t rows,
+                                    size_t hidden, size_t seq, float *out) {
+    if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (!row_exp && rows && seq && hidden) return LARQL_E_ARG;
+    return dev_q4k_gemm(c, w, row_exp, x_bf16, rows, hidden, seq, out);
+}
+
+int larql_hip_dev_q4k_row_exponents(larql_hip_ctx *c, const uint8_t *w, size_t rows, size_t hidden, int32_t *row_exp) {
+    if (!c) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (rows == 0 || hidden == 0) return LARQL_OK;
+    if (hidden % 256 != 0) return fail(c, LARQL_REFUSED_SHAPE, "q4k_row_exponents: hidden not a multiple of 256");
+    if (rows > 0xFFFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "q4k_row_exponents: too large");
+    if (!w || !row_exp || ((uintptr_t)w & 15)) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    HIPCHECK(c, q4k_gemm_prep_launch(c->stream, nullptr, 1, (uint32_t)hidden, 0, nullptr, nullptr, nullptr, nullptr, nullptr, w, (uint32_t)rows,
+                                     (int *)row_exp));
     return LARQL_OK;
 }
 

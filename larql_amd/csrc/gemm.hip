@@ -918,7 +918,7 @@ __global__ void __launch_bounds__(QTHREADS) q4k_gemm_pair_kernel(const uint8_t *
 // activations -> f16 terms, sub-block sums and token scales; with `rexp`, the weight rows' exponents as well
 hipError_t q4k_gemm_prep_launch(hipStream_t s, const void *x, int x_is_bf16, uint32_t hidden, uint32_t seq, uint16_t *xh, uint16_t *xl,
                                 uint16_t *sx, float *tok_scale, int *any_lo, const uint8_t *w, uint32_t rows, int *rexp) {
-    if (seq == 0) return hipSuccess;
+    if (seq == 0 && !(rexp && rows)) return hipSuccess;  // (no tokens: only the rows' exponents, if they are asked for)
     // a token per block; wide activations take more threads per token (two passes over the token: 256 threads on 15360
     // elements are 15 dependent rounds of loads)
     const uint32_t threads = hidden >= 8192 ? 1024u : 256u;

@@ -1164,6 +1164,19 @@ def test_q4k_gemm_mfma_matches_oracle(be, rows, hidden, seq):
     assert rel_l2(got, want) < 5e-4          # stated bar 1e-3; f16 roundings of the sub-block scales and weights give ~3e-4
     # every output element (guards tile-edge and layout mistakes)
     assert np.max(np.abs(got - want)) < 2e-3 * (np.abs(want).mean() + 1e-9)
+    # the rows' exponents computed once per matrix, then handed in: the same bits
+    rexp, do2 = be.malloc(rows * 4 + 64), be.malloc(seq * rows * 4)
+    assert be.dev_q4k_row_exponents(dw, rows, hidden, rexp)
+    assert be.dev_q4k_gemm_prepared(dw, rexp, dx, rows, hidden, seq, do2)
+    be.synchronize()
+    assert np.array_equal(be.d2h(do2, (seq, rows), F).view(np.uint32), got.view(np.uint32))
+    e = be.d2h(rexp, rows, np.int32)
+    hdr = q.reshape(rows, hidden // 256, 144)[:, :, :4].copy().view(np.float16).astype(np.float64)   # d, dmin per super-block
+    m = np.maximum(np.abs(hdr[:, :, 0]), np.abs(hdr[:, :, 1]) / 16.0).max(axis=1)
+    ok = m > 0
+    assert np.all((m[ok] * np.exp2(e[ok].astype(np.float64)) >= 0.5) & (m[ok] * np.exp2(e[ok].astype(np.float64)) < 1.0))
+    with pytest.raises(Exception):                                               # the exponents are not optional here
+        be.dev_q4k_gemm_prepared(dw, 0, dx, rows, hidden, seq, do2)
 
 
 def test_q4k_gemm_row_scales_of_any_size_and_uneven_blocks(be):
