@@ -1415,7 +1415,7 @@ __device__ __forceinline__ f32x4 mx4_step_mfma(const BfOp (&a)[4], const u32x4 q
 
 // tiles [tile_a, tile_b) of one job
 __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, const Mx4Sel &sel, uint32_t tile_a, uint32_t tile_b, uint8_t *lds,
-                                               uint32_t slot_bytes, uint32_t &parity) {
+                                               uint32_t slot_bytes, uint32_t &parity, bool fresh) {
     constexpr int NS = kMx4Stages, R = kMx4BatchTiles;
     const uint32_t lane = threadIdx.x & 63u, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t nw_launch = blockDim.x >> 6;
@@ -1485,8 +1485,9 @@ __device__ __forceinline__ void run_mxfp4_mfma(const GemvJob &j, const Mx4Sel &s
     if (working) mx4_setup_ops(j, xin, ops, cw, lane, ring + (NS - 1) * slot_bytes);  // (768 bytes per step fit the 1024 of a slot's step)
 
     // The two partial-sum areas are laid out for this job's own `hw`; the job this workgroup served before may have used
-    // another layout, and its last row sums may still be read by a slower wavefront: wait for everybody before writing.
-    __builtin_amdgcn_s_barrier();
+    // another layout, and its last row sums may still be read by a slower wavefront: wait for everybody before writing
+    // (`fresh`: the workgroup's first job of the launch has nobody to wait for).
+    if (!fresh) __builtin_amdgcn_s_barrier();
     uint32_t n_use = 0;
     for (uint32_t tb = 0; tb < nt; tb += R) {
         float *pb = part + parity * (R * 16 * nw_launch * hw);
@@ -2964,6 +2965,7 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) gemv_mxfp4_mfma_kernel(Gemv
     const uint32_t p_end = (uint32_t)(P * (blockIdx.x + 1) / gridDim.x);
     const uint32_t lo = first_job_of_share(L, jobs, n_jobs, p);
     uint32_t ji = lo, parity = 0;
+    bool fresh = true;  // no job of this launch has used the workgroup's LDS yet
     while (p < p_end) {
         GemvJob j = uniform_job(jobs + ji);
         Mx4Sel S;
@@ -3011,7 +3013,8 @@ __global__ void __launch_bounds__(kMx4MaxWaves * 64) gemv_mxfp4_mfma_kernel(Gemv
         const uint32_t tile_a = a > su ? (a - su + cpt - 1) / cpt : 0, tile_b = b > su ? (b - su + cpt - 1) / cpt : 0;
         if (tile_a < tile_b) {
             if (j.combine_w) run_mxfp4_fold(j, S, tile_a, tile_b, mx4_lds, L.pad, parity);
-            else run_mxfp4_mfma(j, S, tile_a, tile_b, mx4_lds, L.pad, parity);
+            else run_mxfp4_mfma(j, S, tile_a, tile_b, mx4_lds, L.pad, parity, fresh);
+            fresh = false;
         }
         p = seg_end;
         ji++;
