@@ -99,30 +99,47 @@ class Stack:
         self.be.plan_run(self.plan_q8)
 
 
+def _window(rows, idx, n=48):
+    """First row of an n-row window of result number idx: the first rows, the last rows, or somewhere inside."""
+    return (0, rows - n, ((rows * ((idx * 37) % 97)) // 97) & ~15, (rows // 2 + 8 * idx) % (rows - n))[idx % 4]
+
+
 def verify_and_cpu_baseline(be, stack, lm_rows=16384, min_seconds=10.0):
-    """Check the GPU outputs of a sample (layer 0 + the first lm_head rows) against the CPU
-    oracle, then time the oracle (the reference's CPU algorithm restated, row-chunk
-    threaded as the reference schedules it) on the same sample."""
+    """Check the GPU outputs against the CPU oracle before any time is recorded: every row of layer 0's seven
+    matvecs, a 48-row window of EVERY other Q4_K result of the launch (all layers, all seven matrices; windows at the
+    first rows, the last rows and inside), and three lm_head windows (first, middle and last rows).  Then time the
+    oracle (the reference's CPU algorithm restated, row-chunk threaded as the reference schedules it) on layer 0 +
+    the first lm_head rows."""
     O = _oracle()
     threads = cpu_threads()
     sample, worst = [], 0.0
+
+    def rel(got, want):
+        return float(np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want))
     for (f, w, _, x, out, rows, k), (name, kind, _, _) in zip(stack.q4k_jobs[:7], stack.meta[:7]):
         wb = be.d2h(w, q4k_bytes(rows, k), np.uint8)
         xv = be.d2h(x, k, np.float32)
-        got = be.d2h(out, rows, np.float32)
-        want = O.q4k_matvec_mt(wb, xv, rows, k, threads)
-        worst = max(worst, float(np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want)))
+        worst = max(worst, rel(be.d2h(out, rows, np.float32), O.q4k_matvec_mt(wb, xv, rows, k, threads)))
         sample.append(("q4k", wb, xv, rows, k))
+    windows = 7
+    for idx, (f, w, _, x, out, rows, k) in enumerate(stack.q4k_jobs[7:], start=7):
+        r0 = _window(rows, idx)
+        wb = be.d2h(w + r0 * (k // 256) * 144, q4k_bytes(48, k), np.uint8)
+        worst = max(worst, rel(be.d2h(out + 4 * r0, 48, np.float32), O.q4k_matvec(wb, be.d2h(x, k, np.float32), 48, k)))
+        windows += 1
     (f, w, _, x, out, rows, k) = stack.q8_jobs[0]
     lm_rows = min(lm_rows, rows)
-    wb = be.d2h(w, q8_0_bytes(lm_rows, k), np.uint8)
     xv = be.d2h(x, k, np.float32)
-    got = be.d2h(out, lm_rows, np.float32)
-    want = O.q8_0_gemv_mt(wb, xv, lm_rows, k, threads)
-    worst = max(worst, float(np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want)))
-    sample.append(("q8", wb, xv, lm_rows, k))
+    for r0, n in ((0, lm_rows), (rows // 2 - 1000, 2048), (rows - 2048, 2048)):
+        if r0 < 0 or r0 + n > rows or (r0 and r0 < lm_rows):
+            continue
+        wb = be.d2h(w + r0 * (k // 32) * 34, q8_0_bytes(n, k), np.uint8)
+        worst = max(worst, rel(be.d2h(out + 4 * r0, n, np.float32), O.q8_0_gemv_mt(wb, xv, n, k, threads)))
+        if r0 == 0:
+            sample.append(("q8", wb, xv, n, k))
     if not worst < 1e-3:
         raise SystemExit(f"bench: GPU outputs differ from the CPU oracle (rel-L2 {worst:.3e}); no number recorded")
+    stack.verified = f"{windows} of {len(stack.q4k_jobs)} Q4_K results (layer 0 in full, a 48-row window of every other) + 3 lm_head windows"
 
     sample_bytes = sum(s[1].nbytes for s in sample)
 
@@ -157,12 +174,11 @@ class Chain:
     token and their dependencies, nothing else), then the lm_head on the last layer's output."""
 
     def __init__(self, be, fmt, stack, graph=True):
-        self.be, self.plans = be, []
+        self.be, self.plans, self.jobs = be, [], []
         layers = len(stack.q4k_jobs) // 7
         self.h0 = be.malloc(HIDDEN * 4 + 64)
         assert be.dev_fill_normal(self.h0, HIDDEN, 0x5EED02C0, 1.0)
         h = self.h0
-        self.first = None
         for l in range(layers):
             w = [j[1] for j in stack.q4k_jobs[7 * l:7 * l + 7]]
             buf = {n: be.malloc(r * 4 + 64) for n, r in (("q", 2048), ("k", 1024), ("v", 1024), ("o", 2560), ("gate", 10240), ("up", 10240), ("down", 2560))}
@@ -175,13 +191,13 @@ class Chain:
                 p = be.plan_create(st)
                 assert p, be.last_error()
                 self.plans.append(p)
-            if l == 0:
-                self.first = (w, buf)
+                self.jobs.extend(st)
             h = buf["down"]
         f, w, _, _, out, rows, k = stack.q8_jobs[0]
         p = be.plan_create([(f, w, None, h, out, rows, k)])
         assert p, be.last_error()
         self.plans.append(p)
+        self.lm_head = (w, h, out, rows, k)
 
         self.seq = None
         if graph:
@@ -200,15 +216,31 @@ class Chain:
             self.be.plan_run(p)
 
     def verify(self, O):
-        """Layer 0's chain against the oracle: h0 -> q -> o -> gate -> down."""
+        """Every stage of the walk against the oracle, each on the activation the GPU itself read (the stage before
+        it wrote it): layer 0's chain in full from h0 (h0 -> q -> o -> gate -> down), then a 48-row window of every
+        one of the walk's Q4_K results through the last layer, then three windows of the lm_head on the last layer's
+        output.  By induction over the stages the whole token is held to the oracle."""
         be = self.be
-        w, buf = self.first
+        threads = cpu_threads()
+
+        def rel(got, want):
+            return float(np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want))
         x = be.d2h(self.h0, HIDDEN, np.float32)
         worst = 0.0
-        for wi, name, rows, k in ((0, "q", 2048, 2560), (3, "o", 2560, 2048), (4, "gate", 10240, 2560), (6, "down", 2560, 10240)):
-            x = O.q4k_matvec_mt(be.d2h(w[wi], q4k_bytes(rows, k), np.uint8), x, rows, k, cpu_threads())
-            got = be.d2h(buf[name], rows, np.float32)
-            worst = max(worst, float(np.linalg.norm(got.astype(np.float64) - x) / np.linalg.norm(x)))
+        for ji in (0, 3, 4, 6):                                     # q, o, gate, down of layer 0, chained on the CPU
+            _, w, _, _, out, rows, k = self.jobs[ji]
+            x = O.q4k_matvec_mt(be.d2h(w, q4k_bytes(rows, k), np.uint8), x, rows, k, threads)
+            worst = max(worst, rel(be.d2h(out, rows, np.float32), x))
+        for idx, (_, w, _, xin, out, rows, k) in enumerate(self.jobs):
+            r0 = _window(rows, idx)
+            wb = be.d2h(w + r0 * (k // 256) * 144, q4k_bytes(48, k), np.uint8)
+            want = O.q4k_matvec(wb, be.d2h(xin, k, np.float32), 48, k)
+            worst = max(worst, rel(be.d2h(out + 4 * r0, 48, np.float32), want))
+        w, xin, out, rows, k = self.lm_head
+        xv = be.d2h(xin, k, np.float32)
+        for r0 in (0, rows // 2 - 1000, rows - 2048):
+            wb = be.d2h(w + r0 * (k // 32) * 34, q8_0_bytes(2048, k), np.uint8)
+            worst = max(worst, rel(be.d2h(out + 4 * r0, 2048, np.float32), O.q8_0_gemv_mt(wb, xv, 2048, k, threads)))
         return worst
 
 
@@ -352,17 +384,23 @@ def run_c3(be, fmt, args):
 
             def cpu_one():
                 for b in range(batch):
-                    sc = (O.bf16_gemv(gb.view(np.uint16), xv[b], n, hidden) if variant == "bf16" else O.q4k_matvec_mt(gb, xv[b], n, hidden, threads))
+                    sc = (O.bf16_gemv_mt(gb.view(np.uint16), xv[b], n, hidden, threads) if variant == "bf16"
+                          else O.q4k_matvec_mt(gb, xv[b], n, hidden, threads))
                     O.top_k_by_abs(sc, k)
+
+            def cpu_one_thread():  # one position, one thread
+                sc = (O.bf16_gemv_mt(gb.view(np.uint16), xv[0], n, hidden, 1) if variant == "bf16" else O.q4k_matvec_mt(gb, xv[0], n, hidden, 1))
+                O.top_k_by_abs(sc, k)
             med, nrep = _cpu_time(cpu_one, args.cpu_seconds / 4)
+            med1, _ = _cpu_time(cpu_one_thread, args.cpu_seconds / 8)
             _emit(f"gate-KNN top-64 us/layer ({variant} gate 10240x2560, batch {batch})", round(ms * 1e3, 2), "us/layer", ms * layers,
                   max(3, args.steps // 5), 2,
                   {"workload": f"BASELINE configs[2]: vindex gate-KNN walk, {variant} gate, K=64, 34 layers, batch {batch}",
                    "launches_per_walk": 2, "GBps_weights_once": round(algo / ms / 1e6, 1), "topk_identical_up_to_ties": True},
                   {"kernel": f"gemv_{variant} + topk", "bound": "hbm", "achieved": round(algo / ms / 1e6, 1), "peak": HBM_PEAK_GBS,
                    "unit": "GB/s", "frac": round(algo / ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": None},
-                  {"value": round(med * 1e6, 1), "unit": "us/layer", "cores": threads if variant == "q4k" else 1, "kind": "port",
-                   "sample": f"one layer, batch {batch}, median of {nrep}"}, higher=False)
+                  {"value": round(med * 1e6, 1), "unit": "us/layer", "cores": threads, "kind": "port",
+                   "sample": f"one layer, batch {batch}, median of {nrep}", "one_thread_us_per_position": round(med1 * 1e6, 1)}, higher=False)
             for p in (x, scores, idx, val):
                 be.free(p)
         for g in gates:
@@ -736,7 +774,7 @@ def main():
             "algorithmic_bytes_per_step": algo_bytes, "independent_steps_per_s": round(1e3 / ms_per_step, 1),
             "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
             "q8_0_lm_head": {"ms": round(q8_ms, 4), "GB/s": round(stack.q8_algo_bytes / (q8_ms * 1e-3) / 1e9, 1)},
-            "verified_rel_l2_vs_oracle": worst, "pre_warm_s": args.pre_warm_s,
+            "verified_rel_l2_vs_oracle": worst, "verified": getattr(stack, "verified", None), "pre_warm_s": args.pre_warm_s,
             "dependency_ordered": dependency, "host_tier_us_per_call": host_tier, "other_configs": others,
         },
         "roofline": {"kernel": "gemv_q4k (238 Q4_K matvecs, one launch)", "bound": "hbm", "achieved": round(achieved, 1),
@@ -775,7 +813,7 @@ def dependency_ordered_arm(be, fmt, stack, args):
             "pct_of_hbm_peak": round(100.0 * algo / max(ms, wall_ms) / 1e6 / HBM_PEAK_GBS, 2), "steps": steps,
             "one_host_call_per_stage": {"ms_per_token_device": round(eager_ms, 4), "ms_per_token_wall": round(eager_wall, 4),
                                         "tokens_per_s": round(1e3 / max(eager_ms, eager_wall), 1)},
-            "verified_rel_l2_vs_oracle_layer0": rel,
+            "verified_rel_l2_vs_oracle": rel, "verified": f"every one of the {len(chain.jobs)} Q4_K results of the walk (48-row windows, on the activation the GPU read) + layer 0 chained on the CPU + 3 lm_head windows",
             "note": "matvec launches and their dependencies only (q,k,v | o | gate,up | down per layer, then lm_head); "
                     "device = HIP events around the token, wall = host clock incl. launch overhead"}
 

@@ -1321,7 +1321,7 @@ int lq_moe_block_mxfp4(const float *x, size_t tokens, size_t hidden, size_t inte
 /* ------------------------------------------- multi-threaded CPU baseline */
 
 typedef struct {
-    int kind; /* 0 q4k matvec, 1 q8_0 gemv, 2 mxfp4 gemv, 3 q4k matmul */
+    int kind; /* 0 q4k matvec, 1 q8_0 gemv, 2 mxfp4 gemv, 3 q4k matmul, 4 bf16 gemv */
     float *out; const float *x; const uint8_t *w; const float *sum_x;
     size_t rows, blocks_per_row; int tid, nthreads;
     const uint8_t *aux; size_t seq; float *tmp; /* mxfp4 scales; matmul positions and its [rows, seq] scratch */
@@ -1337,6 +1337,9 @@ static void *mt_worker(void *p) {
         else if (j->kind == 2) {
             moe_matrix m = {1, NULL, j->w, j->aux};
             for (size_t r = r0; r < r1; r++) j->out[r] = moe_row_dot(&m, r, j->blocks_per_row * 32, j->x);
+        } else if (j->kind == 4) {
+            size_t k = j->blocks_per_row;
+            lq_bf16_gemv((const uint16_t *)j->w + r0 * k, j->x, r1 - r0, k, j->out + r0);
         } else { /* the row loop of lq_q4k_matmul_into for rows r0..r1 */
             float wf[256];
             size_t n_blocks = j->blocks_per_row, row_bytes = n_blocks * 144, hidden = n_blocks * 256;
@@ -1366,6 +1369,13 @@ static void mt_run(mt_job proto, int threads) {
 int lq_mxfp4_gemv_mt(const uint8_t *packed, const uint8_t *scales, const float *x, size_t n, size_t k, float *out, int threads) {
     if (k % 32 != 0) return 1;
     mt_job j = {2, out, x, packed, NULL, n, k / 32, 0, 1, scales, 0, NULL};
+    mt_run(j, threads);
+    return 0;
+}
+
+/* lq_bf16_gemv with its rows shared out in chunks of 32 (timing baseline; same bits per row) */
+int lq_bf16_gemv_mt(const uint16_t *w, const float *x, size_t n, size_t k, float *out, int threads) {
+    mt_job j = {4, out, x, (const uint8_t *)w, NULL, n, k, 0, 1, NULL, 0, NULL};
     mt_run(j, threads);
     return 0;
 }

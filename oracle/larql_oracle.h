@@ -128,6 +128,7 @@ int lq_moe_block_mxfp4(const float *x, size_t tokens, size_t hidden, size_t inte
  * them); per-row arithmetic is identical to the serial functions. */
 int lq_q4k_matvec_into_mt(float *out, const float *x, const uint8_t *w, size_t w_len,
                           size_t rows, size_t cols, int threads);
+int lq_bf16_gemv_mt(const uint16_t *w, const float *x, size_t n, size_t k, float *out, int threads);
 int lq_mxfp4_gemv_mt(const uint8_t *packed, const uint8_t *scales, const float *x, size_t n, size_t k, float *out, int threads);
 int lq_q4k_matmul_into_mt(float *out, const float *x, const uint8_t *w, size_t w_len, size_t rows, size_t hidden, size_t seq, int threads);
 int lq_q8_0_gemv_mt(const uint8_t *blocks, size_t blocks_len, const float *x,

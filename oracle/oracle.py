@@ -389,6 +389,15 @@ def bf16_gemv(w_bits, x, n: int, k: int) -> np.ndarray:
     return out
 
 
+def bf16_gemv_mt(w_bits, x, n: int, k: int, threads: int) -> np.ndarray:
+    """bf16_gemv with the rows shared out in chunks of 32 over `threads` threads (timing baseline; same bits)."""
+    w = np.ascontiguousarray(w_bits, dtype=np.uint16).ravel()
+    x = _f32(x).ravel()
+    out = np.empty(n, dtype=np.float32)
+    _tlib.lq_bf16_gemv_mt(_p(w, _u16p), _p(x, _f32p), _sz(n), _sz(k), _p(out, _f32p), C.c_int(threads))
+    return out
+
+
 def f16_gemv(w_bits, x, n: int, k: int) -> np.ndarray:
     w = np.ascontiguousarray(w_bits, dtype=np.uint16).ravel()
     x = _f32(x).ravel()

@@ -12,20 +12,6 @@ pytestmark = pytest.mark.gpu
 F = np.float32
 
 
-@pytest.fixture(scope="module")
-def be():
-    import larql_amd
-    b = larql_amd.HipBackend()
-    yield b
-    b.close()
-
-
-@pytest.fixture(scope="module")
-def fmt():
-    import larql_amd
-    return larql_amd
-
-
 def rel_l2(a, b):
     a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
     return np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30)
@@ -118,6 +104,76 @@ def test_decode_stack_plan_is_deterministic_order_independent_and_linear(be, fmt
     for n in outs:
         for o in outs[n]:
             be.free(o)
+
+
+def sample_window(rows, idx):
+    """A 48-row window of matrix number idx: the first rows, the last rows, or somewhere inside (aligned to the 16-row tiles or not)."""
+    return (0, rows - 48, ((rows * ((idx * 37) % 97)) // 97) & ~15, (rows // 2 + 8 * idx) % (rows - 48))[idx % 4]
+
+
+def test_decode_stack_34_layers_238_jobs_in_one_launch_every_matrix_sampled(be, fmt):
+    """configs[1] as the benchmark times it: all 34 layers x 7 Q4_K matvecs (1.8 GB of weights) recorded as ONE launch.
+    The share-out of a launch depends on its job list, so the 238-job launch gets its own checks: a 48-row window of
+    EVERY one of the 238 results against the oracle (windows at the first rows, the last rows and inside), bit-equal
+    repeats, bit-equal results with the jobs recorded in reverse order, and linearity over all rows."""
+    rng = np.random.default_rng(34)
+    layers = 34
+    xs = {k: rng.standard_normal(k).astype(F) for k in (2560, 2048, 10240)}
+    ys = {k: rng.standard_normal(k).astype(F) for k in xs}
+    a, b = F(0.25), F(-4.0)
+    dev = {"x": {k: be.to_device(v) for k, v in xs.items()}, "y": {k: be.to_device(v) for k, v in ys.items()},
+           "z": {k: be.to_device((a * xs[k] + b * ys[k]).astype(F)) for k in xs}}
+    tmp = be.malloc(10240 * 2560 * 4)
+    mats, jobs, outs = [], {n: [] for n in dev}, {n: [] for n in dev}
+    for l in range(layers):
+        for i, (rows, k) in enumerate(LAYER):
+            w = be.malloc(q4k_bytes(rows, k) + 64)
+            assert be.dev_fill_normal(tmp, rows * k, 0x5EED2200 + 8 * l + i, 0.02) and be.dev_quantize_q4_k(tmp, rows * k, w)
+            mats.append((w, rows, k))
+            for n in dev:
+                o = be.to_device(np.full(rows, np.nan, F))
+                outs[n].append(o)
+                jobs[n].append((fmt.FMT_Q4_K, w, None, dev[n][k], o, rows, k))
+    assert len(mats) == 238
+    plans = {n: be.plan_create(j) for n, j in jobs.items()}
+    assert all(p is not None for p in plans.values()) and be.plan_launch_count(plans["x"]) == 1
+    for p in plans.values():
+        assert be.plan_run(p)
+    be.synchronize()
+    res = {n: [be.d2h(o, m[1], F) for o, m in zip(outs[n], mats)] for n in outs}
+    assert all(np.isfinite(r).all() for r in res["x"])
+    # every one of the 238 matvecs: a window of rows against the oracle
+    worst = 0.0
+    for idx, (w, rows, k) in enumerate(mats):
+        r0 = sample_window(rows, idx)
+        wb = be.d2h(w + r0 * (k // 256) * 144, 48 * (k // 256) * 144, np.uint8)
+        worst = max(worst, rel_l2(res["x"][idx][r0:r0 + 48], O.q4k_matvec(wb, xs[k], 48, k)))
+    assert worst < 2e-5, worst
+    # determinism
+    assert be.plan_run(plans["x"])
+    be.synchronize()
+    for o, m, first in zip(outs["x"], mats, res["x"]):
+        assert np.array_equal(be.d2h(o, m[1], F).view(np.uint32), first.view(np.uint32))
+    # the same 238 jobs recorded in reverse order (another share-out of the same launch): the same bits per matrix
+    rev = be.plan_create(list(reversed(jobs["x"])))
+    for o, m in zip(outs["x"], mats):
+        be.h2d(o, np.full(m[1], np.nan, F))
+    assert be.plan_run(rev)
+    be.synchronize()
+    for o, m, first in zip(outs["x"], mats, res["x"]):
+        assert np.array_equal(be.d2h(o, m[1], F).view(np.uint32), first.view(np.uint32))
+    # and each matrix alone (a one-job launch) gives those bits too, on a sample of the stack
+    for idx in (0, 3, 6, 100, 237):
+        w, rows, k = mats[idx]
+        o = be.malloc(rows * 4)
+        assert be.dev_matvec(fmt.FMT_Q4_K, w, None, dev["x"][k], rows, k, o)
+        be.synchronize()
+        assert np.array_equal(be.d2h(o, rows, F).view(np.uint32), res["x"][idx].view(np.uint32)), idx
+    # linearity over every row of every matrix
+    for rx, ry, rz in zip(res["x"], res["y"], res["z"]):
+        assert rel_l2(rz, a * rx.astype(np.float64) + b * ry.astype(np.float64)) < 2e-5
+    for p in list(plans.values()) + [rev]:
+        be.plan_destroy(p)
 
 
 def test_lm_head_q8_0_full_vocabulary_linearity_and_sampled_rows(be, fmt):

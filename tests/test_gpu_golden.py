@@ -25,14 +25,6 @@ GOLD = os.path.join(os.path.dirname(__file__), "golden")
 
 
 @pytest.fixture(scope="module")
-def be():
-    import larql_amd
-    b = larql_amd.HipBackend()
-    yield b
-    b.close()
-
-
-@pytest.fixture(scope="module")
 def ggml_golden():
     d = json.load(open(os.path.join(GOLD, "ggml_kquant_golden.json")))
     out = {}

@@ -14,20 +14,6 @@ F = np.float32
 TOL = 2e-5
 
 
-@pytest.fixture(scope="module")
-def be():
-    import larql_amd
-    b = larql_amd.HipBackend()
-    yield b
-    b.close()
-
-
-@pytest.fixture(scope="module")
-def fmt():
-    import larql_amd
-    return larql_amd
-
-
 def rel_l2(a, b):
     a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
     return np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30)
@@ -1214,6 +1200,51 @@ def test_q4k_gemm_row_scales_of_any_size_and_uneven_blocks(be):
         n = np.linalg.norm(want_h[:, r].astype(np.float64))
         if n > 0:
             assert np.linalg.norm(got_h[:, r].astype(np.float64) - want_h[:, r]) / n < 2e-5, r
+
+
+def test_q4k_gemm_activation_ranges_token_by_token(be):
+    """The device tier's GEMM scales every token by a power of two into f16.  Tokens far from N(0, 1) — outliers a
+    thousand times the rest, all zeros, 1e-30, 1e20, a single non-zero element, alternating signs of equal size — must
+    each come out at the stated bar (1e-3 relative L2 per token against the oracle), next to ordinary tokens."""
+    rng = np.random.default_rng(101)
+    rows, hidden, seq = 272, 2048, 40
+    q = O.quantize_q4_k((rng.standard_normal((rows, hidden)) * 0.02).astype(F))
+    X = rng.standard_normal((seq, hidden)).astype(F)
+    X[1, rng.integers(0, hidden, 5)] *= F(1000.0)          # a few outliers x1000
+    X[2] = 0.0                                              # an all-zero token
+    X[3] *= F(1e-30)
+    X[4] *= F(1e20)
+    X[5] = 0.0; X[5, 777] = F(3.0)                          # one-hot
+    X[6] = F(0.5) * (1 - 2 * (np.arange(hidden) % 2))       # +-0.5: every sub-block sum is zero
+    X[7, :] = F(2.0 ** -120); X[7, 3] = F(2.0 ** -100)      # small with a 2^20 outlier
+    X[8] *= F(1e-30); X[8, 100] = F(1e8)                    # 38 orders of magnitude inside one token
+    X[9, rng.integers(0, hidden, 40)] *= F(-1000.0)
+    xb = O.f32_to_bf16(X)
+    Xb = (xb.astype(np.uint32) << 16).view(F).reshape(seq, hidden)
+    want = O.q4k_matmul(q, Xb, rows, hidden, seq)           # [seq, rows]
+    dw, dx, do = be.to_device(q), be.to_device(xb), be.malloc(seq * rows * 4)
+    assert be.dev_q4k_gemm(dw, dx, rows, hidden, seq, do)
+    be.synchronize()
+    got = be.d2h(do, (seq, rows), F)
+    assert np.isfinite(got).all()
+    assert np.array_equal(got[2], np.zeros(rows, F))
+    for t in range(seq):
+        n = np.linalg.norm(want[t].astype(np.float64))
+        if n > 0:
+            assert np.linalg.norm(got[t].astype(np.float64) - want[t]) / n < 1e-3, t
+    # an ordinary token's result does not depend on its neighbours: the same bits as in an all-ordinary batch
+    X2 = Xb.copy(); X2[:10] = Xb[10:20]
+    do2 = be.malloc(seq * rows * 4)
+    assert be.dev_q4k_gemm(dw, be.to_device(O.f32_to_bf16(X2)), rows, hidden, seq, do2)
+    be.synchronize()
+    assert np.array_equal(be.d2h(do2, (seq, rows), F)[10:].view(np.uint32), got[10:].view(np.uint32))
+    # host tier (exact integer sums, f32 activations as two f16 terms): the same tokens, unrounded
+    got_h = be.q4k_matmul(q, X, rows, hidden, seq).reshape(seq, rows)
+    want_h = O.q4k_matmul(q, X, rows, hidden, seq)
+    for t in range(seq):
+        n = np.linalg.norm(want_h[t].astype(np.float64))
+        if n > 0:
+            assert np.linalg.norm(got_h[t].astype(np.float64) - want_h[t]) / n < 1e-3, t
 
 
 def test_q4k_matmul_host_tier_uses_gemm_for_prefill_shapes(be):

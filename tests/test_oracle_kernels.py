@@ -193,6 +193,8 @@ def test_dense_gemvs_are_sequential_f32():
     wb = O.f32_to_bf16(w)
     wbf = (wb.astype(np.uint32) << 16).view(F).reshape(n, k)
     assert np.array_equal(bits(O.bf16_gemv(wb, x, n, k)), bits(seq_dot_f32(wbf, x)))
+    w2 = O.f32_to_bf16((rng.standard_normal((70, k)) * 0.02).astype(F))     # the threaded timing baseline: same bits, ragged chunks
+    assert np.array_equal(bits(O.bf16_gemv_mt(w2, x, 70, k, 3)), bits(O.bf16_gemv(w2, x, 70, k)))
     wh = w.astype(np.float16)
     assert np.array_equal(bits(O.f16_gemv(wh.view(np.uint16), x, n, k)), bits(seq_dot_f32(wh.astype(F), x)))
 

@@ -10,14 +10,6 @@ pytestmark = pytest.mark.gpu
 F = np.float32
 
 
-@pytest.fixture(scope="module")
-def be():
-    import larql_amd
-    b = larql_amd.HipBackend()
-    yield b
-    b.close()
-
-
 def encode(fmt, name, w):
     if name == "q4k":
         return fmt.FMT_Q4_K, O.quantize_q4_k(w)
