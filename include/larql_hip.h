@@ -343,8 +343,9 @@ int larql_hip_dev_gate_knn(larql_hip_ctx *ctx, int format, const void *gate,
  * flag.  The calls themselves only raise it: take it after the calls whose scores matter. */
 int larql_hip_dev_take_nan_flag(larql_hip_ctx *ctx, int *flag_out);
 
-/* larql_hip_dev_gate_knn for callers that cannot allocate (code under HIP graph capture, tight serving loops,
- * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same results as
+/* larql_hip_dev_gate_knn for callers that cannot allocate (tight serving loops, harnesses that forbid hipMalloc).
+ * It has no counterpart in the reference.  (It launches on the context's own stream like every other entry point:
+ * it is not a call to make under a caller's graph capture.)  Same results as
  * larql_hip_dev_gate_knn, bit for bit, but the score matrix, the hit counts and the quantised activation of
  * Q4_0 gates live in a fixed array in device memory that the library holds on every GPU it runs on until the
  * process ends (larql_hip_static_scratch_bytes(), about 0.7 MiB); the call itself performs no hipMalloc /
@@ -357,6 +358,10 @@ int larql_hip_dev_take_nan_flag(larql_hip_ctx *ctx, int *flag_out);
 #define LARQL_HIP_STATIC_MAX_SCORES 131072
 #define LARQL_HIP_STATIC_MAX_HIDDEN 16384
 size_t larql_hip_static_scratch_bytes(void);
+/* How often calls on this context have taken device memory, gone through a staging buffer or uploaded a job table so
+ * far (host-side bookkeeping, no GPU work): the number a caller checks before and after a call that must allocate
+ * nothing.  No counterpart in the reference. */
+int larql_hip_debug_alloc_events(larql_hip_ctx *ctx, uint64_t *out);
 int larql_hip_dev_gate_knn_static(larql_hip_ctx *ctx, int format, const void *gate, const float *x, size_t batch,
                                   size_t n_features, size_t hidden, size_t top_k, uint32_t *idx_out, float *score_out,
                                   uint32_t *count_out);
@@ -442,6 +447,58 @@ int larql_hip_dev_moe_mxfp4(larql_hip_ctx *ctx, const larql_hip_mxfp4_experts *b
 int larql_hip_dev_moe_mxfp4_routed(larql_hip_ctx *ctx, const larql_hip_mxfp4_experts *bank, const float *x, size_t tokens, size_t k,
                                    const float *router_logits, int policy, uint32_t *experts, float *weights, float *out,
                                    void *workspace, size_t workspace_bytes);
+
+/* ---- MoE layer: per-expert slices, split scale streams and the router, as MoeLayerWeights brings them ------------
+ * MoeLayerWeights — larql-compute/src/pipeline/moe.rs:469-541 — hands a layer's experts over as PER-EXPERT byte slices
+ * (experts_gate_up[e], experts_down[e]: mmap ranges layers/{L}/{e}/..., anywhere in memory) with the dequantisation
+ * scales either inside the payload (MoeExpertScales::Inline) or as per-expert e8m0 streams index-aligned with them
+ * (MoeExpertScales::Paired, moe.rs:214-238), the fused gate+up rows Interleaved or as ContiguousHalves
+ * (MoeFusedRowLayout, moe.rs:294-332), and the router's own tensors.  larql_hip_moe_layer_create makes such a layer
+ * resident: every slice is uploaded where the expert kernels want it (expert after expert in one region; the halves of
+ * a ContiguousHalves bank apart), so the caller gathers nothing.  Served: expert_data_format MXFP4 with Paired scales
+ * (what a native GPT-OSS bank is; the CPU tier refuses it, cpu/ops/moe/forward.rs:69-75) and MoeGateRule::ClampedGlu;
+ * MXFP4 with Inline scales is LARQL_REFUSED_SHAPE (the format keeps its exponents apart: there is nothing to read them
+ * from), other formats LARQL_UNSUPPORTED.  num_experts <= 64, top_k <= 8. */
+enum { LARQL_MOE_SCALES_INLINE = 0, LARQL_MOE_SCALES_PAIRED = 1 };
+enum { LARQL_MOE_ROWS_CONTIGUOUS_HALVES = 0, LARQL_MOE_ROWS_INTERLEAVED = 1 };
+typedef struct {
+    size_t num_experts, top_k, hidden, intermediate_size;
+    int expert_data_format;                      /* LARQL_FMT_* of the per-expert slices */
+    int fused_row_layout;                        /* LARQL_MOE_ROWS_* */
+    int expert_scales;                           /* LARQL_MOE_SCALES_* */
+    const uint8_t *const *experts_gate_up;       /* [num_experts]: expert e's fused [2*inter, hidden/32, 16] nibble bytes */
+    const size_t *experts_gate_up_len;
+    const uint8_t *const *experts_down;          /* [num_experts]: expert e's [hidden, inter/32, 16] nibble bytes */
+    const size_t *experts_down_len;
+    const uint8_t *const *scales_gate_up;        /* Paired: [num_experts] e8m0 streams [2*inter, hidden/32]; else NULL */
+    const size_t *scales_gate_up_len;
+    const uint8_t *const *scales_down;           /* Paired: [num_experts] e8m0 streams [hidden, inter/32]; else NULL */
+    const size_t *scales_down_len;
+    const float *router_proj;                    /* [num_experts, hidden] */
+    const float *router_bias;                    /* [num_experts], or NULL (the reference: an empty slice) */
+    const float *experts_gate_up_bias;           /* [num_experts, 2*inter] as the checkpoint ships it (interleaved), or NULL */
+    const float *experts_down_bias;              /* [num_experts, hidden], or NULL */
+    const float *router_per_expert_scale;        /* [num_experts], or NULL */
+    int renormalized_softmax;                    /* MoeTopKWeightPolicy::RenormalizedSoftmax (else the softmax's own values) */
+    int per_expert_scale;                        /* MoeExpertScalePolicy::PerExpert */
+    float glu_limit, glu_alpha;                  /* MoeGateRule::ClampedGlu (GPT-OSS: 7, 1.702) */
+} larql_hip_moe_layer_weights;
+typedef struct larql_hip_moe_layer larql_hip_moe_layer;
+int  larql_hip_moe_layer_create(larql_hip_ctx *ctx, const larql_hip_moe_layer_weights *weights, larql_hip_moe_layer **out);
+void larql_hip_moe_layer_destroy(larql_hip_ctx *ctx, larql_hip_moe_layer *layer);
+/* moe_route_from_router_input (cpu/ops/moe/mod.rs:149-186: router_proj . router_in + router_bias, softmax, top_k,
+ * renormalise, per-expert scale) followed by the expert block (cpu/ops/moe/forward.rs:201-270) on host slices:
+ * router_in and x are [tokens, hidden] (the router's and the experts' input: the reference derives both from the
+ * residual under MoeRoutingPolicy, and they may be the same slice), out is [tokens, hidden].  experts_out /
+ * weights_out ([tokens, min(top_k, num_experts)], may be NULL) receive the route.  One submission. */
+int  larql_hip_moe_layer_forward(larql_hip_ctx *ctx, larql_hip_moe_layer *layer, const float *router_in, const float *x,
+                                 size_t tokens, float *out, uint32_t *experts_out, float *weights_out);
+/* The same on resident operands; only enqueues.  The router's projection runs on the device (a [num_experts, hidden]
+ * f32 gemv per token), the selection inside the first expert launch for one token: residual -> output without a host
+ * round trip.  experts / weights: device buffers [tokens, min(top_k, num_experts)]; router_in, x and out 16-byte
+ * aligned with hidden % 4 == 0 (else LARQL_REFUSED_SHAPE). */
+int  larql_hip_dev_moe_layer_forward(larql_hip_ctx *ctx, larql_hip_moe_layer *layer, const float *router_in, const float *x,
+                                     size_t tokens, float *out, uint32_t *experts, float *weights);
 
 /* ---- device tier: encoders (bit-exact with the reference's host encoders) --- */
 /* quantize_q4_k — larql-compute/src/cpu/ops/q4_common/quantize.rs:89-189. */

@@ -18,6 +18,45 @@ pub struct Clock {
     pub gpu_nanos: u64,
 }
 
+#[repr(C)]
+pub struct MoeLayer {
+    _private: [u8; 0],
+}
+
+/// `larql_hip_moe_layer_weights`: `larql_compute::MoeLayerWeights` as plain pointers.
+#[repr(C)]
+pub struct MoeLayerWeights {
+    pub num_experts: usize,
+    pub top_k: usize,
+    pub hidden: usize,
+    pub intermediate_size: usize,
+    pub expert_data_format: c_int,
+    pub fused_row_layout: c_int,
+    pub expert_scales: c_int,
+    pub experts_gate_up: *const *const u8,
+    pub experts_gate_up_len: *const usize,
+    pub experts_down: *const *const u8,
+    pub experts_down_len: *const usize,
+    pub scales_gate_up: *const *const u8,
+    pub scales_gate_up_len: *const usize,
+    pub scales_down: *const *const u8,
+    pub scales_down_len: *const usize,
+    pub router_proj: *const f32,
+    pub router_bias: *const f32,
+    pub experts_gate_up_bias: *const f32,
+    pub experts_down_bias: *const f32,
+    pub router_per_expert_scale: *const f32,
+    pub renormalized_softmax: c_int,
+    pub per_expert_scale: c_int,
+    pub glu_limit: f32,
+    pub glu_alpha: f32,
+}
+
+pub const MOE_SCALES_INLINE: c_int = 0;
+pub const MOE_SCALES_PAIRED: c_int = 1;
+pub const MOE_ROWS_CONTIGUOUS_HALVES: c_int = 0;
+pub const MOE_ROWS_INTERLEAVED: c_int = 1;
+
 pub const OK: c_int = 0;
 
 // QuantFormat discriminants as the library numbers them (the order of larql_compute::QuantFormat)
@@ -92,6 +131,11 @@ extern "C" {
     pub fn larql_hip_gate_knn(ctx: *mut Ctx, format: c_int, gate: *const u8, gate_len: usize, x: *const f32, batch: usize,
                               n_features: usize, hidden: usize, top_k: usize, idx: *mut u32, score: *mut f32,
                               n_out: *mut usize) -> c_int;
+    pub fn larql_hip_moe_layer_create(ctx: *mut Ctx, weights: *const MoeLayerWeights, out: *mut *mut MoeLayer) -> c_int;
+    pub fn larql_hip_moe_layer_destroy(ctx: *mut Ctx, layer: *mut MoeLayer);
+    pub fn larql_hip_moe_layer_forward(ctx: *mut Ctx, layer: *mut MoeLayer, router_in: *const f32, x: *const f32, tokens: usize,
+                                       out: *mut f32, experts_out: *mut u32, weights_out: *mut f32) -> c_int;
+
     pub fn larql_hip_gate_scores(ctx: *mut Ctx, format: c_int, gate: *const u8, gate_len: usize, x: *const f32, batch: usize,
                                  n_features: usize, hidden: usize, scores: *mut f32) -> c_int;
 }

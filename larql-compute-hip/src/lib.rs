@@ -20,7 +20,8 @@ use std::os::raw::c_int;
 use std::ptr;
 
 use larql_compute::{
-    Capability, ComputeBackend, CpuBackend, DecodeBackend, MatMul, QuantFormat, QuantMatVec, SubmissionClock,
+    Capability, ComputeBackend, CpuBackend, DecodeBackend, MatMul, MoeExpertScalePolicy, MoeExpertScales, MoeFusedRowLayout,
+    MoeGateRule, MoeLayerWeights, MoeTopKWeightPolicy, QuantFormat, QuantMatVec, SubmissionClock,
 };
 use ndarray::{Array2, ArrayView2};
 
@@ -39,6 +40,44 @@ unsafe impl Sync for HipBackend {}
 /// or is not a gfx950 part, so a named `--backend hip` fails loudly instead of running on the CPU.
 pub fn hip_backend() -> Option<HipBackend> {
     HipBackend::on_device(0)
+}
+
+/// One MoE layer resident on the device (see [`HipBackend::moe_layer`]).
+pub struct HipMoeLayer<'a> {
+    backend: &'a HipBackend,
+    layer: *mut ffi::MoeLayer,
+    hidden: usize,
+    top_k: usize,
+}
+
+unsafe impl Send for HipMoeLayer<'_> {}
+unsafe impl Sync for HipMoeLayer<'_> {}
+
+impl HipMoeLayer<'_> {
+    /// `moe_route_from_router_input` + the expert block (crates/larql-compute/src/cpu/ops/moe/mod.rs:149-186,
+    /// forward.rs:201-270) for `tokens` rows: `router_in` and `x` are `[tokens, hidden]` (the router's and the experts'
+    /// input as `MoeRoutingPolicy` derives them from the residual).  Returns the block's output and the route.
+    pub fn forward(&self, router_in: &[f32], x: &[f32], tokens: usize) -> Option<(Vec<f32>, Vec<u32>, Vec<f32>)> {
+        let n = tokens.checked_mul(self.hidden)?;
+        if router_in.len() != n || x.len() != n {
+            return None;
+        }
+        let cells = tokens.checked_mul(self.top_k)?;
+        let (mut out, mut experts, mut weights) = (vec![0.0f32; n], vec![0u32; cells], vec![0.0f32; cells]);
+        // SAFETY: the buffers have the sizes the library documents: [tokens, hidden] and [tokens, min(top_k, num_experts)].
+        let rc = unsafe {
+            ffi::larql_hip_moe_layer_forward(self.backend.ctx, self.layer, router_in.as_ptr(), x.as_ptr(), tokens,
+                                             out.as_mut_ptr(), experts.as_mut_ptr(), weights.as_mut_ptr())
+        };
+        some_if_ok(rc, (out, experts, weights))
+    }
+}
+
+impl Drop for HipMoeLayer<'_> {
+    fn drop(&mut self) {
+        // SAFETY: the handle came from larql_hip_moe_layer_create on this context and is dropped once.
+        unsafe { ffi::larql_hip_moe_layer_destroy(self.backend.ctx, self.layer) }
+    }
 }
 
 fn format_code(format: QuantFormat) -> c_int {
@@ -62,6 +101,20 @@ fn some_if_ok<T>(rc: c_int, value: T) -> Option<T> {
         Some(value)
     } else {
         None
+    }
+}
+
+/// The winners the library can order per row (`kTopkMaxK`).
+const TOP_K_MAX: usize = 16384;
+
+/// A caller may pass a very large K to mean "all": K is clamped to the number of candidates BEFORE any buffer is sized
+/// from it, and a K the library does not serve answers `None` here instead of an allocation failure.
+fn clamp_top_k(top_k: usize, candidates: usize) -> Option<usize> {
+    let k = top_k.min(candidates);
+    if k > TOP_K_MAX {
+        None
+    } else {
+        Some(k)
     }
 }
 
@@ -108,6 +161,7 @@ impl HipBackend {
     /// lm_head KNN over a ggml Q8_0 head with the selection on the device
     /// (crates/larql-vindex/src/index/storage/lm_head/knn.rs:126-185, top_k_sorted :315-386).
     pub fn q8_0_gemv_topk(&self, blocks: &[u8], x: &[f32], n: usize, k: usize, top_k: usize) -> Option<Vec<(u32, f32)>> {
+        let top_k = clamp_top_k(top_k, n)?;
         let (mut idx, mut score, mut got) = (vec![0u32; top_k], vec![0.0f32; top_k], 0usize);
         // SAFETY: `idx` / `score` hold top_k entries, what the library copies back; `got` says how many are hits.
         let rc = unsafe {
@@ -122,10 +176,12 @@ impl HipBackend {
     /// `[batch, hidden]`; the result has one hit list per position.
     pub fn gate_knn(&self, format: QuantFormat, gate: &[u8], x: &[f32], batch: usize, n_features: usize, hidden: usize,
                     top_k: usize) -> Option<Vec<Vec<(u32, f32)>>> {
-        if x.len() != batch * hidden {
+        if Some(x.len()) != batch.checked_mul(hidden) {
             return None;
         }
-        let (mut idx, mut score, mut got) = (vec![0u32; batch * top_k], vec![0.0f32; batch * top_k], vec![0usize; batch]);
+        let top_k = clamp_top_k(top_k, n_features)?;
+        let cells = batch.checked_mul(top_k)?;
+        let (mut idx, mut score, mut got) = (vec![0u32; cells], vec![0.0f32; cells], vec![0usize; batch]);
         // SAFETY: the outputs are [batch, top_k] and the counts [batch], as the library documents; `x` was checked above.
         let rc = unsafe {
             ffi::larql_hip_gate_knn(self.ctx, format_code(format), gate.as_ptr(), gate.len(), x.as_ptr(), batch, n_features,
@@ -136,6 +192,69 @@ impl HipBackend {
                 .map(|b| (0..got[b].min(top_k)).map(|i| (idx[b * top_k + i], score[b * top_k + i])).collect())
                 .collect()
         })
+    }
+
+    /// A MoE layer made resident from `MoeLayerWeights` (crates/larql-compute/src/pipeline/moe.rs:469-541): the
+    /// per-expert slices and their paired exponent streams go up expert by expert, wherever their mmap ranges lie.
+    /// `None` where this backend has no kernel for the layer (anything but an MXFP4 bank with `Paired` scales and
+    /// `ClampedGlu`, more than 64 experts, top-k above 8) — the caller keeps `cpu_moe_forward`.
+    pub fn moe_layer<'a>(&'a self, moe: &MoeLayerWeights<'_>, hidden: usize) -> Option<HipMoeLayer<'a>> {
+        let (limit, alpha) = match moe.gate_rule {
+            MoeGateRule::ClampedGlu { limit, alpha } => (limit, alpha),
+            _ => return None,
+        };
+        let (sg, sd): (Vec<&[u8]>, Vec<&[u8]>) = match &moe.expert_scales {
+            MoeExpertScales::Paired { gate_up, down } => (gate_up.clone(), down.clone()),
+            MoeExpertScales::Inline => (Vec::new(), Vec::new()),
+        };
+        let n = moe.num_experts;
+        if moe.experts_gate_up.len() != n || moe.experts_down.len() != n || moe.router_proj.len() != n.checked_mul(hidden)? {
+            return None;
+        }
+        if moe.expert_scales.is_paired() && (sg.len() != n || sd.len() != n) {
+            return None;
+        }
+        let ptrs = |v: &[&[u8]]| v.iter().map(|s| s.as_ptr()).collect::<Vec<*const u8>>();
+        let lens = |v: &[&[u8]]| v.iter().map(|s| s.len()).collect::<Vec<usize>>();
+        let (gp, gl, dp, dl) = (ptrs(&moe.experts_gate_up), lens(&moe.experts_gate_up), ptrs(&moe.experts_down), lens(&moe.experts_down));
+        let (sgp, sgl, sdp, sdl) = (ptrs(&sg), lens(&sg), ptrs(&sd), lens(&sd));
+        let opt = |s: &[f32]| if s.is_empty() { ptr::null() } else { s.as_ptr() };
+        let w = ffi::MoeLayerWeights {
+            num_experts: n,
+            top_k: moe.top_k,
+            hidden,
+            intermediate_size: moe.intermediate_size,
+            expert_data_format: format_code(moe.expert_data_format),
+            fused_row_layout: match moe.fused_row_layout {
+                MoeFusedRowLayout::Interleaved => ffi::MOE_ROWS_INTERLEAVED,
+                MoeFusedRowLayout::ContiguousHalves => ffi::MOE_ROWS_CONTIGUOUS_HALVES,
+            },
+            expert_scales: if moe.expert_scales.is_paired() { ffi::MOE_SCALES_PAIRED } else { ffi::MOE_SCALES_INLINE },
+            experts_gate_up: gp.as_ptr(),
+            experts_gate_up_len: gl.as_ptr(),
+            experts_down: dp.as_ptr(),
+            experts_down_len: dl.as_ptr(),
+            scales_gate_up: if sgp.is_empty() { ptr::null() } else { sgp.as_ptr() },
+            scales_gate_up_len: if sgl.is_empty() { ptr::null() } else { sgl.as_ptr() },
+            scales_down: if sdp.is_empty() { ptr::null() } else { sdp.as_ptr() },
+            scales_down_len: if sdl.is_empty() { ptr::null() } else { sdl.as_ptr() },
+            router_proj: moe.router_proj.as_ptr(),
+            router_bias: opt(moe.router_bias),
+            experts_gate_up_bias: opt(moe.experts_gate_up_bias),
+            experts_down_bias: opt(moe.experts_down_bias),
+            router_per_expert_scale: opt(moe.router_per_expert_scale),
+            renormalized_softmax: (moe.routing_policy.selected_weight == MoeTopKWeightPolicy::RenormalizedSoftmax) as c_int,
+            per_expert_scale: (moe.routing_policy.expert_scale == MoeExpertScalePolicy::PerExpert) as c_int,
+            glu_limit: limit,
+            glu_alpha: alpha,
+        };
+        let mut layer: *mut ffi::MoeLayer = ptr::null_mut();
+        // SAFETY: every table holds `n` entries that outlive the call; the library copies the bytes before it returns.
+        let rc = unsafe { ffi::larql_hip_moe_layer_create(self.ctx, &w, &mut layer) };
+        if rc != ffi::OK || layer.is_null() {
+            return None;
+        }
+        Some(HipMoeLayer { backend: self, layer, hidden, top_k: moe.top_k.min(n) })
     }
 
     /// `gate_scores_batch_backend` (gate_knn/scores_batch.rs:30-57): the full `[batch, n_features]` score matrix.
@@ -358,6 +477,7 @@ impl QuantMatVec for HipBackend {
 
     fn q4k_matvec_topk(&self, q4k_data: &[u8], x: &[f32], num_rows: usize, hidden: usize, top_k: usize)
                        -> Option<Vec<(u32, f32)>> {
+        let top_k = clamp_top_k(top_k, num_rows)?;
         let (mut idx, mut score, mut got) = (vec![0u32; top_k], vec![0.0f32; top_k], 0usize);
         // SAFETY: `idx` / `score` hold top_k entries, what the library copies back; `got` says how many are hits.
         let rc = unsafe {

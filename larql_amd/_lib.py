@@ -33,6 +33,21 @@ class Mxfp4Experts(C.Structure):
                 ("alpha", C.c_float), ("gate_up_interleaved", C.c_int), ("router_bias", vp), ("gate_up_bias", vp), ("down_bias", vp)]
 
 
+MOE_SCALES_INLINE, MOE_SCALES_PAIRED = 0, 1
+MOE_ROWS_CONTIGUOUS_HALVES, MOE_ROWS_INTERLEAVED = 0, 1
+
+
+class MoeLayerWeights(C.Structure):
+    """larql_hip_moe_layer_weights (MoeLayerWeights, larql-compute/src/pipeline/moe.rs:469-541)."""
+    _fields_ = [("num_experts", sz), ("top_k", sz), ("hidden", sz), ("intermediate_size", sz), ("expert_data_format", ci),
+                ("fused_row_layout", ci), ("expert_scales", ci), ("experts_gate_up", C.POINTER(vp)), ("experts_gate_up_len", C.POINTER(sz)),
+                ("experts_down", C.POINTER(vp)), ("experts_down_len", C.POINTER(sz)), ("scales_gate_up", C.POINTER(vp)),
+                ("scales_gate_up_len", C.POINTER(sz)), ("scales_down", C.POINTER(vp)), ("scales_down_len", C.POINTER(sz)),
+                ("router_proj", vp), ("router_bias", vp), ("experts_gate_up_bias", vp), ("experts_down_bias", vp),
+                ("router_per_expert_scale", vp), ("renormalized_softmax", ci), ("per_expert_scale", ci), ("glu_limit", C.c_float),
+                ("glu_alpha", C.c_float)]
+
+
 class MatvecJob(C.Structure):
     _fields_ = [("format", C.c_int32), ("reserved", C.c_int32), ("w", vp), ("aux", vp), ("x", vp),
                 ("out", vp), ("rows", u64), ("k", u64)]
@@ -102,6 +117,7 @@ SIGNATURES = {
     "larql_hip_dev_gate_knn": (ci, [vp, ci, vp, vp, sz, sz, sz, sz, vp, vp, vp, vp]),
     "larql_hip_dev_take_nan_flag": (ci, [vp, C.POINTER(ci)]),
     "larql_hip_static_scratch_bytes": (sz, []),
+    "larql_hip_debug_alloc_events": (ci, [vp, C.POINTER(u64)]),
     "larql_hip_dev_gate_knn_static": (ci, [vp, ci, vp, vp, sz, sz, sz, sz, vp, vp, vp]),
     "larql_hip_dev_gate_walk": (ci, [vp, ci, C.POINTER(vp), sz, vp, sz, sz, sz, sz, sz, vp, vp, vp, vp]),
     "larql_hip_dev_q4k_gemm": (ci, [vp, vp, vp, sz, sz, sz, vp]),
@@ -111,6 +127,10 @@ SIGNATURES = {
     "larql_hip_moe_mxfp4_workspace_bytes": (sz, [sz, sz, sz, sz]),
     "larql_hip_dev_moe_mxfp4": (ci, [vp, C.POINTER(Mxfp4Experts), vp, sz, sz, vp, vp, vp, vp, sz]),
     "larql_hip_dev_moe_mxfp4_routed": (ci, [vp, C.POINTER(Mxfp4Experts), vp, sz, sz, vp, ci, vp, vp, vp, vp, sz]),
+    "larql_hip_moe_layer_create": (ci, [vp, C.POINTER(MoeLayerWeights), C.POINTER(vp)]),
+    "larql_hip_moe_layer_destroy": (None, [vp, vp]),
+    "larql_hip_moe_layer_forward": (ci, [vp, vp, vp, vp, sz, vp, vp, vp]),
+    "larql_hip_dev_moe_layer_forward": (ci, [vp, vp, vp, vp, sz, vp, vp, vp]),
     "larql_hip_dev_quantize_q4_k": (ci, [vp, vp, sz, vp]),
     "larql_hip_dev_quantize_q6_k": (ci, [vp, vp, sz, vp]),
     "larql_hip_dev_quantize_q8_0": (ci, [vp, vp, sz, vp]),

@@ -443,6 +443,12 @@ class HipBackend:
         self._some(lib.larql_hip_dev_take_nan_flag(self._h, C.byref(f)))
         return bool(f.value)
 
+    def debug_alloc_events(self) -> int:
+        """Allocations, stagings and table uploads made through this context so far (host-side counter)."""
+        v = L.u64()
+        self._some(lib.larql_hip_debug_alloc_events(self._h, C.byref(v)))
+        return v.value
+
     def static_scratch_bytes(self) -> int:
         return int(lib.larql_hip_static_scratch_bytes())
 
@@ -485,6 +491,70 @@ class HipBackend:
         written as dev_router_select writes them."""
         return self._some(lib.larql_hip_dev_moe_mxfp4_routed(self._h, C.byref(bank), x, tokens, k, logits, policy, experts, weights,
                                                              out, workspace, workspace_bytes))
+
+    # -- MoE layer: per-expert slices, split scale streams and the router (MoeLayerWeights) ----------------------
+    def moe_layer_create(self, experts_gate_up, experts_down, scales_gate_up, scales_down, router_proj, top_k: int, hidden: int,
+                         inter: int, fused_row_layout: int = L.MOE_ROWS_INTERLEAVED, router_bias=None, gate_up_bias=None,
+                         down_bias=None, per_expert_scale=None, renormalized: bool = True, expert_scales: int = L.MOE_SCALES_PAIRED,
+                         expert_data_format: int = L.FMT_MXFP4, limit: float = 7.0, alpha: float = 1.702) -> Optional[int]:
+        """experts_gate_up / experts_down / scales_*: one uint8 array per expert (separate allocations, as mmap ranges
+        would be).  Returns a layer handle, or None where the backend refuses the layer."""
+        n = len(experts_gate_up)
+        keep = []  # host arrays have to outlive the call
+
+        def table(arrs):
+            if arrs is None:
+                return None, None
+            a = [np.ascontiguousarray(x, dtype=np.uint8).ravel() for x in arrs]
+            keep.append(a)
+            ptrs = (vp_t * max(len(a), 1))(*[x.ctypes.data for x in a])
+            lens = (C.c_size_t * max(len(a), 1))(*[x.size for x in a])
+            keep.append((ptrs, lens))
+            return C.cast(ptrs, C.POINTER(vp_t)), C.cast(lens, C.POINTER(C.c_size_t))
+
+        def f32(a):
+            if a is None:
+                return None
+            a = np.ascontiguousarray(a, dtype=np.float32)
+            keep.append(a)
+            return a.ctypes.data
+        vp_t = C.c_void_p
+        w = L.MoeLayerWeights()
+        w.num_experts, w.top_k, w.hidden, w.intermediate_size = n, top_k, hidden, inter
+        w.expert_data_format, w.fused_row_layout, w.expert_scales = expert_data_format, fused_row_layout, expert_scales
+        w.experts_gate_up, w.experts_gate_up_len = table(experts_gate_up)
+        w.experts_down, w.experts_down_len = table(experts_down)
+        sg, sgl = table(scales_gate_up)
+        sd, sdl = table(scales_down)
+        if sg is not None:
+            w.scales_gate_up, w.scales_gate_up_len = sg, sgl
+        if sd is not None:
+            w.scales_down, w.scales_down_len = sd, sdl
+        w.router_proj, w.router_bias = f32(router_proj), f32(router_bias)
+        w.experts_gate_up_bias, w.experts_down_bias = f32(gate_up_bias), f32(down_bias)
+        w.router_per_expert_scale = f32(per_expert_scale)
+        w.renormalized_softmax, w.per_expert_scale = int(renormalized), int(per_expert_scale is not None)
+        w.glu_limit, w.glu_alpha = limit, alpha
+        h = C.c_void_p()
+        ok = self._some(lib.larql_hip_moe_layer_create(self._h, C.byref(w), C.byref(h)))
+        return h.value if ok else None
+
+    def moe_layer_destroy(self, layer: int) -> None:
+        lib.larql_hip_moe_layer_destroy(self._h, layer)
+
+    def moe_layer_forward(self, layer: int, router_in, x, top_k: int):
+        """Host tier: (out [tokens, hidden], experts [tokens, k], weights [tokens, k]) or None."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        rin = x if router_in is x else np.ascontiguousarray(router_in, dtype=np.float32)
+        tokens = x.shape[0]
+        out = np.empty_like(x)
+        ex, wt = np.zeros((tokens, top_k), np.uint32), np.zeros((tokens, top_k), np.float32)
+        ok = self._some(lib.larql_hip_moe_layer_forward(self._h, layer, rin.ctypes.data, x.ctypes.data, tokens, out.ctypes.data,
+                                                        ex.ctypes.data, wt.ctypes.data))
+        return (out, ex, wt) if ok else None
+
+    def dev_moe_layer_forward(self, layer: int, router_in: int, x: int, tokens: int, out: int, experts: int, weights: int) -> bool:
+        return self._some(lib.larql_hip_dev_moe_layer_forward(self._h, layer, router_in, x, tokens, out, experts, weights))
 
     def dev_quantize_q4_k(self, src: int, n: int, dst: int) -> bool:
         return self._some(lib.larql_hip_dev_quantize_q4_k(self._h, src, n, dst))

@@ -78,6 +78,9 @@ struct larql_hip_ctx {
     int *nan_flag = nullptr;       // [0]: device tier, raised by any call, cleared when taken; [1]: host tier, cleared by every call
     uint8_t *static_scratch = nullptr;  // this device's copy of `scratch` (hipGetSymbolAddress at create)
     larql_hip_submission_clock clock = {0, 0, 0};
+    // Times a call took device memory, staged a host buffer or uploaded a job table (larql_hip_debug_alloc_events):
+    // what the entry point that allocates nothing must never do.
+    uint64_t alloc_events = 0;
 };
 
 namespace {
@@ -99,6 +102,7 @@ int fail(larql_hip_ctx *c, int code, const char *fmt, ...) {
     } while (0)
 
 int ensure(larql_hip_ctx *c, DevBuf &b, size_t bytes) {
+    c->alloc_events++;  // (counted whether or not the buffer has to grow: the caller went through the staging path)
     if (bytes <= b.cap) return LARQL_OK;
     if (b.p) HIPCHECK(c, hipFree(b.p));
     b.p = nullptr; b.cap = 0;
@@ -223,6 +227,7 @@ int prepare_same_kind(larql_hip_ctx *c, GemvJob *live, size_t n_live, void *tabl
     } else {
         // the table: the jobs, then the first job of every workgroup's share (what a workgroup would otherwise find by
         // bisection over the jobs' pass ranges, a dependent load per step)
+        c->alloc_events++;
         const size_t job_bytes = n_live * sizeof(GemvJob);
         const bool with_first = grid >= 1 && grid <= (uint64_t)kTableFirstMax;
         const size_t bytes = job_bytes + (with_first ? (size_t)grid * sizeof(uint32_t) : 0);
@@ -1130,9 +1135,17 @@ int larql_hip_gate_knn(larql_hip_ctx *c, int format, const uint8_t *gate, size_t
 
 // ---- device tier ----------------------------------------------------------------------------
 
+int larql_hip_debug_alloc_events(larql_hip_ctx *c, uint64_t *out) {
+    if (!c || !out) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    *out = c->alloc_events;
+    return LARQL_OK;
+}
+
 int larql_hip_malloc(larql_hip_ctx *c, void **dptr, size_t bytes) {
     if (!c || !dptr) return LARQL_E_ARG;
     std::lock_guard<std::mutex> lk(c->mu);
+    c->alloc_events++;
     HIPCHECK(c, hipSetDevice(c->device));
     HIPCHECK(c, hipMalloc(dptr, bytes ? bytes : 1));
     return LARQL_OK;
@@ -1784,6 +1797,173 @@ int larql_hip_dev_moe_mxfp4_routed(larql_hip_ctx *c, const larql_hip_mxfp4_exper
     if (bank->n_experts > 64 || k > 8) return fail(c, LARQL_UNSUPPORTED, "router_select: at most 64 experts and top-8 on this backend");
     if (!router_logits) return LARQL_E_ARG;
     return moe_mxfp4_block(c, bank, x, tokens, k, experts, weights, out, workspace, workspace_bytes, router_logits, policy);
+}
+
+// ---- MoE layer: per-expert slices + split scales + router, made resident (MoeLayerWeights, pipeline/moe.rs:469-541) ----
+
+struct larql_hip_moe_layer {
+    void *region = nullptr;             // every tensor of the layer, resident
+    larql_hip_mxfp4_experts bank = {};  // device pointers into `region`
+    const float *router_proj = nullptr, *scale = nullptr;
+    size_t n_experts = 0, top_k = 0, hidden = 0, inter = 0;
+    int renormalized = 1, per_expert_scale = 0;
+    DevBuf ws, logits, rin, x, out, experts, weights;  // grown on demand (host tier: staging as well)
+};
+
+void larql_hip_moe_layer_destroy(larql_hip_ctx *c, larql_hip_moe_layer *L) {
+    if (!L) return;
+    if (c) { (void)hipSetDevice(c->device); (void)hipStreamSynchronize(c->stream); }
+    DevBuf *bufs[] = {&L->ws, &L->logits, &L->rin, &L->x, &L->out, &L->experts, &L->weights};
+    for (DevBuf *b : bufs) if (b->p) (void)hipFree(b->p);
+    if (L->region) (void)hipFree(L->region);
+    delete L;
+}
+
+int larql_hip_moe_layer_create(larql_hip_ctx *c, const larql_hip_moe_layer_weights *w, larql_hip_moe_layer **out) {
+    if (!c || !w || !out) return LARQL_E_ARG;
+    *out = nullptr;
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (w->expert_data_format != LARQL_FMT_MXFP4)
+        return fail(c, LARQL_UNSUPPORTED, "moe_layer: only MXFP4 expert banks are served by this backend");
+    if (w->expert_scales != LARQL_MOE_SCALES_PAIRED)
+        return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: an MXFP4 bank keeps its e8m0 exponents in a partner stream (MoeExpertScales::Paired)");
+    const size_t E = w->num_experts, hidden = w->hidden, inter = w->intermediate_size;
+    if (E == 0 || w->top_k == 0 || hidden == 0 || inter == 0) return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: empty layer");
+    if (E > 64 || std::min(w->top_k, E) > 8) return fail(c, LARQL_UNSUPPORTED, "moe_layer: at most 64 experts and top-8 on this backend");
+    if (hidden % 32 != 0 || inter % 32 != 0) return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: hidden and intermediate_size must be multiples of 32");
+    if (w->fused_row_layout != LARQL_MOE_ROWS_INTERLEAVED && w->fused_row_layout != LARQL_MOE_ROWS_CONTIGUOUS_HALVES)
+        return fail(c, LARQL_E_ARG, "moe_layer: unknown fused row layout");
+    if (!w->experts_gate_up || !w->experts_gate_up_len || !w->experts_down || !w->experts_down_len || !w->scales_gate_up ||
+        !w->scales_gate_up_len || !w->scales_down || !w->scales_down_len || !w->router_proj)
+        return LARQL_E_ARG;
+    const size_t gu_p = 2 * inter * (hidden / 32) * 16, gu_s = 2 * inter * (hidden / 32);  // per expert
+    const size_t dn_p = hidden * (inter / 32) * 16, dn_s = hidden * (inter / 32);
+    for (size_t e = 0; e < E; e++) {
+        if (!w->experts_gate_up[e] || !w->experts_down[e] || !w->scales_gate_up[e] || !w->scales_down[e]) return LARQL_E_ARG;
+        if (w->experts_gate_up_len[e] < gu_p || w->scales_gate_up_len[e] < gu_s || w->experts_down_len[e] < dn_p || w->scales_down_len[e] < dn_s)
+            return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: expert %zu's slices are shorter than its geometry", e);
+    }
+    HIPCHECK(c, hipSetDevice(c->device));
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    // region: [gate(+up) nibbles | gate(+up) exponents | down nibbles | down exponents | router_proj | router_bias |
+    //          gate_up_bias | down_bias | per-expert scale], every part 256-byte aligned, 64 bytes of slack at the end
+    size_t off = 0;
+    const size_t o_gup = off; off += up(E * gu_p);
+    const size_t o_gus = off; off += up(E * gu_s);
+    const size_t o_dnp = off; off += up(E * dn_p);
+    const size_t o_dns = off; off += up(E * dn_s);
+    const size_t o_rp = off; off += up(E * hidden * 4);
+    const size_t o_rb = off; off += up(E * 4);
+    const size_t o_gub = off; off += up(E * 2 * inter * 4);
+    const size_t o_db = off; off += up(E * hidden * 4);
+    const size_t o_sc = off; off += up(E * 4);
+    larql_hip_moe_layer *L = new larql_hip_moe_layer();
+    if (hipMalloc(&L->region, off + 64) != hipSuccess) { delete L; return fail(c, LARQL_E_DEVICE, "moe_layer: out of device memory"); }
+    uint8_t *d = (uint8_t *)L->region;
+    const bool inter_rows = w->fused_row_layout == LARQL_MOE_ROWS_INTERLEAVED;
+    hipError_t e = hipSuccess;
+    auto put = [&](size_t dst, const void *src, size_t n) {
+        if (e == hipSuccess && n) e = hipMemcpyAsync(d + dst, src, n, hipMemcpyHostToDevice, c->stream);
+    };
+    for (size_t x = 0; x < E; x++) {
+        if (inter_rows) {  // the fused rows stay as stored: gate on the even, up on the odd rows, walked in place
+            put(o_gup + x * gu_p, w->experts_gate_up[x], gu_p);
+            put(o_gus + x * gu_s, w->scales_gate_up[x], gu_s);
+        } else {           // [gate rows | up rows] per expert: the gate halves of all experts, then the up halves
+            put(o_gup + x * (gu_p / 2), w->experts_gate_up[x], gu_p / 2);
+            put(o_gup + E * (gu_p / 2) + x * (gu_p / 2), w->experts_gate_up[x] + gu_p / 2, gu_p / 2);
+            put(o_gus + x * (gu_s / 2), w->scales_gate_up[x], gu_s / 2);
+            put(o_gus + E * (gu_s / 2) + x * (gu_s / 2), w->scales_gate_up[x] + gu_s / 2, gu_s / 2);
+        }
+        put(o_dnp + x * dn_p, w->experts_down[x], dn_p);
+        put(o_dns + x * dn_s, w->scales_down[x], dn_s);
+    }
+    put(o_rp, w->router_proj, E * hidden * 4);
+    if (w->router_bias) put(o_rb, w->router_bias, E * 4);
+    if (w->experts_gate_up_bias) put(o_gub, w->experts_gate_up_bias, E * 2 * inter * 4);
+    if (w->experts_down_bias) put(o_db, w->experts_down_bias, E * hidden * 4);
+    if (w->router_per_expert_scale) put(o_sc, w->router_per_expert_scale, E * 4);
+    if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+    if (e != hipSuccess) {
+        (void)hipFree(L->region);
+        delete L;
+        return fail(c, LARQL_E_DEVICE, "moe_layer: upload: %s", hipGetErrorString(e));
+    }
+    L->bank.gate_packed = d + o_gup; L->bank.gate_scales = d + o_gus;
+    L->bank.up_packed = inter_rows ? nullptr : d + o_gup + E * (gu_p / 2);
+    L->bank.up_scales = inter_rows ? nullptr : d + o_gus + E * (gu_s / 2);
+    L->bank.down_packed = d + o_dnp; L->bank.down_scales = d + o_dns;
+    L->bank.n_experts = E; L->bank.hidden = hidden; L->bank.inter = inter;
+    L->bank.limit = w->glu_limit; L->bank.alpha = w->glu_alpha;
+    L->bank.gate_up_interleaved = inter_rows ? 1 : 0;
+    L->bank.router_bias = w->router_bias ? (const float *)(d + o_rb) : nullptr;
+    L->bank.gate_up_bias = w->experts_gate_up_bias ? (const float *)(d + o_gub) : nullptr;
+    L->bank.down_bias = w->experts_down_bias ? (const float *)(d + o_db) : nullptr;
+    L->router_proj = (const float *)(d + o_rp);
+    L->scale = w->router_per_expert_scale ? (const float *)(d + o_sc) : nullptr;
+    L->n_experts = E; L->top_k = w->top_k; L->hidden = hidden; L->inter = inter;
+    L->renormalized = w->renormalized_softmax ? 1 : 0;
+    L->per_expert_scale = (w->per_expert_scale && w->router_per_expert_scale) ? 1 : 0;
+    *out = L;
+    return LARQL_OK;
+}
+
+// router logits on the device (one [num_experts, hidden] f32 gemv job per token), then the route and the expert block
+static int moe_layer_enqueue(larql_hip_ctx *c, larql_hip_moe_layer *L, const float *router_in, const float *x, size_t tokens, float *out,
+                             uint32_t *experts, float *weights) {
+    const size_t E = L->n_experts, hidden = L->hidden, k = std::min(L->top_k, E);
+    if (hidden % 4 != 0 || ((uintptr_t)router_in & 15) || ((uintptr_t)x & 15) || ((uintptr_t)out & 15))
+        return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: activations must be 16-byte aligned rows (hidden a multiple of 4)");
+    const size_t wsb = larql_hip_moe_mxfp4_workspace_bytes(tokens, k, hidden, L->inter);
+    int rc = ensure(c, L->ws, wsb); if (rc) return rc;
+    rc = ensure(c, L->logits, tokens * E * 4 + 64); if (rc) return rc;
+    float *logits = (float *)L->logits.p;
+    std::vector<GemvJob> jobs;
+    for (size_t t = 0; t < tokens; t++) jobs.push_back(make_job(KIND_F32, L->router_proj, nullptr, router_in + t * hidden, logits + t * E, E, hidden));
+    rc = enqueue_jobs(c, jobs);
+    if (rc) return rc;
+    // softmax over all, top-k, renormalise == Router::select's NormalisedOverSelected (the same quotient of exponentials);
+    // without the renormalisation the weights are the softmax's own values (SoftmaxThenSelect)
+    const int policy = L->renormalized ? 1 : 0;
+    if (!L->per_expert_scale) return moe_mxfp4_block(c, &L->bank, x, tokens, k, experts, weights, out, L->ws.p, wsb, logits, policy);
+    HIPCHECK(c, router_select_launch(c->stream, logits, L->bank.router_bias, (uint32_t)tokens, (uint32_t)E, (uint32_t)k, policy, experts, weights));
+    HIPCHECK(c, expert_scale_launch(c->stream, weights, experts, L->scale, (uint32_t)(tokens * k), (uint32_t)E));
+    return moe_mxfp4_block(c, &L->bank, x, tokens, k, experts, weights, out, L->ws.p, wsb, nullptr, 0);
+}
+
+int larql_hip_dev_moe_layer_forward(larql_hip_ctx *c, larql_hip_moe_layer *L, const float *router_in, const float *x, size_t tokens,
+                                    float *out, uint32_t *experts, float *weights) {
+    if (!c || !L) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (tokens == 0) return LARQL_OK;
+    if (tokens > (1u << 20)) return fail(c, LARQL_UNSUPPORTED, "moe_layer: too many tokens in one call");
+    if (!router_in || !x || !out || !experts || !weights) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    return moe_layer_enqueue(c, L, router_in, x, tokens, out, experts, weights);
+}
+
+int larql_hip_moe_layer_forward(larql_hip_ctx *c, larql_hip_moe_layer *L, const float *router_in, const float *x, size_t tokens,
+                                float *out, uint32_t *experts_out, float *weights_out) {
+    if (!c || !L) return LARQL_E_ARG;
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (tokens == 0) return LARQL_OK;
+    if (tokens > (1u << 20)) return fail(c, LARQL_UNSUPPORTED, "moe_layer: too many tokens in one call");
+    if (!router_in || !x || !out) return LARQL_E_ARG;
+    HIPCHECK(c, hipSetDevice(c->device));
+    const size_t hidden = L->hidden, k = std::min(L->top_k, L->n_experts), nb = tokens * hidden * 4;
+    int rc = upload(c, L->x, x, nb); if (rc) return rc;
+    const float *d_rin = (const float *)L->x.p;
+    if (router_in != x) { rc = upload(c, L->rin, router_in, nb); if (rc) return rc; d_rin = (const float *)L->rin.p; }
+    rc = ensure(c, L->out, nb + 64); if (rc) return rc;
+    rc = ensure(c, L->experts, tokens * k * 4 + 64); if (rc) return rc;
+    rc = ensure(c, L->weights, tokens * k * 4 + 64); if (rc) return rc;
+    Submission sub(c);
+    rc = moe_layer_enqueue(c, L, d_rin, (const float *)L->x.p, tokens, (float *)L->out.p, (uint32_t *)L->experts.p, (float *)L->weights.p);
+    if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
+    HIPCHECK(c, hipMemcpyAsync(out, L->out.p, nb, hipMemcpyDeviceToHost, c->stream));
+    if (experts_out) HIPCHECK(c, hipMemcpyAsync(experts_out, L->experts.p, tokens * k * 4, hipMemcpyDeviceToHost, c->stream));
+    if (weights_out) HIPCHECK(c, hipMemcpyAsync(weights_out, L->weights.p, tokens * k * 4, hipMemcpyDeviceToHost, c->stream));
+    return sub.finish();
 }
 
 // Gate-KNN over several layers in one submission (the LQL WALK / DESCRIBE shape: every layer of

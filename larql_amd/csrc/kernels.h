@@ -193,6 +193,7 @@ hipError_t moe_plan_launch(hipStream_t s, const float *logits, const float *rout
                            GemvJob *gu_table, uint32_t *gu_hdr, GemvJob *dn_table, uint32_t *dn_hdr, uint32_t *gu_first, uint32_t *dn_first);
 hipError_t clamped_glu_interleaved_launch(hipStream_t s, const float *gu, float *h, size_t n, float limit, float alpha);
 hipError_t clamped_glu_launch(hipStream_t s, const float *g, const float *u, float *h, size_t n, float limit, float alpha);
+hipError_t expert_scale_launch(hipStream_t s, float *weights, const uint32_t *experts, const float *scale, uint32_t n, uint32_t n_scale);
 hipError_t weighted_sum_launch(hipStream_t s, const float *d, const float *weights, const uint32_t *experts, uint32_t n_experts, float *out,
                                uint32_t tokens, uint32_t k, uint32_t hidden);
 

@@ -50,6 +50,16 @@ __global__ void clamped_glu_interleaved_kernel(const float *__restrict__ gu, flo
     h[i] = (uv + 1.0f) * (gv * sig);
 }
 
+// weights[i] *= scale[experts[i]] — MoeExpertScalePolicy::PerExpert (larql-compute/src/cpu/ops/moe/mod.rs:168-176);
+// a selected id outside the scale table keeps its weight, as the reference leaves it.
+__global__ void expert_scale_kernel(float *__restrict__ weights, const uint32_t *__restrict__ experts, const float *__restrict__ scale,
+                                    uint32_t n, uint32_t n_scale) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const uint32_t e = experts[i];
+    if (e < n_scale) weights[i] *= scale[e];
+}
+
 // out[t] = sum over the token's k selected experts, in selection order, of w * down-output
 // (larql-compute/src/cpu/ops/moe/forward.rs:266-270).  A slot whose expert id lies outside the bank is skipped
 // (forward.rs:203-208): its rows of `d` were never written and are not read.
@@ -336,6 +346,12 @@ hipError_t clamped_glu_launch(hipStream_t s, const float *g, const float *u, flo
     hipLaunchKernelGGL(clamped_glu_kernel, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, s, g, u, h, n, limit, alpha);
     return hipGetLastError();
 }
+hipError_t expert_scale_launch(hipStream_t s, float *weights, const uint32_t *experts, const float *scale, uint32_t n, uint32_t n_scale) {
+    if (n == 0 || n_scale == 0) return hipSuccess;
+    hipLaunchKernelGGL(expert_scale_kernel, dim3((n + 255) / 256), dim3(256), 0, s, weights, experts, scale, n, n_scale);
+    return hipGetLastError();
+}
+
 hipError_t weighted_sum_launch(hipStream_t s, const float *d, const float *weights, const uint32_t *experts, uint32_t n_experts, float *out,
                                uint32_t tokens, uint32_t k, uint32_t hidden) {
     if (tokens == 0 || hidden == 0) return hipSuccess;

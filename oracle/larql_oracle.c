@@ -1180,6 +1180,41 @@ void lq_softmax(float *v, size_t n) {
     if (sum > 0.0f) for (size_t i = 0; i < n; i++) v[i] /= sum;
 }
 
+/* moe_router_logits: larql-compute/src/cpu/ops/moe/mod.rs:127-147 — logits[e] = router_in . router_proj[e] + bias[e]
+ * (the bias joins before softmax / selection).  The reference's matmul_vec goes through BLAS, whose summation order
+ * is not fixed; a sequential f32 dot stands in for it. */
+void lq_moe_router_logits(const float *router_in, const float *router_proj, const float *router_bias, size_t n_experts,
+                          size_t hidden, float *logits) {
+    for (size_t e = 0; e < n_experts; e++) {
+        float acc = 0.0f;
+        for (size_t c = 0; c < hidden; c++) acc += router_in[c] * router_proj[e * hidden + c];
+        logits[e] = router_bias ? acc + router_bias[e] : acc;
+    }
+}
+
+/* moe_route_from_router_input: cpu/ops/moe/mod.rs:149-186 — the served tier's route: softmax over ALL logits, top_k
+ * of the probabilities (value descending, index ascending), divided by their sum under
+ * MoeTopKWeightPolicy::RenormalizedSoftmax (only when the sum is positive), then multiplied by
+ * router_per_expert_scale[expert] under MoeExpertScalePolicy::PerExpert (per_expert_scale != NULL here). */
+size_t lq_moe_route_from_router_input(const float *router_in, size_t hidden, const float *router_proj, const float *router_bias,
+                                      size_t n_experts, size_t top_k, int renormalize, const float *per_expert_scale,
+                                      size_t n_scale, uint64_t *experts, float *weights) {
+    float *logits = (float *)malloc((n_experts ? n_experts : 1) * sizeof(float));
+    lq_moe_router_logits(router_in, router_proj, router_bias, n_experts, hidden, logits);
+    lq_softmax(logits, n_experts);
+    size_t k = lq_moe_top_k(logits, n_experts, top_k, experts, weights);
+    if (renormalize) {
+        float sum = 0.0f;
+        for (size_t i = 0; i < k; i++) sum += weights[i];
+        if (sum > 0.0f) for (size_t i = 0; i < k; i++) weights[i] /= sum;
+    }
+    if (per_expert_scale && n_scale)
+        for (size_t i = 0; i < k; i++)
+            if (experts[i] < n_scale) weights[i] *= per_expert_scale[experts[i]];
+    free(logits);
+    return k;
+}
+
 /* MoeGateRule::ClampedGlu: larql-compute/src/pipeline/moe.rs:88-92. */
 float lq_clamped_glu(float g, float u, float limit, float alpha) {
     g = fminf(g, limit);

@@ -111,6 +111,11 @@ size_t lq_router_select(const float *logits, size_t n, size_t k, int policy,
                         uint64_t *experts, float *weights);
 size_t lq_moe_top_k(const float *v, size_t n, size_t k, uint64_t *idx, float *val);
 void   lq_softmax(float *v, size_t n);
+void   lq_moe_router_logits(const float *router_in, const float *router_proj, const float *router_bias, size_t n_experts,
+                            size_t hidden, float *logits);
+size_t lq_moe_route_from_router_input(const float *router_in, size_t hidden, const float *router_proj, const float *router_bias,
+                                      size_t n_experts, size_t top_k, int renormalize, const float *per_expert_scale,
+                                      size_t n_scale, uint64_t *experts, float *weights);
 float  lq_clamped_glu(float g, float u, float limit, float alpha);
 /* ExpertWeightFfn::moe_block (ffn/expert_weight/mod.rs:100-262) on a GPT-OSS-shaped f32 layer; pinned on EXPECTED[48]
  * of larql-compute/tests/test_moe_reference_parity.rs.  router_b / gate_up_bias / down_bias may be NULL. */

@@ -480,6 +480,35 @@ def router_select(logits, k: int, policy: int = NORMALISED_OVER_SELECTED):
     return [(int(e[i]), float(w[i])) for i in range(got)]
 
 
+def moe_router_logits(router_in, router_proj, router_bias=None) -> np.ndarray:
+    """moe_router_logits (cpu/ops/moe/mod.rs:127-147): router_proj is [n_experts, hidden]."""
+    x = _f32(router_in).ravel()
+    w = np.ascontiguousarray(router_proj, dtype=np.float32)
+    n, hidden = w.shape
+    assert hidden == x.size
+    b = None if router_bias is None else _f32(router_bias).ravel()
+    out = np.empty(n, dtype=np.float32)
+    _lib.lq_moe_router_logits(_p(x, _f32p), _p(w, _f32p), _p(b, _f32p) if b is not None else None, _sz(n), _sz(hidden), _p(out, _f32p))
+    return out
+
+
+def moe_route_from_router_input(router_in, router_proj, router_bias, top_k: int, renormalize: bool = True, per_expert_scale=None):
+    """moe_route_from_router_input (cpu/ops/moe/mod.rs:149-186): [(expert, weight)] in selection order."""
+    x = _f32(router_in).ravel()
+    w = np.ascontiguousarray(router_proj, dtype=np.float32)
+    n, hidden = w.shape
+    b = None if router_bias is None else _f32(router_bias).ravel()
+    sc = None if per_expert_scale is None else _f32(per_expert_scale).ravel()
+    cap = max(1, min(top_k, n))
+    e = np.empty(cap, dtype=np.uint64)
+    wt = np.empty(cap, dtype=np.float32)
+    _lib.lq_moe_route_from_router_input.restype = C.c_size_t
+    got = _lib.lq_moe_route_from_router_input(_p(x, _f32p), _sz(hidden), _p(w, _f32p), _p(b, _f32p) if b is not None else None, _sz(n),
+                                              _sz(top_k), C.c_int(1 if renormalize else 0), _p(sc, _f32p) if sc is not None else None,
+                                              _sz(0 if sc is None else sc.size), _p(e, _u64p), _p(wt, _f32p))
+    return [(int(e[i]), float(wt[i])) for i in range(got)]
+
+
 def moe_top_k(v, k: int):
     v = _f32(v).ravel()
     cap = max(1, min(k, v.size))

@@ -1134,6 +1134,92 @@ def test_moe_mxfp4_interleaved_gate_up_bank_equals_separate_banks(be, fmt, T, E,
                          dev["x"], T, k, de, dw_, do, ws, wsb)
 
 
+@pytest.mark.parametrize("T,E,hidden,inter,layout,per_expert,renorm", [
+    (1, 5, 2880, 2880, "interleaved", False, True),       # a GPT-OSS layer's shapes, one token: selection inside the first launch
+    (1, 6, 384, 320, "halves", False, True),
+    (5, 6, 384, 320, "interleaved", True, True),          # several tokens, MoeExpertScalePolicy::PerExpert
+    (9, 8, 2880, 576, "halves", True, False),             # ... and the softmax's own values (no renormalisation)
+    (1, 4, 96, 64, "interleaved", True, True),            # rows the matrix-core kernels do not take
+])
+def test_moe_layer_from_per_expert_slices_with_router_projection(be, fmt, T, E, hidden, inter, layout, per_expert, renorm):
+    """MoeLayerWeights as the reference brings it (pipeline/moe.rs:469-541): per-expert gate+up / down slices in
+    allocations of their own, MoeExpertScales::Paired exponent streams, Interleaved or ContiguousHalves fused rows,
+    router_proj / router_bias / router_per_expert_scale.  The layer goes residual -> output with the router's
+    projection on the device: the route equals moe_route_from_router_input (mod.rs:149-186), the output the checker's
+    expert block under that route; host tier and device tier agree bit for bit."""
+    rng = np.random.default_rng(211 + T + E)
+    k, G, Gd = 4, hidden // 32, inter // 32
+    gate = [O.quantize_mxfp4((rng.standard_normal(inter * hidden) * 0.02).astype(F), inter, hidden) for _ in range(E)]
+    up = [O.quantize_mxfp4((rng.standard_normal(inter * hidden) * 0.02).astype(F), inter, hidden) for _ in range(E)]
+    down = [O.quantize_mxfp4((rng.standard_normal(hidden * inter) * 0.02).astype(F), hidden, inter) for _ in range(E)]
+    gu_p, gu_s = [], []                                   # expert e's fused slice, an allocation of its own
+    for e in range(E):
+        p, s = np.empty((2 * inter, G * 16), np.uint8), np.empty((2 * inter, G), np.uint8)
+        if layout == "interleaved":
+            p[0::2], p[1::2] = gate[e][0].reshape(inter, -1), up[e][0].reshape(inter, -1)
+            s[0::2], s[1::2] = gate[e][1].reshape(inter, -1), up[e][1].reshape(inter, -1)
+        else:
+            p[:inter], p[inter:] = gate[e][0].reshape(inter, -1), up[e][0].reshape(inter, -1)
+            s[:inter], s[inter:] = gate[e][1].reshape(inter, -1), up[e][1].reshape(inter, -1)
+        gu_p.append(np.concatenate([p.reshape(-1), np.full(7 + e, 0xEE, np.uint8)]))     # (slices may be longer than the geometry)
+        gu_s.append(s.reshape(-1).copy())
+    router_w = (rng.standard_normal((E, hidden)) * 0.05).astype(F)
+    router_b = rng.standard_normal(E).astype(F)
+    gub = (rng.standard_normal((E, 2 * inter)) * 0.5).astype(F)
+    db = (rng.standard_normal((E, hidden)) * 0.5).astype(F)
+    scale = rng.uniform(0.5, 2.0, E).astype(F) if per_expert else None
+    x = rng.standard_normal((T, hidden)).astype(F)
+    rin = (x * F(0.5) + F(0.25)).astype(F)                # the router's input is its own tensor (a norm of the residual in the reference)
+    rows = fmt.MOE_ROWS_INTERLEAVED if layout == "interleaved" else fmt.MOE_ROWS_CONTIGUOUS_HALVES
+    layer = be.moe_layer_create(gu_p, [d[0] for d in down], gu_s, [d[1] for d in down], router_w, k, hidden, inter, rows,
+                                router_bias=router_b, gate_up_bias=gub, down_bias=db, per_expert_scale=scale, renormalized=renorm)
+    assert layer
+    got = be.moe_layer_forward(layer, rin, x, k)
+    assert got is not None
+    out, experts, weights = got
+    # the route: moe_route_from_router_input on the same tensors
+    for t in range(T):
+        want = O.moe_route_from_router_input(rin[t], router_w, router_b, k, renormalize=renorm, per_expert_scale=scale)
+        # (the device's f32 gemv adds in another order than the sequential dot: logits differ in the last bits, so a
+        # selection may only differ where two probabilities are that close)
+        assert [int(e) for e in experts[t]] == [e for e, _ in want], t
+        assert np.allclose(weights[t], [w for _, w in want], rtol=5e-5, atol=0)
+    gpb, gsb = np.concatenate([g[0] for g in gate]), np.concatenate([g[1] for g in gate])
+    upb, usb = np.concatenate([u[0] for u in up]), np.concatenate([u[1] for u in up])
+    dpb, dsb = np.concatenate([d[0] for d in down]), np.concatenate([d[1] for d in down])
+    want_out = O.moe_block_mxfp4(x, experts.astype(np.uint64), weights, (gpb, gsb), (upb, usb), (dpb, dsb), E, hidden, inter,
+                                 gate_up_bias=gub, down_bias=db)
+    assert rel_l2(out, want_out) < 1e-5
+    # device tier on resident operands: the same bits, nothing crosses the bus
+    dx, dr, do = be.to_device(x), be.to_device(rin), be.malloc(T * hidden * 4)
+    de, dw_ = be.malloc(T * k * 4), be.malloc(T * k * 4)
+    assert be.dev_moe_layer_forward(layer, dr, dx, T, do, de, dw_)
+    be.synchronize()
+    assert np.array_equal(be.d2h(do, (T, hidden), F).view(np.uint32), out.view(np.uint32))
+    assert np.array_equal(be.d2h(de, (T, k), np.uint32), experts) and np.array_equal(be.d2h(dw_, (T, k), F).view(np.uint32), weights.view(np.uint32))
+    be.moe_layer_destroy(layer)
+
+
+def test_moe_layer_refusals(be, fmt):
+    """What MoeLayerWeights can say and this backend does not serve answers None (never a wrong bank): inline scales on
+    an MXFP4 bank, another expert format, slices shorter than the geometry, more than 64 experts."""
+    rng = np.random.default_rng(3)
+    E, hidden, inter, k = 3, 64, 32, 2
+    gu = [O.quantize_mxfp4((rng.standard_normal(2 * inter * hidden) * 0.02).astype(F), 2 * inter, hidden) for _ in range(E)]
+    dn = [O.quantize_mxfp4((rng.standard_normal(hidden * inter) * 0.02).astype(F), hidden, inter) for _ in range(E)]
+    rw = rng.standard_normal((E, hidden)).astype(F)
+    args = ([g[0] for g in gu], [d[0] for d in dn], [g[1] for g in gu], [d[1] for d in dn], rw, k, hidden, inter)
+    ok = be.moe_layer_create(*args)
+    assert ok
+    be.moe_layer_destroy(ok)
+    assert be.moe_layer_create(*args, expert_scales=fmt.MOE_SCALES_INLINE) is None
+    assert be.moe_layer_create(*args, expert_data_format=fmt.FMT_Q4_K) is None
+    short = ([g[0][:-16] for g in gu],) + args[1:]
+    assert be.moe_layer_create(*short) is None
+    many = ([gu[0][0]] * 65, [dn[0][0]] * 65, [gu[0][1]] * 65, [dn[0][1]] * 65, np.zeros((65, hidden), F), k, hidden, inter)
+    assert be.moe_layer_create(*many) is None
+
+
 # ------------------------------------------------------------- prefill GEMM
 @pytest.mark.parametrize("rows,hidden,seq", [(300, 512, 70), (128, 3840, 128), (1, 256, 1), (257, 768, 33), (520, 8192, 200)])
 def test_q4k_gemm_mfma_matches_oracle(be, rows, hidden, seq):
@@ -1200,6 +1286,46 @@ def test_q4k_gemm_row_scales_of_any_size_and_uneven_blocks(be):
         n = np.linalg.norm(want_h[:, r].astype(np.float64))
         if n > 0:
             assert np.linalg.norm(got_h[:, r].astype(np.float64) - want_h[:, r]) / n < 2e-5, r
+
+
+def test_q4k_gemm_non_finite_and_lopsided_block_headers(be):
+    """The rows' exponents come from max(|d|, |dmin|/16) over a row's super-blocks.  A header that is inf or NaN (a
+    corrupt or adversarial block) makes that row's results non-finite in the reference as well (inf * q, inf - inf);
+    here it must do the same to THAT row and leave every other row's bits alone.  A row with one large super-block and
+    39 tiny ones (their scales fall into f16 subnormals behind the row's exponent) stays within the stated bar."""
+    rng = np.random.default_rng(103)
+    rows, hidden, seq = 96, 10240, 24
+    w = (rng.standard_normal((rows, hidden)) * 0.02).astype(F)
+    w[7, 256:] *= F(2.0 ** -13)                             # one super-block 8192 times the other 39
+    w[8, :] *= F(2.0 ** -13); w[8, 9 * 256:10 * 256] *= F(2.0 ** 13)
+    q = O.quantize_q4_k(w)
+    xb = O.f32_to_bf16(rng.standard_normal((seq, hidden)).astype(F))
+    X = (xb.astype(np.uint32) << 16).view(F).reshape(seq, hidden)
+    dw, dx, do = be.to_device(q), be.to_device(xb), be.malloc(seq * rows * 4)
+    assert be.dev_q4k_gemm(dw, dx, rows, hidden, seq, do)
+    be.synchronize()
+    clean = be.d2h(do, (seq, rows), F)
+    want = O.q4k_matmul(q, X, rows, hidden, seq)
+    for r in (7, 8):
+        assert np.linalg.norm(clean[:, r].astype(np.float64) - want[:, r]) / np.linalg.norm(want[:, r]) < 1e-3, r
+    assert rel_l2(clean, want) < 5e-4
+    bad = q.reshape(rows, hidden // 256, 144).copy()
+    bad[20, 3, 0:2] = np.frombuffer(np.float16(np.inf).tobytes(), np.uint8)        # d = +inf
+    bad[41, 17, 2:4] = np.frombuffer(np.float16(np.nan).tobytes(), np.uint8)       # dmin = NaN
+    bad[60, 0, 0:2] = np.frombuffer(np.float16(-np.inf).tobytes(), np.uint8)       # d = -inf
+    want_bad = O.q4k_matmul(bad.reshape(-1), X, rows, hidden, seq)
+    assert not np.isfinite(want_bad[:, [20, 41, 60]]).any()
+    be.h2d(dw, bad.reshape(-1))
+    assert be.dev_q4k_gemm(dw, dx, rows, hidden, seq, do)
+    be.synchronize()
+    got = be.d2h(do, (seq, rows), F)
+    assert not np.isfinite(got[:, [20, 41, 60]]).any()
+    others = [r for r in range(rows) if r not in (20, 41, 60)]
+    assert np.array_equal(got[:, others].view(np.uint32), clean[:, others].view(np.uint32))
+    # the exact-integer host tier on the same matrix
+    got_h = be.q4k_matmul(bad.reshape(-1), X, rows, hidden, seq).reshape(seq, rows)
+    assert not np.isfinite(got_h[:, [20, 41, 60]]).any()
+    assert rel_l2(got_h[:, others], want[:, others]) < 2e-5
 
 
 def test_q4k_gemm_activation_ranges_token_by_token(be):

@@ -29,7 +29,10 @@ def both(be, f, gate_dev, x, batch, n, hidden, k):
     i2, v2, c2 = be.malloc(batch * k * 4), be.malloc(batch * k * 4), be.malloc(batch * 4)
     try:
         assert be.dev_gate_knn(f, gate_dev, xd, batch, n, hidden, k, sc, i1, v1)
+        events = be.debug_alloc_events()
         assert be.dev_gate_knn_static(f, gate_dev, xd, batch, n, hidden, k, i2, v2, c2)
+        # what the entry point exists for: it took no device memory, staged nothing and uploaded no job table
+        assert be.debug_alloc_events() == events
         be.synchronize()
         m = min(k, n)
         a = be.d2h(i1, (batch, k), np.uint32)[:, :m], be.d2h(v1, (batch, k), np.uint32)[:, :m]
@@ -47,7 +50,8 @@ def test_static_entry_equals_the_allocating_one_on_two_calls_in_a_row(be, name):
     import larql_amd as fmt
     rng = np.random.default_rng(17)
     hidden = 512
-    shapes = [(8, 3000, 64), (3, 700, 17)]      # (batch, features, K): the second call is smaller
+    shapes = [(8, 3000, 64), (3, 700, 17), (2, 2000, 200)]   # (batch, features, K): the second call is smaller; the third
+    #                                                          takes the path for more than 64 winners (a sort in LDS)
     for batch, n, k in shapes:
         w = (rng.standard_normal((n, hidden)) * 0.02).astype(F)
         x = rng.standard_normal((batch, hidden)).astype(F)
