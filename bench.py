@@ -22,8 +22,9 @@ a streaming-bandwidth figure, not a decode rate.  `config.dependency_ordered`
 reports the same weights walked as a token would walk them — per layer the
 stages q,k,v | o | gate,up | down, each stage reading the previous stage's
 output, 137 dependent launches — with its own ms per token.  `config.other_configs`
-carries a short run of BASELINE's other configurations (each verified against
-the oracle in the same run), `config.host_tier_us_per_call` what a trait-shaped
+carries a short run of BASELINE's other configurations and of the other block
+formats of the matvec family (Q6_K, MXFP4), each verified against the oracle in
+the same run, `config.host_tier_us_per_call` what a trait-shaped
 call on host slices costs end to end.
 """
 from __future__ import annotations
@@ -866,7 +867,7 @@ def other_configs(be, fmt, args):
     short.cpu_seconds = 0.4 if args.no_cpu else min(args.cpu_seconds, 4.0)
     _COLLECT = []
     try:
-        for fn in (run_c1, run_c3, run_c4, run_c5):
+        for fn in (run_c1, run_c3, run_c4, run_c5, run_formats):
             fn(be, fmt, short)
         lines = _COLLECT
     finally:

@@ -53,6 +53,14 @@ struct Region {
     uint8_t *dev;
 };
 
+// Page-locked host memory the device can address: small activations go up through it (an asynchronous copy from
+// page-locked memory does not wait for a staging copy inside the runtime) and small results are WRITTEN into it by
+// the kernels themselves, which spares a host-tier call the copy back.
+struct PinBuf {
+    void *host = nullptr, *dev = nullptr;
+    size_t cap = 0;
+};
+
 }  // namespace
 
 constexpr size_t kHostMats = 8;  // matrices one host-tier submission stages (their jobs travel in the kernel arguments)
@@ -78,6 +86,8 @@ struct larql_hip_ctx {
     int *nan_flag = nullptr;       // [0]: device tier, raised by any call, cleared when taken; [1]: host tier, cleared by every call
     uint8_t *static_scratch = nullptr;  // this device's copy of `scratch` (hipGetSymbolAddress at create)
     larql_hip_submission_clock clock = {0, 0, 0};
+    PinBuf pin_up, pin_out;   // host tier: activations on their way up (a ring, see upload()), results written by kernels
+    size_t pin_up_off = 0, pin_up_call = 0;  // next free byte of the ring; bytes staged since the stream was last waited for
     // Times a call took device memory, staged a host buffer or uploaded a job table (larql_hip_debug_alloc_events):
     // what the entry point that allocates nothing must never do.
     uint64_t alloc_events = 0;
@@ -129,10 +139,53 @@ int resolve_weights(larql_hip_ctx *c, const uint8_t *host, size_t len, DevBuf &s
     return LARQL_OK;
 }
 
+constexpr size_t kPinUpBytes = 4u << 20;    // the ring activations go up through
+constexpr size_t kPinSmall = 512u << 10;    // what counts as small enough for page-locked staging / results
+
+int ensure_pinned(larql_hip_ctx *c, PinBuf &b, size_t bytes) {
+    if (bytes <= b.cap) return LARQL_OK;
+    c->alloc_events++;
+    if (b.host) {
+        HIPCHECK(c, hipStreamSynchronize(c->stream));
+        HIPCHECK(c, hipHostFree(b.host));
+    }
+    b.host = b.dev = nullptr; b.cap = 0;
+    const size_t cap = bytes < 65536 ? 65536 : bytes;
+    HIPCHECK(c, hipHostMalloc(&b.host, cap, hipHostMallocDefault));
+    if (hipHostGetDevicePointer(&b.dev, b.host, 0) != hipSuccess || !b.dev) {
+        (void)hipHostFree(b.host);
+        b.host = nullptr;
+        return fail(c, LARQL_E_DEVICE, "page-locked memory is not addressable by the device");
+    }
+    b.cap = cap;
+    return LARQL_OK;
+}
+
+// Every host-tier call ends by waiting for the stream; from then on the whole ring is free again.
+void stream_waited(larql_hip_ctx *c) { c->pin_up_call = 0; }
+hipError_t wait_stream(larql_hip_ctx *c) {
+    const hipError_t e = hipStreamSynchronize(c->stream);
+    stream_waited(c);
+    return e;
+}
+
 int upload(larql_hip_ctx *c, DevBuf &b, const void *host, size_t bytes) {
     int rc = ensure(c, b, bytes + 64);
     if (rc) return rc;
-    if (bytes) HIPCHECK(c, hipMemcpyAsync(b.p, host, bytes, hipMemcpyHostToDevice, c->stream));
+    if (!bytes) return LARQL_OK;
+    // small: through the page-locked ring (slices of one call never overlap: a call that stages more than the ring
+    // holds before it waits for the stream takes the pageable path for the rest)
+    const size_t slice = (bytes + 255) & ~(size_t)255;
+    if (bytes <= kPinSmall && c->pin_up_call + slice <= kPinUpBytes && ensure_pinned(c, c->pin_up, kPinUpBytes) == LARQL_OK) {
+        if (c->pin_up_off + slice > kPinUpBytes) c->pin_up_off = 0;
+        uint8_t *stage = (uint8_t *)c->pin_up.host + c->pin_up_off;
+        memcpy(stage, host, bytes);
+        c->pin_up_off += slice;
+        c->pin_up_call += slice;
+        HIPCHECK(c, hipMemcpyAsync(b.p, stage, bytes, hipMemcpyHostToDevice, c->stream));
+        return LARQL_OK;
+    }
+    HIPCHECK(c, hipMemcpyAsync(b.p, host, bytes, hipMemcpyHostToDevice, c->stream));
     return LARQL_OK;
 }
 
@@ -144,7 +197,7 @@ struct Submission {
     }
     int finish() {
         HIPCHECK(c, hipEventRecord(c->ev1, c->stream));
-        HIPCHECK(c, hipStreamSynchronize(c->stream));
+        HIPCHECK(c, wait_stream(c));
         float ms = 0.f;
         if (hipEventElapsedTime(&ms, c->ev0, c->ev1) == hipSuccess) c->clock.gpu_nanos += (uint64_t)(ms * 1e6);
         c->clock.submissions += 1;
@@ -265,7 +318,7 @@ int prepare_same_kind(larql_hip_ctx *c, GemvJob *live, size_t n_live, void *tabl
             c->table_sent_bytes[stage_slot] = bytes;
         } else {
             HIPCHECK(c, hipMemcpyAsync(table_dst, blob.data(), bytes, hipMemcpyHostToDevice, c->stream));
-            HIPCHECK(c, hipStreamSynchronize(c->stream));  // the host vector may die
+            HIPCHECK(c, wait_stream(c));  // the host vector may die
         }
         P.L.table = (const GemvJob *)table_dst;
         if (with_first) P.L.wg_first = (const uint32_t *)((const uint8_t *)table_dst + job_bytes);
@@ -405,6 +458,8 @@ void larql_hip_destroy(larql_hip_ctx *c) {
         if (c->table_host[i]) (void)hipHostFree(c->table_host[i]);
         if (c->table_ev[i]) (void)hipEventDestroy(c->table_ev[i]);
     }
+    if (c->pin_up.host) (void)hipHostFree(c->pin_up.host);
+    if (c->pin_out.host) (void)hipHostFree(c->pin_out.host);
     if (c->log2_up) (void)hipFree(c->log2_up);
     if (c->nan_flag) (void)hipFree(c->nan_flag);
     if (c->ev0) (void)hipEventDestroy(c->ev0);
@@ -458,7 +513,7 @@ int larql_hip_clear_weight_regions(larql_hip_ctx *c) {
     if (!c) return LARQL_E_ARG;
     std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipSetDevice(c->device));
-    HIPCHECK(c, hipStreamSynchronize(c->stream));
+    HIPCHECK(c, wait_stream(c));
     for (Region &r : c->regions) (void)hipFree(r.dev);
     c->regions.clear();
     return LARQL_OK;
@@ -483,26 +538,35 @@ static int host_matvec_multi(larql_hip_ctx *c, int kind, size_t n_mats, const ui
     if (rc) return rc;
     size_t out_total = 0;
     for (size_t i = 0; i < n_mats; i++) out_total += rows[i];
-    rc = ensure(c, c->out, out_total * sizeof(float) + 64);
-    if (rc) return rc;
+    // small results are written by the kernel straight into page-locked host memory: no copy back
+    const bool direct = out_total * sizeof(float) <= kPinSmall && ensure_pinned(c, c->pin_out, kPinSmall + 64) == LARQL_OK;
+    if (!direct) { rc = ensure(c, c->out, out_total * sizeof(float) + 64); if (rc) return rc; }
+    float *d_out = direct ? (float *)c->pin_out.dev : (float *)c->out.p;
     size_t off = 0;
     for (size_t i = 0; i < n_mats; i++) {
         const uint8_t *dw = nullptr, *da = nullptr;
         rc = resolve_weights(c, w[i], w_len[i], c->w[i], &dw);
         if (rc) return rc;
         if (aux) { rc = resolve_weights(c, aux[i], aux_len[i], c->aux[i], &da); if (rc) return rc; }
-        jobs.push_back(make_job(kind, dw, da, c->x.p, (float *)c->out.p + off, rows[i], k));
+        jobs.push_back(make_job(kind, dw, da, c->x.p, d_out + off, rows[i], k));
         off += rows[i];
     }
     Submission sub(c);
     rc = enqueue_jobs(c, jobs);
-    if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
+    if (rc) { (void)hipStreamSynchronize(c->stream); stream_waited(c); return rc; }
     off = 0;
+    if (!direct)
+        for (size_t i = 0; i < n_mats; i++) {
+            if (rows[i]) HIPCHECK(c, hipMemcpyAsync(out[i], (float *)c->out.p + off, rows[i] * sizeof(float), hipMemcpyDeviceToHost, c->stream));
+            off += rows[i];
+        }
+    rc = sub.finish();
+    if (rc || !direct) return rc;
     for (size_t i = 0; i < n_mats; i++) {
-        if (rows[i]) HIPCHECK(c, hipMemcpyAsync(out[i], (float *)c->out.p + off, rows[i] * sizeof(float), hipMemcpyDeviceToHost, c->stream));
+        if (rows[i]) memcpy(out[i], (const float *)c->pin_out.host + off, rows[i] * sizeof(float));
         off += rows[i];
     }
-    return sub.finish();
+    return LARQL_OK;
 }
 
 static bool q4k_shape_ok(size_t out_len, size_t rows, size_t x_len, size_t cols, size_t w_len) {
@@ -725,7 +789,7 @@ int larql_hip_q4k_matmul(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, c
         HIPCHECK(c, q4k_gemm_prep_launch(c->stream, c->x.p, 0, (uint32_t)hidden, (uint32_t)seq_len, xh, xl, sx, ts, c->nan_flag + 1, nullptr, 0, nullptr));
         int any_lo = 0;
         HIPCHECK(c, hipMemcpyAsync(&any_lo, c->nan_flag + 1, sizeof(int), hipMemcpyDeviceToHost, c->stream));
-        HIPCHECK(c, hipStreamSynchronize(c->stream));
+        HIPCHECK(c, wait_stream(c));
         HIPCHECK(c, hipMemsetAsync(c->nan_flag + 1, 0, sizeof(int), c->stream));
         const uint32_t splits = q4k_gemm_splits((uint32_t)num_rows, (uint32_t)hidden, (uint32_t)seq_len, (uint32_t)c->cu_count);
         float *partial = nullptr;
@@ -747,20 +811,53 @@ int larql_hip_q4k_matmul(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, c
     return sub.finish();
 }
 
-static int topk_download(larql_hip_ctx *c, size_t batch, size_t k, uint32_t *idx_out, float *score_out, size_t *n_out,
-                         bool check_nan) {
-    // misc layout: idx [batch*k] u32 | val [batch*k] f32 | count [batch] u32
-    uint32_t *d_idx = (uint32_t *)c->misc.p;
-    float *d_val = (float *)(d_idx + batch * k);
-    uint32_t *d_cnt = (uint32_t *)(d_val + batch * k);
-    std::vector<uint32_t> cnt(batch);
+// Where a host-tier top-K leaves its hits: idx [batch*k] u32 | val [batch*k] f32 | count [batch] u32.  Small results
+// are written by the kernel straight into page-locked host memory (the NaN flag follows them there by one 4-byte copy
+// queued behind the kernel), so the call waits for the stream once and copies nothing back; large ones stay in device
+// memory and are copied.
+struct TopkArea {
+    uint32_t *idx;
+    float *val;
+    uint32_t *cnt;
+    bool direct;
+};
+
+static int topk_area(larql_hip_ctx *c, size_t batch, size_t k, TopkArea &a) {
+    const size_t bytes = batch * (k * 8 + 4);
+    a.direct = bytes <= kPinSmall && ensure_pinned(c, c->pin_out, kPinSmall + 64) == LARQL_OK;
+    if (!a.direct) { int rc = ensure(c, c->misc, bytes + 64); if (rc) return rc; }
+    a.idx = (uint32_t *)(a.direct ? c->pin_out.dev : c->misc.p);
+    a.val = (float *)(a.idx + batch * k);
+    a.cnt = (uint32_t *)(a.val + batch * k);
+    return LARQL_OK;
+}
+
+// queued behind the top-K launch, before the call waits for the stream
+static int topk_queue_flag(larql_hip_ctx *c, const TopkArea &a) {
+    if (a.direct) HIPCHECK(c, hipMemcpyAsync((uint8_t *)c->pin_out.host + kPinSmall, c->nan_flag + 1, sizeof(int), hipMemcpyDeviceToHost, c->stream));
+    return LARQL_OK;
+}
+
+// after the stream has been waited for
+static int topk_collect(larql_hip_ctx *c, const TopkArea &a, size_t batch, size_t k, uint32_t *idx_out, float *score_out, size_t *n_out,
+                        bool check_nan) {
     int nan = 0;
-    HIPCHECK(c, hipMemcpyAsync(idx_out, d_idx, batch * k * 4, hipMemcpyDeviceToHost, c->stream));
-    HIPCHECK(c, hipMemcpyAsync(score_out, d_val, batch * k * 4, hipMemcpyDeviceToHost, c->stream));
-    HIPCHECK(c, hipMemcpyAsync(cnt.data(), d_cnt, batch * 4, hipMemcpyDeviceToHost, c->stream));
-    HIPCHECK(c, hipMemcpyAsync(&nan, c->nan_flag + 1, sizeof(int), hipMemcpyDeviceToHost, c->stream));
-    HIPCHECK(c, hipStreamSynchronize(c->stream));
-    for (size_t b = 0; b < batch; b++) n_out[b] = cnt[b];
+    if (a.direct) {
+        const uint8_t *h = (const uint8_t *)c->pin_out.host;
+        memcpy(idx_out, h, batch * k * 4);
+        memcpy(score_out, h + batch * k * 4, batch * k * 4);
+        const uint32_t *cnt = (const uint32_t *)(h + batch * k * 8);
+        for (size_t b = 0; b < batch; b++) n_out[b] = cnt[b];
+        memcpy(&nan, h + kPinSmall, sizeof(int));
+    } else {
+        std::vector<uint32_t> cnt(batch);
+        HIPCHECK(c, hipMemcpyAsync(idx_out, a.idx, batch * k * 4, hipMemcpyDeviceToHost, c->stream));
+        HIPCHECK(c, hipMemcpyAsync(score_out, a.val, batch * k * 4, hipMemcpyDeviceToHost, c->stream));
+        HIPCHECK(c, hipMemcpyAsync(cnt.data(), a.cnt, batch * 4, hipMemcpyDeviceToHost, c->stream));
+        HIPCHECK(c, hipMemcpyAsync(&nan, c->nan_flag + 1, sizeof(int), hipMemcpyDeviceToHost, c->stream));
+        HIPCHECK(c, wait_stream(c));
+        for (size_t b = 0; b < batch; b++) n_out[b] = cnt[b];
+    }
     if (check_nan && nan) return fail(c, LARQL_E_NAN, "top-K: NaN score");
     return LARQL_OK;
 }
@@ -776,20 +873,20 @@ static int host_matvec_topk(larql_hip_ctx *c, int kind, const uint8_t *w, size_t
     if (rc) return rc;
     rc = ensure(c, c->scores, num_rows * 4 + 64);
     if (rc) return rc;
-    rc = ensure(c, c->misc, top_k * 8 + 4 + 64);
+    TopkArea hits;
+    rc = topk_area(c, 1, top_k, hits);
     if (rc) return rc;
     std::vector<GemvJob> jobs{make_job(kind, dw, nullptr, c->x.p, (float *)c->scores.p, num_rows, hidden)};
     Submission sub(c);
     rc = enqueue_jobs(c, jobs);
-    if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
-    uint32_t *d_idx = (uint32_t *)c->misc.p;
-    float *d_val = (float *)(d_idx + top_k);
-    uint32_t *d_cnt = (uint32_t *)(d_val + top_k);
-    HIPCHECK(c, topk_launch(c->stream, (const float *)c->scores.p, 1, (uint32_t)num_rows, (uint32_t)top_k, false, d_idx, d_val,
-                            d_cnt, c->nan_flag + 1, nullptr, 0));
+    if (rc) { (void)wait_stream(c); return rc; }
+    HIPCHECK(c, topk_launch(c->stream, (const float *)c->scores.p, 1, (uint32_t)num_rows, (uint32_t)top_k, false, hits.idx, hits.val,
+                            hits.cnt, c->nan_flag + 1, nullptr, 0));
+    rc = topk_queue_flag(c, hits);
+    if (rc) return rc;
     rc = sub.finish();
     if (rc) return rc;
-    return topk_download(c, 1, top_k, idx_out, score_out, n_out, false);
+    return topk_collect(c, hits, 1, top_k, idx_out, score_out, n_out, false);
 }
 
 int larql_hip_q4k_matvec_topk(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, const float *x, size_t x_len,
@@ -1118,19 +1215,18 @@ int larql_hip_gate_knn(larql_hip_ctx *c, int format, const uint8_t *gate, size_t
     rc = resolve_weights(c, gate, n * format_row_bytes(kind, hidden), c->w[0], &dg); if (rc) return rc;
     rc = upload(c, c->x, x, batch * hidden * 4); if (rc) return rc;
     rc = ensure(c, c->scores, batch * n * 4 + 64); if (rc) return rc;
-    rc = ensure(c, c->misc, batch * (top_k * 8 + 4) + 64); if (rc) return rc;
+    TopkArea hits;
+    rc = topk_area(c, batch, top_k, hits); if (rc) return rc;
     HIPCHECK(c, hipMemsetAsync(c->nan_flag + 1, 0, sizeof(int), c->stream));
     Submission sub(c);
     rc = dev_gate_scores(c, kind, dg, (const float *)c->x.p, batch, n, hidden, (float *)c->scores.p);
-    if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
-    uint32_t *d_idx = (uint32_t *)c->misc.p;
-    float *d_val = (float *)(d_idx + batch * top_k);
-    uint32_t *d_cnt = (uint32_t *)(d_val + batch * top_k);
-    HIPCHECK(c, topk_launch(c->stream, (const float *)c->scores.p, (uint32_t)batch, (uint32_t)n, (uint32_t)top_k, true, d_idx,
-                            d_val, d_cnt, c->nan_flag + 1, nullptr, 0));
+    if (rc) { (void)wait_stream(c); return rc; }
+    HIPCHECK(c, topk_launch(c->stream, (const float *)c->scores.p, (uint32_t)batch, (uint32_t)n, (uint32_t)top_k, true, hits.idx,
+                            hits.val, hits.cnt, c->nan_flag + 1, nullptr, 0));
+    rc = topk_queue_flag(c, hits); if (rc) return rc;
     rc = sub.finish();
     if (rc) return rc;
-    return topk_download(c, batch, top_k, idx_out, score_out, n_out, true);
+    return topk_collect(c, hits, batch, top_k, idx_out, score_out, n_out, true);
 }
 
 // ---- device tier ----------------------------------------------------------------------------
@@ -1154,7 +1250,7 @@ int larql_hip_free(larql_hip_ctx *c, void *dptr) {
     if (!c) return LARQL_E_ARG;
     std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipSetDevice(c->device));
-    HIPCHECK(c, hipStreamSynchronize(c->stream));
+    HIPCHECK(c, wait_stream(c));
     HIPCHECK(c, hipFree(dptr));
     return LARQL_OK;
 }
@@ -1163,7 +1259,7 @@ int larql_hip_memcpy_h2d(larql_hip_ctx *c, void *dst, const void *src, size_t by
     std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipSetDevice(c->device));
     HIPCHECK(c, hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, c->stream));
-    HIPCHECK(c, hipStreamSynchronize(c->stream));
+    HIPCHECK(c, wait_stream(c));
     return LARQL_OK;
 }
 int larql_hip_memcpy_d2h(larql_hip_ctx *c, void *dst, const void *src, size_t bytes) {
@@ -1171,7 +1267,7 @@ int larql_hip_memcpy_d2h(larql_hip_ctx *c, void *dst, const void *src, size_t by
     std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipSetDevice(c->device));
     HIPCHECK(c, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, c->stream));
-    HIPCHECK(c, hipStreamSynchronize(c->stream));
+    HIPCHECK(c, wait_stream(c));
     return LARQL_OK;
 }
 int larql_hip_memset(larql_hip_ctx *c, void *dst, int value, size_t bytes) {
@@ -1185,7 +1281,7 @@ int larql_hip_synchronize(larql_hip_ctx *c) {
     if (!c) return LARQL_E_ARG;
     std::lock_guard<std::mutex> lk(c->mu);
     HIPCHECK(c, hipSetDevice(c->device));
-    HIPCHECK(c, hipStreamSynchronize(c->stream));
+    HIPCHECK(c, wait_stream(c));
     return LARQL_OK;
 }
 int larql_hip_event_create(larql_hip_ctx *c, void **event) {
@@ -1307,7 +1403,7 @@ int larql_hip_sequence_create(larql_hip_ctx *c, larql_hip_plan *const *plans, si
     // once eagerly: whatever a kernel's first launch sets up (its LDS limit) happens outside the recording
     for (size_t i = 0; i < n_plans; i++)
         for (const PreparedLaunch &P : plans[i]->launches) HIPCHECK(c, gemv_launch(c->stream, P.kind, P.L, P.threads, P.grid, P.lds));
-    HIPCHECK(c, hipStreamSynchronize(c->stream));
+    HIPCHECK(c, wait_stream(c));
     larql_hip_sequence *seq = new larql_hip_sequence();
     hipError_t e = hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal);
     if (e == hipSuccess) {
@@ -1408,7 +1504,7 @@ int larql_hip_dev_take_nan_flag(larql_hip_ctx *c, int *flag_out) {
     HIPCHECK(c, hipSetDevice(c->device));
     int v = 0;
     HIPCHECK(c, hipMemcpyAsync(&v, c->nan_flag, sizeof(int), hipMemcpyDeviceToHost, c->stream));
-    HIPCHECK(c, hipStreamSynchronize(c->stream));
+    HIPCHECK(c, wait_stream(c));
     *flag_out = v != 0;
     if (v) { int rc = clear_nan_flag(c); if (rc) return rc; }
     return LARQL_OK;
