@@ -478,6 +478,44 @@ def run_c4(be, fmt, args):
                "sample": f"one 2880x2880 MXFP4 matvec (dequant-order loop, rows in chunks of 32 over the threads), median of {nrep}, scaled by {3 * T * k} matvecs"}, higher=False)
         for p in (x, lg, de, dw, out, ws):
             be.free(p)
+    # The same bank handed over as MoeLayerWeights brings it (per-expert slices + Paired exponent streams + router_proj):
+    # residual -> output with the router's projection on the device.
+    G = H // 32
+    fph, fsh = be.d2h(fp, E * per, np.uint8), be.d2h(fs, E * per // 16, np.uint8)
+    dph, dsh = be.d2h(bufs["down"][0], E * per // 2, np.uint8), be.d2h(bufs["down"][1], E * per // 32, np.uint8)
+    gu_p, gu_s = [fph[e * per:(e + 1) * per] for e in range(E)], [fsh[e * per // 16:(e + 1) * per // 16] for e in range(E)]
+    dn_p, dn_s = [dph[e * per // 2:(e + 1) * per // 2] for e in range(E)], [dsh[e * per // 32:(e + 1) * per // 32] for e in range(E)]
+    rng = np.random.default_rng(0x5EED04A0)
+    router_w = (rng.standard_normal((E, H)) * 0.05).astype(np.float32)
+    layer = be.moe_layer_create(gu_p, dn_p, gu_s, dn_s, router_w, k, H, I, fmt.MOE_ROWS_INTERLEAVED)
+    assert layer, be.last_error()
+    for T in (1, 16):
+        x = be.malloc(T * H * 4 + 64)
+        be.dev_fill_normal(x, T * H, 0x5EED04F0 + T, 1.0)
+        de, dw, out = be.malloc(T * k * 4), be.malloc(T * k * 4), be.malloc(T * H * 4)
+
+        def layer_fwd():
+            be.dev_moe_layer_forward(layer, x, x, T, out, de, dw)
+        layer_fwd(); be.synchronize()
+        xv = be.d2h(x, (T, H), np.float32)
+        experts, wts = be.d2h(de, (T, k), np.uint32), be.d2h(dw, (T, k), np.float32)
+        want_route = O.moe_route_from_router_input(xv[0], router_w, None, k)
+        assert [int(e) for e in experts[0]] == [e for e, _ in want_route] and np.allclose(wts[0], [w for _, w in want_route], rtol=5e-5)
+        want = O.moe_block_mxfp4(xv[:1], experts[:1].astype(np.uint64), wts[:1], (fph, fsh), None, (dph, dsh), E, H, I, interleaved=True)
+        got = be.d2h(out, (T, H), np.float32)[:1]
+        rel = float(np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want))
+        assert rel < 1e-3, rel
+        distinct = len(set(int(v) for v in experts.reshape(-1)))
+        ms = _timeit(be, layer_fwd, args.steps)
+        algo = distinct * expert_bytes + E * H * 4 + T * (8 * H + 4 * E)
+        _emit(f"MXFP4 MoE layer us, router projection included (per-expert slices, batch {T})", round(ms * 1e3, 2), "us/block", ms, args.steps, 2,
+              {"workload": f"BASELINE configs[3] as MoeLayerWeights hands it over: 32 per-expert slices, router_proj 32x2880 on the device, top-4, batch {T}",
+               "distinct_experts": distinct, "launches_per_block": 3 if T == 1 else 5, "verified_rel_l2_vs_oracle": rel},
+              {"kernel": "f32 gemv (router) + gemv_mxfp4 (gate/up, down)", "bound": "hbm", "achieved": round(algo / ms / 1e6, 1), "peak": HBM_PEAK_GBS,
+               "unit": "GB/s", "frac": round(algo / ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": None}, None, higher=False)
+        for p in (x, de, dw, out):
+            be.free(p)
+    be.moe_layer_destroy(layer)
 
 
 def run_c5(be, fmt, args):

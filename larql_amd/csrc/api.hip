@@ -528,6 +528,26 @@ int larql_hip_get_submission_clock(larql_hip_ctx *c, larql_hip_submission_clock 
 
 // ---- host tier: quantised matvec -------------------------------------------------
 
+// Where a host-tier call's f32 result goes: page-locked host memory the kernel writes itself when it is small
+// (no copy back), the context's device buffer otherwise.
+struct ResultArea {
+    float *dev;
+    bool direct;
+};
+static int result_area(larql_hip_ctx *c, size_t bytes, ResultArea &r) {
+    r.direct = bytes <= kPinSmall && ensure_pinned(c, c->pin_out, kPinSmall + 64) == LARQL_OK;
+    if (!r.direct) { int rc = ensure(c, c->out, bytes + 64); if (rc) return rc; }
+    r.dev = (float *)(r.direct ? c->pin_out.dev : c->out.p);
+    return LARQL_OK;
+}
+// ends the submission (one wait for the stream) and leaves the result in `dst`
+static int finish_with_result(larql_hip_ctx *c, Submission &sub, const ResultArea &r, void *dst, size_t bytes) {
+    if (!r.direct) HIPCHECK(c, hipMemcpyAsync(dst, r.dev, bytes, hipMemcpyDeviceToHost, c->stream));
+    const int rc = sub.finish();
+    if (rc == LARQL_OK && r.direct) memcpy(dst, c->pin_out.host, bytes);
+    return rc;
+}
+
 static int host_matvec_multi(larql_hip_ctx *c, int kind, size_t n_mats, const uint8_t *const *w, const size_t *w_len,
                              const uint8_t *const *aux, const size_t *aux_len, const size_t *rows, size_t k,
                              const float *x, size_t x_bytes, float *const *out) {
@@ -701,7 +721,8 @@ int larql_hip_q4k_q8k_gemm(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len,
         pack_q8k(packed.data() + s * stride, qs + s * cols, d + s * (cols / 256), sums + s * (cols / 32), cols);
     int rc = upload(c, c->x, (const float *)packed.data(), packed.size());
     if (rc) return rc;
-    rc = ensure(c, c->out, out_len * sizeof(float) + 64);
+    ResultArea res;
+    rc = result_area(c, out_len * sizeof(float), res);
     if (rc) return rc;
     const uint8_t *dw = nullptr;
     rc = resolve_weights(c, q4k, need, c->w[0], &dw);
@@ -709,12 +730,11 @@ int larql_hip_q4k_q8k_gemm(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len,
     std::vector<GemvJob> jobs;
     jobs.reserve(seq);
     for (size_t s = 0; s < seq; s++)
-        jobs.push_back(make_job(KIND_Q4K_Q8K, dw, nullptr, (const uint8_t *)c->x.p + s * stride, (float *)c->out.p + s * num_rows, num_rows, cols));
+        jobs.push_back(make_job(KIND_Q4K_Q8K, dw, nullptr, (const uint8_t *)c->x.p + s * stride, res.dev + s * num_rows, num_rows, cols));
     Submission sub(c);
     rc = enqueue_jobs(c, jobs);
-    if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
-    HIPCHECK(c, hipMemcpyAsync(out, c->out.p, out_len * sizeof(float), hipMemcpyDeviceToHost, c->stream));
-    return sub.finish();
+    if (rc) { (void)wait_stream(c); return rc; }
+    return finish_with_result(c, sub, res, out, out_len * sizeof(float));
 }
 
 int larql_hip_q6k_q8k_matvec(larql_hip_ctx *c, const uint8_t *q6k, size_t q6k_len, const int8_t *qs, size_t qs_len, const float *d,
@@ -932,14 +952,14 @@ int larql_hip_q4_matvec(larql_hip_ctx *c, const uint8_t *q4, size_t q4_len, cons
     if (rc) return rc;
     rc = upload(c, c->q8s, q8_scales, n_scales * 4);
     if (rc) return rc;
-    rc = ensure(c, c->out, num_rows * 4 + 64);
+    ResultArea res;
+    rc = result_area(c, num_rows * 4, res);
     if (rc) return rc;
-    std::vector<GemvJob> jobs{make_job(KIND_Q4_0, dw, c->q8s.p, c->q8.p, (float *)c->out.p, num_rows, hidden)};
+    std::vector<GemvJob> jobs{make_job(KIND_Q4_0, dw, c->q8s.p, c->q8.p, res.dev, num_rows, hidden)};
     Submission sub(c);
     rc = enqueue_jobs(c, jobs);
-    if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
-    HIPCHECK(c, hipMemcpyAsync(out, c->out.p, num_rows * 4, hipMemcpyDeviceToHost, c->stream));
-    return sub.finish();
+    if (rc) { (void)wait_stream(c); return rc; }
+    return finish_with_result(c, sub, res, out, num_rows * 4);
 }
 
 int larql_hip_q8_0_gemv(larql_hip_ctx *c, const uint8_t *blocks, size_t blocks_len, const float *x, size_t x_len, size_t n,
@@ -975,14 +995,14 @@ int larql_hip_quant_matvec(larql_hip_ctx *c, int format, const uint8_t *weights,
             if (rc) return rc;
             rc = ensure(c, c->q8, hidden + 64); if (rc) return rc;
             rc = ensure(c, c->q8s, (hidden / 32) * 4 + 64); if (rc) return rc;
-            rc = ensure(c, c->out, num_rows * 4 + 64); if (rc) return rc;
+            ResultArea res;
+            rc = result_area(c, num_rows * 4, res); if (rc) return rc;
             Submission sub(c);
             HIPCHECK(c, quantize_to_q8_launch(c->stream, (const float *)c->x.p, hidden, (int8_t *)c->q8.p, (float *)c->q8s.p));
-            std::vector<GemvJob> jobs{make_job(KIND_Q4_0, dw, c->q8s.p, c->q8.p, (float *)c->out.p, num_rows, hidden)};
+            std::vector<GemvJob> jobs{make_job(KIND_Q4_0, dw, c->q8s.p, c->q8.p, res.dev, num_rows, hidden)};
             rc = enqueue_jobs(c, jobs);
-            if (rc) { (void)hipStreamSynchronize(c->stream); return rc; }
-            HIPCHECK(c, hipMemcpyAsync(out, c->out.p, num_rows * 4, hipMemcpyDeviceToHost, c->stream));
-            return sub.finish();
+            if (rc) { (void)wait_stream(c); return rc; }
+            return finish_with_result(c, sub, res, out, num_rows * 4);
         }
         default:
             // Q5_K, I2S, MXFP4 (external scales), the trait's own Q8_0 layout and the
