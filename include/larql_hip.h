@@ -403,7 +403,9 @@ int larql_hip_dev_q4k_gemm_prepared(larql_hip_ctx *ctx, const uint8_t *w, const 
  * of `n_experts` logits per token (ties: first index), weights softmaxed over
  * the selected logits (policy 1, NormalisedOverSelected: GPT-OSS) or over all
  * experts (policy 0, SoftmaxThenSelect).  experts/weights are [tokens, k].
- * n_experts <= 64, k <= 8. */
+ * n_experts <= 256, k <= 8 (a launch of the expert block selects for itself up to 64
+ * experts; a wider bank — 128 in the larger GPT-OSS and Gemma 4 checkpoints — goes through the
+ * selection kernel first). */
 int larql_hip_dev_router_select(larql_hip_ctx *ctx, const float *logits, size_t tokens, size_t n_experts, size_t k,
                                 int policy, uint32_t *experts, float *weights);
 /* One bank of MXFP4 experts: gate/up are [n_experts, inter, hidden] and down is
@@ -458,7 +460,7 @@ int larql_hip_dev_moe_mxfp4_routed(larql_hip_ctx *ctx, const larql_hip_mxfp4_exp
  * a ContiguousHalves bank apart), so the caller gathers nothing.  Served: expert_data_format MXFP4 with Paired scales
  * (what a native GPT-OSS bank is; the CPU tier refuses it, cpu/ops/moe/forward.rs:69-75) and MoeGateRule::ClampedGlu;
  * MXFP4 with Inline scales is LARQL_REFUSED_SHAPE (the format keeps its exponents apart: there is nothing to read them
- * from), other formats LARQL_UNSUPPORTED.  num_experts <= 64, top_k <= 8. */
+ * from), other formats LARQL_UNSUPPORTED.  num_experts <= 256, top_k <= 8. */
 enum { LARQL_MOE_SCALES_INLINE = 0, LARQL_MOE_SCALES_PAIRED = 1 };
 enum { LARQL_MOE_ROWS_CONTIGUOUS_HALVES = 0, LARQL_MOE_ROWS_INTERLEAVED = 1 };
 typedef struct {

@@ -197,7 +197,7 @@ impl HipBackend {
     /// A MoE layer made resident from `MoeLayerWeights` (crates/larql-compute/src/pipeline/moe.rs:469-541): the
     /// per-expert slices and their paired exponent streams go up expert by expert, wherever their mmap ranges lie.
     /// `None` where this backend has no kernel for the layer (anything but an MXFP4 bank with `Paired` scales and
-    /// `ClampedGlu`, more than 64 experts, top-k above 8) — the caller keeps `cpu_moe_forward`.
+    /// `ClampedGlu`, more than 256 experts, top-k above 8) — the caller keeps `cpu_moe_forward`.
     pub fn moe_layer<'a>(&'a self, moe: &MoeLayerWeights<'_>, hidden: usize) -> Option<HipMoeLayer<'a>> {
         let (limit, alpha) = match moe.gate_rule {
             MoeGateRule::ClampedGlu { limit, alpha } => (limit, alpha),

@@ -1667,7 +1667,7 @@ int larql_hip_dev_router_select(larql_hip_ctx *c, const float *logits, size_t to
     std::lock_guard<std::mutex> lk(c->mu);
     if (k > n_experts) k = n_experts;  // select(): k.min(logits.len())
     if (tokens == 0 || k == 0) return LARQL_OK;
-    if (n_experts > 64 || k > 8) return fail(c, LARQL_UNSUPPORTED, "router_select: at most 64 experts and top-8 on this backend");
+    if (n_experts > kRouterMaxExperts || k > 8) return fail(c, LARQL_UNSUPPORTED, "router_select: at most 256 experts and top-8 on this backend");
     if (!logits || !experts || !weights) return LARQL_E_ARG;
     HIPCHECK(c, hipSetDevice(c->device));
     HIPCHECK(c, router_select_launch(c->stream, logits, nullptr, (uint32_t)tokens, (uint32_t)n_experts, (uint32_t)k, policy, experts, weights));
@@ -1697,6 +1697,12 @@ static int moe_mxfp4_block(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank
         (!bank->gate_up_interleaved && (!bank->up_packed || !bank->up_scales)))
         return LARQL_E_ARG;
     HIPCHECK(c, hipSetDevice(c->device));
+    if (route_logits && tokens == 1 && bank->n_experts > kRouterInLaunchExperts) {
+        // more experts than a matvec launch selects over by itself: the selection kernel first, then the block on its choice
+        HIPCHECK(c, router_select_launch(c->stream, route_logits, bank->router_bias, 1, (uint32_t)bank->n_experts, (uint32_t)k, route_policy, experts,
+                                         weights));
+        route_logits = nullptr;
+    }
     const size_t slots = tokens * k;
     float *g = (float *)workspace, *u = g + slots * inter, *h = u + slots * inter, *d = h + slots * inter;
     // fused: every expert's gate_up region is one matrix of 2*inter interleaved rows (gate even, up odd), walked in
@@ -1757,7 +1763,7 @@ static int moe_mxfp4_block(larql_hip_ctx *c, const larql_hip_mxfp4_experts *bank
         }
         uint32_t gt = 0, dt = 0;
         size_t gl = 0, dl = 0;
-        if (gu_rows < (1u << 22) && hidden < (1u << 22) && c->cu_count <= 512 && (!route_logits || bank->n_experts <= 64) && moe1_geometry(ga, &gt, &gl) &&
+        if (gu_rows < (1u << 22) && hidden < (1u << 22) && c->cu_count <= 512 && (!route_logits || bank->n_experts <= kRouterInLaunchExperts) && moe1_geometry(ga, &gt, &gl) &&
             moe1_geometry(da, &dt, &dl)) {
             const uint32_t cus = (uint32_t)c->cu_count;
             // a short result is cut into tiles of fewer than 16 rows so that every compute unit gets the same share
@@ -1910,7 +1916,7 @@ int larql_hip_dev_moe_mxfp4_routed(larql_hip_ctx *c, const larql_hip_mxfp4_exper
     std::lock_guard<std::mutex> lk(c->mu);
     if (k > bank->n_experts) k = bank->n_experts;  // select(): k.min(logits.len())
     if (tokens == 0 || k == 0) return LARQL_OK;
-    if (bank->n_experts > 64 || k > 8) return fail(c, LARQL_UNSUPPORTED, "router_select: at most 64 experts and top-8 on this backend");
+    if (bank->n_experts > kRouterMaxExperts || k > 8) return fail(c, LARQL_UNSUPPORTED, "router_select: at most 256 experts and top-8 on this backend");
     if (!router_logits) return LARQL_E_ARG;
     return moe_mxfp4_block(c, bank, x, tokens, k, experts, weights, out, workspace, workspace_bytes, router_logits, policy);
 }
@@ -1945,7 +1951,7 @@ int larql_hip_moe_layer_create(larql_hip_ctx *c, const larql_hip_moe_layer_weigh
         return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: an MXFP4 bank keeps its e8m0 exponents in a partner stream (MoeExpertScales::Paired)");
     const size_t E = w->num_experts, hidden = w->hidden, inter = w->intermediate_size;
     if (E == 0 || w->top_k == 0 || hidden == 0 || inter == 0) return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: empty layer");
-    if (E > 64 || std::min(w->top_k, E) > 8) return fail(c, LARQL_UNSUPPORTED, "moe_layer: at most 64 experts and top-8 on this backend");
+    if (E > kRouterMaxExperts || std::min(w->top_k, E) > 8) return fail(c, LARQL_UNSUPPORTED, "moe_layer: at most 256 experts and top-8 on this backend");
     if (hidden % 32 != 0 || inter % 32 != 0) return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: hidden and intermediate_size must be multiples of 32");
     if (w->fused_row_layout != LARQL_MOE_ROWS_INTERLEAVED && w->fused_row_layout != LARQL_MOE_ROWS_CONTIGUOUS_HALVES)
         return fail(c, LARQL_E_ARG, "moe_layer: unknown fused row layout");

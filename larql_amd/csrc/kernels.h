@@ -183,9 +183,11 @@ bool moe1_geometry(Moe1Args &A, uint32_t *threads, size_t *lds);  // fills cw / 
 hipError_t moe1_launch(hipStream_t s, const Moe1Args &A, bool down, uint32_t grid, uint32_t threads, size_t lds);
 
 // MoE helpers
+constexpr uint32_t kRouterMaxExperts = 256;      // the selection kernel and the planner (four logits per lane)
+constexpr uint32_t kRouterInLaunchExperts = 64;  // a matvec launch that selects for itself (one logit per lane)
 hipError_t router_select_launch(hipStream_t s, const float *logits, const float *bias, uint32_t tokens, uint32_t n_experts, uint32_t k,
                                 int policy, uint32_t *experts, float *weights);
-// (logits != nullptr: the kernel selects the experts itself first — at most 64 experts, top-kRouterMaxK — and writes experts / weights)
+// (logits != nullptr: the kernel selects the experts itself first — at most kRouterMaxExperts, top-kRouterMaxK — and writes experts / weights)
 hipError_t moe_plan_launch(hipStream_t s, const float *logits, const float *router_bias, int policy, float *weights, uint32_t *experts,
                            uint32_t slots, uint32_t k, uint32_t n_experts, const GemvJob &tg,
                            const GemvJob &tu, const GemvJob &td, uint64_t gu_w_stride, uint64_t gu_s_stride, uint64_t dn_w_stride,

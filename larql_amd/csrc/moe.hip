@@ -8,6 +8,8 @@
 
 namespace larql {
 
+static_assert(kRouterMaxExperts == 64u * (uint32_t)kRouterWideSlots, "the wide selection holds kRouterMaxExperts logits");
+
 // router::select for every token: one wavefront per token (router.h).
 __global__ void __launch_bounds__(64) router_select_kernel(const float *__restrict__ logits, const float *__restrict__ bias, uint32_t n_experts,
                                                            uint32_t k, int policy, uint32_t *__restrict__ experts,
@@ -15,7 +17,7 @@ __global__ void __launch_bounds__(64) router_select_kernel(const float *__restri
     const uint32_t t = blockIdx.x, lane = threadIdx.x;
     uint32_t sel_idx[kRouterMaxK];
     float sel_w[kRouterMaxK];
-    router_select_wave(logits + (size_t)t * n_experts, bias, n_experts, k, policy, lane, sel_idx, sel_w);
+    router_select_any(logits + (size_t)t * n_experts, bias, n_experts, k, policy, lane, sel_idx, sel_w);
     if (lane == 0) {
 #pragma unroll
         for (int r = 0; r < kRouterMaxK; r++)
@@ -116,7 +118,7 @@ __global__ void __launch_bounds__(1024) moe_plan_kernel(const float *__restrict_
         for (uint32_t tok = t >> 6; tok < tokens; tok += blockDim.x >> 6) {
             uint32_t sel_idx[kRouterMaxK];
             float sel_w[kRouterMaxK];
-            router_select_wave(logits + (size_t)tok * n_experts, router_bias, n_experts, k, policy, lane, sel_idx, sel_w);
+            router_select_any(logits + (size_t)tok * n_experts, router_bias, n_experts, k, policy, lane, sel_idx, sel_w);
             if (lane == 0) {
 #pragma unroll
                 for (int r = 0; r < kRouterMaxK; r++)

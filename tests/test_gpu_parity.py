@@ -855,7 +855,34 @@ def test_router_select_matches_oracle(be):
             assert np.allclose(w[t], [x for _, x in want], rtol=2e-6, atol=1e-7)
     assert [int(v) for v in e[0]] == [0, 1, 2, 3] and [int(v) for v in e[2][:2]] == [5, 9]
     assert be.dev_router_select(dl, T, E, 0, 1, de, dw)                  # k == 0: nothing to do
-    assert not be.dev_router_select(dl, T, 65, 4, 1, de, dw)             # beyond this kernel: refused
+    assert not be.dev_router_select(dl, T, 257, 4, 1, de, dw)            # beyond this kernel: refused
+
+
+@pytest.mark.parametrize("E,k", [(65, 4), (128, 4), (128, 8), (200, 8), (256, 8), (129, 1)])
+def test_router_select_over_wide_banks_matches_oracle(be, E, k):
+    """Banks of more than 64 experts (128 in the larger GPT-OSS and Gemma 4 checkpoints): a lane holds up to four logits.
+    Same rule — logit descending, the lower index wins a tie, wherever the tied experts sit — both weight policies."""
+    rng = np.random.default_rng(1000 + E + k)
+    T = 40
+    logits = rng.standard_normal((T, E)).astype(F)
+    logits[0, :] = 1.0                                   # all tied -> the first k indices
+    j1 = 69 if E > 69 else E - 1
+    logits[1, 5] = logits[1, j1] = 4.0                   # a tie between two logits of one lane (where the bank has both)
+    logits[2, E - 1] = 5.0; logits[2, 3] = 5.0           # ... and between lanes of different quarters
+    logits[3, :] = -np.arange(E, dtype=F)                # descending by index
+    logits[4, :] = np.arange(E, dtype=F) * F(0.01)       # the last experts win
+    logits[5, :] = -1e30; logits[5, E - 2] = 0.0         # one expert takes all the weight
+    dl, de, dw = be.to_device(logits), be.malloc(T * k * 4), be.malloc(T * k * 4)
+    for policy in (O.NORMALISED_OVER_SELECTED, O.SOFTMAX_THEN_SELECT):
+        assert be.dev_router_select(dl, T, E, k, policy, de, dw)
+        e, w = be.d2h(de, (T, k), np.uint32), be.d2h(dw, (T, k), F)
+        for t in range(T):
+            want = O.router_select(logits[t], k, policy)
+            assert [int(v) for v in e[t]] == [i for i, _ in want], (policy, t)
+            assert np.allclose(w[t], [x for _, x in want], rtol=4e-6, atol=1e-7), (policy, t)
+    assert [int(v) for v in e[0]] == list(range(k))
+    if k >= 2:
+        assert [int(v) for v in e[1][:2]] == [5, j1] and [int(v) for v in e[2][:2]] == [3, E - 1]
 
 
 def _mx_bank(rng, E, n, kk, sigma=0.02):
@@ -1003,11 +1030,13 @@ def test_moe_mxfp4_tokens_sharing_an_expert_equal_single_token_calls(be, fmt):
 
 @pytest.mark.parametrize("T,E,hidden,inter,interleaved,policy", [(1, 8, 2880, 2880, 0, 1), (1, 8, 2880, 2880, 1, 1), (1, 6, 384, 320, 0, 0),
                                                                  (1, 64, 384, 320, 1, 1), (5, 6, 384, 320, 0, 1), (1, 3, 96, 64, 0, 1), (16, 32, 384, 320, 1, 1),
-                                                                 (32, 9, 384, 320, 0, 0), (40, 12, 384, 320, 0, 1)])
+                                                                 (32, 9, 384, 320, 0, 0), (40, 12, 384, 320, 0, 1),
+                                                                 (1, 128, 384, 320, 1, 1), (1, 200, 96, 64, 0, 0), (5, 128, 384, 320, 0, 1),
+                                                                 (20, 256, 96, 64, 0, 1)])
 def test_moe_mxfp4_routed_equals_select_then_block(be, fmt, T, E, hidden, inter, interleaved, policy):
     """Selection and expert block as one call: experts, weights and output bit for bit those of the two calls (one
     token: the selection runs inside the first matvec launch; k = 96 rows are below what that kernel takes and
-    several tokens go through the selection kernel)."""
+    several tokens go through the selection kernel; so does a bank of more than 64 experts)."""
     rng = np.random.default_rng(500 + E + T)
     k = min(4, E)
     g_rows = 2 * inter if interleaved else inter
@@ -1140,6 +1169,9 @@ def test_moe_mxfp4_interleaved_gate_up_bank_equals_separate_banks(be, fmt, T, E,
     (5, 6, 384, 320, "interleaved", True, True),          # several tokens, MoeExpertScalePolicy::PerExpert
     (9, 8, 2880, 576, "halves", True, False),             # ... and the softmax's own values (no renormalisation)
     (1, 4, 96, 64, "interleaved", True, True),            # rows the matrix-core kernels do not take
+    (1, 128, 384, 320, "interleaved", False, True),       # 128 experts, top-8 (Gemma 4 26B-A4B's count): one token
+    (6, 128, 384, 320, "halves", True, True),             # ... several tokens, per-expert scale
+    (3, 128, 384, 320, "interleaved", False, False),      # ... the planner selects
 ])
 def test_moe_layer_from_per_expert_slices_with_router_projection(be, fmt, T, E, hidden, inter, layout, per_expert, renorm):
     """MoeLayerWeights as the reference brings it (pipeline/moe.rs:469-541): per-expert gate+up / down slices in
@@ -1148,7 +1180,7 @@ def test_moe_layer_from_per_expert_slices_with_router_projection(be, fmt, T, E, 
     projection on the device: the route equals moe_route_from_router_input (mod.rs:149-186), the output the checker's
     expert block under that route; host tier and device tier agree bit for bit."""
     rng = np.random.default_rng(211 + T + E)
-    k, G, Gd = 4, hidden // 32, inter // 32
+    k, G, Gd = (8 if E > 64 else 4), hidden // 32, inter // 32
     gate = [O.quantize_mxfp4((rng.standard_normal(inter * hidden) * 0.02).astype(F), inter, hidden) for _ in range(E)]
     up = [O.quantize_mxfp4((rng.standard_normal(inter * hidden) * 0.02).astype(F), inter, hidden) for _ in range(E)]
     down = [O.quantize_mxfp4((rng.standard_normal(hidden * inter) * 0.02).astype(F), hidden, inter) for _ in range(E)]
@@ -1202,7 +1234,7 @@ def test_moe_layer_from_per_expert_slices_with_router_projection(be, fmt, T, E, 
 
 def test_moe_layer_refusals(be, fmt):
     """What MoeLayerWeights can say and this backend does not serve answers None (never a wrong bank): inline scales on
-    an MXFP4 bank, another expert format, slices shorter than the geometry, more than 64 experts."""
+    an MXFP4 bank, another expert format, slices shorter than the geometry, more than 256 experts."""
     rng = np.random.default_rng(3)
     E, hidden, inter, k = 3, 64, 32, 2
     gu = [O.quantize_mxfp4((rng.standard_normal(2 * inter * hidden) * 0.02).astype(F), 2 * inter, hidden) for _ in range(E)]
@@ -1216,7 +1248,7 @@ def test_moe_layer_refusals(be, fmt):
     assert be.moe_layer_create(*args, expert_data_format=fmt.FMT_Q4_K) is None
     short = ([g[0][:-16] for g in gu],) + args[1:]
     assert be.moe_layer_create(*short) is None
-    many = ([gu[0][0]] * 65, [dn[0][0]] * 65, [gu[0][1]] * 65, [dn[0][1]] * 65, np.zeros((65, hidden), F), k, hidden, inter)
+    many = ([gu[0][0]] * 257, [dn[0][0]] * 257, [gu[0][1]] * 257, [dn[0][1]] * 257, np.zeros((257, hidden), F), k, hidden, inter)
     assert be.moe_layer_create(*many) is None
 
 
