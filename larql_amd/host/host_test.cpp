@@ -5,6 +5,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <vector>
 
 #include "hip_backend.hpp"
 
@@ -108,6 +109,127 @@ int main() {
     auto hits = be.gate_knn(larql::QuantFormat::F32, larql::Slice<uint8_t>((const uint8_t *)gate.data(), gate.size() * 4), res, 4, 256, 2);
     CHECK(hits.has_value() && hits->size() == 2 && (*hits)[0].first == 1 && (*hits)[1].first == 2);
     CHECK(std::fabs((*hits)[0].second + 0.9f) < 1e-6);
+
+    // the batch forms: one hit list per position, the union gate_knn_batch returns, the full score matrix
+    {
+        std::vector<float> res2(2 * 256, 0.0f);
+        for (int i = 0; i < 4; i++) res2[i] = res[i];
+        res2[256 + 0] = 0.7f; res2[256 + 3] = -0.2f;
+        const larql::Slice<uint8_t> g8((const uint8_t *)gate.data(), gate.size() * 4);
+        auto per = be.gate_knn_positions(larql::QuantFormat::F32, g8, res2, 2, 4, 256, 2);
+        CHECK(per && per->size() == 2 && (*per)[0].size() == 2 && (*per)[1].size() == 2);
+        CHECK((*per)[0][0].first == 1 && (*per)[0][1].first == 2 && (*per)[1][0].first == 0 && (*per)[1][1].first == 3);
+        auto uni = be.gate_knn_batch(larql::QuantFormat::F32, g8, res2, 2, 4, 256, 2);
+        CHECK(uni && *uni == (std::vector<size_t>{0, 1, 2, 3}));
+        auto sc = be.gate_scores_batch(larql::QuantFormat::F32, g8, res2, 2, 4, 256);
+        CHECK(sc && sc->size() == 8 && std::fabs((*sc)[1] + 0.9f) < 1e-6 && std::fabs((*sc)[4] - 0.7f) < 1e-6 && (*sc)[5] == 0.0f);
+        CHECK(!be.gate_knn_positions(larql::QuantFormat::F32, g8, res2, 3, 4, 256, 2));          // x is not [3, 256]
+        auto all = be.gate_knn(larql::QuantFormat::F32, g8, res, 4, 256, (size_t)1 << 40);          // "every feature"
+        CHECK(all && all->size() == 4);
+    }
+
+    // Q8-input forms (quant_matvec.rs:100-151): codes 2 x scale 0.5 = the activation 1.0 -> the f32 call's bits
+    {
+        std::vector<int8_t> q8(hidden, 2);
+        std::vector<float> q8s(hidden / 32, 0.5f);
+        auto o = be.quant_matvec_q8_input(larql::QuantFormat::Q4_K, w, q8, q8s, rows, hidden);
+        CHECK(o && *o == *out);
+        CHECK(!be.quant_matvec_q8_input(larql::QuantFormat::MXFP4, w, q8, q8s, rows, hidden));
+        // Q4_0: d = 0.5, every nibble 10 -> weight 1.0; activation 3 x 0.25 -> 0.75; 64 of them -> 48
+        std::vector<uint8_t> q40(3 * 2 * 18);
+        for (size_t b = 0; b < 6; b++) { q40[b * 18] = 0x00; q40[b * 18 + 1] = 0x38; std::memset(&q40[b * 18 + 2], 0xAA, 16); }
+        std::vector<int8_t> q8b(64, 3);
+        std::vector<float> q8bs(2, 0.25f);
+        auto o4 = be.q4_matvec(q40, q8b, q8bs, 3, 64);
+        CHECK(o4 && o4->size() == 3 && (*o4)[0] == 48.0f && (*o4)[2] == 48.0f);
+        auto o4b = be.quant_matvec_q8_input(larql::QuantFormat::Q4_0, q40, q8b, q8bs, 3, 64);
+        CHECK(o4b && *o4b == *o4);
+    }
+
+    // ggml Q8_0 head: row r has d = 1 and every code r + 1; x = 1 over k = 64 -> 64 (r + 1); top-2 by value = rows 4, 3
+    {
+        const size_t n = 5, k = 64;
+        std::vector<uint8_t> q8w(n * 2 * 34);
+        for (size_t r = 0; r < n; r++)
+            for (size_t b = 0; b < 2; b++) {
+                uint8_t *blk = &q8w[(r * 2 + b) * 34];
+                blk[0] = 0x00; blk[1] = 0x3C;
+                std::memset(blk + 2, (int)(r + 1), 32);
+            }
+        std::vector<float> ones(k, 1.0f);
+        auto o = be.q8_0_gemv(q8w, ones, n, k);
+        CHECK(o && o->size() == n);
+        for (size_t r = 0; r < n; r++) CHECK((*o)[r] == 64.0f * (float)(r + 1));
+        auto top = be.q8_0_gemv_topk(q8w, ones, n, k, 2);
+        CHECK(top && top->size() == 2 && (*top)[0].first == 4 && (*top)[0].second == 320.0f && (*top)[1].first == 3);
+        auto every = be.q8_0_gemv_topk(q8w, ones, n, k, 1000);   // K beyond the rows: all of them, in order
+        CHECK(every && every->size() == n && (*every)[4].first == 0);
+        CHECK(!be.q8_0_gemv(q8w, ones, n, 48));
+    }
+
+    // dense gemv: bf16 / f16 rows of 2^r against x = 1 (exact), the multi forms equal to the single calls, a bad
+    // matrix refusing the whole batch, the unforced call leaving a tiny matrix to the caller's BLAS
+    {
+        const size_t n = 4, k = 64;
+        const uint16_t bf[4] = {0x3F00, 0x3F80, 0x4000, 0x4080}, hf[4] = {0x3800, 0x3C00, 0x4000, 0x4400};  // 0.5, 1, 2, 4
+        std::vector<uint8_t> wb(n * k * 2), wh(n * k * 2);
+        for (size_t r = 0; r < n; r++)
+            for (size_t c = 0; c < k; c++) { std::memcpy(&wb[(r * k + c) * 2], &bf[r], 2); std::memcpy(&wh[(r * k + c) * 2], &hf[r], 2); }
+        std::vector<float> ones(k, 1.0f);
+        auto ob = be.bf16_gemv_force(wb, ones, n, k), oh = be.f16_gemv_force(wh, ones, n, k);
+        CHECK(ob && oh && (*ob)[0] == 32.0f && (*ob)[3] == 256.0f && *oh == *ob);
+        CHECK(!be.bf16_gemv(wb, ones, n, k) && !be.f16_gemv(wh, ones, n, k));       // below the flop threshold
+        CHECK(be.supports(larql::Capability::F16Gemv) && be.supports(larql::Capability::QuantMatVec));
+        std::vector<larql::DenseMatrix> three = {{wb, n, k}, {larql::Slice<uint8_t>(wb.data(), 2 * k * 2), 2, k}, {wb, n, k}};
+        auto mb = be.bf16_gemv_multi(three, ones);
+        CHECK(mb && mb->size() == 3 && (*mb)[0] == *ob && (*mb)[2] == *ob && (*mb)[1].size() == 2 && (*mb)[1][1] == 64.0f);
+        auto mh = be.f16_gemv_multi({{wh, n, k}}, ones);
+        CHECK(mh && mh->size() == 1 && (*mh)[0] == *oh);
+        three[1].k = 32;
+        CHECK(!be.bf16_gemv_multi(three, ones));
+        auto none = be.bf16_gemv_multi({}, ones);
+        CHECK(none && none->empty());
+        std::vector<float> wf(n * k);
+        for (size_t r = 0; r < n; r++) for (size_t c = 0; c < k; c++) wf[r * k + c] = (float)(r + 1);
+        auto of = be.f32_gemv_force(wf, ones, n, k);
+        CHECK(of && (*of)[2] == 192.0f && !be.f32_gemv(wf, ones, n, k));
+    }
+
+    // mxfp4_gemv_multi == the single calls
+    {
+        std::vector<uint8_t> p2(2 * 16, 0x22), s2 = {127, 128}, s3 = {126, 127};
+        auto mm2 = be.mxfp4_gemv_multi({{p2, s2, 2, 32}, {p2, s3, 2, 32}}, x32);
+        CHECK(mm2 && mm2->size() == 2 && (*mm2)[0][0] == 32.0f && (*mm2)[0][1] == 64.0f && (*mm2)[1][0] == 16.0f && (*mm2)[1][1] == 32.0f);
+        CHECK(!be.mxfp4_gemv_multi({{p2, s2, 2, 32}, {p2, s3, 2, 33}}, x32));
+    }
+
+    // A MoE layer from per-expert slices (MoeLayerWeights, pipeline/moe.rs:469-541), closed form: expert 0 is all ones
+    // (code 2, exponent 127), expert 1 all zeros; x = 1/128 makes every gate and up row dot 1.0, ClampedGlu gives
+    // (1 + 1) * sigmoid(1.702), the down rows sum 128 of those; the router's rows +1 / -1 pick expert 0 with weight 1.
+    {
+        const size_t H = 128, I = 128, G = H / 32;
+        std::vector<uint8_t> gu1(2 * I * G * 16, 0x22), gu0(2 * I * G * 16, 0x00), dn1(H * (I / 32) * 16, 0x22), dn0(H * (I / 32) * 16, 0x00);
+        std::vector<uint8_t> sgu(2 * I * G, 127), sdn(H * (I / 32), 127);
+        std::vector<float> rp(2 * H);
+        for (size_t c = 0; c < H; c++) { rp[c] = 1.0f; rp[H + c] = -1.0f; }
+        larql::MoeLayerWeights m;
+        m.experts_gate_up = {gu1, gu0}; m.experts_down = {dn1, dn0};
+        m.expert_scales.paired = true; m.expert_scales.gate_up = {sgu, sgu}; m.expert_scales.down = {sdn, sdn};
+        m.router_proj = rp; m.num_experts = 2; m.top_k = 1; m.intermediate_size = I;
+        auto layer = be.moe_layer(m, H);
+        CHECK(layer.has_value());
+        std::vector<float> xm(2 * H, 1.0f / 128.0f);
+        for (size_t c = 0; c < H; c++) xm[H + c] = -1.0f / 128.0f;   // the second token's logits are -1 / +1: expert 1, all zeros
+        auto r1 = layer->forward(xm, xm, 2);
+        CHECK(r1 && r1->experts.size() == 2 && r1->experts[0] == 0 && r1->experts[1] == 1 && r1->weights[0] == 1.0f && r1->weights[1] == 1.0f);
+        const double want = 128.0 * 2.0 / (1.0 + std::exp(-1.702));
+        for (size_t c = 0; c < H; c++) { CHECK(std::fabs(r1->out[c] - want) < 1e-4 * want); CHECK(r1->out[H + c] == 0.0f); }
+        CHECK(!layer->forward(xm, larql::Slice<float>(xm.data(), H), 2));                 // x is not [2, H]
+        m.expert_scales.paired = false;                                                    // Inline scales on an MXFP4 bank: refused
+        CHECK(!be.moe_layer(m, H));
+        m.expert_scales.paired = true; m.gate_rule.clamped_glu = false;                    // another gate rule: the caller's CPU path
+        CHECK(!be.moe_layer(m, H));
+    }
 
     auto clock = be.submission_clock();
     CHECK(clock.has_value() && clock->submissions > 0);
