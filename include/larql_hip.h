@@ -460,8 +460,17 @@ int larql_hip_dev_moe_mxfp4_routed(larql_hip_ctx *ctx, const larql_hip_mxfp4_exp
  * a ContiguousHalves bank apart), so the caller gathers nothing.  Served: expert_data_format MXFP4 with Paired scales
  * (what a native GPT-OSS bank is; the CPU tier refuses it, cpu/ops/moe/forward.rs:69-75) and MoeGateRule::ClampedGlu;
  * MXFP4 with Inline scales is LARQL_REFUSED_SHAPE (the format keeps its exponents apart: there is nothing to read them
- * from), other formats LARQL_UNSUPPORTED.  num_experts <= 256, top_k <= 8. */
+ * from).  Also served: expert_data_format Q4_K or Q6_K with Inline scales and ContiguousHalves rows — the per-layer
+ * k-quant files of Gemma 4 26B-A4B, what cpu_moe_forward's integer path reads (cpu/ops/moe/forward.rs:160-330,
+ * expert/q4k.rs:232-351): experts_gate_up[e] is [2*inter, cols] rows, gate half first, cols the stored row width (>= hidden,
+ * a multiple of 256, derived from the slice length as stored_gate_up_cols does, moe.rs:659-690); experts_down[e] is
+ * [hidden, ceil(inter/256)*256]; the scale tables are NULL; any LARQL_MOE_GATE_* rule.  The expert input is quantised to
+ * Q8_K once per token, the gated activation once per expert, and every matvec is the integer Q4_K x Q8_K (Q6_K x Q8_K)
+ * kernel, as on the CPU.  An Interleaved k-quant bank is LARQL_REFUSED_SHAPE (the CPU tier asserts the same,
+ * forward.rs:69-75); rows longer than 10240 elements and other formats LARQL_UNSUPPORTED.  num_experts <= 256, top_k <= 8. */
 enum { LARQL_MOE_SCALES_INLINE = 0, LARQL_MOE_SCALES_PAIRED = 1 };
+/* MoeGateRule (moe.rs:40-118): ClampedGlu{limit, alpha}, Gated(gelu_tanh), Gated(silu). */
+enum { LARQL_MOE_GATE_CLAMPED_GLU = 0, LARQL_MOE_GATE_GELU_TANH = 1, LARQL_MOE_GATE_SILU = 2 };
 enum { LARQL_MOE_ROWS_CONTIGUOUS_HALVES = 0, LARQL_MOE_ROWS_INTERLEAVED = 1 };
 typedef struct {
     size_t num_experts, top_k, hidden, intermediate_size;
@@ -484,6 +493,7 @@ typedef struct {
     int renormalized_softmax;                    /* MoeTopKWeightPolicy::RenormalizedSoftmax (else the softmax's own values) */
     int per_expert_scale;                        /* MoeExpertScalePolicy::PerExpert */
     float glu_limit, glu_alpha;                  /* MoeGateRule::ClampedGlu (GPT-OSS: 7, 1.702) */
+    int gate_rule;                               /* LARQL_MOE_GATE_* (0 = ClampedGlu with the two parameters above) */
 } larql_hip_moe_layer_weights;
 typedef struct larql_hip_moe_layer larql_hip_moe_layer;
 int  larql_hip_moe_layer_create(larql_hip_ctx *ctx, const larql_hip_moe_layer_weights *weights, larql_hip_moe_layer **out);

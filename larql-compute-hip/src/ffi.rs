@@ -50,12 +50,16 @@ pub struct MoeLayerWeights {
     pub per_expert_scale: c_int,
     pub glu_limit: f32,
     pub glu_alpha: f32,
+    pub gate_rule: c_int,
 }
 
 pub const MOE_SCALES_INLINE: c_int = 0;
 pub const MOE_SCALES_PAIRED: c_int = 1;
 pub const MOE_ROWS_CONTIGUOUS_HALVES: c_int = 0;
 pub const MOE_ROWS_INTERLEAVED: c_int = 1;
+pub const MOE_GATE_CLAMPED_GLU: c_int = 0;
+pub const MOE_GATE_GELU_TANH: c_int = 1;
+pub const MOE_GATE_SILU: c_int = 2;
 
 pub const OK: c_int = 0;
 

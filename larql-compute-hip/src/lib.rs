@@ -196,11 +196,17 @@ impl HipBackend {
 
     /// A MoE layer made resident from `MoeLayerWeights` (crates/larql-compute/src/pipeline/moe.rs:469-541): the
     /// per-expert slices and their paired exponent streams go up expert by expert, wherever their mmap ranges lie.
-    /// `None` where this backend has no kernel for the layer (anything but an MXFP4 bank with `Paired` scales and
-    /// `ClampedGlu`, more than 256 experts, top-k above 8) — the caller keeps `cpu_moe_forward`.
+    /// Served: an MXFP4 bank with `Paired` scales under `ClampedGlu` (a native GPT-OSS bank), and a Q4_K / Q6_K bank with
+    /// `Inline` scales and `ContiguousHalves` rows under `ClampedGlu` or `Gated` (the per-layer k-quant files of Gemma 4
+    /// 26B-A4B: `cpu_moe_forward`'s integer path, crates/larql-compute/src/cpu/ops/moe/forward.rs:160-330).  `None` where
+    /// this backend has no kernel for the layer (other formats or rules, more than 256 experts, top-k above 8) — the
+    /// caller keeps `cpu_moe_forward`.
     pub fn moe_layer<'a>(&'a self, moe: &MoeLayerWeights<'_>, hidden: usize) -> Option<HipMoeLayer<'a>> {
-        let (limit, alpha) = match moe.gate_rule {
-            MoeGateRule::ClampedGlu { limit, alpha } => (limit, alpha),
+        // the rules this backend has kernels for: ClampedGlu on any bank, Gated(gelu_tanh | silu) on a k-quant bank
+        let (gate_rule, limit, alpha) = match moe.gate_rule {
+            MoeGateRule::ClampedGlu { limit, alpha } => (ffi::MOE_GATE_CLAMPED_GLU, limit, alpha),
+            MoeGateRule::Gated(activation) if activation.gate_up_is_gelu_tanh() => (ffi::MOE_GATE_GELU_TANH, 0.0, 0.0),
+            MoeGateRule::Gated(_) => (ffi::MOE_GATE_SILU, 0.0, 0.0),
             _ => return None,
         };
         let (sg, sd): (Vec<&[u8]>, Vec<&[u8]>) = match &moe.expert_scales {
@@ -247,6 +253,7 @@ impl HipBackend {
             per_expert_scale: (moe.routing_policy.expert_scale == MoeExpertScalePolicy::PerExpert) as c_int,
             glu_limit: limit,
             glu_alpha: alpha,
+            gate_rule,
         };
         let mut layer: *mut ffi::MoeLayer = ptr::null_mut();
         // SAFETY: every table holds `n` entries that outlive the call; the library copies the bytes before it returns.

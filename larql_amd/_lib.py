@@ -34,6 +34,7 @@ class Mxfp4Experts(C.Structure):
 
 
 MOE_SCALES_INLINE, MOE_SCALES_PAIRED = 0, 1
+MOE_GATE_CLAMPED_GLU, MOE_GATE_GELU_TANH, MOE_GATE_SILU = 0, 1, 2
 MOE_ROWS_CONTIGUOUS_HALVES, MOE_ROWS_INTERLEAVED = 0, 1
 
 
@@ -45,7 +46,7 @@ class MoeLayerWeights(C.Structure):
                 ("scales_gate_up_len", C.POINTER(sz)), ("scales_down", C.POINTER(vp)), ("scales_down_len", C.POINTER(sz)),
                 ("router_proj", vp), ("router_bias", vp), ("experts_gate_up_bias", vp), ("experts_down_bias", vp),
                 ("router_per_expert_scale", vp), ("renormalized_softmax", ci), ("per_expert_scale", ci), ("glu_limit", C.c_float),
-                ("glu_alpha", C.c_float)]
+                ("glu_alpha", C.c_float), ("gate_rule", ci)]
 
 
 class MatvecJob(C.Structure):

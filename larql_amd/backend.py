@@ -496,9 +496,11 @@ class HipBackend:
     def moe_layer_create(self, experts_gate_up, experts_down, scales_gate_up, scales_down, router_proj, top_k: int, hidden: int,
                          inter: int, fused_row_layout: int = L.MOE_ROWS_INTERLEAVED, router_bias=None, gate_up_bias=None,
                          down_bias=None, per_expert_scale=None, renormalized: bool = True, expert_scales: int = L.MOE_SCALES_PAIRED,
-                         expert_data_format: int = L.FMT_MXFP4, limit: float = 7.0, alpha: float = 1.702) -> Optional[int]:
+                         expert_data_format: int = L.FMT_MXFP4, limit: float = 7.0, alpha: float = 1.702,
+                         gate_rule: int = L.MOE_GATE_CLAMPED_GLU) -> Optional[int]:
         """experts_gate_up / experts_down / scales_*: one uint8 array per expert (separate allocations, as mmap ranges
-        would be).  Returns a layer handle, or None where the backend refuses the layer."""
+        would be); a Q4_K / Q6_K bank has no scale tables (None, MOE_SCALES_INLINE) and ContiguousHalves rows.  Returns a
+        layer handle, or None where the backend refuses the layer."""
         n = len(experts_gate_up)
         keep = []  # host arrays have to outlive the call
 
@@ -534,7 +536,7 @@ class HipBackend:
         w.experts_gate_up_bias, w.experts_down_bias = f32(gate_up_bias), f32(down_bias)
         w.router_per_expert_scale = f32(per_expert_scale)
         w.renormalized_softmax, w.per_expert_scale = int(renormalized), int(per_expert_scale is not None)
-        w.glu_limit, w.glu_alpha = limit, alpha
+        w.glu_limit, w.glu_alpha, w.gate_rule = limit, alpha, gate_rule
         h = C.c_void_p()
         ok = self._some(lib.larql_hip_moe_layer_create(self._h, C.byref(w), C.byref(h)))
         return h.value if ok else None

@@ -1929,6 +1929,15 @@ struct larql_hip_moe_layer {
     const float *router_proj = nullptr, *scale = nullptr;
     size_t n_experts = 0, top_k = 0, hidden = 0, inter = 0;
     int renormalized = 1, per_expert_scale = 0;
+    // a k-quant (Q4_K / Q6_K) bank: expert e's gate rows at kq_gate + e * kq_gu_stride, its up rows at kq_up + the same,
+    // its down rows at kq_down + e * kq_dn_stride; rows `cols` (gate, up) and `inter_padded` (down) elements wide
+    int kq_kind = 0;  // 0: an MXFP4 bank (`bank`); else KIND_Q4K_Q8K / KIND_Q6K_Q8K
+    const uint8_t *kq_gate = nullptr, *kq_up = nullptr, *kq_down = nullptr;
+    uint64_t kq_gu_stride = 0, kq_dn_stride = 0;
+    size_t cols = 0, inter_padded = 0;
+    const float *kq_gub = nullptr, *kq_db = nullptr, *router_bias = nullptr;
+    int gate_rule = 0;
+    float glu_limit = 7.0f, glu_alpha = 1.702f;
     DevBuf ws, logits, rin, x, out, experts, weights;  // grown on demand (host tier: staging as well)
 };
 
@@ -1941,12 +1950,98 @@ void larql_hip_moe_layer_destroy(larql_hip_ctx *c, larql_hip_moe_layer *L) {
     delete L;
 }
 
+// A Q4_K / Q6_K bank (the caller holds the context's lock): what cpu_moe_forward's integer path reads.
+static int moe_layer_create_kq(larql_hip_ctx *c, const larql_hip_moe_layer_weights *w, larql_hip_moe_layer **out) {
+    const size_t E = w->num_experts, hidden = w->hidden, inter = w->intermediate_size;
+    const size_t blk = w->expert_data_format == LARQL_FMT_Q6_K ? 210 : 144;
+    if (w->expert_scales != LARQL_MOE_SCALES_INLINE)
+        return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: a k-quant bank carries its scales inside its blocks (MoeExpertScales::Inline)");
+    if (w->fused_row_layout != LARQL_MOE_ROWS_CONTIGUOUS_HALVES)
+        return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: a k-quant bank is read as contiguous gate / up halves, as cpu_moe_forward reads it");
+    if (w->gate_rule != LARQL_MOE_GATE_CLAMPED_GLU && w->gate_rule != LARQL_MOE_GATE_GELU_TANH && w->gate_rule != LARQL_MOE_GATE_SILU)
+        return fail(c, LARQL_UNSUPPORTED, "moe_layer: unknown gate rule");
+    if (E == 0 || w->top_k == 0 || hidden == 0 || inter == 0) return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: empty layer");
+    if (E > kRouterMaxExperts || std::min(w->top_k, E) > 8) return fail(c, LARQL_UNSUPPORTED, "moe_layer: at most 256 experts and top-8 on this backend");
+    if (hidden > (1u << 24) || inter > (1u << 24)) return fail(c, LARQL_UNSUPPORTED, "moe_layer: dimensions beyond this backend");
+    if (!w->experts_gate_up || !w->experts_gate_up_len || !w->experts_down || !w->experts_down_len || !w->router_proj) return LARQL_E_ARG;
+    // the gate/up matrices' stored row width, from the slab length (stored_gate_up_cols, pipeline/moe.rs:659-690)
+    size_t cols = hidden;
+    {
+        const size_t len = w->experts_gate_up_len[0];
+        if (len % (2 * inter) == 0 && (len / (2 * inter)) % blk == 0 && len / (2 * inter) / blk * 256 >= hidden) cols = len / (2 * inter) / blk * 256;
+    }
+    const size_t ip = (inter + 255) / 256 * 256;  // MoeWeightLayout::quant_block_padded_down
+    if (cols % 256 != 0) return fail(c, LARQL_UNSUPPORTED, "moe_layer: k-quant rows must be whole 256-element super-blocks");
+    if (cols / 256 > 40 || ip / 256 > 40) return fail(c, LARQL_UNSUPPORTED, "moe_layer: k-quant rows longer than 10240 elements have no kernel");
+    const size_t half = inter * (cols / 256) * blk, dn = hidden * (ip / 256) * blk;
+    for (size_t e = 0; e < E; e++) {
+        if (!w->experts_gate_up[e] || !w->experts_down[e]) return LARQL_E_ARG;
+        if (w->experts_gate_up_len[e] < 2 * half || w->experts_down_len[e] < dn)
+            return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: expert %zu's slices are shorter than its geometry", e);
+    }
+    HIPCHECK(c, hipSetDevice(c->device));
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    // region: [gate halves | up halves | down | router_proj | router_bias | gate_up_bias | down_bias | per-expert scale]; every
+    // expert's matrix starts on a 256-byte boundary (a Q6_K half is a whole number of 210-byte blocks, not of 16 bytes)
+    const size_t hs = up(half), ds = up(dn);
+    size_t off = 0;
+    const size_t o_g = off; off += E * hs;
+    const size_t o_u = off; off += E * hs;
+    const size_t o_d = off; off += E * ds;
+    const size_t o_rp = off; off += up(E * hidden * 4);
+    const size_t o_rb = off; off += up(E * 4);
+    const size_t o_gub = off; off += up(E * 2 * inter * 4);
+    const size_t o_db = off; off += up(E * hidden * 4);
+    const size_t o_sc = off; off += up(E * 4);
+    larql_hip_moe_layer *L = new larql_hip_moe_layer();
+    if (hipMalloc(&L->region, off + 64) != hipSuccess) { delete L; return fail(c, LARQL_E_DEVICE, "moe_layer: out of device memory"); }
+    uint8_t *d = (uint8_t *)L->region;
+    hipError_t e = hipSuccess;
+    auto put = [&](size_t dst, const void *src, size_t n) {
+        if (e == hipSuccess && n) e = hipMemcpyAsync(d + dst, src, n, hipMemcpyHostToDevice, c->stream);
+    };
+    for (size_t x = 0; x < E; x++) {
+        put(o_g + x * hs, w->experts_gate_up[x], half);
+        put(o_u + x * hs, w->experts_gate_up[x] + half, half);
+        put(o_d + x * ds, w->experts_down[x], dn);
+    }
+    put(o_rp, w->router_proj, E * hidden * 4);
+    if (w->router_bias) put(o_rb, w->router_bias, E * 4);
+    if (w->experts_gate_up_bias) put(o_gub, w->experts_gate_up_bias, E * 2 * inter * 4);
+    if (w->experts_down_bias) put(o_db, w->experts_down_bias, E * hidden * 4);
+    if (w->router_per_expert_scale) put(o_sc, w->router_per_expert_scale, E * 4);
+    if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+    if (e != hipSuccess) {
+        (void)hipFree(L->region);
+        delete L;
+        return fail(c, LARQL_E_DEVICE, "moe_layer: upload: %s", hipGetErrorString(e));
+    }
+    L->kq_kind = w->expert_data_format == LARQL_FMT_Q6_K ? KIND_Q6K_Q8K : KIND_Q4K_Q8K;
+    L->kq_gate = d + o_g; L->kq_up = d + o_u; L->kq_down = d + o_d;
+    L->kq_gu_stride = hs; L->kq_dn_stride = ds;
+    L->cols = cols; L->inter_padded = ip;
+    L->kq_gub = w->experts_gate_up_bias ? (const float *)(d + o_gub) : nullptr;
+    L->kq_db = w->experts_down_bias ? (const float *)(d + o_db) : nullptr;
+    L->router_bias = w->router_bias ? (const float *)(d + o_rb) : nullptr;
+    L->gate_rule = w->gate_rule; L->glu_limit = w->glu_limit; L->glu_alpha = w->glu_alpha;
+    L->router_proj = (const float *)(d + o_rp);
+    L->scale = w->router_per_expert_scale ? (const float *)(d + o_sc) : nullptr;
+    L->n_experts = E; L->top_k = w->top_k; L->hidden = hidden; L->inter = inter;
+    L->renormalized = w->renormalized_softmax ? 1 : 0;
+    L->per_expert_scale = (w->per_expert_scale && w->router_per_expert_scale) ? 1 : 0;
+    *out = L;
+    return LARQL_OK;
+}
+
 int larql_hip_moe_layer_create(larql_hip_ctx *c, const larql_hip_moe_layer_weights *w, larql_hip_moe_layer **out) {
     if (!c || !w || !out) return LARQL_E_ARG;
     *out = nullptr;
     std::lock_guard<std::mutex> lk(c->mu);
+    if (w->expert_data_format == LARQL_FMT_Q4_K || w->expert_data_format == LARQL_FMT_Q6_K) return moe_layer_create_kq(c, w, out);
     if (w->expert_data_format != LARQL_FMT_MXFP4)
-        return fail(c, LARQL_UNSUPPORTED, "moe_layer: only MXFP4 expert banks are served by this backend");
+        return fail(c, LARQL_UNSUPPORTED, "moe_layer: MXFP4, Q4_K and Q6_K expert banks are served by this backend");
+    if (w->gate_rule != LARQL_MOE_GATE_CLAMPED_GLU)
+        return fail(c, LARQL_UNSUPPORTED, "moe_layer: an MXFP4 bank is served under MoeGateRule::ClampedGlu only");
     if (w->expert_scales != LARQL_MOE_SCALES_PAIRED)
         return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: an MXFP4 bank keeps its e8m0 exponents in a partner stream (MoeExpertScales::Paired)");
     const size_t E = w->num_experts, hidden = w->hidden, inter = w->intermediate_size;
@@ -2036,8 +2131,8 @@ static int moe_layer_enqueue(larql_hip_ctx *c, larql_hip_moe_layer *L, const flo
     const size_t E = L->n_experts, hidden = L->hidden, k = std::min(L->top_k, E);
     if (hidden % 4 != 0 || ((uintptr_t)router_in & 15) || ((uintptr_t)x & 15) || ((uintptr_t)out & 15))
         return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: activations must be 16-byte aligned rows (hidden a multiple of 4)");
-    const size_t wsb = larql_hip_moe_mxfp4_workspace_bytes(tokens, k, hidden, L->inter);
-    int rc = ensure(c, L->ws, wsb); if (rc) return rc;
+    const size_t wsb = L->kq_kind ? 0 : larql_hip_moe_mxfp4_workspace_bytes(tokens, k, hidden, L->inter);
+    int rc = L->kq_kind ? LARQL_OK : ensure(c, L->ws, wsb); if (rc) return rc;
     rc = ensure(c, L->logits, tokens * E * 4 + 64); if (rc) return rc;
     float *logits = (float *)L->logits.p;
     std::vector<GemvJob> jobs;
@@ -2047,6 +2142,45 @@ static int moe_layer_enqueue(larql_hip_ctx *c, larql_hip_moe_layer *L, const flo
     // softmax over all, top-k, renormalise == Router::select's NormalisedOverSelected (the same quotient of exponentials);
     // without the renormalisation the weights are the softmax's own values (SoftmaxThenSelect)
     const int policy = L->renormalized ? 1 : 0;
+    if (L->kq_kind) {
+        // The integer expert path of cpu_moe_forward (cpu/ops/moe/forward.rs:160-330): the route, the expert input as one
+        // Q8_K activation per token at the stored row width, gate and up of every slot in one launch (the expert picked
+        // from the bank at run time), the gated activation as Q8_K per slot, the down projections in one launch, and
+        // the weighted sum with the down bias inside the weight.
+        const size_t slots = tokens * k, inter = L->inter, ip = L->inter_padded, cols = L->cols;
+        if (tokens > 65535 || slots > 65535) return fail(c, LARQL_UNSUPPORTED, "moe_layer: too many tokens in one call for a k-quant bank");
+        HIPCHECK(c, router_select_launch(c->stream, logits, L->router_bias, (uint32_t)tokens, (uint32_t)E, (uint32_t)k, policy, experts, weights));
+        if (L->per_expert_scale) HIPCHECK(c, expert_scale_launch(c->stream, weights, experts, L->scale, (uint32_t)slots, (uint32_t)E));
+        const size_t xq_stride = (q8k_bytes(cols) + 255) & ~(size_t)255, aq_stride = (q8k_bytes(ip) + 255) & ~(size_t)255;
+        const size_t f_bytes = ((2 * slots * inter + slots * hidden) * sizeof(float) + 255) & ~(size_t)255;
+        rc = ensure(c, L->ws, f_bytes + tokens * xq_stride + slots * aq_stride + 256); if (rc) return rc;
+        float *g = (float *)L->ws.p, *u = g + slots * inter, *dd = u + slots * inter;
+        uint8_t *xq = (uint8_t *)L->ws.p + f_bytes, *aq = xq + tokens * xq_stride;
+        HIPCHECK(c, quantize_rows_to_q8k_launch(c->stream, x, hidden, (uint32_t)hidden, (uint32_t)cols, (uint32_t)tokens, xq, xq_stride));
+        jobs.clear();
+        for (size_t s = 0; s < slots; s++) {
+            GemvJob a = make_job(L->kq_kind, L->kq_gate, nullptr, xq + (s / k) * xq_stride, g + s * inter, inter, cols);
+            a.sel = experts + s; a.w_sel_stride = L->kq_gu_stride; a.sel_count = (uint32_t)E;
+            GemvJob b = a;
+            b.w = L->kq_up; b.out = u + s * inter;
+            jobs.push_back(a);
+            jobs.push_back(b);
+        }
+        rc = enqueue_jobs(c, jobs);
+        if (rc) return rc;
+        HIPCHECK(c, moe_kq_act_q8k_launch(c->stream, g, u, (uint32_t)inter, (uint32_t)ip, (uint32_t)slots, experts, (uint32_t)E, L->kq_gub, L->gate_rule,
+                                          L->glu_limit, L->glu_alpha, aq, aq_stride));
+        jobs.clear();
+        for (size_t s = 0; s < slots; s++) {
+            GemvJob a = make_job(L->kq_kind, L->kq_down, nullptr, aq + s * aq_stride, dd + s * hidden, hidden, ip);
+            a.sel = experts + s; a.w_sel_stride = L->kq_dn_stride; a.sel_count = (uint32_t)E;
+            jobs.push_back(a);
+        }
+        rc = enqueue_jobs(c, jobs);
+        if (rc) return rc;
+        HIPCHECK(c, weighted_sum_bias_launch(c->stream, dd, weights, experts, (uint32_t)E, L->kq_db, out, (uint32_t)tokens, (uint32_t)k, (uint32_t)hidden));
+        return LARQL_OK;
+    }
     if (!L->per_expert_scale) return moe_mxfp4_block(c, &L->bank, x, tokens, k, experts, weights, out, L->ws.p, wsb, logits, policy);
     HIPCHECK(c, router_select_launch(c->stream, logits, L->bank.router_bias, (uint32_t)tokens, (uint32_t)E, (uint32_t)k, policy, experts, weights));
     HIPCHECK(c, expert_scale_launch(c->stream, weights, experts, L->scale, (uint32_t)(tokens * k), (uint32_t)E));

@@ -2942,7 +2942,13 @@ __global__ void __launch_bounds__(kQ4kMaxWaves * 64) gemv_q4k_q8k_kernel(GemvLau
     const uint32_t lo = first_job_of_share(L, jobs, L.n_jobs, p);
     uint32_t ji = lo, parity = 0;
     while (p < p_end) {
-        const GemvJob j = uniform_job(jobs + ji);
+        GemvJob j = uniform_job(jobs + ji);
+        if (j.sel) {  // run-time expert selection: one bank of equally shaped matrices (an id outside the bank reads matrix 0;
+                      // the caller does not use that result)
+            uint32_t e = __builtin_amdgcn_readfirstlane(*(const GLOBAL_AS uint32_t *)j.sel);
+            e = e < j.sel_count ? e : 0u;
+            j.w += (size_t)e * j.w_sel_stride;
+        }
         const uint32_t seg_end = min(p_end, j.pass_begin + j.n_pass);
         const uint32_t a = p - j.pass_begin, b = seg_end - j.pass_begin, cpt = (uint32_t)j.pad, su = j.pad2;
         const uint32_t tile_a = a > su ? (a - su + cpt - 1) / cpt : 0, tile_b = b > su ? (b - su + cpt - 1) / cpt : 0;

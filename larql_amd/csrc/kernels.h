@@ -196,6 +196,15 @@ hipError_t moe_plan_launch(hipStream_t s, const float *logits, const float *rout
 hipError_t clamped_glu_interleaved_launch(hipStream_t s, const float *gu, float *h, size_t n, float limit, float alpha);
 hipError_t clamped_glu_launch(hipStream_t s, const float *g, const float *u, float *h, size_t n, float limit, float alpha);
 hipError_t expert_scale_launch(hipStream_t s, float *weights, const uint32_t *experts, const float *scale, uint32_t n, uint32_t n_scale);
+// the k-quant expert path: rows -> Q8_K activations of their own (zero-padded to `cols`), the gated activation of every
+// slot -> Q8_K, and the weighted sum with the experts' down bias (rule: 0 ClampedGlu, 1 Gated(gelu_tanh), 2 Gated(silu))
+hipError_t quantize_rows_to_q8k_launch(hipStream_t s, const float *src, size_t src_stride, uint32_t src_cols, uint32_t cols, uint32_t rows,
+                                       uint8_t *dst, size_t dst_stride);
+hipError_t moe_kq_act_q8k_launch(hipStream_t s, const float *g, const float *u, uint32_t inter, uint32_t inter_padded, uint32_t slots,
+                                 const uint32_t *experts, uint32_t n_experts, const float *gub, int rule, float limit, float alpha, uint8_t *dst,
+                                 size_t dst_stride);
+hipError_t weighted_sum_bias_launch(hipStream_t s, const float *d, const float *weights, const uint32_t *experts, uint32_t n_experts,
+                                    const float *bias, float *out, uint32_t tokens, uint32_t k, uint32_t hidden);
 hipError_t weighted_sum_launch(hipStream_t s, const float *d, const float *weights, const uint32_t *experts, uint32_t n_experts, float *out,
                                uint32_t tokens, uint32_t k, uint32_t hidden);
 

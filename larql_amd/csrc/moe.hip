@@ -86,6 +86,113 @@ __global__ void weighted_sum_kernel(const float *__restrict__ d, const float *__
     out[(size_t)t * hidden + i] = acc;
 }
 
+// ---- the k-quant expert path (cpu_moe_forward over Q4_K / Q6_K banks: cpu/ops/moe/forward.rs:160-330) ----------------
+
+// quantize_x_to_q8k (cpu/ops/q4k_q8k_dot/q8k_activation.rs:84-109) of one 256-element super-block that a wavefront
+// holds four elements per lane: d = amax / 127, codes round(x * (1/d)) clamped to +-127, NaN -> 0.  `sum` ends, in the
+// lanes 8s, as the sum of sub-block s's 32 codes.
+__device__ __forceinline__ int q8k_code(float t) {
+    float r = roundf(t);
+    r = r < -127.0f ? -127.0f : (r > 127.0f ? 127.0f : r);
+    return r != r ? 0 : (int)r;
+}
+__device__ __forceinline__ void q8k_block(const float (&v)[4], uint32_t &codes, float &scale, int &sum) {
+    float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));  // fmaxf ignores a NaN operand, as f32::max does
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+    scale = amax > 0.0f ? amax / 127.0f : 0.0f;
+    const float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
+    const int q0 = q8k_code(v[0] * inv), q1 = q8k_code(v[1] * inv), q2 = q8k_code(v[2] * inv), q3 = q8k_code(v[3] * inv);
+    sum = q0 + q1 + q2 + q3;
+    sum += __shfl_xor(sum, 1);
+    sum += __shfl_xor(sum, 2);
+    sum += __shfl_xor(sum, 4);
+    codes = ((uint32_t)q0 & 0xFFu) | (((uint32_t)q1 & 0xFFu) << 8) | (((uint32_t)q2 & 0xFFu) << 16) | (((uint32_t)q3 & 0xFFu) << 24);
+}
+// the device layout of a Q8_K activation of `cols` elements at `o`: [cols codes | cols/256 f32 scales | cols/32 i16 sums]
+__device__ __forceinline__ void q8k_store(uint8_t *o, uint32_t cols, uint32_t sb, uint32_t lane, uint32_t codes, float scale, int sum) {
+    const uint32_t nb = cols / 256;
+    reinterpret_cast<uint32_t *>(o)[sb * 64 + lane] = codes;
+    if (lane == 0) reinterpret_cast<float *>(o + cols)[sb] = scale;
+    if ((lane & 7u) == 0) reinterpret_cast<int16_t *>(o + cols + (size_t)nb * 4)[sb * 8 + (lane >> 3)] = (int16_t)sum;
+}
+
+// Row `blockIdx.y` of src ([rows, src_cols] floats, src_stride apart), zero-padded to `cols` (a multiple of 256: the
+// stored row width of the gate/up matrices, forward.rs:176-184), as a Q8_K activation of its own at dst + row * dst_stride.
+// One wavefront per super-block.
+__global__ void __launch_bounds__(256) quantize_rows_to_q8k_kernel(const float *__restrict__ src, size_t src_stride, uint32_t src_cols, uint32_t cols,
+                                                                  uint8_t *__restrict__ dst, size_t dst_stride) {
+    const uint32_t sb = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63u;
+    if (sb >= cols / 256) return;
+    const float *s = src + (size_t)blockIdx.y * src_stride;
+    const uint32_t j = sb * 256 + 4 * lane;
+    float v[4];
+#pragma unroll
+    for (uint32_t i = 0; i < 4; i++) v[i] = j + i < src_cols ? s[j + i] : 0.0f;
+    uint32_t codes; float scale; int sum;
+    q8k_block(v, codes, scale, sum);
+    q8k_store(dst + (size_t)blockIdx.y * dst_stride, cols, sb, lane, codes, scale, sum);
+}
+
+// math::silu / math::gelu_tanh (cpu/ops/moe/math.rs:54-65) and MoeGateRule::combine (pipeline/moe.rs:73-118)
+__device__ __forceinline__ float moe_combine(int rule, float g, float u, float limit, float alpha) {
+    if (rule == 1) {
+        const float c = 0.7978846f;
+        return 0.5f * g * (1.0f + tanhf(c * (g + 0.044715f * g * g * g))) * u;
+    }
+    if (rule == 2) return g / (1.0f + expf(-g)) * u;
+    const float gv = fminf(g, limit);
+    const float uv = u < -limit ? -limit : (u > limit ? limit : u);
+    return (uv + 1.0f) * (gv * (1.0f / (1.0f + expf(-(gv * alpha)))));
+}
+
+// Slot `blockIdx.y`'s activation: act[j] = combine(g[j] + gate bias, u[j] + up bias) for j < inter (the fused bias row
+// of the slot's expert is interleaved: gate at 2j, up at 2j+1 — ExpertMlp::gate_bias / up_bias, pipeline/moe.rs:150-170),
+// zeros up to inter_padded, quantised to a Q8_K activation of inter_padded elements at dst + slot * dst_stride
+// (run_single_expert_kq_q8k_into, cpu/ops/moe/expert/q4k.rs:300-325).  A slot whose expert lies outside the bank gets
+// no bias; its result is never read.
+__global__ void __launch_bounds__(256) moe_kq_act_q8k_kernel(const float *__restrict__ g, const float *__restrict__ u, uint32_t inter, uint32_t inter_padded,
+                                                            const uint32_t *__restrict__ experts, uint32_t n_experts, const float *__restrict__ gub,
+                                                            int rule, float limit, float alpha, uint8_t *__restrict__ dst, size_t dst_stride) {
+    const uint32_t sb = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63u;
+    if (sb >= inter_padded / 256) return;
+    const uint32_t slot = blockIdx.y;
+    const uint32_t e = experts[slot];
+    const float *b = (gub && e < n_experts) ? gub + (size_t)e * 2 * inter : nullptr;
+    const uint32_t j = sb * 256 + 4 * lane;
+    float v[4];
+#pragma unroll
+    for (uint32_t i = 0; i < 4; i++) {
+        v[i] = 0.0f;
+        if (j + i < inter) {
+            const float gv = g[(size_t)slot * inter + j + i] + (b ? b[2 * (j + i)] : 0.0f);
+            const float uv = u[(size_t)slot * inter + j + i] + (b ? b[2 * (j + i) + 1] : 0.0f);
+            v[i] = moe_combine(rule, gv, uv, limit, alpha);
+        }
+    }
+    uint32_t codes; float scale; int sum;
+    q8k_block(v, codes, scale, sum);
+    q8k_store(dst + (size_t)slot * dst_stride, inter_padded, sb, lane, codes, scale, sum);
+}
+
+// out[t] = sum over the token's k slots, in selection order, of w * (down output + the expert's down bias)
+// (forward.rs:220-228: add_down_bias, then `*a += w * v`); a slot whose expert lies outside the bank is skipped.
+__global__ void weighted_sum_bias_kernel(const float *__restrict__ d, const float *__restrict__ weights, const uint32_t *__restrict__ experts,
+                                         uint32_t n_experts, const float *__restrict__ bias, float *__restrict__ out, uint32_t k, uint32_t hidden) {
+    const uint32_t t = blockIdx.y;
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= hidden) return;
+    float acc = 0.0f;
+    for (uint32_t r = 0; r < k; r++) {
+        const uint32_t e = experts[(size_t)t * k + r];
+        if (e >= n_experts) continue;
+        float v = d[((size_t)t * k + r) * hidden + i];
+        if (bias) v += bias[(size_t)e * hidden + i];
+        acc += weights[(size_t)t * k + r] * v;
+    }
+    out[(size_t)t * hidden + i] = acc;
+}
+
 // Job lists of an expert block, built on the device from the router's choice (no host round trip): the slots
 // (token, rank) that chose the same expert are grouped by `group` (2 or 4), in slot order, and every group becomes one
 // gate, one up and one down job whose activations share the expert's weights (GemvJob::batch = tokens in the group;
@@ -351,6 +458,27 @@ hipError_t clamped_glu_launch(hipStream_t s, const float *g, const float *u, flo
 hipError_t expert_scale_launch(hipStream_t s, float *weights, const uint32_t *experts, const float *scale, uint32_t n, uint32_t n_scale) {
     if (n == 0 || n_scale == 0) return hipSuccess;
     hipLaunchKernelGGL(expert_scale_kernel, dim3((n + 255) / 256), dim3(256), 0, s, weights, experts, scale, n, n_scale);
+    return hipGetLastError();
+}
+
+hipError_t quantize_rows_to_q8k_launch(hipStream_t s, const float *src, size_t src_stride, uint32_t src_cols, uint32_t cols, uint32_t rows,
+                                       uint8_t *dst, size_t dst_stride) {
+    if (rows == 0 || cols < 256) return hipSuccess;
+    hipLaunchKernelGGL(quantize_rows_to_q8k_kernel, dim3((cols / 256 + 3) / 4, rows), dim3(256), 0, s, src, src_stride, src_cols, cols, dst, dst_stride);
+    return hipGetLastError();
+}
+hipError_t moe_kq_act_q8k_launch(hipStream_t s, const float *g, const float *u, uint32_t inter, uint32_t inter_padded, uint32_t slots,
+                                 const uint32_t *experts, uint32_t n_experts, const float *gub, int rule, float limit, float alpha, uint8_t *dst,
+                                 size_t dst_stride) {
+    if (slots == 0 || inter_padded < 256) return hipSuccess;
+    hipLaunchKernelGGL(moe_kq_act_q8k_kernel, dim3((inter_padded / 256 + 3) / 4, slots), dim3(256), 0, s, g, u, inter, inter_padded, experts, n_experts,
+                       gub, rule, limit, alpha, dst, dst_stride);
+    return hipGetLastError();
+}
+hipError_t weighted_sum_bias_launch(hipStream_t s, const float *d, const float *weights, const uint32_t *experts, uint32_t n_experts,
+                                    const float *bias, float *out, uint32_t tokens, uint32_t k, uint32_t hidden) {
+    if (tokens == 0 || hidden == 0) return hipSuccess;
+    hipLaunchKernelGGL(weighted_sum_bias_kernel, dim3((hidden + 255) / 256, tokens), dim3(256), 0, s, d, weights, experts, n_experts, bias, out, k, hidden);
     return hipGetLastError();
 }
 

@@ -51,9 +51,10 @@ struct MoeExpertScales {  // Inline | Paired { gate_up, down } (moe.rs:214-238)
     bool paired = false;
     std::vector<Slice<uint8_t>> gate_up, down;
 };
-struct MoeGateRule {  // the one rule this backend has a kernel for: ClampedGlu { limit, alpha } (moe.rs:88-92)
-    bool clamped_glu = true;
-    float limit = 7.0f, alpha = 1.702f;
+struct MoeGateRule {  // moe.rs:40-118; the rules this backend has kernels for, `Other` standing for the rest
+    enum Kind { ClampedGlu = LARQL_MOE_GATE_CLAMPED_GLU, GatedGeluTanh = LARQL_MOE_GATE_GELU_TANH, GatedSilu = LARQL_MOE_GATE_SILU, Other = -1 };
+    Kind kind = ClampedGlu;
+    float limit = 7.0f, alpha = 1.702f;  // ClampedGlu { limit, alpha }
 };
 struct MoeLayerWeights {
     std::vector<Slice<uint8_t>> experts_gate_up, experts_down;
@@ -278,11 +279,13 @@ class HipBackend {
     }
 
     // A MoE layer made resident from MoeLayerWeights: the per-expert slices and their paired exponent streams go up
-    // expert by expert, wherever they lie.  nullopt where this backend has no kernel for the layer (anything but an
-    // MXFP4 bank with Paired scales and ClampedGlu, more than 256 experts, top-k above 8): the caller keeps cpu_moe_forward.
+    // expert by expert, wherever they lie.  Served: an MXFP4 bank with Paired scales under ClampedGlu, and a Q4_K / Q6_K
+    // bank with Inline scales and ContiguousHalves rows under ClampedGlu or Gated (cpu_moe_forward's integer path).
+    // nullopt where this backend has no kernel for the layer (other formats or rules, more than 256 experts, top-k
+    // above 8): the caller keeps cpu_moe_forward.
     std::optional<HipMoeLayer> moe_layer(const MoeLayerWeights &moe, size_t hidden) {
         const size_t n = moe.num_experts;
-        if (!moe.gate_rule.clamped_glu) return std::nullopt;
+        if (moe.gate_rule.kind == MoeGateRule::Other) return std::nullopt;
         if (moe.experts_gate_up.size() != n || moe.experts_down.size() != n) return std::nullopt;
         if (hidden != 0 && n > (size_t)-1 / hidden) return std::nullopt;
         if (moe.router_proj.len != n * hidden) return std::nullopt;
@@ -307,7 +310,7 @@ class HipBackend {
         w.router_per_expert_scale = opt(moe.router_per_expert_scale);
         w.renormalized_softmax = moe.renormalized_softmax ? 1 : 0;
         w.per_expert_scale = moe.per_expert_scale ? 1 : 0;
-        w.glu_limit = moe.gate_rule.limit; w.glu_alpha = moe.gate_rule.alpha;
+        w.glu_limit = moe.gate_rule.limit; w.glu_alpha = moe.gate_rule.alpha; w.gate_rule = (int)moe.gate_rule.kind;
         larql_hip_moe_layer *layer = nullptr;
         if (larql_hip_moe_layer_create(ctx_, &w, &layer) != LARQL_OK || !layer) return std::nullopt;
         return HipMoeLayer(ctx_, layer, hidden, std::min(moe.top_k, n));

@@ -227,7 +227,39 @@ int main() {
         CHECK(!layer->forward(xm, larql::Slice<float>(xm.data(), H), 2));                 // x is not [2, H]
         m.expert_scales.paired = false;                                                    // Inline scales on an MXFP4 bank: refused
         CHECK(!be.moe_layer(m, H));
-        m.expert_scales.paired = true; m.gate_rule.clamped_glu = false;                    // another gate rule: the caller's CPU path
+        m.expert_scales.paired = true; m.gate_rule.kind = larql::MoeGateRule::GatedSilu;      // an MXFP4 bank under another gate rule: no kernel
+        CHECK(!be.moe_layer(m, H));
+    }
+
+    // The same from a Q4_K bank (Inline scales, ContiguousHalves rows): cpu_moe_forward's integer path in closed form.
+    // Every weight is 0.5 * 1 * 2 = 1.0; x = 127 / 2^14 quantises exactly (d = 2^-14, codes 127), so gate = up =
+    // 256 x = 1.984375 in every row, the SiLU-gated activation is one constant (exact as Q8_K too), and a down row sums
+    // 256 of them.
+    {
+        const size_t H = 256, I = 256;
+        uint8_t blk[144];
+        std::memset(blk, 0, 144);
+        blk[0] = 0x00; blk[1] = 0x38;                                  // d = 0.5, dmin = 0
+        for (int j = 0; j < 4; j++) { blk[4 + j] = 1; blk[12 + j] = 1; }  // every 6-bit scale 1, every min 0
+        std::memset(blk + 16, 0x22, 128);
+        std::vector<uint8_t> gu(2 * I * 144), dn(H * 144);
+        for (size_t r = 0; r < 2 * I; r++) std::memcpy(&gu[r * 144], blk, 144);
+        for (size_t r = 0; r < H; r++) std::memcpy(&dn[r * 144], blk, 144);
+        std::vector<float> rp(H, 0.0f);
+        larql::MoeLayerWeights m;
+        m.experts_gate_up = {gu}; m.experts_down = {dn};
+        m.fused_row_layout = larql::MoeFusedRowLayout::ContiguousHalves;
+        m.expert_data_format = larql::QuantFormat::Q4_K;
+        m.gate_rule.kind = larql::MoeGateRule::GatedSilu;
+        m.router_proj = rp; m.num_experts = 1; m.top_k = 1; m.intermediate_size = I;
+        auto layer = be.moe_layer(m, H);
+        CHECK(layer.has_value());
+        std::vector<float> xm(H, 127.0f / 16384.0f);
+        auto r1 = layer->forward(xm, xm, 1);
+        const double g = 256.0 * 127.0 / 16384.0, want = 256.0 * (g / (1.0 + std::exp(-g))) * g;
+        CHECK(r1 && r1->experts[0] == 0 && r1->weights[0] == 1.0f);
+        for (size_t c = 0; c < H; c++) CHECK(std::fabs(r1->out[c] - want) < 1e-5 * want);
+        m.fused_row_layout = larql::MoeFusedRowLayout::Interleaved;   // the CPU tier refuses an interleaved k-quant bank; so does this one
         CHECK(!be.moe_layer(m, H));
     }
 

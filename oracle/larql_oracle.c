@@ -1353,6 +1353,81 @@ int lq_moe_block_mxfp4(const float *x, size_t tokens, size_t hidden, size_t inte
     return 0;
 }
 
+/* math::silu / math::gelu_tanh — larql-compute/src/cpu/ops/moe/math.rs:54-65. */
+float lq_silu(float x) { return x / (1.0f + expf(-x)); }
+float lq_gelu_tanh(float x) {
+    const float c = 0.7978846f;
+    return 0.5f * x * (1.0f + tanhf(c * (x + 0.044715f * x * x * x)));
+}
+/* MoeGateRule::combine — larql-compute/src/pipeline/moe.rs:73-118, the rules a k-quant bank is served under:
+ * 0 ClampedGlu{limit, alpha}, 1 Gated(gelu_tanh), 2 Gated(silu).  Inputs already carry their biases. */
+float lq_moe_combine(int rule, float g, float u, float limit, float alpha) {
+    if (rule == LQ_GATE_GELU_TANH) return lq_gelu_tanh(g) * u;
+    if (rule == LQ_GATE_SILU) return lq_silu(g) * u;
+    return lq_clamped_glu(g, u, limit, alpha);
+}
+
+/* cpu_moe_forward's integer expert path with the routing given — larql-compute/src/cpu/ops/moe/forward.rs:160-330 and
+ * run_single_expert_kq_q8k_into, cpu/ops/moe/expert/q4k.rs:232-351.  Per token the expert input is zero-padded to the
+ * gate/up matrices' stored row width `cols` (forward.rs:176-184) and quantised to Q8_K once for all its experts; per
+ * selected expert, in selection order: gate and up are the first and second half of its [2*inter, cols] slab
+ * (ContiguousHalves, the only layout this tier serves: forward.rs:69-75), g and u get their biases from the fused row
+ * (gate at 2j, up at 2j+1: ExpertMlp::gate_bias / up_bias, pipeline/moe.rs:150-170), the pair is combined under
+ * `rule`, the activation is zero-padded to inter_padded = ceil(inter/256)*256 and quantised to Q8_K, the down matvec
+ * over [hidden, inter_padded] gets the expert's down bias, and out += w * that (forward.rs:220-228).  An expert id
+ * outside the bank is skipped (forward.rs:203-208).  format: 4 = Q4_K, 6 = Q6_K (one format for the whole bank). */
+int lq_moe_block_kq(const float *x, size_t tokens, size_t hidden, size_t cols, size_t inter, size_t n_experts, size_t top_k,
+                    const uint64_t *experts, const float *weights, const uint8_t *const *gate_up, const uint8_t *const *down,
+                    int format, const float *gate_up_bias, const float *down_bias, int rule, float limit, float alpha, float *out) {
+    if ((format != 4 && format != 6) || cols % 256 != 0 || cols < hidden) return 1;
+    const size_t blk = format == 6 ? 210 : 144;
+    const size_t inter_padded = (inter + 255) / 256 * 256;
+    const size_t half = inter * (cols / 256) * blk, down_bytes = hidden * (inter_padded / 256) * blk;
+    float *xp = (float *)calloc(cols ? cols : 1, sizeof(float));
+    int8_t *xq = (int8_t *)malloc(cols ? cols : 1);
+    float *xd = (float *)malloc((cols / 256 + 1) * sizeof(float));
+    int16_t *xs = (int16_t *)malloc((cols / 32 + 1) * sizeof(int16_t));
+    float *g = (float *)malloc((inter ? inter : 1) * sizeof(float)), *u = (float *)malloc((inter ? inter : 1) * sizeof(float));
+    float *act = (float *)calloc(inter_padded ? inter_padded : 1, sizeof(float));
+    int8_t *aq = (int8_t *)malloc(inter_padded ? inter_padded : 1);
+    float *ad = (float *)malloc((inter_padded / 256 + 1) * sizeof(float));
+    int16_t *as = (int16_t *)malloc((inter_padded / 32 + 1) * sizeof(int16_t));
+    float *h2 = (float *)malloc((hidden ? hidden : 1) * sizeof(float));
+    int rc = 0;
+    for (size_t t = 0; t < tokens && !rc; t++) {
+        float *o = out + t * hidden;
+        for (size_t i = 0; i < hidden; i++) { o[i] = 0.0f; xp[i] = x[t * hidden + i]; }
+        if (inter == 0 || cols == 0) continue;
+        rc |= lq_quantize_x_to_q8k(xp, cols, xq, xd, xs);
+        for (size_t s = 0; s < top_k && !rc; s++) {
+            const uint64_t e = experts[t * top_k + s];
+            const float w = weights[t * top_k + s];
+            if (e >= n_experts) continue;
+            if (format == 6) {
+                rc |= lq_q6k_q8k_matvec(g, inter, xq, cols, xd, gate_up[e], half, inter, cols);
+                rc |= lq_q6k_q8k_matvec(u, inter, xq, cols, xd, gate_up[e] + half, half, inter, cols);
+            } else {
+                rc |= lq_q4k_q8k_matvec(g, inter, xq, cols, xd, xs, gate_up[e], half, inter, cols);
+                rc |= lq_q4k_q8k_matvec(u, inter, xq, cols, xd, xs, gate_up[e] + half, half, inter, cols);
+            }
+            for (size_t j = 0; j < inter; j++) {
+                const float gb = gate_up_bias ? gate_up_bias[e * 2 * inter + 2 * j] : 0.0f;
+                const float ub = gate_up_bias ? gate_up_bias[e * 2 * inter + 2 * j + 1] : 0.0f;
+                act[j] = lq_moe_combine(rule, g[j] + gb, u[j] + ub, limit, alpha);
+            }
+            rc |= lq_quantize_x_to_q8k(act, inter_padded, aq, ad, as);
+            if (format == 6) rc |= lq_q6k_q8k_matvec(h2, hidden, aq, inter_padded, ad, down[e], down_bytes, hidden, inter_padded);
+            else rc |= lq_q4k_q8k_matvec(h2, hidden, aq, inter_padded, ad, as, down[e], down_bytes, hidden, inter_padded);
+            for (size_t i = 0; i < hidden; i++) {
+                const float v = down_bias ? h2[i] + down_bias[e * hidden + i] : h2[i];
+                o[i] += w * v;
+            }
+        }
+    }
+    free(xp); free(xq); free(xd); free(xs); free(g); free(u); free(act); free(aq); free(ad); free(as); free(h2);
+    return rc;
+}
+
 /* ------------------------------------------- multi-threaded CPU baseline */
 
 typedef struct {

@@ -128,6 +128,20 @@ int lq_moe_block_mxfp4(const float *x, size_t tokens, size_t hidden, size_t inte
                        const uint8_t *up_packed, const uint8_t *up_scales, const uint8_t *down_packed, const uint8_t *down_scales,
                        int interleaved, const float *gate_up_bias, const float *down_bias, float limit, float alpha, float *out);
 
+/* math::silu / gelu_tanh (cpu/ops/moe/math.rs:54-65) and MoeGateRule::combine (pipeline/moe.rs:73-118) */
+#define LQ_GATE_CLAMPED_GLU 0
+#define LQ_GATE_GELU_TANH 1
+#define LQ_GATE_SILU 2
+float lq_silu(float x);
+float lq_gelu_tanh(float x);
+float lq_moe_combine(int rule, float g, float u, float limit, float alpha);
+/* cpu_moe_forward's integer expert path over a Q4_K (format 4) or Q6_K (format 6) bank of per-expert slices, routing
+ * given (cpu/ops/moe/forward.rs:160-330, expert/q4k.rs:232-351).  gate_up[e]: [2*inter, cols] rows, gate half first;
+ * down[e]: [hidden, ceil(inter/256)*256]; cols >= hidden is the stored (block-padded) row width. */
+int lq_moe_block_kq(const float *x, size_t tokens, size_t hidden, size_t cols, size_t inter, size_t n_experts, size_t top_k,
+                    const uint64_t *experts, const float *weights, const uint8_t *const *gate_up, const uint8_t *const *down,
+                    int format, const float *gate_up_bias, const float *down_bias, int rule, float limit, float alpha, float *out);
+
 /* ---- multi-threaded drivers for the CPU baseline ----------------------- */
 /* Row-chunk parallel versions (32-row chunks, as the reference schedules
  * them); per-row arithmetic is identical to the serial functions. */

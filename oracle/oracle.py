@@ -91,6 +91,11 @@ _lib.lq_nearest_mxfp4_code.restype = C.c_uint8
 _lib.lq_nearest_mxfp4_code.argtypes = [C.c_float]
 _lib.lq_clamped_glu.restype = C.c_float
 _lib.lq_clamped_glu.argtypes = [C.c_float] * 4
+for _n in ("lq_silu", "lq_gelu_tanh"):
+    getattr(_lib, _n).restype = C.c_float
+    getattr(_lib, _n).argtypes = [C.c_float]
+_lib.lq_moe_combine.restype = C.c_float
+_lib.lq_moe_combine.argtypes = [C.c_int, C.c_float, C.c_float, C.c_float, C.c_float]
 _lib.lq_top_k_by_abs.restype = C.c_long
 _lib.lq_top_k_sorted.restype = C.c_long
 _lib.lq_gate_knn_batch_union.restype = C.c_long
@@ -573,6 +578,51 @@ def moe_block_mxfp4(x, experts, weights, gate, up, down, n_experts: int, hidden:
                                  C.c_int(1 if interleaved else 0), gbp, dbp, C.c_float(limit), C.c_float(alpha), _p(out, _f32p))
     if rc:
         raise ValueError("hidden and inter must be multiples of 32")
+    return out
+
+
+GATE_CLAMPED_GLU, GATE_GELU_TANH, GATE_SILU = 0, 1, 2
+
+
+def silu(x: float) -> float:
+    return _lib.lq_silu(x)
+
+
+def gelu_tanh(x: float) -> float:
+    return _lib.lq_gelu_tanh(x)
+
+
+def moe_combine(rule: int, g: float, u: float, limit: float = 7.0, alpha: float = 1.702) -> float:
+    return _lib.lq_moe_combine(rule, g, u, limit, alpha)
+
+
+def moe_block_kq(x, experts, weights, gate_up, down, hidden: int, cols: int, inter: int, fmt: int = 4, gate_up_bias=None,
+                 down_bias=None, rule: int = GATE_GELU_TANH, limit: float = 7.0, alpha: float = 1.702) -> np.ndarray:
+    """cpu_moe_forward's integer expert path over per-expert k-quant slices (fmt 4 = Q4_K, 6 = Q6_K), routing given.
+    gate_up[e]: bytes of [2*inter, cols] rows (gate half first); down[e]: [hidden, ceil(inter/256)*256] rows."""
+    x = _f32(x)
+    tokens = x.shape[0]
+    ex = np.ascontiguousarray(experts, dtype=np.uint64).reshape(tokens, -1)
+    wt = _f32(weights).reshape(tokens, -1)
+    k = ex.shape[1]
+    gu = [_u8(a).ravel() for a in gate_up]
+    dn = [_u8(a).ravel() for a in down]
+    n_experts = len(gu)
+    blk = 210 if fmt == 6 else 144
+    ip = (inter + 255) // 256 * 256
+    for a, b in zip(gu, dn):
+        if a.size < 2 * inter * (cols // 256) * blk or b.size < hidden * (ip // 256) * blk:
+            raise ValueError("an expert's slices are shorter than the geometry")
+    gup = (C.c_void_p * n_experts)(*[a.ctypes.data for a in gu])
+    dnp = (C.c_void_p * n_experts)(*[a.ctypes.data for a in dn])
+    gb, gbp = _opt_f32(gate_up_bias)
+    db, dbp = _opt_f32(down_bias)
+    out = np.empty((tokens, hidden), np.float32)
+    rc = _lib.lq_moe_block_kq(_p(x, _f32p), _sz(tokens), _sz(hidden), _sz(cols), _sz(inter), _sz(n_experts), _sz(k), _p(ex, _u64p),
+                              _p(wt, _f32p), gup, dnp, C.c_int(fmt), gbp, dbp, C.c_int(rule), C.c_float(limit), C.c_float(alpha),
+                              _p(out, _f32p))
+    if rc:
+        raise ValueError("moe_block_kq: bad geometry")
     return out
 
 

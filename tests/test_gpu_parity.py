@@ -1232,6 +1232,86 @@ def test_moe_layer_from_per_expert_slices_with_router_projection(be, fmt, T, E, 
     be.moe_layer_destroy(layer)
 
 
+@pytest.mark.parametrize("T,E,k,hidden,cols,inter,wfmt,rule,biases,per_expert", [
+    (1, 8, 4, 512, 512, 704, "q4k", 1, False, True),       # Gemma 4 26B-A4B's shape rules in small: inter 704 stored 768 wide, GeluTanh, per-expert scale
+    (5, 128, 8, 768, 768, 256, "q4k", 1, False, True),     # ... its 128 experts, top-8, several tokens
+    (3, 6, 4, 480, 512, 320, "q4k", 0, True, False),       # rows stored wider than hidden (GPT-OSS 2880 -> 3072 in small), ClampedGlu, biases
+    (1, 6, 2, 2816, 2816, 704, "q4k", 1, False, False),    # Gemma 4 26B-A4B's real expert shape
+    (4, 5, 3, 512, 512, 320, "q6k", 2, True, False),       # a Q6_K bank, SiLU
+    (1, 4, 2, 256, 768, 256, "q6k", 1, False, True),
+])
+def test_moe_layer_over_a_k_quant_bank_matches_the_integer_expert_path(be, fmt, T, E, k, hidden, cols, inter, wfmt, rule, biases, per_expert):
+    """MoeLayerWeights with expert_data_format Q4_K / Q6_K (Inline scales, ContiguousHalves rows): cpu_moe_forward's
+    integer path (cpu/ops/moe/forward.rs:160-330) — expert input and gated activation as Q8_K, every matvec the integer
+    kernel.  The route equals moe_route_from_router_input; the output the checker's block under that route (the
+    matvecs are bit-exact, expf / tanhf of the device may move an activation code by one step: 2e-4 is asserted where
+    the stated bar is 1e-3); host tier and device tier agree bit for bit."""
+    rng = np.random.default_rng(700 + T + E + inter)
+    ip = (inter + 255) // 256 * 256
+    quant = O.quantize_q4_k if wfmt == "q4k" else O.quantize_q6_k
+    f = 4 if wfmt == "q4k" else 6
+    gate_up = [quant((rng.standard_normal((2 * inter, cols)) * 0.05).astype(F)) for _ in range(E)]
+    down = [np.concatenate([quant((rng.standard_normal((hidden, ip)) * 0.05).astype(F)), np.full(5 + e, 0xEE, np.uint8)])
+            for e in range(E)]                                                     # (slices may be longer than the geometry)
+    router_w = (rng.standard_normal((E, hidden)) * 0.05).astype(F)
+    router_b = rng.standard_normal(E).astype(F)
+    gub = (rng.standard_normal((E, 2 * inter)) * 0.5).astype(F) if biases else None
+    db = (rng.standard_normal((E, hidden)) * 0.5).astype(F) if biases else None
+    scale = rng.uniform(0.5, 2.0, E).astype(F) if per_expert else None
+    x = rng.standard_normal((T, hidden)).astype(F)
+    rin = (x * F(0.5) + F(0.25)).astype(F)
+    layer = be.moe_layer_create(gate_up, down, None, None, router_w, k, hidden, inter, fmt.MOE_ROWS_CONTIGUOUS_HALVES, router_bias=router_b,
+                                gate_up_bias=gub, down_bias=db, per_expert_scale=scale, expert_scales=fmt.MOE_SCALES_INLINE,
+                                expert_data_format=fmt.FMT_Q4_K if wfmt == "q4k" else fmt.FMT_Q6_K, gate_rule=rule)
+    assert layer, be.last_error()
+    got = be.moe_layer_forward(layer, rin, x, k)
+    assert got is not None, be.last_error()
+    out, experts, weights = got
+    for t in range(T):
+        want = O.moe_route_from_router_input(rin[t], router_w, router_b, k, renormalize=True, per_expert_scale=scale)
+        assert [int(e) for e in experts[t]] == [e for e, _ in want], t
+        assert np.allclose(weights[t], [w for _, w in want], rtol=5e-5, atol=0)
+    want_out = O.moe_block_kq(x, experts, weights, gate_up, down, hidden, cols, inter, f, gub, db, rule)
+    assert rel_l2(out, want_out) < 2e-4
+    dx, dr, do = be.to_device(x), be.to_device(rin), be.malloc(T * hidden * 4)
+    de, dw_ = be.malloc(T * k * 4), be.malloc(T * k * 4)
+    for rep in range(2):                                   # (the second call finds its job tables already on the device)
+        assert be.dev_moe_layer_forward(layer, dr, dx, T, do, de, dw_)
+        be.synchronize()
+        assert np.array_equal(be.d2h(do, (T, hidden), F).view(np.uint32), out.view(np.uint32))
+        assert np.array_equal(be.d2h(de, (T, k), np.uint32), experts)
+    # a token alone gives the token's row of the batch, bit for bit (no arithmetic is shared between tokens)
+    if T > 1:
+        one = be.moe_layer_forward(layer, rin[1:2], x[1:2], k)
+        assert one is not None and np.array_equal(one[0][0].view(np.uint32), out[1].view(np.uint32))
+    be.moe_layer_destroy(layer)
+
+
+def test_moe_layer_k_quant_refusals(be, fmt):
+    """A k-quant bank the CPU tier itself would refuse, or that has no kernel here, answers None: Interleaved rows
+    (forward.rs:69-75), Paired scales, slices shorter than the geometry, rows beyond 10240 elements."""
+    rng = np.random.default_rng(4)
+    E, hidden, inter, k = 3, 256, 256, 2
+    gu = [O.quantize_q4_k((rng.standard_normal((2 * inter, hidden)) * 0.05).astype(F)) for _ in range(E)]
+    dn = [O.quantize_q4_k((rng.standard_normal((hidden, inter)) * 0.05).astype(F)) for _ in range(E)]
+    rw = rng.standard_normal((E, hidden)).astype(F)
+    kw = dict(expert_scales=fmt.MOE_SCALES_INLINE, expert_data_format=fmt.FMT_Q4_K, gate_rule=fmt.MOE_GATE_GELU_TANH)
+    ok = be.moe_layer_create(gu, dn, None, None, rw, k, hidden, inter, fmt.MOE_ROWS_CONTIGUOUS_HALVES, **kw)
+    assert ok
+    be.moe_layer_destroy(ok)
+    assert be.moe_layer_create(gu, dn, None, None, rw, k, hidden, inter, fmt.MOE_ROWS_INTERLEAVED, **kw) is None
+    assert be.moe_layer_create(gu, dn, None, None, rw, k, hidden, inter, fmt.MOE_ROWS_CONTIGUOUS_HALVES,
+                               **dict(kw, expert_scales=fmt.MOE_SCALES_PAIRED)) is None
+    assert be.moe_layer_create(gu, dn, None, None, rw, k, hidden, inter, fmt.MOE_ROWS_CONTIGUOUS_HALVES, **dict(kw, gate_rule=7)) is None
+    assert be.moe_layer_create([g[:-144] for g in gu], dn, None, None, rw, k, hidden, inter, fmt.MOE_ROWS_CONTIGUOUS_HALVES, **kw) is None
+    assert be.moe_layer_create(gu, [d[:-1] for d in dn], None, None, rw, k, hidden, inter, fmt.MOE_ROWS_CONTIGUOUS_HALVES, **kw) is None
+    # an MXFP4 bank under another gate rule: no kernel
+    g4 = [O.quantize_mxfp4((rng.standard_normal(2 * 32 * 64) * 0.02).astype(F), 2 * 32, 64) for _ in range(E)]
+    d4 = [O.quantize_mxfp4((rng.standard_normal(64 * 32) * 0.02).astype(F), 64, 32) for _ in range(E)]
+    assert be.moe_layer_create([g[0] for g in g4], [d[0] for d in d4], [g[1] for g in g4], [d[1] for d in d4], rng.standard_normal((E, 64)).astype(F),
+                               k, 64, 32, gate_rule=fmt.MOE_GATE_SILU) is None
+
+
 def test_moe_layer_refusals(be, fmt):
     """What MoeLayerWeights can say and this backend does not serve answers None (never a wrong bank): inline scales on
     an MXFP4 bank, another expert format, slices shorter than the geometry, more than 256 experts."""
