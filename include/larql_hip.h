@@ -127,7 +127,9 @@ int larql_hip_quantize_x_to_q8k(larql_hip_ctx *ctx, const float *x, size_t n, in
  * bit and so does this one.  Shape rule KernelShapeError::check
  * (cpu/ops/kernel_shape.rs:47-75): out_len == rows, qs_len == cols, cols % 256 == 0,
  * q4k_len >= rows*(cols/256)*144, else REFUSED_SHAPE with `out` untouched; zero
- * dims write zeros.  cols <= 10240 on this backend (longer: UNSUPPORTED). */
+ * dims write zeros.  Rows of more than 10240 elements (the down projections of the larger models) are served as
+ * column ranges whose partial sums are added in range order: the integer sums are the same, the f32 accumulation
+ * meets in another order than the scalar kernel's single chain (about 1e-7 relative instead of bit-exact). */
 int larql_hip_q4k_q8k_matvec(larql_hip_ctx *ctx, const uint8_t *q4k, size_t q4k_len, const int8_t *qs, size_t qs_len,
                              const float *d, const int16_t *sums, size_t num_rows, size_t cols, float *out, size_t out_len);
 /* q4k_q8k_gate_up_into — cpu/ops/q4k_q8k_dot/gate_up.rs:30-57 (shape checks :68-87):

@@ -35,6 +35,15 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 // Clears a few words on the stream (a kernel, not hipMemsetAsync: memset nodes recorded into a captured graph have
 // given wrong results on replays).
+// out[i] = parts[0][i] + parts[1][i] + ... (left to right), the partial vectors `stride` floats apart
+__global__ void sum_partials_kernel(const float *__restrict__ parts, size_t stride, uint32_t n_parts, float *__restrict__ out, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float acc = parts[i];
+    for (uint32_t p = 1; p < n_parts; p++) acc += parts[(size_t)p * stride + i];
+    out[i] = acc;
+}
+
 __global__ void zero_words_kernel(uint32_t *p, uint32_t n) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = 0u;
@@ -74,7 +83,7 @@ struct larql_hip_ctx {
     std::mutex mu;
     std::string name, info, last_error;
     std::vector<Region> regions;
-    DevBuf w[kHostMats], aux[kHostMats], x, out, tables[4], misc, scores, q8, q8s;
+    DevBuf w[kHostMats], aux[kHostMats], x, out, tables[4], misc, scores, q8, q8s, parts;
     // pinned staging for job tables: the upload is asynchronous, the event says when a slot may be rewritten
     void *table_host[4] = {nullptr, nullptr, nullptr, nullptr};
     size_t table_host_cap[4] = {0, 0, 0, 0};
@@ -353,9 +362,77 @@ std::vector<std::vector<GemvJob>> group_by_kind(const std::vector<GemvJob> &jobs
     return groups;
 }
 
+// Q4_K rows longer than the matrix-core kernels take (40 super-blocks of 256) are served as column ranges of at most 40
+// super-blocks: every range a job of its own over the rows of the full matrix (GemvJob::row_stride) into a partial
+// vector of its own, the partial vectors added in range order by sum_partials_kernel.  The ranges of a row of `cpr`
+// super-blocks, as {first super-block, count}: as few as fit, of equal length up to one super-block.
+constexpr uint64_t kQ4kRangeMax = 40;
+std::vector<std::pair<uint64_t, uint64_t>> q4k_row_ranges(uint64_t cpr) {
+    std::vector<std::pair<uint64_t, uint64_t>> r;
+    const uint64_t n = (cpr + kQ4kRangeMax - 1) / kQ4kRangeMax;
+    uint64_t at = 0;
+    for (uint64_t i = 0; i < n; i++) {
+        const uint64_t len = cpr / n + (i < cpr % n ? 1 : 0);
+        r.push_back({at, len});
+        at += len;
+    }
+    return r;
+}
+// The device layout of a Q8_K activation whose row is served in ranges: range after range, each [codes | scales | sums]
+// of its own and 64-byte aligned (the kernel finds a job's scales and sums behind its k codes).
+size_t q8k_ranged_bytes(size_t cols) {
+    size_t total = 0;
+    for (const auto &rg : q4k_row_ranges(cols / 256)) total += (q8k_bytes(rg.second * 256) + 63) & ~(size_t)63;
+    return total;
+}
+struct SplitSum { float *out; size_t parts_off, rows; uint32_t n_parts; };
+// Replaces every plain Q4_K / Q4_K x Q8_K job with rows beyond the kernels' reach by its range jobs (a Q8_K activation
+// must be laid out by q8k_ranged_bytes' rule); `sums` says what to add up afterwards, `parts_floats` how much room the
+// partial vectors take.
+bool split_long_q4k_rows(std::vector<GemvJob> &jobs, std::vector<SplitSum> &sums, size_t &parts_floats) {
+    std::vector<GemvJob> outj;
+    parts_floats = 0;
+    bool any = false;
+    for (const GemvJob &j : jobs) {
+        // (f32 activations: rows of up to 128 super-blocks have the K-slice kernel — one launch, no partial sums, and
+        // measured no slower than ranges plus their addition; the Q8_K kernel has no other way beyond 40)
+        const uint64_t reach = j.kind == KIND_Q4K ? 128 : kQ4kRangeMax;
+        const bool long_row = (j.kind == KIND_Q4K || j.kind == KIND_Q4K_Q8K) && j.k % 256 == 0 && j.k / 256 > reach && j.rows > 0 &&
+                              !j.sel && j.batch <= 1 && !j.bias && !j.row_stride && (j.k / 256) * 144 <= (1ull << 27);
+        if (!long_row) { outj.push_back(j); continue; }
+        any = true;
+        const auto ranges = q4k_row_ranges(j.k / 256);
+        const size_t rows_up = ((size_t)j.rows + 63) & ~(size_t)63;
+        sums.push_back({j.out, parts_floats, (size_t)j.rows, (uint32_t)ranges.size()});
+        size_t q8_off = 0;
+        for (size_t i = 0; i < ranges.size(); i++) {
+            GemvJob s = j;
+            s.w = j.w + ranges[i].first * 144;
+            s.row_stride = (j.k / 256) * 144;
+            s.k = ranges[i].second * 256;
+            if (j.kind == KIND_Q4K) s.x = j.x + ranges[i].first * 256;
+            else { s.x = (const float *)((const uint8_t *)j.x + q8_off); q8_off += (q8k_bytes(s.k) + 63) & ~(size_t)63; }
+            s.out = reinterpret_cast<float *>((uintptr_t)((parts_floats + i * rows_up) * sizeof(float)));  // (a byte offset into the partial area: rebased by the caller)
+            outj.push_back(s);
+        }
+        parts_floats += ranges.size() * rows_up;
+    }
+    if (any) jobs.swap(outj);
+    return any;
+}
+
 // Enqueue `jobs` (device operands): one launch per format present, in first-seen
 // order.  Jobs with no rows are dropped.
-int enqueue_jobs(larql_hip_ctx *c, std::vector<GemvJob> &jobs) {
+int enqueue_jobs(larql_hip_ctx *c, std::vector<GemvJob> &jobs_in) {
+    std::vector<GemvJob> jobs(jobs_in);
+    std::vector<SplitSum> sums;
+    size_t parts_floats = 0;
+    if (split_long_q4k_rows(jobs, sums, parts_floats)) {
+        int rc0 = ensure(c, c->parts, parts_floats * sizeof(float) + 64);
+        if (rc0) return rc0;
+        for (GemvJob &j : jobs)
+            if (j.row_stride) j.out = reinterpret_cast<float *>((uint8_t *)c->parts.p + reinterpret_cast<uintptr_t>(j.out));
+    }
     int rc = check_jobs(c, jobs);
     if (rc) return rc;
     int slot = 0;
@@ -372,6 +449,12 @@ int enqueue_jobs(larql_hip_ctx *c, std::vector<GemvJob> &jobs) {
         rc = prepare_same_kind(c, live.data(), live.size(), tb.p, P, sl);
         if (rc) return rc;
         HIPCHECK(c, gemv_launch(c->stream, P.kind, P.L, P.threads, P.grid, P.lds));
+    }
+    for (const SplitSum &sm : sums) {
+        const size_t rows_up = (sm.rows + 63) & ~(size_t)63;
+        hipLaunchKernelGGL(sum_partials_kernel, dim3((unsigned)((sm.rows + 255) / 256)), dim3(256), 0, c->stream,
+                           (const float *)c->parts.p + sm.parts_off, rows_up, sm.n_parts, sm.out, sm.rows);
+        HIPCHECK(c, hipGetLastError());
     }
     return LARQL_OK;
 }
@@ -448,7 +531,7 @@ void larql_hip_destroy(larql_hip_ctx *c) {
     (void)hipSetDevice(c->device);
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     for (Region &r : c->regions) (void)hipFree(r.dev);
-    DevBuf *bufs[] = {&c->x, &c->out, &c->tables[0], &c->tables[1], &c->tables[2], &c->tables[3], &c->misc, &c->scores, &c->q8, &c->q8s};
+    DevBuf *bufs[] = {&c->x, &c->out, &c->tables[0], &c->tables[1], &c->tables[2], &c->tables[3], &c->misc, &c->scores, &c->q8, &c->q8s, &c->parts};
     for (DevBuf *b : bufs) if (b->p) (void)hipFree(b->p);
     for (size_t i = 0; i < kHostMats; i++) {
         if (c->w[i].p) (void)hipFree(c->w[i].p);
@@ -661,6 +744,16 @@ static void pack_q8k(uint8_t *dst, const int8_t *qs, const float *d, const int16
     memcpy(dst + cols, d, (cols / 256) * 4);
     memcpy(dst + cols + (cols / 256) * 4, sums, (cols / 32) * 2);
 }
+// ... range after range where the row is longer than one job takes (q8k_ranged_bytes; a row of up to 10240 elements is one range)
+static std::vector<uint8_t> pack_q8k_ranged(const int8_t *qs, const float *d, const int16_t *sums, size_t cols) {
+    std::vector<uint8_t> packed(q8k_ranged_bytes(cols), 0);
+    size_t off = 0;
+    for (const auto &rg : q4k_row_ranges(cols / 256)) {
+        pack_q8k(packed.data() + off, qs + rg.first * 256, d + rg.first, sums + rg.first * 8, rg.second * 256);
+        off += (q8k_bytes(rg.second * 256) + 63) & ~(size_t)63;
+    }
+    return packed;
+}
 
 int larql_hip_q4k_q8k_matvec(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_len, const int8_t *qs, size_t qs_len, const float *d,
                              const int16_t *sums, size_t num_rows, size_t cols, float *out, size_t out_len) {
@@ -671,9 +764,8 @@ int larql_hip_q4k_q8k_matvec(larql_hip_ctx *c, const uint8_t *q4k, size_t q4k_le
                     out_len, num_rows, qs_len, cols, q4k_len);
     if (num_rows == 0 || cols == 0) { for (size_t i = 0; i < out_len; i++) out[i] = 0.0f; return LARQL_OK; }
     if (!q4k || !qs || !d || !sums) return LARQL_E_ARG;
-    if (cols / 256 > 40) return fail(c, LARQL_UNSUPPORTED, "q4k_q8k_matvec: rows longer than 10240 have no kernel");
-    std::vector<uint8_t> packed(q8k_bytes(cols));
-    pack_q8k(packed.data(), qs, d, sums, cols);
+    if ((cols / 256) * 144 > (1ull << 27)) return fail(c, LARQL_UNSUPPORTED, "q4k_q8k_matvec: rows this long have no kernel");
+    const std::vector<uint8_t> packed = pack_q8k_ranged(qs, d, sums, cols);
     const size_t need = (cols / 256) * 144 * num_rows;
     return host_matvec_multi(c, KIND_Q4K_Q8K, 1, &q4k, &need, nullptr, nullptr, &num_rows, cols, (const float *)packed.data(), packed.size(), &out);
 }
@@ -689,9 +781,8 @@ int larql_hip_q4k_q8k_gate_up(larql_hip_ctx *c, const uint8_t *gate_w, size_t ga
                     out_len, num_rows, qs_len, cols, gate_len, up_len);
     if (num_rows == 0 || cols == 0) { for (size_t i = 0; i < out_len; i++) { gate_out[i] = 0.0f; up_out[i] = 0.0f; } return LARQL_OK; }
     if (!gate_w || !up_w || !qs || !d || !sums) return LARQL_E_ARG;
-    if (cols / 256 > 40) return fail(c, LARQL_UNSUPPORTED, "q4k_q8k_gate_up: rows longer than 10240 have no kernel");
-    std::vector<uint8_t> packed(q8k_bytes(cols));
-    pack_q8k(packed.data(), qs, d, sums, cols);
+    if ((cols / 256) * 144 > (1ull << 27)) return fail(c, LARQL_UNSUPPORTED, "q4k_q8k_gate_up: rows this long have no kernel");
+    const std::vector<uint8_t> packed = pack_q8k_ranged(qs, d, sums, cols);
     const size_t need = (cols / 256) * 144 * num_rows;
     const uint8_t *w[2] = {gate_w, up_w};
     const size_t needs[2] = {need, need}, rows[2] = {num_rows, num_rows};

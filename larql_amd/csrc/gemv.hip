@@ -3204,6 +3204,7 @@ bool gemv_refine_costs(GemvJob *jobs, size_t n, uint32_t grid) {
 }
 
 bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
+    if (j.row_stride && j.kind != KIND_Q4K_MFMA && j.kind != KIND_Q4K_Q8K) return false;  // (column ranges: those two kernels only)
     if (j.kind == KIND_Q8_0_MFMA) {
         const uint64_t cpr = j.k / 256;
         const uint32_t nw = q8_mfma_waves(cpr);
@@ -3285,6 +3286,10 @@ bool gemv_job_geometry(GemvJob &j, uint32_t threads) {
         j.cpr = (uint32_t)cpr;
         j.rpp = nw;  // wavefronts that work on this job
         j.row_bytes = cpr * 144;
+        if (j.row_stride) {  // a column range of a wider matrix (the kernels form 16 x row_bytes in 32 bits)
+            if (j.row_stride % 144 != 0 || j.row_stride < cpr * 144 || j.row_stride > (1ull << 27)) return false;
+            j.row_bytes = j.row_stride;
+        }
         const uint64_t tiles = (j.rows + 15) / 16;
         uint64_t cpt, startup;
         q4k_tile_cost(cpr, nw, &cpt, &startup);

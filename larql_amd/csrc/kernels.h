@@ -80,7 +80,9 @@ struct GemvJob {
     const float *combine_w;
     // Optional router bias [route_n], added to route_logits before the selection (it changes which experts win).
     const float *route_bias;
-    uint64_t pad3;
+    // Optional (matrix-core Q4_K kernels only): bytes from one weight row to the next when the job covers a column
+    // range of a wider matrix — w points at the range's first super-block of row 0.  0 = rows are packed (row_bytes).
+    uint64_t row_stride;
 };
 static_assert(sizeof(GemvJob) % 16 == 0, "the descriptor is a whole number of 16-byte words (moe_plan_kernel stores it that way)");
 

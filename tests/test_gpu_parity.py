@@ -224,8 +224,48 @@ def test_q4k_q8k_matvec_shape_rules(be):
     assert be.q4k_q8k_matvec(w, *a, 2, 512, out_len=1) is None                             # output shorter than rows
     z = be.q4k_q8k_matvec(np.zeros(0, np.uint8), np.zeros(0, np.int8), np.zeros(0, F), np.zeros(0, np.int16), 3, 0)
     assert z is not None and z.shape == (3,) and not z.any()                               # zero dims give zeros
-    big = O.quantize_x_to_q8k(np.ones(10496, F))                                           # 41 super-blocks: no kernel
-    assert be.q4k_q8k_matvec(np.zeros(41 * 144, np.uint8), *big, 1, 10496) is None
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 10496), (70, 15360), (33, 21504), (19, 28672), (5, 40960)])
+def test_q4k_q8k_rows_beyond_one_pass_are_served_in_column_ranges(be, rows, cols):
+    """Rows longer than 40 super-blocks (the down projections of Gemma-3-12B / 27B and the Llamas: 15360, 21504, 14336,
+    28672) are served as column ranges whose partial sums are added in range order: the integer sums are the reference's,
+    the f32 accumulation meets in another order than q4k_q8k_matvec_scalar's single chain (1e-6 is asserted where rows of
+    up to 10240 elements are bit-exact); gate_up the same, still equal to the single calls bit for bit."""
+    w, x = weights(rows + cols, rows, cols)
+    q = O.quantize_q4_k(w)
+    a = O.quantize_x_to_q8k(x * F(2.5))
+    want = O.q4k_q8k_matvec(q, *a, rows, cols)
+    got = be.q4k_q8k_matvec(q, *a, rows, cols)
+    assert got is not None, be.last_error()
+    assert rel_l2(got, want) < 1e-6 and np.max(np.abs(got - want)) < 1e-5 * (np.abs(want).mean() + 1e-9)
+    assert np.array_equal(got.view(np.uint32), be.q4k_q8k_matvec(q, *a, rows, cols).view(np.uint32))
+    w2, _ = weights(rows + cols + 1, rows, cols)
+    q2 = O.quantize_q4_k(w2)
+    gu = be.q4k_q8k_gate_up(q, q2, *a, rows, cols)
+    assert gu is not None and np.array_equal(gu[0].view(np.uint32), got.view(np.uint32))
+    assert np.array_equal(gu[1].view(np.uint32), be.q4k_q8k_matvec(q2, *a, rows, cols).view(np.uint32))
+
+
+@pytest.mark.parametrize("rows,cols", [(48, 15360), (130, 32768), (3, 33024), (7, 65536), (20, 102400)])
+def test_q4k_rows_of_any_length_are_served(be, fmt, rows, cols):
+    """The f32-activation matvec over long rows: up to 32768 elements the K-slice kernel, beyond that column ranges on the
+    matrix-core kernel with the partial sums added in range order — host tier and device tier (one job, and next to a
+    short-row job in one call)."""
+    w, x = weights(rows * 5 + cols, rows, cols)
+    q = O.quantize_q4_k(w)
+    want = O.q4k_matvec(q, x, rows, cols)
+    got = be.q4k_matvec(q, x, rows, cols)
+    assert got is not None, be.last_error()
+    assert rel_l2(got, want) < TOL and np.max(np.abs(got - want)) < 1e-3 * (np.abs(want).mean() + 1e-12)
+    dw, dx, do, do2 = be.to_device(q), be.to_device(x), be.malloc(rows * 4), be.malloc(64 * 4)
+    w3, _ = weights(9, 64, 512)
+    q3 = O.quantize_q4_k(w3)
+    dw3 = be.to_device(q3)
+    assert be.dev_matvec_batch([(fmt.FMT_Q4_K, dw, 0, dx, do, rows, cols), (fmt.FMT_Q4_K, dw3, 0, dx, do2, 64, 512)])
+    be.synchronize()
+    assert np.array_equal(be.d2h(do, rows, F).view(np.uint32), got.view(np.uint32))
+    assert rel_l2(be.d2h(do2, 64, F), O.q4k_matvec(q3, x[:512], 64, 512)) < TOL
 
 
 def test_q4k_q8k_device_tier_plan_matches_host_tier(be, fmt):
