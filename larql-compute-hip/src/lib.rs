@@ -73,6 +73,24 @@ impl HipMoeLayer<'_> {
     }
 }
 
+impl HipMoeLayer<'_> {
+    /// `cpu_moe_forward(h, moe, norm_offset, eps)` (crates/larql-compute/src/cpu/ops/moe/forward.rs:24-31) for one token,
+    /// the router and the expert block on the device: the inputs are derived from the residual and the output is
+    /// post-normed under `moe.routing_policy` by the reference's own functions (`moe_expert_input`, `moe_router_input`,
+    /// `moe_post_expert_output`, cpu/ops/moe/mod.rs:55-200) — hidden-sized vector work that stays on the host, as it
+    /// does in front of the Metal peer's expert dispatch.  `moe` must be the layer this handle was created from.
+    pub fn forward_residual(&self, h: &[f32], moe: &MoeLayerWeights<'_>, norm_offset: f32, eps: f32) -> Option<Vec<f32>> {
+        use larql_compute::cpu::ops::moe::{moe_expert_input, moe_post_expert_output, moe_router_input};
+        if h.len() != self.hidden {
+            return None;
+        }
+        let expert_input = moe_expert_input(h, moe, norm_offset, eps);
+        let router_in = moe_router_input(h, &expert_input, moe, norm_offset, eps);
+        let (out, _, _) = self.forward(&router_in, &expert_input, 1)?;
+        Some(moe_post_expert_output(&out, moe, norm_offset, eps))
+    }
+}
+
 impl Drop for HipMoeLayer<'_> {
     fn drop(&mut self) {
         // SAFETY: the handle came from larql_hip_moe_layer_create on this context and is dropped once.
