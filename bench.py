@@ -18,7 +18,8 @@ region) and `cpu_baseline` (the CPU oracle's restatement of the reference
 kernels, multi-threaded, on a bounded sample of the same weights).
 
 The headline step submits the 239 matvecs as mutually independent jobs: it is
-a streaming-bandwidth figure, not a decode rate.  `config.dependency_ordered`
+a streaming-bandwidth figure, not a decode rate.  `decode_in_dependency_order`
+(beside `value`; in full under `config.dependency_ordered`)
 reports the same weights walked as a token would walk them — per layer the
 stages q,k,v | o | gate,up | down, each stage reading the previous stage's
 output, 137 dependent launches — with its own ms per token.  `config.other_configs`
@@ -822,6 +823,11 @@ def main():
                      "traffic": read_traffic()},
         "cpu_baseline": cpu,
     }
+    if dependency:
+        # beside the headline: the rate a token sees when every stage waits for the one before it (full detail in config)
+        out["decode_in_dependency_order"] = {
+            "tokens_per_s": dependency["tokens_per_s"], "ms_per_token": dependency["ms_per_token_device"], "GB/s": dependency["GBps"],
+            "frac_of_hbm_peak": round(dependency["pct_of_hbm_peak"] / 100.0, 4), "dependent_launches_per_token": dependency["launches_per_token"]}
     print(json.dumps(out))
 
 
