@@ -216,7 +216,8 @@ impl HipBackend {
     /// per-expert slices and their paired exponent streams go up expert by expert, wherever their mmap ranges lie.
     /// Served: an MXFP4 bank with `Paired` scales under `ClampedGlu` (a native GPT-OSS bank), and a Q4_K / Q6_K bank with
     /// `Inline` scales and `ContiguousHalves` rows under `ClampedGlu` or `Gated` (the per-layer k-quant files of Gemma 4
-    /// 26B-A4B: `cpu_moe_forward`'s integer path, crates/larql-compute/src/cpu/ops/moe/forward.rs:160-330).  `None` where
+    /// 26B-A4B: `cpu_moe_forward`'s integer path, crates/larql-compute/src/cpu/ops/moe/forward.rs:160-330), and a BF16 /
+    /// F16 / F32 bank on that function's f32 arm (forward.rs:246-290).  `None` where
     /// this backend has no kernel for the layer (other formats or rules, more than 256 experts, top-k above 8) — the
     /// caller keeps `cpu_moe_forward`.
     pub fn moe_layer<'a>(&'a self, moe: &MoeLayerWeights<'_>, hidden: usize) -> Option<HipMoeLayer<'a>> {

@@ -2022,7 +2022,8 @@ struct larql_hip_moe_layer {
     int renormalized = 1, per_expert_scale = 0;
     // a k-quant (Q4_K / Q6_K) bank: expert e's gate rows at kq_gate + e * kq_gu_stride, its up rows at kq_up + the same,
     // its down rows at kq_down + e * kq_dn_stride; rows `cols` (gate, up) and `inter_padded` (down) elements wide
-    int kq_kind = 0;  // 0: an MXFP4 bank (`bank`); else KIND_Q4K_Q8K / KIND_Q6K_Q8K
+    int kq_kind = 0;  // 0: an MXFP4 bank (`bank`); else KIND_Q4K_Q8K / KIND_Q6K_Q8K, or (kq_dense) KIND_BF16 / KIND_F16 / KIND_F32
+    bool kq_dense = false;
     const uint8_t *kq_gate = nullptr, *kq_up = nullptr, *kq_down = nullptr;
     uint64_t kq_gu_stride = 0, kq_dn_stride = 0;
     size_t cols = 0, inter_padded = 0;
@@ -2044,11 +2045,15 @@ void larql_hip_moe_layer_destroy(larql_hip_ctx *c, larql_hip_moe_layer *L) {
 // A Q4_K / Q6_K bank (the caller holds the context's lock): what cpu_moe_forward's integer path reads.
 static int moe_layer_create_kq(larql_hip_ctx *c, const larql_hip_moe_layer_weights *w, larql_hip_moe_layer **out) {
     const size_t E = w->num_experts, hidden = w->hidden, inter = w->intermediate_size;
-    const size_t blk = w->expert_data_format == LARQL_FMT_Q6_K ? 210 : 144;
+    // a float bank (BF16: the legacy monolith; F16, F32) takes the same way with f32 activations and the dense matvec
+    // kernels (cpu_moe_forward's f32 arm, forward.rs:246-290); `blk` bytes hold `bel` elements of a row
+    const bool dense = w->expert_data_format == LARQL_FMT_BF16 || w->expert_data_format == LARQL_FMT_F16 || w->expert_data_format == LARQL_FMT_F32;
+    const size_t blk = dense ? (w->expert_data_format == LARQL_FMT_F32 ? 4 : 2) : w->expert_data_format == LARQL_FMT_Q6_K ? 210 : 144;
+    const size_t bel = dense ? 1 : 256;
     if (w->expert_scales != LARQL_MOE_SCALES_INLINE)
-        return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: a k-quant bank carries its scales inside its blocks (MoeExpertScales::Inline)");
+        return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: a k-quant or float bank has no scale stream of its own (MoeExpertScales::Inline)");
     if (w->fused_row_layout != LARQL_MOE_ROWS_CONTIGUOUS_HALVES)
-        return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: a k-quant bank is read as contiguous gate / up halves, as cpu_moe_forward reads it");
+        return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: a k-quant or float bank is read as contiguous gate / up halves, as cpu_moe_forward reads it");
     if (w->gate_rule != LARQL_MOE_GATE_CLAMPED_GLU && w->gate_rule != LARQL_MOE_GATE_GELU_TANH && w->gate_rule != LARQL_MOE_GATE_SILU)
         return fail(c, LARQL_UNSUPPORTED, "moe_layer: unknown gate rule");
     if (E == 0 || w->top_k == 0 || hidden == 0 || inter == 0) return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: empty layer");
@@ -2059,12 +2064,19 @@ static int moe_layer_create_kq(larql_hip_ctx *c, const larql_hip_moe_layer_weigh
     size_t cols = hidden;
     {
         const size_t len = w->experts_gate_up_len[0];
-        if (len % (2 * inter) == 0 && (len / (2 * inter)) % blk == 0 && len / (2 * inter) / blk * 256 >= hidden) cols = len / (2 * inter) / blk * 256;
+        if (len % (2 * inter) == 0 && (len / (2 * inter)) % blk == 0 && len / (2 * inter) / blk * bel >= hidden) cols = len / (2 * inter) / blk * bel;
     }
-    const size_t ip = (inter + 255) / 256 * 256;  // MoeWeightLayout::quant_block_padded_down
-    if (cols % 256 != 0) return fail(c, LARQL_UNSUPPORTED, "moe_layer: k-quant rows must be whole 256-element super-blocks");
-    if (cols / 256 > 40 || ip / 256 > 40) return fail(c, LARQL_UNSUPPORTED, "moe_layer: k-quant rows longer than 10240 elements have no kernel");
-    const size_t half = inter * (cols / 256) * blk, dn = hidden * (ip / 256) * blk;
+    // MoeWeightLayout::quant_block_padded_down (moe.rs:184-200): a block format pads `inter` to whole blocks, a float format does not
+    const size_t ip = dense ? inter : (inter + 255) / 256 * 256;
+    if (dense) {
+        if (cols != hidden) return fail(c, LARQL_UNSUPPORTED, "moe_layer: float expert rows wider than hidden are not served");
+        if (cols % 16 != 0 || inter % 16 != 0 || cols > 8192 || inter > 8192)
+            return fail(c, LARQL_UNSUPPORTED, "moe_layer: float expert rows must be multiples of 16 elements, at most 8192");
+    } else {
+        if (cols % 256 != 0) return fail(c, LARQL_UNSUPPORTED, "moe_layer: k-quant rows must be whole 256-element super-blocks");
+        if (cols / 256 > 40 || ip / 256 > 40) return fail(c, LARQL_UNSUPPORTED, "moe_layer: k-quant rows longer than 10240 elements have no kernel");
+    }
+    const size_t half = inter * (cols / bel) * blk, dn = hidden * (ip / bel) * blk;
     for (size_t e = 0; e < E; e++) {
         if (!w->experts_gate_up[e] || !w->experts_down[e]) return LARQL_E_ARG;
         if (w->experts_gate_up_len[e] < 2 * half || w->experts_down_len[e] < dn)
@@ -2107,7 +2119,8 @@ static int moe_layer_create_kq(larql_hip_ctx *c, const larql_hip_moe_layer_weigh
         delete L;
         return fail(c, LARQL_E_DEVICE, "moe_layer: upload: %s", hipGetErrorString(e));
     }
-    L->kq_kind = w->expert_data_format == LARQL_FMT_Q6_K ? KIND_Q6K_Q8K : KIND_Q4K_Q8K;
+    L->kq_kind = dense ? kind_of_format(w->expert_data_format) : w->expert_data_format == LARQL_FMT_Q6_K ? KIND_Q6K_Q8K : KIND_Q4K_Q8K;
+    L->kq_dense = dense;
     L->kq_gate = d + o_g; L->kq_up = d + o_u; L->kq_down = d + o_d;
     L->kq_gu_stride = hs; L->kq_dn_stride = ds;
     L->cols = cols; L->inter_padded = ip;
@@ -2128,9 +2141,11 @@ int larql_hip_moe_layer_create(larql_hip_ctx *c, const larql_hip_moe_layer_weigh
     if (!c || !w || !out) return LARQL_E_ARG;
     *out = nullptr;
     std::lock_guard<std::mutex> lk(c->mu);
-    if (w->expert_data_format == LARQL_FMT_Q4_K || w->expert_data_format == LARQL_FMT_Q6_K) return moe_layer_create_kq(c, w, out);
+    if (w->expert_data_format == LARQL_FMT_Q4_K || w->expert_data_format == LARQL_FMT_Q6_K || w->expert_data_format == LARQL_FMT_BF16 ||
+        w->expert_data_format == LARQL_FMT_F16 || w->expert_data_format == LARQL_FMT_F32)
+        return moe_layer_create_kq(c, w, out);
     if (w->expert_data_format != LARQL_FMT_MXFP4)
-        return fail(c, LARQL_UNSUPPORTED, "moe_layer: MXFP4, Q4_K and Q6_K expert banks are served by this backend");
+        return fail(c, LARQL_UNSUPPORTED, "moe_layer: MXFP4, Q4_K, Q6_K and float expert banks are served by this backend");
     if (w->gate_rule != LARQL_MOE_GATE_CLAMPED_GLU)
         return fail(c, LARQL_UNSUPPORTED, "moe_layer: an MXFP4 bank is served under MoeGateRule::ClampedGlu only");
     if (w->expert_scales != LARQL_MOE_SCALES_PAIRED)
@@ -2242,12 +2257,16 @@ static int moe_layer_enqueue(larql_hip_ctx *c, larql_hip_moe_layer *L, const flo
         if (tokens > 65535 || slots > 65535) return fail(c, LARQL_UNSUPPORTED, "moe_layer: too many tokens in one call for a k-quant bank");
         HIPCHECK(c, router_select_launch(c->stream, logits, L->router_bias, (uint32_t)tokens, (uint32_t)E, (uint32_t)k, policy, experts, weights));
         if (L->per_expert_scale) HIPCHECK(c, expert_scale_launch(c->stream, weights, experts, L->scale, (uint32_t)slots, (uint32_t)E));
-        const size_t xq_stride = (q8k_bytes(cols) + 255) & ~(size_t)255, aq_stride = (q8k_bytes(ip) + 255) & ~(size_t)255;
+        // (a float bank: the activations stay f32 — x itself, and one row of `inter` floats per slot)
+        const bool dense = L->kq_dense;
+        const size_t xq_stride = dense ? hidden * sizeof(float) : (q8k_bytes(cols) + 255) & ~(size_t)255;
+        const size_t aq_stride = dense ? ((inter * sizeof(float) + 255) & ~(size_t)255) : (q8k_bytes(ip) + 255) & ~(size_t)255;
         const size_t f_bytes = ((2 * slots * inter + slots * hidden) * sizeof(float) + 255) & ~(size_t)255;
-        rc = ensure(c, L->ws, f_bytes + tokens * xq_stride + slots * aq_stride + 256); if (rc) return rc;
+        rc = ensure(c, L->ws, f_bytes + (dense ? 0 : tokens * xq_stride) + slots * aq_stride + 256); if (rc) return rc;
         float *g = (float *)L->ws.p, *u = g + slots * inter, *dd = u + slots * inter;
-        uint8_t *xq = (uint8_t *)L->ws.p + f_bytes, *aq = xq + tokens * xq_stride;
-        HIPCHECK(c, quantize_rows_to_q8k_launch(c->stream, x, hidden, (uint32_t)hidden, (uint32_t)cols, (uint32_t)tokens, xq, xq_stride));
+        uint8_t *xq = dense ? (uint8_t *)const_cast<float *>(x) : (uint8_t *)L->ws.p + f_bytes;
+        uint8_t *aq = dense ? (uint8_t *)L->ws.p + f_bytes : xq + tokens * xq_stride;
+        if (!dense) HIPCHECK(c, quantize_rows_to_q8k_launch(c->stream, x, hidden, (uint32_t)hidden, (uint32_t)cols, (uint32_t)tokens, xq, xq_stride));
         jobs.clear();
         for (size_t s = 0; s < slots; s++) {
             GemvJob a = make_job(L->kq_kind, L->kq_gate, nullptr, xq + (s / k) * xq_stride, g + s * inter, inter, cols);
@@ -2259,8 +2278,12 @@ static int moe_layer_enqueue(larql_hip_ctx *c, larql_hip_moe_layer *L, const flo
         }
         rc = enqueue_jobs(c, jobs);
         if (rc) return rc;
-        HIPCHECK(c, moe_kq_act_q8k_launch(c->stream, g, u, (uint32_t)inter, (uint32_t)ip, (uint32_t)slots, experts, (uint32_t)E, L->kq_gub, L->gate_rule,
-                                          L->glu_limit, L->glu_alpha, aq, aq_stride));
+        if (dense)
+            HIPCHECK(c, moe_act_f32_launch(c->stream, g, u, (uint32_t)inter, (uint32_t)slots, experts, (uint32_t)E, L->kq_gub, L->gate_rule, L->glu_limit,
+                                           L->glu_alpha, (float *)aq, aq_stride / sizeof(float)));
+        else
+            HIPCHECK(c, moe_kq_act_q8k_launch(c->stream, g, u, (uint32_t)inter, (uint32_t)ip, (uint32_t)slots, experts, (uint32_t)E, L->kq_gub, L->gate_rule,
+                                              L->glu_limit, L->glu_alpha, aq, aq_stride));
         jobs.clear();
         for (size_t s = 0; s < slots; s++) {
             GemvJob a = make_job(L->kq_kind, L->kq_down, nullptr, aq + s * aq_stride, dd + s * hidden, hidden, ip);

@@ -175,6 +175,20 @@ __global__ void __launch_bounds__(256) moe_kq_act_q8k_kernel(const float *__rest
     q8k_store(dst + (size_t)slot * dst_stride, inter_padded, sb, lane, codes, scale, sum);
 }
 
+// The same activation kept as f32 (a float bank: cpu_moe_forward's f32 arm, forward.rs:262-267): slot `blockIdx.y`'s row
+// of `inter` floats at act + slot * act_stride.
+__global__ void __launch_bounds__(256) moe_act_f32_kernel(const float *__restrict__ g, const float *__restrict__ u, uint32_t inter,
+                                                         const uint32_t *__restrict__ experts, uint32_t n_experts, const float *__restrict__ gub, int rule,
+                                                         float limit, float alpha, float *__restrict__ act, size_t act_stride) {
+    const uint32_t j = blockIdx.x * blockDim.x + threadIdx.x, slot = blockIdx.y;
+    if (j >= inter) return;
+    const uint32_t e = experts[slot];
+    const float *b = (gub && e < n_experts) ? gub + (size_t)e * 2 * inter : nullptr;
+    const float gv = g[(size_t)slot * inter + j] + (b ? b[2 * j] : 0.0f);
+    const float uv = u[(size_t)slot * inter + j] + (b ? b[2 * j + 1] : 0.0f);
+    act[(size_t)slot * act_stride + j] = moe_combine(rule, gv, uv, limit, alpha);
+}
+
 // out[t] = sum over the token's k slots, in selection order, of w * (down output + the expert's down bias)
 // (forward.rs:220-228: add_down_bias, then `*a += w * v`); a slot whose expert lies outside the bank is skipped.
 __global__ void weighted_sum_bias_kernel(const float *__restrict__ d, const float *__restrict__ weights, const uint32_t *__restrict__ experts,
@@ -473,6 +487,13 @@ hipError_t moe_kq_act_q8k_launch(hipStream_t s, const float *g, const float *u, 
     if (slots == 0 || inter_padded < 256) return hipSuccess;
     hipLaunchKernelGGL(moe_kq_act_q8k_kernel, dim3((inter_padded / 256 + 3) / 4, slots), dim3(256), 0, s, g, u, inter, inter_padded, experts, n_experts,
                        gub, rule, limit, alpha, dst, dst_stride);
+    return hipGetLastError();
+}
+hipError_t moe_act_f32_launch(hipStream_t s, const float *g, const float *u, uint32_t inter, uint32_t slots, const uint32_t *experts, uint32_t n_experts,
+                              const float *gub, int rule, float limit, float alpha, float *act, size_t act_stride) {
+    if (slots == 0 || inter == 0) return hipSuccess;
+    hipLaunchKernelGGL(moe_act_f32_kernel, dim3((inter + 255) / 256, slots), dim3(256), 0, s, g, u, inter, experts, n_experts, gub, rule, limit, alpha,
+                       act, act_stride);
     return hipGetLastError();
 }
 hipError_t weighted_sum_bias_launch(hipStream_t s, const float *d, const float *weights, const uint32_t *experts, uint32_t n_experts,

@@ -280,7 +280,8 @@ class HipBackend {
 
     // A MoE layer made resident from MoeLayerWeights: the per-expert slices and their paired exponent streams go up
     // expert by expert, wherever they lie.  Served: an MXFP4 bank with Paired scales under ClampedGlu, and a Q4_K / Q6_K
-    // bank with Inline scales and ContiguousHalves rows under ClampedGlu or Gated (cpu_moe_forward's integer path).
+    // bank with Inline scales and ContiguousHalves rows under ClampedGlu or Gated (cpu_moe_forward's integer path); a
+    // BF16 / F16 / F32 bank likewise (its f32 arm).
     // nullopt where this backend has no kernel for the layer (other formats or rules, more than 256 experts, top-k
     // above 8): the caller keeps cpu_moe_forward.
     std::optional<HipMoeLayer> moe_layer(const MoeLayerWeights &moe, size_t hidden) {

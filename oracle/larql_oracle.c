@@ -1367,6 +1367,49 @@ float lq_moe_combine(int rule, float g, float u, float limit, float alpha) {
     return lq_clamped_glu(g, u, limit, alpha);
 }
 
+/* cpu_moe_forward's f32 arm (cpu/ops/moe/forward.rs:246-290) over a float bank — format 16 = BF16 (the legacy monolith),
+ * 17 = F16, 32 = F32: the slab is dequantised to f32 and met by matmul_vec (BLAS sgemv there; a sequential f32 dot here,
+ * as in lq_moe_block_f32), gate and up the two halves of [2*inter, cols], down [hidden, inter] unpadded (a float format has
+ * no block to pad to: MoeWeightLayout::down_cols, pipeline/moe.rs:184-200); biases, rule and weighting as below. */
+static void float_gemv(int format, const uint8_t *w, const float *x, size_t n, size_t k, float *out) {
+    if (format == 16) lq_bf16_gemv((const uint16_t *)w, x, n, k, out);
+    else if (format == 17) lq_f16_gemv((const uint16_t *)w, x, n, k, out);
+    else lq_f32_gemv((const float *)w, x, n, k, out);
+}
+static int moe_block_float(const float *x, size_t tokens, size_t hidden, size_t cols, size_t inter, size_t n_experts, size_t top_k,
+                           const uint64_t *experts, const float *weights, const uint8_t *const *gate_up, const uint8_t *const *down,
+                           int format, const float *gate_up_bias, const float *down_bias, int rule, float limit, float alpha, float *out) {
+    if (cols < hidden) return 1;
+    const size_t el = format == 32 ? 4 : 2;
+    float *xp = (float *)calloc(cols ? cols : 1, sizeof(float));
+    float *g = (float *)malloc((inter ? inter : 1) * sizeof(float)), *u = (float *)malloc((inter ? inter : 1) * sizeof(float));
+    float *act = (float *)malloc((inter ? inter : 1) * sizeof(float)), *h2 = (float *)malloc((hidden ? hidden : 1) * sizeof(float));
+    for (size_t t = 0; t < tokens; t++) {
+        float *o = out + t * hidden;
+        for (size_t i = 0; i < hidden; i++) { o[i] = 0.0f; xp[i] = x[t * hidden + i]; }
+        if (inter == 0) continue;
+        for (size_t s = 0; s < top_k; s++) {
+            const uint64_t e = experts[t * top_k + s];
+            const float w = weights[t * top_k + s];
+            if (e >= n_experts) continue;
+            float_gemv(format, gate_up[e], xp, inter, cols, g);
+            float_gemv(format, gate_up[e] + inter * cols * el, xp, inter, cols, u);
+            for (size_t j = 0; j < inter; j++) {
+                const float gb = gate_up_bias ? gate_up_bias[e * 2 * inter + 2 * j] : 0.0f;
+                const float ub = gate_up_bias ? gate_up_bias[e * 2 * inter + 2 * j + 1] : 0.0f;
+                act[j] = lq_moe_combine(rule, g[j] + gb, u[j] + ub, limit, alpha);
+            }
+            float_gemv(format, down[e], act, hidden, inter, h2);
+            for (size_t i = 0; i < hidden; i++) {
+                const float v = down_bias ? h2[i] + down_bias[e * hidden + i] : h2[i];
+                o[i] += w * v;
+            }
+        }
+    }
+    free(xp); free(g); free(u); free(act); free(h2);
+    return 0;
+}
+
 /* cpu_moe_forward's integer expert path with the routing given — larql-compute/src/cpu/ops/moe/forward.rs:160-330 and
  * run_single_expert_kq_q8k_into, cpu/ops/moe/expert/q4k.rs:232-351.  Per token the expert input is zero-padded to the
  * gate/up matrices' stored row width `cols` (forward.rs:176-184) and quantised to Q8_K once for all its experts; per
@@ -1379,6 +1422,9 @@ float lq_moe_combine(int rule, float g, float u, float limit, float alpha) {
 int lq_moe_block_kq(const float *x, size_t tokens, size_t hidden, size_t cols, size_t inter, size_t n_experts, size_t top_k,
                     const uint64_t *experts, const float *weights, const uint8_t *const *gate_up, const uint8_t *const *down,
                     int format, const float *gate_up_bias, const float *down_bias, int rule, float limit, float alpha, float *out) {
+    if (format == 16 || format == 17 || format == 32)
+        return moe_block_float(x, tokens, hidden, cols, inter, n_experts, top_k, experts, weights, gate_up, down, format, gate_up_bias, down_bias,
+                               rule, limit, alpha, out);
     if ((format != 4 && format != 6) || cols % 256 != 0 || cols < hidden) return 1;
     const size_t blk = format == 6 ? 210 : 144;
     const size_t inter_padded = (inter + 255) / 256 * 256;

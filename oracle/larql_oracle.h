@@ -137,7 +137,8 @@ float lq_gelu_tanh(float x);
 float lq_moe_combine(int rule, float g, float u, float limit, float alpha);
 /* cpu_moe_forward's integer expert path over a Q4_K (format 4) or Q6_K (format 6) bank of per-expert slices, routing
  * given (cpu/ops/moe/forward.rs:160-330, expert/q4k.rs:232-351).  gate_up[e]: [2*inter, cols] rows, gate half first;
- * down[e]: [hidden, ceil(inter/256)*256]; cols >= hidden is the stored (block-padded) row width. */
+ * down[e]: [hidden, ceil(inter/256)*256]; cols >= hidden is the stored (block-padded) row width.  Formats 16 (BF16),
+ * 17 (F16) and 32 (F32) take cpu_moe_forward's f32 arm instead (forward.rs:246-290): f32 activations, down [hidden, inter]. */
 int lq_moe_block_kq(const float *x, size_t tokens, size_t hidden, size_t cols, size_t inter, size_t n_experts, size_t top_k,
                     const uint64_t *experts, const float *weights, const uint8_t *const *gate_up, const uint8_t *const *down,
                     int format, const float *gate_up_bias, const float *down_bias, int rule, float limit, float alpha, float *out);

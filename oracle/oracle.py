@@ -599,7 +599,8 @@ def moe_combine(rule: int, g: float, u: float, limit: float = 7.0, alpha: float 
 def moe_block_kq(x, experts, weights, gate_up, down, hidden: int, cols: int, inter: int, fmt: int = 4, gate_up_bias=None,
                  down_bias=None, rule: int = GATE_GELU_TANH, limit: float = 7.0, alpha: float = 1.702) -> np.ndarray:
     """cpu_moe_forward's integer expert path over per-expert k-quant slices (fmt 4 = Q4_K, 6 = Q6_K), routing given.
-    gate_up[e]: bytes of [2*inter, cols] rows (gate half first); down[e]: [hidden, ceil(inter/256)*256] rows."""
+    gate_up[e]: bytes of [2*inter, cols] rows (gate half first); down[e]: [hidden, ceil(inter/256)*256] rows.
+    fmt 16 / 17 / 32 = a BF16 / F16 / F32 bank on the f32 arm: f32 activations, down [hidden, inter]."""
     x = _f32(x)
     tokens = x.shape[0]
     ex = np.ascontiguousarray(experts, dtype=np.uint64).reshape(tokens, -1)
@@ -608,10 +609,15 @@ def moe_block_kq(x, experts, weights, gate_up, down, hidden: int, cols: int, int
     gu = [_u8(a).ravel() for a in gate_up]
     dn = [_u8(a).ravel() for a in down]
     n_experts = len(gu)
-    blk = 210 if fmt == 6 else 144
-    ip = (inter + 255) // 256 * 256
+    if fmt in (16, 17, 32):                       # float banks: BF16 / F16 / F32, rows unpadded
+        el = 4 if fmt == 32 else 2
+        need_gu, need_dn = 2 * inter * cols * el, hidden * inter * el
+    else:
+        blk = 210 if fmt == 6 else 144
+        ip = (inter + 255) // 256 * 256
+        need_gu, need_dn = 2 * inter * (cols // 256) * blk, hidden * (ip // 256) * blk
     for a, b in zip(gu, dn):
-        if a.size < 2 * inter * (cols // 256) * blk or b.size < hidden * (ip // 256) * blk:
+        if a.size < need_gu or b.size < need_dn:
             raise ValueError("an expert's slices are shorter than the geometry")
     gup = (C.c_void_p * n_experts)(*[a.ctypes.data for a in gu])
     dnp = (C.c_void_p * n_experts)(*[a.ctypes.data for a in dn])

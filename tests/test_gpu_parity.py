@@ -1327,6 +1327,89 @@ def test_moe_layer_over_a_k_quant_bank_matches_the_integer_expert_path(be, fmt, 
     be.moe_layer_destroy(layer)
 
 
+def _float_bytes(a, kind):
+    a = np.ascontiguousarray(a, F)
+    if kind == "bf16":
+        return (a.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8).reshape(-1)
+    if kind == "f16":
+        return a.astype(np.float16).view(np.uint8).reshape(-1)
+    return a.view(np.uint8).reshape(-1)
+
+
+@pytest.mark.parametrize("T,E,k,hidden,inter,kind,rule,biases", [
+    (1, 6, 2, 256, 704, "bf16", 1, False),       # the legacy BF16 monolith's arm: GeluTanh, no biases
+    (5, 8, 4, 512, 320, "bf16", 0, True),
+    (3, 4, 2, 128, 96, "f16", 2, True),
+    (2, 3, 1, 64, 48, "f32", 1, True),
+])
+def test_moe_layer_over_a_float_bank_matches_the_f32_arm(be, fmt, T, E, k, hidden, inter, kind, rule, biases):
+    """MoeLayerWeights with expert_data_format BF16 / F16 / F32: cpu_moe_forward's f32 arm (forward.rs:246-290) — f32
+    activations throughout, the dense matvec kernels on the expert picked at run time, down rows unpadded."""
+    rng = np.random.default_rng(900 + T + E + inter)
+    f = {"bf16": 16, "f16": 17, "f32": 32}[kind]
+    dfmt = {"bf16": fmt.FMT_BF16, "f16": fmt.FMT_F16, "f32": fmt.FMT_F32}[kind]
+    gate_up = [_float_bytes(rng.standard_normal((2 * inter, hidden)) * 0.05, kind) for _ in range(E)]
+    down = [_float_bytes(rng.standard_normal((hidden, inter)) * 0.05, kind) for _ in range(E)]
+    router_w = (rng.standard_normal((E, hidden)) * 0.05).astype(F)
+    gub = (rng.standard_normal((E, 2 * inter)) * 0.5).astype(F) if biases else None
+    db = (rng.standard_normal((E, hidden)) * 0.5).astype(F) if biases else None
+    x = rng.standard_normal((T, hidden)).astype(F)
+    layer = be.moe_layer_create(gate_up, down, None, None, router_w, k, hidden, inter, fmt.MOE_ROWS_CONTIGUOUS_HALVES, gate_up_bias=gub,
+                                down_bias=db, expert_scales=fmt.MOE_SCALES_INLINE, expert_data_format=dfmt, gate_rule=rule)
+    assert layer, be.last_error()
+    got = be.moe_layer_forward(layer, x, x, k)
+    assert got is not None, be.last_error()
+    out, experts, weights = got
+    for t in range(T):
+        want = O.moe_route_from_router_input(x[t], router_w, None, k, renormalize=True)
+        assert [int(e) for e in experts[t]] == [e for e, _ in want], t
+    want_out = O.moe_block_kq(x, experts, weights, gate_up, down, hidden, hidden, inter, f, gub, db, rule)
+    assert rel_l2(out, want_out) < 1e-5
+    dx, do, de, dw_ = be.to_device(x), be.malloc(T * hidden * 4), be.malloc(T * k * 4), be.malloc(T * k * 4)
+    assert be.dev_moe_layer_forward(layer, dx, dx, T, do, de, dw_)
+    be.synchronize()
+    assert np.array_equal(be.d2h(do, (T, hidden), F).view(np.uint32), out.view(np.uint32))
+    be.moe_layer_destroy(layer)
+
+
+def test_moe_layer_float_bank_reproduces_the_reference_plumbing_tests(be, fmt):
+    """The hand-derived expectations of the reference's own tests for this path (cpu/ops/moe/expert/tests/bias.rs:52-146:
+    BF16 identity expert, h = [1, 2], asymmetric interleaved biases, tolerance 1e-4), the 2 x 2 identity sitting in a
+    16 x 16 frame of zeros (the dense kernel's rows are multiples of 16 elements): a swapped or dropped bias, the
+    gate / up halves exchanged or another combine rule change these numbers."""
+    H = I = 16
+    gate_up = np.zeros((2 * I, H), F)
+    for row in range(2 * I):
+        gate_up[row, row % I] = 1.0
+    down = np.eye(H, I, dtype=F)
+    gu, dn = _float_bytes(gate_up, "bf16"), _float_bytes(down, "bf16")
+    rw = np.zeros((1, H), F)
+    silu = lambda v: v / (1.0 + np.exp(-v))
+
+    def run(h, rule, gub=None, db=None):
+        layer = be.moe_layer_create([gu], [dn], None, None, rw, 1, H, I, fmt.MOE_ROWS_CONTIGUOUS_HALVES, gate_up_bias=gub, down_bias=db,
+                                    expert_scales=fmt.MOE_SCALES_INLINE, expert_data_format=fmt.FMT_BF16, gate_rule=rule)
+        assert layer, be.last_error()
+        x = np.zeros((1, H), F)
+        x[0, :2] = h
+        out = be.moe_layer_forward(layer, x, x, 1)
+        be.moe_layer_destroy(layer)
+        assert out is not None and out[2][0, 0] == 1.0
+        return out[0][0]
+
+    fused = np.zeros((1, 2 * I), F)
+    fused[0, :4] = [0.5, 3.0, -0.25, 7.0]                        # gate biases [0.5, -0.25], up biases [3, 7], interleaved
+    got = run([1.0, 2.0], fmt.MOE_GATE_SILU, gub=fused)
+    assert np.allclose(got[:2], [silu(1.5) * 4.0, silu(1.75) * 9.0], atol=1e-4) and not got[2:].any()
+    dbias = np.zeros((1, H), F)
+    dbias[0, :2] = [10.0, -20.0]
+    got = run([1.0, 2.0], fmt.MOE_GATE_SILU, db=dbias)
+    assert np.allclose(got[:2], [silu(1.0) * 1.0 + 10.0, silu(2.0) * 2.0 - 20.0], atol=1e-4)
+    got = run([2.0, 0.0], fmt.MOE_GATE_CLAMPED_GLU)
+    assert abs(got[0] - 3.0 * (2.0 / (1.0 + np.exp(-2.0 * 1.702)))) < 1e-4 and got[1] == 0.0
+    assert abs(got[0] - run([2.0, 0.0], fmt.MOE_GATE_SILU)[0]) > 0.5
+
+
 def test_moe_layer_k_quant_refusals(be, fmt):
     """A k-quant bank the CPU tier itself would refuse, or that has no kernel here, answers None: Interleaved rows
     (forward.rs:69-75), Paired scales, slices shorter than the geometry, rows beyond 10240 elements."""
