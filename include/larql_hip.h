@@ -474,8 +474,10 @@ int larql_hip_dev_moe_mxfp4_routed(larql_hip_ctx *ctx, const larql_hip_mxfp4_exp
  * asserts the same, forward.rs:69-75); k-quant rows longer than 10240 elements and other formats LARQL_UNSUPPORTED.
  * num_experts <= 256, top_k <= 8. */
 enum { LARQL_MOE_SCALES_INLINE = 0, LARQL_MOE_SCALES_PAIRED = 1 };
-/* MoeGateRule (moe.rs:40-118): ClampedGlu{limit, alpha}, Gated(gelu_tanh), Gated(silu). */
-enum { LARQL_MOE_GATE_CLAMPED_GLU = 0, LARQL_MOE_GATE_GELU_TANH = 1, LARQL_MOE_GATE_SILU = 2 };
+/* MoeGateRule (moe.rs:16-118): ClampedGlu{limit, alpha}, Gated(gelu_tanh), Gated(silu), SituGlu{beta, linear_beta}
+ * (glu_limit = beta, glu_alpha = linear_beta, 0 for None), ClampedGated{limit, gelu_tanh | silu} (glu_limit = limit). */
+enum { LARQL_MOE_GATE_CLAMPED_GLU = 0, LARQL_MOE_GATE_GELU_TANH = 1, LARQL_MOE_GATE_SILU = 2, LARQL_MOE_GATE_SITU_GLU = 3,
+       LARQL_MOE_GATE_CLAMPED_GELU_TANH = 4, LARQL_MOE_GATE_CLAMPED_SILU = 5 };
 enum { LARQL_MOE_ROWS_CONTIGUOUS_HALVES = 0, LARQL_MOE_ROWS_INTERLEAVED = 1 };
 typedef struct {
     size_t num_experts, top_k, hidden, intermediate_size;

@@ -60,6 +60,9 @@ pub const MOE_ROWS_INTERLEAVED: c_int = 1;
 pub const MOE_GATE_CLAMPED_GLU: c_int = 0;
 pub const MOE_GATE_GELU_TANH: c_int = 1;
 pub const MOE_GATE_SILU: c_int = 2;
+pub const MOE_GATE_SITU_GLU: c_int = 3;
+pub const MOE_GATE_CLAMPED_GELU_TANH: c_int = 4;
+pub const MOE_GATE_CLAMPED_SILU: c_int = 5;
 
 pub const OK: c_int = 0;
 

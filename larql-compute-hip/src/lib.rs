@@ -20,7 +20,7 @@ use std::os::raw::c_int;
 use std::ptr;
 
 use larql_compute::{
-    Capability, ComputeBackend, CpuBackend, DecodeBackend, MatMul, MoeExpertScalePolicy, MoeExpertScales, MoeFusedRowLayout,
+    Activation, Capability, ComputeBackend, CpuBackend, DecodeBackend, MatMul, MoeExpertScalePolicy, MoeExpertScales, MoeFusedRowLayout,
     MoeGateRule, MoeLayerWeights, MoeTopKWeightPolicy, QuantFormat, QuantMatVec, SubmissionClock,
 };
 use ndarray::{Array2, ArrayView2};
@@ -215,18 +215,26 @@ impl HipBackend {
     /// A MoE layer made resident from `MoeLayerWeights` (crates/larql-compute/src/pipeline/moe.rs:469-541): the
     /// per-expert slices and their paired exponent streams go up expert by expert, wherever their mmap ranges lie.
     /// Served: an MXFP4 bank with `Paired` scales under `ClampedGlu` (a native GPT-OSS bank), and a Q4_K / Q6_K bank with
-    /// `Inline` scales and `ContiguousHalves` rows under `ClampedGlu` or `Gated` (the per-layer k-quant files of Gemma 4
+    /// `Inline` scales and `ContiguousHalves` rows under any `MoeGateRule` (the per-layer k-quant files of Gemma 4
     /// 26B-A4B: `cpu_moe_forward`'s integer path, crates/larql-compute/src/cpu/ops/moe/forward.rs:160-330), and a BF16 /
     /// F16 / F32 bank on that function's f32 arm (forward.rs:246-290).  `None` where
     /// this backend has no kernel for the layer (other formats or rules, more than 256 experts, top-k above 8) — the
     /// caller keeps `cpu_moe_forward`.
     pub fn moe_layer<'a>(&'a self, moe: &MoeLayerWeights<'_>, hidden: usize) -> Option<HipMoeLayer<'a>> {
-        // the rules this backend has kernels for: ClampedGlu on any bank, Gated(gelu_tanh | silu) on a k-quant bank
+        // ClampedGlu on any bank, every rule on a k-quant or float bank.  `Activation::ReLU` has no gate/up kernel on the
+        // CPU paths either (it panics there: pipeline/enums.rs:79-88); here it is `None`.
+        let gelu = |a: Activation| match a {
+            Activation::GeluTanh | Activation::GeluExact => Some(true),
+            Activation::Silu => Some(false),
+            _ => None,
+        };
         let (gate_rule, limit, alpha) = match moe.gate_rule {
             MoeGateRule::ClampedGlu { limit, alpha } => (ffi::MOE_GATE_CLAMPED_GLU, limit, alpha),
-            MoeGateRule::Gated(activation) if activation.gate_up_is_gelu_tanh() => (ffi::MOE_GATE_GELU_TANH, 0.0, 0.0),
-            MoeGateRule::Gated(_) => (ffi::MOE_GATE_SILU, 0.0, 0.0),
-            _ => return None,
+            MoeGateRule::Gated(a) => (if gelu(a)? { ffi::MOE_GATE_GELU_TANH } else { ffi::MOE_GATE_SILU }, 0.0, 0.0),
+            MoeGateRule::SituGlu { beta, linear_beta } => (ffi::MOE_GATE_SITU_GLU, beta, linear_beta.unwrap_or(0.0)),
+            MoeGateRule::ClampedGated { limit, activation } => {
+                (if gelu(activation)? { ffi::MOE_GATE_CLAMPED_GELU_TANH } else { ffi::MOE_GATE_CLAMPED_SILU }, limit, 0.0)
+            }
         };
         let (sg, sd): (Vec<&[u8]>, Vec<&[u8]>) = match &moe.expert_scales {
             MoeExpertScales::Paired { gate_up, down } => (gate_up.clone(), down.clone()),

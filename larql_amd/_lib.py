@@ -34,7 +34,7 @@ class Mxfp4Experts(C.Structure):
 
 
 MOE_SCALES_INLINE, MOE_SCALES_PAIRED = 0, 1
-MOE_GATE_CLAMPED_GLU, MOE_GATE_GELU_TANH, MOE_GATE_SILU = 0, 1, 2
+MOE_GATE_CLAMPED_GLU, MOE_GATE_GELU_TANH, MOE_GATE_SILU, MOE_GATE_SITU_GLU, MOE_GATE_CLAMPED_GELU_TANH, MOE_GATE_CLAMPED_SILU = 0, 1, 2, 3, 4, 5
 MOE_ROWS_CONTIGUOUS_HALVES, MOE_ROWS_INTERLEAVED = 0, 1
 
 

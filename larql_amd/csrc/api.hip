@@ -2054,8 +2054,10 @@ static int moe_layer_create_kq(larql_hip_ctx *c, const larql_hip_moe_layer_weigh
         return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: a k-quant or float bank has no scale stream of its own (MoeExpertScales::Inline)");
     if (w->fused_row_layout != LARQL_MOE_ROWS_CONTIGUOUS_HALVES)
         return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: a k-quant or float bank is read as contiguous gate / up halves, as cpu_moe_forward reads it");
-    if (w->gate_rule != LARQL_MOE_GATE_CLAMPED_GLU && w->gate_rule != LARQL_MOE_GATE_GELU_TANH && w->gate_rule != LARQL_MOE_GATE_SILU)
+    if (w->gate_rule < LARQL_MOE_GATE_CLAMPED_GLU || w->gate_rule > LARQL_MOE_GATE_CLAMPED_SILU)
         return fail(c, LARQL_UNSUPPORTED, "moe_layer: unknown gate rule");
+    if (w->gate_rule == LARQL_MOE_GATE_SITU_GLU && !(w->glu_limit > 0.0f))
+        return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: SituGlu needs a positive beta");
     if (E == 0 || w->top_k == 0 || hidden == 0 || inter == 0) return fail(c, LARQL_REFUSED_SHAPE, "moe_layer: empty layer");
     if (E > kRouterMaxExperts || std::min(w->top_k, E) > 8) return fail(c, LARQL_UNSUPPORTED, "moe_layer: at most 256 experts and top-8 on this backend");
     if (hidden > (1u << 24) || inter > (1u << 24)) return fail(c, LARQL_UNSUPPORTED, "moe_layer: dimensions beyond this backend");

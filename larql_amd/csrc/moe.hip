@@ -141,8 +141,15 @@ __device__ __forceinline__ float moe_combine(int rule, float g, float u, float l
         return 0.5f * g * (1.0f + tanhf(c * (g + 0.044715f * g * g * g))) * u;
     }
     if (rule == 2) return g / (1.0f + expf(-g)) * u;
+    if (rule == 3) {  // SituGlu { beta = limit, linear_beta = alpha, 0 for None }
+        const float situ_a = limit * tanhf(g / limit) * (1.0f / (1.0f + expf(-g)));
+        const float uc = alpha != 0.0f ? alpha * tanhf(u / alpha) : u;
+        return situ_a * uc;
+    }
     const float gv = fminf(g, limit);
     const float uv = u < -limit ? -limit : (u > limit ? limit : u);
+    if (rule == 4) return 0.5f * gv * (1.0f + tanhf(0.7978846f * (gv + 0.044715f * gv * gv * gv))) * uv;  // ClampedGated { limit, gelu_tanh }
+    if (rule == 5) return gv / (1.0f + expf(-gv)) * uv;                                                    // ClampedGated { limit, silu }
     return (uv + 1.0f) * (gv * (1.0f / (1.0f + expf(-(gv * alpha)))));
 }
 

@@ -51,10 +51,15 @@ struct MoeExpertScales {  // Inline | Paired { gate_up, down } (moe.rs:214-238)
     bool paired = false;
     std::vector<Slice<uint8_t>> gate_up, down;
 };
-struct MoeGateRule {  // moe.rs:40-118; the rules this backend has kernels for, `Other` standing for the rest
-    enum Kind { ClampedGlu = LARQL_MOE_GATE_CLAMPED_GLU, GatedGeluTanh = LARQL_MOE_GATE_GELU_TANH, GatedSilu = LARQL_MOE_GATE_SILU, Other = -1 };
+struct MoeGateRule {  // moe.rs:16-118; `Other` stands for a rule without a kernel here (Gated(ReLU))
+    enum Kind {
+        ClampedGlu = LARQL_MOE_GATE_CLAMPED_GLU, GatedGeluTanh = LARQL_MOE_GATE_GELU_TANH, GatedSilu = LARQL_MOE_GATE_SILU,
+        SituGlu = LARQL_MOE_GATE_SITU_GLU, ClampedGatedGeluTanh = LARQL_MOE_GATE_CLAMPED_GELU_TANH, ClampedGatedSilu = LARQL_MOE_GATE_CLAMPED_SILU,
+        Other = -1
+    };
     Kind kind = ClampedGlu;
-    float limit = 7.0f, alpha = 1.702f;  // ClampedGlu { limit, alpha }
+    // ClampedGlu { limit, alpha }; SituGlu { beta = limit, linear_beta = alpha (0: None) }; ClampedGated { limit }
+    float limit = 7.0f, alpha = 1.702f;
 };
 struct MoeLayerWeights {
     std::vector<Slice<uint8_t>> experts_gate_up, experts_down;

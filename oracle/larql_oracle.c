@@ -1360,10 +1360,21 @@ float lq_gelu_tanh(float x) {
     return 0.5f * x * (1.0f + tanhf(c * (x + 0.044715f * x * x * x)));
 }
 /* MoeGateRule::combine — larql-compute/src/pipeline/moe.rs:73-118, the rules a k-quant bank is served under:
- * 0 ClampedGlu{limit, alpha}, 1 Gated(gelu_tanh), 2 Gated(silu).  Inputs already carry their biases. */
+ * 0 ClampedGlu{limit, alpha}, 1 Gated(gelu_tanh), 2 Gated(silu), 3 SituGlu{beta, linear_beta}, 4 / 5 ClampedGated{limit,
+ * gelu_tanh / silu}.  Inputs already carry their biases. */
 float lq_moe_combine(int rule, float g, float u, float limit, float alpha) {
     if (rule == LQ_GATE_GELU_TANH) return lq_gelu_tanh(g) * u;
     if (rule == LQ_GATE_SILU) return lq_silu(g) * u;
+    if (rule == LQ_GATE_SITU_GLU) {  /* SituGlu{beta = limit, linear_beta = alpha, 0 for None}: moe.rs:100-107 */
+        const float situ_a = limit * tanhf(g / limit) * (1.0f / (1.0f + expf(-g)));
+        if (alpha != 0.0f) u = alpha * tanhf(u / alpha);
+        return situ_a * u;
+    }
+    if (rule == LQ_GATE_CLAMPED_GELU_TANH || rule == LQ_GATE_CLAMPED_SILU) {  /* ClampedGated{limit, activation}: moe.rs:108-117 */
+        g = fminf(g, limit);
+        u = clampf(u, -limit, limit);
+        return (rule == LQ_GATE_CLAMPED_GELU_TANH ? lq_gelu_tanh(g) : lq_silu(g)) * u;
+    }
     return lq_clamped_glu(g, u, limit, alpha);
 }
 

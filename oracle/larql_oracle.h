@@ -132,6 +132,9 @@ int lq_moe_block_mxfp4(const float *x, size_t tokens, size_t hidden, size_t inte
 #define LQ_GATE_CLAMPED_GLU 0
 #define LQ_GATE_GELU_TANH 1
 #define LQ_GATE_SILU 2
+#define LQ_GATE_SITU_GLU 3          /* limit = beta, alpha = linear_beta (0: none) */
+#define LQ_GATE_CLAMPED_GELU_TANH 4  /* ClampedGated{limit, gelu_tanh} */
+#define LQ_GATE_CLAMPED_SILU 5       /* ClampedGated{limit, silu} */
 float lq_silu(float x);
 float lq_gelu_tanh(float x);
 float lq_moe_combine(int rule, float g, float u, float limit, float alpha);

@@ -581,7 +581,7 @@ def moe_block_mxfp4(x, experts, weights, gate, up, down, n_experts: int, hidden:
     return out
 
 
-GATE_CLAMPED_GLU, GATE_GELU_TANH, GATE_SILU = 0, 1, 2
+GATE_CLAMPED_GLU, GATE_GELU_TANH, GATE_SILU, GATE_SITU_GLU, GATE_CLAMPED_GELU_TANH, GATE_CLAMPED_SILU = 0, 1, 2, 3, 4, 5
 
 
 def silu(x: float) -> float:

@@ -15,6 +15,9 @@ test-data file) and writes small JSON fixtures beside this script:
                             inputs: name, 32 input bit patterns, 34-byte block.
                             Source tables:
                             crates/larql-models/src/quant/ggml/tests/q8_0_ggml_golden.rs
+  situ_glu_golden.json      SiTU-GLU (Kimi-K3's SituAndMul.forward run in PyTorch): per arm beta, linear_beta and 88
+                            (gate, up, out) points.  Source (the arms' data, without the measured controls):
+                            crates/larql-compute/src/ffn/expert_weight/tests/situ_oracle.json
 
 Nothing of the reference is imported or executed.
 """
@@ -42,7 +45,11 @@ def main(ref: str) -> None:
     header = re.search(r"// Expected bytes: (.*)", rs)
     with open(os.path.join(HERE, "q8_0_ggml_golden.json"), "w") as f:
         json.dump({"source": header.group(1) if header else "", "cases": cases}, f, indent=0)
-    print(f"wrote {len(cases)} Q8_0 golden blocks and ggml_kquant_golden.json")
+    situ = json.load(open(os.path.join(ref, "crates/larql-compute/src/ffn/expert_weight/tests/situ_oracle.json")))
+    arms = {name: {k: arm[k] for k in ("beta", "linear_beta", "gate", "up", "out")} for name, arm in situ["arms"].items()}
+    with open(os.path.join(HERE, "situ_glu_golden.json"), "w") as f:
+        json.dump({"source": situ["_source"], "precision": situ["_precision"], "arms": arms}, f, indent=0)
+    print(f"wrote {len(cases)} Q8_0 golden blocks, ggml_kquant_golden.json and {len(arms)} SiTU-GLU arms")
 
 
 if __name__ == "__main__":

@@ -4,6 +4,9 @@ inputs.  Bars: quantised bytes bit-exact; matvec outputs within 1e-3 relative
 L2 (fp32 accumulate; measured ~1e-6, asserted at 2e-5 so a wrong scale or a
 dropped term cannot hide); top-K index sets identical except at score ties
 within 1e-5."""
+import json
+import os
+
 import numpy as np
 import pytest
 
@@ -1408,6 +1411,48 @@ def test_moe_layer_float_bank_reproduces_the_reference_plumbing_tests(be, fmt):
     got = run([2.0, 0.0], fmt.MOE_GATE_CLAMPED_GLU)
     assert abs(got[0] - 3.0 * (2.0 / (1.0 + np.exp(-2.0 * 1.702)))) < 1e-4 and got[1] == 0.0
     assert abs(got[0] - run([2.0, 0.0], fmt.MOE_GATE_SILU)[0]) > 0.5
+
+
+def test_moe_layer_gate_rules_on_reference_held_points(be, fmt):
+    """Every MoeGateRule the layer serves, through the device: SituGlu on the points the reference holds for it
+    (ffn/expert_weight/tests/situ_oracle.json, both arms, its tolerance 1e-5), ClampedGlu on the PyTorch values of
+    ffn/expert_weight/gate.rs:108-117, ClampedGated on that file's points.  An F32 bank with zero gate / up weights and
+    an identity down matrix: the fused bias row carries (gate, up) to the combine rule exactly, the output is the rule's
+    value per element."""
+    arms = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "situ_glu_golden.json")))["arms"]
+    H = I = 96
+    gu = np.zeros((2 * I, H), F).view(np.uint8).reshape(-1)
+    dn = np.eye(H, I, dtype=F).view(np.uint8).reshape(-1)
+    rw = np.zeros((1, H), F)
+    x = np.zeros((1, H), F)
+
+    def run(rule, gate, up, limit, alpha):
+        fused = np.zeros((1, 2 * I), F)
+        fused[0, 0:2 * len(gate):2] = gate
+        fused[0, 1:2 * len(up):2] = up
+        layer = be.moe_layer_create([gu], [dn], None, None, rw, 1, H, I, fmt.MOE_ROWS_CONTIGUOUS_HALVES, gate_up_bias=fused,
+                                    expert_scales=fmt.MOE_SCALES_INLINE, expert_data_format=fmt.FMT_F32, gate_rule=rule, limit=limit, alpha=alpha)
+        assert layer, be.last_error()
+        out = be.moe_layer_forward(layer, x, x, 1)
+        be.moe_layer_destroy(layer)
+        assert out is not None
+        return out[0][0][:len(gate)]
+
+    for name, arm in arms.items():
+        got = run(fmt.MOE_GATE_SITU_GLU, arm["gate"], arm["up"], arm["beta"], arm["linear_beta"] or 0.0)
+        want = np.array(arm["out"], F)
+        assert np.all(np.abs(got - want) <= 1e-5 * np.maximum(1.0, np.abs(want))), name
+    got = run(fmt.MOE_GATE_CLAMPED_GLU, [-2.0, 0.0, 1.5, 9.0], [0.5, -1.0, 2.0, -9.0], 7.0, 1.702)
+    assert np.all(np.abs(got - np.array([-0.0965121, 0.0, 4.174987, -41.999718], F)) < 1e-5)
+    pts = [(0.5, 0.25), (-0.5, 0.25), (25.0, 0.5), (-25.0, 0.5), (0.5, 25.0), (0.5, -25.0), (-40.0, 1.0), (1.0, -40.0)]
+    for rule, orule in ((fmt.MOE_GATE_CLAMPED_SILU, O.GATE_CLAMPED_SILU), (fmt.MOE_GATE_CLAMPED_GELU_TANH, O.GATE_CLAMPED_GELU_TANH),
+                        (fmt.MOE_GATE_SILU, O.GATE_SILU), (fmt.MOE_GATE_GELU_TANH, O.GATE_GELU_TANH)):
+        got = run(rule, [g for g, _ in pts], [u for _, u in pts], 10.0, 0.0)
+        want = np.array([O.moe_combine(orule, g, u, 10.0, 0.0) for g, u in pts], F)
+        assert np.all(np.abs(got - want) <= 2e-6 * np.maximum(1.0, np.abs(want))), rule
+    # SituGlu without a positive beta has no meaning: refused
+    assert be.moe_layer_create([gu], [dn], None, None, rw, 1, H, I, fmt.MOE_ROWS_CONTIGUOUS_HALVES, expert_scales=fmt.MOE_SCALES_INLINE,
+                               expert_data_format=fmt.FMT_F32, gate_rule=fmt.MOE_GATE_SITU_GLU, limit=0.0) is None
 
 
 def test_moe_layer_k_quant_refusals(be, fmt):
