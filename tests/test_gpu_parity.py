@@ -1455,6 +1455,28 @@ def test_moe_layer_gate_rules_on_reference_held_points(be, fmt):
                                expert_data_format=fmt.FMT_F32, gate_rule=fmt.MOE_GATE_SITU_GLU, limit=0.0) is None
 
 
+def test_moe_layer_reproduces_the_reference_moe_fixture(be, fmt):
+    """EXPECTED[48] of larql-compute/tests/test_moe_reference_parity.rs:72-85 — values an independent transcription of
+    the GPT-OSS reference model produced — through the device entry point: the fixture's f32 bank (fused rows
+    de-interleaved into gate / up halves, what a canonicalising extraction stores), its router weights and bias, the
+    interleaved bias rows, both expert biases, ClampedGlu, top-2 of 4 experts over 3 tokens; the inputs regenerated by
+    the fixture's own LCG.  The reference's tolerance: 1e-5."""
+    import test_oracle_moe as ref
+    x, router_w, router_b, fused, fused_bias, down, down_bias = ref.draw()
+    E, H, I = ref.EXPERTS, ref.HIDDEN, ref.INTER
+    gate_up = [np.concatenate([fused[e][0::2], fused[e][1::2]]).astype(F).view(np.uint8).reshape(-1) for e in range(E)]
+    dn = [np.ascontiguousarray(down[e], F).view(np.uint8).reshape(-1) for e in range(E)]
+    layer = be.moe_layer_create(gate_up, dn, None, None, router_w, ref.TOP_K, H, I, fmt.MOE_ROWS_CONTIGUOUS_HALVES, router_bias=router_b,
+                                gate_up_bias=fused_bias, down_bias=down_bias, expert_scales=fmt.MOE_SCALES_INLINE,
+                                expert_data_format=fmt.FMT_F32, gate_rule=fmt.MOE_GATE_CLAMPED_GLU, limit=7.0, alpha=1.702)
+    assert layer, be.last_error()
+    got = be.moe_layer_forward(layer, x, x, ref.TOP_K)
+    be.moe_layer_destroy(layer)
+    assert got is not None
+    assert float(np.max(np.abs(got[0] - ref.EXPECTED))) < ref.TOLERANCE
+    assert set(map(int, got[1][2])) != set(map(int, got[1][0]))        # the fixture's own remark: token 2 routes elsewhere
+
+
 def test_moe_layer_k_quant_refusals(be, fmt):
     """A k-quant bank the CPU tier itself would refuse, or that has no kernel here, answers None: Interleaved rows
     (forward.rs:69-75), Paired scales, slices shorter than the geometry, rows beyond 10240 elements."""
