@@ -470,7 +470,7 @@ int larql_hip_dev_moe_mxfp4_routed(larql_hip_ctx *ctx, const larql_hip_mxfp4_exp
  * Q8_K once per token, the gated activation once per expert, and every matvec is the integer Q4_K x Q8_K (Q6_K x Q8_K)
  * kernel, as on the CPU.  A BF16 (the legacy monolith), F16 or F32 bank takes cpu_moe_forward's f32 arm (forward.rs:246-290):
  * f32 activations, the dense matvec kernels, experts_down[e] [hidden, inter] unpadded; its rows are multiples of 16
- * elements, at most 8192, and as wide as hidden.  An Interleaved k-quant or float bank is LARQL_REFUSED_SHAPE (the CPU tier
+ * elements, at most 8192 (stored wider than hidden: the expert input goes in zero-padded, as on the CPU).  An Interleaved k-quant or float bank is LARQL_REFUSED_SHAPE (the CPU tier
  * asserts the same, forward.rs:69-75); k-quant rows longer than 10240 elements and other formats LARQL_UNSUPPORTED.
  * num_experts <= 256, top_k <= 8. */
 enum { LARQL_MOE_SCALES_INLINE = 0, LARQL_MOE_SCALES_PAIRED = 1 };

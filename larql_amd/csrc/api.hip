@@ -2071,7 +2071,6 @@ static int moe_layer_create_kq(larql_hip_ctx *c, const larql_hip_moe_layer_weigh
     // MoeWeightLayout::quant_block_padded_down (moe.rs:184-200): a block format pads `inter` to whole blocks, a float format does not
     const size_t ip = dense ? inter : (inter + 255) / 256 * 256;
     if (dense) {
-        if (cols != hidden) return fail(c, LARQL_UNSUPPORTED, "moe_layer: float expert rows wider than hidden are not served");
         if (cols % 16 != 0 || inter % 16 != 0 || cols > 8192 || inter > 8192)
             return fail(c, LARQL_UNSUPPORTED, "moe_layer: float expert rows must be multiples of 16 elements, at most 8192");
     } else {
@@ -2261,14 +2260,17 @@ static int moe_layer_enqueue(larql_hip_ctx *c, larql_hip_moe_layer *L, const flo
         if (L->per_expert_scale) HIPCHECK(c, expert_scale_launch(c->stream, weights, experts, L->scale, (uint32_t)slots, (uint32_t)E));
         // (a float bank: the activations stay f32 — x itself, and one row of `inter` floats per slot)
         const bool dense = L->kq_dense;
-        const size_t xq_stride = dense ? hidden * sizeof(float) : (q8k_bytes(cols) + 255) & ~(size_t)255;
+        const bool pad_x = dense && cols != hidden;  // rows stored wider than hidden: x goes in zero-padded
+        const size_t xq_stride = dense ? (pad_x ? cols : hidden) * sizeof(float) : (q8k_bytes(cols) + 255) & ~(size_t)255;
         const size_t aq_stride = dense ? ((inter * sizeof(float) + 255) & ~(size_t)255) : (q8k_bytes(ip) + 255) & ~(size_t)255;
         const size_t f_bytes = ((2 * slots * inter + slots * hidden) * sizeof(float) + 255) & ~(size_t)255;
-        rc = ensure(c, L->ws, f_bytes + (dense ? 0 : tokens * xq_stride) + slots * aq_stride + 256); if (rc) return rc;
+        const size_t x_area = (dense && !pad_x) ? 0 : ((tokens * xq_stride + 255) & ~(size_t)255);
+        rc = ensure(c, L->ws, f_bytes + x_area + slots * aq_stride + 256); if (rc) return rc;
         float *g = (float *)L->ws.p, *u = g + slots * inter, *dd = u + slots * inter;
-        uint8_t *xq = dense ? (uint8_t *)const_cast<float *>(x) : (uint8_t *)L->ws.p + f_bytes;
-        uint8_t *aq = dense ? (uint8_t *)L->ws.p + f_bytes : xq + tokens * xq_stride;
+        uint8_t *xq = (dense && !pad_x) ? (uint8_t *)const_cast<float *>(x) : (uint8_t *)L->ws.p + f_bytes;
+        uint8_t *aq = (uint8_t *)L->ws.p + f_bytes + x_area;
         if (!dense) HIPCHECK(c, quantize_rows_to_q8k_launch(c->stream, x, hidden, (uint32_t)hidden, (uint32_t)cols, (uint32_t)tokens, xq, xq_stride));
+        else if (pad_x) HIPCHECK(c, pad_rows_f32_launch(c->stream, x, hidden, (uint32_t)hidden, (uint32_t)cols, (uint32_t)tokens, (float *)xq));
         jobs.clear();
         for (size_t s = 0; s < slots; s++) {
             GemvJob a = make_job(L->kq_kind, L->kq_gate, nullptr, xq + (s / k) * xq_stride, g + s * inter, inter, cols);

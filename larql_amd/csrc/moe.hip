@@ -134,6 +134,15 @@ __global__ void __launch_bounds__(256) quantize_rows_to_q8k_kernel(const float *
     q8k_store(dst + (size_t)blockIdx.y * dst_stride, cols, sb, lane, codes, scale, sum);
 }
 
+// Row `blockIdx.y` of src ([rows, src_cols] floats, src_stride apart) zero-padded to `cols` floats at dst + row * cols:
+// the expert input of a float bank whose rows are stored wider than hidden (forward.rs:176-184).
+__global__ void __launch_bounds__(256) pad_rows_f32_kernel(const float *__restrict__ src, size_t src_stride, uint32_t src_cols, uint32_t cols,
+                                                          float *__restrict__ dst) {
+    const uint32_t j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= cols) return;
+    dst[(size_t)blockIdx.y * cols + j] = j < src_cols ? src[(size_t)blockIdx.y * src_stride + j] : 0.0f;
+}
+
 // math::silu / math::gelu_tanh (cpu/ops/moe/math.rs:54-65) and MoeGateRule::combine (pipeline/moe.rs:73-118)
 __device__ __forceinline__ float moe_combine(int rule, float g, float u, float limit, float alpha) {
     if (rule == 1) {
@@ -494,6 +503,11 @@ hipError_t moe_kq_act_q8k_launch(hipStream_t s, const float *g, const float *u, 
     if (slots == 0 || inter_padded < 256) return hipSuccess;
     hipLaunchKernelGGL(moe_kq_act_q8k_kernel, dim3((inter_padded / 256 + 3) / 4, slots), dim3(256), 0, s, g, u, inter, inter_padded, experts, n_experts,
                        gub, rule, limit, alpha, dst, dst_stride);
+    return hipGetLastError();
+}
+hipError_t pad_rows_f32_launch(hipStream_t s, const float *src, size_t src_stride, uint32_t src_cols, uint32_t cols, uint32_t rows, float *dst) {
+    if (rows == 0 || cols == 0) return hipSuccess;
+    hipLaunchKernelGGL(pad_rows_f32_kernel, dim3((cols + 255) / 256, rows), dim3(256), 0, s, src, src_stride, src_cols, cols, dst);
     return hipGetLastError();
 }
 hipError_t moe_act_f32_launch(hipStream_t s, const float *g, const float *u, uint32_t inter, uint32_t slots, const uint32_t *experts, uint32_t n_experts,

@@ -1477,6 +1477,31 @@ def test_moe_layer_reproduces_the_reference_moe_fixture(be, fmt):
     assert set(map(int, got[1][2])) != set(map(int, got[1][0]))        # the fixture's own remark: token 2 routes elsewhere
 
 
+def test_moe_layer_properties_the_reference_asserts_for_cpu_moe_forward(be, fmt):
+    """cpu/ops/moe/forward/tests.rs: a bank whose rows are stored wider than hidden gives what the unpadded bank gives
+    (:535-560, the pad columns holding weights the zero-padded activation must cancel), and a zero per-expert scale
+    silences the selected expert (:169-197) — on a BF16 bank of ones, in a 16-wide frame."""
+    H, W, I = 16, 32, 16
+    ones = lambda n: (np.ones(n, F).view(np.uint32) >> 16).astype(np.uint16).view(np.uint8)
+    rw = np.ones((1, H), F)
+    h = np.ones((1, H), F)
+    kw = dict(expert_scales=fmt.MOE_SCALES_INLINE, expert_data_format=fmt.FMT_BF16, gate_rule=fmt.MOE_GATE_SILU)
+
+    def run(gate_up, **more):
+        layer = be.moe_layer_create([gate_up], [ones(H * I)], None, None, rw, 1, H, I, fmt.MOE_ROWS_CONTIGUOUS_HALVES, **dict(kw, **more))
+        assert layer, be.last_error()
+        out = be.moe_layer_forward(layer, h, h, 1)
+        be.moe_layer_destroy(layer)
+        assert out is not None
+        return out[0][0]
+
+    plain, padded = run(ones(2 * I * H)), run(ones(2 * I * W))
+    assert np.array_equal(plain.view(np.uint32), padded.view(np.uint32)) and plain[0] > 1.0
+    g = float(H)                                                                   # every gate and up row sums 16 ones
+    assert np.allclose(plain, I * (g / (1.0 + np.exp(-g))) * g, rtol=1e-6)
+    assert not run(ones(2 * I * H), per_expert_scale=np.zeros(1, F)).any()
+
+
 def test_moe_layer_k_quant_refusals(be, fmt):
     """A k-quant bank the CPU tier itself would refuse, or that has no kernel here, answers None: Interleaved rows
     (forward.rs:69-75), Paired scales, slices shorter than the geometry, rows beyond 10240 elements."""
