@@ -35,13 +35,22 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 // Clears a few words on the stream (a kernel, not hipMemsetAsync: memset nodes recorded into a captured graph have
 // given wrong results on replays).
-// out[i] = parts[0][i] + parts[1][i] + ... (left to right), the partial vectors `stride` floats apart
-__global__ void sum_partials_kernel(const float *__restrict__ parts, size_t stride, uint32_t n_parts, float *__restrict__ out, size_t n) {
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
+// out[i] = parts[0][i] + parts[1][i] + ... (left to right), the partial vectors `stride` floats apart; up to eight
+// such sums per launch (blockIdx.y says which)
+constexpr int kSumBatch = 8;
+struct SumPartialsArgs {
+    const float *parts[kSumBatch];
+    float *out[kSumBatch];
+    uint32_t stride[kSumBatch], n_parts[kSumBatch], n[kSumBatch];
+};
+__global__ void sum_partials_kernel(SumPartialsArgs a) {
+    const uint32_t q = blockIdx.y;
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= a.n[q]) return;
+    const float *parts = a.parts[q];
     float acc = parts[i];
-    for (uint32_t p = 1; p < n_parts; p++) acc += parts[(size_t)p * stride + i];
-    out[i] = acc;
+    for (uint32_t p = 1; p < a.n_parts[q]; p++) acc += parts[(size_t)p * a.stride[q] + i];
+    a.out[q][i] = acc;
 }
 
 __global__ void zero_words_kernel(uint32_t *p, uint32_t n) {
@@ -450,10 +459,22 @@ int enqueue_jobs(larql_hip_ctx *c, std::vector<GemvJob> &jobs_in) {
         if (rc) return rc;
         HIPCHECK(c, gemv_launch(c->stream, P.kind, P.L, P.threads, P.grid, P.lds));
     }
-    for (const SplitSum &sm : sums) {
-        const size_t rows_up = (sm.rows + 63) & ~(size_t)63;
-        hipLaunchKernelGGL(sum_partials_kernel, dim3((unsigned)((sm.rows + 255) / 256)), dim3(256), 0, c->stream,
-                           (const float *)c->parts.p + sm.parts_off, rows_up, sm.n_parts, sm.out, sm.rows);
+    for (size_t at = 0; at < sums.size(); at += kSumBatch) {
+        SumPartialsArgs a;
+        memset(&a, 0, sizeof a);
+        const size_t nb = std::min<size_t>(kSumBatch, sums.size() - at);
+        size_t longest = 0;
+        for (size_t q = 0; q < nb; q++) {
+            const SplitSum &sm = sums[at + q];
+            if (sm.rows > 0xFFFFFFFFull) return fail(c, LARQL_UNSUPPORTED, "matvec: too many rows");
+            a.parts[q] = (const float *)c->parts.p + sm.parts_off;
+            a.out[q] = sm.out;
+            a.stride[q] = (uint32_t)((sm.rows + 63) & ~(size_t)63);
+            a.n_parts[q] = sm.n_parts;
+            a.n[q] = (uint32_t)sm.rows;
+            longest = std::max(longest, sm.rows);
+        }
+        hipLaunchKernelGGL(sum_partials_kernel, dim3((unsigned)((longest + 255) / 256), (unsigned)nb), dim3(256), 0, c->stream, a);
         HIPCHECK(c, hipGetLastError());
     }
     return LARQL_OK;
