@@ -519,6 +519,56 @@ def run_c4(be, fmt, args):
     be.moe_layer_destroy(layer)
 
 
+def run_kq(be, fmt, args):
+    """Beside BASELINE configs[3]: the MoE layer over a Q4_K expert bank at Gemma-4-26B-A4B's shapes (128 experts, top-8,
+    hidden 2816, intermediate 704 stored 768 wide, GeluTanh) — cpu_moe_forward's integer expert path, residual -> output."""
+    O = _oracle()
+    E, k, H, I, IP = 128, 8, 2816, 704, 768
+    rng = np.random.default_rng(0x5EED0600)
+    # (a bank of 128 distinct experts on the device; four distinct weight sets on the host keep the set-up short)
+    gus = [O.quantize_q4_k((rng.standard_normal((2 * I, H)) * 0.05).astype(np.float32)) for _ in range(4)]
+    dns = [O.quantize_q4_k((rng.standard_normal((H, IP)) * 0.05).astype(np.float32)) for _ in range(4)]
+    gate_up, down = [gus[e % 4] for e in range(E)], [dns[e % 4] for e in range(E)]
+    router_w = (rng.standard_normal((E, H)) * 0.05).astype(np.float32)
+    layer = be.moe_layer_create(gate_up, down, None, None, router_w, k, H, I, fmt.MOE_ROWS_CONTIGUOUS_HALVES, expert_scales=fmt.MOE_SCALES_INLINE,
+                                expert_data_format=fmt.FMT_Q4_K, gate_rule=fmt.MOE_GATE_GELU_TANH)
+    assert layer, be.last_error()
+    expert_bytes = gus[0].size + dns[0].size
+    for T in (1, 16):
+        x = be.malloc(T * H * 4 + 64)
+        be.dev_fill_normal(x, T * H, 0x5EED06F0 + T, 1.0)
+        de, dw, out = be.malloc(T * k * 4), be.malloc(T * k * 4), be.malloc(T * H * 4)
+
+        def layer_fwd():
+            be.dev_moe_layer_forward(layer, x, x, T, out, de, dw)
+        layer_fwd(); be.synchronize()
+        xv = be.d2h(x, (T, H), np.float32)
+        experts, wts = be.d2h(de, (T, k), np.uint32), be.d2h(dw, (T, k), np.float32)
+        want_route = O.moe_route_from_router_input(xv[0], router_w, None, k)
+        assert [int(e) for e in experts[0]] == [e for e, _ in want_route] and np.allclose(wts[0], [w for _, w in want_route], rtol=5e-5)
+        t0 = time.perf_counter()
+        want = O.moe_block_kq(xv[:1], experts[:1], wts[:1], gate_up, down, H, H, I, 4, None, None, O.GATE_GELU_TANH)
+        cpu_s = time.perf_counter() - t0
+        got = be.d2h(out, (T, H), np.float32)[:1]
+        rel = float(np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want))
+        assert rel < 1e-3, rel
+        ms = _timeit(be, layer_fwd, args.steps)
+        slots = T * k
+        algo = slots * expert_bytes + E * H * 4 + T * (8 * H + 4 * E)      # every slot reads its expert's matrices (no sharing between tokens yet)
+        _emit(f"Q4_K MoE layer us (Gemma-4-26B-A4B shapes: 128 experts, top-8, batch {T})", round(ms * 1e3, 2), "us/layer", ms, args.steps, 2,
+              {"workload": f"MoE layer over a Q4_K expert bank as MoeLayerWeights hands it over: 128 experts x (gate_up 1408x2816, down 2816x768), "
+                           f"router_proj 128x2816, top-8, GeluTanh, Q8_K activations (the reference's integer expert path), batch {T}",
+               "launches_per_layer": 8, "slots": slots, "distinct_experts": len(set(int(v) for v in experts.reshape(-1))),
+               "verified_rel_l2_vs_oracle": rel},
+              {"kernel": "gemv_q4k_q8k (gate/up, down launches) + the small kernels around them", "bound": "hbm", "achieved": round(algo / ms / 1e6, 1),
+               "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(algo / ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": None},
+              {"value": round(cpu_s * 1e6 * T, 1), "unit": "us/layer", "cores": 1, "kind": "port",
+               "sample": f"one token through the checker's scalar integer expert path, one thread, scaled by {T} tokens"}, higher=False)
+        for p_ in (x, de, dw, out):
+            be.free(p_)
+    be.moe_layer_destroy(layer)
+
+
 def run_c5(be, fmt, args):
     """BASELINE configs[4]: batched-prefill Q4_K GEMM at Gemma-3-12B shapes, 512 tokens, f16 MFMA on integer weights, bf16 activations."""
     O = _oracle()
@@ -722,7 +772,7 @@ def main():
                          "does not survive HIP graph capture in this image)")
     ap.add_argument("--headline-only", action="store_true",
                     help="skip the dependency-ordered arm, the host-tier call timings and the other configurations (profiling runs)")
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "q8k", "formats"],
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "q8k", "formats", "kq"],
                     help="c2 (default) is the headline decode stack; the others are BASELINE's remaining configs")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run the plain 16-byte copy kernel on 1 GiB three times (known size, for scaling "
@@ -756,7 +806,7 @@ def main():
                           "read_only_GBps": round(n / ms_r / 1e6, 1)}))
         return
     if args.workload != "c2":
-        {"c1": run_c1, "c3": run_c3, "c4": run_c4, "c5": run_c5, "q8k": run_q8k, "formats": run_formats}[args.workload](be, fmt, args)
+        {"c1": run_c1, "c3": run_c3, "c4": run_c4, "c5": run_c5, "q8k": run_q8k, "formats": run_formats, "kq": run_kq}[args.workload](be, fmt, args)
         return
     stack = Stack(be, fmt, layers=args.layers)
 
@@ -911,7 +961,7 @@ def other_configs(be, fmt, args):
     short.cpu_seconds = 0.4 if args.no_cpu else min(args.cpu_seconds, 4.0)
     _COLLECT = []
     try:
-        for fn in (run_c1, run_c3, run_c4, run_c5, run_formats):
+        for fn in (run_c1, run_c3, run_c4, run_kq, run_c5, run_formats):
             fn(be, fmt, short)
         lines = _COLLECT
     finally:
