@@ -83,6 +83,11 @@ struct PinBuf {
 
 constexpr size_t kHostMats = 8;  // matrices one host-tier submission stages (their jobs travel in the kernel arguments)
 
+// Job tables of host-tier and enqueue-only calls live in a few device buffers with pinned staging beside them; a call's
+// table goes to the slot its shape hashes to, so that the calls of a loop (a layer's router gemv, gate/up and down
+// launches, every token) each find the table they sent last time still in place.
+constexpr int kTableSlots = 8;
+
 struct larql_hip_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
@@ -92,13 +97,13 @@ struct larql_hip_ctx {
     std::mutex mu;
     std::string name, info, last_error;
     std::vector<Region> regions;
-    DevBuf w[kHostMats], aux[kHostMats], x, out, tables[4], misc, scores, q8, q8s, parts;
+    DevBuf w[kHostMats], aux[kHostMats], x, out, tables[kTableSlots], misc, scores, q8, q8s, parts;
     // pinned staging for job tables: the upload is asynchronous, the event says when a slot may be rewritten
-    void *table_host[4] = {nullptr, nullptr, nullptr, nullptr};
-    size_t table_host_cap[4] = {0, 0, 0, 0};
-    hipEvent_t table_ev[4] = {nullptr, nullptr, nullptr, nullptr};
-    void *table_sent_dst[4] = {nullptr, nullptr, nullptr, nullptr};  // where the table staged in table_host[i] went, and its size:
-    size_t table_sent_bytes[4] = {0, 0, 0, 0};                      // an identical table for the same place is not sent again
+    void *table_host[kTableSlots] = {};
+    size_t table_host_cap[kTableSlots] = {};
+    hipEvent_t table_ev[kTableSlots] = {};
+    void *table_sent_dst[kTableSlots] = {};   // where the table staged in table_host[i] went, and its size:
+    size_t table_sent_bytes[kTableSlots] = {};  // an identical table for the same place is not sent again
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     uint8_t *log2_up = nullptr;  // 256-entry table for the MXFP4 encoder
     int *nan_flag = nullptr;       // [0]: device tier, raised by any call, cleared when taken; [1]: host tier, cleared by every call
@@ -444,9 +449,8 @@ int enqueue_jobs(larql_hip_ctx *c, std::vector<GemvJob> &jobs_in) {
     }
     int rc = check_jobs(c, jobs);
     if (rc) return rc;
-    int slot = 0;
     for (std::vector<GemvJob> &live : group_by_kind(jobs)) {
-        const int sl = slot++ % 4;
+        const int sl = (int)(((size_t)live[0].kind * 31 + live.size() * 7 + ((uintptr_t)live[0].w >> 8) + ((uintptr_t)live[0].out >> 6)) % kTableSlots);
         DevBuf &tb = c->tables[sl];
         if (live.size() > (size_t)kInlineJobs) {
             const void *before = tb.p;
@@ -552,13 +556,14 @@ void larql_hip_destroy(larql_hip_ctx *c) {
     (void)hipSetDevice(c->device);
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     for (Region &r : c->regions) (void)hipFree(r.dev);
-    DevBuf *bufs[] = {&c->x, &c->out, &c->tables[0], &c->tables[1], &c->tables[2], &c->tables[3], &c->misc, &c->scores, &c->q8, &c->q8s, &c->parts};
+    DevBuf *bufs[] = {&c->x, &c->out, &c->misc, &c->scores, &c->q8, &c->q8s, &c->parts};
+    for (DevBuf &t : c->tables) if (t.p) (void)hipFree(t.p);
     for (DevBuf *b : bufs) if (b->p) (void)hipFree(b->p);
     for (size_t i = 0; i < kHostMats; i++) {
         if (c->w[i].p) (void)hipFree(c->w[i].p);
         if (c->aux[i].p) (void)hipFree(c->aux[i].p);
     }
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < kTableSlots; i++) {
         if (c->table_host[i]) (void)hipHostFree(c->table_host[i]);
         if (c->table_ev[i]) (void)hipEventDestroy(c->table_ev[i]);
     }
@@ -2277,10 +2282,12 @@ static int moe_layer_enqueue(larql_hip_ctx *c, larql_hip_moe_layer *L, const flo
         // the weighted sum with the down bias inside the weight.
         const size_t slots = tokens * k, inter = L->inter, ip = L->inter_padded, cols = L->cols;
         if (tokens > 65535 || slots > 65535) return fail(c, LARQL_UNSUPPORTED, "moe_layer: too many tokens in one call for a k-quant bank");
-        HIPCHECK(c, router_select_launch(c->stream, logits, L->router_bias, (uint32_t)tokens, (uint32_t)E, (uint32_t)k, policy, experts, weights));
-        if (L->per_expert_scale) HIPCHECK(c, expert_scale_launch(c->stream, weights, experts, L->scale, (uint32_t)slots, (uint32_t)E));
         // (a float bank: the activations stay f32 — x itself, and one row of `inter` floats per slot)
         const bool dense = L->kq_dense;
+        if (dense) {
+            HIPCHECK(c, router_select_launch(c->stream, logits, L->router_bias, (uint32_t)tokens, (uint32_t)E, (uint32_t)k, policy, experts, weights));
+            if (L->per_expert_scale) HIPCHECK(c, expert_scale_launch(c->stream, weights, experts, L->scale, (uint32_t)slots, (uint32_t)E));
+        }
         const bool pad_x = dense && cols != hidden;  // rows stored wider than hidden: x goes in zero-padded
         const size_t xq_stride = dense ? (pad_x ? cols : hidden) * sizeof(float) : (q8k_bytes(cols) + 255) & ~(size_t)255;
         const size_t aq_stride = dense ? ((inter * sizeof(float) + 255) & ~(size_t)255) : (q8k_bytes(ip) + 255) & ~(size_t)255;
@@ -2290,7 +2297,10 @@ static int moe_layer_enqueue(larql_hip_ctx *c, larql_hip_moe_layer *L, const flo
         float *g = (float *)L->ws.p, *u = g + slots * inter, *dd = u + slots * inter;
         uint8_t *xq = (dense && !pad_x) ? (uint8_t *)const_cast<float *>(x) : (uint8_t *)L->ws.p + f_bytes;
         uint8_t *aq = (uint8_t *)L->ws.p + f_bytes + x_area;
-        if (!dense) HIPCHECK(c, quantize_rows_to_q8k_launch(c->stream, x, hidden, (uint32_t)hidden, (uint32_t)cols, (uint32_t)tokens, xq, xq_stride));
+        if (!dense)  // the route and the Q8_K expert input of every token: one launch
+            HIPCHECK(c, moe_kq_route_quant_launch(c->stream, logits, L->router_bias, (uint32_t)tokens, (uint32_t)E, (uint32_t)k, policy,
+                                                  L->per_expert_scale ? L->scale : nullptr, experts, weights, x, hidden, (uint32_t)hidden, (uint32_t)cols, xq,
+                                                  xq_stride));
         else if (pad_x) HIPCHECK(c, pad_rows_f32_launch(c->stream, x, hidden, (uint32_t)hidden, (uint32_t)cols, (uint32_t)tokens, (float *)xq));
         jobs.clear();
         for (size_t s = 0; s < slots; s++) {

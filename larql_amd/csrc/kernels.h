@@ -205,6 +205,9 @@ hipError_t quantize_rows_to_q8k_launch(hipStream_t s, const float *src, size_t s
 hipError_t moe_kq_act_q8k_launch(hipStream_t s, const float *g, const float *u, uint32_t inter, uint32_t inter_padded, uint32_t slots,
                                  const uint32_t *experts, uint32_t n_experts, const float *gub, int rule, float limit, float alpha, uint8_t *dst,
                                  size_t dst_stride);
+hipError_t moe_kq_route_quant_launch(hipStream_t s, const float *logits, const float *bias, uint32_t tokens, uint32_t n_experts, uint32_t k, int policy,
+                                     const float *scale, uint32_t *experts, float *weights, const float *src, size_t src_stride, uint32_t src_cols,
+                                     uint32_t cols, uint8_t *dst, size_t dst_stride);
 hipError_t pad_rows_f32_launch(hipStream_t s, const float *src, size_t src_stride, uint32_t src_cols, uint32_t cols, uint32_t rows, float *dst);
 hipError_t moe_act_f32_launch(hipStream_t s, const float *g, const float *u, uint32_t inter, uint32_t slots, const uint32_t *experts, uint32_t n_experts,
                               const float *gub, int rule, float limit, float alpha, float *act, size_t act_stride);

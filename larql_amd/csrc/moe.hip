@@ -134,6 +134,40 @@ __global__ void __launch_bounds__(256) quantize_rows_to_q8k_kernel(const float *
     q8k_store(dst + (size_t)blockIdx.y * dst_stride, cols, sb, lane, codes, scale, sum);
 }
 
+// Token `blockIdx.x`'s route and its expert input in one launch (they do not depend on one another): wavefront 0 selects
+// as router_select_kernel does and applies MoeExpertScalePolicy::PerExpert where a scale table is given (as
+// expert_scale_kernel does); the four wavefronts then quantise the token's row as quantize_rows_to_q8k_kernel does.
+__global__ void __launch_bounds__(256) moe_kq_route_quant_kernel(const float *__restrict__ logits, const float *__restrict__ bias, uint32_t n_experts, uint32_t k,
+                                                                int policy, const float *__restrict__ scale, uint32_t *__restrict__ experts,
+                                                                float *__restrict__ weights, const float *__restrict__ src, size_t src_stride,
+                                                                uint32_t src_cols, uint32_t cols, uint8_t *__restrict__ dst, size_t dst_stride) {
+    const uint32_t t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+    if (wave == 0) {
+        uint32_t sel_idx[kRouterMaxK];
+        float sel_w[kRouterMaxK];
+        router_select_any(logits + (size_t)t * n_experts, bias, n_experts, k, policy, lane, sel_idx, sel_w);
+        if (lane == 0) {
+#pragma unroll
+            for (int r = 0; r < kRouterMaxK; r++)
+                if ((uint32_t)r < k) {
+                    const uint32_t e = sel_idx[r];
+                    experts[(size_t)t * k + r] = e;
+                    weights[(size_t)t * k + r] = (scale && e < n_experts) ? sel_w[r] * scale[e] : sel_w[r];
+                }
+        }
+    }
+    const float *s = src + (size_t)t * src_stride;
+    for (uint32_t sb = wave; sb < cols / 256; sb += 4) {
+        const uint32_t j = sb * 256 + 4 * lane;
+        float v[4];
+#pragma unroll
+        for (uint32_t i = 0; i < 4; i++) v[i] = j + i < src_cols ? s[j + i] : 0.0f;
+        uint32_t codes; float sc; int sum;
+        q8k_block(v, codes, sc, sum);
+        q8k_store(dst + (size_t)t * dst_stride, cols, sb, lane, codes, sc, sum);
+    }
+}
+
 // Row `blockIdx.y` of src ([rows, src_cols] floats, src_stride apart) zero-padded to `cols` floats at dst + row * cols:
 // the expert input of a float bank whose rows are stored wider than hidden (forward.rs:176-184).
 __global__ void __launch_bounds__(256) pad_rows_f32_kernel(const float *__restrict__ src, size_t src_stride, uint32_t src_cols, uint32_t cols,
@@ -503,6 +537,14 @@ hipError_t moe_kq_act_q8k_launch(hipStream_t s, const float *g, const float *u, 
     if (slots == 0 || inter_padded < 256) return hipSuccess;
     hipLaunchKernelGGL(moe_kq_act_q8k_kernel, dim3((inter_padded / 256 + 3) / 4, slots), dim3(256), 0, s, g, u, inter, inter_padded, experts, n_experts,
                        gub, rule, limit, alpha, dst, dst_stride);
+    return hipGetLastError();
+}
+hipError_t moe_kq_route_quant_launch(hipStream_t s, const float *logits, const float *bias, uint32_t tokens, uint32_t n_experts, uint32_t k, int policy,
+                                     const float *scale, uint32_t *experts, float *weights, const float *src, size_t src_stride, uint32_t src_cols,
+                                     uint32_t cols, uint8_t *dst, size_t dst_stride) {
+    if (tokens == 0) return hipSuccess;
+    hipLaunchKernelGGL(moe_kq_route_quant_kernel, dim3(tokens), dim3(256), 0, s, logits, bias, n_experts, k, policy, scale, experts, weights, src,
+                       src_stride, src_cols, cols, dst, dst_stride);
     return hipGetLastError();
 }
 hipError_t pad_rows_f32_launch(hipStream_t s, const float *src, size_t src_stride, uint32_t src_cols, uint32_t cols, uint32_t rows, float *dst) {
