@@ -459,7 +459,7 @@ int larql_hip_dev_moe_mxfp4_routed(larql_hip_ctx *ctx, const larql_hip_mxfp4_exp
  * (MoeExpertScales::Paired, moe.rs:214-238), the fused gate+up rows Interleaved or as ContiguousHalves
  * (MoeFusedRowLayout, moe.rs:294-332), and the router's own tensors.  larql_hip_moe_layer_create makes such a layer
  * resident: every slice is uploaded where the expert kernels want it (expert after expert in one region; the halves of
- * a ContiguousHalves bank apart), so the caller gathers nothing.  Served: expert_data_format MXFP4 with Paired scales
+ * a ContiguousHalves MXFP4 bank interleaved row by row on the way up), so the caller gathers nothing.  Served: expert_data_format MXFP4 with Paired scales
  * (what a native GPT-OSS bank is; the CPU tier refuses it, cpu/ops/moe/forward.rs:69-75) and MoeGateRule::ClampedGlu;
  * MXFP4 with Inline scales is LARQL_REFUSED_SHAPE (the format keeps its exponents apart: there is nothing to read them
  * from).  Also served: expert_data_format Q4_K or Q6_K with Inline scales and ContiguousHalves rows — the per-layer

@@ -2219,11 +2219,18 @@ int larql_hip_moe_layer_create(larql_hip_ctx *c, const larql_hip_moe_layer_weigh
         if (inter_rows) {  // the fused rows stay as stored: gate on the even, up on the odd rows, walked in place
             put(o_gup + x * gu_p, w->experts_gate_up[x], gu_p);
             put(o_gus + x * gu_s, w->scales_gate_up[x], gu_s);
-        } else {           // [gate rows | up rows] per expert: the gate halves of all experts, then the up halves
-            put(o_gup + x * (gu_p / 2), w->experts_gate_up[x], gu_p / 2);
-            put(o_gup + E * (gu_p / 2) + x * (gu_p / 2), w->experts_gate_up[x] + gu_p / 2, gu_p / 2);
-            put(o_gus + x * (gu_s / 2), w->scales_gate_up[x], gu_s / 2);
-            put(o_gus + E * (gu_s / 2) + x * (gu_s / 2), w->scales_gate_up[x] + gu_s / 2, gu_s / 2);
+        } else {
+            // [gate rows | up rows] per expert: interleaved on the way up (gate row r to row 2r, up row r to row 2r+1: a
+            // strided copy per half), so that the resident bank is walked as one fused matrix like a bank stored that way —
+            // a one-token block then hands the gated activation from stage to stage as operand terms (20 instead of 24 us)
+            const size_t rb = (hidden / 32) * 16, rs = hidden / 32;  // bytes of a row: nibbles, exponents
+            auto put2d = [&](size_t dst, const uint8_t *src, size_t row) {
+                if (e == hipSuccess) e = hipMemcpy2DAsync(d + dst, 2 * row, src, row, row, inter, hipMemcpyHostToDevice, c->stream);
+            };
+            put2d(o_gup + x * gu_p, w->experts_gate_up[x], rb);
+            put2d(o_gup + x * gu_p + rb, w->experts_gate_up[x] + gu_p / 2, rb);
+            put2d(o_gus + x * gu_s, w->scales_gate_up[x], rs);
+            put2d(o_gus + x * gu_s + rs, w->scales_gate_up[x] + gu_s / 2, rs);
         }
         put(o_dnp + x * dn_p, w->experts_down[x], dn_p);
         put(o_dns + x * dn_s, w->scales_down[x], dn_s);
@@ -2240,12 +2247,12 @@ int larql_hip_moe_layer_create(larql_hip_ctx *c, const larql_hip_moe_layer_weigh
         return fail(c, LARQL_E_DEVICE, "moe_layer: upload: %s", hipGetErrorString(e));
     }
     L->bank.gate_packed = d + o_gup; L->bank.gate_scales = d + o_gus;
-    L->bank.up_packed = inter_rows ? nullptr : d + o_gup + E * (gu_p / 2);
-    L->bank.up_scales = inter_rows ? nullptr : d + o_gus + E * (gu_s / 2);
+    L->bank.up_packed = nullptr;  // (the resident bank is interleaved whichever way the slices came)
+    L->bank.up_scales = nullptr;
     L->bank.down_packed = d + o_dnp; L->bank.down_scales = d + o_dns;
     L->bank.n_experts = E; L->bank.hidden = hidden; L->bank.inter = inter;
     L->bank.limit = w->glu_limit; L->bank.alpha = w->glu_alpha;
-    L->bank.gate_up_interleaved = inter_rows ? 1 : 0;
+    L->bank.gate_up_interleaved = 1;
     L->bank.router_bias = w->router_bias ? (const float *)(d + o_rb) : nullptr;
     L->bank.gate_up_bias = w->experts_gate_up_bias ? (const float *)(d + o_gub) : nullptr;
     L->bank.down_bias = w->experts_down_bias ? (const float *)(d + o_db) : nullptr;
