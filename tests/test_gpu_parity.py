@@ -1282,6 +1282,7 @@ def test_moe_layer_from_per_expert_slices_with_router_projection(be, fmt, T, E, 
     (1, 6, 2, 2816, 2816, 704, "q4k", 1, False, False),    # Gemma 4 26B-A4B's real expert shape
     (4, 5, 3, 512, 512, 320, "q6k", 2, True, False),       # a Q6_K bank, SiLU
     (1, 4, 2, 256, 768, 256, "q6k", 1, False, True),
+    (300, 8, 2, 256, 256, 256, "q4k", 2, True, False),     # many tokens: 600 slots, job tables of 1200 and 600 entries
 ])
 def test_moe_layer_over_a_k_quant_bank_matches_the_integer_expert_path(be, fmt, T, E, k, hidden, cols, inter, wfmt, rule, biases, per_expert):
     """MoeLayerWeights with expert_data_format Q4_K / Q6_K (Inline scales, ContiguousHalves rows): cpu_moe_forward's
@@ -1520,6 +1521,10 @@ def test_moe_layer_k_quant_refusals(be, fmt):
     assert be.moe_layer_create(gu, dn, None, None, rw, k, hidden, inter, fmt.MOE_ROWS_CONTIGUOUS_HALVES, **dict(kw, gate_rule=7)) is None
     assert be.moe_layer_create([g[:-144] for g in gu], dn, None, None, rw, k, hidden, inter, fmt.MOE_ROWS_CONTIGUOUS_HALVES, **kw) is None
     assert be.moe_layer_create(gu, [d[:-1] for d in dn], None, None, rw, k, hidden, inter, fmt.MOE_ROWS_CONTIGUOUS_HALVES, **kw) is None
+    # more (token, expert) slots than one call takes
+    assert be.moe_layer_forward(ok2 := be.moe_layer_create(gu, dn, None, None, rw, k, hidden, inter, fmt.MOE_ROWS_CONTIGUOUS_HALVES, **kw),
+                                np.zeros((40000, hidden), F), np.zeros((40000, hidden), F), k) is None
+    be.moe_layer_destroy(ok2)
     # an MXFP4 bank under another gate rule: no kernel
     g4 = [O.quantize_mxfp4((rng.standard_normal(2 * 32 * 64) * 0.02).astype(F), 2 * 32, 64) for _ in range(E)]
     d4 = [O.quantize_mxfp4((rng.standard_normal(64 * 32) * 0.02).astype(F), 64, 32) for _ in range(E)]
