@@ -509,7 +509,8 @@ void larql_hip_moe_layer_destroy(larql_hip_ctx *ctx, larql_hip_moe_layer *layer)
  * renormalise, per-expert scale) followed by the expert block (cpu/ops/moe/forward.rs:201-270) on host slices:
  * router_in and x are [tokens, hidden] (the router's and the experts' input: the reference derives both from the
  * residual under MoeRoutingPolicy, and they may be the same slice), out is [tokens, hidden].  experts_out /
- * weights_out ([tokens, min(top_k, num_experts)], may be NULL) receive the route.  One submission. */
+ * weights_out ([tokens, min(top_k, num_experts)], may be NULL) receive the route.  One submission.  A k-quant or float
+ * bank takes up to 65535 (token, expert) slots per call (more: LARQL_UNSUPPORTED — split the tokens over calls). */
 int  larql_hip_moe_layer_forward(larql_hip_ctx *ctx, larql_hip_moe_layer *layer, const float *router_in, const float *x,
                                  size_t tokens, float *out, uint32_t *experts_out, float *weights_out);
 /* The same on resident operands; only enqueues.  The router's projection runs on the device (a [num_experts, hidden]
